@@ -1,0 +1,423 @@
+// TEST INFRASTRUCTURE - CPU oracle, never linked into or called by the product.
+//
+// The transformer forward the decode step runs, as the mathematical reference
+// the 2e-2 max-abs / 1e-3 mean-abs logit tolerances are judged against:
+// exact f32 dequantisation of the stored blocks, f32 activations, every
+// reduction accumulated in double, K/V rounded to f16 when stored (the
+// configs' "f16 KV cache").
+//
+// The arithmetic of the reference's forward lives in its llama.cpp fork
+// (.gitmodules:1-4; upstream base ggml-org/llama.cpp@cd8427d0, recorded at
+// crates/retrograd-ffi/runtime/llama.cpp.lock:6-7), which is absent from the
+// reference checkout, so this file follows the published architectures the
+// reference's fixtures name (scripts/gen-tiny-fixture.py:245-261 qwen2 tensor
+// names and metadata keys; scripts/gen-tiny-moe-fixture.py:221-244 MoE names):
+//   llama    : RMSNorm, GQA attention, RoPE on adjacent pairs (2i, 2i+1), SwiGLU
+//   qwen2    : the same with q/k/v biases and RoPE on split halves (i, i+d/2)
+//   qwen3moe : per-head RMSNorm on q and k, split-half RoPE, softmax router,
+//              top-k experts with renormalised weights, SwiGLU experts
+// RMSNorm is x / sqrt(mean(x^2) + eps) with the weight multiply a separate op
+// (generated/rir/rms_norm/kernel.shared_reduce.cu:27-55).
+//
+// PARITY UNPINNED against the reference at float level: no reference test or
+// fixture records absolute logits of a causal model. What pins this file
+// instead (tests/test_oracle_model.py): a numpy float64 transformer written
+// independently from the formulas, permutation invariance over batch rows,
+// chunked prefill == token-by-token decode, seq_cp copy == source.
+#pragma once
+
+#include "gguf.hpp"
+#include "quant.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <memory>
+#include <numeric>
+
+namespace oracle {
+
+struct hparams {
+    std::string arch;
+    int n_layer = 0, n_embd = 0, n_head = 0, n_head_kv = 0, head_dim = 0, n_ff = 0, n_vocab = 0;
+    int n_expert = 0, n_expert_used = 0, n_ff_exp = 0;
+    int rope_dim = 0;
+    bool rope_neox = false;
+    double eps = 1e-5, rope_base = 10000.0;
+};
+
+struct lora_pair {
+    const gguf_tensor * a = nullptr;  // ne = [n_in, r]
+    const gguf_tensor * b = nullptr;  // ne = [r, n_out]
+};
+
+struct adapter {
+    std::unique_ptr<gguf_file> file;
+    double alpha = 0.0;
+    float scale = 1.0f;
+    std::map<std::string, lora_pair> pairs;  // keyed by base weight name
+};
+
+struct model {
+    explicit model(const std::string & path) : file(path) {
+        hparams & h = hp;
+        h.arch = file.s("general.architecture");
+        const std::string p = h.arch + ".";
+        h.n_layer = (int)file.u(p + "block_count");
+        h.n_embd = (int)file.u(p + "embedding_length");
+        h.n_head = (int)file.u(p + "attention.head_count");
+        h.n_head_kv = (int)file.u_or(p + "attention.head_count_kv", h.n_head);
+        h.head_dim = (int)file.u_or(p + "attention.key_length", h.n_embd / h.n_head);
+        h.n_ff = (int)file.u_or(p + "feed_forward_length", 0);
+        h.eps = file.f_or(p + "attention.layer_norm_rms_epsilon", 1e-5);
+        h.rope_base = file.f_or(p + "rope.freq_base", 10000.0);
+        h.rope_dim = (int)file.u_or(p + "rope.dimension_count", h.head_dim);
+        h.n_expert = (int)file.u_or(p + "expert_count", 0);
+        h.n_expert_used = (int)file.u_or(p + "expert_used_count", 0);
+        h.n_ff_exp = (int)file.u_or(p + "expert_feed_forward_length", h.n_ff);
+        if (h.arch == "llama") h.rope_neox = false;
+        else if (h.arch == "qwen2" || h.arch == "qwen3moe" || h.arch == "qwen3") h.rope_neox = true;
+        else throw std::runtime_error("oracle: unsupported architecture " + h.arch);
+        h.n_vocab = (int)file.need("token_embd.weight").ne[1];
+    }
+    gguf_file file;
+    hparams hp;
+    std::map<int, adapter> adapters;
+    int next_adapter = 1;
+};
+
+// ---------------------------------------------------------------------------
+
+// y[t][n] = sum_k W[n][k] x[t][k], W stored row by row (ne = [K, N]) in any
+// supported block format; one thread owns an output feature, so the result
+// does not depend on the thread count.
+inline void matmul(const gguf_tensor & w, const float * x, int T, float * y, int ldy = -1) {
+    const size_t K = w.ne[0];
+    const size_t N = w.ne[1];
+    const size_t rb = row_bytes(w.type, K);
+    if (ldy < 0) ldy = (int)N;
+#pragma omp parallel
+    {
+        std::vector<float> row(K);
+#pragma omp for schedule(static)
+        for (long n = 0; n < (long)N; ++n) {
+            decode_row(w.type, w.data + (size_t)n * rb, K, row.data());
+            for (int t = 0; t < T; ++t) {
+                const float * xt = x + (size_t)t * K;
+                double a0 = 0, a1 = 0, a2 = 0, a3 = 0;
+                size_t k = 0;
+                for (; k + 4 <= K; k += 4) {
+                    a0 += (double)row[k] * xt[k];
+                    a1 += (double)row[k + 1] * xt[k + 1];
+                    a2 += (double)row[k + 2] * xt[k + 2];
+                    a3 += (double)row[k + 3] * xt[k + 3];
+                }
+                for (; k < K; ++k) a0 += (double)row[k] * xt[k];
+                y[(size_t)t * ldy + n] = (float)((a0 + a1) + (a2 + a3));
+            }
+        }
+    }
+}
+
+inline void rmsnorm(const float * x, const float * w, int n, double eps, float * y) {
+    double ss = 0.0;
+    for (int i = 0; i < n; ++i) ss += (double)x[i] * x[i];
+    const float scale = (float)(1.0 / std::sqrt(ss / n + eps));
+    for (int i = 0; i < n; ++i) y[i] = (x[i] * scale) * (w ? w[i] : 1.0f);
+}
+
+inline const float * f32_data(const gguf_tensor & t) {
+    if (t.type != T_F32) throw std::runtime_error("oracle: expected an F32 vector: " + t.name);
+    return (const float *)t.data;
+}
+
+// Rotates one head in place; angle = pos * base^(-2i/d) evaluated in double.
+inline void rope(float * v, int head_dim, int rope_dim, int pos, double base, bool neox) {
+    const int half = rope_dim / 2;
+    for (int i = 0; i < half; ++i) {
+        const double angle = (double)pos * std::pow(base, -2.0 * i / rope_dim);
+        const double c = std::cos(angle), s = std::sin(angle);
+        const int i0 = neox ? i : 2 * i;
+        const int i1 = neox ? i + half : 2 * i + 1;
+        const double a = v[i0], b = v[i1];
+        v[i0] = (float)(a * c - b * s);
+        v[i1] = (float)(a * s + b * c);
+    }
+    (void)head_dim;
+}
+
+struct slot_state {
+    int begin = 0, end = 0;              // resident positions [begin, end)
+    std::vector<std::vector<uint16_t>> k, v;   // per layer: pos * kv_dim halves, indexed by absolute pos
+};
+
+struct context {
+    context(model * m, int n_seq_max) : mdl(m), slots((size_t)n_seq_max) {
+        for (auto & s : slots) {
+            s.k.resize((size_t)m->hp.n_layer);
+            s.v.resize((size_t)m->hp.n_layer);
+        }
+    }
+    model * mdl;
+    std::vector<slot_state> slots;
+
+    int kv_dim() const { return mdl->hp.n_head_kv * mdl->hp.head_dim; }
+
+    void seq_rm(int slot, int p0, int p1) {
+        slot_state & s = slots.at((size_t)slot);
+        if (p0 < 0) p0 = 0;
+        if (p1 < 0) p1 = 1 << 30;
+        if (s.end <= s.begin) return;
+        if (p0 <= s.begin && p1 >= s.end) { s.begin = s.end = 0; return; }
+        if (p1 >= s.end) { s.end = std::max(s.begin, p0); return; }
+        if (p0 <= s.begin) { s.begin = std::min(s.end, p1); return; }
+        throw std::runtime_error("oracle: seq_rm would leave a hole");
+    }
+    void seq_cp(int src, int dst, int p0, int p1) {
+        const slot_state & a = slots.at((size_t)src);
+        slot_state & b = slots.at((size_t)dst);
+        if (p0 < 0) p0 = 0;
+        if (p1 < 0) p1 = 1 << 30;
+        p0 = std::max(p0, a.begin);
+        p1 = std::min(p1, a.end);
+        if (p1 <= p0 || src == dst) return;
+        const size_t kd = (size_t)kv_dim();
+        if (b.end <= b.begin) { b.begin = p0; b.end = p0; }
+        if (p0 != b.end && p1 != b.begin) throw std::runtime_error("oracle: seq_cp range is not adjacent to dst");
+        for (size_t l = 0; l < b.k.size(); ++l) {
+            if (b.k[l].size() < (size_t)p1 * kd) { b.k[l].resize((size_t)p1 * kd); b.v[l].resize((size_t)p1 * kd); }
+            std::copy(a.k[l].begin() + (size_t)p0 * kd, a.k[l].begin() + (size_t)p1 * kd, b.k[l].begin() + (size_t)p0 * kd);
+            std::copy(a.v[l].begin() + (size_t)p0 * kd, a.v[l].begin() + (size_t)p1 * kd, b.v[l].begin() + (size_t)p0 * kd);
+        }
+        b.begin = std::min(b.begin, p0);
+        b.end = std::max(b.end, p1);
+    }
+
+    // y += scale * alpha/r * B (A x) for the adapter each token decodes under.
+    void add_lora(const std::string & wname, const float * x, int T, const int32_t * adapter_of,
+                  float * y, int N) const {
+        if (!adapter_of) return;
+        for (int t = 0; t < T; ++t) {
+            if (adapter_of[t] <= 0) continue;
+            auto ai = mdl->adapters.find(adapter_of[t]);
+            if (ai == mdl->adapters.end()) throw std::runtime_error("oracle: adapter not loaded");
+            auto pi = ai->second.pairs.find(wname);
+            if (pi == ai->second.pairs.end()) continue;
+            const gguf_tensor & A = *pi->second.a;
+            const gguf_tensor & B = *pi->second.b;
+            const int r = (int)A.ne[1];
+            const int K = (int)A.ne[0];
+            std::vector<float> mid((size_t)r), delta((size_t)N);
+            matmul(A, x + (size_t)t * K, 1, mid.data());
+            matmul(B, mid.data(), 1, delta.data());
+            const float s = (float)((double)ai->second.scale * ai->second.alpha / r);
+            for (int n = 0; n < N; ++n) y[(size_t)t * N + n] += s * delta[n];
+        }
+    }
+
+    // One decode over a packed batch. logits_out: n_outputs rows of n_vocab.
+    void step(int T, const int32_t * tok, const int32_t * pos, const int32_t * slot,
+              const int32_t * adapter_of, const uint8_t * want, float * logits_out) {
+        const hparams & h = mdl->hp;
+        const gguf_file & g = mdl->file;
+        const int E = h.n_embd, HD = h.head_dim, NH = h.n_head, NKV = h.n_head_kv;
+        const int QD = NH * HD, KD = NKV * HD;
+        const size_t kd = (size_t)KD;
+        std::vector<float> x((size_t)T * E), xn((size_t)T * E);
+        {
+            const gguf_tensor & emb = g.need("token_embd.weight");
+            const size_t rb = row_bytes(emb.type, (size_t)E);
+            for (int t = 0; t < T; ++t) decode_row(emb.type, emb.data + (size_t)tok[t] * rb, (size_t)E, &x[(size_t)t * E]);
+        }
+        // Make the positions this step writes resident before attention reads them.
+        for (int t = 0; t < T; ++t) {
+            slot_state & s = slots.at((size_t)slot[t]);
+            if (s.end <= s.begin) { s.begin = pos[t]; s.end = pos[t] + 1; }
+            if (pos[t] < s.begin) throw std::runtime_error("oracle: position before the resident range");
+            s.end = std::max(s.end, pos[t] + 1);
+            const size_t need = ((size_t)pos[t] + 1) * kd;
+            for (int l = 0; l < h.n_layer; ++l) {
+                if (s.k[(size_t)l].size() < need) { s.k[(size_t)l].resize(need); s.v[(size_t)l].resize(need); }
+            }
+        }
+        std::vector<float> q((size_t)T * QD), k((size_t)T * KD), v((size_t)T * KD), att((size_t)T * QD), proj((size_t)T * E);
+        for (int l = 0; l < h.n_layer; ++l) {
+            const std::string b = "blk." + std::to_string(l) + ".";
+            const float * wn = f32_data(g.need(b + "attn_norm.weight"));
+            for (int t = 0; t < T; ++t) rmsnorm(&x[(size_t)t * E], wn, E, h.eps, &xn[(size_t)t * E]);
+            matmul(g.need(b + "attn_q.weight"), xn.data(), T, q.data());
+            matmul(g.need(b + "attn_k.weight"), xn.data(), T, k.data());
+            matmul(g.need(b + "attn_v.weight"), xn.data(), T, v.data());
+            add_lora(b + "attn_q.weight", xn.data(), T, adapter_of, q.data(), QD);
+            add_lora(b + "attn_k.weight", xn.data(), T, adapter_of, k.data(), KD);
+            add_lora(b + "attn_v.weight", xn.data(), T, adapter_of, v.data(), KD);
+            if (const gguf_tensor * bq = g.find(b + "attn_q.bias")) {
+                const float * bk = f32_data(g.need(b + "attn_k.bias"));
+                const float * bv = f32_data(g.need(b + "attn_v.bias"));
+                const float * bqd = f32_data(*bq);
+                for (int t = 0; t < T; ++t) {
+                    for (int i = 0; i < QD; ++i) q[(size_t)t * QD + i] += bqd[i];
+                    for (int i = 0; i < KD; ++i) { k[(size_t)t * KD + i] += bk[i]; v[(size_t)t * KD + i] += bv[i]; }
+                }
+            }
+            const gguf_tensor * qn = g.find(b + "attn_q_norm.weight");
+            const gguf_tensor * kn = g.find(b + "attn_k_norm.weight");
+            for (int t = 0; t < T; ++t) {
+                for (int hh = 0; hh < NH; ++hh) {
+                    float * qh = &q[(size_t)t * QD + (size_t)hh * HD];
+                    if (qn) rmsnorm(qh, f32_data(*qn), HD, h.eps, qh);
+                    rope(qh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox);
+                }
+                slot_state & s = slots[(size_t)slot[t]];
+                for (int hh = 0; hh < NKV; ++hh) {
+                    float * kh = &k[(size_t)t * KD + (size_t)hh * HD];
+                    if (kn) rmsnorm(kh, f32_data(*kn), HD, h.eps, kh);
+                    rope(kh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox);
+                }
+                uint16_t * kc = &s.k[(size_t)l][(size_t)pos[t] * kd];
+                uint16_t * vc = &s.v[(size_t)l][(size_t)pos[t] * kd];
+                for (int i = 0; i < KD; ++i) {
+                    kc[i] = float_to_half(k[(size_t)t * KD + i]);
+                    vc[i] = float_to_half(v[(size_t)t * KD + i]);
+                }
+                s.end = std::max(s.end, pos[t] + 1);
+            }
+            const int G = NH / NKV;
+            const double inv_sqrt = 1.0 / std::sqrt((double)HD);
+#pragma omp parallel for collapse(2) schedule(dynamic)
+            for (int t = 0; t < T; ++t) {
+                for (int hh = 0; hh < NH; ++hh) {
+                    const slot_state & s = slots[(size_t)slot[t]];
+                    const int p0 = s.begin, p1 = pos[t] + 1;
+                    const int kvh = hh / G;
+                    const float * qh = &q[(size_t)t * QD + (size_t)hh * HD];
+                    std::vector<double> sc((size_t)(p1 - p0));
+                    double mx = -INFINITY;
+                    for (int p = p0; p < p1; ++p) {
+                        const uint16_t * kc = &s.k[(size_t)l][(size_t)p * kd + (size_t)kvh * HD];
+                        double d = 0.0;
+                        for (int i = 0; i < HD; ++i) d += (double)qh[i] * half_to_float(kc[i]);
+                        d *= inv_sqrt;
+                        sc[(size_t)(p - p0)] = d;
+                        mx = std::max(mx, d);
+                    }
+                    double den = 0.0;
+                    for (auto & e : sc) { e = std::exp(e - mx); den += e; }
+                    std::vector<double> acc((size_t)HD, 0.0);
+                    for (int p = p0; p < p1; ++p) {
+                        const uint16_t * vc = &s.v[(size_t)l][(size_t)p * kd + (size_t)kvh * HD];
+                        const double w = sc[(size_t)(p - p0)];
+                        for (int i = 0; i < HD; ++i) acc[(size_t)i] += w * half_to_float(vc[i]);
+                    }
+                    float * o = &att[(size_t)t * QD + (size_t)hh * HD];
+                    for (int i = 0; i < HD; ++i) o[i] = (float)(acc[(size_t)i] / den);
+                }
+            }
+            matmul(g.need(b + "attn_output.weight"), att.data(), T, proj.data());
+            add_lora(b + "attn_output.weight", att.data(), T, adapter_of, proj.data(), E);
+            for (size_t i = 0; i < x.size(); ++i) x[i] += proj[i];
+
+            const float * wf = f32_data(g.need(b + "ffn_norm.weight"));
+            for (int t = 0; t < T; ++t) rmsnorm(&x[(size_t)t * E], wf, E, h.eps, &xn[(size_t)t * E]);
+            if (h.n_expert > 0) {
+                moe_ffn(b, xn.data(), T, proj.data());
+            } else {
+                const int F = h.n_ff;
+                std::vector<float> gate((size_t)T * F), up((size_t)T * F);
+                matmul(g.need(b + "ffn_gate.weight"), xn.data(), T, gate.data());
+                matmul(g.need(b + "ffn_up.weight"), xn.data(), T, up.data());
+                for (size_t i = 0; i < gate.size(); ++i) gate[i] = silu(gate[i]) * up[i];
+                matmul(g.need(b + "ffn_down.weight"), gate.data(), T, proj.data());
+            }
+            for (size_t i = 0; i < x.size(); ++i) x[i] += proj[i];
+        }
+        // Output rows only.
+        std::vector<int> outs;
+        for (int t = 0; t < T; ++t) if (want[t]) outs.push_back(t);
+        if (outs.empty()) return;
+        const float * wo = f32_data(g.need("output_norm.weight"));
+        std::vector<float> xo(outs.size() * (size_t)E);
+        for (size_t i = 0; i < outs.size(); ++i) rmsnorm(&x[(size_t)outs[i] * E], wo, E, h.eps, &xo[i * (size_t)E]);
+        const gguf_tensor * head = g.find("output.weight");
+        if (!head) head = &g.need("token_embd.weight");
+        matmul(*head, xo.data(), (int)outs.size(), logits_out);
+        if (const gguf_tensor * ob = g.find("output.bias")) {
+            const float * bd = f32_data(*ob);
+            for (size_t i = 0; i < outs.size(); ++i)
+                for (int n = 0; n < h.n_vocab; ++n) logits_out[i * (size_t)h.n_vocab + n] += bd[n];
+        }
+    }
+
+    static float silu(float g) { return (float)((double)g / (1.0 + std::exp(-(double)g))); }
+
+    // Softmax router over all experts, top-k by probability (ties to the lower
+    // index), weights renormalised over the selected experts, SwiGLU experts.
+    void moe_ffn(const std::string & b, const float * xn, int T, float * out) const {
+        const hparams & h = mdl->hp;
+        const gguf_file & g = mdl->file;
+        const int E = h.n_embd, NE = h.n_expert, KU = h.n_expert_used, F = h.n_ff_exp;
+        std::vector<float> rl((size_t)T * NE);
+        matmul(g.need(b + "ffn_gate_inp.weight"), xn, T, rl.data());
+        const gguf_tensor & wg = g.need(b + "ffn_gate_exps.weight");
+        const gguf_tensor & wu = g.need(b + "ffn_up_exps.weight");
+        const gguf_tensor & wd = g.need(b + "ffn_down_exps.weight");
+        const size_t g_bytes = row_bytes(wg.type, (size_t)E) * (size_t)F;
+        const size_t d_bytes = row_bytes(wd.type, (size_t)F) * (size_t)E;
+        std::vector<float> gate((size_t)F), up((size_t)F), down((size_t)E);
+        for (int t = 0; t < T; ++t) {
+            const float * r = &rl[(size_t)t * NE];
+            double mx = -INFINITY;
+            for (int e = 0; e < NE; ++e) mx = std::max(mx, (double)r[e]);
+            std::vector<double> p((size_t)NE);
+            double den = 0.0;
+            for (int e = 0; e < NE; ++e) { p[(size_t)e] = std::exp((double)r[e] - mx); den += p[(size_t)e]; }
+            for (auto & e : p) e /= den;
+            std::vector<int> order((size_t)NE);
+            std::iota(order.begin(), order.end(), 0);
+            std::stable_sort(order.begin(), order.end(), [&](int a, int c) { return p[(size_t)a] > p[(size_t)c]; });
+            double wsum = 0.0;
+            for (int j = 0; j < KU; ++j) wsum += p[(size_t)order[(size_t)j]];
+            std::vector<double> acc((size_t)E, 0.0);
+            for (int j = 0; j < KU; ++j) {
+                const int e = order[(size_t)j];
+                gguf_tensor eg = wg, eu = wu, ed = wd;
+                eg.ne = {(uint64_t)E, (uint64_t)F}; eg.data = wg.data + (size_t)e * g_bytes;
+                eu.ne = {(uint64_t)E, (uint64_t)F}; eu.data = wu.data + (size_t)e * g_bytes;
+                ed.ne = {(uint64_t)F, (uint64_t)E}; ed.data = wd.data + (size_t)e * d_bytes;
+                matmul(eg, xn + (size_t)t * E, 1, gate.data());
+                matmul(eu, xn + (size_t)t * E, 1, up.data());
+                for (int i = 0; i < F; ++i) gate[(size_t)i] = silu(gate[(size_t)i]) * up[(size_t)i];
+                matmul(ed, gate.data(), 1, down.data());
+                const double w = p[(size_t)e] / wsum;
+                for (int i = 0; i < E; ++i) acc[(size_t)i] += w * down[(size_t)i];
+            }
+            for (int i = 0; i < E; ++i) out[(size_t)t * E + i] = (float)acc[(size_t)i];
+        }
+    }
+};
+
+// LoRA adapter file as the reference writes it (retro_lora.cpp:1004-1043,
+// 1143-1153): general.type = "adapter", adapter.type = "lora",
+// adapter.lora.alpha (f32), tensors "<weight>.lora_a" / "<weight>.lora_b".
+inline int load_adapter(model & m, const std::string & path, float scale) {
+    adapter a;
+    a.file.reset(new gguf_file(path));
+    if (a.file->s("general.type") != "adapter" || a.file->s("adapter.type") != "lora")
+        throw std::runtime_error("oracle: not a LoRA adapter file");
+    a.alpha = a.file->f("adapter.lora.alpha");
+    a.scale = scale;
+    for (const gguf_tensor & t : a.file->tensors) {
+        const std::string suffix_a = ".lora_a";
+        if (t.name.size() > suffix_a.size() && t.name.compare(t.name.size() - suffix_a.size(), suffix_a.size(), suffix_a) == 0) {
+            const std::string base = t.name.substr(0, t.name.size() - suffix_a.size());
+            lora_pair p;
+            p.a = &t;
+            p.b = &a.file->need(base + ".lora_b");
+            a.pairs.emplace(base, p);
+        }
+    }
+    const int id = m.next_adapter++;
+    m.adapters.emplace(id, std::move(a));
+    return id;
+}
+
+}  // namespace oracle

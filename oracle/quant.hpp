@@ -1,0 +1,214 @@
+// TEST INFRASTRUCTURE - CPU oracle, never linked into or called by the product.
+//
+// Decoders for the GGUF block formats the decode step reads, restated from the
+// reference's portable dequantisation oracle (crates/rir-core/src/quant.rs),
+// which the reference proves bit-equal to ggml's to_float on identical bytes
+// (tests/rir_quant_oracle.rs:67-103). Block geometry from
+// crates/rir-core/src/quant_table.rs (Q8_0 32 el / 34 B, MXFP4 32 el / 17 B,
+// Q4_K 256 el / 144 B).
+//
+// Pinned by: tests/test_oracle_quant.py (known answers of quant.rs:534-581,
+// exhaustive f16 against numpy, brute-force Q4_K addressing against
+// generated/rir/mul_mat_vec_q4_K/cpu.rs:52-120 semantics).
+#pragma once
+
+#include <cmath>
+#include <cstddef>
+#include <cstdint>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+
+namespace oracle {
+
+// ggml type ids as stored in a GGUF tensor table.
+enum ggml_type_id : uint32_t {
+    T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_BF16 = 30, T_MXFP4 = 39,
+};
+
+struct block_geom { uint32_t elements; uint32_t bytes; };
+
+inline block_geom geom_of(uint32_t type) {
+    switch (type) {
+        case T_F32:   return {1, 4};
+        case T_F16:   return {1, 2};
+        case T_BF16:  return {1, 2};
+        case T_Q8_0:  return {32, 34};
+        case T_MXFP4: return {32, 17};
+        case T_Q4_K:  return {256, 144};
+        default: throw std::runtime_error("oracle: unsupported ggml type " + std::to_string(type));
+    }
+}
+
+inline size_t row_bytes(uint32_t type, size_t n) {
+    const block_geom g = geom_of(type);
+    if (n % g.elements != 0) throw std::runtime_error("oracle: row is not block aligned");
+    return n / g.elements * g.bytes;
+}
+
+// IEEE binary16 -> binary32, exact incl. subnormals (quant.rs:82-103).
+inline float half_to_float(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h >> 15) << 31;
+    const uint32_t e = (h >> 10) & 0x1f;
+    const uint32_t m = h & 0x3ff;
+    uint32_t bits;
+    if (e == 0) {
+        if (m == 0) {
+            bits = sign;
+        } else {
+            // value = m * 2^-24: normalise the mantissa.
+            int shift = 0;
+            uint32_t mm = m;
+            while ((mm & 0x400) == 0) { mm <<= 1; ++shift; }
+            bits = sign | ((uint32_t)(113 - shift) << 23) | ((mm & 0x3ff) << 13);
+        }
+    } else if (e == 31) {
+        bits = sign | 0x7f800000u | (m << 13);
+    } else {
+        bits = sign | ((e + 112) << 23) | (m << 13);
+    }
+    float out;
+    std::memcpy(&out, &bits, 4);
+    return out;
+}
+
+// binary64 -> binary16, round to nearest even in ONE rounding (what Python's
+// struct.pack("<e", x) does on a double; a float argument widens exactly, so
+// this is also the binary32 -> binary16 conversion). Overflow goes to infinity.
+inline uint16_t double_to_half(double v) {
+    const uint16_t sign = std::signbit(v) ? 0x8000 : 0;
+    if (std::isnan(v)) return (uint16_t)(sign | 0x7e00);
+    double a = std::fabs(v);
+    if (std::isinf(a)) return (uint16_t)(sign | 0x7c00);
+    if (a == 0.0) return sign;
+    int e;
+    std::frexp(a, &e);              // a = f * 2^e, f in [0.5, 1)  ->  floor(log2 a) = e - 1
+    int exp2 = e - 1;
+    if (exp2 < -14) exp2 = -14;     // subnormal halves share the quantum 2^-24
+    const double quantum = std::ldexp(1.0, exp2 - 10);
+    double q = std::nearbyint(a / quantum);   // exact division; ties to even
+    if (q == 0.0) return sign;
+    if (q >= 2048.0) { q = 1024.0; ++exp2; }  // mantissa carry
+    if (exp2 > 15) return (uint16_t)(sign | 0x7c00);
+    const uint32_t qi = (uint32_t)q;
+    if (qi < 1024) return (uint16_t)(sign | qi);                       // subnormal
+    return (uint16_t)(sign | ((uint32_t)(exp2 + 15) << 10) | (qi - 1024));
+}
+
+inline uint16_t float_to_half(float f) { return double_to_half((double)f); }
+
+inline float bf16_to_float(uint16_t h) {
+    const uint32_t bits = (uint32_t)h << 16;
+    float out;
+    std::memcpy(&out, &bits, 4);
+    return out;
+}
+
+// E8M0 exponent byte scaled by 1/2 (quant.rs:107-115): 2^(x-128), the two
+// smallest landing in binary32 subnormals.
+inline float e8m0_half(uint8_t x) {
+    uint32_t bits;
+    if (x == 0) bits = 0x00200000u;
+    else if (x == 1) bits = 0x00400000u;
+    else bits = ((uint32_t)x - 1) << 23;
+    float out;
+    std::memcpy(&out, &bits, 4);
+    return out;
+}
+
+inline uint16_t rd16(const uint8_t * p) { return (uint16_t)(p[0] | (p[1] << 8)); }
+
+// 6-bit (scale, min) of sub-block j from the 12 packed bytes (quant.rs:119-128).
+inline void q4k_scale_min(int j, const uint8_t * q, uint8_t & sc, uint8_t & mn) {
+    if (j < 4) {
+        sc = q[j] & 63;
+        mn = q[j + 4] & 63;
+    } else {
+        sc = (uint8_t)((q[j + 4] & 0x0f) | ((q[j - 4] >> 6) << 4));
+        mn = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+static const int8_t k_fp4_doubled[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+
+// Decode n elements (whole blocks) of `type` from src into out.
+inline void decode_row(uint32_t type, const uint8_t * src, size_t n, float * out) {
+    switch (type) {
+        case T_F32:
+            std::memcpy(out, src, n * 4);
+            return;
+        case T_F16:
+            for (size_t i = 0; i < n; ++i) out[i] = half_to_float(rd16(src + 2 * i));
+            return;
+        case T_BF16:
+            for (size_t i = 0; i < n; ++i) out[i] = bf16_to_float(rd16(src + 2 * i));
+            return;
+        case T_Q8_0:  // quant.rs:228-234: d (f16) then 32 signed bytes
+            for (size_t b = 0; b < n / 32; ++b) {
+                const uint8_t * blk = src + b * 34;
+                const float d = half_to_float(rd16(blk));
+                for (int j = 0; j < 32; ++j) out[b * 32 + j] = d * (float)(int8_t)blk[2 + j];
+            }
+            return;
+        case T_MXFP4:  // quant.rs:286-295: e8m0 byte, low nibbles first half
+            for (size_t b = 0; b < n / 32; ++b) {
+                const uint8_t * blk = src + b * 17;
+                const float d = e8m0_half(blk[0]);
+                for (int j = 0; j < 16; ++j) {
+                    const uint8_t q = blk[1 + j];
+                    out[b * 32 + j]      = d * (float)k_fp4_doubled[q & 0x0f];
+                    out[b * 32 + j + 16] = d * (float)k_fp4_doubled[q >> 4];
+                }
+            }
+            return;
+        case T_Q4_K:  // quant.rs:399-416: d, dmin | scales[12] | qs[128]
+            for (size_t b = 0; b < n / 256; ++b) {
+                const uint8_t * blk = src + b * 144;
+                const float d = half_to_float(rd16(blk));
+                const float dmin = half_to_float(rd16(blk + 2));
+                const uint8_t * scales = blk + 4;
+                const uint8_t * qs = blk + 16;
+                float * y = out + b * 256;
+                for (int pair = 0; pair < 4; ++pair) {   // 64 elements per pair of sub-blocks
+                    uint8_t sc1, m1, sc2, m2;
+                    q4k_scale_min(2 * pair, scales, sc1, m1);
+                    q4k_scale_min(2 * pair + 1, scales, sc2, m2);
+                    const float d1 = d * (float)sc1, mm1 = dmin * (float)m1;
+                    const float d2 = d * (float)sc2, mm2 = dmin * (float)m2;
+                    const uint8_t * q = qs + 32 * pair;
+                    for (int l = 0; l < 32; ++l) {
+                        y[64 * pair + l]      = d1 * (float)(q[l] & 0x0f) - mm1;
+                        y[64 * pair + 32 + l] = d2 * (float)(q[l] >> 4) - mm2;
+                    }
+                }
+            }
+            return;
+        default:
+            throw std::runtime_error("oracle: unsupported ggml type " + std::to_string(type));
+    }
+}
+
+// ggml's quantize_row_q8_0_ref as the fixture generator restates it
+// (scripts/gen-tiny-fixture.py:173-197): d = amax/127 stored as f16, the
+// codes use the *unrounded* d, round half away from zero, clamp to 127.
+inline void quantize_q8_0(const float * x, size_t n, uint8_t * dst) {
+    for (size_t b = 0; b < n / 32; ++b) {
+        const float * v = x + b * 32;
+        double amax = 0.0;
+        for (int j = 0; j < 32; ++j) amax = std::fmax(amax, std::fabs((double)v[j]));
+        const double d = amax / 127.0;
+        const double inv = d != 0.0 ? 1.0 / d : 0.0;
+        const uint16_t h = double_to_half(d);
+        uint8_t * blk = dst + b * 34;
+        blk[0] = (uint8_t)(h & 0xff);
+        blk[1] = (uint8_t)(h >> 8);
+        for (int j = 0; j < 32; ++j) {
+            const double scaled = (double)v[j] * inv;
+            double code = std::floor(std::fabs(scaled) + 0.5);
+            if (code > 127.0) code = 127.0;
+            blk[2 + j] = (uint8_t)(int8_t)(scaled >= 0.0 ? code : -code);
+        }
+    }
+}
+
+}  // namespace oracle

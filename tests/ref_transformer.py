@@ -1,0 +1,116 @@
+"""float64 numpy transformer written from the textbook formulas, independent of
+oracle/model.hpp: used to pin the oracle's forward (tests only)."""
+import numpy as np
+
+import oracle
+from gguf_reader import Reader
+
+
+class NumpyModel:
+    def __init__(self, path):
+        r = Reader(path)
+        self.r = r
+        a = r.kv["general.architecture"]
+        self.arch = a
+        g = lambda k, d=None: r.kv.get(a + "." + k, d)
+        self.L = g("block_count")
+        self.E = g("embedding_length")
+        self.H = g("attention.head_count")
+        self.KV = g("attention.head_count_kv", self.H)
+        self.D = g("attention.key_length", self.E // self.H)
+        self.eps = g("attention.layer_norm_rms_epsilon", 1e-5)
+        self.base = g("rope.freq_base", 10000.0)
+        self.n_expert = g("expert_count", 0)
+        self.n_used = g("expert_used_count", 0)
+        self.neox = a != "llama"
+        self.w = {}
+
+    def t(self, name):
+        if name not in self.w:
+            self.w[name] = self.r.dense(name, oracle.decode_row) if name in self.r.tensors else None
+        return self.w[name]
+
+    def norm(self, x, w):
+        return x / np.sqrt((x * x).mean(-1, keepdims=True) + self.eps) * w
+
+    def rope(self, v, pos):
+        # v: [heads, D]
+        D = self.D
+        i = np.arange(D // 2)
+        ang = pos * self.base ** (-2.0 * i / D)
+        c, s = np.cos(ang), np.sin(ang)
+        out = v.copy()
+        if self.neox:
+            a, b = v[:, :D // 2], v[:, D // 2:]
+            out[:, :D // 2] = a * c - b * s
+            out[:, D // 2:] = a * s + b * c
+        else:
+            a, b = v[:, 0::2], v[:, 1::2]
+            out[:, 0::2] = a * c - b * s
+            out[:, 1::2] = a * s + b * c
+        return out
+
+    def forward(self, tokens, pos0=0, lora=None):
+        """Full causal forward of one sequence; returns logits [T, V].
+        lora: dict name -> (A [r, in], B [out, r], scale*alpha/r)."""
+        T = len(tokens)
+        x = self.t("token_embd.weight")[np.asarray(tokens)]
+        G = self.H // self.KV
+
+        def mm(name, v):
+            y = v @ self.t(name).T
+            if lora and name in lora:
+                A, B, s = lora[name]
+                y = y + s * ((v @ A.T) @ B.T)
+            return y
+
+        for l in range(self.L):
+            b = "blk.%d." % l
+            h = self.norm(x, self.t(b + "attn_norm.weight"))
+            q, k, v = mm(b + "attn_q.weight", h), mm(b + "attn_k.weight", h), mm(b + "attn_v.weight", h)
+            if self.t(b + "attn_q.bias") is not None:
+                q = q + self.t(b + "attn_q.bias"); k = k + self.t(b + "attn_k.bias"); v = v + self.t(b + "attn_v.bias")
+            q = q.reshape(T, self.H, self.D); k = k.reshape(T, self.KV, self.D); v = v.reshape(T, self.KV, self.D)
+            if self.t(b + "attn_q_norm.weight") is not None:
+                q = self.norm(q, self.t(b + "attn_q_norm.weight"))
+                k = self.norm(k, self.t(b + "attn_k_norm.weight"))
+            q = np.stack([self.rope(q[t], pos0 + t) for t in range(T)])
+            k = np.stack([self.rope(k[t], pos0 + t) for t in range(T)])
+            k = k.astype(np.float16).astype(np.float64)   # f16 KV cache
+            v = v.astype(np.float16).astype(np.float64)
+            att = np.zeros((T, self.H, self.D))
+            for hh in range(self.H):
+                s = q[:, hh] @ k[:, hh // G].T / np.sqrt(self.D)
+                s = np.where(np.tril(np.ones((T, T), bool)), s, -np.inf)
+                p = np.exp(s - s.max(-1, keepdims=True))
+                p /= p.sum(-1, keepdims=True)
+                att[:, hh] = p @ v[:, hh // G]
+            x = x + mm(b + "attn_output.weight", att.reshape(T, -1))
+            h = self.norm(x, self.t(b + "ffn_norm.weight"))
+            if self.n_expert:
+                x = x + self.moe(b, h)
+            else:
+                gate, up = mm(b + "ffn_gate.weight", h), mm(b + "ffn_up.weight", h)
+                x = x + mm(b + "ffn_down.weight", gate / (1 + np.exp(-gate)) * up)
+        h = self.norm(x, self.t("output_norm.weight"))
+        head = self.t("output.weight")
+        if head is None:
+            head = self.t("token_embd.weight")
+        logits = h @ head.T
+        if self.t("output.bias") is not None:
+            logits = logits + self.t("output.bias")
+        return logits
+
+    def moe(self, b, h):
+        router = h @ self.t(b + "ffn_gate_inp.weight").T
+        p = np.exp(router - router.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+        Wg, Wu, Wd = self.t(b + "ffn_gate_exps.weight"), self.t(b + "ffn_up_exps.weight"), self.t(b + "ffn_down_exps.weight")
+        out = np.zeros_like(h)
+        for t in range(h.shape[0]):
+            top = np.argsort(-p[t], kind="stable")[:self.n_used]
+            wsum = p[t, top].sum()
+            for e in top:
+                g, u = Wg[e] @ h[t], Wu[e] @ h[t]
+                out[t] += p[t, e] / wsum * (Wd[e] @ (g / (1 + np.exp(-g)) * u))
+        return out

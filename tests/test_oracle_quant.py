@@ -1,0 +1,153 @@
+"""Pins oracle/quant.hpp: the known answers the reference's own decoder tests
+hold (reference crates/rir-core/src/quant.rs:534-581), exhaustive f16 against
+numpy, and a brute-force per-element Q4_K / MXFP4 decoder written from the
+addressing the reference's generated mat-vec spells out
+(generated/rir/mul_mat_vec_q4_K/cpu.rs:52-120: d@0, dmin@2, scales@4..16,
+qs@16..144)."""
+import numpy as np
+import pytest
+
+import oracle
+from retrograd_amd import gguf_writer as gw
+
+
+def test_half_conversion_known_answers():
+    # quant.rs:534-541
+    h = np.array([0x3C00, 0xBC00, 0x0000, 0x0001, 0x0400, 0x7BFF], np.uint16)
+    want = np.array([1.0, -1.0, 0.0, 2.0 ** -24, 2.0 ** -14, 65504.0], np.float32)
+    assert np.array_equal(oracle.half_to_float(h), want)
+
+
+def test_half_to_float_exhaustive_against_numpy():
+    h = np.arange(65536, dtype=np.uint16)
+    got = oracle.half_to_float(h)
+    want = h.view(np.float16).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_float_to_half_against_numpy_rounding():
+    rng = np.random.default_rng(0)
+    x = np.concatenate([
+        rng.standard_normal(200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-8, 5, 200000).astype(np.float32),
+        np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32),            # every half is a fixed point
+        np.array([65504.0, 65519.9, 65520.0, 1e9, -1e9, 2.0 ** -25, 2.0 ** -25 * 1.0001, 2.0 ** -24 * 1.5, 0.0, -0.0], np.float32),
+    ])
+    x = x[np.isfinite(x)]
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(oracle.float_to_half(x), want)
+    # halfway cases between adjacent halves round to even
+    h = np.arange(0x0001, 0x7BFE, 7, dtype=np.uint16)
+    lo = h.view(np.float16).astype(np.float64)
+    hi = (h + 1).astype(np.uint16).view(np.float16).astype(np.float64)
+    mid = (lo + hi) / 2
+    want = np.where(h % 2 == 0, h, h + 1).astype(np.uint16)
+    assert np.array_equal(oracle.double_to_half(mid), want)
+
+
+def test_e8m0_half_scale_known_answers():
+    # quant.rs:545-553
+    assert oracle.e8m0_half(127) == 0.5
+    assert oracle.e8m0_half(128) == 1.0
+    assert oracle.e8m0_half(129) == 2.0
+    assert np.float32(oracle.e8m0_half(1)).view(np.uint32) == 0x00400000
+    assert np.float32(oracle.e8m0_half(0)).view(np.uint32) == 0x00200000
+
+
+def test_q8_0_decodes_scale_times_byte():
+    # quant.rs:557-568
+    blk = bytearray(34)
+    blk[0:2] = (0x3C00).to_bytes(2, "little")
+    for j in range(32):
+        blk[2 + j] = (j - 16) & 0xFF
+    v = oracle.decode_row(gw.GGML_Q8_0, bytes(blk), 32)
+    assert np.array_equal(v, np.arange(-16, 16, dtype=np.float32))
+
+
+def _f16(b, off):
+    return np.frombuffer(bytes(b[off:off + 2]), np.float16)[0].astype(np.float32)
+
+
+def _q4k_brute(block: bytes) -> np.ndarray:
+    """One element at a time: element e lives in 64-element group g = e // 64;
+    within it the first 32 are low nibbles, the last 32 high nibbles of the
+    same 32 bytes; sub-block j = e // 32 picks the 6-bit scale/min."""
+    d, dmin = _f16(block, 0), _f16(block, 2)
+    sc = block[4:16]
+    qs = block[16:144]
+    out = np.zeros(256, np.float32)
+    for e in range(256):
+        j = e // 32
+        if j < 4:
+            s, m = sc[j] & 63, sc[j + 4] & 63
+        else:
+            s = (sc[j + 4] & 0x0F) | ((sc[j - 4] >> 6) << 4)
+            m = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4)
+        byte = qs[(e // 64) * 32 + e % 32]
+        q = (byte >> 4) if (e % 64) >= 32 else (byte & 0x0F)
+        out[e] = np.float32(np.float32(d * np.float32(s)) * np.float32(q)) - np.float32(dmin * np.float32(m))
+    return out
+
+
+def test_q4_k_against_bruteforce_addressing():
+    rng = np.random.default_rng(1)
+    for _ in range(20):
+        blk = bytearray(rng.integers(0, 256, 144, dtype=np.uint8).tobytes())
+        blk[0:2] = (0x2400).to_bytes(2, "little")   # pinned finite scales, as quant.rs:206-212
+        blk[2:4] = (0x2000).to_bytes(2, "little")
+        got = oracle.decode_row(gw.GGML_Q4_K, bytes(blk), 256)
+        assert np.array_equal(got, _q4k_brute(bytes(blk)))
+
+
+def test_q4_k_single_nibble_lands_on_one_element():
+    # A lone nibble set in qs must light exactly one element: catches swapped
+    # halves and wrong group strides.
+    for byte_index in (0, 31, 32, 95, 127):
+        for high in (False, True):
+            blk = bytearray(144)
+            blk[0:2] = (0x3C00).to_bytes(2, "little")      # d = 1
+            for j in range(4):
+                blk[4 + j] = 1                              # scales of sub-blocks 0..3 = 1
+                blk[12 + j] = 1                             # low nibble: scales of sub-blocks 4..7 = 1
+            blk[16 + byte_index] = 0x50 if high else 0x05
+            v = oracle.decode_row(gw.GGML_Q4_K, bytes(blk), 256)
+            e = (byte_index // 32) * 64 + (32 if high else 0) + byte_index % 32
+            want = np.zeros(256, np.float32)
+            want[e] = 5.0
+            assert np.array_equal(v, want), (byte_index, high)
+
+
+def test_mxfp4_nibble_halves_and_table():
+    table = [0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12]   # doubled E2M1, quant.rs:61
+    blk = bytearray(17)
+    blk[0] = 128                                    # half-scale 1.0
+    for j in range(16):
+        blk[1 + j] = j | ((15 - j) << 4)
+    v = oracle.decode_row(gw.GGML_MXFP4, bytes(blk), 32)
+    want = np.array([table[j] for j in range(16)] + [table[15 - j] for j in range(16)], np.float32)
+    assert np.array_equal(v, want)
+    blk[0] = 127
+    assert np.array_equal(oracle.decode_row(gw.GGML_MXFP4, bytes(blk), 32), want * 0.5)
+
+
+def test_partial_block_is_refused():
+    with pytest.raises(oracle.OracleError):
+        oracle.row_bytes(gw.GGML_Q4_K, 128)
+    assert oracle.row_bytes(gw.GGML_Q4_K, 4096) == 16 * 144
+    assert oracle.row_bytes(gw.GGML_Q8_0, 4096) == 128 * 34
+    assert oracle.row_bytes(gw.GGML_MXFP4, 64) == 34
+
+
+def test_synthetic_quantisers_round_trip_close():
+    # Not a parity statement: only that the synthetic-model quantisers write
+    # blocks that decode near their input (valid scales, right packing).
+    import torch
+    from retrograd_amd import synth
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(4, 512, generator=g) * 0.02
+    for t, tol in ((gw.GGML_Q8_0, 0.01), (gw.GGML_Q4_K, 0.12), (gw.GGML_MXFP4, 0.3)):
+        raw = synth.encode(x, t)
+        for r in range(4):
+            y = oracle.decode_row(t, raw[r], 512)
+            err = np.abs(y - x[r].numpy()).max() / np.abs(x[r].numpy()).max()
+            assert err < tol, (t, err)

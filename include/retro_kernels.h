@@ -1,0 +1,54 @@
+/*
+ * retro_kernels.h - kernel-level and state-inspection entry points of
+ * libretro_hip.so. None of these has a counterpart in the reference's C ABI
+ * (crates/retrograd-ffi/runtime/include/retro_lora_train.h): they exist so the
+ * parity tests and micro-benchmarks can drive single gfx950 kernels, and read
+ * back device state, through plain C calls. Same error convention as
+ * retro_step.h (0 / -1 / -2, message in retro_last_error()).
+ */
+#ifndef RETRO_KERNELS_H
+#define RETRO_KERNELS_H
+
+#include "retro_step.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* y[t][n] (=|+=) sum_k W[n][k] * f16(x[t][k]) (+ bias[n]) with W given as
+ * n_rows raw GGUF rows of `type`. use_tiles selects the MFMA tile kernel
+ * (K % 256 == 0, n_rows % 16 == 0, Q4_K or Q8_0) instead of the generic one.
+ * y is [n_tokens][n_rows] and is read first when accumulate is set. */
+int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x,
+                        int32_t n_tokens, int32_t use_tiles, const float * bias, int32_t accumulate, float * y);
+
+/* Per logits row: argmax (lowest id on ties), max, sum exp(double(l) - max),
+ * and the k[r] best (id, logit) pairs in (logit desc, id asc) order, written
+ * to out_top_*[r * retro_kernel_max_topk() + j]. */
+int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_vocab, const int32_t * k,
+                                int32_t * out_argmax, float * out_max, double * out_sum_exp,
+                                int32_t * out_top_ids, float * out_top_logits);
+
+int32_t retro_kernel_page_size(void);   /* positions per KV page */
+int32_t retro_kernel_max_topk(void);    /* candidates sample_prepare can return */
+
+/* Logits of the last step's sampling rows, [rows][n_vocab], in row order.
+ * out == NULL only reports the row count. */
+int retro_engine_debug_logits(retro_engine * engine, float * out, size_t n_floats, size_t * out_rows);
+/* The stored f16 K (want_v = 0) or V row of (layer, slot, pos) in natural
+ * element order: n_head_kv * head_dim halves. */
+int retro_engine_debug_kv(retro_engine * engine, int32_t layer, int32_t slot, int32_t pos, int32_t want_v,
+                          uint16_t * out);
+/* The device-side packing of the last step: per-token arrays and
+ * counts[4] = tokens, outputs, attention tiles, attention work items. */
+int retro_engine_debug_pack(retro_engine * engine, int32_t * tok, int32_t * pos, int32_t * seq, int32_t * cell,
+                            int32_t * out_index, int32_t * last_index, size_t cap_tokens, size_t cap_rows,
+                            int32_t * counts);
+/* Page id per page index of a slot (-1 = none); out == NULL reports the length. */
+int retro_engine_debug_pages(retro_engine * engine, int32_t slot, int32_t * out, size_t cap, size_t * out_n);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* RETRO_KERNELS_H */

@@ -1,0 +1,525 @@
+// extern "C" surface of libretro_hip.so: the entry points include/retro_step.h
+// declares, each a thin boundary over retro::Engine. Every body runs inside
+// boundary(), which clears the thread's error string and turns any C++
+// exception into -1 (reference retro_runtime.hpp:1255-1267).
+#include "engine.hpp"
+
+#include <cmath>
+#include <cstring>
+
+using namespace retro;
+
+struct retro_grammar { std::string gbnf; };
+
+namespace {
+
+template <typename Fn> int boundary(Fn && fn) {
+    try {
+        clear_error();
+        return fn();
+    } catch (const std::exception & e) {
+        set_error(e.what());
+        return -1;
+    } catch (...) {
+        set_error("unknown C++ exception");
+        return -1;
+    }
+}
+
+Engine * checked(retro_engine * e) {
+    if (!e) {
+        set_error("engine is required");
+        return nullptr;
+    }
+    return &e->impl;
+}
+
+bool blank(const char * s) { return s == nullptr || s[0] == '\0'; }
+
+// Defaults and validation of the reference (retro_engine.cpp:93-153), plus the
+// refusals of what this library does not contain.
+retro_engine_config default_config() {
+    retro_engine_config c {};
+    c.struct_size = sizeof(retro_engine_config);
+    c.n_ctx = 4096;
+    c.n_seq_max = 8;
+    c.n_batch = 512;
+    c.n_ubatch = 512;
+    c.kv_dtype = RETRO_ENGINE_KV_DTYPE_F16;
+    c.flash_attn = true;
+    c.device = RETRO_DEVICE_AUTO;
+    c.threads = 0;
+    c.verbose = false;
+    c.kv_unified = 1;
+    c.expert_placement = RETRO_EXPERT_PLACEMENT_DEVICE;
+    c.expert_host_layers = 0;
+    c.expert_device_cache_bytes = 0;
+    return c;
+}
+
+bool validate_config(const retro_engine_config & c, bool * invalid_placement) {
+    if (c.n_ctx == 0 || c.n_seq_max == 0) {
+        set_error("engine n_ctx and n_seq_max must be greater than zero");
+        return false;
+    }
+    if (c.n_batch == 0 || c.n_ubatch == 0 || c.n_ubatch > c.n_batch) {
+        set_error("engine n_ubatch must be in (0, n_batch]");
+        return false;
+    }
+    if (c.n_ctx > INT32_MAX || c.n_batch > INT32_MAX || c.n_ubatch > INT32_MAX || c.threads > INT32_MAX) {
+        set_error("engine context, batch and thread counts must fit in int32_t");
+        return false;
+    }
+    if (c.n_seq_max > RETRO_MAX_SEQ || c.n_seq_max > std::min(c.n_batch, c.n_ctx)) {
+        set_error("engine n_seq_max must not exceed LLAMA_MAX_SEQ, n_batch or n_ctx");
+        return false;
+    }
+    if (c.kv_dtype < RETRO_ENGINE_KV_DTYPE_F32 || c.kv_dtype > RETRO_ENGINE_KV_DTYPE_Q4_0) {
+        set_error("engine kv_dtype must be one of retro_engine_kv_dtype");
+        return false;
+    }
+    if ((c.kv_dtype == RETRO_ENGINE_KV_DTYPE_Q8_0 || c.kv_dtype == RETRO_ENGINE_KV_DTYPE_Q4_0) && !c.flash_attn) {
+        set_error("a quantized engine kv_dtype requires flash_attn");
+        return false;
+    }
+    if (c.device < RETRO_DEVICE_AUTO || c.device > RETRO_DEVICE_GPU) {
+        set_error("engine device must be one of retro_device");
+        return false;
+    }
+    if (c.expert_placement != RETRO_EXPERT_PLACEMENT_DEVICE && c.expert_placement != RETRO_EXPERT_PLACEMENT_HOST) {
+        set_error("engine expert_placement must be one of retro_expert_placement");
+        return false;
+    }
+    if (c.device == RETRO_DEVICE_CPU) {
+        set_error("device=cpu requested, but this library only executes on an MI355X GPU");
+        return false;
+    }
+    if (c.kv_dtype != RETRO_ENGINE_KV_DTYPE_F16) {
+        set_error("only the f16 KV cache is implemented by this library");
+        return false;
+    }
+    if (c.expert_placement == RETRO_EXPERT_PLACEMENT_HOST || c.expert_device_cache_bytes != 0) {
+        if (invalid_placement) *invalid_placement = true;
+        set_error("host expert placement is not supported: every tensor lives in device memory");
+        return false;
+    }
+    return true;
+}
+
+// Two-call string contract of the reference (retro_runtime.hpp:551-576).
+int string_out(const std::string & s, char * buffer, size_t n_buffer, size_t * out_n_bytes) {
+    *out_n_bytes = s.size();
+    if (!buffer || n_buffer == 0) return 0;
+    if (s.size() > n_buffer - 1) {
+        set_error("output buffer is too small");
+        return -2;
+    }
+    std::memcpy(buffer, s.data(), s.size());
+    buffer[s.size()] = '\0';
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char * retro_last_error(void) {
+    return last_error().empty() ? "no runtime error" : last_error().c_str();
+}
+
+retro_engine * retro_engine_new(const char * model_path, const retro_engine_config * config) {
+    return retro_engine_new_checked(model_path, config, nullptr);
+}
+
+retro_engine * retro_engine_new_checked(const char * model_path, const retro_engine_config * config,
+                                        bool * out_invalid_placement) {
+    if (out_invalid_placement) *out_invalid_placement = false;
+    try {
+        clear_error();
+        if (blank(model_path)) {
+            set_error("model_path is required");
+            return nullptr;
+        }
+        retro_engine_config resolved = default_config();
+        if (config) {
+            // Read the evolution key before any other field; copy only the
+            // prefix the caller owns (retro_engine.cpp:474-494).
+            uint32_t size = 0;
+            std::memcpy(&size, config, sizeof(size));
+            constexpr size_t required = offsetof(retro_engine_config, verbose) + sizeof(bool);
+            if (size < required) {
+                set_error("retro_engine_config.struct_size is too small for this build");
+                return nullptr;
+            }
+            std::memcpy(&resolved, config, std::min<size_t>(size, sizeof(resolved)));
+        }
+        if (!validate_config(resolved, out_invalid_placement)) return nullptr;
+        return new retro_engine(model_path, resolved);
+    } catch (const std::exception & e) {
+        set_error(e.what());
+        return nullptr;
+    } catch (...) {
+        set_error("unknown C++ exception");
+        return nullptr;
+    }
+}
+
+void retro_engine_free(retro_engine * engine) { delete engine; }
+
+int retro_engine_step(retro_engine * engine, const retro_step_row * rows, size_t n_rows,
+                      retro_step_out_row * out_rows, int32_t * out_top_ids, float * out_top_logprobs,
+                      size_t n_top_stride) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        if (!rows || n_rows == 0 || !out_rows) {
+            set_error("step rows and output rows are required");
+            return -3;
+        }
+        return e->step(nullptr, rows, n_rows, nullptr, out_rows, out_top_ids, out_top_logprobs, n_top_stride);
+    });
+}
+
+int retro_engine_step_v2(retro_engine * engine, const retro_step_row_v2 * rows, size_t n_rows,
+                         retro_step_out_row_v2 * out_rows, int32_t * out_top_ids, float * out_top_logprobs,
+                         size_t n_top_stride) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        if (!rows || n_rows == 0 || !out_rows) {
+            set_error("step rows and output rows are required");
+            return -3;
+        }
+        return e->step(rows, nullptr, n_rows, out_rows, nullptr, out_top_ids, out_top_logprobs, n_top_stride);
+    });
+}
+
+int retro_engine_seq_rm(retro_engine * engine, int32_t slot, int32_t p0, int32_t p1) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->seq_rm(slot, p0, p1) ? 0 : -1;
+    });
+}
+
+int retro_engine_seq_cp(retro_engine * engine, int32_t src, int32_t dst, int32_t p0, int32_t p1) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->seq_cp(src, dst, p0, p1) ? 0 : -1;
+    });
+}
+
+int retro_engine_seq_save(retro_engine * engine, int32_t slot, uint32_t flags, uint8_t * buffer, size_t n_buffer,
+                          size_t * out_n_bytes) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->seq_save(slot, flags, buffer, n_buffer, out_n_bytes);
+    });
+}
+
+int retro_engine_seq_load(retro_engine * engine, int32_t slot, uint32_t flags, const uint8_t * buffer,
+                          size_t n_bytes, size_t * out_n_read) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->seq_load(slot, flags, buffer, n_bytes, out_n_read);
+    });
+}
+
+int retro_engine_seq_pos(retro_engine * engine, int32_t slot, int32_t * out_pos_min, int32_t * out_pos_max) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->seq_pos(slot, out_pos_min, out_pos_max);
+    });
+}
+
+int retro_engine_memory(retro_engine * engine, retro_engine_memory_info * out) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->memory(out);
+    });
+}
+
+int retro_engine_request_free(retro_engine * engine, int32_t request) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        e->request_free(request);
+        return 0;
+    });
+}
+
+int retro_engine_kv_unified(retro_engine * engine, bool * out_unified) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e || !out_unified) {
+            if (e) set_error("out_unified is required");
+            return -1;
+        }
+        *out_unified = e->config().kv_unified != 0;
+        return 0;
+    });
+}
+
+int retro_engine_weights_version(retro_engine * engine, uint64_t * out_version) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e || !out_version) {
+            if (e) set_error("out_version is required");
+            return -1;
+        }
+        *out_version = e->weights_version();
+        return 0;
+    });
+}
+
+int retro_engine_model_fingerprint(retro_engine * engine, uint64_t * out_fingerprint) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e || !out_fingerprint) {
+            if (e) set_error("out_fingerprint is required");
+            return -1;
+        }
+        *out_fingerprint = e->fingerprint();
+        return 0;
+    });
+}
+
+int retro_engine_is_hybrid(retro_engine * engine, bool * out_is_hybrid) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e || !out_is_hybrid) {
+            if (e) set_error("out_is_hybrid is required");
+            return -1;
+        }
+        *out_is_hybrid = false;   // attention-only architectures
+        return 0;
+    });
+}
+
+int retro_engine_eos_token(retro_engine * engine, int32_t * out_token) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e || !out_token) {
+            if (e) set_error("out_token is required");
+            return -1;
+        }
+        *out_token = e->vocab().eos;
+        return 0;
+    });
+}
+
+int retro_engine_vocab_size(retro_engine * engine, uint32_t * out_n_vocab) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e || !out_n_vocab) {
+            if (e) set_error("out_n_vocab is required");
+            return -1;
+        }
+        *out_n_vocab = (uint32_t)e->hparams().n_vocab;
+        return 0;
+    });
+}
+
+int retro_engine_is_eog_token(retro_engine * engine, int32_t token, bool * out_is_eog) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e || !out_is_eog) {
+            if (e) set_error("out_is_eog is required");
+            return -1;
+        }
+        if (token < 0 || token >= e->hparams().n_vocab) {
+            set_error("token is outside the vocabulary");
+            return -1;
+        }
+        const Vocab & v = e->vocab();
+        *out_is_eog = (v.eos >= 0 && token == v.eos) || (v.eot >= 0 && token == v.eot);
+        return 0;
+    });
+}
+
+int retro_engine_context_size(retro_engine * engine, uint32_t * out_n_ctx) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e || !out_n_ctx) {
+            if (e) set_error("out_n_ctx is required");
+            return -1;
+        }
+        *out_n_ctx = e->context_size();
+        return 0;
+    });
+}
+
+// Concatenates the raw pieces: SentencePiece's U+2581 becomes a space, byte
+// tokens "<0xXX>" their byte, control tokens are skipped unless unparse_special.
+int retro_engine_detokenize(retro_engine * engine, const int32_t * tokens, size_t n_tokens, bool unparse_special,
+                            char * buffer, size_t n_buffer, size_t * out_n_bytes) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        if (!out_n_bytes) {
+            set_error("out_n_bytes is required");
+            return -1;
+        }
+        if (n_tokens > 0 && !tokens) {
+            set_error("tokens are required");
+            return -1;
+        }
+        if (n_tokens > (size_t)INT32_MAX) {
+            set_error("too many tokens to detokenize");
+            return -1;
+        }
+        const Vocab & v = e->vocab();
+        const int32_t n_vocab = e->hparams().n_vocab;
+        std::string text;
+        for (size_t i = 0; i < n_tokens; ++i) {
+            const int32_t t = tokens[i];
+            if (t < 0 || t >= n_vocab) {
+                set_error("token " + std::to_string(t) + " at index " + std::to_string(i)
+                          + " is outside the vocabulary of size " + std::to_string(n_vocab));
+                return -1;
+            }
+            if ((size_t)t >= v.pieces.size()) continue;
+            const int32_t type = (size_t)t < v.types.size() ? v.types[(size_t)t] : 1;
+            const std::string & piece = v.pieces[(size_t)t];
+            if (type == 3 || type == 2) {            // control / unknown
+                if (unparse_special) text += piece;
+                continue;
+            }
+            if (type == 6 && piece.size() == 6 && piece.compare(0, 3, "<0x") == 0) {
+                text.push_back((char)std::stoi(piece.substr(3, 2), nullptr, 16));
+                continue;
+            }
+            for (size_t j = 0; j < piece.size();) {
+                if (j + 2 < piece.size() && (unsigned char)piece[j] == 0xE2 && (unsigned char)piece[j + 1] == 0x96
+                        && (unsigned char)piece[j + 2] == 0x81) {
+                    text.push_back(' ');
+                    j += 3;
+                } else {
+                    text.push_back(piece[j++]);
+                }
+            }
+        }
+        return string_out(text, buffer, n_buffer, out_n_bytes);
+    });
+}
+
+int retro_engine_graphs_reused(retro_engine * engine, uint64_t * out_n_reused) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        if (!out_n_reused) {
+            set_error("out_n_reused is required");
+            return -1;
+        }
+        *out_n_reused = 0;   // every step launches its kernels directly; nothing is cached between steps
+        return 0;
+    });
+}
+
+// ---- adapters ---------------------------------------------------------------------------
+
+int retro_engine_load_lora_named(retro_engine * engine, const char * name, const char * adapter_path) {
+    return boundary([&]() -> int {
+        if (!checked(engine)) return -1;
+        (void)name;
+        (void)adapter_path;
+        set_error("named LoRA adapters are not supported by this library yet");
+        return -1;
+    });
+}
+
+int retro_engine_activate_lora(retro_engine * engine, const char * name) {
+    return boundary([&]() -> int {
+        if (!checked(engine)) return -1;
+        if (blank(name)) return 0;   // the base model is what is active
+        set_error("named LoRA adapters are not supported by this library yet");
+        return -1;
+    });
+}
+
+int retro_engine_active_adapter(retro_engine * engine, char * buffer, size_t n_buffer, size_t * out_n_bytes) {
+    return boundary([&]() -> int {
+        if (!checked(engine)) return -1;
+        if (!out_n_bytes) {
+            set_error("out_n_bytes is required");
+            return -1;
+        }
+        return string_out(std::string(), buffer, n_buffer, out_n_bytes);
+    });
+}
+
+int retro_engine_adapter_load(retro_engine * engine, const char * adapter_path, float scale, int32_t * out_id) {
+    return boundary([&]() -> int {
+        if (!checked(engine)) return -1;
+        if (blank(adapter_path)) {
+            set_error("adapter_path is required");
+            return -1;
+        }
+        if (!out_id) {
+            set_error("out_id is required");
+            return -1;
+        }
+        if (!std::isfinite(scale)) {
+            set_error("the adapter scale must be finite");
+            return -1;
+        }
+        set_error("per-row LoRA adapters are not supported by this library yet");
+        return -1;
+    });
+}
+
+int retro_engine_adapter_unload(retro_engine * engine, int32_t id) {
+    return boundary([&]() -> int {
+        if (!checked(engine)) return -1;
+        set_error("no per-row adapter is loaded under id " + std::to_string(id));
+        return -1;
+    });
+}
+
+int retro_engine_adapter_rows_info(retro_engine * engine, retro_adapter_rows_info * out_info) {
+    return boundary([&]() -> int {
+        if (!checked(engine)) return -1;
+        if (!out_info) {
+            set_error("out_info is required");
+            return -1;
+        }
+        *out_info = retro_adapter_rows_info{};
+        out_info->struct_size = sizeof(retro_adapter_rows_info);
+        return 0;
+    });
+}
+
+// ---- grammar handles -------------------------------------------------------------------
+
+retro_grammar * retro_grammar_from_json_schema(const char * json_schema) {
+    clear_error();
+    (void)json_schema;
+    set_error("JSON-schema grammars need llama.cpp's schema converter, which this library does not contain");
+    return nullptr;
+}
+
+retro_grammar * retro_grammar_from_gbnf(const char * gbnf) {
+    clear_error();
+    if (blank(gbnf)) {
+        set_error("gbnf is required");
+        return nullptr;
+    }
+    return new retro_grammar{gbnf};
+}
+
+retro_grammar * retro_grammar_json_object(void) {
+    clear_error();
+    set_error("the built-in JSON grammar is llama.cpp's grammars/json.gbnf, which this library does not contain");
+    return nullptr;
+}
+
+const char * retro_grammar_gbnf(const retro_grammar * grammar) { return grammar ? grammar->gbnf.c_str() : nullptr; }
+
+void retro_grammar_free(retro_grammar * grammar) { delete grammar; }
+
+}  // extern "C"

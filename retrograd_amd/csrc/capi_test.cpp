@@ -1,0 +1,132 @@
+// Kernel-level and state-inspection entry points declared in
+// include/retro_kernels.h. They have no counterpart in the reference ABI: they
+// exist so parity tests can compare single kernels and device state with the
+// CPU oracle through plain C calls.
+#include "../../include/retro_kernels.h"
+#include "engine.hpp"
+
+#include <cstring>
+
+using namespace retro;
+
+
+namespace {
+template <typename Fn> int guarded(Fn && fn) {
+    try {
+        clear_error();
+        return fn();
+    } catch (const std::exception & e) {
+        set_error(e.what());
+        return -1;
+    } catch (...) {
+        set_error("unknown C++ exception");
+        return -1;
+    }
+}
+void ok(hipError_t e, const char * what) {
+    if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+}  // namespace
+
+extern "C" {
+
+int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x,
+                        int32_t n_tokens, int32_t use_tiles, const float * bias, int32_t accumulate, float * y) {
+    return guarded([&]() -> int {
+        const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
+        DevBuf d_raw, d_packed, d_x, d_xh, d_hi, d_lo, d_y, d_bias;
+        d_raw.alloc(bytes);
+        ok(hipMemcpy(d_raw.ptr, raw, bytes, hipMemcpyHostToDevice), "upload weights");
+        rk::Weight w;
+        w.type = type; w.K = (int)k; w.N = (int)n_rows; w.bytes = bytes;
+        if (use_tiles) {
+            if (!rk::can_pack(type, k, n_rows)) throw std::runtime_error("this shape or type has no tile layout");
+            d_packed.alloc(bytes);
+            rk::repack(nullptr, type, d_raw.as<uint8_t>(), d_packed.as<uint8_t>(), (int)k, (int)n_rows);
+            w.packed = d_packed.as<uint8_t>();
+        } else {
+            w.raw = d_raw.as<uint8_t>();
+        }
+        d_x.alloc((size_t)n_tokens * k * 4);
+        ok(hipMemcpy(d_x.ptr, x, d_x.bytes, hipMemcpyHostToDevice), "upload activations");
+        d_xh.alloc((size_t)n_tokens * k * 2);
+        d_hi.alloc((size_t)n_tokens * (k / 32 + 1) * 2);
+        d_lo.alloc((size_t)n_tokens * (k / 32 + 1) * 2);
+        rk::Act act{d_xh.as<__half>(), k % 32 == 0 ? d_hi.as<__half>() : nullptr, k % 32 == 0 ? d_lo.as<__half>() : nullptr, (int)k};
+        rk::to_act(nullptr, d_x.as<float>(), n_tokens, (int)k, act);
+        d_y.alloc((size_t)n_tokens * n_rows * 4);
+        ok(hipMemcpy(d_y.ptr, y, d_y.bytes, hipMemcpyHostToDevice), "upload outputs");
+        if (bias) {
+            d_bias.alloc((size_t)n_rows * 4);
+            ok(hipMemcpy(d_bias.ptr, bias, d_bias.bytes, hipMemcpyHostToDevice), "upload bias");
+        }
+        rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, accumulate ? rk::MM_ADD : rk::MM_STORE,
+                   d_bias.as<float>());
+        ok(hipDeviceSynchronize(), "matmul");
+        ok(hipMemcpy(y, d_y.ptr, d_y.bytes, hipMemcpyDeviceToHost), "download outputs");
+        return 0;
+    });
+}
+
+int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_vocab, const int32_t * k,
+                                int32_t * out_argmax, float * out_max, double * out_sum_exp,
+                                int32_t * out_top_ids, float * out_top_logits) {
+    return guarded([&]() -> int {
+        DevBuf d_l, d_k, d_o;
+        d_l.alloc((size_t)n_rows * n_vocab * 4);
+        d_k.alloc((size_t)n_rows * 4);
+        d_o.alloc((size_t)n_rows * sizeof(rk::SampleOut));
+        ok(hipMemcpy(d_l.ptr, logits, d_l.bytes, hipMemcpyHostToDevice), "upload logits");
+        ok(hipMemcpy(d_k.ptr, k, d_k.bytes, hipMemcpyHostToDevice), "upload k");
+        rk::sample_prepare(nullptr, d_l.as<float>(), n_rows, n_vocab, d_k.as<int32_t>(), d_o.as<rk::SampleOut>());
+        ok(hipDeviceSynchronize(), "sample_prepare");
+        std::vector<rk::SampleOut> h((size_t)n_rows);
+        ok(hipMemcpy(h.data(), d_o.ptr, d_o.bytes, hipMemcpyDeviceToHost), "download");
+        for (int r = 0; r < n_rows; ++r) {
+            out_argmax[r] = h[(size_t)r].argmax;
+            out_max[r] = h[(size_t)r].max;
+            out_sum_exp[r] = h[(size_t)r].sum_exp;
+            for (int j = 0; j < rk::MAX_TOPK; ++j) {
+                out_top_ids[r * rk::MAX_TOPK + j] = j < k[r] ? h[(size_t)r].top_id[j] : -1;
+                out_top_logits[r * rk::MAX_TOPK + j] = j < k[r] ? h[(size_t)r].top_logit[j] : 0.0f;
+            }
+        }
+        return 0;
+    });
+}
+
+int32_t retro_kernel_page_size(void) { return rk::PAGE; }
+int32_t retro_kernel_max_topk(void) { return rk::MAX_TOPK; }
+
+int retro_engine_debug_logits(retro_engine * engine, float * out, size_t n_floats, size_t * out_rows) {
+    return guarded([&]() -> int {
+        if (!engine) { set_error("engine is required"); return -1; }
+        return engine->impl.debug_last_logits(out, n_floats, out_rows);
+    });
+}
+
+int retro_engine_debug_kv(retro_engine * engine, int32_t layer, int32_t slot, int32_t pos, int32_t want_v,
+                          uint16_t * out) {
+    return guarded([&]() -> int {
+        if (!engine) { set_error("engine is required"); return -1; }
+        return engine->impl.debug_read_kv(layer, slot, pos, want_v, out);
+    });
+}
+
+int retro_engine_debug_pack(retro_engine * engine, int32_t * tok, int32_t * pos, int32_t * seq, int32_t * cell,
+                            int32_t * out_index, int32_t * last_index, size_t cap_tokens, size_t cap_rows,
+                            int32_t * counts) {
+    return guarded([&]() -> int {
+        if (!engine) { set_error("engine is required"); return -1; }
+        return engine->impl.debug_pack(tok, pos, seq, cell, out_index, last_index, cap_tokens, cap_rows, counts);
+    });
+}
+
+int retro_engine_debug_pages(retro_engine * engine, int32_t slot, int32_t * out, size_t cap, size_t * out_n) {
+    return guarded([&]() -> int {
+        if (!engine) { set_error("engine is required"); return -1; }
+        return engine->impl.debug_page_table(slot, out, cap, out_n);
+    });
+}
+
+}  // extern "C"

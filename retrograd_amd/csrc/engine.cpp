@@ -1,0 +1,1155 @@
+#include "engine.hpp"
+
+#include <algorithm>
+#include <climits>
+#include <cmath>
+#include <cstring>
+#include <sstream>
+
+namespace retro {
+
+namespace {
+thread_local std::string g_last_error;
+
+void hip_check(hipError_t err, const char * what) {
+    if (err != hipSuccess) {
+        throw std::runtime_error(std::string("HIP error in ") + what + ": " + hipGetErrorString(err));
+    }
+}
+}  // namespace
+
+void set_error(std::string message) { g_last_error = std::move(message); }
+void clear_error() { g_last_error.clear(); }
+const std::string & last_error() { return g_last_error; }
+
+// ---- buffers --------------------------------------------------------------------
+
+DevBuf::~DevBuf() { release(); }
+DevBuf & DevBuf::operator=(DevBuf && o) noexcept {
+    if (this != &o) {
+        release();
+        ptr = o.ptr;
+        bytes = o.bytes;
+        o.ptr = nullptr;
+        o.bytes = 0;
+    }
+    return *this;
+}
+void DevBuf::release() {
+    if (ptr) (void)hipFree(ptr);
+    ptr = nullptr;
+    bytes = 0;
+}
+void DevBuf::alloc(size_t n) {
+    release();
+    if (n == 0) return;
+    hip_check(hipMalloc(&ptr, n), "hipMalloc");
+    bytes = n;
+}
+void DevBuf::ensure(size_t n) {
+    if (n > bytes) alloc(n + n / 4);
+}
+
+HostPinned::~HostPinned() {
+    if (ptr) (void)hipHostFree(ptr);
+}
+void HostPinned::ensure(size_t n) {
+    if (n <= bytes) return;
+    if (ptr) (void)hipHostFree(ptr);
+    ptr = nullptr;
+    bytes = 0;
+    hip_check(hipHostMalloc(&ptr, n + n / 4, hipHostMallocDefault), "hipHostMalloc");
+    bytes = n + n / 4;
+}
+
+// ---- construction -----------------------------------------------------------------
+
+Engine::Engine(const std::string & path, const retro_engine_config & config) : cfg_(config) {
+    int n_dev = 0;
+    if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev == 0) {
+        throw std::runtime_error("no HIP device is available: this library has no CPU path");
+    }
+    hip_check(hipSetDevice(0), "hipSetDevice");
+    hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
+    load_model(path);
+
+    // Per-sequence context: the whole pool when unified, an equal share otherwise.
+    n_ctx_seq_ = cfg_.kv_unified ? (int)cfg_.n_ctx : (int)(cfg_.n_ctx / cfg_.n_seq_max);
+    if (n_ctx_seq_ <= 0) throw std::runtime_error("engine n_ctx is too small for n_seq_max sequences");
+    max_pages_ = (n_ctx_seq_ + rk::PAGE - 1) / rk::PAGE;
+    // A partially filled last page per slot is the only space paging can waste.
+    n_pages_ = (int)((cfg_.n_ctx + rk::PAGE - 1) / rk::PAGE + cfg_.n_seq_max);
+    const int G = hp_.n_head / hp_.n_head_kv;
+    if (hp_.n_head % hp_.n_head_kv != 0 || G > 16) throw std::runtime_error("unsupported attention head grouping");
+    qt_ = std::max(1, 16 / G);
+
+    const size_t pool_halves = (size_t)n_pages_ * hp_.n_head_kv * rk::PAGE * hp_.head_dim;
+    k_pool_.resize((size_t)hp_.n_layer);
+    v_pool_.resize((size_t)hp_.n_layer);
+    for (int l = 0; l < hp_.n_layer; ++l) {
+        k_pool_[(size_t)l].alloc(pool_halves * 2);
+        v_pool_[(size_t)l].alloc(pool_halves * 2);
+        // Pages must never hold non-finite bit patterns: a masked score times a
+        // NaN value would poison the output.
+        hip_check(hipMemsetAsync(k_pool_[(size_t)l].ptr, 0, pool_halves * 2, stream_), "hipMemsetAsync");
+        hip_check(hipMemsetAsync(v_pool_[(size_t)l].ptr, 0, pool_halves * 2, stream_), "hipMemsetAsync");
+    }
+    table_.alloc((size_t)cfg_.n_seq_max * max_pages_ * sizeof(int32_t));
+    hip_check(hipMemsetAsync(table_.ptr, 0xff, table_.bytes, stream_), "hipMemsetAsync");
+    slots_.resize(cfg_.n_seq_max);
+    for (auto & s : slots_) s.pages.assign((size_t)max_pages_, -1);
+    page_ref_.assign((size_t)n_pages_, 0);
+    for (int p = 0; p < n_pages_; ++p) free_pages_.push(p);
+
+    build_buffers();
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+}
+
+Engine::~Engine() {
+    if (stream_) {
+        (void)hipStreamSynchronize(stream_);
+        (void)hipStreamDestroy(stream_);
+    }
+}
+
+void Engine::upload_f32(const TensorInfo * t, DevBuf & out, size_t expect) {
+    if (!t) return;
+    if (t->type != rk::WT_F32) throw std::runtime_error("tensor " + t->name + " must be F32");
+    if (t->nbytes != expect * 4) throw std::runtime_error("tensor " + t->name + " has an unexpected size");
+    out.alloc(t->nbytes);
+    hip_check(hipMemcpy(out.ptr, t->data, t->nbytes, hipMemcpyHostToDevice), "hipMemcpy");
+}
+
+void Engine::upload_weight(const TensorInfo & t, int64_t K, int64_t N, const uint8_t * data, size_t bytes,
+                           bool keep_raw, DevWeight & out) {
+    rk::geom_of(t.type);   // refuses unsupported storage
+    if (rk::row_bytes(t.type, K) * (size_t)N != bytes) throw std::runtime_error("tensor " + t.name + " has an unexpected size");
+    out.w.type = t.type;
+    out.w.K = (int)K;
+    out.w.N = (int)N;
+    out.w.bytes = bytes;
+    DevBuf raw;
+    raw.alloc(bytes);
+    hip_check(hipMemcpy(raw.ptr, data, bytes, hipMemcpyHostToDevice), "hipMemcpy");
+    if (!keep_raw && rk::can_pack(t.type, K, N)) {
+        out.buf.alloc(bytes);
+        rk::repack(stream_, t.type, raw.as<uint8_t>(), out.buf.as<uint8_t>(), (int)K, (int)N);
+        hip_check(hipStreamSynchronize(stream_), "repack");
+        out.w.packed = out.buf.as<uint8_t>();
+        out.w.raw = nullptr;
+    } else {
+        out.buf = std::move(raw);
+        out.w.raw = out.buf.as<uint8_t>();
+        out.w.packed = nullptr;
+    }
+}
+
+// Row-wise concatenation of matrices that share K and storage type: one matmul
+// instead of several. Falls back to separate matrices when they differ.
+void Engine::upload_fused(const std::vector<const TensorInfo *> & parts, std::vector<DevWeight> & out) {
+    bool same = true;
+    for (const TensorInfo * p : parts) same = same && p->type == parts[0]->type && p->ne[0] == parts[0]->ne[0];
+    out.clear();
+    if (same) {
+        std::vector<uint8_t> joined;
+        int64_t N = 0;
+        for (const TensorInfo * p : parts) {
+            joined.insert(joined.end(), p->data, p->data + p->nbytes);
+            N += p->ne[1];
+        }
+        out.emplace_back();
+        upload_weight(*parts[0], parts[0]->ne[0], N, joined.data(), joined.size(), false, out.back());
+    } else {
+        for (const TensorInfo * p : parts) {
+            out.emplace_back();
+            upload_weight(*p, p->ne[0], p->ne[1], p->data, p->nbytes, false, out.back());
+        }
+    }
+}
+
+void Engine::load_model(const std::string & path) {
+    GgufFile g(path);
+    HParams & h = hp_;
+    h.arch = g.get_string("general.architecture");
+    if (h.arch == "llama") h.rope_neox = false;
+    else if (h.arch == "qwen2" || h.arch == "qwen3") h.rope_neox = true;
+    else throw std::runtime_error("unsupported model architecture: " + h.arch);
+    const std::string a = h.arch + ".";
+    h.n_layer = (int)g.need_int(a + "block_count");
+    h.n_embd = (int)g.need_int(a + "embedding_length");
+    h.n_head = (int)g.need_int(a + "attention.head_count");
+    h.n_head_kv = (int)g.get_int(a + "attention.head_count_kv", h.n_head);
+    h.head_dim = (int)g.get_int(a + "attention.key_length", h.n_embd / h.n_head);
+    h.n_ff = (int)g.get_int(a + "feed_forward_length", 0);
+    h.eps = (float)g.get_float(a + "attention.layer_norm_rms_epsilon", 1e-5);
+    h.rope_base = g.get_float(a + "rope.freq_base", 10000.0);
+    h.rope_dim = (int)g.get_int(a + "rope.dimension_count", h.head_dim);
+    h.n_expert = (int)g.get_int(a + "expert_count", 0);
+    if (h.n_expert > 0) throw std::runtime_error("mixture-of-experts models are not supported yet");
+    if (h.head_dim != 32 && h.head_dim != 64 && h.head_dim != 128) throw std::runtime_error("head_dim must be 32, 64 or 128");
+    if (h.rope_dim > h.head_dim || h.rope_dim % 2 != 0) throw std::runtime_error("unsupported rotary width");
+
+    const TensorInfo & emb = g.require("token_embd.weight");
+    h.n_vocab = (int)emb.ne[1];
+    const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim;
+    if (emb.ne[0] != E) throw std::runtime_error("token_embd.weight does not match embedding_length");
+
+    upload_weight(emb, E, h.n_vocab, emb.data, emb.nbytes, true, tok_embd_);
+    const TensorInfo * head = g.find("output.weight");
+    if (!head) head = &emb;   // tied
+    upload_weight(*head, E, h.n_vocab, head->data, head->nbytes, false, lm_head_);
+    upload_f32(&g.require("output_norm.weight"), out_norm_, (size_t)E);
+    upload_f32(g.find("output.bias"), out_bias_, (size_t)h.n_vocab);
+
+    layers_.resize((size_t)h.n_layer);
+    for (int l = 0; l < h.n_layer; ++l) {
+        LayerWeights & L = layers_[(size_t)l];
+        const std::string b = "blk." + std::to_string(l) + ".";
+        upload_f32(&g.require(b + "attn_norm.weight"), L.attn_norm, (size_t)E);
+        upload_f32(&g.require(b + "ffn_norm.weight"), L.ffn_norm, (size_t)E);
+        upload_f32(g.find(b + "attn_q_norm.weight"), L.q_norm, (size_t)h.head_dim);
+        upload_f32(g.find(b + "attn_k_norm.weight"), L.k_norm, (size_t)h.head_dim);
+        const TensorInfo & wq = g.require(b + "attn_q.weight");
+        const TensorInfo & wk = g.require(b + "attn_k.weight");
+        const TensorInfo & wv = g.require(b + "attn_v.weight");
+        if (wq.ne[0] != E || wq.ne[1] != QD || wk.ne[1] != KD || wv.ne[1] != KD) throw std::runtime_error("attention weights of layer " + std::to_string(l) + " have unexpected shapes");
+        upload_fused({&wq, &wk, &wv}, L.qkv);
+        const TensorInfo * bq = g.find(b + "attn_q.bias");
+        if (bq) {
+            const TensorInfo & bk = g.require(b + "attn_k.bias");
+            const TensorInfo & bv = g.require(b + "attn_v.bias");
+            if (bq->type != rk::WT_F32 || bk.type != rk::WT_F32 || bv.type != rk::WT_F32) throw std::runtime_error("attention biases must be F32");
+            std::vector<float> joined((size_t)(QD + 2 * KD));
+            std::memcpy(joined.data(), bq->data, (size_t)QD * 4);
+            std::memcpy(joined.data() + QD, bk.data, (size_t)KD * 4);
+            std::memcpy(joined.data() + QD + KD, bv.data, (size_t)KD * 4);
+            L.qkv_bias.alloc(joined.size() * 4);
+            hip_check(hipMemcpy(L.qkv_bias.ptr, joined.data(), joined.size() * 4, hipMemcpyHostToDevice), "hipMemcpy");
+        }
+        const TensorInfo & wo = g.require(b + "attn_output.weight");
+        upload_weight(wo, QD, E, wo.data, wo.nbytes, false, L.wo);
+        const TensorInfo & wg = g.require(b + "ffn_gate.weight");
+        const TensorInfo & wu = g.require(b + "ffn_up.weight");
+        const TensorInfo & wd = g.require(b + "ffn_down.weight");
+        if (wg.ne[0] != E || wu.ne[0] != E || wg.ne[1] != wu.ne[1] || wd.ne[0] != wg.ne[1] || wd.ne[1] != E) throw std::runtime_error("feed-forward weights of layer " + std::to_string(l) + " have unexpected shapes");
+        h.n_ff = (int)wg.ne[1];
+        upload_fused({&wg, &wu}, L.gate_up);
+        upload_weight(wd, h.n_ff, E, wd.data, wd.nbytes, false, L.down);
+    }
+
+    // rotary frequencies in double: angle = pos * base^(-2i/d)
+    std::vector<double> inv((size_t)(h.rope_dim / 2));
+    for (size_t i = 0; i < inv.size(); ++i) inv[i] = std::pow(h.rope_base, -2.0 * (double)i / h.rope_dim);
+    inv_freq_.alloc(inv.size() * sizeof(double));
+    hip_check(hipMemcpy(inv_freq_.ptr, inv.data(), inv.size() * sizeof(double), hipMemcpyHostToDevice), "hipMemcpy");
+
+    // vocabulary
+    if (const MetaValue * toks = g.meta("tokenizer.ggml.tokens")) vocab_.pieces = toks->sa;
+    if (const MetaValue * types = g.meta("tokenizer.ggml.token_type")) {
+        vocab_.types.assign(types->ia.begin(), types->ia.end());
+    }
+    vocab_.eos = (int32_t)g.get_int("tokenizer.ggml.eos_token_id", -1);
+    vocab_.eot = (int32_t)g.get_int("tokenizer.ggml.eot_token_id", -1);
+
+    // FNV-1a over the path bytes then the u64 weight size
+    // (reference retro_runtime.hpp:856-868).
+    uint64_t hash = UINT64_C(14695981039346656037);
+    auto mix = [&hash](const void * data, size_t n) {
+        const unsigned char * p = (const unsigned char *)data;
+        for (size_t i = 0; i < n; ++i) { hash ^= p[i]; hash *= UINT64_C(1099511628211); }
+    };
+    mix(path.data(), path.size());
+    const uint64_t size = g.tensor_bytes();
+    mix(&size, sizeof(size));
+    fingerprint_ = hash;
+}
+
+void Engine::build_buffers() {
+    const int B = (int)cfg_.n_batch;
+    const int E = hp_.n_embd, QD = hp_.n_head * hp_.head_dim, KD = hp_.n_head_kv * hp_.head_dim, F = hp_.n_ff;
+    auto i32 = [&](size_t n) {
+        pk_store_.emplace_back();
+        pk_store_.back().alloc(n * 4);
+        return pk_store_.back().as<int32_t>();
+    };
+    pk_.tok = i32((size_t)B); pk_.pos = i32((size_t)B); pk_.seq = i32((size_t)B); pk_.row = i32((size_t)B);
+    pk_.cell = i32((size_t)B); pk_.out_index = i32((size_t)B); pk_.out_tok = i32((size_t)B);
+    pk_.last_index = i32((size_t)B); pk_.row_offset = i32((size_t)B + 1); pk_.counts = i32(4);
+    pk_.tile_t0 = i32((size_t)B); pk_.tile_nq = i32((size_t)B); pk_.tile_item0 = i32((size_t)B);
+    pk_.tile_nsplit = i32((size_t)B); pk_.tile_page0 = i32((size_t)B); pk_.tile_kv_begin = i32((size_t)B);
+    pk_.tok_tile = i32((size_t)B);
+    pk_.rope_cos = (float *)i32((size_t)B * (hp_.rope_dim / 2));
+    pk_.rope_sin = (float *)i32((size_t)B * (hp_.rope_dim / 2));
+
+    x_.alloc((size_t)B * E * 4);
+    qkv_.alloc((size_t)B * (QD + 2 * KD) * 4);
+    gu_.alloc((size_t)B * 2 * F * 4);
+    q_half_.alloc((size_t)B * QD * 2);
+    auto act = [&](DevBuf & x, DevBuf & hi, DevBuf & lo, int K) {
+        x.alloc((size_t)B * K * 2);
+        hi.alloc((size_t)B * (K / 32 + 1) * 2);
+        lo.alloc((size_t)B * (K / 32 + 1) * 2);
+    };
+    act(act_e_x_, act_e_hi_, act_e_lo_, E);
+    act(act_q_x_, act_q_hi_, act_q_lo_, QD);
+    act(act_f_x_, act_f_hi_, act_f_lo_, F);
+    act(act_o_x_, act_o_hi_, act_o_lo_, E);
+    sample_k_.alloc((size_t)B * 4);
+    sample_out_.alloc((size_t)B * sizeof(rk::SampleOut));
+    const size_t stage = (size_t)B * (sizeof(rk::RowDesc) + 4) + 65536;
+    d_stage_.alloc(stage);
+    h_stage_.ensure(stage);
+    h_sample_.ensure((size_t)B * sizeof(rk::SampleOut));
+}
+
+// ---- pages ---------------------------------------------------------------------------
+
+int32_t Engine::alloc_page() {
+    if (free_pages_.empty()) return -1;
+    const int32_t p = free_pages_.top();
+    free_pages_.pop();
+    page_ref_[(size_t)p] = 1;
+    return p;
+}
+
+void Engine::release_page(int32_t page) {
+    if (page < 0) return;
+    if (--page_ref_[(size_t)page] == 0) free_pages_.push(page);
+}
+
+void Engine::copy_page(int32_t src, int32_t dst) {
+    for (int l = 0; l < hp_.n_layer; ++l) {
+        rk::kv_copy_page(stream_, k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(),
+                         hp_.n_head_kv, hp_.head_dim, src, dst);
+    }
+}
+
+void Engine::set_page(int32_t slot, int idx, int32_t page) {
+    slots_[(size_t)slot].pages[(size_t)idx] = page;
+    pending_updates_.push_back({slot, idx, page, 0});
+}
+
+void Engine::clear_slot(Slot & s, int32_t slot) {
+    if (s.end > s.begin) {
+        for (int idx = s.begin / rk::PAGE; idx <= (s.end - 1) / rk::PAGE; ++idx) {
+            release_page(s.pages[(size_t)idx]);
+            set_page(slot, idx, -1);
+        }
+    }
+    s.begin = s.end = 0;
+}
+
+bool Engine::seq_rm(int32_t slot, int32_t p0, int32_t p1) {
+    if (slot < 0 || slot >= (int32_t)cfg_.n_seq_max) {
+        set_error("slot is outside the context's sequence range");
+        return false;
+    }
+    Slot & s = slots_[(size_t)slot];
+    if (p0 < 0) p0 = 0;
+    if (p1 < 0) p1 = INT_MAX;
+    if (s.end <= s.begin || p0 >= s.end || p1 <= s.begin || p0 >= p1) return true;
+    if (p0 <= s.begin && p1 >= s.end) {
+        clear_slot(s, slot);
+        return true;
+    }
+    if (p1 >= s.end) {                       // drop a suffix: keep [begin, p0)
+        const int keep_last = (p0 - 1) / rk::PAGE;
+        for (int idx = keep_last + 1; idx <= (s.end - 1) / rk::PAGE; ++idx) {
+            release_page(s.pages[(size_t)idx]);
+            set_page(slot, idx, -1);
+        }
+        s.end = p0;
+        return true;
+    }
+    if (p0 <= s.begin) {                     // drop a prefix: keep [p1, end)
+        const int keep_first = p1 / rk::PAGE;
+        for (int idx = s.begin / rk::PAGE; idx < keep_first; ++idx) {
+            release_page(s.pages[(size_t)idx]);
+            set_page(slot, idx, -1);
+        }
+        s.begin = p1;
+        return true;
+    }
+    set_error("the memory cannot remove that partial range; remove the whole sequence instead");
+    return false;
+}
+
+bool Engine::seq_cp(int32_t src, int32_t dst, int32_t p0, int32_t p1) {
+    const int32_t n = (int32_t)cfg_.n_seq_max;
+    if (src < 0 || src >= n || dst < 0 || dst >= n) {
+        set_error("seq_cp slots are outside the context's sequence range");
+        return false;
+    }
+    if (src == dst) return true;
+    const Slot & a = slots_[(size_t)src];
+    Slot & b = slots_[(size_t)dst];
+    const bool whole = p0 <= 0 && p1 < 0;
+    if (p0 < 0) p0 = 0;
+    if (p1 < 0) p1 = INT_MAX;
+    const int lo = std::max(p0, a.begin), hi = std::min(p1, a.end);
+    if (a.end <= a.begin || hi <= lo) return true;
+    if (!cfg_.kv_unified && !(whole || (lo == a.begin && hi == a.end))) {
+        set_error("a partitioned KV pool only supports whole-sequence copies");
+        return false;
+    }
+    if (b.end > b.begin) {
+        if (lo < b.end && b.begin < hi) {
+            set_error("seq_cp: the copied range of the destination is not empty");
+            return false;
+        }
+        if (lo != b.end && hi != b.begin) {
+            set_error("seq_cp: the copied range is not adjacent to the destination's resident range");
+            return false;
+        }
+    }
+    // Pages are shared by reference; a page either side later writes into is
+    // copied first (see the step), so a partially used last page costs nothing here.
+    for (int idx = lo / rk::PAGE; idx <= (hi - 1) / rk::PAGE; ++idx) {
+        const int32_t sp = a.pages[(size_t)idx];
+        const int32_t dp = b.pages[(size_t)idx];
+        if (dp < 0) {
+            ++page_ref_[(size_t)sp];
+            set_page(dst, idx, sp);
+        } else if (dp != sp) {
+            // The destination already owns part of this page index (adjacent
+            // ranges meeting inside one page): merge position by position.
+            int32_t target = dp;
+            if (page_ref_[(size_t)dp] > 1) {
+                target = alloc_page();
+                if (target < 0) {
+                    set_error("the KV pool is full");
+                    return false;
+                }
+                copy_page(dp, target);
+                release_page(dp);
+                set_page(dst, idx, target);
+            }
+            const int first = std::max(lo, idx * rk::PAGE), last = std::min(hi, (idx + 1) * rk::PAGE);
+            std::vector<int32_t> cells_src, cells_dst;
+            for (int p = first; p < last; ++p) {
+                cells_src.push_back(sp * rk::PAGE + p % rk::PAGE);
+                cells_dst.push_back(target * rk::PAGE + p % rk::PAGE);
+            }
+            const size_t kd = (size_t)hp_.n_head_kv * hp_.head_dim;
+            DevBuf cs, cd, tmp;
+            cs.alloc(cells_src.size() * 4);
+            cd.alloc(cells_dst.size() * 4);
+            tmp.alloc(cells_src.size() * kd * 2);
+            hip_check(hipMemcpyAsync(cs.ptr, cells_src.data(), cs.bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
+            hip_check(hipMemcpyAsync(cd.ptr, cells_dst.data(), cd.bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
+            for (int l = 0; l < hp_.n_layer; ++l) {
+                for (int v = 0; v < 2; ++v) {
+                    __half * pool = v ? v_pool_[(size_t)l].as<__half>() : k_pool_[(size_t)l].as<__half>();
+                    rk::kv_gather(stream_, pool, hp_.n_head_kv, hp_.head_dim, v != 0, cs.as<int32_t>(), (int)cells_src.size(), tmp.as<__half>());
+                    rk::kv_scatter(stream_, pool, hp_.n_head_kv, hp_.head_dim, v != 0, cd.as<int32_t>(), (int)cells_dst.size(), tmp.as<__half>());
+                }
+            }
+            hip_check(hipStreamSynchronize(stream_), "seq_cp merge");
+        }
+    }
+    if (b.end <= b.begin) { b.begin = lo; b.end = hi; }
+    else { b.begin = std::min(b.begin, lo); b.end = std::max(b.end, hi); }
+    return true;
+}
+
+int Engine::seq_pos(int32_t slot, int32_t * out_min, int32_t * out_max) {
+    if (!out_min || !out_max) {
+        set_error("the position outputs are required");
+        return -1;
+    }
+    if (slot < 0 || slot >= (int32_t)cfg_.n_seq_max) {
+        set_error("slot is outside the context's sequence range");
+        return -1;
+    }
+    const Slot & s = slots_[(size_t)slot];
+    if (s.end <= s.begin) { *out_min = -1; *out_max = -1; }
+    else { *out_min = s.begin; *out_max = s.end - 1; }
+    return 0;
+}
+
+int Engine::memory(retro_engine_memory_info * out) {
+    if (!out) {
+        set_error("out is required");
+        return -1;
+    }
+    out->struct_size = sizeof(retro_engine_memory_info);
+    out->n_slots = cfg_.n_seq_max;
+    out->cells_total = cfg_.n_ctx;
+    uint64_t used = 0;
+    for (const Slot & s : slots_) if (s.end > s.begin) used += (uint64_t)(s.end - s.begin);
+    out->cells_used = used;
+    uint64_t kv = 0;
+    for (const auto & b : k_pool_) kv += b.bytes;
+    for (const auto & b : v_pool_) kv += b.bytes;
+    out->kv_bytes = kv;
+    out->recurrent_bytes = 0;
+    return 0;
+}
+
+// ---- snapshots -------------------------------------------------------------------------
+//
+// Byte format (this library's own; only seq_load of the same build reads it):
+//   u32 magic "RKV1", u32 flags, i32 n_layer, i32 kv_dim, i32 begin, i32 end,
+//   then per layer the K rows [end-begin][kv_dim] and the V rows, f16, in
+//   natural element order.
+namespace {
+struct SnapHeader { uint32_t magic, flags; int32_t n_layer, kv_dim, begin, end; };
+constexpr uint32_t kSnapMagic = 0x31564b52u;
+}
+
+int Engine::seq_save(int32_t slot, uint32_t flags, uint8_t * buffer, size_t n_buffer, size_t * out_n_bytes) {
+    if (!out_n_bytes) {
+        set_error("out_n_bytes is required");
+        return -1;
+    }
+    if (flags & ~RETRO_STATE_SEQ_FLAGS_PARTIAL_ONLY) {
+        set_error("only host snapshots (flags 0 or PARTIAL_ONLY) are supported");
+        return -1;
+    }
+    if (slot < 0 || slot >= (int32_t)cfg_.n_seq_max) {
+        set_error("slot is outside the context's sequence range");
+        return -1;
+    }
+    const Slot & s = slots_[(size_t)slot];
+    const size_t kd = (size_t)hp_.n_head_kv * hp_.head_dim;
+    const bool partial_only = (flags & RETRO_STATE_SEQ_FLAGS_PARTIAL_ONLY) != 0;
+    const int n_pos = partial_only ? 0 : std::max(0, s.end - s.begin);   // no recurrent or SWA state exists
+    const size_t required = sizeof(SnapHeader) + (size_t)hp_.n_layer * 2 * (size_t)n_pos * kd * 2;
+    *out_n_bytes = required;
+    if (!buffer) return 0;
+    if (n_buffer < required) {
+        set_error("the save buffer is too small for this sequence's state");
+        return -2;
+    }
+    SnapHeader h{kSnapMagic, flags, hp_.n_layer, (int32_t)kd, partial_only ? 0 : s.begin, partial_only ? 0 : s.begin + n_pos};
+    std::memcpy(buffer, &h, sizeof(h));
+    if (n_pos > 0) {
+        std::vector<int32_t> cells((size_t)n_pos);
+        for (int p = s.begin; p < s.end; ++p) cells[(size_t)(p - s.begin)] = s.pages[(size_t)(p / rk::PAGE)] * rk::PAGE + p % rk::PAGE;
+        DevBuf dc, tmp;
+        dc.alloc(cells.size() * 4);
+        tmp.alloc((size_t)n_pos * kd * 2);
+        hip_check(hipMemcpyAsync(dc.ptr, cells.data(), dc.bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
+        uint8_t * at = buffer + sizeof(h);
+        for (int l = 0; l < hp_.n_layer; ++l) {
+            for (int v = 0; v < 2; ++v) {
+                const __half * pool = v ? v_pool_[(size_t)l].as<__half>() : k_pool_[(size_t)l].as<__half>();
+                rk::kv_gather(stream_, pool, hp_.n_head_kv, hp_.head_dim, v != 0, dc.as<int32_t>(), n_pos, tmp.as<__half>());
+                hip_check(hipMemcpyAsync(at, tmp.ptr, tmp.bytes, hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync");
+                hip_check(hipStreamSynchronize(stream_), "seq_save");
+                at += tmp.bytes;
+            }
+        }
+    }
+    return 0;
+}
+
+int Engine::seq_load(int32_t slot, uint32_t flags, const uint8_t * buffer, size_t n_bytes, size_t * out_n_read) {
+    if (!out_n_read) {
+        set_error("out_n_read is required");
+        return -1;
+    }
+    if (flags & ~RETRO_STATE_SEQ_FLAGS_PARTIAL_ONLY) {
+        set_error("only host snapshots (flags 0 or PARTIAL_ONLY) are supported");
+        return -1;
+    }
+    if (slot < 0 || slot >= (int32_t)cfg_.n_seq_max) {
+        set_error("slot is outside the context's sequence range");
+        return -1;
+    }
+    if (!buffer || n_bytes == 0) {
+        set_error("a snapshot buffer is required");
+        return -1;
+    }
+    const char * refused = "the snapshot was refused (wrong size, flags or corrupted data)";
+    SnapHeader h;
+    if (n_bytes < sizeof(h)) { set_error(refused); return -1; }
+    std::memcpy(&h, buffer, sizeof(h));
+    const size_t kd = (size_t)hp_.n_head_kv * hp_.head_dim;
+    if (h.magic != kSnapMagic || h.flags != flags || h.n_layer != hp_.n_layer || h.kv_dim != (int32_t)kd
+            || h.begin < 0 || h.end < h.begin || h.end > n_ctx_seq_) {
+        set_error(refused);
+        return -1;
+    }
+    const int n_pos = h.end - h.begin;
+    const size_t required = sizeof(h) + (size_t)hp_.n_layer * 2 * (size_t)n_pos * kd * 2;
+    if (n_bytes < required) { set_error(refused); return -1; }
+    if (flags & RETRO_STATE_SEQ_FLAGS_PARTIAL_ONLY) {
+        *out_n_read = required;
+        return 0;
+    }
+    Slot & s = slots_[(size_t)slot];
+    clear_slot(s, slot);
+    if (n_pos > 0) {
+        const int first = h.begin / rk::PAGE, last = (h.end - 1) / rk::PAGE;
+        if ((int)free_pages_.size() < last - first + 1) {
+            set_error("the KV pool is full");
+            return -1;
+        }
+        for (int idx = first; idx <= last; ++idx) set_page(slot, idx, alloc_page());
+        s.begin = h.begin;
+        s.end = h.end;
+        std::vector<int32_t> cells((size_t)n_pos);
+        for (int p = s.begin; p < s.end; ++p) cells[(size_t)(p - s.begin)] = s.pages[(size_t)(p / rk::PAGE)] * rk::PAGE + p % rk::PAGE;
+        DevBuf dc, tmp;
+        dc.alloc(cells.size() * 4);
+        tmp.alloc((size_t)n_pos * kd * 2);
+        hip_check(hipMemcpyAsync(dc.ptr, cells.data(), dc.bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
+        const uint8_t * at = buffer + sizeof(h);
+        for (int l = 0; l < hp_.n_layer; ++l) {
+            for (int v = 0; v < 2; ++v) {
+                __half * pool = v ? v_pool_[(size_t)l].as<__half>() : k_pool_[(size_t)l].as<__half>();
+                hip_check(hipMemcpyAsync(tmp.ptr, at, tmp.bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
+                rk::kv_scatter(stream_, pool, hp_.n_head_kv, hp_.head_dim, v != 0, dc.as<int32_t>(), n_pos, tmp.as<__half>());
+                hip_check(hipStreamSynchronize(stream_), "seq_load");
+                at += tmp.bytes;
+            }
+        }
+    }
+    *out_n_read = required;
+    return 0;
+}
+
+// ---- the step -------------------------------------------------------------------------
+
+namespace {
+
+bool valid_sampling_v1(const retro_sampling_params & s) {
+    if (!(s.temperature > 0.0f) || !std::isfinite(s.temperature)) {
+        set_error("sampling temperature must be finite and greater than zero");
+        return false;
+    }
+    if (!(s.top_p > 0.0f && s.top_p <= 1.0f)) {
+        set_error("sampling top_p must be in (0, 1]");
+        return false;
+    }
+    if (s.max_new_tokens == 0) {
+        set_error("sampling max_new_tokens must be greater than zero");
+        return false;
+    }
+    return true;
+}
+
+bool valid_tokens(const int32_t * tokens, size_t n, int32_t n_vocab) {
+    for (size_t i = 0; i < n; ++i) {
+        if (tokens[i] < 0 || tokens[i] >= n_vocab) {
+            std::ostringstream m;
+            m << "token " << tokens[i] << " at index " << i << " is outside the vocabulary of size " << n_vocab;
+            set_error(m.str());
+            return false;
+        }
+    }
+    return true;
+}
+
+// Same checks, order and messages as the reference (retro_gen_core.cpp:1539-1589).
+bool valid_sampling_v2(const retro_sampling_params_v2 & s, int32_t n_vocab) {
+    if (s.struct_size < sizeof(retro_sampling_params_v2)) {
+        set_error("retro_sampling_params_v2.struct_size is too small for this build");
+        return false;
+    }
+    if (!(s.temperature > 0.0f) || !std::isfinite(s.temperature)) {
+        set_error("sampling temperature must be finite and greater than zero");
+        return false;
+    }
+    if (!(s.top_p > 0.0f && s.top_p <= 1.0f)) {
+        set_error("sampling top_p must be in (0, 1]");
+        return false;
+    }
+    if (!(s.repeat_penalty > 0.0f) || !std::isfinite(s.repeat_penalty)) {
+        set_error("sampling repeat_penalty must be finite and greater than zero");
+        return false;
+    }
+    if (!(s.min_p >= 0.0f && s.min_p <= 1.0f) || !std::isfinite(s.min_p)) {
+        set_error("sampling min_p must be in [0, 1]");
+        return false;
+    }
+    if (!std::isfinite(s.frequency_penalty)) {
+        set_error("sampling frequency_penalty must be finite");
+        return false;
+    }
+    if (!std::isfinite(s.presence_penalty)) {
+        set_error("sampling presence_penalty must be finite");
+        return false;
+    }
+    if (s.n_logit_bias > 4096) {
+        set_error("sampling n_logit_bias must not exceed 4096");
+        return false;
+    }
+    if (s.n_logit_bias > 0) {
+        if (!s.logit_bias_ids || !s.logit_bias_values) {
+            set_error("logit_bias ids and values are required when n_logit_bias is nonzero");
+            return false;
+        }
+        if (!valid_tokens(s.logit_bias_ids, s.n_logit_bias, n_vocab)) return false;
+        for (uint32_t i = 0; i < s.n_logit_bias; ++i) {
+            if (!std::isfinite(s.logit_bias_values[i])) {
+                set_error("logit_bias values must be finite");
+                return false;
+            }
+        }
+    }
+    return true;
+}
+
+}  // namespace
+
+int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, size_t n_rows,
+                 retro_step_out_row_v2 * out2, retro_step_out_row * out1,
+                 int32_t * out_top_ids, float * out_top_logprobs, size_t n_top_stride) {
+    const bool is_v2 = rows2 != nullptr;
+    if ((!rows2 && !rows1) || n_rows == 0 || (!out2 && !out1)) {
+        set_error("step rows and output rows are required");
+        return -3;
+    }
+    const int32_t n_seq_max = (int32_t)cfg_.n_seq_max;
+    const int32_t n_batch = (int32_t)cfg_.n_batch;
+    const int64_t n_ctx_seq = n_ctx_seq_;
+    const int32_t n_vocab = hp_.n_vocab;
+
+    // ---- validation: caller errors are reported before anything decodes
+    // (order and messages follow retro_gen_core.cpp:2353-2516).
+    std::vector<RowView> rows(n_rows);
+    if (is_v2) {
+        for (size_t r = 0; r < n_rows; ++r) {
+            const retro_step_row_v2 & in = rows2[r];
+            if (in.struct_size < offsetof(retro_step_row_v2, adapter) + sizeof(int32_t)) {
+                set_error("retro_step_row_v2.struct_size is too small for this build");
+                return -3;
+            }
+            if (in.sampling.struct_size < sizeof(retro_sampling_params_v2)) {
+                set_error("retro_sampling_params_v2.struct_size is too small for this build");
+                return -3;
+            }
+            RowView & v = rows[r];
+            v.request = in.request; v.slot = in.slot; v.tokens = in.tokens; v.n = in.n; v.pos0 = in.pos0;
+            v.sample = in.sample; v.v2 = &in.sampling; v.v1 = retro_sampling_params{};
+            v.n_top = in.n_top_logprobs; v.want_logprob = in.want_logprob != 0; v.adapter = in.adapter;
+        }
+    } else {
+        for (size_t r = 0; r < n_rows; ++r) {
+            const retro_step_row & in = rows1[r];
+            // Read the evolution key before any other field.
+            if (in.struct_size < offsetof(retro_step_row, adapter) + sizeof(int32_t)) {
+                set_error("retro_step_row.struct_size is too small for this build");
+                return -3;
+            }
+            RowView & v = rows[r];
+            v.request = in.request; v.slot = in.slot; v.tokens = in.tokens; v.n = in.n; v.pos0 = in.pos0;
+            v.sample = in.sample; v.v2 = nullptr; v.v1 = in.sampling;
+            v.n_top = in.n_top_logprobs; v.want_logprob = false; v.adapter = in.adapter;
+        }
+    }
+    if (n_rows > (size_t)n_batch || (n_top_stride != 0 && n_rows > SIZE_MAX / n_top_stride)) {
+        set_error("the step row count or output shape exceeds capacity");
+        return -3;
+    }
+    std::vector<int32_t> seen_requests;
+    size_t total = 0;
+    for (size_t r = 0; r < n_rows; ++r) {
+        const RowView & row = rows[r];
+        if (!row.tokens || row.n == 0) {
+            set_error("a step row requires at least one token");
+            return -3;
+        }
+        if (row.slot < 0 || row.slot >= n_seq_max) {
+            set_error("step row slot is outside the context's sequence range");
+            return -3;
+        }
+        if (row.adapter != 0) {
+            // No per-row adapter is ever loaded in this build (retro_engine_adapter_load
+            // refuses), so the only other legal value is the base model.
+            if (row.adapter != RETRO_STEP_ADAPTER_BASE) {
+                set_error("step row adapter " + std::to_string(row.adapter) + " is not a loaded per-row adapter");
+                return -3;
+            }
+        }
+        if (row.pos0 < 0 || (int64_t)row.pos0 + row.n > n_ctx_seq) {
+            set_error("step row positions exceed the per-sequence context");
+            return -3;
+        }
+        for (size_t prev = 0; prev < r; ++prev) {
+            const RowView & other = rows[prev];
+            if (row.slot == other.slot && row.pos0 < (int64_t)other.pos0 + other.n
+                    && other.pos0 < (int64_t)row.pos0 + row.n) {
+                set_error("step rows overlap in the same sequence slot");
+                return -3;
+            }
+            if (row.slot == other.slot && row.adapter != other.adapter) {
+                set_error("step rows of one sequence slot select different adapters");
+                return -3;
+            }
+        }
+        if (!valid_tokens(row.tokens, row.n, n_vocab)) return -3;
+        if (row.n > (uint32_t)n_batch || total + row.n > (size_t)n_batch) {
+            set_error("the step's tokens exceed the context's physical batch (n_batch)");
+            return -3;
+        }
+        total += row.n;
+        if (row.n_top > 0 && (!out_top_ids || !out_top_logprobs)) {
+            set_error("top logprobs requested but the output buffers are missing");
+            return -3;
+        }
+        if (row.n_top > n_top_stride) {
+            set_error("a step row's n_top_logprobs exceeds the output stride");
+            return -3;
+        }
+        if (row.sample) {
+            if (row.request < 0) {
+                set_error("a sampling step row requires a request id");
+                return -3;
+            }
+            if (row.v2) {
+                if (!valid_sampling_v2(*row.v2, n_vocab)) return -3;
+                if (row.v2->grammar) {
+                    set_error("grammar-constrained rows are not supported by this library");
+                    return -3;
+                }
+            } else {
+                retro_sampling_params s = row.v1;
+                s.max_new_tokens = 1;   // the caller owns stopping
+                if (!valid_sampling_v1(s)) return -3;
+            }
+        }
+        if (row.request >= 0) {
+            if (std::find(seen_requests.begin(), seen_requests.end(), row.request) != seen_requests.end()) {
+                set_error("a request id appears twice in one step");
+                return -3;
+            }
+            seen_requests.push_back(row.request);
+        }
+    }
+
+    // ---- KV placement: positions must extend each slot's resident range.
+    // Nothing is mutated until the whole plan is known to fit.
+    {
+        std::vector<std::pair<int, int>> span(slots_.size());
+        for (size_t i = 0; i < slots_.size(); ++i) span[i] = {slots_[i].begin, slots_[i].end};
+        std::vector<std::pair<int32_t, int>> touched;   // (slot, page index) already paid for
+        size_t need = 0;
+        for (const RowView & row : rows) {
+            auto & sp = span[(size_t)row.slot];
+            if (sp.second > sp.first && row.pos0 != sp.second) {
+                set_error(row.pos0 < sp.second
+                    ? "step row positions are already resident in the slot: remove them with seq_rm first"
+                    : "step row positions leave a gap after the slot's resident range");
+                return -1;
+            }
+            if (sp.second <= sp.first) sp.first = row.pos0;
+            const int last = row.pos0 + (int)row.n;
+            const Slot & s = slots_[(size_t)row.slot];
+            for (int idx = row.pos0 / rk::PAGE; idx <= (last - 1) / rk::PAGE; ++idx) {
+                const std::pair<int32_t, int> key{row.slot, idx};
+                if (std::find(touched.begin(), touched.end(), key) != touched.end()) continue;
+                const int32_t pg = s.pages[(size_t)idx];
+                if (pg < 0 || page_ref_[(size_t)pg] > 1) {   // a fresh page, or a private copy of a shared one
+                    ++need;
+                    touched.push_back(key);
+                }
+            }
+            sp.second = last;
+        }
+        if (need > free_pages_.size()) {
+            set_error("the KV pool is full: the step needs " + std::to_string(need) + " pages, "
+                      + std::to_string(free_pages_.size()) + " are free");
+            return -1;
+        }
+    }
+    for (const RowView & row : rows) {
+        Slot & s = slots_[(size_t)row.slot];
+        if (s.end <= s.begin) { s.begin = row.pos0; s.end = row.pos0; }
+        const int last = row.pos0 + (int)row.n;
+        for (int idx = row.pos0 / rk::PAGE; idx <= (last - 1) / rk::PAGE; ++idx) {
+            const int32_t pg = s.pages[(size_t)idx];
+            if (pg < 0) {
+                set_page(row.slot, idx, alloc_page());
+            } else if (page_ref_[(size_t)pg] > 1) {
+                const int32_t fresh = alloc_page();
+                copy_page(pg, fresh);
+                release_page(pg);
+                set_page(row.slot, idx, fresh);
+            }
+        }
+        s.end = last;
+    }
+
+    // ---- upload the plan and pack it on the device
+    const int T = (int)total;
+    const size_t n_upd = pending_updates_.size();
+    const size_t off_tok = n_rows * sizeof(rk::RowDesc);
+    const size_t off_upd = off_tok + (size_t)T * 4;
+    const size_t stage_bytes = off_upd + n_upd * sizeof(rk::TableUpdate);
+    h_stage_.ensure(stage_bytes);
+    d_stage_.ensure(stage_bytes);
+    rk::RowDesc * hd = h_stage_.as<rk::RowDesc>();
+    int32_t * ht = (int32_t *)((uint8_t *)h_stage_.ptr + off_tok);
+    int n_out = 0;
+    {
+        int at = 0;
+        for (size_t r = 0; r < n_rows; ++r) {
+            const RowView & row = rows[r];
+            hd[r].slot = row.slot; hd[r].pos0 = row.pos0; hd[r].n = (int32_t)row.n; hd[r].tok_off = at;
+            hd[r].sample = row.sample ? 1 : 0; hd[r].kv_begin = slots_[(size_t)row.slot].begin;
+            hd[r].route = 0; hd[r].pad = 0;
+            std::memcpy(ht + at, row.tokens, (size_t)row.n * 4);
+            at += (int)row.n;
+            if (row.sample) ++n_out;
+        }
+    }
+    if (n_upd) std::memcpy((uint8_t *)h_stage_.ptr + off_upd, pending_updates_.data(), n_upd * sizeof(rk::TableUpdate));
+    pending_updates_.clear();
+    int n_tiles = 0, n_items = 0;
+    rk::count_attention_work(hd, (int)n_rows, qt_, hp_.n_head_kv, &n_tiles, &n_items);
+
+    try {
+        hip_check(hipMemcpyAsync(d_stage_.ptr, h_stage_.ptr, stage_bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
+        rk::pack_step(stream_, d_stage_.as<rk::RowDesc>(), (int)n_rows,
+                      (const int32_t *)((const uint8_t *)d_stage_.ptr + off_tok),
+                      (const rk::TableUpdate *)((const uint8_t *)d_stage_.ptr + off_upd), (int)n_upd,
+                      table_.as<int32_t>(), max_pages_, qt_, hp_.n_head_kv, inv_freq_.as<double>(),
+                      hp_.rope_dim / 2, pk_);
+        forward(T, n_out, n_tiles, n_items);
+
+        // ---- sampling: the device scans the vocabulary, the host draws.
+        std::vector<int32_t> kreq((size_t)std::max(n_out, 1), 0);
+        std::vector<int> out_of_row(n_rows, -1);
+        bool any_full = false;
+        {
+            int o = 0;
+            for (size_t r = 0; r < n_rows; ++r) {
+                const RowView & row = rows[r];
+                if (!row.sample) continue;
+                out_of_row[r] = o;
+                const bool fast = row.v2 && sampling::neutral_extras(*row.v2) && row.v2->top_k > 0
+                    && row.v2->top_k <= rk::MAX_TOPK && row.v2->top_k < n_vocab;
+                kreq[(size_t)o] = fast ? row.v2->top_k : 0;
+                any_full = any_full || !fast;
+                ++o;
+            }
+        }
+        if (n_out > 0) {
+            hip_check(hipMemcpyAsync(sample_k_.ptr, kreq.data(), (size_t)n_out * 4, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
+            rk::sample_prepare(stream_, logits_.as<float>(), n_out, n_vocab, sample_k_.as<int32_t>(), sample_out_.as<rk::SampleOut>());
+            hip_check(hipMemcpyAsync(h_sample_.ptr, sample_out_.ptr, (size_t)n_out * sizeof(rk::SampleOut), hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync");
+            if (any_full) {
+                h_logits_.ensure((size_t)n_out * n_vocab * 4);
+                for (size_t r = 0; r < n_rows; ++r) {
+                    const int o = out_of_row[r];
+                    if (o < 0 || kreq[(size_t)o] != 0) continue;
+                    hip_check(hipMemcpyAsync(h_logits_.as<float>() + (size_t)o * n_vocab, logits_.as<float>() + (size_t)o * n_vocab,
+                                             (size_t)n_vocab * 4, hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync");
+                }
+            }
+        }
+        hip_check(hipStreamSynchronize(stream_), "step");
+        last_n_out_ = n_out;
+        ++steps_run_;
+
+        const rk::SampleOut * so = h_sample_.as<rk::SampleOut>();
+        for (size_t r = 0; r < n_rows; ++r) {
+            const RowView & row = rows[r];
+            int32_t token = 0;
+            float logprob = 0.0f, sampled_logprob = 0.0f;
+            uint32_t n_top = 0;
+            uint8_t sampled = 0;
+            if (row.sample) {
+                const int o = out_of_row[r];
+                const rk::SampleOut & s = so[o];
+                RequestState & req = requests_[row.request];
+                if (!req.seeded) {
+                    req.rng.seed(row.v2 ? row.v2->seed : row.v1.seed);
+                    req.seeded = true;
+                }
+                const uint32_t k = std::min<uint32_t>(row.n_top, (uint32_t)std::min<size_t>(n_top_stride, (size_t)n_vocab));
+                int32_t * top_ids = k > 0 ? out_top_ids + r * n_top_stride : nullptr;
+                float * top_lps = k > 0 ? out_top_logprobs + r * n_top_stride : nullptr;
+                const double log_sum = std::log(s.sum_exp);
+                if (row.v2) {
+                    RowSample got;
+                    float token_logit = 0.0f;
+                    if (kreq[(size_t)o] > 0) {
+                        got = sampling::finish_from_candidates(*row.v2, s.top_id, s.top_logit, (size_t)kreq[(size_t)o],
+                                                               (size_t)n_vocab, req.rng, row.want_logprob, k, top_ids, top_lps);
+                        for (int j = 0; j < kreq[(size_t)o]; ++j) if (s.top_id[j] == got.token) token_logit = s.top_logit[j];
+                    } else {
+                        const float * host_row = h_logits_.as<float>() + (size_t)o * n_vocab;
+                        std::string err;
+                        got = sampling::sample_full_row_v2(host_row, (size_t)n_vocab, *row.v2, req.rng, req.history, scratch_,
+                                                           row.want_logprob, k, top_ids, top_lps, err);
+                        if (got.token < 0) {
+                            set_error(err);
+                            return -1;
+                        }
+                        token_logit = host_row[got.token];
+                    }
+                    token = got.token;
+                    sampled_logprob = row.want_logprob ? got.sampled_logprob : 0.0f;
+                    n_top = k;
+                    req.history.push_back(token);
+                    // temperature-1 policy logprob: logit - max - log(sum exp(logit - max))
+                    logprob = (float)((double)token_logit - s.max - log_sum);
+                } else {
+                    const float * host_row = h_logits_.as<float>() + (size_t)o * n_vocab;
+                    float smax = 0.0f;
+                    double stotal = 0.0;
+                    std::string err;
+                    token = sampling::sample_full_row_v1(host_row, (size_t)n_vocab, row.v1.temperature, row.v1.top_p,
+                                                         req.rng, scratch_, smax, stotal, err);
+                    if (token < 0) {
+                        set_error(err);
+                        return -1;
+                    }
+                    logprob = row.v1.temperature == 1.0f
+                        ? (float)((double)host_row[token] - smax - std::log(stotal))
+                        : (float)((double)host_row[token] - s.max - log_sum);
+                    if (k > 0) {
+                        sampling::top_logprobs_dense(host_row, (size_t)n_vocab, k, s.max, log_sum, scratch_.order, top_ids, top_lps);
+                        n_top = k;
+                    }
+                }
+                sampled = 1;
+            }
+            if (out2) {
+                retro_step_out_row_v2 & o = out2[r];
+                o.struct_size = sizeof(retro_step_out_row_v2);
+                o.token = token; o.logprob = logprob; o.n_top = n_top; o.forced = 0; o.sampled = sampled;
+                o.sampled_logprob = sampled_logprob;
+            } else {
+                retro_step_out_row & o = out1[r];
+                o.struct_size = sizeof(retro_step_out_row);
+                o.token = token; o.logprob = logprob; o.n_top = n_top; o.forced = 0; o.sampled = sampled;
+            }
+        }
+    } catch (const std::exception & e) {
+        set_error(std::string("the step failed on the device: ") + e.what()
+                  + " - the KV may hold a prefix of the submitted tokens (query it with the seq_pos entry point)");
+        return -1;
+    }
+    return 0;
+}
+
+void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
+    const HParams & h = hp_;
+    const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim, F = h.n_ff;
+    rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps};
+    rk::Act act_e{act_e_x_.as<__half>(), act_e_hi_.as<__half>(), act_e_lo_.as<__half>(), E};
+    rk::Act act_q{act_q_x_.as<__half>(), act_q_hi_.as<__half>(), act_q_lo_.as<__half>(), QD};
+    rk::Act act_f{act_f_x_.as<__half>(), act_f_hi_.as<__half>(), act_f_lo_.as<__half>(), F};
+    rk::Act act_o{act_o_x_.as<__half>(), act_o_hi_.as<__half>(), act_o_lo_.as<__half>(), E};
+    if (E % 32 != 0) { act_e.xs_hi = act_e.xs_lo = act_o.xs_hi = act_o.xs_lo = nullptr; }
+    if (QD % 32 != 0) { act_q.xs_hi = act_q.xs_lo = nullptr; }
+    if (F % 32 != 0) { act_f.xs_hi = act_f.xs_lo = nullptr; }
+    partial_.ensure(rk::attention_partial_floats(n_items, h.head_dim) * 4);
+    float * x = x_.as<float>();
+    float * qkv = qkv_.as<float>();
+    float * gu = gu_.as<float>();
+
+    rk::embed(stream_, tok_embd_.w, pk_.tok, T, x);
+    for (int l = 0; l < h.n_layer; ++l) {
+        const LayerWeights & L = layers_[(size_t)l];
+        rk::rmsnorm_act(stream_, x, L.attn_norm.as<float>(), E, h.eps, nullptr, T, act_e);
+        {
+            int col = 0;
+            for (const DevWeight & w : L.qkv) {
+                rk::matmul(stream_, w.w, act_e, T, qkv, QD + 2 * KD, col, rk::MM_STORE,
+                           L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr);
+                col += w.w.N;
+            }
+        }
+        rk::rope_store(stream_, qkv, T, sh, pk_, L.q_norm.as<float>(), L.k_norm.as<float>(), q_half_.as<__half>(),
+                       k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>());
+        rk::attention(stream_, q_half_.as<__half>(), sh, pk_, table_.as<int32_t>(), max_pages_,
+                      k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), n_items, n_tiles,
+                      partial_.as<float>());
+        rk::attention_combine(stream_, partial_.as<float>(), T, sh, pk_, act_q);
+        rk::matmul(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr);
+        rk::rmsnorm_act(stream_, x, L.ffn_norm.as<float>(), E, h.eps, nullptr, T, act_e);
+        {
+            int col = 0;
+            for (const DevWeight & w : L.gate_up) {
+                rk::matmul(stream_, w.w, act_e, T, gu, 2 * F, col, rk::MM_STORE, nullptr);
+                col += w.w.N;
+            }
+        }
+        rk::swiglu_act(stream_, gu, T, F, act_f);
+        rk::matmul(stream_, L.down.w, act_f, T, x, E, 0, rk::MM_ADD, nullptr);
+    }
+    if (n_out > 0) {
+        logits_.ensure((size_t)n_out * h.n_vocab * 4);
+        rk::rmsnorm_act(stream_, x, out_norm_.as<float>(), E, h.eps, pk_.out_tok, n_out, act_o);
+        rk::matmul(stream_, lm_head_.w, act_o, n_out, logits_.as<float>(), h.n_vocab, 0, rk::MM_STORE,
+                   out_bias_.as<float>());
+    }
+}
+
+// ---- test hooks -------------------------------------------------------------------------
+
+int Engine::debug_last_logits(float * out, size_t n_floats, size_t * out_rows) {
+    if (out_rows) *out_rows = (size_t)last_n_out_;
+    const size_t need = (size_t)last_n_out_ * hp_.n_vocab;
+    if (!out) return 0;
+    if (n_floats < need) {
+        set_error("the logits buffer is too small");
+        return -2;
+    }
+    if (need) hip_check(hipMemcpy(out, logits_.ptr, need * 4, hipMemcpyDeviceToHost), "hipMemcpy");
+    return 0;
+}
+
+int Engine::debug_read_kv(int layer, int32_t slot, int32_t pos, int want_v, uint16_t * out) {
+    if (layer < 0 || layer >= hp_.n_layer || slot < 0 || slot >= (int32_t)cfg_.n_seq_max) {
+        set_error("layer or slot out of range");
+        return -1;
+    }
+    const Slot & s = slots_[(size_t)slot];
+    if (pos < s.begin || pos >= s.end) {
+        set_error("position is not resident");
+        return -1;
+    }
+    const int32_t cell = s.pages[(size_t)(pos / rk::PAGE)] * rk::PAGE + pos % rk::PAGE;
+    const size_t kd = (size_t)hp_.n_head_kv * hp_.head_dim;
+    DevBuf dc, tmp;
+    dc.alloc(4);
+    tmp.alloc(kd * 2);
+    hip_check(hipMemcpy(dc.ptr, &cell, 4, hipMemcpyHostToDevice), "hipMemcpy");
+    const __half * pool = want_v ? v_pool_[(size_t)layer].as<__half>() : k_pool_[(size_t)layer].as<__half>();
+    rk::kv_gather(stream_, pool, hp_.n_head_kv, hp_.head_dim, want_v != 0, dc.as<int32_t>(), 1, tmp.as<__half>());
+    hip_check(hipStreamSynchronize(stream_), "debug_read_kv");
+    hip_check(hipMemcpy(out, tmp.ptr, kd * 2, hipMemcpyDeviceToHost), "hipMemcpy");
+    return 0;
+}
+
+int Engine::debug_pack(int32_t * tok, int32_t * pos, int32_t * seq, int32_t * cell, int32_t * out_index,
+                       int32_t * last_index, size_t cap_tokens, size_t cap_rows, int32_t * counts) {
+    int32_t c[4];
+    hip_check(hipMemcpy(c, pk_.counts, sizeof(c), hipMemcpyDeviceToHost), "hipMemcpy");
+    std::memcpy(counts, c, sizeof(c));
+    const size_t T = (size_t)c[0];
+    if (T > cap_tokens) {
+        set_error("the token buffers are too small");
+        return -2;
+    }
+    auto get = [&](int32_t * dst, const int32_t * src, size_t n) {
+        if (dst && n) hip_check(hipMemcpy(dst, src, n * 4, hipMemcpyDeviceToHost), "hipMemcpy");
+    };
+    get(tok, pk_.tok, T); get(pos, pk_.pos, T); get(seq, pk_.seq, T); get(cell, pk_.cell, T); get(out_index, pk_.out_index, T);
+    get(last_index, pk_.last_index, std::min(cap_rows, (size_t)cfg_.n_batch));
+    return 0;
+}
+
+int Engine::debug_page_table(int32_t slot, int32_t * out, size_t cap, size_t * out_n) {
+    if (slot < 0 || slot >= (int32_t)cfg_.n_seq_max) {
+        set_error("slot is outside the context's sequence range");
+        return -1;
+    }
+    *out_n = (size_t)max_pages_;
+    if (!out) return 0;
+    if (cap < (size_t)max_pages_) {
+        set_error("the page buffer is too small");
+        return -2;
+    }
+    std::memcpy(out, slots_[(size_t)slot].pages.data(), (size_t)max_pages_ * 4);
+    return 0;
+}
+
+}  // namespace retro

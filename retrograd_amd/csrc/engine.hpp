@@ -1,0 +1,195 @@
+// The engine behind the opaque retro_engine handle: a GGUF model resident in
+// HBM, one paged KV pool, per-request sampler state, and the step that runs
+// one forward pass over a caller-built ragged plan. Mirrors the state the
+// reference keeps in engine_state (crates/retrograd-ffi/runtime/src/
+// retro_engine.cpp:22-74) minus everything that belongs to llama.cpp.
+#pragma once
+
+#include "../../include/retro_step.h"
+#include "gguf_file.hpp"
+#include "kernels.hpp"
+#include "sampler.hpp"
+
+#include <map>
+#include <memory>
+#include <queue>
+#include <string>
+#include <vector>
+
+namespace retro {
+
+void set_error(std::string message);
+void clear_error();
+const std::string & last_error();
+
+// A device allocation released with the object.
+struct DevBuf {
+    void * ptr = nullptr;
+    size_t bytes = 0;
+    DevBuf() = default;
+    ~DevBuf();
+    DevBuf(const DevBuf &) = delete;
+    DevBuf & operator=(const DevBuf &) = delete;
+    DevBuf(DevBuf && o) noexcept : ptr(o.ptr), bytes(o.bytes) { o.ptr = nullptr; o.bytes = 0; }
+    DevBuf & operator=(DevBuf && o) noexcept;
+    void alloc(size_t n);          // frees what it held; n = 0 leaves it empty
+    void ensure(size_t n);         // grows (never shrinks); contents are not kept
+    void release();
+    template <typename T> T * as() const { return (T *)ptr; }
+};
+
+struct HostPinned {
+    void * ptr = nullptr;
+    size_t bytes = 0;
+    ~HostPinned();
+    void ensure(size_t n);
+    template <typename T> T * as() const { return (T *)ptr; }
+};
+
+struct HParams {
+    std::string arch;
+    int n_layer = 0, n_embd = 0, n_head = 0, n_head_kv = 0, head_dim = 0, n_ff = 0, n_vocab = 0;
+    int rope_dim = 0;
+    bool rope_neox = false;
+    float eps = 1e-5f;
+    double rope_base = 10000.0;
+    int n_expert = 0, n_expert_used = 0, n_ff_exp = 0;
+};
+
+struct DevWeight {
+    rk::Weight w;
+    DevBuf buf;
+};
+
+struct LayerWeights {
+    DevBuf attn_norm, ffn_norm, qkv_bias, q_norm, k_norm;
+    std::vector<DevWeight> qkv;    // one fused matrix, or q, k, v separately
+    DevWeight wo;
+    std::vector<DevWeight> gate_up; // one fused matrix, or gate, up separately
+    DevWeight down;
+};
+
+struct Slot {
+    int begin = 0, end = 0;         // resident positions [begin, end)
+    std::vector<int32_t> pages;     // page id per page index (position / PAGE), -1 = none
+};
+
+struct Vocab {
+    std::vector<std::string> pieces;
+    std::vector<int32_t> types;
+    int32_t eos = -1, eot = -1;
+};
+
+class Engine {
+public:
+    Engine(const std::string & path, const retro_engine_config & config);
+    ~Engine();
+
+    // The step; `v2` rows or `v1` rows (exactly one non-null).
+    int step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, size_t n_rows,
+             retro_step_out_row_v2 * out2, retro_step_out_row * out1,
+             int32_t * out_top_ids, float * out_top_logprobs, size_t n_top_stride);
+
+    bool seq_rm(int32_t slot, int32_t p0, int32_t p1);
+    bool seq_cp(int32_t src, int32_t dst, int32_t p0, int32_t p1);
+    int seq_save(int32_t slot, uint32_t flags, uint8_t * buffer, size_t n_buffer, size_t * out_n_bytes);
+    int seq_load(int32_t slot, uint32_t flags, const uint8_t * buffer, size_t n_bytes, size_t * out_n_read);
+    int seq_pos(int32_t slot, int32_t * out_min, int32_t * out_max);
+    int memory(retro_engine_memory_info * out);
+    void request_free(int32_t request) { requests_.erase(request); }
+
+    const retro_engine_config & config() const { return cfg_; }
+    const HParams & hparams() const { return hp_; }
+    const Vocab & vocab() const { return vocab_; }
+    uint32_t context_size() const { return (uint32_t)n_ctx_seq_; }
+    uint64_t weights_version() const { return weights_version_; }
+    uint64_t fingerprint() const { return fingerprint_; }
+    uint64_t steps_run() const { return steps_run_; }
+
+    // Test hooks: copies of device state.
+    int debug_last_logits(float * out, size_t n_floats, size_t * out_rows);
+    int debug_read_kv(int layer, int32_t slot, int32_t pos, int want_v, uint16_t * out);
+    int debug_pack(int32_t * tok, int32_t * pos, int32_t * seq, int32_t * cell, int32_t * out_index,
+                   int32_t * last_index, size_t cap_tokens, size_t cap_rows, int32_t * counts);
+    int debug_page_table(int32_t slot, int32_t * out, size_t cap, size_t * out_n);
+
+private:
+    struct RowView {      // the fields both row versions share
+        int32_t request, slot;
+        const int32_t * tokens;
+        uint32_t n;
+        int32_t pos0;
+        bool sample;
+        const retro_sampling_params_v2 * v2;
+        retro_sampling_params v1;
+        uint32_t n_top;
+        bool want_logprob;
+        int32_t adapter;
+    };
+
+    void load_model(const std::string & path);
+    void upload_weight(const TensorInfo & t, int64_t K, int64_t N, const uint8_t * data, size_t bytes,
+                       bool keep_raw, DevWeight & out);
+    void upload_fused(const std::vector<const TensorInfo *> & parts, std::vector<DevWeight> & out);
+    void upload_f32(const TensorInfo * t, DevBuf & out, size_t expect);
+    void build_buffers();
+
+    int32_t alloc_page();
+    void release_page(int32_t page);
+    void copy_page(int32_t src, int32_t dst);
+    void set_page(int32_t slot, int idx, int32_t page);
+    void clear_slot(Slot & s, int32_t slot);
+    void forward(int T, int n_out, int n_tiles, int n_items);
+
+    retro_engine_config cfg_ {};
+    HParams hp_;
+    Vocab vocab_;
+    uint64_t fingerprint_ = 0;
+    uint64_t weights_version_ = 0;
+    uint64_t steps_run_ = 0;
+    int n_ctx_seq_ = 0;
+    int max_pages_ = 0;       // page indices per slot
+    int n_pages_ = 0;         // pages in the pool
+    int qt_ = 1;              // query tokens per attention tile
+
+    hipStream_t stream_ = nullptr;
+
+    // weights
+    DevWeight tok_embd_;      // raw rows, gathered per token
+    DevWeight lm_head_;
+    DevBuf out_norm_, out_bias_;
+    std::vector<LayerWeights> layers_;
+    DevBuf inv_freq_;         // double[rope_dim/2]
+
+    // KV
+    std::vector<DevBuf> k_pool_, v_pool_;   // per layer
+    DevBuf table_;                          // int32 [n_seq_max][max_pages]
+    std::vector<Slot> slots_;
+    std::vector<int32_t> page_ref_;
+    std::priority_queue<int32_t, std::vector<int32_t>, std::greater<int32_t>> free_pages_;
+    std::vector<rk::TableUpdate> pending_updates_;
+
+    // per-step device buffers
+    DevBuf d_stage_;          // rows | tokens | table updates, as uploaded
+    HostPinned h_stage_;
+    rk::PackBuffers pk_ {};
+    std::vector<DevBuf> pk_store_;
+    DevBuf x_, qkv_, gu_, q_half_, partial_, logits_, sample_k_, sample_out_, out_rows_idx_;
+    DevBuf act_e_x_, act_e_hi_, act_e_lo_;       // n_embd wide
+    DevBuf act_q_x_, act_q_hi_, act_q_lo_;       // n_head * head_dim wide
+    DevBuf act_f_x_, act_f_hi_, act_f_lo_;       // n_ff wide
+    DevBuf act_o_x_, act_o_hi_, act_o_lo_;       // output rows, n_embd wide
+    HostPinned h_sample_, h_logits_;
+    int last_n_out_ = 0;
+
+    std::map<int32_t, RequestState> requests_;
+    sampling::FullScratch scratch_;
+};
+
+}  // namespace retro
+
+// The opaque handle of the C ABI.
+struct retro_engine {
+    retro::Engine impl;
+    retro_engine(const std::string & path, const retro_engine_config & config) : impl(path, config) {}
+};

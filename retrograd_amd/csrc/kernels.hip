@@ -1,0 +1,1269 @@
+// gfx950 (CDNA4, wave64) kernels of the batched decode step.
+//
+// Data layouts (all chosen for this hardware, none inherited from GGUF beyond
+// the bits of each quantised block):
+//
+//  * Weight tiles. A quantised matrix [N][K] (K % 256 == 0, N % 16 == 0) is cut
+//    into tiles of 16 rows x 256 columns. A tile stores first one 16-byte
+//    header per row, then the quantised payload ordered so that lane l of a
+//    wave reads 16 contiguous bytes at offset l*16 of each 1 KiB load:
+//      Q4_K  2304 B = 16 x (d, dmin, scales[12]) + 2 loads;  lane (r = l%16,
+//            g = l/16) of load h holds, as 4 dwords, the 8 nibbles of
+//            elements 32*(4h+j) + 8g .. +8 of row r, j = 0..3. Inside a dword
+//            the nibbles are ordered e0 e2 e4 e6 | e1 e3 e5 e7 so that masking
+//            with 0x000F000F / 0x00F000F0 yields f16 pairs in natural order.
+//      Q8_0  4352 B = 16 x scales[8] (f16) + 4 loads; lane (r, g) of load q
+//            holds elements 32*(2q)+8g..+8 and 32*(2q+1)+8g..+8 of row r.
+//    The byte count equals the GGUF byte count of the same matrix.
+//
+//  * KV pages. A page holds 32 positions of one sequence for one kv head:
+//      K: [dims/32][token half (2)][g (4)][token (16)][8 halves]   - the A operand
+//         of a 16x16x32 MFMA (row = token, k = 8 dims) is one 16-byte load/lane
+//      V: [dims/16][g (4)][dim (16)][8 halves] holding, for k-slot (g, i), the
+//         token 4g+i (i < 4) or 16+4g+(i-4) (i >= 4): exactly the tokens whose
+//         scores lane group g owns after the QK^T MFMAs, so P feeds the PV MFMA
+//         without any cross-lane movement.
+//
+// MFMA operand convention used throughout (v_mfma_f32_16x16x32_f16): lane l
+// supplies row/column l%16 and k-slots (l/16, 0..7) of both operands; the
+// result holds rows 4*(l/16)+i, column l%16. Both operands always use the same
+// (lane group, slot) for the same logical k, so the hardware's internal k
+// order never matters.
+#include "kernels.hpp"
+
+#include <stdexcept>
+#include <string>
+
+namespace rk {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+#define HIP_OK(expr)                                                                        \
+    do {                                                                                    \
+        hipError_t err__ = (expr);                                                          \
+        if (err__ != hipSuccess)                                                            \
+            throw std::runtime_error(std::string("HIP error: ") + hipGetErrorString(err__)  \
+                                     + " at " #expr);                                       \
+    } while (0)
+
+static inline void check_launch(const char * what) {
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess)
+        throw std::runtime_error(std::string("kernel launch failed (") + what + "): " + hipGetErrorString(err));
+}
+
+BlockGeom geom_of(int type) {
+    switch (type) {
+        case WT_F32:   return {1, 4};
+        case WT_F16:   return {1, 2};
+        case WT_BF16:  return {1, 2};
+        case WT_Q8_0:  return {32, 34};
+        case WT_MXFP4: return {32, 17};
+        case WT_Q4_K:  return {256, 144};
+        default: throw std::runtime_error("unsupported tensor type " + std::to_string(type));
+    }
+}
+
+size_t row_bytes(int type, int64_t k) {
+    const BlockGeom g = geom_of(type);
+    if (k % g.elements != 0) throw std::runtime_error("row length is not a whole number of blocks");
+    return (size_t)(k / g.elements) * g.bytes;
+}
+
+bool can_pack(int type, int64_t K, int64_t N) {
+    return (type == WT_Q4_K || type == WT_Q8_0) && K % 256 == 0 && N % 16 == 0 && K > 0 && N > 0;
+}
+
+// ---------------------------------------------------------------------------
+// small device helpers
+
+__device__ __forceinline__ float h2f(uint16_t bits) {
+    return __half2float(__ushort_as_half(bits));
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// f32 -> f16 with saturation, so nothing non-finite is ever stored.
+__device__ __forceinline__ __half sat_half(float v) {
+    v = fminf(fmaxf(v, -65504.0f), 65504.0f);
+    return __float2half_rn(v);
+}
+
+// One element of a raw GGUF row, decoded exactly as the stored blocks define
+// it (two roundings for d*q - m, no contraction).
+__device__ float decode_elem(int type, const uint8_t * row, int k) {
+    switch (type) {
+        case WT_F32: return ((const float *)row)[k];
+        case WT_F16: return h2f(((const uint16_t *)row)[k]);
+        case WT_BF16: return __uint_as_float((uint32_t)((const uint16_t *)row)[k] << 16);
+        case WT_Q8_0: {
+            const uint8_t * b = row + (size_t)(k >> 5) * 34;
+            const float d = h2f(*(const uint16_t *)b);
+            return __fmul_rn(d, (float)(int8_t)b[2 + (k & 31)]);
+        }
+        case WT_MXFP4: {
+            const uint8_t * b = row + (size_t)(k >> 5) * 17;
+            const int e = k & 31;
+            const uint8_t byte = b[1 + (e & 15)];
+            const int code = e < 16 ? (byte & 0x0f) : (byte >> 4);
+            const int mag = code & 7;
+            // doubled E2M1 magnitudes 0 1 2 3 4 6 8 12
+            const int dv = mag < 4 ? mag : (mag == 4 ? 4 : (mag == 5 ? 6 : (mag == 6 ? 8 : 12)));
+            const uint8_t x = b[0];
+            const uint32_t bits = x == 0 ? 0x00200000u : (x == 1 ? 0x00400000u : ((uint32_t)x - 1) << 23);
+            const float d = __uint_as_float(bits);
+            return __fmul_rn(d, (float)((code & 8) ? -dv : dv));
+        }
+        case WT_Q4_K: {
+            const uint8_t * b = row + (size_t)(k >> 8) * 144;
+            const int e = k & 255;
+            const int j = e >> 5;
+            const uint8_t * sc = b + 4;
+            int s, m;
+            if (j < 4) {
+                s = sc[j] & 63;
+                m = sc[j + 4] & 63;
+            } else {
+                s = (sc[j + 4] & 0x0f) | ((sc[j - 4] >> 6) << 4);
+                m = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4);
+            }
+            const uint8_t byte = b[16 + (e >> 6) * 32 + (e & 31)];
+            const int q = (e & 32) ? (byte >> 4) : (byte & 0x0f);
+            const float d = h2f(*(const uint16_t *)b);
+            const float dmin = h2f(*(const uint16_t *)(b + 2));
+            return __fsub_rn(__fmul_rn(__fmul_rn(d, (float)s), (float)q), __fmul_rn(dmin, (float)m));
+        }
+        default: return 0.0f;
+    }
+}
+
+// Writes up to 32 consecutive activations of one row as f16 and, for a whole
+// block, the sum of the rounded values as hi + lo halves.
+__device__ __forceinline__ void store_act_block(const float * v, int count, __half * x, __half * hi, __half * lo) {
+    float sum = 0.0f;
+    for (int i = 0; i < count; ++i) {
+        const __half h = sat_half(v[i]);
+        x[i] = h;
+        sum += __half2float(h);
+    }
+    if (hi && count == 32) {
+        const __half a = sat_half(sum);
+        *hi = a;
+        *lo = __float2half_rn(sum - __half2float(a));
+    }
+}
+
+// ---------------------------------------------------------------------------
+// weight repacking (runs once per tensor at load)
+
+__global__ void k_repack_q4k(const uint8_t * __restrict__ raw, uint8_t * __restrict__ dst, int nsb, int n_tiles) {
+    // one thread per output dword: 576 dwords per (tile, super-block)
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = (size_t)n_tiles * nsb * 576;
+    if (gid >= total) return;
+    const int w = (int)(gid % 576);
+    const size_t ts = gid / 576;
+    const int sb = (int)(ts % nsb);
+    const size_t rt = ts / nsb;
+    uint32_t out;
+    if (w < 64) {                       // headers: row r, dword j
+        const int r = w >> 2, j = w & 3;
+        const uint8_t * blk = raw + ((rt * 16 + r) * nsb + sb) * 144;
+        out = *(const uint32_t *)(blk + 4 * j);
+    } else {
+        const int v = w - 64;           // 0..511
+        const int h = v >> 8;           // load
+        const int lane = (v >> 2) & 63;
+        const int j = v & 3;
+        const int r = lane & 15, g = lane >> 4;
+        const uint8_t * blk = raw + ((rt * 16 + r) * nsb + sb) * 144;
+        const int s = 4 * h + j;        // sub-block
+        uint32_t nib[8];
+        for (int i = 0; i < 8; ++i) {
+            const int e = 32 * s + 8 * g + i;
+            const uint8_t byte = blk[16 + (e >> 6) * 32 + (e & 31)];
+            nib[i] = (e & 32) ? (byte >> 4) : (byte & 0x0f);
+        }
+        out = nib[0] | (nib[2] << 4) | (nib[4] << 8) | (nib[6] << 12)
+            | (nib[1] << 16) | (nib[3] << 20) | (nib[5] << 24) | (nib[7] << 28);
+    }
+    *(uint32_t *)(dst + ts * 2304 + (size_t)w * 4) = out;
+}
+
+__global__ void k_repack_q8_0(const uint8_t * __restrict__ raw, uint8_t * __restrict__ dst, int nsb, int n_tiles) {
+    // 1088 dwords per (tile, group of 8 blocks): 64 header + 1024 payload
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = (size_t)n_tiles * nsb * 1088;
+    if (gid >= total) return;
+    const int w = (int)(gid % 1088);
+    const size_t ts = gid / 1088;
+    const int sb = (int)(ts % nsb);
+    const size_t rt = ts / nsb;
+    uint32_t out;
+    if (w < 64) {                       // row r, scales 2j and 2j+1
+        const int r = w >> 2, j = w & 3;
+        const uint8_t * row = raw + (rt * 16 + r) * (size_t)nsb * 272 + (size_t)sb * 272;
+        const uint32_t a = *(const uint16_t *)(row + (2 * j) * 34);
+        const uint32_t b = *(const uint16_t *)(row + (2 * j + 1) * 34);
+        out = a | (b << 16);
+    } else {
+        const int v = w - 64;           // 0..1023
+        const int q = v >> 8;           // load 0..3
+        const int lane = (v >> 2) & 63;
+        const int j = v & 3;            // dword within the 16 bytes
+        const int r = lane & 15, g = lane >> 4;
+        const int blk = 2 * q + (j >> 1);
+        const int e0 = 8 * g + 4 * (j & 1);
+        const uint8_t * p = raw + (rt * 16 + r) * (size_t)nsb * 272 + (size_t)sb * 272 + (size_t)blk * 34 + 2 + e0;
+        out = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+    }
+    *(uint32_t *)(dst + ts * 4352 + (size_t)w * 4) = out;
+}
+
+void repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int K, int N) {
+    if (!can_pack(type, K, N)) throw std::runtime_error("repack: shape or type has no tile layout");
+    const int nsb = K / 256, n_tiles = N / 16;
+    const size_t per = type == WT_Q4_K ? 576 : 1088;
+    const size_t total = (size_t)n_tiles * nsb * per;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (type == WT_Q4_K) hipLaunchKernelGGL(k_repack_q4k, dim3(blocks), dim3(256), 0, s, raw, packed, nsb, n_tiles);
+    else hipLaunchKernelGGL(k_repack_q8_0, dim3(blocks), dim3(256), 0, s, raw, packed, nsb, n_tiles);
+    check_launch("repack");
+}
+
+// ---------------------------------------------------------------------------
+// matmul over tiled quantised weights (MFMA)
+
+struct MMArgs {
+    const uint8_t * w;
+    const __half * x;
+    const __half * xs_hi;
+    const __half * xs_lo;
+    float * y;
+    const float * bias;
+    int K, N, T, ldy, col0, mode;
+    int n_row_tiles;
+    int ksplit;       // waves of a workgroup that share one row tile along K (1, 2 or 4)
+};
+
+__device__ __forceinline__ h8 load_h8(const __half * p) {
+    return *(const h8 *)p;
+}
+
+template <int NT>
+__device__ __forceinline__ void mm_finish(const MMArgs & a, f4 (&acc)[NT], int rt, int tbase, int nt,
+                                          int wk, int wr, float * lds) {
+    const int lane = threadIdx.x & 63;
+    const int r = lane & 15, g = lane >> 4;
+    if (a.ksplit > 1) {
+        // lds[(wk-1)][wr][tile*4+i][lane]
+        const int rows_per_wg = 4 / a.ksplit;
+        if (wk > 0) {
+            float * dst = lds + ((size_t)((wk - 1) * rows_per_wg + wr) * NT * 4) * 64;
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) dst[(t * 4 + i) * 64 + lane] = acc[t][i];
+        }
+        __syncthreads();
+        if (wk > 0) return;
+        for (int k = 1; k < a.ksplit; ++k) {
+            const float * src = lds + ((size_t)((k - 1) * rows_per_wg + wr) * NT * 4) * 64;
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[t][i] += src[(t * 4 + i) * 64 + lane];
+        }
+    }
+    if (rt >= a.n_row_tiles) return;
+    const int n = rt * 16 + r;
+    const float bias = a.bias ? a.bias[n] : 0.0f;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        if (t >= nt) break;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int tok = tbase + t * 16 + 4 * g + i;
+            if (tok < a.T) {
+                float * p = a.y + (size_t)tok * a.ldy + a.col0 + n;
+                const float v = acc[t][i] + bias;
+                *p = a.mode == MM_ADD ? *p + v : v;
+            }
+        }
+    }
+}
+
+template <int NT>
+__global__ __launch_bounds__(256) void k_mm_q4k(MMArgs a) {
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int wr = wave / a.ksplit, wk = wave % a.ksplit;
+    const int rt = blockIdx.x * (4 / a.ksplit) + wr;
+    const int tbase = blockIdx.y * 64;
+    const int nt = min(NT, (a.T - tbase + 15) >> 4);
+    const int nsb = a.K >> 8;
+    const int nblk = a.K >> 5;
+
+    f4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = (f4){0.f, 0.f, 0.f, 0.f};
+
+    // activation row of this lane for every token tile (clamped: rows past T
+    // are computed on the last row and never stored)
+    const __half * xrow[NT];
+    const __half * shi[NT];
+    const __half * slo[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int tok = min(tbase + t * 16 + r, a.T - 1);
+        xrow[t] = a.x + (size_t)tok * a.K + 8 * g;
+        shi[t] = a.xs_hi + (size_t)tok * nblk;
+        slo[t] = a.xs_lo + (size_t)tok * nblk;
+    }
+
+    if (rt < a.n_row_tiles) {
+        for (int sb = wk; sb < nsb; sb += a.ksplit) {
+            const uint8_t * tile = a.w + ((size_t)rt * nsb + sb) * 2304;
+            const u4 hdr = *(const u4 *)(tile + r * 16);
+            const u4 q0 = *(const u4 *)(tile + 256 + lane * 16);
+            const u4 q1 = *(const u4 *)(tile + 1280 + lane * 16);
+            const float d = h2f((uint16_t)(hdr.x & 0xffff));
+            const float dmin = h2f((uint16_t)(hdr.x >> 16));
+            // scales[12] = bytes of hdr.y, hdr.z, hdr.w
+            uint32_t sc[8], mn[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t lo_b = (hdr.y >> (8 * j)) & 0xff;   // scales[j]
+                const uint32_t md_b = (hdr.z >> (8 * j)) & 0xff;   // scales[j+4]
+                const uint32_t hi_b = (hdr.w >> (8 * j)) & 0xff;   // scales[j+8]
+                sc[j] = lo_b & 63;
+                mn[j] = md_b & 63;
+                sc[j + 4] = (hi_b & 0x0f) | ((lo_b >> 6) << 4);
+                mn[j + 4] = (hi_b >> 4) | ((md_b >> 6) << 4);
+            }
+            f4 accq[NT], accm[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                accq[t] = (f4){0.f, 0.f, 0.f, 0.f};
+                accm[t] = (f4){0.f, 0.f, 0.f, 0.f};
+            }
+            // min term: sum_s m[r][s] * xsum[t][s], k-slots (g=0: hi sums, g=1: lo sums)
+            {
+                h8 mB;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) mB[i] = g < 2 ? (_Float16)(float)mn[i] : (_Float16)0.0f;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    if (t >= nt) break;
+                    h8 sA = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+                    if (g == 0) sA = load_h8(shi[t] + sb * 8);
+                    else if (g == 1) sA = load_h8(slo[t] + sb * 8);
+                    accm[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(sA, mB, accm[t], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const uint32_t wq = s < 4 ? q0[s & 3] : q1[s & 3];
+                const _Float16 sch = (_Float16)(float)sc[s];
+                const h2 k1 = {sch, sch};
+                const h2 c1 = k1 * (_Float16)(-1024.0f);        // exact: sc <= 63
+                const h2 k2 = k1 * (_Float16)(0.0625f);         // exact
+                const h2 c2 = k1 * (_Float16)(-64.0f);          // exact
+                const uint32_t w8 = wq >> 8;
+                const h2 u0 = __builtin_bit_cast(h2, (wq & 0x000F000Fu) | 0x64006400u);   // 1024 + e0, e1
+                const h2 u1 = __builtin_bit_cast(h2, (wq & 0x00F000F0u) | 0x64006400u);   // 1024 + 16*(e2, e3)
+                const h2 u2 = __builtin_bit_cast(h2, (w8 & 0x000F000Fu) | 0x64006400u);
+                const h2 u3 = __builtin_bit_cast(h2, (w8 & 0x00F000F0u) | 0x64006400u);
+                // fused multiply-add: (1024 + e) * sc - 1024 * sc == sc * e exactly (<= 945)
+                const h2 a0 = __builtin_elementwise_fma(u0, k1, c1);
+                const h2 a1 = __builtin_elementwise_fma(u1, k2, c2);
+                const h2 a2 = __builtin_elementwise_fma(u2, k1, c1);
+                const h2 a3 = __builtin_elementwise_fma(u3, k2, c2);
+                const h8 B = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    if (t >= nt) break;
+                    const h8 A = load_h8(xrow[t] + sb * 256 + s * 32);
+                    accq[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, accq[t], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[t][i] = fmaf(-dmin, accm[t][i], fmaf(d, accq[t][i], acc[t][i]));
+        }
+    }
+    mm_finish<NT>(a, acc, rt, tbase, nt, wk, wr, lds);
+}
+
+template <int NT>
+__global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
+    extern __shared__ float lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int wr = wave / a.ksplit, wk = wave % a.ksplit;
+    const int rt = blockIdx.x * (4 / a.ksplit) + wr;
+    const int tbase = blockIdx.y * 64;
+    const int nt = min(NT, (a.T - tbase + 15) >> 4);
+    const int nsb = a.K >> 8;
+
+    f4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = (f4){0.f, 0.f, 0.f, 0.f};
+    const __half * xrow[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        const int tok = min(tbase + t * 16 + r, a.T - 1);
+        xrow[t] = a.x + (size_t)tok * a.K + 8 * g;
+    }
+    const h2 bias1152 = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
+
+    if (rt < a.n_row_tiles) {
+        for (int sb = wk; sb < nsb; sb += a.ksplit) {
+            const uint8_t * tile = a.w + ((size_t)rt * nsb + sb) * 4352;
+            const u4 hdr = *(const u4 *)(tile + r * 16);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const u4 d4 = *(const u4 *)(tile + 256 + q * 1024 + lane * 16);
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int s = 2 * q + half;
+                    const uint32_t sw = hdr[s >> 1];
+                    const float d = h2f((uint16_t)((s & 1) ? (sw >> 16) : (sw & 0xffff)));
+                    // bytes are two's complement; flipping the sign bit gives q + 128 in
+                    // 0..255, and 0x6400 | b is the f16 1024 + b: subtract 1152 for q.
+                    const uint32_t w0 = d4[2 * half] ^ 0x80808080u;
+                    const uint32_t w1 = d4[2 * half + 1] ^ 0x80808080u;
+                    const h2 u0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u));
+                    const h2 u1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u));
+                    const h2 u2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u));
+                    const h2 u3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u));
+                    const h2 a0 = u0 + bias1152, a1 = u1 + bias1152, a2 = u2 + bias1152, a3 = u3 + bias1152;
+                    const h8 B = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        if (t >= nt) break;
+                        const h8 A = load_h8(xrow[t] + sb * 256 + s * 32);
+                        const f4 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) acc[t][i] = fmaf(d, part[i], acc[t][i]);
+                    }
+                }
+            }
+        }
+    }
+    mm_finish<NT>(a, acc, rt, tbase, nt, wk, wr, lds);
+}
+
+// Any type, any shape: one wave per output feature, raw GGUF rows.
+__global__ __launch_bounds__(256) void k_mm_generic(int type, const uint8_t * __restrict__ raw, size_t rb,
+                                                    const __half * __restrict__ x, int K, int N, int T,
+                                                    float * y, int ldy, int col0, int mode, const float * bias) {
+    const int lane = threadIdx.x & 63;
+    const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    const uint8_t * row = raw + (size_t)n * rb;
+    for (int t0 = 0; t0 < T; t0 += 8) {
+        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int k = lane; k < K; k += 64) {
+            const float w = decode_elem(type, row, k);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int t = min(t0 + j, T - 1);
+                acc[j] = fmaf(w, __half2float(x[(size_t)t * K + k]), acc[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float v = wave_sum(acc[j]);
+            if (lane == 0 && t0 + j < T) {
+                float * p = y + (size_t)(t0 + j) * ldy + col0 + n;
+                const float o = v + (bias ? bias[n] : 0.0f);
+                *p = mode == MM_ADD ? *p + o : o;
+            }
+        }
+    }
+}
+
+void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                    int mode, const float * bias) {
+    if (!w.raw) throw std::runtime_error("matmul_generic: the weight has no raw layout");
+    if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
+    if (T <= 0) return;
+    hipLaunchKernelGGL(k_mm_generic, dim3((w.N + 3) / 4), dim3(256), 0, s, w.type, w.raw, row_bytes(w.type, w.K),
+                       x.x, w.K, w.N, T, y, ldy, col0, mode, bias);
+    check_launch("matmul_generic");
+}
+
+template <int NT>
+static void launch_mm(hipStream_t s, int type, const MMArgs & a, dim3 grid, size_t lds) {
+    if (type == WT_Q4_K) hipLaunchKernelGGL(k_mm_q4k<NT>, grid, dim3(256), lds, s, a);
+    else hipLaunchKernelGGL(k_mm_q8_0<NT>, grid, dim3(256), lds, s, a);
+}
+
+void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+            int mode, const float * bias) {
+    if (T <= 0) return;
+    if (!w.packed) {
+        matmul_generic(s, w, x, T, y, ldy, col0, mode, bias);
+        return;
+    }
+    if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
+    if (w.type == WT_Q4_K && (!x.xs_hi || !x.xs_lo)) throw std::runtime_error("matmul: Q4_K needs block sums");
+    MMArgs a;
+    a.w = w.packed; a.x = x.x; a.xs_hi = x.xs_hi; a.xs_lo = x.xs_lo; a.y = y; a.bias = bias;
+    a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
+    a.n_row_tiles = w.N / 16;
+    // Enough waves to cover the chip: split K across the waves of a workgroup
+    // when there are few row tiles.
+    const int nsb = w.K / 256;
+    int ksplit = 1;
+    if (a.n_row_tiles < 1024 && nsb >= 8) ksplit = 4;
+    else if (a.n_row_tiles < 2048 && nsb >= 4) ksplit = 2;
+    a.ksplit = ksplit;
+    const int rows_per_wg = 4 / ksplit;
+    dim3 grid((a.n_row_tiles + rows_per_wg - 1) / rows_per_wg, (T + 63) / 64);
+    const int nt = T >= 49 ? 4 : (T + 15) / 16;
+    const size_t lds = ksplit > 1 ? (size_t)(ksplit - 1) * rows_per_wg * nt * 4 * 64 * sizeof(float) : 0;
+    switch (nt) {
+        case 1: launch_mm<1>(s, w.type, a, grid, lds); break;
+        case 2: launch_mm<2>(s, w.type, a, grid, lds); break;
+        case 3: launch_mm<3>(s, w.type, a, grid, lds); break;
+        default: launch_mm<4>(s, w.type, a, grid, lds); break;
+    }
+    check_launch("matmul");
+}
+
+// ---------------------------------------------------------------------------
+// embedding, RMSNorm, SwiGLU
+
+__global__ void k_embed(int type, const uint8_t * __restrict__ raw, size_t rb, const int32_t * __restrict__ tok,
+                        int E, float * __restrict__ x) {
+    const int t = blockIdx.y;
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= E) return;
+    x[(size_t)t * E + k] = decode_elem(type, raw + (size_t)tok[t] * rb, k);
+}
+
+void embed(hipStream_t s, const Weight & emb, const int32_t * tok, int T, float * x) {
+    if (!emb.raw) throw std::runtime_error("embed: the embedding has no raw layout");
+    if (T <= 0) return;
+    hipLaunchKernelGGL(k_embed, dim3((emb.K + 255) / 256, T), dim3(256), 0, s, emb.type, emb.raw,
+                       row_bytes(emb.type, emb.K), tok, emb.K, x);
+    check_launch("embed");
+}
+
+__global__ __launch_bounds__(256) void k_rmsnorm_act(const float * __restrict__ x, const float * __restrict__ w,
+                                                     int E, float eps, const int32_t * __restrict__ rows, Act out) {
+    __shared__ float red[4];
+    const int o = blockIdx.x;
+    const float * xr = x + (size_t)(rows ? rows[o] : o) * E;
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < E; i += 256) ss += xr[i] * xr[i];
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    const float scale = 1.0f / sqrtf(total / (float)E + eps);
+    const int nblk = (E + 31) / 32;
+    for (int b = threadIdx.x; b < nblk; b += 256) {
+        const int k0 = b * 32;
+        const int count = min(32, E - k0);
+        float v[32];
+        for (int i = 0; i < count; ++i) v[i] = (xr[k0 + i] * scale) * w[k0 + i];
+        store_act_block(v, count, out.x + (size_t)o * E + k0,
+                        out.xs_hi ? out.xs_hi + (size_t)o * (E / 32) + b : nullptr,
+                        out.xs_lo ? out.xs_lo + (size_t)o * (E / 32) + b : nullptr);
+    }
+}
+
+void rmsnorm_act(hipStream_t s, const float * x, const float * w, int E, float eps,
+                 const int32_t * rows, int n_rows, const Act & out) {
+    if (n_rows <= 0) return;
+    Act o = out;
+    if (E % 32 != 0) { o.xs_hi = nullptr; o.xs_lo = nullptr; }
+    hipLaunchKernelGGL(k_rmsnorm_act, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, o);
+    check_launch("rmsnorm");
+}
+
+__global__ __launch_bounds__(256) void k_swiglu_act(const float * __restrict__ gu, int T, int F, Act out) {
+    const int nblk = (F + 31) / 32;
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (size_t)T * nblk) return;
+    const int t = (int)(gid / nblk), b = (int)(gid % nblk);
+    const int k0 = b * 32;
+    const int count = min(32, F - k0);
+    const float * g = gu + (size_t)t * 2 * F + k0;
+    const float * u = g + F;
+    float v[32];
+    for (int i = 0; i < count; ++i) {
+        const float gi = g[i];
+        v[i] = (gi / (1.0f + __expf(-gi))) * u[i];
+    }
+    store_act_block(v, count, out.x + (size_t)t * F + k0,
+                    out.xs_hi ? out.xs_hi + (size_t)t * (F / 32) + b : nullptr,
+                    out.xs_lo ? out.xs_lo + (size_t)t * (F / 32) + b : nullptr);
+}
+
+__global__ __launch_bounds__(256) void k_to_act(const float * __restrict__ x, int T, int K, Act out) {
+    const int nblk = (K + 31) / 32;
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (size_t)T * nblk) return;
+    const int t = (int)(gid / nblk), b = (int)(gid % nblk);
+    const int k0 = b * 32;
+    const int count = min(32, K - k0);
+    float v[32];
+    for (int i = 0; i < count; ++i) v[i] = x[(size_t)t * K + k0 + i];
+    store_act_block(v, count, out.x + (size_t)t * K + k0,
+                    out.xs_hi ? out.xs_hi + (size_t)t * (K / 32) + b : nullptr,
+                    out.xs_lo ? out.xs_lo + (size_t)t * (K / 32) + b : nullptr);
+}
+
+void to_act(hipStream_t s, const float * x, int T, int K, const Act & out) {
+    if (T <= 0) return;
+    Act o = out;
+    if (K % 32 != 0) { o.xs_hi = nullptr; o.xs_lo = nullptr; }
+    const size_t n = (size_t)T * ((K + 31) / 32);
+    hipLaunchKernelGGL(k_to_act, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, T, K, o);
+    check_launch("to_act");
+}
+
+void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out) {
+    if (T <= 0) return;
+    Act o = out;
+    if (F % 32 != 0) { o.xs_hi = nullptr; o.xs_lo = nullptr; }
+    const size_t n = (size_t)T * ((F + 31) / 32);
+    hipLaunchKernelGGL(k_swiglu_act, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, T, F, o);
+    check_launch("swiglu");
+}
+
+// ---------------------------------------------------------------------------
+// step packing
+
+__device__ __forceinline__ int tile_splits(int kv_begin, int kv_hi) {
+    const int p_first = kv_begin / PAGE;
+    const int p_last = (kv_hi - 1) / PAGE;
+    return (p_last - p_first + 1 + SPLIT_PAGES - 1) / SPLIT_PAGES;
+}
+
+// Inclusive scan of one int per thread over a 1024-thread block.
+__device__ int block_scan_incl(int v, int * scratch) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int o = 1; o < 64; o <<= 1) {
+        const int n = __shfl_up(v, o, 64);
+        if (lane >= o) v += n;
+    }
+    if (lane == 63) scratch[wave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int i = 0; i < 16; ++i) { const int c = scratch[i]; scratch[i] = run; run += c; }
+    }
+    __syncthreads();
+    v += scratch[wave];
+    __syncthreads();
+    return v;
+}
+
+__global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows, int n_rows,
+                                               const int32_t * __restrict__ toks,
+                                               const TableUpdate * __restrict__ upd, int n_upd,
+                                               int32_t * __restrict__ table, int max_pages,
+                                               int qt, int n_kv, const double * __restrict__ inv_freq, int pairs,
+                                               PackBuffers o) {
+    __shared__ int scratch[16];
+    __shared__ int carry[3];
+    for (int i = threadIdx.x; i < n_upd; i += 1024) table[(size_t)upd[i].slot * max_pages + upd[i].index] = upd[i].page;
+    if (threadIdx.x == 0) { carry[0] = 0; carry[1] = 0; carry[2] = 0; }
+    __syncthreads();
+
+    // rows in chunks of 1024: per-row tile / item / output counts -> bases
+    for (int base = 0; base < n_rows; base += 1024) {
+        const int r = base + threadIdx.x;
+        int tiles = 0, items = 0, outs = 0;
+        RowDesc d;
+        if (r < n_rows) {
+            d = rows[r];
+            tiles = (d.n + qt - 1) / qt;
+            for (int j = 0; j < tiles; ++j) {
+                const int hi = d.pos0 + min(d.n, (j + 1) * qt);
+                items += n_kv * tile_splits(d.kv_begin, hi);
+            }
+            outs = d.sample ? 1 : 0;
+        }
+        const int tile_end = block_scan_incl(tiles, scratch);
+        const int item_end = block_scan_incl(items, scratch);
+        const int out_end = block_scan_incl(outs, scratch);
+        if (r < n_rows) {
+            int tile_at = carry[0] + tile_end - tiles;
+            int item_at = carry[1] + item_end - items;
+            const int out_at = carry[2] + out_end - outs;
+            o.row_offset[r] = d.tok_off;
+            o.last_index[r] = d.tok_off + d.n - 1;
+            if (d.sample) o.out_tok[out_at] = d.tok_off + d.n - 1;
+            for (int j = 0; j < tiles; ++j) {
+                const int q0 = j * qt;
+                const int nq = min(qt, d.n - q0);
+                const int hi = d.pos0 + q0 + nq;
+                const int ns = tile_splits(d.kv_begin, hi);
+                o.tile_t0[tile_at] = d.tok_off + q0;
+                o.tile_nq[tile_at] = nq;
+                o.tile_item0[tile_at] = item_at;
+                o.tile_nsplit[tile_at] = ns;
+                o.tile_page0[tile_at] = d.kv_begin / PAGE;
+                o.tile_kv_begin[tile_at] = d.kv_begin;
+                for (int i = 0; i < nq; ++i) o.tok_tile[d.tok_off + q0 + i] = tile_at;
+                item_at += n_kv * ns;
+                ++tile_at;
+            }
+            for (int i = 0; i < d.n; ++i) {
+                const int t = d.tok_off + i;
+                const int p = d.pos0 + i;
+                o.tok[t] = toks[t];
+                o.pos[t] = p;
+                o.seq[t] = d.slot;
+                o.row[t] = r;
+                o.cell[t] = table[(size_t)d.slot * max_pages + p / PAGE] * PAGE + p % PAGE;
+                o.out_index[t] = (d.sample && i + 1 == d.n) ? out_at : -1;
+            }
+        }
+        __syncthreads();
+        // rows past n_rows contribute zero, so the last thread's inclusive
+        // sums are the chunk totals
+        if (threadIdx.x == 1023) {
+            carry[0] += tile_end;
+            carry[1] += item_end;
+            carry[2] += out_end;
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const RowDesc last = rows[n_rows - 1];
+        o.row_offset[n_rows] = last.tok_off + last.n;
+        o.counts[0] = last.tok_off + last.n;
+        o.counts[1] = carry[2];
+        o.counts[2] = carry[0];
+        o.counts[3] = carry[1];
+    }
+    // rotary table of the step: angle = pos * base^(-2i/d) in double
+    const RowDesc lastd = rows[n_rows - 1];
+    const int T = lastd.tok_off + lastd.n;
+    for (int i = threadIdx.x; i < T * pairs; i += 1024) {
+        const int t = i / pairs, j = i % pairs;
+        // position of token t: recompute from its row (binary search over tok_off)
+        int lo = 0, hi = n_rows - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (rows[mid].tok_off <= t) lo = mid; else hi = mid - 1;
+        }
+        const double ang = (double)(rows[lo].pos0 + (t - rows[lo].tok_off)) * inv_freq[j];
+        double sv, cv;
+        sincos(ang, &sv, &cv);
+        o.rope_cos[i] = (float)cv;
+        o.rope_sin[i] = (float)sv;
+    }
+}
+
+void pack_step(hipStream_t s, const RowDesc * rows, int n_rows, const int32_t * tokens_concat,
+               const TableUpdate * updates, int n_updates, int32_t * table, int max_pages,
+               int qt, int n_kv_heads, const double * inv_freq, int rope_pairs, const PackBuffers & out) {
+    if (n_rows <= 0) return;
+    hipLaunchKernelGGL(k_pack, dim3(1), dim3(1024), 0, s, rows, n_rows, tokens_concat, updates, n_updates,
+                       table, max_pages, qt, n_kv_heads, inv_freq, rope_pairs, out);
+    check_launch("pack_step");
+}
+
+void count_attention_work(const RowDesc * rows, int n_rows, int qt, int n_kv_heads, int * n_tiles, int * n_items) {
+    int tiles = 0, items = 0;
+    for (int r = 0; r < n_rows; ++r) {
+        const RowDesc & d = rows[r];
+        const int nt = (d.n + qt - 1) / qt;
+        for (int j = 0; j < nt; ++j) {
+            const int hi = d.pos0 + std::min(d.n, (j + 1) * qt);
+            const int p_first = d.kv_begin / PAGE, p_last = (hi - 1) / PAGE;
+            items += n_kv_heads * ((p_last - p_first + 1 + SPLIT_PAGES - 1) / SPLIT_PAGES);
+        }
+        tiles += nt;
+    }
+    *n_tiles = tiles;
+    *n_items = items;
+}
+
+// ---------------------------------------------------------------------------
+// RoPE + KV store
+
+__device__ __forceinline__ size_t k_page_offset(int head_dim, int t32, int e) {
+    // [dims/32][token half][g][token][8]
+    const int j = e >> 5, g = (e >> 3) & 3, i = e & 7;
+    const int tg = t32 >> 4, t = t32 & 15;
+    (void)head_dim;
+    return (size_t)((((j * 2 + tg) * 4 + g) * 16 + t) * 8 + i);
+}
+
+__device__ __forceinline__ size_t v_page_offset(int head_dim, int t32, int e) {
+    // [dims/16][g][dim][8]; slot (g, i) = token 4g+i (i<4) or 16+4g+(i-4)
+    const int dt = e >> 4, d = e & 15;
+    const int tt = t32 & 15;
+    const int g = tt >> 2;
+    const int i = (tt & 3) + ((t32 >> 4) << 2);
+    (void)head_dim;
+    return (size_t)(((dt * 4 + g) * 16 + d) * 8 + i);
+}
+
+struct RopeArgs {
+    const float * qkv;
+    const float * q_norm;
+    const float * k_norm;
+    __half * q_out;
+    __half * k_pool;
+    __half * v_pool;
+    const int32_t * cell;
+    const float * rope_cos;
+    const float * rope_sin;
+    int n_head, n_kv, hd, rope_dim, neox;
+    float eps, qscale;
+};
+
+// One wave per head: lanes own element pairs.
+__global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
+    const int t = blockIdx.x;
+    const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    const int heads_total = a.n_head + 2 * a.n_kv;
+    if (head >= heads_total) return;
+    const int QD = a.n_head * a.hd, KD = a.n_kv * a.hd;
+    const int pairs = a.hd / 2;
+    const int rp = a.rope_dim / 2;
+    const float * src = a.qkv + (size_t)t * (QD + 2 * KD) + (size_t)head * a.hd;
+    const bool is_q = head < a.n_head;
+    const bool is_k = !is_q && head < a.n_head + a.n_kv;
+    const bool active = lane < pairs;
+    // element pair of this lane
+    int i0, i1;
+    if (is_q || is_k) {
+        if (lane < rp) {
+            i0 = a.neox ? lane : 2 * lane;
+            i1 = a.neox ? lane + rp : 2 * lane + 1;
+        } else {          // dims past the rotary width pass through
+            i0 = a.rope_dim + 2 * (lane - rp);
+            i1 = i0 + 1;
+        }
+    } else {
+        i0 = 2 * lane;
+        i1 = i0 + 1;
+    }
+    float x0 = active ? src[i0] : 0.0f;
+    float x1 = active ? src[i1] : 0.0f;
+    const float * nw = is_q ? a.q_norm : (is_k ? a.k_norm : nullptr);
+    if (nw) {
+        const float ss = wave_sum(x0 * x0 + x1 * x1);
+        const float scale = 1.0f / sqrtf(ss / (float)a.hd + a.eps);
+        if (active) {
+            x0 = (x0 * scale) * nw[i0];
+            x1 = (x1 * scale) * nw[i1];
+        }
+    }
+    if (!active) return;
+    if ((is_q || is_k) && lane < rp) {
+        const float c = a.rope_cos[(size_t)t * rp + lane];
+        const float s = a.rope_sin[(size_t)t * rp + lane];
+        const float r0 = x0 * c - x1 * s;
+        const float r1 = x0 * s + x1 * c;
+        x0 = r0;
+        x1 = r1;
+    }
+    if (is_q) {
+        __half * q = a.q_out + (size_t)t * QD + (size_t)head * a.hd;
+        q[i0] = sat_half(x0 * a.qscale);
+        q[i1] = sat_half(x1 * a.qscale);
+        return;
+    }
+    const int cell = a.cell[t];
+    const int page = cell / PAGE, t32 = cell % PAGE;
+    const int kvh = is_k ? head - a.n_head : head - a.n_head - a.n_kv;
+    const size_t page_elems = (size_t)PAGE * a.hd;
+    if (is_k) {
+        __half * dst = a.k_pool + ((size_t)page * a.n_kv + kvh) * page_elems;
+        dst[k_page_offset(a.hd, t32, i0)] = sat_half(x0);
+        dst[k_page_offset(a.hd, t32, i1)] = sat_half(x1);
+    } else {
+        __half * dst = a.v_pool + ((size_t)page * a.n_kv + kvh) * page_elems;
+        dst[v_page_offset(a.hd, t32, i0)] = sat_half(x0);
+        dst[v_page_offset(a.hd, t32, i1)] = sat_half(x1);
+    }
+}
+
+void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, const PackBuffers & pk,
+                const float * q_norm, const float * k_norm, __half * q_out, __half * k_pool, __half * v_pool) {
+    if (T <= 0) return;
+    if (sh.head_dim > 128 || sh.head_dim % 32 != 0) throw std::runtime_error("rope_store: head_dim must be 32, 64, 96 or 128");
+    RopeArgs a;
+    a.qkv = qkv; a.q_norm = q_norm; a.k_norm = k_norm; a.q_out = q_out; a.k_pool = k_pool; a.v_pool = v_pool;
+    a.cell = pk.cell; a.rope_cos = pk.rope_cos; a.rope_sin = pk.rope_sin;
+    a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.hd = sh.head_dim; a.rope_dim = sh.rope_dim; a.neox = sh.rope_neox ? 1 : 0;
+    a.eps = sh.eps;
+    a.qscale = 1.4426950408889634f / sqrtf((float)sh.head_dim);
+    const int heads = sh.n_head + 2 * sh.n_head_kv;
+    hipLaunchKernelGGL(k_rope_store, dim3(T, (heads + 3) / 4), dim3(256), 0, s, a);
+    check_launch("rope_store");
+}
+
+// ---------------------------------------------------------------------------
+// paged attention
+
+struct AttnArgs {
+    const __half * q;
+    const __half * k_pool;
+    const __half * v_pool;
+    const int32_t * table;
+    const int32_t * tile_t0;
+    const int32_t * tile_nq;
+    const int32_t * tile_item0;
+    const int32_t * tile_nsplit;
+    const int32_t * tile_page0;
+    const int32_t * tile_kv_begin;
+    const int32_t * pos;
+    const int32_t * seq;
+    float * partial;
+    int n_tiles, n_items, max_pages;
+    int n_head, n_kv, G;
+};
+
+template <int HD>
+__global__ __launch_bounds__(64) void k_attention(AttnArgs a) {
+    constexpr int KS = HD / 32;     // k-steps of QK^T
+    constexpr int DT = HD / 16;     // dim tiles of PV
+    const int item = blockIdx.x;
+    const int lane = threadIdx.x;
+    const int c = lane & 15, g = lane >> 4;
+    // tile of this item: last tile whose first item <= item
+    int lo = 0, hi = a.n_tiles - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (a.tile_item0[mid] <= item) lo = mid; else hi = mid - 1;
+    }
+    const int tile = lo;
+    const int nsplit = a.tile_nsplit[tile];
+    const int rel = item - a.tile_item0[tile];
+    const int h = rel / nsplit, split = rel % nsplit;
+    const int t0 = a.tile_t0[tile], nq = a.tile_nq[tile];
+    const int kv_begin = a.tile_kv_begin[tile];
+    const int slot = a.seq[t0];
+    const int qi = c / a.G, gi = c % a.G;
+    const bool col_ok = qi < nq;
+    const int tq = t0 + (col_ok ? qi : 0);
+    const int limit = a.pos[tq];                        // this column attends positions <= limit
+    const int kv_hi = a.pos[t0 + nq - 1] + 1;
+    const int page_first = a.tile_page0[tile] + split * SPLIT_PAGES;
+    const int page_end = min((kv_hi - 1) / PAGE + 1, page_first + SPLIT_PAGES);
+
+    const int QD = a.n_head * HD;
+    h8 qreg[KS];
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+        if (col_ok) qreg[j] = load_h8(a.q + (size_t)tq * QD + (size_t)(h * a.G + gi) * HD + 32 * j + 8 * g);
+        else qreg[j] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+    }
+    f4 o[DT];
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o[d] = (f4){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.0f;
+    const size_t page_elems = (size_t)PAGE * HD;
+
+    for (int pi = page_first; pi < page_end; ++pi) {
+        const int pid = a.table[(size_t)slot * a.max_pages + pi];
+        const __half * kp = a.k_pool + ((size_t)pid * a.n_kv + h) * page_elems;
+        const __half * vp = a.v_pool + ((size_t)pid * a.n_kv + h) * page_elems;
+        h8 kreg[KS][2], vreg[DT];
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            kreg[j][0] = load_h8(kp + ((j * 2 + 0) * 64 + lane) * 8);
+            kreg[j][1] = load_h8(kp + ((j * 2 + 1) * 64 + lane) * 8);
+        }
+#pragma unroll
+        for (int d = 0; d < DT; ++d) vreg[d] = load_h8(vp + (d * 64 + lane) * 8);
+
+        f4 s0 = (f4){0.f, 0.f, 0.f, 0.f}, s1 = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg[j], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg[j], s1, 0, 0, 0);
+        }
+        // rows of s0 are tokens 4g+i, of s1 tokens 16+4g+i of this page
+        const int pbase = pi * PAGE + 4 * g;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int p0 = pbase + i, p1 = pbase + 16 + i;
+            if (!(col_ok && p0 >= kv_begin && p0 <= limit)) s0[i] = -INFINITY;
+            if (!(col_ok && p1 >= kv_begin && p1 <= limit)) s1[i] = -INFINITY;
+            mx = fmaxf(mx, fmaxf(s0[i], s1[i]));
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = exp2f(m_run - m_use);       // m_run = -inf -> 0
+        float psum = 0.0f;
+        h8 pt;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float e0 = exp2f(s0[i] - m_use);
+            const float e1 = exp2f(s1[i] - m_use);
+            const _Float16 h0 = (_Float16)e0, h1 = (_Float16)e1;
+            pt[i] = h0;
+            pt[4 + i] = h1;
+            psum += (float)h0 + (float)h1;              // the sum of what PV really multiplies
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[d][i] *= alpha;
+            o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt, o[d], 0, 0, 0);
+        }
+    }
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (col_ok) {
+        float * dst = a.partial + ((size_t)item * 16 + c) * (HD + 2);
+        if (g == 0) { dst[0] = m_run; dst[1] = l_run; }
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dst[2 + d * 16 + 4 * g + i] = o[d][i];
+    }
+}
+
+size_t attention_partial_floats(int n_items, int head_dim) {
+    return (size_t)n_items * 16 * (head_dim + 2);
+}
+
+void attention(hipStream_t s, const __half * q, const AttnShape & sh, const PackBuffers & pk,
+               const int32_t * table, int max_pages, const __half * k_pool, const __half * v_pool,
+               int n_items, int n_tiles, float * partial) {
+    if (n_items <= 0) return;
+    AttnArgs a;
+    a.q = q; a.k_pool = k_pool; a.v_pool = v_pool; a.table = table;
+    a.tile_t0 = pk.tile_t0; a.tile_nq = pk.tile_nq; a.tile_item0 = pk.tile_item0; a.tile_nsplit = pk.tile_nsplit;
+    a.tile_page0 = pk.tile_page0; a.tile_kv_begin = pk.tile_kv_begin; a.pos = pk.pos; a.seq = pk.seq;
+    a.partial = partial; a.n_tiles = n_tiles; a.n_items = n_items; a.max_pages = max_pages;
+    a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.G = sh.n_head / sh.n_head_kv;
+    if (a.G > 16 || sh.n_head % sh.n_head_kv != 0) throw std::runtime_error("attention: unsupported head grouping");
+    switch (sh.head_dim) {
+        case 32:  hipLaunchKernelGGL(k_attention<32>, dim3(n_items), dim3(64), 0, s, a); break;
+        case 64:  hipLaunchKernelGGL(k_attention<64>, dim3(n_items), dim3(64), 0, s, a); break;
+        case 128: hipLaunchKernelGGL(k_attention<128>, dim3(n_items), dim3(64), 0, s, a); break;
+        default: throw std::runtime_error("attention: head_dim must be 32, 64 or 128");
+    }
+    check_launch("attention");
+}
+
+struct CombineArgs {
+    const float * partial;
+    const int32_t * tok_tile;
+    const int32_t * tile_t0;
+    const int32_t * tile_item0;
+    const int32_t * tile_nsplit;
+    Act out;
+    int n_head, G, hd;
+};
+
+// One wave per (token, query head): merges the KV splits and writes the
+// attention output as the O-projection's activations.
+__global__ __launch_bounds__(256) void k_attention_combine(CombineArgs a) {
+    const int t = blockIdx.x;
+    const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (head >= a.n_head) return;
+    const int tile = a.tok_tile[t];
+    const int ns = a.tile_nsplit[tile];
+    const int kvh = head / a.G, gi = head % a.G;
+    const int col = (t - a.tile_t0[tile]) * a.G + gi;
+    const int item0 = a.tile_item0[tile] + kvh * ns;
+    const int stride = a.hd + 2;
+    float M = -INFINITY;
+    for (int s = 0; s < ns; ++s) M = fmaxf(M, a.partial[((size_t)(item0 + s) * 16 + col) * stride]);
+    float L = 0.0f, v0 = 0.0f, v1 = 0.0f;
+    const int e0 = 2 * lane;
+    for (int s = 0; s < ns; ++s) {
+        const float * p = a.partial + ((size_t)(item0 + s) * 16 + col) * stride;
+        const float w = p[0] == -INFINITY ? 0.0f : exp2f(p[0] - M);
+        L += w * p[1];
+        if (e0 < a.hd) {
+            v0 += w * p[2 + e0];
+            v1 += w * p[3 + e0];
+        }
+    }
+    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+    const int QD = a.n_head * a.hd;
+    float r0 = 0.0f, r1 = 0.0f;
+    if (e0 < a.hd) {
+        const __half h0 = sat_half(v0 * inv), h1 = sat_half(v1 * inv);
+        __half * dst = a.out.x + (size_t)t * QD + (size_t)head * a.hd + e0;
+        dst[0] = h0;
+        dst[1] = h1;
+        r0 = __half2float(h0);
+        r1 = __half2float(h1);
+    }
+    if (a.out.xs_hi) {
+        // block of 32 outputs = 16 lanes
+        float sum = r0 + r1;
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o, 64);
+        if ((lane & 15) == 0 && e0 < a.hd) {
+            const size_t b = ((size_t)t * QD + (size_t)head * a.hd + e0) / 32;
+            const __half hi = sat_half(sum);
+            a.out.xs_hi[b] = hi;
+            a.out.xs_lo[b] = __float2half_rn(sum - __half2float(hi));
+        }
+    }
+}
+
+void attention_combine(hipStream_t s, const float * partial, int T, const AttnShape & sh,
+                       const PackBuffers & pk, const Act & out) {
+    if (T <= 0) return;
+    CombineArgs a;
+    a.partial = partial; a.tok_tile = pk.tok_tile; a.tile_t0 = pk.tile_t0; a.tile_item0 = pk.tile_item0;
+    a.tile_nsplit = pk.tile_nsplit; a.out = out;
+    a.n_head = sh.n_head; a.G = sh.n_head / sh.n_head_kv; a.hd = sh.head_dim;
+    hipLaunchKernelGGL(k_attention_combine, dim3(T, (sh.n_head + 3) / 4), dim3(256), 0, s, a);
+    check_launch("attention_combine");
+}
+
+// ---------------------------------------------------------------------------
+// KV page utilities
+
+__global__ void k_kv_gather(const __half * pool, int n_kv, int hd, int is_v, const int32_t * cells, int n,
+                            __half * out, int scatter) {
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int kd = n_kv * hd;
+    if (gid >= (size_t)n * kd) return;
+    const int idx = (int)(gid / kd), e_all = (int)(gid % kd);
+    const int kvh = e_all / hd, e = e_all % hd;
+    const int cell = cells[idx];
+    const int page = cell / PAGE, t32 = cell % PAGE;
+    const size_t off = ((size_t)page * n_kv + kvh) * (size_t)PAGE * hd
+        + (is_v ? v_page_offset(hd, t32, e) : k_page_offset(hd, t32, e));
+    __half * cache = const_cast<__half *>(pool) + off;
+    if (scatter) *cache = out[gid];
+    else out[gid] = *cache;
+}
+
+void kv_gather(hipStream_t s, const __half * pool, int n_kv_heads, int head_dim, bool is_v,
+               const int32_t * cells, int n, __half * out) {
+    if (n <= 0) return;
+    const size_t total = (size_t)n * n_kv_heads * head_dim;
+    hipLaunchKernelGGL(k_kv_gather, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, n_kv_heads,
+                       head_dim, is_v ? 1 : 0, cells, n, out, 0);
+    check_launch("kv_gather");
+}
+
+void kv_scatter(hipStream_t s, __half * pool, int n_kv_heads, int head_dim, bool is_v,
+                const int32_t * cells, int n, const __half * in) {
+    if (n <= 0) return;
+    const size_t total = (size_t)n * n_kv_heads * head_dim;
+    hipLaunchKernelGGL(k_kv_gather, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, n_kv_heads,
+                       head_dim, is_v ? 1 : 0, cells, n, const_cast<__half *>(in), 1);
+    check_launch("kv_scatter");
+}
+
+__global__ void k_kv_copy_page(__half * k_pool, __half * v_pool, size_t page_halves, int src, int dst) {
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (i >= page_halves) return;
+    *(u4 *)(k_pool + (size_t)dst * page_halves + i) = *(const u4 *)(k_pool + (size_t)src * page_halves + i);
+    *(u4 *)(v_pool + (size_t)dst * page_halves + i) = *(const u4 *)(v_pool + (size_t)src * page_halves + i);
+}
+
+void kv_copy_page(hipStream_t s, __half * k_pool, __half * v_pool, int n_kv_heads, int head_dim,
+                  int src_page, int dst_page) {
+    const size_t page_halves = (size_t)n_kv_heads * PAGE * head_dim;
+    hipLaunchKernelGGL(k_kv_copy_page, dim3((unsigned)((page_halves / 8 + 255) / 256)), dim3(256), 0, s,
+                       k_pool, v_pool, page_halves, src_page, dst_page);
+    check_launch("kv_copy_page");
+}
+
+// ---------------------------------------------------------------------------
+// sampling preparation
+
+// (value desc, id asc) order on (float, int) pairs
+__device__ __forceinline__ bool better(float va, int ia, float vb, int ib) {
+    return va > vb || (va == vb && ia < ib);
+}
+
+__global__ __launch_bounds__(1024) void k_sample_prepare(const float * __restrict__ logits, int V,
+                                                         const int32_t * __restrict__ kreq, SampleOut * out) {
+    __shared__ float s_val[16];
+    __shared__ int s_idx[16];
+    __shared__ double s_sum[16];
+    __shared__ float b_val;
+    __shared__ int b_idx;
+    const int row = blockIdx.x;
+    const float * l = logits + (size_t)row * V;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int k = min(kreq ? kreq[row] : 0, MAX_TOPK);
+    float prev_v = INFINITY;
+    int prev_i = -1;
+    float row_max = 0.0f;
+    // selection 0 is the argmax; each later selection is the best entry
+    // strictly after the previous one in (value desc, id asc) order
+    for (int sel = 0; sel < max(k, 1); ++sel) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int i = threadIdx.x; i < V; i += 1024) {
+            const float v = l[i];
+            const bool after_prev = sel == 0 || better(prev_v, prev_i, v, i);
+            if (after_prev && better(v, i, bv, bi)) { bv = v; bi = i; }
+        }
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+        }
+        if (lane == 0) { s_val[wave] = bv; s_idx[wave] = bi; }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float fv = s_val[0];
+            int fi = s_idx[0];
+            for (int w = 1; w < 16; ++w) if (better(s_val[w], s_idx[w], fv, fi)) { fv = s_val[w]; fi = s_idx[w]; }
+            b_val = fv;
+            b_idx = fi;
+            if (sel == 0) { out[row].argmax = fi; out[row].max = fv; }
+            if (sel < k) { out[row].top_id[sel] = fi; out[row].top_logit[sel] = fv; }
+        }
+        __syncthreads();
+        prev_v = b_val;
+        prev_i = b_idx;
+        if (sel == 0) row_max = b_val;
+        __syncthreads();
+    }
+    double acc = 0.0;
+    for (int i = threadIdx.x; i < V; i += 1024) acc += exp((double)l[i] - (double)row_max);
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (lane == 0) s_sum[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double total = 0.0;
+        for (int w = 0; w < 16; ++w) total += s_sum[w];
+        out[row].sum_exp = total;
+    }
+}
+
+void sample_prepare(hipStream_t s, const float * logits, int n_rows, int n_vocab, const int32_t * k,
+                    SampleOut * out) {
+    if (n_rows <= 0) return;
+    hipLaunchKernelGGL(k_sample_prepare, dim3(n_rows), dim3(1024), 0, s, logits, n_vocab, k, out);
+    check_launch("sample_prepare");
+}
+
+}  // namespace rk

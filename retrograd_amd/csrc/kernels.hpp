@@ -1,0 +1,164 @@
+// Host-side launch interface of the gfx950 kernels behind the decode step.
+// Everything here is plain C++ over HIP pointers; the C ABI lives in capi.cpp.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace rk {
+
+// ggml tensor type ids as stored in GGUF.
+enum : int { WT_F32 = 0, WT_F16 = 1, WT_Q8_0 = 8, WT_Q4_K = 12, WT_BF16 = 30, WT_MXFP4 = 39 };
+
+// One KV page holds PAGE consecutive positions of one sequence.
+constexpr int PAGE = 32;
+// One attention work item scans at most SPLIT_PAGES pages of one sequence.
+constexpr int SPLIT_PAGES = 8;
+// Candidates the sampling kernel can return per row.
+constexpr int MAX_TOPK = 64;
+
+struct BlockGeom { int elements; int bytes; };
+BlockGeom geom_of(int type);                 // throws on an unknown type
+size_t row_bytes(int type, int64_t k);       // throws when k is not block aligned
+
+// A weight matrix [N rows][K] in HBM. Exactly one of raw/packed is set:
+// `raw` keeps the GGUF row-major block layout (generic kernel, row gathers);
+// `packed` is the MFMA tile layout of the same bytes (K % 256 == 0, N % 16 == 0).
+struct Weight {
+    int type = 0;
+    int K = 0;
+    int N = 0;
+    const uint8_t * raw = nullptr;
+    const uint8_t * packed = nullptr;
+    size_t bytes = 0;
+};
+
+// Activations handed to a matmul: f16 rows plus, for every 32-wide block of a
+// row, the f32 sum of the (already rounded) f16 values split into two halves
+// hi + lo. The sums are what the Q4_K min term multiplies.
+struct Act {
+    __half * x = nullptr;       // [T][K]
+    __half * xs_hi = nullptr;   // [T][K/32], null when K % 32 != 0
+    __half * xs_lo = nullptr;
+    int K = 0;
+};
+
+bool can_pack(int type, int64_t K, int64_t N);
+// raw (device, GGUF layout) -> packed (device). Both hold `bytes` bytes.
+void repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int K, int N);
+
+enum : int { MM_STORE = 0, MM_ADD = 1 };
+// y[t][col0 + n] (=|+=) sum_k W[n][k] * x[t][k] (+ bias[n]); y has row stride ldy.
+void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+            int mode, const float * bias);
+// Forces the generic (raw layout) kernel; used to cross-check the tile kernels.
+void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                    int mode, const float * bias);
+
+// x[t][:] = decode(raw row tok[t]) as f32.
+void embed(hipStream_t s, const Weight & emb, const int32_t * tok, int T, float * x);
+
+// act = f16(x * rsqrt(mean(x^2) + eps) * w) (+ block sums). `rows` selects the
+// input rows (null: identity), n_rows outputs.
+void rmsnorm_act(hipStream_t s, const float * x, const float * w, int E, float eps,
+                 const int32_t * rows, int n_rows, const Act & out);
+
+// act = f16(x) (+ block sums): the plain conversion every producer fuses.
+void to_act(hipStream_t s, const float * x, int T, int K, const Act & out);
+
+// act = f16(silu(gu[t][i]) * gu[t][F + i]) (+ block sums).
+void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out);
+
+// ---- step packing -----------------------------------------------------------
+struct RowDesc {           // one per step row, written by the host
+    int32_t slot;
+    int32_t pos0;
+    int32_t n;
+    int32_t tok_off;       // flat index of the row's first token
+    int32_t sample;
+    int32_t kv_begin;      // first resident position of the slot
+    int32_t route;         // adapter route (0 = none)
+    int32_t pad;
+};
+struct TableUpdate { int32_t slot; int32_t index; int32_t page; int32_t pad; };
+
+struct PackBuffers {       // device arrays, sized for n_batch tokens / rows
+    int32_t * tok;         // [T] token id
+    int32_t * pos;         // [T] absolute position
+    int32_t * seq;         // [T] slot
+    int32_t * row;         // [T] owning row
+    int32_t * cell;        // [T] page_id * PAGE + pos % PAGE
+    int32_t * out_index;   // [T] index among the output rows, or -1
+    int32_t * out_tok;     // [n_out] flat token index of each output row
+    int32_t * last_index;  // [n_rows] flat index of the row's last token
+    int32_t * row_offset;  // [n_rows + 1]
+    int32_t * counts;      // [4]: n_tokens, n_outputs, n_tiles, n_items
+    // attention query tiles: up to `qt` consecutive tokens of one row
+    int32_t * tile_t0;     // first flat token
+    int32_t * tile_nq;     // tokens in the tile
+    int32_t * tile_item0;  // first work item of the tile
+    int32_t * tile_nsplit; // KV splits per kv head
+    int32_t * tile_page0;  // first page index (within the slot) the tile reads
+    int32_t * tile_kv_begin;
+    int32_t * tok_tile;    // [T] tile of each token
+    float * rope_cos;      // [T][rope_dim/2]
+    float * rope_sin;
+};
+// Applies the block-table updates, then derives every per-token / per-tile
+// array of the step from the row descriptors. One workgroup.
+void pack_step(hipStream_t s, const RowDesc * rows, int n_rows, const int32_t * tokens_concat,
+               const TableUpdate * updates, int n_updates, int32_t * table, int max_pages,
+               int qt, int n_kv_heads, const double * inv_freq, int rope_pairs, const PackBuffers & out);
+
+// Host mirror of the tile/item count (same formula as the kernel).
+void count_attention_work(const RowDesc * rows, int n_rows, int qt, int n_kv_heads,
+                          int * n_tiles, int * n_items);
+
+// ---- attention ----------------------------------------------------------------
+struct AttnShape {
+    int n_head, n_head_kv, head_dim;
+    int rope_dim;
+    bool rope_neox;
+    float eps;
+};
+// qkv f32 [T][QD + 2*KD] (+ optional per-head RMSNorm weights) -> q f16 [T][QD]
+// (rotated, pre-scaled by log2(e)/sqrt(head_dim)) and K/V pages of the layer.
+void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, const PackBuffers & pk,
+                const float * q_norm, const float * k_norm, __half * q_out, __half * k_pool, __half * v_pool);
+
+// Split-KV paged attention over the step's query tiles. partial holds, per
+// (item, column), m (log2 domain), l and head_dim unnormalised outputs.
+void attention(hipStream_t s, const __half * q, const AttnShape & sh, const PackBuffers & pk,
+               const int32_t * table, int max_pages, const __half * k_pool, const __half * v_pool,
+               int n_items, int n_tiles, float * partial);
+// Merges the splits: out act [T][QD] (+ block sums).
+void attention_combine(hipStream_t s, const float * partial, int T, const AttnShape & sh,
+                       const PackBuffers & pk, const Act & out);
+size_t attention_partial_floats(int n_items, int head_dim);
+
+// Gathers the K or V row of one (layer pool, cell) into natural order, and the
+// inverse; used by sequence snapshots and by tests.
+void kv_gather(hipStream_t s, const __half * pool, int n_kv_heads, int head_dim, bool is_v,
+               const int32_t * cells, int n, __half * out);
+void kv_scatter(hipStream_t s, __half * pool, int n_kv_heads, int head_dim, bool is_v,
+                const int32_t * cells, int n, const __half * in);
+// Copies the first `count` positions of page src to page dst in one layer pool.
+void kv_copy_page(hipStream_t s, __half * k_pool, __half * v_pool, int n_kv_heads, int head_dim,
+                  int src_page, int dst_page);
+
+// ---- sampling -------------------------------------------------------------------
+struct SampleOut {          // one per output row, read back by the host
+    int32_t argmax;
+    float max;
+    double sum_exp;         // sum exp(double(logit) - max)
+    int32_t top_id[MAX_TOPK];
+    float top_logit[MAX_TOPK];
+};
+// k[r] candidates per row by (logit desc, id asc); k = 0 rows only get argmax/max/sum.
+void sample_prepare(hipStream_t s, const float * logits, int n_rows, int n_vocab, const int32_t * k,
+                    SampleOut * out);
+
+}  // namespace rk

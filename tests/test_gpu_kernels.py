@@ -1,0 +1,121 @@
+"""Kernel-level parity on the GPU, through the C ABI of include/retro_kernels.h.
+
+Reference values come from the CPU oracle's block decoders: the same stored
+bytes decoded on the host, multiplied in float64 with the f16-rounded
+activations the kernels consume. Tolerance: the kernels accumulate exact
+f16 x integer products in f32, so 2e-5 of the output scale covers them."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from retrograd_amd import engine as E
+from retrograd_amd import gguf_writer as gw
+from retrograd_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _weights(t, n, k, seed):
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(n, k, generator=g) * 0.05
+    raw = synth.encode(w, t)
+    raw = np.ascontiguousarray(raw).view(np.uint8).reshape(n, -1)
+    dense = np.stack([oracle.decode_row(t, raw[i], k) for i in range(n)]).astype(np.float64)
+    return raw, dense
+
+
+def _ref(dense, x):
+    xh = x.astype(np.float16).astype(np.float64)
+    return xh @ dense.T
+
+
+@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0])
+@pytest.mark.parametrize("n,k,T", [(16, 256, 1), (48, 512, 7), (64, 1024, 16), (256, 4096, 33),
+                                   (4096, 2048, 64), (160, 768, 100), (2064, 256, 3)])
+def test_tile_matmul_matches_decoded_blocks(t, n, k, T):
+    print("case", t, n, k, T, flush=True)
+    raw, dense = _weights(t, n, k, seed=n + k + T)
+    x = np.random.default_rng(T).standard_normal((T, k)).astype(np.float32)
+    want = _ref(dense, x)
+    got = E.kernel_matmul(t, raw, n, k, x, use_tiles=True)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-5 * scale + 1e-6
+    gen = E.kernel_matmul(t, raw, n, k, x, use_tiles=False)
+    assert np.abs(gen - want).max() <= 2e-5 * scale + 1e-6
+
+
+@pytest.mark.parametrize("t,k", [(gw.GGML_F16, 344), (gw.GGML_F32, 100), (gw.GGML_Q8_0, 128),
+                                 (gw.GGML_MXFP4, 96), (gw.GGML_Q4_K, 256), (gw.GGML_BF16, 64)])
+def test_generic_matmul_every_storage_type(t, k):
+    print("case", t, k, flush=True)
+    n, T = 37, 11
+    if t == gw.GGML_BF16:
+        g = torch.Generator().manual_seed(1)
+        w = (torch.randn(n, k, generator=g) * 0.05).to(torch.bfloat16)
+        raw = w.view(torch.int16).numpy().view(np.uint8).reshape(n, -1)
+        dense = w.float().numpy().astype(np.float64)
+    else:
+        raw, dense = _weights(t, n, k, seed=k)
+    x = np.random.default_rng(2).standard_normal((T, k)).astype(np.float32)
+    want = _ref(dense, x)
+    got = E.kernel_matmul(t, raw, n, k, x, use_tiles=False)
+    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max() + 1e-6
+
+
+def test_matmul_bias_and_accumulate():
+    t, n, k, T = gw.GGML_Q4_K, 64, 512, 20
+    raw, dense = _weights(t, n, k, seed=5)
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((T, k)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    y0 = rng.standard_normal((T, n)).astype(np.float32)
+    want = _ref(dense, x)
+    for tiles in (True, False):
+        got = E.kernel_matmul(t, raw, n, k, x, use_tiles=tiles, bias=bias)
+        assert np.abs(got - (want + bias)).max() <= 3e-5 * np.abs(want).max()
+        got = E.kernel_matmul(t, raw, n, k, x, use_tiles=tiles, accumulate_into=y0)
+        assert np.abs(got - (want + y0)).max() <= 3e-5 * np.abs(want).max()
+
+
+def test_tile_matmul_exact_on_integer_data():
+    # Small-integer activations and weights whose products and sums are exact
+    # in f32: the tile kernel must be bit-exact, which catches any misplaced
+    # nibble, scale or min.
+    rng = np.random.default_rng(7)
+    n, k, T = 32, 512, 16
+    blocks = rng.integers(0, 256, (n, k // 256, 144), dtype=np.uint8)
+    blocks[..., 0:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    blocks[..., 2:4] = np.frombuffer(np.float16(0.25).tobytes(), np.uint8)
+    raw = blocks.reshape(n, -1)
+    dense = np.stack([oracle.decode_row(gw.GGML_Q4_K, raw[i], k) for i in range(n)]).astype(np.float64)
+    x = rng.integers(-4, 5, (T, k)).astype(np.float32)
+    want = x.astype(np.float64) @ dense.T
+    got = E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x, use_tiles=True)
+    assert np.array_equal(got.astype(np.float64), want)
+    q8 = rng.integers(0, 256, (n, k // 32, 34), dtype=np.uint8)
+    q8[..., 0:2] = np.frombuffer(np.float16(0.125).tobytes(), np.uint8)
+    raw = q8.reshape(n, -1)
+    dense = np.stack([oracle.decode_row(gw.GGML_Q8_0, raw[i], k) for i in range(n)]).astype(np.float64)
+    want = x.astype(np.float64) @ dense.T
+    got = E.kernel_matmul(gw.GGML_Q8_0, raw, n, k, x, use_tiles=True)
+    assert np.array_equal(got.astype(np.float64), want)
+
+
+def test_sample_prepare_matches_numpy():
+    rng = np.random.default_rng(11)
+    V = 5003
+    logits = (rng.standard_normal((6, V)) * 3).astype(np.float32)
+    logits[2, 100] = logits[2, 4000] = logits[2].max() + 1.0      # tie for the maximum: lowest id wins
+    logits[3, :50] = 2.5                                           # ties inside the top-k
+    k = [0, 1, 5, 64, 40, 8]
+    argmax, mx, se, ids, vals = E.kernel_sample_prepare(logits, k)
+    for r in range(6):
+        row = logits[r]
+        assert argmax[r] == int(np.flatnonzero(row == row.max())[0])
+        assert mx[r] == row.max()
+        ref = np.exp(row.astype(np.float64) - float(row.max())).sum()
+        assert abs(se[r] - ref) <= 1e-12 * ref
+        order = np.lexsort((np.arange(V), -row.astype(np.float64)))[:k[r]]
+        assert list(ids[r, :k[r]]) == list(order)
+        assert np.array_equal(vals[r, :k[r]], row[order])

@@ -1,0 +1,219 @@
+"""The decode step on the GPU against the CPU oracle, through the C ABI.
+
+Tolerances are BASELINE's: logits within 2e-2 max-abs and 1e-3 mean-abs
+relative error; packing, cells, slot ranges and greedy token ids bit-exact
+(token ids are compared where the oracle's own top-1/top-2 margin exceeds the
+logit tolerance - a margin below the tolerance is a tie no two float
+implementations are required to break alike)."""
+import numpy as np
+import pytest
+
+import oracle
+from engine_helpers import assert_logits_close, greedy, logit_errors, run_both
+from retrograd_amd import engine as E
+from retrograd_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+SMALL = {
+    "tiny-llama-q8": synth.TINY_LLAMA,
+    "llama-q4k": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
+                              n_ff=1024, n_vocab=1024, name="llama-q4k-small"),
+    "llama-q4k-hd128": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=1024, n_head=8, n_head_kv=2,
+                                    head_dim=128, n_ff=2048, n_vocab=2048, name="llama-q4k-hd128"),
+    "qwen2-q8": synth.scaled(synth.QWEN25_7B_Q8, n_layer=2, n_embd=512, n_head=14, n_head_kv=2, head_dim=32,
+                             n_ff=1024, n_vocab=1024, name="qwen2-small"),
+}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    d = tmp_path_factory.mktemp("gpu_models")
+    out = {}
+    for i, (k, s) in enumerate(SMALL.items()):
+        p = d / (k + ".gguf")
+        synth.write_model(p, s, seed=100 + i, device="cpu", std=0.05 if k != "tiny-llama-q8" else 0.02)
+        out[k] = p
+    return out
+
+
+def _pair(path, n_seq=8, n_ctx=2048, n_batch=256):
+    eng = E.Engine(path, E.EngineConfig(n_ctx=n_ctx, n_seq_max=n_seq, n_batch=n_batch, n_ubatch=n_batch))
+    m = oracle.Model(path)
+    return eng, oracle.Context(m, n_seq), m
+
+
+@pytest.mark.parametrize("key", list(SMALL))
+def test_prefill_and_decode_logits_match_oracle(models, key):
+    print("model", key, flush=True)
+    eng, ctx, m = _pair(models[key])
+    rng = np.random.default_rng(1)
+    lens = [5, 33, 64, 17]
+    prompts = [rng.integers(0, m.n_vocab, n) for n in lens]
+    rows = [(i, i, p, 0, True) for i, p in enumerate(prompts)]
+    out, got, want = run_both(eng, ctx, rows)
+    assert_logits_close(got, want)
+    toks = [r.token for r in out.rows()]
+    for i, t in enumerate(toks):
+        srt = np.sort(want[i])[::-1]
+        if srt[0] - srt[1] > 4e-2:
+            assert t == int(want[i].argmax())
+    # three decode steps, teacher-forced with the oracle's tokens
+    pos = list(lens)
+    for _ in range(3):
+        feed = [int(want[i].argmax()) for i in range(4)]
+        rows = [(i, i, [feed[i]], pos[i], True) for i in range(4)]
+        out, got, want = run_both(eng, ctx, rows)
+        assert_logits_close(got, want)
+        pos = [p + 1 for p in pos]
+    for i in range(4):
+        assert eng.seq_pos(i) == ctx.seq_pos(i) == (0, pos[i] - 1)
+    eng.close()
+
+
+def test_packing_is_bit_exact_with_the_oracle(models):
+    eng, ctx, m = _pair(models["llama-q4k"], n_seq=8, n_ctx=1024, n_batch=128)
+    rng = np.random.default_rng(2)
+    plan = [(3, 40, True), (0, 1, True), (7, 33, False), (5, 9, True)]   # slot, n, sample
+    rows = [(i, s, rng.integers(0, m.n_vocab, n), 0, smp) for i, (s, n, smp) in enumerate(plan)]
+    out = E.StepOutput()
+    eng.step([E.StepRow(r[0], r[1], r[2], r[3], sample=r[4], sampling=greedy()) for r in rows], out)
+    pk = eng.debug_pack(128, 128)
+    want = oracle.pack_rows([(r[1], r[3], r[2], r[4]) for r in rows])
+    assert np.array_equal(pk["token"], want["token"])
+    assert np.array_equal(pk["pos"], want["pos"])
+    assert np.array_equal(pk["seq"], want["seq"])
+    assert np.array_equal(pk["out_index"] >= 0, want["output"].astype(bool))
+    assert np.array_equal(pk["last_index"][:4], want["last_index"])
+    assert list(pk["counts"][:2]) == [83, 3]
+    # block table: lowest free page first, in row order; cells follow the table
+    page = 32
+    tables = np.stack([eng.debug_pages(s) for s in range(8)])
+    assert list(tables[3][:2]) == [0, 1] and tables[0][0] == 2 and list(tables[7][:2]) == [3, 4] and tables[5][0] == 5
+    cells = oracle.pack_cells(want["pos"], want["seq"], tables, page)
+    assert np.array_equal(pk["cell"].astype(np.int64), cells)
+    assert [r.sampled for r in out.rows()] == [True, True, False, True]
+    eng.close()
+
+
+def test_chunked_prefill_matches_one_shot(models):
+    eng, ctx, m = _pair(models["llama-q4k-hd128"], n_batch=128)
+    rng = np.random.default_rng(3)
+    toks = rng.integers(0, m.n_vocab, 100)
+    out = E.StepOutput()
+    eng.step([E.StepRow(0, 0, toks, 0, sample=True, sampling=greedy())], out)
+    one = eng.debug_logits().copy()
+    eng.step([E.StepRow.prefill(1, 1, toks[:37], 0)], out)
+    eng.step([E.StepRow.prefill(1, 1, toks[37:70], 37)], out)
+    eng.step([E.StepRow(1, 1, toks[70:], 70, sample=True, sampling=greedy())], out)
+    chunked = eng.debug_logits()
+    want = ctx.step_rows([(0, 0, toks, True)])
+    assert_logits_close(one, want)
+    assert_logits_close(chunked, want)
+    # K/V written by either schedule are the same f16 values as the oracle's
+    for pos in (0, 36, 37, 99):
+        for want_v in (False, True):
+            a = eng.debug_kv(1, 0, pos, want_v, m.n_head_kv * m.head_dim).astype(np.float32)
+            b = eng.debug_kv(1, 1, pos, want_v, m.n_head_kv * m.head_dim).astype(np.float32)
+            c = ctx.read_kv(1, 0, pos, want_v).astype(np.float32)
+            assert np.abs(a - c).max() <= 2e-2 * np.abs(c).max() + 1e-3
+            assert np.abs(b - c).max() <= 2e-2 * np.abs(c).max() + 1e-3
+    eng.close()
+
+
+def test_seq_cp_seq_rm_and_snapshots(models):
+    eng, ctx, m = _pair(models["llama-q4k"], n_seq=6, n_ctx=1024, n_batch=128)
+    rng = np.random.default_rng(4)
+    toks = rng.integers(0, m.n_vocab, 50)
+    out = E.StepOutput()
+    eng.step([E.StepRow.prefill(0, 0, toks[:45], 0)], out)
+    ctx.step_rows([(0, 0, toks[:45], False)])
+    eng.seq_cp(0, 1)              # whole copy: shares both pages
+    eng.seq_cp(0, 2, 0, 40)       # partial copy [0, 40)
+    ctx.seq_cp(0, 1)
+    ctx.seq_cp(0, 2, 0, 40)
+    assert eng.seq_pos(1) == (0, 44) and eng.seq_pos(2) == (0, 39)
+    assert eng.memory().cells_used == 45 + 45 + 40     # counted once per slot that references them
+    snap = eng.seq_save(0)
+    assert len(snap) == eng.seq_save_len(0)
+    eng.seq_load(3, snap)
+    assert eng.seq_pos(3) == (0, 44)
+    # continue all four: slot 2 first re-decodes positions 40..44
+    eng.step([E.StepRow.prefill(2, 2, toks[40:45], 40)], out)
+    ctx.step_rows([(2, 40, toks[40:45], False)])
+    rows = [(s, s, toks[45:], 45, True) for s in range(3)]
+    o, got, want = run_both(eng, ctx, rows)
+    assert_logits_close(got, want)
+    # copy == source bit for bit (same arithmetic on the same cells / same bytes)
+    assert np.array_equal(got[0], got[1])
+    eng.step([E.StepRow(3, 3, toks[45:], 45, sample=True, sampling=greedy())], out)
+    restored = eng.debug_logits()
+    assert_logits_close(restored, want[:1])
+    # removal
+    eng.seq_rm(1, 30, -1)
+    assert eng.seq_pos(1) == (0, 29)
+    eng.seq_rm(1)
+    assert eng.seq_pos(1) == (-1, -1)
+    with pytest.raises(E.RuntimeFailure):
+        eng.seq_rm(0, 10, 20)      # a hole in the middle cannot be removed
+    with pytest.raises(E.BufferTooSmall):
+        eng.seq_save_into(0, 0, bytearray(16))
+    eng.close()
+
+
+def test_step_argument_errors_are_reported_before_decoding(models):
+    eng, ctx, m = _pair(models["tiny-llama-q8"], n_seq=4, n_ctx=256, n_batch=32)
+    out = E.StepOutput()
+    ok = lambda **kw: E.StepRow(kw.get("request", 0), kw.get("slot", 0), kw.get("tokens", [1, 2]), kw.get("pos0", 0),
+                                sample=kw.get("sample", False), sampling=kw.get("sampling", greedy()),
+                                n_top_logprobs=kw.get("n_top", 0), adapter=kw.get("adapter", E.RowAdapter()))
+    cases = [
+        ([ok(slot=4)], "slot is outside"),
+        ([ok(tokens=[m.n_vocab])], "outside the vocabulary"),
+        ([ok(pos0=255)], "positions exceed"),
+        ([ok(tokens=list(range(33)))], "exceed the context's physical batch"),
+        ([ok(request=0), ok(request=1, slot=0, pos0=1)], "overlap"),
+        ([ok(request=-1, sample=True)], "request id"),
+        ([ok(sample=True, sampling=E.SamplingParamsV2(temperature=0.0))], "temperature"),
+        ([ok(sample=True, sampling=E.SamplingParamsV2(top_p=0.0))], "top_p"),
+        ([ok(sample=True, sampling=E.SamplingParamsV2(min_p=1.5))], "min_p"),
+        ([ok(adapter=E.RowAdapter.loaded(3))], "not a loaded per-row adapter"),
+    ]
+    for rows, needle in cases:
+        with pytest.raises(E.InvalidArgument) as err:
+            eng.step(rows, out)
+        assert needle in str(err.value), (needle, str(err.value))
+        assert eng.seq_pos(0) == (-1, -1)
+    # a request id twice is caught on the caller side too (step.rs:412-505)
+    with pytest.raises(E.InvalidArgument):
+        eng.step([ok(request=5), ok(request=5, slot=1)], out)
+    # capacity is a runtime condition, not an invalid argument
+    eng.step([ok(tokens=list(range(1, 30)))], out)
+    with pytest.raises(E.RuntimeFailure):
+        eng.step([ok(pos0=10)], out)         # already resident
+    eng.close()
+
+
+def test_introspection_and_memory(models):
+    path = models["tiny-llama-q8"]
+    eng = E.Engine(path, E.EngineConfig(n_ctx=512, n_seq_max=4, n_batch=64, n_ubatch=64))
+    assert eng.vocab_size() == 512 and eng.context_size() == 512 and eng.kv_unified()
+    assert not eng.is_hybrid() and eng.weights_version() == 0
+    mem = eng.memory()
+    assert (mem.n_slots, mem.cells_total, mem.cells_used, mem.recurrent_bytes) == (4, 512, 0, 0)
+    assert mem.kv_bytes > 0
+    # FNV-1a over the path bytes, then the u64 payload size (retro_runtime.hpp:856-868)
+    from gguf_reader import Reader
+    r = Reader(path)
+    from retrograd_amd import gguf_writer as gw
+    size = sum(gw.tensor_nbytes(ne, t) for ne, t, _ in r.tensors.values())
+    h = 14695981039346656037
+    for b in str(path).encode() + size.to_bytes(8, "little"):
+        h = ((h ^ b) * 1099511628211) & (2 ** 64 - 1)
+    assert eng.model_fingerprint() == h
+    assert eng.detokenize_bytes([5, 6]) == b"<t5><t6>"
+    assert not eng.is_eog_token(2) and eng.eos_token() == -1
+    part = E.Engine(path, E.EngineConfig(n_ctx=512, n_seq_max=4, n_batch=64, n_ubatch=64, kv_unified=False))
+    assert part.context_size() == 128 and not part.kv_unified()
+    part.close()
+    eng.close()

@@ -34,7 +34,7 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
                         int32_t n_tokens, int32_t use_tiles, const float * bias, int32_t accumulate, float * y) {
     return guarded([&]() -> int {
         const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
-        DevBuf d_raw, d_packed, d_x, d_xh, d_hi, d_lo, d_y, d_bias;
+        DevBuf d_raw, d_packed, d_x, d_xh, d_xl, d_hi, d_lo, d_y, d_bias;
         d_raw.alloc(bytes);
         ok(hipMemcpy(d_raw.ptr, raw, bytes, hipMemcpyHostToDevice), "upload weights");
         rk::Weight w;
@@ -50,9 +50,10 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
         d_x.alloc((size_t)n_tokens * k * 4);
         ok(hipMemcpy(d_x.ptr, x, d_x.bytes, hipMemcpyHostToDevice), "upload activations");
         d_xh.alloc((size_t)n_tokens * k * 2);
+        d_xl.alloc((size_t)n_tokens * k * 2);
         d_hi.alloc((size_t)n_tokens * (k / 32 + 1) * 2);
         d_lo.alloc((size_t)n_tokens * (k / 32 + 1) * 2);
-        rk::Act act{d_xh.as<__half>(), k % 32 == 0 ? d_hi.as<__half>() : nullptr, k % 32 == 0 ? d_lo.as<__half>() : nullptr, (int)k};
+        rk::Act act{d_xh.as<__half>(), d_xl.as<__half>(), k % 32 == 0 ? d_hi.as<__half>() : nullptr, k % 32 == 0 ? d_lo.as<__half>() : nullptr, (int)k};
         rk::to_act(nullptr, d_x.as<float>(), n_tokens, (int)k, act);
         d_y.alloc((size_t)n_tokens * n_rows * 4);
         ok(hipMemcpy(d_y.ptr, y, d_y.bytes, hipMemcpyHostToDevice), "upload outputs");

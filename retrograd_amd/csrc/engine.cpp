@@ -285,15 +285,17 @@ void Engine::build_buffers() {
     qkv_.alloc((size_t)B * (QD + 2 * KD) * 4);
     gu_.alloc((size_t)B * 2 * F * 4);
     q_half_.alloc((size_t)B * QD * 2);
-    auto act = [&](DevBuf & x, DevBuf & hi, DevBuf & lo, int K) {
+    auto act = [&](DevBuf & x, DevBuf & xl, DevBuf & hi, DevBuf & lo, int K) {
         x.alloc((size_t)B * K * 2);
+        xl.alloc((size_t)B * K * 2);
         hi.alloc((size_t)B * (K / 32 + 1) * 2);
         lo.alloc((size_t)B * (K / 32 + 1) * 2);
     };
-    act(act_e_x_, act_e_hi_, act_e_lo_, E);
-    act(act_q_x_, act_q_hi_, act_q_lo_, QD);
-    act(act_f_x_, act_f_hi_, act_f_lo_, F);
-    act(act_o_x_, act_o_hi_, act_o_lo_, E);
+    act(act_e_x_, act_e_xl_, act_e_hi_, act_e_lo_, E);
+    act(act_q_x_, act_q_xl_, act_q_hi_, act_q_lo_, QD);
+    act(act_f_x_, act_f_xl_, act_f_hi_, act_f_lo_, F);
+    act(act_o_x_, act_o_xl_, act_o_hi_, act_o_lo_, E);
+    q_half_lo_.alloc((size_t)B * QD * 2);
     sample_k_.alloc((size_t)B * 4);
     sample_out_.alloc((size_t)B * sizeof(rk::SampleOut));
     const size_t stage = (size_t)B * (sizeof(rk::RowDesc) + 4) + 65536;
@@ -1032,10 +1034,10 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
     const HParams & h = hp_;
     const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim, F = h.n_ff;
     rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps};
-    rk::Act act_e{act_e_x_.as<__half>(), act_e_hi_.as<__half>(), act_e_lo_.as<__half>(), E};
-    rk::Act act_q{act_q_x_.as<__half>(), act_q_hi_.as<__half>(), act_q_lo_.as<__half>(), QD};
-    rk::Act act_f{act_f_x_.as<__half>(), act_f_hi_.as<__half>(), act_f_lo_.as<__half>(), F};
-    rk::Act act_o{act_o_x_.as<__half>(), act_o_hi_.as<__half>(), act_o_lo_.as<__half>(), E};
+    rk::Act act_e{act_e_x_.as<__half>(), act_e_xl_.as<__half>(), act_e_hi_.as<__half>(), act_e_lo_.as<__half>(), E};
+    rk::Act act_q{act_q_x_.as<__half>(), act_q_xl_.as<__half>(), act_q_hi_.as<__half>(), act_q_lo_.as<__half>(), QD};
+    rk::Act act_f{act_f_x_.as<__half>(), act_f_xl_.as<__half>(), act_f_hi_.as<__half>(), act_f_lo_.as<__half>(), F};
+    rk::Act act_o{act_o_x_.as<__half>(), act_o_xl_.as<__half>(), act_o_hi_.as<__half>(), act_o_lo_.as<__half>(), E};
     if (E % 32 != 0) { act_e.xs_hi = act_e.xs_lo = act_o.xs_hi = act_o.xs_lo = nullptr; }
     if (QD % 32 != 0) { act_q.xs_hi = act_q.xs_lo = nullptr; }
     if (F % 32 != 0) { act_f.xs_hi = act_f.xs_lo = nullptr; }
@@ -1057,8 +1059,8 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
             }
         }
         rk::rope_store(stream_, qkv, T, sh, pk_, L.q_norm.as<float>(), L.k_norm.as<float>(), q_half_.as<__half>(),
-                       k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>());
-        rk::attention(stream_, q_half_.as<__half>(), sh, pk_, table_.as<int32_t>(), max_pages_,
+                       q_half_lo_.as<__half>(), k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>());
+        rk::attention(stream_, q_half_.as<__half>(), q_half_lo_.as<__half>(), sh, pk_, table_.as<int32_t>(), max_pages_,
                       k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), n_items, n_tiles,
                       partial_.as<float>());
         rk::attention_combine(stream_, partial_.as<float>(), T, sh, pk_, act_q);

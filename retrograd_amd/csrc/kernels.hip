@@ -144,14 +144,17 @@ __device__ float decode_elem(int type, const uint8_t * row, int k) {
     }
 }
 
-// Writes up to 32 consecutive activations of one row as f16 and, for a whole
-// block, the sum of the rounded values as hi + lo halves.
-__device__ __forceinline__ void store_act_block(const float * v, int count, __half * x, __half * hi, __half * lo) {
+// Writes up to 32 consecutive activations of one row as f16 hi/lo pairs and,
+// for a whole block, the sum of the stored values as hi + lo halves.
+__device__ __forceinline__ void store_act_block(const float * v, int count, __half * x, __half * x_lo,
+                                                __half * hi, __half * lo) {
     float sum = 0.0f;
     for (int i = 0; i < count; ++i) {
         const __half h = sat_half(v[i]);
+        const __half l = __float2half_rn(fminf(fmaxf(v[i], -65504.0f), 65504.0f) - __half2float(h));
         x[i] = h;
-        sum += __half2float(h);
+        x_lo[i] = l;
+        sum += __half2float(h) + __half2float(l);
     }
     if (hi && count == 32) {
         const __half a = sat_half(sum);
@@ -244,6 +247,7 @@ void repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int 
 struct MMArgs {
     const uint8_t * w;
     const __half * x;
+    const __half * x_lo;
     const __half * xs_hi;
     const __half * xs_lo;
     float * y;
@@ -319,12 +323,14 @@ __global__ __launch_bounds__(256) void k_mm_q4k(MMArgs a) {
     // activation row of this lane for every token tile (clamped: rows past T
     // are computed on the last row and never stored)
     const __half * xrow[NT];
+    const __half * xrow_lo[NT];
     const __half * shi[NT];
     const __half * slo[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int tok = min(tbase + t * 16 + r, a.T - 1);
         xrow[t] = a.x + (size_t)tok * a.K + 8 * g;
+        xrow_lo[t] = a.x_lo + (size_t)tok * a.K + 8 * g;
         shi[t] = a.xs_hi + (size_t)tok * nblk;
         slo[t] = a.xs_lo + (size_t)tok * nblk;
     }
@@ -392,7 +398,9 @@ __global__ __launch_bounds__(256) void k_mm_q4k(MMArgs a) {
                 for (int t = 0; t < NT; ++t) {
                     if (t >= nt) break;
                     const h8 A = load_h8(xrow[t] + sb * 256 + s * 32);
+                    const h8 Al = load_h8(xrow_lo[t] + sb * 256 + s * 32);
                     accq[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, accq[t], 0, 0, 0);
+                    accq[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, B, accq[t], 0, 0, 0);
                 }
             }
 #pragma unroll
@@ -420,10 +428,12 @@ __global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[t] = (f4){0.f, 0.f, 0.f, 0.f};
     const __half * xrow[NT];
+    const __half * xrow_lo[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         const int tok = min(tbase + t * 16 + r, a.T - 1);
         xrow[t] = a.x + (size_t)tok * a.K + 8 * g;
+        xrow_lo[t] = a.x_lo + (size_t)tok * a.K + 8 * g;
     }
     const h2 bias1152 = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
 
@@ -453,7 +463,9 @@ __global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
                     for (int t = 0; t < NT; ++t) {
                         if (t >= nt) break;
                         const h8 A = load_h8(xrow[t] + sb * 256 + s * 32);
-                        const f4 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        const h8 Al = load_h8(xrow_lo[t] + sb * 256 + s * 32);
+                        f4 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, B, part, 0, 0, 0);
 #pragma unroll
                         for (int i = 0; i < 4; ++i) acc[t][i] = fmaf(d, part[i], acc[t][i]);
                     }
@@ -466,7 +478,8 @@ __global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
 
 // Any type, any shape: one wave per output feature, raw GGUF rows.
 __global__ __launch_bounds__(256) void k_mm_generic(int type, const uint8_t * __restrict__ raw, size_t rb,
-                                                    const __half * __restrict__ x, int K, int N, int T,
+                                                    const __half * __restrict__ x,
+                                                    const __half * __restrict__ x_lo, int K, int N, int T,
                                                     float * y, int ldy, int col0, int mode, const float * bias) {
     const int lane = threadIdx.x & 63;
     const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -479,7 +492,8 @@ __global__ __launch_bounds__(256) void k_mm_generic(int type, const uint8_t * __
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int t = min(t0 + j, T - 1);
-                acc[j] = fmaf(w, __half2float(x[(size_t)t * K + k]), acc[j]);
+                const float xv = __half2float(x[(size_t)t * K + k]) + __half2float(x_lo[(size_t)t * K + k]);
+                acc[j] = fmaf(w, xv, acc[j]);
             }
         }
 #pragma unroll
@@ -500,7 +514,7 @@ void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
     if (T <= 0) return;
     hipLaunchKernelGGL(k_mm_generic, dim3((w.N + 3) / 4), dim3(256), 0, s, w.type, w.raw, row_bytes(w.type, w.K),
-                       x.x, w.K, w.N, T, y, ldy, col0, mode, bias);
+                       x.x, x.x_lo, w.K, w.N, T, y, ldy, col0, mode, bias);
     check_launch("matmul_generic");
 }
 
@@ -520,7 +534,7 @@ void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, in
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
     if (w.type == WT_Q4_K && (!x.xs_hi || !x.xs_lo)) throw std::runtime_error("matmul: Q4_K needs block sums");
     MMArgs a;
-    a.w = w.packed; a.x = x.x; a.xs_hi = x.xs_hi; a.xs_lo = x.xs_lo; a.y = y; a.bias = bias;
+    a.w = w.packed; a.x = x.x; a.x_lo = x.x_lo; a.xs_hi = x.xs_hi; a.xs_lo = x.xs_lo; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
     a.n_row_tiles = w.N / 16;
     // Enough waves to cover the chip: split K across the waves of a workgroup
@@ -580,7 +594,7 @@ __global__ __launch_bounds__(256) void k_rmsnorm_act(const float * __restrict__ 
         const int count = min(32, E - k0);
         float v[32];
         for (int i = 0; i < count; ++i) v[i] = (xr[k0 + i] * scale) * w[k0 + i];
-        store_act_block(v, count, out.x + (size_t)o * E + k0,
+        store_act_block(v, count, out.x + (size_t)o * E + k0, out.x_lo + (size_t)o * E + k0,
                         out.xs_hi ? out.xs_hi + (size_t)o * (E / 32) + b : nullptr,
                         out.xs_lo ? out.xs_lo + (size_t)o * (E / 32) + b : nullptr);
     }
@@ -609,7 +623,7 @@ __global__ __launch_bounds__(256) void k_swiglu_act(const float * __restrict__ g
         const float gi = g[i];
         v[i] = (gi / (1.0f + __expf(-gi))) * u[i];
     }
-    store_act_block(v, count, out.x + (size_t)t * F + k0,
+    store_act_block(v, count, out.x + (size_t)t * F + k0, out.x_lo + (size_t)t * F + k0,
                     out.xs_hi ? out.xs_hi + (size_t)t * (F / 32) + b : nullptr,
                     out.xs_lo ? out.xs_lo + (size_t)t * (F / 32) + b : nullptr);
 }
@@ -623,7 +637,7 @@ __global__ __launch_bounds__(256) void k_to_act(const float * __restrict__ x, in
     const int count = min(32, K - k0);
     float v[32];
     for (int i = 0; i < count; ++i) v[i] = x[(size_t)t * K + k0 + i];
-    store_act_block(v, count, out.x + (size_t)t * K + k0,
+    store_act_block(v, count, out.x + (size_t)t * K + k0, out.x_lo + (size_t)t * K + k0,
                     out.xs_hi ? out.xs_hi + (size_t)t * (K / 32) + b : nullptr,
                     out.xs_lo ? out.xs_lo + (size_t)t * (K / 32) + b : nullptr);
 }
@@ -824,6 +838,7 @@ struct RopeArgs {
     const float * q_norm;
     const float * k_norm;
     __half * q_out;
+    __half * q_out_lo;
     __half * k_pool;
     __half * v_pool;
     const int32_t * cell;
@@ -882,9 +897,14 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
         x1 = r1;
     }
     if (is_q) {
-        __half * q = a.q_out + (size_t)t * QD + (size_t)head * a.hd;
-        q[i0] = sat_half(x0 * a.qscale);
-        q[i1] = sat_half(x1 * a.qscale);
+        const size_t at = (size_t)t * QD + (size_t)head * a.hd;
+        const float s0 = fminf(fmaxf(x0 * a.qscale, -65504.0f), 65504.0f);
+        const float s1 = fminf(fmaxf(x1 * a.qscale, -65504.0f), 65504.0f);
+        const __half h0 = __float2half_rn(s0), h1 = __float2half_rn(s1);
+        a.q_out[at + i0] = h0;
+        a.q_out[at + i1] = h1;
+        a.q_out_lo[at + i0] = __float2half_rn(s0 - __half2float(h0));
+        a.q_out_lo[at + i1] = __float2half_rn(s1 - __half2float(h1));
         return;
     }
     const int cell = a.cell[t];
@@ -903,11 +923,13 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
 }
 
 void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, const PackBuffers & pk,
-                const float * q_norm, const float * k_norm, __half * q_out, __half * k_pool, __half * v_pool) {
+                const float * q_norm, const float * k_norm, __half * q_out, __half * q_out_lo,
+                __half * k_pool, __half * v_pool) {
     if (T <= 0) return;
     if (sh.head_dim > 128 || sh.head_dim % 32 != 0) throw std::runtime_error("rope_store: head_dim must be 32, 64, 96 or 128");
     RopeArgs a;
-    a.qkv = qkv; a.q_norm = q_norm; a.k_norm = k_norm; a.q_out = q_out; a.k_pool = k_pool; a.v_pool = v_pool;
+    a.qkv = qkv; a.q_norm = q_norm; a.k_norm = k_norm; a.q_out = q_out; a.q_out_lo = q_out_lo;
+    a.k_pool = k_pool; a.v_pool = v_pool;
     a.cell = pk.cell; a.rope_cos = pk.rope_cos; a.rope_sin = pk.rope_sin;
     a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.hd = sh.head_dim; a.rope_dim = sh.rope_dim; a.neox = sh.rope_neox ? 1 : 0;
     a.eps = sh.eps;
@@ -922,6 +944,7 @@ void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, c
 
 struct AttnArgs {
     const __half * q;
+    const __half * q_lo;
     const __half * k_pool;
     const __half * v_pool;
     const int32_t * table;
@@ -967,11 +990,17 @@ __global__ __launch_bounds__(64) void k_attention(AttnArgs a) {
     const int page_end = min((kv_hi - 1) / PAGE + 1, page_first + SPLIT_PAGES);
 
     const int QD = a.n_head * HD;
-    h8 qreg[KS];
+    h8 qreg[KS], qreg_lo[KS];
 #pragma unroll
     for (int j = 0; j < KS; ++j) {
-        if (col_ok) qreg[j] = load_h8(a.q + (size_t)tq * QD + (size_t)(h * a.G + gi) * HD + 32 * j + 8 * g);
-        else qreg[j] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+        if (col_ok) {
+            const size_t at = (size_t)tq * QD + (size_t)(h * a.G + gi) * HD + 32 * j + 8 * g;
+            qreg[j] = load_h8(a.q + at);
+            qreg_lo[j] = load_h8(a.q_lo + at);
+        } else {
+            qreg[j] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+            qreg_lo[j] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+        }
     }
     f4 o[DT];
 #pragma unroll
@@ -997,6 +1026,8 @@ __global__ __launch_bounds__(64) void k_attention(AttnArgs a) {
         for (int j = 0; j < KS; ++j) {
             s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg[j], s0, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg[j], s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg_lo[j], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg_lo[j], s1, 0, 0, 0);
         }
         // rows of s0 are tokens 4g+i, of s1 tokens 16+4g+i of this page
         const int pbase = pi * PAGE + 4 * g;
@@ -1014,7 +1045,7 @@ __global__ __launch_bounds__(64) void k_attention(AttnArgs a) {
         const float m_use = m_new == -INFINITY ? 0.0f : m_new;
         const float alpha = exp2f(m_run - m_use);       // m_run = -inf -> 0
         float psum = 0.0f;
-        h8 pt;
+        h8 pt, pt_lo;                                   // probabilities as f16 hi/lo pairs
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const float e0 = exp2f(s0[i] - m_use);
@@ -1022,7 +1053,9 @@ __global__ __launch_bounds__(64) void k_attention(AttnArgs a) {
             const _Float16 h0 = (_Float16)e0, h1 = (_Float16)e1;
             pt[i] = h0;
             pt[4 + i] = h1;
-            psum += (float)h0 + (float)h1;              // the sum of what PV really multiplies
+            pt_lo[i] = (_Float16)(e0 - (float)h0);
+            pt_lo[4 + i] = (_Float16)(e1 - (float)h1);
+            psum += e0 + e1;
         }
         l_run = l_run * alpha + psum;
         m_run = m_new;
@@ -1031,6 +1064,7 @@ __global__ __launch_bounds__(64) void k_attention(AttnArgs a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) o[d][i] *= alpha;
             o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt, o[d], 0, 0, 0);
+            o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt_lo, o[d], 0, 0, 0);
         }
     }
     l_run += __shfl_xor(l_run, 16, 64);
@@ -1049,12 +1083,12 @@ size_t attention_partial_floats(int n_items, int head_dim) {
     return (size_t)n_items * 16 * (head_dim + 2);
 }
 
-void attention(hipStream_t s, const __half * q, const AttnShape & sh, const PackBuffers & pk,
+void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnShape & sh, const PackBuffers & pk,
                const int32_t * table, int max_pages, const __half * k_pool, const __half * v_pool,
                int n_items, int n_tiles, float * partial) {
     if (n_items <= 0) return;
     AttnArgs a;
-    a.q = q; a.k_pool = k_pool; a.v_pool = v_pool; a.table = table;
+    a.q = q; a.q_lo = q_lo; a.k_pool = k_pool; a.v_pool = v_pool; a.table = table;
     a.tile_t0 = pk.tile_t0; a.tile_nq = pk.tile_nq; a.tile_item0 = pk.tile_item0; a.tile_nsplit = pk.tile_nsplit;
     a.tile_page0 = pk.tile_page0; a.tile_kv_begin = pk.tile_kv_begin; a.pos = pk.pos; a.seq = pk.seq;
     a.partial = partial; a.n_tiles = n_tiles; a.n_items = n_items; a.max_pages = max_pages;
@@ -1109,12 +1143,17 @@ __global__ __launch_bounds__(256) void k_attention_combine(CombineArgs a) {
     const int QD = a.n_head * a.hd;
     float r0 = 0.0f, r1 = 0.0f;
     if (e0 < a.hd) {
-        const __half h0 = sat_half(v0 * inv), h1 = sat_half(v1 * inv);
-        __half * dst = a.out.x + (size_t)t * QD + (size_t)head * a.hd + e0;
-        dst[0] = h0;
-        dst[1] = h1;
-        r0 = __half2float(h0);
-        r1 = __half2float(h1);
+        const float f0 = fminf(fmaxf(v0 * inv, -65504.0f), 65504.0f);
+        const float f1 = fminf(fmaxf(v1 * inv, -65504.0f), 65504.0f);
+        const __half h0 = __float2half_rn(f0), h1 = __float2half_rn(f1);
+        const __half l0 = __float2half_rn(f0 - __half2float(h0)), l1 = __float2half_rn(f1 - __half2float(h1));
+        const size_t at = (size_t)t * QD + (size_t)head * a.hd + e0;
+        a.out.x[at] = h0;
+        a.out.x[at + 1] = h1;
+        a.out.x_lo[at] = l0;
+        a.out.x_lo[at + 1] = l1;
+        r0 = __half2float(h0) + __half2float(l0);
+        r1 = __half2float(h1) + __half2float(l1);
     }
     if (a.out.xs_hi) {
         // block of 32 outputs = 16 lanes

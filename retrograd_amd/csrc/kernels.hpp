@@ -36,11 +36,15 @@ struct Weight {
     size_t bytes = 0;
 };
 
-// Activations handed to a matmul: f16 rows plus, for every 32-wide block of a
-// row, the f32 sum of the (already rounded) f16 values split into two halves
-// hi + lo. The sums are what the Q4_K min term multiplies.
+// Activations handed to a matmul. An f32 value v travels as two f16 numbers,
+// x = f16(v) and x_lo = f16(v - x), which together carry about 22 significant
+// bits: a single f16 (11 bits) leaves a logit error above the parity
+// tolerance once it has passed through a few layers. For every 32-wide block
+// of a row the f32 sum of x + x_lo is kept as well, split the same way; the
+// sums are what the Q4_K min term multiplies.
 struct Act {
     __half * x = nullptr;       // [T][K]
+    __half * x_lo = nullptr;    // [T][K]
     __half * xs_hi = nullptr;   // [T][K/32], null when K % 32 != 0
     __half * xs_lo = nullptr;
     int K = 0;
@@ -124,14 +128,16 @@ struct AttnShape {
     bool rope_neox;
     float eps;
 };
-// qkv f32 [T][QD + 2*KD] (+ optional per-head RMSNorm weights) -> q f16 [T][QD]
-// (rotated, pre-scaled by log2(e)/sqrt(head_dim)) and K/V pages of the layer.
+// qkv f32 [T][QD + 2*KD] (+ optional per-head RMSNorm weights) -> q as an f16
+// hi/lo pair [T][QD] each (rotated, pre-scaled by log2(e)/sqrt(head_dim)) and
+// the K/V pages of the layer (f16, the KV cache precision).
 void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, const PackBuffers & pk,
-                const float * q_norm, const float * k_norm, __half * q_out, __half * k_pool, __half * v_pool);
+                const float * q_norm, const float * k_norm, __half * q_out, __half * q_out_lo,
+                __half * k_pool, __half * v_pool);
 
 // Split-KV paged attention over the step's query tiles. partial holds, per
 // (item, column), m (log2 domain), l and head_dim unnormalised outputs.
-void attention(hipStream_t s, const __half * q, const AttnShape & sh, const PackBuffers & pk,
+void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnShape & sh, const PackBuffers & pk,
                const int32_t * table, int max_pages, const __half * k_pool, const __half * v_pool,
                int n_items, int n_tiles, float * partial);
 // Merges the splits: out act [T][QD] (+ block sums).

@@ -1,9 +1,10 @@
 """Kernel-level parity on the GPU, through the C ABI of include/retro_kernels.h.
 
 Reference values come from the CPU oracle's block decoders: the same stored
-bytes decoded on the host, multiplied in float64 with the f16-rounded
-activations the kernels consume. Tolerance: the kernels accumulate exact
-f16 x integer products in f32, so 2e-5 of the output scale covers them."""
+bytes decoded on the host, multiplied in float64 with the f32
+activations (the kernels carry them as f16 hi/lo pairs, about 22 bits).
+Tolerance: exact products accumulated in f32, so 2e-5 of the output scale
+covers them."""
 import numpy as np
 import pytest
 import torch
@@ -26,8 +27,8 @@ def _weights(t, n, k, seed):
 
 
 def _ref(dense, x):
-    xh = x.astype(np.float16).astype(np.float64)
-    return xh @ dense.T
+    # activations travel as f16 hi/lo pairs (~22 bits): the f32 input is the reference
+    return x.astype(np.float64) @ dense.T
 
 
 @pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0])

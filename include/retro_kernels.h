@@ -47,6 +47,14 @@ int retro_engine_debug_pack(retro_engine * engine, int32_t * tok, int32_t * pos,
 /* Page id per page index of a slot (-1 = none); out == NULL reports the length. */
 int retro_engine_debug_pages(retro_engine * engine, int32_t slot, int32_t * out, size_t cap, size_t * out_n);
 
+/* HIP-event timing of the step's kernel categories on the engine's own stream:
+ * level 0 off, 1 attention only, 2 every category. Categories, in order: pack,
+ * embed, norm, qkv, rope, attention, combine, o_proj, gate_up, swiglu, down,
+ * head, sample. read() returns accumulated milliseconds and span counts. */
+int retro_engine_debug_profile(retro_engine * engine, int32_t level);
+int32_t retro_engine_debug_profile_categories(void);
+int retro_engine_debug_profile_read(retro_engine * engine, double * out_ms, uint64_t * out_launches, int32_t reset);
+
 #ifdef __cplusplus
 }
 #endif

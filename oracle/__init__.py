@@ -77,6 +77,7 @@ def _declare(l: C.CDLL) -> None:
     l.orc_ctx_seq_cp.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_ctx_seq_pos.argtypes = [C.c_void_p, C.c_int, _i32p, _i32p]
     l.orc_ctx_read_kv.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _u16p]
+    l.orc_ctx_import_kv.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _u16p, _u16p]
     l.orc_rng_new.argtypes = [C.c_uint32]
     l.orc_rng_new.restype = C.c_void_p
     l.orc_rng_free.argtypes = [C.c_void_p]
@@ -271,6 +272,25 @@ class Context:
         out = np.empty(self.model.n_head_kv * self.model.head_dim, np.uint16)
         _check(lib().orc_ctx_read_kv(self._h, layer, slot, pos, 1 if want_v else 0, _ptr(out, _u16p)))
         return out.view(np.float16)
+
+    def import_kv(self, layer, slot, begin, end, k_rows: np.ndarray, v_rows: np.ndarray) -> None:
+        k = np.ascontiguousarray(k_rows).view(np.uint16)
+        v = np.ascontiguousarray(v_rows).view(np.uint16)
+        _check(lib().orc_ctx_import_kv(self._h, layer, slot, begin, end, _ptr(k, _u16p), _ptr(v, _u16p)))
+
+    def import_snapshot(self, slot: int, snapshot: bytes) -> None:
+        """Loads a sequence snapshot written by the engine's seq_save (header of
+        six 32-bit words: magic, flags, n_layer, kv_dim, begin, end; then per
+        layer the K rows and the V rows as f16)."""
+        head = np.frombuffer(snapshot, np.int32, 6)
+        n_layer, kd, begin, end = (int(v) for v in head[2:6])
+        n = end - begin
+        body = np.frombuffer(snapshot, np.uint16, offset=24)
+        per = n * kd
+        for l in range(n_layer):
+            k = body[(2 * l) * per:(2 * l + 1) * per]
+            v = body[(2 * l + 1) * per:(2 * l + 2) * per]
+            self.import_kv(l, slot, begin, end, k, v)
 
     def close(self) -> None:
         if self._h:

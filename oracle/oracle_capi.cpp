@@ -162,6 +162,26 @@ int orc_ctx_read_kv(void * c, int layer, int slot, int pos, int want_v, uint16_t
     });
 }
 
+// Installs f16 K and V rows of positions [begin, end) of one layer of a slot
+// (rows of kv_dim halves): lets a decode step be checked or timed at a long
+// context without running the prefill on the CPU first.
+int orc_ctx_import_kv(void * c, int layer, int slot, int begin, int end, const uint16_t * k_rows,
+                      const uint16_t * v_rows) {
+    return guard([&] {
+        context * ctx = (context *)c;
+        slot_state & s = ctx->slots.at((size_t)slot);
+        const size_t kd = (size_t)ctx->kv_dim();
+        auto & kk = s.k.at((size_t)layer);
+        auto & vv = s.v.at((size_t)layer);
+        if (kk.size() < (size_t)end * kd) { kk.resize((size_t)end * kd); vv.resize((size_t)end * kd); }
+        std::copy(k_rows, k_rows + (size_t)(end - begin) * kd, kk.begin() + (size_t)begin * kd);
+        std::copy(v_rows, v_rows + (size_t)(end - begin) * kd, vv.begin() + (size_t)begin * kd);
+        s.begin = begin;
+        s.end = end;
+        return 0;
+    });
+}
+
 // ---- sampling --------------------------------------------------------------
 void * orc_rng_new(uint32_t seed) { return new std::mt19937(seed); }
 void orc_rng_free(void * r) { delete (std::mt19937 *)r; }

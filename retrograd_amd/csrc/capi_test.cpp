@@ -123,6 +123,24 @@ int retro_engine_debug_pack(retro_engine * engine, int32_t * tok, int32_t * pos,
     });
 }
 
+int retro_engine_debug_profile(retro_engine * engine, int32_t level) {
+    return guarded([&]() -> int {
+        if (!engine) { set_error("engine is required"); return -1; }
+        engine->impl.profile_level(level);
+        return 0;
+    });
+}
+
+int32_t retro_engine_debug_profile_categories(void) { return retro::PC_COUNT; }
+
+int retro_engine_debug_profile_read(retro_engine * engine, double * out_ms, uint64_t * out_launches, int32_t reset) {
+    return guarded([&]() -> int {
+        if (!engine) { set_error("engine is required"); return -1; }
+        engine->impl.profile_read(out_ms, out_launches, reset != 0);
+        return 0;
+    });
+}
+
 int retro_engine_debug_pages(retro_engine * engine, int32_t slot, int32_t * out, size_t cap, size_t * out_n) {
     return guarded([&]() -> int {
         if (!engine) { set_error("engine is required"); return -1; }

@@ -106,6 +106,7 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
 }
 
 Engine::~Engine() {
+    for (hipEvent_t e : prof_events_) (void)hipEventDestroy(e);
     if (stream_) {
         (void)hipStreamSynchronize(stream_);
         (void)hipStreamDestroy(stream_);
@@ -328,7 +329,7 @@ void Engine::copy_page(int32_t src, int32_t dst) {
 
 void Engine::set_page(int32_t slot, int idx, int32_t page) {
     slots_[(size_t)slot].pages[(size_t)idx] = page;
-    pending_updates_.push_back({slot, idx, page, 0});
+    pending_updates_[(int64_t)slot * max_pages_ + idx] = page;
 }
 
 void Engine::clear_slot(Slot & s, int32_t slot) {
@@ -875,6 +876,16 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
         s.end = last;
     }
 
+    // Every resident position of a slot the step reads must have a page: a
+    // missing one would send a kernel outside the pool.
+    for (const RowView & row : rows) {
+        const Slot & s = slots_[(size_t)row.slot];
+        for (int idx = s.begin / rk::PAGE; idx <= (s.end - 1) / rk::PAGE; ++idx) {
+            const int32_t pg = s.pages[(size_t)idx];
+            if (pg < 0 || pg >= n_pages_) throw std::runtime_error("internal error: a resident position has no KV page");
+        }
+    }
+
     // ---- upload the plan and pack it on the device
     const int T = (int)total;
     const size_t n_upd = pending_updates_.size();
@@ -898,18 +909,26 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
             if (row.sample) ++n_out;
         }
     }
-    if (n_upd) std::memcpy((uint8_t *)h_stage_.ptr + off_upd, pending_updates_.data(), n_upd * sizeof(rk::TableUpdate));
-    pending_updates_.clear();
+    {
+        rk::TableUpdate * hu = (rk::TableUpdate *)((uint8_t *)h_stage_.ptr + off_upd);
+        size_t i = 0;
+        for (const auto & kv : pending_updates_) {
+            hu[i++] = {(int32_t)(kv.first / max_pages_), (int32_t)(kv.first % max_pages_), kv.second, 0};
+        }
+        pending_updates_.clear();
+    }
     int n_tiles = 0, n_items = 0;
     rk::count_attention_work(hd, (int)n_rows, qt_, hp_.n_head_kv, &n_tiles, &n_items);
 
     try {
         hip_check(hipMemcpyAsync(d_stage_.ptr, h_stage_.ptr, stage_bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
+        const size_t pt_pack = prof_begin(PC_PACK);
         rk::pack_step(stream_, d_stage_.as<rk::RowDesc>(), (int)n_rows,
                       (const int32_t *)((const uint8_t *)d_stage_.ptr + off_tok),
                       (const rk::TableUpdate *)((const uint8_t *)d_stage_.ptr + off_upd), (int)n_upd,
                       table_.as<int32_t>(), max_pages_, qt_, hp_.n_head_kv, inv_freq_.as<double>(),
                       hp_.rope_dim / 2, pk_);
+        prof_end(PC_PACK, pt_pack);
         forward(T, n_out, n_tiles, n_items);
 
         // ---- sampling: the device scans the vocabulary, the host draws.
@@ -931,7 +950,9 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
         }
         if (n_out > 0) {
             hip_check(hipMemcpyAsync(sample_k_.ptr, kreq.data(), (size_t)n_out * 4, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
+            const size_t pt_s = prof_begin(PC_SAMPLE);
             rk::sample_prepare(stream_, logits_.as<float>(), n_out, n_vocab, sample_k_.as<int32_t>(), sample_out_.as<rk::SampleOut>());
+            prof_end(PC_SAMPLE, pt_s);
             hip_check(hipMemcpyAsync(h_sample_.ptr, sample_out_.ptr, (size_t)n_out * sizeof(rk::SampleOut), hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync");
             if (any_full) {
                 h_logits_.ensure((size_t)n_out * n_vocab * 4);
@@ -944,6 +965,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
             }
         }
         hip_check(hipStreamSynchronize(stream_), "step");
+        if (prof_level_) prof_resolve();
         last_n_out_ = n_out;
         ++steps_run_;
 
@@ -1046,26 +1068,39 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
     float * qkv = qkv_.as<float>();
     float * gu = gu_.as<float>();
 
-    rk::embed(stream_, tok_embd_.w, pk_.tok, T, x);
+    { const size_t pt_ = prof_begin(PC_EMBED); rk::embed(stream_, tok_embd_.w, pk_.tok, T, x); prof_end(PC_EMBED, pt_); }
     for (int l = 0; l < h.n_layer; ++l) {
         const LayerWeights & L = layers_[(size_t)l];
-        rk::rmsnorm_act(stream_, x, L.attn_norm.as<float>(), E, h.eps, nullptr, T, act_e);
+        { const size_t pt_ = prof_begin(PC_NORM); rk::rmsnorm_act(stream_, x, L.attn_norm.as<float>(), E, h.eps, nullptr, T, act_e); prof_end(PC_NORM, pt_); }
         {
+            const size_t pt_ = prof_begin(PC_QKV);
             int col = 0;
             for (const DevWeight & w : L.qkv) {
                 rk::matmul(stream_, w.w, act_e, T, qkv, QD + 2 * KD, col, rk::MM_STORE,
                            L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr);
                 col += w.w.N;
             }
+            prof_end(PC_QKV, pt_);
         }
+        size_t pt_ = prof_begin(PC_ROPE);
         rk::rope_store(stream_, qkv, T, sh, pk_, L.q_norm.as<float>(), L.k_norm.as<float>(), q_half_.as<__half>(),
                        q_half_lo_.as<__half>(), k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>());
+        prof_end(PC_ROPE, pt_);
+        pt_ = prof_begin(PC_ATTN);
         rk::attention(stream_, q_half_.as<__half>(), q_half_lo_.as<__half>(), sh, pk_, table_.as<int32_t>(), max_pages_,
                       k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), n_items, n_tiles,
                       partial_.as<float>());
+        prof_end(PC_ATTN, pt_);
+        pt_ = prof_begin(PC_COMBINE);
         rk::attention_combine(stream_, partial_.as<float>(), T, sh, pk_, act_q);
+        prof_end(PC_COMBINE, pt_);
+        pt_ = prof_begin(PC_OPROJ);
         rk::matmul(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr);
+        prof_end(PC_OPROJ, pt_);
+        pt_ = prof_begin(PC_NORM);
         rk::rmsnorm_act(stream_, x, L.ffn_norm.as<float>(), E, h.eps, nullptr, T, act_e);
+        prof_end(PC_NORM, pt_);
+        pt_ = prof_begin(PC_GATEUP);
         {
             int col = 0;
             for (const DevWeight & w : L.gate_up) {
@@ -1073,14 +1108,64 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
                 col += w.w.N;
             }
         }
+        prof_end(PC_GATEUP, pt_);
+        pt_ = prof_begin(PC_SWIGLU);
         rk::swiglu_act(stream_, gu, T, F, act_f);
+        prof_end(PC_SWIGLU, pt_);
+        pt_ = prof_begin(PC_DOWN);
         rk::matmul(stream_, L.down.w, act_f, T, x, E, 0, rk::MM_ADD, nullptr);
+        prof_end(PC_DOWN, pt_);
     }
     if (n_out > 0) {
         logits_.ensure((size_t)n_out * h.n_vocab * 4);
+        const size_t pt_ = prof_begin(PC_HEAD);
         rk::rmsnorm_act(stream_, x, out_norm_.as<float>(), E, h.eps, pk_.out_tok, n_out, act_o);
         rk::matmul(stream_, lm_head_.w, act_o, n_out, logits_.as<float>(), h.n_vocab, 0, rk::MM_STORE,
                    out_bias_.as<float>());
+        prof_end(PC_HEAD, pt_);
+    }
+}
+
+// ---- event timing -------------------------------------------------------------------------
+
+size_t Engine::prof_begin(int cat) {
+    if (prof_level_ == 0 || (prof_level_ == 1 && cat != PC_ATTN)) return (size_t)-1;
+    if (prof_used_ + 2 > prof_events_.size()) {
+        for (int i = 0; i < 2; ++i) {
+            hipEvent_t e;
+            hip_check(hipEventCreate(&e), "hipEventCreate");
+            prof_events_.push_back(e);
+        }
+    }
+    const size_t a = prof_used_;
+    prof_used_ += 2;
+    hip_check(hipEventRecord(prof_events_[a], stream_), "hipEventRecord");
+    return a;
+}
+
+void Engine::prof_end(int cat, size_t token) {
+    if (token == (size_t)-1) return;
+    hip_check(hipEventRecord(prof_events_[token + 1], stream_), "hipEventRecord");
+    prof_spans_.push_back({cat, token, token + 1});
+}
+
+void Engine::prof_resolve() {
+    for (const ProfSpan & sp : prof_spans_) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, prof_events_[sp.a], prof_events_[sp.b]) == hipSuccess) {
+            prof_ms_[sp.cat] += ms;
+            prof_n_[sp.cat] += 1;
+        }
+    }
+    prof_spans_.clear();
+    prof_used_ = 0;
+}
+
+void Engine::profile_read(double * ms, uint64_t * launches, bool reset) {
+    for (int c = 0; c < PC_COUNT; ++c) {
+        ms[c] = prof_ms_[c];
+        launches[c] = prof_n_[c];
+        if (reset) { prof_ms_[c] = 0.0; prof_n_[c] = 0; }
     }
 }
 

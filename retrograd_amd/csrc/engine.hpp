@@ -14,6 +14,7 @@
 #include <memory>
 #include <queue>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 namespace retro {
@@ -80,6 +81,12 @@ struct Vocab {
     int32_t eos = -1, eot = -1;
 };
 
+// Kernel categories of one step, for the optional event-based timing.
+enum ProfCat : int {
+    PC_PACK = 0, PC_EMBED, PC_NORM, PC_QKV, PC_ROPE, PC_ATTN, PC_COMBINE, PC_OPROJ, PC_GATEUP, PC_SWIGLU,
+    PC_DOWN, PC_HEAD, PC_SAMPLE, PC_COUNT
+};
+
 class Engine {
 public:
     Engine(const std::string & path, const retro_engine_config & config);
@@ -105,6 +112,10 @@ public:
     uint64_t weights_version() const { return weights_version_; }
     uint64_t fingerprint() const { return fingerprint_; }
     uint64_t steps_run() const { return steps_run_; }
+
+    // Event timing of kernel categories: level 0 off, 1 attention only, 2 all.
+    void profile_level(int level) { prof_level_ = level; }
+    void profile_read(double * ms, uint64_t * launches, bool reset);
 
     // Test hooks: copies of device state.
     int debug_last_logits(float * out, size_t n_floats, size_t * out_rows);
@@ -167,7 +178,11 @@ private:
     std::vector<Slot> slots_;
     std::vector<int32_t> page_ref_;
     std::priority_queue<int32_t, std::vector<int32_t>, std::greater<int32_t>> free_pages_;
-    std::vector<rk::TableUpdate> pending_updates_;
+    // Device block-table entries that changed since the last step, keyed by
+    // slot * max_pages + index so that only the LAST value of an entry is
+    // uploaded: the packing kernel applies the list with one thread per entry,
+    // in no particular order.
+    std::unordered_map<int64_t, int32_t> pending_updates_;
 
     // per-step device buffers
     DevBuf d_stage_;          // rows | tokens | table updates, as uploaded
@@ -182,6 +197,18 @@ private:
     DevBuf q_half_lo_;
     HostPinned h_sample_, h_logits_;
     int last_n_out_ = 0;
+
+    // event timing
+    struct ProfSpan { int cat; size_t a, b; };
+    int prof_level_ = 0;
+    std::vector<hipEvent_t> prof_events_;
+    size_t prof_used_ = 0;
+    std::vector<ProfSpan> prof_spans_;
+    double prof_ms_[PC_COUNT] = {};
+    uint64_t prof_n_[PC_COUNT] = {};
+    size_t prof_begin(int cat);
+    void prof_end(int cat, size_t token);
+    void prof_resolve();
 
     std::map<int32_t, RequestState> requests_;
     sampling::FullScratch scratch_;

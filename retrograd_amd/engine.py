@@ -122,7 +122,10 @@ STEP_SYMBOLS = [
 KERNEL_SYMBOLS = [
     "retro_kernel_matmul", "retro_kernel_sample_prepare", "retro_kernel_page_size", "retro_kernel_max_topk",
     "retro_engine_debug_logits", "retro_engine_debug_kv", "retro_engine_debug_pack", "retro_engine_debug_pages",
+    "retro_engine_debug_profile", "retro_engine_debug_profile_categories", "retro_engine_debug_profile_read",
 ]
+PROFILE_CATEGORIES = ["pack", "embed", "norm", "qkv", "rope", "attention", "combine", "o_proj", "gate_up", "swiglu",
+                      "down", "head", "sample"]
 
 _lib = None
 _i32p, _f32p, _u8p = C.POINTER(C.c_int32), C.POINTER(C.c_float), C.POINTER(C.c_uint8)
@@ -194,6 +197,9 @@ def load_library() -> C.CDLL:
     lib.retro_engine_debug_pack.argtypes = [C.c_void_p, _i32p, _i32p, _i32p, _i32p, _i32p, _i32p, C.c_size_t,
                                             C.c_size_t, _i32p]
     lib.retro_engine_debug_pages.argtypes = [C.c_void_p, C.c_int32, _i32p, C.c_size_t, C.POINTER(C.c_size_t)]
+    lib.retro_engine_debug_profile.argtypes = [C.c_void_p, C.c_int32]
+    lib.retro_engine_debug_profile_categories.restype = C.c_int32
+    lib.retro_engine_debug_profile_read.argtypes = [C.c_void_p, C.POINTER(C.c_double), C.POINTER(C.c_uint64), C.c_int32]
     _lib = lib
     return lib
 
@@ -633,6 +639,22 @@ class Engine:
         out["last_index"] = last
         out["counts"] = counts
         return out
+
+    def profile(self, level: int) -> None:
+        """HIP-event timing of kernel categories: 0 off, 1 attention only, 2 all."""
+        s = self._lib.retro_engine_debug_profile(self._h, level)
+        if s != 0:
+            _raise(s)
+
+    def profile_read(self, reset: bool = True) -> dict:
+        n = self._lib.retro_engine_debug_profile_categories()
+        assert n == len(PROFILE_CATEGORIES)
+        ms = (C.c_double * n)()
+        cnt = (C.c_uint64 * n)()
+        s = self._lib.retro_engine_debug_profile_read(self._h, ms, cnt, 1 if reset else 0)
+        if s != 0:
+            _raise(s)
+        return {name: (ms[i], int(cnt[i])) for i, name in enumerate(PROFILE_CATEGORIES)}
 
     def debug_pages(self, slot: int) -> np.ndarray:
         n = C.c_size_t()

@@ -161,6 +161,25 @@ def test_seq_cp_seq_rm_and_snapshots(models):
     eng.close()
 
 
+def test_slot_reuse_after_removal(models):
+    # A slot is emptied and refilled between two steps: its block-table entries
+    # change twice (to "none", then to new pages) before the device sees them.
+    eng, ctx, m = _pair(models["llama-q4k"], n_seq=4, n_ctx=512, n_batch=128)
+    rng = np.random.default_rng(9)
+    for cycle in range(4):
+        n = int(rng.integers(20, 90))
+        toks = rng.integers(0, m.n_vocab, n)
+        slot = cycle % 2
+        eng.seq_rm(slot)
+        ctx.seq_rm(slot)
+        o, got, want = run_both(eng, ctx, [(cycle, slot, toks, 0, True)])
+        assert_logits_close(got, want)
+        o, got, want = run_both(eng, ctx, [(cycle, slot, [int(want[0].argmax())], n, True)])
+        assert_logits_close(got, want)
+        eng.request_free(cycle)
+    eng.close()
+
+
 def test_step_argument_errors_are_reported_before_decoding(models):
     eng, ctx, m = _pair(models["tiny-llama-q8"], n_seq=4, n_ctx=256, n_batch=32)
     out = E.StepOutput()

@@ -16,8 +16,9 @@ extern "C" {
 #endif
 
 /* y[t][n] (=|+=) sum_k W[n][k] * f16(x[t][k]) (+ bias[n]) with W given as
- * n_rows raw GGUF rows of `type`. use_tiles selects the MFMA tile kernel
- * (K % 256 == 0, n_rows % 16 == 0, Q4_K or Q8_0) instead of the generic one.
+ * n_rows raw GGUF rows of `type`. use_tiles = 0 runs the generic kernel, 1 the
+ * register-only MFMA tile kernel, 2 the LDS-staged MFMA tile kernel (tiles need
+ * K % 256 == 0, n_rows % 16 == 0, Q4_K or Q8_0).
  * y is [n_tokens][n_rows] and is read first when accumulate is set. */
 int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x,
                         int32_t n_tokens, int32_t use_tiles, const float * bias, int32_t accumulate, float * y);
@@ -28,6 +29,12 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
 int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_vocab, const int32_t * k,
                                 int32_t * out_argmax, float * out_max, double * out_sum_exp,
                                 int32_t * out_top_ids, float * out_top_logits);
+
+/* Micro-benchmark: microseconds per launch of one tile matmul (mode 1 register
+ * tiles, 2 LDS-staged tiles) over `iters` back-to-back launches on device-only
+ * data. debug and force_ksplit are timing experiments (0 = normal). */
+int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,
+                             int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us);
 
 int32_t retro_kernel_page_size(void);   /* positions per KV page */
 int32_t retro_kernel_max_topk(void);    /* candidates sample_prepare can return */

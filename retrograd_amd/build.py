@@ -15,8 +15,8 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libretro_hip.so"
-SOURCES = ["kernels.hip", "engine.cpp", "capi.cpp", "capi_test.cpp"]
-HEADERS = ["kernels.hpp", "engine.hpp", "sampler.hpp", "gguf_file.hpp"]
+SOURCES = ["kernels.hip", "mm_lds.hip", "engine.cpp", "capi.cpp", "capi_test.cpp"]
+HEADERS = ["kernels.hpp", "dev_common.hpp", "engine.hpp", "sampler.hpp", "gguf_file.hpp"]
 
 # packed-fp32 code generation is switched off for every HIP translation unit.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wextra",

@@ -61,8 +61,13 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
             d_bias.alloc((size_t)n_rows * 4);
             ok(hipMemcpy(d_bias.ptr, bias, d_bias.bytes, hipMemcpyHostToDevice), "upload bias");
         }
+        DevBuf d_ws;
+        if (use_tiles == 2) {
+            d_ws.alloc(rk::matmul_workspace_bytes());
+            ok(hipMemset(d_ws.ptr, 0, d_ws.bytes), "clear workspace");
+        }
         rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, accumulate ? rk::MM_ADD : rk::MM_STORE,
-                   d_bias.as<float>());
+                   d_bias.as<float>(), d_ws.ptr);
         ok(hipDeviceSynchronize(), "matmul");
         ok(hipMemcpy(y, d_y.ptr, d_y.bytes, hipMemcpyDeviceToHost), "download outputs");
         return 0;
@@ -92,6 +97,46 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
                 out_top_logits[r * rk::MAX_TOPK + j] = j < k[r] ? h[(size_t)r].top_logit[j] : 0.0f;
             }
         }
+        return 0;
+    });
+}
+
+// Times `iters` launches of one tile matmul on random device data with HIP
+// events; returns microseconds per launch through out_us.
+int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,
+                             int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us) {
+    return guarded([&]() -> int {
+        const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
+        DevBuf d_w, d_xh, d_xl, d_hi, d_lo, d_y, d_ws;
+        d_w.alloc(bytes);
+        ok(hipMemset(d_w.ptr, 0x11, bytes), "fill");
+        d_xh.alloc((size_t)n_tokens * k * 2); d_xl.alloc((size_t)n_tokens * k * 2);
+        d_hi.alloc((size_t)n_tokens * (k / 32 + 1) * 2); d_lo.alloc((size_t)n_tokens * (k / 32 + 1) * 2);
+        ok(hipMemset(d_xh.ptr, 0, d_xh.bytes), "fill"); ok(hipMemset(d_xl.ptr, 0, d_xl.bytes), "fill");
+        ok(hipMemset(d_hi.ptr, 0, d_hi.bytes), "fill"); ok(hipMemset(d_lo.ptr, 0, d_lo.bytes), "fill");
+        d_y.alloc((size_t)n_tokens * n_rows * 4);
+        d_ws.alloc(rk::matmul_workspace_bytes());
+        ok(hipMemset(d_ws.ptr, 0, d_ws.bytes), "fill");
+        rk::Weight w;
+        w.type = type; w.K = (int)k; w.N = (int)n_rows; w.bytes = bytes; w.packed = d_w.as<uint8_t>();
+        rk::Act act{d_xh.as<__half>(), d_xl.as<__half>(), d_hi.as<__half>(), d_lo.as<__half>(), (int)k};
+        rk::g_mm_debug = debug;
+        rk::g_mm_force_ksplit = force_ksplit & 0xff;
+        rk::g_mm_force_r = force_ksplit >> 8;
+        hipEvent_t e0, e1;
+        ok(hipEventCreate(&e0), "event"); ok(hipEventCreate(&e1), "event");
+        for (int i = 0; i < 3; ++i) rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, mode == 2 ? d_ws.ptr : nullptr);
+        ok(hipEventRecord(e0, nullptr), "record");
+        for (int i = 0; i < iters; ++i) rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, mode == 2 ? d_ws.ptr : nullptr);
+        ok(hipEventRecord(e1, nullptr), "record");
+        ok(hipEventSynchronize(e1), "sync");
+        float ms = 0;
+        ok(hipEventElapsedTime(&ms, e0, e1), "elapsed");
+        rk::g_mm_debug = 0;
+        rk::g_mm_force_ksplit = 0;
+        rk::g_mm_force_r = 0;
+        (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+        *out_us = (double)ms * 1e3 / iters;
         return 0;
     });
 }

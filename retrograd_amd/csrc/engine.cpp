@@ -297,6 +297,8 @@ void Engine::build_buffers() {
     act(act_f_x_, act_f_xl_, act_f_hi_, act_f_lo_, F);
     act(act_o_x_, act_o_xl_, act_o_hi_, act_o_lo_, E);
     q_half_lo_.alloc((size_t)B * QD * 2);
+    mm_ws_.alloc(rk::matmul_workspace_bytes());
+    hip_check(hipMemsetAsync(mm_ws_.ptr, 0, mm_ws_.bytes, stream_), "hipMemsetAsync");
     sample_k_.alloc((size_t)B * 4);
     sample_out_.alloc((size_t)B * sizeof(rk::SampleOut));
     const size_t stage = (size_t)B * (sizeof(rk::RowDesc) + 4) + 65536;
@@ -1077,7 +1079,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
             int col = 0;
             for (const DevWeight & w : L.qkv) {
                 rk::matmul(stream_, w.w, act_e, T, qkv, QD + 2 * KD, col, rk::MM_STORE,
-                           L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr);
+                           L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr, mm_ws_.ptr);
                 col += w.w.N;
             }
             prof_end(PC_QKV, pt_);
@@ -1095,7 +1097,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
         rk::attention_combine(stream_, partial_.as<float>(), T, sh, pk_, act_q);
         prof_end(PC_COMBINE, pt_);
         pt_ = prof_begin(PC_OPROJ);
-        rk::matmul(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr);
+        rk::matmul(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
         prof_end(PC_OPROJ, pt_);
         pt_ = prof_begin(PC_NORM);
         rk::rmsnorm_act(stream_, x, L.ffn_norm.as<float>(), E, h.eps, nullptr, T, act_e);
@@ -1104,7 +1106,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
         {
             int col = 0;
             for (const DevWeight & w : L.gate_up) {
-                rk::matmul(stream_, w.w, act_e, T, gu, 2 * F, col, rk::MM_STORE, nullptr);
+                rk::matmul(stream_, w.w, act_e, T, gu, 2 * F, col, rk::MM_STORE, nullptr, mm_ws_.ptr);
                 col += w.w.N;
             }
         }
@@ -1113,7 +1115,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
         rk::swiglu_act(stream_, gu, T, F, act_f);
         prof_end(PC_SWIGLU, pt_);
         pt_ = prof_begin(PC_DOWN);
-        rk::matmul(stream_, L.down.w, act_f, T, x, E, 0, rk::MM_ADD, nullptr);
+        rk::matmul(stream_, L.down.w, act_f, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
         prof_end(PC_DOWN, pt_);
     }
     if (n_out > 0) {
@@ -1121,7 +1123,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
         const size_t pt_ = prof_begin(PC_HEAD);
         rk::rmsnorm_act(stream_, x, out_norm_.as<float>(), E, h.eps, pk_.out_tok, n_out, act_o);
         rk::matmul(stream_, lm_head_.w, act_o, n_out, logits_.as<float>(), h.n_vocab, 0, rk::MM_STORE,
-                   out_bias_.as<float>());
+                   out_bias_.as<float>(), mm_ws_.ptr);
         prof_end(PC_HEAD, pt_);
     }
 }

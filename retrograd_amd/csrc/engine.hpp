@@ -195,6 +195,7 @@ private:
     DevBuf act_f_x_, act_f_xl_, act_f_hi_, act_f_lo_;       // n_ff wide
     DevBuf act_o_x_, act_o_xl_, act_o_hi_, act_o_lo_;       // output rows, n_embd wide
     DevBuf q_half_lo_;
+    DevBuf mm_ws_;            // matmul workspace: split-K partials, counters, zeros
     HostPinned h_sample_, h_logits_;
     int last_n_out_ = 0;
 

@@ -29,31 +29,9 @@
 // result holds rows 4*(l/16)+i, column l%16. Both operands always use the same
 // (lane group, slot) for the same logical k, so the hardware's internal k
 // order never matters.
-#include "kernels.hpp"
-
-#include <stdexcept>
-#include <string>
+#include "dev_common.hpp"
 
 namespace rk {
-
-typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-typedef _Float16 h8 __attribute__((ext_vector_type(8)));
-typedef float f4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-
-#define HIP_OK(expr)                                                                        \
-    do {                                                                                    \
-        hipError_t err__ = (expr);                                                          \
-        if (err__ != hipSuccess)                                                            \
-            throw std::runtime_error(std::string("HIP error: ") + hipGetErrorString(err__)  \
-                                     + " at " #expr);                                       \
-    } while (0)
-
-static inline void check_launch(const char * what) {
-    hipError_t err = hipGetLastError();
-    if (err != hipSuccess)
-        throw std::runtime_error(std::string("kernel launch failed (") + what + "): " + hipGetErrorString(err));
-}
 
 BlockGeom geom_of(int type) {
     switch (type) {
@@ -79,22 +57,6 @@ bool can_pack(int type, int64_t K, int64_t N) {
 
 // ---------------------------------------------------------------------------
 // small device helpers
-
-__device__ __forceinline__ float h2f(uint16_t bits) {
-    return __half2float(__ushort_as_half(bits));
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
-}
-
-// f32 -> f16 with saturation, so nothing non-finite is ever stored.
-__device__ __forceinline__ __half sat_half(float v) {
-    v = fminf(fmaxf(v, -65504.0f), 65504.0f);
-    return __float2half_rn(v);
-}
 
 // One element of a raw GGUF row, decoded exactly as the stored blocks define
 // it (two roundings for d*q - m, no contraction).
@@ -160,6 +122,34 @@ __device__ __forceinline__ void store_act_block(const float * v, int count, __ha
         const __half a = sat_half(sum);
         *hi = a;
         *lo = __float2half_rn(sum - __half2float(a));
+    }
+}
+
+// Eight consecutive activations per lane: hi/lo pairs as two 16-byte stores; the
+// four lanes that own one 32-wide block add their sums with two xor-shuffles.
+__device__ __forceinline__ void store_act8(const float (&v)[8], __half * x, __half * x_lo, __half * hi, __half * lo,
+                                           int lane_in_block) {
+    h8 a, b;
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float c = fminf(fmaxf(v[i], -65504.0f), 65504.0f);
+        const _Float16 h = (_Float16)c;
+        const _Float16 l = (_Float16)(c - (float)h);
+        a[i] = h;
+        b[i] = l;
+        sum += (float)h + (float)l;
+    }
+    *(h8 *)x = a;
+    *(h8 *)x_lo = b;
+    if (hi) {
+        sum += __shfl_xor(sum, 1, 64);
+        sum += __shfl_xor(sum, 2, 64);
+        if (lane_in_block == 0) {
+            const __half s = sat_half(sum);
+            *hi = s;
+            *lo = __float2half_rn(sum - __half2float(s));
+        }
     }
 }
 
@@ -244,22 +234,6 @@ void repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int 
 // ---------------------------------------------------------------------------
 // matmul over tiled quantised weights (MFMA)
 
-struct MMArgs {
-    const uint8_t * w;
-    const __half * x;
-    const __half * x_lo;
-    const __half * xs_hi;
-    const __half * xs_lo;
-    float * y;
-    const float * bias;
-    int K, N, T, ldy, col0, mode;
-    int n_row_tiles;
-    int ksplit;       // waves of a workgroup that share one row tile along K (1, 2 or 4)
-};
-
-__device__ __forceinline__ h8 load_h8(const __half * p) {
-    return *(const h8 *)p;
-}
 
 template <int NT>
 __device__ __forceinline__ void mm_finish(const MMArgs & a, f4 (&acc)[NT], int rt, int tbase, int nt,
@@ -368,7 +342,6 @@ __global__ __launch_bounds__(256) void k_mm_q4k(MMArgs a) {
                 for (int i = 0; i < 8; ++i) mB[i] = g < 2 ? (_Float16)(float)mn[i] : (_Float16)0.0f;
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    if (t >= nt) break;
                     h8 sA = (h8){0, 0, 0, 0, 0, 0, 0, 0};
                     if (g == 0) sA = load_h8(shi[t] + sb * 8);
                     else if (g == 1) sA = load_h8(slo[t] + sb * 8);
@@ -396,7 +369,6 @@ __global__ __launch_bounds__(256) void k_mm_q4k(MMArgs a) {
                 const h8 B = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    if (t >= nt) break;
                     const h8 A = load_h8(xrow[t] + sb * 256 + s * 32);
                     const h8 Al = load_h8(xrow_lo[t] + sb * 256 + s * 32);
                     accq[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, accq[t], 0, 0, 0);
@@ -461,7 +433,6 @@ __global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
                     const h8 B = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
 #pragma unroll
                     for (int t = 0; t < NT; ++t) {
-                        if (t >= nt) break;
                         const h8 A = load_h8(xrow[t] + sb * 256 + s * 32);
                         const h8 Al = load_h8(xrow_lo[t] + sb * 256 + s * 32);
                         f4 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
@@ -525,7 +496,7 @@ static void launch_mm(hipStream_t s, int type, const MMArgs & a, dim3 grid, size
 }
 
 void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
-            int mode, const float * bias) {
+            int mode, const float * bias, void * ws) {
     if (T <= 0) return;
     if (!w.packed) {
         matmul_generic(s, w, x, T, y, ldy, col0, mode, bias);
@@ -533,7 +504,11 @@ void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, in
     }
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
     if (w.type == WT_Q4_K && (!x.xs_hi || !x.xs_lo)) throw std::runtime_error("matmul: Q4_K needs block sums");
-    MMArgs a;
+    if (ws) {
+        matmul_lds(s, w, x, T, y, ldy, col0, mode, bias, ws);
+        return;
+    }
+    MMArgs a {};
     a.w = w.packed; a.x = x.x; a.x_lo = x.x_lo; a.xs_hi = x.xs_hi; a.xs_lo = x.xs_lo; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
     a.n_row_tiles = w.N / 16;
@@ -600,9 +575,41 @@ __global__ __launch_bounds__(256) void k_rmsnorm_act(const float * __restrict__ 
     }
 }
 
+// E % 32 == 0: 8 elements per lane, 16-byte loads and stores.
+__global__ __launch_bounds__(256) void k_rmsnorm_act8(const float * __restrict__ x, const float * __restrict__ w,
+                                                      int E, float eps, const int32_t * __restrict__ rows, Act out) {
+    __shared__ float red[4];
+    const int o = blockIdx.x;
+    const float * xr = x + (size_t)(rows ? rows[o] : o) * E;
+    float ss = 0.0f;
+    for (int k = threadIdx.x * 8; k < E; k += 2048) {
+        const f4 a = *(const f4 *)(xr + k), b = *(const f4 *)(xr + k + 4);
+        ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    const float scale = 1.0f / sqrtf(total / (float)E + eps);
+    const int nblk = E / 32;
+    for (int k = threadIdx.x * 8; k < E; k += 2048) {
+        const f4 a = *(const f4 *)(xr + k), b = *(const f4 *)(xr + k + 4);
+        const f4 wa = *(const f4 *)(w + k), wb = *(const f4 *)(w + k + 4);
+        const float v[8] = {(a.x * scale) * wa.x, (a.y * scale) * wa.y, (a.z * scale) * wa.z, (a.w * scale) * wa.w,
+                            (b.x * scale) * wb.x, (b.y * scale) * wb.y, (b.z * scale) * wb.z, (b.w * scale) * wb.w};
+        store_act8(v, out.x + (size_t)o * E + k, out.x_lo + (size_t)o * E + k,
+                   out.xs_hi + (size_t)o * nblk + k / 32, out.xs_lo + (size_t)o * nblk + k / 32, threadIdx.x & 3);
+    }
+}
+
 void rmsnorm_act(hipStream_t s, const float * x, const float * w, int E, float eps,
                  const int32_t * rows, int n_rows, const Act & out) {
     if (n_rows <= 0) return;
+    if (E % 32 == 0 && out.xs_hi && out.xs_lo) {
+        hipLaunchKernelGGL(k_rmsnorm_act8, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, out);
+        check_launch("rmsnorm");
+        return;
+    }
     Act o = out;
     if (E % 32 != 0) { o.xs_hi = nullptr; o.xs_lo = nullptr; }
     hipLaunchKernelGGL(k_rmsnorm_act, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, o);
@@ -651,8 +658,32 @@ void to_act(hipStream_t s, const float * x, int T, int K, const Act & out) {
     check_launch("to_act");
 }
 
+// F % 32 == 0: 8 elements per lane.
+__global__ __launch_bounds__(256) void k_swiglu_act8(const float * __restrict__ gu, int T, int F, Act out) {
+    const int per = F / 8;
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (size_t)T * per) return;      // whole groups of four lanes leave together (per % 4 == 0)
+    const int t = (int)(gid / per), k = (int)(gid % per) * 8;
+    const float * g = gu + (size_t)t * 2 * F + k;
+    const float * u = g + F;
+    const f4 ga = *(const f4 *)g, gb = *(const f4 *)(g + 4), ua = *(const f4 *)u, ub = *(const f4 *)(u + 4);
+    const float gv[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
+    const float uv[8] = {ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w};
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (gv[i] / (1.0f + __expf(-gv[i]))) * uv[i];
+    const size_t at = (size_t)t * F + k;
+    store_act8(v, out.x + at, out.x_lo + at, out.xs_hi + at / 32, out.xs_lo + at / 32, threadIdx.x & 3);
+}
+
 void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out) {
     if (T <= 0) return;
+    if (F % 32 == 0 && out.xs_hi && out.xs_lo) {
+        const size_t n = (size_t)T * (F / 8);
+        hipLaunchKernelGGL(k_swiglu_act8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, T, F, out);
+        check_launch("swiglu");
+        return;
+    }
     Act o = out;
     if (F % 32 != 0) { o.xs_hi = nullptr; o.xs_lo = nullptr; }
     const size_t n = (size_t)T * ((F + 31) / 32);

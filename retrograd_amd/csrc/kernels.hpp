@@ -56,8 +56,17 @@ void repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int 
 
 enum : int { MM_STORE = 0, MM_ADD = 1 };
 // y[t][col0 + n] (=|+=) sum_k W[n][k] * x[t][k] (+ bias[n]); y has row stride ldy.
+// `ws` is a zero-initialised device workspace of matmul_workspace_bytes() that
+// selects the LDS-staged tile kernels; without it the register-only tile
+// kernels run.
 void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
-            int mode, const float * bias);
+            int mode, const float * bias, void * ws = nullptr);
+size_t matmul_workspace_bytes();
+extern int g_mm_debug;         // timing experiments (see MMArgs::debug)
+extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic
+extern int g_mm_force_r;       // 4 selects four row tiles per wave instead of two
+void matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                int mode, const float * bias, void * ws);
 // Forces the generic (raw layout) kernel; used to cross-check the tile kernels.
 void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
                     int mode, const float * bias);

@@ -120,7 +120,7 @@ STEP_SYMBOLS = [
     "retro_grammar_gbnf", "retro_grammar_free", "retro_last_error",
 ]
 KERNEL_SYMBOLS = [
-    "retro_kernel_matmul", "retro_kernel_sample_prepare", "retro_kernel_page_size", "retro_kernel_max_topk",
+    "retro_kernel_matmul", "retro_kernel_matmul_time", "retro_kernel_sample_prepare", "retro_kernel_page_size", "retro_kernel_max_topk",
     "retro_engine_debug_logits", "retro_engine_debug_kv", "retro_engine_debug_pack", "retro_engine_debug_pages",
     "retro_engine_debug_profile", "retro_engine_debug_profile_categories", "retro_engine_debug_profile_read",
 ]
@@ -189,6 +189,8 @@ def load_library() -> C.CDLL:
                                         _f32p, C.c_int32, _f32p]
     lib.retro_kernel_sample_prepare.argtypes = [_f32p, C.c_int32, C.c_int32, _i32p, _i32p, _f32p,
                                                 C.POINTER(C.c_double), _i32p, _f32p]
+    lib.retro_kernel_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,
+                                             C.c_int32, C.c_int32, C.POINTER(C.c_double)]
     lib.retro_kernel_page_size.restype = C.c_int32
     lib.retro_kernel_max_topk.restype = C.c_int32
     lib.retro_engine_debug_logits.argtypes = [C.c_void_p, _f32p, C.c_size_t, C.POINTER(C.c_size_t)]
@@ -681,7 +683,7 @@ class _GrammarHandle:
 
 # ---- kernel-level calls (tests, micro-benchmarks) -----------------------------------------
 
-def kernel_matmul(ggml_type: int, raw: np.ndarray, n_rows: int, k: int, x: np.ndarray, use_tiles: bool,
+def kernel_matmul(ggml_type: int, raw: np.ndarray, n_rows: int, k: int, x: np.ndarray, use_tiles,
                   bias: np.ndarray | None = None, accumulate_into: np.ndarray | None = None) -> np.ndarray:
     lib = load_library()
     raw = np.ascontiguousarray(raw, np.uint8)
@@ -693,10 +695,21 @@ def kernel_matmul(ggml_type: int, raw: np.ndarray, n_rows: int, k: int, x: np.nd
         bias = np.ascontiguousarray(bias, np.float32)
         b = bias.ctypes.data_as(_f32p)
     s = lib.retro_kernel_matmul(ggml_type, raw.ctypes.data_as(_u8p), n_rows, k, x.ctypes.data_as(_f32p), T,
-                                1 if use_tiles else 0, b, 0 if accumulate_into is None else 1, y.ctypes.data_as(_f32p))
+                                int(use_tiles), b, 0 if accumulate_into is None else 1, y.ctypes.data_as(_f32p))
     if s != 0:
         _raise(s)
     return y
+
+
+def kernel_matmul_time(ggml_type: int, n_rows: int, k: int, n_tokens: int, mode: int = 2, iters: int = 50,
+                       debug: int = 0, force_ksplit: int = 0) -> float:
+    """Microseconds per launch of one tile matmul on device-only data."""
+    out = C.c_double()
+    s = load_library().retro_kernel_matmul_time(ggml_type, n_rows, k, n_tokens, mode, iters, debug, force_ksplit,
+                                                C.byref(out))
+    if s != 0:
+        _raise(s)
+    return out.value
 
 
 def kernel_sample_prepare(logits: np.ndarray, k: Sequence[int]):

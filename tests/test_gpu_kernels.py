@@ -39,9 +39,10 @@ def test_tile_matmul_matches_decoded_blocks(t, n, k, T):
     raw, dense = _weights(t, n, k, seed=n + k + T)
     x = np.random.default_rng(T).standard_normal((T, k)).astype(np.float32)
     want = _ref(dense, x)
-    got = E.kernel_matmul(t, raw, n, k, x, use_tiles=True)
     scale = np.abs(want).max()
-    assert np.abs(got - want).max() <= 2e-5 * scale + 1e-6
+    for mode in (1, 2):      # register-only tiles, LDS-staged tiles
+        got = E.kernel_matmul(t, raw, n, k, x, use_tiles=mode)
+        assert np.abs(got - want).max() <= 2e-5 * scale + 1e-6, mode
     gen = E.kernel_matmul(t, raw, n, k, x, use_tiles=False)
     assert np.abs(gen - want).max() <= 2e-5 * scale + 1e-6
 
@@ -72,7 +73,7 @@ def test_matmul_bias_and_accumulate():
     bias = rng.standard_normal(n).astype(np.float32)
     y0 = rng.standard_normal((T, n)).astype(np.float32)
     want = _ref(dense, x)
-    for tiles in (True, False):
+    for tiles in (2, 1, 0):
         got = E.kernel_matmul(t, raw, n, k, x, use_tiles=tiles, bias=bias)
         assert np.abs(got - (want + bias)).max() <= 3e-5 * np.abs(want).max()
         got = E.kernel_matmul(t, raw, n, k, x, use_tiles=tiles, accumulate_into=y0)
@@ -92,15 +93,34 @@ def test_tile_matmul_exact_on_integer_data():
     dense = np.stack([oracle.decode_row(gw.GGML_Q4_K, raw[i], k) for i in range(n)]).astype(np.float64)
     x = rng.integers(-4, 5, (T, k)).astype(np.float32)
     want = x.astype(np.float64) @ dense.T
-    got = E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x, use_tiles=True)
-    assert np.array_equal(got.astype(np.float64), want)
+    for mode in (1, 2):
+        got = E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x, use_tiles=mode)
+        assert np.array_equal(got.astype(np.float64), want), mode
     q8 = rng.integers(0, 256, (n, k // 32, 34), dtype=np.uint8)
     q8[..., 0:2] = np.frombuffer(np.float16(0.125).tobytes(), np.uint8)
     raw = q8.reshape(n, -1)
     dense = np.stack([oracle.decode_row(gw.GGML_Q8_0, raw[i], k) for i in range(n)]).astype(np.float64)
     want = x.astype(np.float64) @ dense.T
-    got = E.kernel_matmul(gw.GGML_Q8_0, raw, n, k, x, use_tiles=True)
-    assert np.array_equal(got.astype(np.float64), want)
+    for mode in (1, 2):
+        got = E.kernel_matmul(gw.GGML_Q8_0, raw, n, k, x, use_tiles=mode)
+        assert np.array_equal(got.astype(np.float64), want), mode
+
+
+@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0])
+def test_split_k_matmul_is_deterministic_and_exact(t):
+    # 4096 x 4096 at 64 tokens splits K across workgroups; the reduction order
+    # is fixed, so two runs agree bit for bit, and both match the decoded blocks.
+    n, k, T = 4096, 4096, 64
+    raw, dense = _weights(t, n, k, seed=77)
+    x = np.random.default_rng(5).standard_normal((T, k)).astype(np.float32)
+    want = _ref(dense, x)
+    a = E.kernel_matmul(t, raw, n, k, x, use_tiles=2)
+    b = E.kernel_matmul(t, raw, n, k, x, use_tiles=2)
+    assert np.array_equal(a, b)
+    assert np.abs(a - want).max() <= 2e-5 * np.abs(want).max()
+    y0 = np.random.default_rng(6).standard_normal((T, n)).astype(np.float32)
+    c = E.kernel_matmul(t, raw, n, k, x, use_tiles=2, accumulate_into=y0)
+    assert np.abs(c - (want + y0)).max() <= 3e-5 * np.abs(want).max()
 
 
 def test_sample_prepare_matches_numpy():

@@ -34,7 +34,7 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
                         int32_t n_tokens, int32_t use_tiles, const float * bias, int32_t accumulate, float * y) {
     return guarded([&]() -> int {
         const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
-        DevBuf d_raw, d_packed, d_x, d_xh, d_xl, d_hi, d_lo, d_y, d_bias;
+        DevBuf d_raw, d_packed, d_x, d_xh, d_sums, d_y, d_bias;
         d_raw.alloc(bytes);
         ok(hipMemcpy(d_raw.ptr, raw, bytes, hipMemcpyHostToDevice), "upload weights");
         rk::Weight w;
@@ -49,11 +49,11 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
         }
         d_x.alloc((size_t)n_tokens * k * 4);
         ok(hipMemcpy(d_x.ptr, x, d_x.bytes, hipMemcpyHostToDevice), "upload activations");
-        d_xh.alloc((size_t)n_tokens * k * 2);
-        d_xl.alloc((size_t)n_tokens * k * 2);
-        d_hi.alloc((size_t)n_tokens * (k / 32 + 1) * 2);
-        d_lo.alloc((size_t)n_tokens * (k / 32 + 1) * 2);
-        rk::Act act{d_xh.as<__half>(), d_xl.as<__half>(), k % 32 == 0 ? d_hi.as<__half>() : nullptr, k % 32 == 0 ? d_lo.as<__half>() : nullptr, (int)k};
+        d_xh.alloc(rk::act_halves(n_tokens, (int)k) * 2);
+        d_sums.alloc(rk::act_sum_halves(n_tokens, (int)k) * 2);
+        ok(hipMemset(d_xh.ptr, 0, d_xh.bytes), "clear activations");
+        ok(hipMemset(d_sums.ptr, 0, d_sums.bytes), "clear block sums");
+        rk::Act act{d_xh.as<__half>(), k % 32 == 0 ? d_sums.as<__half>() : nullptr, (int)k};
         rk::to_act(nullptr, d_x.as<float>(), n_tokens, (int)k, act);
         d_y.alloc((size_t)n_tokens * n_rows * 4);
         ok(hipMemcpy(d_y.ptr, y, d_y.bytes, hipMemcpyHostToDevice), "upload outputs");
@@ -107,22 +107,20 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
                              int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us) {
     return guarded([&]() -> int {
         const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
-        DevBuf d_w, d_xh, d_xl, d_hi, d_lo, d_y, d_ws;
+        DevBuf d_w, d_xh, d_sums, d_y, d_ws;
         d_w.alloc(bytes);
         ok(hipMemset(d_w.ptr, 0x11, bytes), "fill");
-        d_xh.alloc((size_t)n_tokens * k * 2); d_xl.alloc((size_t)n_tokens * k * 2);
-        d_hi.alloc((size_t)n_tokens * (k / 32 + 1) * 2); d_lo.alloc((size_t)n_tokens * (k / 32 + 1) * 2);
-        ok(hipMemset(d_xh.ptr, 0, d_xh.bytes), "fill"); ok(hipMemset(d_xl.ptr, 0, d_xl.bytes), "fill");
-        ok(hipMemset(d_hi.ptr, 0, d_hi.bytes), "fill"); ok(hipMemset(d_lo.ptr, 0, d_lo.bytes), "fill");
+        d_xh.alloc(rk::act_halves(n_tokens, (int)k) * 2);
+        d_sums.alloc(rk::act_sum_halves(n_tokens, (int)k) * 2);
+        ok(hipMemset(d_xh.ptr, 0, d_xh.bytes), "fill"); ok(hipMemset(d_sums.ptr, 0, d_sums.bytes), "fill");
         d_y.alloc((size_t)n_tokens * n_rows * 4);
         d_ws.alloc(rk::matmul_workspace_bytes());
         ok(hipMemset(d_ws.ptr, 0, d_ws.bytes), "fill");
         rk::Weight w;
         w.type = type; w.K = (int)k; w.N = (int)n_rows; w.bytes = bytes; w.packed = d_w.as<uint8_t>();
-        rk::Act act{d_xh.as<__half>(), d_xl.as<__half>(), d_hi.as<__half>(), d_lo.as<__half>(), (int)k};
+        rk::Act act{d_xh.as<__half>(), d_sums.as<__half>(), (int)k};
         rk::g_mm_debug = debug;
-        rk::g_mm_force_ksplit = force_ksplit & 0xff;
-        rk::g_mm_force_r = force_ksplit >> 8;
+        rk::g_mm_force_ksplit = force_ksplit;
         hipEvent_t e0, e1;
         ok(hipEventCreate(&e0), "event"); ok(hipEventCreate(&e1), "event");
         for (int i = 0; i < 3; ++i) rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, mode == 2 ? d_ws.ptr : nullptr);
@@ -134,7 +132,6 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
         ok(hipEventElapsedTime(&ms, e0, e1), "elapsed");
         rk::g_mm_debug = 0;
         rk::g_mm_force_ksplit = 0;
-        rk::g_mm_force_r = 0;
         (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
         *out_us = (double)ms * 1e3 / iters;
         return 0;

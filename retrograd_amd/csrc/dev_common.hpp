@@ -48,12 +48,38 @@ __device__ __forceinline__ h8 load_h8(const __half * p) {
 }
 
 // Arguments of the tile matmuls.
+// Index, in halves, of element (token, k, hi/lo) of an operand-order activation buffer.
+__device__ __forceinline__ size_t act_chunk_halves(int K) { return (size_t)((K + 31) & ~31) * 128; }
+__device__ __forceinline__ size_t act_at(int tok, int k, int hl, int K) {
+    return (size_t)(tok >> 6) * act_chunk_halves(K) + (size_t)(((k >> 5) * 2 + hl) * 4 + ((tok >> 4) & 3)) * 512
+         + ((((k >> 3) & 3) * 16 + (tok & 15)) * 8) + (k & 7);
+}
+// ... and of the hi/lo sum of 32-wide block `blk` of a token.
+__device__ __forceinline__ size_t act_sum_chunk_halves(int K) { return (size_t)((K + 255) >> 8) * 2048; }
+__device__ __forceinline__ size_t act_sum_at(int tok, int blk, int hl, int K) {
+    return (size_t)(tok >> 6) * act_sum_chunk_halves(K) + (size_t)((blk >> 3) * 4 + ((tok >> 4) & 3)) * 512
+         + ((hl * 16 + (tok & 15)) * 8) + (blk & 7);
+}
+
+// Scales and mins of the eight sub-blocks of a Q4_K super-block, one value per
+// byte (sc[0] = sub-blocks 0-3, sc[1] = 4-7, likewise mn), from a row's tile
+// header: word 0 is d | dmin << 16; the bytes of words 1, 2, 3 hold sc0-3, sc4-7
+// and mn0-3 in their low six bits, and the top two bits of byte j of the three
+// words are bits 0-1, 2-3 and 4-5 of mn(4+j).
+struct Q4KScales { uint32_t sc[2]; uint32_t mn[2]; };
+__device__ __forceinline__ Q4KScales q4k_scales(const u4 & hdr) {
+    Q4KScales s;
+    s.sc[0] = hdr.y & 0x3f3f3f3fu;
+    s.sc[1] = hdr.z & 0x3f3f3f3fu;
+    s.mn[0] = hdr.w & 0x3f3f3f3fu;
+    s.mn[1] = ((hdr.y >> 6) & 0x03030303u) | ((hdr.z >> 4) & 0x0c0c0c0cu) | ((hdr.w >> 2) & 0x30303030u);
+    return s;
+}
+
 struct MMArgs {
     const uint8_t * w;
-    const __half * x;
-    const __half * x_lo;
-    const __half * xs_hi;
-    const __half * xs_lo;
+    const __half * x;         // operand-order activations and block sums (see Act)
+    const __half * sums;
     float * y;
     const float * bias;
     int K, N, T, ldy, col0, mode;
@@ -63,7 +89,6 @@ struct MMArgs {
     int n_row_groups;
     float * partial;          // [ksplit][gridDim.y * 64][N]
     int32_t * counters;       // [n_row_groups * gridDim.y], zero between launches
-    const __half * zeros;     // 16 bytes of zeros
     int debug;                // timing experiments only: bit 0 stage activations once, bit 1 skip the multiplies
 };
 

@@ -286,16 +286,17 @@ void Engine::build_buffers() {
     qkv_.alloc((size_t)B * (QD + 2 * KD) * 4);
     gu_.alloc((size_t)B * 2 * F * 4);
     q_half_.alloc((size_t)B * QD * 2);
-    auto act = [&](DevBuf & x, DevBuf & xl, DevBuf & hi, DevBuf & lo, int K) {
-        x.alloc((size_t)B * K * 2);
-        xl.alloc((size_t)B * K * 2);
-        hi.alloc((size_t)B * (K / 32 + 1) * 2);
-        lo.alloc((size_t)B * (K / 32 + 1) * 2);
+    // operand-order activations; the sums keep zero padding lanes, so they are cleared once
+    auto act = [&](DevBuf & x, DevBuf & sums, int K) {
+        x.alloc(rk::act_halves(B, K) * 2);
+        sums.alloc(rk::act_sum_halves(B, K) * 2);
+        hip_check(hipMemsetAsync(x.ptr, 0, x.bytes, stream_), "hipMemsetAsync");
+        hip_check(hipMemsetAsync(sums.ptr, 0, sums.bytes, stream_), "hipMemsetAsync");
     };
-    act(act_e_x_, act_e_xl_, act_e_hi_, act_e_lo_, E);
-    act(act_q_x_, act_q_xl_, act_q_hi_, act_q_lo_, QD);
-    act(act_f_x_, act_f_xl_, act_f_hi_, act_f_lo_, F);
-    act(act_o_x_, act_o_xl_, act_o_hi_, act_o_lo_, E);
+    act(act_e_x_, act_e_sums_, E);
+    act(act_q_x_, act_q_sums_, QD);
+    act(act_f_x_, act_f_sums_, F);
+    act(act_o_x_, act_o_sums_, E);
     q_half_lo_.alloc((size_t)B * QD * 2);
     mm_ws_.alloc(rk::matmul_workspace_bytes());
     hip_check(hipMemsetAsync(mm_ws_.ptr, 0, mm_ws_.bytes, stream_), "hipMemsetAsync");
@@ -1058,13 +1059,10 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
     const HParams & h = hp_;
     const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim, F = h.n_ff;
     rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps};
-    rk::Act act_e{act_e_x_.as<__half>(), act_e_xl_.as<__half>(), act_e_hi_.as<__half>(), act_e_lo_.as<__half>(), E};
-    rk::Act act_q{act_q_x_.as<__half>(), act_q_xl_.as<__half>(), act_q_hi_.as<__half>(), act_q_lo_.as<__half>(), QD};
-    rk::Act act_f{act_f_x_.as<__half>(), act_f_xl_.as<__half>(), act_f_hi_.as<__half>(), act_f_lo_.as<__half>(), F};
-    rk::Act act_o{act_o_x_.as<__half>(), act_o_xl_.as<__half>(), act_o_hi_.as<__half>(), act_o_lo_.as<__half>(), E};
-    if (E % 32 != 0) { act_e.xs_hi = act_e.xs_lo = act_o.xs_hi = act_o.xs_lo = nullptr; }
-    if (QD % 32 != 0) { act_q.xs_hi = act_q.xs_lo = nullptr; }
-    if (F % 32 != 0) { act_f.xs_hi = act_f.xs_lo = nullptr; }
+    rk::Act act_e{act_e_x_.as<__half>(), E % 32 == 0 ? act_e_sums_.as<__half>() : nullptr, E};
+    rk::Act act_q{act_q_x_.as<__half>(), QD % 32 == 0 ? act_q_sums_.as<__half>() : nullptr, QD};
+    rk::Act act_f{act_f_x_.as<__half>(), F % 32 == 0 ? act_f_sums_.as<__half>() : nullptr, F};
+    rk::Act act_o{act_o_x_.as<__half>(), E % 32 == 0 ? act_o_sums_.as<__half>() : nullptr, E};
     partial_.ensure(rk::attention_partial_floats(n_items, h.head_dim) * 4);
     float * x = x_.as<float>();
     float * qkv = qkv_.as<float>();

@@ -190,12 +190,12 @@ private:
     rk::PackBuffers pk_ {};
     std::vector<DevBuf> pk_store_;
     DevBuf x_, qkv_, gu_, q_half_, partial_, logits_, sample_k_, sample_out_, out_rows_idx_;
-    DevBuf act_e_x_, act_e_xl_, act_e_hi_, act_e_lo_;       // n_embd wide
-    DevBuf act_q_x_, act_q_xl_, act_q_hi_, act_q_lo_;       // n_head * head_dim wide
-    DevBuf act_f_x_, act_f_xl_, act_f_hi_, act_f_lo_;       // n_ff wide
-    DevBuf act_o_x_, act_o_xl_, act_o_hi_, act_o_lo_;       // output rows, n_embd wide
+    DevBuf act_e_x_, act_e_sums_;       // n_embd wide
+    DevBuf act_q_x_, act_q_sums_;       // n_head * head_dim wide
+    DevBuf act_f_x_, act_f_sums_;       // n_ff wide
+    DevBuf act_o_x_, act_o_sums_;       // output rows, n_embd wide
     DevBuf q_half_lo_;
-    DevBuf mm_ws_;            // matmul workspace: split-K partials, counters, zeros
+    DevBuf mm_ws_;            // matmul workspace: split-K partials, counters
     HostPinned h_sample_, h_logits_;
     int last_n_out_ = 0;
 

@@ -7,7 +7,7 @@
 //    into tiles of 16 rows x 256 columns. A tile stores first one 16-byte
 //    header per row, then the quantised payload ordered so that lane l of a
 //    wave reads 16 contiguous bytes at offset l*16 of each 1 KiB load:
-//      Q4_K  2304 B = 16 x (d, dmin, scales[12]) + 2 loads;  lane (r = l%16,
+//      Q4_K  2304 B = 16 x (d, dmin, 12 bytes of re-encoded scales) + 2 loads;  lane (r = l%16,
 //            g = l/16) of load h holds, as 4 dwords, the 8 nibbles of
 //            elements 32*(4h+j) + 8g .. +8 of row r, j = 0..3. Inside a dword
 //            the nibbles are ordered e0 e2 e4 e6 | e1 e3 e5 e7 so that masking
@@ -106,29 +106,28 @@ __device__ float decode_elem(int type, const uint8_t * row, int k) {
     }
 }
 
-// Writes up to 32 consecutive activations of one row as f16 hi/lo pairs and,
-// for a whole block, the sum of the stored values as hi + lo halves.
-__device__ __forceinline__ void store_act_block(const float * v, int count, __half * x, __half * x_lo,
-                                                __half * hi, __half * lo) {
+// Writes up to 32 consecutive activations of one token (k0 a multiple of 32) as
+// f16 hi/lo pairs and, for a whole block, the sum of the stored values as hi + lo halves.
+__device__ __forceinline__ void store_act_block(const float * v, int count, const Act & out, int tok, int k0) {
     float sum = 0.0f;
     for (int i = 0; i < count; ++i) {
         const __half h = sat_half(v[i]);
         const __half l = __float2half_rn(fminf(fmaxf(v[i], -65504.0f), 65504.0f) - __half2float(h));
-        x[i] = h;
-        x_lo[i] = l;
+        out.x[act_at(tok, k0 + i, 0, out.K)] = h;
+        out.x[act_at(tok, k0 + i, 1, out.K)] = l;
         sum += __half2float(h) + __half2float(l);
     }
-    if (hi && count == 32) {
+    if (out.sums && count == 32) {
         const __half a = sat_half(sum);
-        *hi = a;
-        *lo = __float2half_rn(sum - __half2float(a));
+        out.sums[act_sum_at(tok, k0 >> 5, 0, out.K)] = a;
+        out.sums[act_sum_at(tok, k0 >> 5, 1, out.K)] = __float2half_rn(sum - __half2float(a));
     }
 }
 
-// Eight consecutive activations per lane: hi/lo pairs as two 16-byte stores; the
-// four lanes that own one 32-wide block add their sums with two xor-shuffles.
-__device__ __forceinline__ void store_act8(const float (&v)[8], __half * x, __half * x_lo, __half * hi, __half * lo,
-                                           int lane_in_block) {
+// Eight consecutive activations per lane (k a multiple of 8): hi/lo as two
+// 16-byte stores; the four lanes that own one 32-wide block add their sums
+// with two xor-shuffles.
+__device__ __forceinline__ void store_act8(const float (&v)[8], const Act & out, int tok, int k, int lane_in_block) {
     h8 a, b;
     float sum = 0.0f;
 #pragma unroll
@@ -140,15 +139,15 @@ __device__ __forceinline__ void store_act8(const float (&v)[8], __half * x, __ha
         b[i] = l;
         sum += (float)h + (float)l;
     }
-    *(h8 *)x = a;
-    *(h8 *)x_lo = b;
-    if (hi) {
+    *(h8 *)(out.x + act_at(tok, k, 0, out.K)) = a;
+    *(h8 *)(out.x + act_at(tok, k, 1, out.K)) = b;
+    if (out.sums) {
         sum += __shfl_xor(sum, 1, 64);
         sum += __shfl_xor(sum, 2, 64);
         if (lane_in_block == 0) {
             const __half s = sat_half(sum);
-            *hi = s;
-            *lo = __float2half_rn(sum - __half2float(s));
+            out.sums[act_sum_at(tok, k >> 5, 0, out.K)] = s;
+            out.sums[act_sum_at(tok, k >> 5, 1, out.K)] = __float2half_rn(sum - __half2float(s));
         }
     }
 }
@@ -169,7 +168,21 @@ __global__ void k_repack_q4k(const uint8_t * __restrict__ raw, uint8_t * __restr
     if (w < 64) {                       // headers: row r, dword j
         const int r = w >> 2, j = w & 3;
         const uint8_t * blk = raw + ((rt * 16 + r) * nsb + sb) * 144;
-        out = *(const uint32_t *)(blk + 4 * j);
+        if (j == 0) {
+            out = *(const uint32_t *)blk;          // d, dmin
+        } else {
+            // the 6-bit scales and mins, re-encoded one per byte (see q4k_scales)
+            const uint8_t * q = blk + 4;
+            out = 0;
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t sc_lo = q[i] & 63, mn_lo = q[i + 4] & 63;
+                const uint32_t sc_hi = (q[i + 8] & 0x0f) | ((q[i] >> 6) << 4);
+                const uint32_t mn_hi = (q[i + 8] >> 4) | ((q[i + 4] >> 6) << 4);
+                const uint32_t low = j == 1 ? sc_lo : (j == 2 ? sc_hi : mn_lo);
+                const uint32_t top = (mn_hi >> (2 * (j - 1))) & 3;
+                out |= (low | (top << 6)) << (8 * i);
+            }
+        }
     } else {
         const int v = w - 64;           // 0..511
         const int h = v >> 8;           // load
@@ -288,7 +301,6 @@ __global__ __launch_bounds__(256) void k_mm_q4k(MMArgs a) {
     const int tbase = blockIdx.y * 64;
     const int nt = min(NT, (a.T - tbase + 15) >> 4);
     const int nsb = a.K >> 8;
-    const int nblk = a.K >> 5;
 
     f4 acc[NT];
 #pragma unroll
@@ -296,17 +308,12 @@ __global__ __launch_bounds__(256) void k_mm_q4k(MMArgs a) {
 
     // activation row of this lane for every token tile (clamped: rows past T
     // are computed on the last row and never stored)
-    const __half * xrow[NT];
-    const __half * xrow_lo[NT];
-    const __half * shi[NT];
-    const __half * slo[NT];
+    const __half * xt[NT];
+    const __half * st[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        const int tok = min(tbase + t * 16 + r, a.T - 1);
-        xrow[t] = a.x + (size_t)tok * a.K + 8 * g;
-        xrow_lo[t] = a.x_lo + (size_t)tok * a.K + 8 * g;
-        shi[t] = a.xs_hi + (size_t)tok * nblk;
-        slo[t] = a.xs_lo + (size_t)tok * nblk;
+        xt[t] = a.x + (size_t)blockIdx.y * act_chunk_halves(a.K) + t * 512 + lane * 8;
+        st[t] = a.sums + (size_t)blockIdx.y * act_sum_chunk_halves(a.K) + t * 512 + lane * 8;
     }
 
     if (rt < a.n_row_tiles) {
@@ -317,17 +324,12 @@ __global__ __launch_bounds__(256) void k_mm_q4k(MMArgs a) {
             const u4 q1 = *(const u4 *)(tile + 1280 + lane * 16);
             const float d = h2f((uint16_t)(hdr.x & 0xffff));
             const float dmin = h2f((uint16_t)(hdr.x >> 16));
-            // scales[12] = bytes of hdr.y, hdr.z, hdr.w
+            const Q4KScales s4 = q4k_scales(hdr);
             uint32_t sc[8], mn[8];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t lo_b = (hdr.y >> (8 * j)) & 0xff;   // scales[j]
-                const uint32_t md_b = (hdr.z >> (8 * j)) & 0xff;   // scales[j+4]
-                const uint32_t hi_b = (hdr.w >> (8 * j)) & 0xff;   // scales[j+8]
-                sc[j] = lo_b & 63;
-                mn[j] = md_b & 63;
-                sc[j + 4] = (hi_b & 0x0f) | ((lo_b >> 6) << 4);
-                mn[j + 4] = (hi_b >> 4) | ((md_b >> 6) << 4);
+            for (int j = 0; j < 8; ++j) {
+                sc[j] = (s4.sc[j >> 2] >> (8 * (j & 3))) & 0xff;
+                mn[j] = (s4.mn[j >> 2] >> (8 * (j & 3))) & 0xff;
             }
             f4 accq[NT], accm[NT];
 #pragma unroll
@@ -342,9 +344,7 @@ __global__ __launch_bounds__(256) void k_mm_q4k(MMArgs a) {
                 for (int i = 0; i < 8; ++i) mB[i] = g < 2 ? (_Float16)(float)mn[i] : (_Float16)0.0f;
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    h8 sA = (h8){0, 0, 0, 0, 0, 0, 0, 0};
-                    if (g == 0) sA = load_h8(shi[t] + sb * 8);
-                    else if (g == 1) sA = load_h8(slo[t] + sb * 8);
+                    const h8 sA = load_h8(st[t] + (size_t)sb * 2048);
                     accm[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(sA, mB, accm[t], 0, 0, 0);
                 }
             }
@@ -369,8 +369,8 @@ __global__ __launch_bounds__(256) void k_mm_q4k(MMArgs a) {
                 const h8 B = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    const h8 A = load_h8(xrow[t] + sb * 256 + s * 32);
-                    const h8 Al = load_h8(xrow_lo[t] + sb * 256 + s * 32);
+                    const h8 A = load_h8(xt[t] + (size_t)((sb * 8 + s) * 2) * 2048);
+                    const h8 Al = load_h8(xt[t] + (size_t)((sb * 8 + s) * 2 + 1) * 2048);
                     accq[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, accq[t], 0, 0, 0);
                     accq[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, B, accq[t], 0, 0, 0);
                 }
@@ -389,7 +389,7 @@ template <int NT>
 __global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
     extern __shared__ float lds[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r = lane & 15, g = lane >> 4;
+    const int r = lane & 15;
     const int wr = wave / a.ksplit, wk = wave % a.ksplit;
     const int rt = blockIdx.x * (4 / a.ksplit) + wr;
     const int tbase = blockIdx.y * 64;
@@ -399,14 +399,9 @@ __global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
     f4 acc[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[t] = (f4){0.f, 0.f, 0.f, 0.f};
-    const __half * xrow[NT];
-    const __half * xrow_lo[NT];
+    const __half * xt[NT];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-        const int tok = min(tbase + t * 16 + r, a.T - 1);
-        xrow[t] = a.x + (size_t)tok * a.K + 8 * g;
-        xrow_lo[t] = a.x_lo + (size_t)tok * a.K + 8 * g;
-    }
+    for (int t = 0; t < NT; ++t) xt[t] = a.x + (size_t)blockIdx.y * act_chunk_halves(a.K) + t * 512 + lane * 8;
     const h2 bias1152 = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
 
     if (rt < a.n_row_tiles) {
@@ -433,8 +428,8 @@ __global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
                     const h8 B = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
 #pragma unroll
                     for (int t = 0; t < NT; ++t) {
-                        const h8 A = load_h8(xrow[t] + sb * 256 + s * 32);
-                        const h8 Al = load_h8(xrow_lo[t] + sb * 256 + s * 32);
+                        const h8 A = load_h8(xt[t] + (size_t)((sb * 8 + s) * 2) * 2048);
+                        const h8 Al = load_h8(xt[t] + (size_t)((sb * 8 + s) * 2 + 1) * 2048);
                         f4 part = __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                         part = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, B, part, 0, 0, 0);
 #pragma unroll
@@ -449,8 +444,7 @@ __global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
 
 // Any type, any shape: one wave per output feature, raw GGUF rows.
 __global__ __launch_bounds__(256) void k_mm_generic(int type, const uint8_t * __restrict__ raw, size_t rb,
-                                                    const __half * __restrict__ x,
-                                                    const __half * __restrict__ x_lo, int K, int N, int T,
+                                                    const __half * __restrict__ x, int K, int N, int T,
                                                     float * y, int ldy, int col0, int mode, const float * bias) {
     const int lane = threadIdx.x & 63;
     const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -463,7 +457,7 @@ __global__ __launch_bounds__(256) void k_mm_generic(int type, const uint8_t * __
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int t = min(t0 + j, T - 1);
-                const float xv = __half2float(x[(size_t)t * K + k]) + __half2float(x_lo[(size_t)t * K + k]);
+                const float xv = __half2float(x[act_at(t, k, 0, K)]) + __half2float(x[act_at(t, k, 1, K)]);
                 acc[j] = fmaf(w, xv, acc[j]);
             }
         }
@@ -485,7 +479,7 @@ void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
     if (T <= 0) return;
     hipLaunchKernelGGL(k_mm_generic, dim3((w.N + 3) / 4), dim3(256), 0, s, w.type, w.raw, row_bytes(w.type, w.K),
-                       x.x, x.x_lo, w.K, w.N, T, y, ldy, col0, mode, bias);
+                       x.x, w.K, w.N, T, y, ldy, col0, mode, bias);
     check_launch("matmul_generic");
 }
 
@@ -503,13 +497,13 @@ void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, in
         return;
     }
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
-    if (w.type == WT_Q4_K && (!x.xs_hi || !x.xs_lo)) throw std::runtime_error("matmul: Q4_K needs block sums");
+    if (w.type == WT_Q4_K && !x.sums) throw std::runtime_error("matmul: Q4_K needs block sums");
     if (ws) {
         matmul_lds(s, w, x, T, y, ldy, col0, mode, bias, ws);
         return;
     }
     MMArgs a {};
-    a.w = w.packed; a.x = x.x; a.x_lo = x.x_lo; a.xs_hi = x.xs_hi; a.xs_lo = x.xs_lo; a.y = y; a.bias = bias;
+    a.w = w.packed; a.x = x.x; a.sums = x.sums; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
     a.n_row_tiles = w.N / 16;
     // Enough waves to cover the chip: split K across the waves of a workgroup
@@ -569,9 +563,7 @@ __global__ __launch_bounds__(256) void k_rmsnorm_act(const float * __restrict__ 
         const int count = min(32, E - k0);
         float v[32];
         for (int i = 0; i < count; ++i) v[i] = (xr[k0 + i] * scale) * w[k0 + i];
-        store_act_block(v, count, out.x + (size_t)o * E + k0, out.x_lo + (size_t)o * E + k0,
-                        out.xs_hi ? out.xs_hi + (size_t)o * (E / 32) + b : nullptr,
-                        out.xs_lo ? out.xs_lo + (size_t)o * (E / 32) + b : nullptr);
+        store_act_block(v, count, out, o, k0);
     }
 }
 
@@ -591,27 +583,26 @@ __global__ __launch_bounds__(256) void k_rmsnorm_act8(const float * __restrict__
     __syncthreads();
     const float total = (red[0] + red[1]) + (red[2] + red[3]);
     const float scale = 1.0f / sqrtf(total / (float)E + eps);
-    const int nblk = E / 32;
     for (int k = threadIdx.x * 8; k < E; k += 2048) {
         const f4 a = *(const f4 *)(xr + k), b = *(const f4 *)(xr + k + 4);
         const f4 wa = *(const f4 *)(w + k), wb = *(const f4 *)(w + k + 4);
         const float v[8] = {(a.x * scale) * wa.x, (a.y * scale) * wa.y, (a.z * scale) * wa.z, (a.w * scale) * wa.w,
                             (b.x * scale) * wb.x, (b.y * scale) * wb.y, (b.z * scale) * wb.z, (b.w * scale) * wb.w};
-        store_act8(v, out.x + (size_t)o * E + k, out.x_lo + (size_t)o * E + k,
-                   out.xs_hi + (size_t)o * nblk + k / 32, out.xs_lo + (size_t)o * nblk + k / 32, threadIdx.x & 3);
+        store_act8(v, out, o, k, threadIdx.x & 3);
     }
 }
 
 void rmsnorm_act(hipStream_t s, const float * x, const float * w, int E, float eps,
                  const int32_t * rows, int n_rows, const Act & out) {
     if (n_rows <= 0) return;
-    if (E % 32 == 0 && out.xs_hi && out.xs_lo) {
+    if (out.K != E) throw std::runtime_error("rmsnorm: activation width does not match");
+    if (E % 32 == 0 && out.sums) {
         hipLaunchKernelGGL(k_rmsnorm_act8, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, out);
         check_launch("rmsnorm");
         return;
     }
     Act o = out;
-    if (E % 32 != 0) { o.xs_hi = nullptr; o.xs_lo = nullptr; }
+    if (E % 32 != 0) o.sums = nullptr;
     hipLaunchKernelGGL(k_rmsnorm_act, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, o);
     check_launch("rmsnorm");
 }
@@ -630,9 +621,7 @@ __global__ __launch_bounds__(256) void k_swiglu_act(const float * __restrict__ g
         const float gi = g[i];
         v[i] = (gi / (1.0f + __expf(-gi))) * u[i];
     }
-    store_act_block(v, count, out.x + (size_t)t * F + k0, out.x_lo + (size_t)t * F + k0,
-                    out.xs_hi ? out.xs_hi + (size_t)t * (F / 32) + b : nullptr,
-                    out.xs_lo ? out.xs_lo + (size_t)t * (F / 32) + b : nullptr);
+    store_act_block(v, count, out, t, k0);
 }
 
 __global__ __launch_bounds__(256) void k_to_act(const float * __restrict__ x, int T, int K, Act out) {
@@ -644,15 +633,14 @@ __global__ __launch_bounds__(256) void k_to_act(const float * __restrict__ x, in
     const int count = min(32, K - k0);
     float v[32];
     for (int i = 0; i < count; ++i) v[i] = x[(size_t)t * K + k0 + i];
-    store_act_block(v, count, out.x + (size_t)t * K + k0, out.x_lo + (size_t)t * K + k0,
-                    out.xs_hi ? out.xs_hi + (size_t)t * (K / 32) + b : nullptr,
-                    out.xs_lo ? out.xs_lo + (size_t)t * (K / 32) + b : nullptr);
+    store_act_block(v, count, out, t, k0);
 }
 
 void to_act(hipStream_t s, const float * x, int T, int K, const Act & out) {
     if (T <= 0) return;
+    if (out.K != K) throw std::runtime_error("to_act: activation width does not match");
     Act o = out;
-    if (K % 32 != 0) { o.xs_hi = nullptr; o.xs_lo = nullptr; }
+    if (K % 32 != 0) o.sums = nullptr;
     const size_t n = (size_t)T * ((K + 31) / 32);
     hipLaunchKernelGGL(k_to_act, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, T, K, o);
     check_launch("to_act");
@@ -672,20 +660,20 @@ __global__ __launch_bounds__(256) void k_swiglu_act8(const float * __restrict__ 
     float v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = (gv[i] / (1.0f + __expf(-gv[i]))) * uv[i];
-    const size_t at = (size_t)t * F + k;
-    store_act8(v, out.x + at, out.x_lo + at, out.xs_hi + at / 32, out.xs_lo + at / 32, threadIdx.x & 3);
+    store_act8(v, out, t, k, threadIdx.x & 3);
 }
 
 void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out) {
     if (T <= 0) return;
-    if (F % 32 == 0 && out.xs_hi && out.xs_lo) {
+    if (out.K != F) throw std::runtime_error("swiglu: activation width does not match");
+    if (F % 32 == 0 && out.sums) {
         const size_t n = (size_t)T * (F / 8);
         hipLaunchKernelGGL(k_swiglu_act8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, T, F, out);
         check_launch("swiglu");
         return;
     }
     Act o = out;
-    if (F % 32 != 0) { o.xs_hi = nullptr; o.xs_lo = nullptr; }
+    if (F % 32 != 0) o.sums = nullptr;
     const size_t n = (size_t)T * ((F + 31) / 32);
     hipLaunchKernelGGL(k_swiglu_act, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, T, F, o);
     check_launch("swiglu");
@@ -1178,24 +1166,25 @@ __global__ __launch_bounds__(256) void k_attention_combine(CombineArgs a) {
         const float f1 = fminf(fmaxf(v1 * inv, -65504.0f), 65504.0f);
         const __half h0 = __float2half_rn(f0), h1 = __float2half_rn(f1);
         const __half l0 = __float2half_rn(f0 - __half2float(h0)), l1 = __float2half_rn(f1 - __half2float(h1));
-        const size_t at = (size_t)t * QD + (size_t)head * a.hd + e0;
+        const int k = head * a.hd + e0;            // even: k and k + 1 share a group of eight
+        const size_t at = act_at(t, k, 0, QD), at_lo = act_at(t, k, 1, QD);
         a.out.x[at] = h0;
         a.out.x[at + 1] = h1;
-        a.out.x_lo[at] = l0;
-        a.out.x_lo[at + 1] = l1;
+        a.out.x[at_lo] = l0;
+        a.out.x[at_lo + 1] = l1;
         r0 = __half2float(h0) + __half2float(l0);
         r1 = __half2float(h1) + __half2float(l1);
     }
-    if (a.out.xs_hi) {
+    if (a.out.sums) {
         // block of 32 outputs = 16 lanes
         float sum = r0 + r1;
 #pragma unroll
         for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o, 64);
         if ((lane & 15) == 0 && e0 < a.hd) {
-            const size_t b = ((size_t)t * QD + (size_t)head * a.hd + e0) / 32;
+            const int b = (head * a.hd + e0) / 32;
             const __half hi = sat_half(sum);
-            a.out.xs_hi[b] = hi;
-            a.out.xs_lo[b] = __float2half_rn(sum - __half2float(hi));
+            a.out.sums[act_sum_at(t, b, 0, QD)] = hi;
+            a.out.sums[act_sum_at(t, b, 1, QD)] = __float2half_rn(sum - __half2float(hi));
         }
     }
 }

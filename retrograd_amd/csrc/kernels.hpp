@@ -37,18 +37,26 @@ struct Weight {
 };
 
 // Activations handed to a matmul. An f32 value v travels as two f16 numbers,
-// x = f16(v) and x_lo = f16(v - x), which together carry about 22 significant
+// hi = f16(v) and lo = f16(v - hi), which together carry about 22 significant
 // bits: a single f16 (11 bits) leaves a logit error above the parity
 // tolerance once it has passed through a few layers. For every 32-wide block
-// of a row the f32 sum of x + x_lo is kept as well, split the same way; the
+// of a row the f32 sum of hi + lo is kept as well, split the same way; the
 // sums are what the Q4_K min term multiplies.
+//
+// Both buffers are stored in MFMA operand order, so that a matmul stages them
+// with contiguous 1 KiB loads. Tokens are grouped in chunks of 64 (4 tiles of
+// 16); with Kp = K rounded up to 32:
+//   x:    [chunk][k / 32][hi, lo][tile][lane = 16 * ((k % 32) / 8) + token % 16][k % 8]
+//   sums: [chunk][k / 256][tile][lane = 16 * (hi: 0, lo: 1) + token % 16][(k % 256) / 32]
+// The sums blocks also have lanes 32-63, which stay zero from allocation: they
+// pad the operand of the min-term MFMA.
 struct Act {
-    __half * x = nullptr;       // [T][K]
-    __half * x_lo = nullptr;    // [T][K]
-    __half * xs_hi = nullptr;   // [T][K/32], null when K % 32 != 0
-    __half * xs_lo = nullptr;
+    __half * x = nullptr;       // act_halves(T, K) halves
+    __half * sums = nullptr;    // act_sum_halves(T, K) halves, zero-initialised; null when K % 32 != 0
     int K = 0;
 };
+inline size_t act_halves(int T, int K) { return (size_t)((T + 63) / 64) * (size_t)((K + 31) / 32 * 32) * 128; }
+inline size_t act_sum_halves(int T, int K) { return (size_t)((T + 63) / 64) * (size_t)((K + 255) / 256) * 2048; }
 
 bool can_pack(int type, int64_t K, int64_t N);
 // raw (device, GGUF layout) -> packed (device). Both hold `bytes` bytes.
@@ -64,7 +72,6 @@ void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, in
 size_t matmul_workspace_bytes();
 extern int g_mm_debug;         // timing experiments (see MMArgs::debug)
 extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic
-extern int g_mm_force_r;       // 4 selects four row tiles per wave instead of two
 void matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
                 int mode, const float * bias, void * ws);
 // Forces the generic (raw layout) kernel; used to cross-check the tile kernels.

@@ -32,49 +32,41 @@ template <int NT> struct XStage {
 };
 
 // Per-lane source pointers of the activation staging, computed once per kernel:
-// wave w always stages token tile w % NT, and 4/NT waves share the sixteen
-// (k-step, hi/lo) blocks of a tile.
+// wave w of the eight always stages token tile w % NT, and 8/NT waves share the
+// sixteen (k-step, hi/lo) blocks of a tile. The activations are stored in
+// operand order, so every load copies one contiguous 1 KiB block.
 template <int NT> struct StageSrc {
-    const __half * x;        // row of this lane's token in a.x, at k = 8g
-    ptrdiff_t lo_delta;      // a.x_lo - a.x (halves)
-    const __half * sum;      // this lane's block-sum source (hi, lo or zeros)
-    int sum_stride;          // halves to advance per super-block (0 for the zeros)
+    const __half * x;        // block (k-step 0, hi) of this wave's tile, at this lane
+    const __half * sum;      // block sums of super-block 0 of this wave's tile, at this lane
     int tile, slot;
 };
 
 template <int NT>
-__device__ __forceinline__ StageSrc<NT> stage_prepare(const MMArgs & a, int tbase, int lane, int wave) {
+__device__ __forceinline__ StageSrc<NT> stage_prepare(const MMArgs & a, int chunk, int lane, int wave) {
     static_assert(NT == 1 || NT == 2 || NT == 4, "token tiles per chunk");
     StageSrc<NT> s;
-    const int r16 = lane & 15, g = lane >> 4;
     s.tile = wave % NT;
     s.slot = wave / NT;
-    const int tok = min(tbase + s.tile * 16 + r16, a.T - 1);
-    s.x = a.x + (size_t)tok * a.K + 8 * g;
-    s.lo_delta = a.x_lo - a.x;
-    const int nblk = a.K >> 5;
-    if (g == 0) { s.sum = a.xs_hi + (size_t)tok * nblk; s.sum_stride = 8; }
-    else if (g == 1) { s.sum = a.xs_lo + (size_t)tok * nblk; s.sum_stride = 8; }
-    else { s.sum = a.zeros; s.sum_stride = 0; }
+    s.x = a.x + (size_t)chunk * act_chunk_halves(a.K) + s.tile * 512 + lane * 8;
+    s.sum = a.sums ? a.sums + (size_t)chunk * act_sum_chunk_halves(a.K) + s.tile * 512 + lane * 8 : nullptr;
     return s;
 }
 
 // Issues the direct-to-LDS loads of one super-block column of activations.
 template <int NT>
 __device__ __forceinline__ void stage_x(const StageSrc<NT> & s, int sb, uint8_t * buf, bool with_sums) {
-    constexpr int WAVES_PER_TILE = 4 / NT;
+    constexpr int WAVES_PER_TILE = 8 / NT;
     constexpr int PER_WAVE = 16 / WAVES_PER_TILE;
 #pragma unroll
     for (int j = 0; j < PER_WAVE; ++j) {
-        const int c = s.slot + WAVES_PER_TILE * j;      // (k-step, hi/lo) combination, wave-uniform
-        const int ks = c >> 1, hl = c & 1;
-        const __half * src = s.x + (size_t)sb * 256 + ks * 32 + (hl ? s.lo_delta : 0);
+        const int c = s.slot + WAVES_PER_TILE * j;      // (k-step, hi/lo) block of the super-block, wave-uniform
+        const __half * src = s.x + (size_t)(sb * 16 + c) * 2048;
         __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)src,
-                                         (void __attribute__((address_space(3))) *)(buf + ((ks * 2 + hl) * NT + s.tile) * 1024),
+                                         (void __attribute__((address_space(3))) *)(buf + (c * NT + s.tile) * 1024),
                                          16, 0, 0);
     }
     if (with_sums && s.slot == 0) {
-        const __half * src = s.sum + (size_t)sb * s.sum_stride;
+        const __half * src = s.sum + (size_t)sb * 2048;
         __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)src,
                                          (void __attribute__((address_space(3))) *)(buf + (XStage<NT>::X_BLOCKS + s.tile) * 1024),
                                          16, 0, 0);
@@ -89,7 +81,7 @@ __device__ __forceinline__ h8 lds_h8(const uint8_t * buf, int block, int lane) {
 // weight row 16 * rt[r] + r16.
 template <int NT, int R>
 __device__ __forceinline__ void finish(const MMArgs & a, f4 (&acc)[R][NT], const int (&rt)[R], int tbase, int nt,
-                                       int rg, int ks, int * flag) {
+                                       int rg, int ks, int * flag, bool owner) {
     const int lane = threadIdx.x & 63;
     const int r16 = lane & 15, g = lane >> 4;
     if (a.ksplit > 1) {
@@ -97,7 +89,7 @@ __device__ __forceinline__ void finish(const MMArgs & a, f4 (&acc)[R][NT], const
         float * mine = a.partial + (size_t)ks * tpad * a.N;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            if (rt[r] >= a.n_row_tiles) continue;
+            if (!owner || rt[r] >= a.n_row_tiles) continue;
 #pragma unroll
             for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -116,7 +108,7 @@ __device__ __forceinline__ void finish(const MMArgs & a, f4 (&acc)[R][NT], const
             *flag = last;
         }
         __syncthreads();
-        if (!*flag) return;
+        if (!*flag || !owner) return;
         __threadfence();
         // Every partial address was written exactly once, by one workgroup, before
         // its counter increment: plain loads see it. Slice order is the sum order.
@@ -139,6 +131,7 @@ __device__ __forceinline__ void finish(const MMArgs & a, f4 (&acc)[R][NT], const
             }
         }
     }
+    if (!owner) return;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (rt[r] >= a.n_row_tiles) continue;
@@ -160,152 +153,55 @@ __device__ __forceinline__ void finish(const MMArgs & a, f4 (&acc)[R][NT], const
     }
 }
 
+
+// (x & mask) | bits in one instruction
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) {
+    uint32_t d;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(d) : "v"(x), "s"(mask), "v"(bits));
+    return d;
+}
+
+// f16 pair (1024 + byte a, 1024 + byte b) of a word, bytes chosen by the selector
+__device__ __forceinline__ h2 magic_pair(uint32_t word, uint32_t sel) {
+    return __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, word, sel));
+}
+
+constexpr int kWaves = 8;      // 4 row waves x 2 halves of every super-block
+constexpr int kThreads = kWaves * 64;
+
+// The two k-halves of a row wave add their accumulators through LDS; the sum
+// is left in the half-0 waves.
+template <int NT, int R>
+__device__ __forceinline__ void join_halves(f4 (&acc)[R][NT], uint8_t * smem, int rw, int kh, int lane) {
+    __syncthreads();       // every wave is done with the staged activations
+    if (kh == 1) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) *(f4 *)(smem + (((rw * R + r) * NT + t) * 64 + lane) * 16) = acc[r][t];
+    }
+    __syncthreads();
+    if (kh == 0) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const f4 o = *(const f4 *)(smem + (((rw * R + r) * NT + t) * 64 + lane) * 16);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[r][t][i] += o[i];
+            }
+    }
+}
+
 }  // namespace
 
 template <int NT, int R>
-__global__ __launch_bounds__(256, 1) void k_mm2_q4k(MMArgs a) {
+__global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     __shared__ int flag;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r16 = lane & 15, g = lane >> 4;
-    const int rg = blockIdx.x % a.n_row_groups, ks = blockIdx.x / a.n_row_groups;
-    const int tbase = blockIdx.y * 64;
-    const int nt = min(NT, (a.T - tbase + 15) >> 4);
-    const int nsb = a.K >> 8;
-    const int per = (nsb + a.ksplit - 1) / a.ksplit;
-    const int sb0 = ks * per, sb1 = min(nsb, sb0 + per);
-
-    int rt[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) rt[r] = (rg * 4 + wave) * R + r;
-    const StageSrc<NT> stage = stage_prepare<NT>(a, tbase, lane, wave);
-
-    f4 acc[R][NT];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
-
-    const uint8_t * wbase[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) wbase[r] = a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 2304;
-    // weights of one super-block of every row tile: header, two payload loads
-    u4 hdr[R], q0[R], q1[R], n_hdr[R], n_q0[R], n_q1[R];
-    auto load_w = [&](int sb, u4 (&h)[R], u4 (&p0)[R], u4 (&p1)[R]) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            // rows past the matrix read the last tile; their results are never stored
-            const uint8_t * tile = wbase[r] + (size_t)sb * 2304;
-            h[r] = *(const u4 *)(tile + r16 * 16);
-            p0[r] = *(const u4 *)(tile + 256 + lane * 16);
-            p1[r] = *(const u4 *)(tile + 1280 + lane * 16);
-        }
-    };
-
-    if (sb0 < sb1) {
-        stage_x<NT>(stage, sb0, smem, true);
-        load_w(sb0, hdr, q0, q1);
-    }
-    for (int sb = sb0; sb < sb1; ++sb) {
-        uint8_t * cur = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
-        uint8_t * nxt = smem + ((sb - sb0 + 1) & 1) * XStage<NT>::BYTES;
-        // everything issued for this super-block has landed, and every wave is
-        // done reading the buffer the next loads overwrite
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (sb + 1 < sb1) {
-            if (!(a.debug & 1)) stage_x<NT>(stage, sb + 1, nxt, true);
-            load_w(sb + 1, n_hdr, n_q0, n_q1);
-        }
-        if (a.debug & 1) cur = smem;
-
-        f4 accq[R][NT];
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int t = 0; t < NT; ++t) accq[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
-        // 6-bit scales and mins of the 8 sub-blocks, as bytes: sc in the low, min in the high half-word pairs
-        uint32_t sc[R][8], mn[R][8];
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t lo_b = (hdr[r].y >> (8 * j)) & 0xff;
-                const uint32_t md_b = (hdr[r].z >> (8 * j)) & 0xff;
-                const uint32_t hi_b = (hdr[r].w >> (8 * j)) & 0xff;
-                sc[r][j] = lo_b & 63;
-                mn[r][j] = md_b & 63;
-                sc[r][j + 4] = (hi_b & 0x0f) | ((lo_b >> 6) << 4);
-                mn[r][j + 4] = (hi_b >> 4) | ((md_b >> 6) << 4);
-            }
-        // min term: k-slots of lane group 0 carry the hi block sums, group 1 the lo sums
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            const h8 sA = lds_h8(cur, XStage<NT>::X_BLOCKS + t, lane);
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                h8 mB;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) mB[i] = g < 2 ? (_Float16)(float)mn[r][i] : (_Float16)0.0f;
-                const f4 m4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(sA, mB, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                const float ndmin = -h2f((uint16_t)(hdr[r].x >> 16));
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[r][t][i] = fmaf(ndmin, m4[i], acc[r][t][i]);
-            }
-        }
-        if (!(a.debug & 2))
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            h8 A[NT], Al[NT];
-#pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                A[t] = lds_h8(cur, (s * 2 + 0) * NT + t, lane);
-                Al[t] = lds_h8(cur, (s * 2 + 1) * NT + t, lane);
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const uint32_t wq = s < 4 ? q0[r][s & 3] : q1[r][s & 3];
-                const _Float16 sch = (_Float16)(float)sc[r][s];
-                const h2 k1 = {sch, sch};
-                const h2 c1 = k1 * (_Float16)(-1024.0f);
-                const h2 k2 = k1 * (_Float16)(0.0625f);
-                const h2 c2 = k1 * (_Float16)(-64.0f);
-                const uint32_t w8 = wq >> 8;
-                const h2 u0 = __builtin_bit_cast(h2, (wq & 0x000F000Fu) | 0x64006400u);
-                const h2 u1 = __builtin_bit_cast(h2, (wq & 0x00F000F0u) | 0x64006400u);
-                const h2 u2 = __builtin_bit_cast(h2, (w8 & 0x000F000Fu) | 0x64006400u);
-                const h2 u3 = __builtin_bit_cast(h2, (w8 & 0x00F000F0u) | 0x64006400u);
-                const h2 a0 = __builtin_elementwise_fma(u0, k1, c1);   // exactly sc * e (<= 945)
-                const h2 a1 = __builtin_elementwise_fma(u1, k2, c2);
-                const h2 a2 = __builtin_elementwise_fma(u2, k1, c1);
-                const h2 a3 = __builtin_elementwise_fma(u3, k2, c2);
-                const h8 B = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
-#pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[t], B, accq[r][t], 0, 0, 0);
-                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[t], B, accq[r][t], 0, 0, 0);
-                }
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const float d = h2f((uint16_t)(hdr[r].x & 0xffff));
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[r][t][i] = fmaf(d, accq[r][t][i], acc[r][t][i]);
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r) { hdr[r] = n_hdr[r]; q0[r] = n_q0[r]; q1[r] = n_q1[r]; }
-    }
-    finish<NT, R>(a, acc, rt, tbase, nt, rg, ks, &flag);
-}
-
-template <int NT, int R>
-__global__ __launch_bounds__(256, 1) void k_mm2_q8_0(MMArgs a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ int flag;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rw = wave & 3, kh = wave >> 2;
     const int r16 = lane & 15;
     const int rg = blockIdx.x % a.n_row_groups, ks = blockIdx.x / a.n_row_groups;
     const int tbase = blockIdx.y * 64;
@@ -316,8 +212,161 @@ __global__ __launch_bounds__(256, 1) void k_mm2_q8_0(MMArgs a) {
 
     int rt[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) rt[r] = (rg * 4 + wave) * R + r;
-    const StageSrc<NT> stage = stage_prepare<NT>(a, tbase, lane, wave);
+    for (int r = 0; r < R; ++r) rt[r] = (rg * 4 + rw) * R + r;
+    const StageSrc<NT> stage = stage_prepare<NT>(a, blockIdx.y, lane, wave);
+
+    f4 acc[R][NT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
+
+    // rows past the matrix read the last tile; their results are never stored
+    const uint8_t * wbase[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) wbase[r] = a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 2304;
+    // this wave's weights of one super-block: the row headers and its half of the payload
+    struct WSet { u4 hdr[R]; u4 q[R]; };
+    auto load_w = [&](int sb, WSet & w) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint8_t * tile = wbase[r] + (size_t)sb * 2304;
+            w.hdr[r] = *(const u4 *)(tile + r16 * 16);
+            w.q[r] = *(const u4 *)(tile + 256 + kh * 1024 + lane * 16);
+        }
+    };
+    const h2 m1024 = {(_Float16)(-1024.0f), (_Float16)(-1024.0f)};
+    const uint32_t magic1024 = 0x64006400u, magic64 = 0x54005400u;
+
+    // One super-block: wait for its activations, start the loads of what comes
+    // next (activations one super-block ahead, weights two), multiply.
+    auto body = [&](int sb, const WSet & w, WSet & fut) {
+        uint8_t * cur = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
+        uint8_t * nxt = smem + ((sb - sb0 + 1) & 1) * XStage<NT>::BYTES;
+        // All but the newest 2R loads (the weights one super-block ahead) have
+        // landed: this super-block's activations and weights are in.
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R));
+        __syncthreads();   // ... for every wave, and nobody still reads nxt
+        if (sb + 1 < sb1 && !(a.debug & 1)) stage_x<NT>(stage, sb + 1, nxt, true);
+        load_w(min(sb + 2, sb1 - 1), fut);
+        if (a.debug & 1) cur = smem;
+
+        Q4KScales s4[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) s4[r] = q4k_scales(w.hdr[r]);
+
+        // min term: k-slots of lane group 0 carry the hi block sums, group 1 the
+        // lo sums, groups 2-3 zeros; the token tiles are shared out between the halves
+        {
+            h8 mB[R];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const h2 p0 = magic_pair(s4[r].mn[0], 0x04010400u) + m1024;
+                const h2 p1 = magic_pair(s4[r].mn[0], 0x04030402u) + m1024;
+                const h2 p2 = magic_pair(s4[r].mn[1], 0x04010400u) + m1024;
+                const h2 p3 = magic_pair(s4[r].mn[1], 0x04030402u) + m1024;
+                mB[r] = (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+            }
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                if ((NT == 1 ? 0 : (t & 1)) != kh) continue;
+                const h8 sA = lds_h8(cur, XStage<NT>::X_BLOCKS + t, lane);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const f4 m4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(sA, mB[r], (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    const float ndmin = -h2f((uint16_t)(w.hdr[r].x >> 16));
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[r][t][i] = fmaf(ndmin, m4[i], acc[r][t][i]);
+                }
+            }
+        }
+
+        f4 accq[R][NT];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) accq[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
+        const uint8_t * xk = cur + kh * (8 * NT * 1024);      // this half's four k-steps
+        if (!(a.debug & 2))
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            h8 A[NT], Al[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                A[t] = lds_h8(xk, (j * 2 + 0) * NT + t, lane);
+                Al[t] = lds_h8(xk, (j * 2 + 1) * NT + t, lane);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const uint32_t scw = kh ? s4[r].sc[1] : s4[r].sc[0];
+                const h2 k1 = magic_pair(scw, 0x04000400u + 0x00010001u * j) + m1024;   // (sc, sc)
+                const h2 c1 = k1 * (_Float16)(-1024.0f);
+                const h2 c2 = k1 * (_Float16)(-64.0f);
+                const uint32_t wq = w.q[r][j];
+                const uint32_t w8 = wq >> 8;
+                // 1024 + e in the low nibble positions, 64 + e in the high ones
+                const h2 u0 = __builtin_bit_cast(h2, and_or(wq, 0x000F000Fu, magic1024));
+                const h2 u1 = __builtin_bit_cast(h2, and_or(wq, 0x00F000F0u, magic64));
+                const h2 u2 = __builtin_bit_cast(h2, and_or(w8, 0x000F000Fu, magic1024));
+                const h2 u3 = __builtin_bit_cast(h2, and_or(w8, 0x00F000F0u, magic64));
+                const h2 a0 = __builtin_elementwise_fma(u0, k1, c1);   // exactly sc * e (<= 945)
+                const h2 a1 = __builtin_elementwise_fma(u1, k1, c2);
+                const h2 a2 = __builtin_elementwise_fma(u2, k1, c1);
+                const h2 a3 = __builtin_elementwise_fma(u3, k1, c2);
+                const h8 B = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[t], B, accq[r][t], 0, 0, 0);
+                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[t], B, accq[r][t], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float d = h2f((uint16_t)(w.hdr[r].x & 0xffff));
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[r][t][i] = fmaf(d, accq[r][t][i], acc[r][t][i]);
+        }
+    };
+
+    if (sb0 < sb1) {
+        WSet w0, w1, w2;
+        stage_x<NT>(stage, sb0, smem, true);
+        load_w(sb0, w0);
+        load_w(min(sb0 + 1, sb1 - 1), w1);
+        for (int sb = sb0; sb < sb1; sb += 3) {
+            body(sb, w0, w2);
+            if (sb + 1 >= sb1) break;
+            body(sb + 1, w1, w0);
+            if (sb + 2 >= sb1) break;
+            body(sb + 2, w2, w1);
+        }
+    }
+    join_halves<NT, R>(acc, smem, rw, kh, lane);
+    finish<NT, R>(a, acc, rt, tbase, nt, rg, ks, &flag, kh == 0);
+}
+
+template <int NT, int R>
+__global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ int flag;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rw = wave & 3, kh = wave >> 2;
+    const int r16 = lane & 15;
+    const int rg = blockIdx.x % a.n_row_groups, ks = blockIdx.x / a.n_row_groups;
+    const int tbase = blockIdx.y * 64;
+    const int nt = min(NT, (a.T - tbase + 15) >> 4);
+    const int nsb = a.K >> 8;
+    const int per = (nsb + a.ksplit - 1) / a.ksplit;
+    const int sb0 = ks * per, sb1 = min(nsb, sb0 + per);
+
+    int rt[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) rt[r] = (rg * 4 + rw) * R + r;
+    const StageSrc<NT> stage = stage_prepare<NT>(a, blockIdx.y, lane, wave);
     f4 acc[R][NT];
 #pragma unroll
     for (int r = 0; r < R; ++r)
@@ -327,52 +376,45 @@ __global__ __launch_bounds__(256, 1) void k_mm2_q8_0(MMArgs a) {
     const uint8_t * wbase[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) wbase[r] = a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 4352;
-    u4 hdr[R], q[R][4], n_hdr[R], n_q[R][4];
-    auto load_w = [&](int sb, u4 (&h)[R], u4 (&p)[R][4]) {
+    struct WSet { u4 hdr[R]; u4 q[R][2]; };
+    auto load_w = [&](int sb, WSet & w) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const uint8_t * tile = wbase[r] + (size_t)sb * 4352;
-            h[r] = *(const u4 *)(tile + r16 * 16);
+            w.hdr[r] = *(const u4 *)(tile + r16 * 16);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) p[r][j] = *(const u4 *)(tile + 256 + j * 1024 + lane * 16);
+            for (int j = 0; j < 2; ++j) w.q[r][j] = *(const u4 *)(tile + 256 + (2 * kh + j) * 1024 + lane * 16);
         }
     };
     const h2 bias1152 = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
 
-    if (sb0 < sb1) {
-        stage_x<NT>(stage, sb0, smem, false);
-        load_w(sb0, hdr, q);
-    }
-    for (int sb = sb0; sb < sb1; ++sb) {
+    auto body = [&](int sb, const WSet & w, WSet & fut) {
         uint8_t * cur = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
         uint8_t * nxt = smem + ((sb - sb0 + 1) & 1) * XStage<NT>::BYTES;
-        __builtin_amdgcn_s_waitcnt(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * R));
         __syncthreads();
-        if (sb + 1 < sb1) {
-            stage_x<NT>(stage, sb + 1, nxt, false);
-            load_w(sb + 1, n_hdr, n_q);
-        }
+        if (sb + 1 < sb1) stage_x<NT>(stage, sb + 1, nxt, false);
+        load_w(min(sb + 2, sb1 - 1), fut);
+        const uint8_t * xk = cur + kh * (8 * NT * 1024);
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
+        for (int j = 0; j < 4; ++j) {
             h8 A[NT], Al[NT];
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                A[t] = lds_h8(cur, (s * 2 + 0) * NT + t, lane);
-                Al[t] = lds_h8(cur, (s * 2 + 1) * NT + t, lane);
+                A[t] = lds_h8(xk, (j * 2 + 0) * NT + t, lane);
+                Al[t] = lds_h8(xk, (j * 2 + 1) * NT + t, lane);
             }
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                const uint32_t sw = hdr[r][s >> 1];
-                const float d = h2f((uint16_t)((s & 1) ? (sw >> 16) : (sw & 0xffff)));
-                const u4 d4 = q[r][s >> 1];
-                const int half = s & 1;
+                // scales of sub-blocks 4 kh + j: words 2 kh and 2 kh + 1 of the header
+                const uint32_t sw = kh ? (j < 2 ? w.hdr[r].z : w.hdr[r].w) : (j < 2 ? w.hdr[r].x : w.hdr[r].y);
+                const float d = h2f((uint16_t)((j & 1) ? (sw >> 16) : (sw & 0xffff)));
+                const u4 d4 = w.q[r][j >> 1];
+                const int half = j & 1;
                 const uint32_t w0 = d4[2 * half] ^ 0x80808080u;
                 const uint32_t w1 = d4[2 * half + 1] ^ 0x80808080u;
-                const h2 u0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u));
-                const h2 u1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u));
-                const h2 u2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u));
-                const h2 u3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u));
-                const h2 a0 = u0 + bias1152, a1 = u1 + bias1152, a2 = u2 + bias1152, a3 = u3 + bias1152;
+                const h2 a0 = magic_pair(w0, 0x04010400u) + bias1152, a1 = magic_pair(w0, 0x04030402u) + bias1152;
+                const h2 a2 = magic_pair(w1, 0x04010400u) + bias1152, a3 = magic_pair(w1, 0x04030402u) + bias1152;
                 const h8 B = {a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
@@ -383,33 +425,43 @@ __global__ __launch_bounds__(256, 1) void k_mm2_q8_0(MMArgs a) {
                 }
             }
         }
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            hdr[r] = n_hdr[r];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) q[r][j] = n_q[r][j];
+    };
+
+    if (sb0 < sb1) {
+        WSet w0, w1, w2;
+        stage_x<NT>(stage, sb0, smem, false);
+        load_w(sb0, w0);
+        load_w(min(sb0 + 1, sb1 - 1), w1);
+        for (int sb = sb0; sb < sb1; sb += 3) {
+            body(sb, w0, w2);
+            if (sb + 1 >= sb1) break;
+            body(sb + 1, w1, w0);
+            if (sb + 2 >= sb1) break;
+            body(sb + 2, w2, w1);
         }
     }
-    finish<NT, R>(a, acc, rt, tbase, nt, rg, ks, &flag);
+    join_halves<NT, R>(acc, smem, rw, kh, lane);
+    finish<NT, R>(a, acc, rt, tbase, nt, rg, ks, &flag, kh == 0);
 }
 
 template <int NT, int R>
 static void launch2(hipStream_t s, int type, const MMArgs & a, dim3 grid) {
     const size_t lds = 2 * (size_t)XStage<NT>::BYTES;
+    static_assert(2 * XStage<NT>::BYTES >= 4 * R * NT * 1024, "the joined accumulators fit the staging buffers");
     if (type == WT_Q4_K) {
         static bool once = false;
         if (!once) {
             HIP_OK(hipFuncSetAttribute((const void *)k_mm2_q4k<NT, R>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             once = true;
         }
-        hipLaunchKernelGGL((k_mm2_q4k<NT, R>), grid, dim3(256), lds, s, a);
+        hipLaunchKernelGGL((k_mm2_q4k<NT, R>), grid, dim3(kThreads), lds, s, a);
     } else {
         static bool once = false;
         if (!once) {
             HIP_OK(hipFuncSetAttribute((const void *)k_mm2_q8_0<NT, R>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             once = true;
         }
-        hipLaunchKernelGGL((k_mm2_q8_0<NT, R>), grid, dim3(256), lds, s, a);
+        hipLaunchKernelGGL((k_mm2_q8_0<NT, R>), grid, dim3(kThreads), lds, s, a);
     }
 }
 
@@ -421,7 +473,6 @@ size_t matmul_workspace_bytes() {
 // The LDS-staged path; ws must be zero-initialised once.
 int g_mm_debug = 0;
 int g_mm_force_ksplit = 0;
-int g_mm_force_r = 0;
 
 template <int R>
 static void dispatch_nt(hipStream_t s, int type, int nt, const MMArgs & a, dim3 grid) {
@@ -436,17 +487,16 @@ void matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y
                 int mode, const float * bias, void * ws) {
     MMArgs a {};
     a.debug = g_mm_debug;
-    a.w = w.packed; a.x = x.x; a.x_lo = x.x_lo; a.xs_hi = x.xs_hi; a.xs_lo = x.xs_lo; a.y = y; a.bias = bias;
+    a.w = w.packed; a.x = x.x; a.sums = x.sums; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
     a.n_row_tiles = w.N / 16;
     const size_t partial_bytes = (size_t)64 * 16 * 8192 * 4;
     a.partial = (float *)ws;
     a.counters = (int32_t *)((uint8_t *)ws + partial_bytes);
-    a.zeros = (const __half *)((uint8_t *)ws + partial_bytes + 65536);
     const int nsb = w.K / 256;
     const int nt = T > 32 ? 4 : (T > 16 ? 2 : 1);
     const int chunks = (T + 63) / 64;
-    const int R = g_mm_force_r == 4 ? 4 : 2;
+    constexpr int R = 2;
     a.n_row_groups = (a.n_row_tiles + 4 * R - 1) / (4 * R);
     // Split K across workgroups when the row groups alone leave most CUs idle
     // (decode-sized batches only: the partial buffer holds one 64-token chunk).
@@ -463,8 +513,7 @@ void matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y
     }
     a.ksplit = ksplit;
     dim3 grid(a.n_row_groups * ksplit, chunks);
-    if (R == 4) dispatch_nt<4>(s, w.type, nt, a, grid);
-    else dispatch_nt<2>(s, w.type, nt, a, grid);
+    dispatch_nt<R>(s, w.type, nt, a, grid);
     check_launch("matmul_lds");
 }
 

@@ -123,9 +123,14 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
         rk::g_mm_force_ksplit = force_ksplit;
         hipEvent_t e0, e1;
         ok(hipEventCreate(&e0), "event"); ok(hipEventCreate(&e1), "event");
-        for (int i = 0; i < 3; ++i) rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, mode == 2 ? d_ws.ptr : nullptr);
+        auto run = [&]() {
+            // mode 1: register-only tiles, 2: LDS-staged tiles, 3: the same with the K-slices left unreduced
+            if (mode == 3) rk::matmul_deferred(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, d_ws.ptr);
+            else rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, mode == 2 ? d_ws.ptr : nullptr);
+        };
+        for (int i = 0; i < 3; ++i) run();
         ok(hipEventRecord(e0, nullptr), "record");
-        for (int i = 0; i < iters; ++i) rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, mode == 2 ? d_ws.ptr : nullptr);
+        for (int i = 0; i < iters; ++i) run();
         ok(hipEventRecord(e1, nullptr), "record");
         ok(hipEventSynchronize(e1), "sync");
         float ms = 0;

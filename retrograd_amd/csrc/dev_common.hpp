@@ -87,8 +87,7 @@ struct MMArgs {
     int ksplit;       // v1: waves of a workgroup sharing a row tile along K; v2: workgroups sharing a row group
     // v2 only
     int n_row_groups;
-    float * partial;          // [ksplit][gridDim.y * 64][N]
-    int32_t * counters;       // [n_row_groups * gridDim.y], zero between launches
+    float * partial;          // [ksplit][64][N] K-slices of a split matmul
     int debug;                // timing experiments only: bit 0 stage activations once, bit 1 skip the multiplies
 };
 

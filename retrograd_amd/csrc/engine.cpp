@@ -1068,23 +1068,33 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
     float * qkv = qkv_.as<float>();
     float * gu = gu_.as<float>();
 
+    // A matmul into the residual stream may leave its result as K-slices; the
+    // next norm adds them to x.
+    rk::Slices pending;
     { const size_t pt_ = prof_begin(PC_EMBED); rk::embed(stream_, tok_embd_.w, pk_.tok, T, x); prof_end(PC_EMBED, pt_); }
     for (int l = 0; l < h.n_layer; ++l) {
         const LayerWeights & L = layers_[(size_t)l];
-        { const size_t pt_ = prof_begin(PC_NORM); rk::rmsnorm_act(stream_, x, L.attn_norm.as<float>(), E, h.eps, nullptr, T, act_e); prof_end(PC_NORM, pt_); }
+        { const size_t pt_ = prof_begin(PC_NORM); rk::rmsnorm_act(stream_, x, L.attn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending); prof_end(PC_NORM, pt_); }
+        rk::Slices qkv_slices;
         {
             const size_t pt_ = prof_begin(PC_QKV);
-            int col = 0;
-            for (const DevWeight & w : L.qkv) {
-                rk::matmul(stream_, w.w, act_e, T, qkv, QD + 2 * KD, col, rk::MM_STORE,
-                           L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr, mm_ws_.ptr);
-                col += w.w.N;
+            if (L.qkv.size() == 1) {     // fused q, k, v: the rotation kernel can add the slices
+                qkv_slices = rk::matmul_deferred(stream_, L.qkv[0].w, act_e, T, qkv, QD + 2 * KD, 0, rk::MM_STORE,
+                                                 L.qkv_bias.as<float>(), mm_ws_.ptr);
+            } else {
+                int col = 0;
+                for (const DevWeight & w : L.qkv) {
+                    rk::matmul(stream_, w.w, act_e, T, qkv, QD + 2 * KD, col, rk::MM_STORE,
+                               L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr, mm_ws_.ptr);
+                    col += w.w.N;
+                }
             }
             prof_end(PC_QKV, pt_);
         }
         size_t pt_ = prof_begin(PC_ROPE);
         rk::rope_store(stream_, qkv, T, sh, pk_, L.q_norm.as<float>(), L.k_norm.as<float>(), q_half_.as<__half>(),
-                       q_half_lo_.as<__half>(), k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>());
+                       q_half_lo_.as<__half>(), k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(),
+                       qkv_slices);
         prof_end(PC_ROPE, pt_);
         pt_ = prof_begin(PC_ATTN);
         rk::attention(stream_, q_half_.as<__half>(), q_half_lo_.as<__half>(), sh, pk_, table_.as<int32_t>(), max_pages_,
@@ -1095,10 +1105,10 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
         rk::attention_combine(stream_, partial_.as<float>(), T, sh, pk_, act_q);
         prof_end(PC_COMBINE, pt_);
         pt_ = prof_begin(PC_OPROJ);
-        rk::matmul(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
+        pending = rk::matmul_deferred(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
         prof_end(PC_OPROJ, pt_);
         pt_ = prof_begin(PC_NORM);
-        rk::rmsnorm_act(stream_, x, L.ffn_norm.as<float>(), E, h.eps, nullptr, T, act_e);
+        rk::rmsnorm_act(stream_, x, L.ffn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending);
         prof_end(PC_NORM, pt_);
         pt_ = prof_begin(PC_GATEUP);
         {
@@ -1113,13 +1123,13 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
         rk::swiglu_act(stream_, gu, T, F, act_f);
         prof_end(PC_SWIGLU, pt_);
         pt_ = prof_begin(PC_DOWN);
-        rk::matmul(stream_, L.down.w, act_f, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
+        pending = rk::matmul_deferred(stream_, L.down.w, act_f, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
         prof_end(PC_DOWN, pt_);
     }
     if (n_out > 0) {
         logits_.ensure((size_t)n_out * h.n_vocab * 4);
         const size_t pt_ = prof_begin(PC_HEAD);
-        rk::rmsnorm_act(stream_, x, out_norm_.as<float>(), E, h.eps, pk_.out_tok, n_out, act_o);
+        rk::rmsnorm_act(stream_, x, out_norm_.as<float>(), E, h.eps, pk_.out_tok, n_out, act_o, pending);
         rk::matmul(stream_, lm_head_.w, act_o, n_out, logits_.as<float>(), h.n_vocab, 0, rk::MM_STORE,
                    out_bias_.as<float>(), mm_ws_.ptr);
         prof_end(PC_HEAD, pt_);

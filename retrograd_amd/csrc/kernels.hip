@@ -489,19 +489,49 @@ static void launch_mm(hipStream_t s, int type, const MMArgs & a, dim3 grid, size
     else hipLaunchKernelGGL(k_mm_q8_0<NT>, grid, dim3(256), lds, s, a);
 }
 
+__global__ __launch_bounds__(256) void k_reduce_slices(Slices sl, int T, float * y, int ldy, int col0, int mode) {
+    const size_t gid = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (gid >= (size_t)T * sl.N) return;
+    const int t = (int)(gid / sl.N), c = (int)(gid % sl.N);
+    f4 v = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < sl.n; ++k) v += *(const f4 *)(sl.data + (size_t)k * sl.stride + gid);
+    float * p = y + (size_t)t * ldy + col0 + c;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) p[i] = mode == MM_ADD ? p[i] + v[i] : v[i];
+}
+
+void reduce_slices(hipStream_t s, const Slices & sl, int T, float * y, int ldy, int col0, int mode) {
+    if (sl.n <= 0 || T <= 0) return;
+    if (sl.N % 4 != 0) throw std::runtime_error("reduce_slices: the row width must be a multiple of 4");
+    const size_t n = (size_t)T * sl.N / 4;
+    hipLaunchKernelGGL(k_reduce_slices, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, sl, T, y, ldy, col0, mode);
+    check_launch("reduce_slices");
+}
+
+static Slices matmul_impl(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                          int mode, const float * bias, void * ws, bool may_slice);
+
 void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
             int mode, const float * bias, void * ws) {
-    if (T <= 0) return;
+    const Slices sl = matmul_impl(s, w, x, T, y, ldy, col0, mode, bias, ws, true);
+    reduce_slices(s, sl, T, y, ldy, col0, mode);
+}
+
+Slices matmul_deferred(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                       int mode, const float * bias, void * ws) {
+    return matmul_impl(s, w, x, T, y, ldy, col0, mode, bias, ws, true);
+}
+
+static Slices matmul_impl(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                          int mode, const float * bias, void * ws, bool may_slice) {
+    if (T <= 0) return Slices();
     if (!w.packed) {
         matmul_generic(s, w, x, T, y, ldy, col0, mode, bias);
-        return;
+        return Slices();
     }
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
     if (w.type == WT_Q4_K && !x.sums) throw std::runtime_error("matmul: Q4_K needs block sums");
-    if (ws) {
-        matmul_lds(s, w, x, T, y, ldy, col0, mode, bias, ws);
-        return;
-    }
+    if (ws) return matmul_lds(s, w, x, T, y, ldy, col0, mode, bias, ws, may_slice);
     MMArgs a {};
     a.w = w.packed; a.x = x.x; a.sums = x.sums; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
@@ -524,6 +554,7 @@ void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, in
         default: launch_mm<4>(s, w.type, a, grid, lds); break;
     }
     check_launch("matmul");
+    return Slices();
 }
 
 // ---------------------------------------------------------------------------
@@ -545,13 +576,22 @@ void embed(hipStream_t s, const Weight & emb, const int32_t * tok, int T, float 
     check_launch("embed");
 }
 
-__global__ __launch_bounds__(256) void k_rmsnorm_act(const float * __restrict__ x, const float * __restrict__ w,
-                                                     int E, float eps, const int32_t * __restrict__ rows, Act out) {
+__global__ __launch_bounds__(256) void k_rmsnorm_act(float * x, const float * __restrict__ w,
+                                                     int E, float eps, const int32_t * __restrict__ rows, Act out,
+                                                     Slices add) {
     __shared__ float red[4];
     const int o = blockIdx.x;
-    const float * xr = x + (size_t)(rows ? rows[o] : o) * E;
+    const int row = rows ? rows[o] : o;
+    float * xr = x + (size_t)row * E;
     float ss = 0.0f;
-    for (int i = threadIdx.x; i < E; i += 256) ss += xr[i] * xr[i];
+    for (int i = threadIdx.x; i < E; i += 256) {
+        float v = xr[i];
+        if (add.n > 0) {
+            for (int k = 0; k < add.n; ++k) v += add.data[(size_t)k * add.stride + (size_t)row * E + i];
+            xr[i] = v;          // re-read below by the same thread
+        }
+        ss += v * v;
+    }
     ss = wave_sum(ss);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
     __syncthreads();
@@ -568,14 +608,25 @@ __global__ __launch_bounds__(256) void k_rmsnorm_act(const float * __restrict__ 
 }
 
 // E % 32 == 0: 8 elements per lane, 16-byte loads and stores.
-__global__ __launch_bounds__(256) void k_rmsnorm_act8(const float * __restrict__ x, const float * __restrict__ w,
-                                                      int E, float eps, const int32_t * __restrict__ rows, Act out) {
+__global__ __launch_bounds__(256) void k_rmsnorm_act8(float * x, const float * __restrict__ w,
+                                                      int E, float eps, const int32_t * __restrict__ rows, Act out,
+                                                      Slices add) {
     __shared__ float red[4];
     const int o = blockIdx.x;
-    const float * xr = x + (size_t)(rows ? rows[o] : o) * E;
+    const int row = rows ? rows[o] : o;
+    float * xr = x + (size_t)row * E;
     float ss = 0.0f;
     for (int k = threadIdx.x * 8; k < E; k += 2048) {
-        const f4 a = *(const f4 *)(xr + k), b = *(const f4 *)(xr + k + 4);
+        f4 a = *(const f4 *)(xr + k), b = *(const f4 *)(xr + k + 4);
+        if (add.n > 0) {
+            for (int j = 0; j < add.n; ++j) {
+                const float * sl = add.data + (size_t)j * add.stride + (size_t)row * E + k;
+                a += *(const f4 *)sl;
+                b += *(const f4 *)(sl + 4);
+            }
+            *(f4 *)(xr + k) = a;          // re-read below by the same thread
+            *(f4 *)(xr + k + 4) = b;
+        }
         ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
     }
     ss = wave_sum(ss);
@@ -592,18 +643,19 @@ __global__ __launch_bounds__(256) void k_rmsnorm_act8(const float * __restrict__
     }
 }
 
-void rmsnorm_act(hipStream_t s, const float * x, const float * w, int E, float eps,
-                 const int32_t * rows, int n_rows, const Act & out) {
+void rmsnorm_act(hipStream_t s, float * x, const float * w, int E, float eps,
+                 const int32_t * rows, int n_rows, const Act & out, const Slices & add) {
     if (n_rows <= 0) return;
+    if (add.n > 0 && add.N != E) throw std::runtime_error("rmsnorm: the slices do not match the row width");
     if (out.K != E) throw std::runtime_error("rmsnorm: activation width does not match");
     if (E % 32 == 0 && out.sums) {
-        hipLaunchKernelGGL(k_rmsnorm_act8, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, out);
+        hipLaunchKernelGGL(k_rmsnorm_act8, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, out, add);
         check_launch("rmsnorm");
         return;
     }
     Act o = out;
     if (E % 32 != 0) o.sums = nullptr;
-    hipLaunchKernelGGL(k_rmsnorm_act, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, o);
+    hipLaunchKernelGGL(k_rmsnorm_act, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, o, add);
     check_launch("rmsnorm");
 }
 
@@ -865,6 +917,7 @@ struct RopeArgs {
     const float * rope_sin;
     int n_head, n_kv, hd, rope_dim, neox;
     float eps, qscale;
+    Slices from;
 };
 
 // One wave per head: lanes own element pairs.
@@ -877,7 +930,7 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
     const int QD = a.n_head * a.hd, KD = a.n_kv * a.hd;
     const int pairs = a.hd / 2;
     const int rp = a.rope_dim / 2;
-    const float * src = a.qkv + (size_t)t * (QD + 2 * KD) + (size_t)head * a.hd;
+    const size_t src_at = (size_t)t * (QD + 2 * KD) + (size_t)head * a.hd;
     const bool is_q = head < a.n_head;
     const bool is_k = !is_q && head < a.n_head + a.n_kv;
     const bool active = lane < pairs;
@@ -895,8 +948,19 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
         i0 = 2 * lane;
         i1 = i0 + 1;
     }
-    float x0 = active ? src[i0] : 0.0f;
-    float x1 = active ? src[i1] : 0.0f;
+    float x0 = 0.0f, x1 = 0.0f;
+    if (active) {
+        if (a.from.n > 0) {
+            for (int k = 0; k < a.from.n; ++k) {
+                const float * sl = a.from.data + (size_t)k * a.from.stride + src_at;
+                x0 += sl[i0];
+                x1 += sl[i1];
+            }
+        } else {
+            x0 = a.qkv[src_at + i0];
+            x1 = a.qkv[src_at + i1];
+        }
+    }
     const float * nw = is_q ? a.q_norm : (is_k ? a.k_norm : nullptr);
     if (nw) {
         const float ss = wave_sum(x0 * x0 + x1 * x1);
@@ -943,7 +1007,7 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
 
 void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, const PackBuffers & pk,
                 const float * q_norm, const float * k_norm, __half * q_out, __half * q_out_lo,
-                __half * k_pool, __half * v_pool) {
+                __half * k_pool, __half * v_pool, const Slices & from) {
     if (T <= 0) return;
     if (sh.head_dim > 128 || sh.head_dim % 32 != 0) throw std::runtime_error("rope_store: head_dim must be 32, 64, 96 or 128");
     RopeArgs a;
@@ -953,6 +1017,9 @@ void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, c
     a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.hd = sh.head_dim; a.rope_dim = sh.rope_dim; a.neox = sh.rope_neox ? 1 : 0;
     a.eps = sh.eps;
     a.qscale = 1.4426950408889634f / sqrtf((float)sh.head_dim);
+    a.from = from;
+    if (from.n > 0 && from.N != (sh.n_head + 2 * sh.n_head_kv) * sh.head_dim)
+        throw std::runtime_error("rope_store: the slices are not a fused q, k, v product");
     const int heads = sh.n_head + 2 * sh.n_head_kv;
     hipLaunchKernelGGL(k_rope_store, dim3(T, (heads + 3) / 4), dim3(256), 0, s, a);
     check_launch("rope_store");

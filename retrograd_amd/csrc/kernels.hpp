@@ -63,17 +63,33 @@ bool can_pack(int type, int64_t K, int64_t N);
 void repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int K, int N);
 
 enum : int { MM_STORE = 0, MM_ADD = 1 };
+// A matmul result left as n K-slices in the workspace instead of in y: element
+// (t, c) of the product (bias included) is the sum over s < n, in that order,
+// of data[s * stride + t * N + c]. n == 0: there are no slices, y holds the result.
+struct Slices {
+    const float * data = nullptr;
+    int n = 0;
+    size_t stride = 0;
+    int N = 0;
+};
 // y[t][col0 + n] (=|+=) sum_k W[n][k] * x[t][k] (+ bias[n]); y has row stride ldy.
-// `ws` is a zero-initialised device workspace of matmul_workspace_bytes() that
-// selects the LDS-staged tile kernels; without it the register-only tile
-// kernels run.
+// `ws` is a device workspace of matmul_workspace_bytes() that selects the
+// LDS-staged tile kernels; without it the register-only tile kernels run.
 void matmul(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
             int mode, const float * bias, void * ws = nullptr);
+// The same product, but a decode-sized matmul with few output rows may return
+// it as K-slices in ws and leave y untouched: the caller hands the slices to
+// the kernel that consumes the result (rmsnorm_act, rope_store) or to
+// reduce_slices. The slices live until the next matmul that uses ws.
+Slices matmul_deferred(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                       int mode, const float * bias, void * ws);
+// y[t][col0 + c] (=|+=) sum of the slices.
+void reduce_slices(hipStream_t s, const Slices & sl, int T, float * y, int ldy, int col0, int mode);
 size_t matmul_workspace_bytes();
 extern int g_mm_debug;         // timing experiments (see MMArgs::debug)
 extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic
-void matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
-                int mode, const float * bias, void * ws);
+Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                  int mode, const float * bias, void * ws, bool may_slice);
 // Forces the generic (raw layout) kernel; used to cross-check the tile kernels.
 void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
                     int mode, const float * bias);
@@ -82,9 +98,10 @@ void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float
 void embed(hipStream_t s, const Weight & emb, const int32_t * tok, int T, float * x);
 
 // act = f16(x * rsqrt(mean(x^2) + eps) * w) (+ block sums). `rows` selects the
-// input rows (null: identity), n_rows outputs.
-void rmsnorm_act(hipStream_t s, const float * x, const float * w, int E, float eps,
-                 const int32_t * rows, int n_rows, const Act & out);
+// input rows (null: identity), n_rows outputs. With slices, x[row] += their sum
+// first (written back), which completes a deferred matmul into the residual.
+void rmsnorm_act(hipStream_t s, float * x, const float * w, int E, float eps,
+                 const int32_t * rows, int n_rows, const Act & out, const Slices & add = Slices());
 
 // act = f16(x) (+ block sums): the plain conversion every producer fuses.
 void to_act(hipStream_t s, const float * x, int T, int K, const Act & out);
@@ -147,9 +164,10 @@ struct AttnShape {
 // qkv f32 [T][QD + 2*KD] (+ optional per-head RMSNorm weights) -> q as an f16
 // hi/lo pair [T][QD] each (rotated, pre-scaled by log2(e)/sqrt(head_dim)) and
 // the K/V pages of the layer (f16, the KV cache precision).
+// With slices (of a [T][QD + 2*KD] product) the values are their sum and qkv is not read.
 void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, const PackBuffers & pk,
                 const float * q_norm, const float * k_norm, __half * q_out, __half * q_out_lo,
-                __half * k_pool, __half * v_pool);
+                __half * k_pool, __half * v_pool, const Slices & from = Slices());
 
 // Split-KV paged attention over the step's query tiles. partial holds, per
 // (item, column), m (log2 domain), l and head_dim unnormalised outputs.

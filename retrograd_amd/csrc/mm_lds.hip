@@ -15,9 +15,10 @@
 //     the current one is multiplied.
 //
 // Few row tiles (N = 4096 at batch 64) do not give every CU a workgroup, so K
-// can also be split across workgroups: each writes its partial sums to a
-// workspace, and the workgroup that finishes last for a row group adds the
-// partials in slice order - the result does not depend on which one is last.
+// can also be split across workgroups: each writes its sums over its slice of K
+// to a workspace, and whoever consumes the result adds the slices in slice
+// order (the next kernel of the step, or reduce_slices) - no workgroup waits
+// for another and the sum order is fixed.
 #include "dev_common.hpp"
 
 namespace rk {
@@ -77,82 +78,40 @@ __device__ __forceinline__ h8 lds_h8(const uint8_t * buf, int block, int lane) {
     return *(const h8 *)(buf + block * 1024 + lane * 16);
 }
 
-// Stores or reduces the accumulators. acc[r][t][i] is token tbase + 16t + 4g + i,
-// weight row 16 * rt[r] + r16.
+// Stores the accumulators: to y, or (split K) to this workgroup's slice of the
+// workspace, the bias going into slice 0. acc[r][t][i] is token
+// tbase + 16t + 4g + i, weight row 16 * rt[r] + r16.
 template <int NT, int R>
 __device__ __forceinline__ void finish(const MMArgs & a, f4 (&acc)[R][NT], const int (&rt)[R], int tbase, int nt,
-                                       int rg, int ks, int * flag, bool owner) {
+                                       int ks, bool owner) {
+    if (!owner) return;
     const int lane = threadIdx.x & 63;
     const int r16 = lane & 15, g = lane >> 4;
-    if (a.ksplit > 1) {
-        const size_t tpad = (size_t)gridDim.y * 64;
-        float * mine = a.partial + (size_t)ks * tpad * a.N;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            if (!owner || rt[r] >= a.n_row_tiles) continue;
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const size_t tok = (size_t)tbase + t * 16 + 4 * g + i;
-                    mine[tok * a.N + rt[r] * 16 + r16] = acc[r][t][i];
-                }
-        }
-        __threadfence();
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            int32_t * c = a.counters + rg * gridDim.y + blockIdx.y;
-            const int prev = atomicAdd(c, 1);
-            const int last = prev == a.ksplit - 1;
-            if (last) *c = 0;              // ready for the next launch
-            *flag = last;
-        }
-        __syncthreads();
-        if (!*flag || !owner) return;
-        __threadfence();
-        // Every partial address was written exactly once, by one workgroup, before
-        // its counter increment: plain loads see it. Slice order is the sum order.
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int t = 0; t < NT; ++t) acc[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
-        for (int k = 0; k < a.ksplit; ++k) {
-            const float * slice = a.partial + (size_t)k * tpad * a.N;
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                if (rt[r] >= a.n_row_tiles) continue;
-#pragma unroll
-                for (int t = 0; t < NT; ++t)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const size_t tok = (size_t)tbase + t * 16 + 4 * g + i;
-                        acc[r][t][i] += slice[tok * a.N + rt[r] * 16 + r16];
-                    }
-            }
-        }
-    }
-    if (!owner) return;
+    const bool sliced = a.ksplit > 1;
+    float * slice = sliced ? a.partial + (size_t)ks * 64 * a.N : nullptr;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (rt[r] >= a.n_row_tiles) continue;
         const int n = rt[r] * 16 + r16;
-        const float bias = a.bias ? a.bias[n] : 0.0f;
+        const float bias = (a.bias && ks == 0) ? a.bias[n] : 0.0f;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             if (t >= nt) break;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int tok = tbase + t * 16 + 4 * g + i;
-                if (tok < a.T) {
+                if (tok >= a.T) continue;
+                const float v = acc[r][t][i] + bias;
+                if (sliced) {
+                    slice[(size_t)tok * a.N + n] = v;
+                } else {
                     float * p = a.y + (size_t)tok * a.ldy + a.col0 + n;
-                    const float v = acc[r][t][i] + bias;
                     *p = a.mode == MM_ADD ? *p + v : v;
                 }
             }
         }
     }
 }
-
 
 // (x & mask) | bits in one instruction
 __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) {
@@ -198,7 +157,6 @@ __device__ __forceinline__ void join_halves(f4 (&acc)[R][NT], uint8_t * smem, in
 template <int NT, int R>
 __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ int flag;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rw = wave & 3, kh = wave >> 2;
@@ -345,13 +303,12 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
         }
     }
     join_halves<NT, R>(acc, smem, rw, kh, lane);
-    finish<NT, R>(a, acc, rt, tbase, nt, rg, ks, &flag, kh == 0);
+    finish<NT, R>(a, acc, rt, tbase, nt, ks, kh == 0);
 }
 
 template <int NT, int R>
 __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    __shared__ int flag;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int rw = wave & 3, kh = wave >> 2;
@@ -383,7 +340,8 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
             const uint8_t * tile = wbase[r] + (size_t)sb * 4352;
             w.hdr[r] = *(const u4 *)(tile + r16 * 16);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) w.q[r][j] = *(const u4 *)(tile + 256 + (2 * kh + j) * 1024 + lane * 16);
+            for (int j = 0; j < 2; ++j)
+                w.q[r][j] = *(const u4 *)(tile + 256 + (2 * kh + j) * 1024 + lane * 16);
         }
     };
     const h2 bias1152 = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
@@ -441,7 +399,7 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
         }
     }
     join_halves<NT, R>(acc, smem, rw, kh, lane);
-    finish<NT, R>(a, acc, rt, tbase, nt, rg, ks, &flag, kh == 0);
+    finish<NT, R>(a, acc, rt, tbase, nt, ks, kh == 0);
 }
 
 template <int NT, int R>
@@ -466,11 +424,10 @@ static void launch2(hipStream_t s, int type, const MMArgs & a, dim3 grid) {
 }
 
 size_t matmul_workspace_bytes() {
-    // partial sums of a split matmul (<= 64 tokens x 16 slices x 8192 columns), counters, zeros
-    return (size_t)64 * 16 * 8192 * 4 + 65536 + 256;
+    // K-slices of a split matmul: up to 16 slices x 64 tokens x 8192 columns
+    return (size_t)64 * 16 * 8192 * 4;
 }
 
-// The LDS-staged path; ws must be zero-initialised once.
 int g_mm_debug = 0;
 int g_mm_force_ksplit = 0;
 
@@ -483,38 +440,42 @@ static void dispatch_nt(hipStream_t s, int type, int nt, const MMArgs & a, dim3 
     }
 }
 
-void matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
-                int mode, const float * bias, void * ws) {
+Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                  int mode, const float * bias, void * ws, bool may_slice) {
     MMArgs a {};
     a.debug = g_mm_debug;
     a.w = w.packed; a.x = x.x; a.sums = x.sums; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
     a.n_row_tiles = w.N / 16;
-    const size_t partial_bytes = (size_t)64 * 16 * 8192 * 4;
     a.partial = (float *)ws;
-    a.counters = (int32_t *)((uint8_t *)ws + partial_bytes);
     const int nsb = w.K / 256;
     const int nt = T > 32 ? 4 : (T > 16 ? 2 : 1);
     const int chunks = (T + 63) / 64;
     constexpr int R = 2;
     a.n_row_groups = (a.n_row_tiles + 4 * R - 1) / (4 * R);
-    // Split K across workgroups when the row groups alone leave most CUs idle
-    // (decode-sized batches only: the partial buffer holds one 64-token chunk).
+    // One chunk of tokens and few row groups: split K so that about every CU
+    // gets a workgroup, each with at least two super-blocks.
     int ksplit = 1;
-    if (chunks == 1) {
-        while (a.n_row_groups * ksplit < 192 && ksplit * 2 <= 16 && nsb / (ksplit * 2) >= 2
-               && (size_t)ksplit * 2 * 64 * w.N * 4 <= partial_bytes && a.n_row_groups * ksplit * 2 <= 16384) {
-            ksplit *= 2;
+    if (may_slice && chunks == 1) {
+        int want = std::min(16, 256 / a.n_row_groups);
+        if (g_mm_force_ksplit > 0) want = g_mm_force_ksplit;
+        want = std::min(want, nsb / 2);
+        if (want > 1) {
+            const int per = (nsb + want - 1) / want;
+            ksplit = (nsb + per - 1) / per;
         }
-    }
-    if (g_mm_force_ksplit > 0 && chunks == 1) ksplit = g_mm_force_ksplit;
-    if ((size_t)ksplit * 64 * w.N * 4 > partial_bytes || (ksplit > 1 && a.n_row_groups > 16384)) {
-        throw std::runtime_error("matmul_lds: the split does not fit the workspace");
+        if ((size_t)ksplit * 64 * w.N * 4 > matmul_workspace_bytes()) {
+            if (g_mm_force_ksplit > 0) throw std::runtime_error("matmul_lds: the split does not fit the workspace");
+            ksplit = 1;
+        }
     }
     a.ksplit = ksplit;
     dim3 grid(a.n_row_groups * ksplit, chunks);
     dispatch_nt<R>(s, w.type, nt, a, grid);
     check_launch("matmul_lds");
+    Slices out;
+    if (ksplit > 1) { out.data = a.partial; out.n = ksplit; out.stride = (size_t)64 * w.N; out.N = w.N; }
+    return out;
 }
 
 }  // namespace rk

@@ -36,6 +36,12 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
 int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,
                              int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us);
 
+/* Microseconds per launch of a plain streaming kernel over `bytes` of device
+ * memory: a copy (reads and writes `bytes` each) or, read_only, a pure read.
+ * Known traffic: the yardstick the memory counters and bandwidth figures of the
+ * real kernels are scaled by. */
+int retro_kernel_stream_time(int64_t bytes, int32_t read_only, int32_t iters, double * out_us);
+
 int32_t retro_kernel_page_size(void);   /* positions per KV page */
 int32_t retro_kernel_max_topk(void);    /* candidates sample_prepare can return */
 

@@ -143,6 +143,27 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
     });
 }
 
+int retro_kernel_stream_time(int64_t bytes, int32_t read_only, int32_t iters, double * out_us) {
+    return guarded([&]() -> int {
+        DevBuf src, dst;
+        src.alloc((size_t)bytes);
+        dst.alloc(read_only ? (size_t)1 << 16 : (size_t)bytes);
+        ok(hipMemset(src.ptr, 0x5a, src.bytes), "fill");
+        hipEvent_t e0, e1;
+        ok(hipEventCreate(&e0), "event"); ok(hipEventCreate(&e1), "event");
+        for (int i = 0; i < 2; ++i) rk::stream_copy(nullptr, src.ptr, dst.ptr, (size_t)bytes, read_only);
+        ok(hipEventRecord(e0, nullptr), "record");
+        for (int i = 0; i < iters; ++i) rk::stream_copy(nullptr, src.ptr, dst.ptr, (size_t)bytes, read_only);
+        ok(hipEventRecord(e1, nullptr), "record");
+        ok(hipEventSynchronize(e1), "sync");
+        float ms = 0;
+        ok(hipEventElapsedTime(&ms, e0, e1), "elapsed");
+        (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+        *out_us = (double)ms * 1e3 / iters;
+        return 0;
+    });
+}
+
 int32_t retro_kernel_page_size(void) { return rk::PAGE; }
 int32_t retro_kernel_max_topk(void) { return rk::MAX_TOPK; }
 

@@ -153,6 +153,32 @@ __device__ __forceinline__ void store_act8(const float (&v)[8], const Act & out,
 }
 
 // ---------------------------------------------------------------------------
+// plain streaming kernels: the yardstick for memory counters and bandwidth
+
+__global__ __launch_bounds__(256) void k_stream_copy(const u4 * __restrict__ src, u4 * __restrict__ dst, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+
+__global__ __launch_bounds__(256) void k_stream_read(const u4 * __restrict__ src, u4 * __restrict__ sink, size_t n) {
+    u4 acc = {0, 0, 0, 0};
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        const u4 v = src[i];
+        acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w;
+    }
+    // data-dependent and practically never true: keeps the loads alive without a store stream
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[blockIdx.x] = acc;
+}
+
+void stream_copy(hipStream_t s, const void * src, void * dst, size_t bytes, int read_only) {
+    const size_t n = bytes / 16;
+    if (n == 0) return;
+    const unsigned blocks = (unsigned)std::min<size_t>((n + 255) / 256, 256 * 16);
+    if (read_only) hipLaunchKernelGGL(k_stream_read, dim3(blocks), dim3(256), 0, s, (const u4 *)src, (u4 *)dst, n);
+    else hipLaunchKernelGGL(k_stream_copy, dim3(blocks), dim3(256), 0, s, (const u4 *)src, (u4 *)dst, n);
+    check_launch("stream_copy");
+}
+
+// ---------------------------------------------------------------------------
 // weight repacking (runs once per tensor at load)
 
 __global__ void k_repack_q4k(const uint8_t * __restrict__ raw, uint8_t * __restrict__ dst, int nsb, int n_tiles) {

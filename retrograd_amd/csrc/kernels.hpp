@@ -58,6 +58,10 @@ struct Act {
 inline size_t act_halves(int T, int K) { return (size_t)((T + 63) / 64) * (size_t)((K + 31) / 32 * 32) * 128; }
 inline size_t act_sum_halves(int T, int K) { return (size_t)((T + 63) / 64) * (size_t)((K + 255) / 256) * 2048; }
 
+// dst = src (16-byte words, grid-stride) or, read_only, a pure read of src
+// (dst needs 64 KiB): plain streaming kernels of known traffic.
+void stream_copy(hipStream_t s, const void * src, void * dst, size_t bytes, int read_only);
+
 bool can_pack(int type, int64_t K, int64_t N);
 // raw (device, GGUF layout) -> packed (device). Both hold `bytes` bytes.
 void repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int K, int N);

@@ -120,7 +120,7 @@ STEP_SYMBOLS = [
     "retro_grammar_gbnf", "retro_grammar_free", "retro_last_error",
 ]
 KERNEL_SYMBOLS = [
-    "retro_kernel_matmul", "retro_kernel_matmul_time", "retro_kernel_sample_prepare", "retro_kernel_page_size", "retro_kernel_max_topk",
+    "retro_kernel_matmul", "retro_kernel_matmul_time", "retro_kernel_stream_time", "retro_kernel_sample_prepare", "retro_kernel_page_size", "retro_kernel_max_topk",
     "retro_engine_debug_logits", "retro_engine_debug_kv", "retro_engine_debug_pack", "retro_engine_debug_pages",
     "retro_engine_debug_profile", "retro_engine_debug_profile_categories", "retro_engine_debug_profile_read",
 ]
@@ -191,6 +191,7 @@ def load_library() -> C.CDLL:
                                                 C.POINTER(C.c_double), _i32p, _f32p]
     lib.retro_kernel_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,
                                              C.c_int32, C.c_int32, C.POINTER(C.c_double)]
+    lib.retro_kernel_stream_time.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_double)]
     lib.retro_kernel_page_size.restype = C.c_int32
     lib.retro_kernel_max_topk.restype = C.c_int32
     lib.retro_engine_debug_logits.argtypes = [C.c_void_p, _f32p, C.c_size_t, C.POINTER(C.c_size_t)]
@@ -707,6 +708,15 @@ def kernel_matmul_time(ggml_type: int, n_rows: int, k: int, n_tokens: int, mode:
     out = C.c_double()
     s = load_library().retro_kernel_matmul_time(ggml_type, n_rows, k, n_tokens, mode, iters, debug, force_ksplit,
                                                 C.byref(out))
+    if s != 0:
+        _raise(s)
+    return out.value
+
+
+def kernel_stream_time(n_bytes: int, read_only: bool = False, iters: int = 20) -> float:
+    """Microseconds per launch of a plain copy (or pure read) of n_bytes."""
+    out = C.c_double()
+    s = load_library().retro_kernel_stream_time(n_bytes, 1 if read_only else 0, iters, C.byref(out))
     if s != 0:
         _raise(s)
     return out.value

@@ -1074,7 +1074,7 @@ struct AttnArgs {
 };
 
 template <int HD>
-__global__ __launch_bounds__(64) void k_attention(AttnArgs a) {
+__global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     constexpr int KS = HD / 32;     // k-steps of QK^T
     constexpr int DT = HD / 16;     // dim tiles of PV
     const int item = blockIdx.x;
@@ -1120,19 +1120,25 @@ __global__ __launch_bounds__(64) void k_attention(AttnArgs a) {
     float m_run = -INFINITY, l_run = 0.0f;
     const size_t page_elems = (size_t)PAGE * HD;
 
-    for (int pi = page_first; pi < page_end; ++pi) {
-        const int pid = a.table[(size_t)slot * a.max_pages + pi];
+    // page ids of this split, one per lane
+    const int n_pages = page_end - page_first;
+    const int my_pid = lane < n_pages ? a.table[(size_t)slot * a.max_pages + page_first + lane] : 0;
+    auto load_k = [&](int idx, h8 (&kreg)[KS][2]) {
+        const int pid = __builtin_amdgcn_readlane(my_pid, idx);
         const __half * kp = a.k_pool + ((size_t)pid * a.n_kv + h) * page_elems;
-        const __half * vp = a.v_pool + ((size_t)pid * a.n_kv + h) * page_elems;
-        h8 kreg[KS][2], vreg[DT];
 #pragma unroll
         for (int j = 0; j < KS; ++j) {
             kreg[j][0] = load_h8(kp + ((j * 2 + 0) * 64 + lane) * 8);
             kreg[j][1] = load_h8(kp + ((j * 2 + 1) * 64 + lane) * 8);
         }
+    };
+    auto load_v = [&](int idx, h8 (&vreg)[DT]) {
+        const int pid = __builtin_amdgcn_readlane(my_pid, idx);
+        const __half * vp = a.v_pool + ((size_t)pid * a.n_kv + h) * page_elems;
 #pragma unroll
         for (int d = 0; d < DT; ++d) vreg[d] = load_h8(vp + (d * 64 + lane) * 8);
-
+    };
+    auto attend = [&](int pi, const h8 (&kreg)[KS][2], const h8 (&vreg)[DT]) {
         f4 s0 = (f4){0.f, 0.f, 0.f, 0.f}, s1 = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < KS; ++j) {
@@ -1177,6 +1183,21 @@ __global__ __launch_bounds__(64) void k_attention(AttnArgs a) {
             for (int i = 0; i < 4; ++i) o[d][i] *= alpha;
             o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt, o[d], 0, 0, 0);
             o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt_lo, o[d], 0, 0, 0);
+        }
+    };
+    // V of a page loads while its scores are computed, K of the next page while
+    // the page is multiplied: two K register sets, one V set
+    if (n_pages > 0) {
+        h8 kA[KS][2], kB[KS][2], v[DT];
+        load_k(0, kA);
+        for (int i = 0; i < n_pages; i += 2) {
+            load_v(i, v);
+            if (i + 1 < n_pages) load_k(i + 1, kB);
+            attend(page_first + i, kA, v);
+            if (i + 1 >= n_pages) break;
+            load_v(i + 1, v);
+            if (i + 2 < n_pages) load_k(i + 2, kA);
+            attend(page_first + i + 1, kB, v);
         }
     }
     l_run += __shfl_xor(l_run, 16, 64);

@@ -48,6 +48,11 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=16)
     ap.add_argument("--profile-all", action="store_true", help="also print a per-category kernel time breakdown to stderr")
+    ap.add_argument("--stream-probe", type=int, default=0, metavar="MIB",
+                    help="after the timed steps also launch the plain copy kernel over this many MiB (known traffic, "
+                         "for scaling rocprofv3 memory counters)")
+    ap.add_argument("--traffic-file", default=str(ROOT / "profiles" / "k_attention_c2_hbm_traffic.txt"),
+                    help="text summary of the rocprofv3 --pmc runs; its traffic_bytes_per_launch line fills roofline.traffic")
     return ap.parse_args()
 
 
@@ -140,6 +145,23 @@ class Workload:
                     self.finished += 1
                     self.new_request(s.slot)
         return sampled, decode_rows, cells, tokens, dt
+
+
+def read_traffic(path: str, workload: str):
+    """HBM bytes per launch of the dominant kernel as measured with rocprofv3
+    --pmc FETCH_SIZE / WRITE_SIZE (scaled by the copy kernel), from the text
+    summary of those runs; None when there is no summary for this workload."""
+    try:
+        fields = {}
+        for line in Path(path).read_text().splitlines():
+            if "=" in line and not line.startswith("#"):
+                k, v = line.split("=", 1)
+                fields[k.strip()] = v.strip()
+        if fields.get("workload") != workload:
+            return None
+        return float(fields["traffic_bytes_per_launch"])
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def main() -> int:
@@ -274,12 +296,12 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "k_attention<128> (paged split-KV attention, one launch per layer)",
+            "kernel": "k_attention<128, true> (paged split-KV attention of a decode step, one launch per layer)",
             "achieved": round(attn_gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(attn_gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": read_traffic(args.traffic_file, shape.name),
             "algorithmic_bytes_per_launch": round(algo_bytes_per_launch),
             "avg_launch_us": round(attn_avg_s * 1e6, 2),
             "launches_timed": attn_launches,
@@ -290,6 +312,9 @@ def main() -> int:
             },
         },
     }
+    if args.stream_probe > 0:
+        us = E.kernel_stream_time(args.stream_probe << 20, False, 3)
+        print("[bench] copy kernel over %d MiB: %.1f us per launch" % (args.stream_probe, us), file=sys.stderr, flush=True)
     if args.profile_all:
         print("[bench] kernel time per step (ms): " + ", ".join(
             "%s=%.3f" % (k, v[0] / args.steps) for k, v in prof.items()), file=sys.stderr, flush=True)

@@ -932,7 +932,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
                       table_.as<int32_t>(), max_pages_, qt_, hp_.n_head_kv, inv_freq_.as<double>(),
                       hp_.rope_dim / 2, pk_);
         prof_end(PC_PACK, pt_pack);
-        forward(T, n_out, n_tiles, n_items);
+        forward(T, n_out, n_tiles, n_items, (size_t)T == n_rows);
 
         // ---- sampling: the device scans the vocabulary, the host draws.
         std::vector<int32_t> kreq((size_t)std::max(n_out, 1), 0);
@@ -1055,7 +1055,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
     return 0;
 }
 
-void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
+void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_rows) {
     const HParams & h = hp_;
     const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim, F = h.n_ff;
     rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps};
@@ -1099,7 +1099,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items) {
         pt_ = prof_begin(PC_ATTN);
         rk::attention(stream_, q_half_.as<__half>(), q_half_lo_.as<__half>(), sh, pk_, table_.as<int32_t>(), max_pages_,
                       k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), n_items, n_tiles,
-                      partial_.as<float>());
+                      partial_.as<float>(), one_token_rows);
         prof_end(PC_ATTN, pt_);
         pt_ = prof_begin(PC_COMBINE);
         rk::attention_combine(stream_, partial_.as<float>(), T, sh, pk_, act_q);

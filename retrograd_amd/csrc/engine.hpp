@@ -150,7 +150,7 @@ private:
     void copy_page(int32_t src, int32_t dst);
     void set_page(int32_t slot, int idx, int32_t page);
     void clear_slot(Slot & s, int32_t slot);
-    void forward(int T, int n_out, int n_tiles, int n_items);
+    void forward(int T, int n_out, int n_tiles, int n_items, bool one_token_rows);
 
     retro_engine_config cfg_ {};
     HParams hp_;

@@ -1073,7 +1073,8 @@ struct AttnArgs {
     int n_head, n_kv, G;
 };
 
-template <int HD>
+// ONE: every tile holds a single query token (a pure decode step).
+template <int HD, bool ONE>
 __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     constexpr int KS = HD / 32;     // k-steps of QK^T
     constexpr int DT = HD / 16;     // dim tiles of PV
@@ -1090,7 +1091,7 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     const int nsplit = a.tile_nsplit[tile];
     const int rel = item - a.tile_item0[tile];
     const int h = rel / nsplit, split = rel % nsplit;
-    const int t0 = a.tile_t0[tile], nq = a.tile_nq[tile];
+    const int t0 = a.tile_t0[tile], nq = ONE ? 1 : a.tile_nq[tile];
     const int kv_begin = a.tile_kv_begin[tile];
     const int slot = a.seq[t0];
     const int qi = c / a.G, gi = c % a.G;
@@ -1218,7 +1219,7 @@ size_t attention_partial_floats(int n_items, int head_dim) {
 
 void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnShape & sh, const PackBuffers & pk,
                const int32_t * table, int max_pages, const __half * k_pool, const __half * v_pool,
-               int n_items, int n_tiles, float * partial) {
+               int n_items, int n_tiles, float * partial, bool one_token_rows) {
     if (n_items <= 0) return;
     AttnArgs a;
     a.q = q; a.q_lo = q_lo; a.k_pool = k_pool; a.v_pool = v_pool; a.table = table;
@@ -1227,12 +1228,18 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
     a.partial = partial; a.n_tiles = n_tiles; a.n_items = n_items; a.max_pages = max_pages;
     a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.G = sh.n_head / sh.n_head_kv;
     if (a.G > 16 || sh.n_head % sh.n_head_kv != 0) throw std::runtime_error("attention: unsupported head grouping");
+#define ATTN_LAUNCH(HD_) \
+    do { \
+        if (one_token_rows) hipLaunchKernelGGL((k_attention<HD_, true>), dim3(n_items), dim3(64), 0, s, a); \
+        else hipLaunchKernelGGL((k_attention<HD_, false>), dim3(n_items), dim3(64), 0, s, a); \
+    } while (0)
     switch (sh.head_dim) {
-        case 32:  hipLaunchKernelGGL(k_attention<32>, dim3(n_items), dim3(64), 0, s, a); break;
-        case 64:  hipLaunchKernelGGL(k_attention<64>, dim3(n_items), dim3(64), 0, s, a); break;
-        case 128: hipLaunchKernelGGL(k_attention<128>, dim3(n_items), dim3(64), 0, s, a); break;
+        case 32:  ATTN_LAUNCH(32); break;
+        case 64:  ATTN_LAUNCH(64); break;
+        case 128: ATTN_LAUNCH(128); break;
         default: throw std::runtime_error("attention: head_dim must be 32, 64 or 128");
     }
+#undef ATTN_LAUNCH
     check_launch("attention");
 }
 

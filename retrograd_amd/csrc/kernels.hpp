@@ -173,11 +173,12 @@ void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, c
                 const float * q_norm, const float * k_norm, __half * q_out, __half * q_out_lo,
                 __half * k_pool, __half * v_pool, const Slices & from = Slices());
 
-// Split-KV paged attention over the step's query tiles. partial holds, per
+// Split-KV paged attention over the step's query tiles (one_token_rows: every
+// row of the step has a single token, so every tile has a single query). partial holds, per
 // (item, column), m (log2 domain), l and head_dim unnormalised outputs.
 void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnShape & sh, const PackBuffers & pk,
                const int32_t * table, int max_pages, const __half * k_pool, const __half * v_pool,
-               int n_items, int n_tiles, float * partial);
+               int n_items, int n_tiles, float * partial, bool one_token_rows = false);
 // Merges the splits: out act [T][QD] (+ block sums).
 void attention_combine(hipStream_t s, const float * partial, int T, const AttnShape & sh,
                        const PackBuffers & pk, const Act & out);

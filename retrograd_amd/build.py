@@ -16,6 +16,11 @@ CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libretro_hip.so"
 SOURCES = ["kernels.hip", "mm_lds.hip", "engine.cpp", "capi.cpp", "capi_test.cpp"]
+# host-only sources (the step scheduler): plain C++, no device pass
+HOST_SOURCES = ["sched/prefix_tree.cpp", "sched/scheduler.cpp", "sched/fake_backend.cpp", "sched/engine_backend.cpp",
+                "sched/capi_sched.cpp"]
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-Wno-unused-parameter", "-D__HIP_PLATFORM_AMD__",
+              "-I/opt/rocm/include"]
 HEADERS = ["kernels.hpp", "dev_common.hpp", "engine.hpp", "sampler.hpp", "gguf_file.hpp"]
 
 # packed-fp32 code generation is switched off for every HIP translation unit.
@@ -47,6 +52,17 @@ def build(verbose: bool = False) -> Path:
             raise RuntimeError("hipcc failed on %s:\n%s" % (src, err))
         if verbose and err.strip():
             print(err, file=sys.stderr)
+        objs.append(str(obj))
+    for src in HOST_SOURCES:
+        obj = obj_dir / (src.replace("/", "_").rsplit(".", 1)[0] + ".o")
+        cmd = [hipcc(), *HOST_FLAGS, "-x", "c++", "-c", str(CSRC / src), "-o", str(obj)]
+        if verbose:
+            print(" ".join(cmd), file=sys.stderr)
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("hipcc failed on %s:\n%s" % (src, res.stderr))
+        if verbose and res.stderr.strip():
+            print(res.stderr, file=sys.stderr)
         objs.append(str(obj))
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *objs]
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -88,9 +88,12 @@ def test_library_exports_every_declared_symbol():
     lib = E.load_library()
     step = _declared(ROOT / "include" / "retro_step.h")
     kern = [s for s in _declared(ROOT / "include" / "retro_kernels.h") if s not in step]
+    sched = [s for s in _declared(ROOT / "include" / "retro_scheduler.h") if s not in step]
+    from retrograd_amd import scheduler as S
     assert sorted(step) == sorted(E.STEP_SYMBOLS)
     assert sorted(kern) == sorted(E.KERNEL_SYMBOLS)
-    for sym in step + kern:
+    assert sorted(sched) == sorted(S.SCHED_SYMBOLS)
+    for sym in step + kern + sched:
         assert hasattr(lib, sym), sym
 
 

@@ -455,7 +455,8 @@ int retro_engine_active_adapter(retro_engine * engine, char * buffer, size_t n_b
 
 int retro_engine_adapter_load(retro_engine * engine, const char * adapter_path, float scale, int32_t * out_id) {
     return boundary([&]() -> int {
-        if (!checked(engine)) return -1;
+        Engine * e = checked(engine);
+        if (!e) return -1;
         if (blank(adapter_path)) {
             set_error("adapter_path is required");
             return -1;
@@ -468,28 +469,27 @@ int retro_engine_adapter_load(retro_engine * engine, const char * adapter_path, 
             set_error("the adapter scale must be finite");
             return -1;
         }
-        set_error("per-row LoRA adapters are not supported by this library yet");
-        return -1;
+        return e->adapter_load(adapter_path, scale, out_id);
     });
 }
 
 int retro_engine_adapter_unload(retro_engine * engine, int32_t id) {
     return boundary([&]() -> int {
-        if (!checked(engine)) return -1;
-        set_error("no per-row adapter is loaded under id " + std::to_string(id));
-        return -1;
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->adapter_unload(id);
     });
 }
 
 int retro_engine_adapter_rows_info(retro_engine * engine, retro_adapter_rows_info * out_info) {
     return boundary([&]() -> int {
-        if (!checked(engine)) return -1;
+        Engine * e = checked(engine);
+        if (!e) return -1;
         if (!out_info) {
             set_error("out_info is required");
             return -1;
         }
-        *out_info = retro_adapter_rows_info{};
-        out_info->struct_size = sizeof(retro_adapter_rows_info);
+        e->adapter_rows_info(out_info);
         return 0;
     });
 }

@@ -762,13 +762,9 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
             set_error("step row slot is outside the context's sequence range");
             return -3;
         }
-        if (row.adapter != 0) {
-            // No per-row adapter is ever loaded in this build (retro_engine_adapter_load
-            // refuses), so the only other legal value is the base model.
-            if (row.adapter != RETRO_STEP_ADAPTER_BASE) {
-                set_error("step row adapter " + std::to_string(row.adapter) + " is not a loaded per-row adapter");
-                return -3;
-            }
+        if (row.adapter != 0 && row.adapter != RETRO_STEP_ADAPTER_BASE && !row_adapters_.count(row.adapter)) {
+            set_error("step row adapter " + std::to_string(row.adapter) + " is not a loaded per-row adapter");
+            return -3;
         }
         if (row.pos0 < 0 || (int64_t)row.pos0 + row.n > n_ctx_seq) {
             set_error("step row positions exceed the per-sequence context");
@@ -900,13 +896,19 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
     rk::RowDesc * hd = h_stage_.as<rk::RowDesc>();
     int32_t * ht = (int32_t *)((uint8_t *)h_stage_.ptr + off_tok);
     int n_out = 0;
+    bool routed = false;
     {
         int at = 0;
         for (size_t r = 0; r < n_rows; ++r) {
             const RowView & row = rows[r];
             hd[r].slot = row.slot; hd[r].pos0 = row.pos0; hd[r].n = (int32_t)row.n; hd[r].tok_off = at;
             hd[r].sample = row.sample ? 1 : 0; hd[r].kv_begin = slots_[(size_t)row.slot].begin;
+            // route = 1-based index of the adapter in id order (0: the base model)
             hd[r].route = 0; hd[r].pad = 0;
+            if (row.adapter > 0) {
+                hd[r].route = 1 + (int32_t)std::distance(row_adapters_.begin(), row_adapters_.find(row.adapter));
+                routed = true;
+            }
             std::memcpy(ht + at, row.tokens, (size_t)row.n * 4);
             at += (int)row.n;
             if (row.sample) ++n_out;
@@ -932,7 +934,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
                       table_.as<int32_t>(), max_pages_, qt_, hp_.n_head_kv, inv_freq_.as<double>(),
                       hp_.rope_dim / 2, pk_);
         prof_end(PC_PACK, pt_pack);
-        forward(T, n_out, n_tiles, n_items, (size_t)T == n_rows);
+        forward(T, n_out, n_tiles, n_items, (size_t)T == n_rows, routed);
 
         // ---- sampling: the device scans the vocabulary, the host draws.
         std::vector<int32_t> kreq((size_t)std::max(n_out, 1), 0);
@@ -1055,7 +1057,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
     return 0;
 }
 
-void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_rows) {
+void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_rows, bool routed) {
     const HParams & h = hp_;
     const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim, F = h.n_ff;
     rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps};
@@ -1089,6 +1091,15 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
                     col += w.w.N;
                 }
             }
+            if (routed) {
+                // the adapter deltas go where the rotation kernel reads q, k, v from: the first slice or the buffer
+                float * dst = qkv_slices.n > 0 ? const_cast<float *>(qkv_slices.data) : qkv;
+                const rk::RowDesc * rows_d = d_stage_.as<rk::RowDesc>();
+                const int cols[3] = {0, QD, QD + KD}, widths[3] = {QD, KD, KD};
+                for (int tg = 0; tg < 3; ++tg)
+                    rk::lora_apply(stream_, lora_entries(l, tg), rows_d, pk_.row, act_e, T, widths[tg], dst, QD + 2 * KD,
+                                   cols[tg], lora_mid_.as<float>());
+            }
             prof_end(PC_QKV, pt_);
         }
         size_t pt_ = prof_begin(PC_ROPE);
@@ -1106,6 +1117,11 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         prof_end(PC_COMBINE, pt_);
         pt_ = prof_begin(PC_OPROJ);
         pending = rk::matmul_deferred(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
+        if (routed) {
+            float * dst = pending.n > 0 ? const_cast<float *>(pending.data) : x;
+            rk::lora_apply(stream_, lora_entries(l, 3), d_stage_.as<rk::RowDesc>(), pk_.row, act_q, T, E, dst, E, 0,
+                           lora_mid_.as<float>());
+        }
         prof_end(PC_OPROJ, pt_);
         pt_ = prof_begin(PC_NORM);
         rk::rmsnorm_act(stream_, x, L.ffn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending);
@@ -1133,6 +1149,153 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         rk::matmul(stream_, lm_head_.w, act_o, n_out, logits_.as<float>(), h.n_vocab, 0, rk::MM_STORE,
                    out_bias_.as<float>(), mm_ws_.ptr);
         prof_end(PC_HEAD, pt_);
+    }
+}
+
+// ---- per-row adapters -----------------------------------------------------------------------
+
+// A LoRA adapter file as the reference writes it (retro_lora.cpp:1004-1043,
+// 1143-1153): general.type = "adapter", adapter.type = "lora",
+// adapter.lora.alpha, tensors "<weight>.lora_a" ne = [n_in, r] and
+// "<weight>.lora_b" ne = [r, n_out].
+int Engine::adapter_load(const std::string & path, float scale, int32_t * out_id) {
+    if (next_adapter_id_ == INT32_MAX) {
+        set_error("per-row adapter ids are exhausted");
+        return -1;
+    }
+    std::unique_ptr<GgufFile> file;
+    try {
+        file.reset(new GgufFile(path));
+    } catch (const std::exception &) {
+        set_error("failed to load LoRA adapter: " + path);
+        return -1;
+    }
+    if (file->get_string("general.type") != "adapter" || file->get_string("adapter.type") != "lora") {
+        set_error("failed to load LoRA adapter: " + path);
+        return -1;
+    }
+    const HParams & h = hp_;
+    const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim;
+    static const char * kTargets[kLoraTargets] = {"attn_q", "attn_k", "attn_v", "attn_output"};
+    const int n_in[kLoraTargets] = {E, E, E, QD}, n_out[kLoraTargets] = {QD, KD, KD, E};
+    RowAdapterData data;
+    data.scale = scale;
+    data.alpha = file->get_float("adapter.lora.alpha", 0.0);
+    data.a.resize((size_t)h.n_layer * kLoraTargets);
+    data.b.resize((size_t)h.n_layer * kLoraTargets);
+    size_t claimed = 0;
+    for (int l = 0; l < h.n_layer; ++l) {
+        for (int tg = 0; tg < kLoraTargets; ++tg) {
+            const std::string base = "blk." + std::to_string(l) + "." + kTargets[tg] + ".weight";
+            const TensorInfo * ta = file->find(base + ".lora_a");
+            const TensorInfo * tb = file->find(base + ".lora_b");
+            if (!ta && !tb) continue;
+            if (!ta || !tb) {
+                set_error("LoRA adapter tensor " + base + " has no matching lora_a / lora_b pair");
+                return -1;
+            }
+            const int r = (int)ta->ne[1];
+            if (ta->ne[0] != n_in[tg] || tb->ne[1] != n_out[tg] || tb->ne[0] != r || r <= 0) {
+                set_error("LoRA adapter tensor " + base + " does not match the base model's shape");
+                return -1;
+            }
+            if (r > rk::LORA_MAX_RANK) {
+                set_error("LoRA rank " + std::to_string(r) + " exceeds the supported maximum of " + std::to_string(rk::LORA_MAX_RANK));
+                return -1;
+            }
+            if (data.rank != 0 && data.rank != r) {
+                set_error("a per-row adapter must use one rank for all of its targets");
+                return -1;
+            }
+            data.rank = r;
+            auto to_f32 = [&](const TensorInfo & t, int K, int rows, DevBuf & out) {
+                rk::geom_of(t.type);
+                if (rk::row_bytes(t.type, K) * (size_t)rows != t.nbytes) throw std::runtime_error("tensor " + t.name + " has an unexpected size");
+                DevBuf raw;
+                raw.alloc(t.nbytes);
+                hip_check(hipMemcpyAsync(raw.ptr, t.data, t.nbytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
+                out.alloc((size_t)rows * K * 4);
+                rk::decode_rows(stream_, t.type, raw.as<uint8_t>(), K, rows, out.as<float>());
+                hip_check(hipStreamSynchronize(stream_), "decode adapter tensor");
+            };
+            to_f32(*ta, n_in[tg], r, data.a[(size_t)l * kLoraTargets + tg]);      // A: r rows of n_in
+            to_f32(*tb, r, n_out[tg], data.b[(size_t)l * kLoraTargets + tg]);     // B: n_out rows of r
+            data.elements += (uint64_t)n_in[tg] + (uint64_t)n_out[tg];
+            claimed += 2;
+        }
+    }
+    // a target this engine does not route per row (embeddings, FFN, experts) must not be dropped silently
+    size_t lora_tensors = 0;
+    for (const TensorInfo & t : file->tensors()) {
+        const std::string & n = t.name;
+        if (n.size() > 7 && (n.compare(n.size() - 7, 7, ".lora_a") == 0 || n.compare(n.size() - 7, 7, ".lora_b") == 0)) ++lora_tensors;
+    }
+    if (lora_tensors != claimed) {
+        set_error("failed to stack the per-row adapters: only attn_q, attn_k, attn_v and attn_output targets are routed per row");
+        return -1;
+    }
+    if (data.rank == 0) {
+        set_error("failed to load LoRA adapter: " + path + " holds no LoRA tensor pair");
+        return -1;
+    }
+    const int32_t id = next_adapter_id_++;
+    row_adapters_.emplace(id, std::move(data));
+    rebuild_lora_table();
+    *out_id = id;
+    return 0;
+}
+
+int Engine::adapter_unload(int32_t id) {
+    auto it = row_adapters_.find(id);
+    if (it == row_adapters_.end()) {
+        set_error("no per-row adapter is loaded under id " + std::to_string(id));
+        return -1;
+    }
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    row_adapters_.erase(it);
+    rebuild_lora_table();
+    return 0;
+}
+
+// Routes are the 1-based positions of the adapters in id order (reference
+// lora_router_install, retro_gen_core.cpp:2987-3006).
+void Engine::rebuild_lora_table() {
+    lora_routes_ = (int)row_adapters_.size();
+    if (lora_routes_ == 0) return;
+    std::vector<rk::LoraEntry> table((size_t)hp_.n_layer * kLoraTargets * (size_t)lora_routes_);
+    int route = 0;
+    for (const auto & kv : row_adapters_) {
+        const RowAdapterData & d = kv.second;
+        for (int l = 0; l < hp_.n_layer; ++l)
+            for (int tg = 0; tg < kLoraTargets; ++tg) {
+                rk::LoraEntry & e = table[((size_t)l * kLoraTargets + tg) * (size_t)lora_routes_ + (size_t)route];
+                const size_t at = (size_t)l * kLoraTargets + tg;
+                if (!d.a[at].ptr) continue;
+                e.A = d.a[at].as<float>();
+                e.B = d.b[at].as<float>();
+                e.rank = d.rank;
+                e.scale = (float)((double)d.scale * d.alpha / d.rank);
+            }
+        ++route;
+    }
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    lora_table_.alloc(table.size() * sizeof(rk::LoraEntry));
+    hip_check(hipMemcpy(lora_table_.ptr, table.data(), table.size() * sizeof(rk::LoraEntry), hipMemcpyHostToDevice), "hipMemcpy");
+    if (!lora_mid_.ptr) lora_mid_.alloc((size_t)cfg_.n_batch * rk::LORA_MAX_RANK * 4);
+}
+
+// What the stacks cost as the reference builds them: every adapter padded to
+// the widest rank, F32 (retro_gen_core.cpp:3008-3030).
+void Engine::adapter_rows_info(retro_adapter_rows_info * out) const {
+    *out = retro_adapter_rows_info{};
+    out->struct_size = sizeof(retro_adapter_rows_info);
+    uint32_t max_rank = 0;
+    for (const auto & kv : row_adapters_) max_rank = std::max<uint32_t>(max_rank, (uint32_t)kv.second.rank);
+    out->n_adapters = (uint32_t)row_adapters_.size();
+    out->max_rank = max_rank;
+    for (const auto & kv : row_adapters_) {
+        out->stacked_bytes += kv.second.elements * max_rank * 4;
+        out->unpadded_bytes += kv.second.elements * (uint64_t)kv.second.rank * 4;
     }
 }
 

@@ -104,6 +104,11 @@ public:
     int seq_pos(int32_t slot, int32_t * out_min, int32_t * out_max);
     int memory(retro_engine_memory_info * out);
     void request_free(int32_t request) { requests_.erase(request); }
+    // Per-row LoRA adapters (reference retro_engine.cpp:872-960): ids start at 1
+    // and are never reused; loading leaves the resident KV alone.
+    int adapter_load(const std::string & path, float scale, int32_t * out_id);
+    int adapter_unload(int32_t id);
+    void adapter_rows_info(retro_adapter_rows_info * out) const;
 
     const retro_engine_config & config() const { return cfg_; }
     const HParams & hparams() const { return hp_; }
@@ -150,7 +155,7 @@ private:
     void copy_page(int32_t src, int32_t dst);
     void set_page(int32_t slot, int idx, int32_t page);
     void clear_slot(Slot & s, int32_t slot);
-    void forward(int T, int n_out, int n_tiles, int n_items, bool one_token_rows);
+    void forward(int T, int n_out, int n_tiles, int n_items, bool one_token_rows, bool routed);
 
     retro_engine_config cfg_ {};
     HParams hp_;
@@ -210,6 +215,25 @@ private:
     size_t prof_begin(int cat);
     void prof_end(int cat, size_t token);
     void prof_resolve();
+
+    // per-row adapters: targets attn_q, attn_k, attn_v, attn_output of every layer
+    static constexpr int kLoraTargets = 4;
+    struct RowAdapterData {
+        float scale = 1.0f;
+        double alpha = 0.0;
+        int rank = 0;
+        uint64_t elements = 0;                     // sum over pairs of (n_in + n_out)
+        std::vector<DevBuf> a, b;                  // [layer * kLoraTargets + target], empty when the pair is absent
+    };
+    std::map<int32_t, RowAdapterData> row_adapters_;
+    int32_t next_adapter_id_ = 1;
+    DevBuf lora_table_;       // LoraEntry [layer][target][route - 1]
+    DevBuf lora_mid_;         // [n_batch][LORA_MAX_RANK] f32
+    int lora_routes_ = 0;
+    void rebuild_lora_table();
+    const rk::LoraEntry * lora_entries(int layer, int target) const {
+        return lora_table_.as<rk::LoraEntry>() + ((size_t)layer * kLoraTargets + target) * (size_t)lora_routes_;
+    }
 
     std::map<int32_t, RequestState> requests_;
     sampling::FullScratch scratch_;

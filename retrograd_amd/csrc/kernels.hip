@@ -602,6 +602,78 @@ void embed(hipStream_t s, const Weight & emb, const int32_t * tok, int T, float 
     check_launch("embed");
 }
 
+__global__ void k_decode_rows(int type, const uint8_t * __restrict__ raw, size_t rb, int K, float * __restrict__ out) {
+    const int r = blockIdx.y;
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= K) return;
+    out[(size_t)r * K + k] = decode_elem(type, raw + (size_t)r * rb, k);
+}
+
+void decode_rows(hipStream_t s, int type, const uint8_t * raw, int K, int n_rows, float * out) {
+    if (n_rows <= 0 || K <= 0) return;
+    hipLaunchKernelGGL(k_decode_rows, dim3((K + 255) / 256, n_rows), dim3(256), 0, s, type, raw, row_bytes(type, K), K, out);
+    check_launch("decode_rows");
+}
+
+// ---------------------------------------------------------------------------
+// per-row LoRA
+
+// mid[t][r] = sum_k A[r][k] * x[t][k]: one wave per (token, r), lanes own groups of eight k.
+__global__ __launch_bounds__(256) void k_lora_down(const LoraEntry * __restrict__ table, const RowDesc * __restrict__ rows,
+                                                   const int32_t * __restrict__ tok_row, Act x, float * __restrict__ mid) {
+    const int t = blockIdx.x;
+    const int route = rows[tok_row[t]].route;
+    if (route <= 0) return;
+    const LoraEntry e = table[route - 1];
+    const int r = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (!e.A || r >= e.rank) return;
+    const int lane = threadIdx.x & 63;
+    const float * a = e.A + (size_t)r * x.K;
+    float acc = 0.0f;
+    if (x.K % 8 == 0) {
+        for (int k = lane * 8; k < x.K; k += 512) {
+            const h8 hi = load_h8(x.x + act_at(t, k, 0, x.K)), lo = load_h8(x.x + act_at(t, k, 1, x.K));
+            const f4 a0 = *(const f4 *)(a + k), a1 = *(const f4 *)(a + k + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc = fmaf(a0[i], (float)hi[i] + (float)lo[i], acc);
+                acc = fmaf(a1[i], (float)hi[4 + i] + (float)lo[4 + i], acc);
+            }
+        }
+    } else {
+        for (int k = lane; k < x.K; k += 64)
+            acc = fmaf(a[k], __half2float(x.x[act_at(t, k, 0, x.K)]) + __half2float(x.x[act_at(t, k, 1, x.K)]), acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) mid[(size_t)t * LORA_MAX_RANK + r] = acc;
+}
+
+// y[t][col0 + n] += scale * sum_r B[n][r] * mid[t][r]
+__global__ __launch_bounds__(256) void k_lora_up(const LoraEntry * __restrict__ table, const RowDesc * __restrict__ rows,
+                                                 const int32_t * __restrict__ tok_row, const float * __restrict__ mid,
+                                                 int N, float * __restrict__ y, int ldy, int col0) {
+    const int t = blockIdx.x;
+    const int route = rows[tok_row[t]].route;
+    if (route <= 0) return;
+    const LoraEntry e = table[route - 1];
+    const int n = blockIdx.y * 256 + threadIdx.x;
+    if (!e.A || n >= N) return;
+    const float * b = e.B + (size_t)n * e.rank;
+    const float * m = mid + (size_t)t * LORA_MAX_RANK;
+    float acc = 0.0f;
+    for (int r = 0; r < e.rank; ++r) acc = fmaf(b[r], m[r], acc);
+    y[(size_t)t * ldy + col0 + n] += e.scale * acc;
+}
+
+void lora_apply(hipStream_t s, const LoraEntry * table, const RowDesc * rows, const int32_t * tok_row,
+                const Act & x, int T, int N, float * y, int ldy, int col0, float * mid) {
+    if (T <= 0 || N <= 0) return;
+    hipLaunchKernelGGL(k_lora_down, dim3(T, LORA_MAX_RANK / 4), dim3(256), 0, s, table, rows, tok_row, x, mid);
+    check_launch("lora_down");
+    hipLaunchKernelGGL(k_lora_up, dim3(T, (N + 255) / 256), dim3(256), 0, s, table, rows, tok_row, mid, N, y, ldy, col0);
+    check_launch("lora_up");
+}
+
 __global__ __launch_bounds__(256) void k_rmsnorm_act(float * x, const float * __restrict__ w,
                                                      int E, float eps, const int32_t * __restrict__ rows, Act out,
                                                      Slices add) {

@@ -98,6 +98,25 @@ Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float *
 void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
                     int mode, const float * bias);
 
+struct RowDesc;
+// Per-row LoRA. One loaded adapter's pair for one target matrix: A [rank][K] and
+// B [N][rank] as f32, scale = adapter scale * alpha / rank.
+struct LoraEntry {
+    const float * A = nullptr;
+    const float * B = nullptr;
+    int32_t rank = 0;
+    float scale = 0.0f;
+};
+constexpr int LORA_MAX_RANK = 64;
+// For every token whose row routes to an adapter (rows[tok_row[t]].route > 0,
+// entry table[route - 1], skipped when the entry has no pair for this target):
+//   y[t][col0 + n] += scale * sum_r B[n][r] * (sum_k A[r][k] * x[t][k]).
+// mid is scratch of T * LORA_MAX_RANK floats.
+void lora_apply(hipStream_t s, const LoraEntry * table, const RowDesc * rows, const int32_t * tok_row,
+                const Act & x, int T, int N, float * y, int ldy, int col0, float * mid);
+// out[r][k] = decode(raw row r)[k] as f32: any tensor to f32, row by row.
+void decode_rows(hipStream_t s, int type, const uint8_t * raw, int K, int n_rows, float * out);
+
 // x[t][:] = decode(raw row tok[t]) as f32.
 void embed(hipStream_t s, const Weight & emb, const int32_t * tok, int T, float * x);
 

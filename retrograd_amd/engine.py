@@ -608,6 +608,14 @@ class Engine:
         if s != 0:
             _raise(s)
 
+    def adapter_rows_info(self) -> "CAdapterRowsInfo":
+        """n_adapters, max_rank, stacked_bytes, unpadded_bytes (retrograd-engine AdapterRowsInfo)."""
+        info = CAdapterRowsInfo()
+        s = self._lib.retro_engine_adapter_rows_info(self._h, C.byref(info))
+        if s != 0:
+            _raise(s)
+        return info
+
     # -- state inspection (tests) --------------------------------------------------------
     def debug_logits(self) -> np.ndarray:
         rows = C.c_size_t()

@@ -1,0 +1,103 @@
+"""Per-row LoRA on the GPU against the CPU oracle: one step mixes rows decoded
+under different adapters and under the base model (reference
+crates/retrograd-ffi/runtime/src/retro_gen_core.cpp:2539-2564, tests/lora_rows.rs)."""
+import numpy as np
+import pytest
+
+import oracle
+from engine_helpers import assert_logits_close, greedy, logit_errors
+from retrograd_amd import engine as E
+from retrograd_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = synth.scaled(synth.QWEN25_7B_Q8, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
+                     n_ff=1024, n_vocab=1024, name="qwen2-lora")
+
+
+@pytest.fixture(scope="module")
+def files(tmp_path_factory):
+    d = tmp_path_factory.mktemp("lora")
+    model = d / "m.gguf"
+    synth.write_model(model, SHAPE, seed=77, device="cpu", std=0.05)
+    a1, a2 = d / "a1.gguf", d / "a2.gguf"
+    synth.write_lora_adapter(a1, SHAPE, rank=16, alpha=32.0, seed=1, std_a=0.1, std_b=0.1)
+    synth.write_lora_adapter(a2, SHAPE, rank=8, alpha=8.0, seed=2, std_a=0.1, std_b=0.1,
+                             targets=("attn_q", "attn_output"))
+    ffn = d / "ffn.gguf"
+    synth.write_lora_adapter(ffn, SHAPE, rank=4, alpha=4.0, seed=3, targets=("attn_q", "ffn_down"))
+    return model, a1, a2, ffn
+
+
+def test_rows_under_different_adapters_match_the_oracle(files):
+    model, a1, a2, _ = files
+    print("per-row LoRA: %s, ranks 16 and 8" % SHAPE.name, flush=True)
+    eng = E.Engine(model, E.EngineConfig(n_ctx=1024, n_seq_max=4, n_batch=128, n_ubatch=128))
+    m = oracle.Model(model)
+    ctx = oracle.Context(m, 4)
+    ids = [eng.adapter_load(a1, 1.0), eng.adapter_load(a2, 0.5)]
+    oids = [m.load_adapter(a1, 1.0), m.load_adapter(a2, 0.5)]
+    assert ids == oids == [1, 2]
+
+    rng = np.random.default_rng(3)
+    lens = [21, 9, 40, 13]
+    prompts = [rng.integers(0, m.n_vocab, n) for n in lens]
+    route = [ids[0], E.RETRO_STEP_ADAPTER_BASE, ids[1], 0]          # adapter 1, base, adapter 2, context (= base here)
+    out = E.StepOutput()
+    rows = [E.StepRow(i, i, prompts[i], 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(route[i])) for i in range(4)]
+    eng.step(rows, out)
+    got = eng.debug_logits()
+    want = ctx.step_rows([(i, 0, prompts[i], True) for i in range(4)], adapters=[route[0], -1, route[2], -1])
+    assert_logits_close(got, want)
+    # the adapters do something: the same rows under the base model differ visibly
+    base = oracle.Context(m, 4).step_rows([(i, 0, prompts[i], True) for i in range(4)])
+    assert np.abs(want[0] - base[0]).max() > 5e-2 and np.abs(want[2] - base[2]).max() > 1e-2
+    assert np.array_equal(want[1], base[1])
+
+    pos = list(lens)
+    for _ in range(3):       # decode steps (sliced matmuls at T = 4), teacher-forced with the oracle's tokens
+        feed = [int(want[i].argmax()) for i in range(4)]
+        rows = [E.StepRow(i, i, [feed[i]], pos[i], sample=True, sampling=greedy(), adapter=E.RowAdapter(route[i]))
+                for i in range(4)]
+        eng.step(rows, out)
+        got = eng.debug_logits()
+        want = ctx.step_rows([(i, pos[i], [feed[i]], True) for i in range(4)], adapters=[route[0], -1, route[2], -1])
+        assert_logits_close(got, want)
+        pos = [p + 1 for p in pos]
+
+    info = eng.adapter_rows_info()
+    E_, QD, KD = SHAPE.n_embd, SHAPE.n_head * SHAPE.head_dim, SHAPE.n_head_kv * SHAPE.head_dim
+    el1 = SHAPE.n_layer * ((E_ + QD) + 2 * (E_ + KD) + (QD + E_))
+    el2 = SHAPE.n_layer * ((E_ + QD) + (QD + E_))
+    assert (info.n_adapters, info.max_rank) == (2, 16)
+    assert info.stacked_bytes == (el1 + el2) * 16 * 4
+    assert info.unpadded_bytes == el1 * 16 * 4 + el2 * 8 * 4
+    eng.close()
+
+
+def test_adapter_errors_and_unload(files):
+    model, a1, a2, ffn = files
+    print("per-row LoRA: argument errors", flush=True)
+    eng = E.Engine(model, E.EngineConfig(n_ctx=512, n_seq_max=2, n_batch=64, n_ubatch=64))
+    out = E.StepOutput()
+    toks = [1, 2, 3]
+    with pytest.raises(E.InvalidArgument, match="is not a loaded per-row adapter"):
+        eng.step([E.StepRow(0, 0, toks, 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(1))], out)
+    with pytest.raises(E.RuntimeFailure, match="only attn_q, attn_k, attn_v and attn_output"):
+        eng.adapter_load(ffn)
+    with pytest.raises(E.RuntimeFailure, match="failed to load LoRA adapter"):
+        eng.adapter_load(model)
+    aid = eng.adapter_load(a1)
+    assert aid == 1, "a refused load does not consume an id"
+    with pytest.raises(E.InvalidArgument, match="select different adapters"):
+        eng.step([E.StepRow(0, 0, toks, 0, adapter=E.RowAdapter(aid)),
+                  E.StepRow(1, 0, [4], 3, sample=True, sampling=greedy())], out)
+    eng.step([E.StepRow(0, 0, toks, 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(aid))], out)
+    eng.adapter_unload(aid)
+    with pytest.raises(E.RuntimeFailure, match="no per-row adapter is loaded under id 1"):
+        eng.adapter_unload(aid)
+    with pytest.raises(E.InvalidArgument, match="is not a loaded per-row adapter"):
+        eng.step([E.StepRow(0, 1, toks, 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(aid))], out)
+    assert eng.adapter_load(a2) == 2, "ids are never reused"
+    assert eng.adapter_rows_info().n_adapters == 1
+    eng.close()

@@ -145,6 +145,25 @@ void Engine::upload_weight(const TensorInfo & t, int64_t K, int64_t N, const uin
     }
 }
 
+// An expert tensor [K][N][n_expert]: n_expert * N rows of K, tiled per expert.
+void Engine::upload_experts(const TensorInfo & t, int64_t K, int64_t N, DevWeight & out) {
+    const int64_t rows = N * hp_.n_expert;
+    if (!rk::moe_can_pack(t.type, K, N)) throw std::runtime_error("expert tensor " + t.name + " must be MXFP4 or Q8_0 with widths that are multiples of 256 and 16");
+    if (rk::row_bytes(t.type, K) * (size_t)rows != t.nbytes) throw std::runtime_error("tensor " + t.name + " has an unexpected size");
+    out.w.type = t.type;
+    out.w.K = (int)K;
+    out.w.N = (int)N;              // rows per expert
+    out.w.bytes = t.nbytes;
+    DevBuf raw;
+    raw.alloc(t.nbytes);
+    hip_check(hipMemcpy(raw.ptr, t.data, t.nbytes, hipMemcpyHostToDevice), "hipMemcpy");
+    out.buf.alloc(t.nbytes);
+    rk::moe_repack(stream_, t.type, raw.as<uint8_t>(), out.buf.as<uint8_t>(), (int)K, rows);
+    hip_check(hipStreamSynchronize(stream_), "repack");
+    out.w.packed = out.buf.as<uint8_t>();
+    out.w.raw = nullptr;
+}
+
 // Row-wise concatenation of matrices that share K and storage type: one matmul
 // instead of several. Falls back to separate matrices when they differ.
 void Engine::upload_fused(const std::vector<const TensorInfo *> & parts, std::vector<DevWeight> & out) {
@@ -173,7 +192,7 @@ void Engine::load_model(const std::string & path) {
     HParams & h = hp_;
     h.arch = g.get_string("general.architecture");
     if (h.arch == "llama") h.rope_neox = false;
-    else if (h.arch == "qwen2" || h.arch == "qwen3") h.rope_neox = true;
+    else if (h.arch == "qwen2" || h.arch == "qwen3" || h.arch == "qwen3moe") h.rope_neox = true;
     else throw std::runtime_error("unsupported model architecture: " + h.arch);
     const std::string a = h.arch + ".";
     h.n_layer = (int)g.need_int(a + "block_count");
@@ -186,7 +205,10 @@ void Engine::load_model(const std::string & path) {
     h.rope_base = g.get_float(a + "rope.freq_base", 10000.0);
     h.rope_dim = (int)g.get_int(a + "rope.dimension_count", h.head_dim);
     h.n_expert = (int)g.get_int(a + "expert_count", 0);
-    if (h.n_expert > 0) throw std::runtime_error("mixture-of-experts models are not supported yet");
+    h.n_expert_used = (int)g.get_int(a + "expert_used_count", 0);
+    h.n_ff_exp = (int)g.get_int(a + "expert_feed_forward_length", h.n_ff);
+    if (h.n_expert > 0 && (h.n_expert > 256 || h.n_expert_used < 1 || h.n_expert_used > 16 || h.n_expert_used > h.n_expert))
+        throw std::runtime_error("unsupported expert configuration (at most 256 experts, 1 to 16 used per token)");
     if (h.head_dim != 32 && h.head_dim != 64 && h.head_dim != 128) throw std::runtime_error("head_dim must be 32, 64 or 128");
     if (h.rope_dim > h.head_dim || h.rope_dim % 2 != 0) throw std::runtime_error("unsupported rotary width");
 
@@ -229,6 +251,22 @@ void Engine::load_model(const std::string & path) {
         }
         const TensorInfo & wo = g.require(b + "attn_output.weight");
         upload_weight(wo, QD, E, wo.data, wo.nbytes, false, L.wo);
+        if (h.n_expert > 0) {
+            const int F = h.n_ff_exp;
+            const TensorInfo & wr = g.require(b + "ffn_gate_inp.weight");
+            if (wr.type != rk::WT_F32 || wr.ne[0] != E || wr.ne[1] != h.n_expert) throw std::runtime_error("the router of layer " + std::to_string(l) + " must be F32 [n_embd][n_expert]");
+            upload_weight(wr, E, h.n_expert, wr.data, wr.nbytes, true, L.router);
+            const TensorInfo & eg = g.require(b + "ffn_gate_exps.weight");
+            const TensorInfo & eu = g.require(b + "ffn_up_exps.weight");
+            const TensorInfo & ed = g.require(b + "ffn_down_exps.weight");
+            for (const TensorInfo * t : {&eg, &eu})
+                if (t->ne[0] != E || t->ne[1] != F || t->ne[2] != h.n_expert) throw std::runtime_error("expert weights of layer " + std::to_string(l) + " have unexpected shapes");
+            if (ed.ne[0] != F || ed.ne[1] != E || ed.ne[2] != h.n_expert) throw std::runtime_error("expert weights of layer " + std::to_string(l) + " have unexpected shapes");
+            upload_experts(eg, E, F, L.gate_exps);
+            upload_experts(eu, E, F, L.up_exps);
+            upload_experts(ed, F, E, L.down_exps);
+            continue;
+        }
         const TensorInfo & wg = g.require(b + "ffn_gate.weight");
         const TensorInfo & wu = g.require(b + "ffn_up.weight");
         const TensorInfo & wd = g.require(b + "ffn_down.weight");
@@ -284,7 +322,21 @@ void Engine::build_buffers() {
 
     x_.alloc((size_t)B * E * 4);
     qkv_.alloc((size_t)B * (QD + 2 * KD) * 4);
-    gu_.alloc((size_t)B * 2 * F * 4);
+    gu_.alloc((size_t)B * 2 * std::max(F, 1) * 4);
+    if (hp_.n_expert > 0) {
+        const int NE = hp_.n_expert, KU = hp_.n_expert_used, FE = hp_.n_ff_exp;
+        const size_t slots = rk::moe_slots(B, KU, NE);
+        moe_logits_.alloc((size_t)B * NE * 4);
+        moe_sel_.alloc((size_t)B * KU * 4);
+        moe_wgt_.alloc((size_t)B * KU * 4);
+        moe_n_.alloc((size_t)NE * 4);
+        moe_off_.alloc((size_t)(NE + 1) * 4);
+        moe_tok_.alloc(slots * 4);
+        moe_q_.alloc((size_t)B * KU * 4);
+        moe_h_.alloc(rk::act_halves((int)slots, FE) * 2);
+        hip_check(hipMemsetAsync(moe_h_.ptr, 0, moe_h_.bytes, stream_), "hipMemsetAsync");
+        moe_out_.alloc(slots * (size_t)E * 4);
+    }
     q_half_.alloc((size_t)B * QD * 2);
     // operand-order activations; the sums keep zero padding lanes, so they are cleared once
     auto act = [&](DevBuf & x, DevBuf & sums, int K) {
@@ -1126,6 +1178,18 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         pt_ = prof_begin(PC_NORM);
         rk::rmsnorm_act(stream_, x, L.ffn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending);
         prof_end(PC_NORM, pt_);
+        if (h.n_expert > 0) {
+            pt_ = prof_begin(PC_GATEUP);
+            rk::MoeLayer ml{L.router.w, L.gate_exps.w, L.up_exps.w, L.down_exps.w};
+            rk::MoeShape ms{E, h.n_ff_exp, h.n_expert, h.n_expert_used};
+            rk::MoeBuffers mb{moe_logits_.as<float>(), moe_sel_.as<int32_t>(), moe_wgt_.as<float>(), moe_n_.as<int32_t>(),
+                              moe_off_.as<int32_t>(), moe_tok_.as<int32_t>(), moe_q_.as<int32_t>(),
+                              rk::Act{moe_h_.as<__half>(), nullptr, h.n_ff_exp}, moe_out_.as<float>()};
+            rk::moe_ffn(stream_, ml, ms, act_e, T, x, mb);
+            pending = rk::Slices();
+            prof_end(PC_GATEUP, pt_);
+            continue;
+        }
         pt_ = prof_begin(PC_GATEUP);
         {
             int col = 0;

@@ -68,6 +68,8 @@ struct LayerWeights {
     DevWeight wo;
     std::vector<DevWeight> gate_up; // one fused matrix, or gate, up separately
     DevWeight down;
+    // mixture-of-experts layers: F32 router [n_expert][E] and the three expert tensors, tiled per expert
+    DevWeight router, gate_exps, up_exps, down_exps;
 };
 
 struct Slot {
@@ -148,6 +150,7 @@ private:
                        bool keep_raw, DevWeight & out);
     void upload_fused(const std::vector<const TensorInfo *> & parts, std::vector<DevWeight> & out);
     void upload_f32(const TensorInfo * t, DevBuf & out, size_t expect);
+    void upload_experts(const TensorInfo & t, int64_t K, int64_t N, DevWeight & out);
     void build_buffers();
 
     int32_t alloc_page();
@@ -201,6 +204,8 @@ private:
     DevBuf act_o_x_, act_o_sums_;       // output rows, n_embd wide
     DevBuf q_half_lo_;
     DevBuf mm_ws_;            // matmul workspace: split-K partials, counters
+    // mixture-of-experts scratch (allocated for MoE models only)
+    DevBuf moe_logits_, moe_sel_, moe_wgt_, moe_n_, moe_off_, moe_tok_, moe_q_, moe_h_, moe_out_;
     HostPinned h_sample_, h_logits_;
     int last_n_out_ = 0;
 

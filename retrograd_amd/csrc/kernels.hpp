@@ -117,6 +117,27 @@ void lora_apply(hipStream_t s, const LoraEntry * table, const RowDesc * rows, co
 // out[r][k] = decode(raw row r)[k] as f32: any tensor to f32, row by row.
 void decode_rows(hipStream_t s, int type, const uint8_t * raw, int K, int n_rows, float * out);
 
+// Mixture-of-experts feed-forward (qwen3moe). Expert tensors are tiled by
+// moe_repack as one matrix of n_expert * N rows; router is raw F32 [n_expert][E].
+bool moe_can_pack(int type, int64_t K, int64_t N);
+void moe_repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int K, int64_t n_rows);
+struct MoeLayer { Weight router, gate, up, down; };
+struct MoeShape { int E, F, n_expert, k_used; };
+struct MoeBuffers {            // device scratch of one step, sized with moe_slots(n_batch, ...)
+    float * logits;            // [T][n_expert]
+    int32_t * sel;             // [T][k_used] chosen experts, by descending probability
+    float * wgt;               // [T][k_used] renormalised weights
+    int32_t * expert_n;        // [n_expert]
+    int32_t * off_pad;         // [n_expert + 1]
+    int32_t * tok_of_q;        // [slots]
+    int32_t * q_of_pair;       // [T * k_used]
+    Act h;                     // [slots] x F
+    float * out_pair;          // [slots][E]
+};
+size_t moe_slots(int n_tokens, int k_used, int n_expert);
+// x[t] += sum over the token's k_used experts of w * down_e(silu(gate_e xn) * (up_e xn))
+void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act & xn, int T, float * x, const MoeBuffers & b);
+
 // x[t][:] = decode(raw row tok[t]) as f32.
 void embed(hipStream_t s, const Weight & emb, const int32_t * tok, int T, float * x);
 

@@ -1,0 +1,410 @@
+// Mixture-of-experts feed-forward (qwen3moe): softmax router, top-k experts with
+// renormalised weights, SwiGLU experts with MXFP4 or Q8_0 weights.
+//
+// The expert weights dominate the bytes of a step (all experts are touched once
+// a batch has a few dozen tokens), so the work is organised by expert: the
+// (token, choice) pairs of a step are grouped by expert, every expert's range
+// padded to whole 16-token MFMA tiles, and one wave owns one 16-row weight tile
+// of one expert and streams it exactly once per 32 tokens of that expert:
+//
+//   k_moe_route     per token: top-k of the router logits, weights in double
+//   k_moe_group     stable counting sort of the pairs by expert (one workgroup)
+//   k_moe_gate_up   h[q][f] = silu(gate_e x) * (up_e x)       q = slot of a pair
+//   k_moe_down      out[q][:] = down_e h[q]
+//   k_moe_combine   x[t] += sum_j w[t][j] * out[q(t, j)]       in choice order
+//
+// Expert tensors [K][N][n_expert] are tiled as one matrix of n_expert * N rows.
+// MXFP4 tile (16 rows x 256 columns, 2176 B = the GGUF byte count): 16 x 8 E8M0
+// scale bytes, then two 1 KiB loads; lane (r = l % 16, g = l / 16) of load h
+// holds one dword per k-step 4h + j: byte b of it carries element 8g + b in its
+// low nibble and element 8g + 4 + b in its high nibble. The doubled E2M1
+// magnitudes 0 1 2 3 4 6 8 12 are f16 numbers whose low byte is zero, so two
+// byte permutes through an 8-byte table decode four weights at a time, exactly.
+#include "dev_common.hpp"
+
+namespace rk {
+
+bool moe_can_pack(int type, int64_t K, int64_t N) {
+    return (type == WT_MXFP4 || type == WT_Q8_0) && K % 256 == 0 && N % 16 == 0 && K > 0 && N > 0;
+}
+
+__global__ void k_repack_mxfp4(const uint8_t * __restrict__ raw, uint8_t * __restrict__ dst, int nsb, size_t n_tiles) {
+    // one thread per output dword: 544 per (tile, super-block): 32 header + 512 payload
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = n_tiles * (size_t)nsb * 544;
+    if (gid >= total) return;
+    const int w = (int)(gid % 544);
+    const size_t ts = gid / 544;
+    const int sb = (int)(ts % nsb);
+    const size_t rt = ts / nsb;
+    const size_t row_bytes = (size_t)nsb * 8 * 17;
+    uint32_t out = 0;
+    if (w < 32) {                       // row r, scales of blocks 4*half .. +3
+        const int r = w >> 1, half = w & 1;
+        const uint8_t * row = raw + (rt * 16 + r) * row_bytes + (size_t)sb * 8 * 17;
+        for (int i = 0; i < 4; ++i) out |= (uint32_t)row[(size_t)(4 * half + i) * 17] << (8 * i);
+    } else {
+        const int v = w - 32;
+        const int h = v >> 8, lane = (v >> 2) & 63, j = v & 3;
+        const int r = lane & 15, g = lane >> 4;
+        const uint8_t * blk = raw + (rt * 16 + r) * row_bytes + (size_t)(sb * 8 + 4 * h + j) * 17;
+        auto elem = [&](int e) -> uint32_t {
+            const uint8_t byte = blk[1 + (e & 15)];
+            return e < 16 ? (byte & 0x0f) : (byte >> 4);
+        };
+        for (int b = 0; b < 4; ++b) out |= (elem(8 * g + b) | (elem(8 * g + 4 + b) << 4)) << (8 * b);
+    }
+    *(uint32_t *)(dst + ts * 2176 + (size_t)w * 4) = out;
+}
+
+void moe_repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int K, int64_t n_rows) {
+    if (!moe_can_pack(type, K, n_rows)) throw std::runtime_error("moe_repack: shape or type has no tile layout");
+    if (type == WT_Q8_0) {
+        // the dense Q8_0 tile layout, in slabs the dense repack's 32-bit sizes can hold
+        const int64_t slab = 1 << 20;
+        for (int64_t r0 = 0; r0 < n_rows; r0 += slab) {
+            const int64_t n = std::min(slab, n_rows - r0);
+            const size_t off = (size_t)r0 * row_bytes(type, K);
+            repack(s, type, raw + off, packed + off, K, (int)n);
+        }
+        return;
+    }
+    const int nsb = K / 256;
+    const size_t n_tiles = (size_t)n_rows / 16;
+    const size_t total = n_tiles * (size_t)nsb * 544;
+    hipLaunchKernelGGL(k_repack_mxfp4, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, raw, packed, nsb, n_tiles);
+    check_launch("moe_repack");
+}
+
+namespace {
+
+template <int TYPE> struct Tile;
+
+template <> struct Tile<WT_MXFP4> {
+    static constexpr int BYTES = 2176;
+    uint2 hdr;
+    u4 q0, q1;
+    __device__ __forceinline__ void load(const uint8_t * tile, int lane) {
+        hdr = *(const uint2 *)(tile + (lane & 15) * 8);
+        q0 = *(const u4 *)(tile + 128 + lane * 16);
+        q1 = *(const u4 *)(tile + 128 + 1024 + lane * 16);
+    }
+    // half of 2^(x - 127): the E8M0 scale of doubled magnitudes
+    __device__ __forceinline__ float scale(int s) const {
+        const uint32_t x = ((s < 4 ? hdr.x : hdr.y) >> (8 * (s & 3))) & 0xff;
+        const uint32_t bits = x == 0 ? 0x00200000u : (x == 1 ? 0x00400000u : (x - 1) << 23);
+        return __uint_as_float(bits);
+    }
+    __device__ __forceinline__ h8 frag(int s) const {
+        const uint32_t w = s < 4 ? q0[s & 3] : q1[s & 3];
+        // high bytes of the f16 numbers 0 1 2 3 | 4 6 8 12, chosen by the 3-bit magnitude; bit 3 is the sign
+        const uint32_t lo = __builtin_amdgcn_perm(0x4A484644u, 0x42403C00u, w & 0x07070707u) | ((w & 0x08080808u) << 4);
+        const uint32_t hi = __builtin_amdgcn_perm(0x4A484644u, 0x42403C00u, (w >> 4) & 0x07070707u) | (w & 0x80808080u);
+        const h2 p0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0u, lo, 0x010C000Cu));
+        const h2 p1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0u, lo, 0x030C020Cu));
+        const h2 p2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0u, hi, 0x010C000Cu));
+        const h2 p3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0u, hi, 0x030C020Cu));
+        return (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+    }
+};
+
+template <> struct Tile<WT_Q8_0> {
+    static constexpr int BYTES = 4352;
+    u4 hdr;
+    u4 q[4];
+    __device__ __forceinline__ void load(const uint8_t * tile, int lane) {
+        hdr = *(const u4 *)(tile + (lane & 15) * 16);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) q[j] = *(const u4 *)(tile + 256 + j * 1024 + lane * 16);
+    }
+    __device__ __forceinline__ float scale(int s) const {
+        const uint32_t sw = hdr[s >> 1];
+        return h2f((uint16_t)((s & 1) ? (sw >> 16) : (sw & 0xffff)));
+    }
+    __device__ __forceinline__ h8 frag(int s) const {
+        const u4 d4 = q[s >> 1];
+        const int half = s & 1;
+        const uint32_t w0 = d4[2 * half] ^ 0x80808080u, w1 = d4[2 * half + 1] ^ 0x80808080u;
+        const h2 bias = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
+        const h2 a0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u)) + bias;
+        const h2 a1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u)) + bias;
+        const h2 a2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u)) + bias;
+        const h2 a3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)) + bias;
+        return (h8){a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+    }
+};
+
+__device__ __forceinline__ f4 mfma2(const h8 & a_hi, const h8 & a_lo, const h8 & b) {
+    f4 p = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_hi, b, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a_lo, b, p, 0, 0, 0);
+}
+
+}  // namespace
+
+struct MoeArgs {
+    const uint8_t * w0;        // gate (gate_up) or down
+    const uint8_t * w1;        // up
+    Act x;                     // gate_up: the normalised activations by token; down: h by pair slot
+    Act h;                     // gate_up output
+    float * out_pair;          // down output [slot][E]
+    const int32_t * expert_n;  // pairs per expert
+    const int32_t * off_pad;   // first slot of each expert (multiples of 16)
+    const int32_t * tok_of_q;  // token of a slot, -1 for padding
+    int n_expert, K, N;        // N output features per expert, K inputs
+};
+
+// One wave per (expert, 16 output features): gate and up tiles together, SwiGLU in the epilogue.
+template <int TYPE>
+__global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int n_tiles = a.N / 16;
+    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int e = item / n_tiles, ft = item % n_tiles;
+    if (e >= a.n_expert) return;
+    const int n_e = a.expert_n[e];
+    if (n_e == 0) return;
+    const int qb = a.off_pad[e];
+    const int nsb = a.K >> 8;
+    const size_t tile0 = ((size_t)e * n_tiles + ft) * nsb * Tile<TYPE>::BYTES;
+    for (int t0 = 0; t0 < n_e; t0 += 32) {
+        int tok[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int at = t0 + t * 16 + r16;
+            const int tk = at < n_e ? a.tok_of_q[qb + at] : -1;
+            tok[t] = tk < 0 ? 0 : tk;          // padding rows read token 0 and are never stored
+        }
+        f4 ag[2], au[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) { ag[t] = (f4){0.f, 0.f, 0.f, 0.f}; au[t] = (f4){0.f, 0.f, 0.f, 0.f}; }
+        for (int sb = 0; sb < nsb; ++sb) {
+            Tile<TYPE> tg, tu;
+            tg.load(a.w0 + tile0 + (size_t)sb * Tile<TYPE>::BYTES, lane);
+            tu.load(a.w1 + tile0 + (size_t)sb * Tile<TYPE>::BYTES, lane);
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const h8 bg = tg.frag(s), bu = tu.frag(s);
+                const float dg = tg.scale(s), du = tu.scale(s);
+                const int k = sb * 256 + s * 32 + 8 * g;
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const h8 hi = load_h8(a.x.x + act_at(tok[t], k, 0, a.K)), lo = load_h8(a.x.x + act_at(tok[t], k, 1, a.K));
+                    const f4 pg = mfma2(hi, lo, bg), pu = mfma2(hi, lo, bu);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        ag[t][i] = fmaf(dg, pg[i], ag[t][i]);
+                        au[t][i] = fmaf(du, pu[i], au[t][i]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int at = t0 + t * 16 + 4 * g + i;
+                if (at >= n_e) continue;
+                const float gv = ag[t][i];
+                const float v = fminf(fmaxf((gv / (1.0f + __expf(-gv))) * au[t][i], -65504.0f), 65504.0f);
+                const __half hh = __float2half_rn(v);
+                const int f = ft * 16 + r16;
+                a.h.x[act_at(qb + at, f, 0, a.N)] = hh;
+                a.h.x[act_at(qb + at, f, 1, a.N)] = __float2half_rn(v - __half2float(hh));
+            }
+    }
+}
+
+// One wave per (expert, 16 output features of the model width).
+template <int TYPE>
+__global__ __launch_bounds__(256) void k_moe_down(MoeArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int r16 = lane & 15, g = lane >> 4;
+    const int n_tiles = a.N / 16;
+    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int e = item / n_tiles, et = item % n_tiles;
+    if (e >= a.n_expert) return;
+    const int n_e = a.expert_n[e];
+    if (n_e == 0) return;
+    const int qb = a.off_pad[e];
+    const int nsb = a.K >> 8;
+    const size_t tile0 = ((size_t)e * n_tiles + et) * nsb * Tile<TYPE>::BYTES;
+    for (int t0 = 0; t0 < n_e; t0 += 32) {
+        // the second tile of the last pass may lie past the expert's padded range: read the first tile again
+        const int q0 = qb + t0 + r16;
+        const int q1 = t0 + 16 < n_e ? q0 + 16 : q0;
+        f4 acc[2] = {(f4){0.f, 0.f, 0.f, 0.f}, (f4){0.f, 0.f, 0.f, 0.f}};
+        for (int sb = 0; sb < nsb; ++sb) {
+            Tile<TYPE> tw;
+            tw.load(a.w0 + tile0 + (size_t)sb * Tile<TYPE>::BYTES, lane);
+#pragma unroll
+            for (int s = 0; s < 8; ++s) {
+                const h8 b = tw.frag(s);
+                const float d = tw.scale(s);
+                const int k = sb * 256 + s * 32 + 8 * g;
+                const f4 p0 = mfma2(load_h8(a.x.x + act_at(q0, k, 0, a.K)), load_h8(a.x.x + act_at(q0, k, 1, a.K)), b);
+                const f4 p1 = mfma2(load_h8(a.x.x + act_at(q1, k, 0, a.K)), load_h8(a.x.x + act_at(q1, k, 1, a.K)), b);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[0][i] = fmaf(d, p0[i], acc[0][i]);
+                    acc[1][i] = fmaf(d, p1[i], acc[1][i]);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int at = t0 + t * 16 + 4 * g + i;
+                if (at < n_e) a.out_pair[(size_t)(qb + at) * a.N + et * 16 + r16] = acc[t][i];
+            }
+    }
+}
+
+// Per token: the top-k experts by router logit (ties to the lower index - the
+// order of the softmax probabilities) and their weights renormalised over the
+// selection, exp and the sums in double.
+__global__ __launch_bounds__(64) void k_moe_route(const float * __restrict__ logits, int n_expert, int k_used,
+                                                  int32_t * __restrict__ sel, float * __restrict__ wgt) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    float v[4];
+    bool taken[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = lane + 64 * i;
+        v[i] = e < n_expert ? logits[(size_t)t * n_expert + e] : -INFINITY;
+        taken[i] = e >= n_expert;
+    }
+    float top_v[16];
+    float mx = -INFINITY;
+    for (int j = 0; j < k_used; ++j) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (!taken[i] && (bi == 0x7fffffff || v[i] > bv)) { bv = v[i]; bi = lane + 64 * i; }
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64);
+            const int oi = __shfl_xor(bi, o, 64);
+            if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (bi == lane + 64 * i) taken[i] = true;
+        if (j == 0) mx = bv;
+        top_v[j] = bv;
+        if (lane == 0) sel[(size_t)t * k_used + j] = bi;
+    }
+    if (lane == 0) {
+        double p[16], sum = 0.0;
+        for (int j = 0; j < k_used; ++j) { p[j] = exp((double)top_v[j] - (double)mx); sum += p[j]; }
+        for (int j = 0; j < k_used; ++j) wgt[(size_t)t * k_used + j] = (float)(p[j] / sum);
+    }
+}
+
+// Stable counting sort of the pairs by expert, every expert's range padded to a
+// multiple of 16 slots. One workgroup of 1024 threads.
+__global__ __launch_bounds__(1024) void k_moe_group(const int32_t * __restrict__ sel, int n_pairs, int n_expert, int k_used,
+                                                    int32_t * __restrict__ expert_n, int32_t * __restrict__ off_pad,
+                                                    int32_t * __restrict__ tok_of_q, int32_t * __restrict__ q_of_pair) {
+    __shared__ int cnt[256];
+    __shared__ int base[256];
+    __shared__ int wcnt[16][256];
+    __shared__ int total_pad;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid < 256) cnt[tid] = 0;
+    for (int i = tid; i < 16 * 256; i += 1024) (&wcnt[0][0])[i] = 0;
+    __syncthreads();
+    for (int p = tid; p < n_pairs; p += 1024) atomicAdd(&cnt[sel[p]], 1);
+    __syncthreads();
+    if (tid == 0) {
+        int at = 0;
+        for (int e = 0; e < n_expert; ++e) {
+            off_pad[e] = at;
+            base[e] = at;
+            expert_n[e] = cnt[e];
+            at += (cnt[e] + 15) & ~15;
+        }
+        off_pad[n_expert] = at;
+        total_pad = at;
+    }
+    __syncthreads();
+    for (int q = tid; q < total_pad; q += 1024) tok_of_q[q] = -1;
+    __syncthreads();
+    for (int c0 = 0; c0 < n_pairs; c0 += 1024) {
+        const int p = c0 + tid;
+        const int e = p < n_pairs ? sel[p] : -1;
+        int rank = 0;
+        for (int i = 0; i < 64; ++i) {
+            const int other = __shfl(e, i, 64);
+            if (other == e && i < lane) ++rank;
+        }
+        if (e >= 0) atomicMax(&wcnt[wave][e], rank + 1);
+        __syncthreads();
+        if (e >= 0) {
+            int pos = base[e] + rank;
+            for (int w = 0; w < wave; ++w) pos += wcnt[w][e];
+            q_of_pair[p] = pos;
+            tok_of_q[pos] = p / k_used;
+        }
+        __syncthreads();
+        if (tid < n_expert) {
+            int add = 0;
+            for (int w = 0; w < 16; ++w) { add += wcnt[w][tid]; wcnt[w][tid] = 0; }
+            base[tid] += add;
+        }
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(256) void k_moe_combine(const float * __restrict__ out_pair, const int32_t * __restrict__ q_of_pair,
+                                                     const float * __restrict__ wgt, int k_used, int E, float * __restrict__ x) {
+    const int t = blockIdx.x;
+    const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
+    if (c >= E) return;
+    f4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < k_used; ++j) {
+        const float w = wgt[(size_t)t * k_used + j];
+        const f4 v = *(const f4 *)(out_pair + (size_t)q_of_pair[(size_t)t * k_used + j] * E + c);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = fmaf(w, v[i], acc[i]);
+    }
+    f4 * dst = (f4 *)(x + (size_t)t * E + c);
+    *dst += acc;
+}
+
+size_t moe_slots(int n_tokens, int k_used, int n_expert) {
+    return ((size_t)n_tokens * k_used + (size_t)16 * n_expert + 63) / 64 * 64;
+}
+
+void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act & xn, int T, float * x, const MoeBuffers & b) {
+    if (T <= 0) return;
+    if (sh.n_expert > 256 || sh.k_used > 16 || sh.k_used > sh.n_expert) throw std::runtime_error("moe: unsupported expert count");
+    if (sh.E % 256 != 0 || sh.F % 256 != 0) throw std::runtime_error("moe: widths must be multiples of 256");
+    if (L.gate.type != L.up.type || (L.gate.type != WT_MXFP4 && L.gate.type != WT_Q8_0) ||
+        (L.down.type != WT_MXFP4 && L.down.type != WT_Q8_0))
+        throw std::runtime_error("moe: expert weights must be MXFP4 or Q8_0");
+    matmul_generic(s, L.router, xn, T, b.logits, sh.n_expert, 0, MM_STORE, nullptr);
+    hipLaunchKernelGGL(k_moe_route, dim3(T), dim3(64), 0, s, b.logits, sh.n_expert, sh.k_used, b.sel, b.wgt);
+    check_launch("moe_route");
+    hipLaunchKernelGGL(k_moe_group, dim3(1), dim3(1024), 0, s, b.sel, T * sh.k_used, sh.n_expert, sh.k_used, b.expert_n,
+                       b.off_pad, b.tok_of_q, b.q_of_pair);
+    check_launch("moe_group");
+    MoeArgs a {};
+    a.expert_n = b.expert_n; a.off_pad = b.off_pad; a.tok_of_q = b.tok_of_q; a.n_expert = sh.n_expert;
+    a.w0 = L.gate.packed; a.w1 = L.up.packed; a.x = xn; a.h = b.h; a.K = sh.E; a.N = sh.F;
+    const unsigned gu_blocks = (unsigned)(((size_t)sh.n_expert * (sh.F / 16) + 3) / 4);
+    if (L.gate.type == WT_MXFP4) hipLaunchKernelGGL(k_moe_gate_up<WT_MXFP4>, dim3(gu_blocks), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(k_moe_gate_up<WT_Q8_0>, dim3(gu_blocks), dim3(256), 0, s, a);
+    check_launch("moe_gate_up");
+    a.w0 = L.down.packed; a.w1 = nullptr; a.x = b.h; a.out_pair = b.out_pair; a.K = sh.F; a.N = sh.E;
+    const unsigned d_blocks = (unsigned)(((size_t)sh.n_expert * (sh.E / 16) + 3) / 4);
+    if (L.down.type == WT_MXFP4) hipLaunchKernelGGL(k_moe_down<WT_MXFP4>, dim3(d_blocks), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(k_moe_down<WT_Q8_0>, dim3(d_blocks), dim3(256), 0, s, a);
+    check_launch("moe_down");
+    hipLaunchKernelGGL(k_moe_combine, dim3(T, (sh.E / 4 + 255) / 256), dim3(256), 0, s, b.out_pair, b.q_of_pair, b.wgt,
+                       sh.k_used, sh.E, x);
+    check_launch("moe_combine");
+}
+
+}  // namespace rk

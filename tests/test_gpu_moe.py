@@ -1,0 +1,45 @@
+"""Mixture-of-experts layers on the GPU against the CPU oracle (qwen3moe:
+softmax router, top-k experts with renormalised weights, SwiGLU experts;
+MXFP4 and Q8_0 expert weights)."""
+import numpy as np
+import pytest
+
+import oracle
+from engine_helpers import assert_logits_close, greedy, run_both
+from retrograd_amd import engine as E
+from retrograd_amd import gguf_writer as gw
+from retrograd_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+BASE = dict(n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64, n_vocab=1024, n_expert=16, n_expert_used=4,
+            n_ff_exp=256)
+SHAPES = {
+    "mxfp4": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-mxfp4", **BASE),
+    "q8_0": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q8", expert_type=gw.GGML_Q8_0, **BASE),
+}
+
+
+@pytest.mark.parametrize("key", list(SHAPES))
+def test_moe_prefill_and_decode_match_the_oracle(tmp_path, key):
+    shape = SHAPES[key]
+    print("mixture of experts: %s" % shape.name, flush=True)
+    path = tmp_path / "moe.gguf"
+    synth.write_model(path, shape, seed=5, device="cpu", std=0.05)
+    eng = E.Engine(path, E.EngineConfig(n_ctx=2048, n_seq_max=8, n_batch=256, n_ubatch=256))
+    m = oracle.Model(path)
+    ctx = oracle.Context(m, 8)
+    rng = np.random.default_rng(2)
+    lens = [7, 40, 65, 18, 3]                      # 133 tokens: experts see more than 32 tokens each
+    prompts = [rng.integers(0, m.n_vocab, n) for n in lens]
+    rows = [(i, i, p, 0, True) for i, p in enumerate(prompts)]
+    out, got, want = run_both(eng, ctx, rows)
+    assert_logits_close(got, want)
+    pos = list(lens)
+    for _ in range(3):
+        feed = [int(want[i].argmax()) for i in range(len(lens))]
+        rows = [(i, i, [feed[i]], pos[i], True) for i in range(len(lens))]
+        out, got, want = run_both(eng, ctx, rows)
+        assert_logits_close(got, want)
+        pos = [p + 1 for p in pos]
+    eng.close()

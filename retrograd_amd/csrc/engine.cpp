@@ -317,6 +317,7 @@ void Engine::build_buffers() {
     pk_.tile_t0 = i32((size_t)B); pk_.tile_nq = i32((size_t)B); pk_.tile_item0 = i32((size_t)B);
     pk_.tile_nsplit = i32((size_t)B); pk_.tile_page0 = i32((size_t)B); pk_.tile_kv_begin = i32((size_t)B);
     pk_.tok_tile = i32((size_t)B);
+    pk_.tok_merge = (int4 *)i32((size_t)B * 4);
     pk_.rope_cos = (float *)i32((size_t)B * (hp_.rope_dim / 2));
     pk_.rope_sin = (float *)i32((size_t)B * (hp_.rope_dim / 2));
 

@@ -705,38 +705,76 @@ __global__ __launch_bounds__(256) void k_rmsnorm_act(float * x, const float * __
     }
 }
 
-// E % 32 == 0: 8 elements per lane, 16-byte loads and stores.
-__global__ __launch_bounds__(256) void k_rmsnorm_act8(float * x, const float * __restrict__ w,
-                                                      int E, float eps, const int32_t * __restrict__ rows, Act out,
-                                                      Slices add) {
-    __shared__ float red[4];
+// E % 32 == 0: 8 elements per lane, 16-byte loads and stores. NW waves per row:
+// a row is read by one workgroup, and a workgroup's bandwidth grows with the
+// loads it has in flight, so wide rows get more waves.
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void k_rmsnorm_act8(float * x, const float * __restrict__ w,
+                                                          int E, float eps, const int32_t * __restrict__ rows, Act out,
+                                                          Slices add) {
+    constexpr int STEP = NW * 64 * 8;
+    __shared__ float red[NW];
     const int o = blockIdx.x;
     const int row = rows ? rows[o] : o;
     float * xr = x + (size_t)row * E;
     float ss = 0.0f;
-    for (int k = threadIdx.x * 8; k < E; k += 2048) {
+    // the first 2 x STEP elements of the row stay in registers between the two passes
+    constexpr int KEEP = 2;
+    f4 ka[KEEP], kb[KEEP], wa[KEEP], wb[KEEP];
+#pragma unroll
+    for (int c = 0; c < KEEP; ++c) {
+        const int k = threadIdx.x * 8 + c * STEP;
+        if (k < E) { wa[c] = *(const f4 *)(w + k); wb[c] = *(const f4 *)(w + k + 4); }   // independent of everything: issued first
+    }
+    int c = 0;
+    for (int k = threadIdx.x * 8; k < E; k += STEP, ++c) {
         f4 a = *(const f4 *)(xr + k), b = *(const f4 *)(xr + k + 4);
         if (add.n > 0) {
-            for (int j = 0; j < add.n; ++j) {
-                const float * sl = add.data + (size_t)j * add.stride + (size_t)row * E + k;
-                a += *(const f4 *)sl;
-                b += *(const f4 *)(sl + 4);
+            const float * sl = add.data + (size_t)row * E + k;
+            int j = 0;
+            for (; j + 4 <= add.n; j += 4) {          // four slices' loads in flight together
+                f4 sa[4], sb[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    sa[u] = *(const f4 *)(sl + (size_t)(j + u) * add.stride);
+                    sb[u] = *(const f4 *)(sl + (size_t)(j + u) * add.stride + 4);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) { a += sa[u]; b += sb[u]; }
             }
-            *(f4 *)(xr + k) = a;          // re-read below by the same thread
+            for (; j < add.n; ++j) {
+                a += *(const f4 *)(sl + (size_t)j * add.stride);
+                b += *(const f4 *)(sl + (size_t)j * add.stride + 4);
+            }
+            *(f4 *)(xr + k) = a;          // read again below (past the kept part) by the same thread
             *(f4 *)(xr + k + 4) = b;
         }
+#pragma unroll
+        for (int i = 0; i < KEEP; ++i)
+            if (i == c) { ka[i] = a; kb[i] = b; }
         ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
     }
     ss = wave_sum(ss);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
     __syncthreads();
-    const float total = (red[0] + red[1]) + (red[2] + red[3]);
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) total += red[i];
     const float scale = 1.0f / sqrtf(total / (float)E + eps);
-    for (int k = threadIdx.x * 8; k < E; k += 2048) {
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+        const int k = threadIdx.x * 8 + i * STEP;
+        if (k >= E) break;
+        const f4 a = ka[i], b = kb[i];
+        const float v[8] = {(a.x * scale) * wa[i].x, (a.y * scale) * wa[i].y, (a.z * scale) * wa[i].z, (a.w * scale) * wa[i].w,
+                            (b.x * scale) * wb[i].x, (b.y * scale) * wb[i].y, (b.z * scale) * wb[i].z, (b.w * scale) * wb[i].w};
+        store_act8(v, out, o, k, threadIdx.x & 3);
+    }
+    for (int k = threadIdx.x * 8 + KEEP * STEP; k < E; k += STEP) {
         const f4 a = *(const f4 *)(xr + k), b = *(const f4 *)(xr + k + 4);
-        const f4 wa = *(const f4 *)(w + k), wb = *(const f4 *)(w + k + 4);
-        const float v[8] = {(a.x * scale) * wa.x, (a.y * scale) * wa.y, (a.z * scale) * wa.z, (a.w * scale) * wa.w,
-                            (b.x * scale) * wb.x, (b.y * scale) * wb.y, (b.z * scale) * wb.z, (b.w * scale) * wb.w};
+        const f4 xa = *(const f4 *)(w + k), xb = *(const f4 *)(w + k + 4);
+        const float v[8] = {(a.x * scale) * xa.x, (a.y * scale) * xa.y, (a.z * scale) * xa.z, (a.w * scale) * xa.w,
+                            (b.x * scale) * xb.x, (b.y * scale) * xb.y, (b.z * scale) * xb.z, (b.w * scale) * xb.w};
         store_act8(v, out, o, k, threadIdx.x & 3);
     }
 }
@@ -747,7 +785,8 @@ void rmsnorm_act(hipStream_t s, float * x, const float * w, int E, float eps,
     if (add.n > 0 && add.N != E) throw std::runtime_error("rmsnorm: the slices do not match the row width");
     if (out.K != E) throw std::runtime_error("rmsnorm: activation width does not match");
     if (E % 32 == 0 && out.sums) {
-        hipLaunchKernelGGL(k_rmsnorm_act8, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, out, add);
+        if (E >= 4096) hipLaunchKernelGGL(k_rmsnorm_act8<8>, dim3(n_rows), dim3(512), 0, s, x, w, E, eps, rows, out, add);
+        else hipLaunchKernelGGL(k_rmsnorm_act8<4>, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, out, add);
         check_launch("rmsnorm");
         return;
     }
@@ -904,7 +943,10 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
                 o.tile_nsplit[tile_at] = ns;
                 o.tile_page0[tile_at] = d.kv_begin / PAGE;
                 o.tile_kv_begin[tile_at] = d.kv_begin;
-                for (int i = 0; i < nq; ++i) o.tok_tile[d.tok_off + q0 + i] = tile_at;
+                for (int i = 0; i < nq; ++i) {
+                    o.tok_tile[d.tok_off + q0 + i] = tile_at;
+                    o.tok_merge[d.tok_off + q0 + i] = make_int4(item_at, ns, i, 0);
+                }
                 item_at += n_kv * ns;
                 ++tile_at;
             }
@@ -1317,38 +1359,50 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
 
 struct CombineArgs {
     const float * partial;
-    const int32_t * tok_tile;
-    const int32_t * tile_t0;
-    const int32_t * tile_item0;
-    const int32_t * tile_nsplit;
+    const int4 * tok_merge;
     Act out;
     int n_head, G, hd;
 };
 
 // One wave per (token, query head): merges the KV splits and writes the
-// attention output as the O-projection's activations.
+// attention output as the O-projection's activations. The (max, sum) pairs of
+// the splits are read one per lane, the outputs two dimensions per lane.
 __global__ __launch_bounds__(256) void k_attention_combine(CombineArgs a) {
     const int t = blockIdx.x;
     const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (head >= a.n_head) return;
-    const int tile = a.tok_tile[t];
-    const int ns = a.tile_nsplit[tile];
+    const int4 meta = a.tok_merge[t];                  // first item of the token's tile, splits, index in the tile
+    const int ns = meta.y;
     const int kvh = head / a.G, gi = head % a.G;
-    const int col = (t - a.tile_t0[tile]) * a.G + gi;
-    const int item0 = a.tile_item0[tile] + kvh * ns;
+    const int col = meta.z * a.G + gi;
+    const int item0 = meta.x + kvh * ns;
     const int stride = a.hd + 2;
-    float M = -INFINITY;
-    for (int s = 0; s < ns; ++s) M = fmaxf(M, a.partial[((size_t)(item0 + s) * 16 + col) * stride]);
-    float L = 0.0f, v0 = 0.0f, v1 = 0.0f;
     const int e0 = 2 * lane;
-    for (int s = 0; s < ns; ++s) {
-        const float * p = a.partial + ((size_t)(item0 + s) * 16 + col) * stride;
-        const float w = p[0] == -INFINITY ? 0.0f : exp2f(p[0] - M);
-        L += w * p[1];
-        if (e0 < a.hd) {
-            v0 += w * p[2 + e0];
-            v1 += w * p[3 + e0];
+    float M = -INFINITY, L = 0.0f, v0 = 0.0f, v1 = 0.0f;
+    for (int s0 = 0; s0 < ns; s0 += 64) {
+        const int n = min(64, ns - s0);
+        float m_s = -INFINITY, l_s = 0.0f;
+        if (lane < n) {
+            const float * p = a.partial + ((size_t)(item0 + s0 + lane) * 16 + col) * stride;
+            m_s = p[0];
+            l_s = p[1];
+        }
+        float cm = m_s;
+        for (int o = 32; o > 0; o >>= 1) cm = fmaxf(cm, __shfl_xor(cm, o, 64));
+        const float m_new = fmaxf(M, cm);
+        const float keep = M == -INFINITY ? 0.0f : exp2f(M - m_new);
+        L *= keep; v0 *= keep; v1 *= keep;
+        M = m_new;
+        const float w_s = m_s == -INFINITY ? 0.0f : exp2f(m_s - M);
+        L += wave_sum(w_s * l_s);
+        for (int s = 0; s < n; ++s) {
+            const float w = __shfl(w_s, s, 64);
+            if (e0 < a.hd) {
+                const float2 pv = *(const float2 *)(a.partial + ((size_t)(item0 + s0 + s) * 16 + col) * stride + 2 + e0);
+                v0 = fmaf(w, pv.x, v0);
+                v1 = fmaf(w, pv.y, v1);
+            }
         }
     }
     const float inv = L > 0.0f ? 1.0f / L : 0.0f;
@@ -1386,8 +1440,7 @@ void attention_combine(hipStream_t s, const float * partial, int T, const AttnSh
                        const PackBuffers & pk, const Act & out) {
     if (T <= 0) return;
     CombineArgs a;
-    a.partial = partial; a.tok_tile = pk.tok_tile; a.tile_t0 = pk.tile_t0; a.tile_item0 = pk.tile_item0;
-    a.tile_nsplit = pk.tile_nsplit; a.out = out;
+    a.partial = partial; a.tok_merge = pk.tok_merge; a.out = out;
     a.n_head = sh.n_head; a.G = sh.n_head / sh.n_head_kv; a.hd = sh.head_dim;
     hipLaunchKernelGGL(k_attention_combine, dim3(T, (sh.n_head + 3) / 4), dim3(256), 0, s, a);
     check_launch("attention_combine");

@@ -185,6 +185,7 @@ struct PackBuffers {       // device arrays, sized for n_batch tokens / rows
     int32_t * tile_page0;  // first page index (within the slot) the tile reads
     int32_t * tile_kv_begin;
     int32_t * tok_tile;    // [T] tile of each token
+    int4 * tok_merge;      // [T] first work item of the token's tile, its KV splits, the token's index in the tile
     float * rope_cos;      // [T][rope_dim/2]
     float * rope_sin;
 };

@@ -25,6 +25,9 @@ namespace rk {
 
 namespace {
 
+constexpr int kWaves = 8;      // 4 row waves x 2 halves of every super-block
+constexpr int kThreads = kWaves * 64;
+
 template <int NT> struct XStage {
     // 1 KiB blocks: [kstep 8][hi/lo 2][tile NT] activations, then [tile NT] block sums
     static constexpr int X_BLOCKS = 8 * 2 * NT;
@@ -78,37 +81,53 @@ __device__ __forceinline__ h8 lds_h8(const uint8_t * buf, int block, int lane) {
     return *(const h8 *)(buf + block * 1024 + lane * 16);
 }
 
-// Stores the accumulators: to y, or (split K) to this workgroup's slice of the
-// workspace, the bias going into slice 0. acc[r][t][i] is token
-// tbase + 16t + 4g + i, weight row 16 * rt[r] + r16.
+// Adds the accumulators of the two k-halves of every row wave and stores the
+// sums: to y, or (split K) to this workgroup's slice of the workspace, the
+// bias going into slice 0. Both halves leave their accumulators in LDS as
+// [token][row of the group]; then every wave stores whole token rows, 16 R
+// lanes per row with four columns each, so each store instruction writes full
+// cache lines (an accumulator tile stored from its registers covers only a
+// 64-byte piece of four different rows per instruction, which was measured to
+// cost several microseconds per launch at 64 tokens).
+// acc[r][t][i] is token 16t + 4g + i of the chunk, row 16 (rw R + r) + r16 of the group.
 template <int NT, int R>
-__device__ __forceinline__ void finish(const MMArgs & a, f4 (&acc)[R][NT], const int (&rt)[R], int tbase, int nt,
-                                       int ks, bool owner) {
-    if (!owner) return;
-    const int lane = threadIdx.x & 63;
+__device__ __forceinline__ void join_and_store(const MMArgs & a, f4 (&acc)[R][NT], uint8_t * smem, int rg, int rw, int kh,
+                                               int tbase, int ks) {
+    constexpr int S = 64 * R + 4;          // floats per token row in LDS; the pad spreads the four token rows a store touches over the banks
+    constexpr int LPR = 16 * R;            // lanes per token row
+    constexpr int TPI = 64 / LPR;          // token rows per store instruction
+    static_assert(2 * NT * 16 * S * 4 <= 2 * XStage<NT>::BYTES, "both halves' accumulators fit the staging buffers");
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, g = lane >> 4;
+    __syncthreads();       // every wave is done with the staged activations
+    float * mine = (float *)smem + kh * (NT * 16 * S);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mine[(t * 16 + 4 * g + i) * S + (rw * R + r) * 16 + r16] = acc[r][t][i];
+    __syncthreads();
+    if (a.debug & 8) return;
+    const float * h0 = (const float *)smem, * h1 = h0 + NT * 16 * S;
+    const int col = (lane % LPR) * 4;
+    const int n = rg * 64 * R + col;
+    if (n >= a.N) return;
     const bool sliced = a.ksplit > 1;
     float * slice = sliced ? a.partial + (size_t)ks * 64 * a.N : nullptr;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        if (rt[r] >= a.n_row_tiles) continue;
-        const int n = rt[r] * 16 + r16;
-        const float bias = (a.bias && ks == 0) ? a.bias[n] : 0.0f;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            if (t >= nt) break;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int tok = tbase + t * 16 + 4 * g + i;
-                if (tok >= a.T) continue;
-                const float v = acc[r][t][i] + bias;
-                if (sliced) {
-                    slice[(size_t)tok * a.N + n] = v;
-                } else {
-                    float * p = a.y + (size_t)tok * a.ldy + a.col0 + n;
-                    *p = a.mode == MM_ADD ? *p + v : v;
-                }
-            }
+    const f4 bias = (a.bias && ks == 0) ? *(const f4 *)(a.bias + n) : (f4){0.f, 0.f, 0.f, 0.f};
+    const int nrows = min(NT * 16, a.T - tbase);
+    for (int tk = wave * TPI + lane / LPR; tk < nrows; tk += kWaves * TPI) {
+        f4 v = *(const f4 *)(h0 + tk * S + col);
+        v += *(const f4 *)(h1 + tk * S + col);
+        v += bias;
+        const int tok = tbase + tk;
+        if (sliced) {
+            *(f4 *)(slice + (size_t)tok * a.N + n) = v;
+        } else {
+            float * p = a.y + (size_t)tok * a.ldy + a.col0 + n;
+            if (a.mode == MM_ADD) v = *(const f4 *)p + v;
+            *(f4 *)p = v;
         }
     }
 }
@@ -125,32 +144,6 @@ __device__ __forceinline__ h2 magic_pair(uint32_t word, uint32_t sel) {
     return __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, word, sel));
 }
 
-constexpr int kWaves = 8;      // 4 row waves x 2 halves of every super-block
-constexpr int kThreads = kWaves * 64;
-
-// The two k-halves of a row wave add their accumulators through LDS; the sum
-// is left in the half-0 waves.
-template <int NT, int R>
-__device__ __forceinline__ void join_halves(f4 (&acc)[R][NT], uint8_t * smem, int rw, int kh, int lane) {
-    __syncthreads();       // every wave is done with the staged activations
-    if (kh == 1) {
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int t = 0; t < NT; ++t) *(f4 *)(smem + (((rw * R + r) * NT + t) * 64 + lane) * 16) = acc[r][t];
-    }
-    __syncthreads();
-    if (kh == 0) {
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                const f4 o = *(const f4 *)(smem + (((rw * R + r) * NT + t) * 64 + lane) * 16);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[r][t][i] += o[i];
-            }
-    }
-}
 
 }  // namespace
 
@@ -163,7 +156,6 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
     const int r16 = lane & 15;
     const int rg = blockIdx.x % a.n_row_groups, ks = blockIdx.x / a.n_row_groups;
     const int tbase = blockIdx.y * 64;
-    const int nt = min(NT, (a.T - tbase + 15) >> 4);
     const int nsb = a.K >> 8;
     const int per = (nsb + a.ksplit - 1) / a.ksplit;
     const int sb0 = ks * per, sb1 = min(nsb, sb0 + per);
@@ -302,8 +294,191 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
             body(sb + 2, w2, w1);
         }
     }
-    join_halves<NT, R>(acc, smem, rw, kh, lane);
-    finish<NT, R>(a, acc, rt, tbase, nt, ks, kh == 0);
+    join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
+}
+
+// Q4_K with the two k-halves of a workgroup half a super-block out of step.
+// The waves of one half share their SIMDs with the waves of the other, so
+// while one half multiplies (matrix pipe, LDS reads) the other decodes its
+// next weights (vector ALU); run in step, both would want the same pipe at the
+// same time and the phases would add up instead of overlapping. A super-block
+// takes two intervals, each opened by a barrier:
+//   interval a(s): half 0 decodes s,            half 1 multiplies s - 1
+//   interval b(s): half 0 multiplies s,         half 1 decodes s
+// The activations of s + 1 are requested at the start of b(s), when nobody
+// reads their buffer any more (half 1 finished s - 1 in a(s)), and each wave
+// sees its own requests land before the barrier that opens b(s + 1).
+template <int NT, int R>
+__global__ __launch_bounds__(kThreads, 1) void k_mm3_q4k(MMArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rw = wave & 3, kh = wave >> 2;
+    const int r16 = lane & 15;
+    const int rg = blockIdx.x % a.n_row_groups, ks = blockIdx.x / a.n_row_groups;
+    const int tbase = blockIdx.y * 64;
+    const int nsb = a.K >> 8;
+    const int per = (nsb + a.ksplit - 1) / a.ksplit;
+    const int sb0 = ks * per, sb1 = min(nsb, sb0 + per);
+    constexpr int STAGE_LOADS = 16 / (8 / NT);      // activation blocks a wave requests per super-block (sums not counted)
+
+    int rt[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) rt[r] = (rg * 4 + rw) * R + r;
+    const StageSrc<NT> stage = stage_prepare<NT>(a, blockIdx.y, lane, wave);
+
+    f4 acc[R][NT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
+
+    const uint8_t * wbase[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) wbase[r] = a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 2304;
+    struct WSet { u4 hdr[R]; u4 q[R]; };
+    auto load_w = [&](int sb, WSet & w) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint8_t * tile = wbase[r] + (size_t)sb * 2304;
+            w.hdr[r] = *(const u4 *)(tile + r16 * 16);
+            w.q[r] = *(const u4 *)(tile + 256 + kh * 1024 + lane * 16);
+        }
+    };
+    const h2 m1024 = {(_Float16)(-1024.0f), (_Float16)(-1024.0f)};
+    const uint32_t magic1024 = 0x64006400u, magic64 = 0x54005400u;
+
+    // decoded weights of one super-block half: sc * e as exact f16 integers in
+    // operand order, the mins the same way, and the two row factors
+    struct Prep { h8 B[4][R]; h8 mB[R]; float d[R], ndmin[R]; };
+    auto decode = [&](const WSet & w, Prep & p) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const Q4KScales s4 = q4k_scales(w.hdr[r]);
+            const h2 p0 = magic_pair(s4.mn[0], 0x04010400u) + m1024;
+            const h2 p1 = magic_pair(s4.mn[0], 0x04030402u) + m1024;
+            const h2 p2 = magic_pair(s4.mn[1], 0x04010400u) + m1024;
+            const h2 p3 = magic_pair(s4.mn[1], 0x04030402u) + m1024;
+            p.mB[r] = (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
+            p.d[r] = h2f((uint16_t)(w.hdr[r].x & 0xffff));
+            p.ndmin[r] = -h2f((uint16_t)(w.hdr[r].x >> 16));
+            const uint32_t scw = kh ? s4.sc[1] : s4.sc[0];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const h2 k1 = magic_pair(scw, 0x04000400u + 0x00010001u * j) + m1024;   // (sc, sc)
+                const h2 c1 = k1 * (_Float16)(-1024.0f);
+                const h2 c2 = k1 * (_Float16)(-64.0f);
+                const uint32_t wq = w.q[r][j];
+                const uint32_t w8 = wq >> 8;
+                // 1024 + e in the low nibble positions, 64 + e in the high ones
+                const h2 u0 = __builtin_bit_cast(h2, and_or(wq, 0x000F000Fu, magic1024));
+                const h2 u1 = __builtin_bit_cast(h2, and_or(wq, 0x00F000F0u, magic64));
+                const h2 u2 = __builtin_bit_cast(h2, and_or(w8, 0x000F000Fu, magic1024));
+                const h2 u3 = __builtin_bit_cast(h2, and_or(w8, 0x00F000F0u, magic64));
+                const h2 a0 = __builtin_elementwise_fma(u0, k1, c1);   // exactly sc * e (<= 945)
+                const h2 a1 = __builtin_elementwise_fma(u1, k1, c2);
+                const h2 a2 = __builtin_elementwise_fma(u2, k1, c1);
+                const h2 a3 = __builtin_elementwise_fma(u3, k1, c2);
+                p.B[j][r] = (h8){a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+            }
+        }
+    };
+    auto multiply = [&](const Prep & p, const uint8_t * cur) {
+        if (a.debug & 2) return;
+        __builtin_amdgcn_s_setprio(1);
+        // min term: k-slots of lane group 0 carry the hi block sums, group 1 the
+        // lo sums, groups 2-3 zeros; the token tiles are shared out between the halves
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            if ((NT == 1 ? 0 : (t & 1)) != kh) continue;
+            const h8 sA = lds_h8(cur, XStage<NT>::X_BLOCKS + t, lane);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const f4 m4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(sA, p.mB[r], (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[r][t][i] = fmaf(p.ndmin[r], m4[i], acc[r][t][i]);
+            }
+        }
+        f4 accq[R][NT];
+        const uint8_t * xk = cur + kh * (8 * NT * 1024);      // this half's four k-steps
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            h8 A[NT], Al[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                A[t] = lds_h8(xk, (j * 2 + 0) * NT + t, lane);
+                Al[t] = lds_h8(xk, (j * 2 + 1) * NT + t, lane);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    f4 c = j == 0 ? (f4){0.f, 0.f, 0.f, 0.f} : accq[r][t];
+                    c = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[t], p.B[j][r], c, 0, 0, 0);
+                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[t], p.B[j][r], c, 0, 0, 0);
+                }
+        }
+        __builtin_amdgcn_s_setprio(0);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[r][t][i] = fmaf(p.d[r], accq[r][t][i], acc[r][t][i]);
+    };
+    auto buffer = [&](int sb) { return (a.debug & 1) ? smem : smem + ((sb - sb0) & 1) * XStage<NT>::BYTES; };
+    auto request = [&](int sb) {      // activations of super-block sb, if there is one
+        if (sb < sb1 && !((a.debug & 1) && sb > sb0)) stage_x<NT>(stage, sb, smem + ((sb - sb0) & 1) * XStage<NT>::BYTES, true);
+    };
+
+    if (sb0 < sb1) {
+        WSet w0, w1;
+        Prep p;
+        // oldest first: weights of the first two super-blocks, then the first activations
+        load_w(sb0, w0);
+        load_w(min(sb0 + 1, sb1 - 1), w1);
+        request(sb0);
+        if (kh == 0) {
+            auto step = [&](int sb, WSet & w) {
+                // a(sb): the weights of sb have landed when at most the next
+                // super-block's weights and the activation requests are newer
+                __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R + STAGE_LOADS));
+                decode(w, p);
+                load_w(min(sb + 2, sb1 - 1), w);
+                __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R));      // this wave's activation requests for sb
+                __syncthreads();
+                // b(sb)
+                request(sb + 1);
+                multiply(p, buffer(sb));
+                __syncthreads();
+            };
+            for (int sb = sb0; sb < sb1; sb += 2) {
+                step(sb, w0);
+                if (sb + 1 >= sb1) break;
+                step(sb + 1, w1);
+            }
+        } else {
+            auto step = [&](int sb, WSet & w) {
+                // a(sb): multiply the previous super-block
+                if (sb > sb0) multiply(p, buffer(sb - 1));
+                if (sb == sb0) __builtin_amdgcn_s_waitcnt(0x0F70);
+                else __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R));
+                __syncthreads();
+                // b(sb)
+                request(sb + 1);
+                decode(w, p);
+                load_w(min(sb + 2, sb1 - 1), w);
+                __syncthreads();
+            };
+            for (int sb = sb0; sb < sb1; sb += 2) {
+                step(sb, w0);
+                if (sb + 1 >= sb1) break;
+                step(sb + 1, w1);
+            }
+            multiply(p, buffer(sb1 - 1));
+        }
+    }
+    join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
 }
 
 template <int NT, int R>
@@ -315,7 +490,6 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
     const int r16 = lane & 15;
     const int rg = blockIdx.x % a.n_row_groups, ks = blockIdx.x / a.n_row_groups;
     const int tbase = blockIdx.y * 64;
-    const int nt = min(NT, (a.T - tbase + 15) >> 4);
     const int nsb = a.K >> 8;
     const int per = (nsb + a.ksplit - 1) / a.ksplit;
     const int sb0 = ks * per, sb1 = min(nsb, sb0 + per);
@@ -398,19 +572,26 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
             body(sb + 2, w2, w1);
         }
     }
-    join_halves<NT, R>(acc, smem, rw, kh, lane);
-    finish<NT, R>(a, acc, rt, tbase, nt, ks, kh == 0);
+    join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
 }
 
 template <int NT, int R>
 static void launch2(hipStream_t s, int type, const MMArgs & a, dim3 grid) {
     const size_t lds = 2 * (size_t)XStage<NT>::BYTES;
-    static_assert(2 * XStage<NT>::BYTES >= 4 * R * NT * 1024, "the joined accumulators fit the staging buffers");
     if (type == WT_Q4_K) {
         static bool once = false;
         if (!once) {
             HIP_OK(hipFuncSetAttribute((const void *)k_mm2_q4k<NT, R>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             once = true;
+        }
+        if (NT == 4 && !(a.debug & 4)) {
+            static bool once3 = false;
+            if (!once3) {
+                HIP_OK(hipFuncSetAttribute((const void *)k_mm3_q4k<NT, R>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                once3 = true;
+            }
+            hipLaunchKernelGGL((k_mm3_q4k<NT, R>), grid, dim3(kThreads), lds, s, a);
+            return;
         }
         hipLaunchKernelGGL((k_mm2_q4k<NT, R>), grid, dim3(kThreads), lds, s, a);
     } else {
@@ -447,6 +628,9 @@ Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float *
     a.w = w.packed; a.x = x.x; a.sums = x.sums; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
     a.n_row_tiles = w.N / 16;
+    // the epilogue stores four columns per lane
+    if ((ldy & 3) || (col0 & 3) || ((uintptr_t)y & 15) || (bias && ((uintptr_t)bias & 15)))
+        throw std::runtime_error("matmul_lds: y, ldy, col0 and bias must be aligned to four floats");
     a.partial = (float *)ws;
     const int nsb = w.K / 256;
     const int nt = T > 32 ? 4 : (T > 16 ? 2 : 1);

@@ -307,448 +307,6 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
     join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
 }
 
-// Q4_K with the two k-halves of a workgroup half a super-block out of step.
-// The waves of one half share their SIMDs with the waves of the other, so
-// while one half multiplies (matrix pipe, LDS reads) the other decodes its
-// next weights (vector ALU); run in step, both would want the same pipe at the
-// same time and the phases would add up instead of overlapping. A super-block
-// takes two intervals, each opened by a barrier:
-//   interval a(s): half 0 decodes s,            half 1 multiplies s - 1
-//   interval b(s): half 0 multiplies s,         half 1 decodes s
-// The activations of s + 1 are requested at the start of b(s), when nobody
-// reads their buffer any more (half 1 finished s - 1 in a(s)), and each wave
-// sees its own requests land before the barrier that opens b(s + 1).
-template <int NT, int R>
-__global__ __launch_bounds__(kThreads, 1) void k_mm3_q4k(MMArgs a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int rw = wave & 3, kh = wave >> 2;
-    const int r16 = lane & 15;
-    const int rg = blockIdx.x % a.n_row_groups, ks = blockIdx.x / a.n_row_groups;
-    const int tbase = blockIdx.y * 64;
-    const int nsb = a.K >> 8;
-    const int per = (nsb + a.ksplit - 1) / a.ksplit;
-    const int sb0 = ks * per, sb1 = min(nsb, sb0 + per);
-    constexpr int STAGE_LOADS = 16 / (8 / NT);      // activation blocks a wave requests per super-block (sums not counted)
-
-    int rt[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) rt[r] = (rg * 4 + rw) * R + r;
-    const StageSrc<NT> stage = stage_prepare<NT>(a, blockIdx.y, lane, wave);
-
-    f4 acc[R][NT];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
-
-    const uint8_t * wbase[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) wbase[r] = a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 2304;
-    struct WSet { u4 hdr[R]; u4 q[R]; };
-    auto load_w = [&](int sb, WSet & w) __attribute__((always_inline)) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const uint8_t * tile = wbase[r] + (size_t)sb * 2304;
-            w.hdr[r] = *(const u4 *)(tile + r16 * 16);
-            w.q[r] = *(const u4 *)(tile + 256 + kh * 1024 + lane * 16);
-        }
-    };
-    const h2 m1024 = {(_Float16)(-1024.0f), (_Float16)(-1024.0f)};
-    const uint32_t magic1024 = 0x64006400u, magic64 = 0x54005400u;
-
-    // One of this wave's activation requests for super-block sb: block idx of
-    // its share, or (idx 8) the block sums. A burst of requests would hold the
-    // wave at the issue of each until the memory pipeline has taken the one
-    // before, so decode and multiply issue them one at a time between their
-    // own instructions.
-    auto request = [&](int sb, int idx) __attribute__((always_inline)) {
-        if (sb >= sb1 || ((a.debug & 1) && sb > sb0)) return;
-        uint8_t * buf = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
-        constexpr int WAVES_PER_TILE = 8 / NT;
-        if (idx < STAGE_LOADS) {
-            const int c = stage.slot + WAVES_PER_TILE * idx;
-            const __half * src = stage.x + (size_t)(sb * 16 + c) * 2048;
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)src,
-                                             (void __attribute__((address_space(3))) *)(buf + (c * NT + stage.tile) * 1024), 16, 0, 0);
-        } else if (idx == 8 && stage.slot == 0) {
-            const __half * src = stage.sum + (size_t)sb * 2048;
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)src,
-                                             (void __attribute__((address_space(3))) *)(buf + (XStage<NT>::X_BLOCKS + stage.tile) * 1024), 16, 0, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    // decoded weights of one super-block half: sc * e as exact f16 integers in
-    // operand order, the mins the same way, and the two row factors
-    struct Prep { h8 B[4][R]; h8 mB[R]; float d[R], ndmin[R]; };
-    // req: super-block whose activations are requested along the way, or sb1 for none
-    auto decode = [&](const WSet & w, Prep & p, int req) __attribute__((always_inline)) {
-        request(req, 8);
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const Q4KScales s4 = q4k_scales(w.hdr[r]);
-            const h2 p0 = magic_pair(s4.mn[0], 0x04010400u) + m1024;
-            const h2 p1 = magic_pair(s4.mn[0], 0x04030402u) + m1024;
-            const h2 p2 = magic_pair(s4.mn[1], 0x04010400u) + m1024;
-            const h2 p3 = magic_pair(s4.mn[1], 0x04030402u) + m1024;
-            p.mB[r] = (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
-            p.d[r] = h2f((uint16_t)(w.hdr[r].x & 0xffff));
-            p.ndmin[r] = -h2f((uint16_t)(w.hdr[r].x >> 16));
-            const uint32_t scw = kh ? s4.sc[1] : s4.sc[0];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                request(req, (r * 4 + j) * 8 / (4 * R));
-                const h2 k1 = magic_pair(scw, 0x04000400u + 0x00010001u * j) + m1024;   // (sc, sc)
-                const h2 c1 = k1 * (_Float16)(-1024.0f);
-                const h2 c2 = k1 * (_Float16)(-64.0f);
-                const uint32_t wq = w.q[r][j];
-                const uint32_t w8 = wq >> 8;
-                // 1024 + e in the low nibble positions, 64 + e in the high ones
-                const h2 u0 = __builtin_bit_cast(h2, and_or(wq, 0x000F000Fu, magic1024));
-                const h2 u1 = __builtin_bit_cast(h2, and_or(wq, 0x00F000F0u, magic64));
-                const h2 u2 = __builtin_bit_cast(h2, and_or(w8, 0x000F000Fu, magic1024));
-                const h2 u3 = __builtin_bit_cast(h2, and_or(w8, 0x00F000F0u, magic64));
-                const h2 a0 = __builtin_elementwise_fma(u0, k1, c1);   // exactly sc * e (<= 945)
-                const h2 a1 = __builtin_elementwise_fma(u1, k1, c2);
-                const h2 a2 = __builtin_elementwise_fma(u2, k1, c1);
-                const h2 a3 = __builtin_elementwise_fma(u3, k1, c2);
-                p.B[j][r] = (h8){a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
-            }
-        }
-    };
-    // The activation fragments of k-step j + 1 are read from LDS before the
-    // products of k-step j are issued: a wave that reads, waits and then
-    // multiplies leaves the matrix pipe idle for the whole read.
-    auto multiply = [&](const Prep & p, const uint8_t * cur, int req) __attribute__((always_inline)) {
-        if (a.debug & 2) {
-            for (int i = 0; i <= 8; ++i) request(req, i);
-            return;
-        }
-        __builtin_amdgcn_s_setprio(1);
-        const uint8_t * xk = cur + kh * (8 * NT * 1024);      // this half's four k-steps
-        // hi and lo fragments of a k-step are two half-steps, each read from
-        // LDS while the products of the half-step before are issued
-        h8 A[NT], Al[NT];
-        auto read_hi = [&](int j) __attribute__((always_inline)) {
-#pragma unroll
-            for (int t = 0; t < NT; ++t) A[t] = lds_h8(xk, (j * 2 + 0) * NT + t, lane);
-        };
-        auto read_lo = [&](int j) __attribute__((always_inline)) {
-#pragma unroll
-            for (int t = 0; t < NT; ++t) Al[t] = lds_h8(xk, (j * 2 + 1) * NT + t, lane);
-        };
-        // min term: k-slots of lane group 0 carry the hi block sums, group 1 the
-        // lo sums, groups 2-3 zeros; the token tiles are shared out between the halves
-        h8 sA[NT];
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-            if ((NT == 1 ? 0 : (t & 1)) == kh) sA[t] = lds_h8(cur, XStage<NT>::X_BLOCKS + t, lane);
-        read_hi(0);
-        __builtin_amdgcn_sched_barrier(0);
-        request(req, 8);
-#pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            if ((NT == 1 ? 0 : (t & 1)) != kh) continue;
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const f4 m4 = __builtin_amdgcn_mfma_f32_16x16x32_f16(sA[t], p.mB[r], (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[r][t][i] = fmaf(p.ndmin[r], m4[i], acc[r][t][i]);
-            }
-        }
-        f4 accq[R][NT];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            read_lo(j);
-            __builtin_amdgcn_sched_barrier(0);
-            request(req, 2 * j);
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-#pragma unroll
-                for (int t = 0; t < NT; ++t)
-                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[t], p.B[j][r], j == 0 ? (f4){0.f, 0.f, 0.f, 0.f} : accq[r][t], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            if (j + 1 < 4) read_hi(j + 1);
-            __builtin_amdgcn_sched_barrier(0);
-            request(req, 2 * j + 1);
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-#pragma unroll
-                for (int t = 0; t < NT; ++t)
-                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[t], p.B[j][r], accq[r][t], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        __builtin_amdgcn_s_setprio(0);
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[r][t][i] = fmaf(p.d[r], accq[r][t][i], acc[r][t][i]);
-    };
-    auto buffer = [&](int sb) { return (a.debug & 1) ? smem : smem + ((sb - sb0) & 1) * XStage<NT>::BYTES; };
-
-    if (sb0 < sb1) {
-        WSet w0, w1;
-        Prep p;
-        // oldest first: weights of the first two super-blocks, then the first activations
-        load_w(sb0, w0);
-        load_w(min(sb0 + 1, sb1 - 1), w1);
-        for (int i = 0; i <= 8; ++i) request(sb0, i);
-        if (kh == 0) {
-            auto step = [&](int sb, WSet & w) __attribute__((always_inline)) {
-                // a(sb): the weights of sb have landed when at most the next
-                // super-block's weights and the activation requests are newer
-                __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R + STAGE_LOADS));
-                decode(w, p, sb1);
-                load_w(min(sb + 2, sb1 - 1), w);
-                __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R));      // this wave's activation requests for sb
-                __syncthreads();
-                // b(sb)
-                multiply(p, buffer(sb), sb + 1);
-                __syncthreads();
-            };
-            for (int sb = sb0; sb < sb1; sb += 2) {
-                step(sb, w0);
-                if (sb + 1 >= sb1) break;
-                step(sb + 1, w1);
-            }
-        } else {
-            auto step = [&](int sb, WSet & w) __attribute__((always_inline)) {
-                // a(sb): multiply the previous super-block
-                if (sb > sb0) multiply(p, buffer(sb - 1), sb1);
-                if (sb == sb0) __builtin_amdgcn_s_waitcnt(0x0F70);
-                else __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R));
-                __syncthreads();
-                // b(sb)
-                decode(w, p, sb + 1);
-                load_w(min(sb + 2, sb1 - 1), w);
-                __syncthreads();
-            };
-            for (int sb = sb0; sb < sb1; sb += 2) {
-                step(sb, w0);
-                if (sb + 1 >= sb1) break;
-                step(sb + 1, w1);
-            }
-            multiply(p, buffer(sb1 - 1), sb1);
-        }
-    }
-    join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
-}
-
-// Q4_K, every wave running one instruction stream per super-block in which the
-// pieces that occupy different units alternate: a wave issues in order, a
-// 16-byte LDS read holds it for about as long as a matrix instruction, and a
-// burst of memory requests holds it until the memory pipeline has taken them,
-// so the reads of a half k-step are issued before the products of the half
-// step before, the activation requests one at a time between them, and the
-// decode of the next k-step's weights falls into the shadow of the products.
-template <int NT, int R>
-__global__ __launch_bounds__(kThreads, 1) void k_mm4_q4k(MMArgs a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int rw = wave & 3, kh = wave >> 2;
-    const int r16 = lane & 15;
-    const int rg = blockIdx.x % a.n_row_groups, ks = blockIdx.x / a.n_row_groups;
-    const int tbase = blockIdx.y * 64;
-    const int nsb = a.K >> 8;
-    const int per = (nsb + a.ksplit - 1) / a.ksplit;
-    const int sb0 = ks * per, sb1 = min(nsb, sb0 + per);
-    constexpr int STAGE_LOADS = 16 / (8 / NT);      // activation blocks a wave requests per super-block (sums not counted)
-    constexpr int WAVES_PER_TILE = 8 / NT;
-
-    int rt[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) rt[r] = (rg * 4 + rw) * R + r;
-    const StageSrc<NT> stage = stage_prepare<NT>(a, blockIdx.y, lane, wave);
-
-    f4 acc[R][NT];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
-    // min term of token tile MT * kh + i, kept apart so that the stream has no
-    // branch on the half; added to the accumulators once, after the last super-block
-    constexpr int MT = NT == 1 ? 1 : NT / 2;
-    f4 accm[R][MT];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int i = 0; i < MT; ++i) accm[r][i] = (f4){0.f, 0.f, 0.f, 0.f};
-
-    const uint8_t * wbase[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) wbase[r] = a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 2304;
-    struct WSet { u4 hdr[R]; u4 q[R]; };
-    auto load_w = [&](int sb, WSet & w) __attribute__((always_inline)) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const uint8_t * tile = wbase[r] + (size_t)sb * 2304;
-            w.hdr[r] = *(const u4 *)(tile + r16 * 16);
-            w.q[r] = *(const u4 *)(tile + 256 + kh * 1024 + lane * 16);
-        }
-    };
-    const h2 m1024 = {(_Float16)(-1024.0f), (_Float16)(-1024.0f)};
-    const uint32_t magic1024 = 0x64006400u, magic64 = 0x54005400u;
-
-    // One of this wave's activation requests for super-block sb (clamped to the
-    // last one, whose repeated request lands in the buffer nobody reads any
-    // more): block idx of its share, or (idx 8) the block sums.
-    auto request = [&](int sb, int idx) __attribute__((always_inline)) {
-        uint8_t * buf = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
-        sb = min(sb, sb1 - 1);
-        if (idx < STAGE_LOADS) {
-            const int c = stage.slot + WAVES_PER_TILE * idx;
-            const __half * src = stage.x + (size_t)(sb * 16 + c) * 2048;
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)src,
-                                             (void __attribute__((address_space(3))) *)(buf + (c * NT + stage.tile) * 1024), 16, 0, 0);
-        } else if (idx == 8) {
-            // every wave requests sums (waves past slot 0 repeat slot 0's block): no branch in the stream
-            const __half * src = stage.sum + (size_t)sb * 2048;
-            __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)src,
-                                             (void __attribute__((address_space(3))) *)(buf + (XStage<NT>::X_BLOCKS + stage.tile) * 1024), 16, 0, 0);
-        }
-    };
-
-    auto body = [&](int sb, WSet & w) __attribute__((always_inline)) {
-        const uint8_t * cur = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
-        // Only the weights requested at the end of the last super-block may
-        // still be on their way: this one's weights and activations are in.
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R));
-        __syncthreads();   // ... for every wave, and nobody still reads the other buffer
-        const uint8_t * xk = cur + kh * (8 * NT * 1024);      // this half's four k-steps
-        h8 A[NT], Al[NT], sA[MT];
-        auto read_hi = [&](int j) __attribute__((always_inline)) {
-#pragma unroll
-            for (int t = 0; t < NT; ++t) A[t] = lds_h8(xk, (j * 2 + 0) * NT + t, lane);
-        };
-        auto read_lo = [&](int j) __attribute__((always_inline)) {
-#pragma unroll
-            for (int t = 0; t < NT; ++t) Al[t] = lds_h8(xk, (j * 2 + 1) * NT + t, lane);
-        };
-#pragma unroll
-        for (int i = 0; i < MT; ++i) sA[i] = lds_h8(cur, XStage<NT>::X_BLOCKS + (NT == 1 ? 0 : MT * kh + i), lane);
-        read_hi(0);
-
-        uint32_t scw[R];
-        h8 mB[R];
-        float d[R], ndmin[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const Q4KScales s4 = q4k_scales(w.hdr[r]);
-            const h2 p0 = magic_pair(s4.mn[0], 0x04010400u) + m1024;
-            const h2 p1 = magic_pair(s4.mn[0], 0x04030402u) + m1024;
-            const h2 p2 = magic_pair(s4.mn[1], 0x04010400u) + m1024;
-            const h2 p3 = magic_pair(s4.mn[1], 0x04030402u) + m1024;
-            mB[r] = (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
-            d[r] = h2f((uint16_t)(w.hdr[r].x & 0xffff));
-            ndmin[r] = -h2f((uint16_t)(w.hdr[r].x >> 16));
-            scw[r] = kh ? s4.sc[1] : s4.sc[0];
-        }
-        auto decode = [&](int j, int r) __attribute__((always_inline)) {
-            const h2 k1 = magic_pair(scw[r], 0x04000400u + 0x00010001u * j) + m1024;   // (sc, sc)
-            const h2 c1 = k1 * (_Float16)(-1024.0f);
-            const h2 c2 = k1 * (_Float16)(-64.0f);
-            const uint32_t wq = w.q[r][j];
-            const uint32_t w8 = wq >> 8;
-            // 1024 + e in the low nibble positions, 64 + e in the high ones
-            const h2 u0 = __builtin_bit_cast(h2, and_or(wq, 0x000F000Fu, magic1024));
-            const h2 u1 = __builtin_bit_cast(h2, and_or(wq, 0x00F000F0u, magic64));
-            const h2 u2 = __builtin_bit_cast(h2, and_or(w8, 0x000F000Fu, magic1024));
-            const h2 u3 = __builtin_bit_cast(h2, and_or(w8, 0x00F000F0u, magic64));
-            const h2 a0 = __builtin_elementwise_fma(u0, k1, c1);   // exactly sc * e (<= 945)
-            const h2 a1 = __builtin_elementwise_fma(u1, k1, c2);
-            const h2 a2 = __builtin_elementwise_fma(u2, k1, c1);
-            const h2 a3 = __builtin_elementwise_fma(u3, k1, c2);
-            return (h8){a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
-        };
-        h8 B[2][R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) B[0][r] = decode(0, r);
-        request(sb + 1, 8);
-
-        // min term: k-slots of lane group 0 carry the hi block sums, group 1 the
-        // lo sums, groups 2-3 zeros; the token tiles are shared out between the halves
-        f4 m4[R][MT];
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-                m4[r][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(sA[i], mB[r], (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-        f4 accq[R][NT];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            read_lo(j);
-            request(sb + 1, 2 * j);
-            if (j + 1 < 4) {
-#pragma unroll
-                for (int r = 0; r < R; ++r) B[(j + 1) & 1][r] = decode(j + 1, r);
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-#pragma unroll
-                for (int t = 0; t < NT; ++t)
-                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[t], B[j & 1][r], j == 0 ? (f4){0.f, 0.f, 0.f, 0.f} : accq[r][t], 0, 0, 0);
-            if (j + 1 < 4) read_hi(j + 1);
-            request(sb + 1, 2 * j + 1);
-            if (j == 0) {
-#pragma unroll
-                for (int i = 0; i < MT; ++i)
-#pragma unroll
-                    for (int r = 0; r < R; ++r)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) accm[r][i][e] = fmaf(ndmin[r], m4[r][i][e], accm[r][i][e]);
-            }
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-#pragma unroll
-                for (int t = 0; t < NT; ++t)
-                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[t], B[j & 1][r], accq[r][t], 0, 0, 0);
-        }
-        load_w(min(sb + 2, sb1 - 1), w);
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int t = 0; t < NT; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[r][t][i] = fmaf(d[r], accq[r][t][i], acc[r][t][i]);
-    };
-
-    if (sb0 < sb1) {
-        WSet w0, w1;
-        for (int i = 0; i <= 8; ++i) request(sb0, i);
-        load_w(sb0, w0);
-        load_w(min(sb0 + 1, sb1 - 1), w1);
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R));
-        for (int sb = sb0; sb < sb1; sb += 2) {
-            body(sb, w0);
-            if (sb + 1 >= sb1) break;
-            body(sb + 1, w1);
-        }
-        __builtin_amdgcn_s_waitcnt(0x0F70);      // the last, repeated requests have landed before the buffers are reused
-    }
-    if (NT == 1) {
-        if (kh == 0) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) acc[r][0] += accm[r][0];
-        }
-    } else {
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    acc[r][i][e] += kh == 0 ? accm[r][i][e] : 0.0f;
-                    acc[r][MT + i][e] += kh == 1 ? accm[r][i][e] : 0.0f;
-                }
-    }
-    join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
-}
-
 // Memory instructions the kernel below counts itself. The compiler's own wait
 // insertion cannot tell which staging buffer an LDS read touches and, at the
 // loop head, merges the prologue's state into every iteration; both end in a
@@ -776,6 +334,15 @@ __device__ __forceinline__ uint32_t lds_offset(const void * p) {
 }
 
 typedef float f16v __attribute__((ext_vector_type(16)));
+
+// a * b + c into a register of the allocator's choice: left to itself the
+// compiler picks the two-operand form for some of the accumulator updates and
+// pays a register copy in front of each
+__device__ __forceinline__ float fma3(float a, float b, float c) {
+    float d;
+    asm("v_fma_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
 
 // Q4_K for a full chunk of 64 tokens on v_mfma_f32_32x32x16_f16: half as many
 // matrix instructions as with 16x16x32 tiles for the same products, which
@@ -809,7 +376,8 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm5_q4k(MMArgs a) {
     const __half * su = a.sums + (size_t)blockIdx.y * act_sum_chunk_halves(a.K) + st_tile * 512;
     const uint32_t lds0 = lds_offset(smem);
 
-    f16v acc[2], accm;
+    f16v acc[2];
+    float accm[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) { acc[0][i] = 0.0f; acc[1][i] = 0.0f; accm[i] = 0.0f; }
 
@@ -888,14 +456,22 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm5_q4k(MMArgs a) {
         // weight registers could not take the next load without a copy behind a full wait
         asm volatile("" : "+v"(d), "+v"(ndmin));
         const uint32_t scw = kh ? s4.sc[1] : s4.sc[0];
-        h2 k1, c1, c2;
-        auto scales = [&](int j) __attribute__((always_inline)) {
-            k1 = magic_pair(scw, 0x04000400u + 0x00010001u * j) + m1024;   // (sc, sc)
-            c1 = k1 * (_Float16)(-1024.0f);
-            c2 = k1 * (_Float16)(-64.0f);
-        };
+        // scales of the four k-steps as f16 pairs (sc 2i, sc 2i + 1) and their products with the two magic
+        // offsets; the packed FMAs below pick the half they need, so nothing is duplicated per k-step
+        h2 kp[2], c1p[2], c2p[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            kp[i] = magic_pair(scw, i ? 0x04030402u : 0x04010400u) + m1024;
+            c1p[i] = kp[i] * (_Float16)(-1024.0f);
+            c2p[i] = kp[i] * (_Float16)(-64.0f);
+        }
         auto decode = [&](int s) __attribute__((always_inline)) {
-            const uint32_t wq = w.q[s & 1][s >> 1];
+            const int j = s >> 1;
+            const h2 kk = kp[j >> 1], cc1 = c1p[j >> 1], cc2 = c2p[j >> 1];
+            const h2 k1 = (j & 1) ? __builtin_shufflevector(kk, kk, 1, 1) : __builtin_shufflevector(kk, kk, 0, 0);
+            const h2 c1 = (j & 1) ? __builtin_shufflevector(cc1, cc1, 1, 1) : __builtin_shufflevector(cc1, cc1, 0, 0);
+            const h2 c2 = (j & 1) ? __builtin_shufflevector(cc2, cc2, 1, 1) : __builtin_shufflevector(cc2, cc2, 0, 0);
+            const uint32_t wq = w.q[s & 1][j];
             const uint32_t w8 = wq >> 8;
             // 1024 + e in the low nibble positions, 64 + e in the high ones
             const h2 u0 = __builtin_bit_cast(h2, and_or(wq, 0x000F000Fu, magic1024));
@@ -909,7 +485,6 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm5_q4k(MMArgs a) {
             return (h8){a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
         };
         h8 B[2];
-        scales(0);
         B[0] = decode(0);
         // min term: the 16 k-slots are the 8 sub-blocks' hi sums and their lo sums, against the same 8 mins
         f16v zero;
@@ -922,21 +497,19 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm5_q4k(MMArgs a) {
             if (s + 1 < 8) read_step(s + 1);
             __builtin_amdgcn_sched_barrier(0);
             // the activation requests of the next super-block, early enough to have landed by its barrier
-            if (s < 4) { request(sb + 1, 2 * s); request(sb + 1, 2 * s + 1); }
-            if (s == 4) request(sb + 1, 8);
+            if (s < 3) { request(sb + 1, 3 * s); request(sb + 1, 3 * s + 1); request(sb + 1, 3 * s + 2); }
             if (s + 1 < 8) {
-                if (((s + 1) & 1) == 0) scales((s + 1) >> 1);
                 B[(s + 1) & 1] = decode(s + 1);
             }
             // a share of the scaling left by the last super-block, and of this one's min term
 #pragma unroll
             for (int i = 2 * s; i < 2 * s + 2; ++i) {
-                acc[0][i] = fmaf(pd, pq[0][i], acc[0][i]);
-                acc[1][i] = fmaf(pd, pq[1][i], acc[1][i]);
+                acc[0][i] = fma3(pd, pq[0][i], acc[0][i]);
+                acc[1][i] = fma3(pd, pq[1][i], acc[1][i]);
             }
             if (s >= 2 && s < 6) {
 #pragma unroll
-                for (int i = 4 * (s - 2); i < 4 * (s - 2) + 4; ++i) accm[i] = fmaf(ndmin, m16[i], accm[i]);
+                for (int i = 4 * (s - 2); i < 4 * (s - 2) + 4; ++i) accm[i] = fma3(ndmin, m16[i], accm[i]);
             }
 #pragma unroll
             for (int tb = 0; tb < 2; ++tb)
@@ -1098,24 +671,6 @@ static void launch2(hipStream_t s, int type, const MMArgs & a, dim3 grid) {
                 once5 = true;
             }
             hipLaunchKernelGGL(k_mm5_q4k, grid, dim3(kThreads), lds, s, a);
-            return;
-        }
-        if (NT == 4 && !(a.debug & 16)) {
-            static bool once4 = false;
-            if (!once4) {
-                HIP_OK(hipFuncSetAttribute((const void *)k_mm4_q4k<NT, R>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-                once4 = true;
-            }
-            hipLaunchKernelGGL((k_mm4_q4k<NT, R>), grid, dim3(kThreads), lds, s, a);
-            return;
-        }
-        if (NT == 4 && !(a.debug & 4)) {
-            static bool once3 = false;
-            if (!once3) {
-                HIP_OK(hipFuncSetAttribute((const void *)k_mm3_q4k<NT, R>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-                once3 = true;
-            }
-            hipLaunchKernelGGL((k_mm3_q4k<NT, R>), grid, dim3(kThreads), lds, s, a);
             return;
         }
         hipLaunchKernelGGL((k_mm2_q4k<NT, R>), grid, dim3(kThreads), lds, s, a);

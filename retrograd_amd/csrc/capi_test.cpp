@@ -2,6 +2,7 @@
 // include/retro_kernels.h. They have no counterpart in the reference ABI: they
 // exist so parity tests can compare single kernels and device state with the
 // CPU oracle through plain C calls.
+#include <algorithm>
 #include "../../include/retro_kernels.h"
 #include "engine.hpp"
 
@@ -107,9 +108,14 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
                              int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us) {
     return guarded([&]() -> int {
         const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
+        // mode bit 4: every launch reads another copy of the weights, 1 GiB of them in turn,
+        // so that they come from HBM as in a decode step and not from the last-level cache
+        const bool cold = (mode & 16) != 0;
+        mode &= 15;
+        const size_t copies = cold ? std::max<size_t>(2, ((size_t)1 << 30) / bytes) : 1;
         DevBuf d_w, d_xh, d_sums, d_y, d_ws;
-        d_w.alloc(bytes);
-        ok(hipMemset(d_w.ptr, 0x11, bytes), "fill");
+        d_w.alloc(bytes * copies);
+        ok(hipMemset(d_w.ptr, 0x11, bytes * copies), "fill");
         d_xh.alloc(rk::act_halves(n_tokens, (int)k) * 2);
         d_sums.alloc(rk::act_sum_halves(n_tokens, (int)k) * 2);
         ok(hipMemset(d_xh.ptr, 0, d_xh.bytes), "fill"); ok(hipMemset(d_sums.ptr, 0, d_sums.bytes), "fill");
@@ -123,7 +129,9 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
         rk::g_mm_force_ksplit = force_ksplit;
         hipEvent_t e0, e1;
         ok(hipEventCreate(&e0), "event"); ok(hipEventCreate(&e1), "event");
+        size_t turn = 0;
         auto run = [&]() {
+            w.packed = d_w.as<uint8_t>() + (turn++ % copies) * bytes;
             // mode 1: register-only tiles, 2: LDS-staged tiles, 3: the same with the K-slices left unreduced
             if (mode == 3) rk::matmul_deferred(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, d_ws.ptr);
             else rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, mode == 2 ? d_ws.ptr : nullptr);

@@ -976,7 +976,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
         pending_updates_.clear();
     }
     int n_tiles = 0, n_items = 0;
-    rk::count_attention_work(hd, (int)n_rows, qt_, hp_.n_head_kv, &n_tiles, &n_items);
+    rk::count_attention_work(hd, (int)n_rows, qt_, hp_.n_head_kv, &n_tiles, &n_items, &pk_.split_pages);
 
     try {
         hip_check(hipMemcpyAsync(d_stage_.ptr, h_stage_.ptr, stage_bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");

@@ -871,10 +871,10 @@ void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out) 
 // ---------------------------------------------------------------------------
 // step packing
 
-__device__ __forceinline__ int tile_splits(int kv_begin, int kv_hi) {
+__device__ __forceinline__ int tile_splits(int kv_begin, int kv_hi, int split_pages) {
     const int p_first = kv_begin / PAGE;
     const int p_last = (kv_hi - 1) / PAGE;
-    return (p_last - p_first + 1 + SPLIT_PAGES - 1) / SPLIT_PAGES;
+    return (p_last - p_first + 1 + split_pages - 1) / split_pages;
 }
 
 // Inclusive scan of one int per thread over a 1024-thread block.
@@ -918,7 +918,7 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
             tiles = (d.n + qt - 1) / qt;
             for (int j = 0; j < tiles; ++j) {
                 const int hi = d.pos0 + min(d.n, (j + 1) * qt);
-                items += n_kv * tile_splits(d.kv_begin, hi);
+                items += n_kv * tile_splits(d.kv_begin, hi, o.split_pages);
             }
             outs = d.sample ? 1 : 0;
         }
@@ -936,7 +936,7 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
                 const int q0 = j * qt;
                 const int nq = min(qt, d.n - q0);
                 const int hi = d.pos0 + q0 + nq;
-                const int ns = tile_splits(d.kv_begin, hi);
+                const int ns = tile_splits(d.kv_begin, hi, o.split_pages);
                 o.tile_t0[tile_at] = d.tok_off + q0;
                 o.tile_nq[tile_at] = nq;
                 o.tile_item0[tile_at] = item_at;
@@ -1007,20 +1007,33 @@ void pack_step(hipStream_t s, const RowDesc * rows, int n_rows, const int32_t * 
     check_launch("pack_step");
 }
 
-void count_attention_work(const RowDesc * rows, int n_rows, int qt, int n_kv_heads, int * n_tiles, int * n_items) {
-    int tiles = 0, items = 0;
-    for (int r = 0; r < n_rows; ++r) {
-        const RowDesc & d = rows[r];
-        const int nt = (d.n + qt - 1) / qt;
-        for (int j = 0; j < nt; ++j) {
-            const int hi = d.pos0 + std::min(d.n, (j + 1) * qt);
-            const int p_first = d.kv_begin / PAGE, p_last = (hi - 1) / PAGE;
-            items += n_kv_heads * ((p_last - p_first + 1 + SPLIT_PAGES - 1) / SPLIT_PAGES);
+// Counts the step's query tiles and, for the split it chooses, its attention
+// work items. A work item is one wave; the attention kernel's time hardly
+// depends on the split as long as the waves fill the chip, while every split
+// costs the merge kernel a partial result to read, so the largest split that
+// still leaves about a wave per SIMD slot wins, and small steps get the
+// smallest one.
+void count_attention_work(const RowDesc * rows, int n_rows, int qt, int n_kv_heads, int * n_tiles, int * n_items,
+                          int * split_pages) {
+    constexpr int kEnoughItems = 1536;
+    int tiles = 0, items = 0, split = MAX_SPLIT_PAGES;
+    for (;; split /= 2) {
+        tiles = 0; items = 0;
+        for (int r = 0; r < n_rows; ++r) {
+            const RowDesc & d = rows[r];
+            const int nt = (d.n + qt - 1) / qt;
+            for (int j = 0; j < nt; ++j) {
+                const int hi = d.pos0 + std::min(d.n, (j + 1) * qt);
+                const int p_first = d.kv_begin / PAGE, p_last = (hi - 1) / PAGE;
+                items += n_kv_heads * ((p_last - p_first + 1 + split - 1) / split);
+            }
+            tiles += nt;
         }
-        tiles += nt;
+        if (items >= kEnoughItems || split <= 4) break;
     }
     *n_tiles = tiles;
     *n_items = items;
+    *split_pages = split;
 }
 
 // ---------------------------------------------------------------------------
@@ -1185,6 +1198,7 @@ struct AttnArgs {
     float * partial;
     int n_tiles, n_items, max_pages;
     int n_head, n_kv, G;
+    int split_pages;
 };
 
 // ONE: every tile holds a single query token (a pure decode step).
@@ -1213,8 +1227,8 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     const int tq = t0 + (col_ok ? qi : 0);
     const int limit = a.pos[tq];                        // this column attends positions <= limit
     const int kv_hi = a.pos[t0 + nq - 1] + 1;
-    const int page_first = a.tile_page0[tile] + split * SPLIT_PAGES;
-    const int page_end = min((kv_hi - 1) / PAGE + 1, page_first + SPLIT_PAGES);
+    const int page_first = a.tile_page0[tile] + split * a.split_pages;
+    const int page_end = min((kv_hi - 1) / PAGE + 1, page_first + a.split_pages);
 
     const int QD = a.n_head * HD;
     h8 qreg[KS], qreg_lo[KS];
@@ -1341,6 +1355,7 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
     a.tile_page0 = pk.tile_page0; a.tile_kv_begin = pk.tile_kv_begin; a.pos = pk.pos; a.seq = pk.seq;
     a.partial = partial; a.n_tiles = n_tiles; a.n_items = n_items; a.max_pages = max_pages;
     a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.G = sh.n_head / sh.n_head_kv;
+    a.split_pages = pk.split_pages;
     if (a.G > 16 || sh.n_head % sh.n_head_kv != 0) throw std::runtime_error("attention: unsupported head grouping");
 #define ATTN_LAUNCH(HD_) \
     do { \

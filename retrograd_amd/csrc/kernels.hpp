@@ -15,8 +15,9 @@ enum : int { WT_F32 = 0, WT_F16 = 1, WT_Q8_0 = 8, WT_Q4_K = 12, WT_BF16 = 30, WT
 
 // One KV page holds PAGE consecutive positions of one sequence.
 constexpr int PAGE = 32;
-// One attention work item scans at most SPLIT_PAGES pages of one sequence.
-constexpr int SPLIT_PAGES = 8;
+// One attention work item scans at most split_pages pages of one sequence;
+// count_attention_work picks the step's split, at most MAX_SPLIT_PAGES.
+constexpr int MAX_SPLIT_PAGES = 16;
 // Candidates the sampling kernel can return per row.
 constexpr int MAX_TOPK = 64;
 
@@ -188,6 +189,7 @@ struct PackBuffers {       // device arrays, sized for n_batch tokens / rows
     int4 * tok_merge;      // [T] first work item of the token's tile, its KV splits, the token's index in the tile
     float * rope_cos;      // [T][rope_dim/2]
     float * rope_sin;
+    int split_pages = MAX_SPLIT_PAGES;   // pages per attention work item in this step (set from count_attention_work)
 };
 // Applies the block-table updates, then derives every per-token / per-tile
 // array of the step from the row descriptors. One workgroup.
@@ -197,7 +199,7 @@ void pack_step(hipStream_t s, const RowDesc * rows, int n_rows, const int32_t * 
 
 // Host mirror of the tile/item count (same formula as the kernel).
 void count_attention_work(const RowDesc * rows, int n_rows, int qt, int n_kv_heads,
-                          int * n_tiles, int * n_items);
+                          int * n_tiles, int * n_items, int * split_pages);
 
 // ---- attention ----------------------------------------------------------------
 struct AttnShape {

@@ -76,6 +76,34 @@ __device__ __forceinline__ Q4KScales q4k_scales(const u4 & hdr) {
     return s;
 }
 
+// Eight consecutive activations per lane (k a multiple of 8): hi/lo as two
+// 16-byte stores; the four lanes that own one 32-wide block add their sums
+// with two xor-shuffles.
+__device__ __forceinline__ void store_act8(const float (&v)[8], const Act & out, int tok, int k, int lane_in_block) {
+    h8 a, b;
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float c = fminf(fmaxf(v[i], -65504.0f), 65504.0f);
+        const _Float16 h = (_Float16)c;
+        const _Float16 l = (_Float16)(c - (float)h);
+        a[i] = h;
+        b[i] = l;
+        sum += (float)h + (float)l;
+    }
+    *(h8 *)(out.x + act_at(tok, k, 0, out.K)) = a;
+    *(h8 *)(out.x + act_at(tok, k, 1, out.K)) = b;
+    if (out.sums) {
+        sum += __shfl_xor(sum, 1, 64);
+        sum += __shfl_xor(sum, 2, 64);
+        if (lane_in_block == 0) {
+            const __half s = sat_half(sum);
+            out.sums[act_sum_at(tok, k >> 5, 0, out.K)] = s;
+            out.sums[act_sum_at(tok, k >> 5, 1, out.K)] = __float2half_rn(sum - __half2float(s));
+        }
+    }
+}
+
 struct MMArgs {
     const uint8_t * w;
     const __half * x;         // operand-order activations and block sums (see Act)
@@ -89,6 +117,11 @@ struct MMArgs {
     int n_row_groups;
     float * partial;          // [ksplit][64][N] K-slices of a split matmul
     int debug;                // timing experiments only: bit 0 stage activations once, bit 1 skip the multiplies
+    // mode MM_SWIGLU: rows come in groups of 128, 64 gate rows then the 64 up rows of the same
+    // columns; the epilogue writes silu(gate) * up as the activations of the next matmul
+    __half * act_x;
+    __half * act_sums;
+    int act_K;
 };
 
 }  // namespace rk

@@ -187,6 +187,28 @@ void Engine::upload_fused(const std::vector<const TensorInfo *> & parts, std::ve
     }
 }
 
+// Gate and up projections as one matrix whose rows alternate in groups of 64:
+// the 64 gate rows of hidden columns [64 b, 64 b + 64), then their 64 up rows.
+// A matmul workgroup owns 128 consecutive rows, so it holds both factors of
+// its 64 hidden columns and applies SwiGLU in its epilogue. Returns false (and
+// uploads nothing) when the pair does not qualify.
+bool Engine::upload_gate_up_interleaved(const TensorInfo & g, const TensorInfo & u, std::vector<DevWeight> & out) {
+    const int64_t K = g.ne[0], F = g.ne[1];
+    if (g.type != u.type || u.ne[0] != K || u.ne[1] != F || F % 64 != 0) return false;
+    if (!rk::can_pack(g.type, K, 2 * F)) return false;
+    const size_t rb = g.nbytes / (size_t)F;
+    std::vector<uint8_t> joined(2 * g.nbytes);
+    for (int64_t b = 0; b < F / 64; ++b) {
+        std::memcpy(joined.data() + (size_t)(2 * b) * 64 * rb, g.data + (size_t)b * 64 * rb, 64 * rb);
+        std::memcpy(joined.data() + (size_t)(2 * b + 1) * 64 * rb, u.data + (size_t)b * 64 * rb, 64 * rb);
+    }
+    out.clear();
+    out.emplace_back();
+    upload_weight(g, K, 2 * F, joined.data(), joined.size(), false, out.back());
+    if (!out.back().w.packed) { out.clear(); return false; }
+    return true;
+}
+
 void Engine::load_model(const std::string & path) {
     GgufFile g(path);
     HParams & h = hp_;
@@ -272,7 +294,8 @@ void Engine::load_model(const std::string & path) {
         const TensorInfo & wd = g.require(b + "ffn_down.weight");
         if (wg.ne[0] != E || wu.ne[0] != E || wg.ne[1] != wu.ne[1] || wd.ne[0] != wg.ne[1] || wd.ne[1] != E) throw std::runtime_error("feed-forward weights of layer " + std::to_string(l) + " have unexpected shapes");
         h.n_ff = (int)wg.ne[1];
-        upload_fused({&wg, &wu}, L.gate_up);
+        L.gate_up_interleaved = upload_gate_up_interleaved(wg, wu, L.gate_up);
+        if (!L.gate_up_interleaved) upload_fused({&wg, &wu}, L.gate_up);
         upload_weight(wd, h.n_ff, E, wd.data, wd.nbytes, false, L.down);
     }
 
@@ -1192,17 +1215,20 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
             continue;
         }
         pt_ = prof_begin(PC_GATEUP);
-        {
+        if (L.gate_up_interleaved) {
+            rk::matmul_swiglu(stream_, L.gate_up[0].w, act_e, T, act_f, mm_ws_.ptr);
+            prof_end(PC_GATEUP, pt_);
+        } else {
             int col = 0;
             for (const DevWeight & w : L.gate_up) {
                 rk::matmul(stream_, w.w, act_e, T, gu, 2 * F, col, rk::MM_STORE, nullptr, mm_ws_.ptr);
                 col += w.w.N;
             }
+            prof_end(PC_GATEUP, pt_);
+            pt_ = prof_begin(PC_SWIGLU);
+            rk::swiglu_act(stream_, gu, T, F, act_f);
+            prof_end(PC_SWIGLU, pt_);
         }
-        prof_end(PC_GATEUP, pt_);
-        pt_ = prof_begin(PC_SWIGLU);
-        rk::swiglu_act(stream_, gu, T, F, act_f);
-        prof_end(PC_SWIGLU, pt_);
         pt_ = prof_begin(PC_DOWN);
         pending = rk::matmul_deferred(stream_, L.down.w, act_f, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
         prof_end(PC_DOWN, pt_);

@@ -67,6 +67,7 @@ struct LayerWeights {
     std::vector<DevWeight> qkv;    // one fused matrix, or q, k, v separately
     DevWeight wo;
     std::vector<DevWeight> gate_up; // one fused matrix, or gate, up separately
+    bool gate_up_interleaved = false;   // one matrix, 64 gate rows and 64 up rows in turn: SwiGLU runs in the matmul's epilogue
     DevWeight down;
     // mixture-of-experts layers: F32 router [n_expert][E] and the three expert tensors, tiled per expert
     DevWeight router, gate_exps, up_exps, down_exps;
@@ -149,6 +150,7 @@ private:
     void upload_weight(const TensorInfo & t, int64_t K, int64_t N, const uint8_t * data, size_t bytes,
                        bool keep_raw, DevWeight & out);
     void upload_fused(const std::vector<const TensorInfo *> & parts, std::vector<DevWeight> & out);
+    bool upload_gate_up_interleaved(const TensorInfo & g, const TensorInfo & u, std::vector<DevWeight> & out);
     void upload_f32(const TensorInfo * t, DevBuf & out, size_t expect);
     void upload_experts(const TensorInfo & t, int64_t K, int64_t N, DevWeight & out);
     void build_buffers();

@@ -124,34 +124,6 @@ __device__ __forceinline__ void store_act_block(const float * v, int count, cons
     }
 }
 
-// Eight consecutive activations per lane (k a multiple of 8): hi/lo as two
-// 16-byte stores; the four lanes that own one 32-wide block add their sums
-// with two xor-shuffles.
-__device__ __forceinline__ void store_act8(const float (&v)[8], const Act & out, int tok, int k, int lane_in_block) {
-    h8 a, b;
-    float sum = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const float c = fminf(fmaxf(v[i], -65504.0f), 65504.0f);
-        const _Float16 h = (_Float16)c;
-        const _Float16 l = (_Float16)(c - (float)h);
-        a[i] = h;
-        b[i] = l;
-        sum += (float)h + (float)l;
-    }
-    *(h8 *)(out.x + act_at(tok, k, 0, out.K)) = a;
-    *(h8 *)(out.x + act_at(tok, k, 1, out.K)) = b;
-    if (out.sums) {
-        sum += __shfl_xor(sum, 1, 64);
-        sum += __shfl_xor(sum, 2, 64);
-        if (lane_in_block == 0) {
-            const __half s = sat_half(sum);
-            out.sums[act_sum_at(tok, k >> 5, 0, out.K)] = s;
-            out.sums[act_sum_at(tok, k >> 5, 1, out.K)] = __float2half_rn(sum - __half2float(s));
-        }
-    }
-}
-
 // ---------------------------------------------------------------------------
 // plain streaming kernels: the yardstick for memory counters and bandwidth
 

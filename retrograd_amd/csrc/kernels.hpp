@@ -67,7 +67,7 @@ bool can_pack(int type, int64_t K, int64_t N);
 // raw (device, GGUF layout) -> packed (device). Both hold `bytes` bytes.
 void repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int K, int N);
 
-enum : int { MM_STORE = 0, MM_ADD = 1 };
+enum : int { MM_STORE = 0, MM_ADD = 1, MM_SWIGLU = 2 };
 // A matmul result left as n K-slices in the workspace instead of in y: element
 // (t, c) of the product (bias included) is the sum over s < n, in that order,
 // of data[s * stride + t * N + c]. n == 0: there are no slices, y holds the result.
@@ -93,6 +93,10 @@ void reduce_slices(hipStream_t s, const Slices & sl, int T, float * y, int ldy, 
 size_t matmul_workspace_bytes();
 extern int g_mm_debug;         // timing experiments (see MMArgs::debug)
 extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic
+// Fused gate/up matmul and SwiGLU: w holds, for every 64 columns of the hidden
+// layer, their 64 gate rows followed by their 64 up rows (w.N = 2 F, F % 64 == 0,
+// a tile storage type); out (K = F) receives silu(gate) * up as activations.
+void matmul_swiglu(hipStream_t s, const Weight & w, const Act & x, int T, const Act & out, void * ws);
 Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
                   int mode, const float * bias, void * ws, bool may_slice);
 // Forces the generic (raw layout) kernel; used to cross-check the tile kernels.

@@ -93,6 +93,27 @@ __device__ __forceinline__ void store_token_rows(const MMArgs & a, uint8_t * sme
     __syncthreads();
     if (a.debug & 8) return;
     const float * h0 = (const float *)smem, * h1 = h0 + NT * 16 * S;
+    if (a.mode == MM_SWIGLU) {
+        // eight lanes per token, eight hidden columns each: gate in columns c, up in columns 64 + c of the group
+        static_assert(R == 2, "a row group is 64 gate rows and 64 up rows");
+        const int c = (threadIdx.x & 7) * 8;
+        const Act out{a.act_x, a.act_sums, a.act_K};
+        for (int tk = threadIdx.x >> 3; tk < NT * 16; tk += kThreads / 8) {
+            const int tok = tbase + tk;
+            if (tok >= a.T || rg * 64 + c >= a.act_K) continue;      // the four lanes of a 32-wide block leave together
+            const float * g0 = h0 + tk * S + c, * g1 = h1 + tk * S + c;
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i += 4) {
+                const f4 g = *(const f4 *)(g0 + i) + *(const f4 *)(g1 + i);
+                const f4 u = *(const f4 *)(g0 + 64 + i) + *(const f4 *)(g1 + 64 + i);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[i + e] = (g[e] / (1.0f + __expf(-g[e]))) * u[e];
+            }
+            store_act8(v, out, tok, rg * 64 + c, threadIdx.x & 3);
+        }
+        return;
+    }
     const int col = (lane % LPR) * 4;
     const int n = rg * 64 * R + col;
     if (n >= a.N) return;
@@ -701,17 +722,20 @@ static void dispatch_nt(hipStream_t s, int type, int nt, const MMArgs & a, dim3 
     }
 }
 
-Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
-                  int mode, const float * bias, void * ws, bool may_slice) {
+// act_out: destination of mode MM_SWIGLU, else null
+static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                       int mode, const float * bias, void * ws, bool may_slice, const Act * act_out) {
     MMArgs a {};
     a.debug = g_mm_debug;
     a.w = w.packed; a.x = x.x; a.sums = x.sums; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
+    if (act_out) { a.act_x = act_out->x; a.act_sums = act_out->sums; a.act_K = act_out->K; }
     a.n_row_tiles = w.N / 16;
     // the epilogue stores four columns per lane
-    if ((ldy & 3) || (col0 & 3) || ((uintptr_t)y & 15) || (bias && ((uintptr_t)bias & 15)))
+    if (mode != MM_SWIGLU && ((ldy & 3) || (col0 & 3) || ((uintptr_t)y & 15) || (bias && ((uintptr_t)bias & 15))))
         throw std::runtime_error("matmul_lds: y, ldy, col0 and bias must be aligned to four floats");
     a.partial = (float *)ws;
+    if (mode == MM_SWIGLU) may_slice = false;
     const int nsb = w.K / 256;
     const int nt = T > 32 ? 4 : (T > 16 ? 2 : 1);
     const int chunks = (T + 63) / 64;
@@ -740,6 +764,20 @@ Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float *
     Slices out;
     if (ksplit > 1) { out.data = a.partial; out.n = ksplit; out.stride = (size_t)64 * w.N; out.N = w.N; }
     return out;
+}
+
+Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
+                  int mode, const float * bias, void * ws, bool may_slice) {
+    if (mode == MM_SWIGLU) throw std::runtime_error("matmul_lds: use matmul_swiglu");
+    return lds_impl(s, w, x, T, y, ldy, col0, mode, bias, ws, may_slice, nullptr);
+}
+
+void matmul_swiglu(hipStream_t s, const Weight & w, const Act & x, int T, const Act & out, void * ws) {
+    if (T <= 0) return;
+    if (!w.packed || !ws || w.N != 2 * out.K || out.K % 64 != 0 || !out.sums)
+        throw std::runtime_error("matmul_swiglu: needs a tile-packed gate/up matrix interleaved by 64 columns");
+    if (x.K != w.K) throw std::runtime_error("matmul_swiglu: activation width does not match the weight");
+    lds_impl(s, w, x, T, nullptr, 0, 0, MM_SWIGLU, nullptr, ws, false, &out);
 }
 
 }  // namespace rk

@@ -5,14 +5,20 @@
 // 16-row weight tile of a wave (9 B per k), so the activations are what must
 // be reused:
 //
-//   * a workgroup of 4 waves covers 4*R row tiles of 16 weight rows and all
-//     token tiles; the activations of one 256-wide super-block column are
-//     copied global -> LDS once per workgroup with direct-to-LDS loads
-//     (global_load_lds_dwordx4), already in MFMA operand order, double buffered;
+//   * a workgroup of 8 waves (4 row waves x 2 halves of every 256-wide
+//     super-block) covers 4*R row tiles of 16 weight rows and all token tiles;
+//     the activations of one super-block column are copied global -> LDS once
+//     per workgroup with direct-to-LDS loads (global_load_lds_dwordx4),
+//     already in MFMA operand order, double buffered;
 //   * each wave reads an operand from LDS once per k-step and uses it for its R
 //     row tiles;
-//   * the weights of the next super-block are prefetched into registers while
-//     the current one is multiplied.
+//   * the weights of the next super-blocks are prefetched into registers while
+//     the current one is multiplied;
+//   * the two halves add their accumulators through LDS, and the sums leave
+//     the workgroup as whole token rows.
+//
+// k_mm2_* are the general kernels (any number of token tiles, Q4_K and Q8_0);
+// k_mm5_q4k is the kernel of the decode step (Q4_K, a full 64-token chunk).
 //
 // Few row tiles (N = 4096 at batch 64) do not give every CU a workgroup, so K
 // can also be split across workgroups: each writes its sums over its slice of K

@@ -31,8 +31,12 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
                                 int32_t * out_top_ids, float * out_top_logits);
 
 /* Micro-benchmark: microseconds per launch of one tile matmul (mode 1 register
- * tiles, 2 LDS-staged tiles) over `iters` back-to-back launches on device-only
- * data. debug and force_ksplit are timing experiments (0 = normal). */
+ * tiles, 2 LDS-staged tiles, 3 the same with the K-slices left to the
+ * consumer) over `iters` back-to-back launches on device-only data. Adding 16
+ * to the mode gives every launch another copy of the weights (1 GiB of copies
+ * in turn), so that they are read from HBM as in a decode step instead of from
+ * the last-level cache. debug and force_ksplit are timing experiments
+ * (0 = normal). */
 int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,
                              int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us);
 

@@ -35,6 +35,31 @@ namespace {
 constexpr int kWaves = 8;      // 4 row waves x 2 halves of every super-block
 constexpr int kThreads = kWaves * 64;
 
+// A direct-to-LDS request issued from inline assembly. The compiler's own wait
+// insertion cannot tell which staging buffer an LDS read touches, so with the
+// builtin it waits for every request (and, loads retiring in order, for every
+// weight load before it) ahead of each barrier: s_waitcnt vmcnt(0) per
+// super-block, the whole latency of the weight prefetch exposed. Requests it
+// does not see leave only the waits written in the kernels. M0 carries the LDS
+// address. base is wave-uniform; every lane adds its own byte offset.
+__device__ __forceinline__ void lds_dma16(const void * base, uint32_t lane_off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_off), "s"(base), "s"(lds_addr) : "memory");
+}
+// In the general kernels the weight loads are ordinary loads: a load issued from
+// inline assembly hands the compiler a register whose value arrives later, and
+// any copy the register allocator makes of it before the wait (one was seen at
+// a loop latch) reads stale data. The compiler counts only the loads it knows,
+// so its own waits can only be stricter than needed, never too weak. (The
+// decode kernel k_mm5_q4k keeps its prefetch in registers the compiler does not
+// allocate at all.)
+__device__ __forceinline__ u4 load16(const void * base, uint32_t lane_off) {
+    return *(const u4 *)((const uint8_t *)base + lane_off);
+}
+__device__ __forceinline__ uint32_t lds_offset(const void * p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p;
+}
+
 template <int NT> struct XStage {
     // 1 KiB blocks: [kstep 8][hi/lo 2][tile NT] activations, then [tile NT] block sums
     static constexpr int X_BLOCKS = 8 * 2 * NT;
@@ -42,46 +67,43 @@ template <int NT> struct XStage {
     static constexpr int BYTES = BLOCKS * 1024;
 };
 
-// Per-lane source pointers of the activation staging, computed once per kernel:
-// wave w of the eight always stages token tile w % NT, and 8/NT waves share the
-// sixteen (k-step, hi/lo) blocks of a tile. The activations are stored in
-// operand order, so every load copies one contiguous 1 KiB block.
+// Activation staging of a workgroup: wave w of the eight always stages token
+// tile w % NT, and 8/NT waves share the sixteen (k-step, hi/lo) blocks of a
+// tile. The activations are stored in operand order, so every request copies
+// one contiguous 1 KiB block; the bases are wave-uniform, the lanes add lane * 16.
 template <int NT> struct StageSrc {
-    const __half * x;        // block (k-step 0, hi) of this wave's tile, at this lane
-    const __half * sum;      // block sums of super-block 0 of this wave's tile, at this lane
+    const __half * x;        // block (k-step 0, hi) of this wave's tile
+    const __half * sum;      // block sums of super-block 0 of this wave's tile
     int tile, slot;
+    uint32_t lane16;
+    uint32_t lds0;           // LDS address of the first staging buffer
 };
 
 template <int NT>
-__device__ __forceinline__ StageSrc<NT> stage_prepare(const MMArgs & a, int chunk, int lane, int wave) {
+__device__ __forceinline__ StageSrc<NT> stage_prepare(const MMArgs & a, int chunk, int lane, int wave, const uint8_t * smem) {
     static_assert(NT == 1 || NT == 2 || NT == 4, "token tiles per chunk");
     StageSrc<NT> s;
     s.tile = wave % NT;
     s.slot = wave / NT;
-    s.x = a.x + (size_t)chunk * act_chunk_halves(a.K) + s.tile * 512 + lane * 8;
-    s.sum = a.sums ? a.sums + (size_t)chunk * act_sum_chunk_halves(a.K) + s.tile * 512 + lane * 8 : nullptr;
+    s.x = a.x + (size_t)chunk * act_chunk_halves(a.K) + s.tile * 512;
+    s.sum = a.sums ? a.sums + (size_t)chunk * act_sum_chunk_halves(a.K) + s.tile * 512 : nullptr;
+    s.lane16 = lane * 16;
+    s.lds0 = lds_offset(smem);
     return s;
 }
 
-// Issues the direct-to-LDS loads of one super-block column of activations.
+// Requests one super-block column of activations into staging buffer `which`.
 template <int NT>
-__device__ __forceinline__ void stage_x(const StageSrc<NT> & s, int sb, uint8_t * buf, bool with_sums) {
+__device__ __forceinline__ void stage_x(const StageSrc<NT> & s, int sb, int which, bool with_sums) {
     constexpr int WAVES_PER_TILE = 8 / NT;
     constexpr int PER_WAVE = 16 / WAVES_PER_TILE;
+    const uint32_t buf = s.lds0 + which * XStage<NT>::BYTES;
 #pragma unroll
     for (int j = 0; j < PER_WAVE; ++j) {
         const int c = s.slot + WAVES_PER_TILE * j;      // (k-step, hi/lo) block of the super-block, wave-uniform
-        const __half * src = s.x + (size_t)(sb * 16 + c) * 2048;
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)src,
-                                         (void __attribute__((address_space(3))) *)(buf + (c * NT + s.tile) * 1024),
-                                         16, 0, 0);
+        lds_dma16(s.x + (size_t)(sb * 16 + c) * 2048, s.lane16, buf + (c * NT + s.tile) * 1024);
     }
-    if (with_sums && s.slot == 0) {
-        const __half * src = s.sum + (size_t)sb * 2048;
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)src,
-                                         (void __attribute__((address_space(3))) *)(buf + (XStage<NT>::X_BLOCKS + s.tile) * 1024),
-                                         16, 0, 0);
-    }
+    if (with_sums && s.slot == 0) lds_dma16(s.sum + (size_t)sb * 2048, s.lane16, buf + (XStage<NT>::X_BLOCKS + s.tile) * 1024);
 }
 
 __device__ __forceinline__ h8 lds_h8(const uint8_t * buf, int block, int lane) {
@@ -200,7 +222,7 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
     int rt[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) rt[r] = (rg * 4 + rw) * R + r;
-    const StageSrc<NT> stage = stage_prepare<NT>(a, blockIdx.y, lane, wave);
+    const StageSrc<NT> stage = stage_prepare<NT>(a, blockIdx.y, lane, wave, smem);
 
     f4 acc[R][NT];
 #pragma unroll
@@ -214,12 +236,13 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
     for (int r = 0; r < R; ++r) wbase[r] = a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 2304;
     // this wave's weights of one super-block: the row headers and its half of the payload
     struct WSet { u4 hdr[R]; u4 q[R]; };
-    auto load_w = [&](int sb, WSet & w) {
+    const uint32_t off_hdr = r16 * 16, off_q = 256 + kh * 1024 + lane * 16;
+    auto load_w = [&](int sb, WSet & w) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const uint8_t * tile = wbase[r] + (size_t)sb * 2304;
-            w.hdr[r] = *(const u4 *)(tile + r16 * 16);
-            w.q[r] = *(const u4 *)(tile + 256 + kh * 1024 + lane * 16);
+            w.hdr[r] = load16(tile, off_hdr);
+            w.q[r] = load16(tile, off_q);
         }
     };
     const h2 m1024 = {(_Float16)(-1024.0f), (_Float16)(-1024.0f)};
@@ -227,14 +250,13 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
 
     // One super-block: wait for its activations, start the loads of what comes
     // next (activations one super-block ahead, weights two), multiply.
-    auto body = [&](int sb, const WSet & w, WSet & fut) {
+    auto body = [&](int sb, WSet & w, WSet & fut) __attribute__((always_inline)) {
         uint8_t * cur = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
-        uint8_t * nxt = smem + ((sb - sb0 + 1) & 1) * XStage<NT>::BYTES;
         // All but the newest 2R loads (the weights one super-block ahead) have
         // landed: this super-block's activations and weights are in.
         __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R));
-        __syncthreads();   // ... for every wave, and nobody still reads nxt
-        if (sb + 1 < sb1 && !(a.debug & 1)) stage_x<NT>(stage, sb + 1, nxt, true);
+        __syncthreads();   // ... for every wave, and nobody still reads the other buffer
+        if (sb + 1 < sb1 && !(a.debug & 1)) stage_x<NT>(stage, sb + 1, (sb - sb0 + 1) & 1, true);
         load_w(min(sb + 2, sb1 - 1), fut);
         if (a.debug & 1) cur = smem;
 
@@ -320,7 +342,7 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
 
     if (sb0 < sb1) {
         WSet w0, w1, w2;
-        stage_x<NT>(stage, sb0, smem, true);
+        stage_x<NT>(stage, sb0, 0, true);
         load_w(sb0, w0);
         load_w(min(sb0 + 1, sb1 - 1), w1);
         for (int sb = sb0; sb < sb1; sb += 3) {
@@ -332,32 +354,6 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
         }
     }
     join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
-}
-
-// Memory instructions the kernel below counts itself. The compiler's own wait
-// insertion cannot tell which staging buffer an LDS read touches and, at the
-// loop head, merges the prologue's state into every iteration; both end in a
-// full s_waitcnt vmcnt(0) per super-block, which exposes the whole memory
-// latency of the weight prefetch. Issued from inline assembly the loads are
-// invisible to that pass, and the waits written in the kernel are the only ones.
-// base is wave-uniform; every lane adds its own byte offset.
-__device__ __forceinline__ void lds_dma16(const void * base, uint32_t lane_off, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(lane_off), "s"(base), "s"(lds_addr) : "memory");
-}
-// The result is valid only after a later s_waitcnt that names it (wait_for below).
-__device__ __forceinline__ u4 load16_async(const void * base, uint32_t lane_off) {
-    u4 r;
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r) : "v"(lane_off), "s"(base) : "memory");
-    return r;
-}
-__device__ __forceinline__ u4 load16_async_512(const void * base, uint32_t lane_off) {
-    u4 r;
-    asm volatile("global_load_dwordx4 %0, %1, %2 offset:512" : "=v"(r) : "v"(lane_off), "s"(base) : "memory");
-    return r;
-}
-__device__ __forceinline__ uint32_t lds_offset(const void * p) {
-    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p;
 }
 
 typedef float f16v __attribute__((ext_vector_type(16)));
@@ -383,7 +379,7 @@ __device__ __forceinline__ float fma3(float a, float b, float c) {
 // activations and the weight tiles keep the 16x16x32 operand order; only the
 // per-lane addresses differ.
 // acc[tb][i] is token 32 tb + 8 (i / 4) + 4 p + i % 4, row n32.
-__global__ __launch_bounds__(kThreads, 1) void k_mm5_q4k(MMArgs a) {
+__global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_num_vgpr(232))) void k_mm5_q4k(MMArgs a) {
     constexpr int NT = 4;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63;
@@ -413,18 +409,36 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm5_q4k(MMArgs a) {
     const uint8_t * wu = a.w + (size_t)tile0 * nsb * 2304;
     const uint32_t off_tile = (n32 >> 4) * (uint32_t)(tile1 - tile0) * nsb * 2304;
     const uint32_t off_hdr = off_tile + r16 * 16, off_q = off_tile + 256 + kh * 1024 + (p * 16 + r16) * 16;
+    // The two prefetched weight sets live in v[232:243] and v[244:255], above the
+    // registers the compiler may allocate (amdgpu_num_vgpr above): their loads are
+    // issued from inline assembly so that the compiler's wait insertion does not
+    // see them, and a register it knows nothing about cannot be copied, spilled
+    // or reused while its load is still in flight. `take` is the only way a
+    // value gets out: it waits until at most the newest set is pending and hands
+    // the other set over.
     struct WSet { u4 hdr; u4 q[2]; };
-    auto load_w = [&](int sb, WSet & w) __attribute__((always_inline)) {
+    auto load_w = [&](int sb, auto set) __attribute__((always_inline)) {
         const uint8_t * t = wu + (size_t)sb * 2304;
-        w.hdr = load16_async(t, off_hdr);
-        w.q[0] = load16_async(t, off_q);
-        w.q[1] = load16_async_512(t, off_q);
+        const uint32_t oh = off_hdr, oq = off_q;      // named here: an asm operand does not capture in a generic lambda
+        if (decltype(set)::value == 0) {
+            asm volatile("global_load_dwordx4 v[232:235], %0, %2\n\tglobal_load_dwordx4 v[236:239], %1, %2\n\t"
+                         "global_load_dwordx4 v[240:243], %1, %2 offset:512"
+                         :: "v"(oh), "v"(oq), "s"(t)
+                         : "memory", "v232", "v233", "v234", "v235", "v236", "v237", "v238", "v239", "v240", "v241", "v242", "v243");
+        } else {
+            asm volatile("global_load_dwordx4 v[244:247], %0, %2\n\tglobal_load_dwordx4 v[248:251], %1, %2\n\t"
+                         "global_load_dwordx4 v[252:255], %1, %2 offset:512"
+                         :: "v"(oh), "v"(oq), "s"(t)
+                         : "memory", "v244", "v245", "v246", "v247", "v248", "v249", "v250", "v251", "v252", "v253", "v254", "v255");
+        }
     };
-    // at most n younger memory instructions are still on their way; w is valid from here on
-    auto wait_for = [&](WSet & w, auto n) __attribute__((always_inline)) {
-        static_assert(decltype(n)::value == 0 || decltype(n)::value == 3, "");
-        if (decltype(n)::value == 3) asm volatile("s_waitcnt vmcnt(3)" : "+v"(w.hdr), "+v"(w.q[0]), "+v"(w.q[1]) :: "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" : "+v"(w.hdr), "+v"(w.q[0]), "+v"(w.q[1]) :: "memory");
+    auto take = [&](auto set) __attribute__((always_inline)) {
+        WSet w;
+        if (decltype(set)::value == 0)
+            asm volatile("s_waitcnt vmcnt(3)" : "={v[232:235]}"(w.hdr), "={v[236:239]}"(w.q[0]), "={v[240:243]}"(w.q[1]) :: "memory");
+        else
+            asm volatile("s_waitcnt vmcnt(3)" : "={v[244:247]}"(w.hdr), "={v[248:251]}"(w.q[0]), "={v[252:255]}"(w.q[1]) :: "memory");
+        return w;
     };
     const h2 m1024 = {(_Float16)(-1024.0f), (_Float16)(-1024.0f)};
     const uint32_t magic1024 = 0x64006400u, magic64 = 0x54005400u;
@@ -450,11 +464,11 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm5_q4k(MMArgs a) {
 
     // q: this super-block's products (sc e x), scaled by the row's d while the
     // next super-block multiplies; pq, pd: the products and d left by the one before
-    auto body = [&](int sb, WSet & w, f16v (&q)[2], float & d, const f16v (&pq)[2], float pd) __attribute__((always_inline)) {
+    auto body = [&](int sb, auto set, f16v (&q)[2], float & d, const f16v (&pq)[2], float pd) __attribute__((always_inline)) {
         const uint8_t * cur = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
-        // Only the weights requested at the end of the last super-block may
-        // still be on their way: this one's weights and activations are in.
-        wait_for(w, std::integral_constant<int, 3>());
+        // All but the newest three loads (the other weight set) have landed:
+        // this super-block's weights and this wave's activation requests.
+        const WSet w = take(set);
         __syncthreads();   // ... for every wave, and nobody still reads the other buffer
         const uint8_t * xk = cur + lane_x;
         // fragments of step s = 2 j + h: [hi, lo][token block]
@@ -544,7 +558,7 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm5_q4k(MMArgs a) {
 #pragma unroll
             for (int tb = 0; tb < 2; ++tb)
                 q[tb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[s & 1][1][tb], B[s & 1], q[tb], 0, 0, 0);
-            if (s == 7) load_w(min(sb + 2, sb1 - 1), w);
+            if (s == 7) load_w(min(sb + 2, sb1 - 1), set);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -556,21 +570,23 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm5_q4k(MMArgs a) {
     };
 
     if (sb0 < sb1) {
-        WSet w0, w1;
         f16v qa[2], qb[2];
         float da = 0.0f, db = 0.0f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) { qb[0][i] = 0.0f; qb[1][i] = 0.0f; }
+        const std::integral_constant<int, 0> set0;
+        const std::integral_constant<int, 1> set1;
         for (int i = 0; i <= 8; ++i) request(sb0, i);
-        load_w(sb0, w0);
-        load_w(min(sb0 + 1, sb1 - 1), w1);
+        load_w(sb0, set0);
+        load_w(min(sb0 + 1, sb1 - 1), set1);
         for (int sb = sb0; sb < sb1; sb += 2) {
-            body(sb, w0, qa, da, qb, db);
+            body(sb, set0, qa, da, qb, db);
             if (sb + 1 >= sb1) { scale_last(qa, da); break; }
-            body(sb + 1, w1, qb, db, qa, da);
+            body(sb + 1, set1, qb, db, qa, da);
             if (sb + 2 >= sb1) scale_last(qb, db);
         }
-        wait_for(w0, std::integral_constant<int, 0>());      // the last, repeated requests have landed before the buffers are reused
+        // the last, repeated requests have landed before the buffers are reused, and no load is in flight
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     // the min term of token block kh joins its accumulator
 #pragma unroll
@@ -604,7 +620,7 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
     int rt[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) rt[r] = (rg * 4 + rw) * R + r;
-    const StageSrc<NT> stage = stage_prepare<NT>(a, blockIdx.y, lane, wave);
+    const StageSrc<NT> stage = stage_prepare<NT>(a, blockIdx.y, lane, wave, smem);
     f4 acc[R][NT];
 #pragma unroll
     for (int r = 0; r < R; ++r)
@@ -615,24 +631,24 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
 #pragma unroll
     for (int r = 0; r < R; ++r) wbase[r] = a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 4352;
     struct WSet { u4 hdr[R]; u4 q[R][2]; };
-    auto load_w = [&](int sb, WSet & w) {
+    const uint32_t off_hdr = r16 * 16, off_q = 256 + 2 * kh * 1024 + lane * 16;
+    auto load_w = [&](int sb, WSet & w) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const uint8_t * tile = wbase[r] + (size_t)sb * 4352;
-            w.hdr[r] = *(const u4 *)(tile + r16 * 16);
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-                w.q[r][j] = *(const u4 *)(tile + 256 + (2 * kh + j) * 1024 + lane * 16);
+            w.hdr[r] = load16(tile, off_hdr);
+            w.q[r][0] = load16(tile, off_q);
+            w.q[r][1] = load16(tile, off_q + 1024);
         }
     };
     const h2 bias1152 = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
 
-    auto body = [&](int sb, const WSet & w, WSet & fut) {
+    auto body = [&](int sb, WSet & w, WSet & fut) __attribute__((always_inline)) {
         uint8_t * cur = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
-        uint8_t * nxt = smem + ((sb - sb0 + 1) & 1) * XStage<NT>::BYTES;
+        // all but the newest 3R loads (the weights one super-block ahead) have landed
         __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * R));
         __syncthreads();
-        if (sb + 1 < sb1) stage_x<NT>(stage, sb + 1, nxt, false);
+        if (sb + 1 < sb1) stage_x<NT>(stage, sb + 1, (sb - sb0 + 1) & 1, false);
         load_w(min(sb + 2, sb1 - 1), fut);
         const uint8_t * xk = cur + kh * (8 * NT * 1024);
 #pragma unroll
@@ -668,7 +684,7 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
 
     if (sb0 < sb1) {
         WSet w0, w1, w2;
-        stage_x<NT>(stage, sb0, smem, false);
+        stage_x<NT>(stage, sb0, 0, false);
         load_w(sb0, w0);
         load_w(min(sb0 + 1, sb1 - 1), w1);
         for (int sb = sb0; sb < sb1; sb += 3) {

@@ -33,7 +33,7 @@ def _ref(dense, x):
 
 @pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0])
 @pytest.mark.parametrize("n,k,T", [(16, 256, 1), (48, 512, 7), (64, 1024, 16), (256, 4096, 33),
-                                   (4096, 2048, 64), (160, 768, 100), (2064, 256, 3)])
+                                   (4096, 2048, 64), (160, 768, 100), (2064, 256, 3), (96, 1024, 24), (512, 4096, 48)])
 def test_tile_matmul_matches_decoded_blocks(t, n, k, T):
     print("case", t, n, k, T, flush=True)
     raw, dense = _weights(t, n, k, seed=n + k + T)

@@ -210,6 +210,65 @@ int retro_engine_seq_pos(
 int retro_engine_memory(retro_engine * engine, retro_engine_memory_info * out);
 int retro_engine_request_free(retro_engine * engine, int32_t request);
 
+/* ---- batched generators on top of the step: ref h:1238-1242, 1123-1131,
+ * 2511-2534, 2672-2674 (contract text h:1844-1879) --------------------------
+ * The whole generation loop inside one call, over the same step and the same
+ * sampling oracle (mt19937 seeded once per sequence), so a caller-side loop of
+ * retro_engine_step calls composed in the canonical order reproduces them bit
+ * for bit (h:2696-2698).
+ * Outputs are row-major with a stride of n_out_max. A row stops at
+ * max_new_tokens, at an end-of-generation token (included), or when its
+ * sequence context is full. out_logprobs may be NULL; otherwise it receives the
+ * temperature-1 policy log-probability of every emitted token. out_n_tokens
+ * holds n_sequences counts. out_forced may be NULL; otherwise all zeros (no
+ * reasoning budget in this build). Returns 0, or -1 with retro_last_error(). */
+
+/* ref h:1238-1242 */
+typedef struct retro_generation_sequence {
+    const int32_t * prompt_tokens;
+    size_t          n_prompt;
+    retro_sampling_params sampling;
+} retro_generation_sequence;
+
+/* ref h:1123-1131: lifetime counters of the continuous generator's slot-level
+ * prefix reuse; a caller attributes one call by differencing two snapshots. */
+typedef struct retro_generation_stats {
+    uint64_t calls;
+    uint64_t sequences;
+    uint64_t prompt_tokens;      /* what the callers asked to be resident before sampling */
+    uint64_t prefilled_tokens;   /* what was decoded to get there */
+    uint64_t reused_tokens;
+    uint64_t hits;
+    uint64_t evictions;
+} retro_generation_stats;
+
+/* ref h:2514-2524 (retro_gen_core.cpp:1696-1876): n_sequences completions of
+ * one prompt. The prompt is decoded once, its KV copied to one slot per member
+ * (slot i for member i), and all live members advance in one step per token.
+ * Starts from, and leaves, an empty KV. */
+int retro_engine_generate_batch(
+    retro_engine * engine, const int32_t * prompt_tokens, size_t n_prompt,
+    const retro_sampling_params * sampling, size_t n_sequences,
+    int32_t * out_tokens, float * out_logprobs, size_t n_out_max, size_t * out_n_tokens,
+    uint8_t * out_forced);
+
+/* ref h:2526-2534 (retro_gen_core.cpp:317-707, 1878-2049): one completion per
+ * input, heterogeneous prompts. Every launch is built in the canonical order
+ * of the contents (prompt length, prompt tokens, seed, max_new_tokens,
+ * temperature, top_p), equal prompts are prefilled once and copied, and the
+ * slots keep what they decoded between calls: a later call whose prompt
+ * strictly extends a slot's resident tokens decodes only the extension.
+ * RETRO_GENERATION_PREFIX_CACHE=0 (or "false") in the environment turns the
+ * reuse off: every call then starts and ends with an empty KV. A step or a raw
+ * sequence operation through this ABI forgets what the slots hold. */
+int retro_engine_generate_continuous_batch(
+    retro_engine * engine, const retro_generation_sequence * sequences, size_t n_sequences,
+    int32_t * out_tokens, float * out_logprobs, size_t n_out_max, size_t * out_n_tokens,
+    uint8_t * out_forced);
+
+/* ref h:2672-2674 */
+int retro_engine_generation_stats(retro_engine * engine, retro_generation_stats * out_stats);
+
 /* ---- introspection: ref h:2775, 2799, 2803, 2808, 2550-2561, 2612 -------- */
 int retro_engine_kv_unified(retro_engine * engine, bool * out_unified);
 int retro_engine_weights_version(retro_engine * engine, uint64_t * out_version);

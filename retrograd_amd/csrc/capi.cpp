@@ -176,6 +176,7 @@ int retro_engine_step(retro_engine * engine, const retro_step_row * rows, size_t
             set_error("step rows and output rows are required");
             return -3;
         }
+        e->forget_generation_bookkeeping();
         return e->step(nullptr, rows, n_rows, nullptr, out_rows, out_top_ids, out_top_logprobs, n_top_stride);
     });
 }
@@ -190,6 +191,7 @@ int retro_engine_step_v2(retro_engine * engine, const retro_step_row_v2 * rows, 
             set_error("step rows and output rows are required");
             return -3;
         }
+        e->forget_generation_bookkeeping();
         return e->step(rows, nullptr, n_rows, out_rows, nullptr, out_top_ids, out_top_logprobs, n_top_stride);
     });
 }
@@ -198,6 +200,7 @@ int retro_engine_seq_rm(retro_engine * engine, int32_t slot, int32_t p0, int32_t
     return boundary([&]() -> int {
         Engine * e = checked(engine);
         if (!e) return -1;
+        e->forget_generation_bookkeeping();
         return e->seq_rm(slot, p0, p1) ? 0 : -1;
     });
 }
@@ -206,6 +209,7 @@ int retro_engine_seq_cp(retro_engine * engine, int32_t src, int32_t dst, int32_t
     return boundary([&]() -> int {
         Engine * e = checked(engine);
         if (!e) return -1;
+        e->forget_generation_bookkeeping();
         return e->seq_cp(src, dst, p0, p1) ? 0 : -1;
     });
 }
@@ -224,6 +228,7 @@ int retro_engine_seq_load(retro_engine * engine, int32_t slot, uint32_t flags, c
     return boundary([&]() -> int {
         Engine * e = checked(engine);
         if (!e) return -1;
+        e->forget_generation_bookkeeping();
         return e->seq_load(slot, flags, buffer, n_bytes, out_n_read);
     });
 }
@@ -249,6 +254,40 @@ int retro_engine_request_free(retro_engine * engine, int32_t request) {
         Engine * e = checked(engine);
         if (!e) return -1;
         e->request_free(request);
+        return 0;
+    });
+}
+
+int retro_engine_generate_batch(retro_engine * engine, const int32_t * prompt_tokens, size_t n_prompt,
+                                const retro_sampling_params * sampling, size_t n_sequences, int32_t * out_tokens,
+                                float * out_logprobs, size_t n_out_max, size_t * out_n_tokens, uint8_t * out_forced) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->generate_batch(prompt_tokens, n_prompt, sampling, n_sequences, out_tokens, out_logprobs, n_out_max,
+                                 out_n_tokens, out_forced);
+    });
+}
+
+int retro_engine_generate_continuous_batch(retro_engine * engine, const retro_generation_sequence * sequences,
+                                           size_t n_sequences, int32_t * out_tokens, float * out_logprobs,
+                                           size_t n_out_max, size_t * out_n_tokens, uint8_t * out_forced) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->generate_continuous_batch(sequences, n_sequences, out_tokens, out_logprobs, n_out_max, out_n_tokens,
+                                            out_forced);
+    });
+}
+
+int retro_engine_generation_stats(retro_engine * engine, retro_generation_stats * out_stats) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e || !out_stats) {
+            if (e) set_error("out_stats is required");
+            return -1;
+        }
+        *out_stats = e->generation_stats();
         return 0;
     });
 }

@@ -107,6 +107,20 @@ public:
     int seq_pos(int32_t slot, int32_t * out_min, int32_t * out_max);
     int memory(retro_engine_memory_info * out);
     void request_free(int32_t request) { requests_.erase(request); }
+
+    // Batched generators over the step (generate.cpp; reference retro_gen_core.cpp:317-707, 1696-2049).
+    int generate_batch(const int32_t * prompt_tokens, size_t n_prompt, const retro_sampling_params * sampling,
+                       size_t n_sequences, int32_t * out_tokens, float * out_logprobs, size_t n_out_max,
+                       size_t * out_n_tokens, uint8_t * out_forced);
+    int generate_continuous_batch(const retro_generation_sequence * sequences, size_t n_sequences,
+                                  int32_t * out_tokens, float * out_logprobs, size_t n_out_max,
+                                  size_t * out_n_tokens, uint8_t * out_forced);
+    const retro_generation_stats & generation_stats() const { return gen_cache_.stats; }
+    // A step or a raw sequence operation issued by a caller mutates the KV outside the
+    // continuous generator's protocol: what its slots hold is forgotten (retro_gen_core.cpp:2569,
+    // 2795, 2813, 2875), the KV itself stays.
+    void forget_generation_bookkeeping() { gen_cache_.forget(); }
+    void clear_generation_memory();
     // Per-row LoRA adapters (reference retro_engine.cpp:872-960): ids start at 1
     // and are never reused; loading leaves the resident KV alone.
     int adapter_load(const std::string & path, float scale, int32_t * out_id);
@@ -243,6 +257,24 @@ private:
     }
 
     std::map<int32_t, RequestState> requests_;
+
+    // What the continuous generator's slots hold between calls (reference retro_runtime.hpp:244-263).
+    struct GenCache {
+        std::vector<std::vector<int32_t>> slots;   // resident tokens per slot
+        std::vector<uint64_t> used_at;             // last call that extended the slot
+        uint64_t clock = 0;
+        retro_generation_stats stats {};
+        void forget();
+    };
+    GenCache gen_cache_;
+    bool gen_validate_sampling(const retro_sampling_params & s);
+    bool gen_validate_tokens(const int32_t * tokens, size_t n);
+    bool gen_prefill(int32_t slot, const int32_t * tokens, size_t p0, size_t p1);
+    int gen_decode_loop(const std::vector<size_t> & order, const std::vector<int32_t> & slot_of,
+                        const std::vector<size_t> & n_prompt_of, const std::vector<retro_sampling_params> & sampling,
+                        const std::vector<size_t> & limits, std::vector<retro_step_out_row> produced,
+                        int32_t * out_tokens, float * out_logprobs, size_t n_out_max, size_t * out_n_tokens,
+                        uint8_t * out_forced);
     sampling::FullScratch scratch_;
 };
 

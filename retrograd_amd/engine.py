@@ -54,6 +54,15 @@ class CSamplingParams(C.Structure):
                 ("max_new_tokens", C.c_uint32), ("seed", C.c_uint32)]
 
 
+class CGenerationSequence(C.Structure):
+    _fields_ = [("prompt_tokens", C.POINTER(C.c_int32)), ("n_prompt", C.c_size_t), ("sampling", CSamplingParams)]
+
+
+class CGenerationStats(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("calls", "sequences", "prompt_tokens", "prefilled_tokens", "reused_tokens",
+                                          "hits", "evictions")]
+
+
 class CStepRow(C.Structure):
     _fields_ = [("struct_size", C.c_uint32), ("request", C.c_int32), ("slot", C.c_int32),
                 ("tokens", C.POINTER(C.c_int32)), ("n", C.c_uint32), ("pos0", C.c_int32),
@@ -111,6 +120,7 @@ STEP_SYMBOLS = [
     "retro_engine_new", "retro_engine_new_checked", "retro_engine_free", "retro_engine_step",
     "retro_engine_step_v2", "retro_engine_seq_rm", "retro_engine_seq_cp", "retro_engine_seq_save",
     "retro_engine_seq_load", "retro_engine_seq_pos", "retro_engine_memory", "retro_engine_request_free",
+    "retro_engine_generate_batch", "retro_engine_generate_continuous_batch", "retro_engine_generation_stats",
     "retro_engine_kv_unified", "retro_engine_weights_version", "retro_engine_model_fingerprint",
     "retro_engine_is_hybrid", "retro_engine_eos_token", "retro_engine_vocab_size", "retro_engine_is_eog_token",
     "retro_engine_context_size", "retro_engine_detokenize", "retro_engine_graphs_reused",
@@ -151,6 +161,11 @@ def load_library() -> C.CDLL:
                                       _i32p, _f32p, C.c_size_t]
     lib.retro_engine_step_v2.argtypes = [C.c_void_p, C.POINTER(CStepRowV2), C.c_size_t, C.POINTER(CStepOutRowV2),
                                          _i32p, _f32p, C.c_size_t]
+    lib.retro_engine_generate_batch.argtypes = [C.c_void_p, _i32p, C.c_size_t, C.POINTER(CSamplingParams), C.c_size_t,
+                                                _i32p, _f32p, C.c_size_t, C.POINTER(C.c_size_t), _u8p]
+    lib.retro_engine_generate_continuous_batch.argtypes = [C.c_void_p, C.POINTER(CGenerationSequence), C.c_size_t,
+                                                           _i32p, _f32p, C.c_size_t, C.POINTER(C.c_size_t), _u8p]
+    lib.retro_engine_generation_stats.argtypes = [C.c_void_p, C.POINTER(CGenerationStats)]
     lib.retro_engine_seq_rm.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32]
     lib.retro_engine_seq_cp.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_int32]
     lib.retro_engine_seq_save.argtypes = [C.c_void_p, C.c_int32, C.c_uint32, _u8p, C.c_size_t, C.POINTER(C.c_size_t)]
@@ -481,6 +496,65 @@ class Engine:
             _raise(status)
         return ([StepOutRow(o.token, o.logprob, bool(o.forced), bool(o.sampled), o.n_top) for o in outs],
                 ids.reshape(n, -1), lps.reshape(n, -1))
+
+    # -- batched generators -----------------------------------------------------------
+    @staticmethod
+    def _sampling_v1(p) -> CSamplingParams:
+        """p: (temperature, top_p, max_new_tokens, seed)."""
+        c = CSamplingParams()
+        c.temperature, c.top_p, c.max_new_tokens, c.seed = p
+        return c
+
+    def _collect(self, n, n_out_max, toks, lps, counts, forced):
+        return [(toks[i, :counts[i]].tolist(), lps[i, :counts[i]].copy(), forced[i, :counts[i]].astype(bool).tolist())
+                for i in range(n)]
+
+    def generate_batch(self, prompt: Sequence[int], sampling: Sequence[tuple], n_out_max: int | None = None):
+        """retro_engine_generate_batch: one completion per entry of `sampling`
+        ((temperature, top_p, max_new_tokens, seed) each) of the one prompt.
+        Returns [(tokens, logprobs, forced)] per member."""
+        n = len(sampling)
+        n_out_max = n_out_max or max(p[2] for p in sampling)
+        prompt_arr = np.ascontiguousarray(prompt, dtype=np.int32)
+        params = (CSamplingParams * n)(*[self._sampling_v1(p) for p in sampling])
+        toks = np.zeros((n, n_out_max), np.int32)
+        lps = np.zeros((n, n_out_max), np.float32)
+        forced = np.zeros((n, n_out_max), np.uint8)
+        counts = (C.c_size_t * n)()
+        status = self._lib.retro_engine_generate_batch(self._h, prompt_arr.ctypes.data_as(_i32p), prompt_arr.size, params, n,
+                                                       toks.ctypes.data_as(_i32p), lps.ctypes.data_as(_f32p), n_out_max,
+                                                       counts, forced.ctypes.data_as(_u8p))
+        if status != 0:
+            _raise(status)
+        return self._collect(n, n_out_max, toks, lps, list(counts), forced)
+
+    def generate_continuous(self, sequences: Sequence[tuple], n_out_max: int | None = None):
+        """retro_engine_generate_continuous_batch over (prompt, (temperature, top_p,
+        max_new_tokens, seed)) pairs. Returns [(tokens, logprobs, forced)] in input order."""
+        n = len(sequences)
+        n_out_max = n_out_max or max(p[2] for _, p in sequences)
+        keep = [np.ascontiguousarray(prompt, dtype=np.int32) for prompt, _ in sequences]
+        ffi = (CGenerationSequence * n)()
+        for i, (_, p) in enumerate(sequences):
+            ffi[i].prompt_tokens = keep[i].ctypes.data_as(_i32p)
+            ffi[i].n_prompt = keep[i].size
+            ffi[i].sampling = self._sampling_v1(p)
+        toks = np.zeros((n, n_out_max), np.int32)
+        lps = np.zeros((n, n_out_max), np.float32)
+        forced = np.zeros((n, n_out_max), np.uint8)
+        counts = (C.c_size_t * n)()
+        status = self._lib.retro_engine_generate_continuous_batch(self._h, ffi, n, toks.ctypes.data_as(_i32p),
+                                                                  lps.ctypes.data_as(_f32p), n_out_max, counts,
+                                                                  forced.ctypes.data_as(_u8p))
+        if status != 0:
+            _raise(status)
+        return self._collect(n, n_out_max, toks, lps, list(counts), forced)
+
+    def generation_stats(self) -> dict:
+        st = CGenerationStats()
+        if self._lib.retro_engine_generation_stats(self._h, C.byref(st)) != 0:
+            _raise(-1)
+        return {name: int(getattr(st, name)) for name, _ in CGenerationStats._fields_}
 
     # -- sequence operations -----------------------------------------------------------
     def seq_rm(self, slot: int, p0: int = -1, p1: int = -1) -> None:

@@ -15,10 +15,13 @@
 extern "C" {
 #endif
 
-/* y[t][n] (=|+=) sum_k W[n][k] * f16(x[t][k]) (+ bias[n]) with W given as
- * n_rows raw GGUF rows of `type`. use_tiles = 0 runs the generic kernel, 1 the
- * register-only MFMA tile kernel, 2 the LDS-staged MFMA tile kernel (tiles need
- * K % 256 == 0, n_rows % 16 == 0, Q4_K or Q8_0).
+/* y[t][n] (=|+=) sum_k W[n][k] * a[t][k] (+ bias[n]) with W given as n_rows raw
+ * GGUF rows of `type`. The low byte of use_tiles picks the kernel: 0 the generic
+ * one, 1 the register-only MFMA tile kernel, 2 the LDS-staged MFMA tile kernel
+ * (tiles need K % 256 == 0, n_rows % 16 == 0, Q4_K or Q8_0). a is x (carried as
+ * f16 hi/lo pairs) or, with bit 8 (0x100) of use_tiles set, x as ggml's CPU
+ * matmul converts it for this weight type: Q8_K codes times their scale for
+ * Q4_K, Q8_0 ones for Q8_0 and MXFP4, f16 / bf16 rounding for F16 / BF16.
  * y is [n_tokens][n_rows] and is read first when accumulate is set. */
 int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x,
                         int32_t n_tokens, int32_t use_tiles, const float * bias, int32_t accumulate, float * y);

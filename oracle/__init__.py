@@ -57,6 +57,10 @@ def _declare(l: C.CDLL) -> None:
     l.orc_float_to_half.restype = None
     l.orc_double_to_half.argtypes = [_f64p, C.c_size_t, _u16p]
     l.orc_double_to_half.restype = None
+    l.orc_activation_row.argtypes = [C.c_uint32, _f32p, C.c_size_t, _f32p]
+    l.orc_matmul.argtypes = [C.c_uint32, _u8p, C.c_size_t, C.c_size_t, _f32p, C.c_int, _f32p]
+    l.orc_set_exact_activations.argtypes = [C.c_int]
+    l.orc_set_exact_activations.restype = None
     l.orc_e8m0_half.argtypes = [C.c_uint8]
     l.orc_e8m0_half.restype = C.c_float
     l.orc_pack_rows.argtypes = [C.c_size_t, _i32p, _i32p, _u32p, _u8p, _i32p,
@@ -70,6 +74,8 @@ def _declare(l: C.CDLL) -> None:
     l.orc_adapter_load.argtypes = [C.c_void_p, C.c_char_p, C.c_float, _i32p]
     l.orc_ctx_new.argtypes = [C.c_void_p, C.c_int]
     l.orc_ctx_new.restype = C.c_void_p
+    l.orc_ctx_set_exact.argtypes = [C.c_void_p, C.c_int]
+    l.orc_ctx_set_exact.restype = None
     l.orc_ctx_free.argtypes = [C.c_void_p]
     l.orc_ctx_free.restype = None
     l.orc_ctx_step.argtypes = [C.c_void_p, C.c_int, _i32p, _i32p, _i32p, _i32p, _u8p, _f32p]
@@ -117,6 +123,28 @@ def decode_row(ggml_type: int, raw, n: int) -> np.ndarray:
     out = np.empty(n, dtype=np.float32)
     _check(lib().orc_decode_row(ggml_type, _ptr(src, _u8p), n, _ptr(out, _f32p)))
     return out
+
+
+def activation_row(weight_type: int, x: np.ndarray) -> np.ndarray:
+    """The activations a weight of `weight_type` is multiplied with on ggml's CPU path."""
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    out = np.empty_like(x)
+    _check(lib().orc_activation_row(weight_type, _ptr(x, _f32p), x.size, _ptr(out, _f32p)))
+    return out
+
+
+def matmul(ggml_type: int, raw, n_rows: int, k: int, x: np.ndarray) -> np.ndarray:
+    """x [T, k] times the n_rows raw rows, activations converted as ggml's CPU path does."""
+    src = np.ascontiguousarray(raw, dtype=np.uint8)
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, k)
+    y = np.empty((x.shape[0], n_rows), np.float32)
+    _check(lib().orc_matmul(ggml_type, _ptr(src, _u8p), k, n_rows, _ptr(x, _f32p), x.shape[0], _ptr(y, _f32p)))
+    return y
+
+
+def set_exact_activations(on: bool) -> None:
+    """Matmuls of the forward pass take f32 activations as they are (measurements only)."""
+    lib().orc_set_exact_activations(1 if on else 0)
 
 
 def row_bytes(ggml_type: int, n: int) -> int:
@@ -226,13 +254,22 @@ class Model:
 
 
 class Context:
-    """Per-slot dense f16 KV and one decode per step() over a packed batch."""
+    """Per-slot dense f16 KV and one decode per step() over a packed batch.
 
-    def __init__(self, model: Model, n_seq_max: int) -> None:
+    activations: "exact" multiplies every weight with the f32 activations as they
+    are (the product's default arithmetic, on which the logit tolerances are
+    demonstrated); "ggml" converts them first as ggml's CPU matmul does (Q8_K /
+    Q8_0 codes, f16 / bf16 rounding: the reference's CPU arithmetic, which the
+    product runs under RETRO_ACTIVATIONS=ggml)."""
+
+    def __init__(self, model: Model, n_seq_max: int, activations: str = "exact") -> None:
+        if activations not in ("exact", "ggml"):
+            raise ValueError("activations must be 'exact' or 'ggml'")
         self.model = model
         self._h = lib().orc_ctx_new(model._h, n_seq_max)
         if not self._h:
             raise OracleError(lib().orc_last_error().decode())
+        lib().orc_ctx_set_exact(self._h, 1 if activations == "exact" else 0)
 
     def step(self, token, pos, slot, want, adapter_of=None) -> np.ndarray:
         token = np.ascontiguousarray(token, np.int32)

@@ -56,6 +56,23 @@ void orc_double_to_half(const double * f, size_t n, uint16_t * out) {
 }
 float orc_e8m0_half(uint8_t x) { return e8m0_half(x); }
 
+// The activations of one row as ggml's CPU matmul sees them for a weight of `wtype`.
+int orc_activation_row(uint32_t wtype, const float * x, size_t n, float * out) {
+    return guard([&] { ggml_activation_row(wtype, x, n, out); return 0; });
+}
+// y[T][N] = W x^T with W (N rows of K) in raw block format `type`, activations converted as above.
+int orc_matmul(uint32_t type, const uint8_t * raw, size_t K, size_t N, const float * x, int T, float * y) {
+    return guard([&] {
+        gguf_tensor w;
+        w.type = type;
+        w.ne = {K, N};
+        w.data = raw;
+        matmul(w, x, T, y);
+        return 0;
+    });
+}
+void orc_set_exact_activations(int on) { exact_activations() = on != 0; }
+
 // ---- packing ---------------------------------------------------------------
 // The flat batch of one step (retro_gen_core.cpp:2578-2603): rows appended in
 // order, flat index = running token count, pos = pos0 + i, seq id = slot, the
@@ -129,6 +146,7 @@ void * orc_ctx_new(void * m, int n_seq_max) {
     return out;
 }
 void orc_ctx_free(void * c) { delete (context *)c; }
+void orc_ctx_set_exact(void * c, int on) { ((context *)c)->exact = on != 0; }
 
 // adapter_of may be NULL (base model for every token); entries <= 0 mean base.
 int orc_ctx_step(void * c, int n_tokens, const int32_t * tok, const int32_t * pos, const int32_t * slot,

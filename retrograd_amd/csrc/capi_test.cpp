@@ -40,7 +40,7 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
         ok(hipMemcpy(d_raw.ptr, raw, bytes, hipMemcpyHostToDevice), "upload weights");
         rk::Weight w;
         w.type = type; w.K = (int)k; w.N = (int)n_rows; w.bytes = bytes;
-        if (use_tiles) {
+        if (use_tiles & 0xff) {
             if (!rk::can_pack(type, k, n_rows)) throw std::runtime_error("this shape or type has no tile layout");
             d_packed.alloc(bytes);
             rk::repack(nullptr, type, d_raw.as<uint8_t>(), d_packed.as<uint8_t>(), (int)k, (int)n_rows);
@@ -54,7 +54,18 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
         d_sums.alloc(rk::act_sum_halves(n_tokens, (int)k) * 2);
         ok(hipMemset(d_xh.ptr, 0, d_xh.bytes), "clear activations");
         ok(hipMemset(d_sums.ptr, 0, d_sums.bytes), "clear block sums");
-        rk::Act act{d_xh.as<__half>(), k % 32 == 0 ? d_sums.as<__half>() : nullptr, (int)k};
+        // use_tiles bit 8: ggml's arithmetic - the rows are converted (quantised types) or rounded (F16 / BF16)
+        // before the product; otherwise the f32 values are multiplied
+        const bool faithful = (use_tiles & 0x100) != 0;
+        use_tiles &= 0xff;
+        rk::Act act;
+        act.K = (int)k;
+        act.faithful = faithful ? 1 : 0;
+        if (!faithful || rk::act_quant_of(type) == rk::AQ_NONE) {
+            act.x = d_xh.as<__half>(); act.sums = k % 32 == 0 ? d_sums.as<__half>() : nullptr;
+        } else {
+            act.qx = d_xh.as<__half>(); act.qsums = d_sums.as<__half>(); act.quant = rk::act_quant_of(type);
+        }
         rk::to_act(nullptr, d_x.as<float>(), n_tokens, (int)k, act);
         d_y.alloc((size_t)n_tokens * n_rows * 4);
         ok(hipMemcpy(d_y.ptr, y, d_y.bytes, hipMemcpyHostToDevice), "upload outputs");
@@ -124,7 +135,9 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
         ok(hipMemset(d_ws.ptr, 0, d_ws.bytes), "fill");
         rk::Weight w;
         w.type = type; w.K = (int)k; w.N = (int)n_rows; w.bytes = bytes; w.packed = d_w.as<uint8_t>();
-        rk::Act act{d_xh.as<__half>(), d_sums.as<__half>(), (int)k};
+        rk::Act act;
+        act.K = (int)k;
+        act.x = act.qx = d_xh.as<__half>(); act.sums = act.qsums = d_sums.as<__half>(); act.quant = rk::act_quant_of(type);
         rk::g_mm_debug = debug;
         rk::g_mm_force_ksplit = force_ksplit;
         hipEvent_t e0, e1;

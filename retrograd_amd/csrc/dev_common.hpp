@@ -76,10 +76,56 @@ __device__ __forceinline__ Q4KScales q4k_scales(const u4 & hdr) {
     return s;
 }
 
-// Eight consecutive activations per lane (k a multiple of 8): hi/lo as two
-// 16-byte stores; the four lanes that own one 32-wide block add their sums
-// with two xor-shuffles.
-__device__ __forceinline__ void store_act8(const float (&v)[8], const Act & out, int tok, int k, int lane_in_block) {
+// The conversion ggml's CPU matmul applies to an activation row before the dot
+// product, on eight consecutive values per lane. The lanes that share a block
+// (4 for the 32-wide Q8_0 blocks, 32 for the 256-wide Q8_K blocks) must be
+// consecutive, aligned to the group size, hold consecutive pieces of one row
+// and all be here. Returns the values the codes stand for, scale times code.
+//   Q8_0: d = amax / 127, code = roundf(v / d) with the unrounded d (half away
+//         from zero), value = f16(d) * code.
+//   Q8_K: `max` = the first value of largest magnitude, iscale = -127 / max,
+//         code = min(127, rint(iscale * v)) (half to even), value = code / iscale.
+__device__ __forceinline__ void requantise8(float (&v)[8], int quant) {
+    float amax = 0.0f, first = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float ax = fabsf(v[i]);
+        if (ax > amax) { amax = ax; first = v[i]; }
+    }
+    if (quant == AQ_Q8_0) {
+        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+        const float d = __fdiv_rn(amax, 127.0f);
+        const float id = d != 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
+        const float dh = (float)(_Float16)d;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = __fmul_rn(dh, roundf(__fmul_rn(v[i], id)));
+        return;
+    }
+    float gmax = amax;
+#pragma unroll
+    for (int o = 1; o < 32; o <<= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, o, 64));
+    // the lowest lane of the group that holds the extreme has the first occurrence
+    const int lane = __lane_id();
+    const uint64_t holders = __ballot(amax == gmax);
+    const uint32_t in_group = (uint32_t)(holders >> (lane & 32));
+    const float max = __shfl(first, (lane & 32) + __ffs((int)in_group) - 1, 64);
+    if (gmax == 0.0f) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = 0.0f;
+        return;
+    }
+    const float iscale = __fdiv_rn(-127.0f, max);
+    const float d = __fdiv_rn(1.0f, iscale);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = __fmul_rn(d, fminf(127.0f, rintf(__fmul_rn(iscale, v[i]))));
+}
+
+// Eight consecutive values per lane (k a multiple of 8) into one pair of planes:
+// hi/lo as two 16-byte stores; the four lanes that own one 32-wide block add
+// their sums with two xor-shuffles.
+__device__ __forceinline__ void store_act8_planes(const float (&v)[8], __half * x, __half * sums, int K,
+                                                  int tok, int k, int lane_in_block) {
     h8 a, b;
     float sum = 0.0f;
 #pragma unroll
@@ -91,16 +137,29 @@ __device__ __forceinline__ void store_act8(const float (&v)[8], const Act & out,
         b[i] = l;
         sum += (float)h + (float)l;
     }
-    *(h8 *)(out.x + act_at(tok, k, 0, out.K)) = a;
-    *(h8 *)(out.x + act_at(tok, k, 1, out.K)) = b;
-    if (out.sums) {
+    *(h8 *)(x + act_at(tok, k, 0, K)) = a;
+    *(h8 *)(x + act_at(tok, k, 1, K)) = b;
+    if (sums) {
         sum += __shfl_xor(sum, 1, 64);
         sum += __shfl_xor(sum, 2, 64);
         if (lane_in_block == 0) {
             const __half s = sat_half(sum);
-            out.sums[act_sum_at(tok, k >> 5, 0, out.K)] = s;
-            out.sums[act_sum_at(tok, k >> 5, 1, out.K)] = __float2half_rn(sum - __half2float(s));
+            sums[act_sum_at(tok, k >> 5, 0, K)] = s;
+            sums[act_sum_at(tok, k >> 5, 1, K)] = __float2half_rn(sum - __half2float(s));
         }
+    }
+}
+
+// Writes the versions of the row that `out` asks for: the values themselves
+// and / or their conversion (see requantise8 for what the lanes must satisfy).
+__device__ __forceinline__ void store_act8(const float (&v)[8], const Act & out, int tok, int k, int lane_in_block) {
+    if (out.x) store_act8_planes(v, out.x, out.sums, out.K, tok, k, lane_in_block);
+    if (out.qx) {
+        float q[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = v[i];
+        requantise8(q, out.quant);
+        store_act8_planes(q, out.qx, out.qsums, out.K, tok, k, lane_in_block);
     }
 }
 
@@ -119,9 +178,9 @@ struct MMArgs {
     int debug;                // timing experiments only: bit 0 stage activations once, bit 1 skip the multiplies
     // mode MM_SWIGLU: rows come in groups of 128, 64 gate rows then the 64 up rows of the same
     // columns; the epilogue writes silu(gate) * up as the activations of the next matmul
-    __half * act_x;
-    __half * act_sums;
-    int act_K;
+    Act act_out;
+    float * act_f32;          // instead of act_out: the products as f32 rows of act_out.K (when the next matmul's
+                              // conversion needs blocks wider than the 64 columns a workgroup holds)
 };
 
 }  // namespace rk

@@ -1,6 +1,7 @@
 #include "engine.hpp"
 
 #include <algorithm>
+#include <array>
 #include <climits>
 #include <cmath>
 #include <cstring>
@@ -71,6 +72,14 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     }
     hip_check(hipSetDevice(0), "hipSetDevice");
     hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
+    {
+        // RETRO_ACTIVATIONS=ggml: every matmul multiplies the activations as ggml's CPU path converts them
+        // (Q8_K / Q8_0 codes, f16 / bf16 rounding); unset or "exact": the f32 values (as f16 hi/lo pairs).
+        const char * v = std::getenv("RETRO_ACTIVATIONS");
+        const std::string mode = v ? v : "exact";
+        if (mode == "ggml") ggml_activations_ = true;
+        else if (mode != "exact" && !mode.empty()) throw std::runtime_error("RETRO_ACTIVATIONS must be \"exact\" or \"ggml\"");
+    }
     load_model(path);
 
     // Per-sequence context: the whole pool when unified, an equal share otherwise.
@@ -373,6 +382,12 @@ void Engine::build_buffers() {
     act(act_q_x_, act_q_sums_, QD);
     act(act_f_x_, act_f_sums_, F);
     act(act_o_x_, act_o_sums_, E);
+    if (ggml_activations_) {
+        act(act_e_qx_, act_e_qsums_, E);
+        act(act_q_qx_, act_q_qsums_, QD);
+        act(act_f_qx_, act_f_qsums_, F);
+        act(act_o_qx_, act_o_qsums_, E);
+    }
     q_half_lo_.alloc((size_t)B * QD * 2);
     mm_ws_.alloc(rk::matmul_workspace_bytes());
     hip_check(hipMemsetAsync(mm_ws_.ptr, 0, mm_ws_.bytes, stream_), "hipMemsetAsync");
@@ -1137,10 +1152,37 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
     const HParams & h = hp_;
     const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim, F = h.n_ff;
     rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps};
-    rk::Act act_e{act_e_x_.as<__half>(), E % 32 == 0 ? act_e_sums_.as<__half>() : nullptr, E};
-    rk::Act act_q{act_q_x_.as<__half>(), QD % 32 == 0 ? act_q_sums_.as<__half>() : nullptr, QD};
-    rk::Act act_f{act_f_x_.as<__half>(), F % 32 == 0 ? act_f_sums_.as<__half>() : nullptr, F};
-    rk::Act act_o{act_o_x_.as<__half>(), E % 32 == 0 ? act_o_sums_.as<__half>() : nullptr, E};
+    // The versions of a row its consumers need: the values themselves for F32 / F16 / BF16 weights, the
+    // expert router and LoRA factors (`plain`); the converted row for the quantised weights.
+    const bool faithful = ggml_activations_;
+    auto act_for = [faithful](DevBuf & x, DevBuf & sums, DevBuf & qx, DevBuf & qsums, int K, std::initializer_list<int> types,
+                              bool plain) {
+        rk::Act a;
+        a.K = K;
+        a.faithful = faithful ? 1 : 0;
+        if (!faithful) {
+            a.x = x.as<__half>();
+            a.sums = K % 32 == 0 ? sums.as<__half>() : nullptr;
+            return a;
+        }
+        for (int t : types) {
+            const int q = rk::act_quant_of(t);
+            if (q == rk::AQ_NONE) { plain = true; continue; }
+            if (a.quant != rk::AQ_NONE && a.quant != q)
+                throw std::runtime_error("weights that share an input row mix Q8_0 / MXFP4 with Q4_K storage: unsupported");
+            a.quant = q;
+        }
+        if (plain) { a.x = x.as<__half>(); a.sums = K % 32 == 0 ? sums.as<__half>() : nullptr; }
+        if (a.quant != rk::AQ_NONE) { a.qx = qx.as<__half>(); a.qsums = qsums.as<__half>(); }
+        return a;
+    };
+    auto types_of = [](const std::vector<DevWeight> & ws) {
+        int t[3] = {-1, -1, -1};
+        for (size_t i = 0; i < ws.size() && i < 3; ++i) t[i] = ws[i].w.type;
+        for (size_t i = ws.size(); i < 3; ++i) t[i] = ws.empty() ? rk::WT_F32 : ws[0].w.type;
+        return std::array<int, 3>{t[0], t[1], t[2]};
+    };
+    const rk::Act act_o = act_for(act_o_x_, act_o_sums_, act_o_qx_, act_o_qsums_, E, {lm_head_.w.type}, false);
     partial_.ensure(rk::attention_partial_floats(n_items, h.head_dim) * 4);
     float * x = x_.as<float>();
     float * qkv = qkv_.as<float>();
@@ -1152,6 +1194,9 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
     { const size_t pt_ = prof_begin(PC_EMBED); rk::embed(stream_, tok_embd_.w, pk_.tok, T, x); prof_end(PC_EMBED, pt_); }
     for (int l = 0; l < h.n_layer; ++l) {
         const LayerWeights & L = layers_[(size_t)l];
+        const std::array<int, 3> qt = types_of(L.qkv), gt = types_of(L.gate_up);
+        rk::Act act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {qt[0], qt[1], qt[2]}, routed);
+        const rk::Act act_q = act_for(act_q_x_, act_q_sums_, act_q_qx_, act_q_qsums_, QD, {L.wo.w.type}, routed);
         { const size_t pt_ = prof_begin(PC_NORM); rk::rmsnorm_act(stream_, x, L.attn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending); prof_end(PC_NORM, pt_); }
         rk::Slices qkv_slices;
         {
@@ -1200,6 +1245,8 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         }
         prof_end(PC_OPROJ, pt_);
         pt_ = prof_begin(PC_NORM);
+        if (h.n_expert > 0) act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {L.router.w.type, L.gate_exps.w.type}, false);
+        else act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {gt[0], gt[1], gt[2]}, false);
         rk::rmsnorm_act(stream_, x, L.ffn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending);
         prof_end(PC_NORM, pt_);
         if (h.n_expert > 0) {
@@ -1215,8 +1262,9 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
             continue;
         }
         pt_ = prof_begin(PC_GATEUP);
+        const rk::Act act_f = act_for(act_f_x_, act_f_sums_, act_f_qx_, act_f_qsums_, F, {L.down.w.type}, false);
         if (L.gate_up_interleaved) {
-            rk::matmul_swiglu(stream_, L.gate_up[0].w, act_e, T, act_f, mm_ws_.ptr);
+            rk::matmul_swiglu(stream_, L.gate_up[0].w, act_e, T, act_f, mm_ws_.ptr, gu);
             prof_end(PC_GATEUP, pt_);
         } else {
             int col = 0;
@@ -1274,6 +1322,8 @@ int Engine::adapter_load(const std::string & path, float scale, int32_t * out_id
     data.alpha = file->get_float("adapter.lora.alpha", 0.0);
     data.a.resize((size_t)h.n_layer * kLoraTargets);
     data.b.resize((size_t)h.n_layer * kLoraTargets);
+    data.a_type.assign((size_t)h.n_layer * kLoraTargets, rk::WT_F32);
+    data.b_type.assign((size_t)h.n_layer * kLoraTargets, rk::WT_F32);
     size_t claimed = 0;
     for (int l = 0; l < h.n_layer; ++l) {
         for (int tg = 0; tg < kLoraTargets; ++tg) {
@@ -1311,6 +1361,8 @@ int Engine::adapter_load(const std::string & path, float scale, int32_t * out_id
             };
             to_f32(*ta, n_in[tg], r, data.a[(size_t)l * kLoraTargets + tg]);      // A: r rows of n_in
             to_f32(*tb, r, n_out[tg], data.b[(size_t)l * kLoraTargets + tg]);     // B: n_out rows of r
+            data.a_type[(size_t)l * kLoraTargets + tg] = (int32_t)ta->type;
+            data.b_type[(size_t)l * kLoraTargets + tg] = (int32_t)tb->type;
             data.elements += (uint64_t)n_in[tg] + (uint64_t)n_out[tg];
             claimed += 2;
         }
@@ -1366,6 +1418,8 @@ void Engine::rebuild_lora_table() {
                 e.B = d.b[at].as<float>();
                 e.rank = d.rank;
                 e.scale = (float)((double)d.scale * d.alpha / d.rank);
+                e.a_type = ggml_activations_ ? d.a_type[at] : rk::WT_F32;
+                e.b_type = ggml_activations_ ? d.b_type[at] : rk::WT_F32;
             }
         ++route;
     }

@@ -218,6 +218,8 @@ private:
     DevBuf act_q_x_, act_q_sums_;       // n_head * head_dim wide
     DevBuf act_f_x_, act_f_sums_;       // n_ff wide
     DevBuf act_o_x_, act_o_sums_;       // output rows, n_embd wide
+    // the same rows after the conversion ggml's CPU matmul applies for a quantised weight
+    DevBuf act_e_qx_, act_e_qsums_, act_q_qx_, act_q_qsums_, act_f_qx_, act_f_qsums_, act_o_qx_, act_o_qsums_;
     DevBuf q_half_lo_;
     DevBuf mm_ws_;            // matmul workspace: split-K partials, counters
     // mixture-of-experts scratch (allocated for MoE models only)
@@ -245,12 +247,14 @@ private:
         int rank = 0;
         uint64_t elements = 0;                     // sum over pairs of (n_in + n_out)
         std::vector<DevBuf> a, b;                  // [layer * kLoraTargets + target], empty when the pair is absent
+        std::vector<int32_t> a_type, b_type;       // storage types in the adapter file, same index
     };
     std::map<int32_t, RowAdapterData> row_adapters_;
     int32_t next_adapter_id_ = 1;
     DevBuf lora_table_;       // LoraEntry [layer][target][route - 1]
     DevBuf lora_mid_;         // [n_batch][LORA_MAX_RANK] f32
     int lora_routes_ = 0;
+    bool ggml_activations_ = false;   // RETRO_ACTIVATIONS=ggml at construction
     void rebuild_lora_table();
     const rk::LoraEntry * lora_entries(int layer, int target) const {
         return lora_table_.as<rk::LoraEntry>() + ((size_t)layer * kLoraTargets + target) * (size_t)lora_routes_;

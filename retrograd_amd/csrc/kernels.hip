@@ -107,7 +107,9 @@ __device__ float decode_elem(int type, const uint8_t * row, int k) {
 }
 
 // Writes up to 32 consecutive activations of one token (k0 a multiple of 32) as
-// f16 hi/lo pairs and, for a whole block, the sum of the stored values as hi + lo halves.
+// f16 hi/lo pairs and, for a whole block, the sum of the stored values as hi + lo
+// halves. Only the values themselves: rows of a width that is no multiple of 32
+// have no quantised consumer.
 __device__ __forceinline__ void store_act_block(const float * v, int count, const Act & out, int tok, int k0) {
     float sum = 0.0f;
     for (int i = 0; i < count; ++i) {
@@ -121,6 +123,18 @@ __device__ __forceinline__ void store_act_block(const float * v, int count, cons
         const __half a = sat_half(sum);
         out.sums[act_sum_at(tok, k0 >> 5, 0, out.K)] = a;
         out.sums[act_sum_at(tok, k0 >> 5, 1, out.K)] = __float2half_rn(sum - __half2float(a));
+    }
+}
+
+// Host-side check of what a producer is asked to write.
+static void check_act_out(const Act & out, int K, const char * what) {
+    if (out.K != K) throw std::runtime_error(std::string(what) + ": activation width does not match");
+    if (!out.x && !out.qx) throw std::runtime_error(std::string(what) + ": no activation buffer to write");
+    if (out.qx) {
+        if (out.quant != AQ_Q8_0 && out.quant != AQ_Q8_K)
+            throw std::runtime_error(std::string(what) + ": unknown activation conversion");
+        if (K % out.quant != 0)
+            throw std::runtime_error(std::string(what) + ": the row width is no multiple of the conversion's block");
     }
 }
 
@@ -443,7 +457,8 @@ __global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
 // Any type, any shape: one wave per output feature, raw GGUF rows.
 __global__ __launch_bounds__(256) void k_mm_generic(int type, const uint8_t * __restrict__ raw, size_t rb,
                                                     const __half * __restrict__ x, int K, int N, int T,
-                                                    float * y, int ldy, int col0, int mode, const float * bias) {
+                                                    float * y, int ldy, int col0, int mode, const float * bias,
+                                                    int round_as) {
     const int lane = threadIdx.x & 63;
     const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (n >= N) return;
@@ -455,7 +470,15 @@ __global__ __launch_bounds__(256) void k_mm_generic(int type, const uint8_t * __
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int t = min(t0 + j, T - 1);
-                const float xv = __half2float(x[act_at(t, k, 0, K)]) + __half2float(x[act_at(t, k, 1, K)]);
+                // under ggml's arithmetic (round_as = the weight type) F16 weights multiply the activations
+                // rounded to f16 (the hi half is that rounding) and BF16 weights those rounded to bf16
+                float xv = __half2float(x[act_at(t, k, 0, K)]);
+                if (round_as != WT_F16) xv += __half2float(x[act_at(t, k, 1, K)]);
+                if (round_as == WT_BF16) {
+                    uint32_t u = __float_as_uint(xv);
+                    u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+                    xv = __uint_as_float(u);
+                }
                 acc[j] = fmaf(w, xv, acc[j]);
             }
         }
@@ -476,8 +499,10 @@ void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float
     if (!w.raw) throw std::runtime_error("matmul_generic: the weight has no raw layout");
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
     if (T <= 0) return;
+    const Act xo = x.operand(w.type);
+    if (!xo.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
     hipLaunchKernelGGL(k_mm_generic, dim3((w.N + 3) / 4), dim3(256), 0, s, w.type, w.raw, row_bytes(w.type, w.K),
-                       x.x, w.K, w.N, T, y, ldy, col0, mode, bias);
+                       xo.x, w.K, w.N, T, y, ldy, col0, mode, bias, xo.faithful ? w.type : WT_F32);
     check_launch("matmul_generic");
 }
 
@@ -528,10 +553,12 @@ static Slices matmul_impl(hipStream_t s, const Weight & w, const Act & x, int T,
         return Slices();
     }
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
-    if (w.type == WT_Q4_K && !x.sums) throw std::runtime_error("matmul: Q4_K needs block sums");
     if (ws) return matmul_lds(s, w, x, T, y, ldy, col0, mode, bias, ws, may_slice);
+    const Act xo = x.operand(w.type);
+    if (!xo.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
+    if (w.type == WT_Q4_K && !xo.sums) throw std::runtime_error("matmul: Q4_K needs block sums");
     MMArgs a {};
-    a.w = w.packed; a.x = x.x; a.sums = x.sums; a.y = y; a.bias = bias;
+    a.w = w.packed; a.x = xo.x; a.sums = xo.sums; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
     a.n_row_tiles = w.N / 16;
     // Enough waves to cover the chip: split K across the waves of a workgroup
@@ -590,6 +617,18 @@ void decode_rows(hipStream_t s, int type, const uint8_t * raw, int K, int n_rows
 // ---------------------------------------------------------------------------
 // per-row LoRA
 
+// The operand of a dot product with a factor of this storage type.
+__device__ __forceinline__ float lora_operand(float hi, float lo, int type) {
+    if (type == WT_F16) return hi;                   // hi is the f16 rounding of the value
+    float v = hi + lo;
+    if (type == WT_BF16) {
+        uint32_t u = __float_as_uint(v);
+        u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+        v = __uint_as_float(u);
+    }
+    return v;
+}
+
 // mid[t][r] = sum_k A[r][k] * x[t][k]: one wave per (token, r), lanes own groups of eight k.
 __global__ __launch_bounds__(256) void k_lora_down(const LoraEntry * __restrict__ table, const RowDesc * __restrict__ rows,
                                                    const int32_t * __restrict__ tok_row, Act x, float * __restrict__ mid) {
@@ -608,13 +647,13 @@ __global__ __launch_bounds__(256) void k_lora_down(const LoraEntry * __restrict_
             const f4 a0 = *(const f4 *)(a + k), a1 = *(const f4 *)(a + k + 4);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                acc = fmaf(a0[i], (float)hi[i] + (float)lo[i], acc);
-                acc = fmaf(a1[i], (float)hi[4 + i] + (float)lo[4 + i], acc);
+                acc = fmaf(a0[i], lora_operand((float)hi[i], (float)lo[i], e.a_type), acc);
+                acc = fmaf(a1[i], lora_operand((float)hi[4 + i], (float)lo[4 + i], e.a_type), acc);
             }
         }
     } else {
         for (int k = lane; k < x.K; k += 64)
-            acc = fmaf(a[k], __half2float(x.x[act_at(t, k, 0, x.K)]) + __half2float(x.x[act_at(t, k, 1, x.K)]), acc);
+            acc = fmaf(a[k], lora_operand(__half2float(x.x[act_at(t, k, 0, x.K)]), __half2float(x.x[act_at(t, k, 1, x.K)]), e.a_type), acc);
     }
     acc = wave_sum(acc);
     if (lane == 0) mid[(size_t)t * LORA_MAX_RANK + r] = acc;
@@ -633,13 +672,17 @@ __global__ __launch_bounds__(256) void k_lora_up(const LoraEntry * __restrict__ 
     const float * b = e.B + (size_t)n * e.rank;
     const float * m = mid + (size_t)t * LORA_MAX_RANK;
     float acc = 0.0f;
-    for (int r = 0; r < e.rank; ++r) acc = fmaf(b[r], m[r], acc);
+    for (int r = 0; r < e.rank; ++r) {
+        const float hi = (float)(_Float16)fminf(fmaxf(m[r], -65504.0f), 65504.0f);
+        acc = fmaf(b[r], lora_operand(hi, m[r] - hi, e.b_type), acc);
+    }
     y[(size_t)t * ldy + col0 + n] += e.scale * acc;
 }
 
 void lora_apply(hipStream_t s, const LoraEntry * table, const RowDesc * rows, const int32_t * tok_row,
                 const Act & x, int T, int N, float * y, int ldy, int col0, float * mid) {
     if (T <= 0 || N <= 0) return;
+    if (!x.x) throw std::runtime_error("lora: the unconverted activations are missing");
     hipLaunchKernelGGL(k_lora_down, dim3(T, LORA_MAX_RANK / 4), dim3(256), 0, s, table, rows, tok_row, x, mid);
     check_launch("lora_down");
     hipLaunchKernelGGL(k_lora_up, dim3(T, (N + 255) / 256), dim3(256), 0, s, table, rows, tok_row, mid, N, y, ldy, col0);
@@ -755,15 +798,15 @@ void rmsnorm_act(hipStream_t s, float * x, const float * w, int E, float eps,
                  const int32_t * rows, int n_rows, const Act & out, const Slices & add) {
     if (n_rows <= 0) return;
     if (add.n > 0 && add.N != E) throw std::runtime_error("rmsnorm: the slices do not match the row width");
-    if (out.K != E) throw std::runtime_error("rmsnorm: activation width does not match");
-    if (E % 32 == 0 && out.sums) {
+    check_act_out(out, E, "rmsnorm");
+    if (E % 32 == 0) {
         if (E >= 4096) hipLaunchKernelGGL(k_rmsnorm_act8<8>, dim3(n_rows), dim3(512), 0, s, x, w, E, eps, rows, out, add);
         else hipLaunchKernelGGL(k_rmsnorm_act8<4>, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, out, add);
         check_launch("rmsnorm");
         return;
     }
     Act o = out;
-    if (E % 32 != 0) o.sums = nullptr;
+    o.sums = nullptr;
     hipLaunchKernelGGL(k_rmsnorm_act, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, o, add);
     check_launch("rmsnorm");
 }
@@ -797,14 +840,53 @@ __global__ __launch_bounds__(256) void k_to_act(const float * __restrict__ x, in
     store_act_block(v, count, out, t, k0);
 }
 
+// K % 32 == 0: 8 elements per lane.
+__global__ __launch_bounds__(256) void k_to_act8(const float * __restrict__ x, int T, int K, Act out) {
+    const int per = K / 8;
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (size_t)T * per) return;      // whole groups of lanes that share a block leave together
+    const int t = (int)(gid / per), k = (int)(gid % per) * 8;
+    const f4 a = *(const f4 *)(x + (size_t)t * K + k), b = *(const f4 *)(x + (size_t)t * K + k + 4);
+    const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+    store_act8(v, out, t, k, threadIdx.x & 3);
+}
+
 void to_act(hipStream_t s, const float * x, int T, int K, const Act & out) {
     if (T <= 0) return;
-    if (out.K != K) throw std::runtime_error("to_act: activation width does not match");
+    check_act_out(out, K, "to_act");
+    if (K % 32 == 0) {
+        const size_t n = (size_t)T * (K / 8);
+        hipLaunchKernelGGL(k_to_act8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, T, K, out);
+        check_launch("to_act");
+        return;
+    }
     Act o = out;
-    if (K % 32 != 0) o.sums = nullptr;
+    o.sums = nullptr;
     const size_t n = (size_t)T * ((K + 31) / 32);
     hipLaunchKernelGGL(k_to_act, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, T, K, o);
     check_launch("to_act");
+}
+
+// The rows in `src` (hi/lo planes) converted into out.qx; the two may be the same buffer.
+__global__ __launch_bounds__(256) void k_requant_act8(const __half * src, int T, int K, Act out) {
+    const int per = K / 8;
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (size_t)T * per) return;      // whole groups of lanes that share a block leave together
+    const int t = (int)(gid / per), k = (int)(gid % per) * 8;
+    const h8 hi = load_h8(src + act_at(t, k, 0, K)), lo = load_h8(src + act_at(t, k, 1, K));
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (float)hi[i] + (float)lo[i];
+    store_act8(v, out, t, k, threadIdx.x & 3);
+}
+
+void requant_act(hipStream_t s, const __half * src, int T, const Act & out) {
+    if (T <= 0) return;
+    check_act_out(out, out.K, "requant_act");
+    if (out.x || !out.qx) throw std::runtime_error("requant_act: writes the converted rows only");
+    const size_t n = (size_t)T * (out.K / 8);
+    hipLaunchKernelGGL(k_requant_act8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, src, T, out.K, out);
+    check_launch("requant_act");
 }
 
 // F % 32 == 0: 8 elements per lane.
@@ -826,15 +908,15 @@ __global__ __launch_bounds__(256) void k_swiglu_act8(const float * __restrict__ 
 
 void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out) {
     if (T <= 0) return;
-    if (out.K != F) throw std::runtime_error("swiglu: activation width does not match");
-    if (F % 32 == 0 && out.sums) {
+    check_act_out(out, F, "swiglu");
+    if (F % 32 == 0) {
         const size_t n = (size_t)T * (F / 8);
         hipLaunchKernelGGL(k_swiglu_act8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, T, F, out);
         check_launch("swiglu");
         return;
     }
     Act o = out;
-    if (F % 32 != 0) o.sums = nullptr;
+    o.sums = nullptr;
     const size_t n = (size_t)T * ((F + 31) / 32);
     hipLaunchKernelGGL(k_swiglu_act, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, T, F, o);
     check_launch("swiglu");
@@ -1355,77 +1437,126 @@ struct CombineArgs {
 // attention output as the O-projection's activations. The (max, sum) pairs of
 // the splits are read one per lane, the outputs two dimensions per lane.
 __global__ __launch_bounds__(256) void k_attention_combine(CombineArgs a) {
+    __shared__ float blk_amax[4], blk_first[4];
     const int t = blockIdx.x;
-    const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
+    const int wave = threadIdx.x >> 6;
+    const int head = blockIdx.y * 4 + wave;
     const int lane = threadIdx.x & 63;
-    if (head >= a.n_head) return;
-    const int4 meta = a.tok_merge[t];                  // first item of the token's tile, splits, index in the tile
-    const int ns = meta.y;
-    const int kvh = head / a.G, gi = head % a.G;
-    const int col = meta.z * a.G + gi;
-    const int item0 = meta.x + kvh * ns;
-    const int stride = a.hd + 2;
+    const bool live = head < a.n_head;           // a wave without a head still meets the others at the barrier
     const int e0 = 2 * lane;
     float M = -INFINITY, L = 0.0f, v0 = 0.0f, v1 = 0.0f;
-    for (int s0 = 0; s0 < ns; s0 += 64) {
-        const int n = min(64, ns - s0);
-        float m_s = -INFINITY, l_s = 0.0f;
-        if (lane < n) {
-            const float * p = a.partial + ((size_t)(item0 + s0 + lane) * 16 + col) * stride;
-            m_s = p[0];
-            l_s = p[1];
-        }
-        float cm = m_s;
-        for (int o = 32; o > 0; o >>= 1) cm = fmaxf(cm, __shfl_xor(cm, o, 64));
-        const float m_new = fmaxf(M, cm);
-        const float keep = M == -INFINITY ? 0.0f : exp2f(M - m_new);
-        L *= keep; v0 *= keep; v1 *= keep;
-        M = m_new;
-        const float w_s = m_s == -INFINITY ? 0.0f : exp2f(m_s - M);
-        L += wave_sum(w_s * l_s);
-        for (int s = 0; s < n; ++s) {
-            const float w = __shfl(w_s, s, 64);
-            if (e0 < a.hd) {
-                const float2 pv = *(const float2 *)(a.partial + ((size_t)(item0 + s0 + s) * 16 + col) * stride + 2 + e0);
-                v0 = fmaf(w, pv.x, v0);
-                v1 = fmaf(w, pv.y, v1);
+    if (live) {
+        const int4 meta = a.tok_merge[t];                  // first item of the token's tile, splits, index in the tile
+        const int ns = meta.y;
+        const int kvh = head / a.G, gi = head % a.G;
+        const int col = meta.z * a.G + gi;
+        const int item0 = meta.x + kvh * ns;
+        const int stride = a.hd + 2;
+        for (int s0 = 0; s0 < ns; s0 += 64) {
+            const int n = min(64, ns - s0);
+            float m_s = -INFINITY, l_s = 0.0f;
+            if (lane < n) {
+                const float * p = a.partial + ((size_t)(item0 + s0 + lane) * 16 + col) * stride;
+                m_s = p[0];
+                l_s = p[1];
+            }
+            float cm = m_s;
+            for (int o = 32; o > 0; o >>= 1) cm = fmaxf(cm, __shfl_xor(cm, o, 64));
+            const float m_new = fmaxf(M, cm);
+            const float keep = M == -INFINITY ? 0.0f : exp2f(M - m_new);
+            L *= keep; v0 *= keep; v1 *= keep;
+            M = m_new;
+            const float w_s = m_s == -INFINITY ? 0.0f : exp2f(m_s - M);
+            L += wave_sum(w_s * l_s);
+            for (int s = 0; s < n; ++s) {
+                const float w = __shfl(w_s, s, 64);
+                if (e0 < a.hd) {
+                    const float2 pv = *(const float2 *)(a.partial + ((size_t)(item0 + s0 + s) * 16 + col) * stride + 2 + e0);
+                    v0 = fmaf(w, pv.x, v0);
+                    v1 = fmaf(w, pv.y, v1);
+                }
             }
         }
     }
     const float inv = L > 0.0f ? 1.0f / L : 0.0f;
     const int QD = a.n_head * a.hd;
-    float r0 = 0.0f, r1 = 0.0f;
-    if (e0 < a.hd) {
-        const float f0 = fminf(fmaxf(v0 * inv, -65504.0f), 65504.0f);
-        const float f1 = fminf(fmaxf(v1 * inv, -65504.0f), 65504.0f);
-        const __half h0 = __float2half_rn(f0), h1 = __float2half_rn(f1);
-        const __half l0 = __float2half_rn(f0 - __half2float(h0)), l1 = __float2half_rn(f1 - __half2float(h1));
-        const int k = head * a.hd + e0;            // even: k and k + 1 share a group of eight
-        const size_t at = act_at(t, k, 0, QD), at_lo = act_at(t, k, 1, QD);
-        a.out.x[at] = h0;
-        a.out.x[at + 1] = h1;
-        a.out.x[at_lo] = l0;
-        a.out.x[at_lo + 1] = l1;
-        r0 = __half2float(h0) + __half2float(l0);
-        r1 = __half2float(h1) + __half2float(l1);
-    }
-    if (a.out.sums) {
-        // block of 32 outputs = 16 lanes
-        float sum = r0 + r1;
+    const bool mine = live && e0 < a.hd;
+    const float f0 = mine ? v0 * inv : 0.0f, f1 = mine ? v1 * inv : 0.0f;
+    const int k = head * a.hd + e0;            // even: k and k + 1 share a group of eight
+    // 32 outputs = 16 lanes: the block sum of the stored values
+    auto store = [&](__half * x, __half * sums, float g0, float g1) {
+        float r0 = 0.0f, r1 = 0.0f;
+        if (mine) {
+            const float c0 = fminf(fmaxf(g0, -65504.0f), 65504.0f), c1 = fminf(fmaxf(g1, -65504.0f), 65504.0f);
+            const __half h0 = __float2half_rn(c0), h1 = __float2half_rn(c1);
+            const __half l0 = __float2half_rn(c0 - __half2float(h0)), l1 = __float2half_rn(c1 - __half2float(h1));
+            const size_t at = act_at(t, k, 0, QD), at_lo = act_at(t, k, 1, QD);
+            x[at] = h0;
+            x[at + 1] = h1;
+            x[at_lo] = l0;
+            x[at_lo + 1] = l1;
+            r0 = __half2float(h0) + __half2float(l0);
+            r1 = __half2float(h1) + __half2float(l1);
+        }
+        if (sums) {
+            float sum = r0 + r1;
 #pragma unroll
-        for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o, 64);
-        if ((lane & 15) == 0 && e0 < a.hd) {
-            const int b = (head * a.hd + e0) / 32;
-            const __half hi = sat_half(sum);
-            a.out.sums[act_sum_at(t, b, 0, QD)] = hi;
-            a.out.sums[act_sum_at(t, b, 1, QD)] = __float2half_rn(sum - __half2float(hi));
+            for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o, 64);
+            if ((lane & 15) == 0 && mine) {
+                const int b = k / 32;
+                const __half hi = sat_half(sum);
+                sums[act_sum_at(t, b, 0, QD)] = hi;
+                sums[act_sum_at(t, b, 1, QD)] = __float2half_rn(sum - __half2float(hi));
+            }
+        }
+    };
+    if (a.out.x) store(a.out.x, a.out.sums, f0, f1);
+    if (!a.out.qx) return;
+    // the conversion ggml's CPU matmul applies to the row before the output projection (see requantise8)
+    float q0, q1;
+    if (a.out.quant == AQ_Q8_0) {
+        float amax = fmaxf(fabsf(f0), fabsf(f1));
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+        const float d = __fdiv_rn(amax, 127.0f);
+        const float id = d != 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
+        const float dh = (float)(_Float16)d;
+        q0 = __fmul_rn(dh, roundf(__fmul_rn(f0, id)));
+        q1 = __fmul_rn(dh, roundf(__fmul_rn(f1, id)));
+    } else {
+        // a block of 256 = 256 / hd heads = that many waves of this workgroup, in head order
+        float amax = fabsf(f0), first = f0;
+        if (fabsf(f1) > amax) { amax = fabsf(f1); first = f1; }
+        float wmax = amax;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) wmax = fmaxf(wmax, __shfl_xor(wmax, o, 64));
+        const uint64_t holders = __ballot(amax == wmax);
+        first = __shfl(first, __ffsll((long long)holders) - 1, 64);
+        if (lane == 0) { blk_amax[wave] = wmax; blk_first[wave] = first; }
+        __syncthreads();
+        const int per = 256 / a.hd;                 // waves per block: 2 (hd 128) or 4 (hd 64)
+        const int w0 = wave / per * per;
+        float gmax = 0.0f, max = 0.0f;
+        for (int w = w0; w < w0 + per; ++w)
+            if (blk_amax[w] > gmax) { gmax = blk_amax[w]; max = blk_first[w]; }
+        if (gmax == 0.0f) {
+            q0 = q1 = 0.0f;
+        } else {
+            const float iscale = __fdiv_rn(-127.0f, max);
+            const float d = __fdiv_rn(1.0f, iscale);
+            q0 = __fmul_rn(d, fminf(127.0f, rintf(__fmul_rn(iscale, f0))));
+            q1 = __fmul_rn(d, fminf(127.0f, rintf(__fmul_rn(iscale, f1))));
         }
     }
+    store(a.out.qx, a.out.qsums, q0, q1);
 }
 
 void attention_combine(hipStream_t s, const float * partial, int T, const AttnShape & sh,
                        const PackBuffers & pk, const Act & out) {
     if (T <= 0) return;
+    check_act_out(out, sh.n_head * sh.head_dim, "attention_combine");
+    if (out.qx && out.quant == AQ_Q8_K && ((sh.head_dim != 64 && sh.head_dim != 128) || (sh.n_head * sh.head_dim) % 256 != 0))
+        throw std::runtime_error("attention_combine: the Q8_K conversion needs heads of 64 or 128 dimensions");
     CombineArgs a;
     a.partial = partial; a.tok_merge = pk.tok_merge; a.out = out;
     a.n_head = sh.n_head; a.G = sh.n_head / sh.n_head_kv; a.hd = sh.head_dim;

@@ -39,22 +39,54 @@ struct Weight {
 
 // Activations handed to a matmul. An f32 value v travels as two f16 numbers,
 // hi = f16(v) and lo = f16(v - hi), which together carry about 22 significant
-// bits: a single f16 (11 bits) leaves a logit error above the parity
-// tolerance once it has passed through a few layers. For every 32-wide block
-// of a row the f32 sum of hi + lo is kept as well, split the same way; the
-// sums are what the Q4_K min term multiplies.
+// bits. For every 32-wide block of a row the f32 sum of hi + lo is kept as
+// well, split the same way; the sums are what the Q4_K min term multiplies.
 //
-// Both buffers are stored in MFMA operand order, so that a matmul stages them
+// ggml's CPU matmul does not multiply a quantised weight with the f32
+// activations themselves: it first converts the row to the weight type's
+// companion format (Q8_K blocks of 256 for Q4_K; Q8_0 blocks of 32 for Q8_0 and
+// MXFP4; f16 / bf16 rounding for F16 / BF16 weights) and multiplies the codes.
+// An engine can run either arithmetic. In the ggml one (`faithful`) a producer
+// writes up to two versions of a row: the values as they are (x, sums: what
+// F32 / F16 / BF16 weights, the expert router and LoRA factors read, the latter
+// rounding on the way) and the values after the conversion, scale times code
+// (qx, qsums, with `quant` the block rule), which the quantised weights read.
+// In the exact one only x and sums exist and every consumer reads them.
+//
+// All buffers are stored in MFMA operand order, so that a matmul stages them
 // with contiguous 1 KiB loads. Tokens are grouped in chunks of 64 (4 tiles of
 // 16); with Kp = K rounded up to 32:
 //   x:    [chunk][k / 32][hi, lo][tile][lane = 16 * ((k % 32) / 8) + token % 16][k % 8]
 //   sums: [chunk][k / 256][tile][lane = 16 * (hi: 0, lo: 1) + token % 16][(k % 256) / 32]
 // The sums blocks also have lanes 32-63, which stay zero from allocation: they
 // pad the operand of the min-term MFMA.
+enum : int { AQ_NONE = 0, AQ_Q8_0 = 32, AQ_Q8_K = 256 };
+// The conversion ggml's CPU matmul applies for a weight of this storage type.
+inline int act_quant_of(int ggml_type) {
+    switch (ggml_type) {
+        case 12: return AQ_Q8_K;            // Q4_K
+        case 8: case 39: return AQ_Q8_0;    // Q8_0, MXFP4
+        default: return AQ_NONE;
+    }
+}
 struct Act {
     __half * x = nullptr;       // act_halves(T, K) halves
     __half * sums = nullptr;    // act_sum_halves(T, K) halves, zero-initialised; null when K % 32 != 0
     int K = 0;
+    __half * qx = nullptr;      // the converted row, same layouts
+    __half * qsums = nullptr;
+    int quant = AQ_NONE;
+    int faithful = 0;           // ggml's arithmetic: F16 / BF16 operands are rounded as well
+    // What a weight of this type multiplies: the converted row for the quantised
+    // types under ggml's arithmetic, the values themselves otherwise.
+    Act operand(int ggml_type) const {
+        Act a;
+        a.K = K;
+        a.faithful = faithful;
+        if (faithful && act_quant_of(ggml_type) != AQ_NONE) { a.x = qx; a.sums = qsums; }
+        else { a.x = x; a.sums = sums; }
+        return a;
+    }
 };
 inline size_t act_halves(int T, int K) { return (size_t)((T + 63) / 64) * (size_t)((K + 31) / 32 * 32) * 128; }
 inline size_t act_sum_halves(int T, int K) { return (size_t)((T + 63) / 64) * (size_t)((K + 255) / 256) * 2048; }
@@ -96,7 +128,10 @@ extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic
 // Fused gate/up matmul and SwiGLU: w holds, for every 64 columns of the hidden
 // layer, their 64 gate rows followed by their 64 up rows (w.N = 2 F, F % 64 == 0,
 // a tile storage type); out (K = F) receives silu(gate) * up as activations.
-void matmul_swiglu(hipStream_t s, const Weight & w, const Act & x, int T, const Act & out, void * ws);
+// When out asks for the Q8_K conversion, whose blocks are wider than the 64
+// columns a workgroup holds, the products leave as f32 rows in h_f32 ([T][F])
+// and a second launch converts them.
+void matmul_swiglu(hipStream_t s, const Weight & w, const Act & x, int T, const Act & out, void * ws, float * h_f32);
 Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
                   int mode, const float * bias, void * ws, bool may_slice);
 // Forces the generic (raw layout) kernel; used to cross-check the tile kernels.
@@ -111,6 +146,10 @@ struct LoraEntry {
     const float * B = nullptr;
     int32_t rank = 0;
     float scale = 0.0f;
+    // storage types of the factors in the adapter file: an F16 (BF16) factor multiplies
+    // its operand rounded to f16 (bf16), as ggml's CPU dot products do
+    int32_t a_type = WT_F32;
+    int32_t b_type = WT_F32;
 };
 constexpr int LORA_MAX_RANK = 64;
 // For every token whose row routes to an adapter (rows[tok_row[t]].route > 0,
@@ -154,6 +193,9 @@ void rmsnorm_act(hipStream_t s, float * x, const float * w, int E, float eps,
 
 // act = f16(x) (+ block sums): the plain conversion every producer fuses.
 void to_act(hipStream_t s, const float * x, int T, int K, const Act & out);
+// The T rows stored as hi/lo planes at `src` (layout of Act::x, width out.K), converted by
+// out.quant into out.qx / out.qsums; src may be out.qx itself. out.x must be null.
+void requant_act(hipStream_t s, const __half * src, int T, const Act & out);
 
 // act = f16(silu(gu[t][i]) * gu[t][F + i]) (+ block sums).
 void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out);

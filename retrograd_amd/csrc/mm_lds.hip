@@ -125,10 +125,10 @@ __device__ __forceinline__ void store_token_rows(const MMArgs & a, uint8_t * sme
         // eight lanes per token, eight hidden columns each: gate in columns c, up in columns 64 + c of the group
         static_assert(R == 2, "a row group is 64 gate rows and 64 up rows");
         const int c = (threadIdx.x & 7) * 8;
-        const Act out{a.act_x, a.act_sums, a.act_K};
+        const Act & out = a.act_out;
         for (int tk = threadIdx.x >> 3; tk < NT * 16; tk += kThreads / 8) {
             const int tok = tbase + tk;
-            if (tok >= a.T || rg * 64 + c >= a.act_K) continue;      // the four lanes of a 32-wide block leave together
+            if (tok >= a.T || rg * 64 + c >= out.K) continue;      // the four lanes of a 32-wide block leave together
             const float * g0 = h0 + tk * S + c, * g1 = h1 + tk * S + c;
             float v[8];
 #pragma unroll
@@ -138,7 +138,13 @@ __device__ __forceinline__ void store_token_rows(const MMArgs & a, uint8_t * sme
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[i + e] = (g[e] / (1.0f + __expf(-g[e]))) * u[e];
             }
-            store_act8(v, out, tok, rg * 64 + c, threadIdx.x & 3);
+            if (a.act_f32) {
+                float * dst = a.act_f32 + (size_t)tok * out.K + rg * 64 + c;
+                *(f4 *)dst = (f4){v[0], v[1], v[2], v[3]};
+                *(f4 *)(dst + 4) = (f4){v[4], v[5], v[6], v[7]};
+            } else {
+                store_act8(v, out, tok, rg * 64 + c, threadIdx.x & 3);
+            }
         }
         return;
     }
@@ -745,13 +751,16 @@ static void dispatch_nt(hipStream_t s, int type, int nt, const MMArgs & a, dim3 
 }
 
 // act_out: destination of mode MM_SWIGLU, else null
-static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
-                       int mode, const float * bias, void * ws, bool may_slice, const Act * act_out) {
+static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x_all, int T, float * y, int ldy, int col0,
+                       int mode, const float * bias, void * ws, bool may_slice, const Act * act_out, float * act_f32) {
+    const Act x = x_all.operand(w.type);
+    if (!x.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
+    if (w.type == WT_Q4_K && !x.sums) throw std::runtime_error("matmul: Q4_K needs block sums");
     MMArgs a {};
     a.debug = g_mm_debug;
     a.w = w.packed; a.x = x.x; a.sums = x.sums; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
-    if (act_out) { a.act_x = act_out->x; a.act_sums = act_out->sums; a.act_K = act_out->K; }
+    if (act_out) { a.act_out = *act_out; a.act_f32 = act_f32; }
     a.n_row_tiles = w.N / 16;
     // the epilogue stores four columns per lane
     if (mode != MM_SWIGLU && ((ldy & 3) || (col0 & 3) || ((uintptr_t)y & 15) || (bias && ((uintptr_t)bias & 15))))
@@ -791,15 +800,20 @@ static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x, int T, fl
 Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
                   int mode, const float * bias, void * ws, bool may_slice) {
     if (mode == MM_SWIGLU) throw std::runtime_error("matmul_lds: use matmul_swiglu");
-    return lds_impl(s, w, x, T, y, ldy, col0, mode, bias, ws, may_slice, nullptr);
+    return lds_impl(s, w, x, T, y, ldy, col0, mode, bias, ws, may_slice, nullptr, nullptr);
 }
 
-void matmul_swiglu(hipStream_t s, const Weight & w, const Act & x, int T, const Act & out, void * ws) {
+void matmul_swiglu(hipStream_t s, const Weight & w, const Act & x, int T, const Act & out, void * ws, float * h_f32) {
     if (T <= 0) return;
-    if (!w.packed || !ws || w.N != 2 * out.K || out.K % 64 != 0 || !out.sums)
+    if (!w.packed || !ws || w.N != 2 * out.K || out.K % 64 != 0 || (!out.x && !out.qx))
         throw std::runtime_error("matmul_swiglu: needs a tile-packed gate/up matrix interleaved by 64 columns");
     if (x.K != w.K) throw std::runtime_error("matmul_swiglu: activation width does not match the weight");
-    lds_impl(s, w, x, T, nullptr, 0, 0, MM_SWIGLU, nullptr, ws, false, &out);
+    // A workgroup holds 64 hidden columns of a token: enough for the 32-wide blocks of the Q8_0
+    // conversion, not for the 256-wide ones of Q8_K. Those rows leave as f32 and are converted after.
+    const bool via_f32 = out.qx && out.quant == AQ_Q8_K;
+    if (via_f32 && !h_f32) throw std::runtime_error("matmul_swiglu: the Q8_K conversion needs the f32 row buffer");
+    lds_impl(s, w, x, T, nullptr, 0, 0, MM_SWIGLU, nullptr, ws, false, &out, via_f32 ? h_f32 : nullptr);
+    if (via_f32) to_act(s, h_f32, T, out.K, out);
 }
 
 }  // namespace rk

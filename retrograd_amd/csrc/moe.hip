@@ -392,11 +392,19 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     check_launch("moe_group");
     MoeArgs a {};
     a.expert_n = b.expert_n; a.off_pad = b.off_pad; a.tok_of_q = b.tok_of_q; a.n_expert = sh.n_expert;
-    a.w0 = L.gate.packed; a.w1 = L.up.packed; a.x = xn; a.h = b.h; a.K = sh.E; a.N = sh.F;
+    // the experts multiply the rows after ggml's Q8_0 conversion, the router the rows themselves
+    a.w0 = L.gate.packed; a.w1 = L.up.packed; a.x = xn.operand(L.gate.type); a.h = b.h; a.K = sh.E; a.N = sh.F;
+    if (!a.x.x || !b.h.x) throw std::runtime_error("moe: the activations were not prepared for the expert weights");
     const unsigned gu_blocks = (unsigned)(((size_t)sh.n_expert * (sh.F / 16) + 3) / 4);
     if (L.gate.type == WT_MXFP4) hipLaunchKernelGGL(k_moe_gate_up<WT_MXFP4>, dim3(gu_blocks), dim3(256), 0, s, a);
     else hipLaunchKernelGGL(k_moe_gate_up<WT_Q8_0>, dim3(gu_blocks), dim3(256), 0, s, a);
     check_launch("moe_gate_up");
+    if (xn.faithful) {
+        // ggml's arithmetic: the hidden rows are converted, in place, for the down projection
+        Act hq;
+        hq.K = sh.F; hq.qx = b.h.x; hq.qsums = nullptr; hq.quant = act_quant_of(L.down.type);
+        requant_act(s, b.h.x, (int)moe_slots(T, sh.k_used, sh.n_expert), hq);
+    }
     a.w0 = L.down.packed; a.w1 = nullptr; a.x = b.h; a.out_pair = b.out_pair; a.K = sh.F; a.N = sh.E;
     const unsigned d_blocks = (unsigned)(((size_t)sh.n_expert * (sh.E / 16) + 3) / 4);
     if (L.down.type == WT_MXFP4) hipLaunchKernelGGL(k_moe_down<WT_MXFP4>, dim3(d_blocks), dim3(256), 0, s, a);

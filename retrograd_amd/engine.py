@@ -767,8 +767,11 @@ class _GrammarHandle:
 # ---- kernel-level calls (tests, micro-benchmarks) -----------------------------------------
 
 def kernel_matmul(ggml_type: int, raw: np.ndarray, n_rows: int, k: int, x: np.ndarray, use_tiles,
-                  bias: np.ndarray | None = None, accumulate_into: np.ndarray | None = None) -> np.ndarray:
+                  bias: np.ndarray | None = None, accumulate_into: np.ndarray | None = None,
+                  ggml_activations: bool = False) -> np.ndarray:
+    """One matmul kernel on host data; ggml_activations: the rows are converted as ggml's CPU matmul does."""
     lib = load_library()
+    use_tiles = int(use_tiles) | (0x100 if ggml_activations else 0)
     raw = np.ascontiguousarray(raw, np.uint8)
     x = np.ascontiguousarray(x, np.float32)
     T = x.shape[0]

@@ -6,8 +6,50 @@ import oracle
 from gguf_reader import Reader
 
 
+F32, F16, Q8_0, Q4_K, BF16, MXFP4 = 0, 1, 8, 12, 30, 39
+
+
+def ggml_activations(v, weight_type):
+    """The rows of v as ggml's CPU matmul multiplies them with a weight of this
+    type: re-quantised to Q8_K (Q4_K weights; blocks of 256, the first value of
+    largest magnitude maps to -127, codes rounded half to even and capped at
+    127), to Q8_0 (Q8_0 and MXFP4 weights; blocks of 32, scale amax / 127 kept
+    as f16, codes rounded half away from zero with the unrounded scale), or
+    rounded to f16 (F16 weights). Written with numpy's float32 arithmetic,
+    independently of oracle/model.hpp."""
+    x = np.asarray(v, np.float32)
+    f32 = np.float32
+    if weight_type == Q4_K:
+        b = x.reshape(-1, 256)
+        first = np.abs(b).argmax(-1)                      # argmax returns the first maximum
+        mx = b[np.arange(len(b)), first]
+        out = np.zeros_like(b)
+        nz = mx != 0
+        iscale = (f32(-127.0) / mx[nz]).astype(f32)
+        codes = np.minimum(np.rint((b[nz] * iscale[:, None]).astype(f32)), 127)
+        out[nz] = ((f32(1.0) / iscale).astype(f32)[:, None] * codes.astype(f32)).astype(f32)
+        return out.reshape(x.shape).astype(np.float64)
+    if weight_type in (Q8_0, MXFP4):
+        b = x.reshape(-1, 32)
+        d = (np.abs(b).max(-1) / f32(127.0)).astype(f32)
+        inv = np.where(d != 0, f32(1.0) / np.where(d != 0, d, f32(1.0)), f32(0.0)).astype(f32)
+        scaled = (b * inv[:, None]).astype(f32)
+        codes = np.sign(scaled) * np.floor(np.abs(scaled) + f32(0.5))
+        out = d.astype(np.float16).astype(f32)[:, None] * codes.astype(f32)
+        return out.reshape(x.shape).astype(np.float64)
+    if weight_type == F16:
+        return x.astype(np.float16).astype(np.float64)
+    if weight_type == BF16:
+        u = x.view(np.uint32).astype(np.uint64)
+        u = (u + 0x7fff + ((u >> 16) & 1)) & 0xffff0000
+        return u.astype(np.uint32).view(np.float32).reshape(x.shape).astype(np.float64)
+    return np.asarray(v, np.float64)
+
+
 class NumpyModel:
-    def __init__(self, path):
+    def __init__(self, path, activations="exact"):
+        """activations: "exact" (the f32 values are multiplied) or "ggml" (converted first)."""
+        self.ggml = activations == "ggml"
         r = Reader(path)
         self.r = r
         a = r.kv["general.architecture"]
@@ -29,6 +71,9 @@ class NumpyModel:
         if name not in self.w:
             self.w[name] = self.r.dense(name, oracle.decode_row) if name in self.r.tensors else None
         return self.w[name]
+
+    def act(self, name, v):
+        return ggml_activations(v, self.r.tensors[name][1]) if self.ggml else v
 
     def norm(self, x, w):
         return x / np.sqrt((x * x).mean(-1, keepdims=True) + self.eps) * w
@@ -52,16 +97,19 @@ class NumpyModel:
 
     def forward(self, tokens, pos0=0, lora=None):
         """Full causal forward of one sequence; returns logits [T, V].
-        lora: dict name -> (A [r, in], B [out, r], scale*alpha/r)."""
+        lora: dict name -> (A [r, in], B [out, r], scale*alpha/r, storage type of A and B)."""
         T = len(tokens)
         x = self.t("token_embd.weight")[np.asarray(tokens)]
         G = self.H // self.KV
 
         def mm(name, v):
-            y = v @ self.t(name).T
+            y = self.act(name, v) @ self.t(name).T
             if lora and name in lora:
-                A, B, s = lora[name]
-                y = y + s * ((v @ A.T) @ B.T)
+                A, B, s, adapter_type = lora[name]
+                if self.ggml:
+                    y = y + s * (ggml_activations(ggml_activations(v, adapter_type) @ A.T, adapter_type) @ B.T)
+                else:
+                    y = y + s * ((v @ A.T) @ B.T)
             return y
 
         for l in range(self.L):
@@ -96,13 +144,13 @@ class NumpyModel:
         head = self.t("output.weight")
         if head is None:
             head = self.t("token_embd.weight")
-        logits = h @ head.T
+        logits = self.act("output.weight" if self.t("output.weight") is not None else "token_embd.weight", h) @ head.T
         if self.t("output.bias") is not None:
             logits = logits + self.t("output.bias")
         return logits
 
     def moe(self, b, h):
-        router = h @ self.t(b + "ffn_gate_inp.weight").T
+        router = self.act(b + "ffn_gate_inp.weight", h) @ self.t(b + "ffn_gate_inp.weight").T
         p = np.exp(router - router.max(-1, keepdims=True))
         p /= p.sum(-1, keepdims=True)
         Wg, Wu, Wd = self.t(b + "ffn_gate_exps.weight"), self.t(b + "ffn_up_exps.weight"), self.t(b + "ffn_down_exps.weight")
@@ -111,6 +159,6 @@ class NumpyModel:
             top = np.argsort(-p[t], kind="stable")[:self.n_used]
             wsum = p[t, top].sum()
             for e in top:
-                g, u = Wg[e] @ h[t], Wu[e] @ h[t]
-                out[t] += p[t, e] / wsum * (Wd[e] @ (g / (1 + np.exp(-g)) * u))
+                g, u = Wg[e] @ self.act(b + "ffn_gate_exps.weight", h[t]), Wu[e] @ self.act(b + "ffn_up_exps.weight", h[t])
+                out[t] += p[t, e] / wsum * (Wd[e] @ self.act(b + "ffn_down_exps.weight", g / (1 + np.exp(-g)) * u))
         return out

@@ -1,10 +1,13 @@
 """Kernel-level parity on the GPU, through the C ABI of include/retro_kernels.h.
 
 Reference values come from the CPU oracle's block decoders: the same stored
-bytes decoded on the host, multiplied in float64 with the f32
-activations (the kernels carry them as f16 hi/lo pairs, about 22 bits).
-Tolerance: exact products accumulated in f32, so 2e-5 of the output scale
-covers them."""
+bytes decoded on the host, multiplied in float64 with the f32 activations (the
+kernels carry them as f16 hi/lo pairs, about 22 bits) or, under the ggml
+arithmetic, with the activations as ggml's CPU matmul converts them for that
+weight type (Q8_K / Q8_0 codes times their scale, f16 or bf16 rounding; the
+oracle's activation_row). Both sides convert the same f32 inputs, so the
+codes are identical. The products are accumulated in f32: 2e-5 of the output
+scale covers that."""
 import numpy as np
 import pytest
 import torch
@@ -26,31 +29,34 @@ def _weights(t, n, k, seed):
     return raw, dense
 
 
-def _ref(dense, x):
-    # activations travel as f16 hi/lo pairs (~22 bits): the f32 input is the reference
-    return x.astype(np.float64) @ dense.T
+def _ref(t, dense, x, ggml):
+    """ggml: the rows as ggml's CPU matmul converts them for this weight type; else the f32 values."""
+    seen = np.stack([oracle.activation_row(t, row) for row in x]) if ggml else x
+    return seen.astype(np.float64) @ dense.T
 
 
+@pytest.mark.parametrize("ggml", [False, True])
 @pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0])
 @pytest.mark.parametrize("n,k,T", [(16, 256, 1), (48, 512, 7), (64, 1024, 16), (256, 4096, 33),
                                    (4096, 2048, 64), (160, 768, 100), (2064, 256, 3), (96, 1024, 24), (512, 4096, 48)])
-def test_tile_matmul_matches_decoded_blocks(t, n, k, T):
-    print("case", t, n, k, T, flush=True)
+def test_tile_matmul_matches_decoded_blocks(t, n, k, T, ggml):
+    print("case", t, n, k, T, ggml, flush=True)
     raw, dense = _weights(t, n, k, seed=n + k + T)
     x = np.random.default_rng(T).standard_normal((T, k)).astype(np.float32)
-    want = _ref(dense, x)
+    want = _ref(t, dense, x, ggml)
     scale = np.abs(want).max()
     for mode in (1, 2):      # register-only tiles, LDS-staged tiles
-        got = E.kernel_matmul(t, raw, n, k, x, use_tiles=mode)
+        got = E.kernel_matmul(t, raw, n, k, x, use_tiles=mode, ggml_activations=ggml)
         assert np.abs(got - want).max() <= 2e-5 * scale + 1e-6, mode
-    gen = E.kernel_matmul(t, raw, n, k, x, use_tiles=False)
+    gen = E.kernel_matmul(t, raw, n, k, x, use_tiles=False, ggml_activations=ggml)
     assert np.abs(gen - want).max() <= 2e-5 * scale + 1e-6
 
 
+@pytest.mark.parametrize("ggml", [False, True])
 @pytest.mark.parametrize("t,k", [(gw.GGML_F16, 344), (gw.GGML_F32, 100), (gw.GGML_Q8_0, 128),
                                  (gw.GGML_MXFP4, 96), (gw.GGML_Q4_K, 256), (gw.GGML_BF16, 64)])
-def test_generic_matmul_every_storage_type(t, k):
-    print("case", t, k, flush=True)
+def test_generic_matmul_every_storage_type(t, k, ggml):
+    print("case", t, k, ggml, flush=True)
     n, T = 37, 11
     if t == gw.GGML_BF16:
         g = torch.Generator().manual_seed(1)
@@ -60,9 +66,11 @@ def test_generic_matmul_every_storage_type(t, k):
     else:
         raw, dense = _weights(t, n, k, seed=k)
     x = np.random.default_rng(2).standard_normal((T, k)).astype(np.float32)
-    want = _ref(dense, x)
-    got = E.kernel_matmul(t, raw, n, k, x, use_tiles=False)
+    want = _ref(t, dense, x, ggml)
+    got = E.kernel_matmul(t, raw, n, k, x, use_tiles=False, ggml_activations=ggml)
     assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max() + 1e-6
+    if ggml and t in (gw.GGML_F16, gw.GGML_BF16, gw.GGML_Q8_0, gw.GGML_Q4_K, gw.GGML_MXFP4):
+        assert np.abs(want - _ref(t, dense, x, False)).max() > 1e-4 * np.abs(want).max()     # the conversion is visible
 
 
 def test_matmul_bias_and_accumulate():
@@ -72,7 +80,7 @@ def test_matmul_bias_and_accumulate():
     x = rng.standard_normal((T, k)).astype(np.float32)
     bias = rng.standard_normal(n).astype(np.float32)
     y0 = rng.standard_normal((T, n)).astype(np.float32)
-    want = _ref(dense, x)
+    want = _ref(t, dense, x, False)
     for tiles in (2, 1, 0):
         got = E.kernel_matmul(t, raw, n, k, x, use_tiles=tiles, bias=bias)
         assert np.abs(got - (want + bias)).max() <= 3e-5 * np.abs(want).max()
@@ -91,19 +99,25 @@ def test_tile_matmul_exact_on_integer_data():
     blocks[..., 2:4] = np.frombuffer(np.float16(0.25).tobytes(), np.uint8)
     raw = blocks.reshape(n, -1)
     dense = np.stack([oracle.decode_row(gw.GGML_Q4_K, raw[i], k) for i in range(n)]).astype(np.float64)
+    # an extreme of magnitude 127 in every block makes the integers their own Q8_K / Q8_0 codes (scale 1)
     x = rng.integers(-4, 5, (T, k)).astype(np.float32)
+    x[:, ::32] = rng.choice([-127.0, 127.0], (T, k // 32))
+    assert np.array_equal(np.stack([oracle.activation_row(gw.GGML_Q4_K, r) for r in x]), x)
+    assert np.array_equal(np.stack([oracle.activation_row(gw.GGML_Q8_0, r) for r in x]), x)
     want = x.astype(np.float64) @ dense.T
     for mode in (1, 2):
-        got = E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x, use_tiles=mode)
-        assert np.array_equal(got.astype(np.float64), want), mode
+        for ggml in (False, True):
+            got = E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x, use_tiles=mode, ggml_activations=ggml)
+            assert np.array_equal(got.astype(np.float64), want), (mode, ggml)
     q8 = rng.integers(0, 256, (n, k // 32, 34), dtype=np.uint8)
     q8[..., 0:2] = np.frombuffer(np.float16(0.125).tobytes(), np.uint8)
     raw = q8.reshape(n, -1)
     dense = np.stack([oracle.decode_row(gw.GGML_Q8_0, raw[i], k) for i in range(n)]).astype(np.float64)
     want = x.astype(np.float64) @ dense.T
     for mode in (1, 2):
-        got = E.kernel_matmul(gw.GGML_Q8_0, raw, n, k, x, use_tiles=mode)
-        assert np.array_equal(got.astype(np.float64), want), mode
+        for ggml in (False, True):
+            got = E.kernel_matmul(gw.GGML_Q8_0, raw, n, k, x, use_tiles=mode, ggml_activations=ggml)
+            assert np.array_equal(got.astype(np.float64), want), (mode, ggml)
 
 
 @pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0])
@@ -113,7 +127,7 @@ def test_split_k_matmul_is_deterministic_and_exact(t):
     n, k, T = 4096, 4096, 64
     raw, dense = _weights(t, n, k, seed=77)
     x = np.random.default_rng(5).standard_normal((T, k)).astype(np.float32)
-    want = _ref(dense, x)
+    want = _ref(t, dense, x, False)
     a = E.kernel_matmul(t, raw, n, k, x, use_tiles=2)
     b = E.kernel_matmul(t, raw, n, k, x, use_tiles=2)
     assert np.array_equal(a, b)

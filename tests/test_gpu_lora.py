@@ -75,6 +75,31 @@ def test_rows_under_different_adapters_match_the_oracle(files):
     eng.close()
 
 
+def test_rows_under_adapters_with_the_ggml_arithmetic(files, monkeypatch):
+    """RETRO_ACTIVATIONS=ggml: the base weights (Q8_0) multiply the Q8_0 conversion of a row,
+    the F16 LoRA factors the same row rounded to f16 (and B the f16 rounding of A x), as
+    ggml's CPU matmuls do. The criterion is the one of tests/test_gpu_step.py."""
+    model, a1, a2, _ = files
+    monkeypatch.setenv("RETRO_ACTIVATIONS", "ggml")
+    eng = E.Engine(model, E.EngineConfig(n_ctx=1024, n_seq_max=4, n_batch=128, n_ubatch=128))
+    m = oracle.Model(model)
+    ids = [eng.adapter_load(a1, 1.0), eng.adapter_load(a2, 0.5)]
+    assert [m.load_adapter(a1, 1.0), m.load_adapter(a2, 0.5)] == ids
+    rng = np.random.default_rng(3)
+    prompts = [rng.integers(0, m.n_vocab, n) for n in (21, 9, 40, 13)]
+    route = [ids[0], E.RETRO_STEP_ADAPTER_BASE, ids[1], 0]
+    out = E.StepOutput()
+    eng.step([E.StepRow(i, i, prompts[i], 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(route[i])) for i in range(4)], out)
+    got = eng.debug_logits()
+    plan, adapters = [(i, 0, prompts[i], True) for i in range(4)], [route[0], -1, route[2], -1]
+    want = oracle.Context(m, 4, activations="ggml").step_rows(plan, adapters=adapters)
+    exact = oracle.Context(m, 4, activations="exact").step_rows(plan, adapters=adapters)
+    (_, drift), (_, conversion) = logit_errors(got, want), logit_errors(exact, want)
+    print("drift %.2e, conversion %.2e" % (drift, conversion), flush=True)
+    assert drift < 0.6 * conversion, (drift, conversion)
+    eng.close()
+
+
 def test_adapter_errors_and_unload(files):
     model, a1, a2, ffn = files
     print("per-row LoRA: argument errors", flush=True)

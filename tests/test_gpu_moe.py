@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from engine_helpers import assert_logits_close, greedy, run_both
+from engine_helpers import assert_logits_close, greedy, logit_errors, run_both
 from retrograd_amd import engine as E
 from retrograd_amd import gguf_writer as gw
 from retrograd_amd import synth
@@ -42,4 +42,30 @@ def test_moe_prefill_and_decode_match_the_oracle(tmp_path, key):
         out, got, want = run_both(eng, ctx, rows)
         assert_logits_close(got, want)
         pos = [p + 1 for p in pos]
+    eng.close()
+
+
+@pytest.mark.parametrize("key", list(SHAPES))
+def test_moe_under_the_ggml_arithmetic(tmp_path, key, monkeypatch):
+    """RETRO_ACTIVATIONS=ggml: the router (F32) multiplies the rows as they are, the experts
+    their Q8_0 conversion, the hidden rows are converted again for the down projection.
+    End to end the product follows the oracle's ggml arithmetic as closely as rounding-boundary
+    drift allows (tests/test_gpu_step.py explains the criterion): clearly closer than the
+    plain product is."""
+    shape = SHAPES[key]
+    print("mixture of experts, ggml arithmetic: %s" % shape.name, flush=True)
+    path = tmp_path / "moe.gguf"
+    synth.write_model(path, shape, seed=5, device="cpu", std=0.05)
+    monkeypatch.setenv("RETRO_ACTIVATIONS", "ggml")
+    eng = E.Engine(path, E.EngineConfig(n_ctx=2048, n_seq_max=8, n_batch=256, n_ubatch=256))
+    m = oracle.Model(path)
+    rng = np.random.default_rng(2)
+    lens = [7, 40, 65, 18, 3]
+    prompts = [rng.integers(0, m.n_vocab, n) for n in lens]
+    rows = [(i, i, p, 0, True) for i, p in enumerate(prompts)]
+    out, got, want = run_both(eng, oracle.Context(m, 8, activations="ggml"), rows)
+    exact = oracle.Context(m, 8, activations="exact").step_rows([(r[1], r[3], r[2], r[4]) for r in rows])
+    (_, drift), (_, conversion) = logit_errors(got, want), logit_errors(exact, want)
+    print("drift %.2e, conversion %.2e" % (drift, conversion), flush=True)
+    assert drift < 0.6 * conversion, (drift, conversion)
     eng.close()

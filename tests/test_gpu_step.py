@@ -71,6 +71,49 @@ def test_prefill_and_decode_logits_match_oracle(models, key):
     eng.close()
 
 
+@pytest.mark.parametrize("key", list(SMALL))
+def test_ggml_arithmetic_follows_the_oracle_as_closely_as_its_rounding_allows(models, key, monkeypatch):
+    """RETRO_ACTIVATIONS=ggml: activations converted as ggml's CPU matmul does. Per matmul the
+    product and the oracle agree to float rounding (test_gpu_kernels.py). Over a whole forward
+    a value near a rounding boundary takes different codes on the two sides and every later
+    conversion amplifies that, exactly as between the oracle and its float64 restatement
+    (tests/test_oracle_model.py). The yardstick for "as close as rounding allows" is that
+    restatement against itself with its matrices perturbed by 2e-5 relative, the size of an
+    f32 accumulation error: the product must drift from the oracle no further than that,
+    must be clearly closer to the ggml arithmetic than the plain product is, and must pick
+    the same token wherever the margin exceeds the drift."""
+    from ref_transformer import NumpyModel
+    print("model", key, flush=True)
+    monkeypatch.setenv("RETRO_ACTIVATIONS", "ggml")
+    eng = E.Engine(models[key], E.EngineConfig(n_ctx=2048, n_seq_max=8, n_batch=256, n_ubatch=256))
+    m = oracle.Model(models[key])
+    ggml_ctx, exact_ctx = oracle.Context(m, 8, activations="ggml"), oracle.Context(m, 8, activations="exact")
+    rng = np.random.default_rng(1)
+    lens = [5, 33, 64, 17]
+    prompts = [rng.integers(0, m.n_vocab, n) for n in lens]
+    rows = [(i, i, p, 0, True) for i, p in enumerate(prompts)]
+    out, got, want = run_both(eng, ggml_ctx, rows)
+    exact = exact_ctx.step_rows([(r[1], r[3], r[2], r[4]) for r in rows])
+    drift_max, drift = logit_errors(got, want)
+    _, conversion = logit_errors(exact, want)
+    clean, noisy = NumpyModel(models[key], activations="ggml"), NumpyModel(models[key], activations="ggml")
+    noise = np.random.default_rng(7)
+    for name in noisy.r.tensors:
+        w = noisy.t(name)
+        if w is not None and w.ndim >= 2:
+            noisy.w[name] = w * (1 + 2e-5 * noise.standard_normal(w.shape))
+    a = np.stack([clean.forward(p)[-1] for p in prompts])
+    b = np.stack([noisy.forward(p)[-1] for p in prompts])
+    _, yardstick = logit_errors(b, a)
+    print("drift %.2e (max %.2e), yardstick %.2e, conversion %.2e" % (drift, drift_max, yardstick, conversion), flush=True)
+    assert drift <= yardstick and drift < 0.6 * conversion, (drift, yardstick, conversion)
+    for i, r in enumerate(out.rows()):
+        srt = np.sort(want[i])[::-1]
+        if srt[0] - srt[1] > 4 * drift_max:
+            assert r.token == int(want[i].argmax())
+    eng.close()
+
+
 def test_packing_is_bit_exact_with_the_oracle(models):
     eng, ctx, m = _pair(models["llama-q4k"], n_seq=8, n_ctx=1024, n_batch=128)
     rng = np.random.default_rng(2)

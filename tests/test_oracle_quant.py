@@ -151,3 +151,85 @@ def test_synthetic_quantisers_round_trip_close():
             y = oracle.decode_row(t, raw[r], 512)
             err = np.abs(y - x[r].numpy()).max() / np.abs(x[r].numpy()).max()
             assert err < tol, (t, err)
+
+
+# ---- the activations of a matmul as ggml's CPU path sees them -------------------------
+
+Q8_K_WEIGHT, Q8_0_WEIGHT = 12, 8          # Q4_K and Q8_0 weights: Q8_K and Q8_0 activations
+
+
+def test_q8_k_activations_hand_computed():
+    # ggml quantize_row_q8_K_ref: the first value of largest magnitude maps to -127
+    x = np.zeros(256, np.float32)
+    x[:5] = [1.0, -2.0, 0.5, 2.0, 62.5 / 63.5]
+    got = oracle.activation_row(Q8_K_WEIGHT, x)
+    iscale = np.float32(-127.0) / np.float32(-2.0)           # 63.5
+    d = np.float32(1.0) / iscale
+    # 63.5 ties to the even 64; 31.75 -> 32; the opposite extreme reaches +127 (the cap); 62.5 ties to the even 62
+    want = np.array([64, -127, 32, 127, 62], np.float32) * d
+    assert np.array_equal(got[:5], want)
+    assert not got[5:].any()
+    # the sign of the scale follows the FIRST extreme; the values it stands for are the same
+    y = x.copy()
+    y[1], y[3] = 2.0, -2.0
+    got2 = oracle.activation_row(Q8_K_WEIGHT, y)
+    assert np.array_equal(got2[[1, 3]], [2.0, -2.0]) and np.array_equal(got2[[0, 2, 4]], got[[0, 2, 4]])
+    # an all-zero block stays zero, blocks are independent
+    z = np.zeros(512, np.float32)
+    z[256:261] = x[:5] * 3
+    got3 = oracle.activation_row(Q8_K_WEIGHT, z)
+    assert not got3[:256].any() and np.allclose(got3[256:261], want * 3, rtol=1e-6)
+
+
+def test_q8_0_activations_are_the_fixture_pinned_quantiser():
+    # the Q8_0 row quantiser that reproduces the reference's fixture digests, decoded again
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal(32 * 64) * 2).astype(np.float32)
+    x[:32] = 0
+    via_blocks = oracle.decode_row(8, oracle.quantize_q8_0(x), x.size)
+    assert np.array_equal(oracle.activation_row(Q8_0_WEIGHT, x), via_blocks)
+    assert np.array_equal(oracle.activation_row(39, x), via_blocks)        # MXFP4 weights take Q8_0 activations too
+    # half away from zero: 2.5 -> 3 with scale 1 (amax 127)
+    v = np.zeros(32, np.float32)
+    v[:4] = [127.0, 2.5, -2.5, 1.4]
+    assert np.array_equal(oracle.activation_row(Q8_0_WEIGHT, v)[:4], [127.0, 3.0, -3.0, 1.0])
+
+
+def test_activation_conversion_against_the_numpy_restatement():
+    from ref_transformer import ggml_activations
+    rng = np.random.default_rng(0)
+    for wt in (0, 1, 8, 12, 30, 39):
+        for i in range(60):
+            x = (rng.standard_normal(512) * rng.choice([1e-3, 1.0, 50.0])).astype(np.float32)
+            if i % 7 == 0:
+                x[rng.integers(0, 512, 300)] = 0
+            assert np.array_equal(oracle.activation_row(wt, x).astype(np.float64), ggml_activations(x, wt)), (wt, i)
+    x = rng.standard_normal(64).astype(np.float32)
+    assert np.array_equal(oracle.activation_row(0, x), x)                   # F32 weights: untouched
+    assert np.array_equal(oracle.activation_row(1, x), x.astype(np.float16).astype(np.float32))
+
+
+def test_matmul_on_grid_activations_is_the_plain_product():
+    # integers with an extreme of 127 in every block are their own codes (scale 1): nothing is lost
+    rng = np.random.default_rng(1)
+    k, n = 512, 24
+    x = rng.integers(-127, 128, (3, k)).astype(np.float32)
+    x[:, ::32] = 127
+    for wt in (8, 12):
+        w = (rng.standard_normal((n, k)) * 0.1).astype(np.float32)
+        raw = synth_quantise(wt, w)
+        dense = np.stack([oracle.decode_row(wt, raw[i], k) for i in range(n)]).astype(np.float64)
+        got = oracle.matmul(wt, raw, n, k, x)
+        assert np.abs(got - x.astype(np.float64) @ dense.T).max() < 1e-4
+    # and off the grid the product is that of the converted activations
+    xf = rng.standard_normal((3, k)).astype(np.float32)
+    conv = np.stack([oracle.activation_row(12, r) for r in xf]).astype(np.float64)
+    got = oracle.matmul(12, raw, n, k, xf)
+    assert np.abs(got - conv @ dense.T).max() < 1e-5
+    assert np.abs(got - xf.astype(np.float64) @ dense.T).max() > 1e-3
+
+
+def synth_quantise(wt, w):
+    import torch
+    from retrograd_amd import synth
+    return np.asarray(synth.encode(torch.from_numpy(w), wt)).reshape(w.shape[0], -1)

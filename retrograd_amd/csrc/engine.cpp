@@ -853,7 +853,8 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
             set_error("step row slot is outside the context's sequence range");
             return -3;
         }
-        if (row.adapter != 0 && row.adapter != RETRO_STEP_ADAPTER_BASE && !row_adapters_.count(row.adapter)) {
+        if (row.adapter != 0 && row.adapter != RETRO_STEP_ADAPTER_BASE
+                && (row.adapter == kPolicyAdapter || !row_adapters_.count(row.adapter))) {
             set_error("step row adapter " + std::to_string(row.adapter) + " is not a loaded per-row adapter");
             return -3;
         }
@@ -996,8 +997,12 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
             hd[r].sample = row.sample ? 1 : 0; hd[r].kv_begin = slots_[(size_t)row.slot].begin;
             // route = 1-based index of the adapter in id order (0: the base model)
             hd[r].route = 0; hd[r].pad = 0;
-            if (row.adapter > 0) {
-                hd[r].route = 1 + (int32_t)std::distance(row_adapters_.begin(), row_adapters_.find(row.adapter));
+            // adapter 0 follows the context: its default adapter, else the trained adapter when there is one
+            int32_t eff = row.adapter;
+            if (eff == 0) eff = default_adapter_ != 0 ? default_adapter_ : kPolicyAdapter;
+            const auto found = eff > 0 ? row_adapters_.find(eff) : row_adapters_.end();
+            if (found != row_adapters_.end()) {
+                hd[r].route = 1 + (int32_t)std::distance(row_adapters_.begin(), found);
                 routed = true;
             }
             std::memcpy(ht + at, row.tokens, (size_t)row.n * 4);
@@ -1298,10 +1303,110 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
 // adapter.lora.alpha, tensors "<weight>.lora_a" ne = [n_in, r] and
 // "<weight>.lora_b" ne = [r, n_out].
 int Engine::adapter_load(const std::string & path, float scale, int32_t * out_id) {
-    if (next_adapter_id_ == INT32_MAX) {
+    if (next_adapter_id_ == kPolicyAdapter) {
         set_error("per-row adapter ids are exhausted");
         return -1;
     }
+    RowAdapterData data;
+    if (read_adapter(path, scale, data) != 0) return -1;
+    const int32_t id = next_adapter_id_++;
+    row_adapters_.emplace(id, std::move(data));
+    rebuild_lora_table();
+    *out_id = id;
+    return 0;
+}
+
+// The trained adapter of a trainer's generation context: what rows with adapter 0
+// decode under until set_default_adapter() says otherwise. Replaces the one before.
+int Engine::policy_adapter_load(const std::string & path) {
+    RowAdapterData data;
+    if (read_adapter(path, 1.0f, data) != 0) return -1;
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    row_adapters_.erase(kPolicyAdapter);
+    row_adapters_.emplace(kPolicyAdapter, std::move(data));
+    rebuild_lora_table();
+    return 0;
+}
+
+// A frozen device-to-device copy of the trained adapter as a per-row adapter
+// (reference retro_rollout.cpp:184-244).
+int Engine::adapter_snapshot(int32_t replace, float scale, int32_t * out_id) {
+    if (!std::isfinite(scale)) {
+        set_error("the adapter scale must be finite");
+        return -1;
+    }
+    auto policy = row_adapters_.find(kPolicyAdapter);
+    if (policy == row_adapters_.end()) {
+        set_error("a snapshot copies the trained LoRA adapter, and the trainer has none");
+        return -1;
+    }
+    if (replace != 0) {
+        if (replace == kPolicyAdapter || !row_adapters_.count(replace)) {
+            set_error("no per-row adapter is loaded under id " + std::to_string(replace));
+            return -1;
+        }
+        if (default_adapter_ == replace) {
+            default_adapter_ = 0;
+            forget_generation_bookkeeping();
+        }
+        hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+        row_adapters_.erase(replace);       // freed before the copy is made: a refresh never holds two snapshots
+    }
+    if (next_adapter_id_ == kPolicyAdapter) {
+        set_error("per-row adapter ids are exhausted");
+        return -1;
+    }
+    const RowAdapterData & src = policy->second;
+    RowAdapterData copy;
+    copy.scale = scale;
+    copy.alpha = src.alpha;
+    copy.rank = src.rank;
+    copy.elements = src.elements;
+    copy.a_type = src.a_type;
+    copy.b_type = src.b_type;
+    copy.a.resize(src.a.size());
+    copy.b.resize(src.b.size());
+    for (size_t i = 0; i < src.a.size(); ++i) {
+        if (!src.a[i].ptr) continue;
+        copy.a[i].alloc(src.a[i].bytes);
+        copy.b[i].alloc(src.b[i].bytes);
+        hip_check(hipMemcpyAsync(copy.a[i].ptr, src.a[i].ptr, src.a[i].bytes, hipMemcpyDeviceToDevice, stream_), "hipMemcpyAsync");
+        hip_check(hipMemcpyAsync(copy.b[i].ptr, src.b[i].ptr, src.b[i].bytes, hipMemcpyDeviceToDevice, stream_), "hipMemcpyAsync");
+    }
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    const int32_t id = next_adapter_id_++;
+    row_adapters_.emplace(id, std::move(copy));
+    rebuild_lora_table();
+    *out_id = id;
+    return 0;
+}
+
+// What rows with adapter 0 - and with them the batched generators - decode under:
+// 0 the trained adapter (the base model when there is none), RETRO_STEP_ADAPTER_BASE
+// the base model, or a per-row adapter id (reference retro_rollout.cpp:283-303).
+int Engine::set_default_adapter(int32_t adapter) {
+    if (adapter < RETRO_STEP_ADAPTER_BASE || adapter == kPolicyAdapter
+            || (adapter > 0 && !row_adapters_.count(adapter))) {
+        set_error("adapter " + std::to_string(adapter) + " is not a loaded per-row adapter");
+        return -1;
+    }
+    if (default_adapter_ != adapter) {
+        default_adapter_ = adapter;
+        // the generators' prefix bookkeeping does not know which adapter a resident prefix was decoded under
+        forget_generation_bookkeeping();
+    }
+    return 0;
+}
+
+// Every cell of the pool and the generators' bookkeeping: what a change of the
+// weights leaves behind is no prefix of the new model (reference retro_runtime.hpp:515-523).
+void Engine::forget_generation_kv() {
+    clear_generation_memory();
+    forget_generation_bookkeeping();
+    weights_version_ += 1;
+}
+
+int Engine::read_adapter(const std::string & path, float scale, RowAdapterData & data) {
     std::unique_ptr<GgufFile> file;
     try {
         file.reset(new GgufFile(path));
@@ -1317,7 +1422,7 @@ int Engine::adapter_load(const std::string & path, float scale, int32_t * out_id
     const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim;
     static const char * kTargets[kLoraTargets] = {"attn_q", "attn_k", "attn_v", "attn_output"};
     const int n_in[kLoraTargets] = {E, E, E, QD}, n_out[kLoraTargets] = {QD, KD, KD, E};
-    RowAdapterData data;
+    data = RowAdapterData();
     data.scale = scale;
     data.alpha = file->get_float("adapter.lora.alpha", 0.0);
     data.a.resize((size_t)h.n_layer * kLoraTargets);
@@ -1381,18 +1486,18 @@ int Engine::adapter_load(const std::string & path, float scale, int32_t * out_id
         set_error("failed to load LoRA adapter: " + path + " holds no LoRA tensor pair");
         return -1;
     }
-    const int32_t id = next_adapter_id_++;
-    row_adapters_.emplace(id, std::move(data));
-    rebuild_lora_table();
-    *out_id = id;
     return 0;
 }
 
 int Engine::adapter_unload(int32_t id) {
     auto it = row_adapters_.find(id);
-    if (it == row_adapters_.end()) {
+    if (id == kPolicyAdapter || it == row_adapters_.end()) {
         set_error("no per-row adapter is loaded under id " + std::to_string(id));
         return -1;
+    }
+    if (default_adapter_ == id) {
+        default_adapter_ = 0;
+        forget_generation_bookkeeping();
     }
     hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
     row_adapters_.erase(it);
@@ -1435,10 +1540,12 @@ void Engine::adapter_rows_info(retro_adapter_rows_info * out) const {
     *out = retro_adapter_rows_info{};
     out->struct_size = sizeof(retro_adapter_rows_info);
     uint32_t max_rank = 0;
-    for (const auto & kv : row_adapters_) max_rank = std::max<uint32_t>(max_rank, (uint32_t)kv.second.rank);
-    out->n_adapters = (uint32_t)row_adapters_.size();
+    for (const auto & kv : row_adapters_)
+        if (kv.first != kPolicyAdapter) max_rank = std::max<uint32_t>(max_rank, (uint32_t)kv.second.rank);
+    out->n_adapters = (uint32_t)(row_adapters_.size() - row_adapters_.count(kPolicyAdapter));
     out->max_rank = max_rank;
     for (const auto & kv : row_adapters_) {
+        if (kv.first == kPolicyAdapter) continue;
         out->stacked_bytes += kv.second.elements * max_rank * 4;
         out->unpadded_bytes += kv.second.elements * (uint64_t)kv.second.rank * 4;
     }

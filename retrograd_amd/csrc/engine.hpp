@@ -124,6 +124,18 @@ public:
     // Per-row LoRA adapters (reference retro_engine.cpp:872-960): ids start at 1
     // and are never reused; loading leaves the resident KV alone.
     int adapter_load(const std::string & path, float scale, int32_t * out_id);
+    // Rows of token_embd.weight of a model file, read from its header alone.
+    static uint64_t vocab_size_of(const std::string & path) {
+        GgufFile file(path);
+        return (uint64_t)file.require("token_embd.weight").ne[1];
+    }
+    // the generation side of a trainer handle
+    int policy_adapter_load(const std::string & path);
+    bool has_policy_adapter() const { return row_adapters_.count(kPolicyAdapter) != 0; }
+    int adapter_snapshot(int32_t replace, float scale, int32_t * out_id);
+    int set_default_adapter(int32_t adapter);
+    int32_t default_adapter() const { return default_adapter_; }
+    void forget_generation_kv();
     int adapter_unload(int32_t id);
     void adapter_rows_info(retro_adapter_rows_info * out) const;
 
@@ -256,6 +268,10 @@ private:
     int lora_routes_ = 0;
     bool ggml_activations_ = false;   // RETRO_ACTIVATIONS=ggml at construction
     void rebuild_lora_table();
+    int read_adapter(const std::string & path, float scale, RowAdapterData & data);
+    // id of the trained adapter among the per-row adapters: never handed out, never accepted from a caller
+    static constexpr int32_t kPolicyAdapter = INT32_MAX;
+    int32_t default_adapter_ = 0;
     const rk::LoraEntry * lora_entries(int layer, int target) const {
         return lora_table_.as<rk::LoraEntry>() + ((size_t)layer * kLoraTargets + target) * (size_t)lora_routes_;
     }

@@ -11,6 +11,7 @@ from pathlib import Path
 import pytest
 
 from retrograd_amd import engine as E
+from retrograd_amd import trainer as T
 
 ROOT = Path(__file__).resolve().parent.parent
 
@@ -33,6 +34,13 @@ EXPECT = [
                                       "sampled": 17, "sampled_logprob": 20}),
     ("retro_engine_memory_info", 40, 8, {"struct_size": 0, "n_slots": 4, "cells_total": 8, "cells_used": 16,
                                          "kv_bytes": 24, "recurrent_bytes": 32}),
+    # the reference's own layout assertions for RetroTrainConfig (crates/retrograd-ffi/src/lib.rs:2835-2880)
+    ("retro_train_config", 176, 8, {"generation_concurrency": 16, "kv_dtype": 24, "learning_rate": 36, "warmup_steps": 56,
+                                    "device": 68, "chunked_ce_seq_chunk": 80, "chunked_ce_offload_logsoftmax": 84,
+                                    "checkpoint_every_n_layers": 88, "checkpoint_dtype": 92, "require_gpu_resident": 96,
+                                    "generation_batch": 100, "shuffle_dataset": 104, "optimizer": 108,
+                                    "shuffle_seed": 112, "trainable": 120, "muon_momentum": 124, "muon_ns_steps": 136,
+                                    "muon_nesterov": 140, "gefen_variant": 144}),
     ("retro_engine_config", 64, 8, {"struct_size": 0, "n_ctx": 4, "n_seq_max": 8, "n_batch": 12, "n_ubatch": 16,
                                     "kv_dtype": 20, "flash_attn": 24, "device": 28, "threads": 32, "verbose": 36,
                                     "kv_unified": 40, "expert_placement": 44, "expert_host_layers": 48,
@@ -44,12 +52,13 @@ CTYPES = {
     "retro_adapter_rows_info": E.CAdapterRowsInfo, "retro_step_out_row": E.CStepOutRow,
     "retro_sampling_params_v2": E.CSamplingParamsV2, "retro_step_row_v2": E.CStepRowV2,
     "retro_step_out_row_v2": E.CStepOutRowV2, "retro_engine_memory_info": E.CEngineMemoryInfo,
-    "retro_engine_config": E.CEngineConfig,
+    "retro_engine_config": E.CEngineConfig, "retro_train_config": T.CTrainConfig,
 }
 
 
 def test_c_header_layout_matches_the_reference_abi(tmp_path):
-    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "retro_step.h"', "int main(void) {"]
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "retro_step.h"', '#include "retro_trainer.h"',
+             "int main(void) {"]
     for name, size, align, fields in EXPECT:
         lines.append('printf("%s %%zu %%zu\\n", sizeof(%s), _Alignof(%s));' % (name, name, name))
         for f in fields:
@@ -90,6 +99,10 @@ def test_library_exports_every_declared_symbol():
     kern = [s for s in _declared(ROOT / "include" / "retro_kernels.h") if s not in step]
     sched = [s for s in _declared(ROOT / "include" / "retro_scheduler.h") if s not in step]
     from retrograd_amd import scheduler as S
+    trainer = [s for s in _declared(ROOT / "include" / "retro_trainer.h") if s not in step]
+    assert sorted(trainer) == sorted(T.TRAINER_SYMBOLS)
+    for sym in trainer:
+        assert hasattr(lib, sym), sym
     assert sorted(step) == sorted(E.STEP_SYMBOLS)
     assert sorted(kern) == sorted(E.KERNEL_SYMBOLS)
     assert sorted(sched) == sorted(S.SCHED_SYMBOLS)
@@ -137,3 +150,30 @@ def test_engine_creation_fails_loudly_without_a_gpu(tmp_path):
     with pytest.raises(E.RuntimeFailure) as err:
         E.Engine(p)
     assert "no HIP device" in str(err.value) or "HIP" in str(err.value)
+
+
+def test_trainer_creation_checks_its_configuration_and_fails_loudly_without_a_gpu(tmp_path):
+    from retrograd_amd import synth
+    lib = T._library()
+    cfg = T.TrainConfig(n_ctx=64, n_batch=64, generation_concurrency=0).to_ffi()
+    assert not lib.retro_trainer_new(b"/nonexistent.gguf", C.byref(cfg))
+    assert E.last_error() == "generation_concurrency must be between 1 and 256"
+    cfg = T.TrainConfig(n_ctx=64, n_batch=8, generation_concurrency=16).to_ffi()
+    assert not lib.retro_trainer_new(b"/nonexistent.gguf", C.byref(cfg))
+    assert E.last_error() == "generation_concurrency must not exceed n_batch"
+    cfg = T.TrainConfig(n_ctx=64, n_batch=64, generation_kv_dtype=1, fast_generation_context=False).to_ffi()
+    assert not lib.retro_trainer_new(b"/nonexistent.gguf", C.byref(cfg))
+    assert E.last_error() == "a quantized generation_kv_dtype requires fast_generation_context"
+    cfg = T.TrainConfig(n_ctx=64, n_batch=64, device=E.DEVICE_CPU).to_ffi()
+    assert not lib.retro_trainer_new(b"/nonexistent.gguf", C.byref(cfg))
+    assert "only executes on an MI355X GPU" in E.last_error()
+    assert not lib.retro_trainer_new(None, C.byref(cfg)) and E.last_error() == "model_path is required"
+    out = C.c_uint64()
+    assert lib.retro_trainer_generation_weights_version(None, C.byref(out)) == -1
+    assert E.last_error() == "trainer is required"
+    import torch
+    if not torch.cuda.is_available():
+        path = tmp_path / "m.gguf"
+        synth.write_model(path, synth.TINY_LLAMA, seed=1, device="cpu", std=0.02)
+        with pytest.raises(E.RuntimeFailure, match="no HIP device"):
+            T.Trainer(path, T.TrainConfig(n_ctx=64, n_batch=64, generation_concurrency=2))

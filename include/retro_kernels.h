@@ -35,9 +35,11 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
 
 /* Micro-benchmark: microseconds per launch of one tile matmul (mode 1 register
  * tiles, 2 LDS-staged tiles, 3 the same with the K-slices left to the
- * consumer) over `iters` back-to-back launches on device-only data. Adding 16
- * to the mode gives every launch another copy of the weights (1 GiB of copies
- * in turn), so that they are read from HBM as in a decode step instead of from
+ * consumer) over `iters` back-to-back launches on device-only data: weight
+ * codes and activations are pseudo-random (constant operands let the pipes
+ * clock higher and flatter the kernel by 15-20 %). Adding 16 to the mode gives
+ * every launch another copy of the weights (1 GiB of copies in turn; adding 32,
+ * 6 GiB), so that they are read from HBM as in a decode step instead of from
  * the last-level cache. debug and force_ksplit are timing experiments
  * (0 = normal). */
 int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,

@@ -5,6 +5,7 @@
 #include <algorithm>
 #include "../../include/retro_kernels.h"
 #include "engine.hpp"
+#include <vector>
 
 #include <cstring>
 
@@ -121,15 +122,33 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
         const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
         // mode bit 4: every launch reads another copy of the weights, 1 GiB of them in turn,
         // so that they come from HBM as in a decode step and not from the last-level cache
-        const bool cold = (mode & 16) != 0;
+        // mode bit 5: 6 GiB of copies instead (more address space than a decode step's weights)
+        const bool cold = (mode & 48) != 0;
+        const size_t span = (mode & 32) ? (size_t)6 << 30 : (size_t)1 << 30;
         mode &= 15;
-        const size_t copies = cold ? std::max<size_t>(2, ((size_t)1 << 30) / bytes) : 1;
+        const size_t copies = cold ? std::max<size_t>(2, span / bytes) : 1;
         DevBuf d_w, d_xh, d_sums, d_y, d_ws;
         d_w.alloc(bytes * copies);
-        ok(hipMemset(d_w.ptr, 0x11, bytes * copies), "fill");
         d_xh.alloc(rk::act_halves(n_tokens, (int)k) * 2);
         d_sums.alloc(rk::act_sum_halves(n_tokens, (int)k) * 2);
-        ok(hipMemset(d_xh.ptr, 0, d_xh.bytes), "fill"); ok(hipMemset(d_sums.ptr, 0, d_sums.bytes), "fill");
+        {
+            // Pseudo-random codes and activations: how fast the matrix pipes may clock depends on how many
+            // bits toggle, so constant operands would flatter the kernel. Every fourth byte pair that could
+            // be a block scale is kept a small finite f16.
+            std::vector<uint8_t> host(bytes);
+            uint32_t state = 0x9e3779b9u;
+            for (size_t i = 0; i < bytes; ++i) { state = state * 1664525u + 1013904223u; host[i] = (uint8_t)(state >> 24); }
+            const size_t blk = type == rk::WT_Q4_K ? 144 : 34;
+            for (size_t i = 0; i + 4 <= bytes; i += blk) { host[i] = 0x1f; host[i + 1] = 0x21; host[i + 2] = 0x1f; host[i + 3] = 0x21; }
+            for (size_t c = 0; c < copies; ++c) ok(hipMemcpy(d_w.as<uint8_t>() + c * bytes, host.data(), bytes, hipMemcpyHostToDevice), "fill");
+            std::vector<uint16_t> xs(d_xh.bytes / 2);
+            for (size_t i = 0; i < xs.size(); ++i) {
+                state = state * 1664525u + 1013904223u;
+                xs[i] = (uint16_t)(((state >> 16) & 0x83ffu) | 0x3800u);       // +-[0.5, 1)
+            }
+            ok(hipMemcpy(d_xh.ptr, xs.data(), d_xh.bytes, hipMemcpyHostToDevice), "fill");
+            ok(hipMemset(d_sums.ptr, 0, d_sums.bytes), "fill");
+        }
         d_y.alloc((size_t)n_tokens * n_rows * 4);
         d_ws.alloc(rk::matmul_workspace_bytes());
         ok(hipMemset(d_ws.ptr, 0, d_ws.bytes), "fill");

@@ -113,7 +113,7 @@ inline int nearest_int(float v) { return (int)std::nearbyint(v); }
 // (ggml-cpu.c of ggml-org/llama.cpp@cd8427d0, the base the reference's fork pins in
 // crates/retrograd-ffi/runtime/llama.cpp.lock:6-7; the submodule itself is absent)
 // converts every f32 activation row to the weight type's vec_dot_type and the
-// dot product runs on that: Q4_K -> Q8_K, Q8_0 and MXFP4 -> Q8_0, F16 -> F16,
+// dot product runs on that: Q4_K and Q6_K -> Q8_K, Q8_0 and MXFP4 -> Q8_0, F16 -> F16,
 // BF16 -> BF16, F32 -> F32 (type_traits_cpu). This writes the converted row back
 // as the f32 values it stands for (scale times code).
 //   Q8_K (quantize_row_q8_K_ref): per 256 values, `max` is the first value of
@@ -125,7 +125,8 @@ inline int nearest_int(float v) { return (int)std::nearbyint(v); }
 inline void ggml_activation_row(uint32_t wtype, const float * x, size_t K, float * out) {
     if (exact_activations()) { std::copy(x, x + K, out); return; }
     switch (wtype) {
-        case T_Q4_K: {
+        case T_Q4_K:
+        case T_Q6_K: {
             if (K % 256) throw std::runtime_error("oracle: Q8_K activations need K % 256 == 0");
             for (size_t b = 0; b < K; b += 256) {
                 float amax = 0.0f, max = 0.0f;

@@ -23,7 +23,7 @@ namespace oracle {
 
 // ggml type ids as stored in a GGUF tensor table.
 enum ggml_type_id : uint32_t {
-    T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_BF16 = 30, T_MXFP4 = 39,
+    T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_BF16 = 30, T_MXFP4 = 39,
 };
 
 struct block_geom { uint32_t elements; uint32_t bytes; };
@@ -36,6 +36,7 @@ inline block_geom geom_of(uint32_t type) {
         case T_Q8_0:  return {32, 34};
         case T_MXFP4: return {32, 17};
         case T_Q4_K:  return {256, 144};
+        case T_Q6_K:  return {256, 210};
         default: throw std::runtime_error("oracle: unsupported ggml type " + std::to_string(type));
     }
 }
@@ -180,6 +181,25 @@ inline void decode_row(uint32_t type, const uint8_t * src, size_t n, float * out
                         y[64 * pair + l]      = d1 * (float)(q[l] & 0x0f) - mm1;
                         y[64 * pair + 32 + l] = d2 * (float)(q[l] >> 4) - mm2;
                     }
+                }
+            }
+            return;
+        case T_Q6_K:  // quant.rs:444-464: ql[128] | qh[64] | scales[16] (i8) | d (f16)
+            // Element e of a block: half = e / 128, group g = (e % 128) / 32, l = e % 32. Its low four bits
+            // are a nibble of ql[64 half + l + 32 (g & 1)] (the high nibble for g >= 2), its top two bits
+            // are bits 2g, 2g + 1 of qh[32 half + l]; the code is that six-bit number minus 32, the scale
+            // is scales[8 half + 2 g + l / 16], and the value is (d * scale) * code.
+            for (size_t b = 0; b < n / 256; ++b) {
+                const uint8_t * blk = src + b * 210;
+                const float d = half_to_float(rd16(blk + 208));
+                for (int e = 0; e < 256; ++e) {
+                    const int half = e >> 7, g = (e & 127) >> 5, l = e & 31;
+                    const uint8_t lo = blk[64 * half + l + 32 * (g & 1)];
+                    const int nib = g >= 2 ? (lo >> 4) : (lo & 0x0f);
+                    const int top = (blk[128 + 32 * half + l] >> (2 * g)) & 3;
+                    const int code = (nib | (top << 4)) - 32;
+                    const float scale = (float)(int8_t)blk[192 + 8 * half + 2 * g + (l >> 4)];
+                    out[b * 256 + e] = (d * scale) * (float)code;
                 }
             }
             return;

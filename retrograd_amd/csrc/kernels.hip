@@ -41,6 +41,7 @@ BlockGeom geom_of(int type) {
         case WT_Q8_0:  return {32, 34};
         case WT_MXFP4: return {32, 17};
         case WT_Q4_K:  return {256, 144};
+        case WT_Q6_K:  return {256, 210};
         default: throw std::runtime_error("unsupported tensor type " + std::to_string(type));
     }
 }
@@ -101,6 +102,20 @@ __device__ float decode_elem(int type, const uint8_t * row, int k) {
             const float d = h2f(*(const uint16_t *)b);
             const float dmin = h2f(*(const uint16_t *)(b + 2));
             return __fsub_rn(__fmul_rn(__fmul_rn(d, (float)s), (float)q), __fmul_rn(dmin, (float)m));
+        }
+        case WT_Q6_K: {
+            // ql[128] | qh[64] | scales[16] (i8) | d (f16): element e has half = e / 128, group g = (e % 128) / 32,
+            // l = e % 32; low bits from a nibble of ql[64 half + l + 32 (g & 1)] (high nibble for g >= 2),
+            // top two bits from qh[32 half + l] >> 2g; value = (d * scale[8 half + 2 g + l / 16]) * (code - 32)
+            const uint8_t * b = row + (size_t)(k >> 8) * 210;
+            const int e = k & 255;
+            const int half = e >> 7, g = (e & 127) >> 5, l = e & 31;
+            const uint8_t lo = b[64 * half + l + 32 * (g & 1)];
+            const int nib = g >= 2 ? (lo >> 4) : (lo & 0x0f);
+            const int top = (b[128 + 32 * half + l] >> (2 * g)) & 3;
+            const float d = h2f((uint16_t)(b[208] | (b[209] << 8)));
+            const float scale = (float)(int8_t)b[192 + 8 * half + 2 * g + (l >> 4)];
+            return __fmul_rn(__fmul_rn(d, scale), (float)((nib | (top << 4)) - 32));
         }
         default: return 0.0f;
     }

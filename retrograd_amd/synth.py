@@ -40,6 +40,10 @@ class ModelShape:
     qkv_bias: bool = False
     eps: float = 1e-5
     name: str = "synthetic"
+    # the mix of a Q4_K_M file: some matrices kept at a finer type (-1: matrix_type)
+    output_type: int = -1            # output.weight
+    down_type: int = -1              # ffn_down.weight
+    v_type: int = -1                 # attn_v.weight
 
 
 # The five benchmark configurations.
@@ -109,6 +113,32 @@ def quantize_q4_k(x: torch.Tensor) -> torch.Tensor:
     return out.reshape(rows, -1)
 
 
+def quantize_q6_k(x: torch.Tensor) -> torch.Tensor:
+    """[rows, K] float -> uint8 [rows, K/256*210]: six-bit codes (offset 32) with an int8 scale per 16
+    elements against an f16 super-block d, stored as ql[128] | qh[64] | scales[16] | d."""
+    rows, K = x.shape
+    nb = K // 256
+    b = x.reshape(rows, nb, 16, 16).float()
+    sub = b.abs().amax(dim=-1) / 31.0
+    d = (sub.amax(dim=-1, keepdim=True) / 127.0).to(torch.float16)
+    df = d.float()
+    sc = torch.where(df > 0, torch.round(sub / df.clamp(min=1e-30)), torch.zeros_like(sub)).clamp_(0, 127)
+    step = (df * sc).unsqueeze(-1)
+    code = torch.where(step > 0, torch.round(b / step.clamp(min=1e-30)), torch.zeros_like(b)).clamp_(-32, 31) + 32
+    code = code.to(torch.uint8).reshape(rows, nb, 2, 4, 32)          # [half][group of 32][l]
+    low, top = code & 0x0F, code >> 4
+    out = torch.empty(rows, nb, 210, dtype=torch.uint8, device=x.device)
+    ql = torch.empty(rows, nb, 2, 64, dtype=torch.uint8, device=x.device)
+    ql[..., 0:32] = low[..., 0, :] | (low[..., 2, :] << 4)
+    ql[..., 32:64] = low[..., 1, :] | (low[..., 3, :] << 4)
+    out[..., 0:128] = ql.reshape(rows, nb, 128)
+    qh = top[..., 0, :] | (top[..., 1, :] << 2) | (top[..., 2, :] << 4) | (top[..., 3, :] << 6)
+    out[..., 128:192] = qh.reshape(rows, nb, 64)
+    out[..., 192:208] = sc.to(torch.int8).view(torch.uint8)
+    out[..., 208:210] = d.view(torch.uint8).reshape(rows, nb, 2)
+    return out.reshape(rows, -1)
+
+
 _FP4_VALUES = (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0)
 
 
@@ -143,6 +173,8 @@ def encode(x: torch.Tensor, ggml_type: int) -> np.ndarray:
         return quantize_q4_k(x).cpu().numpy()
     if ggml_type == gw.GGML_MXFP4:
         return quantize_mxfp4(x).cpu().numpy()
+    if ggml_type == gw.GGML_Q6_K:
+        return quantize_q6_k(x).cpu().numpy()
     raise ValueError("unsupported ggml type %d" % ggml_type)
 
 
@@ -216,7 +248,7 @@ def write_model(path, shape: ModelShape, seed: int = 0, device: str | None = Non
         vector(b + "attn_norm.weight", E, 1.0)
         matrix(b + "attn_q.weight", E, QD)
         matrix(b + "attn_k.weight", E, KD)
-        matrix(b + "attn_v.weight", E, KD)
+        matrix(b + "attn_v.weight", E, KD, None if s.v_type < 0 else s.v_type)
         if s.qkv_bias:
             vector(b + "attn_q.bias", QD)
             vector(b + "attn_k.bias", KD)
@@ -235,9 +267,9 @@ def write_model(path, shape: ModelShape, seed: int = 0, device: str | None = Non
         else:
             matrix(b + "ffn_gate.weight", E, s.n_ff)
             matrix(b + "ffn_up.weight", E, s.n_ff)
-            matrix(b + "ffn_down.weight", s.n_ff, E)
+            matrix(b + "ffn_down.weight", s.n_ff, E, None if s.down_type < 0 else s.down_type)
     vector("output_norm.weight", E, 1.0)
-    matrix("output.weight", E, s.n_vocab)
+    matrix("output.weight", E, s.n_vocab, None if s.output_type < 0 else s.output_type)
     return w.write(Path(path))
 
 

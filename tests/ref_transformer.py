@@ -6,12 +6,12 @@ import oracle
 from gguf_reader import Reader
 
 
-F32, F16, Q8_0, Q4_K, BF16, MXFP4 = 0, 1, 8, 12, 30, 39
+F32, F16, Q8_0, Q4_K, Q6_K, BF16, MXFP4 = 0, 1, 8, 12, 14, 30, 39
 
 
 def ggml_activations(v, weight_type):
     """The rows of v as ggml's CPU matmul multiplies them with a weight of this
-    type: re-quantised to Q8_K (Q4_K weights; blocks of 256, the first value of
+    type: re-quantised to Q8_K (Q4_K and Q6_K weights; blocks of 256, the first value of
     largest magnitude maps to -127, codes rounded half to even and capped at
     127), to Q8_0 (Q8_0 and MXFP4 weights; blocks of 32, scale amax / 127 kept
     as f16, codes rounded half away from zero with the unrounded scale), or
@@ -19,7 +19,7 @@ def ggml_activations(v, weight_type):
     independently of oracle/model.hpp."""
     x = np.asarray(v, np.float32)
     f32 = np.float32
-    if weight_type == Q4_K:
+    if weight_type in (Q4_K, Q6_K):
         b = x.reshape(-1, 256)
         first = np.abs(b).argmax(-1)                      # argmax returns the first maximum
         mx = b[np.arange(len(b)), first]

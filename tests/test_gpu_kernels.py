@@ -54,7 +54,7 @@ def test_tile_matmul_matches_decoded_blocks(t, n, k, T, ggml):
 
 @pytest.mark.parametrize("ggml", [False, True])
 @pytest.mark.parametrize("t,k", [(gw.GGML_F16, 344), (gw.GGML_F32, 100), (gw.GGML_Q8_0, 128),
-                                 (gw.GGML_MXFP4, 96), (gw.GGML_Q4_K, 256), (gw.GGML_BF16, 64)])
+                                 (gw.GGML_MXFP4, 96), (gw.GGML_Q4_K, 256), (gw.GGML_BF16, 64), (gw.GGML_Q6_K, 512)])
 def test_generic_matmul_every_storage_type(t, k, ggml):
     print("case", t, k, ggml, flush=True)
     n, T = 37, 11
@@ -69,7 +69,7 @@ def test_generic_matmul_every_storage_type(t, k, ggml):
     want = _ref(t, dense, x, ggml)
     got = E.kernel_matmul(t, raw, n, k, x, use_tiles=False, ggml_activations=ggml)
     assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max() + 1e-6
-    if ggml and t in (gw.GGML_F16, gw.GGML_BF16, gw.GGML_Q8_0, gw.GGML_Q4_K, gw.GGML_MXFP4):
+    if ggml and t in (gw.GGML_F16, gw.GGML_BF16, gw.GGML_Q8_0, gw.GGML_Q4_K, gw.GGML_MXFP4, gw.GGML_Q6_K):
         assert np.abs(want - _ref(t, dense, x, False)).max() > 1e-4 * np.abs(want).max()     # the conversion is visible
 
 

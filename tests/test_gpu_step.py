@@ -23,6 +23,9 @@ SMALL = {
                                     head_dim=128, n_ff=2048, n_vocab=2048, name="llama-q4k-hd128"),
     "qwen2-q8": synth.scaled(synth.QWEN25_7B_Q8, n_layer=2, n_embd=512, n_head=14, n_head_kv=2, head_dim=32,
                              n_ff=1024, n_vocab=1024, name="qwen2-small"),
+    # the type mix of a Q4_K_M file: output.weight, ffn_down and attn_v in Q6_K, the rest in Q4_K
+    "llama-q4k-m": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
+                                n_ff=1024, n_vocab=1024, output_type=14, down_type=14, v_type=14, name="llama-q4k-m-small"),
 }
 
 

@@ -19,6 +19,9 @@ SHAPES = {
                              n_ff=256, n_vocab=300, name="qwen2-small"),
     "qwen3moe": synth.scaled(synth.QWEN3_30B_A3B, n_layer=2, n_embd=128, n_head=4, n_head_kv=2, head_dim=64,
                              n_vocab=288, n_expert=8, n_expert_used=2, n_ff_exp=64, name="qwen3moe-small"),
+    # the type mix of a Q4_K_M file: output.weight, ffn_down and attn_v in Q6_K
+    "llama-q4k-m": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=256, n_head=4, n_head_kv=2, head_dim=64,
+                                n_ff=512, n_vocab=320, output_type=14, down_type=14, v_type=14, name="llama-q4k-m-small"),
 }
 
 
@@ -41,8 +44,10 @@ def test_forward_matches_independent_float64_transformer(models, key, activation
     # Under the ggml arithmetic the activations entering a matmul are re-quantised (Q8_K / Q8_0).
     # A value within an ulp of a rounding boundary can take the neighbouring code in one of the
     # two implementations (f32 here, f64 there), which moves the logits by ~1e-3; about one
-    # prompt in five has such a value somewhere (see the next test). This prompt has none.
-    rng = np.random.default_rng(6)
+    # prompt in five has such a value somewhere (see the next test). In either arithmetic the
+    # same happens, at the 1e-5 level, to a K or V value on a rounding boundary of the f16
+    # cache. These prompts have neither.
+    rng = np.random.default_rng(10 if key == "llama-q4k-m" else 6)
     toks = rng.integers(0, m.n_vocab, 12)
     p = {"token": toks, "pos": np.arange(12), "seq": np.zeros(12), "output": np.ones(12)}
     got = ctx.step(p["token"], p["pos"], p["seq"], p["output"])

@@ -233,3 +233,62 @@ def synth_quantise(wt, w):
     import torch
     from retrograd_amd import synth
     return np.asarray(synth.encode(torch.from_numpy(w), wt)).reshape(w.shape[0], -1)
+
+
+# ---- Q6_K (the finer type of a Q4_K_M file: output.weight, half of ffn_down and attn_v) -----------
+
+def _q6_k_by_the_block_loops(blk):
+    """One 210-byte block decoded by the loop structure the reference spells out
+    (crates/rir-core/src/quant.rs:444-464): two halves of 128, 32 positions each feeding four outputs."""
+    ql, qh, sc = blk[0:128], blk[128:192], blk[192:208].view(np.int8)
+    d = np.float32(blk[208:210].view(np.float16)[0])
+    y = np.zeros(256, np.float32)
+    for n in (0, 128):
+        a, h, s = ql[n // 2:], qh[n // 4:], sc[n // 16:]
+        for l in range(32):
+            i = l // 16
+            q1 = ((int(a[l]) & 0xF) | ((int(h[l]) & 3) << 4)) - 32
+            q2 = ((int(a[l + 32]) & 0xF) | (((int(h[l]) >> 2) & 3) << 4)) - 32
+            q3 = ((int(a[l]) >> 4) | (((int(h[l]) >> 4) & 3) << 4)) - 32
+            q4 = ((int(a[l + 32]) >> 4) | (((int(h[l]) >> 6) & 3) << 4)) - 32
+            y[n + l] = d * np.float32(s[i]) * np.float32(q1)
+            y[n + l + 32] = d * np.float32(s[i + 2]) * np.float32(q2)
+            y[n + l + 64] = d * np.float32(s[i + 4]) * np.float32(q3)
+            y[n + l + 96] = d * np.float32(s[i + 6]) * np.float32(q4)
+    return y
+
+
+def test_q6_k_against_the_block_loops_and_single_codes():
+    Q6_K = 14
+    assert oracle.row_bytes(Q6_K, 512) == 2 * 210
+    rng = np.random.default_rng(11)
+    raw = rng.integers(0, 256, 2 * 210, dtype=np.uint8)
+    for b in range(2):
+        raw[b * 210 + 208:b * 210 + 210] = np.frombuffer(np.float16(0.03125 * (b + 1)).tobytes(), np.uint8)
+    got = oracle.decode_row(Q6_K, raw, 512)
+    want = np.concatenate([_q6_k_by_the_block_loops(raw[b * 210:(b + 1) * 210]) for b in range(2)])
+    assert np.array_equal(got, want)
+    # one code, one element: all codes 32 (value 0) except element e, scales 1, d 1
+    for e in (0, 17, 33, 95, 127, 128, 200, 255):
+        blk = np.zeros(210, np.uint8)
+        blk[128:192] = 0xAA                      # top bits 2 everywhere: codes 32 -> 0
+        blk[192:208] = 1
+        blk[208:210] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+        assert not oracle.decode_row(Q6_K, blk, 256).any()
+        half, g, l = e // 128, (e % 128) // 32, e % 32
+        # code 63 (value 31): nibble 15, top bits 3
+        blk[64 * half + l + 32 * (g & 1)] |= 0xF0 if g >= 2 else 0x0F
+        blk[128 + 32 * half + l] |= 3 << (2 * g)
+        y = oracle.decode_row(Q6_K, blk, 256)
+        assert y[e] == 31.0 and np.count_nonzero(y) == 1, e
+    # the synthetic quantiser writes blocks that decode near their input
+    import torch
+    from retrograd_amd import synth
+    x = torch.randn(3, 512, generator=torch.Generator().manual_seed(4)) * 0.05
+    enc = synth.encode(x, Q6_K)
+    for r in range(3):
+        y = oracle.decode_row(Q6_K, enc[r], 512)
+        assert np.abs(y - x[r].numpy()).max() < 0.04 * np.abs(x[r].numpy()).max()
+    # Q6_K weights take Q8_K activations
+    v = rng.standard_normal(256).astype(np.float32)
+    assert np.array_equal(oracle.activation_row(Q6_K, v), oracle.activation_row(12, v))

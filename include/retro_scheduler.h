@@ -111,6 +111,13 @@ typedef struct retro_sched_kv_stats {
 /* Scheduler::new over an engine (`impl DecodeBackend for Engine`, backend.rs:266-371). The engine is
  * borrowed: it must outlive the scheduler and is freed by the caller. */
 retro_scheduler * retro_scheduler_new(retro_engine * engine, const retro_sched_options * options);
+/* Scheduler::new over a trainer's generation context (`impl DecodeBackend for TrainerBackend`,
+ * backend.rs:376-461): rollouts admitted, batched and prefix-cached like serving requests. Rows decode
+ * under the trainer's generation default adapter; the per-sequence context is the whole generation pool
+ * (backend.rs:446-453); a weight change moves weights_version on, which makes the scheduler drop every
+ * cached prefix (scheduler.rs, refresh_key). The trainer is borrowed like the engine above. */
+struct retro_trainer;
+retro_scheduler * retro_scheduler_new_trainer(struct retro_trainer * trainer, const retro_sched_options * options);
 /* Scheduler::new over FakeBackend::new(n_slots, n_ctx_seq, cells_total, vocab, eos, pieces) (fake.rs:77-118):
  * the in-memory backend the reference tests its policy with. */
 retro_scheduler * retro_scheduler_new_fake(uint32_t n_slots, uint32_t n_ctx_seq, uint64_t cells_total, uint32_t vocab,

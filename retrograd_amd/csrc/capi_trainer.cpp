@@ -87,6 +87,11 @@ bool validate(const retro_train_config & c) {
 
 }  // namespace
 
+// The engine behind a trainer's generation context, for the scheduler (capi_sched.cpp).
+namespace retro {
+retro_engine * generation_engine_of(retro_trainer * trainer) { return trainer ? trainer->engine : nullptr; }
+}
+
 extern "C" {
 
 retro_trainer * retro_trainer_new(const char * model_path, const retro_train_config * train_config) {

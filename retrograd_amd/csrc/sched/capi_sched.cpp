@@ -8,6 +8,10 @@
 #include "fake_backend.hpp"
 #include "scheduler.hpp"
 
+// defined with the trainer handle (capi_trainer.cpp)
+struct retro_trainer;
+namespace retro { retro_engine * generation_engine_of(retro_trainer * trainer); }
+
 using namespace sched;
 
 struct retro_scheduler {
@@ -99,6 +103,19 @@ retro_scheduler * retro_scheduler_new(retro_engine * engine, const retro_sched_o
     retro_scheduler * out = nullptr;
     guarded([&]() -> int {
         if (!engine) throw InferError::invalid("engine is required");
+        auto s = std::make_unique<retro_scheduler>();
+        s->impl = std::make_unique<Scheduler>(std::make_unique<EngineBackend>(engine), options_from(options));
+        out = s.release();
+        return 0;
+    });
+    return out;
+}
+
+retro_scheduler * retro_scheduler_new_trainer(retro_trainer * trainer, const retro_sched_options * options) {
+    retro_scheduler * out = nullptr;
+    guarded([&]() -> int {
+        retro_engine * engine = retro::generation_engine_of(trainer);
+        if (!engine) throw InferError::invalid("trainer is required");
         auto s = std::make_unique<retro_scheduler>();
         s->impl = std::make_unique<Scheduler>(std::make_unique<EngineBackend>(engine), options_from(options));
         out = s.release();

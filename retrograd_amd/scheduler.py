@@ -22,7 +22,7 @@ ERROR_KINDS = {1: "InvalidArgument", 2: "Failed", 3: "Overflow", 4: "QueueFull",
                7: "Backend"}
 
 SCHED_SYMBOLS = [
-    "retro_sched_options_default", "retro_scheduler_new", "retro_scheduler_new_fake", "retro_scheduler_free",
+    "retro_sched_options_default", "retro_scheduler_new", "retro_scheduler_new_trainer", "retro_scheduler_new_fake", "retro_scheduler_free",
     "retro_scheduler_initialize", "retro_scheduler_submit", "retro_scheduler_pump", "retro_scheduler_run_until_idle",
     "retro_scheduler_counts", "retro_scheduler_fail_queued", "retro_scheduler_kv_stats", "retro_scheduler_pin_prefix",
     "retro_scheduler_unpin", "retro_scheduler_load_adapter", "retro_scheduler_unload_adapter",
@@ -84,6 +84,8 @@ def _lib() -> C.CDLL:
     if not _bound:
         lib.retro_scheduler_new.restype = C.c_void_p
         lib.retro_scheduler_new.argtypes = [C.c_void_p, C.POINTER(COptions)]
+        lib.retro_scheduler_new_trainer.restype = C.c_void_p
+        lib.retro_scheduler_new_trainer.argtypes = [C.c_void_p, C.POINTER(COptions)]
         lib.retro_scheduler_new_fake.restype = C.c_void_p
         lib.retro_scheduler_new_fake.argtypes = [C.c_uint32, C.c_uint32, C.c_uint64, C.c_uint32, C.c_int32,
                                                  C.POINTER(C.c_char_p), C.c_size_t, C.POINTER(COptions)]
@@ -368,6 +370,12 @@ class Scheduler:
     def over_engine(engine: E.Engine, options: SchedulerOptions) -> "Scheduler":
         opts = options.to_c()
         return Scheduler(_lib().retro_scheduler_new(engine._h, C.byref(opts)), engine=engine)
+
+    @staticmethod
+    def over_trainer(trainer, options: SchedulerOptions) -> "Scheduler":
+        """Scheduler::new over TrainerBackend (backend.rs:376-461): the trainer's generation context."""
+        opts = options.to_c()
+        return Scheduler(_lib().retro_scheduler_new_trainer(trainer._h, C.byref(opts)), engine=trainer)
 
     @staticmethod
     def over_fake(n_slots: int, n_ctx_seq: int, cells_total: int, vocab: int, eos: int, pieces: Sequence[str],

@@ -160,3 +160,45 @@ def test_snapshots_freeze_the_policy_and_the_generation_default_selects_one(file
     assert tr.adapter_rows_info().n_adapters == 0
     for t in (tr, other, eng):
         t.close()
+
+
+def test_rollouts_through_the_scheduler_over_a_trainer(files):
+    """The scheduler over a trainer's generation context (reference backend.rs:376-461): requests decode
+    under the trained adapter, and a weight change makes the scheduler let go of every cached prefix."""
+    from retrograd_amd import scheduler as S
+    model, a1, a2 = files
+    print("trainer: scheduler over the generation context", flush=True)
+    tr = trainer(model)
+    tr.load_lora(a1)
+    sched = S.Scheduler.over_trainer(tr, S.SchedulerOptions(mode=S.CONTINUOUS, n_batch=96, event_capacity=256,
+                                                            min_prefix_len=4))
+    sched.initialize()
+    rng = np.random.default_rng(21)
+    prompts = [[int(t) for t in rng.integers(0, SHAPE.n_vocab, n)] for n in (24, 12)]
+
+    def run(prompt, n_new):
+        stream = sched.submit(S.Request.single(prompt, E.SamplingParamsV2.greedy(max_new_tokens=n_new)))
+        sched.run_until_idle()
+        events = list(stream.drain())
+        assert not [e for e in events if e.type == "Error"]
+        return [e.token for e in events if e.type == "Token"], [e for e in events if e.type == "End"][0]
+
+    first, end = run(prompts[0], 4)
+    assert end.cached_tokens == 0
+    # the same tokens as the plain step under the trained adapter gives
+    eng = engine(model)
+    a1_id = eng.adapter_load(a1, 1.0)
+    assert first == decode(eng, [prompts[0]], [a1_id], n_new=4)[0][0]
+    # a second request that extends the first reuses its cells
+    again, end = run(prompts[0] + first[:2], 2)
+    assert end.cached_tokens >= len(prompts[0]) and sched.kv_stats().hits == 1
+    # new weights: the version moves on and nothing cached under the old ones is reused
+    tr.load_lora(a2)
+    assert tr.weights_version() == 2
+    third, end = run(prompts[0] + first[:2], 2)
+    assert end.cached_tokens == 0
+    a2_id = eng.adapter_load(a2, 1.0)
+    assert third == decode(eng, [prompts[0] + first[:2]], [a2_id], n_new=2)[0][0]
+    sched.close()
+    tr.close()
+    eng.close()

@@ -97,7 +97,12 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
         d_o.alloc((size_t)n_rows * sizeof(rk::SampleOut));
         ok(hipMemcpy(d_l.ptr, logits, d_l.bytes, hipMemcpyHostToDevice), "upload logits");
         ok(hipMemcpy(d_k.ptr, k, d_k.bytes, hipMemcpyHostToDevice), "upload k");
-        rk::sample_prepare(nullptr, d_l.as<float>(), n_rows, n_vocab, d_k.as<int32_t>(), d_o.as<rk::SampleOut>());
+        int max_k = 0;
+        for (int r = 0; r < n_rows; ++r) max_k = std::max(max_k, k[r]);
+        DevBuf d_scratch;
+        d_scratch.alloc(rk::sample_scratch_bytes(n_rows));
+        rk::sample_prepare(nullptr, d_l.as<float>(), n_rows, n_vocab, d_k.as<int32_t>(), d_o.as<rk::SampleOut>(), max_k,
+                           d_scratch.ptr);
         ok(hipDeviceSynchronize(), "sample_prepare");
         std::vector<rk::SampleOut> h((size_t)n_rows);
         ok(hipMemcpy(h.data(), d_o.ptr, d_o.bytes, hipMemcpyDeviceToHost), "download");

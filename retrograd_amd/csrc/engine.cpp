@@ -393,6 +393,7 @@ void Engine::build_buffers() {
     hip_check(hipMemsetAsync(mm_ws_.ptr, 0, mm_ws_.bytes, stream_), "hipMemsetAsync");
     sample_k_.alloc((size_t)B * 4);
     sample_out_.alloc((size_t)B * sizeof(rk::SampleOut));
+    sample_scratch_.alloc(rk::sample_scratch_bytes(B));
     const size_t stage = (size_t)B * (sizeof(rk::RowDesc) + 4) + 65536;
     d_stage_.alloc(stage);
     h_stage_.ensure(stage);
@@ -1052,7 +1053,8 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
         if (n_out > 0) {
             hip_check(hipMemcpyAsync(sample_k_.ptr, kreq.data(), (size_t)n_out * 4, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
             const size_t pt_s = prof_begin(PC_SAMPLE);
-            rk::sample_prepare(stream_, logits_.as<float>(), n_out, n_vocab, sample_k_.as<int32_t>(), sample_out_.as<rk::SampleOut>());
+            rk::sample_prepare(stream_, logits_.as<float>(), n_out, n_vocab, sample_k_.as<int32_t>(), sample_out_.as<rk::SampleOut>(),
+                               *std::max_element(kreq.begin(), kreq.end()), sample_scratch_.ptr);
             prof_end(PC_SAMPLE, pt_s);
             hip_check(hipMemcpyAsync(h_sample_.ptr, sample_out_.ptr, (size_t)n_out * sizeof(rk::SampleOut), hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync");
             if (any_full) {

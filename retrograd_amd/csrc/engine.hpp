@@ -225,7 +225,7 @@ private:
     HostPinned h_stage_;
     rk::PackBuffers pk_ {};
     std::vector<DevBuf> pk_store_;
-    DevBuf x_, qkv_, gu_, q_half_, partial_, logits_, sample_k_, sample_out_, out_rows_idx_;
+    DevBuf x_, qkv_, gu_, q_half_, partial_, logits_, sample_k_, sample_out_, sample_scratch_, out_rows_idx_;
     DevBuf act_e_x_, act_e_sums_;       // n_embd wide
     DevBuf act_q_x_, act_q_sums_;       // n_head * head_dim wide
     DevBuf act_f_x_, act_f_sums_;       // n_ff wide

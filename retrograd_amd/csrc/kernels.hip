@@ -1697,9 +1697,85 @@ __global__ __launch_bounds__(1024) void k_sample_prepare(const float * __restric
     }
 }
 
+// Rows that ask for at most one candidate: the vocabulary is cut into slices, one workgroup each, so that a
+// 64-row step fills the chip instead of 64 compute units. A slice leaves its best entry and the sum of
+// exp(double(logit) - its own maximum); the merge rescales the sums to the row maximum.
+struct SamplePartial { float max; int32_t idx; double sum; };
+
+__global__ __launch_bounds__(256) void k_sample_slices(const float * __restrict__ logits, int V, int len,
+                                                       SamplePartial * __restrict__ part) {
+    __shared__ float s_val[4];
+    __shared__ int s_idx[4];
+    __shared__ double s_sum[4];
+    __shared__ float b_val;
+    const int row = blockIdx.x, slice = blockIdx.y, n_slices = gridDim.y;
+    const int lo = slice * len, hi = min(V, lo + len);
+    const float * l = logits + (size_t)row * V;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += 256) {
+        const float v = l[i];
+        if (better(v, i, bv, bi)) { bv = v; bi = i; }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+    }
+    if (lane == 0) { s_val[wave] = bv; s_idx[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float fv = s_val[0];
+        int fi = s_idx[0];
+        for (int w = 1; w < 4; ++w) if (better(s_val[w], s_idx[w], fv, fi)) { fv = s_val[w]; fi = s_idx[w]; }
+        b_val = fv;
+        part[(size_t)row * n_slices + slice].max = fv;
+        part[(size_t)row * n_slices + slice].idx = fi;
+    }
+    __syncthreads();
+    const float slice_max = b_val;
+    double acc = 0.0;
+    for (int i = lo + threadIdx.x; i < hi; i += 256) acc += exp((double)l[i] - (double)slice_max);
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (lane == 0) s_sum[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) part[(size_t)row * n_slices + slice].sum = (s_sum[0] + s_sum[1]) + (s_sum[2] + s_sum[3]);
+}
+
+__global__ __launch_bounds__(64) void k_sample_merge(const SamplePartial * __restrict__ part, int n_slices,
+                                                     const int32_t * __restrict__ kreq, SampleOut * out) {
+    const int row = blockIdx.x;
+    if (threadIdx.x != 0) return;
+    const SamplePartial * p = part + (size_t)row * n_slices;
+    float fv = -INFINITY;
+    int fi = 0x7fffffff;
+    for (int s = 0; s < n_slices; ++s)
+        if (p[s].idx != 0x7fffffff && better(p[s].max, p[s].idx, fv, fi)) { fv = p[s].max; fi = p[s].idx; }
+    double total = 0.0;
+    for (int s = 0; s < n_slices; ++s)
+        if (p[s].idx != 0x7fffffff) total += p[s].sum * exp((double)p[s].max - (double)fv);
+    out[row].argmax = fi;
+    out[row].max = fv;
+    out[row].sum_exp = total;
+    if (kreq && kreq[row] >= 1) { out[row].top_id[0] = fi; out[row].top_logit[0] = fv; }
+}
+
+size_t sample_scratch_bytes(int n_rows) { return (size_t)std::max(n_rows, 1) * 32 * sizeof(SamplePartial); }
+
 void sample_prepare(hipStream_t s, const float * logits, int n_rows, int n_vocab, const int32_t * k,
-                    SampleOut * out) {
+                    SampleOut * out, int max_k, void * scratch) {
     if (n_rows <= 0) return;
+    if (max_k <= 1 && scratch && n_vocab >= 8192) {
+        int n_slices = 1;
+        while (n_slices < 32 && n_rows * n_slices * 2 <= 1024) n_slices *= 2;
+        const int len = ((n_vocab + n_slices - 1) / n_slices + 3) & ~3;
+        hipLaunchKernelGGL(k_sample_slices, dim3(n_rows, n_slices), dim3(256), 0, s, logits, n_vocab, len, (SamplePartial *)scratch);
+        check_launch("sample_slices");
+        hipLaunchKernelGGL(k_sample_merge, dim3(n_rows), dim3(64), 0, s, (const SamplePartial *)scratch, n_slices, k, out);
+        check_launch("sample_merge");
+        return;
+    }
     hipLaunchKernelGGL(k_sample_prepare, dim3(n_rows), dim3(1024), 0, s, logits, n_vocab, k, out);
     check_launch("sample_prepare");
 }

@@ -291,8 +291,11 @@ struct SampleOut {          // one per output row, read back by the host
     int32_t top_id[MAX_TOPK];
     float top_logit[MAX_TOPK];
 };
-// k[r] candidates per row by (logit desc, id asc); k = 0 rows only get argmax/max/sum.
+// k[r] candidates per row by (logit desc, id asc); k = 0 rows only get argmax/max/sum. max_k is the
+// largest k[r] (known to the host): when no row asks for more than one candidate and scratch
+// (sample_scratch_bytes(n_rows) bytes) is given, a large vocabulary is scanned in slices by many workgroups.
+size_t sample_scratch_bytes(int n_rows);
 void sample_prepare(hipStream_t s, const float * logits, int n_rows, int n_vocab, const int32_t * k,
-                    SampleOut * out);
+                    SampleOut * out, int max_k, void * scratch);
 
 }  // namespace rk

@@ -154,3 +154,24 @@ def test_sample_prepare_matches_numpy():
         order = np.lexsort((np.arange(V), -row.astype(np.float64)))[:k[r]]
         assert list(ids[r, :k[r]]) == list(order)
         assert np.array_equal(vals[r, :k[r]], row[order])
+
+
+@pytest.mark.parametrize("n_rows", [1, 5, 64])
+def test_sample_prepare_in_slices_matches_numpy(n_rows):
+    # rows that ask for at most one candidate over a large vocabulary take the sliced scan
+    rng = np.random.default_rng(13)
+    V = 20011                                                      # no multiple of the slice granularity
+    logits = (rng.standard_normal((n_rows, V)) * 3).astype(np.float32)
+    logits[0, 17] = logits[0, 19000] = logits[0].max() + 1.0      # the maximum twice, in different slices: lowest id wins
+    if n_rows > 2:
+        logits[2, -1] = logits[2].max() + 2.0                      # ... and in the very last position
+    k = [r % 2 for r in range(n_rows)]
+    argmax, mx, se, ids, vals = E.kernel_sample_prepare(logits, k)
+    for r in range(n_rows):
+        row = logits[r]
+        assert argmax[r] == int(np.flatnonzero(row == row.max())[0])
+        assert mx[r] == row.max()
+        ref = np.exp(row.astype(np.float64) - float(row.max())).sum()
+        assert abs(se[r] - ref) <= 1e-12 * ref
+        if k[r]:
+            assert ids[r, 0] == argmax[r] and vals[r, 0] == row.max()

@@ -135,6 +135,11 @@ int retro_scheduler_fail_queued(retro_scheduler * s);                           
 int retro_scheduler_kv_stats(retro_scheduler * s, retro_sched_kv_stats * out);             /* scheduler.rs:427 */
 int retro_scheduler_pin_prefix(retro_scheduler * s, const int32_t * prefix, size_t n, uint64_t * out_pin);  /* :534 */
 int retro_scheduler_unpin(retro_scheduler * s, uint64_t pin, uint8_t * out_released);      /* scheduler.rs:542 */
+/* lend_slot (scheduler.rs:746-777): a slot that no live sequence and no dormant prefix holds, with `cells` of the
+ * pool free beside the dormant prefixes, evicting least recently used prefix nodes until both fit; *out_slot = -1
+ * when nothing more can be evicted. Fails while a sequence is live. The caller empties the slot before the next pump. */
+int retro_scheduler_lend_slot(retro_scheduler * s, uint64_t cells, int32_t * out_slot);
+int retro_scheduler_queue_capacity(retro_scheduler * s, size_t * out_capacity);            /* scheduler.rs, queue_capacity */
 int retro_scheduler_load_adapter(retro_scheduler * s, const char * name, const char * path);   /* scheduler.rs:454 */
 int retro_scheduler_unload_adapter(retro_scheduler * s, const char * name);                /* scheduler.rs:488 */
 int retro_scheduler_set_mode(retro_scheduler * s, int32_t mode);

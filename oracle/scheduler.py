@@ -967,6 +967,24 @@ class Scheduler:
                 if stalled > 1024:
                     raise InferError("Failed", "the scheduler made no progress with requests still queued")
 
+    def lend_slot(self, cells: int) -> Optional[int]:
+        """scheduler.rs:746-777."""
+        if self.live:
+            raise InferError("Failed", "a slot can only be lent while no sequence is live")
+        while True:
+            slots_left, cells_left = self._capacity()
+            if slots_left > 0 and cells_left >= cells:
+                held = set(self.kv.resident_slots())
+                for slot in range(self.n_slots):
+                    if slot not in held:
+                        return slot
+                return None
+            if not self._evict_one_lru():
+                return None
+
+    def queue_capacity(self) -> int:
+        return self.o.queue_capacity
+
     def fail_queued(self):
         while self.queue:
             _, stream = self.queue.pop(0)
@@ -1559,3 +1577,49 @@ def validate(r: Request):
         raise invalid("an adapter name must not be empty")
     if r.retention is not None and r.retention[0] == "":
         raise invalid("a retention key must not be empty")
+
+
+# ---- the synchronous batch driver (crates/retrograd-infer/src/sync.rs:96-149) -----------------------
+
+def run_requests(scheduler: "Scheduler", requests, on_step=None):
+    """Submits in order as the queue has room, pumps until all have ended, drains the streams after every
+    step. Returns per request {"completions": [{tokens, logprobs, forced, text, finish}], "error"}."""
+    pending = list(requests)
+    streams, outcomes = [], []
+    stalled = 0
+
+    def absorb(outcome, e):
+        if e["type"] == "Error":
+            outcome["error"] = e["error"]
+            return
+        member = outcome["completions"][e["index"]]
+        if e["type"] == "Token":
+            member["tokens"].append(e["token"])
+            member["logprobs"].append(e["logprob"])
+            member["forced"].append(e.get("forced", False))
+            member["text"] += e.get("text", "")
+        else:
+            member["finish"] = e["reason"]
+            member["text"] += e.get("text", "")
+
+    while True:
+        while pending and scheduler.queued_len() < scheduler.queue_capacity():
+            request = pending.pop(0)
+            streams.append(scheduler.submit(request))
+            outcomes.append({"completions": [dict(tokens=[], logprobs=[], forced=[], text="", finish=None)
+                                             for _ in range(request.n())], "error": None})
+        if not pending and scheduler.is_idle():
+            break
+        progressed = scheduler.pump()
+        if on_step:
+            on_step(scheduler)
+        for stream, outcome in zip(streams, outcomes):
+            for e in stream.drain():
+                absorb(outcome, e)
+        stalled = 0 if progressed else stalled + 1
+        if stalled > 1024:
+            raise InferError("Failed", "the scheduler made no progress with requests still queued")
+    for stream, outcome in zip(streams, outcomes):
+        for e in stream.drain():
+            absorb(outcome, e)
+    return outcomes

@@ -234,6 +234,22 @@ int retro_scheduler_pin_prefix(retro_scheduler * s, const int32_t * prefix, size
     });
 }
 
+int retro_scheduler_lend_slot(retro_scheduler * s, uint64_t cells, int32_t * out_slot) {
+    return guarded([&]() -> int {
+        if (!out_slot) throw InferError::invalid("out_slot is required");
+        *out_slot = sched_of(s).lend_slot(cells);
+        return 0;
+    });
+}
+
+int retro_scheduler_queue_capacity(retro_scheduler * s, size_t * out_capacity) {
+    return guarded([&]() -> int {
+        if (!out_capacity) throw InferError::invalid("out_capacity is required");
+        *out_capacity = sched_of(s).queue_capacity();
+        return 0;
+    });
+}
+
 int retro_scheduler_unpin(retro_scheduler * s, uint64_t pin, uint8_t * out_released) {
     return guarded([&]() -> int {
         const bool released = sched_of(s).unpin(pin);
@@ -371,6 +387,14 @@ int retro_sched_fake_log(retro_scheduler * s, const char * what, int64_t * buffe
                 flat.push_back(e.slot);
                 flat.push_back(e.flags);
                 flat.push_back((int64_t)e.len);
+            }
+        } else if (w == "seq_pos") {
+            const uint32_t n = f.memory().n_slots;
+            for (uint32_t slot = 0; slot < n; ++slot) {
+                const auto range = f.seq_pos((int32_t)slot);
+                flat.push_back(slot);
+                flat.push_back(range.first);
+                flat.push_back(range.second);
             }
         } else {
             throw InferError::invalid("unknown fake backend log '" + w + "'");

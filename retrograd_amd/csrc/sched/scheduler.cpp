@@ -368,6 +368,23 @@ bool Scheduler::pump() {
     }
 }
 
+// scheduler.rs:755-777
+int32_t Scheduler::lend_slot(uint64_t cells) {
+    if (!live_.empty()) throw InferError::failed("a slot can only be lent while no sequence is live");
+    for (;;) {
+        const auto cap = capacity();
+        if (cap.first > 0 && cap.second >= cells) {
+            std::vector<bool> held(n_slots_, false);
+            for (int32_t slot : kv_.resident_slots())
+                if (slot >= 0 && (size_t)slot < held.size()) held[(size_t)slot] = true;
+            for (size_t slot = 0; slot < held.size(); ++slot)
+                if (!held[slot]) return (int32_t)slot;
+            return -1;
+        }
+        if (!evict_one_lru()) return -1;
+    }
+}
+
 // scheduler.rs:783-789
 void Scheduler::run_until_idle() {
     size_t stalled = 0;

@@ -75,6 +75,11 @@ public:
 
     KvStats kv_stats() const;
     SchedulerStats stats();
+    // One pool slot outside the bookkeeping, for host work between waves: a slot that no live sequence and no
+    // dormant prefix holds, with `cells` of the pool left beside the dormant prefixes; least recently used
+    // prefix nodes are evicted until both fit. -1 when nothing more can be evicted. Only while no sequence
+    // is live (throws otherwise); the caller leaves the slot empty before the next pump. scheduler.rs:746-777
+    int32_t lend_slot(uint64_t cells);
     PinId pin_prefix(const std::vector<int32_t> & prefix);
     bool unpin(PinId id) { return kv_.unpin(id); }
     void load_adapter(const std::string & name, const std::string & path);

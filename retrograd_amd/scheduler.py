@@ -22,7 +22,8 @@ ERROR_KINDS = {1: "InvalidArgument", 2: "Failed", 3: "Overflow", 4: "QueueFull",
                7: "Backend"}
 
 SCHED_SYMBOLS = [
-    "retro_sched_options_default", "retro_scheduler_new", "retro_scheduler_new_trainer", "retro_scheduler_new_fake", "retro_scheduler_free",
+    "retro_sched_options_default", "retro_scheduler_new", "retro_scheduler_new_trainer", "retro_scheduler_new_fake", "retro_scheduler_lend_slot",
+    "retro_scheduler_queue_capacity", "retro_scheduler_free",
     "retro_scheduler_initialize", "retro_scheduler_submit", "retro_scheduler_pump", "retro_scheduler_run_until_idle",
     "retro_scheduler_counts", "retro_scheduler_fail_queued", "retro_scheduler_kv_stats", "retro_scheduler_pin_prefix",
     "retro_scheduler_unpin", "retro_scheduler_load_adapter", "retro_scheduler_unload_adapter",
@@ -84,6 +85,8 @@ def _lib() -> C.CDLL:
     if not _bound:
         lib.retro_scheduler_new.restype = C.c_void_p
         lib.retro_scheduler_new.argtypes = [C.c_void_p, C.POINTER(COptions)]
+        lib.retro_scheduler_lend_slot.argtypes = [C.c_void_p, C.c_uint64, C.POINTER(C.c_int32)]
+        lib.retro_scheduler_queue_capacity.argtypes = [C.c_void_p, C.POINTER(C.c_size_t)]
         lib.retro_scheduler_new_trainer.restype = C.c_void_p
         lib.retro_scheduler_new_trainer.argtypes = [C.c_void_p, C.POINTER(COptions)]
         lib.retro_scheduler_new_fake.restype = C.c_void_p
@@ -316,6 +319,10 @@ class FakeLog:
     def request_order(self):
         return [r[0] for r in self._ints("request_order", 1)]
 
+    def seq_pos(self, slot: int):
+        """(pos_min, pos_max) of a slot of the fake pool, (-1, -1) when empty."""
+        return {s: (lo, hi) for s, lo, hi in self._ints("seq_pos", 3)}[slot]
+
     @property
     def saves(self):
         return self._ints("saves", 3)
@@ -457,6 +464,17 @@ class Scheduler:
         return KvStats(st.hits, st.misses, st.prefilled_cells, st.prompt_cells, st.evictions, st.swaps, st.nodes,
                        st.resident_slots, st.snapshot_bytes)
 
+    def lend_slot(self, cells: int) -> Optional[int]:
+        """scheduler.rs:746-777: a free slot with `cells` of the pool beside the dormant prefixes, or None."""
+        out = C.c_int32()
+        _check(_lib().retro_scheduler_lend_slot(self._h, cells, C.byref(out)))
+        return None if out.value < 0 else out.value
+
+    def queue_capacity(self) -> int:
+        out = C.c_size_t()
+        _check(_lib().retro_scheduler_queue_capacity(self._h, C.byref(out)))
+        return out.value
+
     def pin_prefix(self, prefix: Sequence[int]) -> int:
         arr = (C.c_int32 * max(len(prefix), 1))(*prefix)
         pin = C.c_uint64()
@@ -476,3 +494,71 @@ class Scheduler:
 
     def set_mode(self, mode: int) -> None:
         _check(_lib().retro_scheduler_set_mode(self._h, mode))
+
+
+# ---- the synchronous batch driver (crates/retrograd-infer/src/sync.rs) -----------------------------
+
+@dataclass
+class Completion:
+    """sync.rs:20-37: one completion of a request, assembled from its token events."""
+    tokens: List[int] = field(default_factory=list)
+    logprobs: List[float] = field(default_factory=list)
+    forced: List[bool] = field(default_factory=list)
+    text: str = ""
+    finish: Optional[str] = None
+
+
+@dataclass
+class RequestOutcome:
+    """sync.rs:39-45: one completion per sampling entry, or the error that failed the request."""
+    completions: List[Completion]
+    error: Optional[InferError] = None
+
+    def absorb(self, e: Event) -> None:
+        if e.type == "Error":
+            self.error = e.error
+            return
+        if e.index >= len(self.completions):
+            self.error = InferError("Failed", "a%s event named completion %d, but the request has %d"
+                                    % (" token" if e.type == "Token" else "n end", e.index, len(self.completions)))
+            return
+        member = self.completions[e.index]
+        if e.type == "Token":
+            member.tokens.append(e.token)
+            member.logprobs.append(e.logprob)
+            member.forced.append(e.forced)
+            member.text += e.text
+        else:
+            member.finish = e.reason
+            member.text += e.text
+
+
+def run_requests(scheduler: Scheduler, requests: Sequence[Request], on_step=None) -> List[RequestOutcome]:
+    """sync.rs:96-149: submits the requests in order (as the admission queue has room) and pumps until every
+    one has ended, draining the streams after each step; one outcome per request in submission order. A request
+    whose reservation can never fit comes back as an error in its outcome; a step failure is raised."""
+    pending = list(requests)
+    streams: List[EventStream] = []
+    outcomes: List[RequestOutcome] = []
+    capacity = scheduler.queue_capacity()
+    stalled = 0
+    while True:
+        while pending and scheduler.queued_len() < capacity:
+            request = pending.pop(0)
+            streams.append(scheduler.submit(request))
+            outcomes.append(RequestOutcome([Completion() for _ in request.sampling]))
+        if not pending and scheduler.is_idle():
+            break
+        progressed = scheduler.pump()
+        if on_step:
+            on_step(scheduler)
+        for stream, outcome in zip(streams, outcomes):
+            for event in stream.drain():
+                outcome.absorb(event)
+        stalled = 0 if progressed else stalled + 1
+        if stalled > 1024:
+            raise InferError("Failed", "the scheduler made no progress with requests still queued")
+    for stream, outcome in zip(streams, outcomes):
+        for event in stream.drain():
+            outcome.absorb(event)
+    return outcomes

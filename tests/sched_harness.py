@@ -128,6 +128,29 @@ class Harness:
     def run_until_idle(self):
         self.s.run_until_idle()
 
+    def run_requests(self, requests):
+        """sync.rs run_requests; requests are (prompt, sampling) pairs. Returns per request
+        (completions [(tokens, rounded logprobs, forced, text, finish)], error kind or None)."""
+        if self.kind == "product":
+            reqs = [S.Request(list(p), [_product_sampling(x) for x in samp]) for p, samp in requests]
+            return [([(c.tokens, [_r(v) for v in c.logprobs], c.forced, c.text, c.finish) for c in o.completions],
+                     o.error.kind if o.error else None) for o in S.run_requests(self.s, reqs)]
+        reqs = [O.Request(list(p), [_oracle_sampling(x) for x in samp]) for p, samp in requests]
+        return [([(c["tokens"], [_r(v) for v in c["logprobs"]], c["forced"], c["text"], c["finish"]) for c in o["completions"]],
+                 o["error"].kind if o["error"] else None) for o in O.run_requests(self.s, reqs)]
+
+    def lend_slot(self, cells):
+        return self.s.lend_slot(cells)
+
+    def seq_pos(self, slot):
+        return self.s.fake.seq_pos(slot) if self.kind == "product" else self.backend.seq_pos(slot)
+
+    def cells_used(self):
+        return self.s.fake.cells_used if self.kind == "product" else self.backend.cells_used()
+
+    def is_idle(self):
+        return self.s.is_idle()
+
     def queued(self) -> int:
         return self.s.queued_len()
 

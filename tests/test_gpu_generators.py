@@ -279,3 +279,44 @@ def test_argument_errors(model_path):
         eng.generate_continuous([([1], p(1, top_p=1.5))], 4)
     assert eng.generate_batch([1], [p(1, max_new=2), p(2, max_new=2)], 4)[0][0]
     eng.close()
+
+
+def test_prefix_cache_reuse_matches_cold_generation(model_path):
+    """reference tests/infer_runtime.rs:243-329: requests served from the scheduler's prefix tree (a partial
+    copy of a shared prefix; a fully cached prompt served by replaying its last token) generate what the
+    continuous generator generates cold. The reference asserts it bit for bit on its CPU path; here the
+    warm path prefills a suffix where the cold path prefills the whole prompt, in launches of another
+    shape, so the logits agree to accumulation order and the sampled tokens are compared."""
+    print("prefix cache warm vs cold", flush=True)
+    config = E.EngineConfig(n_ctx=256, n_seq_max=4, n_batch=64, n_ubatch=64)
+    ref = E.Engine(model_path, config)
+    rng = np.random.default_rng(31)
+    shared = [int(t) for t in rng.integers(0, SHAPE.n_vocab, 96)]
+    suffix_a, suffix_b = ([int(t) for t in rng.integers(0, SHAPE.n_vocab, n)] for n in (5, 6))
+    prompt_a = shared + suffix_a
+    ref_a = ref.generate_continuous([(prompt_a, p(81, 5))], 5)
+    wave2 = [(shared + suffix_b, p(82, 5)), (shared, p(83, 5))]
+    ref_b = ref.generate_continuous(wave2, 5)
+    ref.close()
+
+    def v2(params):
+        temperature, top_p, max_new, seed = params
+        return E.SamplingParamsV2(temperature=temperature, top_p=top_p, seed=seed, max_new_tokens=max_new)
+
+    eng = E.Engine(model_path, config)
+    sched = S.Scheduler.over_engine(eng, S.SchedulerOptions(mode=S.LOCKSTEP, n_batch=64, queue_capacity=16, event_capacity=256))
+    sched.initialize()
+    stream = sched.submit(S.Request.single(prompt_a, v2(p(81, 5))))
+    sched.run_until_idle()
+    toks, _, _ = drain(stream)
+    assert toks == ref_a[0][0]
+    assert sched.kv_stats().nodes == 1
+    streams = [sched.submit(S.Request.single(prompt, v2(sampling))) for prompt, sampling in wave2]
+    sched.run_until_idle()
+    for index, stream in enumerate(streams):
+        toks, _, end = drain(stream)
+        assert toks == ref_b[index][0], "wave 2 request %d (request 1 is a full-prompt hit)" % index
+        assert end.cached_tokens == (96 if index == 0 else 95)
+    assert sched.kv_stats().hits == 2
+    sched.close()
+    eng.close()

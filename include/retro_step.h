@@ -283,7 +283,11 @@ int retro_engine_detokenize(
     char * buffer, size_t n_buffer, size_t * out_n_bytes);
 int retro_engine_graphs_reused(retro_engine * engine, uint64_t * out_n_reused);
 
-/* ---- adapters: ref h:2574, 2584, 2616 (named), h:2597-2605 (per row) ----- */
+/* ---- adapters: ref h:2566-2567 (the one context-wide adapter), h:2574, 2584, 2616 (named), h:2597-2605 (per row).
+ * The active context-wide adapter is what rows with adapter 0 decode under. Every change of what is active
+ * is a weight change: all cells and the generators' bookkeeping are dropped, the weights version moves on. */
+int retro_engine_load_lora(retro_engine * engine, const char * adapter_path);
+int retro_engine_set_lora_enabled(retro_engine * engine, bool enabled);
 int retro_engine_load_lora_named(retro_engine * engine, const char * name, const char * adapter_path);
 int retro_engine_activate_lora(retro_engine * engine, const char * name);
 int retro_engine_active_adapter(

@@ -462,33 +462,59 @@ int retro_engine_graphs_reused(retro_engine * engine, uint64_t * out_n_reused) {
 
 // ---- adapters ---------------------------------------------------------------------------
 
+int retro_engine_load_lora(retro_engine * engine, const char * adapter_path) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        if (blank(adapter_path)) {
+            set_error("adapter_path is required");
+            return -1;
+        }
+        return e->load_lora(adapter_path);
+    });
+}
+
+int retro_engine_set_lora_enabled(retro_engine * engine, bool enabled) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->set_lora_enabled(enabled);
+    });
+}
+
 int retro_engine_load_lora_named(retro_engine * engine, const char * name, const char * adapter_path) {
     return boundary([&]() -> int {
-        if (!checked(engine)) return -1;
-        (void)name;
-        (void)adapter_path;
-        set_error("named LoRA adapters are not supported by this library yet");
-        return -1;
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        if (blank(name)) {
+            set_error("name is required");
+            return -1;
+        }
+        if (blank(adapter_path)) {
+            set_error("adapter_path is required");
+            return -1;
+        }
+        return e->load_lora_named(name, adapter_path);
     });
 }
 
 int retro_engine_activate_lora(retro_engine * engine, const char * name) {
     return boundary([&]() -> int {
-        if (!checked(engine)) return -1;
-        if (blank(name)) return 0;   // the base model is what is active
-        set_error("named LoRA adapters are not supported by this library yet");
-        return -1;
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return e->activate_lora(name ? name : "");
     });
 }
 
 int retro_engine_active_adapter(retro_engine * engine, char * buffer, size_t n_buffer, size_t * out_n_bytes) {
     return boundary([&]() -> int {
-        if (!checked(engine)) return -1;
+        Engine * e = checked(engine);
+        if (!e) return -1;
         if (!out_n_bytes) {
             set_error("out_n_bytes is required");
             return -1;
         }
-        return string_out(std::string(), buffer, n_buffer, out_n_bytes);
+        return string_out(e->active_adapter(), buffer, n_buffer, out_n_bytes);
     });
 }
 

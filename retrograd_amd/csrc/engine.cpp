@@ -1358,7 +1358,15 @@ int Engine::adapter_snapshot(int32_t replace, float scale, int32_t * out_id) {
         set_error("per-row adapter ids are exhausted");
         return -1;
     }
-    const RowAdapterData & src = policy->second;
+    RowAdapterData copy = clone_adapter(policy->second, scale);
+    const int32_t id = next_adapter_id_++;
+    row_adapters_.emplace(id, std::move(copy));
+    rebuild_lora_table();
+    *out_id = id;
+    return 0;
+}
+
+Engine::RowAdapterData Engine::clone_adapter(const RowAdapterData & src, float scale) {
     RowAdapterData copy;
     copy.scale = scale;
     copy.alpha = src.alpha;
@@ -1376,10 +1384,66 @@ int Engine::adapter_snapshot(int32_t replace, float scale, int32_t * out_id) {
         hip_check(hipMemcpyAsync(copy.b[i].ptr, src.b[i].ptr, src.b[i].bytes, hipMemcpyDeviceToDevice, stream_), "hipMemcpyAsync");
     }
     hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
-    const int32_t id = next_adapter_id_++;
-    row_adapters_.emplace(id, std::move(copy));
+    return copy;
+}
+
+// ---- context-wide adapters (reference retro_engine.cpp:756-870) ----------------------------
+// Adapters registered under a name, one of them active: what rows with adapter 0 decode under.
+// Every change of what is active is a change of the weights: all cells and the generators'
+// bookkeeping go, the weights version moves on (forget_engine_kv, retro_engine.cpp:322-328).
+
+void Engine::apply_active_adapter() {
+    hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    row_adapters_.erase(kPolicyAdapter);
+    if (!active_adapter_.empty())
+        row_adapters_.emplace(kPolicyAdapter, clone_adapter(named_adapters_.at(active_adapter_), 1.0f));
     rebuild_lora_table();
-    *out_id = id;
+}
+
+int Engine::load_lora_named(const std::string & name, const std::string & path) {
+    RowAdapterData data;
+    if (read_adapter(path, 1.0f, data) != 0) return -1;
+    const bool was_active = active_adapter_ == name;
+    named_adapters_.erase(name);
+    named_adapters_.emplace(name, std::move(data));
+    if (was_active) {              // registered beside the others, not applied - unless it replaces the active one
+        apply_active_adapter();
+        forget_generation_kv();
+    }
+    return 0;
+}
+
+int Engine::load_lora(const std::string & path) {
+    RowAdapterData data;
+    if (read_adapter(path, 1.0f, data) != 0) return -1;
+    named_adapters_.clear();       // the single-adapter contract: every other adapter goes
+    named_adapters_.emplace(path, std::move(data));
+    active_adapter_ = path;
+    apply_active_adapter();
+    forget_generation_kv();
+    return 0;
+}
+
+int Engine::activate_lora(const std::string & name) {
+    if (!name.empty() && !named_adapters_.count(name)) {
+        set_error("no LoRA adapter registered under '" + name + "'");
+        return -1;
+    }
+    active_adapter_ = name;
+    apply_active_adapter();
+    forget_generation_kv();
+    return 0;
+}
+
+int Engine::set_lora_enabled(bool enabled) {
+    if (!enabled) {
+        active_adapter_.clear();
+    } else if (active_adapter_.empty()) {
+        set_error("cannot enable LoRA: no adapter is active");
+        return -1;
+    }
+    apply_active_adapter();
+    forget_generation_kv();
     return 0;
 }
 

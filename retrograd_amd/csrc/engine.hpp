@@ -129,6 +129,12 @@ public:
         GgufFile file(path);
         return (uint64_t)file.require("token_embd.weight").ne[1];
     }
+    // context-wide adapters, registered by name, one active
+    int load_lora(const std::string & path);
+    int load_lora_named(const std::string & name, const std::string & path);
+    int activate_lora(const std::string & name);
+    int set_lora_enabled(bool enabled);
+    const std::string & active_adapter() const { return active_adapter_; }
     // the generation side of a trainer handle
     int policy_adapter_load(const std::string & path);
     bool has_policy_adapter() const { return row_adapters_.count(kPolicyAdapter) != 0; }
@@ -269,6 +275,10 @@ private:
     bool ggml_activations_ = false;   // RETRO_ACTIVATIONS=ggml at construction
     void rebuild_lora_table();
     int read_adapter(const std::string & path, float scale, RowAdapterData & data);
+    RowAdapterData clone_adapter(const RowAdapterData & src, float scale);
+    void apply_active_adapter();
+    std::map<std::string, RowAdapterData> named_adapters_;
+    std::string active_adapter_;
     // id of the trained adapter among the per-row adapters: never handed out, never accepted from a caller
     static constexpr int32_t kPolicyAdapter = INT32_MAX;
     int32_t default_adapter_ = 0;

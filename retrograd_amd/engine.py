@@ -124,6 +124,7 @@ STEP_SYMBOLS = [
     "retro_engine_kv_unified", "retro_engine_weights_version", "retro_engine_model_fingerprint",
     "retro_engine_is_hybrid", "retro_engine_eos_token", "retro_engine_vocab_size", "retro_engine_is_eog_token",
     "retro_engine_context_size", "retro_engine_detokenize", "retro_engine_graphs_reused",
+    "retro_engine_load_lora", "retro_engine_set_lora_enabled",
     "retro_engine_load_lora_named", "retro_engine_activate_lora", "retro_engine_active_adapter",
     "retro_engine_adapter_load", "retro_engine_adapter_unload", "retro_engine_adapter_rows_info",
     "retro_grammar_from_json_schema", "retro_grammar_from_gbnf", "retro_grammar_json_object",
@@ -184,6 +185,8 @@ def load_library() -> C.CDLL:
     lib.retro_engine_detokenize.argtypes = [C.c_void_p, _i32p, C.c_size_t, C.c_bool, C.c_char_p, C.c_size_t,
                                             C.POINTER(C.c_size_t)]
     lib.retro_engine_graphs_reused.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
+    lib.retro_engine_load_lora.argtypes = [C.c_void_p, C.c_char_p]
+    lib.retro_engine_set_lora_enabled.argtypes = [C.c_void_p, C.c_bool]
     lib.retro_engine_load_lora_named.argtypes = [C.c_void_p, C.c_char_p, C.c_char_p]
     lib.retro_engine_activate_lora.argtypes = [C.c_void_p, C.c_char_p]
     lib.retro_engine_active_adapter.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]
@@ -670,6 +673,41 @@ class Engine:
             _raise(s)
         return buf.raw[:n.value]
 
+    # -- context-wide adapters: what rows with adapter 0 decode under ---------------------------
+    def load_lora(self, path) -> None:
+        """The one context-wide adapter: every other registered adapter goes, this one is active."""
+        s = self._lib.retro_engine_load_lora(self._h, os.fsencode(str(path)))
+        if s != 0:
+            _raise(s)
+
+    def set_lora_enabled(self, enabled: bool) -> None:
+        s = self._lib.retro_engine_set_lora_enabled(self._h, enabled)
+        if s != 0:
+            _raise(s)
+
+    def load_lora_named(self, name: str, path) -> None:
+        s = self._lib.retro_engine_load_lora_named(self._h, name.encode(), os.fsencode(str(path)))
+        if s != 0:
+            _raise(s)
+
+    def activate_lora(self, name: str | None) -> None:
+        """None or "": the base model."""
+        s = self._lib.retro_engine_activate_lora(self._h, (name or "").encode())
+        if s != 0:
+            _raise(s)
+
+    def active_adapter(self) -> str:
+        n = C.c_size_t()
+        s = self._lib.retro_engine_active_adapter(self._h, None, 0, C.byref(n))
+        if s != 0:
+            _raise(s)
+        buf = C.create_string_buffer(n.value + 1)
+        s = self._lib.retro_engine_active_adapter(self._h, buf, n.value + 1, C.byref(n))
+        if s != 0:
+            _raise(s)
+        return buf.raw[:n.value].decode()
+
+    # -- per-row adapters --------------------------------------------------------------------
     def adapter_load(self, path, scale: float = 1.0) -> int:
         out = C.c_int32()
         s = self._lib.retro_engine_adapter_load(self._h, os.fsencode(str(path)), scale, C.byref(out))

@@ -100,6 +100,114 @@ def test_rows_under_adapters_with_the_ggml_arithmetic(files, monkeypatch):
     eng.close()
 
 
+def test_the_context_adapter_and_per_row_adapters_share_a_step(files):
+    """reference tests/lora_rows.rs:150-237: the context's own adapter is what rows with adapter 0
+    follow, the others ignore it; every row of the mixed step matches the oracle's row under that
+    adapter alone; unloading restacks; an empty routed set still bypasses the context adapter."""
+    model, a1, a2, _ = files
+    print("context adapter + per-row adapters", flush=True)
+    eng = E.Engine(model, E.EngineConfig(n_ctx=1024, n_seq_max=4, n_batch=128, n_ubatch=128))
+    m = oracle.Model(model)
+    oid_a, oid_b = m.load_adapter(a1, 1.0), m.load_adapter(a2, 1.0)
+    prompt = [int(t) for t in np.random.default_rng(4).integers(0, m.n_vocab, 23)]
+    plan = [(i, 0, prompt, True) for i in range(4)]
+    id_a, id_b = eng.adapter_load(a1, 1.0), eng.adapter_load(a2, 1.0)
+    v0 = eng.weights_version()
+    eng.load_lora(a2)                                 # the context's own adapter is b
+    assert eng.active_adapter() == str(a2) and eng.weights_version() == v0 + 1
+    out = E.StepOutput()
+    route = [id_a, id_b, E.RETRO_STEP_ADAPTER_BASE, 0]
+    eng.step([E.StepRow(i + 1, i, prompt, 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(route[i])) for i in range(4)], out)
+    got = eng.debug_logits()
+    want = oracle.Context(m, 4).step_rows(plan, adapters=[oid_a, oid_b, -1, oid_b])
+    assert_logits_close(got, want)
+    base = oracle.Context(m, 4).step_rows(plan)
+    assert np.abs(want[0] - base[0]).max() > 5e-2, "the adapter must move the distribution, or the parity is vacuous"
+    assert np.array_equal(got[1], got[3]), "a context row and a per-row b row are the same arithmetic"
+    info = eng.adapter_rows_info()
+    assert (info.n_adapters, info.max_rank) == (2, 16) and info.stacked_bytes > info.unpadded_bytes
+
+    # unloading a restacks b alone; ids are not reused
+    eng.adapter_unload(id_a)
+    with pytest.raises(E.RuntimeFailure):
+        eng.adapter_unload(id_a)
+    for slot in range(4):
+        eng.seq_rm(slot)
+    eng.step([E.StepRow(5, 0, prompt, 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(id_b))], out)
+    assert_logits_close(eng.debug_logits(), want[1:2])
+    with pytest.raises(E.InvalidArgument):
+        eng.step([E.StepRow(6, 1, prompt, 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(id_a))], out)
+
+    # an empty routed set still bypasses the context adapter
+    eng.adapter_unload(id_b)
+    for slot in range(4):
+        eng.seq_rm(slot)
+    eng.step([E.StepRow(7 + i, i, prompt, 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(E.RETRO_STEP_ADAPTER_BASE))
+              for i in range(4)], out)
+    assert_logits_close(eng.debug_logits(), base)
+
+    # named adapters: registered beside the others, one active; every switch is a weight change
+    eng.load_lora_named("a", a1)
+    assert eng.active_adapter() == str(a2), "registering does not activate"
+    v1 = eng.weights_version()
+    eng.activate_lora("a")
+    assert eng.active_adapter() == "a" and eng.weights_version() == v1 + 1
+    assert eng.memory().cells_used == 0, "a switch drops every resident cell"
+    eng.step([E.StepRow(20, 0, prompt, 0, sample=True, sampling=greedy())], out)
+    assert_logits_close(eng.debug_logits(), want[0:1])
+    with pytest.raises(E.RuntimeFailure, match="no LoRA adapter registered under 'zzz'"):
+        eng.activate_lora("zzz")
+    eng.set_lora_enabled(False)
+    assert eng.active_adapter() == ""
+    eng.step([E.StepRow(21, 0, prompt, 0, sample=True, sampling=greedy())], out)
+    assert_logits_close(eng.debug_logits(), base[0:1])
+    with pytest.raises(E.RuntimeFailure, match="cannot enable LoRA: no adapter is active"):
+        eng.set_lora_enabled(True)
+    eng.close()
+
+
+def test_the_scheduler_serves_a_named_adapter_through_the_engine(files):
+    """A request that names an adapter (reference crates/retrograd-infer/tests/adapters.rs, there on the
+    fake backend) is decoded under that context-wide adapter of the engine: the tokens are those of the
+    same prompt under the same file as a per-row adapter, and the base model's afterwards."""
+    from retrograd_amd import scheduler as S
+    model, a1, _, _ = files
+    print("scheduler: named adapter over the engine", flush=True)
+    eng = E.Engine(model, E.EngineConfig(n_ctx=512, n_seq_max=4, n_batch=64, n_ubatch=64))
+    sched = S.Scheduler.over_engine(eng, S.SchedulerOptions(mode=S.CONTINUOUS, n_batch=64, event_capacity=64))
+    sched.initialize()
+    sched.load_adapter("tuned", str(a1))
+    prompt = [int(t) for t in np.random.default_rng(8).integers(0, SHAPE.n_vocab, 19)]
+
+    def run(adapter):
+        stream = sched.submit(S.Request(prompt, [E.SamplingParamsV2.greedy(max_new_tokens=4)], adapter=adapter))
+        sched.run_until_idle()
+        events = list(stream.drain())
+        assert not [e for e in events if e.type == "Error"], events
+        return [e.token for e in events if e.type == "Token"]
+
+    tuned, plain = run("tuned"), run(None)
+    assert eng.active_adapter() == ""
+    sched.close()
+    ref = E.Engine(model, E.EngineConfig(n_ctx=512, n_seq_max=4, n_batch=64, n_ubatch=64))
+    rid = ref.adapter_load(a1, 1.0)
+    out = E.StepOutput()
+
+    def greedy_decode(adapter):
+        ref.seq_rm(0)
+        ref.step([E.StepRow(1, 0, prompt, 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(adapter))], out)
+        toks = [out.row(0).token]
+        for i in range(3):
+            ref.step([E.StepRow(1, 0, [toks[-1]], len(prompt) + i, sample=True, sampling=greedy(), adapter=E.RowAdapter(adapter))], out)
+            toks.append(out.row(0).token)
+        return toks
+
+    assert tuned == greedy_decode(rid) and plain == greedy_decode(E.RETRO_STEP_ADAPTER_BASE)
+    assert tuned != plain
+    eng.close()
+    ref.close()
+
+
 def test_adapter_errors_and_unload(files):
     model, a1, a2, ffn = files
     print("per-row LoRA: argument errors", flush=True)

@@ -11,7 +11,7 @@ prefill: when a request finishes and a new one is admitted into its slot, the
 new prompt is prefilled in its own (untimed, separately reported) steps before
 the decode batch resumes with all 64 sequences live.
 
-Workload (BASELINE.json configs[1]): 32 layers, hidden 4096, 32/8 heads of 128,
+Workload (the second configuration of the benchmark set): 32 layers, hidden 4096, 32/8 heads of 128,
 FFN 14336, vocab 128256, Q4_K matrices, f16 KV; 64 concurrent sequences,
 prompt lengths log-uniform in [128, 4096], uniform random token ids, greedy
 (top_k = 1), 256 new tokens each, a new request admitted whenever one finishes.

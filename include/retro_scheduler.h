@@ -4,7 +4,7 @@
  * exposes it as a crate API, not as C functions, so these entry points have no
  * C counterpart there: each one names the Rust item it mirrors. A Rust
  * maintainer would bind them with an `unsafe extern "C"` block and implement
- * `retrograd_infer`'s public types on top (see INTEGRATION.md).
+ * `retrograd_infer`'s public types on top.
  *
  * Every function returns 0 on success and a negative code otherwise:
  * -(retro_sched_error_kind) of the failure, with the message available from

@@ -1,6 +1,6 @@
 """The decode step on the GPU against the CPU oracle, through the C ABI.
 
-Tolerances are BASELINE's: logits within 2e-2 max-abs and 1e-3 mean-abs
+Tolerances of the benchmark definition: logits within 2e-2 max-abs and 1e-3 mean-abs
 relative error; packing, cells, slot ranges and greedy token ids bit-exact
 (token ids are compared where the oracle's own top-1/top-2 margin exceeds the
 logit tolerance - a margin below the tolerance is a tie no two float

@@ -469,7 +469,21 @@ __global__ __launch_bounds__(256) void k_mm_q8_0(MMArgs a) {
     mm_finish<NT>(a, acc, rt, tbase, nt, wk, wr, lds);
 }
 
-// Any type, any shape: one wave per output feature, raw GGUF rows.
+// The operand of a product with a weight of storage type round_as under ggml's arithmetic (WT_F32: as it is).
+__device__ __forceinline__ float generic_operand(float hi, float lo, int round_as) {
+    // F16 weights multiply the activations rounded to f16 (the hi half is that rounding), BF16 weights those
+    // rounded to bf16
+    if (round_as == WT_F16) return hi;
+    float xv = hi + lo;
+    if (round_as == WT_BF16) {
+        uint32_t u = __float_as_uint(xv);
+        u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+        xv = __uint_as_float(u);
+    }
+    return xv;
+}
+
+// Any type, any shape: one wave per output feature and group of eight tokens, raw GGUF rows.
 __global__ __launch_bounds__(256) void k_mm_generic(int type, const uint8_t * __restrict__ raw, size_t rb,
                                                     const __half * __restrict__ x, int K, int N, int T,
                                                     float * y, int ldy, int col0, int mode, const float * bias,
@@ -478,33 +492,39 @@ __global__ __launch_bounds__(256) void k_mm_generic(int type, const uint8_t * __
     const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (n >= N) return;
     const uint8_t * row = raw + (size_t)n * rb;
-    for (int t0 = 0; t0 < T; t0 += 8) {
-        float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int t0 = blockIdx.y * 8;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (K % 8 == 0) {
+        // eight consecutive k per lane: the activations of a token are 16 contiguous bytes per half
+        for (int k = lane * 8; k < K; k += 512) {
+            float w[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) w[i] = decode_elem(type, row, k + i);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int t = min(t0 + j, T - 1);
+                const h8 hi = load_h8(x + act_at(t, k, 0, K)), lo = load_h8(x + act_at(t, k, 1, K));
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[j] = fmaf(w[i], generic_operand((float)hi[i], (float)lo[i], round_as), acc[j]);
+            }
+        }
+    } else {
         for (int k = lane; k < K; k += 64) {
             const float w = decode_elem(type, row, k);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const int t = min(t0 + j, T - 1);
-                // under ggml's arithmetic (round_as = the weight type) F16 weights multiply the activations
-                // rounded to f16 (the hi half is that rounding) and BF16 weights those rounded to bf16
-                float xv = __half2float(x[act_at(t, k, 0, K)]);
-                if (round_as != WT_F16) xv += __half2float(x[act_at(t, k, 1, K)]);
-                if (round_as == WT_BF16) {
-                    uint32_t u = __float_as_uint(xv);
-                    u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
-                    xv = __uint_as_float(u);
-                }
-                acc[j] = fmaf(w, xv, acc[j]);
+                acc[j] = fmaf(w, generic_operand(__half2float(x[act_at(t, k, 0, K)]), __half2float(x[act_at(t, k, 1, K)]), round_as), acc[j]);
             }
         }
+    }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float v = wave_sum(acc[j]);
-            if (lane == 0 && t0 + j < T) {
-                float * p = y + (size_t)(t0 + j) * ldy + col0 + n;
-                const float o = v + (bias ? bias[n] : 0.0f);
-                *p = mode == MM_ADD ? *p + o : o;
-            }
+    for (int j = 0; j < 8; ++j) {
+        const float v = wave_sum(acc[j]);
+        if (lane == 0 && t0 + j < T) {
+            float * p = y + (size_t)(t0 + j) * ldy + col0 + n;
+            const float o = v + (bias ? bias[n] : 0.0f);
+            *p = mode == MM_ADD ? *p + o : o;
         }
     }
 }
@@ -516,7 +536,7 @@ void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float
     if (T <= 0) return;
     const Act xo = x.operand(w.type);
     if (!xo.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
-    hipLaunchKernelGGL(k_mm_generic, dim3((w.N + 3) / 4), dim3(256), 0, s, w.type, w.raw, row_bytes(w.type, w.K),
+    hipLaunchKernelGGL(k_mm_generic, dim3((w.N + 3) / 4, (T + 7) / 8), dim3(256), 0, s, w.type, w.raw, row_bytes(w.type, w.K),
                        xo.x, w.K, w.N, T, y, ldy, col0, mode, bias, xo.faithful ? w.type : WT_F32);
     check_launch("matmul_generic");
 }

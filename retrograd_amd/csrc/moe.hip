@@ -5,7 +5,10 @@
 // a batch has a few dozen tokens), so the work is organised by expert: the
 // (token, choice) pairs of a step are grouped by expert, every expert's range
 // padded to whole 16-token MFMA tiles, and one wave owns one 16-row weight tile
-// of one expert and streams it exactly once per 32 tokens of that expert:
+// of one expert and streams it exactly once per 32 tokens of that expert; the
+// four waves of a workgroup own four tiles of the same expert and share its
+// activations through LDS (read from global memory per wave they cost several
+// times the bytes of the weights):
 //
 //   k_moe_route     per token: top-k of the router logits, weights in double
 //   k_moe_group     stable counting sort of the pairs by expert (one workgroup)
@@ -153,43 +156,94 @@ struct MoeArgs {
     int n_expert, K, N;        // N output features per expert, K inputs
 };
 
-// One wave per (expert, 16 output features): gate and up tiles together, SwiGLU in the epilogue.
+// The activations of one super-block (256 k) for up to two 16-token tiles, staged once per workgroup: its four
+// waves own four row tiles of the same expert and multiply them with the same rows. A tile's share is 8 k-steps
+// x (hi, lo) x 64 lanes of 16 bytes, in the order the MFMA operand wants them, so a wave reads its fragments
+// back with one conflict-free 16-byte read per lane.
+constexpr int kStageTile = 8 * 2 * 64 * 16;        // bytes per token tile and super-block
+
+struct StageRegs { u4 v[8]; };
+
+// rows[32]: for every row of the (up to) two tiles, the row of the activation buffer it reads.
+__device__ __forceinline__ void stage_load(const __half * x, int K, const int * rows, int sb, int nt, StageRegs & regs) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        if (c >= 4 * nt) break;
+        const int chunk = c * 256 + threadIdx.x;
+        const int t = chunk >> 10, rem = chunk & 1023;
+        const int s = rem >> 7, hl = (rem >> 6) & 1, ln = rem & 63;
+        const int k = sb * 256 + s * 32 + 8 * (ln >> 4);
+        regs.v[c] = *(const u4 *)(x + act_at(rows[t * 16 + (ln & 15)], k, hl, K));
+    }
+}
+
+__device__ __forceinline__ void stage_store(uint8_t * buf, int nt, const StageRegs & regs) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        if (c >= 4 * nt) break;
+        *(u4 *)(buf + (size_t)(c * 256 + threadIdx.x) * 16) = regs.v[c];
+    }
+}
+
+__device__ __forceinline__ h8 staged(const uint8_t * buf, int t, int s, int hl, int lane) {
+    return *(const h8 *)(buf + t * kStageTile + ((s * 2 + hl) * 64 + lane) * 16);
+}
+
+// One workgroup per (expert, four consecutive tiles of 16 output features), one wave per tile: gate and up
+// tiles together, SwiGLU in the epilogue. The weights of the next super-block and the activations of the next
+// super-block are requested before the current one is multiplied.
 template <int TYPE>
 __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
-    const int lane = threadIdx.x & 63;
+    __shared__ __attribute__((aligned(16))) uint8_t stage[2][2 * kStageTile];
+    __shared__ int rows[32];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const int n_tiles = a.N / 16;
-    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int e = item / n_tiles, ft = item % n_tiles;
+    const int item0 = blockIdx.x * 4;
+    const int e = item0 / n_tiles, ft = item0 % n_tiles + wave;     // n_tiles % 4 == 0: one expert per workgroup
     if (e >= a.n_expert) return;
     const int n_e = a.expert_n[e];
     if (n_e == 0) return;
     const int qb = a.off_pad[e];
     const int nsb = a.K >> 8;
-    const size_t tile0 = ((size_t)e * n_tiles + ft) * nsb * Tile<TYPE>::BYTES;
+    const uint8_t * wg = a.w0 + ((size_t)e * n_tiles + ft) * nsb * Tile<TYPE>::BYTES;
+    const uint8_t * wu = a.w1 + ((size_t)e * n_tiles + ft) * nsb * Tile<TYPE>::BYTES;
     for (int t0 = 0; t0 < n_e; t0 += 32) {
-        int tok[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            const int at = t0 + t * 16 + r16;
+        const int nt = n_e - t0 > 16 ? 2 : 1;
+        __syncthreads();                       // the last pass is done with rows and the staging buffers
+        if (threadIdx.x < 32) {
+            const int at = t0 + threadIdx.x;
             const int tk = at < n_e ? a.tok_of_q[qb + at] : -1;
-            tok[t] = tk < 0 ? 0 : tk;          // padding rows read token 0 and are never stored
+            rows[threadIdx.x] = tk < 0 ? 0 : tk;        // padding rows read token 0 and are never stored
         }
+        __syncthreads();
+        StageRegs regs;
+        stage_load(a.x.x, a.K, rows, 0, nt, regs);
+        Tile<TYPE> tg, tu;
+        tg.load(wg, lane);
+        tu.load(wu, lane);
+        stage_store(stage[0], nt, regs);
+        __syncthreads();
         f4 ag[2], au[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) { ag[t] = (f4){0.f, 0.f, 0.f, 0.f}; au[t] = (f4){0.f, 0.f, 0.f, 0.f}; }
         for (int sb = 0; sb < nsb; ++sb) {
-            Tile<TYPE> tg, tu;
-            tg.load(a.w0 + tile0 + (size_t)sb * Tile<TYPE>::BYTES, lane);
-            tu.load(a.w1 + tile0 + (size_t)sb * Tile<TYPE>::BYTES, lane);
+            const bool more = sb + 1 < nsb;
+            Tile<TYPE> ng = tg, nu = tu;
+            if (more) {
+                stage_load(a.x.x, a.K, rows, sb + 1, nt, regs);
+                ng.load(wg + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
+                nu.load(wu + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
+            }
+            const uint8_t * cur = stage[sb & 1];
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
                 const h8 bg = tg.frag(s), bu = tu.frag(s);
                 const float dg = tg.scale(s), du = tu.scale(s);
-                const int k = sb * 256 + s * 32 + 8 * g;
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    const h8 hi = load_h8(a.x.x + act_at(tok[t], k, 0, a.K)), lo = load_h8(a.x.x + act_at(tok[t], k, 1, a.K));
+                    if (t >= nt) break;
+                    const h8 hi = staged(cur, t, s, 0, lane), lo = staged(cur, t, s, 1, lane);
                     const f4 pg = mfma2(hi, lo, bg), pu = mfma2(hi, lo, bu);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
@@ -198,13 +252,17 @@ __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
                     }
                 }
             }
+            if (more) stage_store(stage[(sb + 1) & 1], nt, regs);
+            __syncthreads();
+            tg = ng;
+            tu = nu;
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int at = t0 + t * 16 + 4 * g + i;
-                if (at >= n_e) continue;
+                if (t >= nt || at >= n_e) continue;
                 const float gv = ag[t][i];
                 const float v = fminf(fmaxf((gv / (1.0f + __expf(-gv))) * au[t][i], -65504.0f), 65504.0f);
                 const __half hh = __float2half_rn(v);
@@ -215,48 +273,66 @@ __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
     }
 }
 
-// One wave per (expert, 16 output features of the model width).
+// One workgroup per (expert, four consecutive tiles of 16 output features of the model width), one wave per
+// tile; the hidden rows of the expert's pairs are staged like the activations above.
 template <int TYPE>
 __global__ __launch_bounds__(256) void k_moe_down(MoeArgs a) {
-    const int lane = threadIdx.x & 63;
+    __shared__ __attribute__((aligned(16))) uint8_t stage[2][2 * kStageTile];
+    __shared__ int rows[32];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const int n_tiles = a.N / 16;
-    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int e = item / n_tiles, et = item % n_tiles;
+    const int item0 = blockIdx.x * 4;
+    const int e = item0 / n_tiles, et = item0 % n_tiles + wave;
     if (e >= a.n_expert) return;
     const int n_e = a.expert_n[e];
     if (n_e == 0) return;
     const int qb = a.off_pad[e];
     const int nsb = a.K >> 8;
-    const size_t tile0 = ((size_t)e * n_tiles + et) * nsb * Tile<TYPE>::BYTES;
+    const uint8_t * wd = a.w0 + ((size_t)e * n_tiles + et) * nsb * Tile<TYPE>::BYTES;
     for (int t0 = 0; t0 < n_e; t0 += 32) {
-        // the second tile of the last pass may lie past the expert's padded range: read the first tile again
-        const int q0 = qb + t0 + r16;
-        const int q1 = t0 + 16 < n_e ? q0 + 16 : q0;
+        const int nt = n_e - t0 > 16 ? 2 : 1;
+        __syncthreads();
+        // every row of a tile lies in the expert's padded slot range
+        if (threadIdx.x < 32) rows[threadIdx.x] = qb + t0 + (threadIdx.x < 16 * nt ? threadIdx.x : 0);
+        __syncthreads();
+        StageRegs regs;
+        stage_load(a.x.x, a.K, rows, 0, nt, regs);
+        Tile<TYPE> tw;
+        tw.load(wd, lane);
+        stage_store(stage[0], nt, regs);
+        __syncthreads();
         f4 acc[2] = {(f4){0.f, 0.f, 0.f, 0.f}, (f4){0.f, 0.f, 0.f, 0.f}};
         for (int sb = 0; sb < nsb; ++sb) {
-            Tile<TYPE> tw;
-            tw.load(a.w0 + tile0 + (size_t)sb * Tile<TYPE>::BYTES, lane);
+            const bool more = sb + 1 < nsb;
+            Tile<TYPE> nw = tw;
+            if (more) {
+                stage_load(a.x.x, a.K, rows, sb + 1, nt, regs);
+                nw.load(wd + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
+            }
+            const uint8_t * cur = stage[sb & 1];
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
                 const h8 b = tw.frag(s);
                 const float d = tw.scale(s);
-                const int k = sb * 256 + s * 32 + 8 * g;
-                const f4 p0 = mfma2(load_h8(a.x.x + act_at(q0, k, 0, a.K)), load_h8(a.x.x + act_at(q0, k, 1, a.K)), b);
-                const f4 p1 = mfma2(load_h8(a.x.x + act_at(q1, k, 0, a.K)), load_h8(a.x.x + act_at(q1, k, 1, a.K)), b);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    acc[0][i] = fmaf(d, p0[i], acc[0][i]);
-                    acc[1][i] = fmaf(d, p1[i], acc[1][i]);
+                for (int t = 0; t < 2; ++t) {
+                    if (t >= nt) break;
+                    const f4 p = mfma2(staged(cur, t, s, 0, lane), staged(cur, t, s, 1, lane), b);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[t][i] = fmaf(d, p[i], acc[t][i]);
                 }
             }
+            if (more) stage_store(stage[(sb + 1) & 1], nt, regs);
+            __syncthreads();
+            tw = nw;
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int at = t0 + t * 16 + 4 * g + i;
-                if (at < n_e) a.out_pair[(size_t)(qb + at) * a.N + et * 16 + r16] = acc[t][i];
+                if (t < nt && at < n_e) a.out_pair[(size_t)(qb + at) * a.N + et * 16 + r16] = acc[t][i];
             }
     }
 }
@@ -380,6 +456,7 @@ size_t moe_slots(int n_tokens, int k_used, int n_expert) {
 void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act & xn, int T, float * x, const MoeBuffers & b) {
     if (T <= 0) return;
     if (sh.n_expert > 256 || sh.k_used > 16 || sh.k_used > sh.n_expert) throw std::runtime_error("moe: unsupported expert count");
+    // multiples of 256: whole super-blocks along K, and the four waves of a workgroup share an expert (N / 16 % 4 == 0)
     if (sh.E % 256 != 0 || sh.F % 256 != 0) throw std::runtime_error("moe: widths must be multiples of 256");
     if (L.gate.type != L.up.type || (L.gate.type != WT_MXFP4 && L.gate.type != WT_Q8_0) ||
         (L.down.type != WT_MXFP4 && L.down.type != WT_Q8_0))

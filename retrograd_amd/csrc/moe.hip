@@ -162,12 +162,15 @@ struct MoeArgs {
 // back with one conflict-free 16-byte read per lane.
 constexpr int kStageTile = 8 * 2 * 64 * 16;        // bytes per token tile and super-block
 
-struct StageRegs { u4 v[8]; };
+template <int NTMAX> struct StageRegs { u4 v[4 * NTMAX]; };
 
-// rows[32]: for every row of the (up to) two tiles, the row of the activation buffer it reads.
-__device__ __forceinline__ void stage_load(const __half * x, int K, const int * rows, int sb, int nt, StageRegs & regs) {
+// NTMAX = 1 halves the LDS of a workgroup (more of them per compute unit, more weight bytes in flight) and
+// makes an expert with more than 16 pairs stream its weights once per 16 of them: the host picks it for
+// decode-sized steps. rows[32]: for every row of the (up to) two tiles, the row of the activation buffer it reads.
+template <int NTMAX>
+__device__ __forceinline__ void stage_load(const __half * x, int K, const int * rows, int sb, int nt, StageRegs<NTMAX> & regs) {
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
+    for (int c = 0; c < 4 * NTMAX; ++c) {
         if (c >= 4 * nt) break;
         const int chunk = c * 256 + threadIdx.x;
         const int t = chunk >> 10, rem = chunk & 1023;
@@ -177,9 +180,10 @@ __device__ __forceinline__ void stage_load(const __half * x, int K, const int * 
     }
 }
 
-__device__ __forceinline__ void stage_store(uint8_t * buf, int nt, const StageRegs & regs) {
+template <int NTMAX>
+__device__ __forceinline__ void stage_store(uint8_t * buf, int nt, const StageRegs<NTMAX> & regs) {
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
+    for (int c = 0; c < 4 * NTMAX; ++c) {
         if (c >= 4 * nt) break;
         *(u4 *)(buf + (size_t)(c * 256 + threadIdx.x) * 16) = regs.v[c];
     }
@@ -192,9 +196,9 @@ __device__ __forceinline__ h8 staged(const uint8_t * buf, int t, int s, int hl, 
 // One workgroup per (expert, four consecutive tiles of 16 output features), one wave per tile: gate and up
 // tiles together, SwiGLU in the epilogue. The weights of the next super-block and the activations of the next
 // super-block are requested before the current one is multiplied.
-template <int TYPE>
+template <int TYPE, int NTMAX>
 __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t stage[2][2 * kStageTile];
+    __shared__ __attribute__((aligned(16))) uint8_t stage[2][NTMAX * kStageTile];
     __shared__ int rows[32];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, g = lane >> 4;
@@ -208,8 +212,8 @@ __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
     const int nsb = a.K >> 8;
     const uint8_t * wg = a.w0 + ((size_t)e * n_tiles + ft) * nsb * Tile<TYPE>::BYTES;
     const uint8_t * wu = a.w1 + ((size_t)e * n_tiles + ft) * nsb * Tile<TYPE>::BYTES;
-    for (int t0 = 0; t0 < n_e; t0 += 32) {
-        const int nt = n_e - t0 > 16 ? 2 : 1;
+    for (int t0 = 0; t0 < n_e; t0 += 16 * NTMAX) {
+        const int nt = (NTMAX == 2 && n_e - t0 > 16) ? 2 : 1;
         __syncthreads();                       // the last pass is done with rows and the staging buffers
         if (threadIdx.x < 32) {
             const int at = t0 + threadIdx.x;
@@ -217,7 +221,7 @@ __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
             rows[threadIdx.x] = tk < 0 ? 0 : tk;        // padding rows read token 0 and are never stored
         }
         __syncthreads();
-        StageRegs regs;
+        StageRegs<NTMAX> regs;
         stage_load(a.x.x, a.K, rows, 0, nt, regs);
         Tile<TYPE> tg, tu;
         tg.load(wg, lane);
@@ -241,7 +245,7 @@ __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
                 const h8 bg = tg.frag(s), bu = tu.frag(s);
                 const float dg = tg.scale(s), du = tu.scale(s);
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
+                for (int t = 0; t < NTMAX; ++t) {
                     if (t >= nt) break;
                     const h8 hi = staged(cur, t, s, 0, lane), lo = staged(cur, t, s, 1, lane);
                     const f4 pg = mfma2(hi, lo, bg), pu = mfma2(hi, lo, bu);
@@ -275,9 +279,9 @@ __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
 
 // One workgroup per (expert, four consecutive tiles of 16 output features of the model width), one wave per
 // tile; the hidden rows of the expert's pairs are staged like the activations above.
-template <int TYPE>
+template <int TYPE, int NTMAX>
 __global__ __launch_bounds__(256) void k_moe_down(MoeArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t stage[2][2 * kStageTile];
+    __shared__ __attribute__((aligned(16))) uint8_t stage[2][NTMAX * kStageTile];
     __shared__ int rows[32];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, g = lane >> 4;
@@ -290,13 +294,13 @@ __global__ __launch_bounds__(256) void k_moe_down(MoeArgs a) {
     const int qb = a.off_pad[e];
     const int nsb = a.K >> 8;
     const uint8_t * wd = a.w0 + ((size_t)e * n_tiles + et) * nsb * Tile<TYPE>::BYTES;
-    for (int t0 = 0; t0 < n_e; t0 += 32) {
-        const int nt = n_e - t0 > 16 ? 2 : 1;
+    for (int t0 = 0; t0 < n_e; t0 += 16 * NTMAX) {
+        const int nt = (NTMAX == 2 && n_e - t0 > 16) ? 2 : 1;
         __syncthreads();
         // every row of a tile lies in the expert's padded slot range
         if (threadIdx.x < 32) rows[threadIdx.x] = qb + t0 + (threadIdx.x < 16 * nt ? threadIdx.x : 0);
         __syncthreads();
-        StageRegs regs;
+        StageRegs<NTMAX> regs;
         stage_load(a.x.x, a.K, rows, 0, nt, regs);
         Tile<TYPE> tw;
         tw.load(wd, lane);
@@ -316,7 +320,7 @@ __global__ __launch_bounds__(256) void k_moe_down(MoeArgs a) {
                 const h8 b = tw.frag(s);
                 const float d = tw.scale(s);
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
+                for (int t = 0; t < NTMAX; ++t) {
                     if (t >= nt) break;
                     const f4 p = mfma2(staged(cur, t, s, 0, lane), staged(cur, t, s, 1, lane), b);
 #pragma unroll
@@ -473,8 +477,12 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     a.w0 = L.gate.packed; a.w1 = L.up.packed; a.x = xn.operand(L.gate.type); a.h = b.h; a.K = sh.E; a.N = sh.F;
     if (!a.x.x || !b.h.x) throw std::runtime_error("moe: the activations were not prepared for the expert weights");
     const unsigned gu_blocks = (unsigned)(((size_t)sh.n_expert * (sh.F / 16) + 3) / 4);
-    if (L.gate.type == WT_MXFP4) hipLaunchKernelGGL(k_moe_gate_up<WT_MXFP4>, dim3(gu_blocks), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(k_moe_gate_up<WT_Q8_0>, dim3(gu_blocks), dim3(256), 0, s, a);
+    // few pairs per expert (a decode step): one token tile per pass
+    const bool one_tile = (size_t)T * sh.k_used <= (size_t)12 * sh.n_expert;
+    // (measured on the 128-expert shape at 128 rows: the down projection gains a fifth from the smaller
+    // workgroups, gate/up - two weight tiles per wave - loses a tenth, so it keeps two tiles)
+    if (L.gate.type == WT_MXFP4) hipLaunchKernelGGL((k_moe_gate_up<WT_MXFP4, 2>), dim3(gu_blocks), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((k_moe_gate_up<WT_Q8_0, 2>), dim3(gu_blocks), dim3(256), 0, s, a);
     check_launch("moe_gate_up");
     if (xn.faithful) {
         // ggml's arithmetic: the hidden rows are converted, in place, for the down projection
@@ -484,8 +492,13 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     }
     a.w0 = L.down.packed; a.w1 = nullptr; a.x = b.h; a.out_pair = b.out_pair; a.K = sh.F; a.N = sh.E;
     const unsigned d_blocks = (unsigned)(((size_t)sh.n_expert * (sh.E / 16) + 3) / 4);
-    if (L.down.type == WT_MXFP4) hipLaunchKernelGGL(k_moe_down<WT_MXFP4>, dim3(d_blocks), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(k_moe_down<WT_Q8_0>, dim3(d_blocks), dim3(256), 0, s, a);
+    if (L.down.type == WT_MXFP4) {
+        if (one_tile) hipLaunchKernelGGL((k_moe_down<WT_MXFP4, 1>), dim3(d_blocks), dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((k_moe_down<WT_MXFP4, 2>), dim3(d_blocks), dim3(256), 0, s, a);
+    } else {
+        if (one_tile) hipLaunchKernelGGL((k_moe_down<WT_Q8_0, 1>), dim3(d_blocks), dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((k_moe_down<WT_Q8_0, 2>), dim3(d_blocks), dim3(256), 0, s, a);
+    }
     check_launch("moe_down");
     hipLaunchKernelGGL(k_moe_combine, dim3(T, (sh.E / 4 + 255) / 256), dim3(256), 0, s, b.out_pair, b.q_of_pair, b.wgt,
                        sh.k_used, sh.E, x);

@@ -1224,9 +1224,9 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
                 float * dst = qkv_slices.n > 0 ? const_cast<float *>(qkv_slices.data) : qkv;
                 const rk::RowDesc * rows_d = d_stage_.as<rk::RowDesc>();
                 const int cols[3] = {0, QD, QD + KD}, widths[3] = {QD, KD, KD};
-                for (int tg = 0; tg < 3; ++tg)
-                    rk::lora_apply(stream_, lora_entries(l, tg), rows_d, pk_.row, act_e, T, widths[tg], dst, QD + 2 * KD,
-                                   cols[tg], lora_mid_.as<float>());
+                const rk::LoraEntry * tables[3] = {lora_entries(l, 0), lora_entries(l, 1), lora_entries(l, 2)};
+                rk::lora_apply_targets(stream_, 3, tables, widths, cols, rows_d, pk_.row, act_e, T, dst, QD + 2 * KD,
+                                       lora_mid_.as<float>());
             }
             prof_end(PC_QKV, pt_);
         }
@@ -1597,7 +1597,7 @@ void Engine::rebuild_lora_table() {
     hip_check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
     lora_table_.alloc(table.size() * sizeof(rk::LoraEntry));
     hip_check(hipMemcpy(lora_table_.ptr, table.data(), table.size() * sizeof(rk::LoraEntry), hipMemcpyHostToDevice), "hipMemcpy");
-    if (!lora_mid_.ptr) lora_mid_.alloc((size_t)cfg_.n_batch * rk::LORA_MAX_RANK * 4);
+    if (!lora_mid_.ptr) lora_mid_.alloc((size_t)3 * cfg_.n_batch * rk::LORA_MAX_RANK * 4);
 }
 
 // What the stacks cost as the reference builds them: every adapter padded to

@@ -665,12 +665,20 @@ __device__ __forceinline__ float lora_operand(float hi, float lo, int type) {
 }
 
 // mid[t][r] = sum_k A[r][k] * x[t][k]: one wave per (token, r), lanes own groups of eight k.
-__global__ __launch_bounds__(256) void k_lora_down(const LoraEntry * __restrict__ table, const RowDesc * __restrict__ rows,
-                                                   const int32_t * __restrict__ tok_row, Act x, float * __restrict__ mid) {
+// Up to three targets that read the same activations (q, k, v) share a launch: blockIdx.z picks the target.
+struct LoraTargets {
+    const LoraEntry * table[3];
+    int N[3], col0[3];
+};
+
+__global__ __launch_bounds__(256) void k_lora_down(LoraTargets tg, const RowDesc * __restrict__ rows,
+                                                   const int32_t * __restrict__ tok_row, Act x, float * __restrict__ mid_all,
+                                                   int T) {
     const int t = blockIdx.x;
     const int route = rows[tok_row[t]].route;
     if (route <= 0) return;
-    const LoraEntry e = table[route - 1];
+    const LoraEntry e = tg.table[blockIdx.z][route - 1];
+    float * mid = mid_all + (size_t)blockIdx.z * T * LORA_MAX_RANK;
     const int r = blockIdx.y * 4 + (threadIdx.x >> 6);
     if (!e.A || r >= e.rank) return;
     const int lane = threadIdx.x & 63;
@@ -695,13 +703,15 @@ __global__ __launch_bounds__(256) void k_lora_down(const LoraEntry * __restrict_
 }
 
 // y[t][col0 + n] += scale * sum_r B[n][r] * mid[t][r]
-__global__ __launch_bounds__(256) void k_lora_up(const LoraEntry * __restrict__ table, const RowDesc * __restrict__ rows,
-                                                 const int32_t * __restrict__ tok_row, const float * __restrict__ mid,
-                                                 int N, float * __restrict__ y, int ldy, int col0) {
+__global__ __launch_bounds__(256) void k_lora_up(LoraTargets tg, const RowDesc * __restrict__ rows,
+                                                 const int32_t * __restrict__ tok_row, const float * __restrict__ mid_all,
+                                                 float * __restrict__ y, int ldy, int T) {
     const int t = blockIdx.x;
     const int route = rows[tok_row[t]].route;
     if (route <= 0) return;
-    const LoraEntry e = table[route - 1];
+    const LoraEntry e = tg.table[blockIdx.z][route - 1];
+    const int N = tg.N[blockIdx.z], col0 = tg.col0[blockIdx.z];
+    const float * mid = mid_all + (size_t)blockIdx.z * T * LORA_MAX_RANK;
     const int n = blockIdx.y * 256 + threadIdx.x;
     if (!e.A || n >= N) return;
     const float * b = e.B + (size_t)n * e.rank;
@@ -714,14 +724,27 @@ __global__ __launch_bounds__(256) void k_lora_up(const LoraEntry * __restrict__ 
     y[(size_t)t * ldy + col0 + n] += e.scale * acc;
 }
 
+void lora_apply_targets(hipStream_t s, int n_targets, const LoraEntry * const * tables, const int * widths, const int * cols,
+                        const RowDesc * rows, const int32_t * tok_row, const Act & x, int T, float * y, int ldy, float * mid) {
+    if (T <= 0 || n_targets <= 0) return;
+    if (n_targets > 3) throw std::runtime_error("lora: at most three targets share a launch");
+    if (!x.x) throw std::runtime_error("lora: the unconverted activations are missing");
+    LoraTargets tg {};
+    int max_n = 0;
+    for (int i = 0; i < n_targets; ++i) {
+        tg.table[i] = tables[i]; tg.N[i] = widths[i]; tg.col0[i] = cols[i];
+        max_n = std::max(max_n, widths[i]);
+    }
+    if (max_n <= 0) return;
+    hipLaunchKernelGGL(k_lora_down, dim3(T, LORA_MAX_RANK / 4, n_targets), dim3(256), 0, s, tg, rows, tok_row, x, mid, T);
+    check_launch("lora_down");
+    hipLaunchKernelGGL(k_lora_up, dim3(T, (max_n + 255) / 256, n_targets), dim3(256), 0, s, tg, rows, tok_row, mid, y, ldy, T);
+    check_launch("lora_up");
+}
+
 void lora_apply(hipStream_t s, const LoraEntry * table, const RowDesc * rows, const int32_t * tok_row,
                 const Act & x, int T, int N, float * y, int ldy, int col0, float * mid) {
-    if (T <= 0 || N <= 0) return;
-    if (!x.x) throw std::runtime_error("lora: the unconverted activations are missing");
-    hipLaunchKernelGGL(k_lora_down, dim3(T, LORA_MAX_RANK / 4), dim3(256), 0, s, table, rows, tok_row, x, mid);
-    check_launch("lora_down");
-    hipLaunchKernelGGL(k_lora_up, dim3(T, (N + 255) / 256), dim3(256), 0, s, table, rows, tok_row, mid, N, y, ldy, col0);
-    check_launch("lora_up");
+    lora_apply_targets(s, 1, &table, &N, &col0, rows, tok_row, x, T, y, ldy, mid);
 }
 
 __global__ __launch_bounds__(256) void k_rmsnorm_act(float * x, const float * __restrict__ w,

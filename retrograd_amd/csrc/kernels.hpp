@@ -156,6 +156,10 @@ constexpr int LORA_MAX_RANK = 64;
 // entry table[route - 1], skipped when the entry has no pair for this target):
 //   y[t][col0 + n] += scale * sum_r B[n][r] * (sum_k A[r][k] * x[t][k]).
 // mid is scratch of T * LORA_MAX_RANK floats.
+// The same for up to three targets that read the same activations (tables[i], widths[i], cols[i]), in one
+// pair of launches; mid is scratch of n_targets * T * LORA_MAX_RANK floats.
+void lora_apply_targets(hipStream_t s, int n_targets, const LoraEntry * const * tables, const int * widths, const int * cols,
+                        const RowDesc * rows, const int32_t * tok_row, const Act & x, int T, float * y, int ldy, float * mid);
 void lora_apply(hipStream_t s, const LoraEntry * table, const RowDesc * rows, const int32_t * tok_row,
                 const Act & x, int T, int N, float * y, int ldy, int col0, float * mid);
 // out[r][k] = decode(raw row r)[k] as f32: any tensor to f32, row by row.

@@ -175,7 +175,7 @@ struct MMArgs {
     // v2 only
     int n_row_groups;
     float * partial;          // [ksplit][64][N] K-slices of a split matmul
-    int debug;                // timing experiments only: bit 0 stage activations once, bit 1 skip the multiplies
+    int debug;                // timing experiments only: bit 5 sends a full 64-token chunk of Q4_K through the general kernel
     // mode MM_SWIGLU: rows come in groups of 128, 64 gate rows then the 64 up rows of the same
     // columns; the epilogue writes silu(gate) * up as the activations of the next matmul
     Act act_out;

@@ -56,6 +56,15 @@ __device__ __forceinline__ void lds_dma16(const void * base, uint32_t lane_off, 
 __device__ __forceinline__ u4 load16(const void * base, uint32_t lane_off) {
     return *(const u4 *)((const uint8_t *)base + lane_off);
 }
+// The same through a buffer descriptor: `n_bytes` from `base` on (under 4 GiB), wave-uniform; a lane reads 16
+// bytes at lane_off + uniform_off.
+typedef __amdgpu_buffer_rsrc_t WeightRows;
+__device__ __forceinline__ WeightRows weight_rows(const void * base, uint32_t n_bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n_bytes, 0x00020000);
+}
+__device__ __forceinline__ u4 load16(WeightRows rows, uint32_t lane_off, uint32_t uniform_off) {
+    return __builtin_bit_cast(u4, __builtin_amdgcn_raw_buffer_load_b128(rows, (int)lane_off, (int)uniform_off, 0));
+}
 __device__ __forceinline__ uint32_t lds_offset(const void * p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p;
 }
@@ -119,7 +128,6 @@ __device__ __forceinline__ void store_token_rows(const MMArgs & a, uint8_t * sme
     constexpr int TPI = 64 / LPR;          // token rows per store instruction
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     __syncthreads();
-    if (a.debug & 8) return;
     const float * h0 = (const float *)smem, * h1 = h0 + NT * 16 * S;
     if (a.mode == MM_SWIGLU) {
         // eight lanes per token, eight hidden columns each: gate in columns c, up in columns 64 + c of the group
@@ -197,6 +205,22 @@ __device__ __forceinline__ void join_and_store(const MMArgs & a, f4 (&acc)[R][NT
     store_token_rows<NT, R>(a, smem, rg, tbase, ks);
 }
 
+// The super-blocks sb0 .. sb1-1 of a K-slice through `body(sb, current set, set to request into)` with three
+// weight sets in rotation: w0 and w1 hold (or are loading) sb0 and sb0 + 1 on entry. Always whole rounds of
+// three: a body past the end of the slice still waits, synchronises and repeats the request for the last
+// super-block, and only skips its arithmetic. The loop therefore has no exit in the middle of a round; with
+// one, the compiled loop has an edge from mid-round back to its head on which the set about to be read looks
+// as if it were still loading, and the compiler then waits at the head of every round until the requests
+// just issued (the staging requests among them) have landed.
+template <class WSet, class Body>
+__device__ __forceinline__ void rotate_sets(int sb0, int sb1, WSet & w0, WSet & w1, WSet & w2, Body body) {
+    for (int sb = sb0; sb < sb1; sb += 3) {
+        body(sb, w0, w2);
+        body(sb + 1, w1, w0);
+        body(sb + 2, w2, w1);
+    }
+}
+
 // (x & mask) | bits in one instruction
 __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) {
     uint32_t d;
@@ -213,7 +237,7 @@ __device__ __forceinline__ h2 magic_pair(uint32_t word, uint32_t sel) {
 }  // namespace
 
 template <int NT, int R>
-__global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
+__global__ __launch_bounds__(kThreads, NT <= 2 ? 4 : 1) void k_mm2_q4k(MMArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -237,18 +261,22 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
         for (int t = 0; t < NT; ++t) acc[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
 
     // rows past the matrix read the last tile; their results are never stored
-    const uint8_t * wbase[R];
+    // A row tile's super-blocks are one buffer: the loads take the lane's offset and the super-block's as
+    // they are, so no load needs an address computed into a vector register first. (With plain pointers the
+    // compiler built each 64-bit address in the register the load was about to fill, and waited there for
+    // loads it believed were still writing it: the staging requests it had just issued, every third super-block.)
+    WeightRows wbase[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) wbase[r] = a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 2304;
+    for (int r = 0; r < R; ++r)
+        wbase[r] = weight_rows(a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 2304, (uint32_t)nsb * 2304u);
     // this wave's weights of one super-block: the row headers and its half of the payload
     struct WSet { u4 hdr[R]; u4 q[R]; };
     const uint32_t off_hdr = r16 * 16, off_q = 256 + kh * 1024 + lane * 16;
     auto load_w = [&](int sb, WSet & w) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const uint8_t * tile = wbase[r] + (size_t)sb * 2304;
-            w.hdr[r] = load16(tile, off_hdr);
-            w.q[r] = load16(tile, off_q);
+            w.hdr[r] = load16(wbase[r], off_hdr, (uint32_t)sb * 2304u);
+            w.q[r] = load16(wbase[r], off_q, (uint32_t)sb * 2304u);
         }
     };
     const h2 m1024 = {(_Float16)(-1024.0f), (_Float16)(-1024.0f)};
@@ -261,10 +289,15 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
         // All but the newest 2R loads (the weights one super-block ahead) have
         // landed: this super-block's activations and weights are in.
         __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R));
+        // the set is usable from here on and not before (nothing of it is to be touched, and so waited
+        // for, inside the super-block before)
+#pragma unroll
+        for (int r = 0; r < R; ++r) asm volatile("" : "+v"(w.hdr[r]), "+v"(w.q[r]));
         __syncthreads();   // ... for every wave, and nobody still reads the other buffer
-        if (sb + 1 < sb1 && !(a.debug & 1)) stage_x<NT>(stage, sb + 1, (sb - sb0 + 1) & 1, true);
+        if (sb + 1 < sb1) stage_x<NT>(stage, sb + 1, (sb - sb0 + 1) & 1, true);
         load_w(min(sb + 2, sb1 - 1), fut);
-        if (a.debug & 1) cur = smem;
+        __builtin_amdgcn_sched_barrier(0);   // requested now, not wherever the scheduler finds room among the arithmetic
+        if (sb >= sb1) return;       // past the slice: the round is only kept whole
 
         Q4KScales s4[R];
 #pragma unroll
@@ -302,7 +335,6 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
 #pragma unroll
             for (int t = 0; t < NT; ++t) accq[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
         const uint8_t * xk = cur + kh * (8 * NT * 1024);      // this half's four k-steps
-        if (!(a.debug & 2))
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             h8 A[NT], Al[NT];
@@ -350,14 +382,13 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q4k(MMArgs a) {
         WSet w0, w1, w2;
         stage_x<NT>(stage, sb0, 0, true);
         load_w(sb0, w0);
+        // The waits in `body` count loads in program order. Left free, the scheduler interleaves the loads of
+        // the two sets here, and the compiler then has to wait in the loop for the newest loads as well
+        // (the staging requests just issued among them) before it may touch what it believes is still arriving.
+        __builtin_amdgcn_sched_barrier(0);
         load_w(min(sb0 + 1, sb1 - 1), w1);
-        for (int sb = sb0; sb < sb1; sb += 3) {
-            body(sb, w0, w2);
-            if (sb + 1 >= sb1) break;
-            body(sb + 1, w1, w0);
-            if (sb + 2 >= sb1) break;
-            body(sb + 2, w2, w1);
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        rotate_sets(sb0, sb1, w0, w1, w2, body);
     }
     join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
 }
@@ -633,18 +664,18 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
 
-    const uint8_t * wbase[R];
+    WeightRows wbase[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) wbase[r] = a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 4352;
+    for (int r = 0; r < R; ++r)
+        wbase[r] = weight_rows(a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 4352, (uint32_t)nsb * 4352u);
     struct WSet { u4 hdr[R]; u4 q[R][2]; };
     const uint32_t off_hdr = r16 * 16, off_q = 256 + 2 * kh * 1024 + lane * 16;
     auto load_w = [&](int sb, WSet & w) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            const uint8_t * tile = wbase[r] + (size_t)sb * 4352;
-            w.hdr[r] = load16(tile, off_hdr);
-            w.q[r][0] = load16(tile, off_q);
-            w.q[r][1] = load16(tile, off_q + 1024);
+            w.hdr[r] = load16(wbase[r], off_hdr, (uint32_t)sb * 4352u);
+            w.q[r][0] = load16(wbase[r], off_q, (uint32_t)sb * 4352u);
+            w.q[r][1] = load16(wbase[r], off_q + 1024, (uint32_t)sb * 4352u);
         }
     };
     const h2 bias1152 = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
@@ -653,9 +684,15 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
         uint8_t * cur = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
         // all but the newest 3R loads (the weights one super-block ahead) have landed
         __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * R));
+        // The set is usable from here on and not before: without this the scheduler starts on the next
+        // super-block's payload inside this one and waits for it there, the staging requests included.
+#pragma unroll
+        for (int r = 0; r < R; ++r) asm volatile("" : "+v"(w.hdr[r]), "+v"(w.q[r][0]), "+v"(w.q[r][1]));
         __syncthreads();
         if (sb + 1 < sb1) stage_x<NT>(stage, sb + 1, (sb - sb0 + 1) & 1, false);
         load_w(min(sb + 2, sb1 - 1), fut);
+        __builtin_amdgcn_sched_barrier(0);   // requested now, not wherever the scheduler finds room among the arithmetic
+        if (sb >= sb1) return;       // past the slice: the round is only kept whole
         const uint8_t * xk = cur + kh * (8 * NT * 1024);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -692,14 +729,10 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
         WSet w0, w1, w2;
         stage_x<NT>(stage, sb0, 0, false);
         load_w(sb0, w0);
+        __builtin_amdgcn_sched_barrier(0);     // the waits in `body` count loads in program order
         load_w(min(sb0 + 1, sb1 - 1), w1);
-        for (int sb = sb0; sb < sb1; sb += 3) {
-            body(sb, w0, w2);
-            if (sb + 1 >= sb1) break;
-            body(sb + 1, w1, w0);
-            if (sb + 2 >= sb1) break;
-            body(sb + 2, w2, w1);
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        rotate_sets(sb0, sb1, w0, w1, w2, body);
     }
     join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
 }

@@ -124,6 +124,9 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
 int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,
                              int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us) {
     return guarded([&]() -> int {
+        if (type != rk::WT_Q4_K && type != rk::WT_Q8_0) throw std::runtime_error("matmul_time: the tile kernels take Q4_K and Q8_0");
+        if (n_rows <= 0 || k <= 0 || n_rows % 16 != 0 || k % 256 != 0 || n_tokens <= 0 || iters <= 0)
+            throw std::runtime_error("matmul_time: whole 16-row tiles and super-blocks of 256, at least one token and one launch");
         const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
         // mode bit 4: every launch reads another copy of the weights, 1 GiB of them in turn,
         // so that they come from HBM as in a decode step and not from the last-level cache

@@ -588,6 +588,9 @@ static Slices matmul_impl(hipStream_t s, const Weight & w, const Act & x, int T,
         return Slices();
     }
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
+    // the tile kernels know two layouts; anything else handed over as tiles would be read as one of them, out of bounds
+    if (w.type != WT_Q4_K && w.type != WT_Q8_0) throw std::runtime_error("matmul: only Q4_K and Q8_0 matrices come as tiles");
+    if (w.K % 256 != 0 || w.N % 16 != 0) throw std::runtime_error("matmul: a tiled matrix has whole super-blocks and whole 16-row tiles");
     if (ws) return matmul_lds(s, w, x, T, y, ldy, col0, mode, bias, ws, may_slice);
     const Act xo = x.operand(w.type);
     if (!xo.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");

@@ -786,6 +786,8 @@ static void dispatch_nt(hipStream_t s, int type, int nt, const MMArgs & a, dim3 
 // act_out: destination of mode MM_SWIGLU, else null
 static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x_all, int T, float * y, int ldy, int col0,
                        int mode, const float * bias, void * ws, bool may_slice, const Act * act_out, float * act_f32) {
+    if (!w.packed || (w.type != WT_Q4_K && w.type != WT_Q8_0) || w.K % 256 != 0 || w.N % 16 != 0)
+        throw std::runtime_error("matmul_lds: needs a tile-packed Q4_K or Q8_0 matrix of whole super-blocks and 16-row tiles");
     const Act x = x_all.operand(w.type);
     if (!x.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
     if (w.type == WT_Q4_K && !x.sums) throw std::runtime_error("matmul: Q4_K needs block sums");

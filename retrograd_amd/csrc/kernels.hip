@@ -53,7 +53,7 @@ size_t row_bytes(int type, int64_t k) {
 }
 
 bool can_pack(int type, int64_t K, int64_t N) {
-    return (type == WT_Q4_K || type == WT_Q8_0) && K % 256 == 0 && N % 16 == 0 && K > 0 && N > 0;
+    return (type == WT_Q4_K || type == WT_Q8_0 || type == WT_Q6_K) && K % 256 == 0 && N % 16 == 0 && K > 0 && N > 0;
 }
 
 // ---------------------------------------------------------------------------
@@ -260,13 +260,71 @@ __global__ void k_repack_q8_0(const uint8_t * __restrict__ raw, uint8_t * __rest
     *(uint32_t *)(dst + ts * 4352 + (size_t)w * 4) = out;
 }
 
+// Q6_K: 16 rows x one super-block = 3360 bytes, the size of the 16 raw blocks:
+//   [0, 256)      the sixteen i8 scales of row r at 16 r
+//   [256, 288)    d (f16) of row r at 256 + 2 r
+//   [288, 2336)   low nibbles: for k-half h, lane = 16 g + r, k-step j one dword at 288 + 1024 h + 16 lane + 4 j with
+//                 the eight codes c0..c7 of elements 128 h + 32 j + 8 g + i: c(2p) in bits 4p.., c(2p+1) in bits 16 + 4p..
+//   [2336, 3360)  top two bits: one dword per two k-steps at 2336 + 512 h + 8 lane + 4 m. K-step 2m: c(2p) in bits
+//                 4 + 2p.., c(2p+1) in bits 20 + 2p..; k-step 2m + 1: the same places rotated left by eight.
+// so that (low >> 4p) & 0x000F000F and (top >> 2p) & 0x00300030 line a pair of codes up in the two halves of a dword.
+__device__ __forceinline__ uint32_t q6k_code(const uint8_t * blk, int e) {
+    const int half = e >> 7, g = (e & 127) >> 5, l = e & 31;
+    const uint8_t lo = blk[64 * half + l + 32 * (g & 1)];
+    const uint32_t nib = g >= 2 ? (lo >> 4) : (lo & 0x0f);
+    const uint32_t top = (blk[128 + 32 * half + l] >> (2 * g)) & 3;
+    return nib | (top << 4);
+}
+
+__global__ void k_repack_q6k(const uint8_t * __restrict__ raw, uint8_t * __restrict__ dst, int nsb, int n_tiles) {
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = (size_t)n_tiles * nsb * 840;
+    if (gid >= total) return;
+    const int w = (int)(gid % 840);
+    const size_t ts = gid / 840;
+    const int sb = (int)(ts % nsb);
+    const size_t rt = ts / nsb;
+    auto block_of = [&](int r) { return raw + ((rt * 16 + r) * nsb + sb) * 210; };
+    uint32_t out = 0;
+    if (w < 64) {
+        const uint8_t * b = block_of(w >> 2) + 192 + 4 * (w & 3);
+        out = (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) | ((uint32_t)b[3] << 24);
+    } else if (w < 72) {
+        const uint8_t * b0 = block_of(2 * (w - 64)) + 208, * b1 = block_of(2 * (w - 64) + 1) + 208;
+        out = (uint32_t)b0[0] | ((uint32_t)b0[1] << 8) | ((uint32_t)b1[0] << 16) | ((uint32_t)b1[1] << 24);
+    } else if (w < 584) {
+        const int v = w - 72;
+        const int h = v >> 8, lane = (v >> 2) & 63, j = v & 3;
+        const uint8_t * b = block_of(lane & 15);
+        const int e0 = 128 * h + 32 * j + 8 * (lane >> 4);
+        for (int p = 0; p < 4; ++p) {
+            out |= (q6k_code(b, e0 + 2 * p) & 15) << (4 * p);
+            out |= (q6k_code(b, e0 + 2 * p + 1) & 15) << (16 + 4 * p);
+        }
+    } else {
+        const int v = w - 584;
+        const int h = v >> 7, lane = (v >> 1) & 63, m = v & 1;
+        const uint8_t * b = block_of(lane & 15);
+        const int e0 = 128 * h + 64 * m + 8 * (lane >> 4);
+        for (int p = 0; p < 4; ++p) {
+            out |= (q6k_code(b, e0 + 2 * p) >> 4) << (4 + 2 * p);
+            out |= (q6k_code(b, e0 + 2 * p + 1) >> 4) << (20 + 2 * p);
+            out |= (q6k_code(b, e0 + 32 + 2 * p) >> 4) << (12 + 2 * p);
+            out |= (q6k_code(b, e0 + 32 + 2 * p + 1) >> 4) << ((28 + 2 * p) & 31);
+        }
+    }
+    *(uint32_t *)(dst + ts * 3360 + (size_t)w * 4) = out;
+}
+
 void repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int K, int N) {
     if (!can_pack(type, K, N)) throw std::runtime_error("repack: shape or type has no tile layout");
     const int nsb = K / 256, n_tiles = N / 16;
-    const size_t per = type == WT_Q4_K ? 576 : 1088;
+    const size_t per = type == WT_Q4_K ? 576 : (type == WT_Q6_K ? 840 : 1088);     // dwords per tile and super-block
     const size_t total = (size_t)n_tiles * nsb * per;
+    if ((total + 255) / 256 > 0x7fffffffu) throw std::runtime_error("repack: the matrix is too large for one launch");
     const unsigned blocks = (unsigned)((total + 255) / 256);
     if (type == WT_Q4_K) hipLaunchKernelGGL(k_repack_q4k, dim3(blocks), dim3(256), 0, s, raw, packed, nsb, n_tiles);
+    else if (type == WT_Q6_K) hipLaunchKernelGGL(k_repack_q6k, dim3(blocks), dim3(256), 0, s, raw, packed, nsb, n_tiles);
     else hipLaunchKernelGGL(k_repack_q8_0, dim3(blocks), dim3(256), 0, s, raw, packed, nsb, n_tiles);
     check_launch("repack");
 }
@@ -589,9 +647,9 @@ static Slices matmul_impl(hipStream_t s, const Weight & w, const Act & x, int T,
     }
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
     // the tile kernels know two layouts; anything else handed over as tiles would be read as one of them, out of bounds
-    if (w.type != WT_Q4_K && w.type != WT_Q8_0) throw std::runtime_error("matmul: only Q4_K and Q8_0 matrices come as tiles");
-    if (w.K % 256 != 0 || w.N % 16 != 0) throw std::runtime_error("matmul: a tiled matrix has whole super-blocks and whole 16-row tiles");
+    if (!can_pack(w.type, w.K, w.N)) throw std::runtime_error("matmul: this matrix type or shape has no tile layout");
     if (ws) return matmul_lds(s, w, x, T, y, ldy, col0, mode, bias, ws, may_slice);
+    if (w.type == WT_Q6_K) throw std::runtime_error("matmul: Q6_K tiles are multiplied by the LDS kernels only (pass the workspace)");
     const Act xo = x.operand(w.type);
     if (!xo.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
     if (w.type == WT_Q4_K && !xo.sums) throw std::runtime_error("matmul: Q4_K needs block sums");

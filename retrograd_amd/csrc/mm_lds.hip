@@ -46,24 +46,28 @@ __device__ __forceinline__ void lds_dma16(const void * base, uint32_t lane_off, 
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :: "v"(lane_off), "s"(base), "s"(lds_addr) : "memory");
 }
-// In the general kernels the weight loads are ordinary loads: a load issued from
+// In the general kernels the weight loads are loads the compiler knows: a load issued from
 // inline assembly hands the compiler a register whose value arrives later, and
 // any copy the register allocator makes of it before the wait (one was seen at
 // a loop latch) reads stale data. The compiler counts only the loads it knows,
 // so its own waits can only be stricter than needed, never too weak. (The
 // decode kernel k_mm5_q4k keeps its prefetch in registers the compiler does not
-// allocate at all.)
-__device__ __forceinline__ u4 load16(const void * base, uint32_t lane_off) {
-    return *(const u4 *)((const uint8_t *)base + lane_off);
-}
-// The same through a buffer descriptor: `n_bytes` from `base` on (under 4 GiB), wave-uniform; a lane reads 16
-// bytes at lane_off + uniform_off.
+// allocate at all.) They go through a buffer descriptor: `n_bytes` from `base` on
+// (under 4 GiB), wave-uniform; a lane reads at lane_off + uniform_off, and a read
+// past n_bytes returns zero instead of touching memory.
 typedef __amdgpu_buffer_rsrc_t WeightRows;
 __device__ __forceinline__ WeightRows weight_rows(const void * base, uint32_t n_bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n_bytes, 0x00020000);
 }
 __device__ __forceinline__ u4 load16(WeightRows rows, uint32_t lane_off, uint32_t uniform_off) {
     return __builtin_bit_cast(u4, __builtin_amdgcn_raw_buffer_load_b128(rows, (int)lane_off, (int)uniform_off, 0));
+}
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u2 load8(WeightRows rows, uint32_t lane_off, uint32_t uniform_off) {
+    return __builtin_bit_cast(u2, __builtin_amdgcn_raw_buffer_load_b64(rows, (int)lane_off, (int)uniform_off, 0));
+}
+__device__ __forceinline__ uint32_t load4(WeightRows rows, uint32_t lane_off, uint32_t uniform_off) {
+    return __builtin_amdgcn_raw_buffer_load_b32(rows, (int)lane_off, (int)uniform_off, 0);
 }
 __device__ __forceinline__ uint32_t lds_offset(const void * p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p;
@@ -737,6 +741,133 @@ __global__ __launch_bounds__(kThreads, 1) void k_mm2_q8_0(MMArgs a) {
     join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
 }
 
+// Q6_K: value = (d * scale of the 16-wide block) * (code - 32), code of six bits, scale an i8. A lane's eight
+// k-slots of a 32-wide step lie in one 16-wide block, so the block scale can be folded into the weight
+// operand; the product scale * code reaches 4096 and is not always an f16, so the scale goes in as two
+// parts whose products are: its low four bits (0..15, products up to 480) and the rest (a multiple of 16,
+// products multiples of 16 up to 4096). Four matrix instructions per step and tile pair (two scale parts x
+// hi/lo activations) accumulate sum(scale * code * x) exactly as far as f32 goes; d is applied per super-block.
+template <int NT, int R>
+__global__ __launch_bounds__(kThreads, 1) void k_mm2_q6k(MMArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int rw = wave & 3, kh = wave >> 2;
+    const int r16 = lane & 15;
+    const int rg = blockIdx.x % a.n_row_groups, ks = blockIdx.x / a.n_row_groups;
+    const int tbase = blockIdx.y * 64;
+    const int nsb = a.K >> 8;
+    const int per = (nsb + a.ksplit - 1) / a.ksplit;
+    const int sb0 = ks * per, sb1 = min(nsb, sb0 + per);
+
+    int rt[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) rt[r] = (rg * 4 + rw) * R + r;
+    const StageSrc<NT> stage = stage_prepare<NT>(a, blockIdx.y, lane, wave, smem);
+    f4 acc[R][NT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
+
+    WeightRows wbase[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        wbase[r] = weight_rows(a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 3360, (uint32_t)nsb * 3360u);
+    // this wave's weights of one super-block: the rows' scales, d (two rows to a dword), its half of the payload
+    struct WSet { u4 sc[R]; uint32_t d[R]; u4 ql[R]; u2 qh[R]; };
+    const uint32_t off_sc = r16 * 16, off_d = 256 + (r16 >> 1) * 4;
+    const uint32_t off_ql = 288 + kh * 1024 + lane * 16, off_qh = 2336 + kh * 512 + lane * 8;
+    auto load_w = [&](int sb, WSet & w) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            w.sc[r] = load16(wbase[r], off_sc, (uint32_t)sb * 3360u);
+            w.d[r] = load4(wbase[r], off_d, (uint32_t)sb * 3360u);
+            w.ql[r] = load16(wbase[r], off_ql, (uint32_t)sb * 3360u);
+            w.qh[r] = load8(wbase[r], off_qh, (uint32_t)sb * 3360u);
+        }
+    };
+    const h2 bias1056 = {(_Float16)(-1056.0f), (_Float16)(-1056.0f)};
+    const uint32_t magic1024 = 0x64006400u;
+    const int sc_shift = (lane >> 5) * 8;          // the lane's 16-wide block within a 32-wide step
+
+    auto body = [&](int sb, WSet & w, WSet & fut) __attribute__((always_inline)) {
+        uint8_t * cur = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
+        // all but the newest 4R loads (the weights one super-block ahead) have landed
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (4 * R));
+        // the set is usable from here on and not before
+#pragma unroll
+        for (int r = 0; r < R; ++r) asm volatile("" : "+v"(w.sc[r]), "+v"(w.d[r]), "+v"(w.ql[r]), "+v"(w.qh[r]));
+        __syncthreads();
+        if (sb + 1 < sb1) stage_x<NT>(stage, sb + 1, (sb - sb0 + 1) & 1, false);
+        load_w(min(sb + 2, sb1 - 1), fut);
+        __builtin_amdgcn_sched_barrier(0);   // requested now, not wherever the scheduler finds room among the arithmetic
+        if (sb >= sb1) return;       // past the slice: the round is only kept whole
+        const uint8_t * xk = cur + kh * (8 * NT * 1024);
+        f4 accq[R][NT];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < NT; ++t) accq[r][t] = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            h8 A[NT], Al[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                A[t] = lds_h8(xk, (j * 2 + 0) * NT + t, lane);
+                Al[t] = lds_h8(xk, (j * 2 + 1) * NT + t, lane);
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                // scale of block 8 kh + 2 j + (lane / 32): byte 2 (j & 1) + lane / 32 of dword 2 kh + j / 2
+                const uint32_t sw = kh ? (j < 2 ? w.sc[r].z : w.sc[r].w) : (j < 2 ? w.sc[r].x : w.sc[r].y);
+                const int sc = __builtin_amdgcn_sbfe((int)sw, 16 * (j & 1) + sc_shift, 8);
+                const _Float16 s_low = (_Float16)(short)(sc & 15), s_rest = (_Float16)(short)(sc & ~15);
+                const h2 k_low = {s_low, s_low}, k_rest = {s_rest, s_rest};
+                const uint32_t lo = w.ql[r][j];
+                const uint32_t top = (j & 1) ? __builtin_amdgcn_alignbit(w.qh[r][j >> 1], w.qh[r][j >> 1], 8) : w.qh[r][j >> 1];
+                h2 q[4];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    // 1024 + code in both halves, then code - 32
+                    const uint32_t u = and_or(top >> (2 * p), 0x00300030u, and_or(lo >> (4 * p), 0x000F000Fu, magic1024));
+                    q[p] = __builtin_bit_cast(h2, u) + bias1056;
+                }
+                const h2 b0 = q[0] * k_rest, b1 = q[1] * k_rest, b2 = q[2] * k_rest, b3 = q[3] * k_rest;
+                const h2 c0 = q[0] * k_low, c1 = q[1] * k_low, c2 = q[2] * k_low, c3 = q[3] * k_low;
+                const h8 B = {b0.x, b0.y, b1.x, b1.y, b2.x, b2.y, b3.x, b3.y};
+                const h8 Bl = {c0.x, c0.y, c1.x, c1.y, c2.x, c2.y, c3.x, c3.y};
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[t], B, accq[r][t], 0, 0, 0);
+                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[t], B, accq[r][t], 0, 0, 0);
+                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[t], Bl, accq[r][t], 0, 0, 0);
+                    accq[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al[t], Bl, accq[r][t], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float d = h2f((uint16_t)((r16 & 1) ? (w.d[r] >> 16) : (w.d[r] & 0xffff)));
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[r][t][i] = fmaf(d, accq[r][t][i], acc[r][t][i]);
+        }
+    };
+
+    if (sb0 < sb1) {
+        WSet w0, w1, w2;
+        stage_x<NT>(stage, sb0, 0, false);
+        load_w(sb0, w0);
+        __builtin_amdgcn_sched_barrier(0);     // the waits in `body` count loads in program order
+        load_w(min(sb0 + 1, sb1 - 1), w1);
+        __builtin_amdgcn_sched_barrier(0);
+        rotate_sets(sb0, sb1, w0, w1, w2, body);
+    }
+    join_and_store<NT, R>(a, acc, smem, rg, rw, kh, tbase, ks);
+}
+
 template <int NT, int R>
 static void launch2(hipStream_t s, int type, const MMArgs & a, dim3 grid) {
     const size_t lds = 2 * (size_t)XStage<NT>::BYTES;
@@ -756,6 +887,13 @@ static void launch2(hipStream_t s, int type, const MMArgs & a, dim3 grid) {
             return;
         }
         hipLaunchKernelGGL((k_mm2_q4k<NT, R>), grid, dim3(kThreads), lds, s, a);
+    } else if (type == WT_Q6_K) {
+        static bool once = false;
+        if (!once) {
+            HIP_OK(hipFuncSetAttribute((const void *)k_mm2_q6k<NT, R>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            once = true;
+        }
+        hipLaunchKernelGGL((k_mm2_q6k<NT, R>), grid, dim3(kThreads), lds, s, a);
     } else {
         static bool once = false;
         if (!once) {
@@ -786,8 +924,8 @@ static void dispatch_nt(hipStream_t s, int type, int nt, const MMArgs & a, dim3 
 // act_out: destination of mode MM_SWIGLU, else null
 static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x_all, int T, float * y, int ldy, int col0,
                        int mode, const float * bias, void * ws, bool may_slice, const Act * act_out, float * act_f32) {
-    if (!w.packed || (w.type != WT_Q4_K && w.type != WT_Q8_0) || w.K % 256 != 0 || w.N % 16 != 0)
-        throw std::runtime_error("matmul_lds: needs a tile-packed Q4_K or Q8_0 matrix of whole super-blocks and 16-row tiles");
+    if (!w.packed || !can_pack(w.type, w.K, w.N))
+        throw std::runtime_error("matmul_lds: needs a tile-packed Q4_K, Q6_K or Q8_0 matrix of whole super-blocks and 16-row tiles");
     const Act x = x_all.operand(w.type);
     if (!x.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
     if (w.type == WT_Q4_K && !x.sums) throw std::runtime_error("matmul: Q4_K needs block sums");

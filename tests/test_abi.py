@@ -138,9 +138,9 @@ def test_error_string_defaults_and_argument_checks_without_a_device():
     assert g and lib.retro_grammar_gbnf(g) == b'root ::= "a"'
     lib.retro_grammar_free(g)
     assert lib.retro_grammar_from_gbnf(b"") is None and E.last_error() == "gbnf is required"
-    # the timing entry point hands its buffer to the tile kernels as Q4_K or Q8_0 tiles: any other type, or a
+    # the timing entry point hands its buffer to the tile kernels as Q4_K, Q6_K or Q8_0 tiles: any other type, or a
     # shape that is not whole tiles, would be read out of bounds and is refused before anything is allocated
-    for args in ((14, 1024, 4096, 1), (12, 1000, 4096, 1), (12, 1024, 4000, 1), (8, 1024, 4096, 0)):
+    for args in ((39, 1024, 4096, 1), (1, 1024, 4096, 1), (12, 1000, 4096, 1), (14, 1024, 4000, 1), (8, 1024, 4096, 0)):
         with pytest.raises(E.EngineError):
             E.kernel_matmul_time(*args)
         assert "matmul_time" in E.last_error()

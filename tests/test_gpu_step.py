@@ -26,6 +26,9 @@ SMALL = {
     # the type mix of a Q4_K_M file: output.weight, ffn_down and attn_v in Q6_K, the rest in Q4_K
     "llama-q4k-m": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
                                 n_ff=1024, n_vocab=1024, output_type=14, down_type=14, v_type=14, name="llama-q4k-m-small"),
+    # every matrix in Q6_K: the fused qkv matrix and the interleaved gate/up matrix with its SwiGLU epilogue on Q6_K tiles
+    "llama-q6k": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
+                              n_ff=1024, n_vocab=1024, matrix_type=14, name="llama-q6k-small"),
 }
 
 

@@ -174,25 +174,27 @@ void Engine::upload_experts(const TensorInfo & t, int64_t K, int64_t N, DevWeigh
 }
 
 // Row-wise concatenation of matrices that share K and storage type: one matmul
-// instead of several. Falls back to separate matrices when they differ.
+// instead of several. Neighbours that differ stay separate matrices (a Q4_K_M
+// file keeps attn_v in Q6_K: q and k are joined, v follows on its own).
 void Engine::upload_fused(const std::vector<const TensorInfo *> & parts, std::vector<DevWeight> & out) {
-    bool same = true;
-    for (const TensorInfo * p : parts) same = same && p->type == parts[0]->type && p->ne[0] == parts[0]->ne[0];
     out.clear();
-    if (same) {
-        std::vector<uint8_t> joined;
-        int64_t N = 0;
-        for (const TensorInfo * p : parts) {
-            joined.insert(joined.end(), p->data, p->data + p->nbytes);
-            N += p->ne[1];
-        }
+    size_t i = 0;
+    while (i < parts.size()) {
+        size_t j = i + 1;
+        while (j < parts.size() && parts[j]->type == parts[i]->type && parts[j]->ne[0] == parts[i]->ne[0]) ++j;
         out.emplace_back();
-        upload_weight(*parts[0], parts[0]->ne[0], N, joined.data(), joined.size(), false, out.back());
-    } else {
-        for (const TensorInfo * p : parts) {
-            out.emplace_back();
-            upload_weight(*p, p->ne[0], p->ne[1], p->data, p->nbytes, false, out.back());
+        if (j == i + 1) {
+            upload_weight(*parts[i], parts[i]->ne[0], parts[i]->ne[1], parts[i]->data, parts[i]->nbytes, false, out.back());
+        } else {
+            std::vector<uint8_t> joined;
+            int64_t N = 0;
+            for (size_t p = i; p < j; ++p) {
+                joined.insert(joined.end(), parts[p]->data, parts[p]->data + parts[p]->nbytes);
+                N += parts[p]->ne[1];
+            }
+            upload_weight(*parts[i], parts[i]->ne[0], N, joined.data(), joined.size(), false, out.back());
         }
+        i = j;
     }
 }
 
@@ -1212,11 +1214,22 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
                 qkv_slices = rk::matmul_deferred(stream_, L.qkv[0].w, act_e, T, qkv, QD + 2 * KD, 0, rk::MM_STORE,
                                                  L.qkv_bias.as<float>(), mm_ws_.ptr);
             } else {
-                int col = 0;
-                for (const DevWeight & w : L.qkv) {
-                    rk::matmul(stream_, w.w, act_e, T, qkv, QD + 2 * KD, col, rk::MM_STORE,
-                               L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr, mm_ws_.ptr);
-                    col += w.w.N;
+                bool tiled = L.qkv.size() <= 3;
+                const rk::Weight * parts[3] = {nullptr, nullptr, nullptr};
+                for (size_t i = 0; i < L.qkv.size() && tiled; ++i) {
+                    parts[i] = &L.qkv[i].w;
+                    tiled = L.qkv[i].w.packed != nullptr && L.qkv[i].w.K == L.qkv[0].w.K && L.qkv[i].w.N % 4 == 0;
+                }
+                if (tiled) {     // tile matrices of different types: their K-slices side by side, added by the rotation kernel
+                    qkv_slices = rk::matmul_deferred_parts(stream_, parts, (int)L.qkv.size(), act_e, T, qkv, QD + 2 * KD,
+                                                           L.qkv_bias.as<float>(), mm_ws_.ptr);
+                } else {
+                    int col = 0;
+                    for (const DevWeight & w : L.qkv) {
+                        rk::matmul(stream_, w.w, act_e, T, qkv, QD + 2 * KD, col, rk::MM_STORE,
+                                   L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr, mm_ws_.ptr);
+                        col += w.w.N;
+                    }
                 }
             }
             if (routed) {

@@ -132,6 +132,10 @@ extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic
 // columns a workgroup holds, the products leave as f32 rows in h_f32 ([T][F])
 // and a second launch converts them.
 void matmul_swiglu(hipStream_t s, const Weight & w, const Act & x, int T, const Act & out, void * ws, float * h_f32);
+// Several tile-packed matrices over the same activations, outputs side by side in y from column 0 (bias likewise):
+// one launch each, all leaving the same number of K-slices in one set of slices of the full row width.
+Slices matmul_deferred_parts(hipStream_t s, const Weight * const * parts, int n_parts, const Act & x, int T, float * y,
+                             int ldy, const float * bias, void * ws);
 Slices matmul_lds(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
                   int mode, const float * bias, void * ws, bool may_slice);
 // Forces the generic (raw layout) kernel; used to cross-check the tile kernels.

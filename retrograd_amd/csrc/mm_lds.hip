@@ -164,7 +164,7 @@ __device__ __forceinline__ void store_token_rows(const MMArgs & a, uint8_t * sme
     const int n = rg * 64 * R + col;
     if (n >= a.N) return;
     const bool sliced = a.ksplit > 1;
-    float * slice = sliced ? a.partial + (size_t)ks * 64 * a.N : nullptr;
+    float * slice = sliced ? a.partial + (size_t)ks * 64 * a.pld + a.pcol : nullptr;
     const f4 bias = (a.bias && ks == 0) ? *(const f4 *)(a.bias + n) : (f4){0.f, 0.f, 0.f, 0.f};
     const int nrows = min(NT * 16, a.T - tbase);
     for (int tk = wave * TPI + lane / LPR; tk < nrows; tk += kWaves * TPI) {
@@ -173,7 +173,7 @@ __device__ __forceinline__ void store_token_rows(const MMArgs & a, uint8_t * sme
         v += bias;
         const int tok = tbase + tk;
         if (sliced) {
-            *(f4 *)(slice + (size_t)tok * a.N + n) = v;
+            *(f4 *)(slice + (size_t)tok * a.pld + n) = v;
         } else {
             float * p = a.y + (size_t)tok * a.ldy + a.col0 + n;
             if (a.mode == MM_ADD) v = *(const f4 *)p + v;
@@ -922,8 +922,13 @@ static void dispatch_nt(hipStream_t s, int type, int nt, const MMArgs & a, dim3 
 }
 
 // act_out: destination of mode MM_SWIGLU, else null
+// One matrix of several that leave their K-slices side by side: the common slice count, the row width of the
+// slices and this matrix's first column in them.
+struct SharedSlices { int ksplit = 0, ld = 0, col = 0; };
+
 static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x_all, int T, float * y, int ldy, int col0,
-                       int mode, const float * bias, void * ws, bool may_slice, const Act * act_out, float * act_f32) {
+                       int mode, const float * bias, void * ws, bool may_slice, const Act * act_out, float * act_f32,
+                       const SharedSlices * shared = nullptr) {
     if (!w.packed || !can_pack(w.type, w.K, w.N))
         throw std::runtime_error("matmul_lds: needs a tile-packed Q4_K, Q6_K or Q8_0 matrix of whole super-blocks and 16-row tiles");
     const Act x = x_all.operand(w.type);
@@ -961,12 +966,64 @@ static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x_all, int T
             ksplit = 1;
         }
     }
+    a.pld = w.N; a.pcol = 0;
+    if (shared) {
+        if (chunks != 1 || shared->ksplit < 2 || shared->ksplit > nsb || (shared->col & 3) || (shared->ld & 3) ||
+            shared->col + w.N > shared->ld || (size_t)shared->ksplit * 64 * shared->ld * 4 > matmul_workspace_bytes())
+            throw std::runtime_error("matmul_lds: the shared slices do not fit this matrix");
+        const int per = (nsb + shared->ksplit - 1) / shared->ksplit;
+        if ((nsb + per - 1) / per != shared->ksplit) throw std::runtime_error("matmul_lds: the shared slice count leaves an empty slice");
+        ksplit = shared->ksplit;
+        a.pld = shared->ld; a.pcol = shared->col;
+    }
     a.ksplit = ksplit;
     dim3 grid(a.n_row_groups * ksplit, chunks);
     dispatch_nt<R>(s, w.type, nt, a, grid);
     check_launch("matmul_lds");
     Slices out;
-    if (ksplit > 1) { out.data = a.partial; out.n = ksplit; out.stride = (size_t)64 * w.N; out.N = w.N; }
+    if (ksplit > 1) { out.data = a.partial; out.n = ksplit; out.stride = (size_t)64 * a.pld; out.N = a.pld; }
+    return out;
+}
+
+// Several tiled matrices over the same activations whose outputs sit side by side in y (q, k and v of different
+// storage types): each is launched on its own, all with the same number of K-slices into one set of slices of
+// the full row width, so that the consumer adds them as it would for one fused matrix. Returns no slices (and
+// leaves the results in y) when the step is not a single chunk or K too short to split.
+Slices matmul_deferred_parts(hipStream_t s, const Weight * const * parts, int n_parts, const Act & x, int T, float * y,
+                             int ldy, const float * bias, void * ws) {
+    if (T <= 0 || n_parts <= 0) return Slices();
+    int total = 0, K = parts[0]->K;
+    for (int i = 0; i < n_parts; ++i) {
+        if (!parts[i]->packed || parts[i]->K != K || !can_pack(parts[i]->type, K, parts[i]->N) || (parts[i]->N & 3))
+            throw std::runtime_error("matmul_deferred_parts: needs tile-packed matrices of one width");
+        total += parts[i]->N;
+    }
+    if (!ws || total > ldy) throw std::runtime_error("matmul_deferred_parts: needs the workspace and room for every part in y");
+    const int nsb = K / 256, chunks = (T + 63) / 64;
+    int ksplit = 1;
+    if (chunks == 1) {
+        const int groups = (total / 16 + 7) / 8;
+        int want = std::min(std::min(16, 256 / std::max(groups, 1)), nsb / 2);
+        if (want > 1) {
+            const int per = (nsb + want - 1) / want;
+            ksplit = (nsb + per - 1) / per;
+        }
+        if ((size_t)ksplit * 64 * total * 4 > matmul_workspace_bytes()) ksplit = 1;
+    }
+    Slices out;
+    int col = 0;
+    for (int i = 0; i < n_parts; ++i) {
+        const float * b = bias ? bias + col : nullptr;
+        if (ksplit > 1) {
+            SharedSlices sh;
+            sh.ksplit = ksplit; sh.ld = total; sh.col = col;
+            out = lds_impl(s, *parts[i], x, T, y, ldy, col, MM_STORE, b, ws, true, nullptr, nullptr, &sh);
+        } else {
+            lds_impl(s, *parts[i], x, T, y, ldy, col, MM_STORE, b, ws, false, nullptr, nullptr);
+        }
+        col += parts[i]->N;
+    }
+    if (ksplit > 1) { out.data = (const float *)ws; out.n = ksplit; out.stride = (size_t)64 * total; out.N = total; }
     return out;
 }
 

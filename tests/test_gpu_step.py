@@ -29,6 +29,9 @@ SMALL = {
     # every matrix in Q6_K: the fused qkv matrix and the interleaved gate/up matrix with its SwiGLU epilogue on Q6_K tiles
     "llama-q6k": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
                               n_ff=1024, n_vocab=1024, matrix_type=14, name="llama-q6k-small"),
+    # q and k joined in Q4_K, v on its own in Q6_K, with biases: two launches that leave their K-slices side by side
+    "qwen2-q4k-m": synth.scaled(synth.QWEN25_7B_Q8, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
+                                n_ff=1024, n_vocab=1024, matrix_type=12, v_type=14, down_type=14, name="qwen2-q4k-m-small"),
 }
 
 

@@ -42,7 +42,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--shape", default="c2", choices=["c2", "small"], help="small = a reduced shape for a quick functional run")
+    ap.add_argument("--shape", default="c2", choices=["c2", "c2-q4km", "small"],
+                    help="c2-q4km = the same workload on the type mix of a Q4_K_M file (a secondary figure); "
+                         "small = a reduced shape for a quick functional run")
     ap.add_argument("--model-dir", default=os.environ.get("RETRO_BENCH_MODEL_DIR", "/dev/shm"))
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -180,8 +182,8 @@ def main() -> int:
         print("bench.py needs an MI355X: no HIP device is visible", file=sys.stderr)
         return 2
 
-    if args.shape == "c2":
-        shape = synth.LLAMA3_8B_Q4K
+    if args.shape in ("c2", "c2-q4km"):
+        shape = synth.LLAMA3_8B_Q4K if args.shape == "c2" else synth.LLAMA3_8B_Q4K_M
         n_slots, max_new, len_lo, len_hi, n_batch = 64, 256, 128, 4096, 512
     else:
         shape = synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=4, n_vocab=32000, name="llama3-8b-shape-q4_k-4layers")
@@ -261,15 +263,14 @@ def main() -> int:
     attn_gbs = algo_bytes_per_launch / attn_avg_s / 1e9 if attn_avg_s > 0 else 0.0
 
     # ---- whole-step roofline (north star): weights once + KV of every attended cell
-    geom = synth.gw.BLOCK_GEOMETRY[hp.matrix_type]
-    bpe = geom[1] / geom[0]
-    per_layer = hp.n_embd * (hp.n_head * hp.head_dim) * 2 + hp.n_embd * (hp.n_head_kv * hp.head_dim) * 2 + 3 * hp.n_embd * hp.n_ff
-    w_bytes = hp.n_layer * per_layer * bpe + hp.n_vocab * hp.n_embd * bpe
+    w_bytes = synth.streamed_weight_bytes(hp)       # every dense matrix once, at its stored type
     step_bytes = w_bytes + hp.n_layer * kv_bytes_per_cell_layer * (cells / args.steps)
     step_roof_tok_s = (sampled / args.steps) / (step_bytes / (HBM_PEAK_GBS * 1e9))
 
     result = {
-        "metric": "decode tok/s, 8B-shape Q4_K ragged batch 64; % of HBM roofline",
+        "metric": ("decode tok/s, 8B-shape Q4_K ragged batch 64; % of HBM roofline" if args.shape != "c2-q4km" else
+                   "decode tok/s, 8B shape with the Q4_K_M type mix (Q6_K output, ffn_down and attn_v on half the layers), "
+                   "ragged batch 64 (secondary figure)"),
         "value": round(tok_s, 1),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -279,7 +280,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "q4_k weights x f16 hi/lo activations, f32 accumulate, f16 KV",
+        "dtype": ("q4_k" if args.shape != "c2-q4km" else "q4_k / q6_k") + " weights x f16 hi/lo activations, f32 accumulate, f16 KV",
         "data": "synthetic",
         "config": {
             "workload": "configs[1]: %s, %d live sequences, prompts log-uniform [%d,%d], greedy, %d new tokens, continuous batching"

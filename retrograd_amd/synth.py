@@ -44,17 +44,60 @@ class ModelShape:
     output_type: int = -1            # output.weight
     down_type: int = -1              # ffn_down.weight
     v_type: int = -1                 # attn_v.weight
+    finer_layers: str = "all"        # layers whose ffn_down / attn_v take the finer type: "all", or "more_bits" =
+                                     # the first and last eighth and every third layer between (llama.cpp's rule for Q4_K_M)
 
 
 # The five benchmark configurations.
 TINY_LLAMA = ModelShape("llama", 2, 128, 4, 2, 32, 344, 512, 10000.0, gw.GGML_Q8_0, name="tiny-llama-q8_0")
 LLAMA3_8B_Q4K = ModelShape("llama", 32, 4096, 32, 8, 128, 14336, 128256, 500000.0, gw.GGML_Q4_K,
                            name="llama3-8b-shape-q4_k")
+# the same shape with the type mix of a Q4_K_M file: output.weight in Q6_K, ffn_down and attn_v in Q6_K on llama.cpp's layers
+LLAMA3_8B_Q4K_M = ModelShape("llama", 32, 4096, 32, 8, 128, 14336, 128256, 500000.0, gw.GGML_Q4_K,
+                             output_type=gw.GGML_Q6_K, down_type=gw.GGML_Q6_K, v_type=gw.GGML_Q6_K, finer_layers="more_bits",
+                             name="llama3-8b-shape-q4_k_m")
 QWEN25_7B_Q8 = ModelShape("qwen2", 28, 3584, 28, 4, 128, 18944, 152064, 1000000.0, gw.GGML_Q8_0,
                           qkv_bias=True, name="qwen2.5-7b-shape-q8_0")
 QWEN3_30B_A3B = ModelShape("qwen3moe", 48, 2048, 32, 4, 128, 6144, 151936, 1000000.0, gw.GGML_Q8_0,
                            n_expert=128, n_expert_used=8, n_ff_exp=768, eps=1e-6,
                            name="qwen3-30b-a3b-shape-mxfp4")
+
+
+def finer_layer(shape: ModelShape, layer: int) -> bool:
+    """Whether `layer` stores ffn_down and attn_v at the finer type (down_type / v_type)."""
+    if shape.finer_layers == "all":
+        return True
+    n = shape.n_layer
+    return layer < n // 8 or layer >= 7 * n // 8 or (layer - n // 8) % 3 == 2
+
+
+def matrix_types(shape: ModelShape):
+    """(name, n_in, n_out, ggml type) of every dense 2-D matrix of a non-expert model, in file order without the
+    token embedding: what a decode step streams once."""
+    s = shape
+    E, QD, KD = s.n_embd, s.n_head * s.head_dim, s.n_head_kv * s.head_dim
+    out = []
+    for l in range(s.n_layer):
+        fine = finer_layer(s, l)
+        b = "blk.%d." % l
+        out.append((b + "attn_q.weight", E, QD, s.matrix_type))
+        out.append((b + "attn_k.weight", E, KD, s.matrix_type))
+        out.append((b + "attn_v.weight", E, KD, s.v_type if (s.v_type >= 0 and fine) else s.matrix_type))
+        out.append((b + "attn_output.weight", QD, E, s.matrix_type))
+        out.append((b + "ffn_gate.weight", E, s.n_ff, s.matrix_type))
+        out.append((b + "ffn_up.weight", E, s.n_ff, s.matrix_type))
+        out.append((b + "ffn_down.weight", s.n_ff, E, s.down_type if (s.down_type >= 0 and fine) else s.matrix_type))
+    out.append(("output.weight", E, s.n_vocab, s.output_type if s.output_type >= 0 else s.matrix_type))
+    return out
+
+
+def streamed_weight_bytes(shape: ModelShape) -> int:
+    """Bytes of the matrices a decode step of a non-expert model reads once (stored types as written)."""
+    total = 0
+    for _, n_in, n_out, t in matrix_types(shape):
+        el, by = gw.BLOCK_GEOMETRY[storage_type(t, n_in)]
+        total += n_in // el * by * n_out
+    return total
 
 
 def scaled(shape: ModelShape, **kw) -> ModelShape:
@@ -248,7 +291,8 @@ def write_model(path, shape: ModelShape, seed: int = 0, device: str | None = Non
         vector(b + "attn_norm.weight", E, 1.0)
         matrix(b + "attn_q.weight", E, QD)
         matrix(b + "attn_k.weight", E, KD)
-        matrix(b + "attn_v.weight", E, KD, None if s.v_type < 0 else s.v_type)
+        fine = finer_layer(s, l)
+        matrix(b + "attn_v.weight", E, KD, None if (s.v_type < 0 or not fine) else s.v_type)
         if s.qkv_bias:
             vector(b + "attn_q.bias", QD)
             vector(b + "attn_k.bias", KD)
@@ -267,7 +311,7 @@ def write_model(path, shape: ModelShape, seed: int = 0, device: str | None = Non
         else:
             matrix(b + "ffn_gate.weight", E, s.n_ff)
             matrix(b + "ffn_up.weight", E, s.n_ff)
-            matrix(b + "ffn_down.weight", s.n_ff, E, None if s.down_type < 0 else s.down_type)
+            matrix(b + "ffn_down.weight", s.n_ff, E, None if (s.down_type < 0 or not fine) else s.down_type)
     vector("output_norm.weight", E, 1.0)
     matrix("output.weight", E, s.n_vocab, None if s.output_type < 0 else s.output_type)
     return w.write(Path(path))

@@ -32,6 +32,10 @@ SMALL = {
     # q and k joined in Q4_K, v on its own in Q6_K, with biases: two launches that leave their K-slices side by side
     "qwen2-q4k-m": synth.scaled(synth.QWEN25_7B_Q8, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
                                 n_ff=1024, n_vocab=1024, matrix_type=12, v_type=14, down_type=14, name="qwen2-q4k-m-small"),
+    # wide enough (four super-blocks per row) for decode steps to split K: the q+k and v launches share their K-slices
+    "llama-q4k-m-1024": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=1024, n_head=8, n_head_kv=2, head_dim=128,
+                                     n_ff=2048, n_vocab=2048, output_type=14, down_type=14, v_type=14,
+                                     name="llama-q4k-m-1024"),
 }
 
 

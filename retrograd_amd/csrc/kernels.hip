@@ -866,7 +866,17 @@ __global__ __launch_bounds__(NW * 64) void k_rmsnorm_act8(float * x, const float
         if (add.n > 0) {
             const float * sl = add.data + (size_t)row * E + k;
             int j = 0;
-            for (; j + 4 <= add.n; j += 4) {          // four slices' loads in flight together
+            for (; j + 8 <= add.n; j += 8) {          // eight slices' loads in flight together, added in slice order
+                f4 sa[8], sb[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    sa[u] = *(const f4 *)(sl + (size_t)(j + u) * add.stride);
+                    sb[u] = *(const f4 *)(sl + (size_t)(j + u) * add.stride + 4);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { a += sa[u]; b += sb[u]; }
+            }
+            for (; j + 4 <= add.n; j += 4) {          // four
                 f4 sa[4], sb[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {

@@ -28,7 +28,7 @@
 namespace rk {
 
 bool moe_can_pack(int type, int64_t K, int64_t N) {
-    return (type == WT_MXFP4 || type == WT_Q8_0) && K % 256 == 0 && N % 16 == 0 && K > 0 && N > 0;
+    return (type == WT_MXFP4 || type == WT_Q8_0 || type == WT_Q4_K || type == WT_Q6_K) && K % 256 == 0 && N % 16 == 0 && K > 0 && N > 0;
 }
 
 __global__ void k_repack_mxfp4(const uint8_t * __restrict__ raw, uint8_t * __restrict__ dst, int nsb, size_t n_tiles) {
@@ -62,8 +62,8 @@ __global__ void k_repack_mxfp4(const uint8_t * __restrict__ raw, uint8_t * __res
 
 void moe_repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int K, int64_t n_rows) {
     if (!moe_can_pack(type, K, n_rows)) throw std::runtime_error("moe_repack: shape or type has no tile layout");
-    if (type == WT_Q8_0) {
-        // the dense Q8_0 tile layout, in slabs the dense repack's 32-bit sizes can hold
+    if (type != WT_MXFP4) {
+        // the dense tile layouts (Q8_0, Q4_K, Q6_K), in slabs the dense repack's 32-bit sizes can hold
         const int64_t slab = 1 << 20;
         for (int64_t r0 = 0; r0 < n_rows; r0 += slab) {
             const int64_t n = std::min(slab, n_rows - r0);
@@ -82,6 +82,18 @@ void moe_repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, 
 namespace {
 
 template <int TYPE> struct Tile;
+
+// What a tile contributes per 32-wide step: the weight operand(s) and the factors applied after the products.
+// prep(s) decodes once per step, mac() multiplies one token tile (hi and lo halves) and adds into acc.
+struct ScaledOperand { h8 b; float d; };
+
+__device__ __forceinline__ f4 mfma2(const h8 & a_hi, const h8 & a_lo, const h8 & b);
+
+__device__ __forceinline__ void mac(const ScaledOperand & o, const h8 & hi, const h8 & lo, f4 & acc) {
+    const f4 p = mfma2(hi, lo, o.b);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = fmaf(o.d, p[i], acc[i]);
+}
 
 template <> struct Tile<WT_MXFP4> {
     static constexpr int BYTES = 2176;
@@ -109,6 +121,7 @@ template <> struct Tile<WT_MXFP4> {
         const h2 p3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0u, hi, 0x030C020Cu));
         return (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
     }
+    __device__ __forceinline__ ScaledOperand prep(int s) const { return {frag(s), scale(s)}; }
 };
 
 template <> struct Tile<WT_Q8_0> {
@@ -135,12 +148,109 @@ template <> struct Tile<WT_Q8_0> {
         const h2 a3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)) + bias;
         return (h8){a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
     }
+    __device__ __forceinline__ ScaledOperand prep(int s) const { return {frag(s), scale(s)}; }
 };
 
 __device__ __forceinline__ f4 mfma2(const h8 & a_hi, const h8 & a_lo, const h8 & b) {
     f4 p = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_hi, b, (f4){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a_lo, b, p, 0, 0, 0);
 }
+
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t bits) { return (x & mask) | bits; }
+
+// Q4_K, the dense tile (2304 bytes): value = d * sc * e - dmin * m per 32-wide sub-block. sc * e goes into the
+// operand as an exact f16 (at most 945); the min term needs the sum of the activations of the sub-block, which a
+// product with an operand of ones supplies for every token of the tile.
+struct Q4KOperand { h8 b; float d, dm; };
+__device__ __forceinline__ void mac(const Q4KOperand & o, const h8 & hi, const h8 & lo, f4 & acc) {
+    const _Float16 one = (_Float16)1.0f;
+    const h8 ones = {one, one, one, one, one, one, one, one};
+    const f4 p = mfma2(hi, lo, o.b), sum = mfma2(hi, lo, ones);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = fmaf(-o.dm, sum[i], fmaf(o.d, p[i], acc[i]));
+}
+template <> struct Tile<WT_Q4_K> {
+    static constexpr int BYTES = 2304;
+    u4 hdr;
+    u4 q0, q1;
+    __device__ __forceinline__ void load(const uint8_t * tile, int lane) {
+        hdr = *(const u4 *)(tile + (lane & 15) * 16);
+        q0 = *(const u4 *)(tile + 256 + lane * 16);
+        q1 = *(const u4 *)(tile + 256 + 1024 + lane * 16);
+    }
+    __device__ __forceinline__ Q4KOperand prep(int s) const {
+        const Q4KScales s4 = q4k_scales(hdr);
+        const int j = s & 3;
+        const uint32_t scw = s < 4 ? s4.sc[0] : s4.sc[1], mnw = s < 4 ? s4.mn[0] : s4.mn[1];
+        const h2 m1024 = {(_Float16)(-1024.0f), (_Float16)(-1024.0f)};
+        // (1024 + sc, 1024 + sc) from byte j, then (sc, sc)
+        const h2 k1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, scw, 0x04000400u + 0x00010001u * j)) + m1024;
+        const h2 c1 = k1 * (_Float16)(-1024.0f), c2 = k1 * (_Float16)(-64.0f);
+        const uint32_t wq = s < 4 ? q0[j] : q1[j];
+        const uint32_t w8 = wq >> 8;
+        const h2 u0 = __builtin_bit_cast(h2, and_or(wq, 0x000F000Fu, 0x64006400u));     // 1024 + e
+        const h2 u1 = __builtin_bit_cast(h2, and_or(wq, 0x00F000F0u, 0x54005400u));     // 64 + e (nibble one place up)
+        const h2 u2 = __builtin_bit_cast(h2, and_or(w8, 0x000F000Fu, 0x64006400u));
+        const h2 u3 = __builtin_bit_cast(h2, and_or(w8, 0x00F000F0u, 0x54005400u));
+        const h2 a0 = __builtin_elementwise_fma(u0, k1, c1), a1 = __builtin_elementwise_fma(u1, k1, c2);
+        const h2 a2 = __builtin_elementwise_fma(u2, k1, c1), a3 = __builtin_elementwise_fma(u3, k1, c2);
+        Q4KOperand o;
+        o.b = (h8){a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+        o.d = h2f((uint16_t)(hdr.x & 0xffff));
+        o.dm = h2f((uint16_t)(hdr.x >> 16)) * (float)((mnw >> (8 * j)) & 0xffu);
+        return o;
+    }
+};
+
+// Q6_K, the dense tile (3360 bytes): value = d * scale * (code - 32) per 16-wide block; the i8 scale goes into the
+// operand in two parts whose products with a code are exact f16 numbers (its low four bits, and the rest).
+struct Q6KOperand { h8 b_rest, b_low; float d; };
+__device__ __forceinline__ void mac(const Q6KOperand & o, const h8 & hi, const h8 & lo, f4 & acc) {
+    f4 p = mfma2(hi, lo, o.b_rest);
+    p = __builtin_amdgcn_mfma_f32_16x16x32_f16(hi, o.b_low, p, 0, 0, 0);
+    p = __builtin_amdgcn_mfma_f32_16x16x32_f16(lo, o.b_low, p, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = fmaf(o.d, p[i], acc[i]);
+}
+template <> struct Tile<WT_Q6_K> {
+    static constexpr int BYTES = 3360;
+    u4 sc;
+    uint32_t dpair;
+    u4 ql0, ql1;
+    uint2 qh0, qh1;
+    int lane_;
+    __device__ __forceinline__ void load(const uint8_t * tile, int lane) {
+        lane_ = lane;
+        sc = *(const u4 *)(tile + (lane & 15) * 16);
+        dpair = *(const uint32_t *)(tile + 256 + ((lane & 15) >> 1) * 4);
+        ql0 = *(const u4 *)(tile + 288 + lane * 16);
+        ql1 = *(const u4 *)(tile + 288 + 1024 + lane * 16);
+        qh0 = *(const uint2 *)(tile + 2336 + lane * 8);
+        qh1 = *(const uint2 *)(tile + 2336 + 512 + lane * 8);
+    }
+    __device__ __forceinline__ Q6KOperand prep(int s) const {
+        const int j = s & 3;
+        // scale of block 2 s + lane / 32: byte 2 (j & 1) + lane / 32 of scale dword s / 2
+        const int scale = __builtin_amdgcn_sbfe((int)sc[s >> 1], 16 * (j & 1) + 8 * (lane_ >> 5), 8);
+        const _Float16 s_low = (_Float16)(short)(scale & 15), s_rest = (_Float16)(short)(scale & ~15);
+        const h2 k_low = {s_low, s_low}, k_rest = {s_rest, s_rest};
+        const uint32_t lo = s < 4 ? ql0[j] : ql1[j];
+        const uint32_t pair = s < 4 ? (j < 2 ? qh0.x : qh0.y) : (j < 2 ? qh1.x : qh1.y);
+        const uint32_t top = (j & 1) ? __builtin_amdgcn_alignbit(pair, pair, 8) : pair;
+        const h2 bias1056 = {(_Float16)(-1056.0f), (_Float16)(-1056.0f)};
+        h2 q[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+            q[p] = __builtin_bit_cast(h2, and_or(top >> (2 * p), 0x00300030u, and_or(lo >> (4 * p), 0x000F000Fu, 0x64006400u))) + bias1056;
+        const h2 b0 = q[0] * k_rest, b1 = q[1] * k_rest, b2 = q[2] * k_rest, b3 = q[3] * k_rest;
+        const h2 c0 = q[0] * k_low, c1 = q[1] * k_low, c2 = q[2] * k_low, c3 = q[3] * k_low;
+        Q6KOperand o;
+        o.b_rest = (h8){b0.x, b0.y, b1.x, b1.y, b2.x, b2.y, b3.x, b3.y};
+        o.b_low = (h8){c0.x, c0.y, c1.x, c1.y, c2.x, c2.y, c3.x, c3.y};
+        o.d = h2f((uint16_t)((lane_ & 1) ? (dpair >> 16) : (dpair & 0xffff)));
+        return o;
+    }
+};
 
 }  // namespace
 
@@ -242,18 +352,13 @@ __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
             const uint8_t * cur = stage[sb & 1];
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
-                const h8 bg = tg.frag(s), bu = tu.frag(s);
-                const float dg = tg.scale(s), du = tu.scale(s);
+                const auto og = tg.prep(s), ou = tu.prep(s);
 #pragma unroll
                 for (int t = 0; t < NTMAX; ++t) {
                     if (t >= nt) break;
                     const h8 hi = staged(cur, t, s, 0, lane), lo = staged(cur, t, s, 1, lane);
-                    const f4 pg = mfma2(hi, lo, bg), pu = mfma2(hi, lo, bu);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        ag[t][i] = fmaf(dg, pg[i], ag[t][i]);
-                        au[t][i] = fmaf(du, pu[i], au[t][i]);
-                    }
+                    mac(og, hi, lo, ag[t]);
+                    mac(ou, hi, lo, au[t]);
                 }
             }
             if (more) stage_store(stage[(sb + 1) & 1], nt, regs);
@@ -317,14 +422,11 @@ __global__ __launch_bounds__(256) void k_moe_down(MoeArgs a) {
             const uint8_t * cur = stage[sb & 1];
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
-                const h8 b = tw.frag(s);
-                const float d = tw.scale(s);
+                const auto ow = tw.prep(s);
 #pragma unroll
                 for (int t = 0; t < NTMAX; ++t) {
                     if (t >= nt) break;
-                    const f4 p = mfma2(staged(cur, t, s, 0, lane), staged(cur, t, s, 1, lane), b);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) acc[t][i] = fmaf(d, p[i], acc[t][i]);
+                    mac(ow, staged(cur, t, s, 0, lane), staged(cur, t, s, 1, lane), acc[t]);
                 }
             }
             if (more) stage_store(stage[(sb + 1) & 1], nt, regs);
@@ -462,9 +564,9 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     if (sh.n_expert > 256 || sh.k_used > 16 || sh.k_used > sh.n_expert) throw std::runtime_error("moe: unsupported expert count");
     // multiples of 256: whole super-blocks along K, and the four waves of a workgroup share an expert (N / 16 % 4 == 0)
     if (sh.E % 256 != 0 || sh.F % 256 != 0) throw std::runtime_error("moe: widths must be multiples of 256");
-    if (L.gate.type != L.up.type || (L.gate.type != WT_MXFP4 && L.gate.type != WT_Q8_0) ||
-        (L.down.type != WT_MXFP4 && L.down.type != WT_Q8_0))
-        throw std::runtime_error("moe: expert weights must be MXFP4 or Q8_0");
+    auto tiled = [](int t) { return t == WT_MXFP4 || t == WT_Q8_0 || t == WT_Q4_K || t == WT_Q6_K; };
+    if (L.gate.type != L.up.type || !tiled(L.gate.type) || !tiled(L.down.type))
+        throw std::runtime_error("moe: expert weights must be MXFP4, Q8_0, Q4_K or Q6_K, gate and up of one type");
     matmul_generic(s, L.router, xn, T, b.logits, sh.n_expert, 0, MM_STORE, nullptr);
     hipLaunchKernelGGL(k_moe_route, dim3(T), dim3(64), 0, s, b.logits, sh.n_expert, sh.k_used, b.sel, b.wgt);
     check_launch("moe_route");
@@ -481,8 +583,12 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     const bool one_tile = (size_t)T * sh.k_used <= (size_t)12 * sh.n_expert;
     // (measured on the 128-expert shape at 128 rows: the down projection gains a fifth from the smaller
     // workgroups, gate/up - two weight tiles per wave - loses a tenth, so it keeps two tiles)
-    if (L.gate.type == WT_MXFP4) hipLaunchKernelGGL((k_moe_gate_up<WT_MXFP4, 2>), dim3(gu_blocks), dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((k_moe_gate_up<WT_Q8_0, 2>), dim3(gu_blocks), dim3(256), 0, s, a);
+    switch (L.gate.type) {
+        case WT_MXFP4: hipLaunchKernelGGL((k_moe_gate_up<WT_MXFP4, 2>), dim3(gu_blocks), dim3(256), 0, s, a); break;
+        case WT_Q4_K:  hipLaunchKernelGGL((k_moe_gate_up<WT_Q4_K, 2>), dim3(gu_blocks), dim3(256), 0, s, a); break;
+        case WT_Q6_K:  hipLaunchKernelGGL((k_moe_gate_up<WT_Q6_K, 2>), dim3(gu_blocks), dim3(256), 0, s, a); break;
+        default:       hipLaunchKernelGGL((k_moe_gate_up<WT_Q8_0, 2>), dim3(gu_blocks), dim3(256), 0, s, a); break;
+    }
     check_launch("moe_gate_up");
     if (xn.faithful) {
         // ggml's arithmetic: the hidden rows are converted, in place, for the down projection
@@ -492,13 +598,18 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     }
     a.w0 = L.down.packed; a.w1 = nullptr; a.x = b.h; a.out_pair = b.out_pair; a.K = sh.F; a.N = sh.E;
     const unsigned d_blocks = (unsigned)(((size_t)sh.n_expert * (sh.E / 16) + 3) / 4);
-    if (L.down.type == WT_MXFP4) {
-        if (one_tile) hipLaunchKernelGGL((k_moe_down<WT_MXFP4, 1>), dim3(d_blocks), dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((k_moe_down<WT_MXFP4, 2>), dim3(d_blocks), dim3(256), 0, s, a);
-    } else {
-        if (one_tile) hipLaunchKernelGGL((k_moe_down<WT_Q8_0, 1>), dim3(d_blocks), dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((k_moe_down<WT_Q8_0, 2>), dim3(d_blocks), dim3(256), 0, s, a);
+#define RK_MOE_DOWN(TYPE)                                                                                        \
+    do {                                                                                                         \
+        if (one_tile) hipLaunchKernelGGL((k_moe_down<TYPE, 1>), dim3(d_blocks), dim3(256), 0, s, a);              \
+        else hipLaunchKernelGGL((k_moe_down<TYPE, 2>), dim3(d_blocks), dim3(256), 0, s, a);                       \
+    } while (0)
+    switch (L.down.type) {
+        case WT_MXFP4: RK_MOE_DOWN(WT_MXFP4); break;
+        case WT_Q4_K:  RK_MOE_DOWN(WT_Q4_K); break;
+        case WT_Q6_K:  RK_MOE_DOWN(WT_Q6_K); break;
+        default:       RK_MOE_DOWN(WT_Q8_0); break;
     }
+#undef RK_MOE_DOWN
     check_launch("moe_down");
     hipLaunchKernelGGL(k_moe_combine, dim3(T, (sh.E / 4 + 255) / 256), dim3(256), 0, s, b.out_pair, b.q_of_pair, b.wgt,
                        sh.k_used, sh.E, x);

@@ -1,6 +1,6 @@
 """Mixture-of-experts layers on the GPU against the CPU oracle (qwen3moe:
 softmax router, top-k experts with renormalised weights, SwiGLU experts;
-MXFP4 and Q8_0 expert weights)."""
+MXFP4, Q8_0, Q4_K and Q6_K expert weights)."""
 import numpy as np
 import pytest
 
@@ -17,6 +17,9 @@ BASE = dict(n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64, n_vocab=1
 SHAPES = {
     "mxfp4": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-mxfp4", **BASE),
     "q8_0": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q8", expert_type=gw.GGML_Q8_0, **BASE),
+    # the expert types of a Q4_K_M mixture-of-experts file
+    "q4_k": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q4k", expert_type=gw.GGML_Q4_K, **BASE),
+    "q6_k": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q6k", expert_type=gw.GGML_Q6_K, **BASE),
 }
 
 

@@ -37,6 +37,7 @@ class ModelShape:
     n_expert_used: int = 0
     n_ff_exp: int = 0
     expert_type: int = gw.GGML_MXFP4
+    expert_down_type: int = -1       # ffn_down_exps on the finer layers (-1: expert_type)
     qkv_bias: bool = False
     eps: float = 1e-5
     name: str = "synthetic"
@@ -307,7 +308,8 @@ def write_model(path, shape: ModelShape, seed: int = 0, device: str | None = Non
             matrix(b + "ffn_gate_inp.weight", E, s.n_expert, gw.GGML_F32, sd=E ** -0.5)
             matrix(b + "ffn_gate_exps.weight", E, s.n_ff_exp, s.expert_type, s.n_expert)
             matrix(b + "ffn_up_exps.weight", E, s.n_ff_exp, s.expert_type, s.n_expert)
-            matrix(b + "ffn_down_exps.weight", s.n_ff_exp, E, s.expert_type, s.n_expert)
+            matrix(b + "ffn_down_exps.weight", s.n_ff_exp, E,
+                   s.expert_down_type if (s.expert_down_type >= 0 and fine) else s.expert_type, s.n_expert)
         else:
             matrix(b + "ffn_gate.weight", E, s.n_ff)
             matrix(b + "ffn_up.weight", E, s.n_ff)

@@ -20,6 +20,9 @@ SHAPES = {
     # the expert types of a Q4_K_M mixture-of-experts file
     "q4_k": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q4k", expert_type=gw.GGML_Q4_K, **BASE),
     "q6_k": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q6k", expert_type=gw.GGML_Q6_K, **BASE),
+    # the whole mix of such a file: Q4_K matrices and experts, Q6_K for attn_v, the experts' down projection and the head
+    "q4_k_m": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q4km", matrix_type=gw.GGML_Q4_K, v_type=gw.GGML_Q6_K,
+                           output_type=gw.GGML_Q6_K, expert_type=gw.GGML_Q4_K, expert_down_type=gw.GGML_Q6_K, **BASE),
 }
 
 

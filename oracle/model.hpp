@@ -126,6 +126,7 @@ inline void ggml_activation_row(uint32_t wtype, const float * x, size_t K, float
     if (exact_activations()) { std::copy(x, x + K, out); return; }
     switch (wtype) {
         case T_Q4_K:
+        case T_Q5_K:
         case T_Q6_K: {
             if (K % 256) throw std::runtime_error("oracle: Q8_K activations need K % 256 == 0");
             for (size_t b = 0; b < K; b += 256) {

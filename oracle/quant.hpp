@@ -23,7 +23,7 @@ namespace oracle {
 
 // ggml type ids as stored in a GGUF tensor table.
 enum ggml_type_id : uint32_t {
-    T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14, T_BF16 = 30, T_MXFP4 = 39,
+    T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_BF16 = 30, T_MXFP4 = 39,
 };
 
 struct block_geom { uint32_t elements; uint32_t bytes; };
@@ -36,6 +36,7 @@ inline block_geom geom_of(uint32_t type) {
         case T_Q8_0:  return {32, 34};
         case T_MXFP4: return {32, 17};
         case T_Q4_K:  return {256, 144};
+        case T_Q5_K:  return {256, 176};
         case T_Q6_K:  return {256, 210};
         default: throw std::runtime_error("oracle: unsupported ggml type " + std::to_string(type));
     }
@@ -180,6 +181,31 @@ inline void decode_row(uint32_t type, const uint8_t * src, size_t n, float * out
                     for (int l = 0; l < 32; ++l) {
                         y[64 * pair + l]      = d1 * (float)(q[l] & 0x0f) - mm1;
                         y[64 * pair + 32 + l] = d2 * (float)(q[l] >> 4) - mm2;
+                    }
+                }
+            }
+            return;
+        case T_Q5_K:  // quant.rs:418-442: d, dmin | scales[12] | qh[32] | qs[128]
+            // As Q4_K with a fifth bit: element l of sub-block s takes bit s of qh[l] as 16.
+            for (size_t b = 0; b < n / 256; ++b) {
+                const uint8_t * blk = src + b * 176;
+                const float d = half_to_float(rd16(blk));
+                const float dmin = half_to_float(rd16(blk + 2));
+                const uint8_t * scales = blk + 4;
+                const uint8_t * qh = blk + 16;
+                const uint8_t * qs = blk + 48;
+                float * y = out + b * 256;
+                for (int pair = 0; pair < 4; ++pair) {
+                    uint8_t sc1, m1, sc2, m2;
+                    q4k_scale_min(2 * pair, scales, sc1, m1);
+                    q4k_scale_min(2 * pair + 1, scales, sc2, m2);
+                    const float d1 = d * (float)sc1, mm1 = dmin * (float)m1;
+                    const float d2 = d * (float)sc2, mm2 = dmin * (float)m2;
+                    const uint8_t * q = qs + 32 * pair;
+                    for (int l = 0; l < 32; ++l) {
+                        const int h1 = (qh[l] >> (2 * pair)) & 1 ? 16 : 0, h2 = (qh[l] >> (2 * pair + 1)) & 1 ? 16 : 0;
+                        y[64 * pair + l]      = d1 * (float)((q[l] & 0x0f) + h1) - mm1;
+                        y[64 * pair + 32 + l] = d2 * (float)((q[l] >> 4) + h2) - mm2;
                     }
                 }
             }

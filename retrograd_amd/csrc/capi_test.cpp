@@ -124,8 +124,8 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
 int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,
                              int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us) {
     return guarded([&]() -> int {
-        if (type != rk::WT_Q4_K && type != rk::WT_Q8_0 && type != rk::WT_Q6_K)
-            throw std::runtime_error("matmul_time: the tile kernels take Q4_K, Q6_K and Q8_0");
+        if (type != rk::WT_Q4_K && type != rk::WT_Q8_0 && type != rk::WT_Q6_K && type != rk::WT_Q5_K)
+            throw std::runtime_error("matmul_time: the tile kernels take Q4_K, Q5_K, Q6_K and Q8_0");
         if (n_rows <= 0 || k <= 0 || n_rows % 16 != 0 || k % 256 != 0 || n_tokens <= 0 || iters <= 0)
             throw std::runtime_error("matmul_time: whole 16-row tiles and super-blocks of 256, at least one token and one launch");
         const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
@@ -151,7 +151,7 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
                 for (size_t t = 0; t + 3360 <= bytes; t += 3360)
                     for (size_t i = 256; i < 288; i += 2) { host[t + i] = 0x1f; host[t + i + 1] = 0x21; }
             } else {
-                const size_t blk = type == rk::WT_Q4_K ? 144 : 34;
+                const size_t blk = type == rk::WT_Q4_K ? 144 : (type == rk::WT_Q5_K ? 176 : 34);
                 for (size_t i = 0; i + 4 <= bytes; i += blk) { host[i] = 0x1f; host[i + 1] = 0x21; host[i + 2] = 0x1f; host[i + 3] = 0x21; }
             }
             for (size_t c = 0; c < copies; ++c) ok(hipMemcpy(d_w.as<uint8_t>() + c * bytes, host.data(), bytes, hipMemcpyHostToDevice), "fill");

@@ -14,6 +14,8 @@
 //            with 0x000F000F / 0x00F000F0 yields f16 pairs in natural order.
 //      Q8_0  4352 B = 16 x scales[8] (f16) + 4 loads; lane (r, g) of load q
 //            holds elements 32*(2q)+8g..+8 and 32*(2q+1)+8g..+8 of row r.
+//      Q5_K  2816 B = the Q4_K tile of the low nibbles + 512 B of fifth bits (k_repack_q4k<true>).
+//      Q6_K  3360 B = scales, d, a plane of low nibbles and a plane of top bit pairs (k_repack_q6k).
 //    The byte count equals the GGUF byte count of the same matrix.
 //
 //  * KV pages. A page holds 32 positions of one sequence for one kv head:
@@ -41,6 +43,7 @@ BlockGeom geom_of(int type) {
         case WT_Q8_0:  return {32, 34};
         case WT_MXFP4: return {32, 17};
         case WT_Q4_K:  return {256, 144};
+        case WT_Q5_K:  return {256, 176};
         case WT_Q6_K:  return {256, 210};
         default: throw std::runtime_error("unsupported tensor type " + std::to_string(type));
     }
@@ -53,7 +56,7 @@ size_t row_bytes(int type, int64_t k) {
 }
 
 bool can_pack(int type, int64_t K, int64_t N) {
-    return (type == WT_Q4_K || type == WT_Q8_0 || type == WT_Q6_K) && K % 256 == 0 && N % 16 == 0 && K > 0 && N > 0;
+    return (type == WT_Q4_K || type == WT_Q8_0 || type == WT_Q6_K || type == WT_Q5_K) && K % 256 == 0 && N % 16 == 0 && K > 0 && N > 0;
 }
 
 // ---------------------------------------------------------------------------
@@ -84,8 +87,11 @@ __device__ float decode_elem(int type, const uint8_t * row, int k) {
             const float d = __uint_as_float(bits);
             return __fmul_rn(d, (float)((code & 8) ? -dv : dv));
         }
-        case WT_Q4_K: {
-            const uint8_t * b = row + (size_t)(k >> 8) * 144;
+        case WT_Q4_K:
+        case WT_Q5_K: {
+            // Q5_K: d, dmin | scales[12] | qh[32] | qs[128] - a Q4_K block with a fifth bit, bit (e / 32) of qh[e % 32]
+            const bool five = type == WT_Q5_K;
+            const uint8_t * b = row + (size_t)(k >> 8) * (five ? 176 : 144);
             const int e = k & 255;
             const int j = e >> 5;
             const uint8_t * sc = b + 4;
@@ -97,8 +103,9 @@ __device__ float decode_elem(int type, const uint8_t * row, int k) {
                 s = (sc[j + 4] & 0x0f) | ((sc[j - 4] >> 6) << 4);
                 m = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4);
             }
-            const uint8_t byte = b[16 + (e >> 6) * 32 + (e & 31)];
-            const int q = (e & 32) ? (byte >> 4) : (byte & 0x0f);
+            const uint8_t byte = b[(five ? 48 : 16) + (e >> 6) * 32 + (e & 31)];
+            int q = (e & 32) ? (byte >> 4) : (byte & 0x0f);
+            if (five) q += ((b[16 + (e & 31)] >> j) & 1) << 4;
             const float d = h2f(*(const uint16_t *)b);
             const float dmin = h2f(*(const uint16_t *)(b + 2));
             return __fsub_rn(__fmul_rn(__fmul_rn(d, (float)s), (float)q), __fmul_rn(dmin, (float)m));
@@ -182,19 +189,24 @@ void stream_copy(hipStream_t s, const void * src, void * dst, size_t bytes, int 
 // ---------------------------------------------------------------------------
 // weight repacking (runs once per tensor at load)
 
+// FIVE: Q5_K. The tile is the Q4_K tile of the low nibbles followed by 512 bytes of fifth bits, one dword per
+// k-half and lane: for k-step j the bits of the lane's elements 0 and 4 at 2j and 2j + 1, of 2 and 6 at 8 + 2j.., of
+// 1 and 5 at 16 + 2j.., of 3 and 7 at 24 + 2j.. - one shift puts them above the nibbles the Q4_K decode isolates.
+template <bool FIVE>
 __global__ void k_repack_q4k(const uint8_t * __restrict__ raw, uint8_t * __restrict__ dst, int nsb, int n_tiles) {
-    // one thread per output dword: 576 dwords per (tile, super-block)
+    // one thread per output dword: 576 (704) dwords per (tile, super-block)
+    constexpr int DW = FIVE ? 704 : 576, BLK = FIVE ? 176 : 144, QS = FIVE ? 48 : 16;
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t total = (size_t)n_tiles * nsb * 576;
+    const size_t total = (size_t)n_tiles * nsb * DW;
     if (gid >= total) return;
-    const int w = (int)(gid % 576);
-    const size_t ts = gid / 576;
+    const int w = (int)(gid % DW);
+    const size_t ts = gid / DW;
     const int sb = (int)(ts % nsb);
     const size_t rt = ts / nsb;
     uint32_t out;
     if (w < 64) {                       // headers: row r, dword j
         const int r = w >> 2, j = w & 3;
-        const uint8_t * blk = raw + ((rt * 16 + r) * nsb + sb) * 144;
+        const uint8_t * blk = raw + ((rt * 16 + r) * nsb + sb) * BLK;
         if (j == 0) {
             out = *(const uint32_t *)blk;          // d, dmin
         } else {
@@ -210,24 +222,34 @@ __global__ void k_repack_q4k(const uint8_t * __restrict__ raw, uint8_t * __restr
                 out |= (low | (top << 6)) << (8 * i);
             }
         }
+    } else if (FIVE && w >= 576) {
+        const int v = w - 576;
+        const int h = v >> 6, lane = v & 63;
+        const int r = lane & 15, g = lane >> 4;
+        const uint8_t * blk = raw + ((rt * 16 + r) * nsb + sb) * BLK;
+        const int place[8] = {0, 16, 8, 24, 1, 17, 9, 25};      // element i of the lane's eight, at k-step 0
+        out = 0;
+        for (int j = 0; j < 4; ++j)
+            for (int i = 0; i < 8; ++i)
+                out |= (uint32_t)((blk[16 + 8 * g + i] >> (4 * h + j)) & 1) << (place[i] + 2 * j);
     } else {
         const int v = w - 64;           // 0..511
         const int h = v >> 8;           // load
         const int lane = (v >> 2) & 63;
         const int j = v & 3;
         const int r = lane & 15, g = lane >> 4;
-        const uint8_t * blk = raw + ((rt * 16 + r) * nsb + sb) * 144;
+        const uint8_t * blk = raw + ((rt * 16 + r) * nsb + sb) * BLK;
         const int s = 4 * h + j;        // sub-block
         uint32_t nib[8];
         for (int i = 0; i < 8; ++i) {
             const int e = 32 * s + 8 * g + i;
-            const uint8_t byte = blk[16 + (e >> 6) * 32 + (e & 31)];
+            const uint8_t byte = blk[QS + (e >> 6) * 32 + (e & 31)];
             nib[i] = (e & 32) ? (byte >> 4) : (byte & 0x0f);
         }
         out = nib[0] | (nib[2] << 4) | (nib[4] << 8) | (nib[6] << 12)
             | (nib[1] << 16) | (nib[3] << 20) | (nib[5] << 24) | (nib[7] << 28);
     }
-    *(uint32_t *)(dst + ts * 2304 + (size_t)w * 4) = out;
+    *(uint32_t *)(dst + ts * (DW * 4) + (size_t)w * 4) = out;
 }
 
 __global__ void k_repack_q8_0(const uint8_t * __restrict__ raw, uint8_t * __restrict__ dst, int nsb, int n_tiles) {
@@ -319,11 +341,12 @@ __global__ void k_repack_q6k(const uint8_t * __restrict__ raw, uint8_t * __restr
 void repack(hipStream_t s, int type, const uint8_t * raw, uint8_t * packed, int K, int N) {
     if (!can_pack(type, K, N)) throw std::runtime_error("repack: shape or type has no tile layout");
     const int nsb = K / 256, n_tiles = N / 16;
-    const size_t per = type == WT_Q4_K ? 576 : (type == WT_Q6_K ? 840 : 1088);     // dwords per tile and super-block
+    const size_t per = type == WT_Q4_K ? 576 : (type == WT_Q5_K ? 704 : (type == WT_Q6_K ? 840 : 1088));     // dwords per tile and super-block
     const size_t total = (size_t)n_tiles * nsb * per;
     if ((total + 255) / 256 > 0x7fffffffu) throw std::runtime_error("repack: the matrix is too large for one launch");
     const unsigned blocks = (unsigned)((total + 255) / 256);
-    if (type == WT_Q4_K) hipLaunchKernelGGL(k_repack_q4k, dim3(blocks), dim3(256), 0, s, raw, packed, nsb, n_tiles);
+    if (type == WT_Q4_K) hipLaunchKernelGGL(k_repack_q4k<false>, dim3(blocks), dim3(256), 0, s, raw, packed, nsb, n_tiles);
+    else if (type == WT_Q5_K) hipLaunchKernelGGL(k_repack_q4k<true>, dim3(blocks), dim3(256), 0, s, raw, packed, nsb, n_tiles);
     else if (type == WT_Q6_K) hipLaunchKernelGGL(k_repack_q6k, dim3(blocks), dim3(256), 0, s, raw, packed, nsb, n_tiles);
     else hipLaunchKernelGGL(k_repack_q8_0, dim3(blocks), dim3(256), 0, s, raw, packed, nsb, n_tiles);
     check_launch("repack");
@@ -649,7 +672,8 @@ static Slices matmul_impl(hipStream_t s, const Weight & w, const Act & x, int T,
     // the tile kernels know two layouts; anything else handed over as tiles would be read as one of them, out of bounds
     if (!can_pack(w.type, w.K, w.N)) throw std::runtime_error("matmul: this matrix type or shape has no tile layout");
     if (ws) return matmul_lds(s, w, x, T, y, ldy, col0, mode, bias, ws, may_slice);
-    if (w.type == WT_Q6_K) throw std::runtime_error("matmul: Q6_K tiles are multiplied by the LDS kernels only (pass the workspace)");
+    if (w.type == WT_Q6_K || w.type == WT_Q5_K)
+        throw std::runtime_error("matmul: Q5_K and Q6_K tiles are multiplied by the LDS kernels only (pass the workspace)");
     const Act xo = x.operand(w.type);
     if (!xo.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
     if (w.type == WT_Q4_K && !xo.sums) throw std::runtime_error("matmul: Q4_K needs block sums");

@@ -11,7 +11,7 @@
 namespace rk {
 
 // ggml tensor type ids as stored in GGUF.
-enum : int { WT_F32 = 0, WT_F16 = 1, WT_Q8_0 = 8, WT_Q4_K = 12, WT_Q6_K = 14, WT_BF16 = 30, WT_MXFP4 = 39 };
+enum : int { WT_F32 = 0, WT_F16 = 1, WT_Q8_0 = 8, WT_Q4_K = 12, WT_Q5_K = 13, WT_Q6_K = 14, WT_BF16 = 30, WT_MXFP4 = 39 };
 
 // One KV page holds PAGE consecutive positions of one sequence.
 constexpr int PAGE = 32;
@@ -64,7 +64,7 @@ enum : int { AQ_NONE = 0, AQ_Q8_0 = 32, AQ_Q8_K = 256 };
 // The conversion ggml's CPU matmul applies for a weight of this storage type.
 inline int act_quant_of(int ggml_type) {
     switch (ggml_type) {
-        case 12: case 14: return AQ_Q8_K;   // Q4_K, Q6_K
+        case 12: case 13: case 14: return AQ_Q8_K;   // Q4_K, Q5_K, Q6_K
         case 8: case 39: return AQ_Q8_0;    // Q8_0, MXFP4
         default: return AQ_NONE;
     }

@@ -240,8 +240,11 @@ __device__ __forceinline__ h2 magic_pair(uint32_t word, uint32_t sel) {
 
 }  // namespace
 
-template <int NT, int R>
+// FIVE: Q5_K - the same tile followed by a plane of fifth bits (one dword per k-half and lane), which one shift
+// per use puts above the nibbles; sc * e stays an exact f16 (at most 63 * 31).
+template <int NT, int R, bool FIVE = false>
 __global__ __launch_bounds__(kThreads, NT <= 2 ? 4 : 1) void k_mm2_q4k(MMArgs a) {
+    constexpr uint32_t TILE = FIVE ? 2816u : 2304u;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -272,15 +275,18 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 4 : 1) void k_mm2_q4k(MMArgs a)
     WeightRows wbase[R];
 #pragma unroll
     for (int r = 0; r < R; ++r)
-        wbase[r] = weight_rows(a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * 2304, (uint32_t)nsb * 2304u);
+        wbase[r] = weight_rows(a.w + (size_t)min(rt[r], a.n_row_tiles - 1) * nsb * TILE, (uint32_t)nsb * TILE);
     // this wave's weights of one super-block: the row headers and its half of the payload
-    struct WSet { u4 hdr[R]; u4 q[R]; };
-    const uint32_t off_hdr = r16 * 16, off_q = 256 + kh * 1024 + lane * 16;
+    struct WSet { u4 hdr[R]; u4 q[R]; uint32_t top[R]; };
+    constexpr int LOADS = FIVE ? 3 : 2;        // per row tile and set
+    const uint32_t off_hdr = r16 * 16, off_q = 256 + kh * 1024 + lane * 16, off_top = 2304 + kh * 256 + lane * 4;
     auto load_w = [&](int sb, WSet & w) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            w.hdr[r] = load16(wbase[r], off_hdr, (uint32_t)sb * 2304u);
-            w.q[r] = load16(wbase[r], off_q, (uint32_t)sb * 2304u);
+            w.hdr[r] = load16(wbase[r], off_hdr, (uint32_t)sb * TILE);
+            w.q[r] = load16(wbase[r], off_q, (uint32_t)sb * TILE);
+            if (FIVE) w.top[r] = load4(wbase[r], off_top, (uint32_t)sb * TILE);
+            else w.top[r] = 0;
         }
     };
     const h2 m1024 = {(_Float16)(-1024.0f), (_Float16)(-1024.0f)};
@@ -290,13 +296,16 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 4 : 1) void k_mm2_q4k(MMArgs a)
     // next (activations one super-block ahead, weights two), multiply.
     auto body = [&](int sb, WSet & w, WSet & fut) __attribute__((always_inline)) {
         uint8_t * cur = smem + ((sb - sb0) & 1) * XStage<NT>::BYTES;
-        // All but the newest 2R loads (the weights one super-block ahead) have
+        // All but the newest LOADS x R loads (the weights one super-block ahead) have
         // landed: this super-block's activations and weights are in.
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * R));
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS * R));
         // the set is usable from here on and not before (nothing of it is to be touched, and so waited
         // for, inside the super-block before)
 #pragma unroll
-        for (int r = 0; r < R; ++r) asm volatile("" : "+v"(w.hdr[r]), "+v"(w.q[r]));
+        for (int r = 0; r < R; ++r) {
+            asm volatile("" : "+v"(w.hdr[r]), "+v"(w.q[r]));
+            if (FIVE) asm volatile("" : "+v"(w.top[r]));
+        }
         __syncthreads();   // ... for every wave, and nobody still reads the other buffer
         if (sb + 1 < sb1) stage_x<NT>(stage, sb + 1, (sb - sb0 + 1) & 1, true);
         load_w(min(sb + 2, sb1 - 1), fut);
@@ -356,10 +365,20 @@ __global__ __launch_bounds__(kThreads, NT <= 2 ? 4 : 1) void k_mm2_q4k(MMArgs a)
                 const uint32_t wq = w.q[r][j];
                 const uint32_t w8 = wq >> 8;
                 // 1024 + e in the low nibble positions, 64 + e in the high ones
-                const h2 u0 = __builtin_bit_cast(h2, and_or(wq, 0x000F000Fu, magic1024));
-                const h2 u1 = __builtin_bit_cast(h2, and_or(wq, 0x00F000F0u, magic64));
-                const h2 u2 = __builtin_bit_cast(h2, and_or(w8, 0x000F000Fu, magic1024));
-                const h2 u3 = __builtin_bit_cast(h2, and_or(w8, 0x00F000F0u, magic64));
+                uint32_t v0 = and_or(wq, 0x000F000Fu, magic1024), v1 = and_or(wq, 0x00F000F0u, magic64);
+                uint32_t v2 = and_or(w8, 0x000F000Fu, magic1024), v3 = and_or(w8, 0x00F000F0u, magic64);
+                if (FIVE) {
+                    // the fifth bits of this k-step: elements 0, 4 (1, 5) at bits 2j, 2j + 1 (16 + 2j ..), wanted at
+                    // bit 4 (20); elements 2, 6 (3, 7) at 8 + 2j .. (24 + 2j ..), wanted at bit 8 (24)
+                    const uint32_t ta = j < 2 ? w.top[r] << ((4 - 2 * j) & 31) : w.top[r] >> ((2 * j - 4) & 31);
+                    const uint32_t tb = w.top[r] >> (2 * j);
+                    v0 = and_or(ta, 0x00100010u, v0);
+                    v2 = and_or(ta >> 1, 0x00100010u, v2);
+                    v1 = and_or(tb, 0x01000100u, v1);
+                    v3 = and_or(tb >> 1, 0x01000100u, v3);
+                }
+                const h2 u0 = __builtin_bit_cast(h2, v0), u1 = __builtin_bit_cast(h2, v1);
+                const h2 u2 = __builtin_bit_cast(h2, v2), u3 = __builtin_bit_cast(h2, v3);
                 const h2 a0 = __builtin_elementwise_fma(u0, k1, c1);   // exactly sc * e (<= 945)
                 const h2 a1 = __builtin_elementwise_fma(u1, k1, c2);
                 const h2 a2 = __builtin_elementwise_fma(u2, k1, c1);
@@ -887,6 +906,13 @@ static void launch2(hipStream_t s, int type, const MMArgs & a, dim3 grid) {
             return;
         }
         hipLaunchKernelGGL((k_mm2_q4k<NT, R>), grid, dim3(kThreads), lds, s, a);
+    } else if (type == WT_Q5_K) {
+        static bool once = false;
+        if (!once) {
+            HIP_OK(hipFuncSetAttribute((const void *)k_mm2_q4k<NT, R, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            once = true;
+        }
+        hipLaunchKernelGGL((k_mm2_q4k<NT, R, true>), grid, dim3(kThreads), lds, s, a);
     } else if (type == WT_Q6_K) {
         static bool once = false;
         if (!once) {
@@ -930,10 +956,10 @@ static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x_all, int T
                        int mode, const float * bias, void * ws, bool may_slice, const Act * act_out, float * act_f32,
                        const SharedSlices * shared = nullptr) {
     if (!w.packed || !can_pack(w.type, w.K, w.N))
-        throw std::runtime_error("matmul_lds: needs a tile-packed Q4_K, Q6_K or Q8_0 matrix of whole super-blocks and 16-row tiles");
+        throw std::runtime_error("matmul_lds: needs a tile-packed Q4_K, Q5_K, Q6_K or Q8_0 matrix of whole super-blocks and 16-row tiles");
     const Act x = x_all.operand(w.type);
     if (!x.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
-    if (w.type == WT_Q4_K && !x.sums) throw std::runtime_error("matmul: Q4_K needs block sums");
+    if ((w.type == WT_Q4_K || w.type == WT_Q5_K) && !x.sums) throw std::runtime_error("matmul: Q4_K and Q5_K need block sums");
     MMArgs a {};
     a.debug = g_mm_debug;
     a.w = w.packed; a.x = x.x; a.sums = x.sums; a.y = y; a.bias = bias;

@@ -26,10 +26,10 @@ T_UINT8, T_INT8, T_UINT16, T_INT16, T_UINT32, T_INT32, T_FLOAT32, T_BOOL, T_STRI
 T_UINT64, T_INT64, T_FLOAT64 = 10, 11, 12
 
 # ggml tensor types used by the decode step
-GGML_F32, GGML_F16, GGML_Q8_0, GGML_Q4_K, GGML_Q6_K, GGML_BF16, GGML_MXFP4 = 0, 1, 8, 12, 14, 30, 39
+GGML_F32, GGML_F16, GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_BF16, GGML_MXFP4 = 0, 1, 8, 12, 13, 14, 30, 39
 BLOCK_GEOMETRY = {  # type -> (elements per block, bytes per block)
     GGML_F32: (1, 4), GGML_F16: (1, 2), GGML_BF16: (1, 2),
-    GGML_Q8_0: (32, 34), GGML_MXFP4: (32, 17), GGML_Q4_K: (256, 144), GGML_Q6_K: (256, 210),
+    GGML_Q8_0: (32, 34), GGML_MXFP4: (32, 17), GGML_Q4_K: (256, 144), GGML_Q5_K: (256, 176), GGML_Q6_K: (256, 210),
 }
 
 _SCALAR_FMT = {

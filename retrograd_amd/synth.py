@@ -157,6 +157,40 @@ def quantize_q4_k(x: torch.Tensor) -> torch.Tensor:
     return out.reshape(rows, -1)
 
 
+def quantize_q5_k(x: torch.Tensor) -> torch.Tensor:
+    """[rows, K] float -> uint8 [rows, K/256*176]: as Q4_K with five-bit codes, the fifth bit of element l of
+    sub-block s in bit s of qh[l]; stored as d, dmin | scales[12] | qh[32] | qs[128]."""
+    rows, K = x.shape
+    nb = K // 256
+    b = x.reshape(rows, nb, 8, 32).float()
+    mn = b.amin(dim=-1).clamp(max=0.0)
+    mx = b.amax(dim=-1).clamp(min=0.0)
+    scale = (mx - mn) / 31.0
+    nmin = -mn
+    d = (scale.amax(dim=-1, keepdim=True) / 63.0).to(torch.float16)
+    dmin = (nmin.amax(dim=-1, keepdim=True) / 63.0).to(torch.float16)
+    df, dminf = d.float(), dmin.float()
+    sc = torch.where(df > 0, torch.round(scale / df.clamp(min=1e-30)), torch.zeros_like(scale)).clamp_(0, 63)
+    m = torch.where(dminf > 0, torch.round(nmin / dminf.clamp(min=1e-30)), torch.zeros_like(nmin)).clamp_(0, 63)
+    dl = (df * sc).unsqueeze(-1)
+    ml = (dminf * m).unsqueeze(-1)
+    q = torch.where(dl > 0, torch.round((b + ml) / dl.clamp(min=1e-30)), torch.zeros_like(b)).clamp_(0, 31).to(torch.uint8)
+    sc = sc.to(torch.uint8)
+    m = m.to(torch.uint8)
+    out = torch.empty(rows, nb, 176, dtype=torch.uint8, device=x.device)
+    out[..., 0:2] = d.view(torch.uint8).reshape(rows, nb, 2)
+    out[..., 2:4] = dmin.view(torch.uint8).reshape(rows, nb, 2)
+    out[..., 4:8] = (sc[..., 0:4] & 63) | ((sc[..., 4:8] >> 4) << 6)
+    out[..., 8:12] = (m[..., 0:4] & 63) | ((m[..., 4:8] >> 4) << 6)
+    out[..., 12:16] = (sc[..., 4:8] & 0x0F) | ((m[..., 4:8] & 0x0F) << 4)
+    top = q >> 4                                                   # [rows, nb, 8, 32]
+    shifts = torch.arange(8, device=x.device, dtype=torch.uint8).reshape(1, 1, 8, 1)
+    out[..., 16:48] = (top << shifts).sum(dim=2).to(torch.uint8)
+    qp = (q & 0x0F).reshape(rows, nb, 4, 2, 32)
+    out[..., 48:] = (qp[..., 0, :] | (qp[..., 1, :] << 4)).reshape(rows, nb, 128)
+    return out.reshape(rows, -1)
+
+
 def quantize_q6_k(x: torch.Tensor) -> torch.Tensor:
     """[rows, K] float -> uint8 [rows, K/256*210]: six-bit codes (offset 32) with an int8 scale per 16
     elements against an f16 super-block d, stored as ql[128] | qh[64] | scales[16] | d."""
@@ -217,6 +251,8 @@ def encode(x: torch.Tensor, ggml_type: int) -> np.ndarray:
         return quantize_q4_k(x).cpu().numpy()
     if ggml_type == gw.GGML_MXFP4:
         return quantize_mxfp4(x).cpu().numpy()
+    if ggml_type == gw.GGML_Q5_K:
+        return quantize_q5_k(x).cpu().numpy()
     if ggml_type == gw.GGML_Q6_K:
         return quantize_q6_k(x).cpu().numpy()
     raise ValueError("unsupported ggml type %d" % ggml_type)

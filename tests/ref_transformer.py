@@ -6,7 +6,7 @@ import oracle
 from gguf_reader import Reader
 
 
-F32, F16, Q8_0, Q4_K, Q6_K, BF16, MXFP4 = 0, 1, 8, 12, 14, 30, 39
+F32, F16, Q8_0, Q4_K, Q5_K, Q6_K, BF16, MXFP4 = 0, 1, 8, 12, 13, 14, 30, 39
 
 
 def ggml_activations(v, weight_type):
@@ -19,7 +19,7 @@ def ggml_activations(v, weight_type):
     independently of oracle/model.hpp."""
     x = np.asarray(v, np.float32)
     f32 = np.float32
-    if weight_type in (Q4_K, Q6_K):
+    if weight_type in (Q4_K, Q5_K, Q6_K):
         b = x.reshape(-1, 256)
         first = np.abs(b).argmax(-1)                      # argmax returns the first maximum
         mx = b[np.arange(len(b)), first]

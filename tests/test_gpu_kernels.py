@@ -53,12 +53,12 @@ def test_tile_matmul_matches_decoded_blocks(t, n, k, T, ggml):
 
 
 @pytest.mark.parametrize("ggml", [False, True])
+@pytest.mark.parametrize("t", [gw.GGML_Q6_K, gw.GGML_Q5_K])
 @pytest.mark.parametrize("n,k,T", [(16, 256, 1), (48, 512, 7), (64, 1024, 16), (256, 4096, 33), (4096, 2048, 64),
                                    (160, 768, 100), (2064, 256, 3), (96, 1024, 24), (512, 4096, 48), (1024, 14336, 5)])
-def test_q6k_tile_matmul_matches_decoded_blocks(n, k, T, ggml):
-    # Q6_K has LDS-staged tiles only (the finer type of a Q4_K_M file: ffn_down, attn_v, output)
-    print("case q6_k", n, k, T, ggml, flush=True)
-    t = gw.GGML_Q6_K
+def test_q6k_and_q5k_tile_matmul_matches_decoded_blocks(t, n, k, T, ggml):
+    # Q6_K and Q5_K have LDS-staged tiles only (the types of Q4_K_M / Q5_K_M files beside Q4_K)
+    print("case", t, n, k, T, ggml, flush=True)
     raw, dense = _weights(t, n, k, seed=n + k + T)
     x = np.random.default_rng(T).standard_normal((T, k)).astype(np.float32)
     want = _ref(t, dense, x, ggml)
@@ -73,7 +73,8 @@ def test_q6k_tile_matmul_matches_decoded_blocks(n, k, T, ggml):
 
 @pytest.mark.parametrize("ggml", [False, True])
 @pytest.mark.parametrize("t,k", [(gw.GGML_F16, 344), (gw.GGML_F32, 100), (gw.GGML_Q8_0, 128),
-                                 (gw.GGML_MXFP4, 96), (gw.GGML_Q4_K, 256), (gw.GGML_BF16, 64), (gw.GGML_Q6_K, 512)])
+                                 (gw.GGML_MXFP4, 96), (gw.GGML_Q4_K, 256), (gw.GGML_BF16, 64), (gw.GGML_Q6_K, 512),
+                                 (gw.GGML_Q5_K, 512)])
 def test_generic_matmul_every_storage_type(t, k, ggml):
     print("case", t, k, ggml, flush=True)
     n, T = 37, 11
@@ -88,7 +89,7 @@ def test_generic_matmul_every_storage_type(t, k, ggml):
     want = _ref(t, dense, x, ggml)
     got = E.kernel_matmul(t, raw, n, k, x, use_tiles=False, ggml_activations=ggml)
     assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max() + 1e-6
-    if ggml and t in (gw.GGML_F16, gw.GGML_BF16, gw.GGML_Q8_0, gw.GGML_Q4_K, gw.GGML_MXFP4, gw.GGML_Q6_K):
+    if ggml and t in (gw.GGML_F16, gw.GGML_BF16, gw.GGML_Q8_0, gw.GGML_Q4_K, gw.GGML_MXFP4, gw.GGML_Q6_K, gw.GGML_Q5_K):
         assert np.abs(want - _ref(t, dense, x, False)).max() > 1e-4 * np.abs(want).max()     # the conversion is visible
 
 
@@ -166,7 +167,32 @@ def test_q6k_tiles_are_exact_for_every_code_and_scale():
         assert np.array_equal(got[0].astype(np.float64), dense[:16, e]), e
 
 
-@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0, gw.GGML_Q6_K])
+def test_q5k_tiles_are_exact_for_every_code_scale_and_min():
+    # Random bytes: every five-bit code, six-bit scale and min in every tile position; d = dmin = 1 and
+    # small-integer activations keep every product and sum exact in f32.
+    rng = np.random.default_rng(13)
+    n, k, T = 48, 768, 16
+    blocks = rng.integers(0, 256, (n, k // 256, 176), dtype=np.uint8)
+    blocks[..., 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    blocks[..., 2:4] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    raw = blocks.reshape(n, -1)
+    dense = np.stack([oracle.decode_row(gw.GGML_Q5_K, raw[i], k) for i in range(n)]).astype(np.float64)
+    x = rng.integers(-2, 3, (T, k)).astype(np.float32)
+    x[:, ::32] = rng.choice([-127.0, 127.0], (T, k // 32))
+    assert np.array_equal(np.stack([oracle.activation_row(gw.GGML_Q5_K, r) for r in x]), x)
+    want = x.astype(np.float64) @ dense.T
+    assert ((np.abs(x).astype(np.float64) @ np.abs(dense).T) <= 2.0 ** 24).all()
+    for ggml in (False, True):
+        got = E.kernel_matmul(gw.GGML_Q5_K, raw, n, k, x, use_tiles=2, ggml_activations=ggml)
+        assert np.array_equal(got.astype(np.float64), want), ggml
+    for e in (0, 1, 4, 7, 8, 15, 16, 31, 32, 63, 64, 95, 96, 127, 128, 200, 255):
+        one = np.zeros((1, 256), np.float32)
+        one[0, e] = 1.0
+        got = E.kernel_matmul(gw.GGML_Q5_K, raw[:16, :176].copy(), 16, 256, one, use_tiles=2)
+        assert np.array_equal(got[0].astype(np.float64), dense[:16, e]), e
+
+
+@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0, gw.GGML_Q6_K, gw.GGML_Q5_K])
 def test_split_k_matmul_is_deterministic_and_exact(t):
     # 4096 x 4096 at 64 tokens splits K across workgroups; the reduction order
     # is fixed, so two runs agree bit for bit, and both match the decoded blocks.

@@ -36,6 +36,10 @@ SMALL = {
     "llama-q4k-m-1024": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=1024, n_head=8, n_head_kv=2, head_dim=128,
                                      n_ff=2048, n_vocab=2048, output_type=14, down_type=14, v_type=14,
                                      name="llama-q4k-m-1024"),
+    # the type mix of a Q5_K_M file: Q5_K matrices, Q6_K for output.weight, ffn_down and attn_v
+    "llama-q5k-m": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=1024, n_head=8, n_head_kv=2, head_dim=128,
+                                n_ff=2048, n_vocab=2048, matrix_type=13, output_type=14, down_type=14, v_type=14,
+                                name="llama-q5k-m-1024"),
 }
 
 

@@ -292,3 +292,77 @@ def test_q6_k_against_the_block_loops_and_single_codes():
     # Q6_K weights take Q8_K activations
     v = rng.standard_normal(256).astype(np.float32)
     assert np.array_equal(oracle.activation_row(Q6_K, v), oracle.activation_row(12, v))
+
+
+# ---- Q5_K (the main type of a Q5_K_M file) --------------------------------------------------------
+
+def _q5_k_by_the_block_loops(blk):
+    """One 176-byte block decoded by the loop structure the reference spells out
+    (crates/rir-core/src/quant.rs:418-442): four groups of 64, two running bit masks for the fifth bit."""
+    d, dmin = np.float32(blk[0:2].view(np.float16)[0]), np.float32(blk[2:4].view(np.float16)[0])
+    scales, qh, qs = blk[4:16], blk[16:48], blk[48:176]
+
+    def scale_min(j):
+        if j < 4:
+            return int(scales[j]) & 63, int(scales[j + 4]) & 63
+        return (int(scales[j + 4]) & 0xF) | ((int(scales[j - 4]) >> 6) << 4), (int(scales[j + 4]) >> 4) | ((int(scales[j]) >> 6) << 4)
+
+    y = np.zeros(256, np.float32)
+    u1, u2, o = 1, 2, 0
+    for g in range(4):
+        ql = qs[32 * g:]
+        sc1, m1 = scale_min(2 * g)
+        sc2, m2 = scale_min(2 * g + 1)
+        d1, mm1 = d * np.float32(sc1), dmin * np.float32(m1)
+        d2, mm2 = d * np.float32(sc2), dmin * np.float32(m2)
+        for l in range(32):
+            h1 = 16 if int(qh[l]) & u1 else 0
+            h2 = 16 if int(qh[l]) & u2 else 0
+            y[o + l] = d1 * np.float32((int(ql[l]) & 0xF) + h1) - mm1
+            y[o + 32 + l] = d2 * np.float32((int(ql[l]) >> 4) + h2) - mm2
+        o += 64
+        u1 <<= 2
+        u2 <<= 2
+    return y
+
+
+def test_q5_k_against_the_block_loops_and_single_codes():
+    Q5_K = 13
+    assert oracle.row_bytes(Q5_K, 512) == 2 * 176
+    rng = np.random.default_rng(12)
+    raw = rng.integers(0, 256, 2 * 176, dtype=np.uint8)
+    for b in range(2):
+        raw[b * 176:b * 176 + 2] = np.frombuffer(np.float16(0.03125 * (b + 1)).tobytes(), np.uint8)
+        raw[b * 176 + 2:b * 176 + 4] = np.frombuffer(np.float16(0.015625 * (b + 1)).tobytes(), np.uint8)
+    got = oracle.decode_row(Q5_K, raw, 512)
+    want = np.concatenate([_q5_k_by_the_block_loops(raw[b * 176:(b + 1) * 176]) for b in range(2)])
+    assert np.array_equal(got, want)
+    # one code, one element: d = 1, dmin = 0, every scale 1 (the six-bit fields of sub-blocks 0-3 in bytes 4-7,
+    # of 4-7 in the low nibbles of bytes 12-15), all codes 0 except element e, which gets 31
+    for e in (0, 17, 31, 32, 63, 64, 100, 127, 128, 200, 255):
+        blk = np.zeros(176, np.uint8)
+        blk[0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+        blk[4:8] = 1
+        blk[12:16] = 1
+        assert not oracle.decode_row(Q5_K, blk, 256).any()
+        s, l = e // 32, e % 32
+        blk[48 + 32 * (s // 2) + l] |= 0xF0 if s & 1 else 0x0F
+        blk[16 + l] |= 1 << s
+        y = oracle.decode_row(Q5_K, blk, 256)
+        assert y[e] == 31.0 and np.count_nonzero(y) == 1, e
+    # the same bytes without the fifth bits are the Q4_K block with the same header and nibbles
+    blk5 = rng.integers(0, 256, 176, dtype=np.uint8)
+    blk5[16:48] = 0
+    blk4 = np.concatenate([blk5[0:16], blk5[48:176]])
+    assert np.array_equal(oracle.decode_row(Q5_K, blk5, 256), oracle.decode_row(12, blk4, 256))
+    # the synthetic quantiser writes blocks that decode near their input
+    import torch
+    from retrograd_amd import synth
+    x = torch.randn(3, 512, generator=torch.Generator().manual_seed(4)) * 0.05
+    enc = synth.encode(x, Q5_K)
+    for r in range(3):
+        y = oracle.decode_row(Q5_K, enc[r], 512)
+        assert np.abs(y - x[r].numpy()).max() < 0.05 * np.abs(x[r].numpy()).max()
+    # Q5_K weights take Q8_K activations
+    v = rng.standard_normal(256).astype(np.float32)
+    assert np.array_equal(oracle.activation_row(Q5_K, v), oracle.activation_row(12, v))

@@ -41,7 +41,9 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
  * every launch another copy of the weights (1 GiB of copies in turn; adding 32,
  * 6 GiB), so that they are read from HBM as in a decode step instead of from
  * the last-level cache. debug and force_ksplit are timing experiments
- * (0 = normal). */
+ * (0 = normal). type is Q4_K, Q5_K, Q6_K or Q8_0 (Q5_K and Q6_K in modes 2 and
+ * 3 only), n_rows a multiple of 16 and k of 256: anything else is refused
+ * before a buffer is allocated. */
 int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,
                              int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us);
 

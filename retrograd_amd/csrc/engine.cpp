@@ -157,7 +157,7 @@ void Engine::upload_weight(const TensorInfo & t, int64_t K, int64_t N, const uin
 // An expert tensor [K][N][n_expert]: n_expert * N rows of K, tiled per expert.
 void Engine::upload_experts(const TensorInfo & t, int64_t K, int64_t N, DevWeight & out) {
     const int64_t rows = N * hp_.n_expert;
-    if (!rk::moe_can_pack(t.type, K, N)) throw std::runtime_error("expert tensor " + t.name + " must be MXFP4, Q8_0, Q4_K or Q6_K with widths that are multiples of 256 and 16");
+    if (!rk::moe_can_pack(t.type, K, N)) throw std::runtime_error("expert tensor " + t.name + " must be MXFP4, Q8_0, Q4_K, Q5_K or Q6_K with widths that are multiples of 256 and 16");
     if (rk::row_bytes(t.type, K) * (size_t)rows != t.nbytes) throw std::runtime_error("tensor " + t.name + " has an unexpected size");
     out.w.type = t.type;
     out.w.K = (int)K;

@@ -28,7 +28,7 @@
 namespace rk {
 
 bool moe_can_pack(int type, int64_t K, int64_t N) {
-    return (type == WT_MXFP4 || type == WT_Q8_0 || type == WT_Q4_K || type == WT_Q6_K) && K % 256 == 0 && N % 16 == 0 && K > 0 && N > 0;
+    return (type == WT_MXFP4 || type == WT_Q8_0 || type == WT_Q4_K || type == WT_Q5_K || type == WT_Q6_K) && K % 256 == 0 && N % 16 == 0 && K > 0 && N > 0;
 }
 
 __global__ void k_repack_mxfp4(const uint8_t * __restrict__ raw, uint8_t * __restrict__ dst, int nsb, size_t n_tiles) {
@@ -169,14 +169,18 @@ __device__ __forceinline__ void mac(const Q4KOperand & o, const h8 & hi, const h
 #pragma unroll
     for (int i = 0; i < 4; ++i) acc[i] = fmaf(-o.dm, sum[i], fmaf(o.d, p[i], acc[i]));
 }
-template <> struct Tile<WT_Q4_K> {
-    static constexpr int BYTES = 2304;
+// FIVE: Q5_K, the same tile followed by a plane of fifth bits (one dword per k-half and lane).
+template <bool FIVE> struct TileQ45 {
+    static constexpr int BYTES = FIVE ? 2816 : 2304;
     u4 hdr;
     u4 q0, q1;
+    uint32_t top0, top1;
     __device__ __forceinline__ void load(const uint8_t * tile, int lane) {
         hdr = *(const u4 *)(tile + (lane & 15) * 16);
         q0 = *(const u4 *)(tile + 256 + lane * 16);
         q1 = *(const u4 *)(tile + 256 + 1024 + lane * 16);
+        top0 = FIVE ? *(const uint32_t *)(tile + 2304 + lane * 4) : 0u;
+        top1 = FIVE ? *(const uint32_t *)(tile + 2304 + 256 + lane * 4) : 0u;
     }
     __device__ __forceinline__ Q4KOperand prep(int s) const {
         const Q4KScales s4 = q4k_scales(hdr);
@@ -188,10 +192,21 @@ template <> struct Tile<WT_Q4_K> {
         const h2 c1 = k1 * (_Float16)(-1024.0f), c2 = k1 * (_Float16)(-64.0f);
         const uint32_t wq = s < 4 ? q0[j] : q1[j];
         const uint32_t w8 = wq >> 8;
-        const h2 u0 = __builtin_bit_cast(h2, and_or(wq, 0x000F000Fu, 0x64006400u));     // 1024 + e
-        const h2 u1 = __builtin_bit_cast(h2, and_or(wq, 0x00F000F0u, 0x54005400u));     // 64 + e (nibble one place up)
-        const h2 u2 = __builtin_bit_cast(h2, and_or(w8, 0x000F000Fu, 0x64006400u));
-        const h2 u3 = __builtin_bit_cast(h2, and_or(w8, 0x00F000F0u, 0x54005400u));
+        uint32_t v0 = and_or(wq, 0x000F000Fu, 0x64006400u), v1 = and_or(wq, 0x00F000F0u, 0x54005400u);   // 1024 + e; 64 + e (nibble one place up)
+        uint32_t v2 = and_or(w8, 0x000F000Fu, 0x64006400u), v3 = and_or(w8, 0x00F000F0u, 0x54005400u);
+        if (FIVE) {
+            // fifth bits of this k-step: elements 0, 4 (1, 5) at bits 2j, 2j + 1 (16 + 2j ..) of the plane dword,
+            // wanted at bit 4 (20); elements 2, 6 (3, 7) at 8 + 2j .. (24 + 2j ..), wanted at bit 8 (24)
+            const uint32_t top = s < 4 ? top0 : top1;
+            const uint32_t ta = j < 2 ? top << ((4 - 2 * j) & 31) : top >> ((2 * j - 4) & 31);
+            const uint32_t tb = top >> (2 * j);
+            v0 = and_or(ta, 0x00100010u, v0);
+            v2 = and_or(ta >> 1, 0x00100010u, v2);
+            v1 = and_or(tb, 0x01000100u, v1);
+            v3 = and_or(tb >> 1, 0x01000100u, v3);
+        }
+        const h2 u0 = __builtin_bit_cast(h2, v0), u1 = __builtin_bit_cast(h2, v1);
+        const h2 u2 = __builtin_bit_cast(h2, v2), u3 = __builtin_bit_cast(h2, v3);
         const h2 a0 = __builtin_elementwise_fma(u0, k1, c1), a1 = __builtin_elementwise_fma(u1, k1, c2);
         const h2 a2 = __builtin_elementwise_fma(u2, k1, c1), a3 = __builtin_elementwise_fma(u3, k1, c2);
         Q4KOperand o;
@@ -201,6 +216,9 @@ template <> struct Tile<WT_Q4_K> {
         return o;
     }
 };
+
+template <> struct Tile<WT_Q4_K> : TileQ45<false> {};
+template <> struct Tile<WT_Q5_K> : TileQ45<true> {};
 
 // Q6_K, the dense tile (3360 bytes): value = d * scale * (code - 32) per 16-wide block; the i8 scale goes into the
 // operand in two parts whose products with a code are exact f16 numbers (its low four bits, and the rest).
@@ -564,9 +582,9 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     if (sh.n_expert > 256 || sh.k_used > 16 || sh.k_used > sh.n_expert) throw std::runtime_error("moe: unsupported expert count");
     // multiples of 256: whole super-blocks along K, and the four waves of a workgroup share an expert (N / 16 % 4 == 0)
     if (sh.E % 256 != 0 || sh.F % 256 != 0) throw std::runtime_error("moe: widths must be multiples of 256");
-    auto tiled = [](int t) { return t == WT_MXFP4 || t == WT_Q8_0 || t == WT_Q4_K || t == WT_Q6_K; };
+    auto tiled = [](int t) { return t == WT_MXFP4 || t == WT_Q8_0 || t == WT_Q4_K || t == WT_Q5_K || t == WT_Q6_K; };
     if (L.gate.type != L.up.type || !tiled(L.gate.type) || !tiled(L.down.type))
-        throw std::runtime_error("moe: expert weights must be MXFP4, Q8_0, Q4_K or Q6_K, gate and up of one type");
+        throw std::runtime_error("moe: expert weights must be MXFP4, Q8_0, Q4_K, Q5_K or Q6_K, gate and up of one type");
     matmul_generic(s, L.router, xn, T, b.logits, sh.n_expert, 0, MM_STORE, nullptr);
     hipLaunchKernelGGL(k_moe_route, dim3(T), dim3(64), 0, s, b.logits, sh.n_expert, sh.k_used, b.sel, b.wgt);
     check_launch("moe_route");
@@ -586,6 +604,7 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     switch (L.gate.type) {
         case WT_MXFP4: hipLaunchKernelGGL((k_moe_gate_up<WT_MXFP4, 2>), dim3(gu_blocks), dim3(256), 0, s, a); break;
         case WT_Q4_K:  hipLaunchKernelGGL((k_moe_gate_up<WT_Q4_K, 2>), dim3(gu_blocks), dim3(256), 0, s, a); break;
+        case WT_Q5_K:  hipLaunchKernelGGL((k_moe_gate_up<WT_Q5_K, 2>), dim3(gu_blocks), dim3(256), 0, s, a); break;
         case WT_Q6_K:  hipLaunchKernelGGL((k_moe_gate_up<WT_Q6_K, 2>), dim3(gu_blocks), dim3(256), 0, s, a); break;
         default:       hipLaunchKernelGGL((k_moe_gate_up<WT_Q8_0, 2>), dim3(gu_blocks), dim3(256), 0, s, a); break;
     }
@@ -606,6 +625,7 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     switch (L.down.type) {
         case WT_MXFP4: RK_MOE_DOWN(WT_MXFP4); break;
         case WT_Q4_K:  RK_MOE_DOWN(WT_Q4_K); break;
+        case WT_Q5_K:  RK_MOE_DOWN(WT_Q5_K); break;
         case WT_Q6_K:  RK_MOE_DOWN(WT_Q6_K); break;
         default:       RK_MOE_DOWN(WT_Q8_0); break;
     }

@@ -1,6 +1,6 @@
 """Mixture-of-experts layers on the GPU against the CPU oracle (qwen3moe:
 softmax router, top-k experts with renormalised weights, SwiGLU experts;
-MXFP4, Q8_0, Q4_K and Q6_K expert weights)."""
+MXFP4, Q8_0, Q4_K, Q5_K and Q6_K expert weights)."""
 import numpy as np
 import pytest
 
@@ -20,6 +20,7 @@ SHAPES = {
     # the expert types of a Q4_K_M mixture-of-experts file
     "q4_k": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q4k", expert_type=gw.GGML_Q4_K, **BASE),
     "q6_k": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q6k", expert_type=gw.GGML_Q6_K, **BASE),
+    "q5_k": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q5k", expert_type=gw.GGML_Q5_K, **BASE),
     # the whole mix of such a file: Q4_K matrices and experts, Q6_K for attn_v, the experts' down projection and the head
     "q4_k_m": synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-q4km", matrix_type=gw.GGML_Q4_K, v_type=gw.GGML_Q6_K,
                            output_type=gw.GGML_Q6_K, expert_type=gw.GGML_Q4_K, expert_down_type=gw.GGML_Q6_K, **BASE),

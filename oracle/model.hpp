@@ -224,11 +224,13 @@ inline const float * f32_data(const gguf_tensor & t) {
     return (const float *)t.data;
 }
 
-// Rotates one head in place; angle = pos * base^(-2i/d) evaluated in double.
-inline void rope(float * v, int head_dim, int rope_dim, int pos, double base, bool neox) {
+// Rotates one head in place; angle = pos * base^(-2i/d) / factor_i evaluated in double. The factors are the
+// model's rope_freqs.weight (ggml's rope divides theta by them: ggml_rope_cache_init, theta / ff) times the linear
+// scaling factor, null for none.
+inline void rope(float * v, int head_dim, int rope_dim, int pos, double base, bool neox, const double * factors = nullptr) {
     const int half = rope_dim / 2;
     for (int i = 0; i < half; ++i) {
-        const double angle = (double)pos * std::pow(base, -2.0 * i / rope_dim);
+        const double angle = (double)pos * std::pow(base, -2.0 * i / rope_dim) / (factors ? factors[i] : 1.0);
         const double c = std::cos(angle), s = std::sin(angle);
         const int i0 = neox ? i : 2 * i;
         const int i1 = neox ? i + half : 2 * i + 1;
@@ -325,6 +327,24 @@ struct context {
         const int E = h.n_embd, HD = h.head_dim, NH = h.n_head, NKV = h.n_head_kv;
         const int QD = NH * HD, KD = NKV * HD;
         const size_t kd = (size_t)KD;
+        // per-frequency divisors of the rotation angle: rope_freqs.weight and linear scaling (see rope())
+        std::vector<double> rope_div;
+        {
+            const std::string p = h.arch + ".rope.scaling.type";
+            const std::string scaling = g.has(p) ? g.s(p) : std::string("none");
+            double lin = 1.0;
+            if (scaling == "linear") lin = g.f_or(h.arch + ".rope.scaling.factor", 1.0);
+            else if (scaling != "none" && !scaling.empty()) throw std::runtime_error("oracle: rope scaling type " + scaling + " is not modelled");
+            const gguf_tensor * rf = g.find("rope_freqs.weight");
+            if (rf || lin != 1.0) {
+                rope_div.assign((size_t)(h.rope_dim / 2), lin);
+                if (rf) {
+                    if (rf->type != T_F32 || (int)rf->ne[0] != h.rope_dim / 2) throw std::runtime_error("oracle: rope_freqs.weight has an unexpected shape");
+                    for (size_t i = 0; i < rope_div.size(); ++i) rope_div[i] *= (double)f32_data(*rf)[i];
+                }
+            }
+        }
+        const double * rope_factors = rope_div.empty() ? nullptr : rope_div.data();
         std::vector<float> x((size_t)T * E), xn((size_t)T * E);
         {
             const gguf_tensor & emb = g.need("token_embd.weight");
@@ -368,13 +388,13 @@ struct context {
                 for (int hh = 0; hh < NH; ++hh) {
                     float * qh = &q[(size_t)t * QD + (size_t)hh * HD];
                     if (qn) rmsnorm(qh, f32_data(*qn), HD, h.eps, qh);
-                    rope(qh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox);
+                    rope(qh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox, rope_factors);
                 }
                 slot_state & s = slots[(size_t)slot[t]];
                 for (int hh = 0; hh < NKV; ++hh) {
                     float * kh = &k[(size_t)t * KD + (size_t)hh * HD];
                     if (kn) rmsnorm(kh, f32_data(*kn), HD, h.eps, kh);
-                    rope(kh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox);
+                    rope(kh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox, rope_factors);
                 }
                 uint16_t * kc = &s.k[(size_t)l][(size_t)pos[t] * kd];
                 uint16_t * vc = &s.v[(size_t)l][(size_t)pos[t] * kd];

@@ -310,9 +310,31 @@ void Engine::load_model(const std::string & path) {
         upload_weight(wd, h.n_ff, E, wd.data, wd.nbytes, false, L.down);
     }
 
-    // rotary frequencies in double: angle = pos * base^(-2i/d)
+    // rotary frequencies in double: angle = pos * base^(-2i/d), divided by the model's per-frequency factors
+    // (rope_freqs.weight, the long-context rule of Llama 3.1 and later: ggml's rope divides theta by them) and
+    // multiplied by 1 / factor under linear scaling. Other scaling rules (yarn, longrope) are not implemented:
+    // a model that declares one is refused rather than rotated wrongly.
     std::vector<double> inv((size_t)(h.rope_dim / 2));
     for (size_t i = 0; i < inv.size(); ++i) inv[i] = std::pow(h.rope_base, -2.0 * (double)i / h.rope_dim);
+    {
+        const std::string scaling = g.get_string(a + "rope.scaling.type", "none");
+        if (scaling == "linear") {
+            const double factor = g.get_float(a + "rope.scaling.factor", 1.0);
+            if (!(factor > 0.0)) throw std::runtime_error("rope.scaling.factor must be positive");
+            for (double & f : inv) f /= factor;
+        } else if (scaling != "none" && !scaling.empty()) {
+            throw std::runtime_error("rope scaling type '" + scaling + "' is not implemented");
+        }
+        if (const TensorInfo * rf = g.find("rope_freqs.weight")) {
+            if (rf->type != rk::WT_F32 || rf->ne[0] != (int64_t)inv.size() || rf->nbytes != inv.size() * sizeof(float))
+                throw std::runtime_error("rope_freqs.weight must hold rope_dim / 2 f32 factors");
+            const float * ff = (const float *)rf->data;
+            for (size_t i = 0; i < inv.size(); ++i) {
+                if (!(ff[i] > 0.0f)) throw std::runtime_error("rope_freqs.weight holds a factor that is not positive");
+                inv[i] /= (double)ff[i];
+            }
+        }
+    }
     inv_freq_.alloc(inv.size() * sizeof(double));
     hip_check(hipMemcpy(inv_freq_.ptr, inv.data(), inv.size() * sizeof(double), hipMemcpyHostToDevice), "hipMemcpy");
 

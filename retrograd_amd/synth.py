@@ -45,6 +45,9 @@ class ModelShape:
     output_type: int = -1            # output.weight
     down_type: int = -1              # ffn_down.weight
     v_type: int = -1                 # attn_v.weight
+    rope_freqs: bool = False         # write rope_freqs.weight: per-frequency divisors of the rotation angle as
+                                     # Llama 3.1's rule gives them (1 for short wavelengths, 8 for long, a ramp between)
+    rope_scaling_linear: float = 0.0 # > 0: rope.scaling.type = linear with this factor
     finer_layers: str = "all"        # layers whose ffn_down / attn_v take the finer type: "all", or "more_bits" =
                                      # the first and last eighth and every third layer between (llama.cpp's rule for Q4_K_M)
 
@@ -281,6 +284,9 @@ def _common_metadata(w: gw.GGUFWriter, s: ModelShape, with_eos: bool) -> None:
     w.add(a + ".attention.layer_norm_rms_epsilon", gw.T_FLOAT32, s.eps)
     w.add(a + ".rope.dimension_count", gw.T_UINT32, s.head_dim)
     w.add(a + ".rope.freq_base", gw.T_FLOAT32, s.rope_base)
+    if s.rope_scaling_linear > 0:
+        w.add(a + ".rope.scaling.type", gw.T_STRING, "linear")
+        w.add(a + ".rope.scaling.factor", gw.T_FLOAT32, s.rope_scaling_linear)
     if s.n_expert:
         w.add(a + ".expert_count", gw.T_UINT32, s.n_expert)
         w.add(a + ".expert_used_count", gw.T_UINT32, s.n_expert_used)
@@ -350,6 +356,18 @@ def write_model(path, shape: ModelShape, seed: int = 0, device: str | None = Non
             matrix(b + "ffn_gate.weight", E, s.n_ff)
             matrix(b + "ffn_up.weight", E, s.n_ff)
             matrix(b + "ffn_down.weight", s.n_ff, E, None if (s.down_type < 0 or not fine) else s.down_type)
+    if s.rope_freqs:
+        def llama3_factors():
+            # llama.cpp's convert script for Llama 3.1: factor 8, low / high frequency factors 1 / 4, over an
+            # original context of 8192 (scaled here to the rotary base in use)
+            half = s.head_dim // 2
+            freqs = 1.0 / (s.rope_base ** (np.arange(half, dtype=np.float64) * 2.0 / s.head_dim))
+            wavelen = 2.0 * np.pi / freqs
+            old_ctx, factor, lo, hi = 8192.0, 8.0, 1.0, 4.0
+            smooth = np.clip((old_ctx / wavelen - lo) / (hi - lo), 0.0, 1.0)
+            out = np.where(wavelen < old_ctx / hi, 1.0, np.where(wavelen > old_ctx / lo, factor, 1.0 / ((1.0 - smooth) / factor + smooth)))
+            return out.astype(np.float32)
+        w.add_tensor("rope_freqs.weight", [s.head_dim // 2], gw.GGML_F32, llama3_factors)
     vector("output_norm.weight", E, 1.0)
     matrix("output.weight", E, s.n_vocab, None if s.output_type < 0 else s.output_type)
     return w.write(Path(path))

@@ -66,6 +66,12 @@ class NumpyModel:
         self.n_used = g("expert_used_count", 0)
         self.neox = a != "llama"
         self.w = {}
+        # divisors of the rotation angle per frequency: linear scaling and the model's rope_freqs.weight
+        scaling = g("rope.scaling.type", "none")
+        assert scaling in ("none", "linear"), scaling
+        self.rope_div = np.full(self.D // 2, float(g("rope.scaling.factor", 1.0)) if scaling == "linear" else 1.0)
+        if "rope_freqs.weight" in r.tensors:
+            self.rope_div = self.rope_div * np.asarray(self.t("rope_freqs.weight"), np.float64).reshape(-1)
 
     def t(self, name):
         if name not in self.w:
@@ -82,7 +88,7 @@ class NumpyModel:
         # v: [heads, D]
         D = self.D
         i = np.arange(D // 2)
-        ang = pos * self.base ** (-2.0 * i / D)
+        ang = pos * self.base ** (-2.0 * i / D) / self.rope_div
         c, s = np.cos(ang), np.sin(ang)
         out = v.copy()
         if self.neox:

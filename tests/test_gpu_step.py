@@ -40,6 +40,10 @@ SMALL = {
     "llama-q5k-m": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=1024, n_head=8, n_head_kv=2, head_dim=128,
                                 n_ff=2048, n_vocab=2048, matrix_type=13, output_type=14, down_type=14, v_type=14,
                                 name="llama-q5k-m-1024"),
+    # per-frequency rotation divisors (rope_freqs.weight, Llama 3.1's long-context rule) and linear scaling
+    "llama-rope-freqs": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
+                                     n_ff=1024, n_vocab=1024, rope_freqs=True, rope_scaling_linear=2.0,
+                                     name="llama-rope-freqs-small"),
 }
 
 
@@ -296,3 +300,36 @@ def test_introspection_and_memory(models):
     assert part.context_size() == 128 and not part.kv_unified()
     part.close()
     eng.close()
+
+
+def test_rope_frequency_factors_and_linear_scaling_change_the_rotation_as_in_the_oracle(tmp_path):
+    """rope_freqs.weight (per-frequency divisors of the angle: ggml's rope, theta / ff) and rope.scaling.type =
+    linear. The same weights with and without them: each engine follows its own oracle, and the two differ by far
+    more than the tolerance, so an engine that ignored the factors would not pass. A scaling rule that is not
+    implemented is refused at load."""
+    base = synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64, n_ff=1024,
+                        n_vocab=1024, name="rope-plain")
+    with_f = synth.scaled(base, rope_freqs=True, rope_scaling_linear=2.0, name="rope-factors")
+    paths = {}
+    for key, shape in (("plain", base), ("factors", with_f)):
+        paths[key] = tmp_path / (key + ".gguf")
+        synth.write_model(paths[key], shape, seed=31, device="cpu", std=0.05)
+    toks = np.random.default_rng(3).integers(0, 1024, 200)
+    logits = {}
+    for key, path in paths.items():
+        eng, ctx, m = _pair(path, n_seq=2, n_ctx=1024)
+        out, got, want = run_both(eng, ctx, [(1, 0, toks, 0, True)])
+        assert_logits_close(got, want)
+        logits[key] = got
+        eng.close()
+    mx, mr = logit_errors(logits["factors"], logits["plain"])
+    print("the factors move the logits by %.3g (max), %.3g (mean, relative)" % (mx, mr), flush=True)
+    assert mx > 0.2 and mr > 1e-2
+    raw = bytearray(paths["factors"].read_bytes())
+    at = raw.find(b"linear")
+    assert at > 0
+    raw[at:at + 6] = b"yarnxx"
+    bad = tmp_path / "unknown-scaling.gguf"
+    bad.write_bytes(bytes(raw))
+    with pytest.raises(E.EngineError, match="not implemented"):
+        E.Engine(bad, E.EngineConfig(n_ctx=256, n_seq_max=1, n_batch=64, n_ubatch=64))

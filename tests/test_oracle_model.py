@@ -22,6 +22,9 @@ SHAPES = {
     # the type mix of a Q4_K_M file: output.weight, ffn_down and attn_v in Q6_K
     "llama-q4k-m": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=256, n_head=4, n_head_kv=2, head_dim=64,
                                 n_ff=512, n_vocab=320, output_type=14, down_type=14, v_type=14, name="llama-q4k-m-small"),
+    # per-frequency rotation divisors (rope_freqs.weight, Llama 3.1's long-context rule) and linear scaling
+    "llama-rope-freqs": synth.scaled(synth.TINY_LLAMA, rope_freqs=True, rope_scaling_linear=2.0, rope_base=500000.0,
+                                     name="tiny-llama-rope-freqs"),
 }
 
 

@@ -5,11 +5,14 @@
 // which the reference proves bit-equal to ggml's to_float on identical bytes
 // (tests/rir_quant_oracle.rs:67-103). Block geometry from
 // crates/rir-core/src/quant_table.rs (Q8_0 32 el / 34 B, MXFP4 32 el / 17 B,
-// Q4_K 256 el / 144 B).
+// Q4_K 256 el / 144 B, Q5_K 256 el / 176 B, Q6_K 256 el / 210 B).
 //
 // Pinned by: tests/test_oracle_quant.py (known answers of quant.rs:534-581,
 // exhaustive f16 against numpy, brute-force Q4_K addressing against
-// generated/rir/mul_mat_vec_q4_K/cpu.rs:52-120 semantics).
+// generated/rir/mul_mat_vec_q4_K/cpu.rs:52-120 semantics; Q5_K and Q6_K each
+// against an independent restatement of the loops quant.rs:418-464 spell out,
+// single codes placed on single elements, and Q5_K's reduction to Q4_K when
+// its fifth bits are clear).
 #pragma once
 
 #include <cmath>

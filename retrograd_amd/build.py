@@ -35,35 +35,43 @@ def hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
-def build(verbose: bool = False) -> Path:
+def _compile(cmd, src, verbose):
+    if verbose:
+        print(" ".join(cmd), file=sys.stderr)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed on %s:\n%s" % (src, err))
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+
+
+def build(verbose: bool = False, incremental: bool = False) -> Path:
+    """Compiles every source (several at a time) and links the library. `incremental` skips a source whose object
+    is newer than it and than every header; the default recompiles everything."""
+    from concurrent.futures import ThreadPoolExecutor
+
     LIB_DIR.mkdir(exist_ok=True)
     obj_dir = LIB_DIR / "obj"
     obj_dir.mkdir(exist_ok=True)
-    objs = []
-    for src in SOURCES:
-        obj = obj_dir / (src.rsplit(".", 1)[0] + ".o")
-        cmd = [hipcc(), *HIP_FLAGS, "-x", "hip", "-c", str(CSRC / src), "-o", str(obj)]
-        if verbose:
-            print(" ".join(cmd), file=sys.stderr)
-        res = subprocess.run(cmd, capture_output=True, text=True)
-        noise = "is not a recognized feature for this target"
-        err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
-        if res.returncode != 0:
-            raise RuntimeError("hipcc failed on %s:\n%s" % (src, err))
-        if verbose and err.strip():
-            print(err, file=sys.stderr)
-        objs.append(str(obj))
-    for src in HOST_SOURCES:
+    headers = [p for p in CSRC.rglob("*.h*")] + list((PKG.parent / "include").glob("*.h"))
+    newest_header = max(p.stat().st_mtime for p in headers)
+    jobs, objs = [], []
+    for src in SOURCES + HOST_SOURCES:
+        host = src in HOST_SOURCES
         obj = obj_dir / (src.replace("/", "_").rsplit(".", 1)[0] + ".o")
-        cmd = [hipcc(), *HOST_FLAGS, "-x", "c++", "-c", str(CSRC / src), "-o", str(obj)]
-        if verbose:
-            print(" ".join(cmd), file=sys.stderr)
-        res = subprocess.run(cmd, capture_output=True, text=True)
-        if res.returncode != 0:
-            raise RuntimeError("hipcc failed on %s:\n%s" % (src, res.stderr))
-        if verbose and res.stderr.strip():
-            print(res.stderr, file=sys.stderr)
         objs.append(str(obj))
+        if incremental and obj.exists() and obj.stat().st_mtime > max((CSRC / src).stat().st_mtime, newest_header):
+            continue
+        if host:
+            cmd = [hipcc(), *HOST_FLAGS, "-x", "c++", "-c", str(CSRC / src), "-o", str(obj)]
+        else:
+            cmd = [hipcc(), *HIP_FLAGS, "-x", "hip", "-c", str(CSRC / src), "-o", str(obj)]
+        jobs.append((cmd, src))
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        for f in [pool.submit(_compile, cmd, src, verbose) for cmd, src in jobs]:
+            f.result()
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *objs]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
@@ -72,4 +80,4 @@ def build(verbose: bool = False) -> Path:
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, incremental="--incremental" in sys.argv))

@@ -1118,7 +1118,18 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
                 if (row.v2) {
                     RowSample got;
                     float token_logit = 0.0f;
-                    if (kreq[(size_t)o] > 0) {
+                    // Equal logits where an unstable host algorithm of the reference decides which survive - the top_k cut
+                    // (std::partial_sort) or, under top_p < 1, the nucleus order (std::sort): the candidates cannot
+                    // say what those algorithms do with the whole row, so the row is fetched and takes the full path.
+                    bool tied = kreq[(size_t)o] > 0 && s.edge_tie != 0;
+                    if (kreq[(size_t)o] > 1 && row.v2->top_p != 1.0f)
+                        for (int j = 1; j < kreq[(size_t)o] && !tied; ++j) tied = s.top_logit[j] == s.top_logit[j - 1];
+                    if (tied) {
+                        h_logits_.ensure((size_t)n_out * n_vocab * 4);
+                        hip_check(hipMemcpy(h_logits_.as<float>() + (size_t)o * n_vocab, logits_.as<float>() + (size_t)o * n_vocab,
+                                            (size_t)n_vocab * 4, hipMemcpyDeviceToHost), "hipMemcpy");
+                    }
+                    if (kreq[(size_t)o] > 0 && !tied) {
                         got = sampling::finish_from_candidates(*row.v2, s.top_id, s.top_logit, (size_t)kreq[(size_t)o],
                                                                (size_t)n_vocab, req.rng, row.want_logprob, k, top_ids, top_lps);
                         for (int j = 0; j < kreq[(size_t)o]; ++j) if (s.top_id[j] == got.token) token_logit = s.top_logit[j];

@@ -1793,7 +1793,10 @@ __global__ __launch_bounds__(1024) void k_sample_prepare(const float * __restric
     float row_max = 0.0f;
     // selection 0 is the argmax; each later selection is the best entry
     // strictly after the previous one in (value desc, id asc) order
-    for (int sel = 0; sel < max(k, 1); ++sel) {
+    // one selection more than asked for when k > 1: an entry right behind the k-th with the k-th's value means
+    // the cut falls inside a run of equal logits, where which of them survive is the host algorithm's business
+    const int n_sel = k > 1 ? k + 1 : 1;
+    for (int sel = 0; sel < n_sel; ++sel) {
         float bv = -INFINITY;
         int bi = 0x7fffffff;
         for (int i = threadIdx.x; i < V; i += 1024) {
@@ -1814,8 +1817,9 @@ __global__ __launch_bounds__(1024) void k_sample_prepare(const float * __restric
             for (int w = 1; w < 16; ++w) if (better(s_val[w], s_idx[w], fv, fi)) { fv = s_val[w]; fi = s_idx[w]; }
             b_val = fv;
             b_idx = fi;
-            if (sel == 0) { out[row].argmax = fi; out[row].max = fv; }
+            if (sel == 0) { out[row].argmax = fi; out[row].max = fv; out[row].edge_tie = 0; }
             if (sel < k) { out[row].top_id[sel] = fi; out[row].top_logit[sel] = fv; }
+            else if (sel > 0) out[row].edge_tie = (fi != 0x7fffffff && fv == prev_v) ? 1 : 0;
         }
         __syncthreads();
         prev_v = b_val;
@@ -1896,6 +1900,7 @@ __global__ __launch_bounds__(64) void k_sample_merge(const SamplePartial * __res
     out[row].argmax = fi;
     out[row].max = fv;
     out[row].sum_exp = total;
+    out[row].edge_tie = 0;
     if (kreq && kreq[row] >= 1) { out[row].top_id[0] = fi; out[row].top_logit[0] = fv; }
 }
 

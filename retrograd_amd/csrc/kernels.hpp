@@ -296,6 +296,8 @@ struct SampleOut {          // one per output row, read back by the host
     int32_t argmax;
     float max;
     double sum_exp;         // sum exp(double(logit) - max)
+    int32_t edge_tie;       // k > 1 and the entry right behind the k-th candidate has the k-th's logit
+    int32_t pad;
     int32_t top_id[MAX_TOPK];
     float top_logit[MAX_TOPK];
 };

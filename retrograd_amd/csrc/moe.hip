@@ -421,7 +421,7 @@ __global__ __launch_bounds__(256) void k_moe_down(MoeArgs a) {
         const int nt = (NTMAX == 2 && n_e - t0 > 16) ? 2 : 1;
         __syncthreads();
         // every row of a tile lies in the expert's padded slot range
-        if (threadIdx.x < 32) rows[threadIdx.x] = qb + t0 + (threadIdx.x < 16 * nt ? threadIdx.x : 0);
+        if (threadIdx.x < 32) rows[threadIdx.x] = qb + t0 + ((int)threadIdx.x < 16 * nt ? threadIdx.x : 0);
         __syncthreads();
         StageRegs<NTMAX> regs;
         stage_load(a.x.x, a.K, rows, 0, nt, regs);

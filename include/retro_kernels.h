@@ -33,6 +33,26 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
                                 int32_t * out_argmax, float * out_max, double * out_sum_exp,
                                 int32_t * out_top_ids, float * out_top_logits);
 
+/* No counterpart in the reference. For callers that cannot allocate device
+ * memory - code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc: the greedy scan of retro_kernel_sample_prepare (every row
+ * with k = 1: argmax with the lowest id on ties, max, sum exp(double(l) - max))
+ * over DEVICE buffers the caller owns, launched on the caller's stream
+ * (a hipStream_t; NULL = the default stream), not waited for. The per-slice
+ * partial results, which retro_kernel_sample_prepare keeps in a buffer it
+ * allocates, live in a static device array of the library (64 KiB per GPU,
+ * held until the process ends); the call allocates and frees nothing.
+ * d_logits is [n_rows][n_vocab] f32; the three outputs hold n_rows entries.
+ * At most retro_kernel_sample_greedy_noalloc_max_rows() (4096) rows per call:
+ * more is refused with -1 and a message, nothing launched. Every call on one
+ * GPU shares that GPU's array: calls that overlap there (two streams, two
+ * threads) race; calls on one stream are ordered and need no clearing between
+ * them. */
+int retro_kernel_sample_greedy_noalloc(const float * d_logits, int32_t n_rows, int32_t n_vocab,
+                                       int32_t * d_out_argmax, float * d_out_max, double * d_out_sum_exp,
+                                       void * stream);
+int32_t retro_kernel_sample_greedy_noalloc_max_rows(void);
+
 /* Micro-benchmark: microseconds per launch of one tile matmul (mode 1 register
  * tiles, 2 LDS-staged tiles, 3 the same with the K-slices left to the
  * consumer) over `iters` back-to-back launches on device-only data: weight

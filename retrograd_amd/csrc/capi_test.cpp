@@ -119,6 +119,16 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
     });
 }
 
+int32_t retro_kernel_sample_greedy_noalloc_max_rows(void) { return rk::sample_static_max_rows(); }
+
+int retro_kernel_sample_greedy_noalloc(const float * d_logits, int32_t n_rows, int32_t n_vocab, int32_t * d_out_argmax,
+                                       float * d_out_max, double * d_out_sum_exp, void * stream) {
+    return guarded([&]() -> int {
+        rk::sample_greedy_static((hipStream_t)stream, d_logits, n_rows, n_vocab, d_out_argmax, d_out_max, d_out_sum_exp);
+        return 0;
+    });
+}
+
 // Times `iters` launches of one tile matmul on random device data with HIP
 // events; returns microseconds per launch through out_us.
 int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,

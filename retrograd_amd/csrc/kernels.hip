@@ -31,6 +31,7 @@
 // result holds rows 4*(l/16)+i, column l%16. Both operands always use the same
 // (lane group, slot) for the same logical k, so the hardware's internal k
 // order never matters.
+#include <mutex>
 #include "dev_common.hpp"
 
 namespace rk {
@@ -1906,12 +1907,90 @@ __global__ __launch_bounds__(64) void k_sample_merge(const SamplePartial * __res
 
 size_t sample_scratch_bytes(int n_rows) { return (size_t)std::max(n_rows, 1) * 32 * sizeof(SamplePartial); }
 
+// Slices per row of the sliced scan: as many as keep about a thousand workgroups in flight, at most 32.
+static int sample_slices_for(int n_rows) {
+    int n_slices = 1;
+    while (n_slices < 32 && n_rows * n_slices * 2 <= 1024) n_slices *= 2;
+    return n_slices;
+}
+
+// ---- the greedy scan for callers that cannot allocate ---------------------------------------------
+// The slice partials of k_sample_slices / the merge live in this file-scope device array instead of a
+// buffer the library allocates. Every GPU the library runs on holds its own copy at its own address until
+// the process ends; host code never uses the array's name as an address, only what hipGetSymbolAddress
+// returned for the device that is current.
+constexpr int SAMPLE_STATIC_MAX_ROWS = 4096;
+constexpr size_t SAMPLE_STATIC_PARTIALS = SAMPLE_STATIC_MAX_ROWS;      // rows * slices never exceeds max(rows, 512)
+static __device__ __align__(256) unsigned char scratch[SAMPLE_STATIC_PARTIALS * sizeof(SamplePartial)];
+
+int sample_static_max_rows() { return SAMPLE_STATIC_MAX_ROWS; }
+
+// The address of `scratch` on the current device, looked up once per device.
+static void * sample_static_scratch() {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex lock;
+    static void * ptr_of[MAX_DEVICES] = {};
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) throw std::runtime_error(std::string("hipGetDevice: ") + hipGetErrorString(e));
+    if (dev < 0 || dev >= MAX_DEVICES) throw std::runtime_error("sample_greedy_static: device index out of range");
+    std::lock_guard<std::mutex> hold(lock);
+    if (!ptr_of[dev]) {
+        void * ptr = nullptr;
+        e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            throw std::runtime_error(std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(e));
+        ptr_of[dev] = ptr;
+    }
+    return ptr_of[dev];
+}
+
+__global__ __launch_bounds__(64) void k_sample_merge_arrays(const SamplePartial * __restrict__ part, int n_slices,
+                                                            int32_t * __restrict__ out_argmax, float * __restrict__ out_max,
+                                                            double * __restrict__ out_sum) {
+    const int row = blockIdx.x;
+    if (threadIdx.x != 0) return;
+    const SamplePartial * p = part + (size_t)row * n_slices;
+    float fv = -INFINITY;
+    int fi = 0x7fffffff;
+    for (int s = 0; s < n_slices; ++s)
+        if (p[s].idx != 0x7fffffff && better(p[s].max, p[s].idx, fv, fi)) { fv = p[s].max; fi = p[s].idx; }
+    double total = 0.0;
+    for (int s = 0; s < n_slices; ++s)
+        if (p[s].idx != 0x7fffffff) total += p[s].sum * exp((double)p[s].max - (double)fv);
+    out_argmax[row] = fi;
+    out_max[row] = fv;
+    out_sum[row] = total;
+}
+
+// argmax (lowest id on ties), max and sum exp(double(logit) - max) per row, all pointers device memory of the
+// caller, the launches on the caller's stream; no allocation, no synchronisation. Every (row, slice) partial is
+// written by its own workgroup before the merge reads it, so the array needs no clearing between calls; two
+// calls that overlap on one GPU (different streams, or threads) race on it.
+void sample_greedy_static(hipStream_t s, const float * logits, int n_rows, int n_vocab, int32_t * out_argmax,
+                          float * out_max, double * out_sum) {
+    if (n_rows <= 0 || n_rows > SAMPLE_STATIC_MAX_ROWS)
+        throw std::runtime_error("sample_greedy_static: between 1 and " + std::to_string(SAMPLE_STATIC_MAX_ROWS)
+                                 + " rows per call (the static scratch array holds no more), got " + std::to_string(n_rows));
+    if (n_vocab <= 0) throw std::runtime_error("sample_greedy_static: the vocabulary must not be empty");
+    if (!logits || !out_argmax || !out_max || !out_sum) throw std::runtime_error("sample_greedy_static: null pointer");
+    const int n_slices = sample_slices_for(n_rows);
+    if ((size_t)n_rows * n_slices > SAMPLE_STATIC_PARTIALS)
+        throw std::runtime_error("sample_greedy_static: internal error, partials exceed the static scratch array");
+    SamplePartial * part = (SamplePartial *)sample_static_scratch();
+    const int len = ((n_vocab + n_slices - 1) / n_slices + 3) & ~3;
+    hipLaunchKernelGGL(k_sample_slices, dim3(n_rows, n_slices), dim3(256), 0, s, logits, n_vocab, len, part);
+    check_launch("sample_slices");
+    hipLaunchKernelGGL(k_sample_merge_arrays, dim3(n_rows), dim3(64), 0, s, (const SamplePartial *)part, n_slices,
+                       out_argmax, out_max, out_sum);
+    check_launch("sample_merge_arrays");
+}
+
 void sample_prepare(hipStream_t s, const float * logits, int n_rows, int n_vocab, const int32_t * k,
                     SampleOut * out, int max_k, void * scratch) {
     if (n_rows <= 0) return;
     if (max_k <= 1 && scratch && n_vocab >= 8192) {
-        int n_slices = 1;
-        while (n_slices < 32 && n_rows * n_slices * 2 <= 1024) n_slices *= 2;
+        const int n_slices = sample_slices_for(n_rows);
         const int len = ((n_vocab + n_slices - 1) / n_slices + 3) & ~3;
         hipLaunchKernelGGL(k_sample_slices, dim3(n_rows, n_slices), dim3(256), 0, s, logits, n_vocab, len, (SamplePartial *)scratch);
         check_launch("sample_slices");

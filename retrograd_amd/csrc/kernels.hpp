@@ -308,4 +308,11 @@ size_t sample_scratch_bytes(int n_rows);
 void sample_prepare(hipStream_t s, const float * logits, int n_rows, int n_vocab, const int32_t * k,
                     SampleOut * out, int max_k, void * scratch);
 
+// The greedy scan (argmax with the lowest id on ties, max, sum exp(double(logit) - max) per row) over device
+// buffers of the caller, on the caller's stream, with its slice partials in a static device array: allocates
+// nothing and waits for nothing. At most sample_static_max_rows() rows per call.
+int sample_static_max_rows();
+void sample_greedy_static(hipStream_t s, const float * logits, int n_rows, int n_vocab, int32_t * out_argmax,
+                          float * out_max, double * out_sum);
+
 }  // namespace rk

@@ -131,7 +131,7 @@ STEP_SYMBOLS = [
     "retro_grammar_gbnf", "retro_grammar_free", "retro_last_error",
 ]
 KERNEL_SYMBOLS = [
-    "retro_kernel_matmul", "retro_kernel_matmul_time", "retro_kernel_stream_time", "retro_kernel_sample_prepare", "retro_kernel_page_size", "retro_kernel_max_topk",
+    "retro_kernel_matmul", "retro_kernel_matmul_time", "retro_kernel_stream_time", "retro_kernel_sample_prepare", "retro_kernel_sample_greedy_noalloc", "retro_kernel_sample_greedy_noalloc_max_rows", "retro_kernel_page_size", "retro_kernel_max_topk",
     "retro_engine_debug_logits", "retro_engine_debug_kv", "retro_engine_debug_pack", "retro_engine_debug_pages",
     "retro_engine_debug_profile", "retro_engine_debug_profile_categories", "retro_engine_debug_profile_read",
 ]
@@ -207,6 +207,9 @@ def load_library() -> C.CDLL:
                                         _f32p, C.c_int32, _f32p]
     lib.retro_kernel_sample_prepare.argtypes = [_f32p, C.c_int32, C.c_int32, _i32p, _i32p, _f32p,
                                                 C.POINTER(C.c_double), _i32p, _f32p]
+    lib.retro_kernel_sample_greedy_noalloc.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
+                                                       C.c_void_p, C.c_void_p]
+    lib.retro_kernel_sample_greedy_noalloc_max_rows.restype = C.c_int32
     lib.retro_kernel_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,
                                              C.c_int32, C.c_int32, C.POINTER(C.c_double)]
     lib.retro_kernel_stream_time.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_double)]
@@ -863,3 +866,13 @@ def kernel_sample_prepare(logits: np.ndarray, k: Sequence[int]):
     if s != 0:
         _raise(s)
     return argmax, mx, se, ids, vals
+
+
+def kernel_sample_greedy_noalloc(d_logits: int, n_rows: int, n_vocab: int, d_argmax: int, d_max: int, d_sum_exp: int,
+                                 stream: int = 0) -> None:
+    """retro_kernel_sample_greedy_noalloc over raw device addresses (e.g. torch tensors' data_ptr()) on a HIP
+    stream handle (0 = the default stream). Launches only: the caller synchronises its stream."""
+    s = load_library().retro_kernel_sample_greedy_noalloc(d_logits, n_rows, n_vocab, d_argmax, d_max, d_sum_exp,
+                                                          stream or None)
+    if s != 0:
+        _raise(s)

@@ -48,6 +48,8 @@ class ModelShape:
     rope_freqs: bool = False         # write rope_freqs.weight: per-frequency divisors of the rotation angle as
                                      # Llama 3.1's rule gives them (1 for short wavelengths, 8 for long, a ramp between)
     rope_scaling_linear: float = 0.0 # > 0: rope.scaling.type = linear with this factor
+    norm_std: float = 0.0            # > 0: norm vectors are 1 + norm_std * N(0, 1) instead of all ones, so that a test
+                                     # can tell whether (and where) a norm weight is applied
     finer_layers: str = "all"        # layers whose ffn_down / attn_v take the finer type: "all", or "more_bits" =
                                      # the first and last eighth and every third layer between (llama.cpp's rule for Q4_K_M)
 
@@ -322,6 +324,8 @@ def write_model(path, shape: ModelShape, seed: int = 0, device: str | None = Non
 
     def vector(name, n, value=None, sd=std):
         def make():
+            if value is not None and s.norm_std > 0 and value == 1.0:
+                return (1.0 + torch.randn(n, generator=gen, device=device) * s.norm_std).float().cpu().numpy()
             if value is not None:
                 return np.full(n, value, np.float32)
             return (torch.randn(n, generator=gen, device=device) * sd).float().cpu().numpy()

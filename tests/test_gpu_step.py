@@ -333,3 +333,37 @@ def test_rope_frequency_factors_and_linear_scaling_change_the_rotation_as_in_the
     bad.write_bytes(bytes(raw))
     with pytest.raises(E.EngineError, match="not implemented"):
         E.Engine(bad, E.EngineConfig(n_ctx=256, n_seq_max=1, n_batch=64, n_ubatch=64))
+
+
+@pytest.mark.parametrize("key", ["llama", "llama-rope-freqs", "llama-linear", "qwen2", "qwen3moe"])
+def test_engine_reproduces_hugging_face_transformers_logits(tmp_path, key):
+    """The engine against tests/golden/hf_reference_logits.npz (Hugging Face transformers in float64 over the
+    dequantised weights of the same seeded file, K and V rounded to f16): every position's logits, through one
+    step of 14 rows that each prefill a prefix of the prompt into a slot of their own."""
+    import importlib.util
+    from pathlib import Path
+    here = Path(__file__).resolve().parent / "golden"
+    spec = importlib.util.spec_from_file_location("hf_reference_logits", here / "hf_reference_logits.py")
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    golden = np.load(here / "hf_reference_logits.npz")
+    shape, seed, std = mod.CASES[key]
+    path = tmp_path / (key + ".gguf")
+    synth.write_model(path, shape, seed=seed, device="cpu", std=std)
+    assert bytes(golden[key + ".sha256"]).hex() == mod.sha256(path)
+    toks = [int(t) for t in golden[key + ".tokens"]]
+    want = golden[key + ".logits"]
+    print("hf fixture", key, flush=True)
+    n = len(toks)
+    eng = E.Engine(path, E.EngineConfig(n_ctx=n * 32, n_seq_max=n, n_batch=256, n_ubatch=256))
+    out = E.StepOutput()
+    eng.step([E.StepRow(i, i, toks[:i + 1], 0, sample=True, sampling=greedy()) for i in range(n)], out)
+    got = eng.debug_logits()
+    assert_logits_close(got, want)
+    mx, mr = logit_errors(got, want)
+    assert mr <= 1e-4, (mx, mr)       # far inside the tolerance: only f32 / f16-pair rounding separates the two
+    for i, r in enumerate(out.rows()):
+        srt = np.sort(want[i])[::-1]
+        if srt[0] - srt[1] > 4e-2:
+            assert r.token == int(want[i].argmax())
+    eng.close()

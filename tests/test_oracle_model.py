@@ -155,3 +155,63 @@ def test_lora_delta_matches_dense_formula_and_rank_padding(models, tmp_path, act
     assert np.abs(got[0] - want_ad).max() < 2e-5 * max(1.0, np.abs(want_ad).max())
     assert np.abs(got[1] - want_base).max() < 2e-5 * max(1.0, np.abs(want_base).max())
     assert np.abs(want_ad - want_base).max() > 1e-3   # the adapter does something
+
+
+# ---- the forward pass against Hugging Face transformers ------------------------------------------------
+
+def _hf_golden():
+    import importlib.util
+    from pathlib import Path
+    here = Path(__file__).resolve().parent / "golden"
+    spec = importlib.util.spec_from_file_location("hf_reference_logits", here / "hf_reference_logits.py")
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)          # imports numpy and this repository's writer only; transformers stays unloaded
+    return mod, np.load(here / "hf_reference_logits.npz")
+
+
+@pytest.mark.parametrize("key", ["llama", "llama-rope-freqs", "llama-linear", "qwen2", "qwen3moe"])
+def test_forward_reproduces_hugging_face_transformers_logits(tmp_path, key):
+    """tests/golden/hf_reference_logits.npz holds logits of LlamaForCausalLM / Qwen2ForCausalLM /
+    Qwen3MoeForCausalLM (float64, K and V rounded to f16 as the cache stores them) over the dequantised
+    weights of the same seeded files. A wrong RoPE pairing or q/k row permutation, head mapping, bias,
+    q/k-norm, norm weight, frequency divisor, router rule or expert layout moves these logits by the size of
+    the logits themselves; the oracle (f32 between operations) must be within 1e-4 of their scale."""
+    mod, golden = _hf_golden()
+    shape, seed, std = mod.CASES[key]
+    path = tmp_path / (key + ".gguf")
+    synth.write_model(path, shape, seed=seed, device="cpu", std=std)
+    assert bytes(golden[key + ".sha256"]).hex() == mod.sha256(path), \
+        "the seeded model file differs from the one the fixture was made from: run tests/golden/hf_reference_logits.py again"
+    toks = golden[key + ".tokens"]
+    want = golden[key + ".logits"].astype(np.float64)
+    m = oracle.Model(path)
+    # all positions: the step returns one row per output token
+    n = len(toks)
+    got = oracle.Context(m, 1, activations="exact").step(toks, np.arange(n), np.zeros(n), np.ones(n))
+    assert got.shape == want.shape
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 1e-4 * scale, (np.abs(got - want).max(), scale)
+    assert np.abs(got - want).mean() <= 2e-5 * np.abs(want).mean()
+    assert np.array_equal(got.argmax(-1), want.argmax(-1))
+
+
+def test_lora_delta_reproduces_hugging_face_logits_with_the_adapter_merged(tmp_path):
+    """scale * alpha / r * B (A x) on q, k, v and o of a qwen2 file against the Hugging Face model whose dense
+    matrices had scale * alpha / r * B A added."""
+    mod, golden = _hf_golden()
+    L = mod.LORA
+    shape, seed, std = mod.CASES[L["case"]]
+    path, ad = tmp_path / "m.gguf", tmp_path / "a.gguf"
+    synth.write_model(path, shape, seed=seed, device="cpu", std=std)
+    synth.write_lora_adapter(ad, shape, rank=L["rank"], alpha=L["alpha"], seed=L["seed"], std_a=L["std_a"], std_b=L["std_b"])
+    assert bytes(golden[L["case"] + ".lora.sha256"]).hex() == mod.sha256(ad)
+    toks = golden[L["case"] + ".tokens"]
+    want = golden[L["case"] + ".lora.logits"].astype(np.float64)
+    base = golden[L["case"] + ".logits"].astype(np.float64)
+    m = oracle.Model(path)
+    aid = m.load_adapter(ad, L["scale"])
+    n = len(toks)
+    got = oracle.Context(m, 1, activations="exact").step(toks, np.arange(n), np.zeros(n), np.ones(n), adapter_of=np.full(n, aid))
+    # the adapter factors are stored as f16 and multiplied in f32: a little looser than the dense comparison
+    assert np.abs(got - want).max() <= 2e-4 * np.abs(want).max(), np.abs(got - want).max()
+    assert np.abs(want - base).mean() > 0.1

@@ -145,3 +145,47 @@ def test_a_group_of_completions_prefills_once_and_samples_per_member(model_path)
     assert eng.memory().cells_used == 0
     sched.close()
     eng.close()
+
+
+def test_tiny_configuration_as_specified_8_sequences_32_free_running_greedy_tokens(tmp_path):
+    """The first benchmark configuration as written: the tiny Llama file (2 layers, hidden 128, 4 / 2 heads of 32,
+    FFN 344, vocabulary 512, Q8_0 matrices, weights N(0, 0.02), norms 1, f16 KV), 8 sequences with prompt lengths
+    uniform in [8, 64], 32 greedy tokens each, free running through the product's scheduler in continuous mode
+    (no teacher forcing: each sequence is fed what the engine sampled).
+
+    N(0, 0.02) weights give logits of spread ~0.2 whose top two are often closer than the 4e-2 a logit tolerance of
+    2e-2 would call decided; the engine's actual error on this model is ~1e-5, so ids are compared wherever the
+    oracle's margin exceeds 1e-3 (a hundred times that error), and at least 90 % of the 256 tokens must be compared.
+    Where the margin is smaller the engine may break the tie either way; if it breaks it differently the rest of
+    that sequence is no longer comparable and is left out."""
+    path = tmp_path / "tiny.gguf"
+    synth.write_model(path, synth.TINY_LLAMA, seed=2024, device="cpu", std=0.02)
+    rng = np.random.default_rng(2024)
+    lens = [int(n) for n in rng.integers(8, 65, 8)]
+    prompts = [[int(t) for t in rng.integers(0, synth.TINY_LLAMA.n_vocab, n)] for n in lens]
+    print("tiny configuration, prompt lengths", lens, flush=True)
+    eng = E.Engine(path, E.EngineConfig(n_ctx=8 * 128, n_seq_max=8, n_batch=256, n_ubatch=256))
+    sched = S.Scheduler.over_engine(eng, S.SchedulerOptions(mode=S.CONTINUOUS, n_batch=256, queue_capacity=16,
+                                                            event_capacity=256, prefix_cache=False))
+    sched.initialize()
+    streams = [sched.submit(S.Request.single(p, E.SamplingParamsV2.greedy(seed=i, max_new_tokens=32)))
+               for i, p in enumerate(prompts)]
+    sched.run_until_idle()
+    model = oracle.Model(path)
+    compared = left_out = 0
+    for i, s in enumerate(streams):
+        toks, end = drain(s)
+        assert end.reason == "MaxTokens" and len(toks) == 32
+        want, margins = oracle_greedy(model, prompts[i], 32)
+        for j, (t, w, m) in enumerate(zip(toks, want, margins)):
+            if m > 1e-3:
+                assert t == w, (i, j, t, w, m)
+                compared += 1
+            elif t != w:
+                left_out += 32 - j
+                break
+    print("compared %d of 256 tokens, %d left out behind a tie" % (compared, left_out), flush=True)
+    assert compared >= 0.9 * 256, (compared, left_out)
+    assert eng.memory().cells_used == 0
+    sched.close()
+    eng.close()

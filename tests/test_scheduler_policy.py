@@ -1013,3 +1013,95 @@ def test_product_matches_the_oracle_on_random_workloads(seed):
     for key in la:
         same(key, la[key], lb[key])
     same("kv stats", hs[0].kv_stats(), hs[1].kv_stats())
+
+
+# --------------------------------------------------------------------------- the rollout configuration's plan shape
+
+def _rollout_requests(seed, n_requests=32, common=2048, lo=32, hi=512, vocab=1000):
+    rng = random.Random(seed)
+    prefix = [rng.randrange(1, vocab - 1) for _ in range(common)]
+    return [prefix + [rng.randrange(1, vocab - 1) for _ in range(rng.randint(lo, hi))] for _ in range(n_requests)]
+
+
+def _rollout_harness(kind, n_slots, n_ctx_seq=4096, vocab=1000, n_batch=512, **kw):
+    opts = dict(mode=CONTINUOUS, n_batch=n_batch, queue_capacity=64, event_capacity=4096, slow_client_timeout=0.0,
+                prefix_cache=True, min_prefix_len=8, swap_min_tokens=1 << 62)
+    opts.update(kw)
+    return Harness(kind, n_slots, n_ctx_seq, n_slots * n_ctx_seq, vocab=vocab, eos=vocab - 1,
+                   piece_table=["x"] * vocab, **opts)
+
+
+def test_rollout_shape_with_a_slot_per_member_is_32_cold_prefills_and_224_whole_slot_copies():
+    """32 prompts (2048 common tokens + 32..512 of their own), 8 members each, 256 slots, nothing pinned
+    (scheduler.rs:1094-1121, 1326-1336, 1816-1843): the prefix tree only learns a path when a member finishes, and
+    all 32 groups are admitted in one pass, so every group is a cold miss that prefills its whole prompt but the
+    last token once, copies the leader's slot to its 7 members (seq_cp(leader, member, -1, -1)) and reports
+    cached_tokens = 0. The product's plan must equal the policy oracle's call for call."""
+    prompts = _rollout_requests(5)
+    hs = {kind: _rollout_harness(kind, 256) for kind in KINDS}
+    events = {}
+    for kind, h in hs.items():
+        streams = [h.submit(p, [dict(seed=100 * i + m, max_new_tokens=3, temperature=1.0, top_k=40) for m in range(8)])
+                   for i, p in enumerate(prompts)]
+        h.run_until_idle()
+        events[kind] = [h.events(s) for s in streams]
+    la, lb = hs["product"].log(), hs["oracle"].log()
+    for key in la:
+        assert la[key] == lb[key], key
+    assert events["product"] == events["oracle"]
+    assert hs["product"].kv_stats() == hs["oracle"].kv_stats()
+    st = hs["product"].kv_stats()
+    total = sum(len(p) for p in prompts)
+    assert (st["hits"], st["misses"]) == (0, 32)
+    assert st["prompt_cells"] == total
+    # the leader prefills len - 1 tokens; the last prompt token is every member's own terminal row and is not counted
+    assert st["prefilled_cells"] == total - 32
+    copies = la["copies"]
+    assert len(copies) == 224 and all(p0 == -1 and p1 == -1 for _, _, p0, p1 in copies)
+    leaders = {}
+    for src, dst, _, _ in copies:
+        leaders.setdefault(src, []).append(dst)
+    assert len(leaders) == 32 and all(len(v) == 7 for v in leaders.values())
+    assert len({d for v in leaders.values() for d in v} | set(leaders)) == 256        # every slot used exactly once
+    for ev in events["product"]:
+        e = ends(ev)
+        assert len(e) == 8 and all(x[2] == "MaxTokens" and x[4] == 0 for x in e)      # cached_tokens = 0
+        assert all(len(tokens_of(ev, m)) == 3 for m in range(8))
+    # the common prefix was prefilled once per request: 32 x 2048 tokens and more in prefill rows
+    prefill_tokens = sum(n for step in la["steps"] for _, n, r in step if r is None)
+    assert prefill_tokens == total - 32
+
+
+def test_rollout_shape_with_fewer_slots_than_members_reuses_the_common_prefix_by_partial_copies():
+    """72 slots for 256 members, the 32 requests arriving in four waves of 8. (Queued all at once they would never hit:
+    a waiting group is admitted the moment eight slots can be freed, which evicts exactly the eight dormant nodes
+    the tree holds - the policy oracle shows hits = 0 there too.) Groups of the later waves find the common prefix
+    in the tree and take a partial copy [0, hit) from the deepest slot-bearing node (kv.rs:246-260,
+    scheduler.rs:1446-1522) into their leader, then whole-slot copies to the members; the hit is the 2048 common
+    tokens, or one more where two prompts happen to continue alike. Product and policy oracle must agree on every
+    step, copy, removal, event and counter."""
+    prompts = _rollout_requests(6)
+    hs = {kind: _rollout_harness(kind, 72) for kind in KINDS}
+    events = {kind: [] for kind in KINDS}
+    for kind, h in hs.items():
+        for w in range(4):
+            streams = [h.submit(p, [dict(seed=100 * i + m, max_new_tokens=2 + (i + m) % 3, temperature=1.0, top_k=40)
+                                    for m in range(8)]) for i, p in enumerate(prompts[8 * w:8 * w + 8])]
+            h.run_until_idle()
+            events[kind] += [h.events(s) for s in streams]
+    la, lb = hs["product"].log(), hs["oracle"].log()
+    for key in la:
+        assert la[key] == lb[key], key
+    assert events["product"] == events["oracle"]
+    assert hs["product"].kv_stats() == hs["oracle"].kv_stats()
+    st = hs["product"].kv_stats()
+    assert st["misses"] == 8 and st["hits"] == 24, st            # the first wave is cold, every later group hits
+    partial = [(s_, d, p0, p1) for s_, d, p0, p1 in la["copies"] if p0 == 0]
+    assert len(partial) == 24 and all(p1 in (2048, 2049) for _, _, _, p1 in partial), partial[:3]
+    assert len([c for c in la["copies"] if c[2] == -1 and c[3] == -1]) == 224
+    cached = [ends(ev)[0][4] for ev in events["product"]]
+    assert cached[:8] == [0] * 8 and sorted(cached[8:]) == sorted(p1 for _, _, _, p1 in partial)
+    for ev in events["product"]:
+        assert len({x[4] for x in ends(ev)}) == 1                # every member of a group reports its group's hit
+    total = sum(len(p) for p in prompts)
+    assert st["prefilled_cells"] == total - 32 - sum(cached)

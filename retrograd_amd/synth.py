@@ -231,7 +231,9 @@ def quantize_mxfp4(x: torch.Tensor) -> torch.Tensor:
     nb = K // 32
     b = x.reshape(rows, nb, 32).float()
     amax = b.abs().amax(dim=-1, keepdim=True)
-    e = torch.where(amax > 0, torch.floor(torch.log2(amax.clamp(min=1e-38))) - 2.0, torch.full_like(amax, -127.0))
+    # floor(log2(amax)) from the float's own exponent (frexp is exact; log2 differs between machines near powers of two)
+    _, ex = torch.frexp(amax.clamp(min=1e-38))
+    e = torch.where(amax > 0, ex.to(amax.dtype) - 3.0, torch.full_like(amax, -127.0))
     e = e.clamp_(-127, 127)
     s = torch.exp2(e)
     grid = torch.tensor(_FP4_VALUES, device=x.device)

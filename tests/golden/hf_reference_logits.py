@@ -49,8 +49,8 @@ CASES = {
     "llama-linear": (synth.scaled(synth.TINY_LLAMA, norm_std=0.2, rope_scaling_linear=4.0, name="hf-llama-linear"), 43, 0.08),
     "qwen2": (synth.scaled(synth.QWEN25_7B_Q8, n_layer=2, n_embd=128, n_head=4, n_head_kv=2, head_dim=32, n_ff=256,
                            n_vocab=300, norm_std=0.2, name="hf-qwen2"), 44, 0.08),
-    "qwen3moe": (synth.scaled(synth.QWEN3_30B_A3B, n_layer=2, n_embd=128, n_head=4, n_head_kv=2, head_dim=64, n_vocab=288,
-                              n_expert=8, n_expert_used=2, n_ff_exp=64, norm_std=0.2, name="hf-qwen3moe"), 45, 0.08),
+    "qwen3moe": (synth.scaled(synth.QWEN3_30B_A3B, n_layer=2, n_embd=256, n_head=4, n_head_kv=2, head_dim=64, n_vocab=288,
+                              n_expert=8, n_expert_used=2, n_ff_exp=256, norm_std=0.2, name="hf-qwen3moe"), 45, 0.08),
 }
 LORA = {"case": "qwen2", "rank": 4, "alpha": 8.0, "seed": 3, "scale": 0.5, "std_a": 0.1, "std_b": 0.1}
 PROMPT_SEED = 77

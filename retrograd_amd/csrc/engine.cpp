@@ -75,6 +75,7 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     {
         // RETRO_ACTIVATIONS=ggml: every matmul multiplies the activations as ggml's CPU path converts them
         // (Q8_K / Q8_0 codes, f16 / bf16 rounding); unset or "exact": the f32 values (as f16 hi/lo pairs).
+        if (const char * dbg = std::getenv("RETRO_MM_DEBUG")) rk::g_mm_debug = std::atoi(dbg);     // timing experiments
         const char * v = std::getenv("RETRO_ACTIVATIONS");
         const std::string mode = v ? v : "exact";
         if (mode == "ggml") ggml_activations_ = true;
@@ -88,9 +89,11 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     max_pages_ = (n_ctx_seq_ + rk::PAGE - 1) / rk::PAGE;
     // A partially filled last page per slot is the only space paging can waste.
     n_pages_ = (int)((cfg_.n_ctx + rk::PAGE - 1) / rk::PAGE + cfg_.n_seq_max);
+    // [page][kv head]: the other order (a head's pages side by side) was measured 3 % slower in the attention kernel
+    kv_strides_ = rk::kv_strides(n_pages_, hp_.n_head_kv, hp_.head_dim, false);
     const int G = hp_.n_head / hp_.n_head_kv;
     if (hp_.n_head % hp_.n_head_kv != 0 || G > 16) throw std::runtime_error("unsupported attention head grouping");
-    qt_ = std::max(1, 16 / G);
+    qt_ = rk::attention_tile_tokens(G);
 
     const size_t pool_halves = (size_t)n_pages_ * hp_.n_head_kv * rk::PAGE * hp_.head_dim;
     k_pool_.resize((size_t)hp_.n_layer);
@@ -441,7 +444,7 @@ void Engine::release_page(int32_t page) {
 
 void Engine::copy_page(int32_t src, int32_t dst) {
     for (int l = 0; l < hp_.n_layer; ++l) {
-        rk::kv_copy_page(stream_, k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(),
+        rk::kv_copy_page(stream_, k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), kv_strides_,
                          hp_.n_head_kv, hp_.head_dim, src, dst);
     }
 }
@@ -562,8 +565,8 @@ bool Engine::seq_cp(int32_t src, int32_t dst, int32_t p0, int32_t p1) {
             for (int l = 0; l < hp_.n_layer; ++l) {
                 for (int v = 0; v < 2; ++v) {
                     __half * pool = v ? v_pool_[(size_t)l].as<__half>() : k_pool_[(size_t)l].as<__half>();
-                    rk::kv_gather(stream_, pool, hp_.n_head_kv, hp_.head_dim, v != 0, cs.as<int32_t>(), (int)cells_src.size(), tmp.as<__half>());
-                    rk::kv_scatter(stream_, pool, hp_.n_head_kv, hp_.head_dim, v != 0, cd.as<int32_t>(), (int)cells_dst.size(), tmp.as<__half>());
+                    rk::kv_gather(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, cs.as<int32_t>(), (int)cells_src.size(), tmp.as<__half>());
+                    rk::kv_scatter(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, cd.as<int32_t>(), (int)cells_dst.size(), tmp.as<__half>());
                 }
             }
             hip_check(hipStreamSynchronize(stream_), "seq_cp merge");
@@ -656,7 +659,7 @@ int Engine::seq_save(int32_t slot, uint32_t flags, uint8_t * buffer, size_t n_bu
         for (int l = 0; l < hp_.n_layer; ++l) {
             for (int v = 0; v < 2; ++v) {
                 const __half * pool = v ? v_pool_[(size_t)l].as<__half>() : k_pool_[(size_t)l].as<__half>();
-                rk::kv_gather(stream_, pool, hp_.n_head_kv, hp_.head_dim, v != 0, dc.as<int32_t>(), n_pos, tmp.as<__half>());
+                rk::kv_gather(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, dc.as<int32_t>(), n_pos, tmp.as<__half>());
                 hip_check(hipMemcpyAsync(at, tmp.ptr, tmp.bytes, hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync");
                 hip_check(hipStreamSynchronize(stream_), "seq_save");
                 at += tmp.bytes;
@@ -722,7 +725,7 @@ int Engine::seq_load(int32_t slot, uint32_t flags, const uint8_t * buffer, size_
             for (int v = 0; v < 2; ++v) {
                 __half * pool = v ? v_pool_[(size_t)l].as<__half>() : k_pool_[(size_t)l].as<__half>();
                 hip_check(hipMemcpyAsync(tmp.ptr, at, tmp.bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
-                rk::kv_scatter(stream_, pool, hp_.n_head_kv, hp_.head_dim, v != 0, dc.as<int32_t>(), n_pos, tmp.as<__half>());
+                rk::kv_scatter(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, dc.as<int32_t>(), n_pos, tmp.as<__half>());
                 hip_check(hipStreamSynchronize(stream_), "seq_load");
                 at += tmp.bytes;
             }
@@ -1046,6 +1049,10 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
     int n_tiles = 0, n_items = 0;
     rk::count_attention_work(hd, (int)n_rows, qt_, hp_.n_head_kv, &n_tiles, &n_items, &pk_.split_pages);
 
+    if ((size_t)n_items * 32 > item_meta_.bytes) item_meta_.ensure((size_t)n_items * 48);      // some room to grow into
+    pk_.item_a = item_meta_.as<int4>();
+    pk_.item_b = pk_.item_a + n_items;
+
     try {
         hip_check(hipMemcpyAsync(d_stage_.ptr, h_stage_.ptr, stage_bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
         const size_t pt_pack = prof_begin(PC_PACK);
@@ -1193,7 +1200,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
 void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_rows, bool routed) {
     const HParams & h = hp_;
     const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim, F = h.n_ff;
-    rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps};
+    rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps, kv_strides_.page, kv_strides_.head};
     // The versions of a row its consumers need: the values themselves for F32 / F16 / BF16 weights, the
     // expert router and LoRA factors (`plain`); the converted row for the quantised weights.
     const bool faithful = ggml_activations_;
@@ -1737,7 +1744,7 @@ int Engine::debug_read_kv(int layer, int32_t slot, int32_t pos, int want_v, uint
     tmp.alloc(kd * 2);
     hip_check(hipMemcpy(dc.ptr, &cell, 4, hipMemcpyHostToDevice), "hipMemcpy");
     const __half * pool = want_v ? v_pool_[(size_t)layer].as<__half>() : k_pool_[(size_t)layer].as<__half>();
-    rk::kv_gather(stream_, pool, hp_.n_head_kv, hp_.head_dim, want_v != 0, dc.as<int32_t>(), 1, tmp.as<__half>());
+    rk::kv_gather(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, want_v != 0, dc.as<int32_t>(), 1, tmp.as<__half>());
     hip_check(hipStreamSynchronize(stream_), "debug_read_kv");
     hip_check(hipMemcpy(out, tmp.ptr, kd * 2, hipMemcpyDeviceToHost), "hipMemcpy");
     return 0;

@@ -204,6 +204,7 @@ private:
     int max_pages_ = 0;       // page indices per slot
     int n_pages_ = 0;         // pages in the pool
     int qt_ = 1;              // query tokens per attention tile
+    rk::KvStrides kv_strides_ {};   // layout of every KV pool
 
     hipStream_t stream_ = nullptr;
 
@@ -239,6 +240,7 @@ private:
     // the same rows after the conversion ggml's CPU matmul applies for a quantised weight
     DevBuf act_e_qx_, act_e_qsums_, act_q_qx_, act_q_qsums_, act_f_qx_, act_f_qsums_, act_o_qx_, act_o_qsums_;
     DevBuf q_half_lo_;
+    DevBuf item_meta_;        // the step's attention work items (PackBuffers::item_a, item_b), grown as needed
     DevBuf mm_ws_;            // matmul workspace: split-K partials, counters
     // mixture-of-experts scratch (allocated for MoE models only)
     DevBuf moe_logits_, moe_sel_, moe_wgt_, moe_n_, moe_off_, moe_tok_, moe_q_, moe_h_, moe_out_;

@@ -32,6 +32,7 @@
 // (lane group, slot) for the same logical k, so the hardware's internal k
 // order never matters.
 #include <mutex>
+#include <cstdlib>
 #include "dev_common.hpp"
 
 namespace rk {
@@ -1179,6 +1180,22 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
         }
         __syncthreads();
     }
+    // the work items of every (tile, kv head), from the tile and token arrays written above
+    __threadfence_block();
+    __syncthreads();
+    for (int pair = threadIdx.x; pair < carry[0] * n_kv; pair += 1024) {
+        const int tile = pair / n_kv, h = pair % n_kv;
+        const int t0 = o.tile_t0[tile], nq = o.tile_nq[tile], ns = o.tile_nsplit[tile];
+        const int kv_begin = o.tile_kv_begin[tile], pos0 = o.pos[t0], slot = o.seq[t0];
+        const int item0 = o.tile_item0[tile] + h * ns;
+        const int hi = pos0 + nq;
+        for (int sp = 0; sp < ns; ++sp) {
+            const int page_first = kv_begin / PAGE + sp * o.split_pages;
+            const int page_end = min((hi - 1) / PAGE + 1, page_first + o.split_pages);
+            o.item_a[item0 + sp] = make_int4(t0, nq, h, slot);
+            o.item_b[item0 + sp] = make_int4(pos0, kv_begin, page_first, page_end - page_first);
+        }
+    }
     if (threadIdx.x == 0) {
         const RowDesc last = rows[n_rows - 1];
         o.row_offset[n_rows] = last.tok_off + last.n;
@@ -1279,6 +1296,7 @@ struct RopeArgs {
     int n_head, n_kv, hd, rope_dim, neox;
     float eps, qscale;
     Slices from;
+    size_t page_stride, head_stride;
 };
 
 // One wave per head: lanes own element pairs.
@@ -1356,11 +1374,11 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
     const int kvh = is_k ? head - a.n_head : head - a.n_head - a.n_kv;
     const size_t page_elems = (size_t)PAGE * a.hd;
     if (is_k) {
-        __half * dst = a.k_pool + ((size_t)page * a.n_kv + kvh) * page_elems;
+        __half * dst = a.k_pool + (size_t)page * a.page_stride + (size_t)kvh * a.head_stride;
         dst[k_page_offset(a.hd, t32, i0)] = sat_half(x0);
         dst[k_page_offset(a.hd, t32, i1)] = sat_half(x1);
     } else {
-        __half * dst = a.v_pool + ((size_t)page * a.n_kv + kvh) * page_elems;
+        __half * dst = a.v_pool + (size_t)page * a.page_stride + (size_t)kvh * a.head_stride;
         dst[v_page_offset(a.hd, t32, i0)] = sat_half(x0);
         dst[v_page_offset(a.hd, t32, i1)] = sat_half(x1);
     }
@@ -1379,6 +1397,8 @@ void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, c
     a.eps = sh.eps;
     a.qscale = 1.4426950408889634f / sqrtf((float)sh.head_dim);
     a.from = from;
+    a.page_stride = sh.page_stride; a.head_stride = sh.head_stride;
+    if (sh.page_stride == 0 || sh.head_stride == 0) throw std::runtime_error("rope_store: the pool's strides are missing");
     if (from.n > 0 && from.N != (sh.n_head + 2 * sh.n_head_kv) * sh.head_dim)
         throw std::runtime_error("rope_store: the slices are not a fused q, k, v product");
     const int heads = sh.n_head + 2 * sh.n_head_kv;
@@ -1395,48 +1415,43 @@ struct AttnArgs {
     const __half * k_pool;
     const __half * v_pool;
     const int32_t * table;
-    const int32_t * tile_t0;
-    const int32_t * tile_nq;
-    const int32_t * tile_item0;
-    const int32_t * tile_nsplit;
-    const int32_t * tile_page0;
-    const int32_t * tile_kv_begin;
-    const int32_t * pos;
-    const int32_t * seq;
+    const int4 * item_a;
+    const int4 * item_b;
     float * partial;
     int n_tiles, n_items, max_pages;
     int n_head, n_kv, G;
     int split_pages;
+    size_t page_stride, head_stride;
+    int debug;
 };
 
 // ONE: every tile holds a single query token (a pure decode step).
-template <int HD, bool ONE>
+// SPLIT (at most 8 query heads per kv head): a tile holds at most 8 / G tokens. Column c < 8 carries the hi
+// half of the query of (token c / G, head c % G) and column 8 + c its lo half, so that one matrix instruction
+// multiplies both; the two score halves are added across the two lanes before the softmax, column 8 + c
+// multiplies the lo halves of the same probabilities, and the two output halves are added at the end. The
+// arithmetic of a column does not depend on ONE or on what else is in its tile, so a token's result is the
+// same bits in a decode step and in a mixed step. Without SPLIT a tile holds 16 / G tokens and the lo halves
+// take a second instruction each.
+template <int HD, bool ONE, bool SPLIT>
 __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     constexpr int KS = HD / 32;     // k-steps of QK^T
     constexpr int DT = HD / 16;     // dim tiles of PV
     const int item = blockIdx.x;
     const int lane = threadIdx.x;
     const int c = lane & 15, g = lane >> 4;
-    // tile of this item: last tile whose first item <= item
-    int lo = 0, hi = a.n_tiles - 1;
-    while (lo < hi) {
-        const int mid = (lo + hi + 1) >> 1;
-        if (a.tile_item0[mid] <= item) lo = mid; else hi = mid - 1;
-    }
-    const int tile = lo;
-    const int nsplit = a.tile_nsplit[tile];
-    const int rel = item - a.tile_item0[tile];
-    const int h = rel / nsplit, split = rel % nsplit;
-    const int t0 = a.tile_t0[tile], nq = ONE ? 1 : a.tile_nq[tile];
-    const int kv_begin = a.tile_kv_begin[tile];
-    const int slot = a.seq[t0];
-    const int qi = c / a.G, gi = c % a.G;
+    // what the packing kernel left for this item: one round trip instead of a search over the tiles
+    const int4 ia = a.item_a[item], ib = a.item_b[item];
+    const int t0 = ia.x, nq = ONE ? 1 : ia.y, h = ia.z, slot = ia.w;
+    const int kv_begin = ib.y;
+    const int cc = SPLIT ? (c & 7) : c;            // the column's (token, head) index
+    const int qi = cc / a.G, gi = cc % a.G;
     const bool col_ok = qi < nq;
+    const bool lo_col = SPLIT && c >= 8;
     const int tq = t0 + (col_ok ? qi : 0);
-    const int limit = a.pos[tq];                        // this column attends positions <= limit
-    const int kv_hi = a.pos[t0 + nq - 1] + 1;
-    const int page_first = a.tile_page0[tile] + split * a.split_pages;
-    const int page_end = min((kv_hi - 1) / PAGE + 1, page_first + a.split_pages);
+    const int limit = ib.x + (col_ok ? qi : 0);         // this column attends positions <= its own (tokens of a row are consecutive)
+    const int page_first = ib.z;
+    const int page_end = page_first + ib.w;
 
     const int QD = a.n_head * HD;
     h8 qreg[KS], qreg_lo[KS];
@@ -1444,8 +1459,8 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     for (int j = 0; j < KS; ++j) {
         if (col_ok) {
             const size_t at = (size_t)tq * QD + (size_t)(h * a.G + gi) * HD + 32 * j + 8 * g;
-            qreg[j] = load_h8(a.q + at);
-            qreg_lo[j] = load_h8(a.q_lo + at);
+            qreg[j] = load_h8((lo_col ? a.q_lo : a.q) + at);
+            qreg_lo[j] = SPLIT ? qreg[j] : load_h8(a.q_lo + at);
         } else {
             qreg[j] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
             qreg_lo[j] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
@@ -1462,7 +1477,7 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     const int my_pid = lane < n_pages ? a.table[(size_t)slot * a.max_pages + page_first + lane] : 0;
     auto load_k = [&](int idx, h8 (&kreg)[KS][2]) {
         const int pid = __builtin_amdgcn_readlane(my_pid, idx);
-        const __half * kp = a.k_pool + ((size_t)pid * a.n_kv + h) * page_elems;
+        const __half * kp = a.k_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
 #pragma unroll
         for (int j = 0; j < KS; ++j) {
             kreg[j][0] = load_h8(kp + ((j * 2 + 0) * 64 + lane) * 8);
@@ -1471,34 +1486,61 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     };
     auto load_v = [&](int idx, h8 (&vreg)[DT]) {
         const int pid = __builtin_amdgcn_readlane(my_pid, idx);
-        const __half * vp = a.v_pool + ((size_t)pid * a.n_kv + h) * page_elems;
+        const __half * vp = a.v_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
 #pragma unroll
         for (int d = 0; d < DT; ++d) vreg[d] = load_h8(vp + (d * 64 + lane) * 8);
     };
     auto attend = [&](int pi, const h8 (&kreg)[KS][2], const h8 (&vreg)[DT]) {
+        if (a.debug & 1) {       // timing experiment: the loads alone
+            h8 t = kreg[0][0];
+#pragma unroll
+            for (int j = 0; j < KS; ++j) { t += kreg[j][0]; t += kreg[j][1]; }
+#pragma unroll
+            for (int d = 0; d < DT; ++d) t += vreg[d];
+            o[0][0] += (float)t[0] + (float)t[3];
+            return;
+        }
         f4 s0 = (f4){0.f, 0.f, 0.f, 0.f}, s1 = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < KS; ++j) {
             s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg[j], s0, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg[j], s1, 0, 0, 0);
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg_lo[j], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg_lo[j], s1, 0, 0, 0);
+            if (!SPLIT) {
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg_lo[j], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg_lo[j], s1, 0, 0, 0);
+            }
+        }
+        if (SPLIT) {
+            // the hi and lo products of a query sit 8 columns apart: both lanes take the sum
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                s0[i] += __shfl_xor(s0[i], 8, 64);
+                s1[i] += __shfl_xor(s1[i], 8, 64);
+            }
         }
         // rows of s0 are tokens 4g+i, of s1 tokens 16+4g+i of this page
         const int pbase = pi * PAGE + 4 * g;
         float mx = -INFINITY;
+        // only the first and the last page of a sequence hold positions a column must not see
+        const bool edge = !ONE || pi * PAGE < kv_begin || pi * PAGE + PAGE - 1 > limit;     // (a tile of several tokens: causal mask everywhere)
+        if (edge) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int p0 = pbase + i, p1 = pbase + 16 + i;
-            if (!(col_ok && p0 >= kv_begin && p0 <= limit)) s0[i] = -INFINITY;
-            if (!(col_ok && p1 >= kv_begin && p1 <= limit)) s1[i] = -INFINITY;
-            mx = fmaxf(mx, fmaxf(s0[i], s1[i]));
+            for (int i = 0; i < 4; ++i) {
+                const int p0 = pbase + i, p1 = pbase + 16 + i;
+                if (!(col_ok && p0 >= kv_begin && p0 <= limit)) s0[i] = -INFINITY;
+                if (!(col_ok && p1 >= kv_begin && p1 <= limit)) s1[i] = -INFINITY;
+            }
+        } else if (!col_ok) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { s0[i] = -INFINITY; s1[i] = -INFINITY; }
         }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fmaxf(s0[i], s1[i]));
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m_run, mx);
         const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-        const float alpha = exp2f(m_run - m_use);       // m_run = -inf -> 0
+        const float alpha = !col_ok ? 1.0f : exp2f(m_run - m_use);       // m_run = -inf -> 0
         float psum = 0.0f;
         h8 pt, pt_lo;                                   // probabilities as f16 hi/lo pairs
 #pragma unroll
@@ -1506,40 +1548,61 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
             const float e0 = exp2f(s0[i] - m_use);
             const float e1 = exp2f(s1[i] - m_use);
             const _Float16 h0 = (_Float16)e0, h1 = (_Float16)e1;
-            pt[i] = h0;
-            pt[4 + i] = h1;
-            pt_lo[i] = (_Float16)(e0 - (float)h0);
-            pt_lo[4 + i] = (_Float16)(e1 - (float)h1);
+            const _Float16 l0 = (_Float16)(e0 - (float)h0), l1 = (_Float16)(e1 - (float)h1);
+            // SPLIT: the column of the lo query half multiplies the lo half of the same probabilities
+            pt[i] = lo_col ? l0 : h0;
+            pt[4 + i] = lo_col ? l1 : h1;
+            pt_lo[i] = l0;
+            pt_lo[4 + i] = l1;
             psum += e0 + e1;
         }
-        l_run = l_run * alpha + psum;
         m_run = m_new;
+        // the running maximum rarely moves after the first pages: then every column's factor is exactly one,
+        // and multiplying by it would change nothing
+        if (__any(alpha != 1.0f)) {
+            l_run *= alpha;
+#pragma unroll
+            for (int d = 0; d < DT; ++d)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[d][i] *= alpha;
+        }
+        l_run += psum;
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) o[d][i] *= alpha;
             o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt, o[d], 0, 0, 0);
-            o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt_lo, o[d], 0, 0, 0);
+            if (!SPLIT) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt_lo, o[d], 0, 0, 0);
         }
     };
     // V of a page loads while its scores are computed, K of the next page while
     // the page is multiplied: two K register sets, one V set
+    // The request for the next K page is never skipped (past the end it repeats the last page): a load under a
+    // condition makes the number of loads in flight differ between the paths into the arithmetic, the compiler
+    // then waits as if the fewer had been issued, and since loads return in order that wait covered the V page
+    // before the scores needed it and the next K page before the products did - nothing was in flight while a
+    // page was computed.
     if (n_pages > 0) {
         h8 kA[KS][2], kB[KS][2], v[DT];
         load_k(0, kA);
         for (int i = 0; i < n_pages; i += 2) {
             load_v(i, v);
-            if (i + 1 < n_pages) load_k(i + 1, kB);
+            load_k(min(i + 1, n_pages - 1), kB);
             attend(page_first + i, kA, v);
             if (i + 1 >= n_pages) break;
             load_v(i + 1, v);
-            if (i + 2 < n_pages) load_k(i + 2, kA);
+            load_k(min(i + 2, n_pages - 1), kA);
             attend(page_first + i + 1, kB, v);
         }
     }
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
-    if (col_ok) {
+    if (SPLIT) {
+        // the outputs against the lo halves of the probabilities join those against the hi halves
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) o[d][i] += __shfl_xor(o[d][i], 8, 64);
+    }
+    if (col_ok && !lo_col) {
         float * dst = a.partial + ((size_t)item * 16 + c) * (HD + 2);
         if (g == 0) { dst[0] = m_run; dst[1] = l_run; }
 #pragma unroll
@@ -1559,16 +1622,20 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
     if (n_items <= 0) return;
     AttnArgs a;
     a.q = q; a.q_lo = q_lo; a.k_pool = k_pool; a.v_pool = v_pool; a.table = table;
-    a.tile_t0 = pk.tile_t0; a.tile_nq = pk.tile_nq; a.tile_item0 = pk.tile_item0; a.tile_nsplit = pk.tile_nsplit;
-    a.tile_page0 = pk.tile_page0; a.tile_kv_begin = pk.tile_kv_begin; a.pos = pk.pos; a.seq = pk.seq;
+    a.item_a = pk.item_a; a.item_b = pk.item_b;
+    if (!pk.item_a || !pk.item_b) throw std::runtime_error("attention: the step's work items were not packed");
     a.partial = partial; a.n_tiles = n_tiles; a.n_items = n_items; a.max_pages = max_pages;
     a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.G = sh.n_head / sh.n_head_kv;
     a.split_pages = pk.split_pages;
+    a.page_stride = sh.page_stride; a.head_stride = sh.head_stride;
+    if (sh.page_stride == 0 || sh.head_stride == 0) throw std::runtime_error("attention: the pool's strides are missing");
+    { static const int dbg = [] { const char * v = std::getenv("RETRO_ATTN_DEBUG"); return v ? std::atoi(v) : 0; }(); a.debug = dbg; }
     if (a.G > 16 || sh.n_head % sh.n_head_kv != 0) throw std::runtime_error("attention: unsupported head grouping");
 #define ATTN_LAUNCH(HD_) \
     do { \
-        if (one_token_rows) hipLaunchKernelGGL((k_attention<HD_, true>), dim3(n_items), dim3(64), 0, s, a); \
-        else hipLaunchKernelGGL((k_attention<HD_, false>), dim3(n_items), dim3(64), 0, s, a); \
+        if (a.G <= 8 && one_token_rows) hipLaunchKernelGGL((k_attention<HD_, true, true>), dim3(n_items), dim3(64), 0, s, a); \
+        else if (a.G <= 8) hipLaunchKernelGGL((k_attention<HD_, false, true>), dim3(n_items), dim3(64), 0, s, a); \
+        else hipLaunchKernelGGL((k_attention<HD_, false, false>), dim3(n_items), dim3(64), 0, s, a); \
     } while (0)
     switch (sh.head_dim) {
         case 32:  ATTN_LAUNCH(32); break;
@@ -1721,7 +1788,7 @@ void attention_combine(hipStream_t s, const float * partial, int T, const AttnSh
 // ---------------------------------------------------------------------------
 // KV page utilities
 
-__global__ void k_kv_gather(const __half * pool, int n_kv, int hd, int is_v, const int32_t * cells, int n,
+__global__ void k_kv_gather(const __half * pool, KvStrides st, int n_kv, int hd, int is_v, const int32_t * cells, int n,
                             __half * out, int scatter) {
     const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int kd = n_kv * hd;
@@ -1730,43 +1797,45 @@ __global__ void k_kv_gather(const __half * pool, int n_kv, int hd, int is_v, con
     const int kvh = e_all / hd, e = e_all % hd;
     const int cell = cells[idx];
     const int page = cell / PAGE, t32 = cell % PAGE;
-    const size_t off = ((size_t)page * n_kv + kvh) * (size_t)PAGE * hd
+    const size_t off = (size_t)page * st.page + (size_t)kvh * st.head
         + (is_v ? v_page_offset(hd, t32, e) : k_page_offset(hd, t32, e));
     __half * cache = const_cast<__half *>(pool) + off;
     if (scatter) *cache = out[gid];
     else out[gid] = *cache;
 }
 
-void kv_gather(hipStream_t s, const __half * pool, int n_kv_heads, int head_dim, bool is_v,
+void kv_gather(hipStream_t s, const __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
                const int32_t * cells, int n, __half * out) {
     if (n <= 0) return;
     const size_t total = (size_t)n * n_kv_heads * head_dim;
-    hipLaunchKernelGGL(k_kv_gather, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, n_kv_heads,
+    hipLaunchKernelGGL(k_kv_gather, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, st, n_kv_heads,
                        head_dim, is_v ? 1 : 0, cells, n, out, 0);
     check_launch("kv_gather");
 }
 
-void kv_scatter(hipStream_t s, __half * pool, int n_kv_heads, int head_dim, bool is_v,
+void kv_scatter(hipStream_t s, __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
                 const int32_t * cells, int n, const __half * in) {
     if (n <= 0) return;
     const size_t total = (size_t)n * n_kv_heads * head_dim;
-    hipLaunchKernelGGL(k_kv_gather, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, n_kv_heads,
+    hipLaunchKernelGGL(k_kv_gather, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, st, n_kv_heads,
                        head_dim, is_v ? 1 : 0, cells, n, const_cast<__half *>(in), 1);
     check_launch("kv_scatter");
 }
 
-__global__ void k_kv_copy_page(__half * k_pool, __half * v_pool, size_t page_halves, int src, int dst) {
+__global__ void k_kv_copy_page(__half * k_pool, __half * v_pool, size_t head_halves, KvStrides st, int src, int dst) {
     const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
-    if (i >= page_halves) return;
-    *(u4 *)(k_pool + (size_t)dst * page_halves + i) = *(const u4 *)(k_pool + (size_t)src * page_halves + i);
-    *(u4 *)(v_pool + (size_t)dst * page_halves + i) = *(const u4 *)(v_pool + (size_t)src * page_halves + i);
+    if (i >= head_halves) return;
+    const size_t from = (size_t)src * st.page + (size_t)blockIdx.y * st.head + i;
+    const size_t to = (size_t)dst * st.page + (size_t)blockIdx.y * st.head + i;
+    *(u4 *)(k_pool + to) = *(const u4 *)(k_pool + from);
+    *(u4 *)(v_pool + to) = *(const u4 *)(v_pool + from);
 }
 
-void kv_copy_page(hipStream_t s, __half * k_pool, __half * v_pool, int n_kv_heads, int head_dim,
+void kv_copy_page(hipStream_t s, __half * k_pool, __half * v_pool, KvStrides st, int n_kv_heads, int head_dim,
                   int src_page, int dst_page) {
-    const size_t page_halves = (size_t)n_kv_heads * PAGE * head_dim;
-    hipLaunchKernelGGL(k_kv_copy_page, dim3((unsigned)((page_halves / 8 + 255) / 256)), dim3(256), 0, s,
-                       k_pool, v_pool, page_halves, src_page, dst_page);
+    const size_t head_halves = (size_t)PAGE * head_dim;       // one head's share of a page
+    hipLaunchKernelGGL(k_kv_copy_page, dim3((unsigned)((head_halves / 8 + 255) / 256), n_kv_heads), dim3(256), 0, s,
+                       k_pool, v_pool, head_halves, st, src_page, dst_page);
     check_launch("kv_copy_page");
 }
 

@@ -241,6 +241,10 @@ struct PackBuffers {       // device arrays, sized for n_batch tokens / rows
     int32_t * tile_kv_begin;
     int32_t * tok_tile;    // [T] tile of each token
     int4 * tok_merge;      // [T] first work item of the token's tile, its KV splits, the token's index in the tile
+    // attention work items (one wave each), everything a wave needs in two 16-byte loads:
+    int4 * item_a;         // [n_items] first flat token of the tile, tokens in the tile, kv head, slot
+    int4 * item_b;         // [n_items] position of the first token, first resident position of the slot,
+                           //           first page index of this split, pages in this split
     float * rope_cos;      // [T][rope_dim/2]
     float * rope_sin;
     int split_pages = MAX_SPLIT_PAGES;   // pages per attention work item in this step (set from count_attention_work)
@@ -251,6 +255,9 @@ void pack_step(hipStream_t s, const RowDesc * rows, int n_rows, const int32_t * 
                const TableUpdate * updates, int n_updates, int32_t * table, int max_pages,
                int qt, int n_kv_heads, const double * inv_freq, int rope_pairs, const PackBuffers & out);
 
+// Query tokens per attention tile for G query heads per kv head: 8 / G when the hi and lo halves of a query
+// share a matrix instruction (G <= 8), else 16 / G.
+inline int attention_tile_tokens(int G) { return G <= 8 ? 8 / G : (16 / G > 0 ? 16 / G : 1); }
 // Host mirror of the tile/item count (same formula as the kernel).
 void count_attention_work(const RowDesc * rows, int n_rows, int qt, int n_kv_heads,
                           int * n_tiles, int * n_items, int * split_pages);
@@ -261,7 +268,15 @@ struct AttnShape {
     int rope_dim;
     bool rope_neox;
     float eps;
+    // element strides of a KV pool between pages and between the kv heads of a page (see kv_strides)
+    size_t page_stride = 0, head_stride = 0;
 };
+// A pool holds, per page and kv head, PAGE positions x head_dim halves. head_major: [kv head][page], else [page][kv head].
+struct KvStrides { size_t page, head; };
+inline KvStrides kv_strides(int n_pages, int n_kv_heads, int head_dim, bool head_major) {
+    const size_t unit = (size_t)PAGE * head_dim;
+    return head_major ? KvStrides{unit, (size_t)n_pages * unit} : KvStrides{(size_t)n_kv_heads * unit, unit};
+}
 // qkv f32 [T][QD + 2*KD] (+ optional per-head RMSNorm weights) -> q as an f16
 // hi/lo pair [T][QD] each (rotated, pre-scaled by log2(e)/sqrt(head_dim)) and
 // the K/V pages of the layer (f16, the KV cache precision).
@@ -283,12 +298,12 @@ size_t attention_partial_floats(int n_items, int head_dim);
 
 // Gathers the K or V row of one (layer pool, cell) into natural order, and the
 // inverse; used by sequence snapshots and by tests.
-void kv_gather(hipStream_t s, const __half * pool, int n_kv_heads, int head_dim, bool is_v,
+void kv_gather(hipStream_t s, const __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
                const int32_t * cells, int n, __half * out);
-void kv_scatter(hipStream_t s, __half * pool, int n_kv_heads, int head_dim, bool is_v,
+void kv_scatter(hipStream_t s, __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
                 const int32_t * cells, int n, const __half * in);
 // Copies the first `count` positions of page src to page dst in one layer pool.
-void kv_copy_page(hipStream_t s, __half * k_pool, __half * v_pool, int n_kv_heads, int head_dim,
+void kv_copy_page(hipStream_t s, __half * k_pool, __half * v_pool, KvStrides st, int n_kv_heads, int head_dim,
                   int src_page, int dst_page);
 
 // ---- sampling -------------------------------------------------------------------

@@ -54,7 +54,15 @@ def parse_args():
                     help="after the timed steps also launch the plain copy kernel over this many MiB (known traffic, "
                          "for scaling rocprofv3 memory counters)")
     ap.add_argument("--traffic-file", default=str(ROOT / "profiles" / "k_attention_c2_hbm_traffic.txt"),
-                    help="text summary of the rocprofv3 --pmc runs; its traffic_bytes_per_launch line fills roofline.traffic")
+                    help="text summary of the rocprofv3 --pmc runs of the attention kernel; its traffic_ratio line (HBM bytes "
+                         "moved per algorithmic byte) is applied to this run's algorithmic bytes")
+    ap.add_argument("--activations", default="exact", choices=["exact", "ggml"],
+                    help="arithmetic of the measured engine: exact (f16 hi/lo activations, the default and the one the "
+                         "logit tolerances are shown on) or ggml (activations converted to Q8_K / Q8_0 as the reference's CPU path does)")
+    ap.add_argument("--kernel-steps", type=int, default=8, help="decode steps timed per kernel category after the timed region")
+    ap.add_argument("--no-scheduler-leg", action="store_true", help="skip the run of the same workload through the step scheduler")
+    ap.add_argument("--scheduler-requests", type=int, default=128)
+    ap.add_argument("--no-ggml-leg", action="store_true", help="skip the secondary measurement under the ggml arithmetic")
     return ap.parse_args()
 
 
@@ -149,10 +157,10 @@ class Workload:
         return sampled, decode_rows, cells, tokens, dt
 
 
-def read_traffic(path: str, workload: str):
-    """HBM bytes per launch of the dominant kernel as measured with rocprofv3
-    --pmc FETCH_SIZE / WRITE_SIZE (scaled by the copy kernel), from the text
-    summary of those runs; None when there is no summary for this workload."""
+def read_traffic_ratio(path: str, workload: str):
+    """HBM bytes moved per algorithmic byte by the attention kernel, as measured with rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE (scaled by the copy kernel) on a run whose own algorithmic bytes the summary
+    records beside the counters; None when there is no summary for this workload."""
     try:
         fields = {}
         for line in Path(path).read_text().splitlines():
@@ -161,50 +169,42 @@ def read_traffic(path: str, workload: str):
                 fields[k.strip()] = v.strip()
         if fields.get("workload") != workload:
             return None
-        return float(fields["traffic_bytes_per_launch"])
-    except (OSError, KeyError, ValueError):
+        if "traffic_ratio" in fields:
+            return float(fields["traffic_ratio"])
+        return float(fields["traffic_bytes_per_launch"]) / float(fields["algorithmic_bytes_per_launch"])
+    except (OSError, KeyError, ValueError, ZeroDivisionError):
         return None
 
 
-def main() -> int:
-    args = parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: the decode step has no multi-GPU path in this build (--gpus must be 1)", file=sys.stderr)
-        return 2
+def matrix_bytes_by_category(shape, synth, gw):
+    """Stored bytes of the matrices each matmul category of a decode step streams, per launch (one layer;
+    the head once per step)."""
+    cats = {"qkv": 0, "o_proj": 0, "gate_up": 0, "down": 0, "head": 0}
+    for name, n_in, n_out, t in synth.matrix_types(shape):
+        el, by = gw.BLOCK_GEOMETRY[synth.storage_type(t, n_in)]
+        b = n_in // el * by * n_out
+        if name == "output.weight":
+            cats["head"] += b
+        elif not name.startswith("blk.0."):
+            continue
+        elif "attn_q" in name or "attn_k" in name or "attn_v" in name:
+            cats["qkv"] += b
+        elif "attn_output" in name:
+            cats["o_proj"] += b
+        elif "ffn_gate" in name or "ffn_up" in name:
+            cats["gate_up"] += b
+        elif "ffn_down" in name:
+            cats["down"] += b
+    return cats
 
+
+def measure_decode(args, eng, E, synth, gw, shape, geometry, profile_kernels):
+    """Prefills the staggered initial cohort, then times args.steps decode steps (attention launches bracketed
+    by HIP events on the engine's stream), then, with profile_kernels, args.kernel_steps more decode steps with
+    events around every kernel category. Returns the measurements and the workload (still live)."""
     import torch
-
-    import oracle
-    from retrograd_amd import engine as E
-    from retrograd_amd import synth
-
-    if not torch.cuda.is_available():
-        print("bench.py needs an MI355X: no HIP device is visible", file=sys.stderr)
-        return 2
-
-    if args.shape in ("c2", "c2-q4km"):
-        shape = synth.LLAMA3_8B_Q4K if args.shape == "c2" else synth.LLAMA3_8B_Q4K_M
-        n_slots, max_new, len_lo, len_hi, n_batch = 64, 256, 128, 4096, 512
-    else:
-        shape = synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=4, n_vocab=32000, name="llama3-8b-shape-q4_k-4layers")
-        n_slots, max_new, len_lo, len_hi, n_batch = 64, 64, 64, 1024, 512
-    n_ctx = n_slots * (len_hi + max_new)
-
-    model_path = Path(args.model_dir) / ("retro-bench-%s-seed%d.gguf" % (shape.name, args.seed))
-    if not model_path.exists():
-        t0 = time.perf_counter()
-        tmp = model_path.with_suffix(".tmp")
-        synth.write_model(tmp, shape, seed=args.seed, device="cuda")
-        os.replace(tmp, model_path)
-        print("[bench] wrote %s (%.1f GB) in %.1fs" % (model_path, model_path.stat().st_size / 1e9, time.perf_counter() - t0), file=sys.stderr, flush=True)
-    torch.cuda.empty_cache()
-
-    t0 = time.perf_counter()
-    eng = E.Engine(model_path, E.EngineConfig(n_ctx=n_ctx, n_seq_max=n_slots, n_batch=n_batch, n_ubatch=n_batch))
-    print("[bench] engine ready in %.1fs" % (time.perf_counter() - t0), file=sys.stderr, flush=True)
-
+    n_slots, max_new, len_lo, len_hi, n_batch = geometry
     wl = Workload(eng, E, n_slots, n_batch, shape.n_vocab, max_new, len_lo, len_hi, args.seed)
-    # initial cohort, staggered through its generation budget
     stagger = np.random.default_rng(args.seed + 1).integers(1, max_new + 1, n_slots)
     for slot in range(n_slots):
         wl.new_request(slot, budget=int(stagger[slot]))
@@ -217,56 +217,187 @@ def main() -> int:
             print("[bench] initial prefill: %d steps" % n_pre, file=sys.stderr, flush=True)
     print("[bench] initial prefill of %d sequences: %d steps, %.1fs" % (n_slots, n_pre, time.perf_counter() - t0), file=sys.stderr, flush=True)
 
-    def run_decode_steps(n, timed):
-        """n decode steps; prompts of requests admitted on the way are prefilled in
-        their own steps in between. Returns the totals of the decode steps and of
-        the prefill steps."""
+    def run_decode_steps(n, level):
+        """n decode steps; prompts of requests admitted on the way are prefilled in their own steps in between
+        (events off). Returns the totals of the decode steps and of the prefill steps."""
         dec = [0, 0, 0, 0, 0.0]
         pre = [0, 0.0, 0]
         done = 0
         while done < n:
             if wl.prefill_pending():
-                if timed:
-                    eng.profile(0)
+                eng.profile(0)
                 r = wl.step("prefill")
                 pre[0] += r[3]
                 pre[1] += r[4]
                 pre[2] += 1
                 continue
-            if timed:
-                eng.profile(2 if args.profile_all else 1)
+            eng.profile(level)
             r = wl.step("decode")
             for i in range(5):
                 dec[i] += r[i]
             done += 1
+        eng.profile(0)
         return dec, pre
 
-    run_decode_steps(args.warmup, False)
+    run_decode_steps(args.warmup, 0)
     eng.profile_read(reset=True)
+    finished0 = wl.finished
     torch.cuda.synchronize()
     wall0 = time.perf_counter()
-    (sampled, decode_rows, cells, tokens, elapsed), (pre_tokens, pre_seconds, pre_steps) = run_decode_steps(args.steps, True)
+    dec, pre = run_decode_steps(args.steps, 2 if args.profile_all else 1)
     torch.cuda.synchronize()
     wall = time.perf_counter() - wall0
     prof = eng.profile_read(reset=True)
-    eng.profile(0)
+    out = {"dec": dec, "pre": pre, "wall": wall, "prof": prof, "finished": wl.finished - finished0, "kernels": None}
+    if profile_kernels and args.kernel_steps > 0:
+        kdec, _ = run_decode_steps(args.kernel_steps, 2)
+        out["kernels"] = (eng.profile_read(reset=True), kdec, args.kernel_steps)
+    return out, wl
+
+
+def scheduler_leg(args, eng, E, shape, geometry):
+    """The same workload through the product's step scheduler in continuous mode (the policy of
+    crates/retrograd-infer/src/scheduler.rs:933-1404: FIFO admission with cell reservations, decode rows first,
+    prefill chunks of new requests inside the same steps): every request is submitted at once, the scheduler
+    admits them as slots free up, and sampled tokens are counted over the whole run, prefill included."""
+    import torch
+    from retrograd_amd import scheduler as S
+    n_slots, max_new, len_lo, len_hi, n_batch = geometry
+    rng = np.random.default_rng(args.seed + 7)
+    n_req = args.scheduler_requests
+    sched = S.Scheduler.over_engine(eng, S.SchedulerOptions(mode=S.CONTINUOUS, n_batch=n_batch, queue_capacity=n_req,
+                                                            event_capacity=max_new + 8, slow_client_timeout=60.0,
+                                                            prefix_cache=True, min_prefix_len=8, swap_min_tokens=1 << 62))
+    sched.initialize()
+    prompts = []
+    for _ in range(n_req):
+        n = int(round(math.exp(rng.uniform(math.log(len_lo), math.log(len_hi)))))
+        prompts.append(rng.integers(0, shape.n_vocab, min(max(n, len_lo), len_hi)).astype(np.int32))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    streams = [sched.submit(S.Request.single([int(t) for t in p], E.SamplingParamsV2.greedy(seed=i, max_new_tokens=max_new)))
+               for i, p in enumerate(prompts)]
+    steps = 0
+    while not sched.is_idle():
+        sched.pump()
+        steps += 1
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    sampled = 0
+    for s_ in streams:
+        events = s_.drain()
+        sampled += sum(1 for e in events if e.type == "Token")
+        if any(e.type == "Error" for e in events):
+            raise RuntimeError("a scheduled request failed")
+    kv = sched.kv_stats()
+    sched.close()
+    return {
+        "tok_s": round(sampled / seconds, 1), "seconds": round(seconds, 3), "steps": steps, "requests": n_req,
+        "sampled_tokens": sampled, "prompt_tokens": int(sum(len(p) for p in prompts)),
+        "mode": "continuous: decode rows and prefill chunks share steps of at most %d tokens; prefill time included" % n_batch,
+        "kv_stats": {"hits": kv.hits, "misses": kv.misses, "prompt_cells": kv.prompt_cells, "prefilled_cells": kv.prefilled_cells,
+                     "evictions": kv.evictions},
+    }
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the decode step has no multi-GPU path in this build (--gpus must be 1)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    import oracle
+    from retrograd_amd import engine as E
+    from retrograd_amd import gguf_writer as gw
+    from retrograd_amd import synth
+
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X: no HIP device is visible", file=sys.stderr)
+        return 2
+
+    if args.shape in ("c2", "c2-q4km"):
+        shape = synth.LLAMA3_8B_Q4K if args.shape == "c2" else synth.LLAMA3_8B_Q4K_M
+        geometry = (64, 256, 128, 4096, 512)
+    else:
+        shape = synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=4, n_vocab=32000, name="llama3-8b-shape-q4_k-4layers")
+        geometry = (64, 64, 64, 1024, 512)
+    n_slots, max_new, len_lo, len_hi, n_batch = geometry
+    n_ctx = n_slots * (len_hi + max_new)
+
+    model_path = Path(args.model_dir) / ("retro-bench-%s-seed%d.gguf" % (shape.name, args.seed))
+    if not model_path.exists():
+        t0 = time.perf_counter()
+        tmp = model_path.with_suffix(".tmp")
+        synth.write_model(tmp, shape, seed=args.seed, device="cuda")
+        os.replace(tmp, model_path)
+        print("[bench] wrote %s (%.1f GB) in %.1fs" % (model_path, model_path.stat().st_size / 1e9, time.perf_counter() - t0), file=sys.stderr, flush=True)
+    torch.cuda.empty_cache()
+
+    def new_engine(activations):
+        os.environ["RETRO_ACTIVATIONS"] = activations
+        t0 = time.perf_counter()
+        eng = E.Engine(model_path, E.EngineConfig(n_ctx=n_ctx, n_seq_max=n_slots, n_batch=n_batch, n_ubatch=n_batch))
+        print("[bench] engine (%s arithmetic) ready in %.1fs" % (activations, time.perf_counter() - t0), file=sys.stderr, flush=True)
+        return eng
+
+    eng = new_engine(args.activations)
+    m, wl = measure_decode(args, eng, E, synth, gw, shape, geometry, profile_kernels=True)
+    sampled, decode_rows, cells, tokens, elapsed = m["dec"]
+    pre_tokens, pre_seconds, pre_steps = m["pre"]
+    prof = m["prof"]
 
     ms_per_step = elapsed / args.steps * 1e3
     tok_s = sampled / elapsed
 
-    # ---- roofline of the dominant kernel (paged attention, one launch per layer)
+    # ---- roofline of the attention kernel (the largest single launch: one per layer), over the timed region
     hp = shape
     kv_bytes_per_cell_layer = 2 * hp.n_head_kv * hp.head_dim * 2
     attn_ms, attn_launches = prof["attention"]
     algo_bytes_per_launch = kv_bytes_per_cell_layer * cells / args.steps
     attn_avg_s = attn_ms / max(attn_launches, 1) * 1e-3
     attn_gbs = algo_bytes_per_launch / attn_avg_s / 1e9 if attn_avg_s > 0 else 0.0
+    ratio = read_traffic_ratio(args.traffic_file, shape.name)
 
     # ---- whole-step roofline (north star): weights once + KV of every attended cell
     w_bytes = synth.streamed_weight_bytes(hp)       # every dense matrix once, at its stored type
     step_bytes = w_bytes + hp.n_layer * kv_bytes_per_cell_layer * (cells / args.steps)
     step_roof_tok_s = (sampled / args.steps) / (step_bytes / (HBM_PEAK_GBS * 1e9))
 
+    # ---- every kernel family of the step, from the profiled steps after the timed region
+    kernels = []
+    if m["kernels"]:
+        kprof, kdec, ksteps = m["kernels"]
+        kcells = kdec[2] / ksteps
+        cats = matrix_bytes_by_category(hp, synth, gw)
+        mm_name = "k_mm5_q4k" if args.shape == "c2" else "k_mm5_q4k / k_mm2_q6k"
+        fam_ms = fam_bytes = fam_launches = 0.0
+        rows = [("k_attention<128, true, true>", "attention", kv_bytes_per_cell_layer * kcells)]
+        rows += [("%s (%s)" % (mm_name, c), c, cats[c]) for c in ("qkv", "o_proj", "gate_up", "down")]
+        for name, cat, by in rows:
+            ms, n = kprof[cat]
+            if n == 0:
+                continue
+            us = ms / n * 1e3
+            kernels.append({"kernel": name, "launches_per_step": round(n / ksteps, 2), "algorithmic_bytes_per_launch": round(by),
+                            "avg_launch_us": round(us, 2), "ms_per_step": round(ms / ksteps, 3),
+                            "achieved_GBs": round(by / (us * 1e-6) / 1e9, 1), "frac": round(by / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+            if cat != "attention":
+                fam_ms += ms; fam_bytes += by * n; fam_launches += n
+        if fam_launches:
+            us = fam_ms / fam_launches * 1e3
+            kernels.append({"kernel": "%s, the layer matmuls together (furthest from its roof)" % mm_name,
+                            "launches_per_step": round(fam_launches / ksteps, 2),
+                            "algorithmic_bytes_per_launch": round(fam_bytes / fam_launches), "avg_launch_us": round(us, 2),
+                            "ms_per_step": round(fam_ms / ksteps, 3),
+                            "achieved_GBs": round(fam_bytes / fam_launches / (us * 1e-6) / 1e9, 1),
+                            "frac": round(fam_bytes / fam_launches / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)})
+        others = {c: round(kprof[c][0] / ksteps, 3) for c in ("norm", "rope", "combine", "head", "sample", "pack", "embed") if kprof[c][1]}
+        kernels.append({"kernel": "latency-bound kernels, ms per step (events around each launch, which adds a few us to each)", **others})
+
+    arithmetic = ("f16 hi/lo activations (about 22 bits)" if args.activations == "exact" else
+                  "activations converted to Q8_K blocks as the reference's CPU path does (ggml arithmetic)")
     result = {
         "metric": ("decode tok/s, 8B-shape Q4_K ragged batch 64; % of HBM roofline" if args.shape != "c2-q4km" else
                    "decode tok/s, 8B shape with the Q4_K_M type mix (Q6_K output, ffn_down and attn_v on half the layers), "
@@ -280,29 +411,32 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("q4_k" if args.shape != "c2-q4km" else "q4_k / q6_k") + " weights x f16 hi/lo activations, f32 accumulate, f16 KV",
+        "dtype": ("q4_k" if args.shape != "c2-q4km" else "q4_k / q6_k") + " weights x " + arithmetic + ", f32 accumulate, f16 KV",
         "data": "synthetic",
         "config": {
             "workload": "configs[1]: %s, %d live sequences, prompts log-uniform [%d,%d], greedy, %d new tokens, continuous batching"
                         % (shape.name, n_slots, len_lo, len_hi, max_new),
             "n_batch": n_batch,
+            "activations": args.activations,
             "mean_decode_rows_per_step": round(decode_rows / args.steps, 2),
             "mean_tokens_per_step": round(tokens / args.steps, 2),
             "mean_kv_cells_attended_per_step": round(cells / args.steps, 1),
-            "requests_finished_in_window": wl.finished,
+            "requests_finished_in_window": m["finished"],
             "timing": "sum of the %d decode steps' own durations; prefill of admitted requests runs between them, untimed" % args.steps,
             "prefill_between_decode_steps": {"steps": pre_steps, "tokens": pre_tokens,
                                              "tok_s": round(pre_tokens / pre_seconds, 1) if pre_seconds > 0 else None},
-            "mixed_tok_s_including_prefill_time": round(sampled / wall, 1),
+            "mixed_tok_s_including_prefill_time": round(sampled / m["wall"], 1),
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "k_attention<128, true> (paged split-KV attention of a decode step, one launch per layer)",
+            "kernel": "k_attention<128, true, true> (paged split-KV attention of a decode step, one launch per layer: the largest "
+                      "single launch; the kernel furthest from its roof is the matmul family, see kernels[] and step)",
             "achieved": round(attn_gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(attn_gbs / HBM_PEAK_GBS, 4),
-            "traffic": read_traffic(args.traffic_file, shape.name),
+            "traffic": round(ratio * algo_bytes_per_launch) if ratio else None,
+            "traffic_ratio": ratio,
             "algorithmic_bytes_per_launch": round(algo_bytes_per_launch),
             "avg_launch_us": round(attn_avg_s * 1e6, 2),
             "launches_timed": attn_launches,
@@ -311,6 +445,7 @@ def main() -> int:
                 "roofline_tok_s": round(step_roof_tok_s, 1),
                 "frac": round(tok_s / step_roof_tok_s, 4),
             },
+            "kernels": kernels,
         },
     }
     if args.stream_probe > 0:
@@ -321,22 +456,45 @@ def main() -> int:
             "%s=%.3f" % (k, v[0] / args.steps) for k, v in prof.items()), file=sys.stderr, flush=True)
 
     if not args.no_cpu_baseline:
-        result["cpu_baseline"], result["parity_full_size"] = cpu_baseline(eng, E, oracle, wl, model_path, args.cpu_rows)
+        result["cpu_baseline"], result["parity_full_size"] = cpu_baseline(eng, E, oracle, wl, model_path, args.cpu_rows, args.activations)
     else:
         result["cpu_baseline"] = None
 
+    if not args.no_scheduler_leg:
+        for s_ in wl.seqs:                         # the hand-composed cohort gives its slots back
+            if s_ is not None:
+                eng.seq_rm(s_.slot)
+                eng.request_free(s_.request)
+        result["config"]["through_the_step_scheduler"] = scheduler_leg(args, eng, E, shape, geometry)
     eng.close()
+    del eng
+
+    if not args.no_ggml_leg and args.activations == "exact":
+        # secondary figure: the same timed loop with the activations converted as the reference's CPU path converts them
+        eng = new_engine("ggml")
+        m2, wl2 = measure_decode(args, eng, E, synth, gw, shape, geometry, profile_kernels=False)
+        s2, _, c2, _, e2 = m2["dec"]
+        b2 = w_bytes + hp.n_layer * kv_bytes_per_cell_layer * (c2 / args.steps)
+        leg = {"value": round(s2 / e2, 1), "unit": "tok/s", "ms_per_step": round(e2 / args.steps * 1e3, 4),
+               "step_frac_of_hbm_roofline": round((s2 / e2) / ((s2 / args.steps) / (b2 / (HBM_PEAK_GBS * 1e9))), 4),
+               "arithmetic": "RETRO_ACTIVATIONS=ggml: Q8_K / Q8_0 activation conversion before every quantised matmul"}
+        if not args.no_cpu_baseline:
+            _, leg["parity_full_size_against_the_oracle_in_the_same_arithmetic"] = cpu_baseline(eng, E, oracle, wl2, model_path, args.cpu_rows, "ggml", time_it=False)
+        result["ggml_arithmetic"] = leg
+        eng.close()
+    os.environ["RETRO_ACTIVATIONS"] = "exact"
+
     print(json.dumps(result), flush=True)
     return 0
 
 
-def cpu_baseline(eng, E, oracle, wl, model_path, n_rows):
+def cpu_baseline(eng, E, oracle, wl, model_path, n_rows, activations="exact", time_it=True):
     """Times the CPU oracle on one decode step over the first n_rows live
     sequences of the same workload (their KV imported from the engine's own
     snapshots), and compares its logits with the engine's for the same rows."""
     live = [s for s in wl.seqs if s is not None and s.last_token is not None][:n_rows]
     model = oracle.Model(model_path)
-    ctx = oracle.Context(model, max(s.slot for s in live) + 1)
+    ctx = oracle.Context(model, max(s.slot for s in live) + 1, activations=activations)
     t0 = time.perf_counter()
     for s in live:
         ctx.import_snapshot(s.slot, eng.seq_save(s.slot))
@@ -348,7 +506,7 @@ def cpu_baseline(eng, E, oracle, wl, model_path, n_rows):
     # a few more decode steps of the same rows (fed with the oracle's own greedy tokens), for about 10 s of CPU work
     cpu_steps = 1
     feed = [int(r.argmax()) for r in want]
-    while cpu_s < 8.0 and cpu_steps < 8:
+    while time_it and cpu_s < 8.0 and cpu_steps < 8:
         t0 = time.perf_counter()
         more = ctx.step_rows([(s.slot, s.pos + cpu_steps, [feed[i]], True) for i, s in enumerate(live)])
         cpu_s += time.perf_counter() - t0
@@ -368,6 +526,11 @@ def cpu_baseline(eng, E, oracle, wl, model_path, n_rows):
         "mean_abs_relative_error": float(err.mean() / np.abs(want).mean()),
         "greedy_tokens_equal": int(sum(same)),
         "greedy_tokens_equal_where_margin_exceeds_tolerance": "%d/%d" % (sum(s for s, d in zip(same, decided) if d), sum(decided)),
+        "against": "the CPU oracle in the %s arithmetic on the same KV and tokens. The oracle's forward pass is pinned against "
+                   "Hugging Face transformers logits (tests/golden/hf_reference_logits.npz); the reference's own ggml build is "
+                   "absent, so float-level parity with it is unpinned. The reference's CPU path converts activations to Q8_K "
+                   "before every Q4_K matmul, which by the oracle moves logits 3.5-6 %% (mean-abs relative) away from the exact "
+                   "product; the 2e-2 / 1e-3 tolerances are shown on the exact arithmetic." % activations,
     }
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     base = {

@@ -98,13 +98,14 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     const size_t pool_halves = (size_t)n_pages_ * hp_.n_head_kv * rk::PAGE * hp_.head_dim;
     k_pool_.resize((size_t)hp_.n_layer);
     v_pool_.resize((size_t)hp_.n_layer);
+    const size_t pool_bytes = (pool_halves * 2 + 255) / 256 * 256;
+    kv_slab_.alloc(pool_bytes * 2 * (size_t)hp_.n_layer);
+    // Pages must never hold non-finite bit patterns: a masked score times a
+    // NaN value would poison the output.
+    hip_check(hipMemsetAsync(kv_slab_.ptr, 0, kv_slab_.bytes, stream_), "hipMemsetAsync");
     for (int l = 0; l < hp_.n_layer; ++l) {
-        k_pool_[(size_t)l].alloc(pool_halves * 2);
-        v_pool_[(size_t)l].alloc(pool_halves * 2);
-        // Pages must never hold non-finite bit patterns: a masked score times a
-        // NaN value would poison the output.
-        hip_check(hipMemsetAsync(k_pool_[(size_t)l].ptr, 0, pool_halves * 2, stream_), "hipMemsetAsync");
-        hip_check(hipMemsetAsync(v_pool_[(size_t)l].ptr, 0, pool_halves * 2, stream_), "hipMemsetAsync");
+        k_pool_[(size_t)l] = PoolView{(uint8_t *)kv_slab_.ptr + pool_bytes * (2 * (size_t)l), pool_halves * 2};
+        v_pool_[(size_t)l] = PoolView{(uint8_t *)kv_slab_.ptr + pool_bytes * (2 * (size_t)l + 1), pool_halves * 2};
     }
     table_.alloc((size_t)cfg_.n_seq_max * max_pages_ * sizeof(int32_t));
     hip_check(hipMemsetAsync(table_.ptr, 0xff, table_.bytes, stream_), "hipMemsetAsync");

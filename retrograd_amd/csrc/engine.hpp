@@ -216,7 +216,15 @@ private:
     DevBuf inv_freq_;         // double[rope_dim/2]
 
     // KV
-    std::vector<DevBuf> k_pool_, v_pool_;   // per layer
+    // One allocation for every layer's K and V pool (one large mapping instead of 2 x n_layer medium ones);
+    // the per-layer pools are views into it.
+    struct PoolView {
+        void * ptr = nullptr;
+        size_t bytes = 0;
+        template <typename T> T * as() const { return (T *)ptr; }
+    };
+    DevBuf kv_slab_;
+    std::vector<PoolView> k_pool_, v_pool_;   // per layer
     DevBuf table_;                          // int32 [n_seq_max][max_pages]
     std::vector<Slot> slots_;
     std::vector<int32_t> page_ref_;

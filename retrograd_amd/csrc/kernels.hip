@@ -1372,7 +1372,6 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
     const int cell = a.cell[t];
     const int page = cell / PAGE, t32 = cell % PAGE;
     const int kvh = is_k ? head - a.n_head : head - a.n_head - a.n_kv;
-    const size_t page_elems = (size_t)PAGE * a.hd;
     if (is_k) {
         __half * dst = a.k_pool + (size_t)page * a.page_stride + (size_t)kvh * a.head_stride;
         dst[k_page_offset(a.hd, t32, i0)] = sat_half(x0);
@@ -1470,7 +1469,6 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
 #pragma unroll
     for (int d = 0; d < DT; ++d) o[d] = (f4){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.0f;
-    const size_t page_elems = (size_t)PAGE * HD;
 
     // page ids of this split, one per lane
     const int n_pages = page_end - page_first;

@@ -1,0 +1,62 @@
+"""k_mm5_q4k keeps its prefetched weight sets in v[232:255], registers the compiler is told not to allocate
+(amdgpu_num_vgpr(232)); the loads into them are issued from inline assembly the compiler cannot see. If the
+compiler ever used one of those registers for a value of its own - the attribute is a request it may exceed under
+register pressure - a load in flight would overwrite that value, or the value the loaded weights, and the kernel
+would read through garbage addresses. This test compiles the file to gfx950 assembly (no GPU needed) and checks
+that, in every instantiation of the kernel, nothing but the kernel's own global_load_dwordx4 writes v232..v255
+and that the kernel does not spill."""
+import re
+import subprocess
+from pathlib import Path
+
+import pytest
+
+from retrograd_amd import build as B
+
+ROOT = Path(__file__).resolve().parent.parent
+RESERVED = range(232, 256)
+
+
+def _written_registers(line):
+    """Destination VGPRs of one instruction line (first operand)."""
+    m = re.match(r"\s*(\S+)\s+(?:v\[(\d+):(\d+)\]|v(\d+)\b)", line)
+    if not m:
+        return None, []
+    op = m.group(1)
+    if m.group(2):
+        return op, list(range(int(m.group(2)), int(m.group(3)) + 1))
+    return op, [int(m.group(4))]
+
+
+def test_the_compiler_never_writes_the_registers_the_weight_prefetch_owns(tmp_path):
+    out = tmp_path / "mm_lds.s"
+    cmd = [B.hipcc(), *[f for f in B.HIP_FLAGS if f != "-fPIC"], "-x", "hip", "-S", "--cuda-device-only",
+           str(B.CSRC / "mm_lds.hip"), "-o", str(out)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    text = out.read_text().split("\n")
+    starts = [i for i, l in enumerate(text) if re.match(r"^_ZN2rk9k_mm5_q4kILb[01]EEEvNS_6MMArgsE:", l)]
+    assert len(starts) == 2, "both instantiations of k_mm5_q4k are expected in the assembly"
+    for s in starts:
+        end = next(i for i in range(s, len(text)) if text[i].startswith(".Lfunc_end"))
+        body = text[s:end]
+        stores_from_reserved = 0
+        for line in body:
+            code = line.split(";")[0]
+            if not code.strip() or code.strip().endswith(":") or code.strip().startswith("."):
+                continue
+            assert "scratch_" not in code, "k_mm5_q4k spills: " + code.strip()
+            op, regs = _written_registers(code)
+            if op is None or op.startswith(("global_store", "buffer_store", "ds_write", "ds_store", "s_", "v_cmp")):
+                continue            # first operand of a store / compare is not a VGPR destination
+            hit = [r for r in regs if r in RESERVED]
+            if hit:
+                assert op == "global_load_dwordx4", "the compiler writes a reserved register: " + code.strip()
+                stores_from_reserved += 1
+        assert stores_from_reserved >= 6, "the inline-assembly weight loads are expected in the kernel"
+        meta_end = next(i for i in range(end, len(text)) if ".end_amdhsa_kernel" in text[i])
+        meta = "\n".join(text[end:meta_end])
+        m = re.search(r"\.amdhsa_next_free_vgpr (\d+)", meta)
+        assert m and int(m.group(1)) == 256
+        m = re.search(r"\.amdhsa_private_segment_fixed_size (\d+)", meta)
+        assert m and int(m.group(1)) == 0

@@ -54,8 +54,7 @@ def test_the_compiler_never_writes_the_registers_the_weight_prefetch_owns(tmp_pa
                 assert op == "global_load_dwordx4", "the compiler writes a reserved register: " + code.strip()
                 stores_from_reserved += 1
         assert stores_from_reserved >= 6, "the inline-assembly weight loads are expected in the kernel"
-        meta_end = next(i for i in range(end, len(text)) if ".end_amdhsa_kernel" in text[i])
-        meta = "\n".join(text[end:meta_end])
+        meta = "\n".join(body)          # the kernel descriptor directives sit between the code and .Lfunc_end
         m = re.search(r"\.amdhsa_next_free_vgpr (\d+)", meta)
         assert m and int(m.group(1)) == 256
         m = re.search(r"\.amdhsa_private_segment_fixed_size (\d+)", meta)

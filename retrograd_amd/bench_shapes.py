@@ -1,0 +1,134 @@
+"""Decode-step measurements of the other full-shape configurations of the
+benchmark set on one MI355X (secondary figures; bench.py at the repository root
+measures the headline):
+
+    python -m retrograd_amd.bench_shapes c4        # multi-LoRA decode, Qwen2.5-7B shape, Q8_0 base
+    python -m retrograd_amd.bench_shapes c5        # mixture of experts, Qwen3-30B-A3B shape, MXFP4 experts
+    python -m retrograd_amd.bench_shapes c5-q4km   # the same shape with the type mix of a Q4_K_M file
+
+c4: 28 layers, hidden 3584, 28 / 4 heads, FFN 18944, vocabulary 152064, eight
+rank-16 F16 adapters on q/k/v/o (A ~ N(0, 0.02), B ~ N(0, 0.01)), 64 sequences
+each routed at random to one adapter or to the base, prompts uniform in
+[256, 2048], 128 greedy tokens.
+c5: 48 layers, hidden 2048, 32 / 4 heads, 128 experts of width 768 with top-8
+routing, attention in Q8_0, experts in MXFP4, 128 sequences with prompts
+log-uniform in [64, 2048], 128 greedy tokens.
+
+Weights are synthetic (seeded), prompts random token ids. Prefill runs first,
+untimed for the decode figure; then `--new` decode steps over all sequences: the
+first part is timed as it is, the last `--profiled` steps run with an event pair
+around every kernel category (which slows them a little) for the breakdown.
+Prints one JSON line."""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("config", choices=["c4", "c5", "c5-q4km"])
+    ap.add_argument("--new", type=int, default=128)
+    ap.add_argument("--profiled", type=int, default=32)
+    ap.add_argument("--model-dir", default=os.environ.get("RETRO_BENCH_MODEL_DIR", "/dev/shm"))
+    ap.add_argument("--seed", type=int, default=1234)
+    args = ap.parse_args()
+
+    import torch
+
+    from . import engine as E
+    from . import gguf_writer as gw
+    from . import synth
+
+    if not torch.cuda.is_available():
+        print("bench_shapes needs an MI355X: no HIP device is visible", file=sys.stderr)
+        return 2
+    rng = np.random.default_rng(args.seed)
+    if args.config == "c4":
+        shape, n_seq = synth.QWEN25_7B_Q8, 64
+        lengths = rng.integers(256, 2048 + 1, n_seq)
+    else:
+        shape, n_seq = synth.QWEN3_30B_A3B, 128
+        if args.config == "c5-q4km":
+            shape = synth.scaled(shape, matrix_type=gw.GGML_Q4_K, v_type=gw.GGML_Q6_K, output_type=gw.GGML_Q6_K,
+                                 expert_type=gw.GGML_Q4_K, expert_down_type=gw.GGML_Q6_K, finer_layers="more_bits",
+                                 name="qwen3-30b-a3b-shape-q4_k_m")
+        else:
+            shape = synth.scaled(shape, expert_type=gw.GGML_MXFP4)
+        lengths = np.exp(rng.uniform(np.log(64), np.log(2048), n_seq)).astype(np.int64)
+    lengths = [int(n) for n in lengths]
+
+    model_path = Path(args.model_dir) / ("retro-bench-%s-seed%d.gguf" % (shape.name, args.seed))
+    if not model_path.exists():
+        tmp = model_path.with_suffix(".tmp")
+        synth.write_model(tmp, shape, seed=args.seed, device="cuda")
+        os.replace(tmp, model_path)
+    torch.cuda.empty_cache()
+
+    n_ctx = sum((n + args.new + 1 + 31) // 32 * 32 for n in lengths)
+    eng = E.Engine(model_path, E.EngineConfig(n_ctx=n_ctx, n_seq_max=n_seq, n_batch=512, n_ubatch=512))
+    adapters = []
+    if args.config == "c4":
+        for i in range(8):
+            a = Path(args.model_dir) / ("retro-bench-c4-lora-%d-seed%d.gguf" % (i, args.seed))
+            if not a.exists():
+                synth.write_lora_adapter(a, shape, rank=16, alpha=16.0, seed=args.seed + 100 + i, std_a=0.02, std_b=0.01)
+            adapters.append(eng.adapter_load(a, 1.0))
+    route = [int(rng.choice(adapters + [E.RETRO_STEP_ADAPTER_BASE])) if adapters else 0 for _ in range(n_seq)]
+
+    out = E.StepOutput(512)
+    greedy = E.SamplingParamsV2.greedy()
+    last = []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s, n in enumerate(lengths):
+        prompt = rng.integers(0, shape.n_vocab, n).astype(np.int32)
+        for at in range(0, n, 512):
+            eng.step([E.StepRow(s, s, prompt[at:at + 512], at, sample=at + 512 >= n, sampling=greedy,
+                                adapter=E.RowAdapter(route[s]))], out)
+        last.append(out.row(0).token)
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+
+    pos = list(lengths)
+    plain = max(1, args.new - args.profiled)
+    step_s = []
+    prof = {}
+    for it in range(args.new):
+        if it == plain:
+            eng.profile(2)
+            eng.profile_read(reset=True)
+        rows = [E.StepRow(s, s, [last[s]], pos[s], sample=True, sampling=greedy, adapter=E.RowAdapter(route[s]))
+                for s in range(n_seq)]
+        t0 = time.perf_counter()
+        eng.step(rows, out)
+        step_s.append(time.perf_counter() - t0)
+        for s in range(n_seq):
+            last[s] = out.row(s).token
+            pos[s] += 1
+    if args.new > plain:
+        prof = eng.profile_read(reset=True)
+    timed = step_s[2:plain] if plain > 4 else step_s[:plain]
+    ms = 1e3 * float(np.mean(timed))
+    n_prof = args.new - plain
+    line = {
+        "config": args.config, "model": shape.name, "sequences": n_seq,
+        "prompt_tokens": int(sum(lengths)), "mean_context_during_decode": float(np.mean(lengths)) + args.new / 2,
+        "prefill_tok_s": round(sum(lengths) / prefill_s, 1),
+        "decode_ms_per_step": round(ms, 3), "decode_tok_s": round(n_seq / ms * 1e3, 1), "decode_steps_timed": len(timed),
+        "adapters": len(adapters), "rows_routed_to_an_adapter": sum(1 for r in route if r > 0),
+        "kernel_ms_per_step": {k: round(t / n_prof, 4) for k, (t, n) in sorted(prof.items(), key=lambda kv: -kv[1][0]) if n},
+        "kernel_launches_per_step": {k: n // n_prof for k, (t, n) in prof.items() if n},
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -264,6 +264,7 @@ private:
     double prof_ms_[PC_COUNT] = {};
     uint64_t prof_n_[PC_COUNT] = {};
     size_t prof_begin(int cat);
+    int mm_single_mask_ = 0;
     void prof_end(int cat, size_t token);
     void prof_resolve();
 

@@ -88,8 +88,11 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     n_ctx_seq_ = cfg_.kv_unified ? (int)cfg_.n_ctx : (int)(cfg_.n_ctx / cfg_.n_seq_max);
     if (n_ctx_seq_ <= 0) throw std::runtime_error("engine n_ctx is too small for n_seq_max sequences");
     max_pages_ = (n_ctx_seq_ + rk::PAGE - 1) / rk::PAGE;
-    // A partially filled last page per slot is the only space paging can waste.
-    n_pages_ = (int)((cfg_.n_ctx + rk::PAGE - 1) / rk::PAGE + cfg_.n_seq_max);
+    // What paging can waste against a cache that shares single cells: per slot the partially filled last
+    // page, and the page in which the slot left a range it shares with another (its private copy of that
+    // page repeats up to PAGE - 1 shared cells). Two spare pages per slot cover both, so a step that fits
+    // n_ctx distinct cells always finds its pages.
+    n_pages_ = (int)((cfg_.n_ctx + rk::PAGE - 1) / rk::PAGE + 2 * cfg_.n_seq_max);
     // [page][kv head]: the other order (a head's pages side by side) was measured 3 % slower in the attention kernel
     kv_strides_ = rk::kv_strides(n_pages_, hp_.n_head_kv, hp_.head_dim, false);
     const int G = hp_.n_head / hp_.n_head_kv;
@@ -245,6 +248,8 @@ void Engine::load_model(const std::string & path) {
     h.n_expert = (int)g.get_int(a + "expert_count", 0);
     h.n_expert_used = (int)g.get_int(a + "expert_used_count", 0);
     h.n_ff_exp = (int)g.get_int(a + "expert_feed_forward_length", h.n_ff);
+    if (h.n_layer < 1 || h.n_embd < 1 || h.n_head < 1 || h.n_head_kv < 1 || h.n_layer > 4096 || h.n_embd > (1 << 20) || h.n_head > 4096)
+        throw std::runtime_error("the model's block_count, embedding_length and head counts must be positive");
     if (h.n_expert > 0 && (h.n_expert > 256 || h.n_expert_used < 1 || h.n_expert_used > 16 || h.n_expert_used > h.n_expert))
         throw std::runtime_error("unsupported expert configuration (at most 256 experts, 1 to 16 used per token)");
     if (h.head_dim != 32 && h.head_dim != 64 && h.head_dim != 128) throw std::runtime_error("head_dim must be 32, 64 or 128");
@@ -273,13 +278,15 @@ void Engine::load_model(const std::string & path) {
         const TensorInfo & wq = g.require(b + "attn_q.weight");
         const TensorInfo & wk = g.require(b + "attn_k.weight");
         const TensorInfo & wv = g.require(b + "attn_v.weight");
-        if (wq.ne[0] != E || wq.ne[1] != QD || wk.ne[1] != KD || wv.ne[1] != KD) throw std::runtime_error("attention weights of layer " + std::to_string(l) + " have unexpected shapes");
+        if (wq.ne[0] != E || wq.ne[1] != QD || wk.ne[0] != E || wk.ne[1] != KD || wv.ne[0] != E || wv.ne[1] != KD) throw std::runtime_error("attention weights of layer " + std::to_string(l) + " have unexpected shapes");
         upload_fused({&wq, &wk, &wv}, L.qkv);
         const TensorInfo * bq = g.find(b + "attn_q.bias");
         if (bq) {
             const TensorInfo & bk = g.require(b + "attn_k.bias");
             const TensorInfo & bv = g.require(b + "attn_v.bias");
             if (bq->type != rk::WT_F32 || bk.type != rk::WT_F32 || bv.type != rk::WT_F32) throw std::runtime_error("attention biases must be F32");
+            if (bq->nbytes != (size_t)QD * 4 || bk.nbytes != (size_t)KD * 4 || bv.nbytes != (size_t)KD * 4)
+                throw std::runtime_error("attention biases of layer " + std::to_string(l) + " have unexpected lengths");
             std::vector<float> joined((size_t)(QD + 2 * KD));
             std::memcpy(joined.data(), bq->data, (size_t)QD * 4);
             std::memcpy(joined.data() + QD, bk.data, (size_t)KD * 4);

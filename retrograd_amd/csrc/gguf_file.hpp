@@ -173,7 +173,12 @@ private:
             case 14: block = 256; bytes = 210; break;
             default: return 0;
         }
-        for (int d = 0; d < t.n_dims; ++d) elems *= t.ne[d];
+        for (int d = 0; d < t.n_dims; ++d) {
+            if (t.ne[d] <= 0) throw std::runtime_error("tensor " + t.name + " has a dimension that is not positive");
+            if (elems > ((int64_t)1 << 46) / t.ne[d]) throw std::runtime_error("tensor " + t.name + " is larger than any file");
+            elems *= t.ne[d];
+        }
+        if (t.ne[0] % block != 0) throw std::runtime_error("tensor " + t.name + " has rows that are not whole blocks of its type");
         return (size_t)(elems / block * bytes);
     }
 
@@ -184,6 +189,8 @@ private:
         if (version < 2 || version > 3) throw std::runtime_error("unsupported GGUF version");
         const uint64_t n_tensors = c.take<uint64_t>();
         const uint64_t n_kv = c.take<uint64_t>();
+        // every key/value takes at least 12 bytes of the file and every tensor entry at least 24
+        if (n_kv > size_ / 12 || n_tensors > size_ / 24) throw std::runtime_error(path_ + ": the GGUF header counts more entries than the file can hold");
         for (uint64_t k = 0; k < n_kv; ++k) {
             std::string key = c.take_string();
             const uint32_t type = c.take<uint32_t>();
@@ -191,6 +198,7 @@ private:
             if (type == 9) {
                 const uint32_t et = c.take<uint32_t>();
                 const uint64_t n = c.take<uint64_t>();
+                if (n > (uint64_t)(c.end - c.p)) throw std::runtime_error("truncated GGUF array for key " + key);
                 v.kind = et == 8 ? MetaValue::STRING_ARRAY : ((et == 6 || et == 12) ? MetaValue::FLOAT_ARRAY : MetaValue::INT_ARRAY);
                 for (uint64_t i = 0; i < n; ++i) {
                     MetaValue e;
@@ -215,13 +223,19 @@ private:
             t.type = (int)c.take<uint32_t>();
             offsets[i] = c.take<uint64_t>();
         }
-        const uint64_t align = (uint64_t)get_int("general.alignment", 32);
+        const int64_t align_field = get_int("general.alignment", 32);
+        if (align_field < 1 || align_field > (1 << 20) || (align_field & (align_field - 1)) != 0)
+            throw std::runtime_error(path_ + ": general.alignment must be a power of two");
+        const uint64_t align = (uint64_t)align_field;
         const uint64_t header = (uint64_t)(c.p - map_);
         const uint64_t data0 = (header + align - 1) / align * align;
+        if (data0 > size_) throw std::runtime_error(path_ + ": the tensor data starts past the end of the file");
+        const uint64_t room = size_ - data0;
         for (size_t i = 0; i < tensors_.size(); ++i) {
             TensorInfo & t = tensors_[i];
             t.nbytes = payload_bytes(t);
-            if (data0 + offsets[i] + t.nbytes > size_) throw std::runtime_error("tensor " + t.name + " runs past the file");
+            // compared without sums, which a huge offset would wrap
+            if (offsets[i] > room || t.nbytes > room - offsets[i]) throw std::runtime_error("tensor " + t.name + " runs past the file");
             t.data = map_ + data0 + offsets[i];
             by_name_[t.name] = i;
         }

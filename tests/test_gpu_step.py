@@ -225,6 +225,28 @@ def test_seq_cp_seq_rm_and_snapshots(models):
     eng.close()
 
 
+def test_forks_inside_a_page_fit_the_pool_up_to_n_ctx_distinct_cells(models):
+    # Eight slots share a 48-cell prefix that ends in the middle of a page and each decodes 58 cells of its
+    # own: 48 + 8 x 58 = 512 = n_ctx distinct cells. Every fork pays a private copy of the half-filled page
+    # and ends in a partial page, 25 pages in all where 512 cells would be 16.
+    eng, ctx, m = _pair(models["tiny-llama-q8"], n_seq=8, n_ctx=512, n_batch=64)
+    rng = np.random.default_rng(21)
+    prefix = rng.integers(0, m.n_vocab, 48)
+    out = E.StepOutput()
+    eng.step([E.StepRow.prefill(0, 0, prefix, 0)], out)
+    ctx.step_rows([(0, 0, prefix, False)])
+    for s in range(1, 8):
+        eng.seq_cp(0, s)
+        ctx.seq_cp(0, s)
+    tails = rng.integers(0, m.n_vocab, (8, 58))
+    for at in range(0, 58, 8):
+        rows = [(s, s, tails[s, at:at + 8], 48 + at, True) for s in range(8)]
+        o, got, want = run_both(eng, ctx, rows)
+        assert_logits_close(got, want)
+    assert all(eng.seq_pos(s) == (0, 105) for s in range(8))
+    eng.close()
+
+
 def test_slot_reuse_after_removal(models):
     # A slot is emptied and refilled between two steps: its block-table entries
     # change twice (to "none", then to new pages) before the device sees them.

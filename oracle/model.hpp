@@ -448,8 +448,12 @@ struct context {
                 std::vector<float> gate((size_t)T * F), up((size_t)T * F);
                 matmul(g.need(b + "ffn_gate.weight"), xn.data(), T, gate.data());
                 matmul(g.need(b + "ffn_up.weight"), xn.data(), T, up.data());
+                // adapters may target every true matrix of a layer (retro_lora.cpp:165-169)
+                add_lora(b + "ffn_gate.weight", xn.data(), T, adapter_of, gate.data(), F);
+                add_lora(b + "ffn_up.weight", xn.data(), T, adapter_of, up.data(), F);
                 for (size_t i = 0; i < gate.size(); ++i) gate[i] = silu(gate[i]) * up[i];
                 matmul(g.need(b + "ffn_down.weight"), gate.data(), T, proj.data());
+                add_lora(b + "ffn_down.weight", gate.data(), T, adapter_of, proj.data(), E);
             }
             for (size_t i = 0; i < x.size(); ++i) x[i] += proj[i];
         }

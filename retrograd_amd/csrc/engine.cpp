@@ -1213,6 +1213,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
     // The versions of a row its consumers need: the values themselves for F32 / F16 / BF16 weights, the
     // expert router and LoRA factors (`plain`); the converted row for the quantised weights.
     const bool faithful = ggml_activations_;
+    const bool ffn_lora = routed && lora_has_ffn_ && h.n_expert == 0;      // some row may carry feed-forward deltas
     auto act_for = [faithful](DevBuf & x, DevBuf & sums, DevBuf & qx, DevBuf & qsums, int K, std::initializer_list<int> types,
                               bool plain) {
         rk::Act a;
@@ -1315,7 +1316,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         prof_end(PC_OPROJ, pt_);
         pt_ = prof_begin(PC_NORM);
         if (h.n_expert > 0) act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {L.router.w.type, L.gate_exps.w.type}, false);
-        else act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {gt[0], gt[1], gt[2]}, false);
+        else act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {gt[0], gt[1], gt[2]}, ffn_lora);
         rk::rmsnorm_act(stream_, x, L.ffn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending);
         prof_end(PC_NORM, pt_);
         if (h.n_expert > 0) {
@@ -1331,23 +1332,37 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
             continue;
         }
         pt_ = prof_begin(PC_GATEUP);
-        const rk::Act act_f = act_for(act_f_x_, act_f_sums_, act_f_qx_, act_f_qsums_, F, {L.down.w.type}, false);
-        if (L.gate_up_interleaved) {
+        const rk::Act act_f = act_for(act_f_x_, act_f_sums_, act_f_qx_, act_f_qsums_, F, {L.down.w.type}, ffn_lora);
+        if (L.gate_up_interleaved && !ffn_lora) {
             rk::matmul_swiglu(stream_, L.gate_up[0].w, act_e, T, act_f, mm_ws_.ptr, gu);
             prof_end(PC_GATEUP, pt_);
         } else {
+            // gate and up as f32 rows: side by side, or - the interleaved matrix of the fused kernel multiplied
+            // like any other - in alternating groups of 64 columns; the adapter deltas join them before the SiLU
+            const int group = L.gate_up_interleaved ? 64 : F;
             int col = 0;
             for (const DevWeight & w : L.gate_up) {
                 rk::matmul(stream_, w.w, act_e, T, gu, 2 * F, col, rk::MM_STORE, nullptr, mm_ws_.ptr);
                 col += w.w.N;
             }
+            if (ffn_lora) {
+                const int cols[2] = {0, group}, widths[2] = {F, F};
+                const rk::LoraEntry * tables[2] = {lora_entries(l, 4), lora_entries(l, 5)};
+                rk::lora_apply_targets(stream_, 2, tables, widths, cols, d_stage_.as<rk::RowDesc>(), pk_.row, act_e, T, gu,
+                                       2 * F, lora_mid_.as<float>(), L.gate_up_interleaved ? group : 0);
+            }
             prof_end(PC_GATEUP, pt_);
             pt_ = prof_begin(PC_SWIGLU);
-            rk::swiglu_act(stream_, gu, T, F, act_f);
+            rk::swiglu_act(stream_, gu, T, F, act_f, group);
             prof_end(PC_SWIGLU, pt_);
         }
         pt_ = prof_begin(PC_DOWN);
         pending = rk::matmul_deferred(stream_, L.down.w, act_f, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
+        if (ffn_lora) {
+            float * dst = pending.n > 0 ? const_cast<float *>(pending.data) : x;
+            rk::lora_apply(stream_, lora_entries(l, 6), d_stage_.as<rk::RowDesc>(), pk_.row, act_f, T, E, dst, E, 0,
+                           lora_mid_.as<float>());
+        }
         prof_end(PC_DOWN, pt_);
     }
     if (n_out > 0) {
@@ -1548,8 +1563,11 @@ int Engine::read_adapter(const std::string & path, float scale, RowAdapterData &
     }
     const HParams & h = hp_;
     const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim;
-    static const char * kTargets[kLoraTargets] = {"attn_q", "attn_k", "attn_v", "attn_output"};
-    const int n_in[kLoraTargets] = {E, E, E, QD}, n_out[kLoraTargets] = {QD, KD, KD, E};
+    // every true matrix of a layer (reference retro_lora.cpp:165-169); a mixture-of-experts layer has no dense
+    // feed-forward matrices, and its expert stacks are no per-row targets (retro_lora_train.h:2594-2596)
+    static const char * kTargets[kLoraTargets] = {"attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down"};
+    const int F = h.n_expert > 0 ? 0 : h.n_ff;
+    const int n_in[kLoraTargets] = {E, E, E, QD, E, E, F}, n_out[kLoraTargets] = {QD, KD, KD, E, F, F, E};
     data = RowAdapterData();
     data.scale = scale;
     data.alpha = file->get_float("adapter.lora.alpha", 0.0);
@@ -1568,6 +1586,7 @@ int Engine::read_adapter(const std::string & path, float scale, RowAdapterData &
                 set_error("LoRA adapter tensor " + base + " has no matching lora_a / lora_b pair");
                 return -1;
             }
+            if (n_in[tg] <= 0 || n_out[tg] <= 0) continue;       // not a matrix of this model: reported below as unclaimed
             const int r = (int)ta->ne[1];
             if (ta->ne[0] != n_in[tg] || tb->ne[1] != n_out[tg] || tb->ne[0] != r || r <= 0) {
                 set_error("LoRA adapter tensor " + base + " does not match the base model's shape");
@@ -1600,14 +1619,14 @@ int Engine::read_adapter(const std::string & path, float scale, RowAdapterData &
             claimed += 2;
         }
     }
-    // a target this engine does not route per row (embeddings, FFN, experts) must not be dropped silently
+    // a target this engine does not route per row (embeddings, expert stacks) must not be dropped silently
     size_t lora_tensors = 0;
     for (const TensorInfo & t : file->tensors()) {
         const std::string & n = t.name;
         if (n.size() > 7 && (n.compare(n.size() - 7, 7, ".lora_a") == 0 || n.compare(n.size() - 7, 7, ".lora_b") == 0)) ++lora_tensors;
     }
     if (lora_tensors != claimed) {
-        set_error("failed to stack the per-row adapters: only attn_q, attn_k, attn_v and attn_output targets are routed per row");
+        set_error("failed to stack the per-row adapters: only the attention and dense feed-forward matrices of a layer are routed per row");
         return -1;
     }
     if (data.rank == 0) {
@@ -1637,6 +1656,7 @@ int Engine::adapter_unload(int32_t id) {
 // lora_router_install, retro_gen_core.cpp:2987-3006).
 void Engine::rebuild_lora_table() {
     lora_routes_ = (int)row_adapters_.size();
+    lora_has_ffn_ = false;
     if (lora_routes_ == 0) return;
     std::vector<rk::LoraEntry> table((size_t)hp_.n_layer * kLoraTargets * (size_t)lora_routes_);
     int route = 0;
@@ -1647,6 +1667,7 @@ void Engine::rebuild_lora_table() {
                 rk::LoraEntry & e = table[((size_t)l * kLoraTargets + tg) * (size_t)lora_routes_ + (size_t)route];
                 const size_t at = (size_t)l * kLoraTargets + tg;
                 if (!d.a[at].ptr) continue;
+                if (tg >= 4) lora_has_ffn_ = true;
                 e.A = d.a[at].as<float>();
                 e.B = d.b[at].as<float>();
                 e.rank = d.rank;

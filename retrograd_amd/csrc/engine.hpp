@@ -269,7 +269,8 @@ private:
     void prof_resolve();
 
     // per-row adapters: targets attn_q, attn_k, attn_v, attn_output of every layer
-    static constexpr int kLoraTargets = 4;
+    static constexpr int kLoraTargets = 7;      // attn_q, attn_k, attn_v, attn_output, ffn_gate, ffn_up, ffn_down
+    bool lora_has_ffn_ = false;                 // some loaded adapter holds a pair for a feed-forward matrix
     struct RowAdapterData {
         float scale = 1.0f;
         double alpha = 0.0;

@@ -756,6 +756,7 @@ __device__ __forceinline__ float lora_operand(float hi, float lo, int type) {
 struct LoraTargets {
     const LoraEntry * table[3];
     int N[3], col0[3];
+    int group;      // 0: output n is column col0 + n; g > 0: column col0 + (n / g) * 2g + n % g (gate and up interleaved by g)
 };
 
 __global__ __launch_bounds__(256) void k_lora_down(LoraTargets tg, const RowDesc * __restrict__ rows,
@@ -808,15 +809,19 @@ __global__ __launch_bounds__(256) void k_lora_up(LoraTargets tg, const RowDesc *
         const float hi = (float)(_Float16)fminf(fmaxf(m[r], -65504.0f), 65504.0f);
         acc = fmaf(b[r], lora_operand(hi, m[r] - hi, e.b_type), acc);
     }
-    y[(size_t)t * ldy + col0 + n] += e.scale * acc;
+    const int col = tg.group > 0 ? (n / tg.group) * 2 * tg.group + n % tg.group : n;
+    y[(size_t)t * ldy + col0 + col] += e.scale * acc;
 }
 
 void lora_apply_targets(hipStream_t s, int n_targets, const LoraEntry * const * tables, const int * widths, const int * cols,
-                        const RowDesc * rows, const int32_t * tok_row, const Act & x, int T, float * y, int ldy, float * mid) {
+                        const RowDesc * rows, const int32_t * tok_row, const Act & x, int T, float * y, int ldy, float * mid,
+                        int group) {
     if (T <= 0 || n_targets <= 0) return;
+    if (group < 0) throw std::runtime_error("lora: the interleave group must not be negative");
     if (n_targets > 3) throw std::runtime_error("lora: at most three targets share a launch");
     if (!x.x) throw std::runtime_error("lora: the unconverted activations are missing");
     LoraTargets tg {};
+    tg.group = group;
     int max_n = 0;
     for (int i = 0; i < n_targets; ++i) {
         tg.table[i] = tables[i]; tg.N[i] = widths[i]; tg.col0[i] = cols[i];
@@ -831,7 +836,7 @@ void lora_apply_targets(hipStream_t s, int n_targets, const LoraEntry * const * 
 
 void lora_apply(hipStream_t s, const LoraEntry * table, const RowDesc * rows, const int32_t * tok_row,
                 const Act & x, int T, int N, float * y, int ldy, int col0, float * mid) {
-    lora_apply_targets(s, 1, &table, &N, &col0, rows, tok_row, x, T, y, ldy, mid);
+    lora_apply_targets(s, 1, &table, &N, &col0, rows, tok_row, x, T, y, ldy, mid, 0);
 }
 
 __global__ __launch_bounds__(256) void k_rmsnorm_act(float * x, const float * __restrict__ w,
@@ -966,15 +971,17 @@ void rmsnorm_act(hipStream_t s, float * x, const float * w, int E, float eps,
     check_launch("rmsnorm");
 }
 
-__global__ __launch_bounds__(256) void k_swiglu_act(const float * __restrict__ gu, int T, int F, Act out) {
+// gate c of a token sits at column (c / group) * 2 group + c % group and up c `group` columns further: group = F
+// for the two matrices side by side, 64 for the interleaved matrix of the fused kernel.
+__global__ __launch_bounds__(256) void k_swiglu_act(const float * __restrict__ gu, int T, int F, int group, Act out) {
     const int nblk = (F + 31) / 32;
     const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (gid >= (size_t)T * nblk) return;
     const int t = (int)(gid / nblk), b = (int)(gid % nblk);
     const int k0 = b * 32;
     const int count = min(32, F - k0);
-    const float * g = gu + (size_t)t * 2 * F + k0;
-    const float * u = g + F;
+    const float * g = gu + (size_t)t * 2 * F + (k0 / group) * 2 * group + k0 % group;
+    const float * u = g + group;
     float v[32];
     for (int i = 0; i < count; ++i) {
         const float gi = g[i];
@@ -1045,13 +1052,13 @@ void requant_act(hipStream_t s, const __half * src, int T, const Act & out) {
 }
 
 // F % 32 == 0: 8 elements per lane.
-__global__ __launch_bounds__(256) void k_swiglu_act8(const float * __restrict__ gu, int T, int F, Act out) {
+__global__ __launch_bounds__(256) void k_swiglu_act8(const float * __restrict__ gu, int T, int F, int group, Act out) {
     const int per = F / 8;
     const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (gid >= (size_t)T * per) return;      // whole groups of four lanes leave together (per % 4 == 0)
     const int t = (int)(gid / per), k = (int)(gid % per) * 8;
-    const float * g = gu + (size_t)t * 2 * F + k;
-    const float * u = g + F;
+    const float * g = gu + (size_t)t * 2 * F + (k / group) * 2 * group + k % group;
+    const float * u = g + group;
     const f4 ga = *(const f4 *)g, gb = *(const f4 *)(g + 4), ua = *(const f4 *)u, ub = *(const f4 *)(u + 4);
     const float gv[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
     const float uv[8] = {ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w};
@@ -1061,19 +1068,22 @@ __global__ __launch_bounds__(256) void k_swiglu_act8(const float * __restrict__ 
     store_act8(v, out, t, k, threadIdx.x & 3);
 }
 
-void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out) {
+void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out, int group) {
     if (T <= 0) return;
     check_act_out(out, F, "swiglu");
+    if (group <= 0) group = F;
+    // a block of 32 (8) gate columns must not straddle two groups
+    if (group != F && (F % group != 0 || group % 32 != 0)) throw std::runtime_error("swiglu: the interleave group must divide F and be a multiple of 32");
     if (F % 32 == 0) {
         const size_t n = (size_t)T * (F / 8);
-        hipLaunchKernelGGL(k_swiglu_act8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, T, F, out);
+        hipLaunchKernelGGL(k_swiglu_act8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, T, F, group, out);
         check_launch("swiglu");
         return;
     }
     Act o = out;
     o.sums = nullptr;
     const size_t n = (size_t)T * ((F + 31) / 32);
-    hipLaunchKernelGGL(k_swiglu_act, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, T, F, o);
+    hipLaunchKernelGGL(k_swiglu_act, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, gu, T, F, group, o);
     check_launch("swiglu");
 }
 

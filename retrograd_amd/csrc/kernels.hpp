@@ -161,9 +161,11 @@ constexpr int LORA_MAX_RANK = 64;
 //   y[t][col0 + n] += scale * sum_r B[n][r] * (sum_k A[r][k] * x[t][k]).
 // mid is scratch of T * LORA_MAX_RANK floats.
 // The same for up to three targets that read the same activations (tables[i], widths[i], cols[i]), in one
-// pair of launches; mid is scratch of n_targets * T * LORA_MAX_RANK floats.
+// pair of launches; mid is scratch of n_targets * T * LORA_MAX_RANK floats. group > 0: output n of a target
+// lands in column cols[i] + (n / group) * 2 group + n % group (gate and up outputs interleaved by `group`).
 void lora_apply_targets(hipStream_t s, int n_targets, const LoraEntry * const * tables, const int * widths, const int * cols,
-                        const RowDesc * rows, const int32_t * tok_row, const Act & x, int T, float * y, int ldy, float * mid);
+                        const RowDesc * rows, const int32_t * tok_row, const Act & x, int T, float * y, int ldy, float * mid,
+                        int group = 0);
 void lora_apply(hipStream_t s, const LoraEntry * table, const RowDesc * rows, const int32_t * tok_row,
                 const Act & x, int T, int N, float * y, int ldy, int col0, float * mid);
 // out[r][k] = decode(raw row r)[k] as f32: any tensor to f32, row by row.
@@ -206,7 +208,8 @@ void to_act(hipStream_t s, const float * x, int T, int K, const Act & out);
 void requant_act(hipStream_t s, const __half * src, int T, const Act & out);
 
 // act = f16(silu(gu[t][i]) * gu[t][F + i]) (+ block sums).
-void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out);
+// group: gate c at column (c / group) * 2 group + c % group, up c `group` columns further (0: group = F, side by side)
+void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out, int group = 0);
 
 // ---- step packing -----------------------------------------------------------
 struct RowDesc {           // one per step row, written by the host

@@ -52,7 +52,9 @@ CASES = {
     "qwen3moe": (synth.scaled(synth.QWEN3_30B_A3B, n_layer=2, n_embd=256, n_head=4, n_head_kv=2, head_dim=64, n_vocab=288,
                               n_expert=8, n_expert_used=2, n_ff_exp=256, norm_std=0.2, name="hf-qwen3moe"), 45, 0.08),
 }
-LORA = {"case": "qwen2", "rank": 4, "alpha": 8.0, "seed": 3, "scale": 0.5, "std_a": 0.1, "std_b": 0.1}
+LORA = {"case": "qwen2", "rank": 4, "alpha": 8.0, "seed": 3, "scale": 0.5, "std_a": 0.1, "std_b": 0.1,
+        # every true matrix of a layer is a target (reference retro_lora.cpp:165-169)
+        "targets": ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down")}
 PROMPT_SEED = 77
 N_TOKENS = 14
 POS0 = {"llama-linear": 0}
@@ -159,9 +161,9 @@ def build_hf(path, shape, lora=None):
             sd[h + "mlp.experts.gate_up_proj"] = T(np.concatenate([gate, up], axis=1))
             sd[h + "mlp.experts.down_proj"] = T(W(b + "ffn_down_exps.weight"))          # [expert][E][F]
         else:
-            sd[h + "mlp.gate_proj.weight"] = T(W(b + "ffn_gate.weight"))
-            sd[h + "mlp.up_proj.weight"] = T(W(b + "ffn_up.weight"))
-            sd[h + "mlp.down_proj.weight"] = T(W(b + "ffn_down.weight"))
+            sd[h + "mlp.gate_proj.weight"] = T(merged(b + "ffn_gate.weight"))
+            sd[h + "mlp.up_proj.weight"] = T(merged(b + "ffn_up.weight"))
+            sd[h + "mlp.down_proj.weight"] = T(merged(b + "ffn_down.weight"))
     missing, unexpected = model.load_state_dict(sd, strict=False)
     assert not unexpected, unexpected
     assert all("rotary" in m or "inv_freq" in m for m in missing), missing
@@ -198,7 +200,7 @@ def main():
             if key == LORA["case"]:
                 ad = Path(d) / "adapter.gguf"
                 synth.write_lora_adapter(ad, shape, rank=LORA["rank"], alpha=LORA["alpha"], seed=LORA["seed"],
-                                         std_a=LORA["std_a"], std_b=LORA["std_b"])
+                                         std_a=LORA["std_a"], std_b=LORA["std_b"], targets=LORA["targets"])
                 ar = Reader(ad)
                 pairs = {}
                 for name in ar.tensors:

@@ -7,6 +7,7 @@ import pytest
 import oracle
 from engine_helpers import assert_logits_close, greedy, logit_errors
 from retrograd_amd import engine as E
+from retrograd_amd import gguf_writer as gw
 from retrograd_amd import synth
 
 pytestmark = pytest.mark.gpu
@@ -24,8 +25,17 @@ def files(tmp_path_factory):
     synth.write_lora_adapter(a1, SHAPE, rank=16, alpha=32.0, seed=1, std_a=0.1, std_b=0.1)
     synth.write_lora_adapter(a2, SHAPE, rank=8, alpha=8.0, seed=2, std_a=0.1, std_b=0.1,
                              targets=("attn_q", "attn_output"))
-    ffn = d / "ffn.gguf"
-    synth.write_lora_adapter(ffn, SHAPE, rank=4, alpha=4.0, seed=3, targets=("attn_q", "ffn_down"))
+    # a target that is no matrix of a layer: never routed per row (reference retro_lora_train.h:2594-2596)
+    ffn = d / "embd.gguf"
+    w = gw.GGUFWriter()
+    w.add("general.type", gw.T_STRING, "adapter")
+    w.add("general.architecture", gw.T_STRING, SHAPE.arch)
+    w.add("adapter.type", gw.T_STRING, "lora")
+    w.add("adapter.lora.alpha", gw.T_FLOAT32, 4.0)
+    rng = np.random.default_rng(5)
+    w.add_tensor("token_embd.weight.lora_a", [SHAPE.n_embd, 4], gw.GGML_F32, rng.standard_normal((4, SHAPE.n_embd)).astype(np.float32).tobytes())
+    w.add_tensor("token_embd.weight.lora_b", [4, SHAPE.n_vocab], gw.GGML_F32, rng.standard_normal((SHAPE.n_vocab, 4)).astype(np.float32).tobytes())
+    w.write(ffn)
     return model, a1, a2, ffn
 
 
@@ -72,6 +82,72 @@ def test_rows_under_different_adapters_match_the_oracle(files):
     assert (info.n_adapters, info.max_rank) == (2, 16)
     assert info.stacked_bytes == (el1 + el2) * 16 * 4
     assert info.unpadded_bytes == el1 * 16 * 4 + el2 * 8 * 4
+    eng.close()
+
+
+FFN_TARGETS = ("attn_q", "ffn_gate", "ffn_up", "ffn_down")
+# gate and up interleaved for the fused SwiGLU kernel (width a multiple of 64), and side by side on the generic kernels
+FFN_SHAPES = {"interleaved": SHAPE, "side-by-side": synth.TINY_LLAMA}
+
+
+@pytest.mark.parametrize("layout", list(FFN_SHAPES))
+@pytest.mark.parametrize("activations", ["exact", "ggml"])
+def test_adapters_on_the_feed_forward_matrices_match_the_oracle(tmp_path, layout, activations, monkeypatch):
+    """Every true matrix of a layer may carry a pair (reference retro_lora.cpp:165-169): rows under an adapter with
+    ffn_gate / ffn_up / ffn_down pairs, under an attention-only adapter and under the base share steps."""
+    shape = FFN_SHAPES[layout]
+    print("per-row LoRA on feed-forward matrices: %s, %s, %s arithmetic" % (shape.name, layout, activations), flush=True)
+    if activations == "ggml":
+        monkeypatch.setenv("RETRO_ACTIVATIONS", "ggml")
+    model, ffn, attn = tmp_path / "m.gguf", tmp_path / "ffn.gguf", tmp_path / "attn.gguf"
+    synth.write_model(model, shape, seed=31, device="cpu", std=0.05)
+    synth.write_lora_adapter(ffn, shape, rank=4, alpha=8.0, seed=3, std_a=0.1, std_b=0.1, targets=FFN_TARGETS)
+    synth.write_lora_adapter(attn, shape, rank=8, alpha=8.0, seed=4, std_a=0.1, std_b=0.1, targets=("attn_q", "attn_output"))
+    eng = E.Engine(model, E.EngineConfig(n_ctx=1024, n_seq_max=4, n_batch=128, n_ubatch=128))
+    m = oracle.Model(model)
+    ctx = oracle.Context(m, 4, activations=activations)
+    ids = [eng.adapter_load(ffn, 1.0), eng.adapter_load(attn, 0.5)]
+    assert ids == [m.load_adapter(ffn, 1.0), m.load_adapter(attn, 0.5)]
+    rng = np.random.default_rng(8)
+    lens = [17, 33, 9, 66]           # 125 tokens: two 64-token chunks in the prefill step
+    prompts = [rng.integers(0, m.n_vocab, n) for n in lens]
+    route = [ids[0], ids[1], E.RETRO_STEP_ADAPTER_BASE, ids[0]]
+    oroute = [ids[0], ids[1], -1, ids[0]]
+    out = E.StepOutput()
+    eng.step([E.StepRow(i, i, prompts[i], 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(route[i])) for i in range(4)], out)
+    got = eng.debug_logits()
+    want = ctx.step_rows([(i, 0, prompts[i], True) for i in range(4)], adapters=oroute)
+    base = oracle.Context(m, 4, activations=activations).step_rows([(i, 0, prompts[i], True) for i in range(4)])
+    assert np.abs(want[0] - base[0]).max() > 5e-2, "the feed-forward pairs do something"
+    if activations == "exact":
+        assert_logits_close(got, want)
+    else:
+        # two faithful implementations of the conversion drift apart by rounding ties; clearly nearer than the base model
+        assert logit_errors(got, want)[1] < 0.3 * logit_errors(base, want)[1]
+        eng.close()
+        return
+    pos = list(lens)
+    for _ in range(3):
+        feed = [int(want[i].argmax()) for i in range(4)]
+        eng.step([E.StepRow(i, i, [feed[i]], pos[i], sample=True, sampling=greedy(), adapter=E.RowAdapter(route[i]))
+                  for i in range(4)], out)
+        got = eng.debug_logits()
+        want = ctx.step_rows([(i, pos[i], [feed[i]], True) for i in range(4)], adapters=oroute)
+        assert_logits_close(got, want)
+        pos = [p + 1 for p in pos]
+    # a step without a routed row goes back to the fused kernel: same logits as an engine that never loaded an adapter
+    plain = E.Engine(model, E.EngineConfig(n_ctx=1024, n_seq_max=4, n_batch=128, n_ubatch=128))
+    rows = lambda: [E.StepRow(9, 3, prompts[1], 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(E.RETRO_STEP_ADAPTER_BASE))]
+    eng.seq_rm(3)
+    eng.step(rows(), out)
+    plain.step(rows(), out)
+    assert np.array_equal(eng.debug_logits(), plain.debug_logits())
+    info = eng.adapter_rows_info()
+    E_, QD, F = shape.n_embd, shape.n_head * shape.head_dim, shape.n_ff
+    el_ffn = shape.n_layer * ((E_ + QD) + 2 * (E_ + F) + (F + E_))
+    el_attn = shape.n_layer * ((E_ + QD) + (QD + E_))
+    assert info.stacked_bytes == (el_ffn + el_attn) * 8 * 4 and info.unpadded_bytes == el_ffn * 4 * 4 + el_attn * 8 * 4
+    plain.close()
     eng.close()
 
 
@@ -216,7 +292,7 @@ def test_adapter_errors_and_unload(files):
     toks = [1, 2, 3]
     with pytest.raises(E.InvalidArgument, match="is not a loaded per-row adapter"):
         eng.step([E.StepRow(0, 0, toks, 0, sample=True, sampling=greedy(), adapter=E.RowAdapter(1))], out)
-    with pytest.raises(E.RuntimeFailure, match="only attn_q, attn_k, attn_v and attn_output"):
+    with pytest.raises(E.RuntimeFailure, match="only the attention and dense feed-forward matrices"):
         eng.adapter_load(ffn)
     with pytest.raises(E.RuntimeFailure, match="failed to load LoRA adapter"):
         eng.adapter_load(model)

@@ -202,3 +202,54 @@ def test_rollouts_through_the_scheduler_over_a_trainer(files):
     sched.close()
     tr.close()
     eng.close()
+
+
+def test_a_trainer_step_under_the_trained_adapter_follows_the_oracle(files):
+    """The trainer handle exposes no logits, so the comparison goes through what a step returns: for every
+    sampling row the ids of the eight largest logits and their log-probabilities, and the sampled token's,
+    against the CPU oracle with the same adapter file loaded (prefill, then three decode steps)."""
+    import oracle
+    model, a1, _ = files
+    print("trainer: step outputs against the oracle", flush=True)
+    tr = trainer(model)
+    tr.load_lora(a1)
+    m = oracle.Model(model)
+    aid = m.load_adapter(a1, 1.0)
+    ctx = oracle.Context(m, 4)
+    rng = np.random.default_rng(33)
+    lens = [19, 7, 30, 12]
+    prompts = [rng.integers(0, SHAPE.n_vocab, n) for n in lens]
+    out = E.StepOutput(4, 8)
+    feed, pos = prompts, [0] * 4
+    compared = 0
+    for step in range(4):
+        # the whole distribution at temperature 1: the reported log-probabilities are those of the plain softmax
+        tr.step([E.StepRow(i, i, feed[i], pos[i], sample=True, n_top_logprobs=8, want_logprob=True,
+                           sampling=E.SamplingParamsV2(temperature=1.0, top_p=1.0, top_k=0, seed=50 + i))
+                 for i in range(4)], out)
+        want = ctx.step_rows([(i, pos[i], feed[i], True) for i in range(4)], adapters=[aid] * 4).astype(np.float64)
+        nxt = []
+        for i in range(4):
+            lp = want[i] - (np.log(np.exp(want[i] - want[i].max()).sum()) + want[i].max())
+            order = np.argsort(-want[i], kind="stable")
+            ids, lps = out.top(i)
+            assert len(ids) == 8
+            # every reported id is among the oracle's eight largest up to the tolerance, in descending order,
+            # and the first one is the oracle's wherever its margin exceeds the tolerance
+            assert (want[i][ids] >= want[i][order[7]] - 2 * 2e-2).all() and len(set(int(t) for t in ids)) == 8
+            assert (np.diff(lps) <= 0).all()
+            if want[i][order[0]] - want[i][order[1]] > 2 * 2e-2:
+                assert int(ids[0]) == int(order[0])
+                compared += 1
+            assert np.abs(lps.astype(np.float64) - lp[ids]).max() <= 2e-2
+            r = out.row(i)
+            assert abs(float(r.sampled_logprob) - lp[r.token]) <= 2e-2
+            nxt.append([int(r.token)])           # both sides continue with the token the trainer drew
+        pos = [pos[i] + len(feed[i]) for i in range(4)]
+        feed = nxt
+    assert compared >= 10
+    # and the adapter matters: the base model's top id differs somewhere or its log-probabilities move visibly
+    base = oracle.Context(m, 4).step_rows([(i, 0, prompts[i], True) for i in range(4)])
+    with_ad = oracle.Context(m, 4).step_rows([(i, 0, prompts[i], True) for i in range(4)], adapters=[aid] * 4)
+    assert np.abs(base - with_ad).max() > 5e-2
+    tr.close()

@@ -133,7 +133,8 @@ def test_lora_delta_matches_dense_formula_and_rank_padding(models, tmp_path, act
     shape = SHAPES["qwen2-q8"]
     m = oracle.Model(models["qwen2-q8"])
     ad = tmp_path / "a.gguf"
-    synth.write_lora_adapter(ad, shape, rank=4, alpha=8.0, seed=3, std_a=0.1, std_b=0.1)
+    synth.write_lora_adapter(ad, shape, rank=4, alpha=8.0, seed=3, std_a=0.1, std_b=0.1,
+                             targets=("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down"))
     aid = m.load_adapter(ad, 0.5)
     assert aid == 1
     rng = np.random.default_rng(9)
@@ -196,14 +197,15 @@ def test_forward_reproduces_hugging_face_transformers_logits(tmp_path, key):
 
 
 def test_lora_delta_reproduces_hugging_face_logits_with_the_adapter_merged(tmp_path):
-    """scale * alpha / r * B (A x) on q, k, v and o of a qwen2 file against the Hugging Face model whose dense
+    """scale * alpha / r * B (A x) on q, k, v, o, gate, up and down of a qwen2 file against the Hugging Face model whose dense
     matrices had scale * alpha / r * B A added."""
     mod, golden = _hf_golden()
     L = mod.LORA
     shape, seed, std = mod.CASES[L["case"]]
     path, ad = tmp_path / "m.gguf", tmp_path / "a.gguf"
     synth.write_model(path, shape, seed=seed, device="cpu", std=std)
-    synth.write_lora_adapter(ad, shape, rank=L["rank"], alpha=L["alpha"], seed=L["seed"], std_a=L["std_a"], std_b=L["std_b"])
+    synth.write_lora_adapter(ad, shape, rank=L["rank"], alpha=L["alpha"], seed=L["seed"], std_a=L["std_a"], std_b=L["std_b"],
+                             targets=L["targets"])
     assert bytes(golden[L["case"] + ".lora.sha256"]).hex() == mod.sha256(ad)
     toks = golden[L["case"] + ".tokens"]
     want = golden[L["case"] + ".lora.logits"].astype(np.float64)

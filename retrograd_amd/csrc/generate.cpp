@@ -286,69 +286,74 @@ int Engine::generate_continuous_batch(const retro_generation_sequence * sequence
 
     const std::vector<size_t> order = canonical_order(sequences, n_sequences);
 
-    // ---- placement (retro_gen_core.cpp:430-546)
+    // ---- placement: the decisions of place_generation_sequences (reference retro_gen_core.cpp:430-546), stated as
+    // a ranking. In canonical order every sequence takes, of the slots no earlier sequence of the call took, the
+    // one ranked first by (longest resident prefix of its prompt; among slots that hold nothing of it the one
+    // extended longest ago; lowest slot number). Then the slots nobody took give way, least recently extended
+    // first, until what they hold fits beside the cells this call can come to occupy.
     const size_t n_slots = cfg_.n_seq_max;
     std::vector<int32_t> slot_of(n_sequences);
     std::vector<size_t> reuse_of(n_sequences, 0);
     if (!cache) {
         for (size_t i = 0; i < n_sequences; ++i) slot_of[i] = (int32_t)i;
     } else {
-        GenCache & bk = gen_cache_;
-        bk.slots.resize(n_slots);
-        bk.used_at.resize(n_slots, 0);
-        std::vector<bool> claimed(n_slots, false);
+        GenCache & ledger = gen_cache_;
+        ledger.slots.resize(n_slots);
+        ledger.used_at.resize(n_slots, 0);
+        std::vector<bool> taken(n_slots, false);
+        struct Offer { size_t slot, kept; uint64_t age; };
+        auto outranks = [](const Offer & a, const Offer & b) {
+            if (a.kept != b.kept) return a.kept > b.kept;
+            if (a.kept == 0 && a.age != b.age) return a.age < b.age;
+            return a.slot < b.slot;
+        };
         for (const size_t seq : order) {
             const retro_generation_sequence & item = sequences[seq];
-            size_t best_slot = n_slots, best_reuse = 0;
+            Offer pick{n_slots, 0, 0};
             for (size_t slot = 0; slot < n_slots; ++slot) {
-                if (claimed[slot]) continue;
-                const size_t reuse = resident_prefix(bk.slots[slot], item);
-                if (best_slot == n_slots || reuse > best_reuse) {
-                    best_slot = slot;
-                    best_reuse = reuse;
-                    continue;
-                }
-                // nothing worth keeping anywhere: sacrifice the slot that has gone longest without being extended
-                if (reuse == best_reuse && reuse == 0 && bk.used_at[slot] < bk.used_at[best_slot]) best_slot = slot;
+                if (taken[slot]) continue;
+                const Offer offer{slot, resident_prefix(ledger.slots[slot], item), ledger.used_at[slot]};
+                if (pick.slot == n_slots || outranks(offer, pick)) pick = offer;
             }
-            claimed[best_slot] = true;
-            slot_of[seq] = (int32_t)best_slot;
-            reuse_of[seq] = best_reuse;
-            if (best_reuse == 0) {
-                if (!bk.slots[best_slot].empty()) bk.stats.evictions++;
-                (void)seq_rm((int32_t)best_slot, -1, -1);
-                bk.slots[best_slot].clear();
+            taken[pick.slot] = true;
+            slot_of[seq] = (int32_t)pick.slot;
+            reuse_of[seq] = pick.kept;
+            if (pick.kept > 0) {
+                ledger.stats.hits++;
             } else {
-                bk.stats.hits++;
+                // a cold start: whatever the slot held is given up
+                if (!ledger.slots[pick.slot].empty()) ledger.stats.evictions++;
+                (void)seq_rm((int32_t)pick.slot, -1, -1);
+                ledger.slots[pick.slot].clear();
             }
-            bk.stats.sequences++;
-            bk.stats.prompt_tokens += item.n_prompt;
-            bk.stats.reused_tokens += best_reuse;
+            ledger.stats.sequences++;
+            ledger.stats.prompt_tokens += item.n_prompt;
+            ledger.stats.reused_tokens += pick.kept;
         }
-        // dormant slots share the pool with this call's sequences: budget the positions
-        // this call will decode, then drop dormant slots, oldest first, until they fit
-        size_t remaining = cfg_.n_ctx;
+        // cells this call may occupy: every prompt and all but the last of the tokens it can emit
+        size_t room = cfg_.n_ctx;
         for (size_t i = 0; i < n_sequences; ++i) {
             const retro_generation_sequence & item = sequences[i];
-            const size_t emitted = std::min<size_t>(std::min<size_t>(n_out_max, item.sampling.max_new_tokens),
-                                                    n_ctx_seq - item.n_prompt);
-            const size_t decoded = item.n_prompt + emitted - 1;
-            remaining -= std::min(remaining, decoded);
+            const size_t new_tokens = std::min<size_t>(std::min<size_t>(n_out_max, item.sampling.max_new_tokens),
+                                                       n_ctx_seq - item.n_prompt);
+            room -= std::min(room, item.n_prompt + new_tokens - 1);
         }
-        uint64_t dormant = 0;
+        // idle slots by the time they were last extended (slot number breaking ties), oldest first
+        std::vector<size_t> idle;
+        uint64_t idle_cells = 0;
         for (size_t slot = 0; slot < n_slots; ++slot)
-            if (!claimed[slot]) dormant += bk.slots[slot].size();
-        while (dormant > remaining) {
-            size_t oldest = n_slots;
-            for (size_t slot = 0; slot < n_slots; ++slot)
-                if (!claimed[slot] && !bk.slots[slot].empty() && (oldest == n_slots || bk.used_at[slot] < bk.used_at[oldest]))
-                    oldest = slot;
-            if (oldest == n_slots) break;
-            (void)seq_rm((int32_t)oldest, -1, -1);
-            dormant -= bk.slots[oldest].size();
-            bk.slots[oldest].clear();
-            bk.used_at[oldest] = 0;
-            bk.stats.evictions++;
+            if (!taken[slot] && !ledger.slots[slot].empty()) {
+                idle.push_back(slot);
+                idle_cells += ledger.slots[slot].size();
+            }
+        std::stable_sort(idle.begin(), idle.end(), [&](size_t a, size_t b) { return ledger.used_at[a] < ledger.used_at[b]; });
+        for (size_t i = 0; i < idle.size() && idle_cells > room; ++i) {
+            const size_t slot = idle[i];
+            (void)seq_rm((int32_t)slot, -1, -1);
+            idle_cells -= ledger.slots[slot].size();
+            ledger.slots[slot].clear();
+            ledger.used_at[slot] = 0;
+            ledger.stats.evictions++;
         }
     }
 

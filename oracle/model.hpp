@@ -29,11 +29,18 @@
 // RMSNorm is x / sqrt(mean(x^2) + eps) with the weight multiply a separate op
 // (generated/rir/rms_norm/kernel.shared_reduce.cu:27-55).
 //
-// PARITY UNPINNED against the reference at float level: no reference test or
-// fixture records absolute logits of a causal model. What pins this file
-// instead (tests/test_oracle_model.py): a numpy float64 transformer written
-// independently from the formulas, permutation invariance over batch rows,
-// chunked prefill == token-by-token decode, seq_cp copy == source.
+// What pins this file (tests/test_oracle_model.py): logits of Hugging Face
+// transformers' LlamaForCausalLM, Qwen2ForCausalLM and Qwen3MoeForCausalLM in
+// float64 over the dequantised weights of synthetic files, committed as a
+// fixture (tests/golden/hf_reference_logits.npz: adjacent-pair and split-half
+// rotation, rope_freqs / linear scaling, biases, q/k-norm, the expert router,
+// LoRA pairs on all seven layer matrices merged into the dense weights); a
+// numpy float64 transformer written independently from the formulas;
+// permutation invariance over batch rows, chunked prefill == token-by-token
+// decode, seq_cp copy == source.
+// PARITY UNPINNED against the reference's own ggml build at float level: the
+// fork is absent and no reference test or fixture records absolute logits of
+// a causal model.
 #pragma once
 
 #include "gguf.hpp"

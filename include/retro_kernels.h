@@ -79,8 +79,9 @@ int32_t retro_kernel_max_topk(void);    /* candidates sample_prepare can return 
 /* Logits of the last step's sampling rows, [rows][n_vocab], in row order.
  * out == NULL only reports the row count. */
 int retro_engine_debug_logits(retro_engine * engine, float * out, size_t n_floats, size_t * out_rows);
-/* The stored f16 K (want_v = 0) or V row of (layer, slot, pos) in natural
- * element order: n_head_kv * head_dim halves. */
+/* The stored K (want_v = 0) or V row of (layer, slot, pos) in natural element order: n_head_kv * head_dim
+ * halves (an f16 cache), or - a Q8_0 cache - per kv head head_dim code bytes (code + 128) followed by
+ * head_dim / 32 f16 block scales, n_head_kv * (head_dim / 2 + head_dim / 32) 16-bit units in all. */
 int retro_engine_debug_kv(retro_engine * engine, int32_t layer, int32_t slot, int32_t pos, int32_t want_v,
                           uint16_t * out);
 /* The device-side packing of the last step: per-token arrays and

@@ -76,6 +76,9 @@ def _declare(l: C.CDLL) -> None:
     l.orc_ctx_new.restype = C.c_void_p
     l.orc_ctx_set_exact.argtypes = [C.c_void_p, C.c_int]
     l.orc_ctx_set_exact.restype = None
+    l.orc_ctx_set_kv_q8.argtypes = [C.c_void_p, C.c_int]
+    l.orc_ctx_set_kv_q8.restype = None
+    l.orc_ctx_read_kv_f32.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _f32p]
     l.orc_ctx_free.argtypes = [C.c_void_p]
     l.orc_ctx_free.restype = None
     l.orc_ctx_step.argtypes = [C.c_void_p, C.c_int, _i32p, _i32p, _i32p, _i32p, _u8p, _f32p]
@@ -254,7 +257,7 @@ class Model:
 
 
 class Context:
-    """Per-slot dense f16 KV and one decode per step() over a packed batch.
+    """Per-slot dense KV (f16, or Q8_0 blocks with kv="q8_0") and one decode per step() over a packed batch.
 
     activations: "exact" multiplies every weight with the f32 activations as they
     are (the product's default arithmetic, on which the logit tolerances are
@@ -262,14 +265,17 @@ class Context:
     Q8_0 codes, f16 / bf16 rounding: the reference's CPU arithmetic, which the
     product runs under RETRO_ACTIVATIONS=ggml)."""
 
-    def __init__(self, model: Model, n_seq_max: int, activations: str = "exact") -> None:
+    def __init__(self, model: Model, n_seq_max: int, activations: str = "exact", kv: str = "f16") -> None:
         if activations not in ("exact", "ggml"):
             raise ValueError("activations must be 'exact' or 'ggml'")
+        if kv not in ("f16", "q8_0"):
+            raise ValueError("kv must be 'f16' or 'q8_0'")
         self.model = model
         self._h = lib().orc_ctx_new(model._h, n_seq_max)
         if not self._h:
             raise OracleError(lib().orc_last_error().decode())
         lib().orc_ctx_set_exact(self._h, 1 if activations == "exact" else 0)
+        lib().orc_ctx_set_kv_q8(self._h, 1 if kv == "q8_0" else 0)
 
     def step(self, token, pos, slot, want, adapter_of=None) -> np.ndarray:
         token = np.ascontiguousarray(token, np.int32)
@@ -304,6 +310,12 @@ class Context:
         a, b = C.c_int32(), C.c_int32()
         _check(lib().orc_ctx_seq_pos(self._h, slot, C.byref(a), C.byref(b)))
         return a.value, b.value
+
+    def read_kv_values(self, layer, slot, pos, want_v=False) -> np.ndarray:
+        """The stored K or V row as the values the cache holds (f16-rounded, or scale times code of a Q8_0 cache)."""
+        out = np.empty(self.model.n_head_kv * self.model.head_dim, np.float32)
+        _check(lib().orc_ctx_read_kv_f32(self._h, layer, slot, pos, 1 if want_v else 0, _ptr(out, _f32p)))
+        return out
 
     def read_kv(self, layer, slot, pos, want_v=False) -> np.ndarray:
         out = np.empty(self.model.n_head_kv * self.model.head_dim, np.uint16)

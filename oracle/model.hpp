@@ -129,6 +129,19 @@ inline int nearest_int(float v) { return (int)std::nearbyint(v); }
 //   Q8_0 (quantize_row_q8_0_ref): per 32 values, d = amax / 127, code =
 //   roundf(x / d) (half away from zero) with the unrounded d, the value uses d
 //   rounded to f16.
+// A row as Q8_0 blocks hold it (quantize_row_q8_0_ref), written back as scale times code.
+inline void q8_0_row_values(const float * x, size_t K, float * out) {
+    if (K % 32) throw std::runtime_error("oracle: Q8_0 rows need whole blocks of 32");
+    for (size_t b = 0; b < K; b += 32) {
+        float amax = 0.0f;
+        for (int j = 0; j < 32; ++j) amax = std::fmax(amax, std::fabs(x[b + j]));
+        const float d = amax / 127.0f;
+        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        const float dh = half_to_float(float_to_half(d));
+        for (int j = 0; j < 32; ++j) out[b + j] = dh * std::round(x[b + j] * id);
+    }
+}
+
 inline void ggml_activation_row(uint32_t wtype, const float * x, size_t K, float * out) {
     if (exact_activations()) { std::copy(x, x + K, out); return; }
     switch (wtype) {
@@ -154,15 +167,7 @@ inline void ggml_activation_row(uint32_t wtype, const float * x, size_t K, float
         }
         case T_Q8_0:
         case T_MXFP4: {
-            if (K % 32) throw std::runtime_error("oracle: Q8_0 activations need K % 32 == 0");
-            for (size_t b = 0; b < K; b += 32) {
-                float amax = 0.0f;
-                for (int j = 0; j < 32; ++j) amax = std::fmax(amax, std::fabs(x[b + j]));
-                const float d = amax / 127.0f;
-                const float id = d != 0.0f ? 1.0f / d : 0.0f;
-                const float dh = half_to_float(float_to_half(d));
-                for (int j = 0; j < 32; ++j) out[b + j] = dh * std::round(x[b + j] * id);
-            }
+            q8_0_row_values(x, K, out);
             return;
         }
         case T_F16:
@@ -250,7 +255,9 @@ inline void rope(float * v, int head_dim, int rope_dim, int pos, double base, bo
 
 struct slot_state {
     int begin = 0, end = 0;              // resident positions [begin, end)
-    std::vector<std::vector<uint16_t>> k, v;   // per layer: pos * kv_dim halves, indexed by absolute pos
+    // per layer: pos * kv_dim values, indexed by absolute pos; the values the cache's storage type holds for what
+    // was written (f16 rounding, or scale times code of Q8_0 blocks), as floats
+    std::vector<std::vector<float>> k, v;
 };
 
 struct context {
@@ -266,6 +273,12 @@ struct context {
     // told otherwise, and what the logit tolerances are demonstrated on) or as ggml's CPU matmul
     // converts them (see ggml_activation_row).
     bool exact = true;
+    // Storage of the K and V cache: f16, or Q8_0 blocks of 32 along a head's row (the reference's kv_dtype;
+    // retro_engine.cpp:84-91 maps it to ggml's type_k / type_v). A row is quantised as quantize_row_q8_0_ref does
+    // (quant.hpp) when it is stored; attention then reads scale times code. Under the ggml arithmetic ggml's CPU
+    // flash attention would also convert the query row to Q8_0 for the K product (the vec_dot_type of Q8_0): done
+    // here when `exact` is off.
+    bool kv_q8 = false;
 
     int kv_dim() const { return mdl->hp.n_head_kv * mdl->hp.head_dim; }
 
@@ -403,11 +416,17 @@ struct context {
                     if (kn) rmsnorm(kh, f32_data(*kn), HD, h.eps, kh);
                     rope(kh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox, rope_factors);
                 }
-                uint16_t * kc = &s.k[(size_t)l][(size_t)pos[t] * kd];
-                uint16_t * vc = &s.v[(size_t)l][(size_t)pos[t] * kd];
-                for (int i = 0; i < KD; ++i) {
-                    kc[i] = float_to_half(k[(size_t)t * KD + i]);
-                    vc[i] = float_to_half(v[(size_t)t * KD + i]);
+                float * kc = &s.k[(size_t)l][(size_t)pos[t] * kd];
+                float * vc = &s.v[(size_t)l][(size_t)pos[t] * kd];
+                if (kv_q8) {
+                    if (HD % 32 != 0) throw std::runtime_error("oracle: a Q8_0 cache needs heads of whole 32-blocks");
+                    q8_0_row_values(&k[(size_t)t * KD], (size_t)KD, kc);
+                    q8_0_row_values(&v[(size_t)t * KD], (size_t)KD, vc);
+                } else {
+                    for (int i = 0; i < KD; ++i) {
+                        kc[i] = half_to_float(float_to_half(k[(size_t)t * KD + i]));
+                        vc[i] = half_to_float(float_to_half(v[(size_t)t * KD + i]));
+                    }
                 }
                 s.end = std::max(s.end, pos[t] + 1);
             }
@@ -420,12 +439,18 @@ struct context {
                     const int p0 = s.begin, p1 = pos[t] + 1;
                     const int kvh = hh / G;
                     const float * qh = &q[(size_t)t * QD + (size_t)hh * HD];
+                    std::vector<float> qconv;
+                    if (kv_q8 && !exact) {      // ggml: the query row as Q8_0, the companion format of a Q8_0 K row
+                        qconv.resize((size_t)HD);
+                        q8_0_row_values(qh, (size_t)HD, qconv.data());
+                        qh = qconv.data();
+                    }
                     std::vector<double> sc((size_t)(p1 - p0));
                     double mx = -INFINITY;
                     for (int p = p0; p < p1; ++p) {
-                        const uint16_t * kc = &s.k[(size_t)l][(size_t)p * kd + (size_t)kvh * HD];
+                        const float * kc = &s.k[(size_t)l][(size_t)p * kd + (size_t)kvh * HD];
                         double d = 0.0;
-                        for (int i = 0; i < HD; ++i) d += (double)qh[i] * half_to_float(kc[i]);
+                        for (int i = 0; i < HD; ++i) d += (double)qh[i] * kc[i];
                         d *= inv_sqrt;
                         sc[(size_t)(p - p0)] = d;
                         mx = std::max(mx, d);
@@ -434,9 +459,9 @@ struct context {
                     for (auto & e : sc) { e = std::exp(e - mx); den += e; }
                     std::vector<double> acc((size_t)HD, 0.0);
                     for (int p = p0; p < p1; ++p) {
-                        const uint16_t * vc = &s.v[(size_t)l][(size_t)p * kd + (size_t)kvh * HD];
+                        const float * vc = &s.v[(size_t)l][(size_t)p * kd + (size_t)kvh * HD];
                         const double w = sc[(size_t)(p - p0)];
-                        for (int i = 0; i < HD; ++i) acc[(size_t)i] += w * half_to_float(vc[i]);
+                        for (int i = 0; i < HD; ++i) acc[(size_t)i] += w * vc[i];
                     }
                     float * o = &att[(size_t)t * QD + (size_t)hh * HD];
                     for (int i = 0; i < HD; ++i) o[i] = (float)(acc[(size_t)i] / den);

@@ -147,6 +147,19 @@ void * orc_ctx_new(void * m, int n_seq_max) {
 }
 void orc_ctx_free(void * c) { delete (context *)c; }
 void orc_ctx_set_exact(void * c, int on) { ((context *)c)->exact = on != 0; }
+void orc_ctx_set_kv_q8(void * c, int on) { ((context *)c)->kv_q8 = on != 0; }
+// The stored K or V row of (layer, slot, pos) as the kv_dim values the cache holds, f32.
+int orc_ctx_read_kv_f32(void * c, int layer, int slot, int pos, int want_v, float * out) {
+    return guard([&] {
+        context * ctx = (context *)c;
+        const slot_state & s = ctx->slots.at((size_t)slot);
+        if (pos < s.begin || pos >= s.end) throw std::runtime_error("oracle: position not resident");
+        const size_t kd = (size_t)ctx->kv_dim();
+        const auto & src = want_v ? s.v.at((size_t)layer) : s.k.at((size_t)layer);
+        std::copy(src.begin() + (size_t)pos * kd, src.begin() + ((size_t)pos + 1) * kd, out);
+        return 0;
+    });
+}
 
 // adapter_of may be NULL (base model for every token); entries <= 0 mean base.
 int orc_ctx_step(void * c, int n_tokens, const int32_t * tok, const int32_t * pos, const int32_t * slot,
@@ -175,7 +188,7 @@ int orc_ctx_read_kv(void * c, int layer, int slot, int pos, int want_v, uint16_t
         if (pos < s.begin || pos >= s.end) throw std::runtime_error("oracle: position not resident");
         const size_t kd = (size_t)ctx->kv_dim();
         const auto & src = want_v ? s.v.at((size_t)layer) : s.k.at((size_t)layer);
-        std::copy(src.begin() + (size_t)pos * kd, src.begin() + ((size_t)pos + 1) * kd, out);
+        for (size_t i = 0; i < kd; ++i) out[i] = float_to_half(src[(size_t)pos * kd + i]);      // exact for an f16 cache
         return 0;
     });
 }
@@ -192,8 +205,10 @@ int orc_ctx_import_kv(void * c, int layer, int slot, int begin, int end, const u
         auto & kk = s.k.at((size_t)layer);
         auto & vv = s.v.at((size_t)layer);
         if (kk.size() < (size_t)end * kd) { kk.resize((size_t)end * kd); vv.resize((size_t)end * kd); }
-        std::copy(k_rows, k_rows + (size_t)(end - begin) * kd, kk.begin() + (size_t)begin * kd);
-        std::copy(v_rows, v_rows + (size_t)(end - begin) * kd, vv.begin() + (size_t)begin * kd);
+        for (size_t i = 0; i < (size_t)(end - begin) * kd; ++i) {
+            kk[(size_t)begin * kd + i] = half_to_float(k_rows[i]);
+            vv[(size_t)begin * kd + i] = half_to_float(v_rows[i]);
+        }
         s.begin = begin;
         s.end = end;
         return 0;

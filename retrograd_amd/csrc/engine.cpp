@@ -94,12 +94,14 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     // n_ctx distinct cells always finds its pages.
     n_pages_ = (int)((cfg_.n_ctx + rk::PAGE - 1) / rk::PAGE + 2 * cfg_.n_seq_max);
     // [page][kv head]: the other order (a head's pages side by side) was measured 3 % slower in the attention kernel
-    kv_strides_ = rk::kv_strides(n_pages_, hp_.n_head_kv, hp_.head_dim, false);
+    kv_q8_ = cfg_.kv_dtype == RETRO_ENGINE_KV_DTYPE_Q8_0;
+    if (kv_q8_ && hp_.head_dim % 32 != 0) throw std::runtime_error("a Q8_0 KV cache needs head_dim to be a multiple of 32");
+    kv_strides_ = rk::kv_strides(n_pages_, hp_.n_head_kv, hp_.head_dim, false, kv_q8_);
     const int G = hp_.n_head / hp_.n_head_kv;
     if (hp_.n_head % hp_.n_head_kv != 0 || G > 16) throw std::runtime_error("unsupported attention head grouping");
     qt_ = rk::attention_tile_tokens(G);
 
-    const size_t pool_halves = (size_t)n_pages_ * hp_.n_head_kv * rk::PAGE * hp_.head_dim;
+    const size_t pool_halves = (size_t)n_pages_ * hp_.n_head_kv * rk::kv_block_halves(hp_.head_dim, kv_q8_);
     k_pool_.resize((size_t)hp_.n_layer);
     v_pool_.resize((size_t)hp_.n_layer);
     const size_t pool_bytes = (pool_halves * 2 + 255) / 256 * 256;
@@ -454,7 +456,7 @@ void Engine::release_page(int32_t page) {
 void Engine::copy_page(int32_t src, int32_t dst) {
     for (int l = 0; l < hp_.n_layer; ++l) {
         rk::kv_copy_page(stream_, k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), kv_strides_,
-                         hp_.n_head_kv, hp_.head_dim, src, dst);
+                         hp_.n_head_kv, hp_.head_dim, src, dst, kv_q8_);
     }
 }
 
@@ -564,7 +566,7 @@ bool Engine::seq_cp(int32_t src, int32_t dst, int32_t p0, int32_t p1) {
                 cells_src.push_back(sp * rk::PAGE + p % rk::PAGE);
                 cells_dst.push_back(target * rk::PAGE + p % rk::PAGE);
             }
-            const size_t kd = (size_t)hp_.n_head_kv * hp_.head_dim;
+            const size_t kd = rk::kv_row_halves(hp_.n_head_kv, hp_.head_dim, kv_q8_);      // halves of a cell's row
             DevBuf cs, cd, tmp;
             cs.alloc(cells_src.size() * 4);
             cd.alloc(cells_dst.size() * 4);
@@ -574,8 +576,8 @@ bool Engine::seq_cp(int32_t src, int32_t dst, int32_t p0, int32_t p1) {
             for (int l = 0; l < hp_.n_layer; ++l) {
                 for (int v = 0; v < 2; ++v) {
                     __half * pool = v ? v_pool_[(size_t)l].as<__half>() : k_pool_[(size_t)l].as<__half>();
-                    rk::kv_gather(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, cs.as<int32_t>(), (int)cells_src.size(), tmp.as<__half>());
-                    rk::kv_scatter(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, cd.as<int32_t>(), (int)cells_dst.size(), tmp.as<__half>());
+                    rk::kv_gather(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, cs.as<int32_t>(), (int)cells_src.size(), tmp.as<__half>(), kv_q8_);
+                    rk::kv_scatter(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, cd.as<int32_t>(), (int)cells_dst.size(), tmp.as<__half>(), kv_q8_);
                 }
             }
             hip_check(hipStreamSynchronize(stream_), "seq_cp merge");
@@ -623,12 +625,13 @@ int Engine::memory(retro_engine_memory_info * out) {
 // ---- snapshots -------------------------------------------------------------------------
 //
 // Byte format (this library's own; only seq_load of the same build reads it):
-//   u32 magic "RKV1", u32 flags, i32 n_layer, i32 kv_dim, i32 begin, i32 end,
-//   then per layer the K rows [end-begin][kv_dim] and the V rows, f16, in
-//   natural element order.
+//   u32 magic "RKV1" (an f16 cache) or "RKV8" (a Q8_0 cache), u32 flags, i32 n_layer, i32 halves per row,
+//   i32 begin, i32 end, then per layer the K rows [end-begin] and the V rows: kv_dim f16 values in
+//   natural order, or - Q8_0 - per kv head head_dim code bytes (code + 128) and head_dim / 32 f16 scales.
 namespace {
 struct SnapHeader { uint32_t magic, flags; int32_t n_layer, kv_dim, begin, end; };
 constexpr uint32_t kSnapMagic = 0x31564b52u;
+constexpr uint32_t kSnapMagicQ8 = 0x38564b52u;
 }
 
 int Engine::seq_save(int32_t slot, uint32_t flags, uint8_t * buffer, size_t n_buffer, size_t * out_n_bytes) {
@@ -645,7 +648,7 @@ int Engine::seq_save(int32_t slot, uint32_t flags, uint8_t * buffer, size_t n_bu
         return -1;
     }
     const Slot & s = slots_[(size_t)slot];
-    const size_t kd = (size_t)hp_.n_head_kv * hp_.head_dim;
+    const size_t kd = rk::kv_row_halves(hp_.n_head_kv, hp_.head_dim, kv_q8_);
     const bool partial_only = (flags & RETRO_STATE_SEQ_FLAGS_PARTIAL_ONLY) != 0;
     const int n_pos = partial_only ? 0 : std::max(0, s.end - s.begin);   // no recurrent or SWA state exists
     const size_t required = sizeof(SnapHeader) + (size_t)hp_.n_layer * 2 * (size_t)n_pos * kd * 2;
@@ -655,7 +658,7 @@ int Engine::seq_save(int32_t slot, uint32_t flags, uint8_t * buffer, size_t n_bu
         set_error("the save buffer is too small for this sequence's state");
         return -2;
     }
-    SnapHeader h{kSnapMagic, flags, hp_.n_layer, (int32_t)kd, partial_only ? 0 : s.begin, partial_only ? 0 : s.begin + n_pos};
+    SnapHeader h{kv_q8_ ? kSnapMagicQ8 : kSnapMagic, flags, hp_.n_layer, (int32_t)kd, partial_only ? 0 : s.begin, partial_only ? 0 : s.begin + n_pos};
     std::memcpy(buffer, &h, sizeof(h));
     if (n_pos > 0) {
         std::vector<int32_t> cells((size_t)n_pos);
@@ -668,7 +671,7 @@ int Engine::seq_save(int32_t slot, uint32_t flags, uint8_t * buffer, size_t n_bu
         for (int l = 0; l < hp_.n_layer; ++l) {
             for (int v = 0; v < 2; ++v) {
                 const __half * pool = v ? v_pool_[(size_t)l].as<__half>() : k_pool_[(size_t)l].as<__half>();
-                rk::kv_gather(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, dc.as<int32_t>(), n_pos, tmp.as<__half>());
+                rk::kv_gather(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, dc.as<int32_t>(), n_pos, tmp.as<__half>(), kv_q8_);
                 hip_check(hipMemcpyAsync(at, tmp.ptr, tmp.bytes, hipMemcpyDeviceToHost, stream_), "hipMemcpyAsync");
                 hip_check(hipStreamSynchronize(stream_), "seq_save");
                 at += tmp.bytes;
@@ -699,8 +702,8 @@ int Engine::seq_load(int32_t slot, uint32_t flags, const uint8_t * buffer, size_
     SnapHeader h;
     if (n_bytes < sizeof(h)) { set_error(refused); return -1; }
     std::memcpy(&h, buffer, sizeof(h));
-    const size_t kd = (size_t)hp_.n_head_kv * hp_.head_dim;
-    if (h.magic != kSnapMagic || h.flags != flags || h.n_layer != hp_.n_layer || h.kv_dim != (int32_t)kd
+    const size_t kd = rk::kv_row_halves(hp_.n_head_kv, hp_.head_dim, kv_q8_);
+    if (h.magic != (kv_q8_ ? kSnapMagicQ8 : kSnapMagic) || h.flags != flags || h.n_layer != hp_.n_layer || h.kv_dim != (int32_t)kd
             || h.begin < 0 || h.end < h.begin || h.end > n_ctx_seq_) {
         set_error(refused);
         return -1;
@@ -734,7 +737,7 @@ int Engine::seq_load(int32_t slot, uint32_t flags, const uint8_t * buffer, size_
             for (int v = 0; v < 2; ++v) {
                 __half * pool = v ? v_pool_[(size_t)l].as<__half>() : k_pool_[(size_t)l].as<__half>();
                 hip_check(hipMemcpyAsync(tmp.ptr, at, tmp.bytes, hipMemcpyHostToDevice, stream_), "hipMemcpyAsync");
-                rk::kv_scatter(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, dc.as<int32_t>(), n_pos, tmp.as<__half>());
+                rk::kv_scatter(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, v != 0, dc.as<int32_t>(), n_pos, tmp.as<__half>(), kv_q8_);
                 hip_check(hipStreamSynchronize(stream_), "seq_load");
                 at += tmp.bytes;
             }
@@ -1209,7 +1212,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
 void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_rows, bool routed) {
     const HParams & h = hp_;
     const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim, F = h.n_ff;
-    rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps, kv_strides_.page, kv_strides_.head};
+    rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps, kv_strides_.page, kv_strides_.head, kv_q8_, kv_q8_ && ggml_activations_};
     // The versions of a row its consumers need: the values themselves for F32 / F16 / BF16 weights, the
     // expert router and LoRA factors (`plain`); the converted row for the quantised weights.
     const bool faithful = ggml_activations_;
@@ -1774,13 +1777,14 @@ int Engine::debug_read_kv(int layer, int32_t slot, int32_t pos, int want_v, uint
         return -1;
     }
     const int32_t cell = s.pages[(size_t)(pos / rk::PAGE)] * rk::PAGE + pos % rk::PAGE;
-    const size_t kd = (size_t)hp_.n_head_kv * hp_.head_dim;
+    // the row as kv_gather writes it: kv_dim f16 values, or (a Q8_0 cache) per kv head the code bytes and block scales
+    const size_t kd = rk::kv_row_halves(hp_.n_head_kv, hp_.head_dim, kv_q8_);
     DevBuf dc, tmp;
     dc.alloc(4);
     tmp.alloc(kd * 2);
     hip_check(hipMemcpy(dc.ptr, &cell, 4, hipMemcpyHostToDevice), "hipMemcpy");
     const __half * pool = want_v ? v_pool_[(size_t)layer].as<__half>() : k_pool_[(size_t)layer].as<__half>();
-    rk::kv_gather(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, want_v != 0, dc.as<int32_t>(), 1, tmp.as<__half>());
+    rk::kv_gather(stream_, pool, kv_strides_, hp_.n_head_kv, hp_.head_dim, want_v != 0, dc.as<int32_t>(), 1, tmp.as<__half>(), kv_q8_);
     hip_check(hipStreamSynchronize(stream_), "debug_read_kv");
     hip_check(hipMemcpy(out, tmp.ptr, kd * 2, hipMemcpyDeviceToHost), "hipMemcpy");
     return 0;

@@ -265,6 +265,7 @@ private:
     uint64_t prof_n_[PC_COUNT] = {};
     size_t prof_begin(int cat);
     int mm_single_mask_ = 0;
+    bool kv_q8_ = false;       // the KV pools hold Q8_0 blocks (kv_dtype Q8_0)
     void prof_end(int cat, size_t token);
     void prof_resolve();
 

@@ -1307,10 +1307,13 @@ struct RopeArgs {
     float eps, qscale;
     Slices from;
     size_t page_stride, head_stride;
+    int kv_q8;
+    int q_q8;        // the ggml arithmetic over a Q8_0 cache: the query row is converted to Q8_0 as well
 };
 
 // One wave per head: lanes own element pairs.
 __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
+    __shared__ float stash[4][128];          // Q8_0 cache: a head's row in element order, per wave
     const int t = blockIdx.x;
     const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
@@ -1368,8 +1371,38 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
         x0 = r0;
         x1 = r1;
     }
+    // Q8_0 blocks want neighbours where lanes hold rotation pairs: through LDS, then lane L owns elements 2 L and
+    // 2 L + 1 and sixteen lanes a block of 32. d = amax / 127, code = roundf(x / d) with the unrounded d (ggml's
+    // quantize_row_q8_0_ref); returns the codes, d through `d`.
+    auto q8_pair = [&](float & v0, float & v1, float & d) {
+        float * mine = stash[threadIdx.x >> 6];
+        mine[i0] = x0;
+        mine[i1] = x1;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        v0 = mine[2 * lane];
+        v1 = mine[2 * lane + 1];
+        float amax = fmaxf(fabsf(v0), fabsf(v1));
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+        d = __fdiv_rn(amax, 127.0f);
+        const float id = d != 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
+        v0 = roundf(__fmul_rn(v0, id));
+        v1 = roundf(__fmul_rn(v1, id));
+    };
     if (is_q) {
         const size_t at = (size_t)t * QD + (size_t)head * a.hd;
+        if (a.q_q8) {
+            // the query row as Q8_0, the companion format of a Q8_0 K row in ggml's CPU attention: scale times code
+            float c0, c1, d;
+            q8_pair(c0, c1, d);
+            const float dh = __half2float(__float2half_rn(d));
+            x0 = __fmul_rn(dh, c0);
+            x1 = __fmul_rn(dh, c1);
+            i0 = 2 * lane;
+            i1 = i0 + 1;
+        }
         const float s0 = fminf(fmaxf(x0 * a.qscale, -65504.0f), 65504.0f);
         const float s1 = fminf(fmaxf(x1 * a.qscale, -65504.0f), 65504.0f);
         const __half h0 = __float2half_rn(s0), h1 = __float2half_rn(s1);
@@ -1382,6 +1415,25 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
     const int cell = a.cell[t];
     const int page = cell / PAGE, t32 = cell % PAGE;
     const int kvh = is_k ? head - a.n_head : head - a.n_head - a.n_kv;
+    if (a.kv_q8) {
+        float c0, c1, d;
+        q8_pair(c0, c1, d);
+        const int e = 2 * lane;
+        const uint32_t b0 = (uint32_t)((int)c0 + 128), b1 = (uint32_t)((int)c1 + 128);
+        uint8_t * blk = (uint8_t *)((is_k ? a.k_pool : a.v_pool) + (size_t)page * a.page_stride + (size_t)kvh * a.head_stride);
+        const int tg = (t32 & 15) >> 2, ti = (t32 & 3) + 4 * (t32 >> 4);      // the token's place among a lane's eight
+        const int blk_idx = e >> 5;
+        if (is_k) {
+            const int g = (e >> 3) & 3, i = e & 7;
+            *(uint16_t *)(blk + blk_idx * 1024 + (g * 16 + (t32 & 15)) * 16 + (t32 >> 4) * 8 + i) = (uint16_t)(b0 | (b1 << 8));
+        } else {
+            const int hi = (e >> 4) & 1, dd = e & 15;
+            blk[blk_idx * 1024 + (tg * 16 + dd) * 16 + hi * 8 + ti] = (uint8_t)b0;
+            blk[blk_idx * 1024 + (tg * 16 + dd + 1) * 16 + hi * 8 + ti] = (uint8_t)b1;
+        }
+        if ((lane & 15) == 0) ((__half *)(blk + (a.hd / 32) * 1024))[blk_idx * 32 + tg * 8 + ti] = __float2half_rn(d);
+        return;
+    }
     if (is_k) {
         __half * dst = a.k_pool + (size_t)page * a.page_stride + (size_t)kvh * a.head_stride;
         dst[k_page_offset(a.hd, t32, i0)] = sat_half(x0);
@@ -1407,6 +1459,8 @@ void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, c
     a.qscale = 1.4426950408889634f / sqrtf((float)sh.head_dim);
     a.from = from;
     a.page_stride = sh.page_stride; a.head_stride = sh.head_stride;
+    a.kv_q8 = sh.kv_q8 ? 1 : 0;
+    a.q_q8 = sh.kv_q8 && sh.q_q8 ? 1 : 0;
     if (sh.page_stride == 0 || sh.head_stride == 0) throw std::runtime_error("rope_store: the pool's strides are missing");
     if (from.n > 0 && from.N != (sh.n_head + 2 * sh.n_head_kv) * sh.head_dim)
         throw std::runtime_error("rope_store: the slices are not a fused q, k, v product");
@@ -1417,6 +1471,19 @@ void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, c
 
 // ---------------------------------------------------------------------------
 // paged attention
+
+// The K (V) blocks a wave holds for one page: f16 operands, or - a Q8_0 cache - code bytes and block scales.
+template <int N, bool Q8> struct KvRegs { h8 r[N]; };
+template <int N> struct KvRegs<N, true> { u4 raw[N / 2]; u4 sc[N / 2]; };
+// Eight bytes (code + 128) as eight f16 codes: 0x6400 | byte is 1024 + byte, exactly.
+__device__ __forceinline__ h8 codes8(uint32_t w0, uint32_t w1) {
+    const h2 bias = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
+    const h2 a0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04010400u)) + bias;
+    const h2 a1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u)) + bias;
+    const h2 a2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u)) + bias;
+    const h2 a3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)) + bias;
+    return (h8){a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+}
 
 struct AttnArgs {
     const __half * q;
@@ -1442,7 +1509,10 @@ struct AttnArgs {
 // arithmetic of a column does not depend on ONE or on what else is in its tile, so a token's result is the
 // same bits in a decode step and in a mixed step. Without SPLIT a tile holds 16 / G tokens and the lo halves
 // take a second instruction each.
-template <int HD, bool ONE, bool SPLIT>
+// Q8: the pools hold Q8_0 blocks (kernels.hpp). K enters the score products as its codes, one 32-wide k-step
+// being one block, and the block's scale multiplies that step's products; V enters as its codes and its scales
+// join the probabilities, one version of the probability operand per 32-wide block of dimensions.
+template <int HD, bool ONE, bool SPLIT, bool Q8 = false>
 __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     constexpr int KS = HD / 32;     // k-steps of QK^T
     constexpr int DT = HD / 16;     // dim tiles of PV
@@ -1483,23 +1553,62 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     // page ids of this split, one per lane
     const int n_pages = page_end - page_first;
     const int my_pid = lane < n_pages ? a.table[(size_t)slot * a.max_pages + page_first + lane] : 0;
-    auto load_k = [&](int idx, h8 (&kreg)[KS][2]) {
+    typedef KvRegs<2 * KS, Q8> KSet;          // f16: [k-step][token half]
+    typedef KvRegs<DT, Q8> VSet;
+    auto load_k = [&](int idx, KSet & ks) {
         const int pid = __builtin_amdgcn_readlane(my_pid, idx);
         const __half * kp = a.k_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
+        if constexpr (Q8) {
+            const uint8_t * kb = (const uint8_t *)kp;
 #pragma unroll
-        for (int j = 0; j < KS; ++j) {
-            kreg[j][0] = load_h8(kp + ((j * 2 + 0) * 64 + lane) * 8);
-            kreg[j][1] = load_h8(kp + ((j * 2 + 1) * 64 + lane) * 8);
+            for (int j = 0; j < KS; ++j) {
+                ks.raw[j] = *(const u4 *)(kb + j * 1024 + lane * 16);
+                ks.sc[j] = *(const u4 *)(kb + KS * 1024 + (j * 4 + g) * 16);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < KS; ++j) {
+                ks.r[2 * j] = load_h8(kp + ((j * 2 + 0) * 64 + lane) * 8);
+                ks.r[2 * j + 1] = load_h8(kp + ((j * 2 + 1) * 64 + lane) * 8);
+            }
         }
     };
-    auto load_v = [&](int idx, h8 (&vreg)[DT]) {
+    auto load_v = [&](int idx, VSet & vs) {
         const int pid = __builtin_amdgcn_readlane(my_pid, idx);
         const __half * vp = a.v_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
+        if constexpr (Q8) {
+            const uint8_t * vb = (const uint8_t *)vp;
 #pragma unroll
-        for (int d = 0; d < DT; ++d) vreg[d] = load_h8(vp + (d * 64 + lane) * 8);
+            for (int b = 0; b < KS; ++b) {
+                vs.raw[b] = *(const u4 *)(vb + b * 1024 + lane * 16);
+                vs.sc[b] = *(const u4 *)(vb + KS * 1024 + (b * 4 + g) * 16);
+            }
+        } else {
+#pragma unroll
+            for (int d = 0; d < DT; ++d) vs.r[d] = load_h8(vp + (d * 64 + lane) * 8);
+        }
     };
-    auto attend = [&](int pi, const h8 (&kreg)[KS][2], const h8 (&vreg)[DT]) {
-        if (a.debug & 1) {       // timing experiment: the loads alone
+    auto attend = [&](int pi, const KSet & ks, const VSet & vs) {
+        h8 kreg[KS][2], vreg[DT];
+        float dk[KS][8], dv[KS][8];      // Q8: the scales of this lane's eight tokens, per block
+        if constexpr (Q8) {
+#pragma unroll
+            for (int j = 0; j < KS; ++j) {
+                kreg[j][0] = codes8(ks.raw[j].x, ks.raw[j].y);
+                kreg[j][1] = codes8(ks.raw[j].z, ks.raw[j].w);
+                vreg[2 * j] = codes8(vs.raw[j].x, vs.raw[j].y);
+                vreg[2 * j + 1] = codes8(vs.raw[j].z, vs.raw[j].w);
+                const h8 sk = __builtin_bit_cast(h8, ks.sc[j]), sv = __builtin_bit_cast(h8, vs.sc[j]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) { dk[j][i] = (float)sk[i]; dv[j][i] = (float)sv[i]; }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < KS; ++j) { kreg[j][0] = ks.r[2 * j]; kreg[j][1] = ks.r[2 * j + 1]; }
+#pragma unroll
+            for (int d = 0; d < DT; ++d) vreg[d] = vs.r[d];
+        }
+        if (!Q8 && (a.debug & 1)) {       // timing experiment: the loads alone
             h8 t = kreg[0][0];
 #pragma unroll
             for (int j = 0; j < KS; ++j) { t += kreg[j][0]; t += kreg[j][1]; }
@@ -1511,11 +1620,26 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
         f4 s0 = (f4){0.f, 0.f, 0.f, 0.f}, s1 = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int j = 0; j < KS; ++j) {
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg[j], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg[j], s1, 0, 0, 0);
-            if (!SPLIT) {
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg_lo[j], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg_lo[j], s1, 0, 0, 0);
+            if constexpr (Q8) {
+                const f4 zero = (f4){0.f, 0.f, 0.f, 0.f};
+                f4 u0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg[j], zero, 0, 0, 0);
+                f4 u1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg[j], zero, 0, 0, 0);
+                if (!SPLIT) {
+                    u0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg_lo[j], u0, 0, 0, 0);
+                    u1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg_lo[j], u1, 0, 0, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    s0[i] = fmaf(dk[j][i], u0[i], s0[i]);
+                    s1[i] = fmaf(dk[j][4 + i], u1[i], s1[i]);
+                }
+            } else {
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg[j], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg[j], s1, 0, 0, 0);
+                if (!SPLIT) {
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg_lo[j], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg_lo[j], s1, 0, 0, 0);
+                }
             }
         }
         if (SPLIT) {
@@ -1550,20 +1674,27 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
         const float m_use = m_new == -INFINITY ? 0.0f : m_new;
         const float alpha = !col_ok ? 1.0f : exp2f(m_run - m_use);       // m_run = -inf -> 0
         float psum = 0.0f;
-        h8 pt, pt_lo;                                   // probabilities as f16 hi/lo pairs
+        float e[8];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float e0 = exp2f(s0[i] - m_use);
-            const float e1 = exp2f(s1[i] - m_use);
-            const _Float16 h0 = (_Float16)e0, h1 = (_Float16)e1;
-            const _Float16 l0 = (_Float16)(e0 - (float)h0), l1 = (_Float16)(e1 - (float)h1);
-            // SPLIT: the column of the lo query half multiplies the lo half of the same probabilities
-            pt[i] = lo_col ? l0 : h0;
-            pt[4 + i] = lo_col ? l1 : h1;
-            pt_lo[i] = l0;
-            pt_lo[4 + i] = l1;
-            psum += e0 + e1;
+            e[i] = exp2f(s0[i] - m_use);
+            e[4 + i] = exp2f(s1[i] - m_use);
+            psum += e[i] + e[4 + i];
         }
+        // the probabilities (Q8: times the V scale of the token in block `b`) as f16 hi/lo pairs
+        auto operand = [&](int b, h8 & pt, h8 & pt_lo) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float p = Q8 ? e[i] * dv[Q8 ? b : 0][i] : e[i];
+                const _Float16 hi = (_Float16)p;
+                const _Float16 lo = (_Float16)(p - (float)hi);
+                // SPLIT: the column of the lo query half multiplies the lo half of the same probabilities
+                pt[i] = lo_col ? lo : hi;
+                pt_lo[i] = lo;
+            }
+        };
+        h8 pt, pt_lo;
+        if constexpr (!Q8) operand(0, pt, pt_lo);
         m_run = m_new;
         // the running maximum rarely moves after the first pages: then every column's factor is exactly one,
         // and multiplying by it would change nothing
@@ -1577,6 +1708,9 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
         l_run += psum;
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
+            if constexpr (Q8) {
+                if ((d & 1) == 0) operand(d >> 1, pt, pt_lo);
+            }
             o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt, o[d], 0, 0, 0);
             if (!SPLIT) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt_lo, o[d], 0, 0, 0);
         }
@@ -1589,7 +1723,8 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     // before the scores needed it and the next K page before the products did - nothing was in flight while a
     // page was computed.
     if (n_pages > 0) {
-        h8 kA[KS][2], kB[KS][2], v[DT];
+        KSet kA, kB;
+        VSet v;
         load_k(0, kA);
         for (int i = 0; i < n_pages; i += 2) {
             load_v(i, v);
@@ -1639,12 +1774,14 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
     if (sh.page_stride == 0 || sh.head_stride == 0) throw std::runtime_error("attention: the pool's strides are missing");
     { static const int dbg = [] { const char * v = std::getenv("RETRO_ATTN_DEBUG"); return v ? std::atoi(v) : 0; }(); a.debug = dbg; }
     if (a.G > 16 || sh.n_head % sh.n_head_kv != 0) throw std::runtime_error("attention: unsupported head grouping");
-#define ATTN_LAUNCH(HD_) \
+#define ATTN_LAUNCH_Q(HD_, Q8_) \
     do { \
-        if (a.G <= 8 && one_token_rows) hipLaunchKernelGGL((k_attention<HD_, true, true>), dim3(n_items), dim3(64), 0, s, a); \
-        else if (a.G <= 8) hipLaunchKernelGGL((k_attention<HD_, false, true>), dim3(n_items), dim3(64), 0, s, a); \
-        else hipLaunchKernelGGL((k_attention<HD_, false, false>), dim3(n_items), dim3(64), 0, s, a); \
+        if (a.G <= 8 && one_token_rows) hipLaunchKernelGGL((k_attention<HD_, true, true, Q8_>), dim3(n_items), dim3(64), 0, s, a); \
+        else if (a.G <= 8) hipLaunchKernelGGL((k_attention<HD_, false, true, Q8_>), dim3(n_items), dim3(64), 0, s, a); \
+        else hipLaunchKernelGGL((k_attention<HD_, false, false, Q8_>), dim3(n_items), dim3(64), 0, s, a); \
     } while (0)
+#define ATTN_LAUNCH(HD_) \
+    do { if (sh.kv_q8) ATTN_LAUNCH_Q(HD_, true); else ATTN_LAUNCH_Q(HD_, false); } while (0)
     switch (sh.head_dim) {
         case 32:  ATTN_LAUNCH(32); break;
         case 64:  ATTN_LAUNCH(64); break;
@@ -1652,6 +1789,7 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
         default: throw std::runtime_error("attention: head_dim must be 32, 64 or 128");
     }
 #undef ATTN_LAUNCH
+#undef ATTN_LAUNCH_Q
     check_launch("attention");
 }
 
@@ -1812,9 +1950,45 @@ __global__ void k_kv_gather(const __half * pool, KvStrides st, int n_kv, int hd,
     else out[gid] = *cache;
 }
 
+// The Q8_0 pool: one 16-bit unit per thread - a pair of code bytes (elements 2u, 2u + 1 of the head's row) or,
+// past the codes, one block scale. Rows of kv_row_halves units.
+__global__ void k_kv_gather_q8(const __half * pool, KvStrides st, int n_kv, int hd, int is_v, const int32_t * cells, int n,
+                               uint16_t * out, int scatter) {
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int per_head = hd / 2 + hd / 32;
+    if (gid >= (size_t)n * n_kv * per_head) return;
+    const int idx = (int)(gid / ((size_t)n_kv * per_head)), rest = (int)(gid % ((size_t)n_kv * per_head));
+    const int kvh = rest / per_head, u = rest % per_head;
+    const int cell = cells[idx];
+    const int page = cell / PAGE, t32 = cell % PAGE;
+    uint8_t * blk = (uint8_t *)(const_cast<__half *>(pool) + (size_t)page * st.page + (size_t)kvh * st.head);
+    const int tg = (t32 & 15) >> 2, ti = (t32 & 3) + 4 * (t32 >> 4);
+    if (u >= hd / 2) {
+        uint16_t * sc = (uint16_t *)(blk + (hd / 32) * 1024) + (u - hd / 2) * 32 + tg * 8 + ti;
+        if (scatter) *sc = out[gid]; else out[gid] = *sc;
+        return;
+    }
+    const int e = 2 * u, b = e >> 5;
+    if (!is_v) {
+        uint16_t * c = (uint16_t *)(blk + b * 1024 + (((e >> 3) & 3) * 16 + (t32 & 15)) * 16 + (t32 >> 4) * 8 + (e & 7));
+        if (scatter) *c = out[gid]; else out[gid] = *c;
+    } else {
+        uint8_t * c0 = blk + b * 1024 + (tg * 16 + (e & 15)) * 16 + ((e >> 4) & 1) * 8 + ti;
+        if (scatter) { c0[0] = (uint8_t)(out[gid] & 0xff); c0[16] = (uint8_t)(out[gid] >> 8); }
+        else out[gid] = (uint16_t)(c0[0] | (c0[16] << 8));
+    }
+}
+
 void kv_gather(hipStream_t s, const __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
-               const int32_t * cells, int n, __half * out) {
+               const int32_t * cells, int n, __half * out, bool q8) {
     if (n <= 0) return;
+    if (q8) {
+        const size_t total = (size_t)n * kv_row_halves(n_kv_heads, head_dim, true);
+        hipLaunchKernelGGL(k_kv_gather_q8, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, st, n_kv_heads,
+                           head_dim, is_v ? 1 : 0, cells, n, (uint16_t *)out, 0);
+        check_launch("kv_gather");
+        return;
+    }
     const size_t total = (size_t)n * n_kv_heads * head_dim;
     hipLaunchKernelGGL(k_kv_gather, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, st, n_kv_heads,
                        head_dim, is_v ? 1 : 0, cells, n, out, 0);
@@ -1822,8 +1996,15 @@ void kv_gather(hipStream_t s, const __half * pool, KvStrides st, int n_kv_heads,
 }
 
 void kv_scatter(hipStream_t s, __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
-                const int32_t * cells, int n, const __half * in) {
+                const int32_t * cells, int n, const __half * in, bool q8) {
     if (n <= 0) return;
+    if (q8) {
+        const size_t total = (size_t)n * kv_row_halves(n_kv_heads, head_dim, true);
+        hipLaunchKernelGGL(k_kv_gather_q8, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, st, n_kv_heads,
+                           head_dim, is_v ? 1 : 0, cells, n, (uint16_t *)const_cast<__half *>(in), 1);
+        check_launch("kv_scatter");
+        return;
+    }
     const size_t total = (size_t)n * n_kv_heads * head_dim;
     hipLaunchKernelGGL(k_kv_gather, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, st, n_kv_heads,
                        head_dim, is_v ? 1 : 0, cells, n, const_cast<__half *>(in), 1);
@@ -1840,8 +2021,8 @@ __global__ void k_kv_copy_page(__half * k_pool, __half * v_pool, size_t head_hal
 }
 
 void kv_copy_page(hipStream_t s, __half * k_pool, __half * v_pool, KvStrides st, int n_kv_heads, int head_dim,
-                  int src_page, int dst_page) {
-    const size_t head_halves = (size_t)PAGE * head_dim;       // one head's share of a page
+                  int src_page, int dst_page, bool q8) {
+    const size_t head_halves = kv_block_halves(head_dim, q8);       // one head's share of a page (a multiple of 8)
     hipLaunchKernelGGL(k_kv_copy_page, dim3((unsigned)((head_halves / 8 + 255) / 256), n_kv_heads), dim3(256), 0, s,
                        k_pool, v_pool, head_halves, st, src_page, dst_page);
     check_launch("kv_copy_page");

@@ -273,12 +273,31 @@ struct AttnShape {
     float eps;
     // element strides of a KV pool between pages and between the kv heads of a page (see kv_strides)
     size_t page_stride = 0, head_stride = 0;
+    bool kv_q8 = false;        // the pools hold Q8_0 blocks (see kv_block_halves)
+    bool q_q8 = false;         // ... and the query rows are converted to Q8_0 too (ggml's CPU attention over such a cache)
 };
-// A pool holds, per page and kv head, PAGE positions x head_dim halves. head_major: [kv head][page], else [page][kv head].
+// A pool holds one block per page and kv head, PAGE positions of one head. f16: PAGE x head_dim halves in the
+// operand orders of the attention kernel. Q8_0 (blocks of 32 along the head's row, one f16 scale each, as the
+// reference's kv_dtype Q8_0 stores a row): head_dim / 32 loads of 1 KiB of codes, a code as the byte code + 128,
+// then head_dim / 32 groups of 32 f16 scales; 17/32 of the f16 block.
+//   K codes  [j = dim / 32][lane = g * 16 + t][16 B]: bytes 0-7 dims 32 j + 8 g + (0..7) of token t, bytes 8-15 of token 16 + t
+//   V codes  [p = dim / 32][lane = g * 16 + d][16 B]: bytes 0-7 dim 32 p + d, bytes 8-15 dim 32 p + 16 + d, byte i of
+//            either the token 4 g + i (i < 4) or 16 + 4 g + (i - 4)
+//   scales   [j or p][g][8]: the scale of block j (p) of token 4 g + i (i < 4) or 16 + 4 g + (i - 4)
+// All strides and sizes are in halves (2 bytes), also for Q8_0.
+inline size_t kv_block_halves(int head_dim, bool q8) {
+    return q8 ? (size_t)(head_dim / 32) * 544 : (size_t)PAGE * head_dim;
+}
+// head_major: [kv head][page], else [page][kv head].
 struct KvStrides { size_t page, head; };
-inline KvStrides kv_strides(int n_pages, int n_kv_heads, int head_dim, bool head_major) {
-    const size_t unit = (size_t)PAGE * head_dim;
+inline KvStrides kv_strides(int n_pages, int n_kv_heads, int head_dim, bool head_major, bool q8 = false) {
+    const size_t unit = kv_block_halves(head_dim, q8);
     return head_major ? KvStrides{unit, (size_t)n_pages * unit} : KvStrides{(size_t)n_kv_heads * unit, unit};
+}
+// Halves of one cell's K (or V) row over all kv heads in the natural order kv_gather writes: f16 values, or per
+// head head_dim code bytes (code + 128) followed by head_dim / 32 f16 scales.
+inline size_t kv_row_halves(int n_kv_heads, int head_dim, bool q8) {
+    return q8 ? (size_t)n_kv_heads * (head_dim / 2 + head_dim / 32) : (size_t)n_kv_heads * head_dim;
 }
 // qkv f32 [T][QD + 2*KD] (+ optional per-head RMSNorm weights) -> q as an f16
 // hi/lo pair [T][QD] each (rotated, pre-scaled by log2(e)/sqrt(head_dim)) and
@@ -302,12 +321,12 @@ size_t attention_partial_floats(int n_items, int head_dim);
 // Gathers the K or V row of one (layer pool, cell) into natural order, and the
 // inverse; used by sequence snapshots and by tests.
 void kv_gather(hipStream_t s, const __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
-               const int32_t * cells, int n, __half * out);
+               const int32_t * cells, int n, __half * out, bool q8 = false);
 void kv_scatter(hipStream_t s, __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
-                const int32_t * cells, int n, const __half * in);
-// Copies the first `count` positions of page src to page dst in one layer pool.
+                const int32_t * cells, int n, const __half * in, bool q8 = false);
+// Copies page src to page dst in one layer's pools.
 void kv_copy_page(hipStream_t s, __half * k_pool, __half * v_pool, KvStrides st, int n_kv_heads, int head_dim,
-                  int src_page, int dst_page);
+                  int src_page, int dst_page, bool q8 = false);
 
 // ---- sampling -------------------------------------------------------------------
 struct SampleOut {          // one per output row, read back by the host

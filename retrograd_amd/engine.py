@@ -752,6 +752,22 @@ class Engine:
             _raise(s)
         return out.view(np.float16)
 
+    def debug_kv_q8(self, layer: int, slot: int, pos: int, want_v: bool, n_kv: int, head_dim: int) -> np.ndarray:
+        """The K or V row of a Q8_0 cache as the values it stands for (scale times code), f32, kv_dim of them."""
+        per_head = head_dim // 2 + head_dim // 32
+        raw = np.empty(n_kv * per_head, np.uint16)
+        s = self._lib.retro_engine_debug_kv(self._h, layer, slot, pos, 1 if want_v else 0,
+                                            raw.ctypes.data_as(C.POINTER(C.c_uint16)))
+        if s != 0:
+            _raise(s)
+        out = np.empty((n_kv, head_dim), np.float32)
+        for h in range(n_kv):
+            row = raw[h * per_head:(h + 1) * per_head]
+            codes = row[:head_dim // 2].view(np.uint8).astype(np.int32) - 128
+            scales = row[head_dim // 2:].view(np.float16).astype(np.float32)
+            out[h] = (codes.reshape(-1, 32) * scales[:, None]).reshape(-1)
+        return out.reshape(-1)
+
     def debug_pack(self, cap_tokens: int, cap_rows: int) -> dict:
         arrs = {k: np.full(cap_tokens, -7, np.int32) for k in ("token", "pos", "seq", "cell", "out_index")}
         last = np.full(cap_rows, -7, np.int32)

@@ -47,7 +47,8 @@ def ggml_activations(v, weight_type):
 
 
 class NumpyModel:
-    def __init__(self, path, activations="exact"):
+    def __init__(self, path, activations="exact", kv="f16"):
+        self.kv = kv          # "f16", or "q8_0": K and V rows stored as Q8_0 blocks of 32 along a head's row
         """activations: "exact" (the f32 values are multiplied) or "ggml" (converted first)."""
         self.ggml = activations == "ggml"
         r = Reader(path)
@@ -130,8 +131,16 @@ class NumpyModel:
                 k = self.norm(k, self.t(b + "attn_k_norm.weight"))
             q = np.stack([self.rope(q[t], pos0 + t) for t in range(T)])
             k = np.stack([self.rope(k[t], pos0 + t) for t in range(T)])
-            k = k.astype(np.float16).astype(np.float64)   # f16 KV cache
-            v = v.astype(np.float16).astype(np.float64)
+            if self.kv == "q8_0":
+                # blocks of 32 never straddle heads (head_dim is a multiple of 32); under the ggml arithmetic the
+                # query row meets a Q8_0 K row converted to Q8_0 itself
+                k = ggml_activations(k.astype(np.float32), Q8_0)
+                v = ggml_activations(v.astype(np.float32), Q8_0)
+                if self.ggml:
+                    q = ggml_activations(q.astype(np.float32), Q8_0)
+            else:
+                k = k.astype(np.float16).astype(np.float64)   # f16 KV cache
+                v = v.astype(np.float16).astype(np.float64)
             att = np.zeros((T, self.H, self.D))
             for hh in range(self.H):
                 s = q[:, hh] @ k[:, hh // G].T / np.sqrt(self.D)

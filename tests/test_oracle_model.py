@@ -158,6 +158,31 @@ def test_lora_delta_matches_dense_formula_and_rank_padding(models, tmp_path, act
     assert np.abs(want_ad - want_base).max() > 1e-3   # the adapter does something
 
 
+@pytest.mark.parametrize("activations", ["exact", "ggml"])
+def test_a_q8_0_cache_holds_the_reference_quantisers_blocks_and_attention_reads_them(models, activations):
+    """kv="q8_0": K and V rows are stored as quantize_row_q8_0_ref blocks (32 values along a head's row, f16
+    scale) and attention reads scale times code; under the ggml arithmetic the query row is converted as well.
+    Pinned by the fixture-pinned row quantiser (what is stored is a fixed point of it, on its grid) and by the
+    float64 numpy transformer with its own numpy quantiser. Against the reference's ggml build: parity unpinned."""
+    m = oracle.Model(models["qwen2-q8"])
+    rng = np.random.default_rng(12)
+    toks = rng.integers(0, m.n_vocab, 40)
+    c = oracle.Context(m, 1, activations=activations, kv="q8_0")
+    got = c.step_rows([(0, 0, toks, True)])[0]
+    for layer, pos, want_v in ((0, 0, False), (0, 39, True), (1, 17, False), (1, 33, True)):
+        row = c.read_kv_values(layer, 0, pos, want_v)
+        blocks = np.frombuffer(oracle.quantize_q8_0(row), np.uint8).reshape(-1, 34)
+        again = blocks[:, :2].copy().view(np.float16).astype(np.float32) * blocks[:, 2:].view(np.int8).astype(np.float32)
+        assert np.array_equal(again.reshape(-1), row)
+        assert np.abs(blocks[:, 2:].view(np.int8)).max(axis=1).min() == 127 or (row.reshape(-1, 32) == 0).all(axis=1).any()
+    nm = NumpyModel(models["qwen2-q8"], activations=activations, kv="q8_0")
+    want = nm.forward(toks)[-1]
+    # a code on a rounding boundary may fall either way between the two (f32 against float64 rows): looser than the f16 comparison
+    assert np.abs(got - want).max() < 2e-3 * max(1.0, np.abs(want).max())
+    f16 = oracle.Context(m, 1, activations=activations).step_rows([(0, 0, toks, True)])[0]
+    assert np.abs(f16 - got).max() > 20 * np.abs(got - want).max(), "the cache type moves the logits far more than the two disagree"
+
+
 # ---- the forward pass against Hugging Face transformers ------------------------------------------------
 
 def _hf_golden():

@@ -59,6 +59,8 @@ def parse_args():
     ap.add_argument("--activations", default="exact", choices=["exact", "ggml"],
                     help="arithmetic of the measured engine: exact (f16 hi/lo activations, the default and the one the "
                          "logit tolerances are shown on) or ggml (activations converted to Q8_K / Q8_0 as the reference's CPU path does)")
+    ap.add_argument("--kv", default="f16", choices=["f16", "q8_0"],
+                    help="storage of the KV cache; the headline is f16 as the workload names it, q8_0 is a secondary configuration")
     ap.add_argument("--kernel-steps", type=int, default=8, help="decode steps timed per kernel category after the timed region")
     ap.add_argument("--no-scheduler-leg", action="store_true", help="skip the run of the same workload through the step scheduler")
     ap.add_argument("--scheduler-requests", type=int, default=128)
@@ -338,7 +340,8 @@ def main() -> int:
     def new_engine(activations):
         os.environ["RETRO_ACTIVATIONS"] = activations
         t0 = time.perf_counter()
-        eng = E.Engine(model_path, E.EngineConfig(n_ctx=n_ctx, n_seq_max=n_slots, n_batch=n_batch, n_ubatch=n_batch))
+        eng = E.Engine(model_path, E.EngineConfig(n_ctx=n_ctx, n_seq_max=n_slots, n_batch=n_batch, n_ubatch=n_batch,
+                                                  kv_dtype=E.KV_Q8_0 if args.kv == "q8_0" else E.KV_F16))
         print("[bench] engine (%s arithmetic) ready in %.1fs" % (activations, time.perf_counter() - t0), file=sys.stderr, flush=True)
         return eng
 
@@ -353,12 +356,14 @@ def main() -> int:
 
     # ---- roofline of the attention kernel (the largest single launch: one per layer), over the timed region
     hp = shape
-    kv_bytes_per_cell_layer = 2 * hp.n_head_kv * hp.head_dim * 2
+    kv_bytes_per_cell_layer = 2 * hp.n_head_kv * hp.head_dim * 2       # K and V, f16
+    if args.kv == "q8_0":
+        kv_bytes_per_cell_layer = kv_bytes_per_cell_layer * 17 // 32      # 34 bytes per block of 32 values
     attn_ms, attn_launches = prof["attention"]
     algo_bytes_per_launch = kv_bytes_per_cell_layer * cells / args.steps
     attn_avg_s = attn_ms / max(attn_launches, 1) * 1e-3
     attn_gbs = algo_bytes_per_launch / attn_avg_s / 1e9 if attn_avg_s > 0 else 0.0
-    ratio = read_traffic_ratio(args.traffic_file, shape.name)
+    ratio = read_traffic_ratio(args.traffic_file, shape.name) if args.kv == "f16" else None      # measured on the f16 kernel
 
     # ---- whole-step roofline (north star): weights once + KV of every attended cell
     w_bytes = synth.streamed_weight_bytes(hp)       # every dense matrix once, at its stored type
@@ -411,13 +416,14 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("q4_k" if args.shape != "c2-q4km" else "q4_k / q6_k") + " weights x " + arithmetic + ", f32 accumulate, f16 KV",
+        "dtype": ("q4_k" if args.shape != "c2-q4km" else "q4_k / q6_k") + " weights x " + arithmetic + ", f32 accumulate, " + ("f16 KV" if args.kv == "f16" else "Q8_0 KV (a secondary configuration: the workload names an f16 cache)"),
         "data": "synthetic",
         "config": {
             "workload": "configs[1]: %s, %d live sequences, prompts log-uniform [%d,%d], greedy, %d new tokens, continuous batching"
                         % (shape.name, n_slots, len_lo, len_hi, max_new),
             "n_batch": n_batch,
             "activations": args.activations,
+            "kv_cache": args.kv,
             "mean_decode_rows_per_step": round(decode_rows / args.steps, 2),
             "mean_tokens_per_step": round(tokens / args.steps, 2),
             "mean_kv_cells_attended_per_step": round(cells / args.steps, 1),
@@ -456,7 +462,7 @@ def main() -> int:
             "%s=%.3f" % (k, v[0] / args.steps) for k, v in prof.items()), file=sys.stderr, flush=True)
 
     if not args.no_cpu_baseline:
-        result["cpu_baseline"], result["parity_full_size"] = cpu_baseline(eng, E, oracle, wl, model_path, args.cpu_rows, args.activations)
+        result["cpu_baseline"], result["parity_full_size"] = cpu_baseline(eng, E, oracle, wl, model_path, args.cpu_rows, args.activations, kv=args.kv)
     else:
         result["cpu_baseline"] = None
 
@@ -479,7 +485,7 @@ def main() -> int:
                "step_frac_of_hbm_roofline": round((s2 / e2) / ((s2 / args.steps) / (b2 / (HBM_PEAK_GBS * 1e9))), 4),
                "arithmetic": "RETRO_ACTIVATIONS=ggml: Q8_K / Q8_0 activation conversion before every quantised matmul"}
         if not args.no_cpu_baseline:
-            _, leg["parity_full_size_against_the_oracle_in_the_same_arithmetic"] = cpu_baseline(eng, E, oracle, wl2, model_path, args.cpu_rows, "ggml", time_it=False)
+            _, leg["parity_full_size_against_the_oracle_in_the_same_arithmetic"] = cpu_baseline(eng, E, oracle, wl2, model_path, args.cpu_rows, "ggml", time_it=False, kv=args.kv)
         result["ggml_arithmetic"] = leg
         eng.close()
     os.environ["RETRO_ACTIVATIONS"] = "exact"
@@ -488,13 +494,13 @@ def main() -> int:
     return 0
 
 
-def cpu_baseline(eng, E, oracle, wl, model_path, n_rows, activations="exact", time_it=True):
+def cpu_baseline(eng, E, oracle, wl, model_path, n_rows, activations="exact", time_it=True, kv="f16"):
     """Times the CPU oracle on one decode step over the first n_rows live
     sequences of the same workload (their KV imported from the engine's own
     snapshots), and compares its logits with the engine's for the same rows."""
     live = [s for s in wl.seqs if s is not None and s.last_token is not None][:n_rows]
     model = oracle.Model(model_path)
-    ctx = oracle.Context(model, max(s.slot for s in live) + 1, activations=activations)
+    ctx = oracle.Context(model, max(s.slot for s in live) + 1, activations=activations, kv=kv)
     t0 = time.perf_counter()
     for s in live:
         ctx.import_snapshot(s.slot, eng.seq_save(s.slot))

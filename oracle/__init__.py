@@ -79,6 +79,7 @@ def _declare(l: C.CDLL) -> None:
     l.orc_ctx_set_kv_q8.argtypes = [C.c_void_p, C.c_int]
     l.orc_ctx_set_kv_q8.restype = None
     l.orc_ctx_read_kv_f32.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _f32p]
+    l.orc_ctx_import_kv_f32.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _f32p, _f32p]
     l.orc_ctx_free.argtypes = [C.c_void_p]
     l.orc_ctx_free.restype = None
     l.orc_ctx_step.argtypes = [C.c_void_p, C.c_int, _i32p, _i32p, _i32p, _i32p, _u8p, _f32p]
@@ -336,6 +337,22 @@ class Context:
         n = end - begin
         body = np.frombuffer(snapshot, np.uint16, offset=24)
         per = n * kd
+        if int(head[0]) == 0x38564b52:
+            # a Q8_0 cache ("RKV8"): per row and kv head head_dim code bytes (code + 128), then head_dim / 32 f16 scales
+            hd, n_kv = self.model.head_dim, self.model.n_head_kv
+            per_head = hd // 2 + hd // 32
+            assert kd == n_kv * per_head
+
+            def values(units):
+                rows = units.reshape(n, n_kv, per_head)
+                codes = np.ascontiguousarray(rows[:, :, :hd // 2]).view(np.uint8).astype(np.float32) - 128.0
+                scales = np.ascontiguousarray(rows[:, :, hd // 2:]).view(np.float16).astype(np.float32)
+                return np.ascontiguousarray((codes.reshape(n, n_kv, hd // 32, 32) * scales[..., None]).reshape(n, n_kv * hd))
+            for l in range(n_layer):
+                k = values(body[(2 * l) * per:(2 * l + 1) * per])
+                v = values(body[(2 * l + 1) * per:(2 * l + 2) * per])
+                _check(lib().orc_ctx_import_kv_f32(self._h, l, slot, begin, end, _ptr(k, _f32p), _ptr(v, _f32p)))
+            return
         for l in range(n_layer):
             k = body[(2 * l) * per:(2 * l + 1) * per]
             v = body[(2 * l + 1) * per:(2 * l + 2) * per]

@@ -215,6 +215,23 @@ int orc_ctx_import_kv(void * c, int layer, int slot, int begin, int end, const u
     });
 }
 
+// The same with the rows given as the f32 values the cache holds (a Q8_0 cache's scale times code).
+int orc_ctx_import_kv_f32(void * c, int layer, int slot, int begin, int end, const float * k_rows, const float * v_rows) {
+    return guard([&] {
+        context * ctx = (context *)c;
+        slot_state & s = ctx->slots.at((size_t)slot);
+        const size_t kd = (size_t)ctx->kv_dim();
+        auto & kk = s.k.at((size_t)layer);
+        auto & vv = s.v.at((size_t)layer);
+        if (kk.size() < (size_t)end * kd) { kk.resize((size_t)end * kd); vv.resize((size_t)end * kd); }
+        std::copy(k_rows, k_rows + (size_t)(end - begin) * kd, kk.begin() + (size_t)begin * kd);
+        std::copy(v_rows, v_rows + (size_t)(end - begin) * kd, vv.begin() + (size_t)begin * kd);
+        s.begin = begin;
+        s.end = end;
+        return 0;
+    });
+}
+
 // ---- sampling --------------------------------------------------------------
 void * orc_rng_new(uint32_t seed) { return new std::mt19937(seed); }
 void orc_rng_free(void * r) { delete (std::mt19937 *)r; }

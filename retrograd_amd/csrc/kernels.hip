@@ -751,7 +751,9 @@ __device__ __forceinline__ float lora_operand(float hi, float lo, int type) {
     return v;
 }
 
-// mid[t][r] = sum_k A[r][k] * x[t][k]: one wave per (token, r), lanes own groups of eight k.
+// mid[t][r] = sum_k A[r][k] * x[t][k]: one workgroup per (token, four rank rows); its 256 threads stride over k in
+// groups of eight, so the activations are read once for the four rows, and the partial sums meet through LDS.
+// (Both LoRA products in one workgroup per token were measured slower: too few workgroups for the chain of loads.)
 // Up to three targets that read the same activations (q, k, v) share a launch: blockIdx.z picks the target.
 struct LoraTargets {
     const LoraEntry * table[3];
@@ -762,52 +764,80 @@ struct LoraTargets {
 __global__ __launch_bounds__(256) void k_lora_down(LoraTargets tg, const RowDesc * __restrict__ rows,
                                                    const int32_t * __restrict__ tok_row, Act x, float * __restrict__ mid_all,
                                                    int T) {
+    __shared__ float red[4][4];
     const int t = blockIdx.x;
     const int route = rows[tok_row[t]].route;
     if (route <= 0) return;
     const LoraEntry e = tg.table[blockIdx.z][route - 1];
+    const int r0 = blockIdx.y * 4;
+    if (!e.A || r0 >= e.rank) return;                     // the same for every thread of the workgroup
     float * mid = mid_all + (size_t)blockIdx.z * T * LORA_MAX_RANK;
-    const int r = blockIdx.y * 4 + (threadIdx.x >> 6);
-    if (!e.A || r >= e.rank) return;
-    const int lane = threadIdx.x & 63;
-    const float * a = e.A + (size_t)r * x.K;
-    float acc = 0.0f;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nr = min(4, e.rank - r0);
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (x.K % 8 == 0) {
-        for (int k = lane * 8; k < x.K; k += 512) {
+        for (int k = threadIdx.x * 8; k < x.K; k += 2048) {
             const h8 hi = load_h8(x.x + act_at(t, k, 0, x.K)), lo = load_h8(x.x + act_at(t, k, 1, x.K));
-            const f4 a0 = *(const f4 *)(a + k), a1 = *(const f4 *)(a + k + 4);
+            float v[8];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc = fmaf(a0[i], lora_operand((float)hi[i], (float)lo[i], e.a_type), acc);
-                acc = fmaf(a1[i], lora_operand((float)hi[4 + i], (float)lo[4 + i], e.a_type), acc);
+            for (int i = 0; i < 8; ++i) v[i] = lora_operand((float)hi[i], (float)lo[i], e.a_type);
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                if (rr >= nr) break;
+                const float * a = e.A + (size_t)(r0 + rr) * x.K + k;
+                const f4 a0 = *(const f4 *)a, a1 = *(const f4 *)(a + 4);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[rr] = fmaf(a0[i], v[i], acc[rr]);
+                    acc[rr] = fmaf(a1[i], v[4 + i], acc[rr]);
+                }
             }
         }
     } else {
-        for (int k = lane; k < x.K; k += 64)
-            acc = fmaf(a[k], lora_operand(__half2float(x.x[act_at(t, k, 0, x.K)]), __half2float(x.x[act_at(t, k, 1, x.K)]), e.a_type), acc);
+        for (int k = threadIdx.x; k < x.K; k += 256) {
+            const float v = lora_operand(__half2float(x.x[act_at(t, k, 0, x.K)]), __half2float(x.x[act_at(t, k, 1, x.K)]), e.a_type);
+            for (int rr = 0; rr < nr; ++rr) acc[rr] = fmaf(e.A[(size_t)(r0 + rr) * x.K + k], v, acc[rr]);
+        }
     }
-    acc = wave_sum(acc);
-    if (lane == 0) mid[(size_t)t * LORA_MAX_RANK + r] = acc;
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+        const float s = wave_sum(acc[rr]);
+        if (lane == 0) red[wave][rr] = s;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < nr) mid[(size_t)t * LORA_MAX_RANK + r0 + threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
 }
 
 // y[t][col0 + n] += scale * sum_r B[n][r] * mid[t][r]
 __global__ __launch_bounds__(256) void k_lora_up(LoraTargets tg, const RowDesc * __restrict__ rows,
                                                  const int32_t * __restrict__ tok_row, const float * __restrict__ mid_all,
                                                  float * __restrict__ y, int ldy, int T) {
+    __shared__ float ops[LORA_MAX_RANK];        // mid[t][r] as the factor B multiplies, once per workgroup
     const int t = blockIdx.x;
     const int route = rows[tok_row[t]].route;
     if (route <= 0) return;
     const LoraEntry e = tg.table[blockIdx.z][route - 1];
     const int N = tg.N[blockIdx.z], col0 = tg.col0[blockIdx.z];
-    const float * mid = mid_all + (size_t)blockIdx.z * T * LORA_MAX_RANK;
+    if (!e.A) return;
+    const float * m = mid_all + (size_t)blockIdx.z * T * LORA_MAX_RANK + (size_t)t * LORA_MAX_RANK;
+    if ((int)threadIdx.x < e.rank) {
+        const float v = m[threadIdx.x];
+        const float hi = (float)(_Float16)fminf(fmaxf(v, -65504.0f), 65504.0f);
+        ops[threadIdx.x] = lora_operand(hi, v - hi, e.b_type);
+    }
+    __syncthreads();
     const int n = blockIdx.y * 256 + threadIdx.x;
-    if (!e.A || n >= N) return;
+    if (n >= N) return;
     const float * b = e.B + (size_t)n * e.rank;
-    const float * m = mid + (size_t)t * LORA_MAX_RANK;
     float acc = 0.0f;
-    for (int r = 0; r < e.rank; ++r) {
-        const float hi = (float)(_Float16)fminf(fmaxf(m[r], -65504.0f), 65504.0f);
-        acc = fmaf(b[r], lora_operand(hi, m[r] - hi, e.b_type), acc);
+    if (e.rank % 4 == 0) {
+        for (int r = 0; r < e.rank; r += 4) {
+            const f4 b4 = *(const f4 *)(b + r);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc = fmaf(b4[i], ops[r + i], acc);
+        }
+    } else {
+        for (int r = 0; r < e.rank; ++r) acc = fmaf(b[r], ops[r], acc);
     }
     const int col = tg.group > 0 ? (n / tg.group) * 2 * tg.group + n % tg.group : n;
     y[(size_t)t * ldy + col0 + col] += e.scale * acc;

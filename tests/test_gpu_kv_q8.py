@@ -145,3 +145,33 @@ def test_cache_types_this_library_does_not_hold_are_refused(models):
     for dtype in (E.KV_F32, E.KV_Q4_0):
         with pytest.raises(E.EngineError, match="only the f16 and the q8_0 KV cache"):
             E.Engine(models["llama-hd64"], E.EngineConfig(n_ctx=256, n_seq_max=2, n_batch=64, n_ubatch=64, kv_dtype=dtype))
+
+
+def test_a_trainers_quantised_generation_context_decodes_like_an_engine_with_the_same_cache(models):
+    """generation_kv_dtype = Q8_0 (reference tests/engine_runtime.rs:218-238 compares a trainer's quantised generation
+    context with an engine of the same kv_dtype bit for bit): tokens and log-probabilities of a greedy continuation."""
+    from retrograd_amd import trainer as T
+    tr = T.Trainer(models["llama-hd64"], T.TrainConfig(n_ctx=128, n_batch=128, generation_concurrency=2, generation_kv_dtype=1))
+    eng = E.Engine(models["llama-hd64"], E.EngineConfig(n_ctx=256, n_seq_max=2, n_batch=128, n_ubatch=128, kv_dtype=E.KV_Q8_0))
+    f16 = E.Engine(models["llama-hd64"], E.EngineConfig(n_ctx=256, n_seq_max=2, n_batch=128, n_ubatch=128))
+    rng = np.random.default_rng(9)
+    prompts = [rng.integers(0, 1024, n) for n in (40, 23)]
+
+    def run(h):
+        out = E.StepOutput()
+        h.step([E.StepRow(i, i, prompts[i], 0, sample=True, sampling=greedy()) for i in range(2)], out)
+        toks = [[r.token] for r in out.rows()]
+        lps = [[np.float32(r.logprob).view(np.uint32)] for r in out.rows()]
+        for step in range(5):
+            h.step([E.StepRow(i, i, [toks[i][-1]], len(prompts[i]) + step, sample=True, sampling=greedy()) for i in range(2)], out)
+            for i, r in enumerate(out.rows()):
+                toks[i].append(r.token)
+                lps[i].append(np.float32(r.logprob).view(np.uint32))
+        return toks, lps
+    a, b, c = run(tr), run(eng), run(f16)
+    assert a == b
+    assert c[1] != a[1], "an f16 cache gives other log-probabilities"
+    assert tr.memory().kv_bytes * 32 == f16.memory().kv_bytes * 17 or abs(tr.memory().kv_bytes / f16.memory().kv_bytes - 17 / 32) < 1e-3
+    with pytest.raises(E.EngineError, match="only the f16 and the q8_0 KV cache"):
+        T.Trainer(models["llama-hd64"], T.TrainConfig(n_ctx=128, n_batch=128, generation_concurrency=2, generation_kv_dtype=2))
+    tr.close(); eng.close(); f16.close()

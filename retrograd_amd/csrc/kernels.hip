@@ -1620,19 +1620,9 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     };
     auto attend = [&](int pi, const KSet & ks, const VSet & vs) {
         h8 kreg[KS][2], vreg[DT];
-        float dk[KS][8], dv[KS][8];      // Q8: the scales of this lane's eight tokens, per block
-        if constexpr (Q8) {
-#pragma unroll
-            for (int j = 0; j < KS; ++j) {
-                kreg[j][0] = codes8(ks.raw[j].x, ks.raw[j].y);
-                kreg[j][1] = codes8(ks.raw[j].z, ks.raw[j].w);
-                vreg[2 * j] = codes8(vs.raw[j].x, vs.raw[j].y);
-                vreg[2 * j + 1] = codes8(vs.raw[j].z, vs.raw[j].w);
-                const h8 sk = __builtin_bit_cast(h8, ks.sc[j]), sv = __builtin_bit_cast(h8, vs.sc[j]);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) { dk[j][i] = (float)sk[i]; dv[j][i] = (float)sv[i]; }
-            }
-        } else {
+        // Q8: the scales of this lane's eight tokens per block stay packed (ks.sc, vs.sc) and are widened where used,
+        // and the codes are widened one k-step (dim-tile pair) at a time: fewer registers, a third wave per SIMD
+        if constexpr (!Q8) {
 #pragma unroll
             for (int j = 0; j < KS; ++j) { kreg[j][0] = ks.r[2 * j]; kreg[j][1] = ks.r[2 * j + 1]; }
 #pragma unroll
@@ -1652,16 +1642,18 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
         for (int j = 0; j < KS; ++j) {
             if constexpr (Q8) {
                 const f4 zero = (f4){0.f, 0.f, 0.f, 0.f};
-                f4 u0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg[j], zero, 0, 0, 0);
-                f4 u1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg[j], zero, 0, 0, 0);
+                const h8 k0 = codes8(ks.raw[j].x, ks.raw[j].y), k1 = codes8(ks.raw[j].z, ks.raw[j].w);
+                f4 u0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0, qreg[j], zero, 0, 0, 0);
+                f4 u1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1, qreg[j], zero, 0, 0, 0);
                 if (!SPLIT) {
-                    u0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg_lo[j], u0, 0, 0, 0);
-                    u1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg_lo[j], u1, 0, 0, 0);
+                    u0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0, qreg_lo[j], u0, 0, 0, 0);
+                    u1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1, qreg_lo[j], u1, 0, 0, 0);
                 }
+                const h8 dk = __builtin_bit_cast(h8, ks.sc[j]);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    s0[i] = fmaf(dk[j][i], u0[i], s0[i]);
-                    s1[i] = fmaf(dk[j][4 + i], u1[i], s1[i]);
+                    s0[i] = fmaf((float)dk[i], u0[i], s0[i]);
+                    s1[i] = fmaf((float)dk[4 + i], u1[i], s1[i]);
                 }
             } else {
                 s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg[j], s0, 0, 0, 0);
@@ -1713,9 +1705,11 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
         }
         // the probabilities (Q8: times the V scale of the token in block `b`) as f16 hi/lo pairs
         auto operand = [&](int b, h8 & pt, h8 & pt_lo) {
+            h8 dv;
+            if constexpr (Q8) dv = __builtin_bit_cast(h8, vs.sc[b]);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float p = Q8 ? e[i] * dv[Q8 ? b : 0][i] : e[i];
+                const float p = Q8 ? e[i] * (float)dv[i] : e[i];
                 const _Float16 hi = (_Float16)p;
                 const _Float16 lo = (_Float16)(p - (float)hi);
                 // SPLIT: the column of the lo query half multiplies the lo half of the same probabilities
@@ -1738,11 +1732,15 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
         l_run += psum;
 #pragma unroll
         for (int d = 0; d < DT; ++d) {
+            h8 vd;
             if constexpr (Q8) {
                 if ((d & 1) == 0) operand(d >> 1, pt, pt_lo);
+                vd = (d & 1) ? codes8(vs.raw[d >> 1].z, vs.raw[d >> 1].w) : codes8(vs.raw[d >> 1].x, vs.raw[d >> 1].y);
+            } else {
+                vd = vreg[d];
             }
-            o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt, o[d], 0, 0, 0);
-            if (!SPLIT) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt_lo, o[d], 0, 0, 0);
+            o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vd, pt, o[d], 0, 0, 0);
+            if (!SPLIT) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vd, pt_lo, o[d], 0, 0, 0);
         }
     };
     // V of a page loads while its scores are computed, K of the next page while

@@ -95,6 +95,12 @@ int retro_trainer_eos_token(retro_trainer * trainer, int32_t * out_token);
 int retro_trainer_vocab_size(retro_trainer * trainer, uint32_t * out_n_vocab);
 int retro_trainer_is_eog_token(retro_trainer * trainer, int32_t token, bool * out_is_eog);
 int retro_trainer_context_size(retro_trainer * trainer, uint32_t * out_n_ctx);
+/* :1604-1632: text -> token ids on the generation engine's vocabulary, the twins of retro_engine_tokenize_text,
+ * retro_engine_tokenize_fragment and retro_engine_tokenize (same two-call contract and return codes). */
+int retro_trainer_tokenize_text(retro_trainer * trainer, const char * text, int32_t * tokens, size_t n_tokens_max, size_t * out_n_tokens);
+int retro_trainer_tokenize_fragment(retro_trainer * trainer, const char * text, int32_t * tokens, size_t n_tokens_max, size_t * out_n_tokens);
+int retro_trainer_tokenize_with(retro_trainer * trainer, const char * text, bool add_special, bool parse_special, int32_t * tokens,
+                                size_t n_tokens_max, size_t * out_n_tokens);
 int retro_trainer_detokenize(retro_trainer * trainer, const int32_t * tokens, size_t n_tokens, bool unparse_special,
                              char * buffer, size_t n_buffer, size_t * out_n_bytes);
 

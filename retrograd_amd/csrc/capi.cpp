@@ -340,6 +340,63 @@ int retro_engine_is_hybrid(retro_engine * engine, bool * out_is_hybrid) {
     });
 }
 
+// Two-call contract of the reference's tokenize_into (retro_engine.cpp:331-378): with no buffer (or no room at all)
+// the count is reported and the call succeeds; a buffer that is too small is -2 with the count.
+static int tokenize_into(Engine & e, const char * text, bool add_special, bool parse_special, int32_t * tokens,
+                         size_t n_tokens_max, size_t * out_n_tokens) {
+    if (!text || text[0] == '\0') {
+        set_error("text is required");
+        return -1;
+    }
+    if (!out_n_tokens) {
+        set_error("out_n_tokens is required");
+        return -1;
+    }
+    if (std::strlen(text) > (size_t)INT32_MAX) {
+        set_error("text is too large to tokenize");
+        return -1;
+    }
+    const Vocab & v = e.vocab();
+    if (!v.tokenizer_error.empty()) {
+        set_error("this model's vocabulary cannot tokenize: " + v.tokenizer_error);
+        return -1;
+    }
+    const std::vector<int32_t> ids = v.tokenizer.tokenize(text, add_special, parse_special);     // throws for a vocabulary kind that is not built
+    *out_n_tokens = ids.size();
+    if (!tokens || n_tokens_max == 0) return 0;
+    if (ids.size() > n_tokens_max) return -2;
+    std::copy(ids.begin(), ids.end(), tokens);
+    return 0;
+}
+
+/* text with BOS / EOS as the model asks, special-token texts read as tokens (ref retro_engine.cpp:594-607) */
+int retro_engine_tokenize_text(retro_engine * engine, const char * text, int32_t * tokens, size_t n_tokens_max, size_t * out_n_tokens) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return tokenize_into(*e, text, true, true, tokens, n_tokens_max, out_n_tokens);
+    });
+}
+
+/* the same without BOS / EOS (ref retro_engine.cpp:609-622) */
+int retro_engine_tokenize_fragment(retro_engine * engine, const char * text, int32_t * tokens, size_t n_tokens_max, size_t * out_n_tokens) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return tokenize_into(*e, text, false, true, tokens, n_tokens_max, out_n_tokens);
+    });
+}
+
+/* both flags explicit (ref retro_lora_train.h:2879-2889) */
+int retro_engine_tokenize(retro_engine * engine, const char * text, bool add_special, bool parse_special, int32_t * tokens,
+                          size_t n_tokens_max, size_t * out_n_tokens) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        return tokenize_into(*e, text, add_special, parse_special, tokens, n_tokens_max, out_n_tokens);
+    });
+}
+
 int retro_engine_eos_token(retro_engine * engine, int32_t * out_token) {
     return boundary([&]() -> int {
         Engine * e = checked(engine);

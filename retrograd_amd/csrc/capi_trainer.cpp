@@ -160,6 +160,16 @@ int retro_trainer_context_size(retro_trainer * trainer, uint32_t * out_n_ctx) {
         return 0;
     });
 }
+int retro_trainer_tokenize_text(retro_trainer * trainer, const char * text, int32_t * tokens, size_t n_tokens_max, size_t * out_n_tokens) {
+    TWIN(retro_engine_tokenize_text(e, text, tokens, n_tokens_max, out_n_tokens));
+}
+int retro_trainer_tokenize_fragment(retro_trainer * trainer, const char * text, int32_t * tokens, size_t n_tokens_max, size_t * out_n_tokens) {
+    TWIN(retro_engine_tokenize_fragment(e, text, tokens, n_tokens_max, out_n_tokens));
+}
+int retro_trainer_tokenize_with(retro_trainer * trainer, const char * text, bool add_special, bool parse_special, int32_t * tokens,
+                                size_t n_tokens_max, size_t * out_n_tokens) {
+    TWIN(retro_engine_tokenize(e, text, add_special, parse_special, tokens, n_tokens_max, out_n_tokens));
+}
 int retro_trainer_detokenize(retro_trainer * trainer, const int32_t * tokens, size_t n_tokens, bool unparse_special,
                              char * buffer, size_t n_buffer, size_t * out_n_bytes) {
     TWIN(retro_engine_detokenize(e, tokens, n_tokens, unparse_special, buffer, n_buffer, out_n_bytes));

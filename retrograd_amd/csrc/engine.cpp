@@ -359,6 +359,24 @@ void Engine::load_model(const std::string & path) {
     }
     vocab_.eos = (int32_t)g.get_int("tokenizer.ggml.eos_token_id", -1);
     vocab_.eot = (int32_t)g.get_int("tokenizer.ggml.eot_token_id", -1);
+    {
+        Tokenizer & tk = vocab_.tokenizer;
+        tk.model = g.get_string("tokenizer.ggml.model");
+        tk.pieces = vocab_.pieces;
+        tk.types = vocab_.types;
+        if (const MetaValue * sc = g.meta("tokenizer.ggml.scores")) tk.scores.assign(sc->fa.begin(), sc->fa.end());
+        tk.bos = (int32_t)g.get_int("tokenizer.ggml.bos_token_id", -1);
+        tk.eos = vocab_.eos;
+        tk.unk = (int32_t)g.get_int("tokenizer.ggml.unknown_token_id", -1);
+        tk.add_bos = g.get_int("tokenizer.ggml.add_bos_token", 1) != 0;
+        tk.add_eos = g.get_int("tokenizer.ggml.add_eos_token", 0) != 0;
+        tk.add_space_prefix = g.get_int("tokenizer.ggml.add_space_prefix", 1) != 0;
+        try {
+            tk.prepare();
+        } catch (const std::exception & e) {
+            vocab_.tokenizer_error = e.what();      // the model still decodes token ids
+        }
+    }
 
     // FNV-1a over the path bytes then the u64 weight size
     // (reference retro_runtime.hpp:856-868).

@@ -8,6 +8,7 @@
 #include "../../include/retro_step.h"
 #include "gguf_file.hpp"
 #include "kernels.hpp"
+#include "tokenizer.hpp"
 #include "sampler.hpp"
 
 #include <map>
@@ -82,6 +83,8 @@ struct Vocab {
     std::vector<std::string> pieces;
     std::vector<int32_t> types;
     int32_t eos = -1, eot = -1;
+    Tokenizer tokenizer;            // text -> ids (sentencepiece-kind vocabularies)
+    std::string tokenizer_error;    // why the vocabulary cannot tokenize, if it cannot
 };
 
 // Kernel categories of one step, for the optional event-based timing.

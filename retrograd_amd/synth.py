@@ -273,7 +273,7 @@ def storage_type(ggml_type: int, row_len: int) -> int:
 
 # ---- model files ----------------------------------------------------------------
 
-def _common_metadata(w: gw.GGUFWriter, s: ModelShape, with_eos: bool) -> None:
+def _common_metadata(w: gw.GGUFWriter, s: ModelShape, with_eos: bool, vocab: dict | None = None) -> None:
     a = s.arch
     w.add("general.architecture", gw.T_STRING, a)
     w.add("general.name", gw.T_STRING, s.name)
@@ -296,6 +296,17 @@ def _common_metadata(w: gw.GGUFWriter, s: ModelShape, with_eos: bool) -> None:
         w.add(a + ".expert_used_count", gw.T_UINT32, s.n_expert_used)
         w.add(a + ".expert_feed_forward_length", gw.T_UINT32, s.n_ff_exp)
     w.add("tokenizer.ggml.model", gw.T_STRING, "llama")
+    if vocab is not None:
+        # a real sentencepiece-kind vocabulary: pieces, scores, types and the special ids (n_vocab of them)
+        assert len(vocab["tokens"]) == s.n_vocab
+        w.add("tokenizer.ggml.tokens", gw.T_ARRAY, list(vocab["tokens"]), gw.T_STRING)
+        w.add("tokenizer.ggml.scores", gw.T_ARRAY, [float(x) for x in vocab["scores"]], gw.T_FLOAT32)
+        w.add("tokenizer.ggml.token_type", gw.T_ARRAY, [int(x) for x in vocab["types"]], gw.T_INT32)
+        w.add("tokenizer.ggml.bos_token_id", gw.T_UINT32, int(vocab["bos"]))
+        w.add("tokenizer.ggml.eos_token_id", gw.T_UINT32, int(vocab["eos"]))
+        w.add("tokenizer.ggml.unknown_token_id", gw.T_UINT32, int(vocab["unk"]))
+        w.add("general.alignment", gw.T_UINT32, 32)
+        return
     w.add("tokenizer.ggml.tokens", gw.T_ARRAY, ["<t%d>" % i for i in range(s.n_vocab)], gw.T_STRING)
     w.add("tokenizer.ggml.token_type", gw.T_ARRAY, [1] * s.n_vocab, gw.T_INT32)
     if with_eos:
@@ -304,7 +315,7 @@ def _common_metadata(w: gw.GGUFWriter, s: ModelShape, with_eos: bool) -> None:
 
 
 def write_model(path, shape: ModelShape, seed: int = 0, device: str | None = None,
-                with_eos: bool = False, std: float = 0.02) -> int:
+                with_eos: bool = False, std: float = 0.02, vocab: dict | None = None) -> int:
     """Writes a random-weight GGUF of `shape`; returns the file size. One tensor
     is materialised at a time, on `device` (cuda if available)."""
     if device is None:
@@ -313,7 +324,7 @@ def write_model(path, shape: ModelShape, seed: int = 0, device: str | None = Non
     gen.manual_seed(seed)
     s = shape
     w = gw.GGUFWriter()
-    _common_metadata(w, s, with_eos)
+    _common_metadata(w, s, with_eos, vocab)
 
     def matrix(name, n_in, n_out, ggml_type=None, n_mats=1, sd=std):
         t = storage_type(s.matrix_type if ggml_type is None else ggml_type, n_in)

@@ -54,6 +54,9 @@ TWINS = {
     "retro_engine_is_eog_token": "retro_trainer_is_eog_token",
     "retro_engine_context_size": "retro_trainer_context_size",
     "retro_engine_detokenize": "retro_trainer_detokenize",
+    "retro_engine_tokenize_text": "retro_trainer_tokenize_text",
+    "retro_engine_tokenize_fragment": "retro_trainer_tokenize_fragment",
+    "retro_engine_tokenize": "retro_trainer_tokenize_with",
     "retro_engine_generate_batch": "retro_trainer_generate_batch",
     "retro_engine_generate_continuous_batch": "retro_trainer_generate_continuous_batch",
     "retro_engine_generation_stats": "retro_trainer_generation_stats",

@@ -389,3 +389,45 @@ def test_engine_reproduces_hugging_face_transformers_logits(tmp_path, key):
         if srt[0] - srt[1] > 4e-2:
             assert r.token == int(want[i].argmax())
     eng.close()
+
+
+def test_tokenization_through_the_abi_reproduces_sentencepiece_ids_and_round_trips(tmp_path):
+    """retro_engine_tokenize / _text / _fragment over a model file whose vocabulary is the sentencepiece model of
+    tests/golden/spm_reference_ids.json: the library's own ids for every text, the two-call size contract, and
+    detokenize(tokenize(text)) == text."""
+    import ctypes as C
+    import json
+    from pathlib import Path
+    golden = json.loads((Path(__file__).resolve().parent / "golden" / "spm_reference_ids.json").read_text())
+    vocab = {"tokens": [v[0] for v in golden["vocab"]], "scores": [v[1] for v in golden["vocab"]],
+             "types": [v[2] for v in golden["vocab"]], "bos": golden["bos"], "eos": golden["eos"], "unk": golden["unk"]}
+    shape = synth.scaled(synth.TINY_LLAMA, n_vocab=len(vocab["tokens"]), name="tiny-llama-spm")
+    path = tmp_path / "spm.gguf"
+    synth.write_model(path, shape, seed=5, device="cpu", vocab=vocab)
+    eng = E.Engine(path, E.EngineConfig(n_ctx=256, n_seq_max=2, n_batch=64, n_ubatch=64))
+    for c in golden["cases"]:
+        assert eng.tokenize(c["text"], add_special=False, parse_special=False) == c["ids"], c["text"]
+        assert eng.tokenize(c["text"], add_special=True, parse_special=False) == [golden["bos"]] + c["ids"]
+        # round trip: the dummy prefix comes back as a leading space
+        assert eng.detokenize_bytes(c["ids"]).decode() == " " + c["text"], c["text"]
+    ids = eng.tokenize("<s>hello world</s>")                 # tokenize_text's flags: BOS added, special texts parsed
+    assert ids[:2] == [golden["bos"], golden["bos"]] and ids[-1] == golden["eos"]
+    # the size contract: no buffer -> count; too small -> -2 with the count; text required
+    lib, n = eng._lib, C.c_size_t()
+    assert lib.retro_engine_tokenize_text(eng._h, b"hello world", None, 0, C.byref(n)) == 0 and n.value == len(golden["cases"][0]["ids"]) + 1
+    small = (C.c_int32 * 1)()
+    assert lib.retro_engine_tokenize_fragment(eng._h, b"hello world", small, 1, C.byref(n)) == -2 and n.value == len(golden["cases"][0]["ids"])
+    assert lib.retro_engine_tokenize_text(eng._h, b"", None, 0, C.byref(n)) == -1 and "text is required" in E.last_error()
+    # the generated token ids of a greedy step detokenize and re-tokenize consistently with the vocabulary size
+    out = E.StepOutput()
+    eng.step([E.StepRow(0, 0, eng.tokenize("attention is all you need"), 0, sample=True, sampling=greedy())], out)
+    assert 0 <= out.row(0).token < len(vocab["tokens"])
+    eng.close()
+    # the trainer handle's twins (retro_trainer_tokenize_text / _fragment / _with) answer from the same vocabulary
+    from retrograd_amd import trainer as T
+    tr = T.Trainer(path, T.TrainConfig(n_ctx=64, n_batch=64))
+    for c in golden["cases"][:4]:
+        assert tr.tokenize(c["text"], add_special=False, parse_special=False) == c["ids"], c["text"]
+    assert tr._lib.retro_engine_tokenize_text(tr._h, b"hello world", None, 0, C.byref(n)) == 0 and n.value == len(golden["cases"][0]["ids"]) + 1
+    assert tr._lib.retro_engine_tokenize_fragment(tr._h, b"hello world", small, 1, C.byref(n)) == -2
+    tr.close()

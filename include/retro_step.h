@@ -277,8 +277,8 @@ int retro_engine_is_hybrid(retro_engine * engine, bool * out_is_hybrid);
 /* ref h:2538-2549, 2879-2889 (retro_engine.cpp:331-378, 594-622): text -> token ids. tokenize_text adds the model's
  * BOS / EOS and reads the text of a special token as that token; tokenize_fragment adds nothing; tokenize takes both
  * flags. Two calls: with tokens == NULL or n_tokens_max == 0 the count is reported; a buffer that is too small returns
- * -2 with the count. Built for sentencepiece-kind vocabularies (tokenizer.ggml.model = "llama"); byte-pair
- * vocabularies with a pre-tokeniser regex ("gpt2") return -1. */
+ * -2 with the count. Built for sentencepiece-kind vocabularies (tokenizer.ggml.model = "llama") and for byte-level
+ * byte-pair ones ("gpt2") whose tokenizer.ggml.pre names the Llama 3, Qwen 2 or GPT-2 pattern; any other returns -1. */
 int retro_engine_tokenize_text(retro_engine * engine, const char * text, int32_t * tokens, size_t n_tokens_max, size_t * out_n_tokens);
 int retro_engine_tokenize_fragment(retro_engine * engine, const char * text, int32_t * tokens, size_t n_tokens_max, size_t * out_n_tokens);
 int retro_engine_tokenize(retro_engine * engine, const char * text, bool add_special, bool parse_special, int32_t * tokens,

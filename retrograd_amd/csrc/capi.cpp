@@ -451,7 +451,8 @@ int retro_engine_context_size(retro_engine * engine, uint32_t * out_n_ctx) {
 }
 
 // Concatenates the raw pieces: SentencePiece's U+2581 becomes a space, byte
-// tokens "<0xXX>" their byte, control tokens are skipped unless unparse_special.
+// tokens "<0xXX>" their byte, a piece of a byte-pair vocabulary the bytes it spells;
+// control tokens are skipped unless unparse_special.
 int retro_engine_detokenize(retro_engine * engine, const int32_t * tokens, size_t n_tokens, bool unparse_special,
                             char * buffer, size_t n_buffer, size_t * out_n_bytes) {
     return boundary([&]() -> int {
@@ -488,6 +489,10 @@ int retro_engine_detokenize(retro_engine * engine, const int32_t * tokens, size_
             }
             if (type == 6 && piece.size() == 6 && piece.compare(0, 3, "<0x") == 0) {
                 text.push_back((char)std::stoi(piece.substr(3, 2), nullptr, 16));
+                continue;
+            }
+            if (v.tokenizer.model == "gpt2") {           // a byte-pair piece spells its bytes in GPT-2's printable alphabet
+                text += v.tokenizer.spelled_bytes(piece);
                 continue;
             }
             for (size_t j = 0; j < piece.size();) {

@@ -368,9 +368,12 @@ void Engine::load_model(const std::string & path) {
         tk.bos = (int32_t)g.get_int("tokenizer.ggml.bos_token_id", -1);
         tk.eos = vocab_.eos;
         tk.unk = (int32_t)g.get_int("tokenizer.ggml.unknown_token_id", -1);
-        tk.add_bos = g.get_int("tokenizer.ggml.add_bos_token", 1) != 0;
-        tk.add_eos = g.get_int("tokenizer.ggml.add_eos_token", 0) != 0;
-        tk.add_space_prefix = g.get_int("tokenizer.ggml.add_space_prefix", 1) != 0;
+        tk.pre = g.get_string("tokenizer.ggml.pre");
+        if (const MetaValue * mg = g.meta("tokenizer.ggml.merges")) tk.merges = mg->sa;
+        tk.set_kind_defaults();
+        tk.add_bos = g.get_int("tokenizer.ggml.add_bos_token", tk.add_bos) != 0;
+        tk.add_eos = g.get_int("tokenizer.ggml.add_eos_token", tk.add_eos) != 0;
+        tk.add_space_prefix = g.get_int("tokenizer.ggml.add_space_prefix", tk.add_space_prefix) != 0;
         try {
             tk.prepare();
         } catch (const std::exception & e) {

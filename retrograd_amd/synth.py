@@ -295,16 +295,22 @@ def _common_metadata(w: gw.GGUFWriter, s: ModelShape, with_eos: bool, vocab: dic
         w.add(a + ".expert_count", gw.T_UINT32, s.n_expert)
         w.add(a + ".expert_used_count", gw.T_UINT32, s.n_expert_used)
         w.add(a + ".expert_feed_forward_length", gw.T_UINT32, s.n_ff_exp)
-    w.add("tokenizer.ggml.model", gw.T_STRING, "llama")
+    w.add("tokenizer.ggml.model", gw.T_STRING, (vocab or {}).get("model", "llama"))
     if vocab is not None:
-        # a real sentencepiece-kind vocabulary: pieces, scores, types and the special ids (n_vocab of them)
+        # a real vocabulary (n_vocab pieces): sentencepiece-kind with scores and the unknown id, or byte-pair
+        # (model "gpt2") with the pre-tokeniser's name and the merges
         assert len(vocab["tokens"]) == s.n_vocab
         w.add("tokenizer.ggml.tokens", gw.T_ARRAY, list(vocab["tokens"]), gw.T_STRING)
-        w.add("tokenizer.ggml.scores", gw.T_ARRAY, [float(x) for x in vocab["scores"]], gw.T_FLOAT32)
+        if "scores" in vocab:
+            w.add("tokenizer.ggml.scores", gw.T_ARRAY, [float(x) for x in vocab["scores"]], gw.T_FLOAT32)
         w.add("tokenizer.ggml.token_type", gw.T_ARRAY, [int(x) for x in vocab["types"]], gw.T_INT32)
+        if "pre" in vocab:
+            w.add("tokenizer.ggml.pre", gw.T_STRING, vocab["pre"])
+            w.add("tokenizer.ggml.merges", gw.T_ARRAY, list(vocab["merges"]), gw.T_STRING)
         w.add("tokenizer.ggml.bos_token_id", gw.T_UINT32, int(vocab["bos"]))
         w.add("tokenizer.ggml.eos_token_id", gw.T_UINT32, int(vocab["eos"]))
-        w.add("tokenizer.ggml.unknown_token_id", gw.T_UINT32, int(vocab["unk"]))
+        if "unk" in vocab:
+            w.add("tokenizer.ggml.unknown_token_id", gw.T_UINT32, int(vocab["unk"]))
         w.add("general.alignment", gw.T_UINT32, 32)
         return
     w.add("tokenizer.ggml.tokens", gw.T_ARRAY, ["<t%d>" % i for i in range(s.n_vocab)], gw.T_STRING)

@@ -431,3 +431,31 @@ def test_tokenization_through_the_abi_reproduces_sentencepiece_ids_and_round_tri
     assert tr._lib.retro_engine_tokenize_text(tr._h, b"hello world", None, 0, C.byref(n)) == 0 and n.value == len(golden["cases"][0]["ids"]) + 1
     assert tr._lib.retro_engine_tokenize_fragment(tr._h, b"hello world", small, 1, C.byref(n)) == -2
     tr.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("pre", ["llama-bpe", "qwen2", "gpt-2"])
+def test_tokenization_of_a_byte_pair_vocabulary_reproduces_the_tokenizers_librarys_ids(tmp_path, pre):
+    """A model file whose vocabulary is the byte-level byte-pair one of tests/golden/bpe_reference_ids.json
+    (tokenizer.ggml.model = gpt2, with its merges and the name of its pre-tokeniser pattern): the library's own
+    ids through retro_engine_tokenize, BOS by the kind's default, and detokenize(tokenize(text)) == text."""
+    import json
+    from pathlib import Path
+    golden = json.loads((Path(__file__).resolve().parent / "golden" / "bpe_reference_ids.json").read_text())
+    kind = next(k for k in golden["kinds"] if k["pre"] == pre)
+    vocab = {"model": "gpt2", "pre": pre, "tokens": kind["tokens"], "merges": kind["merges"],
+             "types": [3 if i in kind["control"] else 1 for i in range(len(kind["tokens"]))], "bos": 0, "eos": 1}
+    shape = synth.scaled(synth.TINY_LLAMA, n_vocab=len(kind["tokens"]), name="tiny-llama-bpe-" + pre)
+    path = tmp_path / "bpe.gguf"
+    synth.write_model(path, shape, seed=6, device="cpu", vocab=vocab)
+    eng = E.Engine(path, E.EngineConfig(n_ctx=256, n_seq_max=2, n_batch=64, n_ubatch=64))
+    for c in kind["cases"]:
+        special = "<|" in c["text"]
+        assert eng.tokenize(c["text"], add_special=False, parse_special=special) == c["ids"], c["text"]
+        assert eng.detokenize_bytes(c["ids"], unparse_special=True).decode() == c["text"], c["text"]
+    hello = next(c["ids"] for c in kind["cases"] if c["text"] == "Hello world")
+    assert eng.tokenize("Hello world") == ([0] if pre == "llama-bpe" else []) + hello
+    out = E.StepOutput()
+    eng.step([E.StepRow(0, 0, eng.tokenize("attention is all you need"), 0, sample=True, sampling=greedy())], out)
+    assert 0 <= out.row(0).token < len(kind["tokens"])
+    eng.close()

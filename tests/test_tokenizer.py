@@ -1,8 +1,10 @@
-"""Text -> token ids for sentencepiece-kind vocabularies (retrograd_amd/csrc/tokenizer.hpp; the host side of
-retro_engine_tokenize*, reference crates/retrograd-ffi/runtime/src/retro_engine.cpp:331-378) against the ids of the
-sentencepiece library itself, committed as tests/golden/spm_reference_ids.json by tests/golden/spm_reference_ids.py.
+"""Text -> token ids (retrograd_amd/csrc/tokenizer.hpp; the host side of retro_engine_tokenize*, reference
+crates/retrograd-ffi/runtime/src/retro_engine.cpp:331-378) against the ids of the libraries that define the two
+vocabulary kinds: sentencepiece for tokenizer.ggml.model = "llama" (tests/golden/spm_reference_ids.json, written by
+tests/golden/spm_reference_ids.py) and Hugging Face tokenizers for the byte-level byte-pair kind "gpt2" with the
+Llama 3, Qwen 2 and GPT-2 pre-tokeniser patterns (tests/golden/bpe_reference_ids.json, by bpe_reference_ids.py).
 The reference hands the text to llama.cpp's tokenizer (absent from its checkout) and its tests hold no tokenisation
-vectors; llama.cpp's SPM tokenizer reproduces sentencepiece's BPE model, which is what pins this one. CPU only."""
+vectors; llama.cpp's tokenizers reproduce those two libraries, which is what pins this one. CPU only."""
 import json
 import subprocess
 from pathlib import Path
@@ -57,3 +59,58 @@ def test_special_tokens_and_the_flags(harness):
     assert mixed.count(bos) == 1 and mixed != plain["mixed <s> inside"]
     (empty,) = _run(harness, [(1, 1, "")]) or ([],)
     assert empty in ([bos], [])
+
+
+# ---- byte-pair vocabularies ----
+
+BPE = json.loads((ROOT / "tests/golden/bpe_reference_ids.json").read_text())
+
+
+def _run_bpe(harness, kind, cases, what):
+    exe, _, d = harness
+    vocab, merges, texts = d / ("bpe-%s-vocab.txt" % kind["pre"]), d / ("bpe-%s-merges.txt" % kind["pre"]), d / "bpe-texts.txt"
+    vocab.write_text("".join("%s 0 %d\n" % (t.encode().hex(), 3 if i in kind["control"] else 1)
+                             for i, t in enumerate(kind["tokens"])))
+    merges.write_text("".join(m.encode().hex() + "\n" for m in kind["merges"]))
+    texts.write_text("".join("%d %d %s\n" % (a, p, t.encode().hex() or "-") for a, p, t in cases))
+    r = subprocess.run([str(exe), str(vocab), str(texts), "0", "1", "0", kind["pre"], str(merges), what],
+                       capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, r.stdout
+    lines = r.stdout.splitlines()
+    return lines[0], lines[1:]
+
+
+@pytest.mark.parametrize("kind", BPE["kinds"], ids=[k["pre"] for k in BPE["kinds"]])
+def test_words_equal_the_tokenizers_librarys_pre_tokeniser(harness, kind):
+    _, got = _run_bpe(harness, kind, [(0, 0, c["text"]) for c in kind["cases"]], "words")
+    for c, line in zip(kind["cases"], got):
+        assert [bytes.fromhex(w).decode() for w in line.split()] == c["words"], c["text"]
+
+
+@pytest.mark.parametrize("kind", BPE["kinds"], ids=[k["pre"] for k in BPE["kinds"]])
+def test_ids_equal_the_tokenizers_librarys(harness, kind):
+    # the library always reads the text of an added token as that token: such a case runs with parse_special
+    first, got = _run_bpe(harness, kind, [(0, int("<|" in c["text"]), c["text"]) for c in kind["cases"]], "ids")
+    assert first == "add_bos %d" % (kind["pre"] == "llama-bpe")         # only the Llama 3 kind opens with BOS by default
+    for c, line in zip(kind["cases"], got):
+        assert [int(x) for x in line.split()] == c["ids"], c["text"]
+    # merges happened (fewer ids than bytes) and, under ignore_merges, whole words were taken
+    assert any(len(c["ids"]) < len(c["text"].encode()) // 2 for c in kind["cases"])
+    # parse_special: the text of a control token is that token, and what follows is split on its own
+    text = "<|begin_of_text|>Hello world<|end_of_text|>"
+    plain = next(c["ids"] for c in kind["cases"] if c["text"] == "Hello world")
+    _, (parsed, literal) = _run_bpe(harness, kind, [(0, 1, text), (0, 0, text)], "ids")
+    assert [int(x) for x in parsed.split()] == [0] + plain + [1]
+    assert 0 not in [int(x) for x in literal.split()]
+
+
+def test_an_unknown_pattern_is_refused(harness):
+    exe, _, d = harness
+    kind = dict(BPE["kinds"][0], pre="some-other-pattern")
+    vocab, merges, texts = d / "x-vocab.txt", d / "x-merges.txt", d / "x-texts.txt"
+    vocab.write_text("61 0 1\n")
+    merges.write_text("")
+    texts.write_text("0 0 61\n")
+    r = subprocess.run([str(exe), str(vocab), str(texts), "0", "1", "0", kind["pre"], str(merges), "ids"],
+                       capture_output=True, text=True, timeout=60)
+    assert r.returncode == 1 and "some-other-pattern" in r.stdout and "not built" in r.stdout

@@ -145,6 +145,9 @@ inline void q8_0_row_values(const float * x, size_t K, float * out) {
 inline void ggml_activation_row(uint32_t wtype, const float * x, size_t K, float * out) {
     if (exact_activations()) { std::copy(x, x + K, out); return; }
     switch (wtype) {
+        case T_Q2_K:
+        case T_Q3_K:
+        case T_IQ4_XS:
         case T_Q4_K:
         case T_Q5_K:
         case T_Q6_K: {
@@ -165,6 +168,11 @@ inline void ggml_activation_row(uint32_t wtype, const float * x, size_t K, float
             }
             return;
         }
+        case T_Q4_0:
+        case T_Q5_0:
+        case T_IQ4_NL:
+        case T_Q4_1:      // ggml pairs these two with Q8_1, whose codes and scale are Q8_0's
+        case T_Q5_1:
         case T_Q8_0:
         case T_MXFP4: {
             q8_0_row_values(x, K, out);

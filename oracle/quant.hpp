@@ -5,7 +5,9 @@
 // which the reference proves bit-equal to ggml's to_float on identical bytes
 // (tests/rir_quant_oracle.rs:67-103). Block geometry from
 // crates/rir-core/src/quant_table.rs (Q8_0 32 el / 34 B, MXFP4 32 el / 17 B,
-// Q4_K 256 el / 144 B, Q5_K 256 el / 176 B, Q6_K 256 el / 210 B).
+// Q4_K 256 el / 144 B, Q5_K 256 el / 176 B, Q6_K 256 el / 210 B; Q4_0 and
+// IQ4_NL 32 / 18, Q4_1 32 / 20, Q5_0 32 / 22, Q5_1 32 / 24, Q2_K 256 / 84,
+// Q3_K 256 / 110, IQ4_XS 256 / 136).
 //
 // Pinned by: tests/test_oracle_quant.py (known answers of quant.rs:534-581,
 // exhaustive f16 against numpy, brute-force Q4_K addressing against
@@ -26,7 +28,8 @@ namespace oracle {
 
 // ggml type ids as stored in a GGUF tensor table.
 enum ggml_type_id : uint32_t {
-    T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_BF16 = 30, T_MXFP4 = 39,
+    T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q4_1 = 3, T_Q5_0 = 6, T_Q5_1 = 7, T_Q8_0 = 8, T_Q2_K = 10, T_Q3_K = 11,
+    T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_IQ4_NL = 20, T_IQ4_XS = 23, T_BF16 = 30, T_MXFP4 = 39,
 };
 
 struct block_geom { uint32_t elements; uint32_t bytes; };
@@ -37,6 +40,14 @@ inline block_geom geom_of(uint32_t type) {
         case T_F16:   return {1, 2};
         case T_BF16:  return {1, 2};
         case T_Q8_0:  return {32, 34};
+        case T_Q4_0:  return {32, 18};
+        case T_Q4_1:  return {32, 20};
+        case T_Q5_0:  return {32, 22};
+        case T_Q5_1:  return {32, 24};
+        case T_IQ4_NL: return {32, 18};
+        case T_Q2_K:  return {256, 84};
+        case T_Q3_K:  return {256, 110};
+        case T_IQ4_XS: return {256, 136};
         case T_MXFP4: return {32, 17};
         case T_Q4_K:  return {256, 144};
         case T_Q5_K:  return {256, 176};
@@ -134,6 +145,8 @@ inline void q4k_scale_min(int j, const uint8_t * q, uint8_t & sc, uint8_t & mn) 
     }
 }
 
+// quant.rs:56-58: the non-linear code book of IQ4_NL and IQ4_XS
+static const int8_t k_iq4nl[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
 static const int8_t k_fp4_doubled[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
 
 // Decode n elements (whole blocks) of `type` from src into out.
@@ -153,6 +166,128 @@ inline void decode_row(uint32_t type, const uint8_t * src, size_t n, float * out
                 const uint8_t * blk = src + b * 34;
                 const float d = half_to_float(rd16(blk));
                 for (int j = 0; j < 32; ++j) out[b * 32 + j] = d * (float)(int8_t)blk[2 + j];
+            }
+            return;
+        case T_Q4_0:  // quant.rs:236-245: d (f16) | 16 bytes; low nibbles are the first half; value = d * (q - 8)
+        case T_IQ4_NL:  // quant.rs:297-306: the same block with the nibble looked up in the code book
+            for (size_t b = 0; b < n / 32; ++b) {
+                const uint8_t * blk = src + b * 18;
+                const float d = half_to_float(rd16(blk));
+                for (int j = 0; j < 16; ++j) {
+                    const uint8_t q = blk[2 + j];
+                    if (type == T_Q4_0) {
+                        out[b * 32 + j]      = d * (float)((int)(q & 0x0f) - 8);
+                        out[b * 32 + j + 16] = d * (float)((int)(q >> 4) - 8);
+                    } else {
+                        out[b * 32 + j]      = d * (float)k_iq4nl[q & 0x0f];
+                        out[b * 32 + j + 16] = d * (float)k_iq4nl[q >> 4];
+                    }
+                }
+            }
+            return;
+        case T_Q4_1:  // quant.rs:247-256: d, m (f16) | 16 bytes; value = d * q + m
+            for (size_t b = 0; b < n / 32; ++b) {
+                const uint8_t * blk = src + b * 20;
+                const float d = half_to_float(rd16(blk)), m = half_to_float(rd16(blk + 2));
+                for (int j = 0; j < 16; ++j) {
+                    const uint8_t q = blk[4 + j];
+                    out[b * 32 + j]      = d * (float)(q & 0x0f) + m;
+                    out[b * 32 + j + 16] = d * (float)(q >> 4) + m;
+                }
+            }
+            return;
+        case T_Q5_0:  // quant.rs:258-270: d (f16) | qh (u32) | 16 bytes; fifth bit j of qh for the first half, j + 16 for the second
+            for (size_t b = 0; b < n / 32; ++b) {
+                const uint8_t * blk = src + b * 22;
+                const float d = half_to_float(rd16(blk));
+                const uint32_t qh = (uint32_t)blk[2] | ((uint32_t)blk[3] << 8) | ((uint32_t)blk[4] << 16) | ((uint32_t)blk[5] << 24);
+                for (int j = 0; j < 16; ++j) {
+                    const uint8_t q = blk[6 + j];
+                    const uint32_t h0 = ((qh >> j) << 4) & 0x10, h1 = (qh >> (j + 12)) & 0x10;
+                    out[b * 32 + j]      = d * (float)((int)((q & 0x0f) | h0) - 16);
+                    out[b * 32 + j + 16] = d * (float)((int)((q >> 4) | h1) - 16);
+                }
+            }
+            return;
+        case T_Q5_1:  // quant.rs:272-284: d, m (f16) | qh (u32) | 16 bytes; value = d * q5 + m
+            for (size_t b = 0; b < n / 32; ++b) {
+                const uint8_t * blk = src + b * 24;
+                const float d = half_to_float(rd16(blk)), m = half_to_float(rd16(blk + 2));
+                const uint32_t qh = (uint32_t)blk[4] | ((uint32_t)blk[5] << 8) | ((uint32_t)blk[6] << 16) | ((uint32_t)blk[7] << 24);
+                for (int j = 0; j < 16; ++j) {
+                    const uint8_t q = blk[8 + j];
+                    const uint32_t h0 = ((qh >> j) << 4) & 0x10, h1 = (qh >> (j + 12)) & 0x10;
+                    out[b * 32 + j]      = d * (float)((q & 0x0f) | h0) + m;
+                    out[b * 32 + j + 16] = d * (float)((q >> 4) | h1) + m;
+                }
+            }
+            return;
+        case T_Q2_K:  // quant.rs:327-349: scales[16] | qs[64] | d, dmin (f16); sixteen sub-blocks of 16
+            for (size_t b = 0; b < n / 256; ++b) {
+                const uint8_t * blk = src + b * 84;
+                const float d = half_to_float(rd16(blk + 80)), dmin = half_to_float(rd16(blk + 82));
+                float * y = out + b * 256;
+                int o = 0, is = 0;
+                for (int n0 = 0; n0 < 256; n0 += 128) {
+                    const uint8_t * q = blk + 16 + n0 / 4;
+                    for (int j = 0; j < 4; ++j) {
+                        for (int half = 0; half < 2; ++half) {
+                            const uint8_t sc = blk[is++];
+                            const float dl = d * (float)(sc & 0x0f), ml = dmin * (float)(sc >> 4);
+                            for (int l = 0; l < 16; ++l) y[o++] = dl * (float)((q[l + 16 * half] >> (2 * j)) & 3) - ml;
+                        }
+                    }
+                }
+            }
+            return;
+        case T_Q3_K:  // quant.rs:351-396: hmask[32] | qs[64] | scales[12] | d (f16); sixteen 6-bit scales split 4 + 2 bits
+            for (size_t b = 0; b < n / 256; ++b) {
+                const uint8_t * blk = src + b * 110;
+                const float d_all = half_to_float(rd16(blk + 108));
+                uint32_t aux[4] = {0, 0, 0, 0};
+                for (int i = 0; i < 3; ++i)
+                    aux[i] = (uint32_t)blk[96 + 4 * i] | ((uint32_t)blk[97 + 4 * i] << 8) | ((uint32_t)blk[98 + 4 * i] << 16) | ((uint32_t)blk[99 + 4 * i] << 24);
+                const uint32_t kmask1 = 0x03030303u, kmask2 = 0x0f0f0f0fu, tmp = aux[2];
+                aux[2] = ((aux[0] >> 4) & kmask2) | (((tmp >> 4) & kmask1) << 4);
+                aux[3] = ((aux[1] >> 4) & kmask2) | (((tmp >> 6) & kmask1) << 4);
+                aux[0] = (aux[0] & kmask2) | ((tmp & kmask1) << 4);
+                aux[1] = (aux[1] & kmask2) | (((tmp >> 2) & kmask1) << 4);
+                int8_t scales[16];
+                for (int i = 0; i < 4; ++i)
+                    for (int j = 0; j < 4; ++j) scales[4 * i + j] = (int8_t)((aux[i] >> (8 * j)) & 0xff);
+                float * y = out + b * 256;
+                int o = 0, is = 0;
+                uint8_t m = 1;
+                for (int n0 = 0; n0 < 256; n0 += 128) {
+                    const uint8_t * q = blk + 32 + n0 / 4;
+                    for (int j = 0; j < 4; ++j) {
+                        for (int half = 0; half < 2; ++half) {
+                            const float dl = d_all * (float)((int)scales[is++] - 32);
+                            for (int l = 0; l < 16; ++l) {
+                                const int idx = l + 16 * half;
+                                const int qv = (q[idx] >> (2 * j)) & 3;
+                                y[o++] = dl * (float)(qv - ((blk[idx] & m) ? 0 : 4));
+                            }
+                        }
+                        m = (uint8_t)(m << 1);
+                    }
+                }
+            }
+            return;
+        case T_IQ4_XS:  // quant.rs:465-480: d (f16) | scales_h (u16) | scales_l[4] | qs[128]; eight sub-blocks of 32
+            for (size_t b = 0; b < n / 256; ++b) {
+                const uint8_t * blk = src + b * 136;
+                const float d = half_to_float(rd16(blk));
+                const uint32_t scales_h = rd16(blk + 2);
+                for (int ib = 0; ib < 8; ++ib) {
+                    const int ls = ((blk[4 + ib / 2] >> (4 * (ib % 2))) & 0x0f) | (int)(((scales_h >> (2 * ib)) & 3) << 4);
+                    const float dl = d * (float)(ls - 32);
+                    const uint8_t * qs = blk + 8 + 16 * ib;
+                    for (int j = 0; j < 16; ++j) {
+                        out[b * 256 + 32 * ib + j]      = dl * (float)k_iq4nl[qs[j] & 0x0f];
+                        out[b * 256 + 32 * ib + j + 16] = dl * (float)k_iq4nl[qs[j] >> 4];
+                    }
+                }
             }
             return;
         case T_MXFP4:  // quant.rs:286-295: e8m0 byte, low nibbles first half

@@ -167,7 +167,7 @@ void Engine::upload_weight(const TensorInfo & t, int64_t K, int64_t N, const uin
 // An expert tensor [K][N][n_expert]: n_expert * N rows of K, tiled per expert.
 void Engine::upload_experts(const TensorInfo & t, int64_t K, int64_t N, DevWeight & out) {
     const int64_t rows = N * hp_.n_expert;
-    if (!rk::moe_can_pack(t.type, K, N)) throw std::runtime_error("expert tensor " + t.name + " must be MXFP4, Q8_0, Q4_K, Q5_K or Q6_K with widths that are multiples of 256 and 16");
+    if (!rk::moe_can_pack(t.type, K, N)) throw std::runtime_error("expert tensor " + t.name + " must be MXFP4, Q8_0, Q4_K, Q5_K, Q6_K or a type rewritten as Q8_0 (Q4_0, Q5_0, IQ4_NL, Q3_K), with widths that are multiples of 256 and 16");
     if (rk::row_bytes(t.type, K) * (size_t)rows != t.nbytes) throw std::runtime_error("tensor " + t.name + " has an unexpected size");
     out.w.type = t.type;
     out.w.K = (int)K;
@@ -232,6 +232,7 @@ bool Engine::upload_gate_up_interleaved(const TensorInfo & g, const TensorInfo &
 
 void Engine::load_model(const std::string & path) {
     GgufFile g(path);
+    g.rewrite_as_q8_0();      // Q4_0, Q5_0, IQ4_NL and Q3_K tensors become the Q8_0 rows that hold the same values
     HParams & h = hp_;
     h.arch = g.get_string("general.architecture");
     if (h.arch == "llama") h.rope_neox = false;

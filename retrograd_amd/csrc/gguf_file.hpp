@@ -11,6 +11,8 @@
 #include <unordered_map>
 #include <vector>
 
+#include "transcode.hpp"
+
 #include <fcntl.h>
 #include <sys/mman.h>
 #include <sys/stat.h>
@@ -73,11 +75,23 @@ public:
     size_t file_size() const { return size_; }
     // Bytes of all tensor payloads: what llama_model_size reports for a file
     // whose tensors are all loaded.
-    uint64_t tensor_bytes() const {
-        uint64_t total = 0;
-        for (const auto & t : tensors_) total += t.nbytes;
-        return total;
+    uint64_t tensor_bytes() const { return tensor_bytes_; }
+    // Rewrites every tensor of a type Q8_0 holds exactly (transcode.hpp) as Q8_0 rows in memory of this object:
+    // the loader then sees a Q8_0 tensor. tensor_bytes() keeps reporting the file's own sizes.
+    void rewrite_as_q8_0() {
+        for (TensorInfo & t : tensors_) {
+            if (!q8_0_holds(t.type)) continue;
+            size_t elems = 1;
+            for (int d = 0; d < t.n_dims; ++d) elems *= (size_t)t.ne[d];
+            owned_.emplace_back(elems / 32 * 34);
+            to_q8_0(t.type, t.data, elems, owned_.back().data());
+            t.type = GT_Q8_0;
+            t.data = owned_.back().data();
+            t.nbytes = owned_.back().size();
+        }
     }
+    // Frees what rewrite_as_q8_0 allocated; the rewritten tensors must not be read afterwards.
+    void drop_rewritten() { owned_.clear(); owned_.shrink_to_fit(); }
     const std::vector<TensorInfo> & tensors() const { return tensors_; }
     const TensorInfo * find(const std::string & name) const {
         auto it = by_name_.find(name);
@@ -171,6 +185,8 @@ private:
             case 11: block = 256; bytes = 110; break;
             case 13: block = 256; bytes = 176; break;
             case 14: block = 256; bytes = 210; break;
+            case 20: block = 32; bytes = 18; break;
+            case 23: block = 256; bytes = 136; break;
             default: return 0;
         }
         for (int d = 0; d < t.n_dims; ++d) {
@@ -238,6 +254,7 @@ private:
             if (offsets[i] > room || t.nbytes > room - offsets[i]) throw std::runtime_error("tensor " + t.name + " runs past the file");
             t.data = map_ + data0 + offsets[i];
             by_name_[t.name] = i;
+            tensor_bytes_ += t.nbytes;
         }
     }
 
@@ -248,6 +265,8 @@ private:
     std::unordered_map<std::string, MetaValue> meta_;
     std::vector<TensorInfo> tensors_;
     std::unordered_map<std::string, size_t> by_name_;
+    uint64_t tensor_bytes_ = 0;
+    std::vector<std::vector<uint8_t>> owned_;
 };
 
 }  // namespace retro

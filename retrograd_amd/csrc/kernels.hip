@@ -47,6 +47,10 @@ BlockGeom geom_of(int type) {
         case WT_Q4_K:  return {256, 144};
         case WT_Q5_K:  return {256, 176};
         case WT_Q6_K:  return {256, 210};
+        case WT_Q4_1:  return {32, 20};
+        case WT_Q5_1:  return {32, 24};
+        case WT_Q2_K:  return {256, 84};
+        case WT_IQ4_XS: return {256, 136};
         default: throw std::runtime_error("unsupported tensor type " + std::to_string(type));
     }
 }
@@ -125,6 +129,42 @@ __device__ float decode_elem(int type, const uint8_t * row, int k) {
             const float d = h2f((uint16_t)(b[208] | (b[209] << 8)));
             const float scale = (float)(int8_t)b[192 + 8 * half + 2 * g + (l >> 4)];
             return __fmul_rn(__fmul_rn(d, scale), (float)((nib | (top << 4)) - 32));
+        }
+        case WT_Q4_1:
+        case WT_Q5_1: {
+            // d, m (f16) | [qh (u32)] | 16 bytes: element e is a nibble of byte e % 16 (the high one for e >= 16), with
+            // bit e of qh on top for Q5_1; value = d * q + m
+            const bool five = type == WT_Q5_1;
+            const uint8_t * b = row + (size_t)(k >> 5) * (five ? 24 : 20);
+            const int e = k & 31;
+            const uint8_t byte = b[(five ? 8 : 4) + (e & 15)];
+            int q = e < 16 ? (byte & 0x0f) : (byte >> 4);
+            if (five) q |= ((b[4 + (e >> 3)] >> (e & 7)) & 1) << 4;
+            const float d = h2f(*(const uint16_t *)b), m = h2f(*(const uint16_t *)(b + 2));
+            return __fadd_rn(__fmul_rn(d, (float)q), m);
+        }
+        case WT_Q2_K: {
+            // scales[16] | qs[64] | d, dmin (f16): element e reads two bits of qs[32 (e / 128) + e % 32] at 2 ((e / 32) % 4),
+            // its sub-block's byte scales[e / 16] holds the scale (low nibble) and the min (high)
+            const uint8_t * b = row + (size_t)(k >> 8) * 84;
+            const int e = k & 255;
+            const int q = (b[16 + (e >> 7) * 32 + (e & 31)] >> (2 * ((e >> 5) & 3))) & 3;
+            const uint8_t sc = b[e >> 4];
+            const float d = h2f((uint16_t)(b[80] | (b[81] << 8))), dmin = h2f((uint16_t)(b[82] | (b[83] << 8)));
+            return __fsub_rn(__fmul_rn(__fmul_rn(d, (float)(sc & 0x0f)), (float)q), __fmul_rn(dmin, (float)(sc >> 4)));
+        }
+        case WT_IQ4_XS: {
+            // d (f16) | scales_h (u16) | scales_l[4] | qs[128]: sub-block ib = e / 32 has the six-bit scale
+            // (scales_l nibble ib) | (scales_h bits 2 ib, 2 ib + 1) << 4, minus 32; its codes index the IQ4_NL table
+            const int8_t table[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+            const uint8_t * b = row + (size_t)(k >> 8) * 136;
+            const int e = k & 255, ib = e >> 5;
+            const uint8_t byte = b[8 + 16 * ib + (e & 15)];
+            const int code = (e & 16) ? (byte >> 4) : (byte & 0x0f);
+            const int sh = b[2] | (b[3] << 8);
+            const int ls = ((b[4 + (ib >> 1)] >> (4 * (ib & 1))) & 0x0f) | (((sh >> (2 * ib)) & 3) << 4);
+            const float d = h2f((uint16_t)(b[0] | (b[1] << 8)));
+            return __fmul_rn(__fmul_rn(d, (float)(ls - 32)), (float)table[code]);
         }
         default: return 0.0f;
     }

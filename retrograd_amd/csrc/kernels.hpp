@@ -11,7 +11,8 @@
 namespace rk {
 
 // ggml tensor type ids as stored in GGUF.
-enum : int { WT_F32 = 0, WT_F16 = 1, WT_Q8_0 = 8, WT_Q4_K = 12, WT_Q5_K = 13, WT_Q6_K = 14, WT_BF16 = 30, WT_MXFP4 = 39 };
+enum : int { WT_F32 = 0, WT_F16 = 1, WT_Q4_1 = 3, WT_Q5_1 = 7, WT_Q8_0 = 8, WT_Q2_K = 10, WT_Q4_K = 12, WT_Q5_K = 13, WT_Q6_K = 14,
+              WT_IQ4_XS = 23, WT_BF16 = 30, WT_MXFP4 = 39 };
 
 // One KV page holds PAGE consecutive positions of one sequence.
 constexpr int PAGE = 32;
@@ -64,8 +65,8 @@ enum : int { AQ_NONE = 0, AQ_Q8_0 = 32, AQ_Q8_K = 256 };
 // The conversion ggml's CPU matmul applies for a weight of this storage type.
 inline int act_quant_of(int ggml_type) {
     switch (ggml_type) {
-        case 12: case 13: case 14: return AQ_Q8_K;   // Q4_K, Q5_K, Q6_K
-        case 8: case 39: return AQ_Q8_0;    // Q8_0, MXFP4
+        case 10: case 12: case 13: case 14: case 23: return AQ_Q8_K;   // Q2_K, Q4_K, Q5_K, Q6_K, IQ4_XS
+        case 3: case 7: case 8: case 39: return AQ_Q8_0;    // Q4_1, Q5_1 (Q8_1 has Q8_0's codes and scale), Q8_0, MXFP4
         default: return AQ_NONE;
     }
 }

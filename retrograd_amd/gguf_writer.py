@@ -27,9 +27,13 @@ T_UINT64, T_INT64, T_FLOAT64 = 10, 11, 12
 
 # ggml tensor types used by the decode step
 GGML_F32, GGML_F16, GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_BF16, GGML_MXFP4 = 0, 1, 8, 12, 13, 14, 30, 39
+# ... and the types a model file may also hold: rewritten as Q8_0 at load or decoded element by element
+GGML_Q4_0, GGML_Q4_1, GGML_Q5_0, GGML_Q5_1, GGML_Q2_K, GGML_Q3_K, GGML_IQ4_NL, GGML_IQ4_XS = 2, 3, 6, 7, 10, 11, 20, 23
 BLOCK_GEOMETRY = {  # type -> (elements per block, bytes per block)
     GGML_F32: (1, 4), GGML_F16: (1, 2), GGML_BF16: (1, 2),
     GGML_Q8_0: (32, 34), GGML_MXFP4: (32, 17), GGML_Q4_K: (256, 144), GGML_Q5_K: (256, 176), GGML_Q6_K: (256, 210),
+    GGML_Q4_0: (32, 18), GGML_Q4_1: (32, 20), GGML_Q5_0: (32, 22), GGML_Q5_1: (32, 24), GGML_IQ4_NL: (32, 18),
+    GGML_Q2_K: (256, 84), GGML_Q3_K: (256, 110), GGML_IQ4_XS: (256, 136),
 }
 
 _SCALAR_FMT = {

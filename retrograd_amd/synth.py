@@ -246,8 +246,39 @@ def quantize_mxfp4(x: torch.Tensor) -> torch.Tensor:
     return out.reshape(rows, -1)
 
 
+# type -> (offsets of the block's f16 scale fields with their factors, the standard deviation of a block of
+# uniformly random codes at scale 1): Q4_1 and Q5_1 get the min -7.5 d / -15.5 d and Q2_K dmin = 1.5 d, which
+# centre their values on zero
+_RANDOM_BLOCKS = {
+    gw.GGML_Q4_0: ([(0, 1.0)], 4.61), gw.GGML_Q5_0: ([(0, 1.0)], 9.23), gw.GGML_IQ4_NL: ([(0, 1.0)], 67.1),
+    gw.GGML_Q4_1: ([(0, 1.0), (2, -7.5)], 4.61), gw.GGML_Q5_1: ([(0, 1.0), (2, -15.5)], 9.23),
+    gw.GGML_Q2_K: ([(80, 1.0), (82, 1.5)], 13.9), gw.GGML_Q3_K: ([(108, 1.0)], 43.3), gw.GGML_IQ4_XS: ([(0, 1.0)], 1247.5),
+}
+
+
+def random_blocks(x: torch.Tensor, ggml_type: int) -> np.ndarray:
+    """Rows of the legacy and i-quant types for a test model: every payload byte uniformly random (so every code,
+    sub-block scale and high bit occurs), the f16 scale fields set so that the decoded values have about the
+    standard deviation of `x`, with a random sign and a spread of two octaves per block. `x` gives the shape, the
+    spread and the seed; its values are not fitted (no quantiser of these types is needed where the same bytes are
+    decoded on both sides of a comparison)."""
+    rows, K = x.shape
+    el, nb = gw.BLOCK_GEOMETRY[ggml_type]
+    fields, unit = _RANDOM_BLOCKS[ggml_type]
+    sd = float(x.float().std())
+    rng = np.random.default_rng(int(abs(float(x.float().sum())) * 1e6) % (2 ** 32))
+    n = rows * (K // el)
+    raw = rng.integers(0, 256, (n, nb), dtype=np.uint8)
+    d = (sd / unit) * np.exp2(rng.uniform(-1.0, 1.0, n)) * rng.choice([-1.0, 1.0], n)
+    for off, factor in fields:
+        raw[:, off:off + 2] = (d * factor).astype(np.float16).view(np.uint8).reshape(n, 2)
+    return raw.reshape(rows, -1)
+
+
 def encode(x: torch.Tensor, ggml_type: int) -> np.ndarray:
     """[rows, K] float tensor -> numpy bytes of the stored representation."""
+    if ggml_type in _RANDOM_BLOCKS:
+        return random_blocks(x, ggml_type)
     if ggml_type == gw.GGML_F32:
         return x.float().cpu().numpy()
     if ggml_type == gw.GGML_F16:

@@ -366,3 +366,120 @@ def test_q5_k_against_the_block_loops_and_single_codes():
     # Q5_K weights take Q8_K activations
     v = rng.standard_normal(256).astype(np.float32)
     assert np.array_equal(oracle.activation_row(Q5_K, v), oracle.activation_row(12, v))
+
+
+# ---- the legacy and i-quant types (quant.rs:236-306, 327-396, 465-480) ------------------------------
+# Each against a per-element closed form in numpy (element e -> byte, shift and scale index, derived from the
+# layouts, where the oracle follows the reference's running loops), on random blocks with finite scales; the
+# reference's own Q4_0 known answer; and single codes placed on single elements.
+
+_IQ4NL = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.float32)
+
+
+def _h(blk, off):
+    return np.float32(blk[off:off + 2].view(np.float16)[0])
+
+
+def _closed_form(wt, blk):
+    e = np.arange(256 if wt in (10, 11, 23) else 32)
+    u = blk.astype(np.int64)
+    if wt in (2, 20, 3, 6, 7):                                   # blocks of 32: element e is a nibble of byte e % 16
+        head = {2: 2, 20: 2, 3: 4, 6: 6, 7: 8}[wt]
+        nib = (u[head + e % 16] >> (4 * (e // 16))) & 15
+        if wt in (6, 7):
+            qh = int.from_bytes(bytes(blk[head - 4:head]), "little")
+            nib = nib | (((qh >> e) & 1) << 4)                   # the fifth bit of element e is bit e of qh
+        d = _h(blk, 0)
+        if wt == 2:
+            return d * (nib - 8).astype(np.float32)
+        if wt == 20:
+            return d * _IQ4NL[nib]
+        if wt == 6:
+            return d * (nib - 16).astype(np.float32)
+        return d * nib.astype(np.float32) + _h(blk, 2)            # Q4_1, Q5_1
+    if wt == 10:                                                 # Q2_K: scales[16] | qs[64] | d | dmin
+        q = (u[16 + (e >> 7) * 32 + (e & 31)] >> (2 * ((e >> 5) & 3))) & 3
+        sc = u[e >> 4]
+        dl = _h(blk, 80) * (sc & 15).astype(np.float32)
+        ml = _h(blk, 82) * (sc >> 4).astype(np.float32)
+        return dl * q.astype(np.float32) - ml
+    if wt == 11:                                                 # Q3_K: hmask[32] | qs[64] | scales[12] | d
+        q = (u[32 + (e >> 7) * 32 + (e & 31)] >> (2 * ((e >> 5) & 3))) & 3
+        high = (u[e & 31] >> (e >> 5)) & 1
+        i = e >> 4                                               # scale i: four bits from scales[i % 8], two from scales[8 + i % 4]
+        s = ((u[96 + i % 8] >> (4 * (i // 8))) & 15) | (((u[104 + i % 4] >> (2 * (i // 4))) & 3) << 4)
+        dl = _h(blk, 108) * (s - 32).astype(np.float32)
+        return dl * (q - 4 * (1 - high)).astype(np.float32)
+    if wt == 23:                                                 # IQ4_XS: d | scales_h | scales_l[4] | qs[128]
+        ib = e >> 5
+        nib = (u[8 + 16 * ib + e % 16] >> (4 * ((e >> 4) & 1))) & 15
+        sh = int(u[2]) | (int(u[3]) << 8)
+        ls = ((u[4 + ib // 2] >> (4 * (ib % 2))) & 15) | (((sh >> (2 * ib)) & 3) << 4)
+        return (_h(blk, 0) * (ls - 32).astype(np.float32)) * _IQ4NL[nib]
+    raise AssertionError(wt)
+
+
+_LEGACY = {2: (32, 18, [0]), 3: (32, 20, [0, 2]), 6: (32, 22, [0]), 7: (32, 24, [0, 2]), 20: (32, 18, [0]),
+           10: (256, 84, [80, 82]), 11: (256, 110, [108]), 23: (256, 136, [0])}
+
+
+def _random_blocks(wt, n_blocks, rng):
+    el, nb, scale_at = _LEGACY[wt]
+    raw = rng.integers(0, 256, (n_blocks, nb), dtype=np.uint8)
+    for off in scale_at:                                         # finite f16 scales of mixed sign and magnitude
+        raw[:, off:off + 2] = (rng.standard_normal(n_blocks) * 0.05).astype(np.float16).view(np.uint8).reshape(n_blocks, 2)
+    return raw
+
+
+@pytest.mark.parametrize("wt", sorted(_LEGACY), ids=["q4_0", "q4_1", "q5_0", "q5_1", "q2_k", "q3_k", "iq4_nl", "iq4_xs"])
+def test_legacy_and_iquant_types_against_the_closed_form(wt):
+    el, nb, _ = _LEGACY[wt]
+    rng = np.random.default_rng(wt)
+    raw = _random_blocks(wt, 24, rng)
+    got = oracle.decode_row(wt, raw.reshape(-1), 24 * el).reshape(24, el)
+    for b in range(24):
+        np.testing.assert_array_equal(got[b], _closed_form(wt, raw[b]).astype(np.float32))
+    with pytest.raises(oracle.OracleError):
+        oracle.row_bytes(wt, el - 1)
+    assert oracle.row_bytes(wt, 3 * el) == 3 * nb
+
+
+def test_q4_0_known_answer_of_the_reference():
+    """crates/rir-core/src/quant.rs:572-581: d = 1, every byte 0x81 -> low nibbles (first half) 1 - 8, high 8 - 8."""
+    blk = np.zeros(18, np.uint8)
+    blk[0:2] = np.array([0x3c00], np.uint16).view(np.uint8)
+    blk[2:] = 0x81
+    v = oracle.decode_row(2, blk, 32)
+    assert (v[:16] == -7.0).all() and (v[16:] == 0.0).all()
+
+
+def test_single_codes_of_the_super_block_types_land_on_single_elements():
+    one = np.array([0x3c00], np.uint16).view(np.uint8)
+    # Q2_K: all sub-block scales 1 (no mins), one 2-bit code 3 at element 100 = second 32 of the first half, l = 4
+    blk = np.zeros(84, np.uint8)
+    blk[0:16] = 0x01
+    blk[80:82] = one
+    blk[16 + 4] = 3 << 6
+    v = oracle.decode_row(10, blk, 256)
+    assert v[100] == 3.0 and np.count_nonzero(v) == 1
+    # Q3_K: every scale 33 (d * 1), all high bits set (no -4): one code 2 at element 200 = half 1, j = 2, position 8
+    blk = np.zeros(110, np.uint8)
+    blk[0:32] = 0xff
+    blk[96:104] = 0x11                                          # low four bits 1 of all sixteen scales
+    blk[104:108] = 0xaa                                         # high two bits 2 -> 33
+    blk[108:110] = one
+    blk[32 + 32 + 8] = 2 << 4
+    v = oracle.decode_row(11, blk, 256)
+    assert v[200] == 2.0 and np.count_nonzero(v) == 1
+    # ... and with its high bit clear the same element reads 2 - 4
+    blk[8] &= ~np.uint8(1 << 6)
+    assert oracle.decode_row(11, blk, 256)[200] == -2.0
+    # IQ4_XS: sub-block 5 with scale 33, the others 32 (zero): code 15 (113) at element 5 * 32 + 16 + 3
+    blk = np.zeros(136, np.uint8)
+    blk[0:2] = one
+    blk[2:4] = np.array([0xaaaa], np.uint16).view(np.uint8)     # high bits 2 everywhere -> 32 + low
+    blk[4 + 2] = 1 << 4                                         # low nibble of sub-block 5
+    blk[8:] = 0x88                                              # code 8 everywhere: value 1 where the scale is not zero
+    blk[8 + 16 * 5 + 3] = 0xf8
+    v = oracle.decode_row(23, blk, 256)
+    assert v[5 * 32 + 16 + 3] == 113.0 and (np.delete(v[160:192], 19) == 1.0).all() and np.count_nonzero(v) == 32

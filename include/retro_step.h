@@ -306,10 +306,11 @@ int retro_engine_adapter_load(
 int retro_engine_adapter_unload(retro_engine * engine, int32_t id);
 int retro_engine_adapter_rows_info(retro_engine * engine, retro_adapter_rows_info * out_info);
 
-/* ---- grammar handles: ref h:1404-1408 ------------------------------------
- * A handle owns a GBNF string. Rows that carry one are refused by the step
- * (-3): grammar masking needs llama.cpp's GBNF parser, which this library does
- * not contain. from_json_schema is refused for the same reason (NULL). */
+/* ---- grammar handles: ref h:1395-1408 ------------------------------------
+ * A handle owns a GBNF string; all three constructors return NULL with the error set on failure. from_gbnf takes the
+ * text as it is (it is compiled by the step that carries it: -3 there when it is invalid); json_object is a grammar
+ * for one JSON object; from_json_schema converts a subset of JSON Schema and names the keyword it cannot convert.
+ * The handle may be freed as soon as the step call that carried it returns. */
 retro_grammar * retro_grammar_from_json_schema(const char * json_schema);
 retro_grammar * retro_grammar_from_gbnf(const char * gbnf);
 retro_grammar * retro_grammar_json_object(void);

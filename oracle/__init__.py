@@ -101,7 +101,7 @@ def _declare(l: C.CDLL) -> None:
     l.orc_sample_v2.argtypes = [_f32p, C.c_size_t, C.c_float, C.c_float, C.c_int32, C.c_float,
                                 C.c_float, C.c_float, C.c_float, C.c_uint32, C.c_uint32, _i32p, _f32p,
                                 C.c_void_p, _i32p, C.c_size_t, _i32p, _f32p, _f32p,
-                                C.c_size_t, _i32p, _f32p]
+                                C.c_size_t, _i32p, _f32p, _u8p]
     l.orc_token_logprob.argtypes = [_f32p, C.c_size_t, C.c_int32]
     l.orc_token_logprob.restype = C.c_float
     l.orc_top_logprobs.argtypes = [_f32p, C.c_size_t, C.c_size_t, _i32p, _f32p]
@@ -403,8 +403,11 @@ def sample_v1(logits: np.ndarray, temperature: float, top_p: float, rng: Rng, k:
 
 def sample_v2(logits: np.ndarray, rng: Rng, *, temperature=1.0, top_p=1.0, top_k=0, min_p=0.0,
               repeat_penalty=1.0, frequency_penalty=0.0, presence_penalty=0.0, penalty_window=0,
-              bias_ids=(), bias_values=(), history=(), k: int = 0):
+              bias_ids=(), bias_values=(), history=(), k: int = 0, allowed=None):
+    """`allowed`: one flag per token, the set a grammar leaves at this position (None: no grammar)."""
     logits = np.ascontiguousarray(logits, np.float32)
+    mask = None if allowed is None else np.ascontiguousarray(allowed, np.uint8)
+    assert mask is None or mask.size == logits.size
     bi = np.asarray(bias_ids, np.int32)
     bv = np.asarray(bias_values, np.float32)
     hist = np.asarray(history, np.int32)
@@ -415,7 +418,7 @@ def sample_v2(logits: np.ndarray, rng: Rng, *, temperature=1.0, top_p=1.0, top_k
                                repeat_penalty, frequency_penalty, presence_penalty, penalty_window,
                                bi.size, _ptr(bi, _i32p), _ptr(bv, _f32p), rng._h,
                                _ptr(hist, _i32p), hist.size, C.byref(tok), C.byref(lp), C.byref(slp),
-                               k, _ptr(ids, _i32p), _ptr(lps, _f32p)))
+                               k, _ptr(ids, _i32p), _ptr(lps, _f32p), None if mask is None else _ptr(mask, _u8p)))
     return tok.value, lp.value, slp.value, ids[:k], lps[:k]
 
 

@@ -269,7 +269,7 @@ int orc_sample_v2(const float * logits, size_t n_vocab,
                   uint32_t penalty_window, uint32_t n_bias, const int32_t * bias_ids, const float * bias_values,
                   void * rng, const int32_t * history, size_t n_history,
                   int32_t * out_token, float * out_logprob, float * out_sampled_logprob,
-                  size_t k, int32_t * top_ids, float * top_lps) {
+                  size_t k, int32_t * top_ids, float * top_lps, const uint8_t * allowed) {
     return guard([&] {
         params_v2 p;
         p.temperature = temperature; p.top_p = top_p; p.top_k = top_k; p.min_p = min_p;
@@ -278,7 +278,7 @@ int orc_sample_v2(const float * logits, size_t n_vocab,
         p.bias_ids.assign(bias_ids, bias_ids + n_bias);
         p.bias_values.assign(bias_values, bias_values + n_bias);
         std::vector<int32_t> hist(history, history + n_history);
-        sample_result r = sample_v2(logits, n_vocab, p, *(std::mt19937 *)rng, hist);
+        sample_result r = sample_v2(logits, n_vocab, p, *(std::mt19937 *)rng, hist, allowed);
         if (r.token < 0) throw std::runtime_error("oracle: no token");
         *out_token = r.token;
         *out_logprob = token_logprob(logits, n_vocab, r.token);

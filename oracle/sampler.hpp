@@ -9,8 +9,11 @@
 // The reference draws with libstdc++'s std::mt19937 and
 // std::uniform_real_distribution<double>; this file uses the same library
 // classes, so the bit stream is the library's, not a restatement.
-// Grammar masking (step 3 of v2) needs llama.cpp's GBNF engine and is not
-// restated: rows carrying a grammar are outside the oracle.
+// Grammar masking (step 3 of v2, retro_gen_core.cpp:767-795) is restated as
+// what it does to the row: every token outside a given allowed set gets -inf
+// between the penalties and top_k, and a row with no allowed token is an
+// error. Which tokens a GBNF text allows is llama.cpp's grammar engine in the
+// reference; the tests compute the set with a regular-expression library.
 //
 // Pinned by tests/test_oracle_sampler.py: top_k = 1 is argmax with the RNG
 // advanced by one draw; top_p = 1e-6 is argmax with sampled_logprob 0 and -inf
@@ -103,7 +106,7 @@ struct params_v2 {
 };
 
 inline sample_result sample_v2(const float * logits, size_t n, const params_v2 & p, std::mt19937 & rng,
-                               const std::vector<int32_t> & history) {
+                               const std::vector<int32_t> & history, const uint8_t * allowed = nullptr) {
     std::vector<float> t(logits, logits + n);
     for (size_t i = 0; i < p.bias_ids.size(); ++i) t[(size_t)p.bias_ids[i]] += p.bias_values[i];
 
@@ -117,6 +120,14 @@ inline sample_result sample_v2(const float * logits, size_t n, const params_v2 &
             v = v <= 0.0f ? v * p.repeat_penalty : v / p.repeat_penalty;
             v -= (float)kv.second * p.frequency_penalty + (float)(kv.second > 0) * p.presence_penalty;
         }
+    }
+    if (allowed) {
+        bool any = false;
+        for (size_t i = 0; i < n; ++i) {
+            if (!allowed[i]) t[i] = -INFINITY;
+            any = any || t[i] != -INFINITY;
+        }
+        if (!any) throw std::runtime_error("grammar allows no token at this position");
     }
     if (p.top_k > 0 && (size_t)p.top_k < n) {
         std::vector<int32_t> order(n);

@@ -3,13 +3,13 @@
 // boundary(), which clears the thread's error string and turns any C++
 // exception into -1 (reference retro_runtime.hpp:1255-1267).
 #include "engine.hpp"
+#include "json_grammar.hpp"
+#include "json_schema.hpp"
 
 #include <cmath>
 #include <cstring>
 
 using namespace retro;
-
-struct retro_grammar { std::string gbnf; };
 
 namespace {
 
@@ -433,7 +433,7 @@ int retro_engine_is_eog_token(retro_engine * engine, int32_t token, bool * out_i
             return -1;
         }
         const Vocab & v = e->vocab();
-        *out_is_eog = (v.eos >= 0 && token == v.eos) || (v.eot >= 0 && token == v.eot);
+        *out_is_eog = v.is_eog(token);
         return 0;
     });
 }
@@ -450,9 +450,7 @@ int retro_engine_context_size(retro_engine * engine, uint32_t * out_n_ctx) {
     });
 }
 
-// Concatenates the raw pieces: SentencePiece's U+2581 becomes a space, byte
-// tokens "<0xXX>" their byte, a piece of a byte-pair vocabulary the bytes it spells;
-// control tokens are skipped unless unparse_special.
+// Concatenates what the tokens stand for (Vocab::append_text); control tokens are skipped unless unparse_special.
 int retro_engine_detokenize(retro_engine * engine, const int32_t * tokens, size_t n_tokens, bool unparse_special,
                             char * buffer, size_t n_buffer, size_t * out_n_bytes) {
     return boundary([&]() -> int {
@@ -480,30 +478,7 @@ int retro_engine_detokenize(retro_engine * engine, const int32_t * tokens, size_
                           + " is outside the vocabulary of size " + std::to_string(n_vocab));
                 return -1;
             }
-            if ((size_t)t >= v.pieces.size()) continue;
-            const int32_t type = (size_t)t < v.types.size() ? v.types[(size_t)t] : 1;
-            const std::string & piece = v.pieces[(size_t)t];
-            if (type == 3 || type == 2) {            // control / unknown
-                if (unparse_special) text += piece;
-                continue;
-            }
-            if (type == 6 && piece.size() == 6 && piece.compare(0, 3, "<0x") == 0) {
-                text.push_back((char)std::stoi(piece.substr(3, 2), nullptr, 16));
-                continue;
-            }
-            if (v.tokenizer.model == "gpt2") {           // a byte-pair piece spells its bytes in GPT-2's printable alphabet
-                text += v.tokenizer.spelled_bytes(piece);
-                continue;
-            }
-            for (size_t j = 0; j < piece.size();) {
-                if (j + 2 < piece.size() && (unsigned char)piece[j] == 0xE2 && (unsigned char)piece[j + 1] == 0x96
-                        && (unsigned char)piece[j + 2] == 0x81) {
-                    text.push_back(' ');
-                    j += 3;
-                } else {
-                    text.push_back(piece[j++]);
-                }
-            }
+            v.append_text(t, unparse_special, text);
         }
         return string_out(text, buffer, n_buffer, out_n_bytes);
     });
@@ -625,9 +600,16 @@ int retro_engine_adapter_rows_info(retro_engine * engine, retro_adapter_rows_inf
 
 retro_grammar * retro_grammar_from_json_schema(const char * json_schema) {
     clear_error();
-    (void)json_schema;
-    set_error("JSON-schema grammars need llama.cpp's schema converter, which this library does not contain");
-    return nullptr;
+    if (blank(json_schema)) {
+        set_error("json_schema is required");
+        return nullptr;
+    }
+    try {
+        return new retro_grammar{SchemaToGbnf::convert(json_schema)};
+    } catch (const std::exception & e) {
+        set_error(std::string("failed to convert the JSON schema to a grammar: ") + e.what());
+        return nullptr;
+    }
 }
 
 retro_grammar * retro_grammar_from_gbnf(const char * gbnf) {
@@ -641,8 +623,7 @@ retro_grammar * retro_grammar_from_gbnf(const char * gbnf) {
 
 retro_grammar * retro_grammar_json_object(void) {
     clear_error();
-    set_error("the built-in JSON grammar is llama.cpp's grammars/json.gbnf, which this library does not contain");
-    return nullptr;
+    return new retro_grammar{kJsonObjectGbnf};
 }
 
 const char * retro_grammar_gbnf(const retro_grammar * grammar) { return grammar ? grammar->gbnf.c_str() : nullptr; }

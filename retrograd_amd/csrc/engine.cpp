@@ -869,6 +869,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
     // ---- validation: caller errors are reported before anything decodes
     // (order and messages follow retro_gen_core.cpp:2353-2516).
     std::vector<RowView> rows(n_rows);
+    std::vector<std::shared_ptr<Grammar>> compiled(n_rows);
     if (is_v2) {
         for (size_t r = 0; r < n_rows; ++r) {
             const retro_step_row_v2 & in = rows2[r];
@@ -958,8 +959,17 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
             if (row.v2) {
                 if (!valid_sampling_v2(*row.v2, n_vocab)) return -3;
                 if (row.v2->grammar) {
-                    set_error("grammar-constrained rows are not supported by this library");
-                    return -3;
+                    // compiled before anything decodes: an invalid grammar must not leave a prompt in the KV
+                    const std::string & gbnf = row.v2->grammar->gbnf;
+                    auto prev = requests_.find(row.request);
+                    if (prev == requests_.end() || !prev->second.grammar || prev->second.grammar->gbnf() != gbnf) {
+                        try {
+                            compiled[r] = std::make_shared<Grammar>(gbnf);
+                        } catch (const std::exception & e) {
+                            set_error(std::string("failed to compile the request's grammar (invalid GBNF): ") + e.what());
+                            return -3;
+                        }
+                    }
                 }
             } else {
                 retro_sampling_params s = row.v1;
@@ -1157,6 +1167,18 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
                 float * top_lps = k > 0 ? out_top_logprobs + r * n_top_stride : nullptr;
                 const double log_sum = std::log(s.sum_exp);
                 if (row.v2) {
+                    // the grammar of this row becomes (or stays) the request's; a row without one drops it
+                    const GrammarVocab * gv = nullptr;
+                    if (row.v2->grammar) {
+                        if (compiled[r]) req.grammar = compiled[r];
+                        if (!req.grammar || req.grammar->gbnf() != row.v2->grammar->gbnf) {      // the request was freed and reused inside one call
+                            set_error("failed to compile the request's grammar (invalid GBNF)");
+                            return -1;
+                        }
+                        gv = &vocab_.for_grammars(n_vocab);
+                    } else {
+                        req.grammar.reset();
+                    }
                     RowSample got;
                     float token_logit = 0.0f;
                     // Equal logits where an unstable host algorithm of the reference decides which survive - the top_k cut
@@ -1178,7 +1200,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
                         const float * host_row = h_logits_.as<float>() + (size_t)o * n_vocab;
                         std::string err;
                         got = sampling::sample_full_row_v2(host_row, (size_t)n_vocab, *row.v2, req.rng, req.history, scratch_,
-                                                           row.want_logprob, k, top_ids, top_lps, err);
+                                                           row.want_logprob, k, top_ids, top_lps, err, gv ? req.grammar.get() : nullptr, gv);
                         if (got.token < 0) {
                             set_error(err);
                             return -1;
@@ -1189,6 +1211,10 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
                     sampled_logprob = row.want_logprob ? got.sampled_logprob : 0.0f;
                     n_top = k;
                     req.history.push_back(token);
+                    if (gv && !req.grammar->accept(*gv, (uint32_t)token)) {
+                        set_error("the grammar refused the token it had allowed");
+                        return -1;
+                    }
                     // temperature-1 policy logprob: logit - max - log(sum exp(logit - max))
                     logprob = (float)((double)token_logit - s.max - log_sum);
                 } else {

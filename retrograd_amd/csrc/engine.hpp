@@ -9,6 +9,7 @@
 #include "gguf_file.hpp"
 #include "kernels.hpp"
 #include "tokenizer.hpp"
+#include "grammar.hpp"
 #include "sampler.hpp"
 
 #include <map>
@@ -17,6 +18,9 @@
 #include <string>
 #include <unordered_map>
 #include <vector>
+
+// A grammar handle of the C ABI: an owned GBNF text (reference retro_grammar.cpp:20-33).
+struct retro_grammar { std::string gbnf; };
 
 namespace retro {
 
@@ -85,6 +89,51 @@ struct Vocab {
     int32_t eos = -1, eot = -1;
     Tokenizer tokenizer;            // text -> ids (sentencepiece-kind vocabularies)
     std::string tokenizer_error;    // why the vocabulary cannot tokenize, if it cannot
+    GrammarVocab grammar_vocab;     // every token's text as a grammar reads it; built by the first grammar row
+    bool grammar_vocab_ready = false;
+
+    bool is_eog(int32_t t) const { return (eos >= 0 && t == eos) || (eot >= 0 && t == eot); }
+    // The bytes token t stands for, appended to `text`: SentencePiece's U+2581 becomes a space, a byte token
+    // "<0xXX>" its byte, a piece of a byte-pair vocabulary the bytes it spells; control and unknown tokens
+    // contribute their text only with unparse_special.
+    void append_text(int32_t t, bool unparse_special, std::string & text) const {
+        if (t < 0 || (size_t)t >= pieces.size()) return;
+        const int32_t type = (size_t)t < types.size() ? types[(size_t)t] : 1;
+        const std::string & piece = pieces[(size_t)t];
+        if (type == 3 || type == 2) {            // control / unknown
+            if (unparse_special) text += piece;
+            return;
+        }
+        if (type == 6 && piece.size() == 6 && piece.compare(0, 3, "<0x") == 0) {
+            text.push_back((char)std::stoi(piece.substr(3, 2), nullptr, 16));
+            return;
+        }
+        if (tokenizer.model == "gpt2") {
+            text += tokenizer.spelled_bytes(piece);
+            return;
+        }
+        for (size_t j = 0; j < piece.size();) {
+            if (j + 2 < piece.size() && (unsigned char)piece[j] == 0xE2 && (unsigned char)piece[j + 1] == 0x96
+                    && (unsigned char)piece[j + 2] == 0x81) {
+                text.push_back(' ');
+                j += 3;
+            } else {
+                text.push_back(piece[j++]);
+            }
+        }
+    }
+    const GrammarVocab & for_grammars(int32_t n_vocab) {
+        if (!grammar_vocab_ready) {
+            grammar_vocab = GrammarVocab();
+            for (int32_t t = 0; t < n_vocab; ++t) {
+                std::string text;
+                append_text(t, true, text);
+                grammar_vocab.add(text, is_eog(t));
+            }
+            grammar_vocab_ready = true;
+        }
+        return grammar_vocab;
+    }
 };
 
 // Kernel categories of one step, for the optional event-based timing.

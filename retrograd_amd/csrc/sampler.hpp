@@ -15,10 +15,12 @@
 #pragma once
 
 #include "../../include/retro_step.h"
+#include "grammar.hpp"
 
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
+#include <memory>
 #include <numeric>
 #include <random>
 #include <string>
@@ -31,6 +33,7 @@ struct RequestState {
     std::mt19937 rng;
     bool seeded = false;
     std::vector<int32_t> history;   // accepted tokens (v2 rows), what the penalties see
+    std::shared_ptr<Grammar> grammar;   // the request's grammar and where its text so far stands in it
 };
 
 struct RowSample {
@@ -203,12 +206,13 @@ inline int32_t draw_dense(std::vector<double> & w, double total, float top_p, st
     return order[keep - 1];
 }
 
-// v2 chain over a full host row: bias -> penalties(window) -> top_k -> min_p ->
+// v2 chain over a full host row: bias -> penalties(window) -> grammar mask -> top_k -> min_p ->
 // temperature -> top_p -> draw, then post-transformation logprobs.
 inline RowSample sample_full_row_v2(const float * logits, size_t n, const retro_sampling_params_v2 & p,
                                     std::mt19937 & rng, const std::vector<int32_t> & history, FullScratch & s,
                                     bool want_logprob, size_t k_top, int32_t * top_ids, float * top_lps,
-                                    std::string & error) {
+                                    std::string & error, const Grammar * grammar = nullptr,
+                                    const GrammarVocab * grammar_vocab = nullptr) {
     std::vector<float> & t = s.t;
     t.assign(logits, logits + n);
     for (uint32_t i = 0; i < p.n_logit_bias; ++i) t[(size_t)p.logit_bias_ids[i]] += p.logit_bias_values[i];
@@ -223,6 +227,12 @@ inline RowSample sample_full_row_v2(const float * logits, size_t n, const retro_
             if (v <= 0.0f) v *= p.repeat_penalty; else v /= p.repeat_penalty;
             v -= (float)c.second * p.frequency_penalty + (float)(c.second > 0) * p.presence_penalty;
         }
+    }
+    if (grammar && !grammar->mask(*grammar_vocab, t.data(), n)) {
+        error = "grammar allows no token at this position";
+        RowSample bad;
+        bad.token = -1;
+        return bad;
     }
     if (p.top_k > 0 && (size_t)p.top_k < n) {
         s.order.resize(n);

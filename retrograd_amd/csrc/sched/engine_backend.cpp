@@ -23,6 +23,10 @@ void EngineBackend::step(const std::vector<StepRow> & rows, StepOutput & out) {
     bias_ids_.reserve(n_bias);
     bias_values_.reserve(n_bias);
     size_t stride = 0;
+    struct Grammars {
+        std::vector<std::pair<std::string, retro_grammar *>> held;
+        ~Grammars() { for (auto & g : held) retro_grammar_free(g.second); }
+    } grammars;
     for (size_t i = 0; i < rows.size(); ++i) {
         const StepRow & row = rows[i];
         if (row.n == 0) throw InferError::backend("a step row requires at least one token");
@@ -42,8 +46,19 @@ void EngineBackend::step(const std::vector<StepRow> & rows, StepOutput & out) {
         f.adapter = row.adapter;
         const SamplingParamsV2 & p = *row.sampling;
         if (p.logit_bias.size() > 4096) throw InferError::backend("logit_bias takes at most 4096 entries");
-        if (p.grammar_gbnf) throw InferError::backend("grammar-constrained rows are not supported by this engine");
         retro_sampling_params_v2 & s = f.sampling;
+        if (p.grammar_gbnf && row.sample) {
+            // one handle per distinct text of the call (step.rs:440-470), freed when the call is over
+            const retro_grammar * h = nullptr;
+            for (const auto & g : grammars.held) if (g.first == *p.grammar_gbnf) h = g.second;
+            if (!h) {
+                retro_grammar * made = retro_grammar_from_gbnf(p.grammar_gbnf->c_str());
+                if (!made) fail();
+                grammars.held.push_back({*p.grammar_gbnf, made});
+                h = made;
+            }
+            s.grammar = h;
+        }
         s.struct_size = sizeof(retro_sampling_params_v2);
         s.temperature = p.temperature; s.top_p = p.top_p; s.max_new_tokens = p.max_new_tokens; s.seed = p.seed;
         s.top_k = p.top_k; s.min_p = p.min_p; s.repeat_penalty = p.repeat_penalty;

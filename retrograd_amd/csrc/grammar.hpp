@@ -425,15 +425,10 @@ public:
 
     // -inf for every token that cannot come next. Returns whether any token is left.
     bool mask(const GrammarVocab & v, float * logits, size_t n_vocab) const {
-        bool complete = false;
-        for (const Stack & s : stacks_) complete = complete || s.empty();
+        const std::vector<uint8_t> & allowed = allowed_now(v, n_vocab);
         bool any = false;
         for (size_t t = 0; t < n_vocab; ++t) {
-            bool ok;
-            if (t >= v.size()) ok = false;
-            else if (v.eog[t]) ok = complete;
-            else ok = allows(v, (uint32_t)t);
-            if (!ok) logits[t] = -INFINITY;
+            if (!allowed[t]) logits[t] = -INFINITY;
             else any = any || logits[t] != -INFINITY;
         }
         return any;
@@ -469,6 +464,40 @@ private:
         uint32_t floor() const { return length == 2 ? 0x80u : length == 3 ? 0x800u : 0x10000u; }
     };
     Utf8 partial_;                      // what the last accepted token left open
+
+    // The allowed set of a state is a function of the state alone, and generation keeps coming back to a few states
+    // (inside a string, between digits, after a comma): the last sets are kept, keyed by the state.
+    struct Remembered { std::string key; std::vector<uint8_t> allowed; };
+    mutable std::vector<Remembered> remembered_;
+    mutable size_t remembered_next_ = 0;
+
+    const std::vector<uint8_t> & allowed_now(const GrammarVocab & v, size_t n_vocab) const {
+        std::vector<std::string> parts;
+        for (const Stack & s : stacks_) parts.emplace_back((const char *)s.data(), s.size() * sizeof(Pos));
+        std::sort(parts.begin(), parts.end());
+        std::string key;
+        const uint64_t head[2] = {(uint64_t)partial_.value | ((uint64_t)partial_.remain << 32) | ((uint64_t)partial_.length << 40), (uint64_t)n_vocab};
+        key.append((const char *)head, sizeof head);
+        for (const std::string & p : parts) {
+            const uint32_t n = (uint32_t)p.size();
+            key.append((const char *)&n, 4);
+            key += p;
+        }
+        for (const Remembered & r : remembered_) if (r.key == key) return r.allowed;
+        bool complete = false;
+        for (const Stack & s : stacks_) complete = complete || s.empty();
+        std::vector<uint8_t> allowed(n_vocab, 0);
+        for (size_t t = 0; t < n_vocab && t < v.size(); ++t) allowed[t] = v.eog[t] ? complete : allows(v, (uint32_t)t);
+        constexpr size_t kKept = 48;
+        if (remembered_.size() < kKept) {
+            remembered_.push_back({std::move(key), std::move(allowed)});
+            return remembered_.back().allowed;
+        }
+        Remembered & slot = remembered_[remembered_next_++ % kKept];
+        slot.key = std::move(key);
+        slot.allowed = std::move(allowed);
+        return slot.allowed;
+    }
 
     const GrammarSymbol & top(const Stack & s) const {
         const Pos & p = s.back();

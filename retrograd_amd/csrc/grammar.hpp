@@ -87,6 +87,8 @@ private:
     std::map<std::string, uint32_t> ids_;
     std::vector<std::pair<std::string, uint32_t>> used_;
     std::vector<bool> defined_;
+    uint64_t written_ = 0;
+    int depth_ = 0;
 
     [[noreturn]] void fail(const std::string & what) const {
         throw std::runtime_error("invalid GBNF at offset " + std::to_string(at_) + ": " + what);
@@ -205,6 +207,9 @@ private:
     void apply_repeat(Seq & seq, size_t item_from, uint32_t lo, int64_t hi) {      // hi < 0: no upper bound
         const Seq item(seq.begin() + (long)item_from, seq.end());
         if (item.empty()) fail("a repetition needs something to repeat");
+        // repetitions are written out: bounded, so that nested counts cannot ask for more memory than a grammar is worth
+        written_ += (uint64_t)item.size() * (uint64_t)(hi < 0 ? lo + 1 : (uint32_t)hi);
+        if (written_ > (1u << 20)) fail("the grammar's repetitions are too large");
         seq.resize(item_from);
         for (uint32_t i = 0; i < lo; ++i) seq.insert(seq.end(), item.begin(), item.end());
         if (hi < 0) {
@@ -272,6 +277,7 @@ private:
                 at_ += 2;
                 seq.push_back(s);
             } else if (c == '(') {
+                if (++depth_ > 200) fail("groups are nested too deeply");
                 ++at_;
                 skip_space(true);
                 const uint32_t r = fresh_rule();
@@ -280,6 +286,7 @@ private:
                 out_.rules[r] = std::move(alts);
                 if (peek() != ')') fail("')' is expected");
                 ++at_;
+                --depth_;
                 seq.push_back(ref(r));
             } else if (word_char(c)) {
                 const std::string name = parse_name();

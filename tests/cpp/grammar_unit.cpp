@@ -43,6 +43,8 @@ int main(int argc, char ** argv) {
             std::string h; int eog = 0;
             is >> h >> eog;
             vocab.add(unhex(h), eog != 0);
+        } else if (!g && (cmd == "mask" || cmd == "accept")) {
+            std::printf("no grammar\n");
         } else if (cmd == "mask") {
             std::vector<float> logits(vocab.size(), 0.0f);
             const bool any = g->mask(vocab, logits.data(), logits.size());

@@ -37,7 +37,7 @@ def _file(n_tensors=1, n_kv=1, alignment=32, ne=(64, 2), offset=0, ttype=0, payl
 @pytest.fixture(scope="module")
 def reader(tmp_path_factory):
     exe = tmp_path_factory.mktemp("gguf_unit") / "gguf_unit"
-    subprocess.run(["g++", "-std=c++17", "-O1", "-o", str(exe), str(ROOT / "tests/cpp/gguf_unit.cpp")], check=True)
+    subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-o", str(exe), str(ROOT / "tests/cpp/gguf_unit.cpp")], check=True)
     return exe
 
 

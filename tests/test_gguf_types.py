@@ -19,7 +19,7 @@ GEOM = {gw.GGML_Q4_0: (32, 18, [0]), gw.GGML_Q5_0: (32, 22, [0]), gw.GGML_IQ4_NL
 def harness(tmp_path_factory):
     d = tmp_path_factory.mktemp("transcode_unit")
     exe = d / "transcode_unit"
-    subprocess.run(["g++", "-std=c++17", "-O1", "-o", str(exe), str(ROOT / "tests/cpp/transcode_unit.cpp")], check=True)
+    subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-o", str(exe), str(ROOT / "tests/cpp/transcode_unit.cpp")], check=True)
     return exe, d
 
 

@@ -21,7 +21,7 @@ ROOT = Path(__file__).resolve().parent.parent
 def exe(tmp_path_factory):
     d = tmp_path_factory.mktemp("grammar_unit")
     out = d / "grammar_unit"
-    subprocess.run(["g++", "-std=c++17", "-O1", "-o", str(out), str(ROOT / "tests/cpp/grammar_unit.cpp")], check=True)
+    subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-o", str(out), str(ROOT / "tests/cpp/grammar_unit.cpp")], check=True)
     return out, d
 
 
@@ -196,6 +196,8 @@ def test_token_ids_and_text_split_inside_a_character(exe):
     ("root = \"a\"", "'::=' is expected"),
     ("root ::= *", "end of the rule"),
     ("", "no 'root' rule"),
+    ("root ::= \"abcdefghijkl\"{100000}", "too large"),
+    ("root ::= " + "(" * 300 + "\"a\"" + ")" * 300, "nested too deeply"),
 ])
 def test_invalid_grammars_are_refused_with_the_reason(exe, gbnf, message):
     (line,) = run(exe, ["grammar " + hx(gbnf)])
@@ -444,7 +446,7 @@ def _gbnf_of(exe, schema):
     out, d = exe
     unit = d / "schema_unit"
     if not unit.exists():
-        subprocess.run(["g++", "-std=c++17", "-O1", "-o", str(unit), str(ROOT / "tests/cpp/schema_unit.cpp")], check=True)
+        subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-o", str(unit), str(ROOT / "tests/cpp/schema_unit.cpp")], check=True)
     f = d / "schema.json"
     f.write_text(json.dumps(schema))
     r = subprocess.run([str(unit), str(f)], capture_output=True, text=True, timeout=60)

@@ -19,7 +19,7 @@ GOLDEN = json.loads((ROOT / "tests/golden/spm_reference_ids.json").read_text())
 def harness(tmp_path_factory):
     d = tmp_path_factory.mktemp("tokenizer_unit")
     exe = d / "tokenizer_unit"
-    subprocess.run(["g++", "-std=c++17", "-O1", "-o", str(exe), str(ROOT / "tests/cpp/tokenizer_unit.cpp")], check=True)
+    subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-o", str(exe), str(ROOT / "tests/cpp/tokenizer_unit.cpp")], check=True)
     vocab = d / "vocab.txt"
     vocab.write_text("".join("%s %r %d\n" % (p.encode().hex() or "-", s, t) for p, s, t in GOLDEN["vocab"]))
     return exe, vocab, d

@@ -59,8 +59,8 @@ def parse_args():
     ap.add_argument("--activations", default="exact", choices=["exact", "ggml"],
                     help="arithmetic of the measured engine: exact (f16 hi/lo activations, the default and the one the "
                          "logit tolerances are shown on) or ggml (activations converted to Q8_K / Q8_0 as the reference's CPU path does)")
-    ap.add_argument("--kv", default="f16", choices=["f16", "q8_0"],
-                    help="storage of the KV cache; the headline is f16 as the workload names it, q8_0 is a secondary configuration")
+    ap.add_argument("--kv", default="f16", choices=["f16", "q8_0", "q4_0"],
+                    help="storage of the KV cache; the headline is f16 as the workload names it, q8_0 and q4_0 are secondary configurations")
     ap.add_argument("--kernel-steps", type=int, default=8, help="decode steps timed per kernel category after the timed region")
     ap.add_argument("--no-scheduler-leg", action="store_true", help="skip the run of the same workload through the step scheduler")
     ap.add_argument("--scheduler-requests", type=int, default=128)
@@ -341,7 +341,7 @@ def main() -> int:
         os.environ["RETRO_ACTIVATIONS"] = activations
         t0 = time.perf_counter()
         eng = E.Engine(model_path, E.EngineConfig(n_ctx=n_ctx, n_seq_max=n_slots, n_batch=n_batch, n_ubatch=n_batch,
-                                                  kv_dtype=E.KV_Q8_0 if args.kv == "q8_0" else E.KV_F16))
+                                                  kv_dtype={"f16": E.KV_F16, "q8_0": E.KV_Q8_0, "q4_0": E.KV_Q4_0}[args.kv]))
         print("[bench] engine (%s arithmetic) ready in %.1fs" % (activations, time.perf_counter() - t0), file=sys.stderr, flush=True)
         return eng
 
@@ -359,6 +359,8 @@ def main() -> int:
     kv_bytes_per_cell_layer = 2 * hp.n_head_kv * hp.head_dim * 2       # K and V, f16
     if args.kv == "q8_0":
         kv_bytes_per_cell_layer = kv_bytes_per_cell_layer * 17 // 32      # 34 bytes per block of 32 values
+    elif args.kv == "q4_0":
+        kv_bytes_per_cell_layer = kv_bytes_per_cell_layer * 9 // 32       # 18 bytes per block of 32 values
     attn_ms, attn_launches = prof["attention"]
     algo_bytes_per_launch = kv_bytes_per_cell_layer * cells / args.steps
     attn_avg_s = attn_ms / max(attn_launches, 1) * 1e-3
@@ -416,7 +418,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("q4_k" if args.shape != "c2-q4km" else "q4_k / q6_k") + " weights x " + arithmetic + ", f32 accumulate, " + ("f16 KV" if args.kv == "f16" else "Q8_0 KV (a secondary configuration: the workload names an f16 cache)"),
+        "dtype": ("q4_k" if args.shape != "c2-q4km" else "q4_k / q6_k") + " weights x " + arithmetic + ", f32 accumulate, " + ("f16 KV" if args.kv == "f16" else args.kv.upper() + " KV (a secondary configuration: the workload names an f16 cache)"),
         "data": "synthetic",
         "config": {
             "workload": "configs[1]: %s, %d live sequences, prompts log-uniform [%d,%d], greedy, %d new tokens, continuous batching"

@@ -76,7 +76,7 @@ typedef struct retro_train_config {
     float gefen_beta2;
     float gefen_eps;
     int32_t master_weights;
-    int32_t generation_kv_dtype;       /* retro_generation_kv_dtype; only f16 (0) is implemented */
+    int32_t generation_kv_dtype;       /* retro_generation_kv_dtype: f16 (0), q8_0 (1), q4_0 (2) */
 } retro_train_config;
 
 /* :1532 / :2456. */

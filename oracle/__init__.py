@@ -258,7 +258,7 @@ class Model:
 
 
 class Context:
-    """Per-slot dense KV (f16, or Q8_0 blocks with kv="q8_0") and one decode per step() over a packed batch.
+    """Per-slot dense KV (f16, or Q8_0 / Q4_0 blocks with kv="q8_0" / "q4_0") and one decode per step() over a packed batch.
 
     activations: "exact" multiplies every weight with the f32 activations as they
     are (the product's default arithmetic, on which the logit tolerances are
@@ -269,14 +269,14 @@ class Context:
     def __init__(self, model: Model, n_seq_max: int, activations: str = "exact", kv: str = "f16") -> None:
         if activations not in ("exact", "ggml"):
             raise ValueError("activations must be 'exact' or 'ggml'")
-        if kv not in ("f16", "q8_0"):
-            raise ValueError("kv must be 'f16' or 'q8_0'")
+        if kv not in ("f16", "q8_0", "q4_0"):
+            raise ValueError("kv must be 'f16', 'q8_0' or 'q4_0'")
         self.model = model
         self._h = lib().orc_ctx_new(model._h, n_seq_max)
         if not self._h:
             raise OracleError(lib().orc_last_error().decode())
         lib().orc_ctx_set_exact(self._h, 1 if activations == "exact" else 0)
-        lib().orc_ctx_set_kv_q8(self._h, 1 if kv == "q8_0" else 0)
+        lib().orc_ctx_set_kv_q8(self._h, {"f16": 0, "q8_0": 8, "q4_0": 4}[kv])
 
     def step(self, token, pos, slot, want, adapter_of=None) -> np.ndarray:
         token = np.ascontiguousarray(token, np.int32)
@@ -351,6 +351,24 @@ class Context:
             for l in range(n_layer):
                 k = values(body[(2 * l) * per:(2 * l + 1) * per])
                 v = values(body[(2 * l + 1) * per:(2 * l + 2) * per])
+                _check(lib().orc_ctx_import_kv_f32(self._h, l, slot, begin, end, _ptr(k, _f32p), _ptr(v, _f32p)))
+            return
+        if int(head[0]) == 0x34564b52:
+            # a Q4_0 cache ("RKV4"): per row and kv head head_dim / 2 code bytes (element 2 k in the low nibble of
+            # byte k), then head_dim / 32 f16 scales; a value is scale times (code - 8)
+            hd, n_kv = self.model.head_dim, self.model.n_head_kv
+            per_head = hd // 4 + hd // 32
+            assert kd == n_kv * per_head
+
+            def values4(units):
+                rows = units.reshape(n, n_kv, per_head)
+                packed = np.ascontiguousarray(rows[:, :, :hd // 4]).view(np.uint8)
+                codes = np.stack([packed & 15, packed >> 4], axis=-1).reshape(n, n_kv, hd).astype(np.float32) - 8.0
+                scales = np.ascontiguousarray(rows[:, :, hd // 4:]).view(np.float16).astype(np.float32)
+                return np.ascontiguousarray((codes.reshape(n, n_kv, hd // 32, 32) * scales[..., None]).reshape(n, n_kv * hd))
+            for l in range(n_layer):
+                k = values4(body[(2 * l) * per:(2 * l + 1) * per])
+                v = values4(body[(2 * l + 1) * per:(2 * l + 2) * per])
                 _check(lib().orc_ctx_import_kv_f32(self._h, l, slot, begin, end, _ptr(k, _f32p), _ptr(v, _f32p)))
             return
         for l in range(n_layer):

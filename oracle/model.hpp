@@ -142,6 +142,27 @@ inline void q8_0_row_values(const float * x, size_t K, float * out) {
     }
 }
 
+// A row as Q4_0 blocks hold it (ggml's quantize_row_q4_0_ref: per 32 values the element m of largest magnitude, the
+// first of equals; d = m / -8; code = min(15, (int8)(x / d + 8.5)) with the unrounded d), written back as
+// (code - 8) times d rounded to f16 (quant.rs:236-245 decodes such a block the same way).
+inline void q4_0_row_values(const float * x, size_t K, float * out) {
+    if (K % 32) throw std::runtime_error("oracle: Q4_0 rows need whole blocks of 32");
+    for (size_t b = 0; b < K; b += 32) {
+        float amax = 0.0f, mx = 0.0f;
+        for (int j = 0; j < 32; ++j) {
+            const float v = x[b + j];
+            if (amax < std::fabs(v)) { amax = std::fabs(v); mx = v; }
+        }
+        const float d = mx / -8.0f;
+        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        const float dh = half_to_float(float_to_half(d));
+        for (int j = 0; j < 32; ++j) {
+            const int q = std::min(15, (int)(int8_t)(x[b + j] * id + 8.5f));
+            out[b + j] = dh * (float)(q - 8);
+        }
+    }
+}
+
 inline void ggml_activation_row(uint32_t wtype, const float * x, size_t K, float * out) {
     if (exact_activations()) { std::copy(x, x + K, out); return; }
     switch (wtype) {
@@ -286,7 +307,7 @@ struct context {
     // (quant.hpp) when it is stored; attention then reads scale times code. Under the ggml arithmetic ggml's CPU
     // flash attention would also convert the query row to Q8_0 for the K product (the vec_dot_type of Q8_0): done
     // here when `exact` is off.
-    bool kv_q8 = false;
+    int kv_q8 = 0;          // 0: an f16 cache; 8 / 4: Q8_0 / Q4_0 blocks
 
     int kv_dim() const { return mdl->hp.n_head_kv * mdl->hp.head_dim; }
 
@@ -427,9 +448,9 @@ struct context {
                 float * kc = &s.k[(size_t)l][(size_t)pos[t] * kd];
                 float * vc = &s.v[(size_t)l][(size_t)pos[t] * kd];
                 if (kv_q8) {
-                    if (HD % 32 != 0) throw std::runtime_error("oracle: a Q8_0 cache needs heads of whole 32-blocks");
-                    q8_0_row_values(&k[(size_t)t * KD], (size_t)KD, kc);
-                    q8_0_row_values(&v[(size_t)t * KD], (size_t)KD, vc);
+                    if (HD % 32 != 0) throw std::runtime_error("oracle: a quantised cache needs heads of whole 32-blocks");
+                    (kv_q8 == 4 ? q4_0_row_values : q8_0_row_values)(&k[(size_t)t * KD], (size_t)KD, kc);
+                    (kv_q8 == 4 ? q4_0_row_values : q8_0_row_values)(&v[(size_t)t * KD], (size_t)KD, vc);
                 } else {
                     for (int i = 0; i < KD; ++i) {
                         kc[i] = half_to_float(float_to_half(k[(size_t)t * KD + i]));
@@ -448,7 +469,7 @@ struct context {
                     const int kvh = hh / G;
                     const float * qh = &q[(size_t)t * QD + (size_t)hh * HD];
                     std::vector<float> qconv;
-                    if (kv_q8 && !exact) {      // ggml: the query row as Q8_0, the companion format of a Q8_0 K row
+                    if (kv_q8 && !exact) {      // ggml: the query row as Q8_0, the companion format of a Q8_0 or Q4_0 K row
                         qconv.resize((size_t)HD);
                         q8_0_row_values(qh, (size_t)HD, qconv.data());
                         qh = qconv.data();

@@ -147,7 +147,7 @@ void * orc_ctx_new(void * m, int n_seq_max) {
 }
 void orc_ctx_free(void * c) { delete (context *)c; }
 void orc_ctx_set_exact(void * c, int on) { ((context *)c)->exact = on != 0; }
-void orc_ctx_set_kv_q8(void * c, int on) { ((context *)c)->kv_q8 = on != 0; }
+void orc_ctx_set_kv_q8(void * c, int bits) { ((context *)c)->kv_q8 = bits == 8 || bits == 4 ? bits : 0; }
 // The stored K or V row of (layer, slot, pos) as the kv_dim values the cache holds, f32.
 int orc_ctx_read_kv_f32(void * c, int layer, int slot, int pos, int want_v, float * out) {
     return guard([&] {

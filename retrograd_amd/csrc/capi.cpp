@@ -94,8 +94,8 @@ bool validate_config(const retro_engine_config & c, bool * invalid_placement) {
         set_error("device=cpu requested, but this library only executes on an MI355X GPU");
         return false;
     }
-    if (c.kv_dtype != RETRO_ENGINE_KV_DTYPE_F16 && c.kv_dtype != RETRO_ENGINE_KV_DTYPE_Q8_0) {
-        set_error("only the f16 and the q8_0 KV cache are implemented by this library");
+    if (c.kv_dtype == RETRO_ENGINE_KV_DTYPE_F32) {
+        set_error("the f32 KV cache is not implemented by this library (f16, q8_0 and q4_0 are)");
         return false;
     }
     if (c.expert_placement == RETRO_EXPERT_PLACEMENT_HOST || c.expert_device_cache_bytes != 0) {

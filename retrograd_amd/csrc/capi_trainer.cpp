@@ -70,10 +70,6 @@ bool validate(const retro_train_config & c) {
         set_error("a quantized generation_kv_dtype requires fast_generation_context");
         return false;
     }
-    if (c.generation_kv_dtype == 2) {
-        set_error("only the f16 and the q8_0 KV cache are implemented by this library");
-        return false;
-    }
     if (c.device < RETRO_DEVICE_AUTO || c.device > RETRO_DEVICE_GPU) {
         set_error("device must be one of retro_device");
         return false;
@@ -117,7 +113,8 @@ retro_trainer * retro_trainer_new(const char * model_path, const retro_train_con
         batch = std::max(batch, train_config->generation_concurrency);
         ec.n_batch = batch;
         ec.n_ubatch = batch;
-        ec.kv_dtype = train_config->generation_kv_dtype == 1 ? RETRO_ENGINE_KV_DTYPE_Q8_0 : RETRO_ENGINE_KV_DTYPE_F16;
+        ec.kv_dtype = train_config->generation_kv_dtype == 1 ? RETRO_ENGINE_KV_DTYPE_Q8_0
+                    : train_config->generation_kv_dtype == 2 ? RETRO_ENGINE_KV_DTYPE_Q4_0 : RETRO_ENGINE_KV_DTYPE_F16;
         ec.flash_attn = true;
         ec.device = train_config->device;
         ec.threads = train_config->threads;

@@ -94,8 +94,8 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     // n_ctx distinct cells always finds its pages.
     n_pages_ = (int)((cfg_.n_ctx + rk::PAGE - 1) / rk::PAGE + 2 * cfg_.n_seq_max);
     // [page][kv head]: the other order (a head's pages side by side) was measured 3 % slower in the attention kernel
-    kv_q8_ = cfg_.kv_dtype == RETRO_ENGINE_KV_DTYPE_Q8_0;
-    if (kv_q8_ && hp_.head_dim % 32 != 0) throw std::runtime_error("a Q8_0 KV cache needs head_dim to be a multiple of 32");
+    kv_q8_ = cfg_.kv_dtype == RETRO_ENGINE_KV_DTYPE_Q8_0 ? rk::KV_Q8 : cfg_.kv_dtype == RETRO_ENGINE_KV_DTYPE_Q4_0 ? rk::KV_Q4 : rk::KV_F16;
+    if (kv_q8_ != rk::KV_F16 && hp_.head_dim % 32 != 0) throw std::runtime_error("a Q8_0 or Q4_0 KV cache needs head_dim to be a multiple of 32");
     kv_strides_ = rk::kv_strides(n_pages_, hp_.n_head_kv, hp_.head_dim, false, kv_q8_);
     const int G = hp_.n_head / hp_.n_head_kv;
     if (hp_.n_head % hp_.n_head_kv != 0 || G > 16) throw std::runtime_error("unsupported attention head grouping");
@@ -647,14 +647,18 @@ int Engine::memory(retro_engine_memory_info * out) {
 // ---- snapshots -------------------------------------------------------------------------
 //
 // Byte format (this library's own; only seq_load of the same build reads it):
-//   u32 magic "RKV1" (an f16 cache) or "RKV8" (a Q8_0 cache), u32 flags, i32 n_layer, i32 halves per row,
+//   u32 magic "RKV1" (an f16 cache), "RKV8" (Q8_0) or "RKV4" (Q4_0), u32 flags, i32 n_layer, i32 halves per row,
 //   i32 begin, i32 end, then per layer the K rows [end-begin] and the V rows: kv_dim f16 values in
-//   natural order, or - Q8_0 - per kv head head_dim code bytes (code + 128) and head_dim / 32 f16 scales.
+//   natural order, or per kv head the codes (Q8_0: head_dim bytes, code + 128; Q4_0: head_dim / 2 bytes, element
+//   2 k in the low nibble of byte k) and head_dim / 32 f16 scales.
 namespace {
 struct SnapHeader { uint32_t magic, flags; int32_t n_layer, kv_dim, begin, end; };
 constexpr uint32_t kSnapMagic = 0x31564b52u;
 constexpr uint32_t kSnapMagicQ8 = 0x38564b52u;
+constexpr uint32_t kSnapMagicQ4 = 0x34564b52u;        // "RKV4"
 }
+
+uint32_t Engine::snap_magic() const { return kv_q8_ == rk::KV_Q8 ? kSnapMagicQ8 : kv_q8_ == rk::KV_Q4 ? kSnapMagicQ4 : kSnapMagic; }
 
 int Engine::seq_save(int32_t slot, uint32_t flags, uint8_t * buffer, size_t n_buffer, size_t * out_n_bytes) {
     if (!out_n_bytes) {
@@ -680,7 +684,7 @@ int Engine::seq_save(int32_t slot, uint32_t flags, uint8_t * buffer, size_t n_bu
         set_error("the save buffer is too small for this sequence's state");
         return -2;
     }
-    SnapHeader h{kv_q8_ ? kSnapMagicQ8 : kSnapMagic, flags, hp_.n_layer, (int32_t)kd, partial_only ? 0 : s.begin, partial_only ? 0 : s.begin + n_pos};
+    SnapHeader h{snap_magic(), flags, hp_.n_layer, (int32_t)kd, partial_only ? 0 : s.begin, partial_only ? 0 : s.begin + n_pos};
     std::memcpy(buffer, &h, sizeof(h));
     if (n_pos > 0) {
         std::vector<int32_t> cells((size_t)n_pos);
@@ -725,7 +729,7 @@ int Engine::seq_load(int32_t slot, uint32_t flags, const uint8_t * buffer, size_
     if (n_bytes < sizeof(h)) { set_error(refused); return -1; }
     std::memcpy(&h, buffer, sizeof(h));
     const size_t kd = rk::kv_row_halves(hp_.n_head_kv, hp_.head_dim, kv_q8_);
-    if (h.magic != (kv_q8_ ? kSnapMagicQ8 : kSnapMagic) || h.flags != flags || h.n_layer != hp_.n_layer || h.kv_dim != (int32_t)kd
+    if (h.magic != snap_magic() || h.flags != flags || h.n_layer != hp_.n_layer || h.kv_dim != (int32_t)kd
             || h.begin < 0 || h.end < h.begin || h.end > n_ctx_seq_) {
         set_error(refused);
         return -1;
@@ -1260,7 +1264,7 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
 void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_rows, bool routed) {
     const HParams & h = hp_;
     const int E = h.n_embd, QD = h.n_head * h.head_dim, KD = h.n_head_kv * h.head_dim, F = h.n_ff;
-    rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps, kv_strides_.page, kv_strides_.head, kv_q8_, kv_q8_ && ggml_activations_};
+    rk::AttnShape sh{h.n_head, h.n_head_kv, h.head_dim, h.rope_dim, h.rope_neox, h.eps, kv_strides_.page, kv_strides_.head, kv_q8_, kv_q8_ != rk::KV_F16 && ggml_activations_};
     // The versions of a row its consumers need: the values themselves for F32 / F16 / BF16 weights, the
     // expert router and LoRA factors (`plain`); the converted row for the quantised weights.
     const bool faithful = ggml_activations_;

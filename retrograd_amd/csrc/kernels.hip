@@ -1377,8 +1377,8 @@ struct RopeArgs {
     float eps, qscale;
     Slices from;
     size_t page_stride, head_stride;
-    int kv_q8;
-    int q_q8;        // the ggml arithmetic over a Q8_0 cache: the query row is converted to Q8_0 as well
+    int kv_quant;    // KV_F16, KV_Q8 or KV_Q4
+    int q_q8;        // the ggml arithmetic over a quantised cache: the query row is converted to Q8_0 as well
 };
 
 // One wave per head: lanes own element pairs.
@@ -1485,7 +1485,7 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
     const int cell = a.cell[t];
     const int page = cell / PAGE, t32 = cell % PAGE;
     const int kvh = is_k ? head - a.n_head : head - a.n_head - a.n_kv;
-    if (a.kv_q8) {
+    if (a.kv_quant == KV_Q8) {
         float c0, c1, d;
         q8_pair(c0, c1, d);
         const int e = 2 * lane;
@@ -1502,6 +1502,57 @@ __global__ __launch_bounds__(256) void k_rope_store(RopeArgs a) {
             blk[blk_idx * 1024 + (tg * 16 + dd + 1) * 16 + hi * 8 + ti] = (uint8_t)b1;
         }
         if ((lane & 15) == 0) ((__half *)(blk + (a.hd / 32) * 1024))[blk_idx * 32 + tg * 8 + ti] = __float2half_rn(d);
+        return;
+    }
+    if (a.kv_quant == KV_Q4) {
+        // ggml's quantize_row_q4_0_ref: d = m / -8 for the element m of largest magnitude (the first of equals),
+        // code = min(15, (int)(x / d + 8.5)) with the unrounded d. Lane L owns elements 2 L and 2 L + 1 after the
+        // exchange through LDS, sixteen lanes a block.
+        float * mine = stash[threadIdx.x >> 6];
+        mine[i0] = x0;
+        mine[i1] = x1;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        const float v0 = mine[2 * lane], v1 = mine[2 * lane + 1];
+        float amax = fabsf(v0), mval = v0;
+        int midx = 2 * lane;
+        if (fabsf(v1) > amax) { amax = fabsf(v1); mval = v1; midx = 2 * lane + 1; }
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) {
+            const float oa = __shfl_xor(amax, o, 64), ov = __shfl_xor(mval, o, 64);
+            const int oi = __shfl_xor(midx, o, 64);
+            if (oa > amax || (oa == amax && oi < midx)) { amax = oa; mval = ov; midx = oi; }
+        }
+        const float d = __fdiv_rn(mval, -8.0f);
+        const float id = d != 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
+        const uint32_t q0 = (uint32_t)min(15, (int)(int8_t)__fadd_rn(__fmul_rn(v0, id), 8.5f));
+        const uint32_t q1 = (uint32_t)min(15, (int)(int8_t)__fadd_rn(__fmul_rn(v1, id), 8.5f));
+        const int e = 2 * lane;
+        uint8_t * blk = (uint8_t *)((is_k ? a.k_pool : a.v_pool) + (size_t)page * a.page_stride + (size_t)kvh * a.head_stride);
+        const int tg = (t32 & 15) >> 2, ti = (t32 & 3) + 4 * (t32 >> 4);      // the token's place among a lane's eight
+        const int blk_idx = e >> 5;
+        if (is_k) {
+            // four lanes hold the eight codes of one 32-bit word (this token's dims 8 g .. 8 g + 7): joined, then one store
+            const int g = (e >> 3) & 3, i = e & 7;
+            uint32_t word = (q0 << (4 * kv_nibble(i))) | (q1 << (4 * kv_nibble(i + 1)));
+            word |= __shfl_xor(word, 1, 64);
+            word |= __shfl_xor(word, 2, 64);
+            if ((lane & 3) == 0)
+                *(uint32_t *)(blk + blk_idx * 512 + (g * 16 + (t32 & 15)) * 8 + (t32 >> 4) * 4) = word;
+        } else {
+            // a word of V holds one dimension of eight tokens: this token's nibble is replaced atomically, other
+            // tokens of the step may be writing theirs into the same word
+            const int hi = (e >> 4) & 1, dd = e & 15;
+            const int sh = 4 * kv_nibble(ti);
+            uint32_t * w0 = (uint32_t *)(blk + blk_idx * 512 + (tg * 16 + dd) * 8 + hi * 4);
+            uint32_t * w1 = (uint32_t *)(blk + blk_idx * 512 + (tg * 16 + dd + 1) * 8 + hi * 4);
+            atomicAnd(w0, ~(0xfu << sh));
+            atomicOr(w0, q0 << sh);
+            atomicAnd(w1, ~(0xfu << sh));
+            atomicOr(w1, q1 << sh);
+        }
+        if ((lane & 15) == 0) ((__half *)(blk + (a.hd / 32) * 512))[blk_idx * 32 + tg * 8 + ti] = __float2half_rn(d);
         return;
     }
     if (is_k) {
@@ -1529,8 +1580,9 @@ void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, c
     a.qscale = 1.4426950408889634f / sqrtf((float)sh.head_dim);
     a.from = from;
     a.page_stride = sh.page_stride; a.head_stride = sh.head_stride;
-    a.kv_q8 = sh.kv_q8 ? 1 : 0;
-    a.q_q8 = sh.kv_q8 && sh.q_q8 ? 1 : 0;
+    a.kv_quant = sh.kv_quant;
+    a.q_q8 = sh.kv_quant != KV_F16 && sh.q_q8 ? 1 : 0;
+    if (sh.kv_quant != KV_F16 && sh.kv_quant != KV_Q8 && sh.kv_quant != KV_Q4) throw std::runtime_error("rope_store: unknown cache type");
     if (sh.page_stride == 0 || sh.head_stride == 0) throw std::runtime_error("rope_store: the pool's strides are missing");
     if (from.n > 0 && from.N != (sh.n_head + 2 * sh.n_head_kv) * sh.head_dim)
         throw std::runtime_error("rope_store: the slices are not a fused q, k, v product");
@@ -1542,9 +1594,11 @@ void rope_store(hipStream_t s, const float * qkv, int T, const AttnShape & sh, c
 // ---------------------------------------------------------------------------
 // paged attention
 
-// The K (V) blocks a wave holds for one page: f16 operands, or - a Q8_0 cache - code bytes and block scales.
-template <int N, bool Q8> struct KvRegs { h8 r[N]; };
-template <int N> struct KvRegs<N, true> { u4 raw[N / 2]; u4 sc[N / 2]; };
+// The K (V) blocks a wave holds for one page: f16 operands, or - a Q8_0 / Q4_0 cache - codes and block scales.
+typedef uint32_t kv_u2 __attribute__((ext_vector_type(2)));
+template <int N, int KVQ> struct KvRegs { h8 r[N]; };
+template <int N> struct KvRegs<N, KV_Q8> { u4 raw[N / 2]; u4 sc[N / 2]; };
+template <int N> struct KvRegs<N, KV_Q4> { kv_u2 raw[N / 2]; u4 sc[N / 2]; };
 // Eight bytes (code + 128) as eight f16 codes: 0x6400 | byte is 1024 + byte, exactly.
 __device__ __forceinline__ h8 codes8(uint32_t w0, uint32_t w1) {
     const h2 bias = {(_Float16)(-1152.0f), (_Float16)(-1152.0f)};
@@ -1552,6 +1606,17 @@ __device__ __forceinline__ h8 codes8(uint32_t w0, uint32_t w1) {
     const h2 a1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w0, 0x04030402u)) + bias;
     const h2 a2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04010400u)) + bias;
     const h2 a3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0x64646464u, w1, 0x04030402u)) + bias;
+    return (h8){a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
+}
+
+// Eight four-bit codes q of a word as eight f16 values q - 8, in the order kv_nibble stores them: a mask leaves
+// nibbles 0 and 4 of the (shifted) word in the low bits of two halves whose other bits are those of 1024.
+__device__ __forceinline__ h8 codes4(uint32_t w) {
+    const h2 bias = {(_Float16)(-1032.0f), (_Float16)(-1032.0f)};
+    const h2 a0 = __builtin_bit_cast(h2, (w & 0x000f000fu) | 0x64006400u) + bias;
+    const h2 a1 = __builtin_bit_cast(h2, ((w >> 4) & 0x000f000fu) | 0x64006400u) + bias;
+    const h2 a2 = __builtin_bit_cast(h2, ((w >> 8) & 0x000f000fu) | 0x64006400u) + bias;
+    const h2 a3 = __builtin_bit_cast(h2, ((w >> 12) & 0x000f000fu) | 0x64006400u) + bias;
     return (h8){a0.x, a0.y, a1.x, a1.y, a2.x, a2.y, a3.x, a3.y};
 }
 
@@ -1579,11 +1644,12 @@ struct AttnArgs {
 // arithmetic of a column does not depend on ONE or on what else is in its tile, so a token's result is the
 // same bits in a decode step and in a mixed step. Without SPLIT a tile holds 16 / G tokens and the lo halves
 // take a second instruction each.
-// Q8: the pools hold Q8_0 blocks (kernels.hpp). K enters the score products as its codes, one 32-wide k-step
-// being one block, and the block's scale multiplies that step's products; V enters as its codes and its scales
-// join the probabilities, one version of the probability operand per 32-wide block of dimensions.
-template <int HD, bool ONE, bool SPLIT, bool Q8 = false>
+// KVQ = KV_Q8 / KV_Q4: the pools hold Q8_0 / Q4_0 blocks (kernels.hpp). K enters the score products as its codes,
+// one 32-wide k-step being one block, and the block's scale multiplies that step's products; V enters as its codes
+// and its scales join the probabilities, one version of the probability operand per 32-wide block of dimensions.
+template <int HD, bool ONE, bool SPLIT, int KVQ = KV_F16>
 __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
+    constexpr bool Q8 = KVQ != KV_F16;       // a quantised cache of either width
     constexpr int KS = HD / 32;     // k-steps of QK^T
     constexpr int DT = HD / 16;     // dim tiles of PV
     const int item = blockIdx.x;
@@ -1623,17 +1689,24 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     // page ids of this split, one per lane
     const int n_pages = page_end - page_first;
     const int my_pid = lane < n_pages ? a.table[(size_t)slot * a.max_pages + page_first + lane] : 0;
-    typedef KvRegs<2 * KS, Q8> KSet;          // f16: [k-step][token half]
-    typedef KvRegs<DT, Q8> VSet;
+    typedef KvRegs<2 * KS, KVQ> KSet;          // f16: [k-step][token half]
+    typedef KvRegs<DT, KVQ> VSet;
     auto load_k = [&](int idx, KSet & ks) {
         const int pid = __builtin_amdgcn_readlane(my_pid, idx);
         const __half * kp = a.k_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
-        if constexpr (Q8) {
+        if constexpr (KVQ == KV_Q8) {
             const uint8_t * kb = (const uint8_t *)kp;
 #pragma unroll
             for (int j = 0; j < KS; ++j) {
                 ks.raw[j] = *(const u4 *)(kb + j * 1024 + lane * 16);
                 ks.sc[j] = *(const u4 *)(kb + KS * 1024 + (j * 4 + g) * 16);
+            }
+        } else if constexpr (KVQ == KV_Q4) {
+            const uint8_t * kb = (const uint8_t *)kp;
+#pragma unroll
+            for (int j = 0; j < KS; ++j) {
+                ks.raw[j] = *(const kv_u2 *)(kb + j * 512 + lane * 8);
+                ks.sc[j] = *(const u4 *)(kb + KS * 512 + (j * 4 + g) * 16);
             }
         } else {
 #pragma unroll
@@ -1646,12 +1719,19 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     auto load_v = [&](int idx, VSet & vs) {
         const int pid = __builtin_amdgcn_readlane(my_pid, idx);
         const __half * vp = a.v_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
-        if constexpr (Q8) {
+        if constexpr (KVQ == KV_Q8) {
             const uint8_t * vb = (const uint8_t *)vp;
 #pragma unroll
             for (int b = 0; b < KS; ++b) {
                 vs.raw[b] = *(const u4 *)(vb + b * 1024 + lane * 16);
                 vs.sc[b] = *(const u4 *)(vb + KS * 1024 + (b * 4 + g) * 16);
+            }
+        } else if constexpr (KVQ == KV_Q4) {
+            const uint8_t * vb = (const uint8_t *)vp;
+#pragma unroll
+            for (int b = 0; b < KS; ++b) {
+                vs.raw[b] = *(const kv_u2 *)(vb + b * 512 + lane * 8);
+                vs.sc[b] = *(const u4 *)(vb + KS * 512 + (b * 4 + g) * 16);
             }
         } else {
 #pragma unroll
@@ -1682,7 +1762,9 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
         for (int j = 0; j < KS; ++j) {
             if constexpr (Q8) {
                 const f4 zero = (f4){0.f, 0.f, 0.f, 0.f};
-                const h8 k0 = codes8(ks.raw[j].x, ks.raw[j].y), k1 = codes8(ks.raw[j].z, ks.raw[j].w);
+                h8 k0, k1;
+                if constexpr (KVQ == KV_Q8) { k0 = codes8(ks.raw[j].x, ks.raw[j].y); k1 = codes8(ks.raw[j].z, ks.raw[j].w); }
+                else { k0 = codes4(ks.raw[j].x); k1 = codes4(ks.raw[j].y); }
                 f4 u0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0, qreg[j], zero, 0, 0, 0);
                 f4 u1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1, qreg[j], zero, 0, 0, 0);
                 if (!SPLIT) {
@@ -1775,7 +1857,8 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
             h8 vd;
             if constexpr (Q8) {
                 if ((d & 1) == 0) operand(d >> 1, pt, pt_lo);
-                vd = (d & 1) ? codes8(vs.raw[d >> 1].z, vs.raw[d >> 1].w) : codes8(vs.raw[d >> 1].x, vs.raw[d >> 1].y);
+                if constexpr (KVQ == KV_Q8) vd = (d & 1) ? codes8(vs.raw[d >> 1].z, vs.raw[d >> 1].w) : codes8(vs.raw[d >> 1].x, vs.raw[d >> 1].y);
+                else vd = (d & 1) ? codes4(vs.raw[d >> 1].y) : codes4(vs.raw[d >> 1].x);
             } else {
                 vd = vreg[d];
             }
@@ -1849,7 +1932,12 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
         else hipLaunchKernelGGL((k_attention<HD_, false, false, Q8_>), dim3(n_items), dim3(64), 0, s, a); \
     } while (0)
 #define ATTN_LAUNCH(HD_) \
-    do { if (sh.kv_q8) ATTN_LAUNCH_Q(HD_, true); else ATTN_LAUNCH_Q(HD_, false); } while (0)
+    do { \
+        if (sh.kv_quant == KV_Q8) ATTN_LAUNCH_Q(HD_, KV_Q8); \
+        else if (sh.kv_quant == KV_Q4) ATTN_LAUNCH_Q(HD_, KV_Q4); \
+        else if (sh.kv_quant == KV_F16) ATTN_LAUNCH_Q(HD_, KV_F16); \
+        else throw std::runtime_error("attention: unknown cache type"); \
+    } while (0)
     switch (sh.head_dim) {
         case 32:  ATTN_LAUNCH(32); break;
         case 64:  ATTN_LAUNCH(64); break;
@@ -2047,16 +2135,59 @@ __global__ void k_kv_gather_q8(const __half * pool, KvStrides st, int n_kv, int 
     }
 }
 
+// The Q4_0 pool: one 16-bit unit per thread - four codes (elements 4u .. 4u + 3 of the head's row, element 2 k in
+// the low nibble of byte k) or, past the codes, one block scale. Rows of kv_row_halves units. Scattered codes
+// replace their nibbles atomically: the words they sit in hold other elements (K) or other tokens (V) as well.
+__global__ void k_kv_gather_q4(const __half * pool, KvStrides st, int n_kv, int hd, int is_v, const int32_t * cells, int n,
+                               uint16_t * out, int scatter) {
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int per_head = hd / 4 + hd / 32;
+    if (gid >= (size_t)n * n_kv * per_head) return;
+    const int idx = (int)(gid / ((size_t)n_kv * per_head)), rest = (int)(gid % ((size_t)n_kv * per_head));
+    const int kvh = rest / per_head, u = rest % per_head;
+    const int cell = cells[idx];
+    const int page = cell / PAGE, t32 = cell % PAGE;
+    uint8_t * blk = (uint8_t *)(const_cast<__half *>(pool) + (size_t)page * st.page + (size_t)kvh * st.head);
+    const int tg = (t32 & 15) >> 2, ti = (t32 & 3) + 4 * (t32 >> 4);
+    if (u >= hd / 4) {
+        uint16_t * sc = (uint16_t *)(blk + (hd / 32) * 512) + (u - hd / 4) * 32 + tg * 8 + ti;
+        if (scatter) *sc = out[gid]; else out[gid] = *sc;
+        return;
+    }
+    const int e0 = 4 * u, b = e0 >> 5;
+    uint32_t unit = scatter ? out[gid] : 0;
+    for (int k = 0; k < 4; ++k) {
+        const int e = e0 + k;
+        uint32_t * word;
+        int sh;
+        if (!is_v) {
+            word = (uint32_t *)(blk + b * 512 + (((e >> 3) & 3) * 16 + (t32 & 15)) * 8 + (t32 >> 4) * 4);
+            sh = 4 * kv_nibble(e & 7);
+        } else {
+            word = (uint32_t *)(blk + b * 512 + (tg * 16 + (e & 15)) * 8 + ((e >> 4) & 1) * 4);
+            sh = 4 * kv_nibble(ti);
+        }
+        if (scatter) {
+            atomicAnd(word, ~(0xfu << sh));
+            atomicOr(word, ((unit >> (4 * k)) & 0xfu) << sh);
+        } else {
+            unit |= ((*word >> sh) & 0xfu) << (4 * k);
+        }
+    }
+    if (!scatter) out[gid] = (uint16_t)unit;
+}
+
 void kv_gather(hipStream_t s, const __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
-               const int32_t * cells, int n, __half * out, bool q8) {
+               const int32_t * cells, int n, __half * out, int kvq) {
     if (n <= 0) return;
-    if (q8) {
-        const size_t total = (size_t)n * kv_row_halves(n_kv_heads, head_dim, true);
-        hipLaunchKernelGGL(k_kv_gather_q8, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, st, n_kv_heads,
-                           head_dim, is_v ? 1 : 0, cells, n, (uint16_t *)out, 0);
+    if (kvq == KV_Q8 || kvq == KV_Q4) {
+        const size_t total = (size_t)n * kv_row_halves(n_kv_heads, head_dim, kvq);
+        hipLaunchKernelGGL(kvq == KV_Q8 ? k_kv_gather_q8 : k_kv_gather_q4, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                           pool, st, n_kv_heads, head_dim, is_v ? 1 : 0, cells, n, (uint16_t *)out, 0);
         check_launch("kv_gather");
         return;
     }
+    if (kvq != KV_F16) throw std::runtime_error("kv_gather: unknown cache type");
     const size_t total = (size_t)n * n_kv_heads * head_dim;
     hipLaunchKernelGGL(k_kv_gather, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, st, n_kv_heads,
                        head_dim, is_v ? 1 : 0, cells, n, out, 0);
@@ -2064,15 +2195,16 @@ void kv_gather(hipStream_t s, const __half * pool, KvStrides st, int n_kv_heads,
 }
 
 void kv_scatter(hipStream_t s, __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
-                const int32_t * cells, int n, const __half * in, bool q8) {
+                const int32_t * cells, int n, const __half * in, int kvq) {
     if (n <= 0) return;
-    if (q8) {
-        const size_t total = (size_t)n * kv_row_halves(n_kv_heads, head_dim, true);
-        hipLaunchKernelGGL(k_kv_gather_q8, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, st, n_kv_heads,
-                           head_dim, is_v ? 1 : 0, cells, n, (uint16_t *)const_cast<__half *>(in), 1);
+    if (kvq == KV_Q8 || kvq == KV_Q4) {
+        const size_t total = (size_t)n * kv_row_halves(n_kv_heads, head_dim, kvq);
+        hipLaunchKernelGGL(kvq == KV_Q8 ? k_kv_gather_q8 : k_kv_gather_q4, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                           pool, st, n_kv_heads, head_dim, is_v ? 1 : 0, cells, n, (uint16_t *)const_cast<__half *>(in), 1);
         check_launch("kv_scatter");
         return;
     }
+    if (kvq != KV_F16) throw std::runtime_error("kv_scatter: unknown cache type");
     const size_t total = (size_t)n * n_kv_heads * head_dim;
     hipLaunchKernelGGL(k_kv_gather, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, pool, st, n_kv_heads,
                        head_dim, is_v ? 1 : 0, cells, n, const_cast<__half *>(in), 1);
@@ -2089,8 +2221,8 @@ __global__ void k_kv_copy_page(__half * k_pool, __half * v_pool, size_t head_hal
 }
 
 void kv_copy_page(hipStream_t s, __half * k_pool, __half * v_pool, KvStrides st, int n_kv_heads, int head_dim,
-                  int src_page, int dst_page, bool q8) {
-    const size_t head_halves = kv_block_halves(head_dim, q8);       // one head's share of a page (a multiple of 8)
+                  int src_page, int dst_page, int kvq) {
+    const size_t head_halves = kv_block_halves(head_dim, kvq);       // one head's share of a page (a multiple of 8)
     hipLaunchKernelGGL(k_kv_copy_page, dim3((unsigned)((head_halves / 8 + 255) / 256), n_kv_heads), dim3(256), 0, s,
                        k_pool, v_pool, head_halves, st, src_page, dst_page);
     check_launch("kv_copy_page");

@@ -274,8 +274,8 @@ struct AttnShape {
     float eps;
     // element strides of a KV pool between pages and between the kv heads of a page (see kv_strides)
     size_t page_stride = 0, head_stride = 0;
-    bool kv_q8 = false;        // the pools hold Q8_0 blocks (see kv_block_halves)
-    bool q_q8 = false;         // ... and the query rows are converted to Q8_0 too (ggml's CPU attention over such a cache)
+    int kv_quant = 0;          // 0: f16 pools; 8 / 4: the pools hold Q8_0 / Q4_0 blocks (see kv_block_halves)
+    bool q_q8 = false;         // over such blocks: the query rows are converted to Q8_0 too (ggml's CPU attention)
 };
 // A pool holds one block per page and kv head, PAGE positions of one head. f16: PAGE x head_dim halves in the
 // operand orders of the attention kernel. Q8_0 (blocks of 32 along the head's row, one f16 scale each, as the
@@ -285,20 +285,28 @@ struct AttnShape {
 //   V codes  [p = dim / 32][lane = g * 16 + d][16 B]: bytes 0-7 dim 32 p + d, bytes 8-15 dim 32 p + 16 + d, byte i of
 //            either the token 4 g + i (i < 4) or 16 + 4 g + (i - 4)
 //   scales   [j or p][g][8]: the scale of block j (p) of token 4 g + i (i < 4) or 16 + 4 g + (i - 4)
-// All strides and sizes are in halves (2 bytes), also for Q8_0.
-inline size_t kv_block_halves(int head_dim, bool q8) {
-    return q8 ? (size_t)(head_dim / 32) * 544 : (size_t)PAGE * head_dim;
+// Q4_0 (kv_dtype Q4_0: the same blocks with four-bit codes q, value d (q - 8)): the same arrangement with 8 bytes
+// per lane, i.e. two 32-bit words where Q8_0 has two groups of eight bytes; the code of index i among a word's eight
+// is the nibble at bits 4 p(i) with p(i) = i / 2 + 4 (i % 2), the order in which one mask and shift pair widens
+// them to f16 (kv_nibble). head_dim / 32 loads of 512 bytes of codes, then the scales as above; 9/32 of the f16 block.
+// All strides and sizes are in halves (2 bytes), also for the quantised pools.
+enum : int { KV_F16 = 0, KV_Q8 = 8, KV_Q4 = 4 };
+constexpr int kv_nibble(int i) { return (i >> 1) + 4 * (i & 1); }
+inline size_t kv_block_halves(int head_dim, int kvq) {
+    return kvq == KV_Q8 ? (size_t)(head_dim / 32) * 544 : kvq == KV_Q4 ? (size_t)(head_dim / 32) * 288 : (size_t)PAGE * head_dim;
 }
 // head_major: [kv head][page], else [page][kv head].
 struct KvStrides { size_t page, head; };
-inline KvStrides kv_strides(int n_pages, int n_kv_heads, int head_dim, bool head_major, bool q8 = false) {
-    const size_t unit = kv_block_halves(head_dim, q8);
+inline KvStrides kv_strides(int n_pages, int n_kv_heads, int head_dim, bool head_major, int kvq = KV_F16) {
+    const size_t unit = kv_block_halves(head_dim, kvq);
     return head_major ? KvStrides{unit, (size_t)n_pages * unit} : KvStrides{(size_t)n_kv_heads * unit, unit};
 }
 // Halves of one cell's K (or V) row over all kv heads in the natural order kv_gather writes: f16 values, or per
-// head head_dim code bytes (code + 128) followed by head_dim / 32 f16 scales.
-inline size_t kv_row_halves(int n_kv_heads, int head_dim, bool q8) {
-    return q8 ? (size_t)n_kv_heads * (head_dim / 2 + head_dim / 32) : (size_t)n_kv_heads * head_dim;
+// head the codes in element order (Q8_0: head_dim bytes, code + 128; Q4_0: head_dim / 2 bytes, element 2 k in the
+// low nibble of byte k) followed by head_dim / 32 f16 scales.
+inline size_t kv_row_halves(int n_kv_heads, int head_dim, int kvq) {
+    return kvq == KV_Q8 ? (size_t)n_kv_heads * (head_dim / 2 + head_dim / 32)
+         : kvq == KV_Q4 ? (size_t)n_kv_heads * (head_dim / 4 + head_dim / 32) : (size_t)n_kv_heads * head_dim;
 }
 // qkv f32 [T][QD + 2*KD] (+ optional per-head RMSNorm weights) -> q as an f16
 // hi/lo pair [T][QD] each (rotated, pre-scaled by log2(e)/sqrt(head_dim)) and
@@ -322,12 +330,12 @@ size_t attention_partial_floats(int n_items, int head_dim);
 // Gathers the K or V row of one (layer pool, cell) into natural order, and the
 // inverse; used by sequence snapshots and by tests.
 void kv_gather(hipStream_t s, const __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
-               const int32_t * cells, int n, __half * out, bool q8 = false);
+               const int32_t * cells, int n, __half * out, int kvq = KV_F16);
 void kv_scatter(hipStream_t s, __half * pool, KvStrides st, int n_kv_heads, int head_dim, bool is_v,
-                const int32_t * cells, int n, const __half * in, bool q8 = false);
+                const int32_t * cells, int n, const __half * in, int kvq = KV_F16);
 // Copies page src to page dst in one layer's pools.
 void kv_copy_page(hipStream_t s, __half * k_pool, __half * v_pool, KvStrides st, int n_kv_heads, int head_dim,
-                  int src_page, int dst_page, bool q8 = false);
+                  int src_page, int dst_page, int kvq = KV_F16);
 
 // ---- sampling -------------------------------------------------------------------
 struct SampleOut {          // one per output row, read back by the host

@@ -769,9 +769,11 @@ class Engine:
             _raise(s)
         return out.view(np.float16)
 
-    def debug_kv_q8(self, layer: int, slot: int, pos: int, want_v: bool, n_kv: int, head_dim: int) -> np.ndarray:
-        """The K or V row of a Q8_0 cache as the values it stands for (scale times code), f32, kv_dim of them."""
-        per_head = head_dim // 2 + head_dim // 32
+    def debug_kv_q8(self, layer: int, slot: int, pos: int, want_v: bool, n_kv: int, head_dim: int, bits: int = 8) -> np.ndarray:
+        """The K or V row of a Q8_0 (bits 8) or Q4_0 (bits 4) cache as the values it stands for (scale times code),
+        f32, kv_dim of them."""
+        code_units = head_dim // 2 if bits == 8 else head_dim // 4
+        per_head = code_units + head_dim // 32
         raw = np.empty(n_kv * per_head, np.uint16)
         s = self._lib.retro_engine_debug_kv(self._h, layer, slot, pos, 1 if want_v else 0,
                                             raw.ctypes.data_as(C.POINTER(C.c_uint16)))
@@ -780,8 +782,12 @@ class Engine:
         out = np.empty((n_kv, head_dim), np.float32)
         for h in range(n_kv):
             row = raw[h * per_head:(h + 1) * per_head]
-            codes = row[:head_dim // 2].view(np.uint8).astype(np.int32) - 128
-            scales = row[head_dim // 2:].view(np.float16).astype(np.float32)
+            packed = row[:code_units].view(np.uint8).astype(np.int32)
+            if bits == 8:
+                codes = packed - 128
+            else:               # element 2 k in the low nibble of byte k, a value is scale times (code - 8)
+                codes = np.stack([packed & 15, packed >> 4], axis=-1).reshape(-1) - 8
+            scales = row[code_units:].view(np.float16).astype(np.float32)
             out[h] = (codes.reshape(-1, 32) * scales[:, None]).reshape(-1)
         return out.reshape(-1)
 

@@ -9,6 +9,21 @@ from gguf_reader import Reader
 F32, F16, Q8_0, Q4_K, Q5_K, Q6_K, BF16, MXFP4 = 0, 1, 8, 12, 13, 14, 30, 39
 
 
+def q4_0_cache_rows(v):
+    """Rows as a Q4_0 KV cache holds them (ggml's quantize_row_q4_0_ref, in numpy's float32 arithmetic): per 32
+    values the first value m of largest magnitude, d = m / -8, codes min(15, trunc(x / d + 8.5)) with the unrounded
+    d, values (code - 8) times d rounded to f16."""
+    x = np.asarray(v, np.float32)
+    f32 = np.float32
+    b = x.reshape(-1, 32)
+    first = np.abs(b).argmax(-1)
+    d = (b[np.arange(len(b)), first] / f32(-8.0)).astype(f32)
+    inv = np.where(d != 0, f32(1.0) / np.where(d != 0, d, f32(1.0)), f32(0.0)).astype(f32)
+    codes = np.minimum(np.trunc((b * inv[:, None]).astype(f32) + f32(8.5)), 15)
+    out = d.astype(np.float16).astype(f32)[:, None] * (codes - 8).astype(f32)
+    return out.reshape(x.shape).astype(np.float64)
+
+
 def ggml_activations(v, weight_type):
     """The rows of v as ggml's CPU matmul multiplies them with a weight of this
     type: re-quantised to Q8_K (Q4_K and Q6_K weights; blocks of 256, the first value of
@@ -131,11 +146,14 @@ class NumpyModel:
                 k = self.norm(k, self.t(b + "attn_k_norm.weight"))
             q = np.stack([self.rope(q[t], pos0 + t) for t in range(T)])
             k = np.stack([self.rope(k[t], pos0 + t) for t in range(T)])
-            if self.kv == "q8_0":
+            if self.kv in ("q8_0", "q4_0"):
                 # blocks of 32 never straddle heads (head_dim is a multiple of 32); under the ggml arithmetic the
-                # query row meets a Q8_0 K row converted to Q8_0 itself
-                k = ggml_activations(k.astype(np.float32), Q8_0)
-                v = ggml_activations(v.astype(np.float32), Q8_0)
+                # query row meets a Q8_0 or Q4_0 K row converted to Q8_0 itself
+                if self.kv == "q4_0":
+                    k, v = q4_0_cache_rows(k), q4_0_cache_rows(v)
+                else:
+                    k = ggml_activations(k.astype(np.float32), Q8_0)
+                    v = ggml_activations(v.astype(np.float32), Q8_0)
                 if self.ggml:
                     q = ggml_activations(q.astype(np.float32), Q8_0)
             else:

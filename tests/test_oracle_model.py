@@ -242,3 +242,34 @@ def test_lora_delta_reproduces_hugging_face_logits_with_the_adapter_merged(tmp_p
     # the adapter factors are stored as f16 and multiplied in f32: a little looser than the dense comparison
     assert np.abs(got - want).max() <= 2e-4 * np.abs(want).max(), np.abs(got - want).max()
     assert np.abs(want - base).mean() > 0.1
+
+
+@pytest.mark.parametrize("activations", ["exact", "ggml"])
+def test_a_q4_0_cache_holds_four_bit_blocks_and_attention_reads_them(models, activations):
+    """kv="q4_0": K and V rows are stored as quantize_row_q4_0_ref blocks (32 values along a head's row; d = m / -8
+    for the value m of largest magnitude, so m itself is stored exactly as code 0; the other codes 0..15) and
+    attention reads d (code - 8). What is stored lies on that grid, and the logits follow the float64 numpy
+    transformer with its own numpy quantiser. Against the reference's ggml build: parity unpinned."""
+    m = oracle.Model(models["qwen2-q8"])
+    rng = np.random.default_rng(13)
+    toks = rng.integers(0, m.n_vocab, 40)
+    c = oracle.Context(m, 1, activations=activations, kv="q4_0")
+    got = c.step_rows([(0, 0, toks, True)])[0]
+    f16c = oracle.Context(m, 1, activations=activations)
+    f16 = f16c.step_rows([(0, 0, toks, True)])[0]
+    for layer, pos, want_v in ((0, 0, False), (0, 39, True), (1, 17, False), (1, 33, True)):
+        row = c.read_kv_values(layer, 0, pos, want_v).reshape(-1, 32)
+        peak = row[np.arange(len(row)), np.abs(row).argmax(-1)]
+        d = (peak / np.float32(-8.0)).astype(np.float32)
+        codes = row / d[:, None] + 8
+        assert np.array_equal(codes, np.rint(codes)) and codes.min() == 0 and codes.max() <= 15
+        assert (codes.min(axis=1) == 0).all()
+        if layer == 0:           # the first layer's rows come from the same inputs as the f16 cache's: within half a step of them
+            plain = f16c.read_kv_values(layer, 0, pos, want_v).reshape(-1, 32)
+            assert (np.abs(row - plain) <= 0.5001 * np.abs(d)[:, None] + 1e-3 * np.abs(plain)).all() or \
+                   (np.abs(row - plain) <= 1.0001 * np.abs(d)[:, None]).all()
+    nm = NumpyModel(models["qwen2-q8"], activations=activations, kv="q4_0")
+    want = nm.forward(toks)[-1]
+    # a code on a rounding boundary may fall either way between the two (f32 against float64 rows), and a four-bit step is coarse
+    assert np.abs(got - want).max() < 2e-2 * max(1.0, np.abs(want).max())
+    assert np.abs(f16 - got).max() > 5 * np.abs(got - want).max(), "the cache type moves the logits far more than the two disagree"

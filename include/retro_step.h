@@ -274,6 +274,10 @@ int retro_engine_kv_unified(retro_engine * engine, bool * out_unified);
 int retro_engine_weights_version(retro_engine * engine, uint64_t * out_version);
 int retro_engine_model_fingerprint(retro_engine * engine, uint64_t * out_fingerprint);
 int retro_engine_is_hybrid(retro_engine * engine, bool * out_is_hybrid);
+/* ref h:2890-2899: the text of one token (what detokenize appends for it); `special` renders a control token as its
+ * text instead of nothing. Two calls: with no buffer the byte count is reported, a buffer that is too small returns -2. */
+int retro_engine_token_piece(retro_engine * engine, int32_t token, bool special, char * buffer, size_t n_buffer, size_t * out_n_bytes);
+
 /* ref h:2538-2549, 2879-2889 (retro_engine.cpp:331-378, 594-622): text -> token ids. tokenize_text adds the model's
  * BOS / EOS and reads the text of a special token as that token; tokenize_fragment adds nothing; tokenize takes both
  * flags. Two calls: with tokens == NULL or n_tokens_max == 0 the count is reported; a buffer that is too small returns

@@ -484,6 +484,24 @@ int retro_engine_detokenize(retro_engine * engine, const int32_t * tokens, size_
     });
 }
 
+int retro_engine_token_piece(retro_engine * engine, int32_t token, bool special, char * buffer, size_t n_buffer, size_t * out_n_bytes) {
+    return boundary([&]() -> int {
+        Engine * e = checked(engine);
+        if (!e) return -1;
+        if (!out_n_bytes) {
+            set_error("out_n_bytes is required");
+            return -1;
+        }
+        if (token < 0 || token >= e->hparams().n_vocab) {
+            set_error("token is outside the vocabulary");
+            return -1;
+        }
+        std::string text;
+        e->vocab().append_text(token, special, text);
+        return string_out(text, buffer, n_buffer, out_n_bytes);
+    });
+}
+
 int retro_engine_graphs_reused(retro_engine * engine, uint64_t * out_n_reused) {
     return boundary([&]() -> int {
         Engine * e = checked(engine);

@@ -124,7 +124,7 @@ STEP_SYMBOLS = [
     "retro_engine_kv_unified", "retro_engine_weights_version", "retro_engine_model_fingerprint",
     "retro_engine_is_hybrid", "retro_engine_eos_token", "retro_engine_vocab_size", "retro_engine_is_eog_token",
     "retro_engine_context_size", "retro_engine_detokenize", "retro_engine_graphs_reused",
-    "retro_engine_tokenize_text", "retro_engine_tokenize_fragment", "retro_engine_tokenize",
+    "retro_engine_tokenize_text", "retro_engine_tokenize_fragment", "retro_engine_tokenize", "retro_engine_token_piece",
     "retro_engine_load_lora", "retro_engine_set_lora_enabled",
     "retro_engine_load_lora_named", "retro_engine_activate_lora", "retro_engine_active_adapter",
     "retro_engine_adapter_load", "retro_engine_adapter_unload", "retro_engine_adapter_rows_info",
@@ -186,6 +186,7 @@ def load_library() -> C.CDLL:
     lib.retro_engine_tokenize.argtypes = [C.c_void_p, C.c_char_p, C.c_bool, C.c_bool, _i32p, C.c_size_t, C.POINTER(C.c_size_t)]
     lib.retro_engine_tokenize_text.argtypes = [C.c_void_p, C.c_char_p, _i32p, C.c_size_t, C.POINTER(C.c_size_t)]
     lib.retro_engine_tokenize_fragment.argtypes = [C.c_void_p, C.c_char_p, _i32p, C.c_size_t, C.POINTER(C.c_size_t)]
+    lib.retro_engine_token_piece.argtypes = [C.c_void_p, C.c_int32, C.c_bool, C.c_char_p, C.c_size_t, C.POINTER(C.c_size_t)]
     lib.retro_engine_detokenize.argtypes = [C.c_void_p, _i32p, C.c_size_t, C.c_bool, C.c_char_p, C.c_size_t,
                                             C.POINTER(C.c_size_t)]
     lib.retro_engine_graphs_reused.argtypes = [C.c_void_p, C.POINTER(C.c_uint64)]
@@ -679,6 +680,17 @@ class Engine:
         if s != 0:
             _raise(s)
         return [int(t) for t in out[:n.value]]
+
+    def token_piece(self, token: int, special: bool = False) -> bytes:
+        n = C.c_size_t()
+        s = self._lib.retro_engine_token_piece(self._h, token, special, None, 0, C.byref(n))
+        if s != 0:
+            _raise(s)
+        buf = C.create_string_buffer(n.value + 1)
+        s = self._lib.retro_engine_token_piece(self._h, token, special, buf, n.value + 1, C.byref(n))
+        if s != 0:
+            _raise(s)
+        return buf.raw[:n.value]
 
     def detokenize_bytes(self, tokens: Sequence[int], unparse_special: bool = False) -> bytes:
         toks = np.ascontiguousarray(tokens, dtype=np.int32)

@@ -455,6 +455,10 @@ def test_tokenization_of_a_byte_pair_vocabulary_reproduces_the_tokenizers_librar
         assert eng.detokenize_bytes(c["ids"], unparse_special=True).decode() == c["text"], c["text"]
     hello = next(c["ids"] for c in kind["cases"] if c["text"] == "Hello world")
     assert eng.tokenize("Hello world") == ([0] if pre == "llama-bpe" else []) + hello
+    assert b"".join(eng.token_piece(t) for t in hello) == b"Hello world"
+    assert eng.token_piece(0) == b"" and eng.token_piece(0, special=True) == b"<|begin_of_text|>"
+    with pytest.raises(E.EngineError, match="outside the vocabulary"):
+        eng.token_piece(len(kind["tokens"]))
     out = E.StepOutput()
     eng.step([E.StepRow(0, 0, eng.tokenize("attention is all you need"), 0, sample=True, sampling=greedy())], out)
     assert 0 <= out.row(0).token < len(kind["tokens"])

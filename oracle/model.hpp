@@ -267,12 +267,16 @@ inline const float * f32_data(const gguf_tensor & t) {
 
 // Rotates one head in place; angle = pos * base^(-2i/d) / factor_i evaluated in double. The factors are the
 // model's rope_freqs.weight (ggml's rope divides theta by them: ggml_rope_cache_init, theta / ff) times the linear
-// scaling factor, null for none.
-inline void rope(float * v, int head_dim, int rope_dim, int pos, double base, bool neox, const double * factors = nullptr) {
+// scaling factor, null for none; under yarn scaling (ggml's rope_yarn: theta = theta_interp (1 - mix) + theta_extrap mix
+// with mix = the ramp 1 - clamp((i - low) / (high - low), 0, 1) over the pair index between the correction
+// dimensions of beta_fast = 32 and beta_slow = 1 rotations within the original context) the divisor is
+// 1 / ((1 - mix) / factor + mix) and cosine and sine are multiplied by `magnitude` = attn_factor (1 + 0.1 ln factor).
+inline void rope(float * v, int head_dim, int rope_dim, int pos, double base, bool neox, const double * factors = nullptr,
+                 double magnitude = 1.0) {
     const int half = rope_dim / 2;
     for (int i = 0; i < half; ++i) {
         const double angle = (double)pos * std::pow(base, -2.0 * i / rope_dim) / (factors ? factors[i] : 1.0);
-        const double c = std::cos(angle), s = std::sin(angle);
+        const double c = std::cos(angle) * magnitude, s = std::sin(angle) * magnitude;
         const int i0 = neox ? i : 2 * i;
         const int i1 = neox ? i + half : 2 * i + 1;
         const double a = v[i0], b = v[i1];
@@ -378,19 +382,34 @@ struct context {
         const size_t kd = (size_t)KD;
         // per-frequency divisors of the rotation angle: rope_freqs.weight and linear scaling (see rope())
         std::vector<double> rope_div;
+        double rope_magnitude = 1.0;
         {
             const std::string p = h.arch + ".rope.scaling.type";
             const std::string scaling = g.has(p) ? g.s(p) : std::string("none");
             double lin = 1.0;
             if (scaling == "linear") lin = g.f_or(h.arch + ".rope.scaling.factor", 1.0);
-            else if (scaling != "none" && !scaling.empty()) throw std::runtime_error("oracle: rope scaling type " + scaling + " is not modelled");
+            else if (scaling != "none" && !scaling.empty() && scaling != "yarn") throw std::runtime_error("oracle: rope scaling type " + scaling + " is not modelled");
             const gguf_tensor * rf = g.find("rope_freqs.weight");
-            if (rf || lin != 1.0) {
+            if (rf || lin != 1.0 || scaling == "yarn") {
                 rope_div.assign((size_t)(h.rope_dim / 2), lin);
                 if (rf) {
                     if (rf->type != T_F32 || (int)rf->ne[0] != h.rope_dim / 2) throw std::runtime_error("oracle: rope_freqs.weight has an unexpected shape");
                     for (size_t i = 0; i < rope_div.size(); ++i) rope_div[i] *= (double)f32_data(*rf)[i];
                 }
+            }
+            if (scaling == "yarn") {
+                const double factor = g.f_or(h.arch + ".rope.scaling.factor", 1.0);
+                const double n_orig = (double)g.u_or(h.arch + ".rope.scaling.original_context_length", 0);
+                if (!(factor > 0.0) || !(n_orig > 0.0)) throw std::runtime_error("oracle: yarn scaling needs a factor and the original context length");
+                const double n_dims = (double)h.rope_dim;
+                auto corr_dim = [&](double n_rot) { return n_dims * std::log(n_orig / (n_rot * 2.0 * M_PI)) / (2.0 * std::log(h.rope_base)); };
+                const double low = std::max(0.0, std::floor(corr_dim(g.f_or(h.arch + ".rope.scaling.yarn_beta_fast", 32.0))));
+                const double high = std::min(n_dims - 1.0, std::ceil(corr_dim(g.f_or(h.arch + ".rope.scaling.yarn_beta_slow", 1.0))));
+                for (size_t i = 0; i < rope_div.size(); ++i) {
+                    const double mix = 1.0 - std::min(1.0, std::max(0.0, ((double)i - low) / std::max(0.001, high - low)));
+                    rope_div[i] /= (1.0 - mix) / factor + mix;
+                }
+                rope_magnitude = g.f_or(h.arch + ".rope.scaling.attn_factor", 1.0) * (1.0 + 0.1 * std::log(factor));
             }
         }
         const double * rope_factors = rope_div.empty() ? nullptr : rope_div.data();
@@ -437,13 +456,13 @@ struct context {
                 for (int hh = 0; hh < NH; ++hh) {
                     float * qh = &q[(size_t)t * QD + (size_t)hh * HD];
                     if (qn) rmsnorm(qh, f32_data(*qn), HD, h.eps, qh);
-                    rope(qh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox, rope_factors);
+                    rope(qh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox, rope_factors, rope_magnitude);
                 }
                 slot_state & s = slots[(size_t)slot[t]];
                 for (int hh = 0; hh < NKV; ++hh) {
                     float * kh = &k[(size_t)t * KD + (size_t)hh * HD];
                     if (kn) rmsnorm(kh, f32_data(*kn), HD, h.eps, kh);
-                    rope(kh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox, rope_factors);
+                    rope(kh, HD, h.rope_dim, pos[t], h.rope_base, h.rope_neox, rope_factors, rope_magnitude);
                 }
                 float * kc = &s.k[(size_t)l][(size_t)pos[t] * kd];
                 float * vc = &s.v[(size_t)l][(size_t)pos[t] * kd];

@@ -327,20 +327,17 @@ void Engine::load_model(const std::string & path) {
 
     // rotary frequencies in double: angle = pos * base^(-2i/d), divided by the model's per-frequency factors
     // (rope_freqs.weight, the long-context rule of Llama 3.1 and later: ggml's rope divides theta by them) and
-    // multiplied by 1 / factor under linear scaling. Other scaling rules (yarn, longrope) are not implemented:
-    // a model that declares one is refused rather than rotated wrongly.
+    // multiplied by 1 / factor under linear scaling. Under yarn scaling (ggml's rope_yarn) the frequencies below the
+    // correction range are interpolated (1 / factor), those above it kept, those inside mixed along a linear ramp
+    // over the pair index, and cosines and sines are multiplied by attn_factor (1 + 0.1 ln factor). Another rule
+    // (longrope) is not implemented: a model that declares one is refused rather than rotated wrongly.
     std::vector<double> inv((size_t)(h.rope_dim / 2));
     for (size_t i = 0; i < inv.size(); ++i) inv[i] = std::pow(h.rope_base, -2.0 * (double)i / h.rope_dim);
+    double magnitude = 1.0;
     {
         const std::string scaling = g.get_string(a + "rope.scaling.type", "none");
-        if (scaling == "linear") {
-            const double factor = g.get_float(a + "rope.scaling.factor", 1.0);
-            if (!(factor > 0.0)) throw std::runtime_error("rope.scaling.factor must be positive");
-            for (double & f : inv) f /= factor;
-        } else if (scaling != "none" && !scaling.empty()) {
-            throw std::runtime_error("rope scaling type '" + scaling + "' is not implemented");
-        }
-        if (const TensorInfo * rf = g.find("rope_freqs.weight")) {
+        const TensorInfo * rf = g.find("rope_freqs.weight");
+        if (rf) {
             if (rf->type != rk::WT_F32 || rf->ne[0] != (int64_t)inv.size() || rf->nbytes != inv.size() * sizeof(float))
                 throw std::runtime_error("rope_freqs.weight must hold rope_dim / 2 f32 factors");
             const float * ff = (const float *)rf->data;
@@ -349,7 +346,32 @@ void Engine::load_model(const std::string & path) {
                 inv[i] /= (double)ff[i];
             }
         }
+        if (scaling == "linear" || scaling == "yarn") {
+            const double factor = g.get_float(a + "rope.scaling.factor", 1.0);
+            if (!(factor > 0.0)) throw std::runtime_error("rope.scaling.factor must be positive");
+            if (scaling == "linear") {
+                for (double & f : inv) f /= factor;
+            } else {
+                const double n_orig = (double)g.get_int(a + "rope.scaling.original_context_length", 0);
+                if (!(n_orig > 0.0)) throw std::runtime_error("yarn scaling needs rope.scaling.original_context_length");
+                const double beta_fast = g.get_float(a + "rope.scaling.yarn_beta_fast", 32.0);
+                const double beta_slow = g.get_float(a + "rope.scaling.yarn_beta_slow", 1.0);
+                const double n_dims = (double)h.rope_dim;
+                auto corr = [&](double n_rot) { return n_dims * std::log(n_orig / (n_rot * 2.0 * M_PI)) / (2.0 * std::log(h.rope_base)); };
+                const double low = std::max(0.0, std::floor(corr(beta_fast)));
+                const double high = std::min(n_dims - 1.0, std::ceil(corr(beta_slow)));
+                for (size_t i = 0; i < inv.size(); ++i) {
+                    const double y = ((double)i - low) / std::max(0.001, high - low);
+                    const double keep = 1.0 - std::min(1.0, std::max(0.0, y));      // 1: the frequency as it is, 0: interpolated
+                    inv[i] *= (1.0 - keep) / factor + keep;
+                }
+                magnitude = g.get_float(a + "rope.scaling.attn_factor", 1.0) * (1.0 + 0.1 * std::log(factor));
+            }
+        } else if (scaling != "none" && !scaling.empty()) {
+            throw std::runtime_error("rope scaling type '" + scaling + "' is not implemented");
+        }
     }
+    inv.push_back(magnitude);
     inv_freq_.alloc(inv.size() * sizeof(double));
     hip_check(hipMemcpy(inv_freq_.ptr, inv.data(), inv.size() * sizeof(double), hipMemcpyHostToDevice), "hipMemcpy");
 

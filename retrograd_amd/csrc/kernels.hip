@@ -1284,7 +1284,9 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
         o.counts[2] = carry[0];
         o.counts[3] = carry[1];
     }
-    // rotary table of the step: angle = pos * base^(-2i/d) in double
+    // rotary table of the step: angle = pos * inv_freq[j] in double; inv_freq[pairs] is the magnitude factor of the
+    // rotation (1 unless the model's frequency scaling rule asks for another)
+    const double magnitude = inv_freq[pairs];
     const RowDesc lastd = rows[n_rows - 1];
     const int T = lastd.tok_off + lastd.n;
     for (int i = threadIdx.x; i < T * pairs; i += 1024) {
@@ -1298,8 +1300,8 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
         const double ang = (double)(rows[lo].pos0 + (t - rows[lo].tok_off)) * inv_freq[j];
         double sv, cv;
         sincos(ang, &sv, &cv);
-        o.rope_cos[i] = (float)cv;
-        o.rope_sin[i] = (float)sv;
+        o.rope_cos[i] = (float)(cv * magnitude);
+        o.rope_sin[i] = (float)(sv * magnitude);
     }
 }
 

@@ -254,7 +254,8 @@ struct PackBuffers {       // device arrays, sized for n_batch tokens / rows
     int split_pages = MAX_SPLIT_PAGES;   // pages per attention work item in this step (set from count_attention_work)
 };
 // Applies the block-table updates, then derives every per-token / per-tile
-// array of the step from the row descriptors. One workgroup.
+// array of the step from the row descriptors. One workgroup. inv_freq holds rope_pairs angles per position and
+// one more value, the factor on the rotation's cosines and sines (1 for a plain rotation).
 void pack_step(hipStream_t s, const RowDesc * rows, int n_rows, const int32_t * tokens_concat,
                const TableUpdate * updates, int n_updates, int32_t * table, int max_pages,
                int qt, int n_kv_heads, const double * inv_freq, int rope_pairs, const PackBuffers & out);

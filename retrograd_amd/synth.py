@@ -48,6 +48,8 @@ class ModelShape:
     rope_freqs: bool = False         # write rope_freqs.weight: per-frequency divisors of the rotation angle as
                                      # Llama 3.1's rule gives them (1 for short wavelengths, 8 for long, a ramp between)
     rope_scaling_linear: float = 0.0 # > 0: rope.scaling.type = linear with this factor
+    rope_scaling_yarn: float = 0.0   # > 0: rope.scaling.type = yarn with this factor ...
+    rope_original_context: int = 0   # ... over this original context length
     norm_std: float = 0.0            # > 0: norm vectors are 1 + norm_std * N(0, 1) instead of all ones, so that a test
                                      # can tell whether (and where) a norm weight is applied
     finer_layers: str = "all"        # layers whose ffn_down / attn_v take the finer type: "all", or "more_bits" =
@@ -322,6 +324,10 @@ def _common_metadata(w: gw.GGUFWriter, s: ModelShape, with_eos: bool, vocab: dic
     if s.rope_scaling_linear > 0:
         w.add(a + ".rope.scaling.type", gw.T_STRING, "linear")
         w.add(a + ".rope.scaling.factor", gw.T_FLOAT32, s.rope_scaling_linear)
+    if s.rope_scaling_yarn > 0:
+        w.add(a + ".rope.scaling.type", gw.T_STRING, "yarn")
+        w.add(a + ".rope.scaling.factor", gw.T_FLOAT32, s.rope_scaling_yarn)
+        w.add(a + ".rope.scaling.original_context_length", gw.T_UINT32, s.rope_original_context)
     if s.n_expert:
         w.add(a + ".expert_count", gw.T_UINT32, s.n_expert)
         w.add(a + ".expert_used_count", gw.T_UINT32, s.n_expert_used)

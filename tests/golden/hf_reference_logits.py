@@ -11,7 +11,7 @@ which pins the oracle's forward pass against a library that is not this reposito
   * grouped-query head mapping (query head h reads KV head h // (H / KV)), 1/sqrt(D) scaling, causal mask;
   * q/k/v biases (qwen2); per-head q/k RMSNorm before the rotation (qwen3moe); RMSNorm with its weight
     (norm vectors are random here, not all ones);
-  * rope_freqs.weight (Llama 3.1's frequency divisors = Hugging Face rope_type "llama3") and linear scaling;
+  * rope_freqs.weight (Llama 3.1's frequency divisors = Hugging Face rope_type "llama3"), linear and yarn scaling;
   * the expert router: softmax over all experts, top-k, renormalise (norm_topk_prob), SwiGLU experts;
   * the LoRA delta scale * alpha / r * B (A x): merged into the dense Hugging Face matrices.
 
@@ -47,6 +47,9 @@ CASES = {
     "llama-rope-freqs": (synth.scaled(synth.TINY_LLAMA, norm_std=0.2, rope_freqs=True, rope_base=500000.0,
                                       name="hf-llama-rope-freqs"), 42, 0.08),
     "llama-linear": (synth.scaled(synth.TINY_LLAMA, norm_std=0.2, rope_scaling_linear=4.0, name="hf-llama-linear"), 43, 0.08),
+    # yarn: with 32 rotary dims, base 1e4 and an original context of 32 the correction range is pairs 0..3
+    "llama-yarn": (synth.scaled(synth.TINY_LLAMA, norm_std=0.2, rope_scaling_yarn=4.0, rope_original_context=32,
+                                name="hf-llama-yarn"), 46, 0.08),
     "qwen2": (synth.scaled(synth.QWEN25_7B_Q8, n_layer=2, n_embd=128, n_head=4, n_head_kv=2, head_dim=32, n_ff=256,
                            n_vocab=300, norm_std=0.2, name="hf-qwen2"), 44, 0.08),
     "qwen3moe": (synth.scaled(synth.QWEN3_30B_A3B, n_layer=2, n_embd=256, n_head=4, n_head_kv=2, head_dim=64, n_vocab=288,
@@ -110,6 +113,9 @@ def build_hf(path, shape, lora=None):
                 "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}
     if s.rope_scaling_linear > 0:
         rope = {"rope_theta": float(s.rope_base), "rope_type": "linear", "factor": float(s.rope_scaling_linear)}
+    if s.rope_scaling_yarn > 0:
+        rope = {"rope_theta": float(s.rope_base), "rope_type": "yarn", "factor": float(s.rope_scaling_yarn),
+                "original_max_position_embeddings": int(s.rope_original_context), "beta_fast": 32.0, "beta_slow": 1.0}
     common = dict(vocab_size=s.n_vocab, hidden_size=s.n_embd, num_hidden_layers=s.n_layer, num_attention_heads=s.n_head,
                   num_key_value_heads=s.n_head_kv, rms_norm_eps=s.eps, max_position_embeddings=131072,
                   tie_word_embeddings=False, rope_parameters=rope, attn_implementation="eager", experts_implementation="eager")

@@ -84,10 +84,20 @@ class NumpyModel:
         self.w = {}
         # divisors of the rotation angle per frequency: linear scaling and the model's rope_freqs.weight
         scaling = g("rope.scaling.type", "none")
-        assert scaling in ("none", "linear"), scaling
+        assert scaling in ("none", "linear", "yarn"), scaling
         self.rope_div = np.full(self.D // 2, float(g("rope.scaling.factor", 1.0)) if scaling == "linear" else 1.0)
+        self.rope_magnitude = 1.0
         if "rope_freqs.weight" in r.tensors:
             self.rope_div = self.rope_div * np.asarray(self.t("rope_freqs.weight"), np.float64).reshape(-1)
+        if scaling == "yarn":
+            # the YaRN rule as its paper states it: below the correction range interpolate (1 / factor), above it keep,
+            # a linear ramp over the pair index between; amplitudes times 0.1 ln(factor) + 1
+            factor, n_orig = float(g("rope.scaling.factor")), float(g("rope.scaling.original_context_length"))
+            corr = lambda rot: self.D * np.log(n_orig / (rot * 2 * np.pi)) / (2 * np.log(self.base))
+            low, high = max(np.floor(corr(32.0)), 0), min(np.ceil(corr(1.0)), self.D - 1)
+            keep = 1 - np.clip((np.arange(self.D // 2) - low) / max(high - low, 0.001), 0, 1)
+            self.rope_div = self.rope_div / ((1 - keep) / factor + keep)
+            self.rope_magnitude = 0.1 * np.log(factor) + 1.0
 
     def t(self, name):
         if name not in self.w:
@@ -105,7 +115,7 @@ class NumpyModel:
         D = self.D
         i = np.arange(D // 2)
         ang = pos * self.base ** (-2.0 * i / D) / self.rope_div
-        c, s = np.cos(ang), np.sin(ang)
+        c, s = np.cos(ang) * self.rope_magnitude, np.sin(ang) * self.rope_magnitude
         out = v.copy()
         if self.neox:
             a, b = v[:, :D // 2], v[:, D // 2:]

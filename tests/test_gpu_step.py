@@ -44,6 +44,10 @@ SMALL = {
     "llama-rope-freqs": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
                                      n_ff=1024, n_vocab=1024, rope_freqs=True, rope_scaling_linear=2.0,
                                      name="llama-rope-freqs-small"),
+    # yarn scaling: interpolated, mixed and kept frequencies, cosines and sines times 1 + 0.1 ln(factor)
+    "llama-yarn": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
+                               n_ff=1024, n_vocab=1024, rope_base=10000.0, rope_scaling_yarn=4.0, rope_original_context=64,
+                               name="llama-yarn-small"),
 }
 
 

@@ -195,7 +195,7 @@ def _hf_golden():
     return mod, np.load(here / "hf_reference_logits.npz")
 
 
-@pytest.mark.parametrize("key", ["llama", "llama-rope-freqs", "llama-linear", "qwen2", "qwen3moe"])
+@pytest.mark.parametrize("key", ["llama", "llama-rope-freqs", "llama-linear", "llama-yarn", "qwen2", "qwen3moe"])
 def test_forward_reproduces_hugging_face_transformers_logits(tmp_path, key):
     """tests/golden/hf_reference_logits.npz holds logits of LlamaForCausalLM / Qwen2ForCausalLM /
     Qwen3MoeForCausalLM (float64, K and V rounded to f16 as the cache stores them) over the dequantised

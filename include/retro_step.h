@@ -230,6 +230,14 @@ typedef struct retro_generation_sequence {
     retro_sampling_params sampling;
 } retro_generation_sequence;
 
+/* ref h:1352-1362: a row of the v2 continuous generator - the prompt and the extended sampling parameters, an
+ * optional grammar handle among them, which constrains every token the row samples. */
+typedef struct retro_generation_sequence_v2 {
+    const int32_t * prompt_tokens;
+    size_t          n_prompt;
+    retro_sampling_params_v2 sampling;
+} retro_generation_sequence_v2;
+
 /* ref h:1123-1131: lifetime counters of the continuous generator's slot-level
  * prefix reuse; a caller attributes one call by differencing two snapshots. */
 typedef struct retro_generation_stats {

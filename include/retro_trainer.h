@@ -140,6 +140,12 @@ int retro_trainer_generate_batch(retro_trainer * trainer, const int32_t * prompt
 int retro_trainer_generate_continuous_batch(retro_trainer * trainer, const retro_generation_sequence * sequences,
                                             size_t n_sequences, int32_t * out_tokens, float * out_logprobs,
                                             size_t n_out_max, size_t * out_n_tokens, uint8_t * out_forced);
+/* :1880-1897: the same over v2 rows (extended sampling, an optional grammar per row); every token is sampled through
+ * the v2 chain with the row's own generator, history and grammar. out_logprobs holds the temperature-1 policy
+ * log-probability of each emitted token, as the v1 entry point's does. Only on the trainer handle, as in the reference. */
+int retro_trainer_generate_continuous_batch_v2(retro_trainer * trainer, const retro_generation_sequence_v2 * sequences,
+                                               size_t n_sequences, int32_t * out_tokens, float * out_logprobs,
+                                               size_t n_out_max, size_t * out_n_tokens, uint8_t * out_forced);
 int retro_trainer_generation_stats(retro_trainer * trainer, retro_generation_stats * out_stats);
 
 /* :1438-1453: per-row adapters of the generation context. A snapshot is a

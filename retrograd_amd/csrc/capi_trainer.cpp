@@ -230,6 +230,19 @@ int retro_trainer_generate_continuous_batch(retro_trainer * trainer, const retro
     TWIN(retro_engine_generate_continuous_batch(e, sequences, n_sequences, out_tokens, out_logprobs, n_out_max,
                                                 out_n_tokens, out_forced));
 }
+int retro_trainer_generate_continuous_batch_v2(retro_trainer * trainer, const retro_generation_sequence_v2 * sequences,
+                                               size_t n_sequences, int32_t * out_tokens, float * out_logprobs,
+                                               size_t n_out_max, size_t * out_n_tokens, uint8_t * out_forced) {
+    retro_engine * e = checked(trainer);
+    if (!e) return -1;
+    try {
+        clear_error();
+        return e->impl.generate_continuous_batch_v2(sequences, n_sequences, out_tokens, out_logprobs, n_out_max, out_n_tokens, out_forced);
+    } catch (const std::exception & ex) {
+        set_error(ex.what());
+        return -1;
+    }
+}
 int retro_trainer_generation_stats(retro_trainer * trainer, retro_generation_stats * out_stats) {
     TWIN(retro_engine_generation_stats(e, out_stats));
 }

@@ -827,7 +827,9 @@ bool valid_tokens(const int32_t * tokens, size_t n, int32_t n_vocab) {
     return true;
 }
 
-// Same checks, order and messages as the reference (retro_gen_core.cpp:1539-1589).
+}  // namespace
+
+// Same checks, order and messages as the reference (retro_gen_core.cpp:1539-1589). Also read by the v2 generator.
 bool valid_sampling_v2(const retro_sampling_params_v2 & s, int32_t n_vocab) {
     if (s.struct_size < sizeof(retro_sampling_params_v2)) {
         set_error("retro_sampling_params_v2.struct_size is too small for this build");
@@ -877,7 +879,6 @@ bool valid_sampling_v2(const retro_sampling_params_v2 & s, int32_t n_vocab) {
     return true;
 }
 
-}  // namespace
 
 int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, size_t n_rows,
                  retro_step_out_row_v2 * out2, retro_step_out_row * out1,

@@ -167,6 +167,9 @@ public:
     int generate_continuous_batch(const retro_generation_sequence * sequences, size_t n_sequences,
                                   int32_t * out_tokens, float * out_logprobs, size_t n_out_max,
                                   size_t * out_n_tokens, uint8_t * out_forced);
+    int generate_continuous_batch_v2(const retro_generation_sequence_v2 * sequences, size_t n_sequences,
+                                     int32_t * out_tokens, float * out_logprobs, size_t n_out_max,
+                                     size_t * out_n_tokens, uint8_t * out_forced);
     const retro_generation_stats & generation_stats() const { return gen_cache_.stats; }
     // A step or a raw sequence operation issued by a caller mutates the KV outside the
     // continuous generator's protocol: what its slots hold is forgotten (retro_gen_core.cpp:2569,
@@ -366,8 +369,17 @@ private:
     bool gen_validate_sampling(const retro_sampling_params & s);
     bool gen_validate_tokens(const int32_t * tokens, size_t n);
     bool gen_prefill(int32_t slot, const int32_t * tokens, size_t p0, size_t p1);
+    // how a generator's sequence samples: exactly one of the two is set
+    struct GenSampling { const retro_sampling_params * v1 = nullptr; const retro_sampling_params_v2 * v2 = nullptr; };
+    struct GenRow { size_t seq; int32_t slot; const int32_t * tokens; uint32_t n; int32_t pos0; bool sample; };
+    int gen_sample_rows(const std::vector<GenRow> & specs, const std::vector<GenSampling> & sampling,
+                        std::vector<retro_step_out_row> & outs);
+    int generate_continuous_impl(const retro_generation_sequence * sequences, const std::vector<GenSampling> & sampling,
+                                 const std::vector<uint32_t> & max_new, size_t n_sequences,
+                                 int32_t * out_tokens, float * out_logprobs, size_t n_out_max,
+                                 size_t * out_n_tokens, uint8_t * out_forced);
     int gen_decode_loop(const std::vector<size_t> & order, const std::vector<int32_t> & slot_of,
-                        const std::vector<size_t> & n_prompt_of, const std::vector<retro_sampling_params> & sampling,
+                        const std::vector<size_t> & n_prompt_of, const std::vector<GenSampling> & sampling,
                         const std::vector<size_t> & limits, std::vector<retro_step_out_row> produced,
                         int32_t * out_tokens, float * out_logprobs, size_t n_out_max, size_t * out_n_tokens,
                         uint8_t * out_forced);
@@ -375,6 +387,9 @@ private:
 };
 
 }  // namespace retro
+
+// The v2 sampling parameters' checks (engine.cpp), shared by the step and the v2 generator.
+namespace retro { bool valid_sampling_v2(const retro_sampling_params_v2 & s, int32_t n_vocab); }
 
 // The opaque handle of the C ABI.
 struct retro_engine {

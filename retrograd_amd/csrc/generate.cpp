@@ -128,11 +128,52 @@ bool Engine::gen_prefill(int32_t slot, const int32_t * tokens, size_t p0, size_t
     return true;
 }
 
+// One step of sampling rows for the generators' own requests, one token span per row. A row samples with the v1 or
+// the v2 parameters of its sequence (all rows of a call alike); what comes back is the part both versions share.
+int Engine::gen_sample_rows(const std::vector<GenRow> & specs, const std::vector<GenSampling> & sampling,
+                            std::vector<retro_step_out_row> & outs) {
+    outs.assign(specs.size(), retro_step_out_row{});
+    if (specs.empty()) return 0;
+    if (!sampling[specs[0].seq].v2) {
+        std::vector<retro_step_row> rows;
+        for (const GenRow & g : specs)
+            rows.push_back(v1_row(kGenRequestBase + (int32_t)g.seq, g.slot, g.tokens, g.n, g.pos0, g.sample, *sampling[g.seq].v1));
+        return step(nullptr, rows.data(), rows.size(), nullptr, outs.data(), nullptr, nullptr, 0);
+    }
+    std::vector<retro_step_row_v2> rows(specs.size());
+    std::vector<retro_step_out_row_v2> outs2(specs.size());
+    for (size_t i = 0; i < specs.size(); ++i) {
+        const GenRow & g = specs[i];
+        retro_step_row_v2 & row = rows[i];
+        row = retro_step_row_v2{};
+        row.struct_size = (uint32_t)sizeof(retro_step_row_v2);
+        row.request = kGenRequestBase + (int32_t)g.seq;
+        row.slot = g.slot;
+        row.tokens = g.tokens;
+        row.n = g.n;
+        row.pos0 = g.pos0;
+        row.sample = g.sample;
+        row.sampling = *sampling[g.seq].v2;
+        row.adapter = 0;     // the context adapter, as the batched generators decode
+        outs2[i].struct_size = (uint32_t)sizeof(retro_step_out_row_v2);
+    }
+    const int status = step(rows.data(), nullptr, rows.size(), outs2.data(), nullptr, nullptr, nullptr, 0);
+    if (status != 0) return status;
+    for (size_t i = 0; i < specs.size(); ++i) {
+        outs[i].struct_size = (uint32_t)sizeof(retro_step_out_row);
+        outs[i].token = outs2[i].token;
+        outs[i].logprob = outs2[i].logprob;      // the temperature-1 policy log-probability, as a v1 row reports it
+        outs[i].forced = outs2[i].forced;
+        outs[i].sampled = outs2[i].sampled;
+    }
+    return 0;
+}
+
 // The decode loop both generators share (retro_gen_core.cpp:1798-1875, 1982-2041):
 // `first` holds what the terminal prompt rows sampled; every pass records one
 // token per live row, in `order`, and decodes the rows that go on.
 int Engine::gen_decode_loop(const std::vector<size_t> & order, const std::vector<int32_t> & slot_of,
-                            const std::vector<size_t> & n_prompt_of, const std::vector<retro_sampling_params> & sampling,
+                            const std::vector<size_t> & n_prompt_of, const std::vector<GenSampling> & sampling,
                             const std::vector<size_t> & limits, std::vector<retro_step_out_row> produced,
                             int32_t * out_tokens, float * out_logprobs, size_t n_out_max, size_t * out_n_tokens,
                             uint8_t * out_forced) {
@@ -140,7 +181,7 @@ int Engine::gen_decode_loop(const std::vector<size_t> & order, const std::vector
     std::vector<bool> live(n, true);
     size_t n_live = n;
     std::vector<size_t> active;
-    std::vector<retro_step_row> rows;
+    std::vector<GenRow> rows;
     std::vector<retro_step_out_row> outs;
     while (n_live > 0) {
         active.clear();
@@ -163,13 +204,11 @@ int Engine::gen_decode_loop(const std::vector<size_t> & order, const std::vector
         }
         if (active.empty()) break;
         rows.clear();
-        outs.assign(active.size(), retro_step_out_row{});
         for (const size_t seq : active) {
             const size_t count = out_n_tokens[seq];
-            rows.push_back(v1_row(kGenRequestBase + (int32_t)seq, slot_of[seq], out_tokens + seq * n_out_max + count - 1, 1,
-                                  (int32_t)(n_prompt_of[seq] + count - 1), true, sampling[seq]));
+            rows.push_back({seq, slot_of[seq], out_tokens + seq * n_out_max + count - 1, 1, (int32_t)(n_prompt_of[seq] + count - 1), true});
         }
-        if (step(nullptr, rows.data(), rows.size(), nullptr, outs.data(), nullptr, nullptr, 0) != 0) return -1;
+        if (gen_sample_rows(rows, sampling, outs) != 0) return -1;
         for (size_t r = 0; r < active.size(); ++r) produced[active[r]] = outs[r];
     }
     return 0;
@@ -233,8 +272,9 @@ int Engine::generate_batch(const int32_t * prompt_tokens, size_t n_prompt, const
     std::vector<int32_t> slot_of(n_sequences);
     std::iota(slot_of.begin(), slot_of.end(), 0);
     std::vector<size_t> n_prompt_of(n_sequences, n_prompt), limits(n_sequences);
-    std::vector<retro_sampling_params> params(sampling, sampling + n_sequences);
+    std::vector<GenSampling> params(n_sequences);
     for (size_t i = 0; i < n_sequences; ++i) {
+        params[i].v1 = &sampling[i];
         limits[i] = std::min<size_t>(std::min<size_t>(n_out_max, sampling[i].max_new_tokens), n_ctx - n_prompt);
         out_n_tokens[i] = 0;
     }
@@ -265,6 +305,8 @@ int Engine::generate_continuous_batch(const retro_generation_sequence * sequence
         return -1;
     }
     const size_t n_ctx_seq = (size_t)n_ctx_seq_;
+    std::vector<GenSampling> sampling(n_sequences);
+    std::vector<uint32_t> max_new(n_sequences);
     for (size_t i = 0; i < n_sequences; ++i) {
         const retro_generation_sequence & item = sequences[i];
         clear_error();
@@ -274,7 +316,69 @@ int Engine::generate_continuous_batch(const retro_generation_sequence * sequence
             return -1;
         }
         out_n_tokens[i] = 0;
+        sampling[i].v1 = &item.sampling;
+        max_new[i] = item.sampling.max_new_tokens;
     }
+    return generate_continuous_impl(sequences, sampling, max_new, n_sequences, out_tokens, out_logprobs, n_out_max, out_n_tokens,
+                                    out_forced);
+}
+
+// The v2 rows of retro_trainer_generate_continuous_batch_v2 (reference retro_gen_core.cpp:2051-2254): the same
+// placement, prefill and bookkeeping over a view of the rows that holds their prompts only (so the canonical order and
+// the cell budget do not see the sampling parameters, as in the reference), every token sampled through the v2 chain
+// with the row's own generator, history and grammar.
+int Engine::generate_continuous_batch_v2(const retro_generation_sequence_v2 * sequences, size_t n_sequences,
+                                         int32_t * out_tokens, float * out_logprobs, size_t n_out_max,
+                                         size_t * out_n_tokens, uint8_t * out_forced) {
+    if (!sequences || n_sequences == 0 || !out_tokens || !out_n_tokens || n_out_max == 0) {
+        set_error("continuous v2 generation inputs and output buffers are required");
+        return -1;
+    }
+    if (n_sequences > cfg_.n_seq_max || n_sequences > cfg_.n_batch) {
+        set_error("continuous v2 generation batch exceeds the configured sequence or batch capacity");
+        return -1;
+    }
+    if (n_sequences > SIZE_MAX / n_out_max) {
+        set_error("continuous v2 generation output shape overflows size_t");
+        return -1;
+    }
+    const size_t n_ctx_seq = (size_t)n_ctx_seq_;
+    std::vector<retro_generation_sequence> view(n_sequences);
+    std::vector<GenSampling> sampling(n_sequences);
+    std::vector<uint32_t> max_new(n_sequences);
+    for (size_t i = 0; i < n_sequences; ++i) {
+        const retro_generation_sequence_v2 & item = sequences[i];
+        clear_error();
+        if (!item.prompt_tokens || item.n_prompt == 0 || item.n_prompt >= n_ctx_seq || !valid_sampling_v2(item.sampling, hp_.n_vocab)
+                || item.sampling.max_new_tokens == 0 || !gen_validate_tokens(item.prompt_tokens, item.n_prompt)) {
+            if (last_error().empty()) set_error("invalid continuous v2 generation prompt");
+            return -1;
+        }
+        if (item.sampling.grammar) {
+            try {
+                Grammar check(item.sampling.grammar->gbnf);
+            } catch (const std::exception & e) {
+                set_error(std::string("failed to compile the row's grammar (invalid GBNF): ") + e.what());
+                clear_generation_memory();
+                return -1;
+            }
+        }
+        out_n_tokens[i] = 0;
+        view[i] = retro_generation_sequence{};
+        view[i].prompt_tokens = item.prompt_tokens;
+        view[i].n_prompt = item.n_prompt;
+        sampling[i].v2 = &item.sampling;
+        max_new[i] = item.sampling.max_new_tokens;
+    }
+    return generate_continuous_impl(view.data(), sampling, max_new, n_sequences, out_tokens, out_logprobs, n_out_max, out_n_tokens,
+                                    out_forced);
+}
+
+int Engine::generate_continuous_impl(const retro_generation_sequence * sequences, const std::vector<GenSampling> & sampling,
+                                     const std::vector<uint32_t> & max_new, size_t n_sequences,
+                                     int32_t * out_tokens, float * out_logprobs, size_t n_out_max,
+                                     size_t * out_n_tokens, uint8_t * out_forced) {
+    const size_t n_ctx_seq = (size_t)n_ctx_seq_;
     const bool cache = prefix_cache_enabled();
     if (!cache) clear_generation_memory();
     gen_cache_.stats.calls++;
@@ -373,7 +477,7 @@ int Engine::generate_continuous_batch(const retro_generation_sequence * sequence
         const size_t members = group_end - group_start;
         const size_t terminal = item.n_prompt - 1;
         gen_cache_.stats.prefilled_tokens += (terminal - reuse) + members;
-        std::vector<retro_step_row> rows;
+        std::vector<GenRow> rows;
         std::vector<retro_step_out_row> outs;
         if (members > 1) {
             // the prefix has to be resident before it can be copied
@@ -385,10 +489,8 @@ int Engine::generate_continuous_batch(const retro_generation_sequence * sequence
                 const size_t stop = std::min(group_end, m + cfg_.n_batch);
                 rows.clear();
                 for (size_t k = m; k < stop; ++k)
-                    rows.push_back(v1_row(kGenRequestBase + (int32_t)order[k], slot_of[order[k]], item.prompt_tokens + terminal, 1,
-                                          (int32_t)terminal, true, sequences[order[k]].sampling));
-                outs.assign(rows.size(), retro_step_out_row{});
-                if (step(nullptr, rows.data(), rows.size(), nullptr, outs.data(), nullptr, nullptr, 0) != 0) return fail();
+                    rows.push_back({order[k], slot_of[order[k]], item.prompt_tokens + terminal, 1, (int32_t)terminal, true});
+                if (gen_sample_rows(rows, sampling, outs) != 0) return fail();
                 for (size_t k = m; k < stop; ++k) produced[order[k]] = outs[k - m];
             }
         } else {
@@ -399,11 +501,9 @@ int Engine::generate_continuous_batch(const retro_generation_sequence * sequence
             while (at < item.n_prompt) {
                 const size_t n = std::min(n_batch, item.n_prompt - at);
                 const bool last = at + n == item.n_prompt;
-                const retro_step_row row = v1_row(kGenRequestBase + (int32_t)leader, slot_of[leader], item.prompt_tokens + at,
-                                                  (uint32_t)n, (int32_t)at, last, item.sampling);
-                retro_step_out_row out {};
-                if (step(nullptr, &row, 1, nullptr, &out, nullptr, nullptr, 0) != 0) return fail();
-                if (last) produced[leader] = out;
+                rows.assign(1, GenRow{leader, slot_of[leader], item.prompt_tokens + at, (uint32_t)n, (int32_t)at, last});
+                if (gen_sample_rows(rows, sampling, outs) != 0) return fail();
+                if (last) produced[leader] = outs[0];
                 at += n;
             }
         }
@@ -412,14 +512,11 @@ int Engine::generate_continuous_batch(const retro_generation_sequence * sequence
 
     // ---- decode
     std::vector<size_t> n_prompt_of(n_sequences), limits(n_sequences);
-    std::vector<retro_sampling_params> params(n_sequences);
     for (size_t i = 0; i < n_sequences; ++i) {
         n_prompt_of[i] = sequences[i].n_prompt;
-        params[i] = sequences[i].sampling;
-        limits[i] = std::min<size_t>(std::min<size_t>(n_out_max, sequences[i].sampling.max_new_tokens),
-                                     n_ctx_seq - sequences[i].n_prompt);
+        limits[i] = std::min<size_t>(std::min<size_t>(n_out_max, max_new[i]), n_ctx_seq - sequences[i].n_prompt);
     }
-    if (gen_decode_loop(order, slot_of, n_prompt_of, params, limits, std::move(produced), out_tokens, out_logprobs, n_out_max,
+    if (gen_decode_loop(order, slot_of, n_prompt_of, sampling, limits, std::move(produced), out_tokens, out_logprobs, n_out_max,
                         out_n_tokens, out_forced) != 0)
         return fail();
 

@@ -58,6 +58,10 @@ class CGenerationSequence(C.Structure):
     _fields_ = [("prompt_tokens", C.POINTER(C.c_int32)), ("n_prompt", C.c_size_t), ("sampling", CSamplingParams)]
 
 
+class CGenerationSequenceV2(C.Structure):
+    pass      # fields set below, once CSamplingParamsV2 is known
+
+
 class CGenerationStats(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in ("calls", "sequences", "prompt_tokens", "prefilled_tokens", "reused_tokens",
                                           "hits", "evictions")]
@@ -82,6 +86,9 @@ class CSamplingParamsV2(C.Structure):
                 ("presence_penalty", C.c_float), ("penalty_window", C.c_uint32), ("n_logit_bias", C.c_uint32),
                 ("logit_bias_ids", C.POINTER(C.c_int32)), ("logit_bias_values", C.POINTER(C.c_float)),
                 ("grammar", C.c_void_p)]
+
+
+CGenerationSequenceV2._fields_ = [("prompt_tokens", C.POINTER(C.c_int32)), ("n_prompt", C.c_size_t), ("sampling", CSamplingParamsV2)]
 
 
 class CStepRowV2(C.Structure):
@@ -450,31 +457,7 @@ class Engine:
             f.request, f.slot = r.request, r.slot
             f.tokens = toks.ctypes.data_as(_i32p)
             f.n, f.pos0, f.sample = toks.size, r.pos0, r.sample
-            s = r.sampling
-            p = f.sampling
-            p.struct_size = C.sizeof(CSamplingParamsV2)
-            p.temperature, p.top_p, p.max_new_tokens, p.seed = s.temperature, s.top_p, s.max_new_tokens, s.seed & 0xFFFFFFFF
-            p.top_k, p.min_p, p.repeat_penalty = s.top_k, s.min_p, s.repeat_penalty
-            p.frequency_penalty, p.presence_penalty, p.penalty_window = s.frequency_penalty, s.presence_penalty, s.penalty_window
-            if s.logit_bias:
-                ids = np.array([b[0] for b in s.logit_bias], np.int32)
-                vals = np.array([b[1] for b in s.logit_bias], np.float32)
-                keep.extend((ids, vals))
-                p.n_logit_bias = ids.size
-                p.logit_bias_ids = ids.ctypes.data_as(_i32p)
-                p.logit_bias_values = vals.ctypes.data_as(_f32p)
-            else:
-                p.n_logit_bias = 0
-                p.logit_bias_ids = None
-                p.logit_bias_values = None
-            if s.grammar is not None:
-                g = self._lib.retro_grammar_from_gbnf(s.grammar.encode())
-                if not g:
-                    raise InvalidArgument(last_error())
-                keep.append(_GrammarHandle(self._lib, g))
-                p.grammar = g
-            else:
-                p.grammar = None
+            self._fill_sampling_v2(f.sampling, r.sampling, keep)
             f.n_top_logprobs, f.want_logprob, f.adapter = r.n_top_logprobs, 1 if r.want_logprob else 0, r.adapter.value
         top_ids = out.top_ids.ctypes.data_as(_i32p) if stride else None
         top_lps = out.top_logprobs.ctypes.data_as(_f32p) if stride else None
@@ -538,6 +521,32 @@ class Engine:
         if status != 0:
             _raise(status)
         return self._collect(n, n_out_max, toks, lps, list(counts), forced)
+
+    def _fill_sampling_v2(self, p, s, keep: list) -> None:
+        """Stages SamplingParamsV2 `s` into the FFI struct `p`; what `p` points at is appended to `keep`."""
+        p.struct_size = C.sizeof(CSamplingParamsV2)
+        p.temperature, p.top_p, p.max_new_tokens, p.seed = s.temperature, s.top_p, s.max_new_tokens, s.seed & 0xFFFFFFFF
+        p.top_k, p.min_p, p.repeat_penalty = s.top_k, s.min_p, s.repeat_penalty
+        p.frequency_penalty, p.presence_penalty, p.penalty_window = s.frequency_penalty, s.presence_penalty, s.penalty_window
+        if s.logit_bias:
+            ids = np.array([b[0] for b in s.logit_bias], np.int32)
+            vals = np.array([b[1] for b in s.logit_bias], np.float32)
+            keep.extend((ids, vals))
+            p.n_logit_bias = ids.size
+            p.logit_bias_ids = ids.ctypes.data_as(_i32p)
+            p.logit_bias_values = vals.ctypes.data_as(_f32p)
+        else:
+            p.n_logit_bias = 0
+            p.logit_bias_ids = None
+            p.logit_bias_values = None
+        if s.grammar is not None:
+            g = self._lib.retro_grammar_from_gbnf(s.grammar.encode())
+            if not g:
+                raise InvalidArgument(last_error())
+            keep.append(_GrammarHandle(self._lib, g))
+            p.grammar = g
+        else:
+            p.grammar = None
 
     def generate_continuous(self, sequences: Sequence[tuple], n_out_max: int | None = None):
         """retro_engine_generate_continuous_batch over (prompt, (temperature, top_p,

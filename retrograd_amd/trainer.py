@@ -65,7 +65,8 @@ TWINS = {
 }
 TRAINER_SYMBOLS = sorted(set(TWINS.values()) | {
     "retro_trainer_new", "retro_trainer_free", "retro_trainer_load_lora", "retro_trainer_generation_adapter_snapshot",
-    "retro_trainer_get_generation_adapter", "retro_trainer_set_generation_adapter"})
+    "retro_trainer_get_generation_adapter", "retro_trainer_set_generation_adapter",
+    "retro_trainer_generate_continuous_batch_v2"})
 
 _ready = False
 
@@ -82,6 +83,9 @@ def _library() -> C.CDLL:
         lib.retro_trainer_generation_adapter_snapshot.argtypes = [C.c_void_p, C.c_int32, C.c_float, _i32p]
         lib.retro_trainer_get_generation_adapter.argtypes = [C.c_void_p, _i32p]
         lib.retro_trainer_set_generation_adapter.argtypes = [C.c_void_p, C.c_int32]
+        lib.retro_trainer_generate_continuous_batch_v2.argtypes = [
+            C.c_void_p, C.POINTER(E.CGenerationSequenceV2), C.c_size_t, _i32p, C.POINTER(C.c_float), C.c_size_t,
+            C.POINTER(C.c_size_t), C.POINTER(C.c_uint8)]
         for engine_name, twin in TWINS.items():
             getattr(lib, twin).argtypes = getattr(lib, engine_name).argtypes
         _ready = True
@@ -143,6 +147,29 @@ class Trainer(E.Engine):
         s = self._lib.retro_trainer_load_lora(self._h, str(path).encode())
         if s != 0:
             E._raise(s)
+
+    def generate_continuous_v2(self, sequences, n_out_max: int | None = None):
+        """retro_trainer_generate_continuous_batch_v2 over (prompt, SamplingParamsV2) pairs (a grammar text among the
+        parameters constrains the row). Returns [(tokens, logprobs, forced)] in input order."""
+        import numpy as np
+        n = len(sequences)
+        n_out_max = n_out_max or max(p.max_new_tokens for _, p in sequences)
+        keep = [np.ascontiguousarray(prompt, dtype=np.int32) for prompt, _ in sequences]
+        ffi = (E.CGenerationSequenceV2 * n)()
+        for i, (_, p) in enumerate(sequences):
+            ffi[i].prompt_tokens = keep[i].ctypes.data_as(_i32p)
+            ffi[i].n_prompt = keep[i].size
+            self._fill_sampling_v2(ffi[i].sampling, p, keep)
+        toks = np.zeros((n, n_out_max), np.int32)
+        lps = np.zeros((n, n_out_max), np.float32)
+        forced = np.zeros((n, n_out_max), np.uint8)
+        counts = (C.c_size_t * n)()
+        status = self._lib.retro_trainer_generate_continuous_batch_v2(
+            self._h, ffi, n, toks.ctypes.data_as(_i32p), lps.ctypes.data_as(C.POINTER(C.c_float)), n_out_max, counts,
+            forced.ctypes.data_as(C.POINTER(C.c_uint8)))
+        if status != 0:
+            E._raise(status)
+        return self._collect(n, n_out_max, toks, lps, list(counts), forced)
 
     def generation_adapter_snapshot(self, replace: int = 0, scale: float = 1.0) -> int:
         out = C.c_int32()

@@ -177,3 +177,96 @@ def test_two_rows_of_one_step_keep_their_own_grammars(model_path):
     assert list(doc)[:2] == ["verdict", "score"] and doc["verdict"] in ("pass", "fail") and isinstance(doc["score"], int)
     assert all(isinstance(n, str) and len(n) <= 6 for n in doc.get("notes", [])) and len(doc.get("notes", [])) <= 2
     sched.close()
+
+
+# ---- the v2 continuous generator (retro_trainer_generate_continuous_batch_v2, reference retro_gen_core.cpp:2051-2254)
+
+def _trainer(path, n_seq=4):
+    from retrograd_amd import trainer as T
+    return T.Trainer(path, T.TrainConfig(n_ctx=96, n_batch=16, generation_concurrency=n_seq))
+
+
+def test_the_v2_generator_keeps_each_rows_grammar(model_path):
+    """tests/engine_contracts.rs:36-60 as written: `root ::= "yes"` and `root ::= "no"` in one call; every row's text
+    is its grammar's sentence, within its budget, nothing forced; a zero budget is an error."""
+    tr = _trainer(model_path)
+    prompt = tr.tokenize("Answer:")
+    params = lambda answer, n=8: E.SamplingParamsV2(temperature=1.0, top_p=1.0, max_new_tokens=n, seed=7, grammar='root ::= "%s"' % answer)
+    rows = tr.generate_continuous_v2([(prompt, params("yes")), (prompt, params("no"))])
+    for (tokens, logprobs, forced), expected in zip(rows, ("yes", "no")):
+        assert tr.detokenize_bytes(tokens).decode() == expected          # the closing end-of-generation token has no text
+        assert tokens[-1] == EOS and len(tokens) <= 8 and len(forced) == len(tokens) and not any(forced)
+        assert len(logprobs) == len(tokens) and all(lp <= 0 for lp in logprobs)
+    with pytest.raises(E.EngineError):
+        tr.generate_continuous_v2([(prompt, params("yes", 0))], n_out_max=4)
+    with pytest.raises(E.EngineError, match="invalid GBNF"):
+        tr.generate_continuous_v2([(prompt, E.SamplingParamsV2(max_new_tokens=4, grammar="root ::= missing"))])
+    assert tr.seq_pos(0) == (-1, -1) or tr.generation_stats()["calls"] >= 1
+    tr.close()
+
+
+def test_a_v2_step_loop_in_canonical_order_reproduces_the_v2_generator_bit_for_bit(model_path, monkeypatch):
+    """The relation the reference tests for the v1 generator (tests/engine_runtime.rs:676-724), for the v2 one: the
+    canonical order sees the prompts only (the rows' sampling parameters are not part of it), equal prompts are
+    decoded once and copied, every row draws from its own generator, history and grammar."""
+    monkeypatch.setenv("RETRO_GENERATION_PREFIX_CACHE", "0")
+    tr = _trainer(model_path)
+    a, b = tr.tokenize("attention is all"), tr.tokenize("the quick brown fox jumps")
+    sp = [E.SamplingParamsV2(temperature=0.9, top_p=0.95, top_k=40, max_new_tokens=7, seed=11, repeat_penalty=1.2, penalty_window=4),
+          E.SamplingParamsV2(temperature=1.0, top_p=1.0, top_k=0, max_new_tokens=6, seed=12, min_p=0.02, logit_bias=[(5, 1.5)]),
+          E.SamplingParamsV2(temperature=1.0, top_p=1.0, max_new_tokens=9, seed=13, grammar='root ::= [a-z ]+ "."', logit_bias=[(EOS, 2.0)]),
+          E.SamplingParamsV2(temperature=1.3, top_p=0.8, top_k=5, max_new_tokens=5, seed=14)]
+    wave = [(b, sp[0]), (a, sp[1]), (b, sp[2]), (a, sp[3])]
+    reference = tr.generate_continuous_v2(wave, 9)
+
+    order = sorted(range(len(wave)), key=lambda i: (len(wave[i][0]), list(wave[i][0]), i))
+    slot_of = {seq: slot for slot, seq in enumerate(order)}
+    for slot in range(len(order)):
+        tr.seq_rm(slot)
+    out = E.StepOutput()
+    nxt, tokens, lps = {}, {s: [] for s in order}, {s: [] for s in order}
+
+    def row(seq, toks, pos0, sample):
+        return E.StepRow(100 + seq, slot_of[seq], toks, pos0, sample=sample, sampling=wave[seq][1])
+    g = 0
+    while g < len(order):
+        leader = order[g]
+        prompt = list(wave[leader][0])
+        e = g + 1
+        while e < len(order) and list(wave[order[e]][0]) == prompt:
+            e += 1
+        members = order[g:e]
+        assert len(members) == 2
+        for at in range(0, len(prompt) - 1, 16):
+            tr.step([row(leader, prompt[at:min(at + 16, len(prompt) - 1)], at, False)], out)
+        for m in members[1:]:
+            tr.seq_cp(slot_of[leader], slot_of[m])
+        tr.step([row(m, [prompt[-1]], len(prompt) - 1, True) for m in members], out)
+        for i, m in enumerate(members):
+            nxt[m] = out.row(i)
+        g = e
+    live = set(order)
+    while live:
+        active = []
+        for s in order:
+            if s not in live:
+                continue
+            tokens[s].append(nxt[s].token)
+            lps[s].append(np.float32(nxt[s].logprob))
+            if nxt[s].token == EOS or len(tokens[s]) == wave[s][1].max_new_tokens:
+                live.discard(s)
+            else:
+                active.append(s)
+        if not active:
+            break
+        tr.step([row(s, [tokens[s][-1]], len(wave[s][0]) + len(tokens[s]) - 1, True) for s in active], out)
+        for i, s in enumerate(active):
+            nxt[s] = out.row(i)
+    for s in order:
+        tr.request_free(100 + s)
+    for s, (toks, logprobs, _) in enumerate(reference):
+        assert toks == tokens[s], (s, toks, tokens[s])
+        assert np.array_equal(np.asarray(logprobs, np.float32).view(np.uint32), np.array(lps[s], np.float32).view(np.uint32))
+    text = tr.detokenize_bytes([t for t in reference[2][0] if t != EOS]).decode()
+    assert regex.fullmatch(r"[a-z ]+\.?", text), text
+    tr.close()

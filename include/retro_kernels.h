@@ -22,6 +22,9 @@ extern "C" {
  * f16 hi/lo pairs) or, with bit 8 (0x100) of use_tiles set, x as ggml's CPU
  * matmul converts it for this weight type: Q8_K codes times their scale for
  * Q4_K, Q8_0 ones for Q8_0 and MXFP4, f16 / bf16 rounding for F16 / BF16.
+ * With bit 9 (0x200) as well (Q4_K tiles, at most two tokens) the conversion
+ * leaves the Q8_K blocks themselves and the integer matrix-vector kernel of very
+ * small steps multiplies the codes; anything else with that bit is refused.
  * y is [n_tokens][n_rows] and is read first when accumulate is set. */
 int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x,
                         int32_t n_tokens, int32_t use_tiles, const float * bias, int32_t accumulate, float * y);
@@ -63,7 +66,9 @@ int32_t retro_kernel_sample_greedy_noalloc_max_rows(void);
  * the last-level cache. debug and force_ksplit are timing experiments
  * (0 = normal). type is Q4_K, Q5_K, Q6_K or Q8_0 (Q5_K and Q6_K in modes 2 and
  * 3 only), n_rows a multiple of 16 and k of 256: anything else is refused
- * before a buffer is allocated. */
+ * before a buffer is allocated. Mode 4 times the integer matrix-vector kernel
+ * of very small steps under the ggml arithmetic instead (Q4_K, at most two
+ * tokens, pseudo-random Q8_K blocks). */
 int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,
                              int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us);
 

@@ -57,7 +57,9 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
         ok(hipMemset(d_sums.ptr, 0, d_sums.bytes), "clear block sums");
         // use_tiles bit 8: ggml's arithmetic - the rows are converted (quantised types) or rounded (F16 / BF16)
         // before the product; otherwise the f32 values are multiplied
-        const bool faithful = (use_tiles & 0x100) != 0;
+        // bit 9 (with bit 8, Q8_K conversions, at most GEMV_MAX_T = 2 tokens): the producer leaves the Q8_K blocks as
+        // well and the integer matrix-vector kernel multiplies them
+        const bool faithful = (use_tiles & 0x100) != 0, integer = (use_tiles & 0x200) != 0;
         use_tiles &= 0xff;
         rk::Act act;
         act.K = (int)k;
@@ -66,6 +68,16 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
             act.x = d_xh.as<__half>(); act.sums = k % 32 == 0 ? d_sums.as<__half>() : nullptr;
         } else {
             act.qx = d_xh.as<__half>(); act.qsums = d_sums.as<__half>(); act.quant = rk::act_quant_of(type);
+        }
+        DevBuf d_codes, d_scales, d_bsums;
+        if (integer) {
+            if (!faithful || act.quant != rk::AQ_Q8_K || n_tokens > rk::GEMV_MAX_T)
+                throw std::runtime_error("the integer kernel takes Q8_K conversions of at most " + std::to_string(rk::GEMV_MAX_T) + " tokens");
+            d_codes.alloc((size_t)n_tokens * k);
+            d_scales.alloc((size_t)n_tokens * (k / 256) * 4);
+            d_bsums.alloc((size_t)n_tokens * (k / 32) * 2);
+            act.qc = d_codes.as<int8_t>(); act.qd = d_scales.as<float>(); act.qbs = d_bsums.as<int16_t>();
+            if (!rk::gemv_can(w, act.operand(type), n_tokens)) throw std::runtime_error("the integer kernel does not take this matrix");
         }
         rk::to_act(nullptr, d_x.as<float>(), n_tokens, (int)k, act);
         d_y.alloc((size_t)n_tokens * n_rows * 4);
@@ -181,6 +193,24 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
         rk::Act act;
         act.K = (int)k;
         act.x = act.qx = d_xh.as<__half>(); act.sums = act.qsums = d_sums.as<__half>(); act.quant = rk::act_quant_of(type);
+        // mode 4: the integer matrix-vector kernel over pseudo-random Q8_K blocks (Q4_K, at most GEMV_MAX_T tokens)
+        DevBuf d_codes, d_scales, d_bsums;
+        if (mode == 4) {
+            if (type != rk::WT_Q4_K || n_tokens > rk::GEMV_MAX_T) throw std::runtime_error("matmul_time: the integer kernel takes Q4_K and at most " + std::to_string(rk::GEMV_MAX_T) + " tokens");
+            std::vector<uint8_t> codes((size_t)n_tokens * k);
+            uint32_t state = 0x85ebca6bu;
+            for (uint8_t & c : codes) { state = state * 1664525u + 1013904223u; c = (uint8_t)(state >> 24); }
+            std::vector<float> scales((size_t)n_tokens * (k / 256), 0.01f);
+            std::vector<int16_t> bsums((size_t)n_tokens * (k / 32));
+            for (int16_t & b : bsums) { state = state * 1664525u + 1013904223u; b = (int16_t)((int)(state >> 20) - 2048); }
+            d_codes.alloc(codes.size()); d_scales.alloc(scales.size() * 4); d_bsums.alloc(bsums.size() * 2);
+            ok(hipMemcpy(d_codes.ptr, codes.data(), d_codes.bytes, hipMemcpyHostToDevice), "fill");
+            ok(hipMemcpy(d_scales.ptr, scales.data(), d_scales.bytes, hipMemcpyHostToDevice), "fill");
+            ok(hipMemcpy(d_bsums.ptr, bsums.data(), d_bsums.bytes, hipMemcpyHostToDevice), "fill");
+            act.faithful = 1;
+            act.qc = d_codes.as<int8_t>(); act.qd = d_scales.as<float>(); act.qbs = d_bsums.as<int16_t>();
+            if (!rk::gemv_can(w, act.operand(type), n_tokens)) throw std::runtime_error("matmul_time: the integer kernel does not take this shape");
+        }
         rk::g_mm_debug = debug;
         rk::g_mm_force_ksplit = force_ksplit;
         hipEvent_t e0, e1;
@@ -190,7 +220,7 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
             w.packed = d_w.as<uint8_t>() + (turn++ % copies) * bytes;
             // mode 1: register-only tiles, 2: LDS-staged tiles, 3: the same with the K-slices left unreduced
             if (mode == 3) rk::matmul_deferred(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, d_ws.ptr);
-            else rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, mode == 2 ? d_ws.ptr : nullptr);
+            else rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, mode == 2 || mode == 4 ? d_ws.ptr : nullptr);
         };
         for (int i = 0; i < 3; ++i) run();
         ok(hipEventRecord(e0, nullptr), "record");

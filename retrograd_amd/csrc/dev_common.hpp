@@ -85,7 +85,9 @@ __device__ __forceinline__ Q4KScales q4k_scales(const u4 & hdr) {
 //         from zero), value = f16(d) * code.
 //   Q8_K: `max` = the first value of largest magnitude, iscale = -127 / max,
 //         code = min(127, rint(iscale * v)) (half to even), value = code / iscale.
-__device__ __forceinline__ void requantise8(float (&v)[8], int quant) {
+// With `codes` (Q8_K only) the integer codes are returned as well, and the block scale 1 / iscale is the
+// function's value (0 for a block of zeros).
+__device__ __forceinline__ float requantise8(float (&v)[8], int quant, float * codes = nullptr) {
     float amax = 0.0f, first = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -100,7 +102,7 @@ __device__ __forceinline__ void requantise8(float (&v)[8], int quant) {
         const float dh = (float)(_Float16)d;
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = __fmul_rn(dh, roundf(__fmul_rn(v[i], id)));
-        return;
+        return dh;
     }
     float gmax = amax;
 #pragma unroll
@@ -113,12 +115,42 @@ __device__ __forceinline__ void requantise8(float (&v)[8], int quant) {
     if (gmax == 0.0f) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = 0.0f;
-        return;
+        if (codes) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) codes[i] = 0.0f;
+        }
+        return 0.0f;
     }
     const float iscale = __fdiv_rn(-127.0f, max);
     const float d = __fdiv_rn(1.0f, iscale);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = __fmul_rn(d, fminf(127.0f, rintf(__fmul_rn(iscale, v[i]))));
+    for (int i = 0; i < 8; ++i) {
+        const float c = fminf(127.0f, rintf(__fmul_rn(iscale, v[i])));
+        if (codes) codes[i] = c;
+        v[i] = __fmul_rn(d, c);
+    }
+    return d;
+}
+
+// The Q8_K codes of eight consecutive values (k a multiple of 8) into the buffers of the integer
+// matrix-vector kernel (Act::qc, qd, qbs): 8 bytes in the order of act_code_pos, the sum of a 32-wide
+// block from its four lanes, the block scale from the lane that holds the block's first values.
+__device__ __forceinline__ void store_codes8(const float (&c)[8], float d, const Act & out, int tok, int k, int lane_in_block) {
+    uint32_t w0 = 0, w1 = 0;
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int q = (int)c[i];
+        sum += q;
+        const uint32_t byte = (uint32_t)q & 0xffu;
+        const int pos = act_code_pos(i);
+        if (pos < 4) w0 |= byte << (8 * pos); else w1 |= byte << (8 * (pos - 4));
+    }
+    *(uint2 *)(out.qc + (size_t)tok * out.K + k) = make_uint2(w0, w1);
+    sum += __shfl_xor(sum, 1, 64);
+    sum += __shfl_xor(sum, 2, 64);
+    if (lane_in_block == 0) out.qbs[(size_t)tok * (out.K >> 5) + (k >> 5)] = (int16_t)sum;
+    if ((k & 255) == 0) out.qd[(size_t)tok * (out.K >> 8) + (k >> 8)] = d;
 }
 
 // Eight consecutive values per lane (k a multiple of 8) into one pair of planes:
@@ -158,7 +190,13 @@ __device__ __forceinline__ void store_act8(const float (&v)[8], const Act & out,
         float q[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) q[i] = v[i];
-        requantise8(q, out.quant);
+        if (out.qc) {
+            float c[8];
+            const float d = requantise8(q, out.quant, c);
+            store_codes8(c, d, out, tok, k, lane_in_block);
+        } else {
+            requantise8(q, out.quant);
+        }
         store_act8_planes(q, out.qx, out.qsums, out.K, tok, k, lane_in_block);
     }
 }

@@ -77,6 +77,9 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
         // (Q8_K / Q8_0 codes, f16 / bf16 rounding); unset or "exact": the f32 values (as f16 hi/lo pairs).
         if (const char * dbg = std::getenv("RETRO_MM_DEBUG")) rk::g_mm_debug = std::atoi(dbg);     // timing experiments
         if (const char * dbg = std::getenv("RETRO_MM_SINGLE")) mm_single_mask_ = std::atoi(dbg);
+        // steps of at most this many tokens go through the integer matrix-vector kernel under the ggml arithmetic (0: never)
+        const char * g = std::getenv("RETRO_GEMV_MAX_T");
+        rk::g_gemv_max_t = g ? std::max(0, std::min(std::atoi(g), rk::GEMV_MAX_T)) : rk::GEMV_MAX_T;
         const char * v = std::getenv("RETRO_ACTIVATIONS");
         const std::string mode = v ? v : "exact";
         if (mode == "ggml") ggml_activations_ = true;
@@ -469,6 +472,16 @@ void Engine::build_buffers() {
         act(act_q_qx_, act_q_qsums_, QD);
         act(act_f_qx_, act_f_qsums_, F);
         act(act_o_qx_, act_o_qsums_, E);
+        auto codes = [&](ActCodes & c, int K) {
+            if (K % 256 != 0) return;          // no Q8_K conversion of such rows
+            c.codes.alloc((size_t)rk::GEMV_MAX_T * K);
+            c.d.alloc((size_t)rk::GEMV_MAX_T * (K / 256) * 4);
+            c.bsums.alloc((size_t)rk::GEMV_MAX_T * (K / 32) * 2);
+        };
+        codes(act_e_codes_, E);
+        codes(act_q_codes_, QD);
+        codes(act_f_codes_, F);
+        codes(act_o_codes_, E);
     }
     q_half_lo_.alloc((size_t)B * QD * 2);
     mm_ws_.alloc(rk::matmul_workspace_bytes());
@@ -1292,8 +1305,9 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
     // expert router and LoRA factors (`plain`); the converted row for the quantised weights.
     const bool faithful = ggml_activations_;
     const bool ffn_lora = routed && lora_has_ffn_ && h.n_expert == 0;      // some row may carry feed-forward deltas
-    auto act_for = [faithful](DevBuf & x, DevBuf & sums, DevBuf & qx, DevBuf & qsums, int K, std::initializer_list<int> types,
-                              bool plain) {
+    const bool small_step = T <= rk::g_gemv_max_t;      // the producers leave the Q8_K blocks for the integer kernel as well
+    auto act_for = [faithful, small_step](DevBuf & x, DevBuf & sums, DevBuf & qx, DevBuf & qsums, int K, std::initializer_list<int> types,
+                                          bool plain, ActCodes * codes = nullptr) {
         rk::Act a;
         a.K = K;
         a.faithful = faithful ? 1 : 0;
@@ -1311,6 +1325,9 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         }
         if (plain) { a.x = x.as<__half>(); a.sums = K % 32 == 0 ? sums.as<__half>() : nullptr; }
         if (a.quant != rk::AQ_NONE) { a.qx = qx.as<__half>(); a.qsums = qsums.as<__half>(); }
+        if (a.quant == rk::AQ_Q8_K && small_step && codes && codes->codes.ptr) {
+            a.qc = codes->codes.as<int8_t>(); a.qd = codes->d.as<float>(); a.qbs = codes->bsums.as<int16_t>();
+        }
         return a;
     };
     auto types_of = [](const std::vector<DevWeight> & ws) {
@@ -1319,7 +1336,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         for (size_t i = ws.size(); i < 3; ++i) t[i] = ws.empty() ? rk::WT_F32 : ws[0].w.type;
         return std::array<int, 3>{t[0], t[1], t[2]};
     };
-    const rk::Act act_o = act_for(act_o_x_, act_o_sums_, act_o_qx_, act_o_qsums_, E, {lm_head_.w.type}, false);
+    const rk::Act act_o = act_for(act_o_x_, act_o_sums_, act_o_qx_, act_o_qsums_, E, {lm_head_.w.type}, false, &act_o_codes_);
     partial_.ensure(rk::attention_partial_floats(n_items, h.head_dim) * 4);
     float * x = x_.as<float>();
     float * qkv = qkv_.as<float>();
@@ -1332,8 +1349,8 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
     for (int l = 0; l < h.n_layer; ++l) {
         const LayerWeights & L = layers_[(size_t)l];
         const std::array<int, 3> qt = types_of(L.qkv), gt = types_of(L.gate_up);
-        rk::Act act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {qt[0], qt[1], qt[2]}, routed);
-        const rk::Act act_q = act_for(act_q_x_, act_q_sums_, act_q_qx_, act_q_qsums_, QD, {L.wo.w.type}, routed);
+        rk::Act act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {qt[0], qt[1], qt[2]}, routed, &act_e_codes_);
+        const rk::Act act_q = act_for(act_q_x_, act_q_sums_, act_q_qx_, act_q_qsums_, QD, {L.wo.w.type}, routed, &act_q_codes_);
         { const size_t pt_ = prof_begin(PC_NORM); rk::rmsnorm_act(stream_, x, L.attn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending); prof_end(PC_NORM, pt_); }
         rk::Slices qkv_slices;
         {
@@ -1394,7 +1411,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         prof_end(PC_OPROJ, pt_);
         pt_ = prof_begin(PC_NORM);
         if (h.n_expert > 0) act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {L.router.w.type, L.gate_exps.w.type}, false);
-        else act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {gt[0], gt[1], gt[2]}, ffn_lora);
+        else act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {gt[0], gt[1], gt[2]}, ffn_lora, &act_e_codes_);
         rk::rmsnorm_act(stream_, x, L.ffn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending);
         prof_end(PC_NORM, pt_);
         if (h.n_expert > 0) {
@@ -1410,7 +1427,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
             continue;
         }
         pt_ = prof_begin(PC_GATEUP);
-        const rk::Act act_f = act_for(act_f_x_, act_f_sums_, act_f_qx_, act_f_qsums_, F, {L.down.w.type}, ffn_lora);
+        const rk::Act act_f = act_for(act_f_x_, act_f_sums_, act_f_qx_, act_f_qsums_, F, {L.down.w.type}, ffn_lora, &act_f_codes_);
         if (L.gate_up_interleaved && !ffn_lora) {
             rk::matmul_swiglu(stream_, L.gate_up[0].w, act_e, T, act_f, mm_ws_.ptr, gu);
             prof_end(PC_GATEUP, pt_);

@@ -1,0 +1,206 @@
+// The integer matrix-vector kernel of very small steps under ggml's arithmetic (gfx950, wave64).
+//
+// A step of one or two tokens reads every weight once and has nothing to amortise the conversion of the
+// 4-bit codes to f16 matrix operands over: the tile kernels then spend their time issuing vector instructions,
+// not waiting for memory. When the activations are Q8_K blocks anyway (what ggml's CPU dot product of a Q4_K
+// row multiplies, ggml-quants.c ggml_vec_dot_q4_K_q8_K), the products can stay integers: one mask (and one
+// shift) turns a dword of eight nibbles into two dwords of four bytes, and a four-way integer dot product
+// multiplies each with four activation codes - about a quarter of the vector instructions per weight.
+//
+//   sum_k w[n][k] x[k] = sum over super-blocks of
+//       d_x * ( d_w * sum_s sc_s * (sum_{k in s} q_k c_k)  -  dmin_w * sum_s m_s * bsum_s )
+//
+// with q the 4-bit codes, c the activation codes, sc / m the 6-bit scales and mins of the eight sub-blocks s,
+// bsum_s the sum of the activation codes of s: all integer up to the two float factors per super-block, exactly
+// the quantities ggml's kernel forms (its order of the float additions is one of several, per instruction set).
+//
+// The matrix is the Q4_K tile layout of the tile kernels (16 rows x 256 columns, 16-byte row headers, then two
+// 1 KiB loads in which lane (r = l % 16, g = l / 16) of load h holds, as dword j, the eight nibbles of columns
+// 32 (4h + j) + 8g .. + 8 of row r, in the order e0 e2 e4 e6 e1 e3 e5 e7). Masking a dword with 0x0F0F0F0F gives
+// the bytes e0 e4 e1 e5, the same after a shift by four e2 e6 e3 e7: the activation codes are stored in that
+// byte order (act_code_pos), so no lane ever permutes anything.
+#include "dev_common.hpp"
+
+namespace rk {
+
+int g_gemv_max_t = GEMV_MAX_T;
+
+struct GemvArgs {
+    const uint8_t * w;         // Q4_K tiles
+    const int8_t * codes;      // [T][K]
+    const float * d;           // [T][K / 256]
+    const int16_t * bsums;     // [T][K / 32]
+    float * y;
+    const float * bias;
+    int K, N, T, ldy, col0, mode, n_tiles;
+};
+
+// NT: tokens held (rows of the step beyond a.T read as zeros). PER: super-blocks of a tile per wave; a workgroup
+// has nw waves (PER 2: half the row's super-blocks; PER 4, rows wider than 32 super-blocks: 16), wave w takes
+// super-blocks w + u * nw. A matrix read once has
+// nothing to hide the memory latency behind, so the loads are issued as early as they can be: a wave holds two
+// super-blocks at a time and requests the next two as soon as those registers are free - the first pair before the
+// step's rows are staged, the first pair of the next tile before the partial sums of this one meet in LDS (one
+// barrier per tile: the sums alternate between two buffers). Holding all four of a wide row at once was slower.
+// Dynamic LDS: codes NT * K bytes | block sums NT * K / 16 bytes | scales NT * K / 64 bytes | 2 * nw * NT * 16 floats.
+template <int NT, int PER>
+__global__ __launch_bounds__(1024) void k_gemv_q4k(GemvArgs a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int K = a.K, nsb = K >> 8;
+    const int nthreads = blockDim.x, nw = nthreads >> 6;
+    int8_t * l_codes = (int8_t *)lds;
+    int16_t * l_bsums = (int16_t *)(lds + (size_t)NT * K);
+    float * l_d = (float *)(lds + (size_t)NT * K + (size_t)NT * (K >> 4));
+    float * l_red = l_d + NT * nsb;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+
+    // two super-blocks are held at a time: u0 and u0 + 1 of the wave's PER
+    u4 hdr[2], q[2][2];
+    auto request = [&](int tile, int u0) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int sb = wave + (u0 + u) * nw;
+            if (sb < nsb) {
+                const uint8_t * tp = a.w + ((size_t)tile * nsb + sb) * 2304;
+                hdr[u] = *(const u4 *)(tp + r * 16);
+                q[u][0] = *(const u4 *)(tp + 256 + lane * 16);
+                q[u][1] = *(const u4 *)(tp + 1280 + lane * 16);
+            }
+        }
+    };
+    int tile = blockIdx.x;
+    if (tile < a.n_tiles) request(tile, 0);
+
+    // stage the rows of the step: 16-byte words of codes, dwords of block sums, scales
+    for (int i = tid; i < NT * (K >> 4); i += nthreads) {
+        const int t = i / (K >> 4);
+        u4 v = {0u, 0u, 0u, 0u};
+        if (t < a.T) v = ((const u4 *)a.codes)[i];
+        ((u4 *)l_codes)[i] = v;
+    }
+    for (int i = tid; i < NT * (K >> 6); i += nthreads) {
+        const int t = i / (K >> 6);
+        ((uint32_t *)l_bsums)[i] = t < a.T ? ((const uint32_t *)a.bsums)[i] : 0u;
+    }
+    for (int i = tid; i < NT * nsb; i += nthreads) l_d[i] = i / nsb < a.T ? a.d[i] : 0.0f;
+    __syncthreads();
+
+    float acc[NT];
+    // super-block sb of the tile, held in register set u, times the rows of the step
+    auto multiply = [&](int sb, int u) {
+        const Q4KScales S = q4k_scales(hdr[u]);
+        int dot[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) dot[t] = 0;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t wq = j == 0 ? q[u][h].x : (j == 1 ? q[u][h].y : (j == 2 ? q[u][h].z : q[u][h].w));
+                const int lo = (int)(wq & 0x0F0F0F0Fu), hi = (int)((wq >> 4) & 0x0F0F0F0Fu);
+                const int sc = (int)((S.sc[h] >> (8 * j)) & 0xffu);
+                const int k0 = (sb << 8) + ((4 * h + j) << 5) + (g << 3);
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const uint2 c = *(const uint2 *)(l_codes + t * K + k0);
+                    int is = __builtin_amdgcn_sdot4(lo, (int)c.x, 0, false);
+                    is = __builtin_amdgcn_sdot4(hi, (int)c.y, is, false);
+                    dot[t] += __mul24(sc, is);
+                }
+            }
+        }
+        // the min term: lane group g takes sub-blocks 2g and 2g + 1
+        const uint32_t mword = (g < 2 ? S.mn[0] : S.mn[1]) >> (16 * (g & 1));
+        const int m0 = (int)(mword & 0xffu), m1 = (int)((mword >> 8) & 0xffu);
+        const float dw = h2f((uint16_t)(hdr[u].x & 0xffffu)), dmin = h2f((uint16_t)(hdr[u].x >> 16));
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const int bs = *(const int *)(l_bsums + t * (K >> 5) + (sb << 3) + 2 * g);
+            const int mins = __mul24(m0, (int)(int16_t)(bs & 0xffff)) + __mul24(m1, bs >> 16);
+            acc[t] += l_d[t * nsb + sb] * (dw * (float)dot[t] - dmin * (float)mins);
+        }
+    };
+
+    for (int turn = 0; tile < a.n_tiles; tile += gridDim.x, turn ^= 1) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
+#pragma unroll
+        for (int u0 = 0; u0 < PER; u0 += 2) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int sb = wave + (u0 + u) * nw;
+                if (sb < nsb) multiply(sb, u);
+            }
+            // the registers are free again: the wave's next pair of this tile, or its first of the next tile
+            if (u0 + 2 < PER) request(tile, u0 + 2);
+            else if (tile + (int)gridDim.x < a.n_tiles) request(tile + (int)gridDim.x, 0);
+        }
+        // the four lane groups of a row, then the waves of the workgroup
+        float * red = l_red + turn * (nw * NT * 16);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            acc[t] += __shfl_xor(acc[t], 16, 64);
+            acc[t] += __shfl_xor(acc[t], 32, 64);
+            if (g == 0) red[(wave * NT + t) * 16 + r] = acc[t];
+        }
+        __syncthreads();
+        if (tid < NT * 16) {
+            const int t = tid >> 4, row = tid & 15;
+            if (t < a.T) {
+                float v = 0.0f;
+                for (int w = 0; w < nw; ++w) v += red[(w * NT + t) * 16 + row];
+                const int n = tile * 16 + row;
+                if (a.bias) v += a.bias[n];
+                float * dst = a.y + (size_t)t * a.ldy + a.col0 + n;
+                *dst = a.mode == MM_ADD ? *dst + v : v;
+            }
+        }
+    }
+}
+
+constexpr size_t kGemvMaxLds = 96 * 1024;     // of the CU's 160 KiB; two tokens of 16,384 columns take 39 KiB
+static size_t gemv_lds_bytes(int NT, int NW, int K) {
+    return (size_t)NT * K + (size_t)NT * (K >> 4) + (size_t)NT * (K >> 8) * 4 + (size_t)2 * NW * NT * 16 * 4;
+}
+
+bool gemv_can(const Weight & w, const Act & x, int T) {
+    return w.type == WT_Q4_K && w.packed && x.qc && x.qd && x.qbs && T >= 1 && T <= g_gemv_max_t && T <= GEMV_MAX_T
+        && w.K % 256 == 0 && w.N % 16 == 0 && w.K > 0 && w.N > 0 && x.K == w.K
+        && w.K <= 256 * 4 * 16 && gemv_lds_bytes(GEMV_MAX_T, 16, w.K) <= kGemvMaxLds;
+}
+
+template <int NT, int PER>
+static void launch_gemv(hipStream_t s, const GemvArgs & a) {
+    const int nsb = a.K / 256;
+    const int nw = PER == 2 ? (nsb + 1) / 2 : 16;
+    const size_t lds = gemv_lds_bytes(NT, nw, a.K);
+    static bool once = false;
+    if (!once) {
+        HIP_OK(hipFuncSetAttribute((const void *)k_gemv_q4k<NT, PER>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvMaxLds));
+        once = true;
+    }
+    // a workgroup stages the step's rows once and then walks tiles: as many workgroups as the chip holds at
+    // once, fewer when that gives every workgroup the same number of tiles
+    const int capacity = 256 * std::max(1, 2048 / (nw * 64));
+    const int turns = (a.n_tiles + capacity - 1) / capacity;
+    const unsigned grid = (unsigned)((a.n_tiles + turns - 1) / turns);
+    hipLaunchKernelGGL((k_gemv_q4k<NT, PER>), dim3(grid), dim3(nw * 64), lds, s, a);
+}
+
+void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias) {
+    if (!gemv_can(w, x, T)) throw std::runtime_error("gemv: needs Q4_K tiles, Q8_K code buffers and at most " + std::to_string(GEMV_MAX_T) + " tokens");
+    if (mode != MM_STORE && mode != MM_ADD) throw std::runtime_error("gemv: stores or adds");
+    if (col0 < 0 || col0 + w.N > ldy) throw std::runtime_error("gemv: the outputs do not fit the row");
+    GemvArgs a {};
+    a.w = w.packed; a.codes = x.qc; a.d = x.qd; a.bsums = x.qbs; a.y = y; a.bias = bias;
+    a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode; a.n_tiles = w.N / 16;
+    // two super-blocks of a tile per wave while sixteen waves cover the row, four beyond
+    const bool two = w.K <= 256 * 2 * 16;
+    static_assert(GEMV_MAX_T == 2, "one instantiation per token count");
+    if (T == 1) { if (two) launch_gemv<1, 2>(s, a); else launch_gemv<1, 4>(s, a); }
+    else { if (two) launch_gemv<2, 2>(s, a); else launch_gemv<2, 4>(s, a); }
+    check_launch("gemv");
+}
+
+}  // namespace rk

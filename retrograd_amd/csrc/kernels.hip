@@ -191,7 +191,10 @@ __device__ __forceinline__ void store_act_block(const float * v, int count, cons
 }
 
 // Host-side check of what a producer is asked to write.
-static void check_act_out(const Act & out, int K, const char * what) {
+static void check_act_out(const Act & out, int K, const char * what, int n_rows) {
+    if (out.qc && (out.quant != AQ_Q8_K || !out.qx || !out.qd || !out.qbs || n_rows > GEMV_MAX_T))
+        throw std::runtime_error(std::string(what) + ": the integer code buffers go with the Q8_K conversion of at most "
+                                 + std::to_string(GEMV_MAX_T) + " rows");
     if (out.K != K) throw std::runtime_error(std::string(what) + ": activation width does not match");
     if (!out.x && !out.qx) throw std::runtime_error(std::string(what) + ": no activation buffer to write");
     if (out.qx) {
@@ -713,6 +716,13 @@ static Slices matmul_impl(hipStream_t s, const Weight & w, const Act & x, int T,
     if (x.K != w.K) throw std::runtime_error("matmul: activation width does not match the weight");
     // the tile kernels know two layouts; anything else handed over as tiles would be read as one of them, out of bounds
     if (!can_pack(w.type, w.K, w.N)) throw std::runtime_error("matmul: this matrix type or shape has no tile layout");
+    if (T <= GEMV_MAX_T) {     // a very small step whose producer left the Q8_K blocks themselves
+        const Act xg = x.operand(w.type);
+        if ((mode == MM_STORE || mode == MM_ADD) && gemv_can(w, xg, T)) {
+            gemv(s, w, xg, T, y, ldy, col0, mode, bias);
+            return Slices();
+        }
+    }
     if (ws) return matmul_lds(s, w, x, T, y, ldy, col0, mode, bias, ws, may_slice);
     if (w.type == WT_Q6_K || w.type == WT_Q5_K)
         throw std::runtime_error("matmul: Q5_K and Q6_K tiles are multiplied by the LDS kernels only (pass the workspace)");
@@ -1028,7 +1038,7 @@ void rmsnorm_act(hipStream_t s, float * x, const float * w, int E, float eps,
                  const int32_t * rows, int n_rows, const Act & out, const Slices & add) {
     if (n_rows <= 0) return;
     if (add.n > 0 && add.N != E) throw std::runtime_error("rmsnorm: the slices do not match the row width");
-    check_act_out(out, E, "rmsnorm");
+    check_act_out(out, E, "rmsnorm", n_rows);
     if (E % 32 == 0) {
         if (E >= 4096) hipLaunchKernelGGL(k_rmsnorm_act8<8>, dim3(n_rows), dim3(512), 0, s, x, w, E, eps, rows, out, add);
         else hipLaunchKernelGGL(k_rmsnorm_act8<4>, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, out, add);
@@ -1085,7 +1095,7 @@ __global__ __launch_bounds__(256) void k_to_act8(const float * __restrict__ x, i
 
 void to_act(hipStream_t s, const float * x, int T, int K, const Act & out) {
     if (T <= 0) return;
-    check_act_out(out, K, "to_act");
+    check_act_out(out, K, "to_act", T);
     if (K % 32 == 0) {
         const size_t n = (size_t)T * (K / 8);
         hipLaunchKernelGGL(k_to_act8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, T, K, out);
@@ -1114,7 +1124,7 @@ __global__ __launch_bounds__(256) void k_requant_act8(const __half * src, int T,
 
 void requant_act(hipStream_t s, const __half * src, int T, const Act & out) {
     if (T <= 0) return;
-    check_act_out(out, out.K, "requant_act");
+    check_act_out(out, out.K, "requant_act", T);
     if (out.x || !out.qx) throw std::runtime_error("requant_act: writes the converted rows only");
     const size_t n = (size_t)T * (out.K / 8);
     hipLaunchKernelGGL(k_requant_act8, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, src, T, out.K, out);
@@ -1140,7 +1150,7 @@ __global__ __launch_bounds__(256) void k_swiglu_act8(const float * __restrict__ 
 
 void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out, int group) {
     if (T <= 0) return;
-    check_act_out(out, F, "swiglu");
+    check_act_out(out, F, "swiglu", T);
     if (group <= 0) group = F;
     // a block of 32 (8) gate columns must not straddle two groups
     if (group != F && (F % group != 0 || group % 32 != 0)) throw std::runtime_error("swiglu: the interleave group must divide F and be a multiple of 32");
@@ -2064,13 +2074,29 @@ __global__ __launch_bounds__(256) void k_attention_combine(CombineArgs a) {
         float gmax = 0.0f, max = 0.0f;
         for (int w = w0; w < w0 + per; ++w)
             if (blk_amax[w] > gmax) { gmax = blk_amax[w]; max = blk_first[w]; }
+        float c0 = 0.0f, c1 = 0.0f, d = 0.0f;
         if (gmax == 0.0f) {
             q0 = q1 = 0.0f;
         } else {
             const float iscale = __fdiv_rn(-127.0f, max);
-            const float d = __fdiv_rn(1.0f, iscale);
-            q0 = __fmul_rn(d, fminf(127.0f, rintf(__fmul_rn(iscale, f0))));
-            q1 = __fmul_rn(d, fminf(127.0f, rintf(__fmul_rn(iscale, f1))));
+            d = __fdiv_rn(1.0f, iscale);
+            c0 = fminf(127.0f, rintf(__fmul_rn(iscale, f0)));
+            c1 = fminf(127.0f, rintf(__fmul_rn(iscale, f1)));
+            q0 = __fmul_rn(d, c0);
+            q1 = __fmul_rn(d, c1);
+        }
+        if (a.out.qc) {      // the blocks themselves, for the integer matrix-vector kernel (see store_codes8)
+            const int i0 = (int)c0, i1 = (int)c1;
+            int sum = i0 + i1;
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o, 64);
+            if (mine) {
+                int8_t * grp = a.out.qc + (size_t)t * QD + (k & ~7);
+                grp[act_code_pos(k & 7)] = (int8_t)i0;
+                grp[act_code_pos((k & 7) + 1)] = (int8_t)i1;
+                if ((lane & 15) == 0) a.out.qbs[(size_t)t * (QD >> 5) + (k >> 5)] = (int16_t)sum;
+                if (wave == w0 && lane == 0) a.out.qd[(size_t)t * (QD >> 8) + (k >> 8)] = d;
+            }
         }
     }
     store(a.out.qx, a.out.qsums, q0, q1);
@@ -2079,7 +2105,7 @@ __global__ __launch_bounds__(256) void k_attention_combine(CombineArgs a) {
 void attention_combine(hipStream_t s, const float * partial, int T, const AttnShape & sh,
                        const PackBuffers & pk, const Act & out) {
     if (T <= 0) return;
-    check_act_out(out, sh.n_head * sh.head_dim, "attention_combine");
+    check_act_out(out, sh.n_head * sh.head_dim, "attention_combine", T);
     if (out.qx && out.quant == AQ_Q8_K && ((sh.head_dim != 64 && sh.head_dim != 128) || (sh.n_head * sh.head_dim) % 256 != 0))
         throw std::runtime_error("attention_combine: the Q8_K conversion needs heads of 64 or 128 dimensions");
     CombineArgs a;

@@ -78,17 +78,28 @@ struct Act {
     __half * qsums = nullptr;
     int quant = AQ_NONE;
     int faithful = 0;           // ggml's arithmetic: F16 / BF16 operands are rounded as well
+    // With quant == AQ_Q8_K a producer can leave the Q8_K blocks themselves as well, for the integer
+    // matrix-vector kernel that multiplies very small steps (gemv): the int8 codes [token][K], the eight
+    // codes of a group k / 8 in the order 0 4 1 5 2 6 3 7 (act_code_pos; the order in which a Q4_K tile's
+    // nibbles unpack into bytes); the block scales 1 / iscale, f32 [token][K / 256]; and the sums of the
+    // codes of every 32, int16 [token][K / 32].
+    int8_t * qc = nullptr;
+    float * qd = nullptr;
+    int16_t * qbs = nullptr;
     // What a weight of this type multiplies: the converted row for the quantised
     // types under ggml's arithmetic, the values themselves otherwise.
     Act operand(int ggml_type) const {
         Act a;
         a.K = K;
         a.faithful = faithful;
-        if (faithful && act_quant_of(ggml_type) != AQ_NONE) { a.x = qx; a.sums = qsums; }
-        else { a.x = x; a.sums = sums; }
+        if (faithful && act_quant_of(ggml_type) != AQ_NONE) {
+            a.x = qx; a.sums = qsums;
+            if (act_quant_of(ggml_type) == AQ_Q8_K && quant == AQ_Q8_K) { a.qc = qc; a.qd = qd; a.qbs = qbs; }
+        } else { a.x = x; a.sums = sums; }
         return a;
     }
 };
+constexpr int act_code_pos(int i) { return (i & 3) * 2 + (i >> 2); }    // byte of code i within its group of eight
 inline size_t act_halves(int T, int K) { return (size_t)((T + 63) / 64) * (size_t)((K + 31) / 32 * 32) * 128; }
 inline size_t act_sum_halves(int T, int K) { return (size_t)((T + 63) / 64) * (size_t)((K + 255) / 256) * 2048; }
 
@@ -124,6 +135,14 @@ Slices matmul_deferred(hipStream_t s, const Weight & w, const Act & x, int T, fl
 // y[t][col0 + c] (=|+=) sum of the slices.
 void reduce_slices(hipStream_t s, const Slices & sl, int T, float * y, int ldy, int col0, int mode);
 size_t matmul_workspace_bytes();
+// The integer matrix-vector kernel: a Q4_K tile matrix times the Q8_K blocks of one or two tokens, as
+// ggml's CPU dot product multiplies them (integer sums of code products per sub-block, times the integer
+// sub-block scale, one float multiply per super-block). One workgroup per 16-row tile, the waves of a
+// workgroup share the tile's super-blocks; no K-slices. x is the operand (Act::operand) of the weight.
+constexpr int GEMV_MAX_T = 2;     // beyond two tokens the tile kernels are as fast
+bool gemv_can(const Weight & w, const Act & x, int T);
+void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias);
+extern int g_gemv_max_t;       // steps of at most this many tokens take the kernel (default GEMV_MAX_T; 0 switches it off)
 extern int g_mm_debug;         // timing experiments (see MMArgs::debug)
 extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic
 // Fused gate/up matmul and SwiGLU: w holds, for every 64 columns of the hidden
@@ -131,7 +150,8 @@ extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic
 // a tile storage type); out (K = F) receives silu(gate) * up as activations.
 // When out asks for the Q8_K conversion, whose blocks are wider than the 64
 // columns a workgroup holds, the products leave as f32 rows in h_f32 ([T][F])
-// and a second launch converts them.
+// and a second launch converts them. h_f32 has room for [T][2 F]: a very small step whose rows came with
+// Q8_K code buffers is multiplied by the integer kernel (gemv) into gate and up rows there.
 void matmul_swiglu(hipStream_t s, const Weight & w, const Act & x, int T, const Act & out, void * ws, float * h_f32);
 // Several tile-packed matrices over the same activations, outputs side by side in y from column 0 (bias likewise):
 // one launch each, all leaving the same number of K-slices in one set of slices of the full row width.

@@ -1031,6 +1031,18 @@ Slices matmul_deferred_parts(hipStream_t s, const Weight * const * parts, int n_
         total += parts[i]->N;
     }
     if (!ws || total > ldy) throw std::runtime_error("matmul_deferred_parts: needs the workspace and room for every part in y");
+    if (T <= GEMV_MAX_T) {     // every part by the integer matrix-vector kernel, or none
+        bool all = true;
+        for (int i = 0; i < n_parts; ++i) all = all && gemv_can(*parts[i], x.operand(parts[i]->type), T);
+        if (all) {
+            int at = 0;
+            for (int i = 0; i < n_parts; ++i) {
+                gemv(s, *parts[i], x.operand(parts[i]->type), T, y, ldy, at, MM_STORE, bias ? bias + at : nullptr);
+                at += parts[i]->N;
+            }
+            return Slices();
+        }
+    }
     const int nsb = K / 256, chunks = (T + 63) / 64;
     int ksplit = 1;
     if (chunks == 1) {
@@ -1072,6 +1084,12 @@ void matmul_swiglu(hipStream_t s, const Weight & w, const Act & x, int T, const 
     if (x.K != w.K) throw std::runtime_error("matmul_swiglu: activation width does not match the weight");
     // A workgroup holds 64 hidden columns of a token: enough for the 32-wide blocks of the Q8_0
     // conversion, not for the 256-wide ones of Q8_K. Those rows leave as f32 and are converted after.
+    if (h_f32 && T <= GEMV_MAX_T && gemv_can(w, x.operand(w.type), T)) {
+        // a very small step: gate and up as f32 rows (in their groups of 64) by the integer kernel, then the SiLU
+        gemv(s, w, x.operand(w.type), T, h_f32, w.N, 0, MM_STORE, nullptr);
+        swiglu_act(s, h_f32, T, out.K, out, 64);
+        return;
+    }
     const bool via_f32 = out.qx && out.quant == AQ_Q8_K;
     if (via_f32 && !h_f32) throw std::runtime_error("matmul_swiglu: the Q8_K conversion needs the f32 row buffer");
     lds_impl(s, w, x, T, nullptr, 0, 0, MM_SWIGLU, nullptr, ws, false, &out, via_f32 ? h_f32 : nullptr);

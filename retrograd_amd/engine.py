@@ -869,10 +869,11 @@ class _GrammarHandle:
 
 def kernel_matmul(ggml_type: int, raw: np.ndarray, n_rows: int, k: int, x: np.ndarray, use_tiles,
                   bias: np.ndarray | None = None, accumulate_into: np.ndarray | None = None,
-                  ggml_activations: bool = False) -> np.ndarray:
-    """One matmul kernel on host data; ggml_activations: the rows are converted as ggml's CPU matmul does."""
+                  ggml_activations: bool = False, integer: bool = False) -> np.ndarray:
+    """One matmul kernel on host data; ggml_activations: the rows are converted as ggml's CPU matmul does;
+    integer (with it, Q4_K tiles, at most two rows): the Q8_K blocks go through the integer matrix-vector kernel."""
     lib = load_library()
-    use_tiles = int(use_tiles) | (0x100 if ggml_activations else 0)
+    use_tiles = int(use_tiles) | (0x100 if ggml_activations else 0) | (0x200 if integer else 0)
     raw = np.ascontiguousarray(raw, np.uint8)
     x = np.ascontiguousarray(x, np.float32)
     T = x.shape[0]

@@ -140,6 +140,66 @@ def test_tile_matmul_exact_on_integer_data():
             assert np.array_equal(got.astype(np.float64), want), (mode, ggml)
 
 
+@pytest.mark.parametrize("n,k,T", [(16, 256, 1), (48, 512, 2), (2064, 256, 2), (64, 1024, 1), (256, 4096, 1), (32, 8192, 2),
+                                   (128, 14336, 2), (4096, 4096, 2), (1024, 14336, 1), (320, 16384, 2), (16, 8448, 1)])
+def test_integer_matvec_matches_decoded_blocks(n, k, T):
+    # The kernel of very small steps under the ggml arithmetic: integer products of the stored codes with the
+    # Q8_K codes of the rows. Its sums are those of the converted values times the decoded weights, so the
+    # reference of the tile kernels is its reference too.
+    print("case", n, k, T, flush=True)
+    t = gw.GGML_Q4_K
+    raw, dense = _weights(t, n, k, seed=n + k + T)
+    rng = np.random.default_rng(T + k)
+    x = rng.standard_normal((T, k)).astype(np.float32)
+    x[0, :256] = 0.0                                    # a block of zeros: scale 0, codes 0
+    want = _ref(t, dense, x, True)
+    scale = np.abs(want).max()
+    got = E.kernel_matmul(t, raw, n, k, x, use_tiles=2, ggml_activations=True, integer=True)
+    assert np.abs(got - want).max() <= 2e-5 * scale + 1e-6
+    tiles = E.kernel_matmul(t, raw, n, k, x, use_tiles=2, ggml_activations=True)
+    assert np.abs(got - tiles).max() <= 2e-5 * scale + 1e-6
+    bias = rng.standard_normal(n).astype(np.float32)
+    y0 = rng.standard_normal((T, n)).astype(np.float32)
+    got = E.kernel_matmul(t, raw, n, k, x, use_tiles=2, ggml_activations=True, integer=True, bias=bias)
+    assert np.abs(got - (want + bias)).max() <= 3e-5 * scale + 1e-6
+    got = E.kernel_matmul(t, raw, n, k, x, use_tiles=2, ggml_activations=True, integer=True, accumulate_into=y0)
+    assert np.abs(got - (want + y0)).max() <= 3e-5 * scale + 1e-6
+
+
+def test_integer_matvec_exact_on_integer_data_and_refusals():
+    # Random bytes in every position of the tile (every code, scale and min), dyadic d and dmin, activations
+    # that are their own Q8_K codes: every product and sum is exact in i32 and f32, so a misplaced nibble,
+    # scale, min or activation byte shows as a wrong bit.
+    rng = np.random.default_rng(17)
+    n, k = 48, 768
+    blocks = rng.integers(0, 256, (n, k // 256, 144), dtype=np.uint8)
+    blocks[..., 0:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    blocks[..., 2:4] = np.frombuffer(np.float16(0.25).tobytes(), np.uint8)
+    raw = blocks.reshape(n, -1)
+    dense = np.stack([oracle.decode_row(gw.GGML_Q4_K, raw[i], k) for i in range(n)]).astype(np.float64)
+    for T in (1, 2):
+        x = rng.integers(-4, 5, (T, k)).astype(np.float32)
+        x[:, ::32] = rng.choice([-127.0, 127.0], (T, k // 32))
+        assert np.array_equal(np.stack([oracle.activation_row(gw.GGML_Q4_K, r) for r in x]), x)
+        want = x.astype(np.float64) @ dense.T
+        got = E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x, use_tiles=2, ggml_activations=True, integer=True)
+        assert np.array_equal(got.astype(np.float64), want), T
+    # one activation at a time: element e alone is non-zero, which places every byte of the code order
+    for e in (0, 1, 2, 3, 4, 5, 6, 7, 8, 31, 32, 100, 255, 256, 767):
+        one = np.zeros((1, k), np.float32)
+        one[0, e] = -127.0
+        got = E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, one, use_tiles=2, ggml_activations=True, integer=True)
+        assert np.array_equal(got[0].astype(np.float64), -127.0 * dense[:, e]), e
+    x = rng.standard_normal((3, k)).astype(np.float32)
+    with pytest.raises(E.EngineError, match="at most 2 tokens"):
+        E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x, use_tiles=2, ggml_activations=True, integer=True)
+    with pytest.raises(E.EngineError, match="at most 2 tokens"):
+        E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x[:1], use_tiles=2, integer=True)      # the exact arithmetic has no codes
+    q8, _ = _weights(gw.GGML_Q8_0, 16, 256, seed=1)
+    with pytest.raises(E.EngineError, match="at most 2 tokens"):
+        E.kernel_matmul(gw.GGML_Q8_0, q8, 16, 256, x[:1, :256], use_tiles=2, ggml_activations=True, integer=True)
+
+
 def test_q6k_tiles_are_exact_for_every_code_and_scale():
     # Random bytes: every six-bit code, every i8 scale (-128 and 127 included, whose products with a code
     # are not all f16 numbers) in every position of the tile. With d = 1 and small-integer activations all

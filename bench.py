@@ -474,6 +474,7 @@ def main() -> int:
                 eng.seq_rm(s_.slot)
                 eng.request_free(s_.request)
         result["config"]["through_the_step_scheduler"] = scheduler_leg(args, eng, E, shape, geometry)
+        result["config"]["one_sequence"] = {args.activations: one_sequence_leg(eng, E, shape, n_slots, w_bytes, kv_bytes_per_cell_layer)}
     eng.close()
     del eng
 
@@ -488,12 +489,45 @@ def main() -> int:
                "arithmetic": "RETRO_ACTIVATIONS=ggml: Q8_K / Q8_0 activation conversion before every quantised matmul"}
         if not args.no_cpu_baseline:
             _, leg["parity_full_size_against_the_oracle_in_the_same_arithmetic"] = cpu_baseline(eng, E, oracle, wl2, model_path, args.cpu_rows, "ggml", time_it=False, kv=args.kv)
+        for s_ in wl2.seqs:
+            if s_ is not None:
+                eng.seq_rm(s_.slot)
+                eng.request_free(s_.request)
+        leg["one_sequence"] = one_sequence_leg(eng, E, shape, n_slots, w_bytes, kv_bytes_per_cell_layer)
         result["ggml_arithmetic"] = leg
         eng.close()
     os.environ["RETRO_ACTIVATIONS"] = "exact"
 
     print(json.dumps(result), flush=True)
     return 0
+
+
+def one_sequence_leg(eng, E, shape, n_slots, w_bytes, kv_bytes_per_cell_layer, context=512, steps=48):
+    """Decode steps of a single sequence at a fixed context on an engine whose slots are free again: the small-batch
+    end of the same step (under the ggml arithmetic its Q4_K matrices go through the integer matrix-vector kernel)."""
+    for slot in range(n_slots):
+        eng.seq_rm(slot)
+    rng = np.random.default_rng(99)
+    out = E.StepOutput(8)
+    greedy = E.SamplingParamsV2.greedy()
+    request = 1 << 40
+    prompt = rng.integers(0, shape.n_vocab, context).astype(np.int32)
+    eng.step([E.StepRow(request, 0, prompt, 0, sample=True, sampling=greedy)], out)
+    token, pos, times = out.row(0).token, context, []
+    for i in range(steps):
+        t0 = time.perf_counter()
+        eng.step([E.StepRow(request, 0, [token], pos, sample=True, sampling=greedy)], out)
+        dt = time.perf_counter() - t0
+        token, pos = out.row(0).token, pos + 1
+        if i >= 8:
+            times.append(dt)
+    eng.seq_rm(0)
+    eng.request_free(request)
+    sec = float(np.median(times))
+    step_bytes = w_bytes + shape.n_layer * kv_bytes_per_cell_layer * (context + steps // 2)
+    return {"context": context, "ms_per_step": round(sec * 1e3, 4), "tok_s": round(1.0 / sec, 1),
+            "step_frac_of_hbm_roofline": round(step_bytes / (HBM_PEAK_GBS * 1e9) / sec, 4),
+            "timing": "median of %d single-row decode steps, host clock around each step" % len(times)}
 
 
 def cpu_baseline(eng, E, oracle, wl, model_path, n_rows, activations="exact", time_it=True, kv="f16"):

@@ -65,6 +65,9 @@ def parse_args():
     ap.add_argument("--no-scheduler-leg", action="store_true", help="skip the run of the same workload through the step scheduler")
     ap.add_argument("--scheduler-requests", type=int, default=128)
     ap.add_argument("--no-ggml-leg", action="store_true", help="skip the secondary measurement under the ggml arithmetic")
+    ap.add_argument("--one-sequence", action="store_true",
+                    help="measure only the single-sequence decode steps (512-token context) in the chosen arithmetic and "
+                         "print their JSON: the workload of the small-batch kernel profiles")
     return ap.parse_args()
 
 
@@ -345,6 +348,14 @@ def main() -> int:
         print("[bench] engine (%s arithmetic) ready in %.1fs" % (activations, time.perf_counter() - t0), file=sys.stderr, flush=True)
         return eng
 
+    if args.one_sequence:
+        eng = new_engine(args.activations)
+        kvb = 2 * shape.n_head_kv * shape.head_dim * 2 * {"f16": 32, "q8_0": 17, "q4_0": 9}[args.kv] // 32
+        leg = one_sequence_leg(eng, E, shape, n_slots, synth.streamed_weight_bytes(shape), kvb, steps=args.steps)
+        eng.close()
+        print(json.dumps({"metric": "single-sequence decode steps, 8B-shape Q4_K", "activations": args.activations,
+                          "kv_cache": args.kv, **leg}), flush=True)
+        return 0
     eng = new_engine(args.activations)
     m, wl = measure_decode(args, eng, E, synth, gw, shape, geometry, profile_kernels=True)
     sampled, decode_rows, cells, tokens, elapsed = m["dec"]

@@ -32,6 +32,14 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
 /* Per logits row: argmax (lowest id on ties), max, sum exp(double(l) - max),
  * and the k[r] best (id, logit) pairs in (logit desc, id asc) order, written
  * to out_top_*[r * retro_kernel_max_topk() + j]. */
+/* The integer matrix-vector kernel with the producer of its rows fused into its staging, beside the same product
+ * as two launches. kind 1: x is [n_tokens][k] residual rows, the rows multiplied are their RMSNorm (norm_w, eps)
+ * converted to Q8_K; kind 2: x is [n_tokens][2 k] gate and up values in alternating groups of `group` columns
+ * (0: side by side), the rows are silu(gate) * up converted to Q8_K. raw: n_rows Q4_K rows of k. Both results are
+ * [n_tokens][n_rows]; at most two tokens. */
+int retro_kernel_gemv_fused(int32_t kind, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, const float * norm_w,
+                            float eps, int32_t n_tokens, int32_t group, float * y_fused, float * y_unfused);
+
 int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_vocab, const int32_t * k,
                                 int32_t * out_argmax, float * out_max, double * out_sum_exp,
                                 int32_t * out_top_ids, float * out_top_logits);

@@ -99,6 +99,52 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
     });
 }
 
+int retro_kernel_gemv_fused(int32_t kind, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, const float * norm_w,
+                            float eps, int32_t n_tokens, int32_t group, float * y_fused, float * y_unfused) {
+    return guarded([&]() -> int {
+        if ((kind != 1 && kind != 2) || n_tokens < 1 || n_tokens > rk::GEMV_MAX_T || k <= 0 || k % 256 != 0 || n_rows <= 0 || n_rows % 16 != 0)
+            throw std::runtime_error("gemv_fused: kind 1 (RMSNorm) or 2 (SwiGLU), whole tiles and super-blocks, at most " + std::to_string(rk::GEMV_MAX_T) + " tokens");
+        if (kind == 1 && !norm_w) throw std::runtime_error("gemv_fused: the RMSNorm needs its weights");
+        const int type = rk::WT_Q4_K;
+        const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
+        const size_t in_floats = (size_t)n_tokens * k * (kind == 2 ? 2 : 1);
+        DevBuf d_raw, d_packed, d_x, d_w, d_xh, d_sums, d_codes, d_scales, d_bsums, d_y;
+        d_raw.alloc(bytes); d_packed.alloc(bytes);
+        ok(hipMemcpy(d_raw.ptr, raw, bytes, hipMemcpyHostToDevice), "upload weights");
+        rk::repack(nullptr, type, d_raw.as<uint8_t>(), d_packed.as<uint8_t>(), (int)k, (int)n_rows);
+        rk::Weight w;
+        w.type = type; w.K = (int)k; w.N = (int)n_rows; w.bytes = bytes; w.packed = d_packed.as<uint8_t>();
+        d_x.alloc(in_floats * 4);
+        ok(hipMemcpy(d_x.ptr, x, d_x.bytes, hipMemcpyHostToDevice), "upload rows");
+        if (kind == 1) {
+            d_w.alloc((size_t)k * 4);
+            ok(hipMemcpy(d_w.ptr, norm_w, d_w.bytes, hipMemcpyHostToDevice), "upload norm weights");
+        }
+        d_xh.alloc(rk::act_halves(n_tokens, (int)k) * 2);
+        d_sums.alloc(rk::act_sum_halves(n_tokens, (int)k) * 2);
+        ok(hipMemset(d_xh.ptr, 0, d_xh.bytes), "clear"); ok(hipMemset(d_sums.ptr, 0, d_sums.bytes), "clear");
+        d_codes.alloc((size_t)n_tokens * k); d_scales.alloc((size_t)n_tokens * (k / 256) * 4); d_bsums.alloc((size_t)n_tokens * (k / 32) * 2);
+        rk::Act act;
+        act.K = (int)k; act.faithful = 1; act.quant = rk::AQ_Q8_K;
+        act.qx = d_xh.as<__half>(); act.qsums = d_sums.as<__half>();
+        act.qc = d_codes.as<int8_t>(); act.qd = d_scales.as<float>(); act.qbs = d_bsums.as<int16_t>();
+        d_y.alloc((size_t)n_tokens * n_rows * 4);
+        // the two launches: the producer leaves the blocks, the kernel multiplies them
+        if (kind == 1) rk::rmsnorm_act(nullptr, d_x.as<float>(), d_w.as<float>(), (int)k, eps, nullptr, n_tokens, act);
+        else rk::swiglu_act(nullptr, d_x.as<float>(), n_tokens, (int)k, act, group);
+        rk::gemv(nullptr, w, act.operand(type), n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr);
+        ok(hipDeviceSynchronize(), "gemv");
+        ok(hipMemcpy(y_unfused, d_y.ptr, d_y.bytes, hipMemcpyDeviceToHost), "download");
+        ok(hipMemset(d_y.ptr, 0, d_y.bytes), "clear");
+        // one launch: the kernel makes the blocks while it stages them
+        if (kind == 1) rk::gemv_norm(nullptr, w, d_x.as<float>(), d_w.as<float>(), eps, nullptr, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr);
+        else rk::gemv_swiglu(nullptr, w, d_x.as<float>(), group, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE);
+        ok(hipDeviceSynchronize(), "gemv fused");
+        ok(hipMemcpy(y_fused, d_y.ptr, d_y.bytes, hipMemcpyDeviceToHost), "download");
+        return 0;
+    });
+}
+
 int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_vocab, const int32_t * k,
                                 int32_t * out_argmax, float * out_max, double * out_sum_exp,
                                 int32_t * out_top_ids, float * out_top_logits) {

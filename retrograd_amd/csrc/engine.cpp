@@ -77,6 +77,7 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
         // (Q8_K / Q8_0 codes, f16 / bf16 rounding); unset or "exact": the f32 values (as f16 hi/lo pairs).
         if (const char * dbg = std::getenv("RETRO_MM_DEBUG")) rk::g_mm_debug = std::atoi(dbg);     // timing experiments
         if (const char * dbg = std::getenv("RETRO_MM_SINGLE")) mm_single_mask_ = std::atoi(dbg);
+        if (const char * f = std::getenv("RETRO_GEMV_FUSE")) gemv_fuse_ = std::atoi(f) != 0;      // 0: producers keep their own launches
         // steps of at most this many tokens go through the integer matrix-vector kernel under the ggml arithmetic (0: never)
         const char * g = std::getenv("RETRO_GEMV_MAX_T");
         rk::g_gemv_max_t = g ? std::max(0, std::min(std::atoi(g), rk::GEMV_MAX_T)) : rk::GEMV_MAX_T;
@@ -1306,6 +1307,18 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
     const bool faithful = ggml_activations_;
     const bool ffn_lora = routed && lora_has_ffn_ && h.n_expert == 0;      // some row may carry feed-forward deltas
     const bool small_step = T <= rk::g_gemv_max_t;      // the producers leave the Q8_K blocks for the integer kernel as well
+    // ... or, where every consumer of a row is that kernel and nothing else wants the row (no adapters), the kernel
+    // makes the blocks itself while it stages them and the producer's launch is saved
+    // (single-token steps only: the blocks of a second row cost every workgroup more than the launch saves)
+    const bool fuse = faithful && small_step && T == 1 && !routed && gemv_fuse_;
+    auto all_gemv = [&](const std::vector<DevWeight> & ws, int K, int room) {
+        int total = 0;
+        for (const DevWeight & w : ws) {
+            if (!rk::gemv_can_weight(w.w, T) || w.w.K != K) return false;
+            total += w.w.N;
+        }
+        return !ws.empty() && total <= room;
+    };
     auto act_for = [faithful, small_step](DevBuf & x, DevBuf & sums, DevBuf & qx, DevBuf & qsums, int K, std::initializer_list<int> types,
                                           bool plain, ActCodes * codes = nullptr) {
         rk::Act a;
@@ -1351,11 +1364,19 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         const std::array<int, 3> qt = types_of(L.qkv), gt = types_of(L.gate_up);
         rk::Act act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {qt[0], qt[1], qt[2]}, routed, &act_e_codes_);
         const rk::Act act_q = act_for(act_q_x_, act_q_sums_, act_q_qx_, act_q_qsums_, QD, {L.wo.w.type}, routed, &act_q_codes_);
-        { const size_t pt_ = prof_begin(PC_NORM); rk::rmsnorm_act(stream_, x, L.attn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending); prof_end(PC_NORM, pt_); }
+        const bool qkv_fused = fuse && pending.n == 0 && all_gemv(L.qkv, E, QD + 2 * KD);
+        if (!qkv_fused) { const size_t pt_ = prof_begin(PC_NORM); rk::rmsnorm_act(stream_, x, L.attn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending); prof_end(PC_NORM, pt_); }
         rk::Slices qkv_slices;
         {
             const size_t pt_ = prof_begin(PC_QKV);
-            if (L.qkv.size() == 1) {     // fused q, k, v: the rotation kernel can add the slices
+            if (qkv_fused) {
+                int col = 0;
+                for (const DevWeight & w : L.qkv) {
+                    rk::gemv_norm(stream_, w.w, x, L.attn_norm.as<float>(), h.eps, nullptr, T, qkv, QD + 2 * KD, col, rk::MM_STORE,
+                                  L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr);
+                    col += w.w.N;
+                }
+            } else if (L.qkv.size() == 1) {     // fused q, k, v: the rotation kernel can add the slices
                 qkv_slices = rk::matmul_deferred(stream_, L.qkv[0].w, act_e, T, qkv, QD + 2 * KD, 0, rk::MM_STORE,
                                                  L.qkv_bias.as<float>(), mm_ws_.ptr);
             } else {
@@ -1409,6 +1430,27 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
                            lora_mid_.as<float>());
         }
         prof_end(PC_OPROJ, pt_);
+        if (fuse && h.n_expert == 0 && pending.n == 0 && all_gemv(L.gate_up, E, 2 * F)) {
+            pt_ = prof_begin(PC_GATEUP);
+            int col = 0;
+            for (const DevWeight & w : L.gate_up) {
+                rk::gemv_norm(stream_, w.w, x, L.ffn_norm.as<float>(), h.eps, nullptr, T, gu, 2 * F, col, rk::MM_STORE, nullptr);
+                col += w.w.N;
+            }
+            prof_end(PC_GATEUP, pt_);
+            const int group = L.gate_up_interleaved ? 64 : F;
+            pt_ = prof_begin(PC_DOWN);
+            if (rk::gemv_can_weight(L.down.w, T) && L.down.w.K == F && L.down.w.N == E) {
+                rk::gemv_swiglu(stream_, L.down.w, gu, group, T, x, E, 0, rk::MM_ADD);
+                pending = rk::Slices();
+            } else {
+                const rk::Act act_f = act_for(act_f_x_, act_f_sums_, act_f_qx_, act_f_qsums_, F, {L.down.w.type}, false, &act_f_codes_);
+                rk::swiglu_act(stream_, gu, T, F, act_f, group);
+                pending = rk::matmul_deferred(stream_, L.down.w, act_f, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
+            }
+            prof_end(PC_DOWN, pt_);
+            continue;
+        }
         pt_ = prof_begin(PC_NORM);
         if (h.n_expert > 0) act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {L.router.w.type, L.gate_exps.w.type}, false);
         else act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {gt[0], gt[1], gt[2]}, ffn_lora, &act_e_codes_);
@@ -1463,9 +1505,14 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
     if (n_out > 0) {
         logits_.ensure((size_t)n_out * h.n_vocab * 4);
         const size_t pt_ = prof_begin(PC_HEAD);
-        rk::rmsnorm_act(stream_, x, out_norm_.as<float>(), E, h.eps, pk_.out_tok, n_out, act_o, pending);
-        rk::matmul(stream_, lm_head_.w, act_o, n_out, logits_.as<float>(), h.n_vocab, 0, rk::MM_STORE,
-                   out_bias_.as<float>(), mm_ws_.ptr);
+        if (fuse && pending.n == 0 && rk::gemv_can_weight(lm_head_.w, n_out) && lm_head_.w.K == E && lm_head_.w.N == h.n_vocab) {
+            rk::gemv_norm(stream_, lm_head_.w, x, out_norm_.as<float>(), h.eps, pk_.out_tok, n_out, logits_.as<float>(), h.n_vocab, 0,
+                          rk::MM_STORE, out_bias_.as<float>());
+        } else {
+            rk::rmsnorm_act(stream_, x, out_norm_.as<float>(), E, h.eps, pk_.out_tok, n_out, act_o, pending);
+            rk::matmul(stream_, lm_head_.w, act_o, n_out, logits_.as<float>(), h.n_vocab, 0, rk::MM_STORE,
+                       out_bias_.as<float>(), mm_ws_.ptr);
+        }
         prof_end(PC_HEAD, pt_);
     }
 }

@@ -33,7 +33,14 @@ struct GemvArgs {
     float * y;
     const float * bias;
     int K, N, T, ldy, col0, mode, n_tiles;
+    // SRC_NORM / SRC_SWIGLU: the f32 rows the Q8_K blocks are made from while they are staged
+    const float * xin;         // NORM: rows of K floats; SWIGLU: rows of 2 K floats, gate and up in alternating groups of 64
+    const float * norm_w;      // NORM: the RMSNorm weights
+    const int32_t * rows;      // NORM: row t is xin row rows[t] (null: t)
+    float eps;
+    int group;                 // SWIGLU: gate c at column (c / group) * 2 group + c % group, up c `group` columns further
 };
+enum : int { SRC_CODES = 0, SRC_NORM = 1, SRC_SWIGLU = 2 };
 
 // NT: tokens held (rows of the step beyond a.T read as zeros). PER: super-blocks of a tile per wave; a workgroup
 // has nw waves (PER 2: half the row's super-blocks; PER 4, rows wider than 32 super-blocks: 16), wave w takes
@@ -42,8 +49,13 @@ struct GemvArgs {
 // super-blocks at a time and requests the next two as soon as those registers are free - the first pair before the
 // step's rows are staged, the first pair of the next tile before the partial sums of this one meet in LDS (one
 // barrier per tile: the sums alternate between two buffers). Holding all four of a wide row at once was slower.
+// SRC: where the Q8_K blocks come from. SRC_CODES: the buffers a producer left. SRC_NORM: every workgroup makes them
+// itself from the residual rows - RMSNorm (the sum of squares in the order k_rmsnorm_act8 adds it, so a row of 4096
+// gives the same codes bit for bit) and the conversion, straight into LDS - which saves the step a launch of four to
+// five microseconds for about one of redundant work per workgroup, hidden behind the weight requests already in
+// flight. SRC_SWIGLU: likewise silu(gate) * up of the gate/up product's f32 rows. NT is exactly the token count then.
 // Dynamic LDS: codes NT * K bytes | block sums NT * K / 16 bytes | scales NT * K / 64 bytes | 2 * nw * NT * 16 floats.
-template <int NT, int PER>
+template <int NT, int PER, int SRC>
 __global__ __launch_bounds__(1024) void k_gemv_q4k(GemvArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
     const int K = a.K, nsb = K >> 8;
@@ -69,21 +81,86 @@ __global__ __launch_bounds__(1024) void k_gemv_q4k(GemvArgs a) {
             }
         }
     };
+    // The inputs of a thread's first eight values of row 0 are requested ahead of the weights: loads return in
+    // order, so a wait for anything requested after the weights would be a wait for the weights as well.
+    auto row_of = [&](int t) -> const float * {
+        if (SRC == SRC_NORM) return a.xin + (size_t)(a.rows ? a.rows[t] : t) * K;
+        return a.xin + (size_t)t * 2 * K;
+    };
+    // NORM: eight row values and their norm weights; SWIGLU: eight gate and eight up values
+    auto load_in = [&](const float * xr, int k, f4 (&in)[4]) {
+        if (SRC == SRC_NORM) {
+            in[0] = *(const f4 *)(xr + k); in[1] = *(const f4 *)(xr + k + 4);
+            in[2] = *(const f4 *)(a.norm_w + k); in[3] = *(const f4 *)(a.norm_w + k + 4);
+        } else {
+            const float * gp = xr + (size_t)(k / a.group) * 2 * a.group + k % a.group, * up = gp + a.group;
+            in[0] = *(const f4 *)gp; in[1] = *(const f4 *)(gp + 4); in[2] = *(const f4 *)up; in[3] = *(const f4 *)(up + 4);
+        }
+    };
+    f4 first[4];
+    if (SRC != SRC_CODES && tid * 8 < K) load_in(row_of(0), tid * 8, first);
     int tile = blockIdx.x;
     if (tile < a.n_tiles) request(tile, 0);
 
-    // stage the rows of the step: 16-byte words of codes, dwords of block sums, scales
-    for (int i = tid; i < NT * (K >> 4); i += nthreads) {
-        const int t = i / (K >> 4);
-        u4 v = {0u, 0u, 0u, 0u};
-        if (t < a.T) v = ((const u4 *)a.codes)[i];
-        ((u4 *)l_codes)[i] = v;
+    if (SRC == SRC_CODES) {
+        // stage the rows of the step: 16-byte words of codes, dwords of block sums, scales
+        for (int i = tid; i < NT * (K >> 4); i += nthreads) {
+            const int t = i / (K >> 4);
+            u4 v = {0u, 0u, 0u, 0u};
+            if (t < a.T) v = ((const u4 *)a.codes)[i];
+            ((u4 *)l_codes)[i] = v;
+        }
+        for (int i = tid; i < NT * (K >> 6); i += nthreads) {
+            const int t = i / (K >> 6);
+            ((uint32_t *)l_bsums)[i] = t < a.T ? ((const uint32_t *)a.bsums)[i] : 0u;
+        }
+        for (int i = tid; i < NT * nsb; i += nthreads) l_d[i] = i / nsb < a.T ? a.d[i] : 0.0f;
+    } else {
+        // make the blocks here: eight consecutive values per thread, the 32 threads of a block together (requantise8)
+        Act lout;
+        lout.K = K; lout.qc = l_codes; lout.qd = l_d; lout.qbs = l_bsums;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const float * xr = row_of(t);
+            float scale = 1.0f;
+            if (SRC == SRC_NORM) {
+                float ss = 0.0f;
+                for (int k = tid * 8; k < K; k += nthreads * 8) {
+                    f4 in[4];
+                    if (t == 0 && k == tid * 8) { in[0] = first[0]; in[1] = first[1]; }
+                    else { in[0] = *(const f4 *)(xr + k); in[1] = *(const f4 *)(xr + k + 4); }
+                    const f4 p = in[0], q4 = in[1];
+                    ss += p.x * p.x + p.y * p.y + p.z * p.z + p.w * p.w + q4.x * q4.x + q4.y * q4.y + q4.z * q4.z + q4.w * q4.w;
+                }
+                ss = wave_sum(ss);
+                if (lane == 0) l_red[wave] = ss;
+                __syncthreads();
+                float total = 0.0f;
+                for (int i = 0; i < nw; ++i) total += l_red[i];
+                scale = 1.0f / sqrtf(total / (float)K + a.eps);
+                __syncthreads();                   // l_red is written again for the next row and by the tiles
+            }
+            for (int k = tid * 8; k < K; k += nthreads * 8) {
+                f4 in[4];
+                if (t == 0 && k == tid * 8) { in[0] = first[0]; in[1] = first[1]; in[2] = first[2]; in[3] = first[3]; }
+                else load_in(xr, k, in);
+                float v[8], c[8];
+                if (SRC == SRC_NORM) {
+                    v[0] = (in[0].x * scale) * in[2].x; v[1] = (in[0].y * scale) * in[2].y;
+                    v[2] = (in[0].z * scale) * in[2].z; v[3] = (in[0].w * scale) * in[2].w;
+                    v[4] = (in[1].x * scale) * in[3].x; v[5] = (in[1].y * scale) * in[3].y;
+                    v[6] = (in[1].z * scale) * in[3].z; v[7] = (in[1].w * scale) * in[3].w;
+                } else {
+                    const float gv[8] = {in[0].x, in[0].y, in[0].z, in[0].w, in[1].x, in[1].y, in[1].z, in[1].w};
+                    const float uv[8] = {in[2].x, in[2].y, in[2].z, in[2].w, in[3].x, in[3].y, in[3].z, in[3].w};
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[i] = (gv[i] / (1.0f + __expf(-gv[i]))) * uv[i];
+                }
+                const float d = requantise8(v, AQ_Q8_K, c);
+                store_codes8(c, d, lout, t, k, tid & 3);
+            }
+        }
     }
-    for (int i = tid; i < NT * (K >> 6); i += nthreads) {
-        const int t = i / (K >> 6);
-        ((uint32_t *)l_bsums)[i] = t < a.T ? ((const uint32_t *)a.bsums)[i] : 0u;
-    }
-    for (int i = tid; i < NT * nsb; i += nthreads) l_d[i] = i / nsb < a.T ? a.d[i] : 0.0f;
     __syncthreads();
 
     float acc[NT];
@@ -164,20 +241,19 @@ static size_t gemv_lds_bytes(int NT, int NW, int K) {
     return (size_t)NT * K + (size_t)NT * (K >> 4) + (size_t)NT * (K >> 8) * 4 + (size_t)2 * NW * NT * 16 * 4;
 }
 
+bool gemv_can_weight(const Weight & w, int T);
 bool gemv_can(const Weight & w, const Act & x, int T) {
-    return w.type == WT_Q4_K && w.packed && x.qc && x.qd && x.qbs && T >= 1 && T <= g_gemv_max_t && T <= GEMV_MAX_T
-        && w.K % 256 == 0 && w.N % 16 == 0 && w.K > 0 && w.N > 0 && x.K == w.K
-        && w.K <= 256 * 4 * 16 && gemv_lds_bytes(GEMV_MAX_T, 16, w.K) <= kGemvMaxLds;
+    return x.qc && x.qd && x.qbs && x.K == w.K && gemv_can_weight(w, T);
 }
 
-template <int NT, int PER>
+template <int NT, int PER, int SRC>
 static void launch_gemv(hipStream_t s, const GemvArgs & a) {
     const int nsb = a.K / 256;
     const int nw = PER == 2 ? (nsb + 1) / 2 : 16;
     const size_t lds = gemv_lds_bytes(NT, nw, a.K);
     static bool once = false;
     if (!once) {
-        HIP_OK(hipFuncSetAttribute((const void *)k_gemv_q4k<NT, PER>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvMaxLds));
+        HIP_OK(hipFuncSetAttribute((const void *)k_gemv_q4k<NT, PER, SRC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvMaxLds));
         once = true;
     }
     // a workgroup stages the step's rows once and then walks tiles: as many workgroups as the chip holds at
@@ -185,22 +261,56 @@ static void launch_gemv(hipStream_t s, const GemvArgs & a) {
     const int capacity = 256 * std::max(1, 2048 / (nw * 64));
     const int turns = (a.n_tiles + capacity - 1) / capacity;
     const unsigned grid = (unsigned)((a.n_tiles + turns - 1) / turns);
-    hipLaunchKernelGGL((k_gemv_q4k<NT, PER>), dim3(grid), dim3(nw * 64), lds, s, a);
+    hipLaunchKernelGGL((k_gemv_q4k<NT, PER, SRC>), dim3(grid), dim3(nw * 64), lds, s, a);
+}
+
+template <int SRC>
+static void launch_gemv_src(hipStream_t s, const GemvArgs & a) {
+    static_assert(GEMV_MAX_T == 2, "one instantiation per token count");
+    // two super-blocks of a tile per wave while sixteen waves cover the row, four beyond
+    const bool two = a.K <= 256 * 2 * 16;
+    if (a.T == 1) { if (two) launch_gemv<1, 2, SRC>(s, a); else launch_gemv<1, 4, SRC>(s, a); }
+    else { if (two) launch_gemv<2, 2, SRC>(s, a); else launch_gemv<2, 4, SRC>(s, a); }
+    check_launch("gemv");
+}
+
+static GemvArgs gemv_args(const Weight & w, int T, float * y, int ldy, int col0, int mode, const float * bias) {
+    if (mode != MM_STORE && mode != MM_ADD) throw std::runtime_error("gemv: stores or adds");
+    if (col0 < 0 || col0 + w.N > ldy) throw std::runtime_error("gemv: the outputs do not fit the row");
+    GemvArgs a {};
+    a.w = w.packed; a.y = y; a.bias = bias;
+    a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode; a.n_tiles = w.N / 16;
+    return a;
 }
 
 void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias) {
     if (!gemv_can(w, x, T)) throw std::runtime_error("gemv: needs Q4_K tiles, Q8_K code buffers and at most " + std::to_string(GEMV_MAX_T) + " tokens");
-    if (mode != MM_STORE && mode != MM_ADD) throw std::runtime_error("gemv: stores or adds");
-    if (col0 < 0 || col0 + w.N > ldy) throw std::runtime_error("gemv: the outputs do not fit the row");
-    GemvArgs a {};
-    a.w = w.packed; a.codes = x.qc; a.d = x.qd; a.bsums = x.qbs; a.y = y; a.bias = bias;
-    a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode; a.n_tiles = w.N / 16;
-    // two super-blocks of a tile per wave while sixteen waves cover the row, four beyond
-    const bool two = w.K <= 256 * 2 * 16;
-    static_assert(GEMV_MAX_T == 2, "one instantiation per token count");
-    if (T == 1) { if (two) launch_gemv<1, 2>(s, a); else launch_gemv<1, 4>(s, a); }
-    else { if (two) launch_gemv<2, 2>(s, a); else launch_gemv<2, 4>(s, a); }
-    check_launch("gemv");
+    GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
+    a.codes = x.qc; a.d = x.qd; a.bsums = x.qbs;
+    launch_gemv_src<SRC_CODES>(s, a);
+}
+
+bool gemv_can_weight(const Weight & w, int T) {
+    return w.type == WT_Q4_K && w.packed && T >= 1 && T <= g_gemv_max_t && T <= GEMV_MAX_T
+        && w.K % 256 == 0 && w.N % 16 == 0 && w.K > 0 && w.N > 0
+        && w.K <= 256 * 4 * 16 && gemv_lds_bytes(GEMV_MAX_T, 16, w.K) <= kGemvMaxLds;
+}
+
+void gemv_norm(hipStream_t s, const Weight & w, const float * x, const float * norm_w, float eps, const int32_t * rows, int T,
+               float * y, int ldy, int col0, int mode, const float * bias) {
+    if (!gemv_can_weight(w, T) || !x || !norm_w) throw std::runtime_error("gemv_norm: needs Q4_K tiles, the rows and the norm weights");
+    GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
+    a.xin = x; a.norm_w = norm_w; a.rows = rows; a.eps = eps;
+    launch_gemv_src<SRC_NORM>(s, a);
+}
+
+void gemv_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, int T, float * y, int ldy, int col0, int mode) {
+    if (group <= 0) group = w.K;
+    if (!gemv_can_weight(w, T) || !gu || w.K % group != 0 || group % 8 != 0)
+        throw std::runtime_error("gemv_swiglu: needs Q4_K tiles and gate / up rows in groups that divide the width");
+    GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, nullptr);
+    a.xin = gu; a.group = group;
+    launch_gemv_src<SRC_SWIGLU>(s, a);
 }
 
 }  // namespace rk

@@ -142,6 +142,14 @@ size_t matmul_workspace_bytes();
 constexpr int GEMV_MAX_T = 2;     // beyond two tokens the tile kernels are as fast
 bool gemv_can(const Weight & w, const Act & x, int T);
 void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias);
+// The weight's side of gemv_can. With it the same product can take its rows as f32 and make the Q8_K blocks while
+// it stages them, one launch instead of two: gemv_norm from the residual rows (x row rows[t], or t; RMSNorm with
+// norm_w and eps as rmsnorm_act computes it, then the conversion), gemv_swiglu from the f32 rows of a gate/up product
+// (gu rows of 2 K floats laid out as swiglu_act reads them with `group`).
+bool gemv_can_weight(const Weight & w, int T);
+void gemv_norm(hipStream_t s, const Weight & w, const float * x, const float * norm_w, float eps, const int32_t * rows, int T,
+               float * y, int ldy, int col0, int mode, const float * bias);
+void gemv_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, int T, float * y, int ldy, int col0, int mode);
 extern int g_gemv_max_t;       // steps of at most this many tokens take the kernel (default GEMV_MAX_T; 0 switches it off)
 extern int g_mm_debug;         // timing experiments (see MMArgs::debug)
 extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic

@@ -139,7 +139,7 @@ STEP_SYMBOLS = [
     "retro_grammar_gbnf", "retro_grammar_free", "retro_last_error",
 ]
 KERNEL_SYMBOLS = [
-    "retro_kernel_matmul", "retro_kernel_matmul_time", "retro_kernel_stream_time", "retro_kernel_sample_prepare", "retro_kernel_sample_greedy_noalloc", "retro_kernel_sample_greedy_noalloc_max_rows", "retro_kernel_page_size", "retro_kernel_max_topk",
+    "retro_kernel_matmul", "retro_kernel_gemv_fused", "retro_kernel_matmul_time", "retro_kernel_stream_time", "retro_kernel_sample_prepare", "retro_kernel_sample_greedy_noalloc", "retro_kernel_sample_greedy_noalloc_max_rows", "retro_kernel_page_size", "retro_kernel_max_topk",
     "retro_engine_debug_logits", "retro_engine_debug_kv", "retro_engine_debug_pack", "retro_engine_debug_pages",
     "retro_engine_debug_profile", "retro_engine_debug_profile_categories", "retro_engine_debug_profile_read",
 ]
@@ -222,6 +222,9 @@ def load_library() -> C.CDLL:
     lib.retro_kernel_sample_greedy_noalloc.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
                                                        C.c_void_p, C.c_void_p]
     lib.retro_kernel_sample_greedy_noalloc_max_rows.restype = C.c_int32
+    lib.retro_kernel_gemv_fused.argtypes = [C.c_int32, _u8p, C.c_int64, C.c_int64, _f32p, _f32p, C.c_float, C.c_int32, C.c_int32,
+                                            _f32p, _f32p]
+    lib.retro_kernel_gemv_fused.restype = C.c_int
     lib.retro_kernel_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,
                                              C.c_int32, C.c_int32, C.POINTER(C.c_double)]
     lib.retro_kernel_stream_time.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_double)]
@@ -887,6 +890,26 @@ def kernel_matmul(ggml_type: int, raw: np.ndarray, n_rows: int, k: int, x: np.nd
     if s != 0:
         _raise(s)
     return y
+
+
+def kernel_gemv_fused(kind: int, raw: np.ndarray, n_rows: int, k: int, x: np.ndarray, norm_w: np.ndarray | None = None,
+                      eps: float = 1e-5, group: int = 0):
+    """The integer matrix-vector kernel with RMSNorm (kind 1) or SwiGLU (kind 2) fused into its staging, and the same
+    product as producer launch plus kernel: returns (fused, unfused), each [tokens][n_rows]."""
+    lib = load_library()
+    raw = np.ascontiguousarray(raw, np.uint8)
+    x = np.ascontiguousarray(x, np.float32)
+    T = x.shape[0]
+    w = None
+    if norm_w is not None:
+        norm_w = np.ascontiguousarray(norm_w, np.float32)
+        w = norm_w.ctypes.data_as(_f32p)
+    fused, unfused = np.zeros((T, n_rows), np.float32), np.zeros((T, n_rows), np.float32)
+    s = lib.retro_kernel_gemv_fused(kind, raw.ctypes.data_as(_u8p), n_rows, k, x.ctypes.data_as(_f32p), w, eps, T, group,
+                                    fused.ctypes.data_as(_f32p), unfused.ctypes.data_as(_f32p))
+    if s != 0:
+        _raise(s)
+    return fused, unfused
 
 
 def kernel_matmul_time(ggml_type: int, n_rows: int, k: int, n_tokens: int, mode: int = 2, iters: int = 50,

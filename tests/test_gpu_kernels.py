@@ -200,6 +200,44 @@ def test_integer_matvec_exact_on_integer_data_and_refusals():
         E.kernel_matmul(gw.GGML_Q8_0, q8, 16, 256, x[:1, :256], use_tiles=2, ggml_activations=True, integer=True)
 
 
+@pytest.mark.parametrize("kind", [1, 2])
+@pytest.mark.parametrize("n,k,T", [(64, 4096, 1), (64, 4096, 2), (32, 512, 1), (48, 1024, 2), (32, 14336, 1), (16, 14336, 2),
+                                   (16, 8448, 2), (32, 2048, 1)])
+def test_integer_matvec_with_its_producer_fused(kind, n, k, T):
+    # The Q8_K blocks made by the kernel itself while it stages them (RMSNorm of residual rows, or SwiGLU of a gate/up
+    # product) against the producer's own launch followed by the kernel, and against the CPU: the norm / SiLU in
+    # float64, the conversion by the oracle, the decoded weights. A row of 4096 is normalised in the very order the
+    # standalone kernel uses, so there the two paths agree bit for bit; elsewhere the sum of squares is added in
+    # another order and a code on a rounding boundary may differ.
+    print("case", kind, n, k, T, flush=True)
+    t = gw.GGML_Q4_K
+    raw, dense = _weights(t, n, k, seed=n + k + T + kind)
+    rng = np.random.default_rng(k + T)
+    eps = 1e-5
+    if kind == 1:
+        x = (rng.standard_normal((T, k)) * 3.0).astype(np.float32)
+        w = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+        fused, unfused = E.kernel_gemv_fused(1, raw, n, k, x, norm_w=w, eps=eps)
+        x64 = x.astype(np.float64)
+        rows = x64 / np.sqrt((x64 * x64).mean(-1, keepdims=True) + eps) * w
+    else:
+        group = 64 if k % 64 == 0 else 0
+        gu = rng.standard_normal((T, 2 * k)).astype(np.float32)
+        fused, unfused = E.kernel_gemv_fused(2, raw, n, k, gu, group=group)
+        g64 = gu.astype(np.float64).reshape(T, k // 64, 2, 64)
+        rows = (g64[:, :, 0] / (1 + np.exp(-g64[:, :, 0])) * g64[:, :, 1]).reshape(T, k)
+    want = _ref(t, dense, rows.astype(np.float32), True)
+    scale = np.abs(want).max()
+    # a code that flips moves one product by d_x * |w|: allow a few of them on top of the float rounding
+    flip = np.abs(rows).max() / 127.0 * np.abs(dense).max()
+    assert np.abs(unfused - want).max() <= 2e-5 * scale + 8 * flip
+    assert np.abs(fused - want).max() <= 2e-5 * scale + 8 * flip
+    if kind == 2 or k == 4096:
+        assert np.array_equal(fused, unfused)
+    else:
+        assert np.abs(fused - unfused).max() <= 8 * flip + 1e-6
+
+
 def test_q6k_tiles_are_exact_for_every_code_and_scale():
     # Random bytes: every six-bit code, every i8 scale (-128 and 127 included, whose products with a code
     # are not all f16 numbers) in every position of the tile. With d = 1 and small-integer activations all

@@ -142,10 +142,12 @@ def test_ggml_arithmetic_follows_the_oracle_as_closely_as_its_rounding_allows(mo
 @pytest.mark.parametrize("key", ["llama-q4k", "llama-q4k-hd128", "llama-q4k-m-1024"])
 def test_small_steps_under_the_ggml_arithmetic_take_the_integer_kernel(models, key, monkeypatch):
     """Steps of one or two tokens under RETRO_ACTIVATIONS=ggml multiply their Q4_K matrices by integer products of
-    the stored codes with the rows' Q8_K codes (Q6_K matrices of the same model stay on the tile kernels). Against
-    the oracle's ggml arithmetic such a step must drift no further than the same step through the tile kernels
-    (RETRO_GEMV_MAX_T=0) does - both differ from it by float rounding that later conversions amplify - and the two
-    engines must stay as close to each other as either is to the oracle."""
+    the stored codes with the rows' Q8_K codes (Q6_K matrices of the same model stay on the tile kernels), and where
+    every consumer of a row is that kernel it makes the codes itself from the residual or gate/up rows (the default;
+    RETRO_GEMV_FUSE=0 keeps the producers' own launches). Against the oracle's ggml arithmetic such a step must
+    drift no further than the same step through the tile kernels (RETRO_GEMV_MAX_T=0) does - all differ from it by
+    float rounding that later conversions amplify - and the engines must stay as close to each other as either is
+    to the oracle."""
     print("model", key, flush=True)
     monkeypatch.setenv("RETRO_ACTIVATIONS", "ggml")
     cfg = E.EngineConfig(n_ctx=2048, n_seq_max=8, n_batch=256, n_ubatch=256)
@@ -156,11 +158,12 @@ def test_small_steps_under_the_ggml_arithmetic_take_the_integer_kernel(models, k
     plans = [[0, 1, 2, 3], [1, 3], [2], [0, 1, 3], [0], [0, 1, 2, 3]]      # the slots of each decode step
     feeds = [[int(t) for t in rng.integers(0, m.n_vocab, len(p))] for p in plans]
     runs = {}
-    for name, limit in (("integer", None), ("tiles", "0")):
-        if limit is None:
-            monkeypatch.delenv("RETRO_GEMV_MAX_T", raising=False)
-        else:
-            monkeypatch.setenv("RETRO_GEMV_MAX_T", limit)
+    for name, limit, fuse in (("integer", None, None), ("unfused", None, "0"), ("tiles", "0", None)):
+        for var, value in (("RETRO_GEMV_MAX_T", limit), ("RETRO_GEMV_FUSE", fuse)):
+            if value is None:
+                monkeypatch.delenv(var, raising=False)
+            else:
+                monkeypatch.setenv(var, value)
         eng = E.Engine(models[key], cfg)
         ctx = oracle.Context(m, 8, activations="ggml")
         run_both(eng, ctx, [(i, i, p, 0, True) for i, p in enumerate(prompts)])
@@ -180,8 +183,13 @@ def test_small_steps_under_the_ggml_arithmetic_take_the_integer_kernel(models, k
         _, drift_i = logit_errors(gi, want)
         _, drift_t = logit_errors(gt, want)
         _, apart = logit_errors(gi, gt)
-        print("step of %d rows: integer %.2e, tiles %.2e from the oracle, %.2e apart" % (len(plan), drift_i, drift_t, apart), flush=True)
+        gu, _ = runs["unfused"][i]
+        _, drift_u = logit_errors(gu, want)
+        _, apart_u = logit_errors(gi, gu)
+        print("step of %d rows: integer %.2e, its producers unfused %.2e, tiles %.2e from the oracle; %.2e and %.2e apart"
+              % (len(plan), drift_i, drift_u, drift_t, apart_u, apart), flush=True)
         assert drift_i <= 2 * drift_t + 1e-4 and apart <= 2 * max(drift_i, drift_t) + 1e-4, (i, drift_i, drift_t, apart)
+        assert drift_u <= 2 * drift_t + 1e-4 and apart_u <= 2 * max(drift_i, drift_u) + 1e-4, (i, drift_u, apart_u)
         assert drift_i <= 5e-2
 
 

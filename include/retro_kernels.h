@@ -22,24 +22,25 @@ extern "C" {
  * f16 hi/lo pairs) or, with bit 8 (0x100) of use_tiles set, x as ggml's CPU
  * matmul converts it for this weight type: Q8_K codes times their scale for
  * Q4_K, Q8_0 ones for Q8_0 and MXFP4, f16 / bf16 rounding for F16 / BF16.
- * With bit 9 (0x200) as well (Q4_K tiles, at most two tokens) the conversion
- * leaves the Q8_K blocks themselves and the integer matrix-vector kernel of very
+ * With bit 9 (0x200) as well (Q4_K or Q8_0 tiles, at most two tokens) the conversion
+ * leaves the converted blocks themselves and the integer matrix-vector kernel of very
  * small steps multiplies the codes; anything else with that bit is refused.
  * y is [n_tokens][n_rows] and is read first when accumulate is set. */
 int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x,
                         int32_t n_tokens, int32_t use_tiles, const float * bias, int32_t accumulate, float * y);
 
+/* The integer matrix-vector kernel with the producer of its rows fused into its staging, beside the same product
+ * as two launches. kind 1: x is [n_tokens][k] residual rows, the rows multiplied are their RMSNorm (norm_w, eps)
+ * converted as ggml converts them for the weight type; kind 2: x is [n_tokens][2 k] gate and up values in alternating
+ * groups of `group` columns (0: side by side), the rows are silu(gate) * up converted likewise. raw: n_rows rows of
+ * k, Q4_K (the rows become Q8_K blocks) or Q8_0 (Q8_0 blocks). Both results are [n_tokens][n_rows]; at most two
+ * tokens. */
+int retro_kernel_gemv_fused(int32_t kind, int32_t type, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, const float * norm_w,
+                            float eps, int32_t n_tokens, int32_t group, float * y_fused, float * y_unfused);
+
 /* Per logits row: argmax (lowest id on ties), max, sum exp(double(l) - max),
  * and the k[r] best (id, logit) pairs in (logit desc, id asc) order, written
  * to out_top_*[r * retro_kernel_max_topk() + j]. */
-/* The integer matrix-vector kernel with the producer of its rows fused into its staging, beside the same product
- * as two launches. kind 1: x is [n_tokens][k] residual rows, the rows multiplied are their RMSNorm (norm_w, eps)
- * converted to Q8_K; kind 2: x is [n_tokens][2 k] gate and up values in alternating groups of `group` columns
- * (0: side by side), the rows are silu(gate) * up converted to Q8_K. raw: n_rows Q4_K rows of k. Both results are
- * [n_tokens][n_rows]; at most two tokens. */
-int retro_kernel_gemv_fused(int32_t kind, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, const float * norm_w,
-                            float eps, int32_t n_tokens, int32_t group, float * y_fused, float * y_unfused);
-
 int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_vocab, const int32_t * k,
                                 int32_t * out_argmax, float * out_max, double * out_sum_exp,
                                 int32_t * out_top_ids, float * out_top_logits);
@@ -75,8 +76,8 @@ int32_t retro_kernel_sample_greedy_noalloc_max_rows(void);
  * (0 = normal). type is Q4_K, Q5_K, Q6_K or Q8_0 (Q5_K and Q6_K in modes 2 and
  * 3 only), n_rows a multiple of 16 and k of 256: anything else is refused
  * before a buffer is allocated. Mode 4 times the integer matrix-vector kernel
- * of very small steps under the ggml arithmetic instead (Q4_K, at most two
- * tokens, pseudo-random Q8_K blocks). */
+ * of very small steps under the ggml arithmetic instead (Q4_K or Q8_0, at most
+ * two tokens, pseudo-random activation blocks). */
 int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,
                              int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us);
 

@@ -85,8 +85,8 @@ __device__ __forceinline__ Q4KScales q4k_scales(const u4 & hdr) {
 //         from zero), value = f16(d) * code.
 //   Q8_K: `max` = the first value of largest magnitude, iscale = -127 / max,
 //         code = min(127, rint(iscale * v)) (half to even), value = code / iscale.
-// With `codes` (Q8_K only) the integer codes are returned as well, and the block scale 1 / iscale is the
-// function's value (0 for a block of zeros).
+// With `codes` the integer codes are returned as well; the function's value is the block scale (Q8_K: 1 / iscale,
+// 0 for a block of zeros; Q8_0: d rounded to f16).
 __device__ __forceinline__ float requantise8(float (&v)[8], int quant, float * codes = nullptr) {
     float amax = 0.0f, first = 0.0f;
 #pragma unroll
@@ -101,7 +101,11 @@ __device__ __forceinline__ float requantise8(float (&v)[8], int quant, float * c
         const float id = d != 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
         const float dh = (float)(_Float16)d;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = __fmul_rn(dh, roundf(__fmul_rn(v[i], id)));
+        for (int i = 0; i < 8; ++i) {
+            const float c = roundf(__fmul_rn(v[i], id));
+            if (codes) codes[i] = c;
+            v[i] = __fmul_rn(dh, c);
+        }
         return dh;
     }
     float gmax = amax;
@@ -132,21 +136,27 @@ __device__ __forceinline__ float requantise8(float (&v)[8], int quant, float * c
     return d;
 }
 
-// The Q8_K codes of eight consecutive values (k a multiple of 8) into the buffers of the integer
-// matrix-vector kernel (Act::qc, qd, qbs): 8 bytes in the order of act_code_pos, the sum of a 32-wide
-// block from its four lanes, the block scale from the lane that holds the block's first values.
+// The codes of eight consecutive values (k a multiple of 8) into the buffers of the integer matrix-vector kernel
+// (Act::qc, qd, qbs). Q8_K: 8 bytes in the order of act_code_pos, the sum of a 32-wide block from its four lanes, the
+// block scale from the lane that holds the block's first values. Q8_0: 8 bytes in element order, the scale of the
+// 32-wide block from its first lane.
 __device__ __forceinline__ void store_codes8(const float (&c)[8], float d, const Act & out, int tok, int k, int lane_in_block) {
     uint32_t w0 = 0, w1 = 0;
     int sum = 0;
+    const bool natural = out.quant == AQ_Q8_0;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int q = (int)c[i];
         sum += q;
         const uint32_t byte = (uint32_t)q & 0xffu;
-        const int pos = act_code_pos(i);
+        const int pos = natural ? i : act_code_pos(i);
         if (pos < 4) w0 |= byte << (8 * pos); else w1 |= byte << (8 * (pos - 4));
     }
     *(uint2 *)(out.qc + (size_t)tok * out.K + k) = make_uint2(w0, w1);
+    if (natural) {
+        if (lane_in_block == 0) out.qd[(size_t)tok * (out.K >> 5) + (k >> 5)] = d;
+        return;
+    }
     sum += __shfl_xor(sum, 1, 64);
     sum += __shfl_xor(sum, 2, 64);
     if (lane_in_block == 0) out.qbs[(size_t)tok * (out.K >> 5) + (k >> 5)] = (int16_t)sum;

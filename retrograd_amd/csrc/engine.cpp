@@ -476,7 +476,7 @@ void Engine::build_buffers() {
         auto codes = [&](ActCodes & c, int K) {
             if (K % 256 != 0) return;          // no Q8_K conversion of such rows
             c.codes.alloc((size_t)rk::GEMV_MAX_T * K);
-            c.d.alloc((size_t)rk::GEMV_MAX_T * (K / 256) * 4);
+            c.d.alloc((size_t)rk::GEMV_MAX_T * (K / 32) * 4);          // one scale per 32 (Q8_0) or per 256 (Q8_K)
             c.bsums.alloc((size_t)rk::GEMV_MAX_T * (K / 32) * 2);
         };
         codes(act_e_codes_, E);
@@ -1338,7 +1338,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         }
         if (plain) { a.x = x.as<__half>(); a.sums = K % 32 == 0 ? sums.as<__half>() : nullptr; }
         if (a.quant != rk::AQ_NONE) { a.qx = qx.as<__half>(); a.qsums = qsums.as<__half>(); }
-        if (a.quant == rk::AQ_Q8_K && small_step && codes && codes->codes.ptr) {
+        if (a.quant != rk::AQ_NONE && small_step && codes && codes->codes.ptr) {
             a.qc = codes->codes.as<int8_t>(); a.qd = codes->d.as<float>(); a.qbs = codes->bsums.as<int16_t>();
         }
         return a;

@@ -302,7 +302,7 @@ private:
     DevBuf act_o_x_, act_o_sums_;       // output rows, n_embd wide
     // the same rows after the conversion ggml's CPU matmul applies for a quantised weight
     DevBuf act_e_qx_, act_e_qsums_, act_q_qx_, act_q_qsums_, act_f_qx_, act_f_qsums_, act_o_qx_, act_o_qsums_;
-    // ggml arithmetic only: the Q8_K blocks themselves (codes, scales, block sums) of steps of at most
+    // ggml arithmetic only: the Q8_K / Q8_0 blocks themselves (codes, scales, block sums) of steps of at most
     // rk::GEMV_MAX_T tokens, for the integer matrix-vector kernel
     struct ActCodes { DevBuf codes, d, bsums; };
     ActCodes act_e_codes_, act_q_codes_, act_f_codes_, act_o_codes_;

@@ -1,24 +1,29 @@
 // The integer matrix-vector kernel of very small steps under ggml's arithmetic (gfx950, wave64).
 //
-// A step of one or two tokens reads every weight once and has nothing to amortise the conversion of the
-// 4-bit codes to f16 matrix operands over: the tile kernels then spend their time issuing vector instructions,
-// not waiting for memory. When the activations are Q8_K blocks anyway (what ggml's CPU dot product of a Q4_K
-// row multiplies, ggml-quants.c ggml_vec_dot_q4_K_q8_K), the products can stay integers: one mask (and one
-// shift) turns a dword of eight nibbles into two dwords of four bytes, and a four-way integer dot product
-// multiplies each with four activation codes - about a quarter of the vector instructions per weight.
+// A step of one or two tokens reads every weight once and has nothing to amortise the conversion of the stored
+// codes to f16 matrix operands over: the tile kernels then spend their time issuing vector instructions, not
+// waiting for memory. When the activations are Q8_K / Q8_0 blocks anyway (what ggml's CPU dot products multiply:
+// ggml-quants.c ggml_vec_dot_q4_K_q8_K, ggml_vec_dot_q8_0_q8_0), the products can stay integers and a four-way
+// integer dot product (v_dot4c_i32_i8) multiplies four weight codes with four activation codes at a time.
 //
+// Q4_K (activations Q8_K):
 //   sum_k w[n][k] x[k] = sum over super-blocks of
 //       d_x * ( d_w * sum_s sc_s * (sum_{k in s} q_k c_k)  -  dmin_w * sum_s m_s * bsum_s )
-//
 // with q the 4-bit codes, c the activation codes, sc / m the 6-bit scales and mins of the eight sub-blocks s,
 // bsum_s the sum of the activation codes of s: all integer up to the two float factors per super-block, exactly
 // the quantities ggml's kernel forms (its order of the float additions is one of several, per instruction set).
-//
 // The matrix is the Q4_K tile layout of the tile kernels (16 rows x 256 columns, 16-byte row headers, then two
 // 1 KiB loads in which lane (r = l % 16, g = l / 16) of load h holds, as dword j, the eight nibbles of columns
 // 32 (4h + j) + 8g .. + 8 of row r, in the order e0 e2 e4 e6 e1 e3 e5 e7). Masking a dword with 0x0F0F0F0F gives
 // the bytes e0 e4 e1 e5, the same after a shift by four e2 e6 e3 e7: the activation codes are stored in that
-// byte order (act_code_pos), so no lane ever permutes anything.
+// byte order (act_code_pos), so no lane ever permutes anything: about a quarter of the tile kernels' vector
+// instructions per weight.
+//
+// Q8_0 (activations Q8_0):
+//   sum_k w[n][k] x[k] = sum over blocks of 32 of  (d_w d_x) * sum_{k in block} q_k c_k
+// The Q8_0 tile (16 x 8 f16 scales, then four 1 KiB loads in which lane (r, g) of load q holds columns 8g .. 8g + 8
+// of blocks 2q and 2q + 1 of row r, bytes in element order) needs no unpacking at all; the activation codes stay in
+// element order.
 #include "dev_common.hpp"
 
 namespace rk {
@@ -26,15 +31,15 @@ namespace rk {
 int g_gemv_max_t = GEMV_MAX_T;
 
 struct GemvArgs {
-    const uint8_t * w;         // Q4_K tiles
+    const uint8_t * w;         // tiles
     const int8_t * codes;      // [T][K]
-    const float * d;           // [T][K / 256]
-    const int16_t * bsums;     // [T][K / 32]
+    const float * d;           // [T][K / 256] (Q8_K) or [T][K / 32] (Q8_0)
+    const int16_t * bsums;     // [T][K / 32] (Q8_K only)
     float * y;
     const float * bias;
     int K, N, T, ldy, col0, mode, n_tiles;
-    // SRC_NORM / SRC_SWIGLU: the f32 rows the Q8_K blocks are made from while they are staged
-    const float * xin;         // NORM: rows of K floats; SWIGLU: rows of 2 K floats, gate and up in alternating groups of 64
+    // SRC_NORM / SRC_SWIGLU: the f32 rows the blocks are made from while they are staged
+    const float * xin;         // NORM: rows of K floats; SWIGLU: rows of 2 K floats, gate and up in alternating groups
     const float * norm_w;      // NORM: the RMSNorm weights
     const int32_t * rows;      // NORM: row t is xin row rows[t] (null: t)
     float eps;
@@ -42,42 +47,50 @@ struct GemvArgs {
 };
 enum : int { SRC_CODES = 0, SRC_NORM = 1, SRC_SWIGLU = 2 };
 
-// NT: tokens held (rows of the step beyond a.T read as zeros). PER: super-blocks of a tile per wave; a workgroup
-// has nw waves (PER 2: half the row's super-blocks; PER 4, rows wider than 32 super-blocks: 16), wave w takes
-// super-blocks w + u * nw. A matrix read once has
-// nothing to hide the memory latency behind, so the loads are issued as early as they can be: a wave holds two
-// super-blocks at a time and requests the next two as soon as those registers are free - the first pair before the
-// step's rows are staged, the first pair of the next tile before the partial sums of this one meet in LDS (one
-// barrier per tile: the sums alternate between two buffers). Holding all four of a wide row at once was slower.
-// SRC: where the Q8_K blocks come from. SRC_CODES: the buffers a producer left. SRC_NORM: every workgroup makes them
-// itself from the residual rows - RMSNorm (the sum of squares in the order k_rmsnorm_act8 adds it, so a row of 4096
-// gives the same codes bit for bit) and the conversion, straight into LDS - which saves the step a launch of four to
-// five microseconds for about one of redundant work per workgroup, hidden behind the weight requests already in
-// flight. SRC_SWIGLU: likewise silu(gate) * up of the gate/up product's f32 rows. NT is exactly the token count then.
-// Dynamic LDS: codes NT * K bytes | block sums NT * K / 16 bytes | scales NT * K / 64 bytes | 2 * nw * NT * 16 floats.
-template <int NT, int PER, int SRC>
-__global__ __launch_bounds__(1024) void k_gemv_q4k(GemvArgs a) {
+template <int WT> struct GemvTile;
+template <> struct GemvTile<WT_Q4_K> { static constexpr int BYTES = 2304, LOADS = 2, QUANT = AQ_Q8_K; };
+template <> struct GemvTile<WT_Q8_0> { static constexpr int BYTES = 4352, LOADS = 4, QUANT = AQ_Q8_0; };
+
+// WT: the weight type. NT: tokens held (rows of the step beyond a.T read as zeros). PER: super-blocks of a tile per
+// wave; a workgroup has nw waves (PER 2: half the row's super-blocks; wider rows: 16), wave w takes super-blocks
+// w + u * nw. A matrix read once has nothing to hide the memory latency behind, so the loads are issued as early as
+// they can be: a wave holds two super-blocks at a time and requests the next two as soon as those registers are
+// free - the first pair before the step's rows are staged, the first pair of the next tile before the partial sums
+// of this one meet in LDS (one barrier per tile: the sums alternate between two buffers). Holding all four of a wide
+// row at once was slower.
+// SRC: where the activation blocks come from. SRC_CODES: the buffers a producer left. SRC_NORM: every workgroup makes
+// them itself from the residual rows - RMSNorm (the sum of squares in the order k_rmsnorm_act8 adds it, so a row of
+// 4096 gives the same codes bit for bit) and the conversion, straight into LDS - which saves the step a launch of
+// four to five microseconds for about one and a half of redundant work per workgroup. SRC_SWIGLU: likewise
+// silu(gate) * up of the gate/up product's f32 rows. NT is exactly the token count then.
+// Dynamic LDS: codes NT * K bytes | scales NT * nd floats (nd = K / 256 or K / 32) | Q8_K: block sums NT * K / 16
+// bytes | 2 * nw * NT * 16 floats.
+template <int WT, int NT, int PER, int SRC>
+__global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
+    using Tile = GemvTile<WT>;
+    constexpr bool Q4 = WT == WT_Q4_K;
     extern __shared__ __align__(16) uint8_t lds[];
     const int K = a.K, nsb = K >> 8;
+    const int nd = Q4 ? nsb : (K >> 5);
     const int nthreads = blockDim.x, nw = nthreads >> 6;
     int8_t * l_codes = (int8_t *)lds;
-    int16_t * l_bsums = (int16_t *)(lds + (size_t)NT * K);
-    float * l_d = (float *)(lds + (size_t)NT * K + (size_t)NT * (K >> 4));
-    float * l_red = l_d + NT * nsb;
+    float * l_d = (float *)(lds + (size_t)NT * K);
+    int16_t * l_bsums = (int16_t *)(l_d + NT * nd);
+    float * l_red = Q4 ? (float *)((uint8_t *)l_bsums + (size_t)NT * (K >> 4)) : (float *)l_bsums;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
 
     // two super-blocks are held at a time: u0 and u0 + 1 of the wave's PER
-    u4 hdr[2], q[2][2];
+    u4 hdr[2], q[2][Tile::LOADS];
     auto request = [&](int tile, int u0) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int sb = wave + (u0 + u) * nw;
             if (sb < nsb) {
-                const uint8_t * tp = a.w + ((size_t)tile * nsb + sb) * 2304;
+                const uint8_t * tp = a.w + ((size_t)tile * nsb + sb) * Tile::BYTES;
                 hdr[u] = *(const u4 *)(tp + r * 16);
-                q[u][0] = *(const u4 *)(tp + 256 + lane * 16);
-                q[u][1] = *(const u4 *)(tp + 1280 + lane * 16);
+#pragma unroll
+                for (int i = 0; i < Tile::LOADS; ++i) q[u][i] = *(const u4 *)(tp + 256 + i * 1024 + lane * 16);
             }
         }
     };
@@ -103,22 +116,24 @@ __global__ __launch_bounds__(1024) void k_gemv_q4k(GemvArgs a) {
     if (tile < a.n_tiles) request(tile, 0);
 
     if (SRC == SRC_CODES) {
-        // stage the rows of the step: 16-byte words of codes, dwords of block sums, scales
+        // stage the rows of the step: 16-byte words of codes, scales, dwords of block sums
         for (int i = tid; i < NT * (K >> 4); i += nthreads) {
             const int t = i / (K >> 4);
             u4 v = {0u, 0u, 0u, 0u};
             if (t < a.T) v = ((const u4 *)a.codes)[i];
             ((u4 *)l_codes)[i] = v;
         }
-        for (int i = tid; i < NT * (K >> 6); i += nthreads) {
-            const int t = i / (K >> 6);
-            ((uint32_t *)l_bsums)[i] = t < a.T ? ((const uint32_t *)a.bsums)[i] : 0u;
+        for (int i = tid; i < NT * nd; i += nthreads) l_d[i] = i / nd < a.T ? a.d[i] : 0.0f;
+        if (Q4) {
+            for (int i = tid; i < NT * (K >> 6); i += nthreads) {
+                const int t = i / (K >> 6);
+                ((uint32_t *)l_bsums)[i] = t < a.T ? ((const uint32_t *)a.bsums)[i] : 0u;
+            }
         }
-        for (int i = tid; i < NT * nsb; i += nthreads) l_d[i] = i / nsb < a.T ? a.d[i] : 0.0f;
     } else {
-        // make the blocks here: eight consecutive values per thread, the 32 threads of a block together (requantise8)
+        // make the blocks here: eight consecutive values per thread, the threads of a block together (requantise8)
         Act lout;
-        lout.K = K; lout.qc = l_codes; lout.qd = l_d; lout.qbs = l_bsums;
+        lout.K = K; lout.quant = Tile::QUANT; lout.qc = l_codes; lout.qd = l_d; lout.qbs = l_bsums;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const float * xr = row_of(t);
@@ -126,7 +141,7 @@ __global__ __launch_bounds__(1024) void k_gemv_q4k(GemvArgs a) {
             if (SRC == SRC_NORM) {
                 float ss = 0.0f;
                 for (int k = tid * 8; k < K; k += nthreads * 8) {
-                    f4 in[4];
+                    f4 in[2];
                     if (t == 0 && k == tid * 8) { in[0] = first[0]; in[1] = first[1]; }
                     else { in[0] = *(const f4 *)(xr + k); in[1] = *(const f4 *)(xr + k + 4); }
                     const f4 p = in[0], q4 = in[1];
@@ -156,7 +171,7 @@ __global__ __launch_bounds__(1024) void k_gemv_q4k(GemvArgs a) {
 #pragma unroll
                     for (int i = 0; i < 8; ++i) v[i] = (gv[i] / (1.0f + __expf(-gv[i]))) * uv[i];
                 }
-                const float d = requantise8(v, AQ_Q8_K, c);
+                const float d = requantise8(v, Tile::QUANT, c);
                 store_codes8(c, d, lout, t, k, tid & 3);
             }
         }
@@ -166,36 +181,58 @@ __global__ __launch_bounds__(1024) void k_gemv_q4k(GemvArgs a) {
     float acc[NT];
     // super-block sb of the tile, held in register set u, times the rows of the step
     auto multiply = [&](int sb, int u) {
-        const Q4KScales S = q4k_scales(hdr[u]);
-        int dot[NT];
+        if constexpr (Q4) {
+            const Q4KScales S = q4k_scales(hdr[u]);
+            int dot[NT];
 #pragma unroll
-        for (int t = 0; t < NT; ++t) dot[t] = 0;
+            for (int t = 0; t < NT; ++t) dot[t] = 0;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+            for (int h = 0; h < 2; ++h) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t wq = j == 0 ? q[u][h].x : (j == 1 ? q[u][h].y : (j == 2 ? q[u][h].z : q[u][h].w));
-                const int lo = (int)(wq & 0x0F0F0F0Fu), hi = (int)((wq >> 4) & 0x0F0F0F0Fu);
-                const int sc = (int)((S.sc[h] >> (8 * j)) & 0xffu);
-                const int k0 = (sb << 8) + ((4 * h + j) << 5) + (g << 3);
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t wq = j == 0 ? q[u][h].x : (j == 1 ? q[u][h].y : (j == 2 ? q[u][h].z : q[u][h].w));
+                    const int lo = (int)(wq & 0x0F0F0F0Fu), hi = (int)((wq >> 4) & 0x0F0F0F0Fu);
+                    const int sc = (int)((S.sc[h] >> (8 * j)) & 0xffu);
+                    const int k0 = (sb << 8) + ((4 * h + j) << 5) + (g << 3);
 #pragma unroll
-                for (int t = 0; t < NT; ++t) {
-                    const uint2 c = *(const uint2 *)(l_codes + t * K + k0);
-                    int is = __builtin_amdgcn_sdot4(lo, (int)c.x, 0, false);
-                    is = __builtin_amdgcn_sdot4(hi, (int)c.y, is, false);
-                    dot[t] += __mul24(sc, is);
+                    for (int t = 0; t < NT; ++t) {
+                        const uint2 c = *(const uint2 *)(l_codes + t * K + k0);
+                        int is = __builtin_amdgcn_sdot4(lo, (int)c.x, 0, false);
+                        is = __builtin_amdgcn_sdot4(hi, (int)c.y, is, false);
+                        dot[t] += __mul24(sc, is);
+                    }
                 }
             }
-        }
-        // the min term: lane group g takes sub-blocks 2g and 2g + 1
-        const uint32_t mword = (g < 2 ? S.mn[0] : S.mn[1]) >> (16 * (g & 1));
-        const int m0 = (int)(mword & 0xffu), m1 = (int)((mword >> 8) & 0xffu);
-        const float dw = h2f((uint16_t)(hdr[u].x & 0xffffu)), dmin = h2f((uint16_t)(hdr[u].x >> 16));
+            // the min term: lane group g takes sub-blocks 2g and 2g + 1
+            const uint32_t mword = (g < 2 ? S.mn[0] : S.mn[1]) >> (16 * (g & 1));
+            const int m0 = (int)(mword & 0xffu), m1 = (int)((mword >> 8) & 0xffu);
+            const float dw = h2f((uint16_t)(hdr[u].x & 0xffffu)), dmin = h2f((uint16_t)(hdr[u].x >> 16));
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            const int bs = *(const int *)(l_bsums + t * (K >> 5) + (sb << 3) + 2 * g);
-            const int mins = __mul24(m0, (int)(int16_t)(bs & 0xffff)) + __mul24(m1, bs >> 16);
-            acc[t] += l_d[t * nsb + sb] * (dw * (float)dot[t] - dmin * (float)mins);
+            for (int t = 0; t < NT; ++t) {
+                const int bs = *(const int *)(l_bsums + t * (K >> 5) + (sb << 3) + 2 * g);
+                const int mins = __mul24(m0, (int)(int16_t)(bs & 0xffff)) + __mul24(m1, bs >> 16);
+                acc[t] += l_d[t * nsb + sb] * (dw * (float)dot[t] - dmin * (float)mins);
+            }
+        } else {
+            // the row's eight block scales: f16 pairs in the header's four dwords
+#pragma unroll
+            for (int qi = 0; qi < 4; ++qi) {
+                const uint32_t pair = qi == 0 ? hdr[u].x : (qi == 1 ? hdr[u].y : (qi == 2 ? hdr[u].z : hdr[u].w));
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int blk = 2 * qi + half;
+                    const float dw = h2f((uint16_t)(half ? pair >> 16 : pair & 0xffffu));
+                    const int w0 = (int)(half ? q[u][qi].z : q[u][qi].x), w1 = (int)(half ? q[u][qi].w : q[u][qi].y);
+                    const int k0 = (sb << 8) + (blk << 5) + (g << 3);
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        const uint2 c = *(const uint2 *)(l_codes + t * K + k0);
+                        int is = __builtin_amdgcn_sdot4(w0, (int)c.x, 0, false);
+                        is = __builtin_amdgcn_sdot4(w1, (int)c.y, is, false);
+                        acc[t] += (dw * l_d[t * nd + (sb << 3) + blk]) * (float)is;
+                    }
+                }
+            }
         }
     };
 
@@ -236,24 +273,32 @@ __global__ __launch_bounds__(1024) void k_gemv_q4k(GemvArgs a) {
     }
 }
 
-constexpr size_t kGemvMaxLds = 96 * 1024;     // of the CU's 160 KiB; two tokens of 16,384 columns take 39 KiB
-static size_t gemv_lds_bytes(int NT, int NW, int K) {
-    return (size_t)NT * K + (size_t)NT * (K >> 4) + (size_t)NT * (K >> 8) * 4 + (size_t)2 * NW * NT * 16 * 4;
+constexpr size_t kGemvMaxLds = 96 * 1024;     // of the CU's 160 KiB; two tokens of 24,576 columns take 57 KiB
+constexpr int kGemvMaxSb = 16 * 6;            // sixteen waves, at most six super-blocks of a tile each
+static size_t gemv_lds_bytes(int type, int NT, int NW, int K) {
+    const size_t scales = type == WT_Q4_K ? (size_t)NT * (K >> 8) * 4 + (size_t)NT * (K >> 4) : (size_t)NT * (K >> 5) * 4;
+    return (size_t)NT * K + scales + (size_t)2 * NW * NT * 16 * 4;
 }
 
-bool gemv_can_weight(const Weight & w, int T);
+bool gemv_can_weight(const Weight & w, int T) {
+    return (w.type == WT_Q4_K || w.type == WT_Q8_0) && w.packed && T >= 1 && T <= g_gemv_max_t && T <= GEMV_MAX_T
+        && w.K % 256 == 0 && w.N % 16 == 0 && w.K > 0 && w.N > 0
+        && w.K <= 256 * kGemvMaxSb && gemv_lds_bytes(w.type, GEMV_MAX_T, 16, w.K) <= kGemvMaxLds;
+}
+
 bool gemv_can(const Weight & w, const Act & x, int T) {
-    return x.qc && x.qd && x.qbs && x.K == w.K && gemv_can_weight(w, T);
+    if (!x.qc || !x.qd || x.K != w.K || !gemv_can_weight(w, T)) return false;
+    return w.type == WT_Q4_K ? (x.quant == AQ_Q8_K && x.qbs != nullptr) : x.quant == AQ_Q8_0;
 }
 
-template <int NT, int PER, int SRC>
+template <int WT, int NT, int PER, int SRC>
 static void launch_gemv(hipStream_t s, const GemvArgs & a) {
     const int nsb = a.K / 256;
     const int nw = PER == 2 ? (nsb + 1) / 2 : 16;
-    const size_t lds = gemv_lds_bytes(NT, nw, a.K);
+    const size_t lds = gemv_lds_bytes(WT, NT, nw, a.K);
     static bool once = false;
     if (!once) {
-        HIP_OK(hipFuncSetAttribute((const void *)k_gemv_q4k<NT, PER, SRC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvMaxLds));
+        HIP_OK(hipFuncSetAttribute((const void *)k_gemv<WT, NT, PER, SRC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvMaxLds));
         once = true;
     }
     // a workgroup stages the step's rows once and then walks tiles: as many workgroups as the chip holds at
@@ -261,17 +306,30 @@ static void launch_gemv(hipStream_t s, const GemvArgs & a) {
     const int capacity = 256 * std::max(1, 2048 / (nw * 64));
     const int turns = (a.n_tiles + capacity - 1) / capacity;
     const unsigned grid = (unsigned)((a.n_tiles + turns - 1) / turns);
-    hipLaunchKernelGGL((k_gemv_q4k<NT, PER, SRC>), dim3(grid), dim3(nw * 64), lds, s, a);
+    hipLaunchKernelGGL((k_gemv<WT, NT, PER, SRC>), dim3(grid), dim3(nw * 64), lds, s, a);
+}
+
+template <int WT, int SRC>
+static void launch_gemv_tokens(hipStream_t s, const GemvArgs & a) {
+    static_assert(GEMV_MAX_T == 2, "one instantiation per token count");
+    // two super-blocks of a tile per wave while sixteen waves cover the row, four or six beyond
+    const int nsb = a.K / 256;
+    if (a.T == 1) {
+        if (nsb <= 32) launch_gemv<WT, 1, 2, SRC>(s, a);
+        else if (nsb <= 64) launch_gemv<WT, 1, 4, SRC>(s, a);
+        else launch_gemv<WT, 1, 6, SRC>(s, a);
+    } else {
+        if (nsb <= 32) launch_gemv<WT, 2, 2, SRC>(s, a);
+        else if (nsb <= 64) launch_gemv<WT, 2, 4, SRC>(s, a);
+        else launch_gemv<WT, 2, 6, SRC>(s, a);
+    }
+    check_launch("gemv");
 }
 
 template <int SRC>
-static void launch_gemv_src(hipStream_t s, const GemvArgs & a) {
-    static_assert(GEMV_MAX_T == 2, "one instantiation per token count");
-    // two super-blocks of a tile per wave while sixteen waves cover the row, four beyond
-    const bool two = a.K <= 256 * 2 * 16;
-    if (a.T == 1) { if (two) launch_gemv<1, 2, SRC>(s, a); else launch_gemv<1, 4, SRC>(s, a); }
-    else { if (two) launch_gemv<2, 2, SRC>(s, a); else launch_gemv<2, 4, SRC>(s, a); }
-    check_launch("gemv");
+static void launch_gemv_src(hipStream_t s, int type, const GemvArgs & a) {
+    if (type == WT_Q4_K) launch_gemv_tokens<WT_Q4_K, SRC>(s, a);
+    else launch_gemv_tokens<WT_Q8_0, SRC>(s, a);
 }
 
 static GemvArgs gemv_args(const Weight & w, int T, float * y, int ldy, int col0, int mode, const float * bias) {
@@ -284,33 +342,28 @@ static GemvArgs gemv_args(const Weight & w, int T, float * y, int ldy, int col0,
 }
 
 void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias) {
-    if (!gemv_can(w, x, T)) throw std::runtime_error("gemv: needs Q4_K tiles, Q8_K code buffers and at most " + std::to_string(GEMV_MAX_T) + " tokens");
+    if (!gemv_can(w, x, T))
+        throw std::runtime_error("gemv: needs Q4_K or Q8_0 tiles, the code buffers of their conversion and at most " + std::to_string(GEMV_MAX_T) + " tokens");
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
     a.codes = x.qc; a.d = x.qd; a.bsums = x.qbs;
-    launch_gemv_src<SRC_CODES>(s, a);
-}
-
-bool gemv_can_weight(const Weight & w, int T) {
-    return w.type == WT_Q4_K && w.packed && T >= 1 && T <= g_gemv_max_t && T <= GEMV_MAX_T
-        && w.K % 256 == 0 && w.N % 16 == 0 && w.K > 0 && w.N > 0
-        && w.K <= 256 * 4 * 16 && gemv_lds_bytes(GEMV_MAX_T, 16, w.K) <= kGemvMaxLds;
+    launch_gemv_src<SRC_CODES>(s, w.type, a);
 }
 
 void gemv_norm(hipStream_t s, const Weight & w, const float * x, const float * norm_w, float eps, const int32_t * rows, int T,
                float * y, int ldy, int col0, int mode, const float * bias) {
-    if (!gemv_can_weight(w, T) || !x || !norm_w) throw std::runtime_error("gemv_norm: needs Q4_K tiles, the rows and the norm weights");
+    if (!gemv_can_weight(w, T) || !x || !norm_w) throw std::runtime_error("gemv_norm: needs Q4_K or Q8_0 tiles, the rows and the norm weights");
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
     a.xin = x; a.norm_w = norm_w; a.rows = rows; a.eps = eps;
-    launch_gemv_src<SRC_NORM>(s, a);
+    launch_gemv_src<SRC_NORM>(s, w.type, a);
 }
 
 void gemv_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, int T, float * y, int ldy, int col0, int mode) {
     if (group <= 0) group = w.K;
     if (!gemv_can_weight(w, T) || !gu || w.K % group != 0 || group % 8 != 0)
-        throw std::runtime_error("gemv_swiglu: needs Q4_K tiles and gate / up rows in groups that divide the width");
+        throw std::runtime_error("gemv_swiglu: needs Q4_K or Q8_0 tiles and gate / up rows in groups that divide the width");
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, nullptr);
     a.xin = gu; a.group = group;
-    launch_gemv_src<SRC_SWIGLU>(s, a);
+    launch_gemv_src<SRC_SWIGLU>(s, w.type, a);
 }
 
 }  // namespace rk

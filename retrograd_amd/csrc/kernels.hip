@@ -192,8 +192,8 @@ __device__ __forceinline__ void store_act_block(const float * v, int count, cons
 
 // Host-side check of what a producer is asked to write.
 static void check_act_out(const Act & out, int K, const char * what, int n_rows) {
-    if (out.qc && (out.quant != AQ_Q8_K || !out.qx || !out.qd || !out.qbs || n_rows > GEMV_MAX_T))
-        throw std::runtime_error(std::string(what) + ": the integer code buffers go with the Q8_K conversion of at most "
+    if (out.qc && ((out.quant != AQ_Q8_K && out.quant != AQ_Q8_0) || !out.qx || !out.qd || (out.quant == AQ_Q8_K && !out.qbs) || n_rows > GEMV_MAX_T))
+        throw std::runtime_error(std::string(what) + ": the integer code buffers go with a Q8_K or Q8_0 conversion of at most "
                                  + std::to_string(GEMV_MAX_T) + " rows");
     if (out.K != K) throw std::runtime_error(std::string(what) + ": activation width does not match");
     if (!out.x && !out.qx) throw std::runtime_error(std::string(what) + ": no activation buffer to write");
@@ -2056,8 +2056,15 @@ __global__ __launch_bounds__(256) void k_attention_combine(CombineArgs a) {
         const float d = __fdiv_rn(amax, 127.0f);
         const float id = d != 0.0f ? __fdiv_rn(1.0f, d) : 0.0f;
         const float dh = (float)(_Float16)d;
-        q0 = __fmul_rn(dh, roundf(__fmul_rn(f0, id)));
-        q1 = __fmul_rn(dh, roundf(__fmul_rn(f1, id)));
+        const float c0 = roundf(__fmul_rn(f0, id)), c1 = roundf(__fmul_rn(f1, id));
+        q0 = __fmul_rn(dh, c0);
+        q1 = __fmul_rn(dh, c1);
+        if (a.out.qc && mine) {      // the blocks themselves, for the integer matrix-vector kernel (see store_codes8)
+            int8_t * at = a.out.qc + (size_t)t * QD + k;
+            at[0] = (int8_t)(int)c0;
+            at[1] = (int8_t)(int)c1;
+            if ((lane & 15) == 0) a.out.qd[(size_t)t * (QD >> 5) + (k >> 5)] = dh;
+        }
     } else {
         // a block of 256 = 256 / hd heads = that many waves of this workgroup, in head order
         float amax = fabsf(f0), first = f0;

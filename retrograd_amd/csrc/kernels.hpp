@@ -78,11 +78,12 @@ struct Act {
     __half * qsums = nullptr;
     int quant = AQ_NONE;
     int faithful = 0;           // ggml's arithmetic: F16 / BF16 operands are rounded as well
-    // With quant == AQ_Q8_K a producer can leave the Q8_K blocks themselves as well, for the integer
-    // matrix-vector kernel that multiplies very small steps (gemv): the int8 codes [token][K], the eight
-    // codes of a group k / 8 in the order 0 4 1 5 2 6 3 7 (act_code_pos; the order in which a Q4_K tile's
-    // nibbles unpack into bytes); the block scales 1 / iscale, f32 [token][K / 256]; and the sums of the
-    // codes of every 32, int16 [token][K / 32].
+    // A producer can leave the blocks of the conversion themselves as well, for the integer matrix-vector
+    // kernel that multiplies very small steps (gemv). Q8_K: the int8 codes [token][K], the eight codes of a
+    // group k / 8 in the order 0 4 1 5 2 6 3 7 (act_code_pos; the order in which a Q4_K tile's nibbles unpack
+    // into bytes); the block scales 1 / iscale, f32 [token][K / 256]; and the sums of the codes of every 32,
+    // int16 [token][K / 32]. Q8_0: the codes in element order, the scales (f16 values) as f32 [token][K / 32],
+    // no sums.
     int8_t * qc = nullptr;
     float * qd = nullptr;
     int16_t * qbs = nullptr;
@@ -94,7 +95,7 @@ struct Act {
         a.faithful = faithful;
         if (faithful && act_quant_of(ggml_type) != AQ_NONE) {
             a.x = qx; a.sums = qsums;
-            if (act_quant_of(ggml_type) == AQ_Q8_K && quant == AQ_Q8_K) { a.qc = qc; a.qd = qd; a.qbs = qbs; }
+            if (act_quant_of(ggml_type) == quant) { a.qc = qc; a.qd = qd; a.qbs = qbs; a.quant = quant; }
         } else { a.x = x; a.sums = sums; }
         return a;
     }
@@ -135,10 +136,10 @@ Slices matmul_deferred(hipStream_t s, const Weight & w, const Act & x, int T, fl
 // y[t][col0 + c] (=|+=) sum of the slices.
 void reduce_slices(hipStream_t s, const Slices & sl, int T, float * y, int ldy, int col0, int mode);
 size_t matmul_workspace_bytes();
-// The integer matrix-vector kernel: a Q4_K tile matrix times the Q8_K blocks of one or two tokens, as
-// ggml's CPU dot product multiplies them (integer sums of code products per sub-block, times the integer
-// sub-block scale, one float multiply per super-block). One workgroup per 16-row tile, the waves of a
-// workgroup share the tile's super-blocks; no K-slices. x is the operand (Act::operand) of the weight.
+// The integer matrix-vector kernel: a Q4_K (Q8_0) tile matrix times the Q8_K (Q8_0) blocks of one or two
+// tokens, as ggml's CPU dot products multiply them (integer sums of code products per block, Q4_K: times
+// the integer sub-block scale, one float multiply per super-block). One workgroup per 16-row tile, the
+// waves of a workgroup share the tile's super-blocks; no K-slices. x is the operand (Act::operand) of the weight.
 constexpr int GEMV_MAX_T = 2;     // beyond two tokens the tile kernels are as fast
 bool gemv_can(const Weight & w, const Act & x, int T);
 void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias);

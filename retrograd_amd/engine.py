@@ -222,7 +222,7 @@ def load_library() -> C.CDLL:
     lib.retro_kernel_sample_greedy_noalloc.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_void_p,
                                                        C.c_void_p, C.c_void_p]
     lib.retro_kernel_sample_greedy_noalloc_max_rows.restype = C.c_int32
-    lib.retro_kernel_gemv_fused.argtypes = [C.c_int32, _u8p, C.c_int64, C.c_int64, _f32p, _f32p, C.c_float, C.c_int32, C.c_int32,
+    lib.retro_kernel_gemv_fused.argtypes = [C.c_int32, C.c_int32, _u8p, C.c_int64, C.c_int64, _f32p, _f32p, C.c_float, C.c_int32, C.c_int32,
                                             _f32p, _f32p]
     lib.retro_kernel_gemv_fused.restype = C.c_int
     lib.retro_kernel_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,
@@ -874,7 +874,7 @@ def kernel_matmul(ggml_type: int, raw: np.ndarray, n_rows: int, k: int, x: np.nd
                   bias: np.ndarray | None = None, accumulate_into: np.ndarray | None = None,
                   ggml_activations: bool = False, integer: bool = False) -> np.ndarray:
     """One matmul kernel on host data; ggml_activations: the rows are converted as ggml's CPU matmul does;
-    integer (with it, Q4_K tiles, at most two rows): the Q8_K blocks go through the integer matrix-vector kernel."""
+    integer (with it, Q4_K or Q8_0 tiles, at most two rows): the converted blocks go through the integer matrix-vector kernel."""
     lib = load_library()
     use_tiles = int(use_tiles) | (0x100 if ggml_activations else 0) | (0x200 if integer else 0)
     raw = np.ascontiguousarray(raw, np.uint8)
@@ -892,7 +892,7 @@ def kernel_matmul(ggml_type: int, raw: np.ndarray, n_rows: int, k: int, x: np.nd
     return y
 
 
-def kernel_gemv_fused(kind: int, raw: np.ndarray, n_rows: int, k: int, x: np.ndarray, norm_w: np.ndarray | None = None,
+def kernel_gemv_fused(kind: int, ggml_type: int, raw: np.ndarray, n_rows: int, k: int, x: np.ndarray, norm_w: np.ndarray | None = None,
                       eps: float = 1e-5, group: int = 0):
     """The integer matrix-vector kernel with RMSNorm (kind 1) or SwiGLU (kind 2) fused into its staging, and the same
     product as producer launch plus kernel: returns (fused, unfused), each [tokens][n_rows]."""
@@ -905,7 +905,7 @@ def kernel_gemv_fused(kind: int, raw: np.ndarray, n_rows: int, k: int, x: np.nda
         norm_w = np.ascontiguousarray(norm_w, np.float32)
         w = norm_w.ctypes.data_as(_f32p)
     fused, unfused = np.zeros((T, n_rows), np.float32), np.zeros((T, n_rows), np.float32)
-    s = lib.retro_kernel_gemv_fused(kind, raw.ctypes.data_as(_u8p), n_rows, k, x.ctypes.data_as(_f32p), w, eps, T, group,
+    s = lib.retro_kernel_gemv_fused(kind, ggml_type, raw.ctypes.data_as(_u8p), n_rows, k, x.ctypes.data_as(_f32p), w, eps, T, group,
                                     fused.ctypes.data_as(_f32p), unfused.ctypes.data_as(_f32p))
     if s != 0:
         _raise(s)

@@ -141,17 +141,18 @@ def test_tile_matmul_exact_on_integer_data():
 
 
 @pytest.mark.parametrize("n,k,T", [(16, 256, 1), (48, 512, 2), (2064, 256, 2), (64, 1024, 1), (256, 4096, 1), (32, 8192, 2),
-                                   (128, 14336, 2), (4096, 4096, 2), (1024, 14336, 1), (320, 16384, 2), (16, 8448, 1)])
-def test_integer_matvec_matches_decoded_blocks(n, k, T):
+                                   (128, 14336, 2), (4096, 4096, 2), (1024, 14336, 1), (320, 16384, 2), (16, 8448, 1),
+                                   (64, 18944, 2), (48, 24576, 1), (112, 3584, 2)])
+@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0])
+def test_integer_matvec_matches_decoded_blocks(t, n, k, T):
     # The kernel of very small steps under the ggml arithmetic: integer products of the stored codes with the
     # Q8_K codes of the rows. Its sums are those of the converted values times the decoded weights, so the
     # reference of the tile kernels is its reference too.
-    print("case", n, k, T, flush=True)
-    t = gw.GGML_Q4_K
+    print("case", t, n, k, T, flush=True)
     raw, dense = _weights(t, n, k, seed=n + k + T)
     rng = np.random.default_rng(T + k)
     x = rng.standard_normal((T, k)).astype(np.float32)
-    x[0, :256] = 0.0                                    # a block of zeros: scale 0, codes 0
+    x[0, :256] = 0.0                                    # blocks of zeros: scale 0, codes 0
     want = _ref(t, dense, x, True)
     scale = np.abs(want).max()
     got = E.kernel_matmul(t, raw, n, k, x, use_tiles=2, ggml_activations=True, integer=True)
@@ -190,40 +191,56 @@ def test_integer_matvec_exact_on_integer_data_and_refusals():
         one[0, e] = -127.0
         got = E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, one, use_tiles=2, ggml_activations=True, integer=True)
         assert np.array_equal(got[0].astype(np.float64), -127.0 * dense[:, e]), e
+    # Q8_0: every byte value as a weight code (-128 included), d = 0.125, the same self-coding activations
+    q8 = rng.integers(0, 256, (n, k // 32, 34), dtype=np.uint8)
+    q8[..., 0:2] = np.frombuffer(np.float16(0.125).tobytes(), np.uint8)
+    raw8 = q8.reshape(n, -1)
+    dense8 = np.stack([oracle.decode_row(gw.GGML_Q8_0, raw8[i], k) for i in range(n)]).astype(np.float64)
+    for T in (1, 2):
+        x = rng.integers(-4, 5, (T, k)).astype(np.float32)
+        x[:, ::32] = rng.choice([-127.0, 127.0], (T, k // 32))
+        assert np.array_equal(np.stack([oracle.activation_row(gw.GGML_Q8_0, r) for r in x]), x)
+        got = E.kernel_matmul(gw.GGML_Q8_0, raw8, n, k, x, use_tiles=2, ggml_activations=True, integer=True)
+        assert np.array_equal(got.astype(np.float64), x.astype(np.float64) @ dense8.T), T
+    for e in (0, 1, 3, 4, 7, 8, 31, 32, 33, 255, 256, 767):
+        one = np.zeros((1, k), np.float32)
+        one[0, e] = 127.0
+        got = E.kernel_matmul(gw.GGML_Q8_0, raw8, n, k, one, use_tiles=2, ggml_activations=True, integer=True)
+        assert np.array_equal(got[0].astype(np.float64), 127.0 * dense8[:, e]), e
     x = rng.standard_normal((3, k)).astype(np.float32)
     with pytest.raises(E.EngineError, match="at most 2 tokens"):
         E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x, use_tiles=2, ggml_activations=True, integer=True)
     with pytest.raises(E.EngineError, match="at most 2 tokens"):
         E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x[:1], use_tiles=2, integer=True)      # the exact arithmetic has no codes
-    q8, _ = _weights(gw.GGML_Q8_0, 16, 256, seed=1)
-    with pytest.raises(E.EngineError, match="at most 2 tokens"):
-        E.kernel_matmul(gw.GGML_Q8_0, q8, 16, 256, x[:1, :256], use_tiles=2, ggml_activations=True, integer=True)
+    q6, _ = _weights(gw.GGML_Q6_K, 16, 256, seed=1)
+    with pytest.raises(E.EngineError, match="does not take this matrix"):
+        E.kernel_matmul(gw.GGML_Q6_K, q6, 16, 256, x[:1, :256], use_tiles=2, ggml_activations=True, integer=True)
 
 
+@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0])
 @pytest.mark.parametrize("kind", [1, 2])
 @pytest.mark.parametrize("n,k,T", [(64, 4096, 1), (64, 4096, 2), (32, 512, 1), (48, 1024, 2), (32, 14336, 1), (16, 14336, 2),
-                                   (16, 8448, 2), (32, 2048, 1)])
-def test_integer_matvec_with_its_producer_fused(kind, n, k, T):
+                                   (16, 8448, 2), (32, 2048, 1), (32, 3584, 1), (16, 18944, 1)])
+def test_integer_matvec_with_its_producer_fused(t, kind, n, k, T):
     # The Q8_K blocks made by the kernel itself while it stages them (RMSNorm of residual rows, or SwiGLU of a gate/up
     # product) against the producer's own launch followed by the kernel, and against the CPU: the norm / SiLU in
     # float64, the conversion by the oracle, the decoded weights. A row of 4096 is normalised in the very order the
     # standalone kernel uses, so there the two paths agree bit for bit; elsewhere the sum of squares is added in
     # another order and a code on a rounding boundary may differ.
-    print("case", kind, n, k, T, flush=True)
-    t = gw.GGML_Q4_K
+    print("case", t, kind, n, k, T, flush=True)
     raw, dense = _weights(t, n, k, seed=n + k + T + kind)
     rng = np.random.default_rng(k + T)
     eps = 1e-5
     if kind == 1:
         x = (rng.standard_normal((T, k)) * 3.0).astype(np.float32)
         w = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
-        fused, unfused = E.kernel_gemv_fused(1, raw, n, k, x, norm_w=w, eps=eps)
+        fused, unfused = E.kernel_gemv_fused(1, t, raw, n, k, x, norm_w=w, eps=eps)
         x64 = x.astype(np.float64)
         rows = x64 / np.sqrt((x64 * x64).mean(-1, keepdims=True) + eps) * w
     else:
         group = 64 if k % 64 == 0 else 0
         gu = rng.standard_normal((T, 2 * k)).astype(np.float32)
-        fused, unfused = E.kernel_gemv_fused(2, raw, n, k, gu, group=group)
+        fused, unfused = E.kernel_gemv_fused(2, t, raw, n, k, gu, group=group)
         g64 = gu.astype(np.float64).reshape(T, k // 64, 2, 64)
         rows = (g64[:, :, 0] / (1 + np.exp(-g64[:, :, 0])) * g64[:, :, 1]).reshape(T, k)
     want = _ref(t, dense, rows.astype(np.float32), True)

@@ -353,7 +353,7 @@ def main() -> int:
         kvb = 2 * shape.n_head_kv * shape.head_dim * 2 * {"f16": 32, "q8_0": 17, "q4_0": 9}[args.kv] // 32
         leg = one_sequence_leg(eng, E, shape, n_slots, synth.streamed_weight_bytes(shape), kvb, steps=args.steps)
         eng.close()
-        print(json.dumps({"metric": "single-sequence decode steps, 8B-shape Q4_K", "activations": args.activations,
+        print(json.dumps({"metric": "single-sequence decode steps, %s" % shape.name, "activations": args.activations,
                           "kv_cache": args.kv, **leg}), flush=True)
         return 0
     eng = new_engine(args.activations)

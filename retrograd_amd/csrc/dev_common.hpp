@@ -137,8 +137,8 @@ __device__ __forceinline__ float requantise8(float (&v)[8], int quant, float * c
 }
 
 // The codes of eight consecutive values (k a multiple of 8) into the buffers of the integer matrix-vector kernel
-// (Act::qc, qd, qbs). Q8_K: 8 bytes in the order of act_code_pos, the sum of a 32-wide block from its four lanes, the
-// block scale from the lane that holds the block's first values. Q8_0: 8 bytes in element order, the scale of the
+// (Act::qc, qd, qbs). Q8_K: 8 bytes in the order of act_code_pos, the sum of every 16 codes from their two lanes (ggml's
+// Q8_K bsums), the block scale from the lane that holds the block's first values. Q8_0: 8 bytes in element order, the scale of the
 // 32-wide block from its first lane.
 __device__ __forceinline__ void store_codes8(const float (&c)[8], float d, const Act & out, int tok, int k, int lane_in_block) {
     uint32_t w0 = 0, w1 = 0;
@@ -158,8 +158,7 @@ __device__ __forceinline__ void store_codes8(const float (&c)[8], float d, const
         return;
     }
     sum += __shfl_xor(sum, 1, 64);
-    sum += __shfl_xor(sum, 2, 64);
-    if (lane_in_block == 0) out.qbs[(size_t)tok * (out.K >> 5) + (k >> 5)] = (int16_t)sum;
+    if ((lane_in_block & 1) == 0) out.qbs[(size_t)tok * (out.K >> 4) + (k >> 4)] = (int16_t)sum;
     if ((k & 255) == 0) out.qd[(size_t)tok * (out.K >> 8) + (k >> 8)] = d;
 }
 

@@ -477,7 +477,7 @@ void Engine::build_buffers() {
             if (K % 256 != 0) return;          // no Q8_K conversion of such rows
             c.codes.alloc((size_t)rk::GEMV_MAX_T * K);
             c.d.alloc((size_t)rk::GEMV_MAX_T * (K / 32) * 4);          // one scale per 32 (Q8_0) or per 256 (Q8_K)
-            c.bsums.alloc((size_t)rk::GEMV_MAX_T * (K / 32) * 2);
+            c.bsums.alloc((size_t)rk::GEMV_MAX_T * (K / 16) * 2);
         };
         codes(act_e_codes_, E);
         codes(act_q_codes_, QD);

@@ -19,6 +19,13 @@
 // byte order (act_code_pos), so no lane ever permutes anything: about a quarter of the tile kernels' vector
 // instructions per weight.
 //
+// Q6_K (activations Q8_K; the finer type of a Q4_K_M file):
+//   sum over super-blocks of  d_w d_x * sum_b sc_b * ( sum_{k in b} u_k c_k  -  32 bsum_b )
+// over the sixteen blocks b of 16 with their i8 scales, u the unsigned 6-bit codes. The tile keeps the low nibbles
+// in the Q4_K order and the top bit pairs in a plane of their own (see k_repack_q6k); two shifts and masks per dword
+// move them above the nibbles of the two byte dwords, which costs about twice the Q4_K kernel's vector instructions
+// per weight - still fewer than the tile kernel spends, and without its four matrix instructions per step.
+//
 // Q8_0 (activations Q8_0):
 //   sum_k w[n][k] x[k] = sum over blocks of 32 of  (d_w d_x) * sum_{k in block} q_k c_k
 // The Q8_0 tile (16 x 8 f16 scales, then four 1 KiB loads in which lane (r, g) of load q holds columns 8g .. 8g + 8
@@ -34,7 +41,7 @@ struct GemvArgs {
     const uint8_t * w;         // tiles
     const int8_t * codes;      // [T][K]
     const float * d;           // [T][K / 256] (Q8_K) or [T][K / 32] (Q8_0)
-    const int16_t * bsums;     // [T][K / 32] (Q8_K only)
+    const int16_t * bsums;     // [T][K / 16] (Q8_K only)
     float * y;
     const float * bias;
     int K, N, T, ldy, col0, mode, n_tiles;
@@ -50,6 +57,9 @@ enum : int { SRC_CODES = 0, SRC_NORM = 1, SRC_SWIGLU = 2 };
 template <int WT> struct GemvTile;
 template <> struct GemvTile<WT_Q4_K> { static constexpr int BYTES = 2304, LOADS = 2, QUANT = AQ_Q8_K; };
 template <> struct GemvTile<WT_Q8_0> { static constexpr int BYTES = 4352, LOADS = 4, QUANT = AQ_Q8_0; };
+// Q6_K: register set = the row's sixteen scales | low nibbles of the two k-halves | top bits of the two k-halves
+// (8 bytes a lane each, held as one 16-byte word) | d
+template <> struct GemvTile<WT_Q6_K> { static constexpr int BYTES = 3360, LOADS = 3, QUANT = AQ_Q8_K; };
 
 // WT: the weight type. NT: tokens held (rows of the step beyond a.T read as zeros). PER: super-blocks of a tile per
 // wave; a workgroup has nw waves (PER 2: half the row's super-blocks; wider rows: 16), wave w takes super-blocks
@@ -63,25 +73,26 @@ template <> struct GemvTile<WT_Q8_0> { static constexpr int BYTES = 4352, LOADS 
 // 4096 gives the same codes bit for bit) and the conversion, straight into LDS - which saves the step a launch of
 // four to five microseconds for about one and a half of redundant work per workgroup. SRC_SWIGLU: likewise
 // silu(gate) * up of the gate/up product's f32 rows. NT is exactly the token count then.
-// Dynamic LDS: codes NT * K bytes | scales NT * nd floats (nd = K / 256 or K / 32) | Q8_K: block sums NT * K / 16
+// Dynamic LDS: codes NT * K bytes | scales NT * nd floats (nd = K / 256 or K / 32) | Q8_K: block sums NT * K / 8
 // bytes | 2 * nw * NT * 16 floats.
 template <int WT, int NT, int PER, int SRC>
 __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
     using Tile = GemvTile<WT>;
-    constexpr bool Q4 = WT == WT_Q4_K;
+    constexpr bool Q4 = WT == WT_Q4_K, Q6 = WT == WT_Q6_K, K8 = Tile::QUANT == AQ_Q8_K;
     extern __shared__ __align__(16) uint8_t lds[];
     const int K = a.K, nsb = K >> 8;
-    const int nd = Q4 ? nsb : (K >> 5);
+    const int nd = K8 ? nsb : (K >> 5);
     const int nthreads = blockDim.x, nw = nthreads >> 6;
     int8_t * l_codes = (int8_t *)lds;
     float * l_d = (float *)(lds + (size_t)NT * K);
     int16_t * l_bsums = (int16_t *)(l_d + NT * nd);
-    float * l_red = Q4 ? (float *)((uint8_t *)l_bsums + (size_t)NT * (K >> 4)) : (float *)l_bsums;
+    float * l_red = K8 ? (float *)((uint8_t *)l_bsums + (size_t)NT * (K >> 3)) : (float *)l_bsums;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
 
     // two super-blocks are held at a time: u0 and u0 + 1 of the wave's PER
     u4 hdr[2], q[2][Tile::LOADS];
+    uint16_t dq6[2] = {0, 0};          // Q6_K: the row's d
     auto request = [&](int tile, int u0) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
@@ -89,8 +100,16 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
             if (sb < nsb) {
                 const uint8_t * tp = a.w + ((size_t)tile * nsb + sb) * Tile::BYTES;
                 hdr[u] = *(const u4 *)(tp + r * 16);
+                if constexpr (Q6) {
+                    q[u][0] = *(const u4 *)(tp + 288 + lane * 16);
+                    q[u][1] = *(const u4 *)(tp + 1312 + lane * 16);
+                    const uint2 t0 = *(const uint2 *)(tp + 2336 + lane * 8), t1 = *(const uint2 *)(tp + 2848 + lane * 8);
+                    q[u][2] = u4{t0.x, t0.y, t1.x, t1.y};
+                    dq6[u] = *(const uint16_t *)(tp + 256 + 2 * r);
+                } else {
 #pragma unroll
-                for (int i = 0; i < Tile::LOADS; ++i) q[u][i] = *(const u4 *)(tp + 256 + i * 1024 + lane * 16);
+                    for (int i = 0; i < Tile::LOADS; ++i) q[u][i] = *(const u4 *)(tp + 256 + i * 1024 + lane * 16);
+                }
             }
         }
     };
@@ -124,9 +143,9 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
             ((u4 *)l_codes)[i] = v;
         }
         for (int i = tid; i < NT * nd; i += nthreads) l_d[i] = i / nd < a.T ? a.d[i] : 0.0f;
-        if (Q4) {
-            for (int i = tid; i < NT * (K >> 6); i += nthreads) {
-                const int t = i / (K >> 6);
+        if (K8) {
+            for (int i = tid; i < NT * (K >> 5); i += nthreads) {
+                const int t = i / (K >> 5);
                 ((uint32_t *)l_bsums)[i] = t < a.T ? ((const uint32_t *)a.bsums)[i] : 0u;
             }
         }
@@ -209,9 +228,51 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
             const float dw = h2f((uint16_t)(hdr[u].x & 0xffffu)), dmin = h2f((uint16_t)(hdr[u].x >> 16));
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
-                const int bs = *(const int *)(l_bsums + t * (K >> 5) + (sb << 3) + 2 * g);
-                const int mins = __mul24(m0, (int)(int16_t)(bs & 0xffff)) + __mul24(m1, bs >> 16);
+                const int2 bs = *(const int2 *)(l_bsums + t * (K >> 4) + (sb << 4) + 4 * g);      // four sums of 16
+                const int s0 = (int)(int16_t)(bs.x & 0xffff) + (bs.x >> 16), s1 = (int)(int16_t)(bs.y & 0xffff) + (bs.y >> 16);
+                const int mins = __mul24(m0, s0) + __mul24(m1, s1);
                 acc[t] += l_d[t * nsb + sb] * (dw * (float)dot[t] - dmin * (float)mins);
+            }
+        } else if constexpr (Q6) {
+            int dot[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) dot[t] = 0;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t wq = j == 0 ? q[u][h].x : (j == 1 ? q[u][h].y : (j == 2 ? q[u][h].z : q[u][h].w));
+                    // the top bit pairs of k-steps 2m and 2m + 1 share a dword, the odd step's rotated left by eight
+                    const uint32_t tw = h == 0 ? (j < 2 ? q[u][2].x : q[u][2].y) : (j < 2 ? q[u][2].z : q[u][2].w);
+                    const uint32_t top = (j & 1) ? __builtin_amdgcn_alignbit(tw, tw, 8) : tw;
+                    // codes 0 4 1 5 and 2 6 3 7 as bytes: nibble | top pair << 4
+                    const int lo = (int)((wq & 0x0F0F0F0Fu) | (top & 0x00300030u) | ((top << 4) & 0x30003000u));
+                    const int hi = (int)(((wq >> 4) & 0x0F0F0F0Fu) | ((top >> 2) & 0x00300030u) | ((top << 2) & 0x30003000u));
+                    // the block of 16 these eight columns belong to: 8h + 2j + g / 2; its i8 scale
+                    const int b = 8 * h + 2 * j + (g >> 1);
+                    const uint32_t sw = (b >> 2) == 0 ? hdr[u].x : ((b >> 2) == 1 ? hdr[u].y : ((b >> 2) == 2 ? hdr[u].z : hdr[u].w));
+                    const int sc = (int)(int8_t)((sw >> (8 * (b & 3))) & 0xffu);
+                    const int k0 = (sb << 8) + ((4 * h + j) << 5) + (g << 3);
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        const uint2 c = *(const uint2 *)(l_codes + t * K + k0);
+                        int is = __builtin_amdgcn_sdot4(lo, (int)c.x, 0, false);
+                        is = __builtin_amdgcn_sdot4(hi, (int)c.y, is, false);
+                        dot[t] += __mul24(sc, is);
+                    }
+                }
+            }
+            // the offset of 32: lane group g takes blocks 4g .. 4g + 3 (the bytes of header dword g)
+            const uint32_t sw = g == 0 ? hdr[u].x : (g == 1 ? hdr[u].y : (g == 2 ? hdr[u].z : hdr[u].w));
+            const float dw = h2f(dq6[u]);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const int2 bs = *(const int2 *)(l_bsums + t * (K >> 4) + (sb << 4) + 4 * g);
+                int corr = __mul24((int)(int8_t)(sw & 0xffu), (int)(int16_t)(bs.x & 0xffff));
+                corr += __mul24((int)(int8_t)((sw >> 8) & 0xffu), bs.x >> 16);
+                corr += __mul24((int)(int8_t)((sw >> 16) & 0xffu), (int)(int16_t)(bs.y & 0xffff));
+                corr += __mul24((int)(int8_t)(sw >> 24), bs.y >> 16);
+                acc[t] += (dw * l_d[t * nsb + sb]) * (float)(dot[t] - 32 * corr);
             }
         } else {
             // the row's eight block scales: f16 pairs in the header's four dwords
@@ -276,19 +337,19 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
 constexpr size_t kGemvMaxLds = 96 * 1024;     // of the CU's 160 KiB; two tokens of 24,576 columns take 57 KiB
 constexpr int kGemvMaxSb = 16 * 6;            // sixteen waves, at most six super-blocks of a tile each
 static size_t gemv_lds_bytes(int type, int NT, int NW, int K) {
-    const size_t scales = type == WT_Q4_K ? (size_t)NT * (K >> 8) * 4 + (size_t)NT * (K >> 4) : (size_t)NT * (K >> 5) * 4;
+    const size_t scales = type == WT_Q8_0 ? (size_t)NT * (K >> 5) * 4 : (size_t)NT * (K >> 8) * 4 + (size_t)NT * (K >> 3);
     return (size_t)NT * K + scales + (size_t)2 * NW * NT * 16 * 4;
 }
 
 bool gemv_can_weight(const Weight & w, int T) {
-    return (w.type == WT_Q4_K || w.type == WT_Q8_0) && w.packed && T >= 1 && T <= g_gemv_max_t && T <= GEMV_MAX_T
+    return (w.type == WT_Q4_K || w.type == WT_Q8_0 || w.type == WT_Q6_K) && w.packed && T >= 1 && T <= g_gemv_max_t && T <= GEMV_MAX_T
         && w.K % 256 == 0 && w.N % 16 == 0 && w.K > 0 && w.N > 0
         && w.K <= 256 * kGemvMaxSb && gemv_lds_bytes(w.type, GEMV_MAX_T, 16, w.K) <= kGemvMaxLds;
 }
 
 bool gemv_can(const Weight & w, const Act & x, int T) {
     if (!x.qc || !x.qd || x.K != w.K || !gemv_can_weight(w, T)) return false;
-    return w.type == WT_Q4_K ? (x.quant == AQ_Q8_K && x.qbs != nullptr) : x.quant == AQ_Q8_0;
+    return w.type == WT_Q8_0 ? x.quant == AQ_Q8_0 : (x.quant == AQ_Q8_K && x.qbs != nullptr);
 }
 
 template <int WT, int NT, int PER, int SRC>
@@ -329,6 +390,7 @@ static void launch_gemv_tokens(hipStream_t s, const GemvArgs & a) {
 template <int SRC>
 static void launch_gemv_src(hipStream_t s, int type, const GemvArgs & a) {
     if (type == WT_Q4_K) launch_gemv_tokens<WT_Q4_K, SRC>(s, a);
+    else if (type == WT_Q6_K) launch_gemv_tokens<WT_Q6_K, SRC>(s, a);
     else launch_gemv_tokens<WT_Q8_0, SRC>(s, a);
 }
 
@@ -343,7 +405,7 @@ static GemvArgs gemv_args(const Weight & w, int T, float * y, int ldy, int col0,
 
 void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias) {
     if (!gemv_can(w, x, T))
-        throw std::runtime_error("gemv: needs Q4_K or Q8_0 tiles, the code buffers of their conversion and at most " + std::to_string(GEMV_MAX_T) + " tokens");
+        throw std::runtime_error("gemv: needs Q4_K, Q6_K or Q8_0 tiles, the code buffers of their conversion and at most " + std::to_string(GEMV_MAX_T) + " tokens");
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
     a.codes = x.qc; a.d = x.qd; a.bsums = x.qbs;
     launch_gemv_src<SRC_CODES>(s, w.type, a);
@@ -351,7 +413,7 @@ void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int 
 
 void gemv_norm(hipStream_t s, const Weight & w, const float * x, const float * norm_w, float eps, const int32_t * rows, int T,
                float * y, int ldy, int col0, int mode, const float * bias) {
-    if (!gemv_can_weight(w, T) || !x || !norm_w) throw std::runtime_error("gemv_norm: needs Q4_K or Q8_0 tiles, the rows and the norm weights");
+    if (!gemv_can_weight(w, T) || !x || !norm_w) throw std::runtime_error("gemv_norm: needs Q4_K, Q6_K or Q8_0 tiles, the rows and the norm weights");
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
     a.xin = x; a.norm_w = norm_w; a.rows = rows; a.eps = eps;
     launch_gemv_src<SRC_NORM>(s, w.type, a);
@@ -360,7 +422,7 @@ void gemv_norm(hipStream_t s, const Weight & w, const float * x, const float * n
 void gemv_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, int T, float * y, int ldy, int col0, int mode) {
     if (group <= 0) group = w.K;
     if (!gemv_can_weight(w, T) || !gu || w.K % group != 0 || group % 8 != 0)
-        throw std::runtime_error("gemv_swiglu: needs Q4_K or Q8_0 tiles and gate / up rows in groups that divide the width");
+        throw std::runtime_error("gemv_swiglu: needs Q4_K, Q6_K or Q8_0 tiles and gate / up rows in groups that divide the width");
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, nullptr);
     a.xin = gu; a.group = group;
     launch_gemv_src<SRC_SWIGLU>(s, w.type, a);

@@ -2094,14 +2094,14 @@ __global__ __launch_bounds__(256) void k_attention_combine(CombineArgs a) {
         }
         if (a.out.qc) {      // the blocks themselves, for the integer matrix-vector kernel (see store_codes8)
             const int i0 = (int)c0, i1 = (int)c1;
-            int sum = i0 + i1;
+            int sum = i0 + i1;          // of 16 codes: eight lanes
 #pragma unroll
-            for (int o = 1; o < 16; o <<= 1) sum += __shfl_xor(sum, o, 64);
+            for (int o = 1; o < 8; o <<= 1) sum += __shfl_xor(sum, o, 64);
             if (mine) {
                 int8_t * grp = a.out.qc + (size_t)t * QD + (k & ~7);
                 grp[act_code_pos(k & 7)] = (int8_t)i0;
                 grp[act_code_pos((k & 7) + 1)] = (int8_t)i1;
-                if ((lane & 15) == 0) a.out.qbs[(size_t)t * (QD >> 5) + (k >> 5)] = (int16_t)sum;
+                if ((lane & 7) == 0) a.out.qbs[(size_t)t * (QD >> 4) + (k >> 4)] = (int16_t)sum;
                 if (wave == w0 && lane == 0) a.out.qd[(size_t)t * (QD >> 8) + (k >> 8)] = d;
             }
         }

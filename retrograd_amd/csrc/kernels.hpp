@@ -81,8 +81,8 @@ struct Act {
     // A producer can leave the blocks of the conversion themselves as well, for the integer matrix-vector
     // kernel that multiplies very small steps (gemv). Q8_K: the int8 codes [token][K], the eight codes of a
     // group k / 8 in the order 0 4 1 5 2 6 3 7 (act_code_pos; the order in which a Q4_K tile's nibbles unpack
-    // into bytes); the block scales 1 / iscale, f32 [token][K / 256]; and the sums of the codes of every 32,
-    // int16 [token][K / 32]. Q8_0: the codes in element order, the scales (f16 values) as f32 [token][K / 32],
+    // into bytes); the block scales 1 / iscale, f32 [token][K / 256]; and the sums of the codes of every 16,
+    // int16 [token][K / 16] (ggml's bsums). Q8_0: the codes in element order, the scales (f16 values) as f32 [token][K / 32],
     // no sums.
     int8_t * qc = nullptr;
     float * qd = nullptr;

@@ -105,7 +105,7 @@ int retro_kernel_gemv_fused(int32_t kind, int32_t type, const uint8_t * raw, int
         if ((kind != 1 && kind != 2) || n_tokens < 1 || n_tokens > rk::GEMV_MAX_T || k <= 0 || k % 256 != 0 || n_rows <= 0 || n_rows % 16 != 0)
             throw std::runtime_error("gemv_fused: kind 1 (RMSNorm) or 2 (SwiGLU), whole tiles and super-blocks, at most " + std::to_string(rk::GEMV_MAX_T) + " tokens");
         if (kind == 1 && !norm_w) throw std::runtime_error("gemv_fused: the RMSNorm needs its weights");
-        if (type != rk::WT_Q4_K && type != rk::WT_Q8_0 && type != rk::WT_Q6_K) throw std::runtime_error("gemv_fused: Q4_K, Q6_K or Q8_0 rows");
+        if (type != rk::WT_Q4_K && type != rk::WT_Q5_K && type != rk::WT_Q6_K && type != rk::WT_Q8_0) throw std::runtime_error("gemv_fused: Q4_K, Q5_K, Q6_K or Q8_0 rows");
         const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
         const size_t in_floats = (size_t)n_tokens * k * (kind == 2 ? 2 : 1);
         DevBuf d_raw, d_packed, d_x, d_w, d_xh, d_sums, d_codes, d_scales, d_bsums, d_y;
@@ -242,8 +242,8 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
         // mode 4: the integer matrix-vector kernel over pseudo-random Q8_K blocks (Q4_K, at most GEMV_MAX_T tokens)
         DevBuf d_codes, d_scales, d_bsums;
         if (mode == 4) {
-            if ((type != rk::WT_Q4_K && type != rk::WT_Q8_0 && type != rk::WT_Q6_K) || n_tokens > rk::GEMV_MAX_T)
-                throw std::runtime_error("matmul_time: the integer kernel takes Q4_K, Q6_K or Q8_0 and at most " + std::to_string(rk::GEMV_MAX_T) + " tokens");
+            if ((type != rk::WT_Q4_K && type != rk::WT_Q5_K && type != rk::WT_Q6_K && type != rk::WT_Q8_0) || n_tokens > rk::GEMV_MAX_T)
+                throw std::runtime_error("matmul_time: the integer kernel takes Q4_K, Q5_K, Q6_K or Q8_0 and at most " + std::to_string(rk::GEMV_MAX_T) + " tokens");
             std::vector<uint8_t> codes((size_t)n_tokens * k);
             uint32_t state = 0x85ebca6bu;
             for (uint8_t & c : codes) { state = state * 1664525u + 1013904223u; c = (uint8_t)(state >> 24); }

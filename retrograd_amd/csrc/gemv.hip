@@ -26,6 +26,10 @@
 // move them above the nibbles of the two byte dwords, which costs about twice the Q4_K kernel's vector instructions
 // per weight - still fewer than the tile kernel spends, and without its four matrix instructions per step.
 //
+// Q5_K (activations Q8_K; the main type of a Q5_K_M file): the Q4_K formula with 5-bit codes. The tile is the Q4_K
+// tile of the low nibbles followed by one dword of fifth bits per k-half and lane (see k_repack_q4k); a shift by the
+// k-step and two masked shifts per byte dword put them above the nibbles.
+//
 // Q8_0 (activations Q8_0):
 //   sum_k w[n][k] x[k] = sum over blocks of 32 of  (d_w d_x) * sum_{k in block} q_k c_k
 // The Q8_0 tile (16 x 8 f16 scales, then four 1 KiB loads in which lane (r, g) of load q holds columns 8g .. 8g + 8
@@ -60,6 +64,8 @@ template <> struct GemvTile<WT_Q8_0> { static constexpr int BYTES = 4352, LOADS 
 // Q6_K: register set = the row's sixteen scales | low nibbles of the two k-halves | top bits of the two k-halves
 // (8 bytes a lane each, held as one 16-byte word) | d
 template <> struct GemvTile<WT_Q6_K> { static constexpr int BYTES = 3360, LOADS = 3, QUANT = AQ_Q8_K; };
+// Q5_K: the two loads of low nibbles; the two dwords of fifth bits travel apart (fifth[])
+template <> struct GemvTile<WT_Q5_K> { static constexpr int BYTES = 2816, LOADS = 2, QUANT = AQ_Q8_K; };
 
 // WT: the weight type. NT: tokens held (rows of the step beyond a.T read as zeros). PER: super-blocks of a tile per
 // wave; a workgroup has nw waves (PER 2: half the row's super-blocks; wider rows: 16), wave w takes super-blocks
@@ -78,7 +84,7 @@ template <> struct GemvTile<WT_Q6_K> { static constexpr int BYTES = 3360, LOADS 
 template <int WT, int NT, int PER, int SRC>
 __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
     using Tile = GemvTile<WT>;
-    constexpr bool Q4 = WT == WT_Q4_K, Q6 = WT == WT_Q6_K, K8 = Tile::QUANT == AQ_Q8_K;
+    constexpr bool Q5 = WT == WT_Q5_K, Q4 = WT == WT_Q4_K || Q5, Q6 = WT == WT_Q6_K, K8 = Tile::QUANT == AQ_Q8_K;
     extern __shared__ __align__(16) uint8_t lds[];
     const int K = a.K, nsb = K >> 8;
     const int nd = K8 ? nsb : (K >> 5);
@@ -93,6 +99,7 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
     // two super-blocks are held at a time: u0 and u0 + 1 of the wave's PER
     u4 hdr[2], q[2][Tile::LOADS];
     uint16_t dq6[2] = {0, 0};          // Q6_K: the row's d
+    uint32_t fifth[2][2] = {{0, 0}, {0, 0}};      // Q5_K: the fifth bits of the two k-halves
     auto request = [&](int tile, int u0) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
@@ -109,6 +116,10 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
                 } else {
 #pragma unroll
                     for (int i = 0; i < Tile::LOADS; ++i) q[u][i] = *(const u4 *)(tp + 256 + i * 1024 + lane * 16);
+                    if constexpr (Q5) {
+                        fifth[u][0] = *(const uint32_t *)(tp + 2304 + lane * 4);
+                        fifth[u][1] = *(const uint32_t *)(tp + 2560 + lane * 4);
+                    }
                 }
             }
         }
@@ -210,7 +221,13 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const uint32_t wq = j == 0 ? q[u][h].x : (j == 1 ? q[u][h].y : (j == 2 ? q[u][h].z : q[u][h].w));
-                    const int lo = (int)(wq & 0x0F0F0F0Fu), hi = (int)((wq >> 4) & 0x0F0F0F0Fu);
+                    int lo = (int)(wq & 0x0F0F0F0Fu), hi = (int)((wq >> 4) & 0x0F0F0F0Fu);
+                    if constexpr (Q5) {
+                        // after the shift by the k-step: the fifth bits of elements 0 4 | 2 6 | 1 5 | 3 7 at bits 0 1 | 8 9 | 16 17 | 24 25
+                        const uint32_t f = fifth[u][h] >> (2 * j);
+                        lo |= (int)(((f << 4) & 0x00100010u) | ((f << 11) & 0x10001000u));
+                        hi |= (int)(((f >> 4) & 0x00100010u) | ((f << 3) & 0x10001000u));
+                    }
                     const int sc = (int)((S.sc[h] >> (8 * j)) & 0xffu);
                     const int k0 = (sb << 8) + ((4 * h + j) << 5) + (g << 3);
 #pragma unroll
@@ -342,7 +359,7 @@ static size_t gemv_lds_bytes(int type, int NT, int NW, int K) {
 }
 
 bool gemv_can_weight(const Weight & w, int T) {
-    return (w.type == WT_Q4_K || w.type == WT_Q8_0 || w.type == WT_Q6_K) && w.packed && T >= 1 && T <= g_gemv_max_t && T <= GEMV_MAX_T
+    return (w.type == WT_Q4_K || w.type == WT_Q5_K || w.type == WT_Q6_K || w.type == WT_Q8_0) && w.packed && T >= 1 && T <= g_gemv_max_t && T <= GEMV_MAX_T
         && w.K % 256 == 0 && w.N % 16 == 0 && w.K > 0 && w.N > 0
         && w.K <= 256 * kGemvMaxSb && gemv_lds_bytes(w.type, GEMV_MAX_T, 16, w.K) <= kGemvMaxLds;
 }
@@ -390,6 +407,7 @@ static void launch_gemv_tokens(hipStream_t s, const GemvArgs & a) {
 template <int SRC>
 static void launch_gemv_src(hipStream_t s, int type, const GemvArgs & a) {
     if (type == WT_Q4_K) launch_gemv_tokens<WT_Q4_K, SRC>(s, a);
+    else if (type == WT_Q5_K) launch_gemv_tokens<WT_Q5_K, SRC>(s, a);
     else if (type == WT_Q6_K) launch_gemv_tokens<WT_Q6_K, SRC>(s, a);
     else launch_gemv_tokens<WT_Q8_0, SRC>(s, a);
 }
@@ -405,7 +423,7 @@ static GemvArgs gemv_args(const Weight & w, int T, float * y, int ldy, int col0,
 
 void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias) {
     if (!gemv_can(w, x, T))
-        throw std::runtime_error("gemv: needs Q4_K, Q6_K or Q8_0 tiles, the code buffers of their conversion and at most " + std::to_string(GEMV_MAX_T) + " tokens");
+        throw std::runtime_error("gemv: needs Q4_K, Q5_K, Q6_K or Q8_0 tiles, the code buffers of their conversion and at most " + std::to_string(GEMV_MAX_T) + " tokens");
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
     a.codes = x.qc; a.d = x.qd; a.bsums = x.qbs;
     launch_gemv_src<SRC_CODES>(s, w.type, a);
@@ -413,7 +431,7 @@ void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int 
 
 void gemv_norm(hipStream_t s, const Weight & w, const float * x, const float * norm_w, float eps, const int32_t * rows, int T,
                float * y, int ldy, int col0, int mode, const float * bias) {
-    if (!gemv_can_weight(w, T) || !x || !norm_w) throw std::runtime_error("gemv_norm: needs Q4_K, Q6_K or Q8_0 tiles, the rows and the norm weights");
+    if (!gemv_can_weight(w, T) || !x || !norm_w) throw std::runtime_error("gemv_norm: needs Q4_K, Q5_K, Q6_K or Q8_0 tiles, the rows and the norm weights");
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
     a.xin = x; a.norm_w = norm_w; a.rows = rows; a.eps = eps;
     launch_gemv_src<SRC_NORM>(s, w.type, a);
@@ -422,7 +440,7 @@ void gemv_norm(hipStream_t s, const Weight & w, const float * x, const float * n
 void gemv_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, int T, float * y, int ldy, int col0, int mode) {
     if (group <= 0) group = w.K;
     if (!gemv_can_weight(w, T) || !gu || w.K % group != 0 || group % 8 != 0)
-        throw std::runtime_error("gemv_swiglu: needs Q4_K, Q6_K or Q8_0 tiles and gate / up rows in groups that divide the width");
+        throw std::runtime_error("gemv_swiglu: needs Q4_K, Q5_K, Q6_K or Q8_0 tiles and gate / up rows in groups that divide the width");
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, nullptr);
     a.xin = gu; a.group = group;
     launch_gemv_src<SRC_SWIGLU>(s, w.type, a);

@@ -143,7 +143,7 @@ def test_tile_matmul_exact_on_integer_data():
 @pytest.mark.parametrize("n,k,T", [(16, 256, 1), (48, 512, 2), (2064, 256, 2), (64, 1024, 1), (256, 4096, 1), (32, 8192, 2),
                                    (128, 14336, 2), (4096, 4096, 2), (1024, 14336, 1), (320, 16384, 2), (16, 8448, 1),
                                    (64, 18944, 2), (48, 24576, 1), (112, 3584, 2)])
-@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0, gw.GGML_Q6_K])
+@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0, gw.GGML_Q6_K, gw.GGML_Q5_K])
 def test_integer_matvec_matches_decoded_blocks(t, n, k, T):
     # The kernel of very small steps under the ggml arithmetic: integer products of the stored codes with the
     # Q8_K codes of the rows. Its sums are those of the converted values times the decoded weights, so the
@@ -212,9 +212,24 @@ def test_integer_matvec_exact_on_integer_data_and_refusals():
         E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x, use_tiles=2, ggml_activations=True, integer=True)
     with pytest.raises(E.EngineError, match="at most 2 tokens"):
         E.kernel_matmul(gw.GGML_Q4_K, raw, n, k, x[:1], use_tiles=2, integer=True)      # the exact arithmetic has no codes
-    q5, _ = _weights(gw.GGML_Q5_K, 16, 256, seed=1)
-    with pytest.raises(E.EngineError, match="does not take this matrix"):
-        E.kernel_matmul(gw.GGML_Q5_K, q5, 16, 256, x[:1, :256], use_tiles=2, ggml_activations=True, integer=True)
+    # Q5_K: the same with a fifth bit per code (blocks of 176 bytes: d, dmin, scales, 32 bytes of fifth bits, nibbles)
+    b5 = rng.integers(0, 256, (n, k // 256, 176), dtype=np.uint8)
+    b5[..., 0:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)
+    b5[..., 2:4] = np.frombuffer(np.float16(0.25).tobytes(), np.uint8)
+    raw5 = b5.reshape(n, -1)
+    dense5 = np.stack([oracle.decode_row(gw.GGML_Q5_K, raw5[i], k) for i in range(n)]).astype(np.float64)
+    for T in (1, 2):
+        x = rng.integers(-4, 5, (T, k)).astype(np.float32)
+        x[:, ::32] = rng.choice([-127.0, 127.0], (T, k // 32))
+        got = E.kernel_matmul(gw.GGML_Q5_K, raw5, n, k, x, use_tiles=2, ggml_activations=True, integer=True)
+        assert np.array_equal(got.astype(np.float64), x.astype(np.float64) @ dense5.T), T
+    for e in (0, 1, 2, 3, 4, 5, 6, 7, 8, 31, 32, 39, 64, 100, 255, 256, 767):
+        one = np.zeros((1, k), np.float32)
+        one[0, e] = -127.0
+        got = E.kernel_matmul(gw.GGML_Q5_K, raw5, n, k, one, use_tiles=2, ggml_activations=True, integer=True)
+        assert np.array_equal(got[0].astype(np.float64), -127.0 * dense5[:, e]), e
+    with pytest.raises(E.EngineError, match="takes Q8_K or Q8_0 conversions"):      # an F16 matrix has none
+        E.kernel_matmul(gw.GGML_F16, np.zeros((16, 512), np.uint8), 16, 256, x[:1, :256], use_tiles=0, ggml_activations=True, integer=True)
 
 
 def test_integer_matvec_q6k_exact_for_every_code_and_scale():
@@ -242,7 +257,7 @@ def test_integer_matvec_q6k_exact_for_every_code_and_scale():
         assert np.array_equal(got[0].astype(np.float64), -127.0 * dense[:, e]), e
 
 
-@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0, gw.GGML_Q6_K])
+@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0, gw.GGML_Q6_K, gw.GGML_Q5_K])
 @pytest.mark.parametrize("kind", [1, 2])
 @pytest.mark.parametrize("n,k,T", [(64, 4096, 1), (64, 4096, 2), (32, 512, 1), (48, 1024, 2), (32, 14336, 1), (16, 14336, 2),
                                    (16, 8448, 2), (32, 2048, 1), (32, 3584, 1), (16, 18944, 1)])

@@ -139,7 +139,7 @@ def test_ggml_arithmetic_follows_the_oracle_as_closely_as_its_rounding_allows(mo
     eng.close()
 
 
-@pytest.mark.parametrize("key", ["llama-q4k", "llama-q4k-hd128", "llama-q4k-m-1024", "qwen2-q8", "tiny-llama-q8", "llama-q6k", "qwen2-q4k-m"])
+@pytest.mark.parametrize("key", ["llama-q4k", "llama-q4k-hd128", "llama-q4k-m-1024", "qwen2-q8", "tiny-llama-q8", "llama-q6k", "qwen2-q4k-m", "llama-q5k-m"])
 def test_small_steps_under_the_ggml_arithmetic_take_the_integer_kernel(models, key, monkeypatch):
     """Steps of one or two tokens under RETRO_ACTIVATIONS=ggml multiply their Q4_K matrices by integer products of
     the stored codes with the rows' Q8_K codes (Q6_K matrices of the same model stay on the tile kernels), and where

@@ -161,9 +161,29 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
             }
         }
     } else {
-        // make the blocks here: eight consecutive values per thread, the threads of a block together (requantise8)
-        Act lout;
-        lout.K = K; lout.quant = Tile::QUANT; lout.qc = l_codes; lout.qd = l_d; lout.qbs = l_bsums;
+        // make the blocks here: eight consecutive values per thread, the threads of a block together (requantise8);
+        // what store_codes8 writes for a producer, written to LDS (through LDS pointers, so that the stores are LDS
+        // instructions and not flat ones, whose completion would be counted with the weight requests in flight)
+        auto store_lds = [&](const float (&c)[8], float d, int t, int k) {
+            uint32_t w0 = 0, w1 = 0;
+            int sum = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int q8 = (int)c[i];
+                sum += q8;
+                const uint32_t byte = (uint32_t)q8 & 0xffu;
+                const int pos = K8 ? act_code_pos(i) : i;
+                if (pos < 4) w0 |= byte << (8 * pos); else w1 |= byte << (8 * (pos - 4));
+            }
+            *(uint2 *)(l_codes + t * K + k) = make_uint2(w0, w1);
+            if (K8) {
+                sum += __shfl_xor(sum, 1, 64);
+                if ((tid & 1) == 0) l_bsums[t * (K >> 4) + (k >> 4)] = (int16_t)sum;
+                if ((k & 255) == 0) l_d[t * nsb + (k >> 8)] = d;
+            } else if ((tid & 3) == 0) {
+                l_d[t * nd + (k >> 5)] = d;
+            }
+        };
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const float * xr = row_of(t);
@@ -202,7 +222,7 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
                     for (int i = 0; i < 8; ++i) v[i] = (gv[i] / (1.0f + __expf(-gv[i]))) * uv[i];
                 }
                 const float d = requantise8(v, Tile::QUANT, c);
-                store_codes8(c, d, lout, t, k, tid & 3);
+                store_lds(c, d, t, k);
             }
         }
     }

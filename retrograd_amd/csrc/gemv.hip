@@ -203,7 +203,7 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
                 float total = 0.0f;
                 for (int i = 0; i < nw; ++i) total += l_red[i];
                 scale = 1.0f / sqrtf(total / (float)K + a.eps);
-                __syncthreads();                   // l_red is written again for the next row and by the tiles
+                if (t + 1 < NT) __syncthreads();   // l_red is written again for the next row (the tiles write it behind the barrier below)
             }
             for (int k = tid * 8; k < K; k += nthreads * 8) {
                 f4 in[4];

@@ -260,7 +260,7 @@ def test_integer_matvec_q6k_exact_for_every_code_and_scale():
 @pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0, gw.GGML_Q6_K, gw.GGML_Q5_K])
 @pytest.mark.parametrize("kind", [1, 2])
 @pytest.mark.parametrize("n,k,T", [(64, 4096, 1), (64, 4096, 2), (32, 512, 1), (48, 1024, 2), (32, 14336, 1), (16, 14336, 2),
-                                   (16, 8448, 2), (32, 2048, 1), (32, 3584, 1), (16, 18944, 1)])
+                                   (16, 8448, 2), (32, 2048, 1), (32, 3584, 1), (16, 18944, 1), (16, 256, 1), (16, 256, 2), (32, 768, 2)])
 def test_integer_matvec_with_its_producer_fused(t, kind, n, k, T):
     # The Q8_K blocks made by the kernel itself while it stages them (RMSNorm of residual rows, or SwiGLU of a gate/up
     # product) against the producer's own launch followed by the kernel, and against the CPU: the norm / SiLU in

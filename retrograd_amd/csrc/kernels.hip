@@ -2003,12 +2003,22 @@ __global__ __launch_bounds__(256) void k_attention_combine(CombineArgs a) {
             M = m_new;
             const float w_s = m_s == -INFINITY ? 0.0f : exp2f(m_s - M);
             L += wave_sum(w_s * l_s);
-            for (int s = 0; s < n; ++s) {
-                const float w = __shfl(w_s, s, 64);
-                if (e0 < a.hd) {
-                    const float2 pv = *(const float2 *)(a.partial + ((size_t)(item0 + s0 + s) * 16 + col) * stride + 2 + e0);
-                    v0 = fmaf(w, pv.x, v0);
-                    v1 = fmaf(w, pv.y, v1);
+            // the splits' outputs eight at a time: their loads are in flight together, the sums keep the split order
+            for (int s1 = 0; s1 < n; s1 += 8) {
+                float2 pv[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    pv[u] = make_float2(0.0f, 0.0f);
+                    if (s1 + u < n && e0 < a.hd)
+                        pv[u] = *(const float2 *)(a.partial + ((size_t)(item0 + s0 + s1 + u) * 16 + col) * stride + 2 + e0);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (s1 + u < n) {
+                        const float w = __shfl(w_s, s1 + u, 64);
+                        v0 = fmaf(w, pv[u].x, v0);
+                        v1 = fmaf(w, pv[u].y, v1);
+                    }
                 }
             }
         }

@@ -655,6 +655,64 @@ __global__ __launch_bounds__(256) void k_mm_generic(int type, const uint8_t * __
     }
 }
 
+// F32 rows (the expert router; unquantised heads) for more than a few tokens. The generic kernel gives a wave one
+// output feature and eight tokens, so the activations - eight times the bytes of a weight row - are read once per
+// feature, and its k-chunks of 512 follow one another. Here a workgroup owns EW features and eight tokens, its four
+// waves take the k-chunks in turn (all loads of a launch are in flight at once for K <= 2048), every wave keeps its
+// chunk's activations in registers for the EW features, and the waves' sums meet in LDS in wave order.
+template <int EW>
+__global__ __launch_bounds__(256) void k_mm_f32_rows(const float * __restrict__ wm, const __half * __restrict__ x, int K, int N, int T,
+                                                     float * y, int ldy, int col0, int mode, const float * bias) {
+    __shared__ float part[4][EW][8];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * EW;
+    const int t0 = blockIdx.y * 8;
+    float acc[EW][8];
+#pragma unroll
+    for (int e = 0; e < EW; ++e)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[e][j] = 0.0f;
+    for (int k = wave * 512 + lane * 8; k < K; k += 2048) {
+        float xv[8][8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int t = min(t0 + j, T - 1);
+            const h8 hi = load_h8(x + act_at(t, k, 0, K)), lo = load_h8(x + act_at(t, k, 1, K));
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[j][i] = (float)hi[i] + (float)lo[i];
+        }
+#pragma unroll
+        for (int e = 0; e < EW; ++e) {
+            if (n0 + e < N) {
+                const f4 wa = *(const f4 *)(wm + (size_t)(n0 + e) * K + k), wb = *(const f4 *)(wm + (size_t)(n0 + e) * K + k + 4);
+                const float w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) acc[e][j] = fmaf(w[i], xv[j][i], acc[e][j]);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < EW; ++e) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float v = wave_sum(acc[e][j]);
+            if (lane == 0) part[wave][e][j] = v;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < EW * 8) {
+        const int e = threadIdx.x >> 3, j = threadIdx.x & 7;
+        if (n0 + e < N && t0 + j < T) {
+            const float v = ((part[0][e][j] + part[1][e][j]) + part[2][e][j]) + part[3][e][j];
+            float * p = y + (size_t)(t0 + j) * ldy + col0 + n0 + e;
+            const float o = v + (bias ? bias[n0 + e] : 0.0f);
+            *p = mode == MM_ADD ? *p + o : o;
+        }
+    }
+}
+
 void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0,
                     int mode, const float * bias) {
     if (!w.raw) throw std::runtime_error("matmul_generic: the weight has no raw layout");
@@ -662,6 +720,14 @@ void matmul_generic(hipStream_t s, const Weight & w, const Act & x, int T, float
     if (T <= 0) return;
     const Act xo = x.operand(w.type);
     if (!xo.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
+    if (w.type == WT_F32 && w.K % 8 == 0 && ((uintptr_t)w.raw & 15) == 0 && T > 8) {
+        // several token groups (a step of few tokens keeps the generic kernel's feature per wave for the parallelism)
+        constexpr int EW = 4;
+        hipLaunchKernelGGL(k_mm_f32_rows<EW>, dim3((w.N + EW - 1) / EW, (T + 7) / 8), dim3(256), 0, s, (const float *)w.raw,
+                           xo.x, w.K, w.N, T, y, ldy, col0, mode, bias);
+        check_launch("matmul_generic");
+        return;
+    }
     hipLaunchKernelGGL(k_mm_generic, dim3((w.N + 3) / 4, (T + 7) / 8), dim3(256), 0, s, w.type, w.raw, row_bytes(w.type, w.K),
                        xo.x, w.K, w.N, T, y, ldy, col0, mode, bias, xo.faithful ? w.type : WT_F32);
     check_launch("matmul_generic");

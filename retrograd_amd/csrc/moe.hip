@@ -511,22 +511,38 @@ __global__ __launch_bounds__(1024) void k_moe_group(const int32_t * __restrict__
     __shared__ int base[256];
     __shared__ int wcnt[16][256];
     __shared__ int total_pad;
+    __shared__ int wsum[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid < 256) cnt[tid] = 0;
     for (int i = tid; i < 16 * 256; i += 1024) (&wcnt[0][0])[i] = 0;
     __syncthreads();
     for (int p = tid; p < n_pairs; p += 1024) atomicAdd(&cnt[sel[p]], 1);
     __syncthreads();
-    if (tid == 0) {
-        int at = 0;
-        for (int e = 0; e < n_expert; ++e) {
-            off_pad[e] = at;
-            base[e] = at;
-            expert_n[e] = cnt[e];
-            at += (cnt[e] + 15) & ~15;
+    // exclusive prefix sums of the padded counts: a scan inside each of the first four waves, then the waves' totals
+    int padded = 0, incl = 0;
+    if (tid < 256) {
+        padded = tid < n_expert ? (cnt[tid] + 15) & ~15 : 0;
+        incl = padded;
+        for (int o = 1; o < 64; o <<= 1) {
+            const int up = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += up;
         }
-        off_pad[n_expert] = at;
-        total_pad = at;
+        if (lane == 63) wsum[wave] = incl;
+    }
+    __syncthreads();
+    if (tid < 256) {
+        int before = 0;
+        for (int w = 0; w < wave; ++w) before += wsum[w];
+        const int at = before + incl - padded;
+        if (tid < n_expert) {
+            off_pad[tid] = at;
+            base[tid] = at;
+            expert_n[tid] = cnt[tid];
+        }
+        if (tid == n_expert - 1) {
+            off_pad[n_expert] = at + padded;
+            total_pad = at + padded;
+        }
     }
     __syncthreads();
     for (int q = tid; q < total_pad; q += 1024) tok_of_q[q] = -1;

@@ -93,6 +93,30 @@ def test_generic_matmul_every_storage_type(t, k, ggml):
         assert np.abs(want - _ref(t, dense, x, False)).max() > 1e-4 * np.abs(want).max()     # the conversion is visible
 
 
+@pytest.mark.parametrize("ggml", [False, True])
+@pytest.mark.parametrize("n,k,T", [(128, 2048, 128), (5, 512, 9), (130, 2304, 33), (7, 4104, 17), (16, 8, 64), (33, 1024, 512)])
+def test_f32_rows_over_many_tokens(n, k, T, ggml):
+    # F32 matrices (the expert router) over more than eight tokens have a kernel of their own: a workgroup per four
+    # features and eight tokens. Ragged feature and token counts, rows shorter and longer than its four k-chunks;
+    # up to eight tokens the generic kernel still runs and must give the same numbers to rounding.
+    print("case", n, k, T, ggml, flush=True)
+    rng = np.random.default_rng(n + k + T)
+    w = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    raw = w.view(np.uint8).reshape(n, -1)
+    x = rng.standard_normal((T, k)).astype(np.float32)
+    want = x.astype(np.float64) @ w.astype(np.float64).T
+    scale = np.abs(want).max()
+    bias = rng.standard_normal(n).astype(np.float32)
+    got = E.kernel_matmul(gw.GGML_F32, raw, n, k, x, use_tiles=False, ggml_activations=ggml, bias=bias)
+    assert np.abs(got - (want + bias)).max() <= 2e-5 * scale + 1e-6
+    y0 = rng.standard_normal((T, n)).astype(np.float32)
+    got = E.kernel_matmul(gw.GGML_F32, raw, n, k, x, use_tiles=False, ggml_activations=ggml, accumulate_into=y0)
+    assert np.abs(got - (want + y0)).max() <= 3e-5 * scale + 1e-6
+    few = E.kernel_matmul(gw.GGML_F32, raw, n, k, x[:8], use_tiles=False, ggml_activations=ggml)
+    many = E.kernel_matmul(gw.GGML_F32, raw, n, k, x, use_tiles=False, ggml_activations=ggml)
+    assert np.abs(few - many[:8]).max() <= 2e-6 * scale + 1e-7
+
+
 def test_matmul_bias_and_accumulate():
     t, n, k, T = gw.GGML_Q4_K, 64, 512, 20
     raw, dense = _weights(t, n, k, seed=5)

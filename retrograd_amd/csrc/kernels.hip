@@ -1269,6 +1269,7 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
                                                PackBuffers o) {
     __shared__ int scratch[16];
     __shared__ int carry[3];
+    __shared__ int len_count[MAX_SPLIT_PAGES + 1], len_base[MAX_SPLIT_PAGES + 1];
     for (int i = threadIdx.x; i < n_upd; i += 1024) table[(size_t)upd[i].slot * max_pages + upd[i].index] = upd[i].page;
     if (threadIdx.x == 0) { carry[0] = 0; carry[1] = 0; carry[2] = 0; }
     __syncthreads();
@@ -1339,18 +1340,39 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
     // the work items of every (tile, kv head), from the tile and token arrays written above
     __threadfence_block();
     __syncthreads();
-    for (int pair = threadIdx.x; pair < carry[0] * n_kv; pair += 1024) {
-        const int tile = pair / n_kv, h = pair % n_kv;
-        const int t0 = o.tile_t0[tile], nq = o.tile_nq[tile], ns = o.tile_nsplit[tile];
-        const int kv_begin = o.tile_kv_begin[tile], pos0 = o.pos[t0], slot = o.seq[t0];
-        const int item0 = o.tile_item0[tile] + h * ns;
-        const int hi = pos0 + nq;
-        for (int sp = 0; sp < ns; ++sp) {
-            const int page_first = kv_begin / PAGE + sp * o.split_pages;
-            const int page_end = min((hi - 1) / PAGE + 1, page_first + o.split_pages);
-            o.item_a[item0 + sp] = make_int4(t0, nq, h, slot);
-            o.item_b[item0 + sp] = make_int4(pos0, kv_begin, page_first, page_end - page_first);
+    // The descriptors are stored longest first (by pages): workgroups start in index order, so the items that start
+    // last - the tail of the launch, when few waves are left to hide each other's latency - are the short ones. An
+    // item keeps its number (a tile's items of a kv head are consecutive numbers, which the merge relies on) inside
+    // its descriptor; only the place of the descriptor changes. Two passes: count the items of every length, then
+    // place them (the order among items of one length is whatever the atomics give: it changes no result).
+    for (int i = threadIdx.x; i <= MAX_SPLIT_PAGES; i += 1024) len_count[i] = 0;
+    __syncthreads();
+    for (int pass = 0; pass < 2; ++pass) {
+        for (int pair = threadIdx.x; pair < carry[0] * n_kv; pair += 1024) {
+            const int tile = pair / n_kv, h = pair % n_kv;
+            const int t0 = o.tile_t0[tile], nq = o.tile_nq[tile], ns = o.tile_nsplit[tile];
+            const int kv_begin = o.tile_kv_begin[tile], pos0 = o.pos[t0], slot = o.seq[t0];
+            const int item0 = o.tile_item0[tile] + h * ns;
+            const int hi = pos0 + nq;
+            for (int sp = 0; sp < ns; ++sp) {
+                const int page_first = kv_begin / PAGE + sp * o.split_pages;
+                const int page_end = min((hi - 1) / PAGE + 1, page_first + o.split_pages);
+                const int len = min(max(page_end - page_first, 0), MAX_SPLIT_PAGES);
+                if (pass == 0) {
+                    atomicAdd(&len_count[len], 1);
+                } else {
+                    const int at = atomicAdd(&len_base[len], 1);
+                    o.item_a[at] = make_int4(t0, nq | (h << 8), item0 + sp, slot);
+                    o.item_b[at] = make_int4(pos0, kv_begin, page_first, page_end - page_first);
+                }
+            }
         }
+        __syncthreads();
+        if (pass == 0 && threadIdx.x == 0) {
+            int at = 0;
+            for (int len = MAX_SPLIT_PAGES; len >= 0; --len) { len_base[len] = at; at += len_count[len]; }
+        }
+        __syncthreads();
     }
     if (threadIdx.x == 0) {
         const RowDesc last = rows[n_rows - 1];
@@ -1730,12 +1752,13 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
     constexpr bool Q8 = KVQ != KV_F16;       // a quantised cache of either width
     constexpr int KS = HD / 32;     // k-steps of QK^T
     constexpr int DT = HD / 16;     // dim tiles of PV
-    const int item = blockIdx.x;
     const int lane = threadIdx.x;
     const int c = lane & 15, g = lane >> 4;
-    // what the packing kernel left for this item: one round trip instead of a search over the tiles
-    const int4 ia = a.item_a[item], ib = a.item_b[item];
-    const int t0 = ia.x, nq = ONE ? 1 : ia.y, h = ia.z, slot = ia.w;
+    // what the packing kernel left for the workgroup's place (the longest items come first): one round trip instead
+    // of a search over the tiles; the item's own number, which places its partial results, is part of it
+    const int4 ia = a.item_a[blockIdx.x], ib = a.item_b[blockIdx.x];
+    const int item = ia.z;
+    const int t0 = ia.x, nq = ONE ? 1 : (ia.y & 0xff), h = ia.y >> 8, slot = ia.w;
     const int kv_begin = ib.y;
     const int cc = SPLIT ? (c & 7) : c;            // the column's (token, head) index
     const int qi = cc / a.G, gi = cc % a.G;

@@ -275,7 +275,7 @@ struct PackBuffers {       // device arrays, sized for n_batch tokens / rows
     int32_t * tok_tile;    // [T] tile of each token
     int4 * tok_merge;      // [T] first work item of the token's tile, its KV splits, the token's index in the tile
     // attention work items (one wave each), everything a wave needs in two 16-byte loads:
-    int4 * item_a;         // [n_items] first flat token of the tile, tokens in the tile, kv head, slot
+    int4 * item_a;         // [n_items, longest first] first flat token of the tile, tokens in the tile | kv head << 8, the item's number, slot
     int4 * item_b;         // [n_items] position of the first token, first resident position of the slot,
                            //           first page index of this split, pages in this split
     float * rope_cos;      // [T][rope_dim/2]

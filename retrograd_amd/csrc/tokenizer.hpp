@@ -19,11 +19,12 @@
 //
 //   * special-token texts split the input as above; nothing is put in front of a stretch;
 //   * a stretch is cut into words by the pattern that tokenizer.ggml.pre names, matched by hand here
-//     (split_words): the Llama 3 pattern ("llama-bpe", "llama3", "llama-v3", "falcon3": case-insensitive
+//     (split_words): the Llama 3 pattern ("llama-bpe", "llama3", "llama-v3", "falcon3", "falcon-h1", "pixtral",
+//     "midm-2.0", "lfm2": case-insensitive
 //     contractions, a letter run with one optional leading character that is neither a letter, a number nor a
 //     line break, numbers in runs of at most three, punctuation with an optional leading space and trailing
 //     line breaks, line-break and space runs), the Qwen 2 pattern ("qwen2", "deepseek-r1-qwen": the same with
-//     numbers one digit at a time) and GPT-2's own ("gpt-2", "gpt2": case-sensitive contractions, an optional
+//     numbers one digit at a time) and GPT-2's own ("gpt-2", "gpt2", "phi-2": case-sensitive contractions, an optional
 //     space before a letter, number or punctuation run). Another tokenizer.ggml.pre is refused;
 //   * the bytes of a word are spelled in GPT-2's printable alphabet (bytes_to_unicode) and the adjacent pair of
 //     lowest rank in tokenizer.ggml.merges is merged first, the leftmost on ties, until no pair has a rank;
@@ -67,11 +68,17 @@ struct Tokenizer {
     std::string byte_spelling[256];          // a byte in GPT-2's printable alphabet, as UTF-8
     std::unordered_map<uint32_t, uint8_t> spelled_byte;      // and back
 
+    // The names llama.cpp gives the Llama 3 pattern with its whole-word rule and BOS default (llama-vocab.cpp).
+    bool llama3_family() const {
+        return pre == "llama3" || pre == "llama-v3" || pre == "llama-bpe" || pre == "falcon3" || pre == "falcon-h1"
+            || pre == "pixtral" || pre == "midm-2.0" || pre == "lfm2";
+    }
+
     // The defaults of a vocabulary kind that the file's own keys then override (call before reading them).
     void set_kind_defaults() {
         if (model != "gpt2") return;
         add_space_prefix = false;
-        add_bos = pre == "llama3" || pre == "llama-v3" || pre == "llama-bpe" || pre == "falcon3";
+        add_bos = llama3_family();
         add_eos = false;
     }
 
@@ -84,12 +91,12 @@ struct Tokenizer {
         pattern = P_NONE;
         ignore_merges = false;
         if (model == "gpt2") {
-            if (pre == "llama3" || pre == "llama-v3" || pre == "llama-bpe" || pre == "falcon3") {
+            if (llama3_family()) {
                 pattern = P_LLAMA3;
                 ignore_merges = true;
             } else if (pre == "qwen2" || pre == "deepseek-r1-qwen") {
                 pattern = P_QWEN2;
-            } else if (pre == "gpt-2" || pre == "gpt2") {
+            } else if (pre == "gpt-2" || pre == "gpt2" || pre == "phi-2") {
                 pattern = P_GPT2;
             } else {
                 throw std::runtime_error("the pre-tokeniser pattern \"" + pre + "\" (tokenizer.ggml.pre) is not built: llama-bpe, qwen2 and gpt-2 are");

@@ -104,6 +104,18 @@ def test_ids_equal_the_tokenizers_librarys(harness, kind):
     assert 0 not in [int(x) for x in literal.split()]
 
 
+@pytest.mark.parametrize("alias,of", [("lfm2", "llama-bpe"), ("pixtral", "llama-bpe"), ("falcon-h1", "llama-bpe"), ("midm-2.0", "llama-bpe"),
+                                      ("llama3", "llama-bpe"), ("phi-2", "gpt-2"), ("deepseek-r1-qwen", "qwen2")])
+def test_pattern_names_that_llama_cpp_maps_to_one_pattern_tokenize_alike(harness, alias, of):
+    # llama.cpp's vocabulary loader gives several tokenizer.ggml.pre names the same pattern and defaults
+    # (llama-vocab.cpp); the reference's own CPU fixture model names "lfm2". Same words, same ids, same BOS default.
+    kind = next(k for k in BPE["kinds"] if k["pre"] == of)
+    cases = [(0, int("<|" in c["text"]), c["text"]) for c in kind["cases"]]
+    first, want = _run_bpe(harness, kind, cases, "ids")
+    again, got = _run_bpe(harness, dict(kind, pre=alias), cases, "ids")
+    assert again == first and got == want
+
+
 def test_an_unknown_pattern_is_refused(harness):
     exe, _, d = harness
     kind = dict(BPE["kinds"][0], pre="some-other-pattern")

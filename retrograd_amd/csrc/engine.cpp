@@ -77,7 +77,9 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
         // (Q8_K / Q8_0 codes, f16 / bf16 rounding); unset or "exact": the f32 values (as f16 hi/lo pairs).
         if (const char * dbg = std::getenv("RETRO_MM_DEBUG")) rk::g_mm_debug = std::atoi(dbg);     // timing experiments
         if (const char * dbg = std::getenv("RETRO_MM_SINGLE")) mm_single_mask_ = std::atoi(dbg);
-        if (const char * f = std::getenv("RETRO_GEMV_FUSE")) gemv_fuse_ = std::atoi(f) != 0;      // 0: producers keep their own launches
+        if (const char * f = std::getenv("RETRO_GEMV_FUSE")) gemv_fuse_ = std::atoi(f) != 0;
+        // ... and the output projection merges at most this many attention splits per kv head itself (0: never)
+        if (const char * f = std::getenv("RETRO_GEMV_MERGE_SPLITS")) merge_max_splits_ = std::max(0, std::min(std::atoi(f), rk::GEMV_COMBINE_MAX_SPLITS));      // 0: producers keep their own launches
         // steps of at most this many tokens go through the integer matrix-vector kernel under the ggml arithmetic (0: never)
         const char * g = std::getenv("RETRO_GEMV_MAX_T");
         rk::g_gemv_max_t = g ? std::max(0, std::min(std::atoi(g), rk::GEMV_MAX_T)) : rk::GEMV_MAX_T;
@@ -1419,6 +1421,17 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
                       k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), n_items, n_tiles,
                       partial_.as<float>(), one_token_rows);
         prof_end(PC_ATTN, pt_);
+        // a single token with few splits: the output projection merges them itself (n_items = kv heads x splits)
+        const int n_split = T == 1 && n_tiles == 1 ? n_items / h.n_head_kv : 0;
+        const bool merge_in_oproj = fuse && n_split >= 1 && n_split <= merge_max_splits_ && n_split * h.n_head_kv == n_items
+                                    && rk::gemv_can_weight(L.wo.w, 1) && L.wo.w.K == QD && L.wo.w.N == E;
+        if (merge_in_oproj) {
+            pt_ = prof_begin(PC_OPROJ);
+            rk::gemv_combine(stream_, L.wo.w, partial_.as<float>(), 0, n_split, h.n_head, h.n_head / h.n_head_kv, h.head_dim, x, E, 0,
+                             rk::MM_ADD);
+            pending = rk::Slices();
+            prof_end(PC_OPROJ, pt_);
+        } else {
         pt_ = prof_begin(PC_COMBINE);
         rk::attention_combine(stream_, partial_.as<float>(), T, sh, pk_, act_q);
         prof_end(PC_COMBINE, pt_);
@@ -1430,6 +1443,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
                            lora_mid_.as<float>());
         }
         prof_end(PC_OPROJ, pt_);
+        }
         if (fuse && h.n_expert == 0 && pending.n == 0 && all_gemv(L.gate_up, E, 2 * F)) {
             pt_ = prof_begin(PC_GATEUP);
             int col = 0;

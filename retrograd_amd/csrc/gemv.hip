@@ -55,8 +55,12 @@ struct GemvArgs {
     const int32_t * rows;      // NORM: row t is xin row rows[t] (null: t)
     float eps;
     int group;                 // SWIGLU: gate c at column (c / group) * 2 group + c % group, up c `group` columns further
+    // SRC_COMBINE: the split partials of the step's single token (what attention_combine merges)
+    const float * partial;     // per (item, column): m (log2 domain), l, head_dim unnormalised outputs
+    int item0, n_split;        // the token's first work item; splits per kv head
+    int att_G, att_hd;         // query heads per kv head, head_dim
 };
-enum : int { SRC_CODES = 0, SRC_NORM = 1, SRC_SWIGLU = 2 };
+enum : int { SRC_CODES = 0, SRC_NORM = 1, SRC_SWIGLU = 2, SRC_COMBINE = 3 };
 
 template <int WT> struct GemvTile;
 template <> struct GemvTile<WT_Q4_K> { static constexpr int BYTES = 2304, LOADS = 2, QUANT = AQ_Q8_K; };
@@ -78,7 +82,8 @@ template <> struct GemvTile<WT_Q5_K> { static constexpr int BYTES = 2816, LOADS 
 // them itself from the residual rows - RMSNorm (the sum of squares in the order k_rmsnorm_act8 adds it, so a row of
 // 4096 gives the same codes bit for bit) and the conversion, straight into LDS - which saves the step a launch of
 // four to five microseconds for about one and a half of redundant work per workgroup. SRC_SWIGLU: likewise
-// silu(gate) * up of the gate/up product's f32 rows. NT is exactly the token count then.
+// silu(gate) * up of the gate/up product's f32 rows. SRC_COMBINE (one token, few splits): the merge of the attention
+// splits - what k_attention_combine computes - for the output projection. NT is exactly the token count then.
 // Dynamic LDS: codes NT * K bytes | scales NT * nd floats (nd = K / 256 or K / 32) | Q8_K: block sums NT * K / 8
 // bytes | 2 * nw * NT * 16 floats.
 template <int WT, int NT, int PER, int SRC>
@@ -141,10 +146,33 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
         }
     };
     f4 first[4];
-    if (SRC != SRC_CODES && tid * 8 < K) load_in(row_of(0), tid * 8, first);
+    if (SRC != SRC_CODES && SRC != SRC_COMBINE && tid * 8 < K) load_in(row_of(0), tid * 8, first);
     int tile = blockIdx.x;
     if (tile < a.n_tiles) request(tile, 0);
 
+    // The blocks a fused source makes: what store_codes8 writes for a producer, written to LDS (through LDS pointers,
+    // so that the stores are LDS instructions and not flat ones, whose completion would be counted with the weight
+    // requests in flight)
+    auto store_lds = [&](const float (&c)[8], float d, int t, int k) {
+        uint32_t w0 = 0, w1 = 0;
+        int sum = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int q8 = (int)c[i];
+            sum += q8;
+            const uint32_t byte = (uint32_t)q8 & 0xffu;
+            const int pos = K8 ? act_code_pos(i) : i;
+            if (pos < 4) w0 |= byte << (8 * pos); else w1 |= byte << (8 * (pos - 4));
+        }
+        *(uint2 *)(l_codes + t * K + k) = make_uint2(w0, w1);
+        if (K8) {
+            sum += __shfl_xor(sum, 1, 64);
+            if ((tid & 1) == 0) l_bsums[t * (K >> 4) + (k >> 4)] = (int16_t)sum;
+            if ((k & 255) == 0) l_d[t * nsb + (k >> 8)] = d;
+        } else if ((tid & 3) == 0) {
+            l_d[t * nd + (k >> 5)] = d;
+        }
+    };
     if (SRC == SRC_CODES) {
         // stage the rows of the step: 16-byte words of codes, scales, dwords of block sums
         for (int i = tid; i < NT * (K >> 4); i += nthreads) {
@@ -160,30 +188,36 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
                 ((uint32_t *)l_bsums)[i] = t < a.T ? ((const uint32_t *)a.bsums)[i] : 0u;
             }
         }
-    } else {
-        // make the blocks here: eight consecutive values per thread, the threads of a block together (requantise8);
-        // what store_codes8 writes for a producer, written to LDS (through LDS pointers, so that the stores are LDS
-        // instructions and not flat ones, whose completion would be counted with the weight requests in flight)
-        auto store_lds = [&](const float (&c)[8], float d, int t, int k) {
-            uint32_t w0 = 0, w1 = 0;
-            int sum = 0;
+    } else if (SRC == SRC_COMBINE) {
+        // eight consecutive dimensions of one query head per thread: the splits' (max, sum) pairs, the weights
+        // 2^(m_s - M), the weighted outputs over the weighted sums, then the conversion as for any other row
+        for (int k = tid * 8; k < K; k += nthreads * 8) {
+            const int head = k / a.att_hd, e0 = k % a.att_hd;
+            const int kvh = head / a.att_G, col = head % a.att_G;
+            const int stride = a.att_hd + 2;
+            const float * base = a.partial + ((size_t)(a.item0 + kvh * a.n_split) * 16 + col) * stride;
+            float M = -INFINITY;
+            for (int sp = 0; sp < a.n_split; ++sp) M = fmaxf(M, base[(size_t)sp * 16 * stride]);
+            float L = 0.0f, v[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (int sp = 0; sp < a.n_split; ++sp) {
+                const float * p = base + (size_t)sp * 16 * stride;
+                const float m_s = p[0];
+                const float w_s = m_s == -INFINITY ? 0.0f : exp2f(m_s - M);
+                L = fmaf(w_s, p[1], L);
+                const float2 o0 = *(const float2 *)(p + 2 + e0), o1 = *(const float2 *)(p + 4 + e0);
+                const float2 o2 = *(const float2 *)(p + 6 + e0), o3 = *(const float2 *)(p + 8 + e0);
+                v[0] = fmaf(w_s, o0.x, v[0]); v[1] = fmaf(w_s, o0.y, v[1]); v[2] = fmaf(w_s, o1.x, v[2]); v[3] = fmaf(w_s, o1.y, v[3]);
+                v[4] = fmaf(w_s, o2.x, v[4]); v[5] = fmaf(w_s, o2.y, v[5]); v[6] = fmaf(w_s, o3.x, v[6]); v[7] = fmaf(w_s, o3.y, v[7]);
+            }
+            const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+            float c[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int q8 = (int)c[i];
-                sum += q8;
-                const uint32_t byte = (uint32_t)q8 & 0xffu;
-                const int pos = K8 ? act_code_pos(i) : i;
-                if (pos < 4) w0 |= byte << (8 * pos); else w1 |= byte << (8 * (pos - 4));
-            }
-            *(uint2 *)(l_codes + t * K + k) = make_uint2(w0, w1);
-            if (K8) {
-                sum += __shfl_xor(sum, 1, 64);
-                if ((tid & 1) == 0) l_bsums[t * (K >> 4) + (k >> 4)] = (int16_t)sum;
-                if ((k & 255) == 0) l_d[t * nsb + (k >> 8)] = d;
-            } else if ((tid & 3) == 0) {
-                l_d[t * nd + (k >> 5)] = d;
-            }
-        };
+            for (int i = 0; i < 8; ++i) v[i] *= inv;
+            const float d = requantise8(v, Tile::QUANT, c);
+            store_lds(c, d, 0, k);
+        }
+    } else {
+        // make the blocks here: eight consecutive values per thread, the threads of a block together (requantise8)
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const float * xr = row_of(t);
@@ -455,6 +489,17 @@ void gemv_norm(hipStream_t s, const Weight & w, const float * x, const float * n
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
     a.xin = x; a.norm_w = norm_w; a.rows = rows; a.eps = eps;
     launch_gemv_src<SRC_NORM>(s, w.type, a);
+}
+
+void gemv_combine(hipStream_t s, const Weight & w, const float * partial, int item0, int n_split, int n_head, int G, int head_dim,
+                  float * y, int ldy, int col0, int mode) {
+    if (!gemv_can_weight(w, 1) || !partial || item0 < 0 || n_split < 1 || n_split > GEMV_COMBINE_MAX_SPLITS || G < 1 || n_head % G != 0
+        || head_dim % 8 != 0 || w.K != n_head * head_dim)
+        throw std::runtime_error("gemv_combine: needs Q4_K, Q5_K, Q6_K or Q8_0 tiles over the heads' outputs and at most "
+                                 + std::to_string(GEMV_COMBINE_MAX_SPLITS) + " splits");
+    GemvArgs a = gemv_args(w, 1, y, ldy, col0, mode, nullptr);
+    a.partial = partial; a.item0 = item0; a.n_split = n_split; a.att_G = G; a.att_hd = head_dim;
+    launch_gemv_src<SRC_COMBINE>(s, w.type, a);
 }
 
 void gemv_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, int T, float * y, int ldy, int col0, int mode) {

@@ -151,6 +151,12 @@ bool gemv_can_weight(const Weight & w, int T);
 void gemv_norm(hipStream_t s, const Weight & w, const float * x, const float * norm_w, float eps, const int32_t * rows, int T,
                float * y, int ldy, int col0, int mode, const float * bias);
 void gemv_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, int T, float * y, int ldy, int col0, int mode);
+// ... and gemv_combine from the split partials of a single-token step's attention (the token's work items start at
+// item0, n_split per kv head, at most GEMV_COMBINE_MAX_SPLITS: every workgroup merges all heads itself, which pays
+// while the partials are few): the product of the output projection without attention_combine's launch.
+constexpr int GEMV_COMBINE_MAX_SPLITS = 16;
+void gemv_combine(hipStream_t s, const Weight & w, const float * partial, int item0, int n_split, int n_head, int G, int head_dim,
+                  float * y, int ldy, int col0, int mode);
 extern int g_gemv_max_t;       // steps of at most this many tokens take the kernel (default GEMV_MAX_T; 0 switches it off)
 extern int g_mm_debug;         // timing experiments (see MMArgs::debug)
 extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic

@@ -143,8 +143,9 @@ def test_ggml_arithmetic_follows_the_oracle_as_closely_as_its_rounding_allows(mo
 def test_small_steps_under_the_ggml_arithmetic_take_the_integer_kernel(models, key, monkeypatch):
     """Steps of one or two tokens under RETRO_ACTIVATIONS=ggml multiply their Q4_K matrices by integer products of
     the stored codes with the rows' Q8_K codes (Q6_K matrices of the same model stay on the tile kernels), and where
-    every consumer of a row is that kernel it makes the codes itself from the residual or gate/up rows (the default;
-    RETRO_GEMV_FUSE=0 keeps the producers' own launches). Against the oracle's ggml arithmetic such a step must
+    every consumer of a row is that kernel it makes the codes itself from the residual or gate/up rows, and the
+    output projection of a single-token step merges the attention splits itself (the default; RETRO_GEMV_FUSE=0 keeps
+    the producers' own launches). Against the oracle's ggml arithmetic such a step must
     drift no further than the same step through the tile kernels (RETRO_GEMV_MAX_T=0) does - all differ from it by
     float rounding that later conversions amplify - and the engines must stay as close to each other as either is
     to the oracle."""
@@ -153,9 +154,9 @@ def test_small_steps_under_the_ggml_arithmetic_take_the_integer_kernel(models, k
     cfg = E.EngineConfig(n_ctx=2048, n_seq_max=8, n_batch=256, n_ubatch=256)
     m = oracle.Model(models[key])
     rng = np.random.default_rng(5)
-    lens = [5, 33, 64, 17]
+    lens = [5, 33, 200, 17]         # slot 2: seven pages, two attention splits per kv head in a single-token step
     prompts = [rng.integers(0, m.n_vocab, n) for n in lens]
-    plans = [[0, 1, 2, 3], [1, 3], [2], [0, 1, 3], [0], [0, 1, 2, 3]]      # the slots of each decode step
+    plans = [[0, 1, 2, 3], [1, 3], [2], [0, 1, 3], [0], [0, 1, 2, 3], [2]]      # the slots of each decode step
     feeds = [[int(t) for t in rng.integers(0, m.n_vocab, len(p))] for p in plans]
     runs = {}
     for name, limit, fuse in (("integer", None, None), ("unfused", None, "0"), ("tiles", "0", None)):

@@ -70,6 +70,9 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
             act.qx = d_xh.as<__half>(); act.qsums = d_sums.as<__half>(); act.quant = rk::act_quant_of(type);
         }
         DevBuf d_codes, d_scales, d_bsums;
+        // the switch an engine's configuration may have left off is on for the call
+        struct Restore { int was; ~Restore() { rk::g_gemv_max_t = was; } } restore{rk::g_gemv_max_t};
+        if (integer) rk::g_gemv_max_t = rk::GEMV_MAX_T;
         if (integer) {
             if (!faithful || act.quant == rk::AQ_NONE || n_tokens > rk::GEMV_MAX_T)
                 throw std::runtime_error("the integer kernel takes Q8_K or Q8_0 conversions of at most " + std::to_string(rk::GEMV_MAX_T) + " tokens");
@@ -106,6 +109,8 @@ int retro_kernel_gemv_fused(int32_t kind, int32_t type, const uint8_t * raw, int
             throw std::runtime_error("gemv_fused: kind 1 (RMSNorm) or 2 (SwiGLU), whole tiles and super-blocks, at most " + std::to_string(rk::GEMV_MAX_T) + " tokens");
         if (kind == 1 && !norm_w) throw std::runtime_error("gemv_fused: the RMSNorm needs its weights");
         if (type != rk::WT_Q4_K && type != rk::WT_Q5_K && type != rk::WT_Q6_K && type != rk::WT_Q8_0) throw std::runtime_error("gemv_fused: Q4_K, Q5_K, Q6_K or Q8_0 rows");
+        struct Restore { int was; ~Restore() { rk::g_gemv_max_t = was; } } restore{rk::g_gemv_max_t};
+        rk::g_gemv_max_t = rk::GEMV_MAX_T;      // whatever an engine's configuration left
         const size_t bytes = rk::row_bytes(type, k) * (size_t)n_rows;
         const size_t in_floats = (size_t)n_tokens * k * (kind == 2 ? 2 : 1);
         DevBuf d_raw, d_packed, d_x, d_w, d_xh, d_sums, d_codes, d_scales, d_bsums, d_y;
@@ -239,7 +244,9 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
         rk::Act act;
         act.K = (int)k;
         act.x = act.qx = d_xh.as<__half>(); act.sums = act.qsums = d_sums.as<__half>(); act.quant = rk::act_quant_of(type);
-        // mode 4: the integer matrix-vector kernel over pseudo-random Q8_K blocks (Q4_K, at most GEMV_MAX_T tokens)
+        struct Restore { int was; ~Restore() { rk::g_gemv_max_t = was; } } restore{rk::g_gemv_max_t};
+        if (mode == 4) rk::g_gemv_max_t = rk::GEMV_MAX_T;      // whatever an engine's configuration left
+        // mode 4: the integer matrix-vector kernel over pseudo-random activation blocks (Q4_K, Q5_K, Q6_K, Q8_0; at most GEMV_MAX_T tokens)
         DevBuf d_codes, d_scales, d_bsums;
         if (mode == 4) {
             if ((type != rk::WT_Q4_K && type != rk::WT_Q5_K && type != rk::WT_Q6_K && type != rk::WT_Q8_0) || n_tokens > rk::GEMV_MAX_T)

@@ -82,7 +82,7 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
         if (const char * f = std::getenv("RETRO_GEMV_MERGE_SPLITS")) merge_max_splits_ = std::max(0, std::min(std::atoi(f), rk::GEMV_COMBINE_MAX_SPLITS));      // 0: producers keep their own launches
         // steps of at most this many tokens go through the integer matrix-vector kernel under the ggml arithmetic (0: never)
         const char * g = std::getenv("RETRO_GEMV_MAX_T");
-        rk::g_gemv_max_t = g ? std::max(0, std::min(std::atoi(g), rk::GEMV_MAX_T)) : rk::GEMV_MAX_T;
+        gemv_max_t_ = g ? std::max(0, std::min(std::atoi(g), rk::GEMV_MAX_T)) : rk::GEMV_MAX_T;
         const char * v = std::getenv("RETRO_ACTIVATIONS");
         const std::string mode = v ? v : "exact";
         if (mode == "ggml") ggml_activations_ = true;
@@ -1308,6 +1308,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
     // expert router and LoRA factors (`plain`); the converted row for the quantised weights.
     const bool faithful = ggml_activations_;
     const bool ffn_lora = routed && lora_has_ffn_ && h.n_expert == 0;      // some row may carry feed-forward deltas
+    rk::g_gemv_max_t = gemv_max_t_;     // this engine's setting, for the matmul entry points called below
     const bool small_step = T <= rk::g_gemv_max_t;      // the producers leave the Q8_K blocks for the integer kernel as well
     // ... or, where every consumer of a row is that kernel and nothing else wants the row (no adapters), the kernel
     // makes the blocks itself while it stages them and the producer's launch is saved

@@ -306,6 +306,7 @@ private:
     // rk::GEMV_MAX_T tokens, for the integer matrix-vector kernel
     struct ActCodes { DevBuf codes, d, bsums; };
     ActCodes act_e_codes_, act_q_codes_, act_f_codes_, act_o_codes_;
+    int gemv_max_t_ = rk::GEMV_MAX_T;
     int merge_max_splits_ = 8;       // about a 1,000-token context: beyond it the merge kernel's own launch is cheaper
     bool gemv_fuse_ = true;      // small steps: the integer kernel makes its Q8_K blocks from the f32 rows itself where it can
     DevBuf q_half_lo_;

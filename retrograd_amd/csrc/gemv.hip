@@ -39,7 +39,7 @@
 
 namespace rk {
 
-int g_gemv_max_t = GEMV_MAX_T;
+thread_local int g_gemv_max_t = GEMV_MAX_T;
 
 struct GemvArgs {
     const uint8_t * w;         // tiles

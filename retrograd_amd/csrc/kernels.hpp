@@ -157,7 +157,8 @@ void gemv_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, i
 constexpr int GEMV_COMBINE_MAX_SPLITS = 16;
 void gemv_combine(hipStream_t s, const Weight & w, const float * partial, int item0, int n_split, int n_head, int G, int head_dim,
                   float * y, int ldy, int col0, int mode);
-extern int g_gemv_max_t;       // steps of at most this many tokens take the kernel (default GEMV_MAX_T; 0 switches it off)
+extern thread_local int g_gemv_max_t;   // steps of at most this many tokens take the kernel (default GEMV_MAX_T; 0 switches it off);
+                                        // an engine sets it from its own configuration at the start of every forward pass
 extern int g_mm_debug;         // timing experiments (see MMArgs::debug)
 extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic
 // Fused gate/up matmul and SwiGLU: w holds, for every 64 columns of the hidden

@@ -72,8 +72,9 @@ int32_t retro_kernel_sample_greedy_noalloc_max_rows(void);
  * clock higher and flatter the kernel by 15-20 %). Adding 16 to the mode gives
  * every launch another copy of the weights (1 GiB of copies in turn; adding 32,
  * 6 GiB), so that they are read from HBM as in a decode step instead of from
- * the last-level cache. debug and force_ksplit are timing experiments
- * (0 = normal). type is Q4_K, Q5_K, Q6_K or Q8_0 (Q5_K and Q6_K in modes 2 and
+ * the last-level cache. debug must be 0 (the library carries no switches that
+ * change results); force_ksplit > 0 overrides the number of K-slices for this
+ * call. type is Q4_K, Q5_K, Q6_K or Q8_0 (Q5_K and Q6_K in modes 2 and
  * 3 only), n_rows a multiple of 16 and k of 256: anything else is refused
  * before a buffer is allocated. Mode 4 times the integer matrix-vector kernel
  * of very small steps under the ggml arithmetic instead (Q4_K or Q8_0, at most

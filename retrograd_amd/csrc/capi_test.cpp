@@ -265,7 +265,7 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
             act.qc = d_codes.as<int8_t>(); act.qd = d_scales.as<float>(); act.qbs = d_bsums.as<int16_t>();
             if (!rk::gemv_can(w, act.operand(type), n_tokens)) throw std::runtime_error("matmul_time: the integer kernel does not take this shape");
         }
-        rk::g_mm_debug = debug;
+        if (debug != 0) throw std::runtime_error("matmul_time: the library has no timing switches; debug must be 0");
         rk::g_mm_force_ksplit = force_ksplit;
         hipEvent_t e0, e1;
         ok(hipEventCreate(&e0), "event"); ok(hipEventCreate(&e1), "event");
@@ -283,7 +283,6 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
         ok(hipEventSynchronize(e1), "sync");
         float ms = 0;
         ok(hipEventElapsedTime(&ms, e0, e1), "elapsed");
-        rk::g_mm_debug = 0;
         rk::g_mm_force_ksplit = 0;
         (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
         *out_us = (double)ms * 1e3 / iters;

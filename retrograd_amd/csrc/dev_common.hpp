@@ -223,7 +223,6 @@ struct MMArgs {
     int n_row_groups;
     float * partial;          // [ksplit][64][pld] K-slices of a split matmul; this matrix fills columns pcol .. pcol + N
     int pld, pcol;            // (pld = N, pcol = 0 unless several matrices share the slices)
-    int debug;                // timing experiments only: bit 5 sends a full 64-token chunk of Q4_K through the general kernel
     // mode MM_SWIGLU: rows come in groups of 128, 64 gate rows then the 64 up rows of the same
     // columns; the epilogue writes silu(gate) * up as the activations of the next matmul
     Act act_out;

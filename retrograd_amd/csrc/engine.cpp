@@ -75,8 +75,6 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     {
         // RETRO_ACTIVATIONS=ggml: every matmul multiplies the activations as ggml's CPU path converts them
         // (Q8_K / Q8_0 codes, f16 / bf16 rounding); unset or "exact": the f32 values (as f16 hi/lo pairs).
-        if (const char * dbg = std::getenv("RETRO_MM_DEBUG")) rk::g_mm_debug = std::atoi(dbg);     // timing experiments
-        if (const char * dbg = std::getenv("RETRO_MM_SINGLE")) mm_single_mask_ = std::atoi(dbg);
         if (const char * f = std::getenv("RETRO_GEMV_FUSE")) gemv_fuse_ = std::atoi(f) != 0;
         // ... and the output projection merges at most this many attention splits per kv head itself (0: never)
         if (const char * f = std::getenv("RETRO_GEMV_MERGE_SPLITS")) merge_max_splits_ = std::max(0, std::min(std::atoi(f), rk::GEMV_COMBINE_MAX_SPLITS));      // 0: producers keep their own launches
@@ -1860,12 +1858,6 @@ void Engine::adapter_rows_info(retro_adapter_rows_info * out) const {
 // ---- event timing -------------------------------------------------------------------------
 
 size_t Engine::prof_begin(int cat) {
-    // accuracy experiment: RETRO_MM_SINGLE is a mask of matrix kinds (1 qkv, 2 attention output, 4 gate/up, 8 down,
-    // 16 head) whose 64-token Q4_K products use only the hi half of the activations
-    if (mm_single_mask_) {
-        const int bit = cat == PC_QKV ? 1 : cat == PC_OPROJ ? 2 : cat == PC_GATEUP ? 4 : cat == PC_DOWN ? 8 : cat == PC_HEAD ? 16 : 0;
-        rk::g_mm_debug = (rk::g_mm_debug & ~64) | ((mm_single_mask_ & bit) ? 64 : 0);
-    }
     if (prof_level_ == 0 || (prof_level_ == 1 && cat != PC_ATTN)) return (size_t)-1;
     if (prof_used_ + 2 > prof_events_.size()) {
         for (int i = 0; i < 2; ++i) {

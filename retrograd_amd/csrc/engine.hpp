@@ -326,7 +326,6 @@ private:
     double prof_ms_[PC_COUNT] = {};
     uint64_t prof_n_[PC_COUNT] = {};
     size_t prof_begin(int cat);
-    int mm_single_mask_ = 0;
     int kv_q8_ = 0;            // rk::KV_F16, or KV_Q8 / KV_Q4: the KV pools hold Q8_0 / Q4_0 blocks (kv_dtype)
     uint32_t snap_magic() const;
     void prof_end(int cat, size_t token);

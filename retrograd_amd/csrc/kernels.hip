@@ -1733,7 +1733,6 @@ struct AttnArgs {
     int n_head, n_kv, G;
     int split_pages;
     size_t page_stride, head_stride;
-    int debug;
 };
 
 // ONE: every tile holds a single query token (a pure decode step).
@@ -1848,15 +1847,6 @@ __global__ __launch_bounds__(64, 2) void k_attention(AttnArgs a) {
             for (int j = 0; j < KS; ++j) { kreg[j][0] = ks.r[2 * j]; kreg[j][1] = ks.r[2 * j + 1]; }
 #pragma unroll
             for (int d = 0; d < DT; ++d) vreg[d] = vs.r[d];
-        }
-        if (!Q8 && (a.debug & 1)) {       // timing experiment: the loads alone
-            h8 t = kreg[0][0];
-#pragma unroll
-            for (int j = 0; j < KS; ++j) { t += kreg[j][0]; t += kreg[j][1]; }
-#pragma unroll
-            for (int d = 0; d < DT; ++d) t += vreg[d];
-            o[0][0] += (float)t[0] + (float)t[3];
-            return;
         }
         f4 s0 = (f4){0.f, 0.f, 0.f, 0.f}, s1 = (f4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -2024,7 +2014,6 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
     a.split_pages = pk.split_pages;
     a.page_stride = sh.page_stride; a.head_stride = sh.head_stride;
     if (sh.page_stride == 0 || sh.head_stride == 0) throw std::runtime_error("attention: the pool's strides are missing");
-    { static const int dbg = [] { const char * v = std::getenv("RETRO_ATTN_DEBUG"); return v ? std::atoi(v) : 0; }(); a.debug = dbg; }
     if (a.G > 16 || sh.n_head % sh.n_head_kv != 0) throw std::runtime_error("attention: unsupported head grouping");
 #define ATTN_LAUNCH_Q(HD_, Q8_) \
     do { \

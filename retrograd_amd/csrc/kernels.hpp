@@ -159,8 +159,7 @@ void gemv_combine(hipStream_t s, const Weight & w, const float * partial, int it
                   float * y, int ldy, int col0, int mode);
 extern thread_local int g_gemv_max_t;   // steps of at most this many tokens take the kernel (default GEMV_MAX_T; 0 switches it off);
                                         // an engine sets it from its own configuration at the start of every forward pass
-extern int g_mm_debug;         // timing experiments (see MMArgs::debug)
-extern int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic
+extern thread_local int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic for the calling thread (kernel-level timing entry point)
 // Fused gate/up matmul and SwiGLU: w holds, for every 64 columns of the hidden
 // layer, their 64 gate rows followed by their 64 up rows (w.N = 2 F, F % 64 == 0,
 // a tile storage type); out (K = F) receives silu(gate) * up as activations.

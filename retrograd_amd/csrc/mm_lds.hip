@@ -439,7 +439,6 @@ __device__ __forceinline__ float fma3(float a, float b, float c) {
 // activations and the weight tiles keep the 16x16x32 operand order; only the
 // per-lane addresses differ.
 // acc[tb][i] is token 32 tb + 8 (i / 4) + 4 p + i % 4, row n32.
-template <bool SINGLE>
 __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_num_vgpr(232))) void k_mm5_q4k(MMArgs a) {
     constexpr int NT = 4;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -513,7 +512,6 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_num_vgpr(232))) 
         sb = min(sb, sb1 - 1);
         if (idx < 8) {
             const int c = st_slot + WAVES_PER_TILE * idx;
-            if (SINGLE && st_slot == 1 && (a.debug & 128)) return;      // timing experiment: the lo blocks are not staged
             lds_dma16(xu + (size_t)(sb * 16 + c) * 2048, lane16, buf + (c * NT + st_tile) * 1024);
         } else {
             // every wave requests sums (waves past slot 0 repeat slot 0's block): no branch in the stream
@@ -538,7 +536,7 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_num_vgpr(232))) 
         auto read_step = [&](int s) __attribute__((always_inline)) {
             const int j = s >> 1, h = s & 1;
 #pragma unroll
-            for (int hl = 0; hl < (SINGLE ? 1 : 2); ++hl)
+            for (int hl = 0; hl < 2; ++hl)
 #pragma unroll
                 for (int tb = 0; tb < 2; ++tb)
                     A[s & 1][hl][tb] = *(const h8 *)(xk + ((j * 2 + hl) * NT + 2 * tb) * 1024 + h * 512);
@@ -617,11 +615,9 @@ __global__ __launch_bounds__(kThreads, 1) __attribute__((amdgpu_num_vgpr(232))) 
 #pragma unroll
             for (int tb = 0; tb < 2; ++tb)
                 q[tb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[s & 1][0][tb], B[s & 1], s == 0 ? zero : q[tb], 0, 0, 0);
-            if (!SINGLE) {
 #pragma unroll
-                for (int tb = 0; tb < 2; ++tb)
-                    q[tb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[s & 1][1][tb], B[s & 1], q[tb], 0, 0, 0);
-            }
+            for (int tb = 0; tb < 2; ++tb)
+                q[tb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[s & 1][1][tb], B[s & 1], q[tb], 0, 0, 0);
             if (s == 7) load_w(min(sb + 2, sb1 - 1), set);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -900,15 +896,13 @@ static void launch2(hipStream_t s, int type, const MMArgs & a, dim3 grid) {
             HIP_OK(hipFuncSetAttribute((const void *)k_mm2_q4k<NT, R>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
             once = true;
         }
-        if (NT == 4 && R == 2 && !(a.debug & 32)) {
+        if (NT == 4 && R == 2) {
             static bool once5 = false;
             if (!once5) {
-                HIP_OK(hipFuncSetAttribute((const void *)k_mm5_q4k<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-                HIP_OK(hipFuncSetAttribute((const void *)k_mm5_q4k<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+                HIP_OK(hipFuncSetAttribute((const void *)k_mm5_q4k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
                 once5 = true;
             }
-            if (a.debug & 64) hipLaunchKernelGGL(k_mm5_q4k<true>, grid, dim3(kThreads), lds, s, a);
-            else hipLaunchKernelGGL(k_mm5_q4k<false>, grid, dim3(kThreads), lds, s, a);
+            hipLaunchKernelGGL(k_mm5_q4k, grid, dim3(kThreads), lds, s, a);
             return;
         }
         hipLaunchKernelGGL((k_mm2_q4k<NT, R>), grid, dim3(kThreads), lds, s, a);
@@ -941,8 +935,7 @@ size_t matmul_workspace_bytes() {
     return (size_t)64 * 16 * 8192 * 4;
 }
 
-int g_mm_debug = 0;
-int g_mm_force_ksplit = 0;
+thread_local int g_mm_force_ksplit = 0;
 
 template <int R>
 static void dispatch_nt(hipStream_t s, int type, int nt, const MMArgs & a, dim3 grid) {
@@ -967,7 +960,6 @@ static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x_all, int T
     if (!x.x) throw std::runtime_error("matmul: the activations were not prepared for this weight type");
     if ((w.type == WT_Q4_K || w.type == WT_Q5_K) && !x.sums) throw std::runtime_error("matmul: Q4_K and Q5_K need block sums");
     MMArgs a {};
-    a.debug = g_mm_debug;
     a.w = w.packed; a.x = x.x; a.sums = x.sums; a.y = y; a.bias = bias;
     a.K = w.K; a.N = w.N; a.T = T; a.ldy = ldy; a.col0 = col0; a.mode = mode;
     if (act_out) { a.act_out = *act_out; a.act_f32 = act_f32; }

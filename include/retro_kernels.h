@@ -59,7 +59,9 @@ int retro_kernel_sample_prepare(const float * logits, int32_t n_rows, int32_t n_
  * more is refused with -1 and a message, nothing launched. Every call on one
  * GPU shares that GPU's array: calls that overlap there (two streams, two
  * threads) race; calls on one stream are ordered and need no clearing between
- * them. */
+ * them. The array's address on a device is looked up once, by engine creation
+ * or else by the first call on that device: in a process that creates no
+ * engine, make the first call outside stream capture. */
 int retro_kernel_sample_greedy_noalloc(const float * d_logits, int32_t n_rows, int32_t n_vocab,
                                        int32_t * d_out_argmax, float * d_out_max, double * d_out_sum_exp,
                                        void * stream);

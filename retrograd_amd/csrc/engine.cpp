@@ -72,6 +72,7 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     }
     hip_check(hipSetDevice(0), "hipSetDevice");
     hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
+    rk::sample_static_prepare();       // the no-allocation greedy scan then only launches, also under stream capture
     {
         // RETRO_ACTIVATIONS=ggml: every matmul multiplies the activations as ggml's CPU path converts them
         // (Q8_K / Q8_0 codes, f16 / bf16 rounding); unset or "exact": the f32 values (as f16 hi/lo pairs).

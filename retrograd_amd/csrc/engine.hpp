@@ -104,9 +104,9 @@ struct Vocab {
             if (unparse_special) text += piece;
             return;
         }
-        if (type == 6 && piece.size() == 6 && piece.compare(0, 3, "<0x") == 0) {
-            text.push_back((char)std::stoi(piece.substr(3, 2), nullptr, 16));
-            return;
+        if (type == 6) {
+            const int v = byte_piece_value(piece);
+            if (v >= 0) { text.push_back((char)v); return; }
         }
         if (tokenizer.model == "gpt2") {
             text += tokenizer.spelled_bytes(piece);

@@ -512,10 +512,19 @@ private:
     }
 
     // Rule references on top are replaced by their alternatives until every stack is empty or waits for a terminal.
-    void expand(Stack s, std::vector<Stack> & out) const {
+    // The grammar text comes with a request: a chain of rules that only name the next one is as deep as the chain is
+    // long, and an ambiguous grammar can hold exponentially many stacks, so both are bounded and a grammar past
+    // the bounds is an error of the call (which reports it), not a crash of the process.
+    static constexpr int kMaxExpandDepth = 1024;
+    static constexpr size_t kMaxStacks = 4096;
+    void expand(Stack s, std::vector<Stack> & out, int depth = 0) const {
+        if (depth > kMaxExpandDepth) throw std::runtime_error("grammar: rules are nested deeper than 1024 references");
         while (!s.empty() && s.back().idx >= rules_.rules[s.back().rule][s.back().alt].size()) s.pop_back();
         if (s.empty() || top(s).kind != GrammarSymbol::RULE) {
-            if (std::find(out.begin(), out.end(), s) == out.end()) out.push_back(std::move(s));
+            if (std::find(out.begin(), out.end(), s) == out.end()) {
+                if (out.size() >= kMaxStacks) throw std::runtime_error("grammar: more than 4096 alternatives are open at once (the grammar is too ambiguous)");
+                out.push_back(std::move(s));
+            }
             return;
         }
         const Pos p = s.back();
@@ -525,7 +534,7 @@ private:
         for (uint32_t a = 0; a < rules_.rules[callee].size(); ++a) {
             Stack t = s;
             t.push_back({callee, a, 0});
-            expand(std::move(t), out);
+            expand(std::move(t), out, depth + 1);
         }
     }
     void step_over_top(const Stack & s, std::vector<Stack> & out) const {

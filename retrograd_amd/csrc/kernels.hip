@@ -2460,7 +2460,9 @@ __global__ __launch_bounds__(256) void k_sample_slices(const float * __restrict_
     __syncthreads();
     const float slice_max = b_val;
     double acc = 0.0;
-    for (int i = lo + threadIdx.x; i < hi; i += 256) acc += exp((double)l[i] - (double)slice_max);
+    // a slice whose logits are all -inf adds nothing (exp(-inf - -inf) would be a NaN that the merge multiplies by 0)
+    if (slice_max != -INFINITY)
+        for (int i = lo + threadIdx.x; i < hi; i += 256) acc += exp((double)l[i] - (double)slice_max);
     for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
     if (lane == 0) s_sum[wave] = acc;
     __syncthreads();
@@ -2478,7 +2480,7 @@ __global__ __launch_bounds__(64) void k_sample_merge(const SamplePartial * __res
         if (p[s].idx != 0x7fffffff && better(p[s].max, p[s].idx, fv, fi)) { fv = p[s].max; fi = p[s].idx; }
     double total = 0.0;
     for (int s = 0; s < n_slices; ++s)
-        if (p[s].idx != 0x7fffffff) total += p[s].sum * exp((double)p[s].max - (double)fv);
+        if (p[s].idx != 0x7fffffff && p[s].max != -INFINITY) total += p[s].sum * exp((double)p[s].max - (double)fv);
     out[row].argmax = fi;
     out[row].max = fv;
     out[row].sum_exp = total;
@@ -2501,12 +2503,14 @@ static int sample_slices_for(int n_rows) {
 // the process ends; host code never uses the array's name as an address, only what hipGetSymbolAddress
 // returned for the device that is current.
 constexpr int SAMPLE_STATIC_MAX_ROWS = 4096;
-constexpr size_t SAMPLE_STATIC_PARTIALS = SAMPLE_STATIC_MAX_ROWS;      // rows * slices never exceeds max(rows, 512)
+constexpr size_t SAMPLE_STATIC_PARTIALS = SAMPLE_STATIC_MAX_ROWS;      // rows * slices never exceeds max(rows, 1024): see sample_slices_for
 static __device__ __align__(256) unsigned char scratch[SAMPLE_STATIC_PARTIALS * sizeof(SamplePartial)];
 
 int sample_static_max_rows() { return SAMPLE_STATIC_MAX_ROWS; }
 
-// The address of `scratch` on the current device, looked up once per device.
+// The address of `scratch` on the current device, looked up once per device: at engine creation
+// (sample_static_prepare) or, in a process that creates no engine, by the first call - which must then be made
+// outside stream capture, since the lookup may load the code object.
 static void * sample_static_scratch() {
     constexpr int MAX_DEVICES = 64;
     static std::mutex lock;
@@ -2526,6 +2530,8 @@ static void * sample_static_scratch() {
     return ptr_of[dev];
 }
 
+void sample_static_prepare() { (void)sample_static_scratch(); }
+
 __global__ __launch_bounds__(64) void k_sample_merge_arrays(const SamplePartial * __restrict__ part, int n_slices,
                                                             int32_t * __restrict__ out_argmax, float * __restrict__ out_max,
                                                             double * __restrict__ out_sum) {
@@ -2538,7 +2544,7 @@ __global__ __launch_bounds__(64) void k_sample_merge_arrays(const SamplePartial 
         if (p[s].idx != 0x7fffffff && better(p[s].max, p[s].idx, fv, fi)) { fv = p[s].max; fi = p[s].idx; }
     double total = 0.0;
     for (int s = 0; s < n_slices; ++s)
-        if (p[s].idx != 0x7fffffff) total += p[s].sum * exp((double)p[s].max - (double)fv);
+        if (p[s].idx != 0x7fffffff && p[s].max != -INFINITY) total += p[s].sum * exp((double)p[s].max - (double)fv);
     out_argmax[row] = fi;
     out_max[row] = fv;
     out_sum[row] = total;

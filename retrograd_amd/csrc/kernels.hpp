@@ -394,6 +394,9 @@ void sample_prepare(hipStream_t s, const float * logits, int n_rows, int n_vocab
 // buffers of the caller, on the caller's stream, with its slice partials in a static device array: allocates
 // nothing and waits for nothing. At most sample_static_max_rows() rows per call.
 int sample_static_max_rows();
+// Looks the static array's address up for the current device (a host-side call that may load the code object), so
+// that later calls of sample_greedy_static do nothing but launch; engine creation calls it.
+void sample_static_prepare();
 void sample_greedy_static(hipStream_t s, const float * logits, int n_rows, int n_vocab, int32_t * out_argmax,
                           float * out_max, double * out_sum);
 

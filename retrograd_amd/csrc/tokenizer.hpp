@@ -42,6 +42,22 @@
 
 #include "unicode_ranges.hpp"
 
+// The byte a piece of exactly the form "<0xHH>" (two hexadecimal digits, either case) stands for, or -1.
+inline int byte_piece_value(const std::string & p) {
+    if (p.size() != 6 || p.compare(0, 3, "<0x") != 0 || p[5] != '>') return -1;
+    int v = 0;
+    for (int i = 3; i < 5; ++i) {
+        const char c = p[(size_t)i];
+        int d;
+        if (c >= '0' && c <= '9') d = c - '0';
+        else if (c >= 'a' && c <= 'f') d = c - 'a' + 10;
+        else if (c >= 'A' && c <= 'F') d = c - 'A' + 10;
+        else return -1;
+        v = v * 16 + d;
+    }
+    return v;
+}
+
 namespace retro {
 
 struct Tokenizer {
@@ -117,10 +133,9 @@ struct Tokenizer {
         for (size_t i = 0; i < pieces.size(); ++i) {
             const int32_t t = types.empty() ? (int32_t)NORMAL : types[i];
             if (t == BYTE) {
-                // "<0xXX>"
-                const std::string & p = pieces[i];
-                if (p.size() == 6 && p.compare(0, 3, "<0x") == 0 && p[5] == '>') {
-                    const int v = std::stoi(p.substr(3, 2), nullptr, 16);
+                // "<0xXX>"; a BYTE piece of any other form stands for no byte and is never produced
+                const int v = byte_piece_value(pieces[i]);
+                if (v >= 0) {
                     byte_id[v] = (int32_t)i;
                     has_bytes = true;
                 }

@@ -45,7 +45,7 @@ int main(int argc, char ** argv) {
             vocab.add(unhex(h), eog != 0);
         } else if (!g && (cmd == "mask" || cmd == "accept")) {
             std::printf("no grammar\n");
-        } else if (cmd == "mask") {
+        } else if (cmd == "mask") try {
             std::vector<float> logits(vocab.size(), 0.0f);
             const bool any = g->mask(vocab, logits.data(), logits.size());
             bool first = true;
@@ -54,10 +54,14 @@ int main(int argc, char ** argv) {
             if (first) std::printf("none");
             if (any == first) std::printf(" INCONSISTENT");
             std::printf("\n");
-        } else if (cmd == "accept") {
+        } catch (const std::exception & e) {
+            std::printf("error: %s\n", e.what());
+        } else if (cmd == "accept") try {
             unsigned id = 0;
             is >> id;
             std::printf(g->accept(vocab, id) ? "ok\n" : "refused\n");
+        } catch (const std::exception & e) {
+            std::printf("error: %s\n", e.what());
         }
     }
     return 0;

@@ -198,8 +198,18 @@ def test_token_ids_and_text_split_inside_a_character(exe):
     ("", "no 'root' rule"),
     ("root ::= \"abcdefghijkl\"{100000}", "too large"),
     ("root ::= " + "(" * 300 + "\"a\"" + ")" * 300, "nested too deeply"),
+    # a chain of 5000 rules that each only name the next: as deep as it is long
+    ("root ::= r0\n" + "".join("r%d ::= r%d\n" % (i, i + 1) for i in range(5000)) + "r5000 ::= \"a\"", "nested deeper"),
+    # 2^14 ways to read the same text: the alternatives open at once are bounded
+    ("root ::= x0\n" + "".join("x%d ::= \"a\" x%d \"b\" | \"a\" x%d \"c\"\n" % (i, i + 1, i + 1) for i in range(14)) + "x14 ::= \"!\"", None),
 ])
 def test_invalid_grammars_are_refused_with_the_reason(exe, gbnf, message):
+    if message is None:
+        # valid, but walking "a" fourteen times doubles the open alternatives each time: an error, never a crash
+        lines = run(exe, ["token 61 0", "grammar " + hx(gbnf)] + ["accept 0"] * 14)
+        assert lines[0] == "ok"
+        assert any(l.startswith("error: ") and "too ambiguous" in l for l in lines[1:]), lines
+        return
     (line,) = run(exe, ["grammar " + hx(gbnf)])
     assert line.startswith("error: ") and message in line, line
 

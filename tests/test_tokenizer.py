@@ -126,3 +126,19 @@ def test_an_unknown_pattern_is_refused(harness):
     r = subprocess.run([str(exe), str(vocab), str(texts), "0", "1", "0", kind["pre"], str(merges), "ids"],
                        capture_output=True, text=True, timeout=60)
     assert r.returncode == 1 and "some-other-pattern" in r.stdout and "not built" in r.stdout
+
+
+def test_byte_pieces_that_are_not_two_hex_digits_stand_for_no_byte(harness):
+    # A malformed vocabulary: BYTE-type pieces "<0x-1>", "<0xZZ>", "<0x+7>", "<0x 1>" must neither index the byte
+    # table out of bounds nor throw (the harness runs under the address and undefined-behaviour sanitizers); the
+    # ids of the well-formed vocabulary in front of them do not change.
+    exe, vocab, d = harness
+    bad = d / "vocab_bad.txt"
+    extra = ["<0x-1>", "<0xZZ>", "<0x+7>", "<0x 1>"]
+    bad.write_text(vocab.read_text() + "".join("%s 0.0 6\n" % p.encode().hex() for p in extra))
+    case = GOLDEN["cases"][0]
+    texts = d / "texts_bad.txt"
+    texts.write_text("0 0 %s\n" % (case["text"].encode().hex() or "-"))
+    r = subprocess.run([str(exe), str(bad), str(texts), str(GOLDEN["bos"]), str(GOLDEN["eos"]), "0"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert [int(x) for x in r.stdout.split()] == case["ids"]

@@ -63,3 +63,39 @@ def test_sizes_beyond_the_static_array_are_refused_before_any_launch():
             E.kernel_sample_greedy_noalloc(x.data_ptr(), rows, vocab, x.data_ptr(), x.data_ptr(), x.data_ptr(), 0)
     with pytest.raises(E.EngineError):
         E.kernel_sample_greedy_noalloc(0, 4, 8192, x.data_ptr(), x.data_ptr(), x.data_ptr(), 0)
+
+
+def test_the_call_inside_a_captured_graph_replays_like_the_eager_call():
+    # What the entry point is for: callers under stream capture. The address lookup happened before (an engine's
+    # creation, or the eager calls of the tests above); the captured region holds the two kernels and nothing else
+    # (no memset node). Replayed several times, with eager work and synchronisations in between, over changing
+    # logits: every replay must equal the eager call on the same logits.
+    import torch
+    n_rows, n_vocab = 24, 32000
+    rng = np.random.default_rng(9)
+    d_logits = torch.zeros((n_rows, n_vocab), dtype=torch.float32, device="cuda")
+    d_argmax = torch.full((n_rows,), -7, dtype=torch.int32, device="cuda")
+    d_max = torch.zeros(n_rows, dtype=torch.float32, device="cuda")
+    d_sum = torch.zeros(n_rows, dtype=torch.float64, device="cuda")
+    warm = torch.cuda.Stream()
+    with torch.cuda.stream(warm):        # one eager call on a side stream first, as torch asks before a capture
+        E.kernel_sample_greedy_noalloc(d_logits.data_ptr(), n_rows, n_vocab, d_argmax.data_ptr(), d_max.data_ptr(),
+                                       d_sum.data_ptr(), warm.cuda_stream)
+    warm.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    print("no-alloc greedy scan: capture", flush=True)
+    with torch.cuda.graph(graph):
+        E.kernel_sample_greedy_noalloc(d_logits.data_ptr(), n_rows, n_vocab, d_argmax.data_ptr(), d_max.data_ptr(),
+                                       d_sum.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    for it in range(4):
+        logits = (rng.standard_normal((n_rows, n_vocab)) * 3).astype(np.float32)
+        d_logits.copy_(torch.from_numpy(logits))
+        d_argmax.fill_(-7)
+        torch.cuda.synchronize()
+        print("no-alloc greedy scan: replay", it, flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = E.kernel_sample_prepare(logits, [1] * n_rows)
+        assert np.array_equal(d_argmax.cpu().numpy(), want[0]), it
+        assert np.array_equal(d_max.cpu().numpy(), want[1]), it
+        assert np.array_equal(d_sum.cpu().numpy(), want[2]), it

@@ -76,6 +76,10 @@ def build(verbose: bool = False, incremental: bool = False) -> Path:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("link failed:\n" + res.stderr)
+    # the stand-alone micro-benchmark of the compute unit's issue and LDS rates (no part of the library)
+    ub_src, ub_bin = CSRC / "ubench" / "issue_model.hip", LIB_DIR / "ubench_issue_model"
+    if not (incremental and ub_bin.exists() and ub_bin.stat().st_mtime > ub_src.stat().st_mtime):
+        _compile([hipcc(), *[f for f in HIP_FLAGS if f != "-fPIC"], "-o", str(ub_bin), str(ub_src)], "ubench/issue_model.hip", verbose)
     return LIB_PATH
 
 

@@ -73,6 +73,7 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     hip_check(hipSetDevice(0), "hipSetDevice");
     hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
     rk::sample_static_prepare();       // the no-allocation greedy scan then only launches, also under stream capture
+    if (const char * v = std::getenv("RETRO_FUSED_DECODE_ATTENTION")) fused_decode_attention_ = std::atoi(v) != 0;
     {
         // RETRO_ACTIVATIONS=ggml: every matmul multiplies the activations as ggml's CPU path converts them
         // (Q8_K / Q8_0 codes, f16 / bf16 rounding); unset or "exact": the f32 values (as f16 hi/lo pairs).
@@ -436,6 +437,7 @@ void Engine::build_buffers() {
     pk_.tile_t0 = i32((size_t)B); pk_.tile_nq = i32((size_t)B); pk_.tile_item0 = i32((size_t)B);
     pk_.tile_nsplit = i32((size_t)B); pk_.tile_page0 = i32((size_t)B); pk_.tile_kv_begin = i32((size_t)B);
     pk_.tok_tile = i32((size_t)B);
+    pk_.dec_order = i32((size_t)B);
     pk_.tok_merge = (int4 *)i32((size_t)B * 4);
     pk_.rope_cos = (float *)i32((size_t)B * (hp_.rope_dim / 2));
     pk_.rope_sin = (float *)i32((size_t)B * (hp_.rope_dim / 2));
@@ -1103,12 +1105,14 @@ int Engine::step(const retro_step_row_v2 * rows2, const retro_step_row * rows1, 
     int32_t * ht = (int32_t *)((uint8_t *)h_stage_.ptr + off_tok);
     int n_out = 0;
     bool routed = false;
+    step_max_resident_ = 0;
     {
         int at = 0;
         for (size_t r = 0; r < n_rows; ++r) {
             const RowView & row = rows[r];
             hd[r].slot = row.slot; hd[r].pos0 = row.pos0; hd[r].n = (int32_t)row.n; hd[r].tok_off = at;
             hd[r].sample = row.sample ? 1 : 0; hd[r].kv_begin = slots_[(size_t)row.slot].begin;
+            step_max_resident_ = std::max(step_max_resident_, row.pos0 + (int32_t)row.n - hd[r].kv_begin);
             // route = 1-based index of the adapter in id order (0: the base model)
             hd[r].route = 0; hd[r].pad = 0;
             // adapter 0 follows the context: its default adapter, else the trained adapter when there is one
@@ -1411,7 +1415,26 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
             }
             prof_end(PC_QKV, pt_);
         }
-        size_t pt_ = prof_begin(PC_ROPE);
+        // every row decodes one token over an f16 cache in the exact arithmetic: rotation, KV store, attention and
+        // split merge are one launch (the output projection's plain activation planes are all it writes)
+        const bool fused_decode = one_token_rows && fused_decode_attention_ && !faithful
+                                  && rk::attention_decode_can(sh, L.q_norm.ptr != nullptr || L.k_norm.ptr != nullptr, step_max_resident_);
+        size_t pt_;
+        if (fused_decode) {
+            pt_ = prof_begin(PC_ATTN);
+            rk::attention_decode(stream_, qkv, qkv_slices, T, sh, pk_, table_.as<int32_t>(), max_pages_,
+                                 k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), act_q);
+            prof_end(PC_ATTN, pt_);
+            pt_ = prof_begin(PC_OPROJ);
+            pending = rk::matmul_deferred(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
+            if (routed) {
+                float * dst = pending.n > 0 ? const_cast<float *>(pending.data) : x;
+                rk::lora_apply(stream_, lora_entries(l, 3), d_stage_.as<rk::RowDesc>(), pk_.row, act_q, T, E, dst, E, 0,
+                               lora_mid_.as<float>());
+            }
+            prof_end(PC_OPROJ, pt_);
+        } else {
+        pt_ = prof_begin(PC_ROPE);
         rk::rope_store(stream_, qkv, T, sh, pk_, L.q_norm.as<float>(), L.k_norm.as<float>(), q_half_.as<__half>(),
                        q_half_lo_.as<__half>(), k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(),
                        qkv_slices);
@@ -1443,6 +1466,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
                            lora_mid_.as<float>());
         }
         prof_end(PC_OPROJ, pt_);
+        }
         }
         if (fuse && h.n_expert == 0 && pending.n == 0 && all_gemv(L.gate_up, E, 2 * F)) {
             pt_ = prof_begin(PC_GATEUP);

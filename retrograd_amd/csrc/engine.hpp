@@ -307,6 +307,8 @@ private:
     struct ActCodes { DevBuf codes, d, bsums; };
     ActCodes act_e_codes_, act_q_codes_, act_f_codes_, act_o_codes_;
     int gemv_max_t_ = rk::GEMV_MAX_T;
+    bool fused_decode_attention_ = true;     // pure decode steps: rotation, KV store, attention and split merge in one launch (RETRO_FUSED_DECODE_ATTENTION=0: the three kernels)
+    int32_t step_max_resident_ = 0;          // longest resident span (positions) among the rows of the step being run
     int merge_max_splits_ = 8;       // about a 1,000-token context: beyond it the merge kernel's own launch is cheaper
     bool gemv_fuse_ = true;      // small steps: the integer kernel makes its Q8_K blocks from the f32 rows itself where it can
     DevBuf q_half_lo_;

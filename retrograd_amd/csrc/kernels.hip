@@ -1270,6 +1270,7 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
     __shared__ int scratch[16];
     __shared__ int carry[3];
     __shared__ int len_count[MAX_SPLIT_PAGES + 1], len_base[MAX_SPLIT_PAGES + 1];
+    __shared__ int row_len[1024];
     for (int i = threadIdx.x; i < n_upd; i += 1024) table[(size_t)upd[i].slot * max_pages + upd[i].index] = upd[i].page;
     if (threadIdx.x == 0) { carry[0] = 0; carry[1] = 0; carry[2] = 0; }
     __syncthreads();
@@ -1373,6 +1374,20 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
             for (int len = MAX_SPLIT_PAGES; len >= 0; --len) { len_base[len] = at; at += len_count[len]; }
         }
         __syncthreads();
+    }
+    // the rows by resident length, longest first (ties in row order): the decode-step attention starts one
+    // workgroup per row and kv head in this order, so that the launch's tail is made of short sequences
+    if (n_rows <= 1024) {
+        if ((int)threadIdx.x < n_rows) { const RowDesc d = rows[threadIdx.x]; row_len[threadIdx.x] = d.pos0 + d.n - d.kv_begin; }
+        __syncthreads();
+        if ((int)threadIdx.x < n_rows) {
+            const int mine = row_len[threadIdx.x];
+            int rank = 0;
+            for (int j = 0; j < n_rows; ++j) rank += (row_len[j] > mine || (row_len[j] == mine && j < (int)threadIdx.x)) ? 1 : 0;
+            o.dec_order[rank] = rows[threadIdx.x].tok_off;
+        }
+    } else {
+        for (int r = threadIdx.x; r < n_rows; r += 1024) o.dec_order[r] = rows[r].tok_off;
     }
     if (threadIdx.x == 0) {
         const RowDesc last = rows[n_rows - 1];
@@ -2208,6 +2223,364 @@ void attention_combine(hipStream_t s, const float * partial, int T, const AttnSh
     a.n_head = sh.n_head; a.G = sh.n_head / sh.n_head_kv; a.hd = sh.head_dim;
     hipLaunchKernelGGL(k_attention_combine, dim3(T, (sh.n_head + 3) / 4), dim3(256), 0, s, a);
     check_launch("attention_combine");
+}
+
+// ---------------------------------------------------------------------------
+// the attention of a pure decode step in one launch
+
+struct DecodeAttnArgs {
+    const float * qkv;                      // [T][QD + 2 KD] f32 (with the biases), when there are no slices
+    Slices from;                            // or the K-slices of the fused q, k, v product, added in slice order
+    const float * rope_cos, * rope_sin;     // [T][head_dim / 2]
+    const int32_t * pos, * seq, * kv_begin; // per row (= token) of the step
+    const int32_t * order;                  // rows, longest sequence first
+    const int32_t * table;
+    int max_pages;
+    __half * k_pool, * v_pool;
+    size_t page_stride, head_stride;
+    Act out;                                // the output projection's activations (hi/lo planes and block sums)
+    int n_head, n_kv, G, neox;
+    float qscale;
+};
+
+// One workgroup of eight waves per (row, kv head) of a step in which every row decodes one token, f16 cache, at
+// most eight query heads per kv head; it does what k_rope_store, k_attention<HD, true, true> and
+// k_attention_combine do for such a step in three launches:
+//   * every lane builds its part of the query operand itself: the K-slices of the q columns added in slice order,
+//     rotated (a rotation pair lies inside a lane's dims in both pairings), scaled, split into f16 hi and lo;
+//   * the sequence's pages are divided evenly among the eight waves (a division that depends on the sequence alone,
+//     so a row's result does not depend on what else the step holds); each wave runs the same online softmax over
+//     its pages as k_attention does over a work item;
+//   * the wave that owns the page of the new position also makes the new K and V row (slices, rotation, f16),
+//     stores them into the page for later steps and puts them into the operand registers it loaded for that page -
+//     no other wave of the launch reads that cell;
+//   * the eight partial results meet in LDS and waves 0 .. G - 1 merge them, one query head each, with
+//     k_attention_combine's arithmetic, and store the output projection's activations.
+template <int HD, int NW>
+__global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttnArgs a) {
+    constexpr int KS = HD / 32;     // k-steps of QK^T
+    constexpr int DT = HD / 16;     // dim tiles of PV
+    constexpr int PS = HD + 2;      // floats of one partial result: max, sum, output
+    constexpr int NT = NW * 64;
+    __shared__ float part[NW][8][PS];
+    __shared__ __attribute__((aligned(16))) _Float16 q_hi[8][HD], q_lo[8][HD], k_row[HD], v_row[HD];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const int t = a.order[blockIdx.x / a.n_kv], h = blockIdx.x % a.n_kv;
+    const int pos = a.pos[t], kv_begin = a.kv_begin[t], slot = a.seq[t];
+    const int cc = c & 7;
+    const bool col_ok = cc < a.G;
+    const bool lo_col = c >= 8;
+    const int QD = a.n_head * HD, KD = a.n_kv * HD, ROW = QD + 2 * KD;
+    const int page_first = kv_begin / PAGE, n_pages = pos / PAGE - page_first + 1;
+    const int per_wave = (n_pages + NW - 1) / NW;
+    const int my_first = page_first + wave * per_wave;
+    const int my_n = min(per_wave, max(0, n_pages - wave * per_wave));
+    const int last_owner = (n_pages - 1) / per_wave;
+    const int t32 = pos % PAGE;
+
+    // page ids of this wave's share, one per lane
+    const int my_pid = lane < my_n ? a.table[(size_t)slot * a.max_pages + my_first + lane] : 0;
+
+    // The workgroup's part of the step's q, k, v row, one column per thread and turn: the G query heads of this
+    // kv head, its k row and its v row ((G + 2) HD columns). A column is the sum of its K-slices in slice order; q
+    // and k columns are rotated with their partner column (which the thread adds up as well), q is scaled and
+    // split into f16 hi and lo. Everything lands in LDS, in element order.
+    auto column = [&](int col) {
+        float v = 0.0f;
+        if (a.from.n > 0) {
+            for (int k = 0; k < a.from.n; ++k) v += a.from.data[(size_t)k * a.from.stride + (size_t)t * ROW + col];
+        } else {
+            v = a.qkv[(size_t)t * ROW + col];
+        }
+        return v;
+    };
+    const float * cs = a.rope_cos + (size_t)t * (HD / 2), * sn = a.rope_sin + (size_t)t * (HD / 2);
+    for (int idx = threadIdx.x; idx < (a.G + 2) * HD; idx += NT) {
+        const int hh = idx / HD, d = idx % HD;          // hh < G: query head, G: k, G + 1: v
+        const int col0 = hh < a.G ? (h * a.G + hh) * HD : (hh == a.G ? QD + h * HD : QD + KD + h * HD);
+        float x = column(col0 + d);
+        if (hh <= a.G) {
+            // partner of the rotation pair and this element's place in it
+            const int pd = a.neox ? (d < HD / 2 ? d + HD / 2 : d - HD / 2) : (d ^ 1);
+            const bool first = a.neox ? d < HD / 2 : (d & 1) == 0;
+            const int i = a.neox ? (d < HD / 2 ? d : d - HD / 2) : (d >> 1);
+            const float y = column(col0 + pd);
+            const float cv = cs[i], sv = sn[i];
+            x = first ? x * cv - y * sv : y * sv + x * cv;
+        }
+        if (hh < a.G) {
+            const float sc = fminf(fmaxf(x * a.qscale, -65504.0f), 65504.0f);
+            const _Float16 hi = (_Float16)sc;
+            q_hi[hh][d] = hi;
+            q_lo[hh][d] = (_Float16)(sc - (float)hi);
+        } else {
+            const _Float16 v = (_Float16)fminf(fmaxf(x, -65504.0f), 65504.0f);
+            if (hh == a.G) k_row[d] = v; else v_row[d] = v;
+        }
+    }
+    __syncthreads();
+
+    h8 qreg[KS];
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+        if (col_ok) qreg[j] = *(const h8 *)&(lo_col ? q_lo : q_hi)[cc][32 * j + 8 * g];
+        else qreg[j] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+    }
+
+    // The new position's K and V row, by the wave that owns its page. K: lane (g, t32 % 16) holds dims 32 j + 8 g ..
+    // of the token in operand register 2 j + t32 / 16; V: lane (g = (t32 % 16) / 4, d) holds the token in slot
+    // (t32 % 4) + 4 (t32 / 16) of dim 16 dt + d. Those lanes keep the values for the operand registers of the page
+    // and store them into it for later steps.
+    const bool owner = wave == last_owner;
+    const bool k_lane = owner && (lane & 15) == (t32 & 15);
+    const bool v_lane = owner && g == ((t32 & 15) >> 2);
+    const int v_slot = (t32 & 3) + 4 * (t32 >> 4);
+    h8 k_new[KS];
+    _Float16 v_new[DT];
+#pragma unroll
+    for (int j = 0; j < KS; ++j) k_new[j] = (h8){0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int d = 0; d < DT; ++d) v_new[d] = (_Float16)0.0f;
+    if (owner) {
+        const int pid = __builtin_amdgcn_readlane(my_pid, my_n - 1);
+        if (k_lane) {
+            __half * dst = a.k_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
+#pragma unroll
+            for (int j = 0; j < KS; ++j) {
+                k_new[j] = *(const h8 *)&k_row[32 * j + 8 * g];
+                *(h8 *)(dst + ((((j * 2 + (t32 >> 4)) * 4 + g) * 16 + (t32 & 15)) * 8)) = k_new[j];
+            }
+        }
+        if (v_lane) {
+            __half * dst = a.v_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
+#pragma unroll
+            for (int d = 0; d < DT; ++d) {
+                v_new[d] = v_row[16 * d + (lane & 15)];
+                dst[((d * 4 + g) * 16 + (lane & 15)) * 8 + v_slot] = __builtin_bit_cast(__half, v_new[d]);
+            }
+        }
+    }
+
+    f4 o[DT];
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o[d] = (f4){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.0f;
+    struct KSet { h8 r[2 * KS]; };
+    struct VSet { h8 r[DT]; };
+    auto load_k = [&](int idx, KSet & ks) {
+        const int pid = __builtin_amdgcn_readlane(my_pid, idx);
+        const __half * kp = a.k_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            ks.r[2 * j] = load_h8(kp + ((j * 2 + 0) * 64 + lane) * 8);
+            ks.r[2 * j + 1] = load_h8(kp + ((j * 2 + 1) * 64 + lane) * 8);
+        }
+    };
+    auto load_v = [&](int idx, VSet & vs) {
+        const int pid = __builtin_amdgcn_readlane(my_pid, idx);
+        const __half * vp = a.v_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) vs.r[d] = load_h8(vp + (d * 64 + lane) * 8);
+    };
+    auto attend = [&](int pi, const KSet & ks, const VSet & vs, bool newest) {
+        h8 kreg[KS][2], vreg[DT];
+#pragma unroll
+        for (int j = 0; j < KS; ++j) { kreg[j][0] = ks.r[2 * j]; kreg[j][1] = ks.r[2 * j + 1]; }
+#pragma unroll
+        for (int d = 0; d < DT; ++d) vreg[d] = vs.r[d];
+        if (newest) {
+            // the page of the new position: what was loaded from its cell is replaced by the row made above
+            if (k_lane) {
+#pragma unroll
+                for (int j = 0; j < KS; ++j) {
+                    if (t32 >> 4) kreg[j][1] = k_new[j]; else kreg[j][0] = k_new[j];
+                }
+            }
+            if (v_lane) {
+#pragma unroll
+                for (int d = 0; d < DT; ++d)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) if (i == v_slot) vreg[d][i] = v_new[d];
+            }
+        }
+        f4 s0 = (f4){0.f, 0.f, 0.f, 0.f}, s1 = (f4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][0], qreg[j], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(kreg[j][1], qreg[j], s1, 0, 0, 0);
+        }
+        // the hi and lo products of a query sit 8 columns apart: both lanes take the sum
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            s0[i] += __shfl_xor(s0[i], 8, 64);
+            s1[i] += __shfl_xor(s1[i], 8, 64);
+        }
+        const int pbase = pi * PAGE + 4 * g;
+        float mx = -INFINITY;
+        // only the first and the last page of a sequence hold positions a column must not see
+        const bool edge = pi * PAGE < kv_begin || pi * PAGE + PAGE - 1 > pos;
+        if (edge) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int p0 = pbase + i, p1 = pbase + 16 + i;
+                if (!(col_ok && p0 >= kv_begin && p0 <= pos)) s0[i] = -INFINITY;
+                if (!(col_ok && p1 >= kv_begin && p1 <= pos)) s1[i] = -INFINITY;
+            }
+        } else if (!col_ok) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { s0[i] = -INFINITY; s1[i] = -INFINITY; }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fmaxf(s0[i], s1[i]));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = !col_ok ? 1.0f : exp2f(m_run - m_use);       // m_run = -inf -> 0
+        float psum = 0.0f;
+        h8 pt;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float e0 = exp2f(s0[i] - m_use), e1 = exp2f(s1[i] - m_use);
+            psum += e0 + e1;
+            const _Float16 h0 = (_Float16)e0, h1 = (_Float16)e1;
+            // the column of the lo query half multiplies the lo half of the same probabilities
+            pt[i] = lo_col ? (_Float16)(e0 - (float)h0) : h0;
+            pt[4 + i] = lo_col ? (_Float16)(e1 - (float)h1) : h1;
+        }
+        m_run = m_new;
+        // the running maximum rarely moves after the first pages: then every column's factor is exactly one
+        if (__any(alpha != 1.0f)) {
+            l_run *= alpha;
+#pragma unroll
+            for (int d = 0; d < DT; ++d)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) o[d][i] *= alpha;
+        }
+        l_run += psum;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt, o[d], 0, 0, 0);
+    };
+    // V of a page loads while its scores are computed, K of the next page (never skipped: past the end the last
+    // page again, so that the number of loads in flight is the same on every path) while the page is multiplied
+    if (my_n > 0) {
+        KSet kA, kB;
+        VSet v;
+        load_k(0, kA);
+        for (int i = 0; i < my_n; i += 2) {
+            load_v(i, v);
+            load_k(min(i + 1, my_n - 1), kB);
+            attend(my_first + i, kA, v, owner && i == my_n - 1);
+            if (i + 1 >= my_n) break;
+            load_v(i + 1, v);
+            load_k(min(i + 2, my_n - 1), kA);
+            attend(my_first + i + 1, kB, v, owner && i + 1 == my_n - 1);
+        }
+    }
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[d][i] += __shfl_xor(o[d][i], 8, 64);
+    if (col_ok && !lo_col) {
+        float * dst = part[wave][cc];
+        if (g == 0) { dst[0] = m_run; dst[1] = l_run; }
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dst[2 + d * 16 + 4 * g + i] = o[d][i];
+    }
+    __syncthreads();
+    // wave gi merges the eight partial results of query head h G + gi (a wave without pages left max = -inf, sum = 0)
+    for (int gi = wave; gi < a.G; gi += NW) {
+    const int e0 = 2 * lane;
+    float m_s = -INFINITY, l_s = 0.0f;
+    if (lane < NW) { m_s = part[lane][gi][0]; l_s = part[lane][gi][1]; }
+    float M = m_s;
+    for (int ofs = 32; ofs > 0; ofs >>= 1) M = fmaxf(M, __shfl_xor(M, ofs, 64));
+    const float w_s = m_s == -INFINITY ? 0.0f : exp2f(m_s - M);
+    const float L = wave_sum(w_s * l_s);
+    float v0 = 0.0f, v1 = 0.0f;
+    if (e0 < HD) {
+#pragma unroll
+        for (int sp = 0; sp < NW; ++sp) {
+            const float w = __shfl(w_s, sp, 64);
+            v0 = fmaf(w, part[sp][gi][2 + e0], v0);
+            v1 = fmaf(w, part[sp][gi][2 + e0 + 1], v1);
+        }
+    } else {
+#pragma unroll
+        for (int sp = 0; sp < NW; ++sp) (void)__shfl(w_s, sp, 64);
+    }
+    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+    const bool mine = e0 < HD;
+    const float f0 = mine ? v0 * inv : 0.0f, f1 = mine ? v1 * inv : 0.0f;
+    const int k = (h * a.G + gi) * HD + e0;
+    float r0 = 0.0f, r1 = 0.0f;
+    if (mine) {
+        const float c0 = fminf(fmaxf(f0, -65504.0f), 65504.0f), c1 = fminf(fmaxf(f1, -65504.0f), 65504.0f);
+        const __half h0 = __float2half_rn(c0), h1 = __float2half_rn(c1);
+        const __half l0 = __float2half_rn(c0 - __half2float(h0)), l1 = __float2half_rn(c1 - __half2float(h1));
+        const size_t at = act_at(t, k, 0, QD), at_lo = act_at(t, k, 1, QD);
+        a.out.x[at] = h0;
+        a.out.x[at + 1] = h1;
+        a.out.x[at_lo] = l0;
+        a.out.x[at_lo + 1] = l1;
+        r0 = __half2float(h0) + __half2float(l0);
+        r1 = __half2float(h1) + __half2float(l1);
+    }
+    if (a.out.sums) {
+        float sum = r0 + r1;
+#pragma unroll
+        for (int ofs = 1; ofs < 16; ofs <<= 1) sum += __shfl_xor(sum, ofs, 64);
+        if ((lane & 15) == 0 && mine) {
+            const int b = k / 32;
+            const __half hi = sat_half(sum);
+            a.out.sums[act_sum_at(t, b, 0, QD)] = hi;
+            a.out.sums[act_sum_at(t, b, 1, QD)] = __float2half_rn(sum - __half2float(hi));
+        }
+    }
+    }
+}
+
+bool attention_decode_can(const AttnShape & sh, bool q_or_k_norm, int max_positions) {
+    const int G = sh.n_head_kv > 0 ? sh.n_head / sh.n_head_kv : 0;
+    return sh.kv_quant == KV_F16 && !q_or_k_norm && (sh.head_dim == 128 || sh.head_dim == 64) && sh.rope_dim == sh.head_dim
+        && G >= 1 && G <= 8 && sh.n_head % sh.n_head_kv == 0 && max_positions <= 4 * 64 * PAGE;       // a wave holds one page id per lane, and a workgroup may have four waves
+}
+
+void attention_decode(hipStream_t s, const float * qkv, const Slices & from, int n_rows, const AttnShape & sh,
+                      const PackBuffers & pk, const int32_t * table, int max_pages, __half * k_pool, __half * v_pool,
+                      const Act & out) {
+    if (n_rows <= 0) return;
+    if (!attention_decode_can(sh, false, 0)) throw std::runtime_error("attention_decode: unsupported shape or cache type");
+    check_act_out(out, sh.n_head * sh.head_dim, "attention_decode", n_rows);
+    if (!out.x) throw std::runtime_error("attention_decode: needs the plain activation planes");
+    if (sh.page_stride == 0 || sh.head_stride == 0) throw std::runtime_error("attention_decode: the pool's strides are missing");
+    const int ROW = (sh.n_head + 2 * sh.n_head_kv) * sh.head_dim;
+    if (from.n > 0 && from.N != ROW) throw std::runtime_error("attention_decode: the slices are not a fused q, k, v product");
+    if (!pk.dec_order) throw std::runtime_error("attention_decode: the step's rows were not ordered");
+    DecodeAttnArgs a;
+    a.qkv = qkv; a.from = from; a.rope_cos = pk.rope_cos; a.rope_sin = pk.rope_sin;
+    a.pos = pk.pos; a.seq = pk.seq; a.kv_begin = pk.tile_kv_begin; a.order = pk.dec_order;
+    a.table = table; a.max_pages = max_pages; a.k_pool = k_pool; a.v_pool = v_pool;
+    a.page_stride = sh.page_stride; a.head_stride = sh.head_stride;
+    a.out = out;
+    a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.G = sh.n_head / sh.n_head_kv; a.neox = sh.rope_neox ? 1 : 0;
+    a.qscale = 1.4426950408889634f / sqrtf((float)sh.head_dim);
+    const dim3 grid(n_rows * sh.n_head_kv);
+    static const int nw = [] { const char * v = std::getenv("RETRO_DECODE_ATTENTION_WAVES"); return v && std::atoi(v) == 4 ? 4 : 8; }();
+    if (nw == 8) {
+        if (sh.head_dim == 128) hipLaunchKernelGGL((k_attention_decode<128, 8>), grid, dim3(512), 0, s, a);
+        else hipLaunchKernelGGL((k_attention_decode<64, 8>), grid, dim3(512), 0, s, a);
+    } else {
+        if (sh.head_dim == 128) hipLaunchKernelGGL((k_attention_decode<128, 4>), grid, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL((k_attention_decode<64, 4>), grid, dim3(256), 0, s, a);
+    }
+    check_launch("attention_decode");
 }
 
 // ---------------------------------------------------------------------------

@@ -284,6 +284,7 @@ struct PackBuffers {       // device arrays, sized for n_batch tokens / rows
     int4 * item_a;         // [n_items, longest first] first flat token of the tile, tokens in the tile | kv head << 8, the item's number, slot
     int4 * item_b;         // [n_items] position of the first token, first resident position of the slot,
                            //           first page index of this split, pages in this split
+    int32_t * dec_order;   // [n_rows] rows by resident length, longest first (the order the decode-step attention starts its workgroups in)
     float * rope_cos;      // [T][rope_dim/2]
     float * rope_sin;
     int split_pages = MAX_SPLIT_PAGES;   // pages per attention work item in this step (set from count_attention_work)
@@ -359,6 +360,14 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
                const int32_t * table, int max_pages, const __half * k_pool, const __half * v_pool,
                int n_items, int n_tiles, float * partial, bool one_token_rows = false);
 // Merges the splits: out act [T][QD] (+ block sums).
+// The three launches above in one, for a step in which every row decodes one token over an f16 cache (see
+// k_attention_decode): reads the q, k, v product (its K-slices or the buffer), stores the new K and V rows, writes the
+// output projection's activations. attention_decode_can: whether the shape allows it (head dims 64 / 128 rotated
+// over their whole width, at most eight query heads per kv head, no q / k norm, sequences of at most 16384 positions).
+bool attention_decode_can(const AttnShape & sh, bool q_or_k_norm, int max_positions);
+void attention_decode(hipStream_t s, const float * qkv, const Slices & from, int n_rows, const AttnShape & sh,
+                      const PackBuffers & pk, const int32_t * table, int max_pages, __half * k_pool, __half * v_pool,
+                      const Act & out);
 void attention_combine(hipStream_t s, const float * partial, int T, const AttnShape & sh,
                        const PackBuffers & pk, const Act & out);
 size_t attention_partial_floats(int n_items, int head_dim);

@@ -1,0 +1,79 @@
+"""The one-launch attention of pure decode steps (k_attention_decode: rotation, KV store, attention and split merge)
+against the three launches it replaces (k_rope_store, k_attention, k_attention_combine; RETRO_FUSED_DECODE_ATTENTION=0)
+on the same model and requests, and against the CPU oracle: llama's adjacent-pair rotation with heads of 128 and the
+NeoX pairing with heads of 64 and q/k/v biases, sequences from one page to many (so that the eight waves of a
+workgroup hold nothing, one page or several), a sequence whose beginning was removed, and steps of one row."""
+import numpy as np
+import pytest
+
+import oracle
+from engine_helpers import assert_logits_close, greedy, logit_errors
+from retrograd_amd import engine as E
+from retrograd_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = {
+    "llama-hd128": synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, n_embd=1024, n_head=8, n_head_kv=2, head_dim=128,
+                                n_ff=2048, n_vocab=2048, name="llama-q4k-hd128"),
+    "qwen2-hd64": synth.scaled(synth.QWEN25_7B_Q8, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
+                               n_ff=1024, n_vocab=1024, matrix_type=12, name="qwen2-q4k-hd64"),
+}
+
+
+@pytest.mark.parametrize("key", list(SHAPES))
+def test_one_launch_equals_three_and_the_oracle(key, tmp_path, monkeypatch):
+    shape = SHAPES[key]
+    print("decode attention:", shape.name, flush=True)
+    path = tmp_path / "m.gguf"
+    synth.write_model(path, shape, seed=31, device="cpu", std=0.05)
+    cfg = E.EngineConfig(n_ctx=8 * 1024, n_seq_max=8, n_batch=256, n_ubatch=256)
+    monkeypatch.setenv("RETRO_FUSED_DECODE_ATTENTION", "1")
+    one = E.Engine(path, cfg)
+    monkeypatch.setenv("RETRO_FUSED_DECODE_ATTENTION", "0")
+    three = E.Engine(path, cfg)
+    m = oracle.Model(path)
+    ctx = oracle.Context(m, 8)
+    rng = np.random.default_rng(4)
+    lens = [1, 31, 32, 33, 250, 700, 95]          # positions 0 .. len - 1 resident before the decode steps
+    prompts = [rng.integers(0, shape.n_vocab, n) for n in lens]
+    out = E.StepOutput()
+    for eng in (one, three):
+        for i, p in enumerate(prompts):
+            for at in range(0, len(p), 256):
+                eng.step([E.StepRow(i, i, p[at:at + 256], at, sample=False, sampling=greedy())], out)
+    for i, p in enumerate(prompts):
+        ctx.step_rows([(i, 0, p, False)])
+    # slot 5 loses its first 100 positions: its resident span starts inside a page
+    for x in (one, three, ctx):
+        x.seq_rm(5, 0, 100)
+    pos = list(lens)
+    feed = [int(t) for t in rng.integers(0, shape.n_vocab, len(lens))]
+    for step in range(3):
+        rows = list(range(len(lens))) if step != 1 else [4]          # all rows, one row, all rows
+        got = {}
+        for name, eng in (("one", one), ("three", three)):
+            eng.step([E.StepRow(i, i, [feed[i]], pos[i], sample=True, sampling=greedy()) for i in rows], out)
+            got[name] = (eng.debug_logits().copy(), [out.row(j).token for j in range(len(rows))])
+        want = ctx.step_rows([(i, pos[i], [feed[i]], True) for i in rows])
+        assert_logits_close(got["one"][0], want)
+        assert_logits_close(got["three"][0], want)
+        mx, rel = logit_errors(got["one"][0], got["three"][0])
+        print("step %d: one launch against three, max %.2e rel %.2e" % (step, mx, rel), flush=True)
+        assert rel <= 2e-5, (mx, rel)
+        # the rows written into the cache are the same values
+        kd = shape.n_head_kv * shape.head_dim
+        for i in rows:
+            for want_v in (False, True):
+                a = one.debug_kv(1, i, pos[i], want_v, kd).astype(np.float32)
+                b = three.debug_kv(1, i, pos[i], want_v, kd).astype(np.float32)
+                bad = np.flatnonzero(~np.isclose(a, b, rtol=2e-3, atol=1e-4 * np.abs(b).max()))      # layer 1 sees layer 0's attention, equal to 1e-5
+                assert bad.size == 0, (i, want_v, bad[:8], a[bad[:8]], b[bad[:8]])
+        for j, i in enumerate(rows):
+            srt = np.sort(want[j])[::-1]
+            if srt[0] - srt[1] > 4e-2:
+                assert got["one"][1][j] == int(want[j].argmax())
+            feed[i] = int(want[j].argmax())
+            pos[i] += 1
+    one.close()
+    three.close()

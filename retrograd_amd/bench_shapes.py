@@ -5,6 +5,7 @@ measures the headline):
     python -m retrograd_amd.bench_shapes c4        # multi-LoRA decode, Qwen2.5-7B shape, Q8_0 base
     python -m retrograd_amd.bench_shapes c5        # mixture of experts, Qwen3-30B-A3B shape, MXFP4 experts
     python -m retrograd_amd.bench_shapes c5-q4km   # the same shape with the type mix of a Q4_K_M file
+    python -m retrograd_amd.bench_shapes mxfp4-scaled   # the block-scaled FP4 x FP8 product at c5's expert sizes
 
 c4: 28 layers, hidden 3584, 28 / 4 heads, FFN 18944, vocabulary 152064, eight
 rank-16 F16 adapters on q/k/v/o (A ~ N(0, 0.02), B ~ N(0, 0.01)), 64 sequences
@@ -18,7 +19,12 @@ Weights are synthetic (seeded), prompts random token ids. Prefill runs first,
 untimed for the decode figure; then `--new` decode steps over all sequences: the
 first part is timed as it is, the last `--profiled` steps run with an event pair
 around every kernel category (which slows them a little) for the breakdown.
-Prints one JSON line."""
+Prints one JSON line.
+
+mxfp4-scaled times one kernel, not a step: MXFP4 rows times 1 to 16 tokens under ggml's arithmetic on the
+block-scaled matrix instruction, as one dense matrix of the size of a layer's expert weights (gate and up of 128
+experts: 196608 rows of 2048; down: 262144 rows of 768), every launch on another copy of the weights so that they
+come from HBM."""
 from __future__ import annotations
 
 import argparse
@@ -33,7 +39,7 @@ import numpy as np
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("config", choices=["c4", "c5", "c5-q4km"])
+    ap.add_argument("config", choices=["c4", "c5", "c5-q4km", "mxfp4-scaled"])
     ap.add_argument("--new", type=int, default=128)
     ap.add_argument("--profiled", type=int, default=32)
     ap.add_argument("--model-dir", default=os.environ.get("RETRO_BENCH_MODEL_DIR", "/dev/shm"))
@@ -49,6 +55,17 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench_shapes needs an MI355X: no HIP device is visible", file=sys.stderr)
         return 2
+    if args.config == "mxfp4-scaled":
+        out = {"kernel": "k_mxs", "arithmetic": "ggml (Q8_0 activation blocks)", "weights": "pseudo-random, from HBM", "cases": []}
+        for what, n, k in (("gate_up", 2 * 128 * 768, 2048), ("down", 128 * 2048, 768)):
+            for t in (1, 4, 8, 16):
+                us = E.kernel_mxfp4_scaled_time(n, k, t, True, 50)
+                nbytes = n * (k // 32) * 17
+                out["cases"].append({"matrix": what, "rows": n, "k": k, "tokens": t, "us": round(us, 2),
+                                     "weight_bytes": nbytes, "tb_per_s": round(nbytes / us / 1e6, 3),
+                                     "frac_of_8_tb_per_s": round(nbytes / us / 1e6 / 8.0, 3)})
+        print(json.dumps(out))
+        return 0
     rng = np.random.default_rng(args.seed)
     if args.config == "c4":
         shape, n_seq = synth.QWEN25_7B_Q8, 64

@@ -15,7 +15,7 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libretro_hip.so"
-SOURCES = ["kernels.hip", "mm_lds.hip", "gemv.hip", "moe.hip", "engine.cpp", "generate.cpp", "capi.cpp", "capi_trainer.cpp", "capi_test.cpp"]
+SOURCES = ["kernels.hip", "mm_lds.hip", "gemv.hip", "moe.hip", "mxfp4_scaled.hip", "engine.cpp", "generate.cpp", "capi.cpp", "capi_trainer.cpp", "capi_test.cpp"]
 # host-only sources (the step scheduler): plain C++, no device pass
 HOST_SOURCES = ["sched/prefix_tree.cpp", "sched/scheduler.cpp", "sched/fake_backend.cpp", "sched/engine_backend.cpp",
                 "sched/capi_sched.cpp"]

@@ -290,6 +290,74 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
     });
 }
 
+int retro_kernel_mxfp4_scaled(const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, int32_t n_tokens, float * y) {
+    return guarded([&]() -> int {
+        if (!rk::mxs_can(k, n_rows, n_tokens))
+            throw std::runtime_error("mxfp4_scaled: rows in 16s, columns in 256s (at most 4608), 1..16 tokens");
+        const size_t bytes = (size_t)n_rows * (size_t)(k / 32) * 17;
+        DevBuf d_raw, d_packed, d_x, d_ops, d_dx, d_y;
+        d_raw.alloc(bytes);
+        ok(hipMemcpy(d_raw.ptr, raw, bytes, hipMemcpyHostToDevice), "upload weights");
+        d_packed.alloc(rk::mxs_packed_bytes(k, n_rows));
+        rk::mxs_repack(nullptr, d_raw.as<uint8_t>(), d_packed.as<uint8_t>(), (int)k, n_rows);
+        d_x.alloc((size_t)n_tokens * k * 4);
+        ok(hipMemcpy(d_x.ptr, x, d_x.bytes, hipMemcpyHostToDevice), "upload activations");
+        d_ops.alloc(rk::mxs_operand_bytes((int)k));
+        d_dx.alloc(rk::mxs_scale_bytes((int)k));
+        rk::mxs_quantise(nullptr, d_x.as<float>(), n_tokens, (int)k, d_ops.as<uint8_t>(), d_dx.as<float>());
+        d_y.alloc((size_t)n_tokens * n_rows * 4);
+        rk::mxs_matmul(nullptr, d_packed.as<uint8_t>(), d_ops.as<uint8_t>(), d_dx.as<float>(), (int)k, n_rows, n_tokens, d_y.as<float>());
+        ok(hipMemcpy(y, d_y.ptr, d_y.bytes, hipMemcpyDeviceToHost), "download");
+        return 0;
+    });
+}
+
+int retro_kernel_mxfp4_scaled_time(int64_t n_rows, int64_t k, int32_t n_tokens, int32_t cold, int32_t iters, double * out_us) {
+    return guarded([&]() -> int {
+        if (!rk::mxs_can(k, n_rows, n_tokens) || iters <= 0)
+            throw std::runtime_error("mxfp4_scaled_time: rows in 16s, columns in 256s (at most 4608), 1..16 tokens, at least one launch");
+        const size_t bytes = rk::mxs_packed_bytes(k, n_rows);
+        const size_t copies = cold ? std::max<size_t>(2, ((size_t)1 << 30) / bytes) : 1;
+        DevBuf d_w, d_x, d_ops, d_dx, d_y;
+        d_w.alloc(bytes * copies);
+        {
+            // pseudo-random nibbles; the exponent bytes (the last 128 of every 2176) between 2^-8 and 2^7
+            std::vector<uint8_t> host(bytes);
+            uint32_t state = 0x9e3779b9u;
+            for (size_t i = 0; i < bytes; ++i) {
+                state = state * 1664525u + 1013904223u;
+                host[i] = (i % 2176 >= 2048) ? (uint8_t)(119 + ((state >> 24) & 15)) : (uint8_t)(state >> 24);
+            }
+            for (size_t c = 0; c < copies; ++c) ok(hipMemcpy(d_w.as<uint8_t>() + c * bytes, host.data(), bytes, hipMemcpyHostToDevice), "fill");
+            std::vector<float> xs((size_t)n_tokens * k);
+            for (float & v : xs) { state = state * 1664525u + 1013904223u; v = (float)((int)(state >> 16) - 32768) / 32768.0f; }
+            d_x.alloc(xs.size() * 4);
+            ok(hipMemcpy(d_x.ptr, xs.data(), d_x.bytes, hipMemcpyHostToDevice), "fill");
+        }
+        d_ops.alloc(rk::mxs_operand_bytes((int)k));
+        d_dx.alloc(rk::mxs_scale_bytes((int)k));
+        rk::mxs_quantise(nullptr, d_x.as<float>(), n_tokens, (int)k, d_ops.as<uint8_t>(), d_dx.as<float>());
+        d_y.alloc((size_t)n_tokens * n_rows * 4);
+        hipEvent_t e0, e1;
+        ok(hipEventCreate(&e0), "event"); ok(hipEventCreate(&e1), "event");
+        size_t turn = 0;
+        auto run = [&]() {
+            rk::mxs_matmul(nullptr, d_w.as<uint8_t>() + (turn++ % copies) * bytes, d_ops.as<uint8_t>(), d_dx.as<float>(), (int)k, n_rows,
+                           n_tokens, d_y.as<float>());
+        };
+        for (int i = 0; i < 3; ++i) run();
+        ok(hipEventRecord(e0, nullptr), "record");
+        for (int i = 0; i < iters; ++i) run();
+        ok(hipEventRecord(e1, nullptr), "record");
+        ok(hipEventSynchronize(e1), "sync");
+        float ms = 0;
+        ok(hipEventElapsedTime(&ms, e0, e1), "elapsed");
+        (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+        *out_us = (double)ms * 1e3 / iters;
+        return 0;
+    });
+}
+
 int retro_kernel_stream_time(int64_t bytes, int32_t read_only, int32_t iters, double * out_us) {
     return guarded([&]() -> int {
         DevBuf src, dst;

@@ -143,6 +143,21 @@ size_t matmul_workspace_bytes();
 constexpr int GEMV_MAX_T = 2;     // beyond two tokens the tile kernels are as fast
 bool gemv_can(const Weight & w, const Act & x, int T);
 void gemv(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias);
+// MXFP4 weights times the Q8_0 blocks of at most MXS_MAX_TOKENS tokens on the block-scaled FP4 x FP8 matrix
+// instruction (ggml's arithmetic for MXFP4: integer code products per block of 32, times both block scales).
+// mxs_repack lays the GGUF rows out in the kernel's records (mxs_packed_bytes), mxs_quantise converts f32 rows to
+// the kernel's activation operands (mxs_operand_bytes) and block scales (mxs_scale_bytes), mxs_matmul writes
+// y [n_tokens][N]. Columns in 128s, rows in 16s; K is bounded by the operands having to fit LDS (mxs_lds_bytes).
+constexpr int MXS_MAX_TOKENS = 16;
+bool mxs_can(int64_t K, int64_t N, int n_tokens);
+size_t mxs_packed_bytes(int64_t K, int64_t N);
+size_t mxs_operand_bytes(int K);
+size_t mxs_scale_bytes(int K);
+size_t mxs_lds_bytes(int K);
+void mxs_repack(hipStream_t s, const uint8_t * raw, uint8_t * packed, int K, int64_t N);
+void mxs_quantise(hipStream_t s, const float * x, int n_tokens, int K, uint8_t * operands, float * scales);
+void mxs_matmul(hipStream_t s, const uint8_t * packed, const uint8_t * operands, const float * scales, int K, int64_t N,
+                int n_tokens, float * y);
 // The weight's side of gemv_can. With it the same product can take its rows as f32 and make the Q8_K blocks while
 // it stages them, one launch instead of two: gemv_norm from the residual rows (x row rows[t], or t; RMSNorm with
 // norm_w and eps as rmsnorm_act computes it, then the conversion), gemv_swiglu from the f32 rows of a gate/up product

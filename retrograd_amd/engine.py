@@ -139,7 +139,7 @@ STEP_SYMBOLS = [
     "retro_grammar_gbnf", "retro_grammar_free", "retro_last_error",
 ]
 KERNEL_SYMBOLS = [
-    "retro_kernel_matmul", "retro_kernel_gemv_fused", "retro_kernel_matmul_time", "retro_kernel_stream_time", "retro_kernel_sample_prepare", "retro_kernel_sample_greedy_noalloc", "retro_kernel_sample_greedy_noalloc_max_rows", "retro_kernel_page_size", "retro_kernel_max_topk",
+    "retro_kernel_matmul", "retro_kernel_gemv_fused", "retro_kernel_matmul_time", "retro_kernel_mxfp4_scaled", "retro_kernel_mxfp4_scaled_time", "retro_kernel_stream_time", "retro_kernel_sample_prepare", "retro_kernel_sample_greedy_noalloc", "retro_kernel_sample_greedy_noalloc_max_rows", "retro_kernel_page_size", "retro_kernel_max_topk",
     "retro_engine_debug_logits", "retro_engine_debug_kv", "retro_engine_debug_pack", "retro_engine_debug_pages",
     "retro_engine_debug_profile", "retro_engine_debug_profile_categories", "retro_engine_debug_profile_read",
 ]
@@ -227,6 +227,8 @@ def load_library() -> C.CDLL:
     lib.retro_kernel_gemv_fused.restype = C.c_int
     lib.retro_kernel_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,
                                              C.c_int32, C.c_int32, C.POINTER(C.c_double)]
+    lib.retro_kernel_mxfp4_scaled.argtypes = [_u8p, C.c_int64, C.c_int64, _f32p, C.c_int32, _f32p]
+    lib.retro_kernel_mxfp4_scaled_time.argtypes = [C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_double)]
     lib.retro_kernel_stream_time.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_double)]
     lib.retro_kernel_page_size.restype = C.c_int32
     lib.retro_kernel_max_topk.restype = C.c_int32
@@ -918,6 +920,28 @@ def kernel_matmul_time(ggml_type: int, n_rows: int, k: int, n_tokens: int, mode:
     out = C.c_double()
     s = load_library().retro_kernel_matmul_time(ggml_type, n_rows, k, n_tokens, mode, iters, debug, force_ksplit,
                                                 C.byref(out))
+    if s != 0:
+        _raise(s)
+    return out.value
+
+
+def kernel_mxfp4_scaled(raw, n_rows: int, k: int, x: np.ndarray) -> np.ndarray:
+    """MXFP4 rows times at most 16 tokens on the block-scaled matrix instruction, ggml's arithmetic."""
+    src = np.ascontiguousarray(raw, np.uint8)
+    x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
+    y = np.empty((x.shape[0], n_rows), np.float32)
+    s = load_library().retro_kernel_mxfp4_scaled(src.ctypes.data_as(C.POINTER(C.c_uint8)), n_rows, k,
+                                                 x.ctypes.data_as(C.POINTER(C.c_float)), x.shape[0],
+                                                 y.ctypes.data_as(C.POINTER(C.c_float)))
+    if s != 0:
+        _raise(s)
+    return y
+
+
+def kernel_mxfp4_scaled_time(n_rows: int, k: int, n_tokens: int, cold: bool = True, iters: int = 50) -> float:
+    """Microseconds per launch of kernel_mxfp4_scaled's product on device-only data."""
+    out = C.c_double()
+    s = load_library().retro_kernel_mxfp4_scaled_time(n_rows, k, n_tokens, 1 if cold else 0, iters, C.byref(out))
     if s != 0:
         _raise(s)
     return out.value

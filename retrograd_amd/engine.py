@@ -98,6 +98,28 @@ class CStepRowV2(C.Structure):
                 ("want_logprob", C.c_uint8), ("adapter", C.c_int32)]
 
 
+def _ffi_row_dtype() -> np.dtype:
+    """CStepRowV2 as a numpy record (pointers as addresses, the sampling block's fields under "s.")."""
+    kinds = {C.c_uint32: "<u4", C.c_int32: "<i4", C.c_float: "<f4", C.c_bool: "?", C.c_uint8: "u1"}
+    names, formats, offsets = [], [], []
+
+    def walk(struct, base, prefix):
+        for name, ctype in struct._fields_:
+            at = base + getattr(struct, name).offset
+            if isinstance(ctype, type) and issubclass(ctype, C.Structure):
+                walk(ctype, at, "s.")
+                continue
+            names.append(prefix + name)
+            formats.append(kinds.get(ctype, "<u8"))        # the rest are pointers
+            offsets.append(at)
+
+    walk(CStepRowV2, 0, "")
+    return np.dtype({"names": names, "formats": formats, "offsets": offsets, "itemsize": C.sizeof(CStepRowV2)})
+
+
+_FFI_ROW_DTYPE = _ffi_row_dtype()
+
+
 class CStepOutRowV2(C.Structure):
     _fields_ = [("struct_size", C.c_uint32), ("token", C.c_int32), ("logprob", C.c_float),
                 ("n_top", C.c_uint32), ("forced", C.c_uint8), ("sampled", C.c_uint8),
@@ -373,6 +395,7 @@ class StepOutput:
         self.n_top_stride = 0
         self.n_rows = 0
         self._ffi_rows = None
+        self._view = None
         self._rows = None
         self.top_ids = np.zeros(0, np.int32)
         self.top_logprobs = np.zeros(0, np.float32)
@@ -383,6 +406,7 @@ class StepOutput:
         if n_rows > self._cap:
             self._cap = max(n_rows, 2 * self._cap)
             self._ffi_rows = (CStepRowV2 * self._cap)()
+            self._view = np.frombuffer(self._ffi_rows, dtype=_FFI_ROW_DTYPE)
             self._rows = (CStepOutRowV2 * self._cap)()
         if stride != self.n_top_stride or self.top_ids.size < self._cap * stride:
             self.n_top_stride = stride
@@ -437,15 +461,71 @@ class Engine:
         stride = max((r.n_top_logprobs for r in rows), default=0)
         out._reserve(n, stride)
         out._keep = keep = []
+        lens = [len(r.tokens) for r in rows]
+        requests = [r.request for r in rows]
+        pos0 = [r.pos0 for r in rows]
+        sample = [bool(r.sample) for r in rows]
+        sp = [r.sampling for r in rows]
+        self._check_rows(rows, lens, requests, pos0, sample, sp)
+        if n:
+            # The FFI rows are filled column by column through a numpy view of the ctypes array (a Python
+            # assignment per field and row costs several times the C call's own host work at 64 rows).
+            v = out._view[:n]
+            if max(lens) == 1:
+                flat = np.array([r.tokens[0] for r in rows], dtype=np.int32)
+            else:
+                flat = np.concatenate([np.asarray(r.tokens, dtype=np.int32).ravel() for r in rows])
+            keep.append(flat)
+            lens_a = np.array(lens, dtype=np.uint64)
+            v["struct_size"] = C.sizeof(CStepRowV2)
+            v["tokens"] = flat.ctypes.data + 4 * (np.cumsum(lens_a) - lens_a)
+            v["n"] = lens_a
+            v["request"] = requests
+            v["slot"] = [r.slot for r in rows]
+            v["pos0"] = pos0
+            v["sample"] = sample
+            v["n_top_logprobs"] = [r.n_top_logprobs for r in rows]
+            v["want_logprob"] = [1 if r.want_logprob else 0 for r in rows]
+            v["adapter"] = [r.adapter.value for r in rows]
+            v["s.struct_size"] = C.sizeof(CSamplingParamsV2)
+            one = sp[0] if all(s is sp[0] for s in sp) else None        # rows that share one parameter object
+            for name in ("temperature", "top_p", "max_new_tokens", "top_k", "min_p", "repeat_penalty",
+                         "frequency_penalty", "presence_penalty", "penalty_window"):
+                v["s." + name] = getattr(one, name) if one is not None else [getattr(s, name) for s in sp]
+            v["s.seed"] = one.seed & 0xFFFFFFFF if one is not None else [s.seed & 0xFFFFFFFF for s in sp]
+            v["s.n_logit_bias"] = 0
+            v["s.logit_bias_ids"] = 0
+            v["s.logit_bias_values"] = 0
+            v["s.grammar"] = 0
+            for i, s in enumerate(sp):           # the rows that point at more: bias lists, a grammar text
+                if s.logit_bias or s.grammar is not None:
+                    self._fill_sampling_v2(out._ffi_rows[i].sampling, s, keep)
+        top_ids = out.top_ids.ctypes.data_as(_i32p) if stride else None
+        top_lps = out.top_logprobs.ctypes.data_as(_f32p) if stride else None
+        status = self._lib.retro_engine_step_v2(self._h, out._ffi_rows, n, out._rows, top_ids, top_lps, stride)
+        out._keep = []
+        if status != 0:
+            _raise(status)
+        out.n_rows = n
+
+    @staticmethod
+    def _check_rows(rows, lens, requests, pos0, sample, sp) -> None:
+        """The caller-side checks of StepRow::to_ffi_v2 / step_with (reference step.rs:150-203, 412-505): one
+        pass over the columns decides whether anything is wrong; the error is then the first in row order."""
+        if not rows:
+            return
+        live = [q for q in requests if q >= 0]
+        if (min(lens) > 0 and min(pos0) >= 0 and max(p + n for p, n in zip(pos0, lens)) <= 2 ** 31 - 1
+                and len(set(live)) == len(live) and not any(s and q < 0 for s, q in zip(sample, requests))
+                and not any(len(s.logit_bias) > 4096 for s in sp if s.logit_bias)):
+            return
         seen = set()
-        for i, r in enumerate(rows):
-            # Same caller-side checks as StepRow::to_ffi_v2 / step_with
-            # (reference step.rs:150-203, 412-505).
-            if len(r.tokens) == 0:
+        for r, n_tok in zip(rows, lens):
+            if n_tok == 0:
                 raise InvalidArgument("a step row requires at least one token")
             if r.pos0 < 0:
                 raise InvalidArgument("a step row's pos0 must be >= 0")
-            if r.pos0 + len(r.tokens) > 2 ** 31 - 1:
+            if r.pos0 + n_tok > 2 ** 31 - 1:
                 raise EngineError("a step row's position range overflows i32")
             if r.sample and r.request < 0:
                 raise InvalidArgument("a sampling step row requires a request id >= 0")
@@ -455,22 +535,6 @@ class Engine:
                 if r.request in seen:
                     raise InvalidArgument("a request id appears twice in one step")
                 seen.add(r.request)
-            toks = np.ascontiguousarray(r.tokens, dtype=np.int32)
-            keep.append(toks)
-            f = out._ffi_rows[i]
-            f.struct_size = C.sizeof(CStepRowV2)
-            f.request, f.slot = r.request, r.slot
-            f.tokens = toks.ctypes.data_as(_i32p)
-            f.n, f.pos0, f.sample = toks.size, r.pos0, r.sample
-            self._fill_sampling_v2(f.sampling, r.sampling, keep)
-            f.n_top_logprobs, f.want_logprob, f.adapter = r.n_top_logprobs, 1 if r.want_logprob else 0, r.adapter.value
-        top_ids = out.top_ids.ctypes.data_as(_i32p) if stride else None
-        top_lps = out.top_logprobs.ctypes.data_as(_f32p) if stride else None
-        status = self._lib.retro_engine_step_v2(self._h, out._ffi_rows, n, out._rows, top_ids, top_lps, stride)
-        out._keep = []
-        if status != 0:
-            _raise(status)
-        out.n_rows = n
 
     def step_v1(self, rows: Sequence[tuple], n_top_stride: int = 0):
         """retro_engine_step with v1 rows: (request, slot, tokens, pos0, sample,

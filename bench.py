@@ -395,7 +395,9 @@ def main() -> int:
         kcells = kdec[2] / ksteps
         cats = matrix_bytes_by_category(hp, synth, gw)
         fam_ms = fam_bytes = fam_launches = 0.0
-        rows = [("k_attention<128, true, true>", "attention", kv_bytes_per_cell_layer * kcells)]
+        attn_name = ("k_attention_decode<128, 8> (rotation, KV store, attention and split merge of a pure decode step)"
+                     if args.kv == "f16" else "k_attention<128, true, true> over a %s cache" % args.kv)
+        rows = [(attn_name, "attention", kv_bytes_per_cell_layer * kcells)]
         rows += [("%s (%s)" % (mm_name, c), c, cats[c]) for c in ("qkv", "o_proj", "gate_up", "down")]
         for name, cat, by in rows:
             ms, n = kprof[cat]

@@ -2287,29 +2287,88 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
     // kv head, its k row and its v row ((G + 2) HD columns). A column is the sum of its K-slices in slice order; q
     // and k columns are rotated with their partner column (which the thread adds up as well), q is scaled and
     // split into f16 hi and lo. Everything lands in LDS, in element order.
-    auto column = [&](int col) {
-        float v = 0.0f;
-        if (a.from.n > 0) {
-            for (int k = 0; k < a.from.n; ++k) v += a.from.data[(size_t)k * a.from.stride + (size_t)t * ROW + col];
-        } else {
-            v = a.qkv[(size_t)t * ROW + col];
-        }
-        return v;
-    };
+    // The order of the memory requests matters, because a wave's loads return in the order they were issued: first
+    // the columns (every slice of a column and of its partner at once - one after the other they cost eight trips to
+    // the L2), then the wave's first K page, and only then the arithmetic on the columns, so that the page's trip to
+    // HBM runs under the rotation, the LDS exchange and the barrier.
+    constexpr int TURNS = (10 * HD + NT - 1) / NT;          // G <= 8
+    const int n_cols = (a.G + 2) * HD;
+    const bool fast = a.from.n >= 1 && a.from.n <= 4;
+    float xs[TURNS][4], ys[TURNS][4], cvs[TURNS], svs[TURNS];
     const float * cs = a.rope_cos + (size_t)t * (HD / 2), * sn = a.rope_sin + (size_t)t * (HD / 2);
-    for (int idx = threadIdx.x; idx < (a.G + 2) * HD; idx += NT) {
-        const int hh = idx / HD, d = idx % HD;          // hh < G: query head, G: k, G + 1: v
+    auto place = [&](int idx, int & col, int & partner, int & hh, int & d) {
+        hh = idx / HD; d = idx % HD;          // hh < G: query head, G: k, G + 1: v
         const int col0 = hh < a.G ? (h * a.G + hh) * HD : (hh == a.G ? QD + h * HD : QD + KD + h * HD);
-        float x = column(col0 + d);
-        if (hh <= a.G) {
-            // partner of the rotation pair and this element's place in it
-            const int pd = a.neox ? (d < HD / 2 ? d + HD / 2 : d - HD / 2) : (d ^ 1);
-            const bool first = a.neox ? d < HD / 2 : (d & 1) == 0;
-            const int i = a.neox ? (d < HD / 2 ? d : d - HD / 2) : (d >> 1);
-            const float y = column(col0 + pd);
-            const float cv = cs[i], sv = sn[i];
-            x = first ? x * cv - y * sv : y * sv + x * cv;
+        // partner of the rotation pair (v columns have none: the column itself)
+        const int pd = hh > a.G ? d : (a.neox ? (d < HD / 2 ? d + HD / 2 : d - HD / 2) : (d ^ 1));
+        col = col0 + d; partner = col0 + pd;
+    };
+#pragma unroll
+    for (int u = 0; u < TURNS; ++u) {
+        const int idx = min((int)threadIdx.x + u * NT, n_cols - 1);
+        int col, partner, hh, d;
+        place(idx, col, partner, hh, d);
+        const int i = a.neox ? (d < HD / 2 ? d : d - HD / 2) : (d >> 1);
+        cvs[u] = cs[i];
+        svs[u] = sn[i];
+        if (fast) {
+            const float * base = a.from.data + (size_t)t * ROW;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const size_t at = (size_t)min(k, a.from.n - 1) * a.from.stride;
+                xs[u][k] = base[at + col];
+                ys[u][k] = base[at + partner];
+            }
         }
+    }
+    asm volatile("" : : : "memory");
+    struct KSet { h8 r[2 * KS]; };
+    struct VSet { h8 r[DT]; };
+    auto load_k = [&](int idx, KSet & ks) {
+        const int pid = __builtin_amdgcn_readlane(my_pid, idx);
+        const __half * kp = a.k_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
+#pragma unroll
+        for (int j = 0; j < KS; ++j) {
+            ks.r[2 * j] = load_h8(kp + ((j * 2 + 0) * 64 + lane) * 8);
+            ks.r[2 * j + 1] = load_h8(kp + ((j * 2 + 1) * 64 + lane) * 8);
+        }
+    };
+    KSet kA;
+    // (the new position's own cell in its page is not stored yet: the owner wave replaces it in registers below)
+    if (my_n > 0) load_k(0, kA);
+    asm volatile("" : : : "memory");
+    auto column_pair = [&](int col, int partner, float & x, float & y) {
+        x = 0.0f; y = 0.0f;
+        if (a.from.n > 0) {
+            const float * base = a.from.data + (size_t)t * ROW;
+            for (int k = 0; k < a.from.n; ++k) {
+                x += base[(size_t)k * a.from.stride + col];
+                y += base[(size_t)k * a.from.stride + partner];
+            }
+        } else {
+            x = a.qkv[(size_t)t * ROW + col];
+            y = a.qkv[(size_t)t * ROW + partner];
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < TURNS; ++u) {
+        const int idx = threadIdx.x + u * NT;
+        if (idx >= n_cols) break;
+        int col, partner, hh, d;
+        place(idx, col, partner, hh, d);
+        const bool first = a.neox ? d < HD / 2 : (d & 1) == 0;
+        const float cv = cvs[u], sv = svs[u];
+        float x = 0.0f, y = 0.0f;
+        if (fast) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                x += k < a.from.n ? xs[u][k] : 0.0f;
+                y += k < a.from.n ? ys[u][k] : 0.0f;
+            }
+        } else {
+            column_pair(col, partner, x, y);
+        }
+        if (hh <= a.G) x = first ? x * cv - y * sv : y * sv + x * cv;
         if (hh < a.G) {
             const float sc = fminf(fmaxf(x * a.qscale, -65504.0f), 65504.0f);
             const _Float16 hi = (_Float16)sc;
@@ -2367,17 +2426,6 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
 #pragma unroll
     for (int d = 0; d < DT; ++d) o[d] = (f4){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.0f;
-    struct KSet { h8 r[2 * KS]; };
-    struct VSet { h8 r[DT]; };
-    auto load_k = [&](int idx, KSet & ks) {
-        const int pid = __builtin_amdgcn_readlane(my_pid, idx);
-        const __half * kp = a.k_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
-#pragma unroll
-        for (int j = 0; j < KS; ++j) {
-            ks.r[2 * j] = load_h8(kp + ((j * 2 + 0) * 64 + lane) * 8);
-            ks.r[2 * j + 1] = load_h8(kp + ((j * 2 + 1) * 64 + lane) * 8);
-        }
-    };
     auto load_v = [&](int idx, VSet & vs) {
         const int pid = __builtin_amdgcn_readlane(my_pid, idx);
         const __half * vp = a.v_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
@@ -2466,9 +2514,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
     // V of a page loads while its scores are computed, K of the next page (never skipped: past the end the last
     // page again, so that the number of loads in flight is the same on every path) while the page is multiplied
     if (my_n > 0) {
-        KSet kA, kB;
+        KSet kB;
         VSet v;
-        load_k(0, kA);
         for (int i = 0; i < my_n; i += 2) {
             load_v(i, v);
             load_k(min(i + 1, my_n - 1), kB);

@@ -37,6 +37,28 @@ from pathlib import Path
 import numpy as np
 
 
+def step_algorithmic_bytes(shape, synth, gw, n_seq: int, mean_context: float) -> dict:
+    """HBM bytes one decode step has to move: every dense matrix once at its stored type, the experts the step's rows
+    touch (their expected number under uniform routing), and K and V of every attended cell (f16)."""
+    kv = shape.n_layer * 2 * shape.n_head_kv * shape.head_dim * 2 * mean_context * n_seq
+    if shape.n_expert == 0:
+        return {"weights": synth.streamed_weight_bytes(shape), "experts": 0, "kv": round(kv)}
+    dense = 0
+    for name, n_in, n_out, t in synth.matrix_types(shape):
+        if ".ffn_" in name:
+            continue
+        el, by = gw.BLOCK_GEOMETRY[synth.storage_type(t, n_in)]
+        dense += n_in // el * by * n_out
+    dense += shape.n_layer * shape.n_embd * shape.n_expert * 4          # the F32 routers
+    touched = shape.n_expert * (1.0 - (1.0 - shape.n_expert_used / shape.n_expert) ** n_seq)
+    el, by = gw.BLOCK_GEOMETRY[shape.expert_type]
+    gate_up = 2 * shape.n_embd // el * by * shape.n_ff_exp
+    el, by = gw.BLOCK_GEOMETRY[shape.expert_down_type if shape.expert_down_type >= 0 else shape.expert_type]
+    down = shape.n_ff_exp // el * by * shape.n_embd
+    return {"weights": dense, "experts": round(shape.n_layer * touched * (gate_up + down)), "kv": round(kv),
+            "experts_touched_per_layer": round(touched, 2)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("config", choices=["c4", "c5", "c5-q4km", "mxfp4-scaled"])
@@ -134,11 +156,15 @@ def main() -> int:
     timed = step_s[2:plain] if plain > 4 else step_s[:plain]
     ms = 1e3 * float(np.mean(timed))
     n_prof = args.new - plain
+    # the timed steps are the first `plain` ones: their mean context
+    by = step_algorithmic_bytes(shape, synth, gw, n_seq, float(np.mean(lengths)) + (2 + plain) / 2)
+    total_bytes = by["weights"] + by["experts"] + by["kv"]
     line = {
         "config": args.config, "model": shape.name, "sequences": n_seq,
         "prompt_tokens": int(sum(lengths)), "mean_context_during_decode": float(np.mean(lengths)) + args.new / 2,
         "prefill_tok_s": round(sum(lengths) / prefill_s, 1),
         "decode_ms_per_step": round(ms, 3), "decode_tok_s": round(n_seq / ms * 1e3, 1), "decode_steps_timed": len(timed),
+        "algorithmic_bytes_per_step": by, "step_frac_of_hbm_roofline": round(total_bytes / 8e12 / (ms * 1e-3), 4),
         "adapters": len(adapters), "rows_routed_to_an_adapter": sum(1 for r in route if r > 0),
         "kernel_ms_per_step": {k: round(t / n_prof, 4) for k, (t, n) in sorted(prof.items(), key=lambda kv: -kv[1][0]) if n},
         "kernel_launches_per_step": {k: n // n_prof for k, (t, n) in prof.items() if n},

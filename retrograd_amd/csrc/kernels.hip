@@ -2596,7 +2596,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
 bool attention_decode_can(const AttnShape & sh, bool q_or_k_norm, int max_positions) {
     const int G = sh.n_head_kv > 0 ? sh.n_head / sh.n_head_kv : 0;
     return sh.kv_quant == KV_F16 && !q_or_k_norm && (sh.head_dim == 128 || sh.head_dim == 64) && sh.rope_dim == sh.head_dim
-        && G >= 1 && G <= 8 && sh.n_head % sh.n_head_kv == 0 && max_positions <= 4 * 64 * PAGE;       // a wave holds one page id per lane, and a workgroup may have four waves
+        && G >= 1 && G <= 8 && sh.n_head % sh.n_head_kv == 0 && max_positions <= 8 * 64 * PAGE;       // a wave holds one page id per lane, a workgroup has eight waves
 }
 
 void attention_decode(hipStream_t s, const float * qkv, const Slices & from, int n_rows, const AttnShape & sh,
@@ -2619,14 +2619,9 @@ void attention_decode(hipStream_t s, const float * qkv, const Slices & from, int
     a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.G = sh.n_head / sh.n_head_kv; a.neox = sh.rope_neox ? 1 : 0;
     a.qscale = 1.4426950408889634f / sqrtf((float)sh.head_dim);
     const dim3 grid(n_rows * sh.n_head_kv);
-    static const int nw = [] { const char * v = std::getenv("RETRO_DECODE_ATTENTION_WAVES"); return v && std::atoi(v) == 4 ? 4 : 8; }();
-    if (nw == 8) {
-        if (sh.head_dim == 128) hipLaunchKernelGGL((k_attention_decode<128, 8>), grid, dim3(512), 0, s, a);
-        else hipLaunchKernelGGL((k_attention_decode<64, 8>), grid, dim3(512), 0, s, a);
-    } else {
-        if (sh.head_dim == 128) hipLaunchKernelGGL((k_attention_decode<128, 4>), grid, dim3(256), 0, s, a);
-        else hipLaunchKernelGGL((k_attention_decode<64, 4>), grid, dim3(256), 0, s, a);
-    }
+    // eight waves per workgroup, one workgroup per CU (four waves and two workgroups per CU measured slower)
+    if (sh.head_dim == 128) hipLaunchKernelGGL((k_attention_decode<128, 8>), grid, dim3(512), 0, s, a);
+    else hipLaunchKernelGGL((k_attention_decode<64, 8>), grid, dim3(512), 0, s, a);
     check_launch("attention_decode");
 }
 

@@ -480,18 +480,22 @@ class Engine:
             v["struct_size"] = C.sizeof(CStepRowV2)
             v["tokens"] = flat.ctypes.data + 4 * (np.cumsum(lens_a) - lens_a)
             v["n"] = lens_a
-            v["request"] = requests
-            v["slot"] = [r.slot for r in rows]
+            # integer fields wrap to their C width as a ctypes field assignment does
+            i32 = lambda values: np.array(values, dtype=np.int64).astype(np.int32)
+            u32 = lambda values: np.array(values, dtype=np.int64).astype(np.uint32)
+            v["request"] = i32(requests)
+            v["slot"] = i32([r.slot for r in rows])
             v["pos0"] = pos0
             v["sample"] = sample
-            v["n_top_logprobs"] = [r.n_top_logprobs for r in rows]
+            v["n_top_logprobs"] = u32([r.n_top_logprobs for r in rows])
             v["want_logprob"] = [1 if r.want_logprob else 0 for r in rows]
-            v["adapter"] = [r.adapter.value for r in rows]
+            v["adapter"] = i32([r.adapter.value for r in rows])
             v["s.struct_size"] = C.sizeof(CSamplingParamsV2)
             one = sp[0] if all(s is sp[0] for s in sp) else None        # rows that share one parameter object
-            for name in ("temperature", "top_p", "max_new_tokens", "top_k", "min_p", "repeat_penalty",
-                         "frequency_penalty", "presence_penalty", "penalty_window"):
+            for name in ("temperature", "top_p", "min_p", "repeat_penalty", "frequency_penalty", "presence_penalty"):
                 v["s." + name] = getattr(one, name) if one is not None else [getattr(s, name) for s in sp]
+            for name, conv in (("max_new_tokens", u32), ("top_k", i32), ("penalty_window", u32)):
+                v["s." + name] = conv([getattr(one, name)])[0] if one is not None else conv([getattr(s, name) for s in sp])
             v["s.seed"] = one.seed & 0xFFFFFFFF if one is not None else [s.seed & 0xFFFFFFFF for s in sp]
             v["s.n_logit_bias"] = 0
             v["s.logit_bias_ids"] = 0

@@ -106,6 +106,20 @@ def test_rows_left_from_a_larger_step_do_not_leak_into_a_smaller_one():
     assert [g == _expect(r) for g, r in zip(rec.rows, plain)] == [True] * 3
 
 
+def test_integers_wider_than_their_field_wrap_as_a_ctypes_assignment_does():
+    eng, rec = _engine()
+    out = E.StepOutput()
+    rows = [E.StepRow((1 << 40) + i, i, [1], 0, sample=True, sampling=E.SamplingParamsV2(max_new_tokens=(1 << 32) + 7, top_k=-1))
+            for i in range(3)]
+    eng.step(rows, out)
+    assert [g["request"] for g in rec.rows] == [0, 1, 2]
+    assert [g["max_new_tokens"] for g in rec.rows] == [7, 7, 7]
+    assert [g["top_k"] for g in rec.rows] == [-1, -1, -1]
+    shared = E.SamplingParamsV2(max_new_tokens=(1 << 32) + 9)
+    eng.step([E.StepRow((1 << 40) + i, i, [1], 0, sample=True, sampling=shared) for i in range(3)], out)
+    assert [g["max_new_tokens"] for g in rec.rows] == [9, 9, 9]
+
+
 def test_caller_side_errors_come_in_row_order():
     eng, _ = _engine()
     out = E.StepOutput()

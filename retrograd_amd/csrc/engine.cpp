@@ -1418,12 +1418,13 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         // every row decodes one token over an f16 cache in the exact arithmetic: rotation, KV store, attention and
         // split merge are one launch (the output projection's plain activation planes are all it writes)
         const bool fused_decode = one_token_rows && fused_decode_attention_ && !faithful
-                                  && rk::attention_decode_can(sh, L.q_norm.ptr != nullptr || L.k_norm.ptr != nullptr, step_max_resident_);
+                                  && rk::attention_decode_can(sh, step_max_resident_);
         size_t pt_;
         if (fused_decode) {
             pt_ = prof_begin(PC_ATTN);
             rk::attention_decode(stream_, qkv, qkv_slices, T, sh, pk_, table_.as<int32_t>(), max_pages_,
-                                 k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), act_q);
+                                 k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), L.q_norm.as<float>(),
+                                 L.k_norm.as<float>(), act_q);
             prof_end(PC_ATTN, pt_);
             pt_ = prof_begin(PC_OPROJ);
             pending = rk::matmul_deferred(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);

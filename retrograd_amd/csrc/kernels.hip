@@ -2241,6 +2241,8 @@ struct DecodeAttnArgs {
     Act out;                                // the output projection's activations (hi/lo planes and block sums)
     int n_head, n_kv, G, neox;
     float qscale;
+    const float * q_norm, * k_norm;         // per-head RMSNorm weights of the q and k rows ([head_dim]), or null
+    float eps;
 };
 
 // One workgroup of eight waves per (row, kv head) of a step in which every row decodes one token, f16 cache, at
@@ -2350,6 +2352,53 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
             y = a.qkv[(size_t)t * ROW + partner];
         }
     };
+    // the columns' sums in slice order
+    float xv[TURNS], yv[TURNS];
+#pragma unroll
+    for (int u = 0; u < TURNS; ++u) {
+        const int idx = threadIdx.x + u * NT;
+        float x = 0.0f, y = 0.0f;
+        if (fast) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                x += k < a.from.n ? xs[u][k] : 0.0f;
+                y += k < a.from.n ? ys[u][k] : 0.0f;
+            }
+        } else if (idx < n_cols) {
+            int col, partner, hh, d;
+            place(idx, col, partner, hh, d);
+            column_pair(col, partner, x, y);
+        }
+        xv[u] = x; yv[u] = y;
+    }
+    // Architectures that normalise the q and k rows per head (RMSNorm over the head's dims, before the rotation): a
+    // head's columns sit in consecutive threads of one turn - one wave for 64 dims, an even and an odd wave for 128 -
+    // so the sum of squares is a wave sum, and for 128 dims the two halves meet in LDS.
+    if (a.q_norm || a.k_norm) {
+        float * half_ss = &part[0][0][0];          // free until the waves leave their partial results there
+#pragma unroll
+        for (int u = 0; u < TURNS; ++u) {
+            const int idx = threadIdx.x + u * NT;
+            const float mine = idx < n_cols ? xv[u] * xv[u] : 0.0f;
+            const float ws = wave_sum(mine);
+            if (lane == 0) half_ss[u * NW + wave] = ws;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < TURNS; ++u) {
+            const int idx = min((int)threadIdx.x + u * NT, n_cols - 1);
+            int col, partner, hh, d;
+            place(idx, col, partner, hh, d);
+            const float * nw = hh < a.G ? a.q_norm : (hh == a.G ? a.k_norm : nullptr);
+            if (nw) {
+                const float ss = HD == 128 ? half_ss[u * NW + (wave & ~1)] + half_ss[u * NW + (wave | 1)] : half_ss[u * NW + wave];
+                const float scale = 1.0f / sqrtf(ss / (float)HD + a.eps);
+                xv[u] = (xv[u] * scale) * nw[d];
+                yv[u] = (yv[u] * scale) * nw[partner - (col - d)];
+            }
+        }
+        __syncthreads();          // half_ss is read before the partial results may overwrite it
+    }
 #pragma unroll
     for (int u = 0; u < TURNS; ++u) {
         const int idx = threadIdx.x + u * NT;
@@ -2358,16 +2407,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
         place(idx, col, partner, hh, d);
         const bool first = a.neox ? d < HD / 2 : (d & 1) == 0;
         const float cv = cvs[u], sv = svs[u];
-        float x = 0.0f, y = 0.0f;
-        if (fast) {
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                x += k < a.from.n ? xs[u][k] : 0.0f;
-                y += k < a.from.n ? ys[u][k] : 0.0f;
-            }
-        } else {
-            column_pair(col, partner, x, y);
-        }
+        float x = xv[u];
+        const float y = yv[u];
         if (hh <= a.G) x = first ? x * cv - y * sv : y * sv + x * cv;
         if (hh < a.G) {
             const float sc = fminf(fmaxf(x * a.qscale, -65504.0f), 65504.0f);
@@ -2593,17 +2634,17 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
     }
 }
 
-bool attention_decode_can(const AttnShape & sh, bool q_or_k_norm, int max_positions) {
+bool attention_decode_can(const AttnShape & sh, int max_positions) {
     const int G = sh.n_head_kv > 0 ? sh.n_head / sh.n_head_kv : 0;
-    return sh.kv_quant == KV_F16 && !q_or_k_norm && (sh.head_dim == 128 || sh.head_dim == 64) && sh.rope_dim == sh.head_dim
+    return sh.kv_quant == KV_F16 && (sh.head_dim == 128 || sh.head_dim == 64) && sh.rope_dim == sh.head_dim
         && G >= 1 && G <= 8 && sh.n_head % sh.n_head_kv == 0 && max_positions <= 8 * 64 * PAGE;       // a wave holds one page id per lane, a workgroup has eight waves
 }
 
 void attention_decode(hipStream_t s, const float * qkv, const Slices & from, int n_rows, const AttnShape & sh,
                       const PackBuffers & pk, const int32_t * table, int max_pages, __half * k_pool, __half * v_pool,
-                      const Act & out) {
+                      const float * q_norm, const float * k_norm, const Act & out) {
     if (n_rows <= 0) return;
-    if (!attention_decode_can(sh, false, 0)) throw std::runtime_error("attention_decode: unsupported shape or cache type");
+    if (!attention_decode_can(sh, 0)) throw std::runtime_error("attention_decode: unsupported shape or cache type");
     check_act_out(out, sh.n_head * sh.head_dim, "attention_decode", n_rows);
     if (!out.x) throw std::runtime_error("attention_decode: needs the plain activation planes");
     if (sh.page_stride == 0 || sh.head_stride == 0) throw std::runtime_error("attention_decode: the pool's strides are missing");
@@ -2618,6 +2659,7 @@ void attention_decode(hipStream_t s, const float * qkv, const Slices & from, int
     a.out = out;
     a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.G = sh.n_head / sh.n_head_kv; a.neox = sh.rope_neox ? 1 : 0;
     a.qscale = 1.4426950408889634f / sqrtf((float)sh.head_dim);
+    a.q_norm = q_norm; a.k_norm = k_norm; a.eps = sh.eps;
     const dim3 grid(n_rows * sh.n_head_kv);
     // eight waves per workgroup, one workgroup per CU (four waves and two workgroups per CU measured slower)
     if (sh.head_dim == 128) hipLaunchKernelGGL((k_attention_decode<128, 8>), grid, dim3(512), 0, s, a);

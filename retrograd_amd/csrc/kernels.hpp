@@ -378,11 +378,11 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
 // The three launches above in one, for a step in which every row decodes one token over an f16 cache (see
 // k_attention_decode): reads the q, k, v product (its K-slices or the buffer), stores the new K and V rows, writes the
 // output projection's activations. attention_decode_can: whether the shape allows it (head dims 64 / 128 rotated
-// over their whole width, at most eight query heads per kv head, no q / k norm, sequences of at most 16384 positions).
-bool attention_decode_can(const AttnShape & sh, bool q_or_k_norm, int max_positions);
+// over their whole width, at most eight query heads per kv head, sequences of at most 16384 positions; q_norm / k_norm: the per-head RMSNorm weights of architectures that have them, or null).
+bool attention_decode_can(const AttnShape & sh, int max_positions);
 void attention_decode(hipStream_t s, const float * qkv, const Slices & from, int n_rows, const AttnShape & sh,
                       const PackBuffers & pk, const int32_t * table, int max_pages, __half * k_pool, __half * v_pool,
-                      const Act & out);
+                      const float * q_norm, const float * k_norm, const Act & out);
 void attention_combine(hipStream_t s, const float * partial, int T, const AttnShape & sh,
                        const PackBuffers & pk, const Act & out);
 size_t attention_partial_floats(int n_items, int head_dim);

@@ -1,7 +1,8 @@
 """The one-launch attention of pure decode steps (k_attention_decode: rotation, KV store, attention and split merge)
 against the three launches it replaces (k_rope_store, k_attention, k_attention_combine; RETRO_FUSED_DECODE_ATTENTION=0)
 on the same model and requests, and against the CPU oracle: llama's adjacent-pair rotation with heads of 128 and the
-NeoX pairing with heads of 64 and q/k/v biases, sequences from one page to many (so that the eight waves of a
+NeoX pairing with heads of 64 and q/k/v biases, per-head q / k RMSNorm (qwen3moe, heads of 64 and of 128, norm weights
+away from one), sequences from one page to many (so that the eight waves of a
 workgroup hold nothing, one page or several), a sequence whose beginning was removed, and steps of one row."""
 import numpy as np
 import pytest
@@ -18,6 +19,10 @@ SHAPES = {
                                 n_ff=2048, n_vocab=2048, name="llama-q4k-hd128"),
     "qwen2-hd64": synth.scaled(synth.QWEN25_7B_Q8, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64,
                                n_ff=1024, n_vocab=1024, matrix_type=12, name="qwen2-q4k-hd64"),
+    "qwen3moe-hd64": synth.scaled(synth.QWEN3_30B_A3B, n_layer=2, n_embd=512, n_head=8, n_head_kv=2, head_dim=64, n_vocab=1024,
+                                  n_expert=16, n_expert_used=4, n_ff_exp=256, norm_std=0.2, name="qwen3moe-qknorm-hd64"),
+    "qwen3moe-hd128": synth.scaled(synth.QWEN3_30B_A3B, n_layer=2, n_embd=512, n_head=8, n_head_kv=4, head_dim=128, n_vocab=1024,
+                                   n_expert=16, n_expert_used=4, n_ff_exp=256, norm_std=0.2, name="qwen3moe-qknorm-hd128"),
 }
 
 

@@ -64,6 +64,8 @@ def parse_args():
     ap.add_argument("--kv", default="f16", choices=["f16", "q8_0", "q4_0"],
                     help="storage of the KV cache; the headline is f16 as the workload names it, q8_0 and q4_0 are secondary configurations")
     ap.add_argument("--kernel-steps", type=int, default=8, help="decode steps timed per kernel category after the timed region")
+    ap.add_argument("--attention-timeline", default="", metavar="FILE",
+                    help="after the timed region, record the workgroup timeline of one decode attention launch and write a text summary")
     ap.add_argument("--no-scheduler-leg", action="store_true", help="skip the run of the same workload through the step scheduler")
     ap.add_argument("--scheduler-requests", type=int, default=128)
     ap.add_argument("--no-ggml-leg", action="store_true", help="skip the secondary measurement under the ggml arithmetic")
@@ -266,7 +268,42 @@ def measure_decode(args, eng, E, synth, gw, shape, geometry, profile_kernels):
     if profile_kernels and args.kernel_steps > 0:
         kdec, _ = run_decode_steps(args.kernel_steps, 2)
         out["kernels"] = (eng.profile_read(reset=True), kdec, args.kernel_steps)
+    if profile_kernels and args.attention_timeline:
+        eng.attention_timeline(True)
+        run_decode_steps(3, 0)
+        stamps = eng.attention_timeline_read()
+        eng.attention_timeline(False)
+        Path(args.attention_timeline).write_text(attention_timeline_summary(stamps))
     return out, wl
+
+
+def attention_timeline_summary(stamps) -> str:
+    """Text summary of one decode attention launch from the six values its workgroups leave (clock ticks of 10 ns at
+    the start, after the prologue, when the first wave is done, when all waves are done, at the end; the row's pages)."""
+    if len(stamps) == 0:
+        return "no decode step took the one-launch attention\n"
+    st = stamps.astype(np.int64)
+    t0 = st[:, 0].min()
+    us = lambda col: (st[:, col] - t0) / 100.0
+    start, pro, first, allw, end, pages = us(0), us(1), us(2), us(3), us(4), st[:, 5]
+    lines = ["workgroups %d, pages %d (16 KiB of K and V each: %.1f MB), launch span %.1f us (first start to last end): %.2f TB/s"
+             % (len(st), pages.sum(), pages.sum() * 16384 / 1e6, end.max(), pages.sum() * 16384 / end.max() / 1e6),
+             "per workgroup, mean: prologue %.2f us, pages streamed in %.2f us (%.3f us per page; the first wave is done after "
+             "%.0f %% of that), merge and store %.2f us"
+             % ((pro - start).mean(), (allw - pro).mean(), ((allw - pro) / pages).mean(),
+                100.0 * ((first - pro) / np.maximum(allw - pro, 1e-9)).mean(), (end - allw).mean()),
+             "", "time us | workgroups resident | of them streaming pages | started so far | finished so far"]
+    for t in np.arange(0.0, end.max() + 5.0, 5.0):
+        lines.append("%7.0f | %19d | %24d | %14d | %15d" % (t, ((start <= t) & (end > t)).sum(), ((pro <= t) & (allw > t)).sum(),
+                                                              (start <= t).sum(), (end <= t).sum()))
+    lines += ["", "workgroups by pages of their row: pages | count | mean start us | mean duration us | us per page"]
+    edges = [0, 8, 16, 32, 48, 64, 96, 128, 1 << 30]
+    for lo, hi in zip(edges[:-1], edges[1:]):
+        sel = (pages > lo) & (pages <= hi)
+        if sel.any():
+            lines.append("%4d..%-4s | %5d | %13.1f | %16.1f | %.3f" % (lo + 1, hi if hi < (1 << 30) else "", sel.sum(), start[sel].mean(),
+                                                                       (end - start)[sel].mean(), ((allw - pro)[sel] / pages[sel]).mean()))
+    return "\n".join(lines) + "\n"
 
 
 def scheduler_leg(args, eng, E, shape, geometry):

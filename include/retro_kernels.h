@@ -133,6 +133,15 @@ int retro_engine_debug_profile(retro_engine * engine, int32_t level);
 int32_t retro_engine_debug_profile_categories(void);
 int retro_engine_debug_profile_read(retro_engine * engine, double * out_ms, uint64_t * out_launches, int32_t reset);
 
+/* Timeline of the decode attention launch (the one launch of a pure decode step that rotates, stores the KV cell,
+ * attends and merges; one workgroup per row and kv head). While enabled, the launch of the model's middle layer
+ * leaves six values per workgroup, in launch order of the workgroups: the GPU's constant 100 MHz clock at the
+ * workgroup's start, after the prologue's barrier, when its first wave has attended its pages, after the barrier
+ * behind all its waves, at its end, and the number of KV pages of its row. read() copies those of the last such
+ * launch ([workgroups][6]; out == NULL reports the count; 0 workgroups when no step took that launch). */
+int retro_engine_debug_attention_timeline(retro_engine * engine, int32_t enable);
+int retro_engine_debug_attention_timeline_read(retro_engine * engine, uint64_t * out, size_t cap_workgroups, size_t * out_workgroups);
+
 #ifdef __cplusplus
 }
 #endif

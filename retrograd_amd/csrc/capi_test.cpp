@@ -424,6 +424,22 @@ int retro_engine_debug_profile_read(retro_engine * engine, double * out_ms, uint
     });
 }
 
+int retro_engine_debug_attention_timeline(retro_engine * engine, int32_t enable) {
+    return guarded([&]() -> int {
+        if (!engine) { set_error("engine is required"); return -1; }
+        engine->impl.attention_timeline(enable != 0);
+        return 0;
+    });
+}
+
+int retro_engine_debug_attention_timeline_read(retro_engine * engine, uint64_t * out, size_t cap_workgroups, size_t * out_workgroups) {
+    return guarded([&]() -> int {
+        if (!engine) { set_error("engine is required"); return -1; }
+        static_assert(sizeof(uint64_t) == sizeof(unsigned long long), "clock values are 64 bits");
+        return engine->impl.attention_timeline_read((unsigned long long *)out, cap_workgroups, out_workgroups);
+    });
+}
+
 int retro_engine_debug_pages(retro_engine * engine, int32_t slot, int32_t * out, size_t cap, size_t * out_n) {
     return guarded([&]() -> int {
         if (!engine) { set_error("engine is required"); return -1; }

@@ -438,6 +438,8 @@ void Engine::build_buffers() {
     pk_.tile_nsplit = i32((size_t)B); pk_.tile_page0 = i32((size_t)B); pk_.tile_kv_begin = i32((size_t)B);
     pk_.tok_tile = i32((size_t)B);
     pk_.dec_order = i32((size_t)B);
+    pk_.dec_desc = (int4 *)i32((size_t)B * 4);
+    pk_.dec_pid = i32((size_t)B * 8);
     pk_.tok_merge = (int4 *)i32((size_t)B * 4);
     pk_.rope_cos = (float *)i32((size_t)B * (hp_.rope_dim / 2));
     pk_.rope_sin = (float *)i32((size_t)B * (hp_.rope_dim / 2));
@@ -1421,10 +1423,16 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
                                   && rk::attention_decode_can(sh, step_max_resident_);
         size_t pt_;
         if (fused_decode) {
+            unsigned long long * stamps = nullptr;
+            if (attn_timeline_ && l == h.n_layer / 2) {
+                attn_stamped_wgs_ = (size_t)T * (size_t)h.n_head_kv;
+                attn_stamps_.ensure(attn_stamped_wgs_ * 6 * sizeof(unsigned long long));
+                stamps = attn_stamps_.as<unsigned long long>();
+            }
             pt_ = prof_begin(PC_ATTN);
             rk::attention_decode(stream_, qkv, qkv_slices, T, sh, pk_, table_.as<int32_t>(), max_pages_,
                                  k_pool_[(size_t)l].as<__half>(), v_pool_[(size_t)l].as<__half>(), L.q_norm.as<float>(),
-                                 L.k_norm.as<float>(), act_q);
+                                 L.k_norm.as<float>(), act_q, stamps);
             prof_end(PC_ATTN, pt_);
             pt_ = prof_begin(PC_OPROJ);
             pending = rk::matmul_deferred(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
@@ -1977,6 +1985,20 @@ int Engine::debug_pack(int32_t * tok, int32_t * pos, int32_t * seq, int32_t * ce
     };
     get(tok, pk_.tok, T); get(pos, pk_.pos, T); get(seq, pk_.seq, T); get(cell, pk_.cell, T); get(out_index, pk_.out_index, T);
     get(last_index, pk_.last_index, std::min(cap_rows, (size_t)cfg_.n_batch));
+    return 0;
+}
+
+void Engine::attention_timeline(bool on) {
+    attn_timeline_ = on;
+    if (!on) attn_stamped_wgs_ = 0;
+}
+
+int Engine::attention_timeline_read(unsigned long long * out, size_t cap_workgroups, size_t * n_workgroups) {
+    hip_check(hipStreamSynchronize(stream_), "attention_timeline_read");
+    if (n_workgroups) *n_workgroups = attn_stamped_wgs_;
+    if (!out || attn_stamped_wgs_ == 0) return 0;
+    if (cap_workgroups < attn_stamped_wgs_) { set_error("attention timeline: the buffer is too small"); return -2; }
+    hip_check(hipMemcpy(out, attn_stamps_.ptr, attn_stamped_wgs_ * 6 * sizeof(unsigned long long), hipMemcpyDeviceToHost), "hipMemcpy");
     return 0;
 }
 

@@ -210,6 +210,10 @@ public:
 
     // Event timing of kernel categories: level 0 off, 1 attention only, 2 all.
     void profile_level(int level) { prof_level_ = level; }
+    // The decode attention launch of the middle layer leaves six clock values per workgroup while this is on;
+    // read returns those of the last such launch ([workgroup][6]) and the number of workgroups.
+    void attention_timeline(bool on);
+    int attention_timeline_read(unsigned long long * out, size_t cap_workgroups, size_t * n_workgroups);
     void profile_read(double * ms, uint64_t * launches, bool reset);
 
     // Test hooks: copies of device state.
@@ -322,6 +326,9 @@ private:
     // event timing
     struct ProfSpan { int cat; size_t a, b; };
     int prof_level_ = 0;
+    DevBuf attn_stamps_;
+    bool attn_timeline_ = false;
+    size_t attn_stamped_wgs_ = 0;
     std::vector<hipEvent_t> prof_events_;
     size_t prof_used_ = 0;
     std::vector<ProfSpan> prof_spans_;

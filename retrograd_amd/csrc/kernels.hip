@@ -1377,6 +1377,18 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
     }
     // the rows by resident length, longest first (ties in row order): the decode-step attention starts one
     // workgroup per row and kv head in this order, so that the launch's tail is made of short sequences
+    // Beside the order, per row in that order: what a workgroup of that launch needs to start (token index, position,
+    // first resident position, slot) and, with the row's pages dealt evenly to eight waves, the id of each wave's
+    // first page - so that the workgroup's first loads depend on one lookup, not on a chain of three.
+    auto describe = [&](int rank, const RowDesc & d) {
+        o.dec_order[rank] = d.tok_off;
+        const int pos = d.pos0 + d.n - 1;
+        o.dec_desc[rank] = make_int4(d.tok_off + d.n - 1, pos, d.kv_begin, d.slot);
+        const int page_first = d.kv_begin / PAGE, n_pages = pos / PAGE - page_first + 1;
+        const int per_wave = (n_pages + 7) / 8;
+        for (int w = 0; w < 8; ++w)
+            o.dec_pid[rank * 8 + w] = w * per_wave < n_pages ? table[(size_t)d.slot * max_pages + page_first + w * per_wave] : 0;
+    };
     if (n_rows <= 1024) {
         if ((int)threadIdx.x < n_rows) { const RowDesc d = rows[threadIdx.x]; row_len[threadIdx.x] = d.pos0 + d.n - d.kv_begin; }
         __syncthreads();
@@ -1384,10 +1396,10 @@ __global__ __launch_bounds__(1024) void k_pack(const RowDesc * __restrict__ rows
             const int mine = row_len[threadIdx.x];
             int rank = 0;
             for (int j = 0; j < n_rows; ++j) rank += (row_len[j] > mine || (row_len[j] == mine && j < (int)threadIdx.x)) ? 1 : 0;
-            o.dec_order[rank] = rows[threadIdx.x].tok_off;
+            describe(rank, rows[threadIdx.x]);
         }
     } else {
-        for (int r = threadIdx.x; r < n_rows; r += 1024) o.dec_order[r] = rows[r].tok_off;
+        for (int r = threadIdx.x; r < n_rows; r += 1024) describe(r, rows[r]);
     }
     if (threadIdx.x == 0) {
         const RowDesc last = rows[n_rows - 1];
@@ -2232,8 +2244,8 @@ struct DecodeAttnArgs {
     const float * qkv;                      // [T][QD + 2 KD] f32 (with the biases), when there are no slices
     Slices from;                            // or the K-slices of the fused q, k, v product, added in slice order
     const float * rope_cos, * rope_sin;     // [T][head_dim / 2]
-    const int32_t * pos, * seq, * kv_begin; // per row (= token) of the step
-    const int32_t * order;                  // rows, longest sequence first
+    const int4 * desc;                      // per row, longest sequence first: {token index, position, first resident position, slot}
+    const int32_t * first_pid;              // [row in that order][8]: the id of each wave's first page
     const int32_t * table;
     int max_pages;
     __half * k_pool, * v_pool;
@@ -2243,6 +2255,9 @@ struct DecodeAttnArgs {
     float qscale;
     const float * q_norm, * k_norm;         // per-head RMSNorm weights of the q and k rows ([head_dim]), or null
     float eps;
+    unsigned long long * stamps;            // null, or [workgroup][6]: the constant 100 MHz clock at the workgroup's start,
+                                            // after the prologue's barrier, when its first wave has attended its pages, after
+                                            // the barrier behind all waves, at the end; the row's pages
 };
 
 // One workgroup of eight waves per (row, kv head) of a step in which every row decodes one token, f16 cache, at
@@ -2260,6 +2275,8 @@ struct DecodeAttnArgs {
 //     k_attention_combine's arithmetic, and store the output projection's activations.
 template <int HD, int NW>
 __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttnArgs a) {
+    unsigned long long * stamp = a.stamps && threadIdx.x == 0 ? a.stamps + (size_t)blockIdx.x * 6 : nullptr;
+    if (stamp) stamp[0] = wall_clock64();
     constexpr int KS = HD / 32;     // k-steps of QK^T
     constexpr int DT = HD / 16;     // dim tiles of PV
     constexpr int PS = HD + 2;      // floats of one partial result: max, sum, output
@@ -2269,8 +2286,11 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c = lane & 15, g = lane >> 4;
-    const int t = a.order[blockIdx.x / a.n_kv], h = blockIdx.x % a.n_kv;
-    const int pos = a.pos[t], kv_begin = a.kv_begin[t], slot = a.seq[t];
+    static_assert(NW == 8, "k_pack deals a row's pages to eight waves");
+    const int4 dd = a.desc[blockIdx.x / a.n_kv];
+    const int t = dd.x, h = blockIdx.x % a.n_kv;
+    const int pos = dd.y, kv_begin = dd.z, slot = dd.w;
+    const int pid0 = a.first_pid[(blockIdx.x / a.n_kv) * 8 + wave];
     const int cc = c & 7;
     const bool col_ok = cc < a.G;
     const bool lo_col = c >= 8;
@@ -2326,8 +2346,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
     asm volatile("" : : : "memory");
     struct KSet { h8 r[2 * KS]; };
     struct VSet { h8 r[DT]; };
-    auto load_k = [&](int idx, KSet & ks) {
-        const int pid = __builtin_amdgcn_readlane(my_pid, idx);
+    auto load_k_page = [&](int pid, KSet & ks) {
         const __half * kp = a.k_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
 #pragma unroll
         for (int j = 0; j < KS; ++j) {
@@ -2335,10 +2354,22 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
             ks.r[2 * j + 1] = load_h8(kp + ((j * 2 + 1) * 64 + lane) * 8);
         }
     };
+    auto load_k = [&](int idx, KSet & ks) { load_k_page(__builtin_amdgcn_readlane(my_pid, idx), ks); };
     KSet kA;
-    // (the new position's own cell in its page is not stored yet: the owner wave replaces it in registers below)
-    if (my_n > 0) load_k(0, kA);
+    // The wave's first page by the id k_pack left, so that the request does not wait for the table lookup above.
+    // (The new position's own cell in its page is not stored yet: the owner wave replaces it in registers below.)
+    // A wave without pages requests page 0 and never looks at it: with a branch around the request the waits
+    // below could not tell the two paths apart and would wait for everything.
+    load_k_page(pid0, kA);
     asm volatile("" : : : "memory");
+    // The column values are first looked at here: left alone, the compiler adds a turn's first slices right behind
+    // their loads (to reuse the registers) and so waits a trip to memory per turn before it requests the next.
+    if (fast) {
+#pragma unroll
+        for (int u = 0; u < TURNS; ++u)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) asm volatile("" : "+v"(xs[u][k]), "+v"(ys[u][k]));
+    }
     auto column_pair = [&](int col, int partner, float & x, float & y) {
         x = 0.0f; y = 0.0f;
         if (a.from.n > 0) {
@@ -2421,6 +2452,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
         }
     }
     __syncthreads();
+    if (stamp) stamp[1] = wall_clock64();
 
     h8 qreg[KS];
 #pragma unroll
@@ -2567,6 +2599,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
             attend(my_first + i + 1, kB, v, owner && i + 1 == my_n - 1);
         }
     }
+    if (stamp) stamp[2] = wall_clock64();
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
 #pragma unroll
@@ -2582,6 +2615,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
             for (int i = 0; i < 4; ++i) dst[2 + d * 16 + 4 * g + i] = o[d][i];
     }
     __syncthreads();
+    if (stamp) { stamp[3] = wall_clock64(); stamp[5] = (unsigned long long)n_pages; }
     // wave gi merges the eight partial results of query head h G + gi (a wave without pages left max = -inf, sum = 0)
     for (int gi = wave; gi < a.G; gi += NW) {
     const int e0 = 2 * lane;
@@ -2632,6 +2666,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
         }
     }
     }
+    if (stamp) stamp[4] = wall_clock64();
 }
 
 bool attention_decode_can(const AttnShape & sh, int max_positions) {
@@ -2642,7 +2677,7 @@ bool attention_decode_can(const AttnShape & sh, int max_positions) {
 
 void attention_decode(hipStream_t s, const float * qkv, const Slices & from, int n_rows, const AttnShape & sh,
                       const PackBuffers & pk, const int32_t * table, int max_pages, __half * k_pool, __half * v_pool,
-                      const float * q_norm, const float * k_norm, const Act & out) {
+                      const float * q_norm, const float * k_norm, const Act & out, unsigned long long * stamps) {
     if (n_rows <= 0) return;
     if (!attention_decode_can(sh, 0)) throw std::runtime_error("attention_decode: unsupported shape or cache type");
     check_act_out(out, sh.n_head * sh.head_dim, "attention_decode", n_rows);
@@ -2650,16 +2685,17 @@ void attention_decode(hipStream_t s, const float * qkv, const Slices & from, int
     if (sh.page_stride == 0 || sh.head_stride == 0) throw std::runtime_error("attention_decode: the pool's strides are missing");
     const int ROW = (sh.n_head + 2 * sh.n_head_kv) * sh.head_dim;
     if (from.n > 0 && from.N != ROW) throw std::runtime_error("attention_decode: the slices are not a fused q, k, v product");
-    if (!pk.dec_order) throw std::runtime_error("attention_decode: the step's rows were not ordered");
+    if (!pk.dec_desc || !pk.dec_pid) throw std::runtime_error("attention_decode: the step's rows were not described");
     DecodeAttnArgs a;
     a.qkv = qkv; a.from = from; a.rope_cos = pk.rope_cos; a.rope_sin = pk.rope_sin;
-    a.pos = pk.pos; a.seq = pk.seq; a.kv_begin = pk.tile_kv_begin; a.order = pk.dec_order;
+    a.desc = pk.dec_desc; a.first_pid = pk.dec_pid;
     a.table = table; a.max_pages = max_pages; a.k_pool = k_pool; a.v_pool = v_pool;
     a.page_stride = sh.page_stride; a.head_stride = sh.head_stride;
     a.out = out;
     a.n_head = sh.n_head; a.n_kv = sh.n_head_kv; a.G = sh.n_head / sh.n_head_kv; a.neox = sh.rope_neox ? 1 : 0;
     a.qscale = 1.4426950408889634f / sqrtf((float)sh.head_dim);
     a.q_norm = q_norm; a.k_norm = k_norm; a.eps = sh.eps;
+    a.stamps = stamps;
     const dim3 grid(n_rows * sh.n_head_kv);
     // eight waves per workgroup, one workgroup per CU (four waves and two workgroups per CU measured slower)
     if (sh.head_dim == 128) hipLaunchKernelGGL((k_attention_decode<128, 8>), grid, dim3(512), 0, s, a);

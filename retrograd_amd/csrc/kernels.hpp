@@ -300,6 +300,8 @@ struct PackBuffers {       // device arrays, sized for n_batch tokens / rows
     int4 * item_b;         // [n_items] position of the first token, first resident position of the slot,
                            //           first page index of this split, pages in this split
     int32_t * dec_order;   // [n_rows] rows by resident length, longest first (the order the decode-step attention starts its workgroups in)
+    int4 * dec_desc;       // [n_rows] in that order: {the row's token index, its position, the first resident position, the slot}
+    int32_t * dec_pid;     // [n_rows][8] in that order: with the row's pages dealt evenly to eight waves, the id of each wave's first page
     float * rope_cos;      // [T][rope_dim/2]
     float * rope_sin;
     int split_pages = MAX_SPLIT_PAGES;   // pages per attention work item in this step (set from count_attention_work)
@@ -378,11 +380,12 @@ void attention(hipStream_t s, const __half * q, const __half * q_lo, const AttnS
 // The three launches above in one, for a step in which every row decodes one token over an f16 cache (see
 // k_attention_decode): reads the q, k, v product (its K-slices or the buffer), stores the new K and V rows, writes the
 // output projection's activations. attention_decode_can: whether the shape allows it (head dims 64 / 128 rotated
-// over their whole width, at most eight query heads per kv head, sequences of at most 16384 positions; q_norm / k_norm: the per-head RMSNorm weights of architectures that have them, or null).
+// over their whole width, at most eight query heads per kv head, sequences of at most 16384 positions; q_norm / k_norm: the per-head RMSNorm weights of architectures that have them, or null; stamps: null, or six
+// clock values per workgroup (n_rows * n_head_kv of them) for a timeline of the launch).
 bool attention_decode_can(const AttnShape & sh, int max_positions);
 void attention_decode(hipStream_t s, const float * qkv, const Slices & from, int n_rows, const AttnShape & sh,
                       const PackBuffers & pk, const int32_t * table, int max_pages, __half * k_pool, __half * v_pool,
-                      const float * q_norm, const float * k_norm, const Act & out);
+                      const float * q_norm, const float * k_norm, const Act & out, unsigned long long * stamps = nullptr);
 void attention_combine(hipStream_t s, const float * partial, int T, const AttnShape & sh,
                        const PackBuffers & pk, const Act & out);
 size_t attention_partial_floats(int n_items, int head_dim);

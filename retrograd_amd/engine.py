@@ -164,6 +164,7 @@ KERNEL_SYMBOLS = [
     "retro_kernel_matmul", "retro_kernel_gemv_fused", "retro_kernel_matmul_time", "retro_kernel_mxfp4_scaled", "retro_kernel_mxfp4_scaled_time", "retro_kernel_stream_time", "retro_kernel_sample_prepare", "retro_kernel_sample_greedy_noalloc", "retro_kernel_sample_greedy_noalloc_max_rows", "retro_kernel_page_size", "retro_kernel_max_topk",
     "retro_engine_debug_logits", "retro_engine_debug_kv", "retro_engine_debug_pack", "retro_engine_debug_pages",
     "retro_engine_debug_profile", "retro_engine_debug_profile_categories", "retro_engine_debug_profile_read",
+    "retro_engine_debug_attention_timeline", "retro_engine_debug_attention_timeline_read",
 ]
 PROFILE_CATEGORIES = ["pack", "embed", "norm", "qkv", "rope", "attention", "combine", "o_proj", "gate_up", "swiglu",
                       "down", "head", "sample"]
@@ -261,6 +262,8 @@ def load_library() -> C.CDLL:
                                             C.c_size_t, _i32p]
     lib.retro_engine_debug_pages.argtypes = [C.c_void_p, C.c_int32, _i32p, C.c_size_t, C.POINTER(C.c_size_t)]
     lib.retro_engine_debug_profile.argtypes = [C.c_void_p, C.c_int32]
+    lib.retro_engine_debug_attention_timeline.argtypes = [C.c_void_p, C.c_int32]
+    lib.retro_engine_debug_attention_timeline_read.argtypes = [C.c_void_p, C.POINTER(C.c_uint64), C.c_size_t, C.POINTER(C.c_size_t)]
     lib.retro_engine_debug_profile_categories.restype = C.c_int32
     lib.retro_engine_debug_profile_read.argtypes = [C.c_void_p, C.POINTER(C.c_double), C.POINTER(C.c_uint64), C.c_int32]
     _lib = lib
@@ -904,6 +907,26 @@ class Engine:
         s = self._lib.retro_engine_debug_profile(self._h, level)
         if s != 0:
             _raise(s)
+
+    def attention_timeline(self, on: bool) -> None:
+        """While on, the decode attention launch of the middle layer records six clock values per workgroup."""
+        s = self._lib.retro_engine_debug_attention_timeline(self._h, 1 if on else 0)
+        if s != 0:
+            _raise(s)
+
+    def attention_timeline_read(self) -> np.ndarray:
+        """[workgroups][6] of the last recorded launch: start, after the prologue, first wave done, all waves done,
+        end (ticks of the 100 MHz clock) and the row's KV pages; empty when no step took that launch."""
+        n = C.c_size_t()
+        s = self._lib.retro_engine_debug_attention_timeline_read(self._h, None, 0, C.byref(n))
+        if s != 0:
+            _raise(s)
+        out = np.zeros((n.value, 6), np.uint64)
+        if n.value:
+            s = self._lib.retro_engine_debug_attention_timeline_read(self._h, out.ctypes.data_as(C.POINTER(C.c_uint64)), n.value, C.byref(n))
+            if s != 0:
+                _raise(s)
+        return out
 
     def profile_read(self, reset: bool = True) -> dict:
         n = self._lib.retro_engine_debug_profile_categories()

@@ -82,3 +82,32 @@ def test_one_launch_equals_three_and_the_oracle(key, tmp_path, monkeypatch):
             pos[i] += 1
     one.close()
     three.close()
+
+
+def test_the_timeline_records_every_workgroup_and_changes_nothing(tmp_path):
+    shape = SHAPES["llama-hd128"]
+    path = tmp_path / "m.gguf"
+    synth.write_model(path, shape, seed=31, device="cpu", std=0.05)
+    eng = E.Engine(path, E.EngineConfig(n_ctx=4 * 512, n_seq_max=4, n_batch=256, n_ubatch=256))
+    rng = np.random.default_rng(5)
+    lens = [40, 200, 7]
+    out = E.StepOutput()
+    for i, n in enumerate(lens):
+        eng.step([E.StepRow(i, i, rng.integers(0, shape.n_vocab, n), 0, sample=False, sampling=greedy())], out)
+    assert eng.attention_timeline_read().shape == (0, 6)
+    rows = lambda extra: [E.StepRow(i, i, [5 + i], lens[i] + extra, sample=True, sampling=greedy()) for i in range(3)]
+    eng.step(rows(0), out)
+    plain = eng.debug_logits().copy()
+    for i in range(3):
+        eng.seq_rm(i, lens[i], -1)
+    eng.attention_timeline(True)
+    eng.step(rows(0), out)
+    assert np.array_equal(eng.debug_logits(), plain)
+    st = eng.attention_timeline_read().astype(np.int64)
+    assert st.shape == (3 * shape.n_head_kv, 6)
+    assert sorted(st[:, 5].tolist()) == sorted([n // 32 + 1 for n in lens] * shape.n_head_kv)        # pages per row
+    assert (np.diff(st[:, :5], axis=1)[:, [0, 2, 3]] >= 0).all() and (st[:, 3] >= st[:, 1]).all()
+    assert (st[:, 4] - st[:, 0]).max() < 100 * 1000          # a workgroup of this size ends within a millisecond
+    eng.attention_timeline(False)
+    assert eng.attention_timeline_read().shape == (0, 6)
+    eng.close()

@@ -111,3 +111,43 @@ def test_the_timeline_records_every_workgroup_and_changes_nothing(tmp_path):
     eng.attention_timeline(False)
     assert eng.attention_timeline_read().shape == (0, 6)
     eng.close()
+
+
+def test_the_longest_sequences_the_one_launch_takes_and_the_first_it_leaves(tmp_path, monkeypatch):
+    """A workgroup's eight waves hold 64 page ids each: 512 pages, 16384 positions. A sequence decodes across that
+    boundary - on the one launch up to it, on the three launches beyond - and equals an engine that never takes the
+    one launch."""
+    shape = SHAPES["qwen2-hd64"]
+    path = tmp_path / "m.gguf"
+    synth.write_model(path, shape, seed=32, device="cpu", std=0.05)
+    cfg = E.EngineConfig(n_ctx=17 * 1024, n_seq_max=2, n_batch=512, n_ubatch=512)
+    monkeypatch.setenv("RETRO_FUSED_DECODE_ATTENTION", "1")
+    one = E.Engine(path, cfg)
+    monkeypatch.setenv("RETRO_FUSED_DECODE_ATTENTION", "0")
+    three = E.Engine(path, cfg)
+    rng = np.random.default_rng(6)
+    n0 = 16384 - 3
+    prompt = rng.integers(0, shape.n_vocab, n0).astype(np.int32)
+    out = E.StepOutput()
+    for eng in (one, three):
+        for at in range(0, n0, 512):
+            eng.step([E.StepRow(0, 0, prompt[at:at + 512], at, sample=False, sampling=greedy())], out)
+        eng.step([E.StepRow(1, 1, prompt[:40], 0, sample=False, sampling=greedy())], out)
+    one.attention_timeline(True)
+    tok = [7, 9]
+    for step in range(6):          # positions 16381 .. 16386 of slot 0: the last three on the fallback
+        got = []
+        for eng in (one, three):
+            eng.step([E.StepRow(0, 0, [tok[0]], n0 + step, sample=True, sampling=greedy()),
+                      E.StepRow(1, 1, [tok[1]], 40 + step, sample=True, sampling=greedy())], out)
+            got.append((eng.debug_logits().copy(), [out.row(0).token, out.row(1).token]))
+        mx, rel = logit_errors(got[0][0], got[1][0])
+        took_one_launch = len(one.attention_timeline_read()) > 0
+        print("position %d: one launch %s, max %.2e rel %.2e" % (n0 + step, took_one_launch, mx, rel), flush=True)
+        assert took_one_launch == (n0 + step + 1 <= 16384)
+        assert rel <= 2e-5, (step, mx, rel)
+        one.attention_timeline(False)          # forget the recorded launch, so that the next read tells this step's path
+        one.attention_timeline(True)
+        tok = got[1][1]
+    one.close()
+    three.close()

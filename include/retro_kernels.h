@@ -86,19 +86,25 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
 
 /* MXFP4 rows (GGUF block_mxfp4: an E8M0 byte and 16 nibble bytes per 32
  * values) times at most 16 tokens on the block-scaled FP4 x FP8 matrix
- * instruction, in ggml's arithmetic for this type: the activations become Q8_0
+ * instruction. y is [n_tokens][n_rows].
+ * exact == 0: ggml's arithmetic for this type - the activations become Q8_0
  * blocks (quantize_row_q8_0_ref), the integer code products of a block are
  * summed and scaled by both block scales (ggml_vec_dot_mxfp4_q8_0 of
  * ggml-org/llama.cpp@cd8427d0, the base of the fork pinned in reference
- * crates/retrograd-ffi/runtime/llama.cpp.lock:6-7). y is [n_tokens][n_rows].
- * n_rows in 16s, k in 256s and at most 4608 (the activation operands stay in
- * LDS). A kernel-level entry for measurement and parity: the engine's
- * mixture-of-experts path does not call it. */
-int retro_kernel_mxfp4_scaled(const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, int32_t n_tokens, float * y);
+ * crates/retrograd-ffi/runtime/llama.cpp.lock:6-7). n_rows in 16s, k in 256s
+ * and at most 4608 (the activation operands stay in LDS).
+ * exact != 0: the f32 activations themselves, to f32-accumulation accuracy
+ * (each written as a power of two times six signed hexadecimal digits, which
+ * are exact FP8 values with power-of-two block scales). n_rows in 32s, k in
+ * 256s.
+ * Kernel-level entries for measurement and parity; the engine's expert block
+ * runs the exact variant's mixture-of-experts form only under
+ * RETRO_MOE_SCALED=1 (measured slower there than its default kernels). */
+int retro_kernel_mxfp4_scaled(const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, int32_t n_tokens, int32_t exact, float * y);
 /* Microseconds per launch of the same product over pseudo-random device data;
  * cold != 0 gives every launch another copy of the weights (1 GiB of copies in
  * turn), so that they come from HBM. */
-int retro_kernel_mxfp4_scaled_time(int64_t n_rows, int64_t k, int32_t n_tokens, int32_t cold, int32_t iters, double * out_us);
+int retro_kernel_mxfp4_scaled_time(int64_t n_rows, int64_t k, int32_t n_tokens, int32_t exact, int32_t cold, int32_t iters, double * out_us);
 
 /* Microseconds per launch of a plain streaming kernel over `bytes` of device
  * memory: a copy (reads and writes `bytes` each) or, read_only, a pure read.

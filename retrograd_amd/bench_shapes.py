@@ -21,8 +21,8 @@ first part is timed as it is, the last `--profiled` steps run with an event pair
 around every kernel category (which slows them a little) for the breakdown.
 Prints one JSON line.
 
-mxfp4-scaled times one kernel, not a step: MXFP4 rows times 1 to 16 tokens under ggml's arithmetic on the
-block-scaled matrix instruction, as one dense matrix of the size of a layer's expert weights (gate and up of 128
+mxfp4-scaled times two kernels, not a step: MXFP4 rows times 1 to 16 tokens on the block-scaled matrix instruction,
+under ggml's arithmetic and under the exact one, as one dense matrix of the size of a layer's expert weights (gate and up of 128
 experts: 196608 rows of 2048; down: 262144 rows of 768), every launch on another copy of the weights so that they
 come from HBM."""
 from __future__ import annotations
@@ -78,14 +78,16 @@ def main() -> int:
         print("bench_shapes needs an MI355X: no HIP device is visible", file=sys.stderr)
         return 2
     if args.config == "mxfp4-scaled":
-        out = {"kernel": "k_mxs", "arithmetic": "ggml (Q8_0 activation blocks)", "weights": "pseudo-random, from HBM", "cases": []}
-        for what, n, k in (("gate_up", 2 * 128 * 768, 2048), ("down", 128 * 2048, 768)):
-            for t in (1, 4, 8, 16):
-                us = E.kernel_mxfp4_scaled_time(n, k, t, True, 50)
-                nbytes = n * (k // 32) * 17
-                out["cases"].append({"matrix": what, "rows": n, "k": k, "tokens": t, "us": round(us, 2),
-                                     "weight_bytes": nbytes, "tb_per_s": round(nbytes / us / 1e6, 3),
-                                     "frac_of_8_tb_per_s": round(nbytes / us / 1e6 / 8.0, 3)})
+        out = {"kernels": {"ggml": "k_mxs (Q8_0 activation blocks)", "exact": "k_mxe (f32 activations as six hexadecimal digits)"},
+               "weights": "pseudo-random, from HBM", "cases": []}
+        for exact in (False, True):
+            for what, n, k in (("gate_up", 2 * 128 * 768, 2048), ("down", 128 * 2048, 768)):
+                for t in (1, 4, 8, 16):
+                    us = E.kernel_mxfp4_scaled_time(n, k, t, True, 50, exact=exact)
+                    nbytes = n * (k // 32) * 17
+                    out["cases"].append({"arithmetic": "exact" if exact else "ggml", "matrix": what, "rows": n, "k": k, "tokens": t,
+                                         "us": round(us, 2), "weight_bytes": nbytes, "tb_per_s": round(nbytes / us / 1e6, 3),
+                                         "frac_of_8_tb_per_s": round(nbytes / us / 1e6 / 8.0, 3)})
         print(json.dumps(out))
         return 0
     rng = np.random.default_rng(args.seed)

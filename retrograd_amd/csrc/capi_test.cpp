@@ -290,10 +290,11 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
     });
 }
 
-int retro_kernel_mxfp4_scaled(const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, int32_t n_tokens, float * y) {
+int retro_kernel_mxfp4_scaled(const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, int32_t n_tokens, int32_t exact, float * y) {
     return guarded([&]() -> int {
-        if (!rk::mxs_can(k, n_rows, n_tokens))
-            throw std::runtime_error("mxfp4_scaled: rows in 16s, columns in 256s (at most 4608), 1..16 tokens");
+        if (exact ? !rk::mxe_can(k, n_rows, n_tokens) : !rk::mxs_can(k, n_rows, n_tokens))
+            throw std::runtime_error(exact ? "mxfp4_scaled, exact: rows in 32s, columns in 256s, 1..16 tokens"
+                                           : "mxfp4_scaled: rows in 16s, columns in 256s (at most 4608), 1..16 tokens");
         const size_t bytes = (size_t)n_rows * (size_t)(k / 32) * 17;
         DevBuf d_raw, d_packed, d_x, d_ops, d_dx, d_y;
         d_raw.alloc(bytes);
@@ -302,19 +303,26 @@ int retro_kernel_mxfp4_scaled(const uint8_t * raw, int64_t n_rows, int64_t k, co
         rk::mxs_repack(nullptr, d_raw.as<uint8_t>(), d_packed.as<uint8_t>(), (int)k, n_rows);
         d_x.alloc((size_t)n_tokens * k * 4);
         ok(hipMemcpy(d_x.ptr, x, d_x.bytes, hipMemcpyHostToDevice), "upload activations");
-        d_ops.alloc(rk::mxs_operand_bytes((int)k));
-        d_dx.alloc(rk::mxs_scale_bytes((int)k));
-        rk::mxs_quantise(nullptr, d_x.as<float>(), n_tokens, (int)k, d_ops.as<uint8_t>(), d_dx.as<float>());
         d_y.alloc((size_t)n_tokens * n_rows * 4);
-        rk::mxs_matmul(nullptr, d_packed.as<uint8_t>(), d_ops.as<uint8_t>(), d_dx.as<float>(), (int)k, n_rows, n_tokens, d_y.as<float>());
+        if (exact) {
+            d_ops.alloc(rk::mxe_operand_bytes((int)k));
+            d_dx.alloc(rk::mxe_scale_bytes((int)k));
+            rk::mxe_pieces(nullptr, d_x.as<float>(), n_tokens, (int)k, d_ops.as<uint8_t>(), d_dx.as<uint8_t>());
+            rk::mxe_matmul(nullptr, d_packed.as<uint8_t>(), d_ops.as<uint8_t>(), d_dx.as<uint8_t>(), (int)k, n_rows, n_tokens, d_y.as<float>());
+        } else {
+            d_ops.alloc(rk::mxs_operand_bytes((int)k));
+            d_dx.alloc(rk::mxs_scale_bytes((int)k));
+            rk::mxs_quantise(nullptr, d_x.as<float>(), n_tokens, (int)k, d_ops.as<uint8_t>(), d_dx.as<float>());
+            rk::mxs_matmul(nullptr, d_packed.as<uint8_t>(), d_ops.as<uint8_t>(), d_dx.as<float>(), (int)k, n_rows, n_tokens, d_y.as<float>());
+        }
         ok(hipMemcpy(y, d_y.ptr, d_y.bytes, hipMemcpyDeviceToHost), "download");
         return 0;
     });
 }
 
-int retro_kernel_mxfp4_scaled_time(int64_t n_rows, int64_t k, int32_t n_tokens, int32_t cold, int32_t iters, double * out_us) {
+int retro_kernel_mxfp4_scaled_time(int64_t n_rows, int64_t k, int32_t n_tokens, int32_t exact, int32_t cold, int32_t iters, double * out_us) {
     return guarded([&]() -> int {
-        if (!rk::mxs_can(k, n_rows, n_tokens) || iters <= 0)
+        if ((exact ? !rk::mxe_can(k, n_rows, n_tokens) : !rk::mxs_can(k, n_rows, n_tokens)) || iters <= 0)
             throw std::runtime_error("mxfp4_scaled_time: rows in 16s, columns in 256s (at most 4608), 1..16 tokens, at least one launch");
         const size_t bytes = rk::mxs_packed_bytes(k, n_rows);
         const size_t copies = cold ? std::max<size_t>(2, ((size_t)1 << 30) / bytes) : 1;
@@ -334,16 +342,23 @@ int retro_kernel_mxfp4_scaled_time(int64_t n_rows, int64_t k, int32_t n_tokens, 
             d_x.alloc(xs.size() * 4);
             ok(hipMemcpy(d_x.ptr, xs.data(), d_x.bytes, hipMemcpyHostToDevice), "fill");
         }
-        d_ops.alloc(rk::mxs_operand_bytes((int)k));
-        d_dx.alloc(rk::mxs_scale_bytes((int)k));
-        rk::mxs_quantise(nullptr, d_x.as<float>(), n_tokens, (int)k, d_ops.as<uint8_t>(), d_dx.as<float>());
+        if (exact) {
+            d_ops.alloc(rk::mxe_operand_bytes((int)k));
+            d_dx.alloc(rk::mxe_scale_bytes((int)k));
+            rk::mxe_pieces(nullptr, d_x.as<float>(), n_tokens, (int)k, d_ops.as<uint8_t>(), d_dx.as<uint8_t>());
+        } else {
+            d_ops.alloc(rk::mxs_operand_bytes((int)k));
+            d_dx.alloc(rk::mxs_scale_bytes((int)k));
+            rk::mxs_quantise(nullptr, d_x.as<float>(), n_tokens, (int)k, d_ops.as<uint8_t>(), d_dx.as<float>());
+        }
         d_y.alloc((size_t)n_tokens * n_rows * 4);
         hipEvent_t e0, e1;
         ok(hipEventCreate(&e0), "event"); ok(hipEventCreate(&e1), "event");
         size_t turn = 0;
         auto run = [&]() {
-            rk::mxs_matmul(nullptr, d_w.as<uint8_t>() + (turn++ % copies) * bytes, d_ops.as<uint8_t>(), d_dx.as<float>(), (int)k, n_rows,
-                           n_tokens, d_y.as<float>());
+            const uint8_t * w = d_w.as<uint8_t>() + (turn++ % copies) * bytes;
+            if (exact) rk::mxe_matmul(nullptr, w, d_ops.as<uint8_t>(), d_dx.as<uint8_t>(), (int)k, n_rows, n_tokens, d_y.as<float>());
+            else rk::mxs_matmul(nullptr, w, d_ops.as<uint8_t>(), d_dx.as<float>(), (int)k, n_rows, n_tokens, d_y.as<float>());
         };
         for (int i = 0; i < 3; ++i) run();
         ok(hipEventRecord(e0, nullptr), "record");

@@ -74,6 +74,7 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
     hip_check(hipStreamCreate(&stream_), "hipStreamCreate");
     rk::sample_static_prepare();       // the no-allocation greedy scan then only launches, also under stream capture
     if (const char * v = std::getenv("RETRO_FUSED_DECODE_ATTENTION")) fused_decode_attention_ = std::atoi(v) != 0;
+    if (const char * v = std::getenv("RETRO_MOE_SCALED")) moe_scaled_ = std::atoi(v) != 0;
     {
         // RETRO_ACTIVATIONS=ggml: every matmul multiplies the activations as ggml's CPU path converts them
         // (Q8_K / Q8_0 codes, f16 / bf16 rounding); unset or "exact": the f32 values (as f16 hi/lo pairs).
@@ -187,6 +188,13 @@ void Engine::upload_experts(const TensorInfo & t, int64_t K, int64_t N, DevWeigh
     hip_check(hipStreamSynchronize(stream_), "repack");
     out.w.packed = out.buf.as<uint8_t>();
     out.w.raw = nullptr;
+    // MXFP4 experts of the exact arithmetic also in the records of the block-scaled kernels (decode-sized steps take them)
+    if (t.type == rk::WT_MXFP4 && moe_scaled_ && !ggml_activations_ && rk::mxe_moe_can((int)K, (int)N)) {
+        out.records.alloc(rk::mxs_packed_bytes(K, rows));
+        rk::mxs_repack(stream_, raw.as<uint8_t>(), out.records.as<uint8_t>(), (int)K, rows);
+        hip_check(hipStreamSynchronize(stream_), "repack");
+        out.w.records = out.records.as<uint8_t>();
+    }
 }
 
 // Row-wise concatenation of matrices that share K and storage type: one matmul
@@ -460,6 +468,15 @@ void Engine::build_buffers() {
         moe_h_.alloc(rk::act_halves((int)slots, FE) * 2);
         hip_check(hipMemsetAsync(moe_h_.ptr, 0, moe_h_.bytes, stream_), "hipMemsetAsync");
         moe_out_.alloc(slots * (size_t)E * 4);
+        if (moe_scaled_ && !ggml_activations_ && rk::mxe_moe_can(E, FE)) {
+            // the block-scaled expert path serves steps of at most 12 pairs per expert on average
+            const int t_small = std::min(B, 12 * NE / KU);
+            moe_mx_slots_ = rk::moe_slots(t_small, KU, NE);
+            const int wide = std::max(E, FE);
+            moe_mx_ops_.alloc(rk::mxe_moe_operand_bytes(wide, moe_mx_slots_));
+            moe_mx_scales_.alloc(rk::mxe_moe_scale_bytes(wide, moe_mx_slots_));
+            moe_mx_h_.alloc(moe_mx_slots_ * (size_t)FE * 4);
+        }
     }
     q_half_.alloc((size_t)B * QD * 2);
     // operand-order activations; the sums keep zero padding lanes, so they are cleared once
@@ -1510,6 +1527,8 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
             rk::MoeBuffers mb{moe_logits_.as<float>(), moe_sel_.as<int32_t>(), moe_wgt_.as<float>(), moe_n_.as<int32_t>(),
                               moe_off_.as<int32_t>(), moe_tok_.as<int32_t>(), moe_q_.as<int32_t>(),
                               rk::Act{moe_h_.as<__half>(), nullptr, h.n_ff_exp}, moe_out_.as<float>()};
+            mb.mx_ops = moe_mx_ops_.as<uint8_t>(); mb.mx_scales = moe_mx_scales_.as<uint8_t>(); mb.mx_h = moe_mx_h_.as<float>();
+            mb.mx_slots = moe_mx_slots_;
             rk::moe_ffn(stream_, ml, ms, act_e, T, x, mb);
             pending = rk::Slices();
             prof_end(PC_GATEUP, pt_);

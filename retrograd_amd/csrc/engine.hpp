@@ -65,6 +65,7 @@ struct HParams {
 struct DevWeight {
     rk::Weight w;
     DevBuf buf;
+    DevBuf records;      // MXFP4 expert tensors: the rows again in the block-scaled kernels' records
 };
 
 struct LayerWeights {
@@ -357,6 +358,10 @@ private:
     DevBuf lora_mid_;         // [n_batch][LORA_MAX_RANK] f32
     int lora_routes_ = 0;
     bool ggml_activations_ = false;   // RETRO_ACTIVATIONS=ggml at construction
+    bool moe_scaled_ = false;         // RETRO_MOE_SCALED=1: decode-sized steps multiply MXFP4 experts on the block-scaled matrix
+                                      // instruction (measured slower than the f16 tile kernels end to end, so it is off by default)
+    DevBuf moe_mx_ops_, moe_mx_scales_, moe_mx_h_;
+    size_t moe_mx_slots_ = 0;
     void rebuild_lora_table();
     int read_adapter(const std::string & path, float scale, RowAdapterData & data);
     RowAdapterData clone_adapter(const RowAdapterData & src, float scale);

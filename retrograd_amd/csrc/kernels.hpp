@@ -36,6 +36,7 @@ struct Weight {
     const uint8_t * raw = nullptr;
     const uint8_t * packed = nullptr;
     size_t bytes = 0;
+    const uint8_t * records = nullptr;      // MXFP4 expert rows again, in the records of the block-scaled kernels (mxs_repack)
 };
 
 // Activations handed to a matmul. An f32 value v travels as two f16 numbers,
@@ -158,6 +159,26 @@ void mxs_repack(hipStream_t s, const uint8_t * raw, uint8_t * packed, int K, int
 void mxs_quantise(hipStream_t s, const float * x, int n_tokens, int K, uint8_t * operands, float * scales);
 void mxs_matmul(hipStream_t s, const uint8_t * packed, const uint8_t * operands, const float * scales, int K, int64_t N,
                 int n_tokens, float * y);
+// The same product on f32 activations to f32-accumulation accuracy: mxe_pieces writes every activation as a power of
+// two times six signed hexadecimal digits (operands mxe_operand_bytes, scales mxe_scale_bytes), mxe_matmul multiplies
+// them with the records mxs_repack made (rows in 32s, columns in 256s of any length).
+bool mxe_can(int64_t K, int64_t N, int n_tokens);
+size_t mxe_operand_bytes(int K);
+size_t mxe_scale_bytes(int K);
+void mxe_pieces(hipStream_t s, const float * x, int n_tokens, int K, uint8_t * operands, uint8_t * scales);
+void mxe_matmul(hipStream_t s, const uint8_t * packed, const uint8_t * operands, const uint8_t * scales, int K, int64_t N,
+                int n_tokens, float * y);
+// The expert products of a mixture-of-experts step on the same instruction (MXFP4 experts whose rows are also held as
+// records, f32-accumulation accuracy): per group of 16 pair slots the activation rows are written as digits
+// (operands mxe_moe_operand_bytes, scales mxe_moe_scale_bytes for `slots` slots of width K), then gate and up with
+// SwiGLU leave f32 rows h [slot][F], and down leaves out_pair [slot][E]. Widths in 256s.
+bool mxe_moe_can(int E, int F);
+size_t mxe_moe_operand_bytes(int K, size_t slots);
+size_t mxe_moe_scale_bytes(int K, size_t slots);
+void mxe_moe_gate_up(hipStream_t s, const uint8_t * gate, const uint8_t * up, const Act & x, int E, int F, int n_expert,
+                     const int32_t * off_pad, const int32_t * tok_of_q, size_t slots, uint8_t * ops, uint8_t * scales, float * h);
+void mxe_moe_down(hipStream_t s, const uint8_t * down, const float * h, int E, int F, int n_expert, const int32_t * off_pad,
+                  const int32_t * tok_of_q, size_t slots, uint8_t * ops, uint8_t * scales, float * out_pair);
 // The weight's side of gemv_can. With it the same product can take its rows as f32 and make the Q8_K blocks while
 // it stages them, one launch instead of two: gemv_norm from the residual rows (x row rows[t], or t; RMSNorm with
 // norm_w and eps as rmsnorm_act computes it, then the conversion), gemv_swiglu from the f32 rows of a gate/up product
@@ -238,6 +259,12 @@ struct MoeBuffers {            // device scratch of one step, sized with moe_slo
     int32_t * q_of_pair;       // [T * k_used]
     Act h;                     // [slots] x F
     float * out_pair;          // [slots][E]
+    // the block-scaled path of MXFP4 experts (decode-sized steps of the exact arithmetic), or null: activation operands
+    // and scales for mx_slots pair slots of the wider of the two products, and the hidden rows as f32 [mx_slots][F]
+    uint8_t * mx_ops = nullptr;
+    uint8_t * mx_scales = nullptr;
+    float * mx_h = nullptr;
+    size_t mx_slots = 0;
 };
 size_t moe_slots(int n_tokens, int k_used, int n_expert);
 // x[t] += sum over the token's k_used experts of w * down_e(silu(gate_e xn) * (up_e xn))

@@ -615,6 +615,20 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     const unsigned gu_blocks = (unsigned)(((size_t)sh.n_expert * (sh.F / 16) + 3) / 4);
     // few pairs per expert (a decode step): one token tile per pass
     const bool one_tile = (size_t)T * sh.k_used <= (size_t)12 * sh.n_expert;
+    // MXFP4 experts in such a step, exact arithmetic: the block-scaled FP4 x FP8 matrix instruction takes the stored
+    // codes and exponents as they are (no decode), the activations as hexadecimal digits
+    const size_t slots = moe_slots(T, sh.k_used, sh.n_expert);
+    if (one_tile && !xn.faithful && L.gate.type == WT_MXFP4 && L.down.type == WT_MXFP4 && L.gate.records && L.up.records
+        && L.down.records && b.mx_ops && slots <= b.mx_slots && mxe_moe_can(sh.E, sh.F)) {
+        mxe_moe_gate_up(s, L.gate.records, L.up.records, xn, sh.E, sh.F, sh.n_expert, b.off_pad, b.tok_of_q, slots, b.mx_ops,
+                        b.mx_scales, b.mx_h);
+        mxe_moe_down(s, L.down.records, b.mx_h, sh.E, sh.F, sh.n_expert, b.off_pad, b.tok_of_q, slots, b.mx_ops, b.mx_scales,
+                     b.out_pair);
+        hipLaunchKernelGGL(k_moe_combine, dim3(T, (sh.E / 4 + 255) / 256), dim3(256), 0, s, b.out_pair, b.q_of_pair, b.wgt,
+                           sh.k_used, sh.E, x);
+        check_launch("moe_combine");
+        return;
+    }
     // (measured on the 128-expert shape at 128 rows: the down projection gains a fifth from the smaller
     // workgroups, gate/up - two weight tiles per wave - loses a tenth, so it keeps two tiles)
     switch (L.gate.type) {

@@ -250,8 +250,8 @@ def load_library() -> C.CDLL:
     lib.retro_kernel_gemv_fused.restype = C.c_int
     lib.retro_kernel_matmul_time.argtypes = [C.c_int32, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,
                                              C.c_int32, C.c_int32, C.POINTER(C.c_double)]
-    lib.retro_kernel_mxfp4_scaled.argtypes = [_u8p, C.c_int64, C.c_int64, _f32p, C.c_int32, _f32p]
-    lib.retro_kernel_mxfp4_scaled_time.argtypes = [C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_double)]
+    lib.retro_kernel_mxfp4_scaled.argtypes = [_u8p, C.c_int64, C.c_int64, _f32p, C.c_int32, C.c_int32, _f32p]
+    lib.retro_kernel_mxfp4_scaled_time.argtypes = [C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_double)]
     lib.retro_kernel_stream_time.argtypes = [C.c_int64, C.c_int32, C.c_int32, C.POINTER(C.c_double)]
     lib.retro_kernel_page_size.restype = C.c_int32
     lib.retro_kernel_max_topk.restype = C.c_int32
@@ -1016,23 +1016,24 @@ def kernel_matmul_time(ggml_type: int, n_rows: int, k: int, n_tokens: int, mode:
     return out.value
 
 
-def kernel_mxfp4_scaled(raw, n_rows: int, k: int, x: np.ndarray) -> np.ndarray:
-    """MXFP4 rows times at most 16 tokens on the block-scaled matrix instruction, ggml's arithmetic."""
+def kernel_mxfp4_scaled(raw, n_rows: int, k: int, x: np.ndarray, exact: bool = False) -> np.ndarray:
+    """MXFP4 rows times at most 16 tokens on the block-scaled matrix instruction: ggml's arithmetic (Q8_0 activation
+    blocks), or with `exact` the f32 activations themselves."""
     src = np.ascontiguousarray(raw, np.uint8)
     x = np.ascontiguousarray(x, np.float32).reshape(-1, k)
     y = np.empty((x.shape[0], n_rows), np.float32)
     s = load_library().retro_kernel_mxfp4_scaled(src.ctypes.data_as(C.POINTER(C.c_uint8)), n_rows, k,
-                                                 x.ctypes.data_as(C.POINTER(C.c_float)), x.shape[0],
+                                                 x.ctypes.data_as(C.POINTER(C.c_float)), x.shape[0], 1 if exact else 0,
                                                  y.ctypes.data_as(C.POINTER(C.c_float)))
     if s != 0:
         _raise(s)
     return y
 
 
-def kernel_mxfp4_scaled_time(n_rows: int, k: int, n_tokens: int, cold: bool = True, iters: int = 50) -> float:
+def kernel_mxfp4_scaled_time(n_rows: int, k: int, n_tokens: int, cold: bool = True, iters: int = 50, exact: bool = False) -> float:
     """Microseconds per launch of kernel_mxfp4_scaled's product on device-only data."""
     out = C.c_double()
-    s = load_library().retro_kernel_mxfp4_scaled_time(n_rows, k, n_tokens, 1 if cold else 0, iters, C.byref(out))
+    s = load_library().retro_kernel_mxfp4_scaled_time(n_rows, k, n_tokens, 1 if exact else 0, 1 if cold else 0, iters, C.byref(out))
     if s != 0:
         _raise(s)
     return out.value

@@ -52,6 +52,57 @@ def test_moe_prefill_and_decode_match_the_oracle(tmp_path, key):
     eng.close()
 
 
+def test_mxfp4_experts_on_the_block_scaled_instruction(tmp_path, monkeypatch):
+    """RETRO_MOE_SCALED=1: decode-sized steps multiply the MXFP4 experts on the block-scaled FP4 x FP8 matrix
+    instruction (the stored codes and exponents as they are, the activations as hexadecimal digits); larger steps keep
+    the tile kernels. Against the oracle, and against the default engine: close, and not the same bits, so the step did
+    take the other path. An expert with more than 16 pairs (two groups of slots) and experts with none are among them."""
+    shape = synth.scaled(synth.QWEN3_30B_A3B, name="qwen3moe-small-mxfp4-wide", n_layer=2, n_embd=512, n_head=8, n_head_kv=2,
+                         head_dim=64, n_vocab=1024, n_expert=16, n_expert_used=4, n_ff_exp=768)
+    print("mixture of experts on the block-scaled instruction: %s" % shape.name, flush=True)
+    path = tmp_path / "moe.gguf"
+    synth.write_model(path, shape, seed=6, device="cpu", std=0.05)
+    cfg = E.EngineConfig(n_ctx=4096, n_seq_max=48, n_batch=256, n_ubatch=256)
+    plain = E.Engine(path, cfg)
+    monkeypatch.setenv("RETRO_MOE_SCALED", "1")
+    scaled = E.Engine(path, cfg)
+    m = oracle.Model(path)
+    ctx = oracle.Context(m, 48)
+    rng = np.random.default_rng(3)
+    n_seq = 40                                     # 160 pairs over 16 experts: ten on average, some above 16
+    lens = [int(n) for n in rng.integers(3, 30, n_seq)]
+    prompts = [rng.integers(0, m.n_vocab, n) for n in lens]
+    rows = [(i, i, p, 0, True) for i, p in enumerate(prompts)]
+    out = E.StepOutput()
+    for at in range(0, n_seq, 8):                  # prefill steps of more than 12 pairs per expert: the tile kernels
+        for eng in (plain, scaled):
+            eng.step([E.StepRow(r[0], r[1], r[2], r[3], sample=True, sampling=greedy()) for r in rows[at:at + 8]], out)
+        ctx.step_rows([(r[1], r[3], r[2], r[4]) for r in rows[at:at + 8]])
+    pos = list(lens)
+    feed = [int(t) for t in rng.integers(0, m.n_vocab, n_seq)]
+    differs = False
+    for step in range(3):
+        live = list(range(n_seq)) if step != 1 else [0, 5, 6]          # 160 pairs, then 12 (most experts idle), then 160
+        steprows = [E.StepRow(i, i, [feed[i]], pos[i], sample=True, sampling=greedy()) for i in live]
+        plain.step(steprows, out)
+        a = plain.debug_logits().copy()
+        scaled.step(steprows, out)
+        b = scaled.debug_logits().copy()
+        want = ctx.step_rows([(i, pos[i], [feed[i]], True) for i in live])
+        assert_logits_close(a, want)
+        assert_logits_close(b, want)
+        mx, rel = logit_errors(b, a)
+        print("step %d: scaled against tile kernels, max %.2e rel %.2e" % (step, mx, rel), flush=True)
+        assert rel <= 2e-5
+        differs = differs or not np.array_equal(a, b)
+        for j, i in enumerate(live):
+            feed[i] = int(want[j].argmax())
+            pos[i] += 1
+    assert differs
+    plain.close()
+    scaled.close()
+
+
 @pytest.mark.parametrize("key", list(SHAPES))
 def test_moe_under_the_ggml_arithmetic(tmp_path, key, monkeypatch):
     """RETRO_ACTIVATIONS=ggml: the router (F32) multiplies the rows as they are, the experts

@@ -452,7 +452,7 @@ struct MxeMoeArgs {
     int nb, tiles_per_expert, N, parts, chunk_records, n_chunks;
 };
 
-template <bool GATE_UP>
+template <bool GATE_UP, int MAXP>
 __global__ __launch_bounds__(1024, 1) void k_mxe_moe(MxeMoeArgs a) {
     extern __shared__ __align__(16) uint8_t lds[];
     __shared__ int s_expert;
@@ -468,8 +468,9 @@ __global__ __launch_bounds__(1024, 1) void k_mxe_moe(MxeMoeArgs a) {
     const size_t tile_bytes = (size_t)ng * MXS_RECORD;
     const int n_pairs = GATE_UP ? a.tiles_per_expert : a.tiles_per_expert / 2;
     const int per_part = (n_pairs + a.parts - 1) / a.parts;
-    const int ip0 = part * per_part + 2 * wave;
-    const int n_mine = min(2, max(0, min(per_part - 2 * wave, n_pairs - ip0)));
+    // a wave's tile pairs of the part: MAXP consecutive ones
+    const int ip0 = part * per_part + MAXP * wave;
+    const int n_mine = min(MAXP, max(0, min(per_part - MAXP * wave, n_pairs - ip0)));
     // first tile of a pair and the distance to its second
     auto tile_of = [&](int ip) { return (size_t)expert * a.tiles_per_expert + (GATE_UP ? ip : 2 * ip); };
     const ptrdiff_t second = GATE_UP ? (a.w1 - a.w0) : (ptrdiff_t)tile_bytes;
@@ -478,9 +479,9 @@ __global__ __launch_bounds__(1024, 1) void k_mxe_moe(MxeMoeArgs a) {
     const int * l_scales = (const int *)(lds + (size_t)chunk_pairs * MXE_PAIR_BYTES);
     const uint8_t * g_ops = a.ops + (size_t)g * (a.nb / 2) * MXE_PAIR_BYTES;
     const uint8_t * g_scales = a.scales + (size_t)g * (a.nb / 2) * MXE_PAIR_SCALES;
-    f4v acc[2][2];
+    f4v acc[MAXP][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) { acc[i][0] = f4v{0.f, 0.f, 0.f, 0.f}; acc[i][1] = f4v{0.f, 0.f, 0.f, 0.f}; }
+    for (int i = 0; i < MAXP; ++i) { acc[i][0] = f4v{0.f, 0.f, 0.f, 0.f}; acc[i][1] = f4v{0.f, 0.f, 0.f, 0.f}; }
     for (int c = 0; c < a.n_chunks; ++c) {
         const int rec0 = c * a.chunk_records, n_rec = min(a.chunk_records, ng - rec0);
         const int n_items = n_mine * n_rec * 2;
@@ -512,40 +513,42 @@ __global__ __launch_bounds__(1024, 1) void k_mxe_moe(MxeMoeArgs a) {
             for (int i0 = tid; i0 < n_rec * 4 * 64; i0 += 1024) sdst[i0] = ssrc[i0];
         }
         __syncthreads();
-        int cg = 0, ct = 0;
-        for (int it = 0; it < n_items; it += 2) {
-            {
-                const uint8_t * po = l_ops + (size_t)(2 * cg) * MXE_PAIR_BYTES;
-                const int * ps = l_scales + (2 * cg) * 64;
-                f4v & x0 = acc[ct][0], & x1 = acc[ct][1];
-                mxe_pair<0>(G0[0].a[0], G0[0].e, G0[1].a[0], G0[1].e, po, ps, lane, x0, x1);
-                mxe_pair<1>(G0[0].a[1], G0[0].e, G0[1].a[1], G0[1].e, po + MXE_PAIR_BYTES, ps + 64, lane, x0, x1);
-                asm volatile("" : "+v"(x0), "+v"(x1) : : "memory");
-                __builtin_amdgcn_sched_barrier(0);
-                mxe_load(G0[0], lp, 0, lane_at); mxe_load(G0[1], lp + second, 0, lane_at);
-                __builtin_amdgcn_sched_barrier(0);
-                advance();
-                ++cg;
-            }
-            {
-                const uint8_t * po = l_ops + (size_t)(2 * cg) * MXE_PAIR_BYTES;
-                const int * ps = l_scales + (2 * cg) * 64;
-                f4v & x0 = acc[ct][0], & x1 = acc[ct][1];
-                mxe_pair<2>(G1[0].a[0], G1[0].e, G1[1].a[0], G1[1].e, po, ps, lane, x0, x1);
-                mxe_pair<3>(G1[0].a[1], G1[0].e, G1[1].a[1], G1[1].e, po + MXE_PAIR_BYTES, ps + 64, lane, x0, x1);
-                asm volatile("" : "+v"(x0), "+v"(x1) : : "memory");
-                __builtin_amdgcn_sched_barrier(0);
-                mxe_load(G1[0], lp, 1, lane_at); mxe_load(G1[1], lp + second, 1, lane_at);
-                __builtin_amdgcn_sched_barrier(0);
-                advance();
-                if (++cg == 2 * n_rec) { cg = 0; ++ct; }
+#pragma unroll
+        for (int i = 0; i < MAXP; ++i) {
+            if (i >= n_mine) break;
+            f4v & x0 = acc[i][0], & x1 = acc[i][1];
+            for (int cg = 0; cg < 2 * n_rec; cg += 2) {
+                {
+                    const uint8_t * po = l_ops + (size_t)(2 * cg) * MXE_PAIR_BYTES;
+                    const int * ps = l_scales + (2 * cg) * 64;
+                    mxe_pair<0>(G0[0].a[0], G0[0].e, G0[1].a[0], G0[1].e, po, ps, lane, x0, x1);
+                    mxe_pair<1>(G0[0].a[1], G0[0].e, G0[1].a[1], G0[1].e, po + MXE_PAIR_BYTES, ps + 64, lane, x0, x1);
+                    asm volatile("" : "+v"(x0), "+v"(x1) : : "memory");
+                    __builtin_amdgcn_sched_barrier(0);
+                    mxe_load(G0[0], lp, 0, lane_at); mxe_load(G0[1], lp + second, 0, lane_at);
+                    __builtin_amdgcn_sched_barrier(0);
+                    advance();
+                }
+                {
+                    const uint8_t * po = l_ops + (size_t)(2 * cg + 2) * MXE_PAIR_BYTES;
+                    const int * ps = l_scales + (2 * cg + 2) * 64;
+                    mxe_pair<2>(G1[0].a[0], G1[0].e, G1[1].a[0], G1[1].e, po, ps, lane, x0, x1);
+                    mxe_pair<3>(G1[0].a[1], G1[0].e, G1[1].a[1], G1[1].e, po + MXE_PAIR_BYTES, ps + 64, lane, x0, x1);
+                    asm volatile("" : "+v"(x0), "+v"(x1) : : "memory");
+                    __builtin_amdgcn_sched_barrier(0);
+                    mxe_load(G1[0], lp, 1, lane_at); mxe_load(G1[1], lp + second, 1, lane_at);
+                    __builtin_amdgcn_sched_barrier(0);
+                    advance();
+                }
             }
         }
         __syncthreads();
     }
     // lane l holds pair slot slot0 + l % 16, rows 4 (l / 16) .. + 3 of a tile
     float * row = a.out + (size_t)(slot0 + r) * a.N;
-    for (int i = 0; i < n_mine; ++i) {
+#pragma unroll
+    for (int i = 0; i < MAXP; ++i) {
+        if (i >= n_mine) break;
         if (GATE_UP) {
             float v[4];
 #pragma unroll
@@ -555,6 +558,7 @@ __global__ __launch_bounds__(1024, 1) void k_mxe_moe(MxeMoeArgs a) {
             }
             *(float4 *)(row + (size_t)(ip0 + i) * 16 + 4 * q) = make_float4(v[0], v[1], v[2], v[3]);
         } else {
+#pragma unroll
             for (int tl = 0; tl < 2; ++tl)
                 *(float4 *)(row + (size_t)(2 * (ip0 + i) + tl) * 16 + 4 * q) = make_float4(acc[i][tl][0], acc[i][tl][1], acc[i][tl][2], acc[i][tl][3]);
         }
@@ -635,27 +639,42 @@ bool mxe_moe_can(int E, int F) { return E % 256 == 0 && F % 256 == 0 && E > 0 &&
 size_t mxe_moe_operand_bytes(int K, size_t slots) { return slots / 16 * (size_t)(K / 64) * MXE_PAIR_BYTES; }
 size_t mxe_moe_scale_bytes(int K, size_t slots) { return slots / 16 * (size_t)(K / 64) * MXE_PAIR_SCALES; }
 
-static void mxe_moe_launch(hipStream_t s, bool gate_up, const uint8_t * w0, const uint8_t * w1, const uint8_t * ops,
-                           const uint8_t * scales, const int32_t * off_pad, int n_expert, size_t slots, int K, int N, float * out) {
+template <bool GATE_UP, int MAXP>
+static void mxe_moe_launch_as(hipStream_t s, const MxeMoeArgs & a, unsigned grid, size_t lds) {
     static bool raised = false;
     if (!raised) {
         // (the kernel also holds a word of static LDS: six records' operands are 150 KiB)
-        HIP_OK(hipFuncSetAttribute((const void *)k_mxe_moe<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024));
-        HIP_OK(hipFuncSetAttribute((const void *)k_mxe_moe<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024));
+        HIP_OK(hipFuncSetAttribute((const void *)k_mxe_moe<GATE_UP, MAXP>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024));
         raised = true;
     }
+    hipLaunchKernelGGL((k_mxe_moe<GATE_UP, MAXP>), dim3(grid), dim3(1024), lds, s, a);
+}
+
+static void mxe_moe_launch(hipStream_t s, bool gate_up, const uint8_t * w0, const uint8_t * w1, const uint8_t * ops,
+                           const uint8_t * scales, const int32_t * off_pad, int n_expert, size_t slots, int K, int N, float * out) {
     MxeMoeArgs a {};
     a.w0 = w0; a.w1 = w1; a.ops = ops; a.scales = scales; a.off_pad = off_pad; a.n_expert = n_expert; a.out = out;
     a.nb = K / 32; a.tiles_per_expert = N / 16; a.N = N;
+    // a workgroup of 16 waves takes a group of 16 pair slots and, when it can, all tile pairs of the expert (up to
+    // four per wave): the fewer workgroups share a group, the less its operands are re-read, and about one
+    // workgroup per expert fits the chip in one turn
     const int n_pairs = gate_up ? N / 16 : N / 32;
-    a.parts = (n_pairs + 31) / 32;
+    const int maxp = std::min(4, (n_pairs + 15) / 16);
+    a.parts = (n_pairs + 16 * maxp - 1) / (16 * maxp);
     const int ng = K / 256;
     a.n_chunks = (ng + 5) / 6;
     a.chunk_records = (ng + a.n_chunks - 1) / a.n_chunks;
     const size_t lds = (size_t)a.chunk_records * 4 * (MXE_PAIR_BYTES + MXE_PAIR_SCALES);
     const unsigned grid = (unsigned)(slots / 16 * a.parts);
-    if (gate_up) hipLaunchKernelGGL(k_mxe_moe<true>, dim3(grid), dim3(1024), lds, s, a);
-    else hipLaunchKernelGGL(k_mxe_moe<false>, dim3(grid), dim3(1024), lds, s, a);
+#define RK_MXE_MOE(GU)                                                          \
+    switch (maxp) {                                                             \
+        case 1: mxe_moe_launch_as<GU, 1>(s, a, grid, lds); break;               \
+        case 2: mxe_moe_launch_as<GU, 2>(s, a, grid, lds); break;               \
+        case 3: mxe_moe_launch_as<GU, 3>(s, a, grid, lds); break;               \
+        default: mxe_moe_launch_as<GU, 4>(s, a, grid, lds); break;              \
+    }
+    if (gate_up) { RK_MXE_MOE(true) } else { RK_MXE_MOE(false) }
+#undef RK_MXE_MOE
     check_launch("k_mxe_moe");
 }
 

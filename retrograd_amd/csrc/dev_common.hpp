@@ -221,8 +221,9 @@ struct MMArgs {
     int ksplit;       // v1: waves of a workgroup sharing a row tile along K; v2: workgroups sharing a row group
     // v2 only
     int n_row_groups;
-    float * partial;          // [ksplit][64][pld] K-slices of a split matmul; this matrix fills columns pcol .. pcol + N
+    float * partial;          // [ksplit][slice_rows][pld] K-slices of a split matmul; this matrix fills columns pcol .. pcol + N
     int pld, pcol;            // (pld = N, pcol = 0 unless several matrices share the slices)
+    int slice_rows;           // token rows of a slice: 64 per chunk of the step
     // mode MM_SWIGLU: rows come in groups of 128, 64 gate rows then the 64 up rows of the same
     // columns; the epilogue writes silu(gate) * up as the activations of the next matmul
     Act act_out;

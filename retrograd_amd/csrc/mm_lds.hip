@@ -164,7 +164,7 @@ __device__ __forceinline__ void store_token_rows(const MMArgs & a, uint8_t * sme
     const int n = rg * 64 * R + col;
     if (n >= a.N) return;
     const bool sliced = a.ksplit > 1;
-    float * slice = sliced ? a.partial + (size_t)ks * 64 * a.pld + a.pcol : nullptr;
+    float * slice = sliced ? a.partial + (size_t)ks * a.slice_rows * a.pld + a.pcol : nullptr;
     const f4 bias = (a.bias && ks == 0) ? *(const f4 *)(a.bias + n) : (f4){0.f, 0.f, 0.f, 0.f};
     const int nrows = min(NT * 16, a.T - tbase);
     for (int tk = wave * TPI + lane / LPR; tk < nrows; tk += kWaves * TPI) {
@@ -995,26 +995,27 @@ static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x_all, int T
     const int chunks = (T + 63) / 64;
     constexpr int R = 2;
     a.n_row_groups = (a.n_row_tiles + 4 * R - 1) / (4 * R);
-    // One chunk of tokens and few row groups: split K so that about every CU
+    // Few row groups and chunks of tokens: split K so that about every CU
     // gets a workgroup, each with at least two super-blocks.
     int ksplit = 1;
-    if (may_slice && chunks == 1) {
-        int want = std::min(16, 256 / a.n_row_groups);
+    a.slice_rows = chunks * 64;
+    if (may_slice) {
+        int want = std::min(16, 256 / (a.n_row_groups * chunks));
         if (g_mm_force_ksplit > 0) want = g_mm_force_ksplit;
         want = std::min(want, nsb / 2);
         if (want > 1) {
             const int per = (nsb + want - 1) / want;
             ksplit = (nsb + per - 1) / per;
         }
-        if ((size_t)ksplit * 64 * w.N * 4 > matmul_workspace_bytes()) {
+        if ((size_t)ksplit * a.slice_rows * w.N * 4 > matmul_workspace_bytes()) {
             if (g_mm_force_ksplit > 0) throw std::runtime_error("matmul_lds: the split does not fit the workspace");
             ksplit = 1;
         }
     }
     a.pld = w.N; a.pcol = 0;
     if (shared) {
-        if (chunks != 1 || shared->ksplit < 2 || shared->ksplit > nsb || (shared->col & 3) || (shared->ld & 3) ||
-            shared->col + w.N > shared->ld || (size_t)shared->ksplit * 64 * shared->ld * 4 > matmul_workspace_bytes())
+        if (shared->ksplit < 2 || shared->ksplit > nsb || (shared->col & 3) || (shared->ld & 3) ||
+            shared->col + w.N > shared->ld || (size_t)shared->ksplit * a.slice_rows * shared->ld * 4 > matmul_workspace_bytes())
             throw std::runtime_error("matmul_lds: the shared slices do not fit this matrix");
         const int per = (nsb + shared->ksplit - 1) / shared->ksplit;
         if ((nsb + per - 1) / per != shared->ksplit) throw std::runtime_error("matmul_lds: the shared slice count leaves an empty slice");
@@ -1026,14 +1027,14 @@ static Slices lds_impl(hipStream_t s, const Weight & w, const Act & x_all, int T
     dispatch_nt<R>(s, w.type, nt, a, grid);
     check_launch("matmul_lds");
     Slices out;
-    if (ksplit > 1) { out.data = a.partial; out.n = ksplit; out.stride = (size_t)64 * a.pld; out.N = a.pld; }
+    if (ksplit > 1) { out.data = a.partial; out.n = ksplit; out.stride = (size_t)a.slice_rows * a.pld; out.N = a.pld; }
     return out;
 }
 
 // Several tiled matrices over the same activations whose outputs sit side by side in y (q, k and v of different
 // storage types): each is launched on its own, all with the same number of K-slices into one set of slices of
 // the full row width, so that the consumer adds them as it would for one fused matrix. Returns no slices (and
-// leaves the results in y) when the step is not a single chunk or K too short to split.
+// leaves the results in y) when the row groups and token chunks already fill the chip or K is too short to split.
 Slices matmul_deferred_parts(hipStream_t s, const Weight * const * parts, int n_parts, const Act & x, int T, float * y,
                              int ldy, const float * bias, void * ws) {
     if (T <= 0 || n_parts <= 0) return Slices();
@@ -1058,14 +1059,14 @@ Slices matmul_deferred_parts(hipStream_t s, const Weight * const * parts, int n_
     }
     const int nsb = K / 256, chunks = (T + 63) / 64;
     int ksplit = 1;
-    if (chunks == 1) {
+    {
         const int groups = (total / 16 + 7) / 8;
-        int want = std::min(std::min(16, 256 / std::max(groups, 1)), nsb / 2);
+        int want = std::min(std::min(16, 256 / std::max(groups * chunks, 1)), nsb / 2);
         if (want > 1) {
             const int per = (nsb + want - 1) / want;
             ksplit = (nsb + per - 1) / per;
         }
-        if ((size_t)ksplit * 64 * total * 4 > matmul_workspace_bytes()) ksplit = 1;
+        if ((size_t)ksplit * chunks * 64 * total * 4 > matmul_workspace_bytes()) ksplit = 1;
     }
     Slices out;
     int col = 0;
@@ -1080,7 +1081,7 @@ Slices matmul_deferred_parts(hipStream_t s, const Weight * const * parts, int n_
         }
         col += parts[i]->N;
     }
-    if (ksplit > 1) { out.data = (const float *)ws; out.n = ksplit; out.stride = (size_t)64 * total; out.N = total; }
+    if (ksplit > 1) { out.data = (const float *)ws; out.n = ksplit; out.stride = (size_t)chunks * 64 * total; out.N = total; }
     return out;
 }
 

@@ -461,21 +461,76 @@ __global__ __launch_bounds__(256) void k_moe_down(MoeArgs a) {
     }
 }
 
+// Router logits on the f32 matrix instruction (32x32x2: exact f32 products, f32 sums): one wave per (32 experts,
+// 32 tokens, 128 columns of K) leaves its sums as a K-slice [slice][token][expert]; k_moe_route adds the slices
+// in slice order. The rows are the f32 router weights, the tokens' values hi + lo of the activation planes.
+typedef float f16v __attribute__((ext_vector_type(16)));
+constexpr int ROUTER_KSLICE = 128;
+__global__ __launch_bounds__(64) void k_moe_router(const float * __restrict__ wm, const __half * __restrict__ x, int K, int N, int T,
+                                                   float * __restrict__ slices) {
+    const int lane = threadIdx.x, j = lane & 31, g = lane >> 5;
+    const int t = min((int)blockIdx.y * 32 + j, T - 1);
+    const float * wr = wm + (size_t)(blockIdx.x * 32 + j) * K;
+    const int k0 = blockIdx.z * ROUTER_KSLICE + 8 * g;
+    f4 wa[8], wb[8];
+    h8 hi[8], lo[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {          // lanes 0-31 take columns 16u .. 16u+7 of the slice, lanes 32-63 the next eight
+        const int k = k0 + 16 * u;
+        wa[u] = *(const f4 *)(wr + k);
+        wb[u] = *(const f4 *)(wr + k + 4);
+        hi[u] = load_h8(x + act_at(t, k, 0, K));
+        lo[u] = load_h8(x + act_at(t, k, 1, K));
+    }
+    f16v acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+        const float w[8] = {wa[u].x, wa[u].y, wa[u].z, wa[u].w, wb[u].x, wb[u].y, wb[u].z, wb[u].w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w[i], (float)hi[u][i] + (float)lo[u][i], acc, 0, 0, 0);
+    }
+    // acc[4 b + i] = expert 8 b + 4 g + i of the tile, token j
+    const int tok = blockIdx.y * 32 + j;
+    if (tok >= T) return;
+    float * dst = slices + ((size_t)blockIdx.z * T + tok) * N + blockIdx.x * 32 + 4 * g;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) *(f4 *)(dst + 8 * b) = (f4){acc[4 * b], acc[4 * b + 1], acc[4 * b + 2], acc[4 * b + 3]};
+}
+
 // Per token: the top-k experts by router logit (ties to the lower index - the
 // order of the softmax probabilities) and their weights renormalised over the
-// selection, exp and the sums in double.
-__global__ __launch_bounds__(64) void k_moe_route(const float * __restrict__ logits, int n_expert, int k_used,
-                                                  int32_t * __restrict__ sel, float * __restrict__ wgt) {
+// selection, exp and the sums in double. The logits are the sum of n_slices
+// K-slices `stride` floats apart, added in slice order.
+__global__ __launch_bounds__(64) void k_moe_route(const float * __restrict__ logits, int n_slices, size_t stride, int n_expert,
+                                                  int k_used, int32_t * __restrict__ sel, float * __restrict__ wgt) {
     const int t = blockIdx.x, lane = threadIdx.x;
     float v[4];
     bool taken[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int e = lane + 64 * i;
-        v[i] = e < n_expert ? logits[(size_t)t * n_expert + e] : -INFINITY;
+        v[i] = e < n_expert ? 0.0f : -INFINITY;
         taken[i] = e >= n_expert;
     }
-    float top_v[16];
+    for (int s0 = 0; s0 < n_slices; s0 += 8) {       // eight slices' loads in flight together, added in slice order
+        float part[8][4];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int e = min(lane + 64 * i, n_expert - 1);
+                part[u][i] = logits[(size_t)min(s0 + u, n_slices - 1) * stride + (size_t)t * n_expert + e];
+            }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (s0 + u < n_slices && lane + 64 * i < n_expert) v[i] = s0 + u == 0 ? part[u][i] : v[i] + part[u][i];
+    }
+    float mine = -INFINITY;       // lane j keeps the j-th largest logit
     float mx = -INFINITY;
     for (int j = 0; j < k_used; ++j) {
         float bv = -INFINITY;
@@ -492,14 +547,14 @@ __global__ __launch_bounds__(64) void k_moe_route(const float * __restrict__ log
         for (int i = 0; i < 4; ++i)
             if (bi == lane + 64 * i) taken[i] = true;
         if (j == 0) mx = bv;
-        top_v[j] = bv;
+        if (lane == j) mine = bv;
         if (lane == 0) sel[(size_t)t * k_used + j] = bi;
     }
-    if (lane == 0) {
-        double p[16], sum = 0.0;
-        for (int j = 0; j < k_used; ++j) { p[j] = exp((double)top_v[j] - (double)mx); sum += p[j]; }
-        for (int j = 0; j < k_used; ++j) wgt[(size_t)t * k_used + j] = (float)(p[j] / sum);
-    }
+    // every lane below k_used its own exp; the sum in selection order, the same in every lane
+    const double p = lane < k_used ? exp((double)mine - (double)mx) : 0.0;
+    double sum = 0.0;
+    for (int j = 0; j < k_used; ++j) sum += __shfl(p, j, 64);
+    if (lane < k_used) wgt[(size_t)t * k_used + lane] = (float)(p / sum);
 }
 
 // Stable counting sort of the pairs by expert, every expert's range padded to a
@@ -601,8 +656,22 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     auto tiled = [](int t) { return t == WT_MXFP4 || t == WT_Q8_0 || t == WT_Q4_K || t == WT_Q5_K || t == WT_Q6_K; };
     if (L.gate.type != L.up.type || !tiled(L.gate.type) || !tiled(L.down.type))
         throw std::runtime_error("moe: expert weights must be MXFP4, Q8_0, Q4_K, Q5_K or Q6_K, gate and up of one type");
-    matmul_generic(s, L.router, xn, T, b.logits, sh.n_expert, 0, MM_STORE, nullptr);
-    hipLaunchKernelGGL(k_moe_route, dim3(T), dim3(64), 0, s, b.logits, sh.n_expert, sh.k_used, b.sel, b.wgt);
+    // The router: f32 rows on the f32 matrix instruction, K split into slices of 128 columns that the selection
+    // adds (the slices borrow the pairs' output rows, which nothing holds yet); any other router by the generic kernel.
+    const Act xr = xn.operand(L.router.type);
+    const int r_slices = sh.E / ROUTER_KSLICE;
+    if (L.router.type == WT_F32 && L.router.raw && ((uintptr_t)L.router.raw & 15) == 0 && xr.x && sh.n_expert % 32 == 0
+        && L.router.K == sh.E && L.router.N == sh.n_expert
+        && (size_t)r_slices * T * sh.n_expert <= moe_slots(T, sh.k_used, sh.n_expert) * (size_t)sh.E) {
+        hipLaunchKernelGGL(k_moe_router, dim3(sh.n_expert / 32, (T + 31) / 32, r_slices), dim3(64), 0, s,
+                           (const float *)L.router.raw, xr.x, sh.E, sh.n_expert, T, b.out_pair);
+        check_launch("moe_router");
+        hipLaunchKernelGGL(k_moe_route, dim3(T), dim3(64), 0, s, b.out_pair, r_slices, (size_t)T * sh.n_expert, sh.n_expert,
+                           sh.k_used, b.sel, b.wgt);
+    } else {
+        matmul_generic(s, L.router, xn, T, b.logits, sh.n_expert, 0, MM_STORE, nullptr);
+        hipLaunchKernelGGL(k_moe_route, dim3(T), dim3(64), 0, s, b.logits, 1, (size_t)0, sh.n_expert, sh.k_used, b.sel, b.wgt);
+    }
     check_launch("moe_route");
     hipLaunchKernelGGL(k_moe_group, dim3(1), dim3(1024), 0, s, b.sel, T * sh.k_used, sh.n_expert, sh.k_used, b.expert_n,
                        b.off_pad, b.tok_of_q, b.q_of_pair);

@@ -388,6 +388,25 @@ def test_split_k_matmul_is_deterministic_and_exact(t):
     assert np.abs(c - (want + y0)).max() <= 3e-5 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0, gw.GGML_Q6_K, gw.GGML_Q5_K])
+@pytest.mark.parametrize("T", [65, 100, 128, 192])
+def test_split_k_matmul_over_several_token_chunks(t, T):
+    # 2048 rows are 16 row groups: at two or three 64-token chunks K is still split across workgroups, every
+    # slice holding all the chunks' rows; the slices are added in slice order.
+    print("case", t, T, flush=True)
+    n, k = 2048, 4096
+    raw, dense = _weights(t, n, k, seed=31 + T)
+    x = np.random.default_rng(T).standard_normal((T, k)).astype(np.float32)
+    want = _ref(t, dense, x, False)
+    a = E.kernel_matmul(t, raw, n, k, x, use_tiles=2)
+    b = E.kernel_matmul(t, raw, n, k, x, use_tiles=2)
+    assert np.array_equal(a, b)
+    assert np.abs(a - want).max() <= 2e-5 * np.abs(want).max()
+    y0 = np.random.default_rng(6).standard_normal((T, n)).astype(np.float32)
+    c = E.kernel_matmul(t, raw, n, k, x, use_tiles=2, accumulate_into=y0)
+    assert np.abs(c - (want + y0)).max() <= 3e-5 * np.abs(want).max()
+
+
 def test_sample_prepare_matches_numpy():
     rng = np.random.default_rng(11)
     V = 5003

@@ -107,8 +107,7 @@ template <> struct Tile<WT_MXFP4> {
     // half of 2^(x - 127): the E8M0 scale of doubled magnitudes
     __device__ __forceinline__ float scale(int s) const {
         const uint32_t x = ((s < 4 ? hdr.x : hdr.y) >> (8 * (s & 3))) & 0xff;
-        const uint32_t bits = x == 0 ? 0x00200000u : (x == 1 ? 0x00400000u : (x - 1) << 23);
-        return __uint_as_float(bits);
+        return __builtin_ldexpf(0.5f, (int)x - 127);      // one instruction; exponents 0 and 1 give the subnormals 2^-128, 2^-127
     }
     __device__ __forceinline__ h8 frag(int s) const {
         const uint32_t w = s < 4 ? q0[s & 3] : q1[s & 3];
@@ -291,20 +290,33 @@ struct MoeArgs {
 constexpr int kStageTile = 8 * 2 * 64 * 16;        // bytes per token tile and super-block
 
 template <int NTMAX> struct StageRegs { u4 v[4 * NTMAX]; };
+// where a thread's 16-byte pieces of super-block 0 lie in the activation buffer (in halves); super-block sb lies
+// kStageStep halves further per step
+template <int NTMAX> struct StageAt { uint32_t off[4 * NTMAX]; };
+constexpr uint32_t kStageStep = 8 * 2 * 4 * 512;
 
 // NTMAX = 1 halves the LDS of a workgroup (more of them per compute unit, more weight bytes in flight) and
 // makes an expert with more than 16 pairs stream its weights once per 16 of them: the host picks it for
 // decode-sized steps. rows[32]: for every row of the (up to) two tiles, the row of the activation buffer it reads.
 template <int NTMAX>
-__device__ __forceinline__ void stage_load(const __half * x, int K, const int * rows, int sb, int nt, StageRegs<NTMAX> & regs) {
+__device__ __forceinline__ void stage_prepare(int K, const int * rows, int nt, StageAt<NTMAX> & at) {
 #pragma unroll
     for (int c = 0; c < 4 * NTMAX; ++c) {
         if (c >= 4 * nt) break;
         const int chunk = c * 256 + threadIdx.x;
         const int t = chunk >> 10, rem = chunk & 1023;
         const int s = rem >> 7, hl = (rem >> 6) & 1, ln = rem & 63;
-        const int k = sb * 256 + s * 32 + 8 * (ln >> 4);
-        regs.v[c] = *(const u4 *)(x + act_at(rows[t * 16 + (ln & 15)], k, hl, K));
+        at.off[c] = (uint32_t)act_at(rows[t * 16 + (ln & 15)], s * 32 + 8 * (ln >> 4), hl, K);
+    }
+}
+
+template <int NTMAX>
+__device__ __forceinline__ void stage_load(const __half * x, const StageAt<NTMAX> & at, int sb, int nt, StageRegs<NTMAX> & regs) {
+    const __half * xs = x + (size_t)sb * kStageStep;
+#pragma unroll
+    for (int c = 0; c < 4 * NTMAX; ++c) {
+        if (c >= 4 * nt) break;
+        regs.v[c] = *(const u4 *)(xs + at.off[c]);
     }
 }
 
@@ -324,8 +336,10 @@ __device__ __forceinline__ h8 staged(const uint8_t * buf, int t, int s, int hl, 
 // One workgroup per (expert, four consecutive tiles of 16 output features), one wave per tile: gate and up
 // tiles together, SwiGLU in the epilogue. The weights of the next super-block and the activations of the next
 // super-block are requested before the current one is multiplied.
+// (Two workgroups fit a CU's LDS, two waves a SIMD: told so, the compiler keeps the products in vector registers
+// instead of parking them in accumulation registers and copying them back.)
 template <int TYPE, int NTMAX>
-__global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_moe_gate_up(MoeArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][NTMAX * kStageTile];
     __shared__ int rows[32];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -350,7 +364,9 @@ __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
         }
         __syncthreads();
         StageRegs<NTMAX> regs;
-        stage_load(a.x.x, a.K, rows, 0, nt, regs);
+        StageAt<NTMAX> at;
+        stage_prepare(a.K, rows, nt, at);
+        stage_load(a.x.x, at, 0, nt, regs);
         Tile<TYPE> tg, tu;
         tg.load(wg, lane);
         tu.load(wu, lane);
@@ -363,7 +379,7 @@ __global__ __launch_bounds__(256) void k_moe_gate_up(MoeArgs a) {
             const bool more = sb + 1 < nsb;
             Tile<TYPE> ng = tg, nu = tu;
             if (more) {
-                stage_load(a.x.x, a.K, rows, sb + 1, nt, regs);
+                stage_load(a.x.x, at, sb + 1, nt, regs);
                 ng.load(wg + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
                 nu.load(wu + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
             }
@@ -427,7 +443,9 @@ void k_moe_down(MoeArgs a) {
         if (threadIdx.x < 32) rows[threadIdx.x] = qb + t0 + ((int)threadIdx.x < 16 * nt ? threadIdx.x : 0);
         __syncthreads();
         StageRegs<NTMAX> regs;
-        stage_load(a.x.x, a.K, rows, 0, nt, regs);
+        StageAt<NTMAX> at;
+        stage_prepare(a.K, rows, nt, at);
+        stage_load(a.x.x, at, 0, nt, regs);
         Tile<TYPE> tw;
         tw.load(wd, lane);
         stage_store(stage[0], nt, regs);
@@ -437,7 +455,7 @@ void k_moe_down(MoeArgs a) {
             const bool more = sb + 1 < nsb;
             Tile<TYPE> nw = tw;
             if (more) {
-                stage_load(a.x.x, a.K, rows, sb + 1, nt, regs);
+                stage_load(a.x.x, at, sb + 1, nt, regs);
                 nw.load(wd + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
             }
             const uint8_t * cur = stage[sb & 1];

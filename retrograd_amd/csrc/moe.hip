@@ -19,10 +19,11 @@
 // Expert tensors [K][N][n_expert] are tiled as one matrix of n_expert * N rows.
 // MXFP4 tile (16 rows x 256 columns, 2176 B = the GGUF byte count): 16 x 8 E8M0
 // scale bytes, then two 1 KiB loads; lane (r = l % 16, g = l / 16) of load h
-// holds one dword per k-step 4h + j: byte b of it carries element 8g + b in its
-// low nibble and element 8g + 4 + b in its high nibble. The doubled E2M1
-// magnitudes 0 1 2 3 4 6 8 12 are f16 numbers whose low byte is zero, so two
-// byte permutes through an 8-byte table decode four weights at a time, exactly.
+// holds one dword per k-step 4h + j: byte b of it carries element 8g + 2b in its
+// low nibble and element 8g + 2b + 1 in its high nibble, the order in which
+// v_cvt_scalef32_pk_f16_fp4 turns a byte into two f16 numbers (exactly; with the
+// factor 2 they are the doubled E2M1 magnitudes 0 1 2 3 4 6 8 12 that ggml's
+// half scale multiplies): four instructions decode a lane's eight weights.
 #include "dev_common.hpp"
 
 namespace rk {
@@ -55,7 +56,7 @@ __global__ void k_repack_mxfp4(const uint8_t * __restrict__ raw, uint8_t * __res
             const uint8_t byte = blk[1 + (e & 15)];
             return e < 16 ? (byte & 0x0f) : (byte >> 4);
         };
-        for (int b = 0; b < 4; ++b) out |= (elem(8 * g + b) | (elem(8 * g + 4 + b) << 4)) << (8 * b);
+        for (int b = 0; b < 4; ++b) out |= (elem(8 * g + 2 * b) | (elem(8 * g + 2 * b + 1) << 4)) << (8 * b);
     }
     *(uint32_t *)(dst + ts * 2176 + (size_t)w * 4) = out;
 }
@@ -111,13 +112,11 @@ template <> struct Tile<WT_MXFP4> {
     }
     __device__ __forceinline__ h8 frag(int s) const {
         const uint32_t w = s < 4 ? q0[s & 3] : q1[s & 3];
-        // high bytes of the f16 numbers 0 1 2 3 | 4 6 8 12, chosen by the 3-bit magnitude; bit 3 is the sign
-        const uint32_t lo = __builtin_amdgcn_perm(0x4A484644u, 0x42403C00u, w & 0x07070707u) | ((w & 0x08080808u) << 4);
-        const uint32_t hi = __builtin_amdgcn_perm(0x4A484644u, 0x42403C00u, (w >> 4) & 0x07070707u) | (w & 0x80808080u);
-        const h2 p0 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0u, lo, 0x010C000Cu));
-        const h2 p1 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0u, lo, 0x030C020Cu));
-        const h2 p2 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0u, hi, 0x010C000Cu));
-        const h2 p3 = __builtin_bit_cast(h2, __builtin_amdgcn_perm(0u, hi, 0x030C020Cu));
+        // byte b: (low nibble, high nibble) -> the doubled magnitudes of elements 2b, 2b + 1
+        const h2 p0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 2.0f, 0);
+        const h2 p1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 2.0f, 1);
+        const h2 p2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 2.0f, 2);
+        const h2 p3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 2.0f, 3);
         return (h8){p0.x, p0.y, p1.x, p1.y, p2.x, p2.y, p3.x, p3.y};
     }
     __device__ __forceinline__ ScaledOperand prep(int s) const { return {frag(s), scale(s)}; }

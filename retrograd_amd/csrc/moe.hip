@@ -417,10 +417,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 // One workgroup per (expert, four consecutive tiles of 16 output features of the model width), one wave per
 // tile; the hidden rows of the expert's pairs are staged like the activations above.
+constexpr int down_waves(int type, int ntmax) {
+    return ntmax != 1 ? 2 : (type == WT_MXFP4 || type == WT_Q8_0 ? 4 : (type == WT_Q6_K ? 3 : 2));
+}
 // (One token tile of MXFP4 or Q8_0 weights fits 128 registers without spilling: four waves a SIMD instead of the
-// three the compiler settles for; measured 40.6 -> 37.6 us per layer at the 128-expert shape.)
+// three the compiler settles for; measured 40.6 -> 37.6 us per layer at the 128-expert shape. Q6_K fits three; everything else
+// runs two waves a SIMD and may use their 256 registers, which keeps the products out of the accumulation registers.)
 template <int TYPE, int NTMAX>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NTMAX == 1 && (TYPE == WT_MXFP4 || TYPE == WT_Q8_0) ? 4 : 1)))
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(down_waves(TYPE, NTMAX), down_waves(TYPE, NTMAX))))
 void k_moe_down(MoeArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][NTMAX * kStageTile];
     __shared__ int rows[32];

@@ -464,6 +464,7 @@ void Engine::build_buffers() {
         moe_n_.alloc((size_t)NE * 4);
         moe_off_.alloc((size_t)(NE + 1) * 4);
         moe_tok_.alloc(slots * 4);
+        moe_pair_.alloc(slots * 4);
         moe_q_.alloc((size_t)B * KU * 4);
         moe_h_.alloc(rk::act_halves((int)slots, FE) * 2);
         hip_check(hipMemsetAsync(moe_h_.ptr, 0, moe_h_.bytes, stream_), "hipMemsetAsync");
@@ -1529,8 +1530,8 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
                               rk::Act{moe_h_.as<__half>(), nullptr, h.n_ff_exp}, moe_out_.as<float>()};
             mb.mx_ops = moe_mx_ops_.as<uint8_t>(); mb.mx_scales = moe_mx_scales_.as<uint8_t>(); mb.mx_h = moe_mx_h_.as<float>();
             mb.mx_slots = moe_mx_slots_;
-            rk::moe_ffn(stream_, ml, ms, act_e, T, x, mb);
-            pending = rk::Slices();
+            mb.pair_of_q = moe_pair_.as<int32_t>();
+            pending = rk::moe_ffn(stream_, ml, ms, act_e, T, x, mb, true);     // the next norm adds the experts' weighted sum
             prof_end(PC_GATEUP, pt_);
             continue;
         }

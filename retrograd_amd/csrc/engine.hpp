@@ -320,7 +320,7 @@ private:
     DevBuf item_meta_;        // the step's attention work items (PackBuffers::item_a, item_b), grown as needed
     DevBuf mm_ws_;            // matmul workspace: split-K partials, counters
     // mixture-of-experts scratch (allocated for MoE models only)
-    DevBuf moe_logits_, moe_sel_, moe_wgt_, moe_n_, moe_off_, moe_tok_, moe_q_, moe_h_, moe_out_;
+    DevBuf moe_logits_, moe_sel_, moe_wgt_, moe_n_, moe_off_, moe_tok_, moe_q_, moe_h_, moe_out_, moe_pair_;
     HostPinned h_sample_, h_logits_;
     int last_n_out_ = 0;
 

@@ -996,7 +996,16 @@ __global__ __launch_bounds__(256) void k_rmsnorm_act(float * x, const float * __
     for (int i = threadIdx.x; i < E; i += 256) {
         float v = xr[i];
         if (add.n > 0) {
-            for (int k = 0; k < add.n; ++k) v += add.data[(size_t)k * add.stride + (size_t)row * E + i];
+            if (add.weight) {
+                float c = 0.0f;
+                for (int k = 0; k < add.n; ++k) {
+                    const size_t term = (size_t)row * add.n + k;
+                    c = fmaf(add.weight[term], add.data[(add.gather ? (size_t)add.gather[term] : term) * E + i], c);
+                }
+                v += c;
+            } else {
+                for (int k = 0; k < add.n; ++k) v += add.data[(size_t)k * add.stride + (size_t)row * E + i];
+            }
             xr[i] = v;          // re-read below by the same thread
         }
         ss += v * v;
@@ -1040,7 +1049,34 @@ __global__ __launch_bounds__(NW * 64) void k_rmsnorm_act8(float * x, const float
     int c = 0;
     for (int k = threadIdx.x * 8; k < E; k += STEP, ++c) {
         f4 a = *(const f4 *)(xr + k), b = *(const f4 *)(xr + k + 4);
-        if (add.n > 0) {
+        if (add.n > 0 && add.weight) {
+            // the weighted sum of the row's terms, eight terms' loads in flight together
+            f4 ca = {0.f, 0.f, 0.f, 0.f}, cb = {0.f, 0.f, 0.f, 0.f};
+            const size_t term0 = (size_t)row * add.n;
+            const float * gw = add.weight + term0;
+            for (int j = 0; j < add.n; j += 8) {
+                f4 sa[8], sb[8];
+                float wj[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int jj = min(j + u, add.n - 1);
+                    const float * src = add.data + (add.gather ? (size_t)add.gather[term0 + jj] : term0 + jj) * E + k;
+                    wj[u] = gw[jj];
+                    sa[u] = *(const f4 *)src;
+                    sb[u] = *(const f4 *)(src + 4);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (j + u >= add.n) break;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { ca[i] = fmaf(wj[u], sa[u][i], ca[i]); cb[i] = fmaf(wj[u], sb[u][i], cb[i]); }
+                }
+            }
+            a += ca;
+            b += cb;
+            *(f4 *)(xr + k) = a;
+            *(f4 *)(xr + k + 4) = b;
+        } else if (add.n > 0) {
             const float * sl = add.data + (size_t)row * E + k;
             int j = 0;
             for (; j + 8 <= add.n; j += 8) {          // eight slices' loads in flight together, added in slice order

@@ -122,6 +122,11 @@ struct Slices {
     int n = 0;
     size_t stride = 0;
     int N = 0;
+    // or (weight != null) a weighted sum of n rows per row: term j of row t is weight[t n + j] * data[t n + j][:] - or
+    // data[gather[t n + j]][:] with a gather list - the terms added with fused multiply-adds in order j, their sum added
+    // to the row (what k_moe_combine computes)
+    const float * weight = nullptr;
+    const int32_t * gather = nullptr;
 };
 // y[t][col0 + n] (=|+=) sum_k W[n][k] * x[t][k] (+ bias[n]); y has row stride ldy.
 // `ws` is a device workspace of matmul_workspace_bytes() that selects the
@@ -265,10 +270,14 @@ struct MoeBuffers {            // device scratch of one step, sized with moe_slo
     uint8_t * mx_scales = nullptr;
     float * mx_h = nullptr;
     size_t mx_slots = 0;
+    int32_t * pair_of_q = nullptr;   // [slots] the pair (token * k_used + choice) of a slot, -1 for padding; or null: then the
+                                     // down projection leaves its rows in slot order instead of pair order
 };
 size_t moe_slots(int n_tokens, int k_used, int n_expert);
 // x[t] += sum over the token's k_used experts of w * down_e(silu(gate_e xn) * (up_e xn))
-void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act & xn, int T, float * x, const MoeBuffers & b);
+// With defer_combine the weighted sum is not added to x: it is returned as gathered slices for the next rmsnorm_act.
+Slices moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act & xn, int T, float * x, const MoeBuffers & b,
+               bool defer_combine = false);
 
 // x[t][:] = decode(raw row tok[t]) as f32.
 void embed(hipStream_t s, const Weight & emb, const int32_t * tok, int T, float * x);

@@ -14,7 +14,8 @@
 //   k_moe_group     stable counting sort of the pairs by expert (one workgroup)
 //   k_moe_gate_up   h[q][f] = silu(gate_e x) * (up_e x)       q = slot of a pair
 //   k_moe_down      out[q][:] = down_e h[q]
-//   k_moe_combine   x[t] += sum_j w[t][j] * out[q(t, j)]       in choice order
+//   k_moe_combine   x[t] += sum_j w[t][j] * out[q(t, j)]       in choice order (in the engine's steps the next
+//                   RMSNorm launch adds this sum instead: k_moe_down leaves its rows in pair order for it)
 //
 // Expert tensors [K][N][n_expert] are tiled as one matrix of n_expert * N rows.
 // MXFP4 tile (16 rows x 256 columns, 2176 B = the GGUF byte count): 16 x 8 E8M0
@@ -279,6 +280,7 @@ struct MoeArgs {
     const int32_t * expert_n;  // pairs per expert
     const int32_t * off_pad;   // first slot of each expert (multiples of 16)
     const int32_t * tok_of_q;  // token of a slot, -1 for padding
+    const int32_t * pair_of_q; // down: the output row of a slot (its pair), or null: the slot itself
     int n_expert, K, N;        // N output features per expert, K inputs
 };
 
@@ -427,7 +429,7 @@ template <int TYPE, int NTMAX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(down_waves(TYPE, NTMAX), down_waves(TYPE, NTMAX))))
 void k_moe_down(MoeArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][NTMAX * kStageTile];
-    __shared__ int rows[32];
+    __shared__ int rows[32], out_rows[32];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, g = lane >> 4;
     const int n_tiles = a.N / 16;
@@ -443,7 +445,11 @@ void k_moe_down(MoeArgs a) {
         const int nt = (NTMAX == 2 && n_e - t0 > 16) ? 2 : 1;
         __syncthreads();
         // every row of a tile lies in the expert's padded slot range
-        if (threadIdx.x < 32) rows[threadIdx.x] = qb + t0 + ((int)threadIdx.x < 16 * nt ? threadIdx.x : 0);
+        if (threadIdx.x < 32) {
+            const int slot = qb + t0 + ((int)threadIdx.x < 16 * nt ? threadIdx.x : 0);
+            rows[threadIdx.x] = slot;
+            out_rows[threadIdx.x] = a.pair_of_q && t0 + (int)threadIdx.x < n_e ? a.pair_of_q[slot] : slot;
+        }
         __syncthreads();
         StageRegs<NTMAX> regs;
         StageAt<NTMAX> at;
@@ -480,7 +486,7 @@ void k_moe_down(MoeArgs a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int at = t0 + t * 16 + 4 * g + i;
-                if (t < nt && at < n_e) a.out_pair[(size_t)(qb + at) * a.N + et * 16 + r16] = acc[t][i];
+                if (t < nt && at < n_e) a.out_pair[(size_t)out_rows[t * 16 + 4 * g + i] * a.N + et * 16 + r16] = acc[t][i];
             }
     }
 }
@@ -585,7 +591,8 @@ __global__ __launch_bounds__(64) void k_moe_route(const float * __restrict__ log
 // multiple of 16 slots. One workgroup of 1024 threads.
 __global__ __launch_bounds__(1024) void k_moe_group(const int32_t * __restrict__ sel, int n_pairs, int n_expert, int k_used,
                                                     int32_t * __restrict__ expert_n, int32_t * __restrict__ off_pad,
-                                                    int32_t * __restrict__ tok_of_q, int32_t * __restrict__ q_of_pair) {
+                                                    int32_t * __restrict__ tok_of_q, int32_t * __restrict__ q_of_pair,
+                                                    int32_t * __restrict__ pair_of_q) {
     __shared__ int cnt[256];
     __shared__ int base[256];
     __shared__ int wcnt[16][256];
@@ -641,6 +648,7 @@ __global__ __launch_bounds__(1024) void k_moe_group(const int32_t * __restrict__
             for (int w = 0; w < wave; ++w) pos += wcnt[w][e];
             q_of_pair[p] = pos;
             tok_of_q[pos] = p / k_used;
+            if (pair_of_q) pair_of_q[pos] = p;
         }
         __syncthreads();
         if (tid < n_expert) {
@@ -672,8 +680,23 @@ size_t moe_slots(int n_tokens, int k_used, int n_expert) {
     return ((size_t)n_tokens * k_used + (size_t)16 * n_expert + 63) / 64 * 64;
 }
 
-void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act & xn, int T, float * x, const MoeBuffers & b) {
-    if (T <= 0) return;
+Slices moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act & xn, int T, float * x, const MoeBuffers & b,
+               bool defer_combine) {
+    if (T <= 0) return Slices();
+    // the weighted sum over a token's experts: added to x here, or left to the next RMSNorm launch as gathered slices
+    auto combine = [&](bool pair_order) -> Slices {
+        if (defer_combine) {
+            Slices sl;
+            sl.data = b.out_pair; sl.n = sh.k_used; sl.N = sh.E; sl.weight = b.wgt;
+            sl.gather = pair_order ? nullptr : b.q_of_pair;
+            return sl;
+        }
+        if (pair_order) throw std::runtime_error("moe: rows in pair order are combined by the next RMSNorm");
+        hipLaunchKernelGGL(k_moe_combine, dim3(T, (sh.E / 4 + 255) / 256), dim3(256), 0, s, b.out_pair, b.q_of_pair, b.wgt,
+                           sh.k_used, sh.E, x);
+        check_launch("moe_combine");
+        return Slices();
+    };
     if (sh.n_expert > 256 || sh.k_used > 16 || sh.k_used > sh.n_expert) throw std::runtime_error("moe: unsupported expert count");
     // multiples of 256: whole super-blocks along K, and the four waves of a workgroup share an expert (N / 16 % 4 == 0)
     if (sh.E % 256 != 0 || sh.F % 256 != 0) throw std::runtime_error("moe: widths must be multiples of 256");
@@ -698,7 +721,7 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     }
     check_launch("moe_route");
     hipLaunchKernelGGL(k_moe_group, dim3(1), dim3(1024), 0, s, b.sel, T * sh.k_used, sh.n_expert, sh.k_used, b.expert_n,
-                       b.off_pad, b.tok_of_q, b.q_of_pair);
+                       b.off_pad, b.tok_of_q, b.q_of_pair, b.pair_of_q);
     check_launch("moe_group");
     MoeArgs a {};
     a.expert_n = b.expert_n; a.off_pad = b.off_pad; a.tok_of_q = b.tok_of_q; a.n_expert = sh.n_expert;
@@ -717,10 +740,7 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
                         b.mx_scales, b.mx_h);
         mxe_moe_down(s, L.down.records, b.mx_h, sh.E, sh.F, sh.n_expert, b.off_pad, b.tok_of_q, slots, b.mx_ops, b.mx_scales,
                      b.out_pair);
-        hipLaunchKernelGGL(k_moe_combine, dim3(T, (sh.E / 4 + 255) / 256), dim3(256), 0, s, b.out_pair, b.q_of_pair, b.wgt,
-                           sh.k_used, sh.E, x);
-        check_launch("moe_combine");
-        return;
+        return combine(false);
     }
     // (measured on the 128-expert shape at 128 rows: the down projection gains a fifth from the smaller
     // workgroups, gate/up - two weight tiles per wave - loses a tenth, so it keeps two tiles)
@@ -739,6 +759,8 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
         requant_act(s, b.h.x, (int)moe_slots(T, sh.k_used, sh.n_expert), hq);
     }
     a.w0 = L.down.packed; a.w1 = nullptr; a.x = b.h; a.out_pair = b.out_pair; a.K = sh.F; a.N = sh.E;
+    // deferred: the rows leave in pair order, so that the norm reads a token's rows without looking up their slots
+    a.pair_of_q = defer_combine ? b.pair_of_q : nullptr;
     const unsigned d_blocks = (unsigned)(((size_t)sh.n_expert * (sh.E / 16) + 3) / 4);
 #define RK_MOE_DOWN(TYPE)                                                                                        \
     do {                                                                                                         \
@@ -754,9 +776,7 @@ void moe_ffn(hipStream_t s, const MoeLayer & L, const MoeShape & sh, const Act &
     }
 #undef RK_MOE_DOWN
     check_launch("moe_down");
-    hipLaunchKernelGGL(k_moe_combine, dim3(T, (sh.E / 4 + 255) / 256), dim3(256), 0, s, b.out_pair, b.q_of_pair, b.wgt,
-                       sh.k_used, sh.E, x);
-    check_launch("moe_combine");
+    return combine(a.pair_of_q != nullptr);
 }
 
 }  // namespace rk

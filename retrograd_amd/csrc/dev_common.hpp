@@ -210,6 +210,21 @@ __device__ __forceinline__ void store_act8(const float (&v)[8], const Act & out,
     }
 }
 
+// A direct-to-LDS request issued from inline assembly. The compiler's own wait
+// insertion cannot tell which staging buffer an LDS read touches, so with the
+// builtin it waits for every request (and, loads retiring in order, for every
+// weight load before it) ahead of each barrier: s_waitcnt vmcnt(0) per
+// super-block, the whole latency of the weight prefetch exposed. Requests it
+// does not see leave only the waits written in the kernels. M0 carries the LDS
+// address. base is wave-uniform; every lane adds its own byte offset.
+__device__ __forceinline__ void lds_dma16(const void * base, uint32_t lane_off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_off), "s"(base), "s"(lds_addr) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_offset(const void * p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p;
+}
+
 struct MMArgs {
     const uint8_t * w;
     const __half * x;         // operand-order activations and block sums (see Act)

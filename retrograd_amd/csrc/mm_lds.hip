@@ -35,17 +35,6 @@ namespace {
 constexpr int kWaves = 8;      // 4 row waves x 2 halves of every super-block
 constexpr int kThreads = kWaves * 64;
 
-// A direct-to-LDS request issued from inline assembly. The compiler's own wait
-// insertion cannot tell which staging buffer an LDS read touches, so with the
-// builtin it waits for every request (and, loads retiring in order, for every
-// weight load before it) ahead of each barrier: s_waitcnt vmcnt(0) per
-// super-block, the whole latency of the weight prefetch exposed. Requests it
-// does not see leave only the waits written in the kernels. M0 carries the LDS
-// address. base is wave-uniform; every lane adds its own byte offset.
-__device__ __forceinline__ void lds_dma16(const void * base, uint32_t lane_off, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :: "v"(lane_off), "s"(base), "s"(lds_addr) : "memory");
-}
 // In the general kernels the weight loads are loads the compiler knows: a load issued from
 // inline assembly hands the compiler a register whose value arrives later, and
 // any copy the register allocator makes of it before the wait (one was seen at
@@ -68,9 +57,6 @@ __device__ __forceinline__ u2 load8(WeightRows rows, uint32_t lane_off, uint32_t
 }
 __device__ __forceinline__ uint32_t load4(WeightRows rows, uint32_t lane_off, uint32_t uniform_off) {
     return __builtin_amdgcn_raw_buffer_load_b32(rows, (int)lane_off, (int)uniform_off, 0);
-}
-__device__ __forceinline__ uint32_t lds_offset(const void * p) {
-    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t *)p;
 }
 
 template <int NT> struct XStage {

@@ -343,7 +343,7 @@ template <int TYPE, int NTMAX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_moe_gate_up(MoeArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][NTMAX * kStageTile];
     __shared__ int rows[32];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, g = lane >> 4;
     const int n_tiles = a.N / 16;
     const int item0 = blockIdx.x * 4;
@@ -364,30 +364,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             rows[threadIdx.x] = tk < 0 ? 0 : tk;        // padding rows read token 0 and are never stored
         }
         __syncthreads();
-        StageRegs<NTMAX> regs;
         StageAt<NTMAX> at;
         stage_prepare(a.K, rows, nt, at);
-        stage_load(a.x.x, at, 0, nt, regs);
-        Tile<TYPE> tg, tu;
-        tg.load(wg, lane);
-        tu.load(wu, lane);
-        stage_store(stage[0], nt, regs);
-        __syncthreads();
         f4 ag[2], au[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) { ag[t] = (f4){0.f, 0.f, 0.f, 0.f}; au[t] = (f4){0.f, 0.f, 0.f, 0.f}; }
-        for (int sb = 0; sb < nsb; ++sb) {
-            const bool more = sb + 1 < nsb;
-            Tile<TYPE> ng = tg, nu = tu;
-            if (more) {
-                stage_load(a.x.x, at, sb + 1, nt, regs);
-                ng.load(wg + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
-                nu.load(wu + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
-            }
+        auto multiply = [&](int sb, const Tile<TYPE> & cg, const Tile<TYPE> & cu) __attribute__((always_inline)) {
             const uint8_t * cur = stage[sb & 1];
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
-                const auto og = tg.prep(s), ou = tu.prep(s);
+                const auto og = cg.prep(s), ou = cu.prep(s);
 #pragma unroll
                 for (int t = 0; t < NTMAX; ++t) {
                     if (t >= nt) break;
@@ -396,10 +382,70 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     mac(ou, hi, lo, au[t]);
                 }
             }
-            if (more) stage_store(stage[(sb + 1) & 1], nt, regs);
+        };
+        if constexpr (TYPE == WT_MXFP4) {
+            // The small tiles are multiplied faster than a request returns: the activations go global -> LDS directly
+            // (no registers, no store phase), the weights are requested two super-blocks ahead into three sets in
+            // rotation, and the waits are written here - the compiler does not see the direct requests, and its own
+            // waits for the weight loads it does see come after these and find them done. A wave's requests return in
+            // order: at the top of super-block sb everything but the six loads of set sb + 1 must have landed.
+            const uint32_t lds0 = lds_offset(&stage[0][0]);
+            auto request_x = [&](int sb) __attribute__((always_inline)) {
+                const __half * xs = a.x.x + (size_t)sb * kStageStep;
+#pragma unroll
+                for (int c = 0; c < 4 * NTMAX; ++c) {
+                    if (c >= 4 * nt) break;
+                    lds_dma16(xs, at.off[c] * 2u, lds0 + (uint32_t)(sb & 1) * (NTMAX * kStageTile) + (uint32_t)(c * 256 + wave * 64) * 16u);
+                }
+            };
+            auto request_w = [&](int sb, Tile<TYPE> & tg, Tile<TYPE> & tu) __attribute__((always_inline)) {
+                const size_t o = (size_t)min(sb, nsb - 1) * Tile<TYPE>::BYTES;
+                tg.load(wg + o, lane);
+                tu.load(wu + o, lane);
+            };
+            Tile<TYPE> g0, u0, g1, u1, g2, u2;
+            request_x(0);
+            request_w(0, g0, u0);
+            __builtin_amdgcn_sched_barrier(0);
+            request_w(1, g1, u1);
+            __builtin_amdgcn_sched_barrier(0);
+            auto body = [&](int sb, Tile<TYPE> & cg, Tile<TYPE> & cu, Tile<TYPE> & fg, Tile<TYPE> & fu) __attribute__((always_inline)) {
+                __builtin_amdgcn_s_waitcnt(0x0F70 | 6);
+                asm volatile("" : "+v"(cg.hdr.x), "+v"(cg.hdr.y), "+v"(cg.q0), "+v"(cg.q1), "+v"(cu.hdr.x), "+v"(cu.hdr.y), "+v"(cu.q0), "+v"(cu.q1));
+                __syncthreads();           // every wave's part of super-block sb is in LDS, and none still reads the other buffer
+                if (sb + 1 < nsb) request_x(sb + 1);
+                request_w(sb + 2, fg, fu);
+                __builtin_amdgcn_sched_barrier(0);
+                if (sb >= nsb) return;     // past the end: the round of three is only kept whole
+                multiply(sb, cg, cu);
+            };
+            for (int sb = 0; sb < nsb; sb += 3) {
+                body(sb, g0, u0, g2, u2);
+                body(sb + 1, g1, u1, g0, u0);
+                body(sb + 2, g2, u2, g1, u1);
+            }
+        } else {
+            StageRegs<NTMAX> regs;
+            stage_load(a.x.x, at, 0, nt, regs);
+            Tile<TYPE> tg, tu;
+            tg.load(wg, lane);
+            tu.load(wu, lane);
+            stage_store(stage[0], nt, regs);
             __syncthreads();
-            tg = ng;
-            tu = nu;
+            for (int sb = 0; sb < nsb; ++sb) {
+                const bool more = sb + 1 < nsb;
+                Tile<TYPE> ng = tg, nu = tu;
+                if (more) {
+                    stage_load(a.x.x, at, sb + 1, nt, regs);
+                    ng.load(wg + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
+                    nu.load(wu + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
+                }
+                multiply(sb, tg, tu);
+                if (more) stage_store(stage[(sb + 1) & 1], nt, regs);
+                __syncthreads();
+                tg = ng;
+                tu = nu;
+            }
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -430,7 +476,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(down_waves(
 void k_moe_down(MoeArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t stage[2][NTMAX * kStageTile];
     __shared__ int rows[32], out_rows[32];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, g = lane >> 4;
     const int n_tiles = a.N / 16;
     const int item0 = blockIdx.x * 4;
@@ -451,35 +497,75 @@ void k_moe_down(MoeArgs a) {
             out_rows[threadIdx.x] = a.pair_of_q && t0 + (int)threadIdx.x < n_e ? a.pair_of_q[slot] : slot;
         }
         __syncthreads();
-        StageRegs<NTMAX> regs;
         StageAt<NTMAX> at;
         stage_prepare(a.K, rows, nt, at);
-        stage_load(a.x.x, at, 0, nt, regs);
-        Tile<TYPE> tw;
-        tw.load(wd, lane);
-        stage_store(stage[0], nt, regs);
-        __syncthreads();
         f4 acc[2] = {(f4){0.f, 0.f, 0.f, 0.f}, (f4){0.f, 0.f, 0.f, 0.f}};
-        for (int sb = 0; sb < nsb; ++sb) {
-            const bool more = sb + 1 < nsb;
-            Tile<TYPE> nw = tw;
-            if (more) {
-                stage_load(a.x.x, at, sb + 1, nt, regs);
-                nw.load(wd + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
-            }
+        auto multiply = [&](int sb, const Tile<TYPE> & cw) __attribute__((always_inline)) {
             const uint8_t * cur = stage[sb & 1];
 #pragma unroll
             for (int s = 0; s < 8; ++s) {
-                const auto ow = tw.prep(s);
+                const auto ow = cw.prep(s);
 #pragma unroll
                 for (int t = 0; t < NTMAX; ++t) {
                     if (t >= nt) break;
                     mac(ow, staged(cur, t, s, 0, lane), staged(cur, t, s, 1, lane), acc[t]);
                 }
             }
-            if (more) stage_store(stage[(sb + 1) & 1], nt, regs);
+        };
+        if constexpr (TYPE == WT_MXFP4) {
+            // (as in k_moe_gate_up: direct requests into LDS, three weight sets, the waits written here; a set is three loads)
+            const uint32_t lds0 = lds_offset(&stage[0][0]);
+            auto request_x = [&](int sb) __attribute__((always_inline)) {
+                const __half * xs = a.x.x + (size_t)sb * kStageStep;
+#pragma unroll
+                for (int c = 0; c < 4 * NTMAX; ++c) {
+                    if (c >= 4 * nt) break;
+                    lds_dma16(xs, at.off[c] * 2u, lds0 + (uint32_t)(sb & 1) * (NTMAX * kStageTile) + (uint32_t)(c * 256 + wave * 64) * 16u);
+                }
+            };
+            auto request_w = [&](int sb, Tile<TYPE> & tw) __attribute__((always_inline)) {
+                tw.load(wd + (size_t)min(sb, nsb - 1) * Tile<TYPE>::BYTES, lane);
+            };
+            Tile<TYPE> w0, w1, w2;
+            request_x(0);
+            request_w(0, w0);
+            __builtin_amdgcn_sched_barrier(0);
+            request_w(1, w1);
+            __builtin_amdgcn_sched_barrier(0);
+            auto body = [&](int sb, Tile<TYPE> & cw, Tile<TYPE> & fw) __attribute__((always_inline)) {
+                __builtin_amdgcn_s_waitcnt(0x0F70 | 3);
+                asm volatile("" : "+v"(cw.hdr.x), "+v"(cw.hdr.y), "+v"(cw.q0), "+v"(cw.q1));
+                __syncthreads();
+                if (sb + 1 < nsb) request_x(sb + 1);
+                request_w(sb + 2, fw);
+                __builtin_amdgcn_sched_barrier(0);
+                if (sb >= nsb) return;
+                multiply(sb, cw);
+            };
+            for (int sb = 0; sb < nsb; sb += 3) {
+                body(sb, w0, w2);
+                body(sb + 1, w1, w0);
+                body(sb + 2, w2, w1);
+            }
+        } else {
+            StageRegs<NTMAX> regs;
+            stage_load(a.x.x, at, 0, nt, regs);
+            Tile<TYPE> tw;
+            tw.load(wd, lane);
+            stage_store(stage[0], nt, regs);
             __syncthreads();
-            tw = nw;
+            for (int sb = 0; sb < nsb; ++sb) {
+                const bool more = sb + 1 < nsb;
+                Tile<TYPE> nw = tw;
+                if (more) {
+                    stage_load(a.x.x, at, sb + 1, nt, regs);
+                    nw.load(wd + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
+                }
+                multiply(sb, tw);
+                if (more) stage_store(stage[(sb + 1) & 1], nt, regs);
+                __syncthreads();
+                tw = nw;
+            }
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t)

@@ -2397,6 +2397,14 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
     // A wave without pages requests page 0 and never looks at it: with a branch around the request the waits
     // below could not tell the two paths apart and would wait for everything.
     load_k_page(pid0, kA);
+    // ... and its V page behind it (the pages of a wave are attended with the next page's K and V in flight)
+    auto load_v_page = [&](int pid, VSet & vs) {
+        const __half * vp = a.v_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) vs.r[d] = load_h8(vp + (d * 64 + lane) * 8);
+    };
+    VSet vA;
+    load_v_page(pid0, vA);
     asm volatile("" : : : "memory");
     // The column values are first looked at here: left alone, the compiler adds a turn's first slices right behind
     // their loads (to reuse the registers) and so waits a trip to memory per turn before it requests the next.
@@ -2535,12 +2543,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
 #pragma unroll
     for (int d = 0; d < DT; ++d) o[d] = (f4){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.0f;
-    auto load_v = [&](int idx, VSet & vs) {
-        const int pid = __builtin_amdgcn_readlane(my_pid, idx);
-        const __half * vp = a.v_pool + (size_t)pid * a.page_stride + (size_t)h * a.head_stride;
-#pragma unroll
-        for (int d = 0; d < DT; ++d) vs.r[d] = load_h8(vp + (d * 64 + lane) * 8);
-    };
+    auto load_v = [&](int idx, VSet & vs) { load_v_page(__builtin_amdgcn_readlane(my_pid, idx), vs); };
     auto attend = [&](int pi, const KSet & ks, const VSet & vs, bool newest) {
         h8 kreg[KS][2], vreg[DT];
 #pragma unroll
@@ -2620,19 +2623,19 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
 #pragma unroll
         for (int d = 0; d < DT; ++d) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vreg[d], pt, o[d], 0, 0, 0);
     };
-    // V of a page loads while its scores are computed, K of the next page (never skipped: past the end the last
-    // page again, so that the number of loads in flight is the same on every path) while the page is multiplied
+    // K and V of the next page load while a page is attended (never skipped: past the end the last page again, so
+    // that the number of loads in flight is the same on every path)
     if (my_n > 0) {
         KSet kB;
-        VSet v;
+        VSet vB;
         for (int i = 0; i < my_n; i += 2) {
-            load_v(i, v);
             load_k(min(i + 1, my_n - 1), kB);
-            attend(my_first + i, kA, v, owner && i == my_n - 1);
+            load_v(min(i + 1, my_n - 1), vB);
+            attend(my_first + i, kA, vA, owner && i == my_n - 1);
             if (i + 1 >= my_n) break;
-            load_v(i + 1, v);
             load_k(min(i + 2, my_n - 1), kA);
-            attend(my_first + i + 1, kB, v, owner && i + 1 == my_n - 1);
+            load_v(min(i + 2, my_n - 1), vA);
+            attend(my_first + i + 1, kB, vB, owner && i + 1 == my_n - 1);
         }
     }
     if (stamp) stamp[2] = wall_clock64();

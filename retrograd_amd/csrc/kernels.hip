@@ -2427,24 +2427,37 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
             y = a.qkv[(size_t)t * ROW + partner];
         }
     };
-    // the columns' sums in slice order
+    // The columns' sums in slice order. One branch around all turns, not one per turn: where the two paths meet the
+    // compiler treats the other path's loads as possibly in flight, and a meeting point per turn made every turn
+    // wait for everything requested so far - the wave's first K and V page included.
     float xv[TURNS], yv[TURNS];
+    if (fast) {
 #pragma unroll
-    for (int u = 0; u < TURNS; ++u) {
-        const int idx = threadIdx.x + u * NT;
-        float x = 0.0f, y = 0.0f;
-        if (fast) {
+        for (int u = 0; u < TURNS; ++u) {
+            float x = 0.0f, y = 0.0f;
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 x += k < a.from.n ? xs[u][k] : 0.0f;
                 y += k < a.from.n ? ys[u][k] : 0.0f;
             }
-        } else if (idx < n_cols) {
-            int col, partner, hh, d;
-            place(idx, col, partner, hh, d);
-            column_pair(col, partner, x, y);
+            xv[u] = x; yv[u] = y;
         }
-        xv[u] = x; yv[u] = y;
+    } else {
+#pragma unroll
+        for (int u = 0; u < TURNS; ++u) {
+            const int idx = threadIdx.x + u * NT;
+            float x = 0.0f, y = 0.0f;
+            if (idx < n_cols) {
+                int col, partner, hh, d;
+                place(idx, col, partner, hh, d);
+                column_pair(col, partner, x, y);
+            }
+            xv[u] = x; yv[u] = y;
+        }
+        // (this path's loads land before the paths meet: a load that could still be in flight into a register the
+        // other path writes would make that path wait for every request before it)
+#pragma unroll
+        for (int u = 0; u < TURNS; ++u) asm volatile("" : "+v"(xv[u]), "+v"(yv[u]));
     }
     // Architectures that normalise the q and k rows per head (RMSNorm over the head's dims, before the rotation): a
     // head's columns sit in consecutive threads of one turn - one wave for 64 dims, an even and an odd wave for 128 -

@@ -2352,7 +2352,7 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
     constexpr int TURNS = (10 * HD + NT - 1) / NT;          // G <= 8
     const int n_cols = (a.G + 2) * HD;
     const bool fast = a.from.n >= 1 && a.from.n <= 4;
-    float xs[TURNS][4], ys[TURNS][4], cvs[TURNS], svs[TURNS];
+    float xs[TURNS][4], ys[TURNS][4], cvs[TURNS], svs[TURNS], nxs[TURNS], nys[TURNS];
     const float * cs = a.rope_cos + (size_t)t * (HD / 2), * sn = a.rope_sin + (size_t)t * (HD / 2);
     auto place = [&](int idx, int & col, int & partner, int & hh, int & d) {
         hh = idx / HD; d = idx % HD;          // hh < G: query head, G: k, G + 1: v
@@ -2369,6 +2369,12 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
         const int i = a.neox ? (d < HD / 2 ? d : d - HD / 2) : (d >> 1);
         cvs[u] = cs[i];
         svs[u] = sn[i];
+        // the norm weights of the column and of its partner, where the architecture normalises q and k per head
+        // (else any valid word: the request is made on every path, and before the first pages are requested - a
+        // load behind them would have to wait for them)
+        const float * nw = hh < a.G ? a.q_norm : (hh == a.G ? a.k_norm : nullptr);
+        nxs[u] = nw ? nw[d] : cs[0];
+        nys[u] = nw ? nw[partner - (col - d)] : cs[0];
         if (fast) {
             const float * base = a.from.data + (size_t)t * ROW;
 #pragma unroll
@@ -2481,8 +2487,8 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void k_attention_decode(DecodeAttn
             if (nw) {
                 const float ss = HD == 128 ? half_ss[u * NW + (wave & ~1)] + half_ss[u * NW + (wave | 1)] : half_ss[u * NW + wave];
                 const float scale = 1.0f / sqrtf(ss / (float)HD + a.eps);
-                xv[u] = (xv[u] * scale) * nw[d];
-                yv[u] = (yv[u] * scale) * nw[partner - (col - d)];
+                xv[u] = (xv[u] * scale) * nxs[u];
+                yv[u] = (yv[u] * scale) * nys[u];
             }
         }
         __syncthreads();          // half_ss is read before the partial results may overwrite it

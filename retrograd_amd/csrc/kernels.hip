@@ -1046,8 +1046,8 @@ __global__ __launch_bounds__(NW * 64) void k_rmsnorm_act8(float * x, const float
         const int k = threadIdx.x * 8 + c * STEP;
         if (k < E) { wa[c] = *(const f4 *)(w + k); wb[c] = *(const f4 *)(w + k + 4); }   // independent of everything: issued first
     }
-    int c = 0;
-    for (int k = threadIdx.x * 8; k < E; k += STEP, ++c) {
+    // eight elements of the row: the residual value plus what `add` holds for it; c counts the thread's groups
+    auto group = [&](int k, int c) __attribute__((always_inline)) {
         f4 a = *(const f4 *)(xr + k), b = *(const f4 *)(xr + k + 4);
         if (add.n > 0 && add.weight) {
             // the weighted sum of the row's terms, eight terms' loads in flight together
@@ -1078,8 +1078,8 @@ __global__ __launch_bounds__(NW * 64) void k_rmsnorm_act8(float * x, const float
             *(f4 *)(xr + k + 4) = b;
         } else if (add.n > 0) {
             const float * sl = add.data + (size_t)row * E + k;
-            int j = 0;
-            for (; j + 8 <= add.n; j += 8) {          // eight slices' loads in flight together, added in slice order
+            // eight slices' loads in flight together, added in slice order
+            auto add_eight = [&](int j) __attribute__((always_inline)) {
                 f4 sa[8], sb[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
@@ -1088,7 +1088,12 @@ __global__ __launch_bounds__(NW * 64) void k_rmsnorm_act8(float * x, const float
                 }
 #pragma unroll
                 for (int u = 0; u < 8; ++u) { a += sa[u]; b += sb[u]; }
-            }
+            };
+            int j = 0;
+            // The first eight outside the loop: ahead of a loop that adds to values still on their way the compiler
+            // waits for them, and the row itself would have to arrive before its slices are even requested.
+            if (add.n >= 8) { add_eight(0); j = 8; }
+            for (; j + 8 <= add.n; j += 8) add_eight(j);
             for (; j + 4 <= add.n; j += 4) {          // four
                 f4 sa[4], sb[4];
 #pragma unroll
@@ -1110,6 +1115,15 @@ __global__ __launch_bounds__(NW * 64) void k_rmsnorm_act8(float * x, const float
         for (int i = 0; i < KEEP; ++i)
             if (i == c) { ka[i] = a; kb[i] = b; }
         ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w + b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+    };
+    // A row of one group per thread (the common widths) is not a loop: inside a loop the compiler waits for
+    // everything requested so far before the slices' loads go out (a load of the pass before could still be on its
+    // way into their registers, for all it knows), and the row would arrive before its slices are even requested.
+    if (E <= STEP) {
+        if ((int)threadIdx.x * 8 < E) group(threadIdx.x * 8, 0);
+    } else {
+        int c = 0;
+        for (int k = threadIdx.x * 8; k < E; k += STEP, ++c) group(k, c);
     }
     ss = wave_sum(ss);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;

@@ -334,6 +334,13 @@ __device__ __forceinline__ h8 staged(const uint8_t * buf, int t, int s, int hl, 
     return *(const h8 *)(buf + t * kStageTile + ((s * 2 + hl) * 64 + lane) * 16);
 }
 
+// The rotating weight sets of the MXFP4 pipeline (members only where the pipeline is built: as plain locals of every
+// instantiation they cost the other weight types registers).
+template <int TYPE, bool ON> struct GateUpSets { Tile<TYPE> g0, u0, g1, u1, g2, u2; };
+template <int TYPE> struct GateUpSets<TYPE, false> {};
+template <int TYPE, bool ON> struct DownSets { Tile<TYPE> w0, w1, w2; };
+template <int TYPE> struct DownSets<TYPE, false> {};
+
 // One workgroup per (expert, four consecutive tiles of 16 output features), one wave per tile: gate and up
 // tiles together, SwiGLU in the epilogue. The weights of the next super-block and the activations of the next
 // super-block are requested before the current one is multiplied.
@@ -349,15 +356,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int item0 = blockIdx.x * 4;
     const int e = item0 / n_tiles, ft = item0 % n_tiles + wave;     // n_tiles % 4 == 0: one expert per workgroup
     if (e >= a.n_expert) return;
-    const int n_e = a.expert_n[e];
-    if (n_e == 0) return;
-    const int qb = a.off_pad[e];
     const int nsb = a.K >> 8;
     const uint8_t * wg = a.w0 + ((size_t)e * n_tiles + ft) * nsb * Tile<TYPE>::BYTES;
     const uint8_t * wu = a.w1 + ((size_t)e * n_tiles + ft) * nsb * Tile<TYPE>::BYTES;
+    // MXFP4: three weight sets in rotation (below); the first two are requested before the expert's pair count and
+    // slots are looked up - two trips to memory that the weights' own trip then runs under
+    GateUpSets<TYPE, TYPE == WT_MXFP4> ws;
+    auto request_w = [&](int sb, Tile<TYPE> & tg, Tile<TYPE> & tu) __attribute__((always_inline)) {
+        const size_t o = (size_t)min(sb, nsb - 1) * Tile<TYPE>::BYTES;
+        tg.load(wg + o, lane);
+        tu.load(wu + o, lane);
+    };
+    if constexpr (TYPE == WT_MXFP4) {
+        request_w(0, ws.g0, ws.u0);
+        request_w(1, ws.g1, ws.u1);
+    }
+    const int n_e = a.expert_n[e];
+    if (n_e == 0) return;
+    const int qb = a.off_pad[e];
     for (int t0 = 0; t0 < n_e; t0 += 16 * NTMAX) {
         const int nt = (NTMAX == 2 && n_e - t0 > 16) ? 2 : 1;
         __syncthreads();                       // the last pass is done with rows and the staging buffers
+        if constexpr (TYPE == WT_MXFP4) {
+            if (t0 > 0) { request_w(0, ws.g0, ws.u0); request_w(1, ws.g1, ws.u1); }
+        }
         if (threadIdx.x < 32) {
             const int at = t0 + threadIdx.x;
             const int tk = at < n_e ? a.tok_of_q[qb + at] : -1;
@@ -388,7 +410,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             // (no registers, no store phase), the weights are requested two super-blocks ahead into three sets in
             // rotation, and the waits are written here - the compiler does not see the direct requests, and its own
             // waits for the weight loads it does see come after these and find them done. A wave's requests return in
-            // order: at the top of super-block sb everything but the six loads of set sb + 1 must have landed.
+            // order: at the top of super-block sb > 0 everything but the six loads of set sb + 1 must have landed.
             const uint32_t lds0 = lds_offset(&stage[0][0]);
             auto request_x = [&](int sb) __attribute__((always_inline)) {
                 const __half * xs = a.x.x + (size_t)sb * kStageStep;
@@ -398,19 +420,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     lds_dma16(xs, at.off[c] * 2u, lds0 + (uint32_t)(sb & 1) * (NTMAX * kStageTile) + (uint32_t)(c * 256 + wave * 64) * 16u);
                 }
             };
-            auto request_w = [&](int sb, Tile<TYPE> & tg, Tile<TYPE> & tu) __attribute__((always_inline)) {
-                const size_t o = (size_t)min(sb, nsb - 1) * Tile<TYPE>::BYTES;
-                tg.load(wg + o, lane);
-                tu.load(wu + o, lane);
-            };
-            Tile<TYPE> g0, u0, g1, u1, g2, u2;
             request_x(0);
-            request_w(0, g0, u0);
-            __builtin_amdgcn_sched_barrier(0);
-            request_w(1, g1, u1);
             __builtin_amdgcn_sched_barrier(0);
             auto body = [&](int sb, Tile<TYPE> & cg, Tile<TYPE> & cu, Tile<TYPE> & fg, Tile<TYPE> & fu) __attribute__((always_inline)) {
-                __builtin_amdgcn_s_waitcnt(0x0F70 | 6);
+                // super-block 0: its activations were requested last, after both weight sets - everything lands
+                if (sb == 0) __builtin_amdgcn_s_waitcnt(0x0F70); else __builtin_amdgcn_s_waitcnt(0x0F70 | 6);
                 asm volatile("" : "+v"(cg.hdr.x), "+v"(cg.hdr.y), "+v"(cg.q0), "+v"(cg.q1), "+v"(cu.hdr.x), "+v"(cu.hdr.y), "+v"(cu.q0), "+v"(cu.q1));
                 __syncthreads();           // every wave's part of super-block sb is in LDS, and none still reads the other buffer
                 if (sb + 1 < nsb) request_x(sb + 1);
@@ -420,9 +434,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 multiply(sb, cg, cu);
             };
             for (int sb = 0; sb < nsb; sb += 3) {
-                body(sb, g0, u0, g2, u2);
-                body(sb + 1, g1, u1, g0, u0);
-                body(sb + 2, g2, u2, g1, u1);
+                body(sb, ws.g0, ws.u0, ws.g2, ws.u2);
+                body(sb + 1, ws.g1, ws.u1, ws.g0, ws.u0);
+                body(sb + 2, ws.g2, ws.u2, ws.g1, ws.u1);
             }
         } else {
             StageRegs<NTMAX> regs;
@@ -440,7 +454,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     ng.load(wg + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
                     nu.load(wu + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
                 }
-                multiply(sb, tg, tu);
+                const uint8_t * cur = stage[sb & 1];
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+                    const auto og = tg.prep(s), ou = tu.prep(s);
+#pragma unroll
+                    for (int t = 0; t < NTMAX; ++t) {
+                        if (t >= nt) break;
+                        const h8 hi = staged(cur, t, s, 0, lane), lo = staged(cur, t, s, 1, lane);
+                        mac(og, hi, lo, ag[t]);
+                        mac(ou, hi, lo, au[t]);
+                    }
+                }
                 if (more) stage_store(stage[(sb + 1) & 1], nt, regs);
                 __syncthreads();
                 tg = ng;
@@ -482,14 +507,25 @@ void k_moe_down(MoeArgs a) {
     const int item0 = blockIdx.x * 4;
     const int e = item0 / n_tiles, et = item0 % n_tiles + wave;
     if (e >= a.n_expert) return;
+    const int nsb = a.K >> 8;
+    const uint8_t * wd = a.w0 + ((size_t)e * n_tiles + et) * nsb * Tile<TYPE>::BYTES;
+    DownSets<TYPE, TYPE == WT_MXFP4> ws;          // (MXFP4, as in k_moe_gate_up: the first two sets requested before the lookups)
+    auto request_w = [&](int sb, Tile<TYPE> & tw) __attribute__((always_inline)) {
+        tw.load(wd + (size_t)min(sb, nsb - 1) * Tile<TYPE>::BYTES, lane);
+    };
+    if constexpr (TYPE == WT_MXFP4) {
+        request_w(0, ws.w0);
+        request_w(1, ws.w1);
+    }
     const int n_e = a.expert_n[e];
     if (n_e == 0) return;
     const int qb = a.off_pad[e];
-    const int nsb = a.K >> 8;
-    const uint8_t * wd = a.w0 + ((size_t)e * n_tiles + et) * nsb * Tile<TYPE>::BYTES;
     for (int t0 = 0; t0 < n_e; t0 += 16 * NTMAX) {
         const int nt = (NTMAX == 2 && n_e - t0 > 16) ? 2 : 1;
         __syncthreads();
+        if constexpr (TYPE == WT_MXFP4) {
+            if (t0 > 0) { request_w(0, ws.w0); request_w(1, ws.w1); }
+        }
         // every row of a tile lies in the expert's padded slot range
         if (threadIdx.x < 32) {
             const int slot = qb + t0 + ((int)threadIdx.x < 16 * nt ? threadIdx.x : 0);
@@ -523,17 +559,10 @@ void k_moe_down(MoeArgs a) {
                     lds_dma16(xs, at.off[c] * 2u, lds0 + (uint32_t)(sb & 1) * (NTMAX * kStageTile) + (uint32_t)(c * 256 + wave * 64) * 16u);
                 }
             };
-            auto request_w = [&](int sb, Tile<TYPE> & tw) __attribute__((always_inline)) {
-                tw.load(wd + (size_t)min(sb, nsb - 1) * Tile<TYPE>::BYTES, lane);
-            };
-            Tile<TYPE> w0, w1, w2;
             request_x(0);
-            request_w(0, w0);
-            __builtin_amdgcn_sched_barrier(0);
-            request_w(1, w1);
             __builtin_amdgcn_sched_barrier(0);
             auto body = [&](int sb, Tile<TYPE> & cw, Tile<TYPE> & fw) __attribute__((always_inline)) {
-                __builtin_amdgcn_s_waitcnt(0x0F70 | 3);
+                if (sb == 0) __builtin_amdgcn_s_waitcnt(0x0F70); else __builtin_amdgcn_s_waitcnt(0x0F70 | 3);
                 asm volatile("" : "+v"(cw.hdr.x), "+v"(cw.hdr.y), "+v"(cw.q0), "+v"(cw.q1));
                 __syncthreads();
                 if (sb + 1 < nsb) request_x(sb + 1);
@@ -543,9 +572,9 @@ void k_moe_down(MoeArgs a) {
                 multiply(sb, cw);
             };
             for (int sb = 0; sb < nsb; sb += 3) {
-                body(sb, w0, w2);
-                body(sb + 1, w1, w0);
-                body(sb + 2, w2, w1);
+                body(sb, ws.w0, ws.w2);
+                body(sb + 1, ws.w1, ws.w0);
+                body(sb + 2, ws.w2, ws.w1);
             }
         } else {
             StageRegs<NTMAX> regs;
@@ -561,7 +590,16 @@ void k_moe_down(MoeArgs a) {
                     stage_load(a.x.x, at, sb + 1, nt, regs);
                     nw.load(wd + (size_t)(sb + 1) * Tile<TYPE>::BYTES, lane);
                 }
-                multiply(sb, tw);
+                const uint8_t * cur = stage[sb & 1];
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+                    const auto ow = tw.prep(s);
+#pragma unroll
+                    for (int t = 0; t < NTMAX; ++t) {
+                        if (t >= nt) break;
+                        mac(ow, staged(cur, t, s, 0, lane), staged(cur, t, s, 1, lane), acc[t]);
+                    }
+                }
                 if (more) stage_store(stage[(sb + 1) & 1], nt, regs);
                 __syncthreads();
                 tw = nw;

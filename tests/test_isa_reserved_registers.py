@@ -59,3 +59,33 @@ def test_the_compiler_never_writes_the_registers_the_weight_prefetch_owns(tmp_pa
         assert m and int(m.group(1)) == 256
         m = re.search(r"\.amdhsa_private_segment_fixed_size (\d+)", meta)
         assert m and int(m.group(1)) == 0
+
+
+# Kernels whose inner loops are sized to the register file: a spill there costs the kernel its speed without failing
+# any numerical test (seen once: a refactoring of the expert kernels' step loop into a lambda spilled 21-45
+# registers in the Q4_K / Q5_K / Q6_K variants). The private segment of these must stay empty.
+NO_SPILL = {
+    "moe.hip": [r"k_moe_gate_upILi\d+ELi2E", r"k_moe_downILi\d+ELi[12]E"],
+    "mm_lds.hip": [r"k_mm2_q4kILi\dELi2ELb[01]E", r"k_mm2_q8_0ILi\dELi2E", r"k_mm2_q6kILi\dELi2E"],
+    "kernels.hip": [r"k_attention_decodeILi\d+ELi8E", r"k_rmsnorm_act8ILi\dE"],
+}
+
+
+@pytest.mark.parametrize("source", sorted(NO_SPILL))
+def test_the_register_bound_kernels_do_not_spill(tmp_path, source):
+    out = tmp_path / (source + ".s")
+    cmd = [B.hipcc(), *[f for f in B.HIP_FLAGS if f != "-fPIC"], "-x", "hip", "-S", "--cuda-device-only",
+           str(B.CSRC / source), "-o", str(out)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    text = out.read_text()
+    # the kernel descriptor of every kernel: .amdhsa_kernel <name> ... .amdhsa_private_segment_fixed_size N
+    found = 0
+    for m in re.finditer(r"\.amdhsa_kernel (\S+)(.*?)\.end_amdhsa_kernel", text, re.S):
+        name, desc = m.group(1), m.group(2)
+        if not any(re.search(p, name) for p in NO_SPILL[source]):
+            continue
+        found += 1
+        size = re.search(r"\.amdhsa_private_segment_fixed_size (\d+)", desc)
+        assert size and int(size.group(1)) == 0, "%s spills (%s bytes of scratch per lane)" % (name, size.group(1) if size else "?")
+    assert found >= len(NO_SPILL[source]), "the kernels named here are expected in " + source

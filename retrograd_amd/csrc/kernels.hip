@@ -1156,7 +1156,8 @@ void rmsnorm_act(hipStream_t s, float * x, const float * w, int E, float eps,
     if (add.n > 0 && add.N != E) throw std::runtime_error("rmsnorm: the slices do not match the row width");
     check_act_out(out, E, "rmsnorm", n_rows);
     if (E % 32 == 0) {
-        if (E >= 4096) hipLaunchKernelGGL(k_rmsnorm_act8<8>, dim3(n_rows), dim3(512), 0, s, x, w, E, eps, rows, out, add);
+        // eight waves where four would need two groups of eight elements per thread (a loop: see the kernel)
+        if (E > 2048) hipLaunchKernelGGL(k_rmsnorm_act8<8>, dim3(n_rows), dim3(512), 0, s, x, w, E, eps, rows, out, add);
         else hipLaunchKernelGGL(k_rmsnorm_act8<4>, dim3(n_rows), dim3(256), 0, s, x, w, E, eps, rows, out, add);
         check_launch("rmsnorm");
         return;

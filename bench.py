@@ -72,6 +72,9 @@ def parse_args():
     ap.add_argument("--one-sequence", action="store_true",
                     help="measure only the single-sequence decode steps (512-token context) in the chosen arithmetic and "
                          "print their JSON: the workload of the small-batch kernel profiles")
+    ap.add_argument("--single-token-matvec", action="store_true",
+                    help="with --one-sequence in the exact arithmetic: the matrix-vector kernel with f32 rows instead of the tile kernels "
+                         "(what RETRO_GEMV_EXACT=1 selects)")
     return ap.parse_args()
 
 
@@ -396,11 +399,13 @@ def main() -> int:
 
     if args.one_sequence:
         eng = new_engine(args.activations)
+        if args.single_token_matvec:
+            eng.single_token_matvec(True)
         kvb = 2 * shape.n_head_kv * shape.head_dim * 2 * {"f16": 32, "q8_0": 17, "q4_0": 9}[args.kv] // 32
         leg = one_sequence_leg(eng, E, shape, n_slots, synth.streamed_weight_bytes(shape), kvb, steps=args.steps)
         eng.close()
         print(json.dumps({"metric": "single-sequence decode steps, %s" % shape.name, "activations": args.activations,
-                          "kv_cache": args.kv, **leg}), flush=True)
+                          "single_token_matvec": bool(args.single_token_matvec), "kv_cache": args.kv, **leg}), flush=True)
         return 0
     eng = new_engine(args.activations)
     m, wl = measure_decode(args, eng, E, synth, gw, shape, geometry, profile_kernels=True)
@@ -552,6 +557,12 @@ def main() -> int:
                 eng.request_free(s_.request)
         result["config"]["through_the_step_scheduler"] = scheduler_leg(args, eng, E, shape, geometry)
         result["config"]["one_sequence"] = {args.activations: one_sequence_leg(eng, E, shape, n_slots, w_bytes, kv_bytes_per_cell_layer)}
+        if args.activations == "exact":
+            # opt-in (RETRO_GEMV_EXACT=1): the matrix-vector kernel with f32 rows; a sequence decoded alone then differs
+            # in the last bits from the same sequence inside a batch, so the tile kernels stay the default
+            eng.single_token_matvec(True)
+            result["config"]["one_sequence"]["exact_with_the_single_token_matvec_kernel"] = one_sequence_leg(eng, E, shape, n_slots, w_bytes, kv_bytes_per_cell_layer)
+            eng.single_token_matvec(False)
         result["config"]["small_steps"] = [one_sequence_leg(eng, E, shape, n_slots, w_bytes, kv_bytes_per_cell_layer, n_seq=n) for n in (8, 32)]
     eng.close()
     del eng

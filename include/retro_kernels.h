@@ -34,7 +34,9 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
  * converted as ggml converts them for the weight type; kind 2: x is [n_tokens][2 k] gate and up values in alternating
  * groups of `group` columns (0: side by side), the rows are silu(gate) * up converted likewise. raw: n_rows rows of
  * k, Q4_K (the rows become Q8_K blocks) or Q8_0 (Q8_0 blocks). Both results are [n_tokens][n_rows]; at most two
- * tokens. */
+ * tokens. kinds 11 and 12: the same two producers for the exact arithmetic's matrix-vector kernel (one token): the row
+ * stays f32 when the kernel makes it itself (y_fused) and is read back from the hi / lo f16 planes the producer's launch
+ * leaves otherwise (y_unfused). */
 int retro_kernel_gemv_fused(int32_t kind, int32_t type, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, const float * norm_w,
                             float eps, int32_t n_tokens, int32_t group, float * y_fused, float * y_unfused);
 
@@ -80,7 +82,8 @@ int32_t retro_kernel_sample_greedy_noalloc_max_rows(void);
  * 3 only), n_rows a multiple of 16 and k of 256: anything else is refused
  * before a buffer is allocated. Mode 4 times the integer matrix-vector kernel
  * of very small steps under the ggml arithmetic instead (Q4_K or Q8_0, at most
- * two tokens, pseudo-random activation blocks). */
+ * two tokens, pseudo-random activation blocks), mode 5 the exact arithmetic's
+ * matrix-vector kernel over the hi / lo planes (one token). */
 int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_tokens, int32_t mode,
                              int32_t iters, int32_t debug, int32_t force_ksplit, double * out_us);
 
@@ -147,6 +150,13 @@ int retro_engine_debug_profile_read(retro_engine * engine, double * out_ms, uint
  * launch ([workgroups][6]; out == NULL reports the count; 0 workgroups when no step took that launch). */
 int retro_engine_debug_attention_timeline(retro_engine * engine, int32_t enable);
 int retro_engine_debug_attention_timeline_read(retro_engine * engine, uint64_t * out, size_t cap_workgroups, size_t * out_workgroups);
+
+/* Single-token steps of the exact arithmetic on the matrix-vector kernel with f32 rows (RMSNorm and SwiGLU made in its
+ * staging, the attention output read from the planes the attention launch leaves) instead of the tile kernels: what
+ * RETRO_GEMV_EXACT=1 selects when the engine is created. Off by default: a sequence decoded alone then no longer gives
+ * bit for bit the logprobs it gives inside a batch, which the tile kernels do for steps of up to 16 tokens and the
+ * reference's tests hold (tests/engine_runtime.rs:713-722). */
+int retro_engine_debug_single_token_matvec(retro_engine * engine, int32_t enable);
 
 #ifdef __cplusplus
 }

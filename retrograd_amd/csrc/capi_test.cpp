@@ -105,8 +105,12 @@ int retro_kernel_matmul(int32_t type, const uint8_t * raw, int64_t n_rows, int64
 int retro_kernel_gemv_fused(int32_t kind, int32_t type, const uint8_t * raw, int64_t n_rows, int64_t k, const float * x, const float * norm_w,
                             float eps, int32_t n_tokens, int32_t group, float * y_fused, float * y_unfused) {
     return guarded([&]() -> int {
-        if ((kind != 1 && kind != 2) || n_tokens < 1 || n_tokens > rk::GEMV_MAX_T || k <= 0 || k % 256 != 0 || n_rows <= 0 || n_rows % 16 != 0)
-            throw std::runtime_error("gemv_fused: kind 1 (RMSNorm) or 2 (SwiGLU), whole tiles and super-blocks, at most " + std::to_string(rk::GEMV_MAX_T) + " tokens");
+        // kinds 11 and 12: the exact arithmetic's kernel (f32 rows, a single token) for the same two producers
+        const bool exact = kind == 11 || kind == 12;
+        if (exact) kind -= 10;
+        if ((kind != 1 && kind != 2) || n_tokens < 1 || n_tokens > (exact ? 1 : rk::GEMV_MAX_T) || k <= 0 || k % 256 != 0 || n_rows <= 0 || n_rows % 16 != 0)
+            throw std::runtime_error("gemv_fused: kind 1 / 11 (RMSNorm) or 2 / 12 (SwiGLU), whole tiles and super-blocks, at most " + std::to_string(rk::GEMV_MAX_T)
+                                     + " tokens (kinds 11 and 12: one)");
         if (kind == 1 && !norm_w) throw std::runtime_error("gemv_fused: the RMSNorm needs its weights");
         if (type != rk::WT_Q4_K && type != rk::WT_Q5_K && type != rk::WT_Q6_K && type != rk::WT_Q8_0) throw std::runtime_error("gemv_fused: Q4_K, Q5_K, Q6_K or Q8_0 rows");
         struct Restore { int was; ~Restore() { rk::g_gemv_max_t = was; } } restore{rk::g_gemv_max_t};
@@ -130,20 +134,32 @@ int retro_kernel_gemv_fused(int32_t kind, int32_t type, const uint8_t * raw, int
         ok(hipMemset(d_xh.ptr, 0, d_xh.bytes), "clear"); ok(hipMemset(d_sums.ptr, 0, d_sums.bytes), "clear");
         d_codes.alloc((size_t)n_tokens * k); d_scales.alloc((size_t)n_tokens * (k / 32) * 4); d_bsums.alloc((size_t)n_tokens * (k / 16) * 2);
         rk::Act act;
-        act.K = (int)k; act.faithful = 1; act.quant = rk::act_quant_of(type);
-        act.qx = d_xh.as<__half>(); act.qsums = d_sums.as<__half>();
-        act.qc = d_codes.as<int8_t>(); act.qd = d_scales.as<float>(); act.qbs = d_bsums.as<int16_t>();
+        act.K = (int)k;
+        if (exact) {
+            if (!rk::gemv_f32_can_weight(w, n_tokens)) throw std::runtime_error("gemv_fused: the exact kernel does not take this matrix");
+            act.x = d_xh.as<__half>(); act.sums = d_sums.as<__half>();
+        } else {
+            act.faithful = 1; act.quant = rk::act_quant_of(type);
+            act.qx = d_xh.as<__half>(); act.qsums = d_sums.as<__half>();
+            act.qc = d_codes.as<int8_t>(); act.qd = d_scales.as<float>(); act.qbs = d_bsums.as<int16_t>();
+        }
         d_y.alloc((size_t)n_tokens * n_rows * 4);
-        // the two launches: the producer leaves the blocks, the kernel multiplies them
+        // the two launches: the producer leaves the blocks (exact: the hi / lo planes), the kernel multiplies them
         if (kind == 1) rk::rmsnorm_act(nullptr, d_x.as<float>(), d_w.as<float>(), (int)k, eps, nullptr, n_tokens, act);
         else rk::swiglu_act(nullptr, d_x.as<float>(), n_tokens, (int)k, act, group);
-        rk::gemv(nullptr, w, act.operand(type), n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr);
+        if (exact) rk::gemv_f32(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr);
+        else rk::gemv(nullptr, w, act.operand(type), n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr);
         ok(hipDeviceSynchronize(), "gemv");
         ok(hipMemcpy(y_unfused, d_y.ptr, d_y.bytes, hipMemcpyDeviceToHost), "download");
         ok(hipMemset(d_y.ptr, 0, d_y.bytes), "clear");
-        // one launch: the kernel makes the blocks while it stages them
-        if (kind == 1) rk::gemv_norm(nullptr, w, d_x.as<float>(), d_w.as<float>(), eps, nullptr, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr);
-        else rk::gemv_swiglu(nullptr, w, d_x.as<float>(), group, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE);
+        // one launch: the kernel makes the rows while it stages them
+        if (exact) {
+            if (kind == 1) rk::gemv_f32_norm(nullptr, w, d_x.as<float>(), d_w.as<float>(), eps, nullptr, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr);
+            else rk::gemv_f32_swiglu(nullptr, w, d_x.as<float>(), group, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE);
+        } else {
+            if (kind == 1) rk::gemv_norm(nullptr, w, d_x.as<float>(), d_w.as<float>(), eps, nullptr, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr);
+            else rk::gemv_swiglu(nullptr, w, d_x.as<float>(), group, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE);
+        }
         ok(hipDeviceSynchronize(), "gemv fused");
         ok(hipMemcpy(y_fused, d_y.ptr, d_y.bytes, hipMemcpyDeviceToHost), "download");
         return 0;
@@ -273,7 +289,9 @@ int retro_kernel_matmul_time(int32_t type, int64_t n_rows, int64_t k, int32_t n_
         auto run = [&]() {
             w.packed = d_w.as<uint8_t>() + (turn++ % copies) * bytes;
             // mode 1: register-only tiles, 2: LDS-staged tiles, 3: the same with the K-slices left unreduced
-            if (mode == 3) rk::matmul_deferred(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, d_ws.ptr);
+            // mode 5: the exact arithmetic's matrix-vector kernel over the hi / lo planes (one token)
+            if (mode == 5) rk::gemv_f32(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr);
+            else if (mode == 3) rk::matmul_deferred(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, d_ws.ptr);
             else rk::matmul(nullptr, w, act, n_tokens, d_y.as<float>(), (int)n_rows, 0, rk::MM_STORE, nullptr, mode == 2 || mode == 4 ? d_ws.ptr : nullptr);
         };
         for (int i = 0; i < 3; ++i) run();
@@ -443,6 +461,14 @@ int retro_engine_debug_attention_timeline(retro_engine * engine, int32_t enable)
     return guarded([&]() -> int {
         if (!engine) { set_error("engine is required"); return -1; }
         engine->impl.attention_timeline(enable != 0);
+        return 0;
+    });
+}
+
+int retro_engine_debug_single_token_matvec(retro_engine * engine, int32_t enable) {
+    return guarded([&]() -> int {
+        if (!engine) { set_error("engine is required"); return -1; }
+        engine->impl.single_token_matvec(enable != 0);
         return 0;
     });
 }

@@ -79,6 +79,7 @@ Engine::Engine(const std::string & path, const retro_engine_config & config) : c
         // RETRO_ACTIVATIONS=ggml: every matmul multiplies the activations as ggml's CPU path converts them
         // (Q8_K / Q8_0 codes, f16 / bf16 rounding); unset or "exact": the f32 values (as f16 hi/lo pairs).
         if (const char * f = std::getenv("RETRO_GEMV_FUSE")) gemv_fuse_ = std::atoi(f) != 0;
+        if (const char * f = std::getenv("RETRO_GEMV_EXACT")) gemv_exact_ = std::atoi(f) != 0;
         // ... and the output projection merges at most this many attention splits per kv head itself (0: never)
         if (const char * f = std::getenv("RETRO_GEMV_MERGE_SPLITS")) merge_max_splits_ = std::max(0, std::min(std::atoi(f), rk::GEMV_COMBINE_MAX_SPLITS));      // 0: producers keep their own launches
         // steps of at most this many tokens go through the integer matrix-vector kernel under the ggml arithmetic (0: never)
@@ -1337,13 +1338,22 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
     // makes the blocks itself while it stages them and the producer's launch is saved
     // (single-token steps only: the blocks of a second row cost every workgroup more than the launch saves)
     const bool fuse = faithful && small_step && T == 1 && !routed && gemv_fuse_;
+    // The exact arithmetic's single-token steps: the same kernel with f32 rows (gemv_f32*), the same fusions, and the
+    // output projection from the planes the attention launch leaves. One flag selects the flavour below.
+    const bool fuse_x = !faithful && T == 1 && !routed && gemv_fuse_ && gemv_exact_;
+    auto can_gemv = [&](const rk::Weight & w, int tokens) { return fuse_x ? rk::gemv_f32_can_weight(w, tokens) : rk::gemv_can_weight(w, tokens); };
     auto all_gemv = [&](const std::vector<DevWeight> & ws, int K, int room) {
         int total = 0;
         for (const DevWeight & w : ws) {
-            if (!rk::gemv_can_weight(w.w, T) || w.w.K != K) return false;
+            if (!can_gemv(w.w, T) || w.w.K != K) return false;
             total += w.w.N;
         }
         return !ws.empty() && total <= room;
+    };
+    auto gemv_norm = [&](const rk::Weight & w, const float * rows, const float * norm_w, const int32_t * which, int tokens, float * y,
+                         int ldy, int col, const float * bias) {
+        if (fuse_x) rk::gemv_f32_norm(stream_, w, rows, norm_w, h.eps, which, tokens, y, ldy, col, rk::MM_STORE, bias);
+        else rk::gemv_norm(stream_, w, rows, norm_w, h.eps, which, tokens, y, ldy, col, rk::MM_STORE, bias);
     };
     auto act_for = [faithful, small_step](DevBuf & x, DevBuf & sums, DevBuf & qx, DevBuf & qsums, int K, std::initializer_list<int> types,
                                           bool plain, ActCodes * codes = nullptr) {
@@ -1390,7 +1400,7 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         const std::array<int, 3> qt = types_of(L.qkv), gt = types_of(L.gate_up);
         rk::Act act_e = act_for(act_e_x_, act_e_sums_, act_e_qx_, act_e_qsums_, E, {qt[0], qt[1], qt[2]}, routed, &act_e_codes_);
         const rk::Act act_q = act_for(act_q_x_, act_q_sums_, act_q_qx_, act_q_qsums_, QD, {L.wo.w.type}, routed, &act_q_codes_);
-        const bool qkv_fused = fuse && pending.n == 0 && all_gemv(L.qkv, E, QD + 2 * KD);
+        const bool qkv_fused = (fuse || fuse_x) && pending.n == 0 && all_gemv(L.qkv, E, QD + 2 * KD);
         if (!qkv_fused) { const size_t pt_ = prof_begin(PC_NORM); rk::rmsnorm_act(stream_, x, L.attn_norm.as<float>(), E, h.eps, nullptr, T, act_e, pending); prof_end(PC_NORM, pt_); }
         rk::Slices qkv_slices;
         {
@@ -1398,8 +1408,8 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
             if (qkv_fused) {
                 int col = 0;
                 for (const DevWeight & w : L.qkv) {
-                    rk::gemv_norm(stream_, w.w, x, L.attn_norm.as<float>(), h.eps, nullptr, T, qkv, QD + 2 * KD, col, rk::MM_STORE,
-                                  L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr);
+                    gemv_norm(w.w, x, L.attn_norm.as<float>(), nullptr, T, qkv, QD + 2 * KD, col,
+                              L.qkv_bias.ptr ? L.qkv_bias.as<float>() + col : nullptr);
                     col += w.w.N;
                 }
             } else if (L.qkv.size() == 1) {     // fused q, k, v: the rotation kernel can add the slices
@@ -1453,7 +1463,12 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
                                  L.k_norm.as<float>(), act_q, stamps);
             prof_end(PC_ATTN, pt_);
             pt_ = prof_begin(PC_OPROJ);
-            pending = rk::matmul_deferred(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
+            if (fuse_x && rk::gemv_f32_can_weight(L.wo.w, T) && L.wo.w.K == QD && L.wo.w.N == E) {
+                rk::gemv_f32(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr);
+                pending = rk::Slices();
+            } else {
+                pending = rk::matmul_deferred(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
+            }
             if (routed) {
                 float * dst = pending.n > 0 ? const_cast<float *>(pending.data) : x;
                 rk::lora_apply(stream_, lora_entries(l, 3), d_stage_.as<rk::RowDesc>(), pk_.row, act_q, T, E, dst, E, 0,
@@ -1486,7 +1501,12 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         rk::attention_combine(stream_, partial_.as<float>(), T, sh, pk_, act_q);
         prof_end(PC_COMBINE, pt_);
         pt_ = prof_begin(PC_OPROJ);
-        pending = rk::matmul_deferred(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
+        if (fuse_x && rk::gemv_f32_can_weight(L.wo.w, T) && L.wo.w.K == QD && L.wo.w.N == E) {
+            rk::gemv_f32(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr);
+            pending = rk::Slices();
+        } else {
+            pending = rk::matmul_deferred(stream_, L.wo.w, act_q, T, x, E, 0, rk::MM_ADD, nullptr, mm_ws_.ptr);
+        }
         if (routed) {
             float * dst = pending.n > 0 ? const_cast<float *>(pending.data) : x;
             rk::lora_apply(stream_, lora_entries(l, 3), d_stage_.as<rk::RowDesc>(), pk_.row, act_q, T, E, dst, E, 0,
@@ -1495,18 +1515,19 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
         prof_end(PC_OPROJ, pt_);
         }
         }
-        if (fuse && h.n_expert == 0 && pending.n == 0 && all_gemv(L.gate_up, E, 2 * F)) {
+        if ((fuse || fuse_x) && h.n_expert == 0 && pending.n == 0 && all_gemv(L.gate_up, E, 2 * F)) {
             pt_ = prof_begin(PC_GATEUP);
             int col = 0;
             for (const DevWeight & w : L.gate_up) {
-                rk::gemv_norm(stream_, w.w, x, L.ffn_norm.as<float>(), h.eps, nullptr, T, gu, 2 * F, col, rk::MM_STORE, nullptr);
+                gemv_norm(w.w, x, L.ffn_norm.as<float>(), nullptr, T, gu, 2 * F, col, nullptr);
                 col += w.w.N;
             }
             prof_end(PC_GATEUP, pt_);
             const int group = L.gate_up_interleaved ? 64 : F;
             pt_ = prof_begin(PC_DOWN);
-            if (rk::gemv_can_weight(L.down.w, T) && L.down.w.K == F && L.down.w.N == E) {
-                rk::gemv_swiglu(stream_, L.down.w, gu, group, T, x, E, 0, rk::MM_ADD);
+            if (can_gemv(L.down.w, T) && L.down.w.K == F && L.down.w.N == E) {
+                if (fuse_x) rk::gemv_f32_swiglu(stream_, L.down.w, gu, group, T, x, E, 0, rk::MM_ADD);
+                else rk::gemv_swiglu(stream_, L.down.w, gu, group, T, x, E, 0, rk::MM_ADD);
                 pending = rk::Slices();
             } else {
                 const rk::Act act_f = act_for(act_f_x_, act_f_sums_, act_f_qx_, act_f_qsums_, F, {L.down.w.type}, false, &act_f_codes_);
@@ -1572,9 +1593,8 @@ void Engine::forward(int T, int n_out, int n_tiles, int n_items, bool one_token_
     if (n_out > 0) {
         logits_.ensure((size_t)n_out * h.n_vocab * 4);
         const size_t pt_ = prof_begin(PC_HEAD);
-        if (fuse && pending.n == 0 && rk::gemv_can_weight(lm_head_.w, n_out) && lm_head_.w.K == E && lm_head_.w.N == h.n_vocab) {
-            rk::gemv_norm(stream_, lm_head_.w, x, out_norm_.as<float>(), h.eps, pk_.out_tok, n_out, logits_.as<float>(), h.n_vocab, 0,
-                          rk::MM_STORE, out_bias_.as<float>());
+        if ((fuse || fuse_x) && pending.n == 0 && can_gemv(lm_head_.w, n_out) && lm_head_.w.K == E && lm_head_.w.N == h.n_vocab) {
+            gemv_norm(lm_head_.w, x, out_norm_.as<float>(), pk_.out_tok, n_out, logits_.as<float>(), h.n_vocab, 0, out_bias_.as<float>());
         } else {
             rk::rmsnorm_act(stream_, x, out_norm_.as<float>(), E, h.eps, pk_.out_tok, n_out, act_o, pending);
             rk::matmul(stream_, lm_head_.w, act_o, n_out, logits_.as<float>(), h.n_vocab, 0, rk::MM_STORE,

@@ -214,6 +214,7 @@ public:
     // The decode attention launch of the middle layer leaves six clock values per workgroup while this is on;
     // read returns those of the last such launch ([workgroup][6]) and the number of workgroups.
     void attention_timeline(bool on);
+    void single_token_matvec(bool on) { gemv_exact_ = on; }
     int attention_timeline_read(unsigned long long * out, size_t cap_workgroups, size_t * n_workgroups);
     void profile_read(double * ms, uint64_t * launches, bool reset);
 
@@ -316,6 +317,11 @@ private:
     int32_t step_max_resident_ = 0;          // longest resident span (positions) among the rows of the step being run
     int merge_max_splits_ = 8;       // about a 1,000-token context: beyond it the merge kernel's own launch is cheaper
     bool gemv_fuse_ = true;      // small steps: the integer kernel makes its Q8_K blocks from the f32 rows itself where it can
+    // Single-token steps of the exact arithmetic on the matrix-vector kernel with f32 rows (RETRO_GEMV_EXACT=1). Off by
+    // default: its sums are added in another order than the tile kernels', so a sequence decoded alone would no longer
+    // give bit for bit the logprobs it gives inside a batch - a relation the reference's tests hold
+    // (tests/engine_runtime.rs:713-722).
+    bool gemv_exact_ = false;
     DevBuf q_half_lo_;
     DevBuf item_meta_;        // the step's attention work items (PackBuffers::item_a, item_b), grown as needed
     DevBuf mm_ws_;            // matmul workspace: split-K partials, counters

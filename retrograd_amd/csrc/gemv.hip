@@ -59,6 +59,8 @@ struct GemvArgs {
     const float * partial;     // per (item, column): m (log2 domain), l, head_dim unnormalised outputs
     int item0, n_split;        // the token's first work item; splits per kv head
     int att_G, att_hd;         // query heads per kv head, head_dim
+    // k_gemv_f32, SRC_CODES: the hi / lo f16 planes a producer left (Act::x)
+    const __half * planes;
 };
 enum : int { SRC_CODES = 0, SRC_NORM = 1, SRC_SWIGLU = 2, SRC_COMBINE = 3 };
 
@@ -405,17 +407,316 @@ __global__ __launch_bounds__(1024) void k_gemv(GemvArgs a) {
     }
 }
 
+// The same kernel for the exact arithmetic: the rows of the step stay f32 in LDS and every weight code is converted
+// (v_cvt_f32_ubyte) and multiplied by a fused multiply-add - about four times the integer kernel's vector
+// instructions per weight, which one or two tokens still hide behind the memory. Per eight columns a lane forms
+// p = sum q_k x_k in f32 and adds sc * p (Q4_K, Q5_K, Q6_K) to the super-block's sum; the offsets (Q4_K / Q5_K:
+// dmin * m_s * sum of the sub-block's x; Q6_K: 32 * sc_b * sum of the block's x) come from the sums of every sixteen
+// values made while the rows are staged. Q8_0: d_b * p per block. Sources: SRC_CODES - here the hi / lo planes a
+// producer left (the value is hi + lo) -, SRC_NORM and SRC_SWIGLU as above, the values kept as they are computed.
+// Dynamic LDS: NT * K floats | K-quants: NT * K / 16 floats | 2 * nw * NT * 16 floats.
+template <int WT, int NT, int PER, int SRC>
+__global__ __launch_bounds__(1024) void k_gemv_f32(GemvArgs a) {
+    using Tile = GemvTile<WT>;
+    constexpr bool Q5 = WT == WT_Q5_K, Q4 = WT == WT_Q4_K || Q5, Q6 = WT == WT_Q6_K, KQ = WT != WT_Q8_0;
+    static_assert(SRC == SRC_CODES || SRC == SRC_NORM || SRC == SRC_SWIGLU, "planes, RMSNorm or SwiGLU");
+    extern __shared__ __align__(16) uint8_t lds[];
+    const int K = a.K, nsb = K >> 8;
+    const int nthreads = blockDim.x, nw = nthreads >> 6;
+    float * l_x = (float *)lds;
+    float * l_s = l_x + NT * K;
+    float * l_red = KQ ? l_s + NT * (K >> 4) : l_s;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+
+    u4 hdr[2], q[2][Tile::LOADS];
+    uint16_t dq6[2] = {0, 0};
+    uint32_t fifth[2][2] = {{0, 0}, {0, 0}};
+    auto request = [&](int tile, int u0) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int sb = wave + (u0 + u) * nw;
+            if (sb < nsb) {
+                const uint8_t * tp = a.w + ((size_t)tile * nsb + sb) * Tile::BYTES;
+                hdr[u] = *(const u4 *)(tp + r * 16);
+                if constexpr (Q6) {
+                    q[u][0] = *(const u4 *)(tp + 288 + lane * 16);
+                    q[u][1] = *(const u4 *)(tp + 1312 + lane * 16);
+                    const uint2 t0 = *(const uint2 *)(tp + 2336 + lane * 8), t1 = *(const uint2 *)(tp + 2848 + lane * 8);
+                    q[u][2] = u4{t0.x, t0.y, t1.x, t1.y};
+                    dq6[u] = *(const uint16_t *)(tp + 256 + 2 * r);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < Tile::LOADS; ++i) q[u][i] = *(const u4 *)(tp + 256 + i * 1024 + lane * 16);
+                    if constexpr (Q5) {
+                        fifth[u][0] = *(const uint32_t *)(tp + 2304 + lane * 4);
+                        fifth[u][1] = *(const uint32_t *)(tp + 2560 + lane * 4);
+                    }
+                }
+            }
+        }
+    };
+    // as in k_gemv: what a thread's first eight values of row 0 are made from is requested ahead of the weights
+    auto row_of = [&](int t) -> const float * {
+        if (SRC == SRC_NORM) return a.xin + (size_t)(a.rows ? a.rows[t] : t) * K;
+        return a.xin + (size_t)t * 2 * K;
+    };
+    auto load_in = [&](int t, int k, f4 (&in)[4]) {
+        if (SRC == SRC_NORM) {
+            const float * xr = row_of(t);
+            in[0] = *(const f4 *)(xr + k); in[1] = *(const f4 *)(xr + k + 4);
+            in[2] = *(const f4 *)(a.norm_w + k); in[3] = *(const f4 *)(a.norm_w + k + 4);
+        } else if (SRC == SRC_SWIGLU) {
+            const float * gp = row_of(t) + (size_t)(k / a.group) * 2 * a.group + k % a.group, * up = gp + a.group;
+            in[0] = *(const f4 *)gp; in[1] = *(const f4 *)(gp + 4); in[2] = *(const f4 *)up; in[3] = *(const f4 *)(up + 4);
+        } else {
+            // the hi and lo halves of eight values: sixteen bytes each
+            in[0] = *(const f4 *)(a.planes + act_at(t, k, 0, K));
+            in[1] = *(const f4 *)(a.planes + act_at(t, k, 1, K));
+        }
+    };
+    f4 first[4];
+    if (tid * 8 < K) load_in(0, tid * 8, first);
+    int tile = blockIdx.x;
+    if (tile < a.n_tiles) request(tile, 0);
+
+    auto store8 = [&](const float (&v)[8], int t, int k) {
+        *(f4 *)(l_x + t * K + k) = (f4){v[0], v[1], v[2], v[3]};
+        *(f4 *)(l_x + t * K + k + 4) = (f4){v[4], v[5], v[6], v[7]};
+        if (KQ) {
+            float sum = ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+            sum += __shfl_xor(sum, 1, 64);
+            if ((tid & 1) == 0) l_s[t * (K >> 4) + (k >> 4)] = sum;
+        }
+    };
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        float scale = 1.0f;
+        if (SRC == SRC_NORM) {
+            const float * xr = row_of(t);
+            float ss = 0.0f;
+            for (int k = tid * 8; k < K; k += nthreads * 8) {
+                f4 in[2];
+                if (t == 0 && k == tid * 8) { in[0] = first[0]; in[1] = first[1]; }
+                else { in[0] = *(const f4 *)(xr + k); in[1] = *(const f4 *)(xr + k + 4); }
+                const f4 p = in[0], q4 = in[1];
+                ss += p.x * p.x + p.y * p.y + p.z * p.z + p.w * p.w + q4.x * q4.x + q4.y * q4.y + q4.z * q4.z + q4.w * q4.w;
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) l_red[wave] = ss;
+            __syncthreads();
+            float total = 0.0f;
+            for (int i = 0; i < nw; ++i) total += l_red[i];
+            scale = 1.0f / sqrtf(total / (float)K + a.eps);
+            if (t + 1 < NT) __syncthreads();
+        }
+        for (int k = tid * 8; k < K; k += nthreads * 8) {
+            f4 in[4];
+            if (t == 0 && k == tid * 8) { in[0] = first[0]; in[1] = first[1]; in[2] = first[2]; in[3] = first[3]; }
+            else load_in(t, k, in);
+            float v[8];
+            if (SRC == SRC_NORM) {
+                v[0] = (in[0].x * scale) * in[2].x; v[1] = (in[0].y * scale) * in[2].y;
+                v[2] = (in[0].z * scale) * in[2].z; v[3] = (in[0].w * scale) * in[2].w;
+                v[4] = (in[1].x * scale) * in[3].x; v[5] = (in[1].y * scale) * in[3].y;
+                v[6] = (in[1].z * scale) * in[3].z; v[7] = (in[1].w * scale) * in[3].w;
+            } else if (SRC == SRC_SWIGLU) {
+                const float gv[8] = {in[0].x, in[0].y, in[0].z, in[0].w, in[1].x, in[1].y, in[1].z, in[1].w};
+                const float uv[8] = {in[2].x, in[2].y, in[2].z, in[2].w, in[3].x, in[3].y, in[3].z, in[3].w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = (gv[i] / (1.0f + __expf(-gv[i]))) * uv[i];
+            } else {
+                const h8 hi = __builtin_bit_cast(h8, in[0]), lo = __builtin_bit_cast(h8, in[1]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = t < a.T ? (float)hi[i] + (float)lo[i] : 0.0f;
+            }
+            store8(v, t, k);
+        }
+    }
+    __syncthreads();
+
+    float acc[NT];
+    // eight codes as bytes in the order 0 4 1 5 (word a) and 2 6 3 7 (word b) times eight values
+    auto dot8 = [&](uint32_t wa, uint32_t wb, const f4 & xa, const f4 & xb) {
+        float p = (float)(wa & 0xffu) * xa.x;
+        p = fmaf((float)((wa >> 16) & 0xffu), xa.y, p);
+        p = fmaf((float)(wb & 0xffu), xa.z, p);
+        p = fmaf((float)((wb >> 16) & 0xffu), xa.w, p);
+        p = fmaf((float)((wa >> 8) & 0xffu), xb.x, p);
+        p = fmaf((float)(wa >> 24), xb.y, p);
+        p = fmaf((float)((wb >> 8) & 0xffu), xb.z, p);
+        p = fmaf((float)(wb >> 24), xb.w, p);
+        return p;
+    };
+    // The values of a lane's eight columns of sub-block d of super-block sb, every token's. A lane reads one group
+    // ahead of the one it multiplies and no further, and converts a group's codes when the group before is done (the
+    // fence in the loops below): left to itself the compiler requests the values and converts the codes of a whole
+    // super-block at once, and with two tokens they do not fit the registers.
+    struct X8 { f4 a[NT], b[NT]; };
+    auto xload = [&](int sb, int d, X8 & x) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const float * at = l_x + t * K + (sb << 8) + (d << 5) + (g << 3);
+            x.a[t] = *(const f4 *)at; x.b[t] = *(const f4 *)(at + 4);
+        }
+    };
+    auto multiply = [&](int sb, int u) {
+        if constexpr (Q4) {
+            const Q4KScales S = q4k_scales(hdr[u]);
+            float dot[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) dot[t] = 0.0f;
+            X8 x;
+            xload(sb, 0, x);
+#pragma unroll
+            for (int d = 0; d < 8; ++d) {
+                const int h = d >> 2, j = d & 3;
+                X8 nx;
+                if (d < 7) xload(sb, d + 1, nx);
+                uint32_t wq = j == 0 ? q[u][h].x : (j == 1 ? q[u][h].y : (j == 2 ? q[u][h].z : q[u][h].w));
+                asm volatile("" : "+v"(wq), "+v"(dot[0]) :: "memory");     // this group's codes behind the last group's products
+                uint32_t lo = wq & 0x0F0F0F0Fu, hi = (wq >> 4) & 0x0F0F0F0Fu;
+                if constexpr (Q5) {
+                    const uint32_t f = fifth[u][h] >> (2 * j);
+                    lo |= ((f << 4) & 0x00100010u) | ((f << 11) & 0x10001000u);
+                    hi |= ((f >> 4) & 0x00100010u) | ((f << 3) & 0x10001000u);
+                }
+                const float sc = (float)((S.sc[h] >> (8 * j)) & 0xffu);
+#pragma unroll
+                for (int t = 0; t < NT; ++t) dot[t] = fmaf(sc, dot8(lo, hi, x.a[t], x.b[t]), dot[t]);
+                if (d < 7) x = nx;
+            }
+            // the min term: lane group g takes sub-blocks 2g and 2g + 1 (sums of sixteen 4g .. 4g + 3)
+            const uint32_t mword = (g < 2 ? S.mn[0] : S.mn[1]) >> (16 * (g & 1));
+            const float m0 = (float)(mword & 0xffu), m1 = (float)((mword >> 8) & 0xffu);
+            const float dw = h2f((uint16_t)(hdr[u].x & 0xffffu)), dmin = h2f((uint16_t)(hdr[u].x >> 16));
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const f4 bs = *(const f4 *)(l_s + t * (K >> 4) + (sb << 4) + 4 * g);
+                const float mins = fmaf(m0, bs.x + bs.y, m1 * (bs.z + bs.w));
+                acc[t] += dw * dot[t] - dmin * mins;
+            }
+        } else if constexpr (Q6) {
+            float dot[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) dot[t] = 0.0f;
+            X8 x;
+            xload(sb, 0, x);
+#pragma unroll
+            for (int d = 0; d < 8; ++d) {
+                const int h = d >> 2, j = d & 3;
+                X8 nx;
+                if (d < 7) xload(sb, d + 1, nx);
+                uint32_t wq = j == 0 ? q[u][h].x : (j == 1 ? q[u][h].y : (j == 2 ? q[u][h].z : q[u][h].w));
+                asm volatile("" : "+v"(wq), "+v"(dot[0]) :: "memory");     // this group's codes behind the last group's products
+                const uint32_t tw = h == 0 ? (j < 2 ? q[u][2].x : q[u][2].y) : (j < 2 ? q[u][2].z : q[u][2].w);
+                const uint32_t top = (j & 1) ? __builtin_amdgcn_alignbit(tw, tw, 8) : tw;
+                const uint32_t lo = (wq & 0x0F0F0F0Fu) | (top & 0x00300030u) | ((top << 4) & 0x30003000u);
+                const uint32_t hi = ((wq >> 4) & 0x0F0F0F0Fu) | ((top >> 2) & 0x00300030u) | ((top << 2) & 0x30003000u);
+                const int b = 8 * h + 2 * j + (g >> 1);
+                const uint32_t sw = (b >> 2) == 0 ? hdr[u].x : ((b >> 2) == 1 ? hdr[u].y : ((b >> 2) == 2 ? hdr[u].z : hdr[u].w));
+                const float sc = (float)(int)(int8_t)((sw >> (8 * (b & 3))) & 0xffu);
+#pragma unroll
+                for (int t = 0; t < NT; ++t) dot[t] = fmaf(sc, dot8(lo, hi, x.a[t], x.b[t]), dot[t]);
+                if (d < 7) x = nx;
+            }
+            // the offset of 32: lane group g takes blocks 4g .. 4g + 3 (the bytes of header dword g)
+            const uint32_t sw = g == 0 ? hdr[u].x : (g == 1 ? hdr[u].y : (g == 2 ? hdr[u].z : hdr[u].w));
+            const float dw = h2f(dq6[u]);
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                const f4 bs = *(const f4 *)(l_s + t * (K >> 4) + (sb << 4) + 4 * g);
+                float corr = (float)(int)(int8_t)(sw & 0xffu) * bs.x;
+                corr = fmaf((float)(int)(int8_t)((sw >> 8) & 0xffu), bs.y, corr);
+                corr = fmaf((float)(int)(int8_t)((sw >> 16) & 0xffu), bs.z, corr);
+                corr = fmaf((float)(int)(int8_t)(sw >> 24), bs.w, corr);
+                acc[t] += dw * fmaf(-32.0f, corr, dot[t]);
+            }
+        } else {
+#pragma unroll
+            for (int qi = 0; qi < 4; ++qi) {
+                const uint32_t pair = qi == 0 ? hdr[u].x : (qi == 1 ? hdr[u].y : (qi == 2 ? hdr[u].z : hdr[u].w));
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int blk = 2 * qi + half;
+                    const float dw = h2f((uint16_t)(half ? pair >> 16 : pair & 0xffffu));
+                    const uint32_t w0 = half ? q[u][qi].z : q[u][qi].x, w1 = half ? q[u][qi].w : q[u][qi].y;
+                    const int k0 = (sb << 8) + (blk << 5) + (g << 3);
+                    float c[8];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        c[i] = (float)(int)(int8_t)((w0 >> (8 * i)) & 0xffu);
+                        c[4 + i] = (float)(int)(int8_t)((w1 >> (8 * i)) & 0xffu);
+                    }
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) {
+                        const f4 xa = *(const f4 *)(l_x + t * K + k0), xb = *(const f4 *)(l_x + t * K + k0 + 4);
+                        float p = c[0] * xa.x;
+                        p = fmaf(c[1], xa.y, p); p = fmaf(c[2], xa.z, p); p = fmaf(c[3], xa.w, p);
+                        p = fmaf(c[4], xb.x, p); p = fmaf(c[5], xb.y, p); p = fmaf(c[6], xb.z, p); p = fmaf(c[7], xb.w, p);
+                        acc[t] = fmaf(dw, p, acc[t]);
+                    }
+                }
+            }
+        }
+    };
+
+    for (int turn = 0; tile < a.n_tiles; tile += gridDim.x, turn ^= 1) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = 0.0f;
+#pragma unroll
+        for (int u0 = 0; u0 < PER; u0 += 2) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int sb = wave + (u0 + u) * nw;
+                if (sb < nsb) multiply(sb, u);
+            }
+            if (u0 + 2 < PER) request(tile, u0 + 2);
+            else if (tile + (int)gridDim.x < a.n_tiles) request(tile + (int)gridDim.x, 0);
+        }
+        float * red = l_red + turn * (nw * NT * 16);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            acc[t] += __shfl_xor(acc[t], 16, 64);
+            acc[t] += __shfl_xor(acc[t], 32, 64);
+            if (g == 0) red[(wave * NT + t) * 16 + r] = acc[t];
+        }
+        __syncthreads();
+        if (tid < NT * 16) {
+            const int t = tid >> 4, row = tid & 15;
+            if (t < a.T) {
+                float v = 0.0f;
+                for (int w = 0; w < nw; ++w) v += red[(w * NT + t) * 16 + row];
+                const int n = tile * 16 + row;
+                if (a.bias) v += a.bias[n];
+                float * dst = a.y + (size_t)t * a.ldy + a.col0 + n;
+                *dst = a.mode == MM_ADD ? *dst + v : v;
+            }
+        }
+    }
+}
+
 constexpr size_t kGemvMaxLds = 96 * 1024;     // of the CU's 160 KiB; two tokens of 24,576 columns take 57 KiB
+constexpr size_t kGemvMaxLdsF32 = 112 * 1024; // the f32 row: 24,576 columns take 104 KiB
 constexpr int kGemvMaxSb = 16 * 6;            // sixteen waves, at most six super-blocks of a tile each
 static size_t gemv_lds_bytes(int type, int NT, int NW, int K) {
     const size_t scales = type == WT_Q8_0 ? (size_t)NT * (K >> 5) * 4 : (size_t)NT * (K >> 8) * 4 + (size_t)NT * (K >> 3);
     return (size_t)NT * K + scales + (size_t)2 * NW * NT * 16 * 4;
+}
+static size_t gemv_f32_lds_bytes(int type, int NT, int NW, int K) {
+    return (size_t)NT * K * 4 + (type == WT_Q8_0 ? 0 : (size_t)NT * (K >> 4) * 4) + (size_t)2 * NW * NT * 16 * 4;
 }
 
 bool gemv_can_weight(const Weight & w, int T) {
     return (w.type == WT_Q4_K || w.type == WT_Q5_K || w.type == WT_Q6_K || w.type == WT_Q8_0) && w.packed && T >= 1 && T <= g_gemv_max_t && T <= GEMV_MAX_T
         && w.K % 256 == 0 && w.N % 16 == 0 && w.K > 0 && w.N > 0
         && w.K <= 256 * kGemvMaxSb && gemv_lds_bytes(w.type, GEMV_MAX_T, 16, w.K) <= kGemvMaxLds;
+}
+
+bool gemv_f32_can_weight(const Weight & w, int T) {
+    return (w.type == WT_Q4_K || w.type == WT_Q5_K || w.type == WT_Q6_K || w.type == WT_Q8_0) && w.packed && T == 1
+        && w.K % 256 == 0 && w.N % 16 == 0 && w.K > 0 && w.N > 0
+        && w.K <= 256 * kGemvMaxSb && gemv_f32_lds_bytes(w.type, T, 16, w.K) <= kGemvMaxLdsF32;
 }
 
 bool gemv_can(const Weight & w, const Act & x, int T) {
@@ -466,6 +767,45 @@ static void launch_gemv_src(hipStream_t s, int type, const GemvArgs & a) {
     else launch_gemv_tokens<WT_Q8_0, SRC>(s, a);
 }
 
+template <int WT, int NT, int PER, int SRC>
+static void launch_gemv_f32(hipStream_t s, const GemvArgs & a) {
+    const int nsb = a.K / 256;
+    const int nw = PER == 2 ? (nsb + 1) / 2 : 16;
+    const size_t lds = gemv_f32_lds_bytes(WT, NT, nw, a.K);
+    static bool once = false;
+    if (!once) {
+        HIP_OK(hipFuncSetAttribute((const void *)k_gemv_f32<WT, NT, PER, SRC>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemvMaxLdsF32));
+        once = true;
+    }
+    // as many workgroups as the chip holds at once (by threads and by LDS), fewer when that gives every
+    // workgroup the same number of tiles
+    const int per_cu = std::max(1, std::min(2048 / (nw * 64), (int)((160 * 1024) / lds)));
+    const int capacity = 256 * per_cu;
+    const int turns = (a.n_tiles + capacity - 1) / capacity;
+    const unsigned grid = (unsigned)((a.n_tiles + turns - 1) / turns);
+    hipLaunchKernelGGL((k_gemv_f32<WT, NT, PER, SRC>), dim3(grid), dim3(nw * 64), lds, s, a);
+}
+
+template <int WT, int SRC>
+static void launch_gemv_f32_tokens(hipStream_t s, const GemvArgs & a) {
+    // single-token steps only: with two tokens' values and products the kernel does not fit the 128 registers a
+    // workgroup of sixteen waves leaves a lane (the compiler spills the staged values), and the tile kernels take the step
+    const int nsb = a.K / 256;
+    if (a.T != 1) throw std::runtime_error("gemv_f32: one token");
+    if (nsb <= 32) launch_gemv_f32<WT, 1, 2, SRC>(s, a);
+    else if (nsb <= 64) launch_gemv_f32<WT, 1, 4, SRC>(s, a);
+    else launch_gemv_f32<WT, 1, 6, SRC>(s, a);
+    check_launch("gemv_f32");
+}
+
+template <int SRC>
+static void launch_gemv_f32_src(hipStream_t s, int type, const GemvArgs & a) {
+    if (type == WT_Q4_K) launch_gemv_f32_tokens<WT_Q4_K, SRC>(s, a);
+    else if (type == WT_Q5_K) launch_gemv_f32_tokens<WT_Q5_K, SRC>(s, a);
+    else if (type == WT_Q6_K) launch_gemv_f32_tokens<WT_Q6_K, SRC>(s, a);
+    else launch_gemv_f32_tokens<WT_Q8_0, SRC>(s, a);
+}
+
 static GemvArgs gemv_args(const Weight & w, int T, float * y, int ldy, int col0, int mode, const float * bias) {
     if (mode != MM_STORE && mode != MM_ADD) throw std::runtime_error("gemv: stores or adds");
     if (col0 < 0 || col0 + w.N > ldy) throw std::runtime_error("gemv: the outputs do not fit the row");
@@ -509,6 +849,31 @@ void gemv_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, i
     GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, nullptr);
     a.xin = gu; a.group = group;
     launch_gemv_src<SRC_SWIGLU>(s, w.type, a);
+}
+
+void gemv_f32(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias) {
+    if (!gemv_f32_can_weight(w, T) || !x.x || x.K != w.K)
+        throw std::runtime_error("gemv_f32: needs Q4_K, Q5_K, Q6_K or Q8_0 tiles, the hi / lo planes of the row and a single token");
+    GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
+    a.planes = x.x;
+    launch_gemv_f32_src<SRC_CODES>(s, w.type, a);
+}
+
+void gemv_f32_norm(hipStream_t s, const Weight & w, const float * x, const float * norm_w, float eps, const int32_t * rows, int T,
+                   float * y, int ldy, int col0, int mode, const float * bias) {
+    if (!gemv_f32_can_weight(w, T) || !x || !norm_w) throw std::runtime_error("gemv_f32_norm: needs Q4_K, Q5_K, Q6_K or Q8_0 tiles, the rows and the norm weights");
+    GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, bias);
+    a.xin = x; a.norm_w = norm_w; a.rows = rows; a.eps = eps;
+    launch_gemv_f32_src<SRC_NORM>(s, w.type, a);
+}
+
+void gemv_f32_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, int T, float * y, int ldy, int col0, int mode) {
+    if (group <= 0) group = w.K;
+    if (!gemv_f32_can_weight(w, T) || !gu || w.K % group != 0 || group % 8 != 0)
+        throw std::runtime_error("gemv_f32_swiglu: needs Q4_K, Q5_K, Q6_K or Q8_0 tiles and gate / up rows in groups that divide the width");
+    GemvArgs a = gemv_args(w, T, y, ldy, col0, mode, nullptr);
+    a.xin = gu; a.group = group;
+    launch_gemv_f32_src<SRC_SWIGLU>(s, w.type, a);
 }
 
 }  // namespace rk

@@ -198,6 +198,13 @@ void gemv_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, i
 constexpr int GEMV_COMBINE_MAX_SPLITS = 16;
 void gemv_combine(hipStream_t s, const Weight & w, const float * partial, int item0, int n_split, int n_head, int G, int head_dim,
                   float * y, int ldy, int col0, int mode);
+// The same kernel in the exact arithmetic (f32 rows, every code converted and multiplied by a fused multiply-add):
+// from the hi / lo planes a producer left (x.x), from residual rows through RMSNorm, from a gate/up product through SwiGLU.
+bool gemv_f32_can_weight(const Weight & w, int T);
+void gemv_f32(hipStream_t s, const Weight & w, const Act & x, int T, float * y, int ldy, int col0, int mode, const float * bias);
+void gemv_f32_norm(hipStream_t s, const Weight & w, const float * x, const float * norm_w, float eps, const int32_t * rows, int T,
+                   float * y, int ldy, int col0, int mode, const float * bias);
+void gemv_f32_swiglu(hipStream_t s, const Weight & w, const float * gu, int group, int T, float * y, int ldy, int col0, int mode);
 extern thread_local int g_gemv_max_t;   // steps of at most this many tokens take the kernel (default GEMV_MAX_T; 0 switches it off);
                                         // an engine sets it from its own configuration at the start of every forward pass
 extern thread_local int g_mm_force_ksplit;  // > 0 overrides the split-K heuristic for the calling thread (kernel-level timing entry point)

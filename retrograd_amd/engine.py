@@ -164,7 +164,7 @@ KERNEL_SYMBOLS = [
     "retro_kernel_matmul", "retro_kernel_gemv_fused", "retro_kernel_matmul_time", "retro_kernel_mxfp4_scaled", "retro_kernel_mxfp4_scaled_time", "retro_kernel_stream_time", "retro_kernel_sample_prepare", "retro_kernel_sample_greedy_noalloc", "retro_kernel_sample_greedy_noalloc_max_rows", "retro_kernel_page_size", "retro_kernel_max_topk",
     "retro_engine_debug_logits", "retro_engine_debug_kv", "retro_engine_debug_pack", "retro_engine_debug_pages",
     "retro_engine_debug_profile", "retro_engine_debug_profile_categories", "retro_engine_debug_profile_read",
-    "retro_engine_debug_attention_timeline", "retro_engine_debug_attention_timeline_read",
+    "retro_engine_debug_attention_timeline", "retro_engine_debug_attention_timeline_read", "retro_engine_debug_single_token_matvec",
 ]
 PROFILE_CATEGORIES = ["pack", "embed", "norm", "qkv", "rope", "attention", "combine", "o_proj", "gate_up", "swiglu",
                       "down", "head", "sample"]
@@ -263,6 +263,7 @@ def load_library() -> C.CDLL:
     lib.retro_engine_debug_pages.argtypes = [C.c_void_p, C.c_int32, _i32p, C.c_size_t, C.POINTER(C.c_size_t)]
     lib.retro_engine_debug_profile.argtypes = [C.c_void_p, C.c_int32]
     lib.retro_engine_debug_attention_timeline.argtypes = [C.c_void_p, C.c_int32]
+    lib.retro_engine_debug_single_token_matvec.argtypes = [C.c_void_p, C.c_int32]
     lib.retro_engine_debug_attention_timeline_read.argtypes = [C.c_void_p, C.POINTER(C.c_uint64), C.c_size_t, C.POINTER(C.c_size_t)]
     lib.retro_engine_debug_profile_categories.restype = C.c_int32
     lib.retro_engine_debug_profile_read.argtypes = [C.c_void_p, C.POINTER(C.c_double), C.POINTER(C.c_uint64), C.c_int32]
@@ -905,6 +906,13 @@ class Engine:
     def profile(self, level: int) -> None:
         """HIP-event timing of kernel categories: 0 off, 1 attention only, 2 all."""
         s = self._lib.retro_engine_debug_profile(self._h, level)
+        if s != 0:
+            _raise(s)
+
+    def single_token_matvec(self, on: bool) -> None:
+        """Single-token steps of the exact arithmetic on the matrix-vector kernel with f32 rows instead of the tile
+        kernels (what RETRO_GEMV_EXACT=1 selects at creation; off by default, see include/retro_kernels.h)."""
+        s = self._lib.retro_engine_debug_single_token_matvec(self._h, 1 if on else 0)
         if s != 0:
             _raise(s)
 

@@ -193,3 +193,48 @@ def test_ggml_arithmetic_at_the_real_widths_two_layers_deep(tmp_path_factory, mo
     compare([5], "one row (integer matrix-vector kernel)")
     compare([9, 40], "two rows (integer matrix-vector kernel)")
     eng.close()
+
+
+def test_single_row_steps_of_the_exact_arithmetic_at_the_real_widths(tmp_path_factory, monkeypatch):
+    # A step of one token runs the matrix-vector kernel with f32 rows (RMSNorm, SwiGLU fused into its staging, the
+    # output projection from the attention launch's planes): its logits against the oracle at the stated tolerances,
+    # and against the tile kernels (RETRO_GEMV_EXACT=0) on the same KV; the fused steps launch no norm of their own.
+    shape = synth.scaled(synth.LLAMA3_8B_Q4K, n_layer=2, name="llama3-8b-widths-2-layers-q4_k")
+    print("exact single-row steps: %s" % shape.name, flush=True)
+    model = _cached(tmp_path_factory, "retro-test-%s-seed77.gguf" % shape.name,
+                    lambda p: synth.write_model(p, shape, seed=77, device="cuda"))
+    n_seq = 4
+    rng = np.random.default_rng(21)
+    lens = [int(n) for n in rng.integers(4, 40, n_seq)]
+    prompts = [rng.integers(0, shape.n_vocab, n).astype(np.int32) for n in lens]
+    m = oracle.Model(model)
+    ctx = oracle.Context(m, n_seq, activations="exact")
+    logits = {}
+    for exact_kernel in (1, 0):
+        monkeypatch.setenv("RETRO_GEMV_EXACT", str(exact_kernel))
+        eng = E.Engine(model, E.EngineConfig(n_ctx=n_seq * 128, n_seq_max=n_seq, n_batch=512, n_ubatch=512))
+        out = E.StepOutput(n_seq)
+        eng.step([E.StepRow(i, i, prompts[i], 0, sample=True, sampling=greedy()) for i in range(n_seq)], out)
+        feed = [out.row(i).token for i in range(n_seq)]
+        if exact_kernel:
+            for s in range(n_seq):
+                ctx.import_snapshot(s, eng.seq_save(s))
+        eng.profile(2)
+        eng.profile_read()
+        got = []
+        for s in range(n_seq):
+            eng.step([E.StepRow(s, s, [feed[s]], lens[s], sample=True, sampling=greedy())], out)
+            got.append(eng.debug_logits()[0].copy())
+        prof = eng.profile_read()
+        eng.profile(0)
+        # two layers: four norm launches per step on the tile kernels (the final norm counts with the head), none on the fused path
+        assert prof["norm"][1] == (0 if exact_kernel else n_seq * 4), prof["norm"]
+        logits[exact_kernel] = np.stack(got)
+        eng.close()
+    want = ctx.step_rows([(s, lens[s], [feed[s]], True) for s in range(n_seq)])
+    assert_logits_close(logits[1], want)
+    assert_logits_close(logits[0], want)
+    mx, mr = logit_errors(logits[1], logits[0])
+    print("matrix-vector kernel against the tile kernels: max %.2e, mean relative %.2e" % (mx, mr), flush=True)
+    assert mx <= 2e-3 and mr <= 1e-4
+

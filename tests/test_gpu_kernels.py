@@ -319,6 +319,60 @@ def test_integer_matvec_with_its_producer_fused(t, kind, n, k, T):
         assert np.abs(fused - unfused).max() <= 8 * flip + 1e-6
 
 
+@pytest.mark.parametrize("t", [gw.GGML_Q4_K, gw.GGML_Q8_0, gw.GGML_Q6_K, gw.GGML_Q5_K])
+@pytest.mark.parametrize("kind", [11, 12])
+@pytest.mark.parametrize("n,k", [(64, 4096), (32, 512), (48, 1024), (32, 14336), (16, 8448), (32, 2048), (32, 3584), (16, 18944), (16, 256),
+                                 (32, 768), (16, 24576)])
+def test_exact_matvec_with_its_producer_fused(t, kind, n, k):
+    # The exact arithmetic's single-token kernel: f32 rows times the decoded weights, the row made by the kernel itself
+    # (RMSNorm of a residual row, SwiGLU of a gate/up product) or read back from the hi / lo planes the producer's own
+    # launch leaves, against the float64 product of the decoded weights with the float64 norm / SiLU. The fused row
+    # keeps all of f32; the planes keep 22 bits of every value.
+    print("case", t, kind, n, k, flush=True)
+    raw, dense = _weights(t, n, k, seed=n + k + kind)
+    rng = np.random.default_rng(k + kind)
+    eps = 1e-5
+    if kind == 11:
+        x = (rng.standard_normal((1, k)) * 3.0).astype(np.float32)
+        w = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+        fused, unfused = E.kernel_gemv_fused(11, t, raw, n, k, x, norm_w=w, eps=eps)
+        x64 = x.astype(np.float64)
+        rows = x64 / np.sqrt((x64 * x64).mean(-1, keepdims=True) + eps) * w
+    else:
+        group = 64 if k % 64 == 0 else 0
+        gu = rng.standard_normal((1, 2 * k)).astype(np.float32)
+        fused, unfused = E.kernel_gemv_fused(12, t, raw, n, k, gu, group=group)
+        g64 = gu.astype(np.float64).reshape(1, k // 64, 2, 64)
+        rows = (g64[:, :, 0] / (1 + np.exp(-g64[:, :, 0])) * g64[:, :, 1]).reshape(1, k)
+    want = rows @ dense.astype(np.float64).T
+    # what f32 products and sums of k terms may lose, against the sum of the terms' magnitudes
+    bound = 4e-7 * (np.abs(rows) @ np.abs(dense).astype(np.float64).T) + 1e-6
+    assert (np.abs(fused - want) <= 8 * bound).all(), float(np.abs(fused - want).max())
+    assert (np.abs(unfused - want) <= 8 * bound).all(), float(np.abs(unfused - want).max())
+    scale = np.abs(want).max()
+    assert np.abs(fused - want).max() <= 2e-5 * scale and np.abs(unfused - want).max() <= 2e-5 * scale
+
+
+def test_exact_matvec_places_every_code():
+    # One non-zero activation at a time: the product is that column of the decoded weights, bit for bit (a single
+    # product per row, nothing to round) - every position of a tile, every sub-block scale and offset.
+    rng = np.random.default_rng(5)
+    for t in (gw.GGML_Q4_K, gw.GGML_Q5_K, gw.GGML_Q6_K, gw.GGML_Q8_0):
+        n, k = 32, 768
+        raw, dense = _weights(t, n, k, seed=int(t) + 3)
+        w = np.ones(k, np.float32)
+        for e in list(range(0, 40)) + [63, 64, 127, 128, 255, 256, 300, 511, 512, 767] + [int(v) for v in rng.integers(0, k, 8)]:
+            gu = np.zeros((1, 2 * k), np.float32)
+            # SwiGLU of (gate, up) = (big, u): silu(40) = 40 to f32 precision, so the staged value is 40 * u
+            blk, off = divmod(e, 64)
+            gu[0, blk * 128 + off] = 40.0
+            gu[0, blk * 128 + 64 + off] = 0.025
+            fused, unfused = E.kernel_gemv_fused(12, t, raw, n, k, gu, group=64)
+            v = np.float32(np.float32(40.0) / (np.float32(1.0) + np.exp(np.float32(-40.0)))) * np.float32(0.025)
+            want = (np.float64(v) * dense[:, e].astype(np.float64))
+            assert np.abs(fused[0] - want).max() <= 1e-6 * np.abs(want).max() + 1e-12, (t, e)
+
+
 def test_q6k_tiles_are_exact_for_every_code_and_scale():
     # Random bytes: every six-bit code, every i8 scale (-128 and 127 included, whose products with a code
     # are not all f16 numbers) in every position of the tile. With d = 1 and small-integer activations all

@@ -1265,6 +1265,38 @@ __global__ __launch_bounds__(256) void k_swiglu_act8(const float * __restrict__ 
     store_act8(v, out, t, k, threadIdx.x & 3);
 }
 
+// The same from a gate/up product left as K-slices (rows of sl.N columns in groups of 128: 64 gate, then the 64 up
+// columns of the same hidden columns): the slices are added in slice order, and hidden column c of the product is
+// column col0 + c of `out`. Eight columns per lane, the four lanes of a 32-wide block together.
+__global__ __launch_bounds__(256) void k_swiglu_slices(Slices sl, int T, int col0, Act out) {
+    const int per = sl.N / 16;
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= (size_t)T * per) return;      // whole groups of four lanes leave together (per % 4 == 0)
+    const int t = (int)(gid / per), c = (int)(gid % per) * 8;
+    const float * g = sl.data + (size_t)t * sl.N + (c / 64) * 128 + c % 64;
+    f4 ga = {0.f, 0.f, 0.f, 0.f}, gb = ga, ua = ga, ub = ga;
+    for (int i = 0; i < sl.n; ++i, g += sl.stride) {
+        ga += *(const f4 *)g; gb += *(const f4 *)(g + 4);
+        ua += *(const f4 *)(g + 64); ub += *(const f4 *)(g + 68);
+    }
+    const float gv[8] = {ga.x, ga.y, ga.z, ga.w, gb.x, gb.y, gb.z, gb.w};
+    const float uv[8] = {ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w};
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (gv[i] / (1.0f + __expf(-gv[i]))) * uv[i];
+    store_act8(v, out, t, col0 + c, threadIdx.x & 3);
+}
+
+void swiglu_slices(hipStream_t s, const Slices & sl, int T, const Act & out, int col0) {
+    if (T <= 0) return;
+    if (!sl.data || sl.n < 1 || sl.weight || sl.N % 128 != 0 || col0 % 32 != 0 || col0 + sl.N / 2 > out.K || (!out.x && !out.qx)
+        || (out.qx && out.quant == AQ_Q8_K))
+        throw std::runtime_error("swiglu_slices: needs plain K-slices of whole groups of 128 columns inside the output row (and no 256-wide conversion)");
+    const size_t n = (size_t)T * (sl.N / 16);
+    hipLaunchKernelGGL(k_swiglu_slices, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, sl, T, col0, out);
+    check_launch("swiglu_slices");
+}
+
 void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out, int group) {
     if (T <= 0) return;
     check_act_out(out, F, "swiglu", T);

@@ -304,6 +304,8 @@ void requant_act(hipStream_t s, const __half * src, int T, const Act & out);
 // act = f16(silu(gu[t][i]) * gu[t][F + i]) (+ block sums).
 // group: gate c at column (c / group) * 2 group + c % group, up c `group` columns further (0: group = F, side by side)
 void swiglu_act(hipStream_t s, const float * gu, int T, int F, const Act & out, int group = 0);
+// silu(gate) * up of a gate/up product left as K-slices (groups of 128 columns: 64 gate, 64 up) into columns col0 .. of out
+void swiglu_slices(hipStream_t s, const Slices & sl, int T, const Act & out, int col0);
 
 // ---- step packing -----------------------------------------------------------
 struct RowDesc {           // one per step row, written by the host

@@ -1092,6 +1092,24 @@ void matmul_swiglu(hipStream_t s, const Weight & w, const Act & x, int T, const 
     }
     const bool via_f32 = out.qx && out.quant == AQ_Q8_K;
     if (via_f32 && !h_f32) throw std::runtime_error("matmul_swiglu: the Q8_K conversion needs the f32 row buffer");
+    // One workgroup per CU and more row groups than CUs: the last round of workgroups would run on a few CUs only
+    // (18944 hidden columns: 296 groups, the second round 40 of 256 CUs for as long as the first). Whole rounds keep
+    // the fused epilogue; the groups left over are multiplied with K split over as many workgroups as fill the chip,
+    // and a small launch adds their slices and applies the SiLU.
+    const int groups = w.N / 128, tail = groups % 256;
+    if (!via_f32 && T > 32 && T <= 64 && w.N % 128 == 0 && groups > 256 && tail > 0 && tail <= 128 && w.K / 256 >= 4 && g_mm_force_ksplit == 0) {
+        const size_t tile = w.type == WT_Q4_K ? 2304 : (w.type == WT_Q5_K ? 2816 : (w.type == WT_Q6_K ? 3360 : 4352));
+        Weight head = w, rest = w;
+        head.N = (groups - tail) * 128;
+        rest.N = tail * 128;
+        rest.packed = w.packed + (size_t)(groups - tail) * 8 * (size_t)(w.K / 256) * tile;
+        head.bytes = rest.bytes = 0;       // views: the bytes belong to w
+        lds_impl(s, head, x, T, nullptr, 0, 0, MM_SWIGLU, nullptr, ws, false, &out, nullptr);
+        const Slices sl = lds_impl(s, rest, x, T, nullptr, rest.N, 0, MM_STORE, nullptr, ws, true, nullptr, nullptr);
+        if (sl.n < 2) throw std::runtime_error("matmul_swiglu: the left-over row groups were not split");
+        swiglu_slices(s, sl, T, out, (groups - tail) * 64);
+        return;
+    }
     lds_impl(s, w, x, T, nullptr, 0, 0, MM_SWIGLU, nullptr, ws, false, &out, via_f32 ? h_f32 : nullptr);
     if (via_f32) to_act(s, h_f32, T, out.K, out);
 }

@@ -238,3 +238,46 @@ def test_single_row_steps_of_the_exact_arithmetic_at_the_real_widths(tmp_path_fa
     print("matrix-vector kernel against the tile kernels: max %.2e, mean relative %.2e" % (mx, mr), flush=True)
     assert mx <= 2e-3 and mr <= 1e-4
 
+
+@pytest.mark.parametrize("matrix_type", [gw.GGML_Q8_0, gw.GGML_Q4_K])
+def test_a_gate_up_matrix_wider_than_the_chip_has_workgroups(tmp_path_factory, matrix_type):
+    # FFN 18944 (the Qwen2.5-7B width) is 296 groups of 128 fused gate/up rows for 256 CUs: steps of 33 to 64 tokens
+    # multiply the first 256 groups with the fused SiLU epilogue and the other 40 with K split over workgroups, a
+    # small launch adding the slices. One layer at hidden 1024 against the oracle, at 64, 40 (split) and 20 rows
+    # (one launch: smaller workgroups share a CU), and the hidden columns on either side of the seam by a copy.
+    shape = synth.scaled(synth.QWEN25_7B_Q8, n_layer=1, n_embd=1024, n_head=8, n_head_kv=2, n_vocab=1024,
+                         matrix_type=matrix_type, name="one-layer-ffn-18944-%d" % matrix_type)
+    print("gate/up with left-over row groups: %s" % shape.name, flush=True)
+    model = _cached(tmp_path_factory, "retro-test-%s-seed5.gguf" % shape.name,
+                    lambda p: synth.write_model(p, shape, seed=5, device="cuda"))
+    n_seq = 64
+    eng = E.Engine(model, E.EngineConfig(n_ctx=n_seq * 64, n_seq_max=n_seq + 1, n_batch=512, n_ubatch=512))
+    rng = np.random.default_rng(3)
+    lens = [int(n) for n in rng.integers(2, 12, n_seq)]
+    prompts = [rng.integers(0, shape.n_vocab, n).astype(np.int32) for n in lens]
+    out = E.StepOutput(n_seq)
+    m = oracle.Model(model)
+    ctx = oracle.Context(m, n_seq + 1)
+    eng.step([E.StepRow(i, i, prompts[i], 0, sample=True, sampling=greedy()) for i in range(n_seq)], out)
+    ctx.step_rows([(i, 0, prompts[i], True) for i in range(n_seq)])
+    feed = [out.row(i).token for i in range(n_seq)]
+    for rows in (64, 40, 20):
+        eng.step([E.StepRow(s, s, [feed[s]], lens[s], sample=True, sampling=greedy()) for s in range(rows)], out)
+        got = eng.debug_logits().copy()
+        want = ctx.step_rows([(s, lens[s], [feed[s]], True) for s in range(rows)])
+        assert_logits_close(got, want)
+        if rows == 64:
+            eng.seq_cp(7, n_seq)
+            eng.seq_rm(n_seq, lens[7], -1)
+            eng.step([E.StepRow(n_seq, n_seq, [feed[7]], lens[7], sample=True, sampling=greedy())]
+                     + [E.StepRow(s, s, [feed[s]], lens[s] + 1, sample=True, sampling=greedy()) for s in range(39)], out)
+            again = eng.debug_logits()[0].copy()
+            eng.seq_rm(n_seq)
+            for s in range(39):
+                eng.seq_rm(s, lens[s] + 1, -1)
+            assert np.array_equal(again, got[7]), "a copy decodes like its source, wherever its row stands"
+        for s in range(rows):
+            eng.seq_rm(s, lens[s], -1)
+            ctx.seq_rm(s, lens[s], -1)
+    eng.close()
+

@@ -281,3 +281,38 @@ def test_a_gate_up_matrix_wider_than_the_chip_has_workgroups(tmp_path_factory, m
             ctx.seq_rm(s, lens[s], -1)
     eng.close()
 
+
+def test_the_left_over_gate_up_groups_under_the_ggml_arithmetic(tmp_path_factory, monkeypatch):
+    # The same split with Q8_0 weights under the ggml arithmetic: the small launch that adds the slices also makes the
+    # Q8_0 blocks of the down projection's rows. One layer deep the engine stays well inside the distance the
+    # conversion itself moves the logits.
+    shape = synth.scaled(synth.QWEN25_7B_Q8, n_layer=1, n_embd=1024, n_head=8, n_head_kv=2, n_vocab=1024,
+                         matrix_type=gw.GGML_Q8_0, name="one-layer-ffn-18944-%d" % gw.GGML_Q8_0)
+    print("gate/up with left-over row groups, ggml arithmetic: %s" % shape.name, flush=True)
+    model = _cached(tmp_path_factory, "retro-test-%s-seed5.gguf" % shape.name,
+                    lambda p: synth.write_model(p, shape, seed=5, device="cuda"))
+    monkeypatch.setenv("RETRO_ACTIVATIONS", "ggml")
+    n_seq = 48
+    eng = E.Engine(model, E.EngineConfig(n_ctx=n_seq * 64, n_seq_max=n_seq, n_batch=512, n_ubatch=512))
+    rng = np.random.default_rng(4)
+    lens = [int(n) for n in rng.integers(2, 12, n_seq)]
+    prompts = [rng.integers(0, shape.n_vocab, n).astype(np.int32) for n in lens]
+    out = E.StepOutput(n_seq)
+    eng.step([E.StepRow(i, i, prompts[i], 0, sample=True, sampling=greedy()) for i in range(n_seq)], out)
+    feed = [out.row(i).token for i in range(n_seq)]
+    m = oracle.Model(model)
+    ggml_ctx, exact_ctx = oracle.Context(m, n_seq, activations="ggml"), oracle.Context(m, n_seq, activations="exact")
+    for s in range(n_seq):
+        snap = eng.seq_save(s)
+        ggml_ctx.import_snapshot(s, snap)
+        exact_ctx.import_snapshot(s, snap)
+    rows = [(s, lens[s], [feed[s]], True) for s in range(n_seq)]
+    eng.step([E.StepRow(s, s, [feed[s]], lens[s], sample=True, sampling=greedy()) for s in range(n_seq)], out)
+    got = eng.debug_logits().copy()
+    want, exact = ggml_ctx.step_rows(rows), exact_ctx.step_rows(rows)
+    drift_max, drift = logit_errors(got, want)
+    _, conversion = logit_errors(exact, want)
+    print("drift %.2e (max %.2e), conversion %.2e" % (drift, drift_max, conversion), flush=True)
+    assert drift < 0.6 * conversion, (drift, conversion)
+    eng.close()
+
